@@ -1,0 +1,175 @@
+/*
+ * peregrine_hip.h -- C ABI of libperegrine_hip.so: peregrine's quantized-inference
+ * operators served by hand-written HIP kernels for AMD MI355X (gfx950).
+ *
+ * Every entry point replaces one function of the reference crate
+ * (etam103/peregrine v0.32.0); the file:line it replaces is cited beside it.
+ * Conventions:
+ *   - plain pointers and sizes only; all matrices are dense row-major;
+ *   - every function returns pg_status (0 = PG_OK) and never aborts or unwinds
+ *     across the ABI; pg_last_error() gives the message of the last failure.
+ *     The reference panics on shape mismatch (assert!/assert_eq!); a binding
+ *     that wants that contract turns a non-zero status into a panic;
+ *   - functions without a `_dev` suffix take HOST pointers, are synchronous, and
+ *     the caller allocates every output (sizes are closed-form);
+ *   - `_dev` functions take DEVICE pointers, are ordered on the context's HIP
+ *     stream, and return without waiting (pg_sync() waits);
+ *   - one pg_ctx = one device + one HIP stream; a context is not internally
+ *     locked (the reference's callers are single-threaded: Tensor is
+ *     Rc<RefCell>, src/tensor.rs:864); distinct contexts may be used from
+ *     distinct threads;
+ *   - the library keeps no host pointer past the return of a call.
+ */
+#ifndef PEREGRINE_HIP_H
+#define PEREGRINE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int pg_status;
+enum {
+    PG_OK = 0,
+    PG_EINVAL = 1,       /* shape / argument mismatch (the reference's assert!s) */
+    PG_EDEVICE = 2,      /* a HIP call failed */
+    PG_ENOMEM = 3,       /* device or host allocation failed */
+    PG_EUNSUPPORTED = 4  /* valid request this build has no kernel for */
+};
+
+/* GGML block types, numbered as src/gguf.rs:14-33 does. */
+enum { PG_GGML_Q4_0 = 2, PG_GGML_Q4_1 = 3, PG_GGML_Q8_0 = 8 };
+
+/* Expert activation of the grouped MoE FFN. */
+enum {
+    PG_ACT_SILU = 0,      /* Tensor::silu  src/tensor.rs:6120-6135 (deepseek/llama experts) */
+    PG_ACT_GELU_TANH = 1  /* Tensor::gelu  src/tensor.rs:3163-3179 (grok1 experts)          */
+};
+
+typedef struct pg_ctx pg_ctx;
+/* Device-resident quant::QuantizedTensor (src/quant.rs:12-23). */
+typedef struct pg_qtensor pg_qtensor;
+/* Device-resident GGUF block tensor ([n_out, k_in], blocks of 32 along k_in). */
+typedef struct pg_gguf_tensor pg_gguf_tensor;
+
+/* ---- context ------------------------------------------------------------
+ * Replaces the thread-local Metal GpuContext singleton
+ * (src/metal/context.rs:2472-2510).  `hip_stream` may be NULL (the library
+ * creates its own default-priority stream) or an existing hipStream_t the
+ * caller owns (for example the stream a host framework launches on). */
+pg_status pg_ctx_create(int device, void *hip_stream, pg_ctx **out);
+void pg_ctx_destroy(pg_ctx *ctx);
+/* GpuContext::sync (used as gpu.sync() in tests/quant_parity.rs:102-107). */
+pg_status pg_sync(pg_ctx *ctx);
+void *pg_ctx_stream(pg_ctx *ctx);
+/* Message of the most recent failure on this thread ("" if none). */
+const char *pg_last_error(void);
+const char *pg_status_string(pg_status st);
+
+/* Device memory for callers that have no HIP binding of their own
+ * (GpuContext::alloc / upload / GpuBuffer::read, src/metal/buffer.rs). */
+pg_status pg_dev_alloc(pg_ctx *ctx, size_t bytes, void **dptr);
+pg_status pg_dev_free(pg_ctx *ctx, void *dptr);
+pg_status pg_memcpy_h2d(pg_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+pg_status pg_memcpy_d2h(pg_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+
+/* ---- quant::* (src/quant.rs) ---------------------------------------------- */
+
+/* quant::quantize_weights  src/quant.rs:27-75.
+ * w [rows, cols] f32 -> q [rows, cols] i8, q_t [cols, rows] i8 (may be NULL),
+ * scales [cols].  scale[n] = absmax(w[:, n]) / 127 (1.0 for a zero column),
+ * q = round_half_away(w / scale) clamped to [-127, 127]. */
+pg_status pg_quantize_weights(pg_ctx *ctx, const float *w, size_t rows, size_t cols,
+                              int8_t *q, int8_t *q_t, float *scales);
+
+/* quant::quantize_activations  src/quant.rs:79-112 (x86 branch :97-109).
+ * a [rows, cols] f32 -> q [rows, cols] i8, row_scales [rows]. */
+pg_status pg_quantize_activations(pg_ctx *ctx, const float *a, size_t rows, size_t cols,
+                                  int8_t *q, float *row_scales);
+pg_status pg_quantize_activations_dev(pg_ctx *ctx, const float *a_dev, size_t rows,
+                                      size_t cols, int8_t *q_dev, float *row_scales_dev);
+
+/* quant::dequantize  src/quant.rs:115-123.  out[m, n] = (q[m, n] as f32) * scales[n]. */
+pg_status pg_dequantize(pg_ctx *ctx, const int8_t *q, const float *scales, size_t rows,
+                        size_t cols, float *out);
+
+/* QuantizedTensor::to_gpu  src/quant.rs:174-181: upload data_i8 [rows, cols] and
+ * scales [cols].  The device copy is kept K-contiguous ([cols, rows], the
+ * reference's data_i8_t, src/quant.rs:57-62) and zero-padded for the kernels. */
+pg_status pg_qtensor_upload(pg_ctx *ctx, const int8_t *q, const float *scales, size_t rows,
+                            size_t cols, pg_qtensor **out);
+/* quantize_weights followed by to_gpu without the round trip through the host:
+ * w is a host (`pg_qtensor_from_f32`) or device (`_dev`) [rows, cols] f32 matrix. */
+pg_status pg_qtensor_from_f32(pg_ctx *ctx, const float *w, size_t rows, size_t cols,
+                              pg_qtensor **out);
+pg_status pg_qtensor_from_f32_dev(pg_ctx *ctx, const float *w_dev, size_t rows, size_t cols,
+                                  pg_qtensor **out);
+/* QuantizedTensor::from_gpu  src/quant.rs:183-190 (q, q_t, scales: any may be NULL). */
+pg_status pg_qtensor_download(pg_ctx *ctx, const pg_qtensor *t, int8_t *q, int8_t *q_t,
+                              float *scales);
+pg_status pg_qtensor_shape(const pg_qtensor *t, size_t *rows, size_t *cols);
+void pg_qtensor_free(pg_ctx *ctx, pg_qtensor *t);
+
+/* quant::matmul_quantized  src/quant.rs:129-169 (the W8A8 CPU semantics: per-row
+ * dynamic i8 activations, i32 accumulate, out = (acc as f32) * a_scale[m] * w_scale[n])
+ * in the slot of quant::matmul_quantized_gpu  src/quant.rs:196-218 /
+ * GpuContext::dispatch_matmul_dequant_i8  src/metal/context.rs:2226-2306.
+ * a [m, k] f32, k == rows of w; out [m, cols of w]. */
+pg_status pg_matmul_quantized(pg_ctx *ctx, const float *a, size_t m, size_t k,
+                              const pg_qtensor *w, float *out);
+/* Device-pointer form.  acc_dev (may be NULL) receives the raw i32 accumulators [m, n]. */
+pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
+                                  const pg_qtensor *w, float *out_dev, int32_t *acc_dev);
+
+/* ---- gguf::* (src/gguf.rs) -------------------------------------------------- */
+
+/* gguf::f16_to_f32  src/gguf.rs:354-382, applied to n values (bit-exact, NaN payloads
+ * included). */
+pg_status pg_f16_to_f32(pg_ctx *ctx, const uint16_t *bits, size_t n, float *out);
+/* gguf::dequant_q8_0  src/gguf.rs:286-302;  gguf::dequant_q4_0  src/gguf.rs:307-326;
+ * gguf::dequant_q4_1  src/gguf.rs:331-351.  num_elements must be a multiple of 32;
+ * data holds num_elements/32 blocks of 34 / 18 / 20 bytes. */
+pg_status pg_dequant_q8_0(pg_ctx *ctx, const uint8_t *data, size_t num_elements, float *out);
+pg_status pg_dequant_q4_0(pg_ctx *ctx, const uint8_t *data, size_t num_elements, float *out);
+pg_status pg_dequant_q4_1(pg_ctx *ctx, const uint8_t *data, size_t num_elements, float *out);
+
+/* Keep a GGUF weight quantised on the device instead of materialising f32 as
+ * GgufFile::load_tensor_f32 + load_transposed_weight do
+ * (src/gguf.rs:485-517, src/models/llama/model.rs:243-257).
+ * blocks: the tensor's raw block bytes, [n_out, k_in] with blocks of 32 along k_in. */
+pg_status pg_gguf_upload(pg_ctx *ctx, const void *blocks, int ggml_type, size_t n_out,
+                         size_t k_in, pg_gguf_tensor **out);
+pg_status pg_gguf_shape(const pg_gguf_tensor *t, size_t *n_out, size_t *k_in, int *ggml_type);
+void pg_gguf_free(pg_ctx *ctx, pg_gguf_tensor *t);
+
+/* The dequantise-then-matmul of models::llama, fused:
+ * y [m, n_out] = x [m, k_in] . dequant(w)^T, i.e. Tensor::matmul
+ * (src/tensor.rs:1342-1353) applied to the transposed dequantised weight. */
+pg_status pg_gguf_matmul(pg_ctx *ctx, const float *x, size_t m, const pg_gguf_tensor *w,
+                         float *y);
+pg_status pg_gguf_matmul_dev(pg_ctx *ctx, const float *x_dev, size_t m,
+                             const pg_gguf_tensor *w, float *y_dev);
+
+/* ---- grouped MoE expert FFN ------------------------------------------------- */
+
+/* MoELayer::forward after the router matmul  examples/grok1/moe.rs:70-109
+ * (expert body examples/grok1/moe.rs:27-34 or examples/deepseek/moe.rs:55-59):
+ *   probs = softmax(router_logits) per token; top_k experts by stable descending
+ *   sort; out[t] = sum_k prob_k * ( act(x_t.Wg_e) * (x_t.Wu_e) ) . Wd_e, k order.
+ * x [T, d]; router_logits [T, E]; gate[e], up[e]: [ffn, d] block tensors;
+ * down[e]: [d, ffn]; out [T, d]. */
+pg_status pg_moe_ffn(pg_ctx *ctx, const float *x, size_t T, const float *router_logits,
+                     size_t E, size_t top_k, const pg_gguf_tensor *const *gate,
+                     const pg_gguf_tensor *const *up, const pg_gguf_tensor *const *down,
+                     int act, float *out);
+pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
+                         const float *router_logits_dev, size_t E, size_t top_k,
+                         const pg_gguf_tensor *const *gate, const pg_gguf_tensor *const *up,
+                         const pg_gguf_tensor *const *down, int act, float *out_dev);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PEREGRINE_HIP_H */

@@ -1,0 +1,433 @@
+/*
+ * peregrine_oracle.c -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * A scalar, single-threaded CPU restatement of the arithmetic of peregrine's
+ * quantized-inference path (the non-aarch64 / non-macOS branches), written
+ * from the reference's source text.  Only tests, the smoke check and the
+ * CPU-baseline leg of the benchmark may load this file's shared object; the
+ * HIP library never links or calls it.
+ *
+ * Compile WITHOUT floating-point contraction and WITHOUT fast-math
+ * (see oracle/Makefile: -O2 -ffp-contract=off -fno-fast-math): Rust never
+ * contracts a*b+c into an FMA and never reassociates.
+ *
+ * Language-semantics pins used throughout (Rust -> C):
+ *   f32::round           == roundf            (half away from zero)
+ *   f32::max(a, b)       == fmaxf             (returns the non-NaN operand)
+ *   f32::clamp(lo, hi)   keeps NaN as NaN
+ *   `as i8` from f32     saturates, NaN -> 0
+ *   `as f32` from i32    round-to-nearest-even (C cast does the same)
+ *
+ * Parity status of each function (what pins it) is listed in
+ * tests/test_oracle_*.py; every function below is pinned by at least one of:
+ * the reference's own known-answer tests, its golden fixture files, a closed
+ * form, or an independent brute-force restatement in NumPy.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* Rust `f32 as i8`: saturating, NaN -> 0. */
+static inline int8_t sat_i8(float v) {
+    if (v != v) return 0;
+    if (v <= -128.0f) return (int8_t)-128;
+    if (v >= 127.0f) return (int8_t)127;
+    return (int8_t)v; /* truncation toward zero, value already in range */
+}
+
+/* Rust `f32::clamp(-127.0, 127.0)`: NaN stays NaN. */
+static inline float clamp127(float v) {
+    if (v != v) return v;
+    if (v < -127.0f) return -127.0f;
+    if (v > 127.0f) return 127.0f;
+    return v;
+}
+
+/* ------------------------------------------------------------------------
+ * quant::quantize_weights            reference: src/quant.rs:27-75
+ *   w       [rows, cols] f32 row-major   (rows = K, cols = N)
+ *   q       [rows, cols] i8
+ *   q_t     [cols, rows] i8  (q_t[n*rows + k] = q[k*cols + n])
+ *   scales  [cols]
+ * ---------------------------------------------------------------------- */
+ORC_API void orc_quantize_weights(const float *w, size_t rows, size_t cols,
+                                  int8_t *q, int8_t *q_t, float *scales) {
+    /* per-column absmax with a strict `>` compare: NaN never wins (quant.rs:31-39) */
+    for (size_t n = 0; n < cols; ++n) scales[n] = 0.0f;
+    for (size_t m = 0; m < rows; ++m)
+        for (size_t n = 0; n < cols; ++n) {
+            float v = fabsf(w[m * cols + n]);
+            if (v > scales[n]) scales[n] = v;
+        }
+    /* scale = amax / 127, or 1.0 for an all-zero column (quant.rs:42-45) */
+    for (size_t n = 0; n < cols; ++n)
+        scales[n] = (scales[n] == 0.0f) ? 1.0f : scales[n] / 127.0f;
+    /* q = round(w / scale) with a true divide (quant.rs:48-54) */
+    for (size_t m = 0; m < rows; ++m)
+        for (size_t n = 0; n < cols; ++n) {
+            float v = w[m * cols + n] / scales[n];
+            q[m * cols + n] = sat_i8(clamp127(roundf(v)));
+        }
+    /* transpose for the GEMM (quant.rs:57-62) */
+    if (q_t)
+        for (size_t k = 0; k < rows; ++k)
+            for (size_t n = 0; n < cols; ++n) q_t[n * rows + k] = q[k * cols + n];
+}
+
+/* ------------------------------------------------------------------------
+ * quant::quantize_activations        reference: src/quant.rs:79-112
+ *   (the cfg(not(target_arch = "aarch64")) branch, quant.rs:97-109)
+ *   a [rows, cols] f32 -> q [rows, cols] i8, row_scales [rows]
+ * ---------------------------------------------------------------------- */
+ORC_API void orc_quantize_activations(const float *a, size_t rows, size_t cols,
+                                      int8_t *q, float *row_scales) {
+    for (size_t m = 0; m < rows; ++m) {
+        const float *row = a + m * cols;
+        float amax = 0.0f;
+        for (size_t k = 0; k < cols; ++k) amax = fmaxf(amax, fabsf(row[k]));
+        float scale = (amax == 0.0f) ? 1.0f : amax / 127.0f;
+        row_scales[m] = scale;
+        float inv_scale = 1.0f / scale; /* multiply by reciprocal, not a divide */
+        for (size_t k = 0; k < cols; ++k)
+            q[m * cols + k] = sat_i8(clamp127(roundf(row[k] * inv_scale)));
+    }
+}
+
+/* quant::dequantize                  reference: src/quant.rs:115-123 */
+ORC_API void orc_dequantize(const int8_t *q, const float *scales, size_t rows,
+                            size_t cols, float *out) {
+    for (size_t m = 0; m < rows; ++m)
+        for (size_t n = 0; n < cols; ++n)
+            out[m * cols + n] = (float)q[m * cols + n] * scales[n];
+}
+
+/* ------------------------------------------------------------------------
+ * The i8 x i8 -> i32 GEMM with f32 rescale of quant::matmul_quantized
+ *                                    reference: src/quant.rs:154-166
+ *   a_i8 [m, k], b_t [n, k] (the pre-transposed weights), out [m, n].
+ *   acc_out (optional) receives the raw i32 accumulators.
+ *   Epilogue order is ((acc as f32) * a_scale[m]) * w_scale[n].
+ * ---------------------------------------------------------------------- */
+ORC_API void orc_gemm_i8(const int8_t *a_i8, const float *a_scales,
+                         const int8_t *b_t, const float *w_scales, size_t m,
+                         size_t n, size_t k, float *out, int32_t *acc_out) {
+    for (size_t mi = 0; mi < m; ++mi)
+        for (size_t ni = 0; ni < n; ++ni) {
+            int32_t acc = 0;
+            const int8_t *ar = a_i8 + mi * k;
+            const int8_t *br = b_t + ni * k;
+            for (size_t ki = 0; ki < k; ++ki) acc += (int32_t)ar[ki] * (int32_t)br[ki];
+            if (acc_out) acc_out[mi * n + ni] = acc;
+            if (out) out[mi * n + ni] = (float)acc * a_scales[mi] * w_scales[ni];
+        }
+}
+
+/* quant::matmul_quantized            reference: src/quant.rs:129-169
+ *   a [m, k] f32; weights given as (q_t [n, k], w_scales [n]).
+ *   Returns 0, or -1 if scratch allocation failed. */
+ORC_API int orc_matmul_quantized(const float *a, size_t m, size_t k,
+                                 const int8_t *q_t, const float *w_scales,
+                                 size_t n, float *out, int32_t *acc_out) {
+    int8_t *a_i8 = (int8_t *)malloc((m * k) > 0 ? m * k : 1);
+    float *a_sc = (float *)malloc((m ? m : 1) * sizeof(float));
+    if (!a_i8 || !a_sc) { free(a_i8); free(a_sc); return -1; }
+    orc_quantize_activations(a, m, k, a_i8, a_sc);
+    orc_gemm_i8(a_i8, a_sc, q_t, w_scales, m, n, k, out, acc_out);
+    free(a_i8);
+    free(a_sc);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------
+ * gguf::f16_to_f32                   reference: src/gguf.rs:354-382
+ *   Bit-level IEEE half -> single, including the subnormal normalise loop
+ *   and NaN payload = mant << 13 (signalling NaNs are NOT quietened).
+ * ---------------------------------------------------------------------- */
+ORC_API uint32_t orc_f16_to_f32_bits(uint16_t bits) {
+    uint32_t sign = (bits >> 15) & 1u;
+    uint32_t exp = (bits >> 10) & 0x1Fu;
+    uint32_t mant = bits & 0x3FFu;
+    if (exp == 0) {
+        if (mant == 0) return sign << 31;
+        uint32_t m = mant;
+        int32_t e = 0;
+        while ((m & 0x400u) == 0) { m <<= 1; e -= 1; }
+        m &= 0x3FFu;
+        uint32_t f32_exp = (uint32_t)(127 - 15 + 1 + e);
+        return (sign << 31) | (f32_exp << 23) | (m << 13);
+    }
+    if (exp == 31) return (sign << 31) | (0xFFu << 23) | (mant << 13);
+    return (sign << 31) | ((exp + 127 - 15) << 23) | (mant << 13);
+}
+
+static inline float f16_to_f32(uint16_t bits) {
+    uint32_t u = orc_f16_to_f32_bits(bits);
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+ORC_API float orc_f16_to_f32(uint16_t bits) { return f16_to_f32(bits); }
+
+/* gguf::dequant_q8_0                 reference: src/gguf.rs:286-302
+ *   block = [f16 d, little-endian][32 x i8]; out[32b+i] = (q as f32) * d.
+ *   Returns 0, or -1 if n is not a multiple of 32 (the reference asserts). */
+ORC_API int orc_dequant_q8_0(const uint8_t *data, size_t n, float *out) {
+    if (n % 32) return -1;
+    size_t nb = n / 32;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t *blk = data + b * 34;
+        float d = f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        for (int i = 0; i < 32; ++i) out[b * 32 + i] = (float)(int8_t)blk[2 + i] * d;
+    }
+    return 0;
+}
+
+/* gguf::dequant_q4_0                 reference: src/gguf.rs:307-326
+ *   block = [f16 d][16 bytes]; byte i -> out[32b+2i]   = ((byte & 15) - 8) * d
+ *                                        out[32b+2i+1] = ((byte >> 4) - 8) * d
+ *   (interleaved element order, as the reference has it). */
+ORC_API int orc_dequant_q4_0(const uint8_t *data, size_t n, float *out) {
+    if (n % 32) return -1;
+    size_t nb = n / 32;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t *blk = data + b * 18;
+        float d = f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        for (int i = 0; i < 16; ++i) {
+            int32_t lo = (int32_t)(blk[2 + i] & 0x0F) - 8;
+            int32_t hi = (int32_t)((blk[2 + i] >> 4) & 0x0F) - 8;
+            out[b * 32 + 2 * i] = (float)lo * d;
+            out[b * 32 + 2 * i + 1] = (float)hi * d;
+        }
+    }
+    return 0;
+}
+
+/* gguf::dequant_q4_1                 reference: src/gguf.rs:331-351
+ *   block = [f16 d][f16 m][16 bytes]; value = nibble * d + m (mul then add). */
+ORC_API int orc_dequant_q4_1(const uint8_t *data, size_t n, float *out) {
+    if (n % 32) return -1;
+    size_t nb = n / 32;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t *blk = data + b * 20;
+        float d = f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        float mn = f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+        for (int i = 0; i < 16; ++i) {
+            float lo = (float)(blk[4 + i] & 0x0F);
+            float hi = (float)((blk[4 + i] >> 4) & 0x0F);
+            out[b * 32 + 2 * i] = lo * d + mn;
+            out[b * 32 + 2 * i + 1] = hi * d + mn;
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------
+ * Tensor::matmul, non-macOS branch   reference: src/tensor.rs:1342-1353
+ *   a [m, k] . b [k, n] -> out [m, n]; sum starts at 0, `sum += a*b`
+ *   K-sequential, separate multiply and add.
+ * ---------------------------------------------------------------------- */
+ORC_API void orc_matmul_f32(const float *a, const float *b, size_t m, size_t k,
+                            size_t n, float *out) {
+    for (size_t i = 0; i < m; ++i)
+        for (size_t j = 0; j < n; ++j) {
+            float sum = 0.0f;
+            for (size_t p = 0; p < k; ++p) sum += a[i * k + p] * b[p * n + j];
+            out[i * n + j] = sum;
+        }
+}
+
+/* Same sums as orc_matmul_f32 when b is given transposed (bt [n, k]):
+ * identical operands in identical order, only the memory walk differs, so
+ * results are bit-identical.  Used to make full-size checks tractable. */
+static void matmul_f32_bt(const float *a, const float *bt, size_t m, size_t k,
+                          size_t n, float *out) {
+    for (size_t i = 0; i < m; ++i)
+        for (size_t j = 0; j < n; ++j) {
+            float sum = 0.0f;
+            const float *ar = a + i * k, *br = bt + j * k;
+            for (size_t p = 0; p < k; ++p) sum += ar[p] * br[p];
+            out[i * n + j] = sum;
+        }
+}
+
+/* ------------------------------------------------------------------------
+ * GGUF dequant-matmul as models::llama composes it:
+ *   load_tensor_f32 (gguf.rs:485-517) -> dequant_q8_0 / dequant_q4_0 of the
+ *   whole [n_out, k_in] tensor, transpose to [k_in, n_out]
+ *   (models/llama/model.rs:243-257), then x.matmul(w) (tensor.rs:1342-1353).
+ *   ggml_type: 2 = Q4_0, 3 = Q4_1, 8 = Q8_0 (gguf.rs:30-45 numbering).
+ *   y [m, n_out].  Returns 0 on success.
+ * ---------------------------------------------------------------------- */
+ORC_API int orc_gguf_matmul(const float *x, size_t m, const uint8_t *blocks,
+                            int ggml_type, size_t n_out, size_t k_in, float *y) {
+    float *wf = (float *)malloc(n_out * k_in * sizeof(float) + 4);
+    if (!wf) return -1;
+    int rc;
+    if (ggml_type == 8) rc = orc_dequant_q8_0(blocks, n_out * k_in, wf);
+    else if (ggml_type == 2) rc = orc_dequant_q4_0(blocks, n_out * k_in, wf);
+    else if (ggml_type == 3) rc = orc_dequant_q4_1(blocks, n_out * k_in, wf);
+    else rc = -2;
+    if (rc == 0) matmul_f32_bt(x, wf, m, k_in, n_out, y); /* wf is [n_out, k_in] = b^T */
+    free(wf);
+    return rc;
+}
+
+/* Tensor::softmax over the last dim, non-aarch64 branch
+ *                                    reference: src/tensor.rs:2833-2858 */
+ORC_API void orc_softmax_rows(const float *x, size_t rows, size_t cols, float *out) {
+    for (size_t r = 0; r < rows; ++r) {
+        const float *xi = x + r * cols;
+        float *oi = out + r * cols;
+        float mx = -INFINITY;
+        for (size_t d = 0; d < cols; ++d)
+            if (xi[d] > mx) mx = xi[d];
+        float sum = 0.0f;
+        for (size_t d = 0; d < cols; ++d) {
+            float e = expf(xi[d] - mx);
+            oi[d] = e;
+            sum += e;
+        }
+        for (size_t d = 0; d < cols; ++d) oi[d] /= sum;
+    }
+}
+
+/* Tensor::silu, non-aarch64          reference: src/tensor.rs:6129-6133 */
+static inline float silu_tensor(float x) {
+    float sig = 1.0f / (1.0f + expf(-x));
+    return x * sig;
+}
+/* Llama SwiGLU glue, non-macOS       reference: src/models/llama/decoder.rs:143-150 */
+static inline float silu_llama(float g) { return g / (1.0f + expf(-g)); }
+/* Tensor::gelu, non-aarch64 (tanh form) reference: src/tensor.rs:3163-3179 */
+static inline float gelu_tanh(float x) {
+    float c = sqrtf(2.0f / 3.14159265358979323846f);
+    float inner = c * (x + 0.044715f * x * x * x);
+    return 0.5f * x * (1.0f + tanhf(inner));
+}
+
+ORC_API void orc_silu(const float *x, size_t n, float *out) {
+    for (size_t i = 0; i < n; ++i) out[i] = silu_tensor(x[i]);
+}
+ORC_API void orc_gelu_tanh(const float *x, size_t n, float *out) {
+    for (size_t i = 0; i < n; ++i) out[i] = gelu_tanh(x[i]);
+}
+ORC_API void orc_swiglu_llama(const float *g, const float *u, size_t n, float *out) {
+    for (size_t i = 0; i < n; ++i) out[i] = silu_llama(g[i]) * u[i];
+}
+
+/* ------------------------------------------------------------------------
+ * MoE layer forward with block-quantised experts.
+ *   Routing and accumulation: examples/grok1/moe.rs:70-109
+ *     probs = softmax(logits) per token; stable sort descending by prob
+ *     (ties keep the lower expert index first); for k < top_k:
+ *     out[t] += prob * expert(x[t]), in k order, raw (unrenormalised) probs.
+ *   Expert:  act(x.Wg) * (x.Wu) . Wd
+ *     act = 0: Tensor::silu  (examples/deepseek/moe.rs:55-59)
+ *     act = 1: Tensor::gelu  (examples/grok1/moe.rs:27-34)
+ *   Each expert matrix is GGUF block data in [out, in] orientation and goes
+ *   through the dequant -> transpose -> f32 matmul composition above.
+ *     gate[e], up[e]: n_out = ffn, k_in = d;   down[e]: n_out = d, k_in = ffn
+ *   x [T, d], logits [T, E], out [T, d].  Returns 0 on success.
+ *   topk_idx / topk_prob (optional, [T, top_k]) receive the routing.
+ * ---------------------------------------------------------------------- */
+ORC_API int orc_moe_ffn(const float *x, size_t T, size_t d, size_t ffn, size_t E,
+                        size_t top_k, const float *logits,
+                        const uint8_t *const *gate, const uint8_t *const *up,
+                        const uint8_t *const *down, int ggml_type, int act,
+                        float *out, int32_t *topk_idx, float *topk_prob) {
+    if (top_k > E) return -3;
+    float *probs = (float *)malloc(T * E * sizeof(float) + 4);
+    float *g = (float *)malloc(ffn * sizeof(float));
+    float *u = (float *)malloc(ffn * sizeof(float));
+    float *h = (float *)malloc(ffn * sizeof(float));
+    float *y = (float *)malloc(d * sizeof(float));
+    size_t *order = (size_t *)malloc((E ? E : 1) * sizeof(size_t));
+    int rc = 0;
+    if (!probs || !g || !u || !h || !y || !order) { rc = -1; goto done; }
+    orc_softmax_rows(logits, T, E, probs);
+    memset(out, 0, T * d * sizeof(float));
+    for (size_t t = 0; t < T; ++t) {
+        const float *p = probs + t * E;
+        /* stable insertion sort, descending: equal probs keep index order */
+        for (size_t e = 0; e < E; ++e) {
+            size_t j = e;
+            while (j > 0 && p[order[j - 1]] < p[e]) { order[j] = order[j - 1]; --j; }
+            order[j] = e;
+        }
+        const float *xt = x + t * d;
+        for (size_t k = 0; k < top_k; ++k) {
+            size_t e = order[k];
+            float prob = p[e];
+            if (topk_idx) topk_idx[t * top_k + k] = (int32_t)e;
+            if (topk_prob) topk_prob[t * top_k + k] = prob;
+            if ((rc = orc_gguf_matmul(xt, 1, gate[e], ggml_type, ffn, d, g))) goto done;
+            if ((rc = orc_gguf_matmul(xt, 1, up[e], ggml_type, ffn, d, u))) goto done;
+            for (size_t i = 0; i < ffn; ++i)
+                h[i] = (act == 1 ? gelu_tanh(g[i]) : silu_tensor(g[i])) * u[i];
+            if ((rc = orc_gguf_matmul(h, 1, down[e], ggml_type, d, ffn, y))) goto done;
+            for (size_t i = 0; i < d; ++i) out[t * d + i] += prob * y[i];
+        }
+    }
+done:
+    free(probs); free(g); free(u); free(h); free(y); free(order);
+    return rc;
+}
+
+/* ------------------------------------------------------------------------
+ * Input synthesis: SplitMix64-seeded Xoshiro256++ and Box-Muller normals
+ *                                    reference: src/random.rs:16-53, 311-380
+ *   (the sequential generator; the reference switches to a Philox path above
+ *   a size threshold, which is not restated).
+ * ---------------------------------------------------------------------- */
+typedef struct { uint64_t s[4]; } orc_rng;
+
+static inline uint64_t rotl64(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+
+ORC_API void orc_rng_seed(orc_rng *r, uint64_t seed) {
+    uint64_t sm = seed;
+    for (int i = 0; i < 4; ++i) {
+        sm += 0x9E3779B97F4A7C15ull;
+        uint64_t z = sm;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        r->s[i] = z ^ (z >> 31);
+    }
+}
+
+ORC_API uint64_t orc_rng_next_u64(orc_rng *r) {
+    uint64_t *s = r->s;
+    uint64_t result = rotl64(s[0] + s[3], 23) + s[0];
+    uint64_t t = s[1] << 17;
+    s[2] ^= s[0];
+    s[3] ^= s[1];
+    s[1] ^= s[2];
+    s[0] ^= s[3];
+    s[2] ^= t;
+    s[3] = rotl64(s[3], 45);
+    return result;
+}
+
+static inline float rng_next_f32(orc_rng *r) {
+    return (float)(orc_rng_next_u64(r) >> 40) / (float)(1ull << 24);
+}
+
+ORC_API void orc_rng_normal(uint64_t seed, size_t n, float mean, float std, float *out) {
+    orc_rng r;
+    orc_rng_seed(&r, seed);
+    size_t pairs = (n + 1) / 2;
+    /* the reference draws all (u1, u2) pairs first, then transforms them;
+     * drawing pair by pair consumes the stream in the same order */
+    for (size_t i = 0; i < pairs; ++i) {
+        float u1 = fmaxf(rng_next_f32(&r), 1e-10f);
+        float u2 = rng_next_f32(&r);
+        float rad = sqrtf(-2.0f * logf(u1));
+        float theta = 2.0f * 3.14159265358979323846f * u2;
+        out[2 * i] = mean + std * rad * cosf(theta);
+        if (2 * i + 1 < n) out[2 * i + 1] = mean + std * rad * sinf(theta);
+    }
+}

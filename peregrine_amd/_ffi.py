@@ -1,0 +1,84 @@
+"""ctypes binding of libperegrine_hip.so (the C ABI declared in include/peregrine_hip.h)."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libperegrine_hip.so")
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+        "or `make -C peregrine_amd/csrc`. peregrine_amd has no CPU fallback."
+    )
+
+lib = C.CDLL(LIB_PATH)
+
+PG_OK, PG_EINVAL, PG_EDEVICE, PG_ENOMEM, PG_EUNSUPPORTED = 0, 1, 2, 3, 4
+GGML_Q4_0, GGML_Q4_1, GGML_Q8_0 = 2, 3, 8
+ACT_SILU, ACT_GELU_TANH = 0, 1
+
+_vp, _sz, _int = C.c_void_p, C.c_size_t, C.c_int
+_pp = C.POINTER(C.c_void_p)
+
+# name -> argtypes; every function returns pg_status unless listed in _OTHER_RESTYPE.
+SIGNATURES = {
+    "pg_ctx_create": [_int, _vp, _pp],
+    "pg_ctx_destroy": [_vp],
+    "pg_sync": [_vp],
+    "pg_ctx_stream": [_vp],
+    "pg_last_error": [],
+    "pg_status_string": [_int],
+    "pg_dev_alloc": [_vp, _sz, _pp],
+    "pg_dev_free": [_vp, _vp],
+    "pg_memcpy_h2d": [_vp, _vp, _vp, _sz],
+    "pg_memcpy_d2h": [_vp, _vp, _vp, _sz],
+    "pg_quantize_weights": [_vp, _vp, _sz, _sz, _vp, _vp, _vp],
+    "pg_quantize_activations": [_vp, _vp, _sz, _sz, _vp, _vp],
+    "pg_quantize_activations_dev": [_vp, _vp, _sz, _sz, _vp, _vp],
+    "pg_dequantize": [_vp, _vp, _vp, _sz, _sz, _vp],
+    "pg_qtensor_upload": [_vp, _vp, _vp, _sz, _sz, _pp],
+    "pg_qtensor_from_f32": [_vp, _vp, _sz, _sz, _pp],
+    "pg_qtensor_from_f32_dev": [_vp, _vp, _sz, _sz, _pp],
+    "pg_qtensor_download": [_vp, _vp, _vp, _vp, _vp],
+    "pg_qtensor_shape": [_vp, C.POINTER(_sz), C.POINTER(_sz)],
+    "pg_qtensor_free": [_vp, _vp],
+    "pg_matmul_quantized": [_vp, _vp, _sz, _sz, _vp, _vp],
+    "pg_matmul_quantized_dev": [_vp, _vp, _sz, _sz, _vp, _vp, _vp],
+    "pg_f16_to_f32": [_vp, _vp, _sz, _vp],
+    "pg_dequant_q8_0": [_vp, _vp, _sz, _vp],
+    "pg_dequant_q4_0": [_vp, _vp, _sz, _vp],
+    "pg_dequant_q4_1": [_vp, _vp, _sz, _vp],
+    "pg_gguf_upload": [_vp, _vp, _int, _sz, _sz, _pp],
+    "pg_gguf_shape": [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_int)],
+    "pg_gguf_free": [_vp, _vp],
+    "pg_gguf_matmul": [_vp, _vp, _sz, _vp, _vp],
+    "pg_gguf_matmul_dev": [_vp, _vp, _sz, _vp, _vp],
+    "pg_moe_ffn": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
+    "pg_moe_ffn_dev": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
+}
+_OTHER_RESTYPE = {
+    "pg_ctx_destroy": None,
+    "pg_qtensor_free": None,
+    "pg_gguf_free": None,
+    "pg_ctx_stream": _vp,
+    "pg_last_error": C.c_char_p,
+    "pg_status_string": C.c_char_p,
+}
+
+for _name, _args in SIGNATURES.items():
+    _fn = getattr(lib, _name)  # AttributeError here = header and library disagree
+    _fn.argtypes = _args
+    _fn.restype = _OTHER_RESTYPE.get(_name, _int)
+
+
+class PeregrineError(RuntimeError):
+    """A non-zero pg_status.  The reference panics in these places (assert!/expect)."""
+
+    def __init__(self, status, message):
+        super().__init__(f"[{lib.pg_status_string(status).decode()}] {message}")
+        self.status = status
+
+
+def check(status):
+    if status != PG_OK:
+        raise PeregrineError(status, lib.pg_last_error().decode())

@@ -1,0 +1,138 @@
+// Context, status and device-memory entry points of libperegrine_hip.
+#include <stdarg.h>
+#include <stdio.h>
+#include <new>
+#include "pg_internal.h"
+
+static thread_local char g_err[512] = "";
+
+pg_status pg_fail(pg_status st, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return st;
+}
+
+PG_API const char *pg_last_error(void) { return g_err; }
+
+PG_API const char *pg_status_string(pg_status st) {
+    switch (st) {
+        case PG_OK: return "ok";
+        case PG_EINVAL: return "invalid argument";
+        case PG_EDEVICE: return "device error";
+        case PG_ENOMEM: return "out of memory";
+        case PG_EUNSUPPORTED: return "unsupported";
+        default: return "unknown status";
+    }
+}
+
+pg_status pg_use(pg_ctx *ctx) {
+    PG_CHECK_ARG(ctx != nullptr, "null context");
+    PG_HIP(hipSetDevice(ctx->device));
+    return PG_OK;
+}
+
+pg_status pg_launch_check(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return pg_fail(PG_EDEVICE, "launch of %s failed: %s", what, hipGetErrorString(e));
+    return PG_OK;
+}
+
+pg_status pg_workspace(pg_ctx *ctx, size_t bytes, void **out) {
+    if (bytes > ctx->ws_bytes) {
+        // Work already queued may still use the old arena: drain before replacing it.
+        PG_HIP(hipStreamSynchronize(ctx->stream));
+        if (ctx->ws) PG_HIP(hipFree(ctx->ws));
+        ctx->ws = nullptr;
+        ctx->ws_bytes = 0;
+        size_t want = pg_round_up(bytes + bytes / 4, 1 << 20);
+        PG_HIP(hipMalloc(&ctx->ws, want));
+        ctx->ws_bytes = want;
+    }
+    *out = ctx->ws;
+    return PG_OK;
+}
+
+PG_API pg_status pg_ctx_create(int device, void *hip_stream, pg_ctx **out) {
+    PG_CHECK_ARG(out != nullptr, "pg_ctx_create: out is null");
+    *out = nullptr;
+    int count = 0;
+    PG_HIP(hipGetDeviceCount(&count));
+    PG_CHECK_ARG(device >= 0 && device < count, "pg_ctx_create: device %d of %d", device, count);
+    PG_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    PG_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return pg_fail(PG_EUNSUPPORTED, "device %d is %s; this library holds gfx950 code only",
+                       device, prop.gcnArchName);
+    pg_ctx *ctx = new (std::nothrow) pg_ctx();
+    if (!ctx) return pg_fail(PG_ENOMEM, "pg_ctx_create: host allocation failed");
+    ctx->device = device;
+    ctx->ws = nullptr;
+    ctx->ws_bytes = 0;
+    ctx->num_cu = prop.multiProcessorCount;
+    if (hip_stream) {
+        ctx->stream = static_cast<hipStream_t>(hip_stream);
+        ctx->owns_stream = false;
+    } else {
+        hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+        if (e != hipSuccess) {
+            delete ctx;
+            return pg_fail(PG_EDEVICE, "hipStreamCreate failed: %s", hipGetErrorString(e));
+        }
+        ctx->owns_stream = true;
+    }
+    *out = ctx;
+    return PG_OK;
+}
+
+PG_API void pg_ctx_destroy(pg_ctx *ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->ws) (void)hipFree(ctx->ws);
+    if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+PG_API pg_status pg_sync(pg_ctx *ctx) {
+    PG_TRY(pg_use(ctx));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+PG_API void *pg_ctx_stream(pg_ctx *ctx) { return ctx ? static_cast<void *>(ctx->stream) : nullptr; }
+
+PG_API pg_status pg_dev_alloc(pg_ctx *ctx, size_t bytes, void **dptr) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(dptr != nullptr, "pg_dev_alloc: dptr is null");
+    PG_HIP(hipMalloc(dptr, bytes ? bytes : 1));
+    return PG_OK;
+}
+
+PG_API pg_status pg_dev_free(pg_ctx *ctx, void *dptr) {
+    PG_TRY(pg_use(ctx));
+    if (!dptr) return PG_OK;
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    PG_HIP(hipFree(dptr));
+    return PG_OK;
+}
+
+PG_API pg_status pg_memcpy_h2d(pg_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes) {
+    PG_TRY(pg_use(ctx));
+    if (!bytes) return PG_OK;
+    PG_CHECK_ARG(dst_dev && src_host, "pg_memcpy_h2d: null pointer");
+    PG_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+PG_API pg_status pg_memcpy_d2h(pg_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
+    PG_TRY(pg_use(ctx));
+    if (!bytes) return PG_OK;
+    PG_CHECK_ARG(dst_host && src_dev, "pg_memcpy_d2h: null pointer");
+    PG_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}

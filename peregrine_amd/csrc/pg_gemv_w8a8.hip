@@ -1,0 +1,127 @@
+// Decode-shaped W8A8 product (m <= 4 activation rows): a weight-streaming
+// dot-product kernel.  HBM-bound: every weight byte is read exactly once with
+// 128-bit loads, multiplied with v_dot4_i32_i8 against the quantised
+// activation rows held in LDS, and reduced across the wavefront.
+//
+//   out[m, n] = (float)(sum_k a_i8[m, k] * w_t[n, k]) * a_scale[m] * w_scale[n]
+//
+// Integer sums are exact, so the lane/chunk order does not matter; the f32
+// epilogue keeps the reference's multiplication order (src/quant.rs:163).
+#include "pg_internal.h"
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int wave_sum_i32(int v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ int dot16(v4i w, v4i x, int acc) {
+    acc = __builtin_amdgcn_sdot4(w.x, x.x, acc, false);
+    acc = __builtin_amdgcn_sdot4(w.y, x.y, acc, false);
+    acc = __builtin_amdgcn_sdot4(w.z, x.z, acc, false);
+    acc = __builtin_amdgcn_sdot4(w.w, x.w, acc, false);
+    return acc;
+}
+
+// One wavefront owns R consecutive weight rows (output columns); a workgroup is
+// 4 wavefronts.  Lane l reads the 16-byte chunks l, l+64, ... of each row, so a
+// wavefront load covers 1 KiB of contiguous weights.  w_t rows are padded to
+// n_pad (a multiple of 4*R*gridDim granularity) and k_pad, so no load needs a
+// bounds check; only the final store is masked by n.
+template <int R, int M>
+__global__ __launch_bounds__(256) void gemv_w8a8_kernel(
+    const int8_t *__restrict__ w_t, int k_pad, const float *__restrict__ w_scales,
+    const int8_t *__restrict__ a_i8, int a_stride, const float *__restrict__ a_scales, int n,
+    float *__restrict__ out, int32_t *__restrict__ acc_out) {
+    extern __shared__ v4i xs[];  // [M][k_pad / 16]
+    const int nchunk = k_pad >> 4;
+    for (int i = threadIdx.x; i < M * nchunk; i += 256) {
+        const int m = i / nchunk, c = i - m * nchunk;
+        xs[i] = reinterpret_cast<const v4i *>(a_i8 + (size_t)m * a_stride)[c];
+    }
+    __syncthreads();
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row0 = (blockIdx.x * 4 + wave) * R;
+    const v4i *wp = reinterpret_cast<const v4i *>(w_t + (size_t)row0 * k_pad);
+    int acc[R][M];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < M; ++m) acc[r][m] = 0;
+
+#pragma unroll 2
+    for (int c = lane; c < nchunk; c += 64) {
+        v4i w[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) w[r] = __builtin_nontemporal_load(wp + (size_t)r * nchunk + c);
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const v4i x = xs[m * nchunk + c];
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r][m] = dot16(w[r], x, acc[r][m]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < M; ++m) acc[r][m] = wave_sum_i32(acc[r][m]);
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int col = row0 + r;
+            if (col < n) {
+                const float ws = w_scales[col];
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    out[(size_t)m * n + col] = (float)acc[r][m] * a_scales[m] * ws;
+                    if (acc_out) acc_out[(size_t)m * n + col] = acc[r][m];
+                }
+            }
+        }
+    }
+}
+
+template <int R, int M>
+pg_status launch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                 const pg_qtensor *w, float *out, int32_t *acc) {
+    const size_t lds = (size_t)M * w->k_pad;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)gemv_w8a8_kernel<R, M>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return pg_fail(PG_EDEVICE, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    }
+    const unsigned grid = (unsigned)(w->n_pad / (4 * R));
+    gemv_w8a8_kernel<R, M><<<grid, 256, lds, ctx->stream>>>(w->w_t, (int)w->k_pad, w->scales, a_i8,
+                                                          (int)a_stride, a_scales, (int)w->cols, out, acc);
+    return pg_launch_check("gemv_w8a8");
+}
+
+template <int M>
+pg_status launch_m(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                   const pg_qtensor *w, float *out, int32_t *acc) {
+    // Aim for >= 8 wavefronts per CU: fewer rows per wavefront when the matrix is narrow.
+    const size_t want_waves = (size_t)ctx->num_cu * 8;
+    if (w->n_pad / 4 >= want_waves) return launch<4, M>(ctx, a_i8, a_stride, a_scales, w, out, acc);
+    if (w->n_pad / 2 >= want_waves) return launch<2, M>(ctx, a_i8, a_stride, a_scales, w, out, acc);
+    return launch<1, M>(ctx, a_i8, a_stride, a_scales, w, out, acc);
+}
+
+}  // namespace
+
+pg_status pg_launch_gemv_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
+                              const float *a_scales, const pg_qtensor *w, size_t m, float *out,
+                              int32_t *acc) {
+    if ((size_t)m * w->k_pad > 150 * 1024)
+        return pg_launch_gemm_w8a8(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
+    switch (m) {
+        case 1: return launch_m<1>(ctx, a_i8, a_stride, a_scales, w, out, acc);
+        case 2: return launch_m<2>(ctx, a_i8, a_stride, a_scales, w, out, acc);
+        case 3: return launch_m<3>(ctx, a_i8, a_stride, a_scales, w, out, acc);
+        case 4: return launch_m<4>(ctx, a_i8, a_stride, a_scales, w, out, acc);
+        default: return pg_launch_gemm_w8a8(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
+    }
+}

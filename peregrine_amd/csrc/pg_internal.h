@@ -1,0 +1,122 @@
+// Internal definitions shared by the HIP translation units of libperegrine_hip.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+#include "peregrine_hip.h"
+
+#define PG_API extern "C" __attribute__((visibility("default")))
+
+// One device + one stream + one growable scratch arena.
+struct pg_ctx {
+    int device;
+    hipStream_t stream;
+    bool owns_stream;
+    void *ws;        // scratch arena (quantised activations, partial results)
+    size_t ws_bytes;
+    int num_cu;
+};
+
+// Device-resident quantised weight, K-contiguous and zero-padded:
+//   w_t    [n_pad, k_pad] i8, w_t[n*k_pad + k] = q[k, n]; padding is 0
+//   scales [n_pad] f32 (padding 1.0)
+struct pg_qtensor {
+    int8_t *w_t;
+    float *scales;
+    size_t rows, cols;    // rows = K, cols = N (the reference's naming)
+    size_t k_pad, n_pad;  // multiples of PG_KPAD / PG_NPAD
+};
+
+// GGUF block tensor split into planes at upload:
+//   qs     [n_out, k_in/32, QB] quant bytes (QB = 16 for Q4_0, 32 for Q8_0)
+//   d      [n_out, k_in/32]     f16 block scales
+struct pg_gguf_tensor {
+    uint8_t *qs;
+    uint16_t *d;
+    int ggml_type;
+    size_t n_out, k_in;
+};
+
+constexpr size_t PG_KPAD = 128;  // device K stride is a multiple of this
+constexpr size_t PG_NPAD = 256;  // device weight rows are padded to this
+
+static inline size_t pg_round_up(size_t v, size_t m) { return (v + m - 1) / m * m; }
+
+// Error plumbing --------------------------------------------------------------
+pg_status pg_fail(pg_status st, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define PG_CHECK_ARG(cond, ...)                                   \
+    do {                                                          \
+        if (!(cond)) return pg_fail(PG_EINVAL, __VA_ARGS__);      \
+    } while (0)
+
+#define PG_HIP(call)                                                              \
+    do {                                                                          \
+        hipError_t e_ = (call);                                                   \
+        if (e_ != hipSuccess)                                                     \
+            return pg_fail(e_ == hipErrorOutOfMemory ? PG_ENOMEM : PG_EDEVICE,    \
+                           "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), \
+                           __FILE__, __LINE__);                                   \
+    } while (0)
+
+#define PG_TRY(call)                    \
+    do {                                \
+        pg_status s_ = (call);          \
+        if (s_ != PG_OK) return s_;     \
+    } while (0)
+
+// Make ctx's device current for the calling thread.
+pg_status pg_use(pg_ctx *ctx);
+// Scratch arena of at least `bytes` (256-byte aligned); contents undefined.
+pg_status pg_workspace(pg_ctx *ctx, size_t bytes, void **out);
+// Check the launch just made.
+pg_status pg_launch_check(const char *what);
+
+// RAII device temporary for the host-pointer entry points.
+struct pg_tmp {
+    void *p = nullptr;
+    ~pg_tmp() { if (p) (void)hipFree(p); }
+    pg_status alloc(size_t bytes) {
+        hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+        if (e != hipSuccess) { p = nullptr; return pg_fail(PG_ENOMEM, "hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e)); }
+        return PG_OK;
+    }
+    template <class T> T *as() const { return static_cast<T *>(p); }
+};
+
+// Kernel launchers implemented per translation unit (device pointers, stream ordered).
+pg_status pg_launch_quantize_activations(pg_ctx *ctx, const float *a, size_t rows, size_t cols,
+                                         int8_t *q, size_t q_stride, float *row_scales);
+pg_status pg_launch_gemm_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
+                              const float *a_scales, const pg_qtensor *w, size_t m,
+                              float *out, int32_t *acc);
+pg_status pg_launch_gemv_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
+                              const float *a_scales, const pg_qtensor *w, size_t m,
+                              float *out, int32_t *acc);
+// Activation rows rewritten as three byte-digit planes (see pg_gguf.hip).
+struct pg_xdigits {
+    int8_t *digits;  // [3][rows][k]
+    float *xs;       // [rows] power-of-two scale
+    int *bsum;       // [3][rows][k/32] per-block digit sums
+    size_t rows, k;
+};
+size_t pg_xdigits_bytes(size_t rows, size_t k);
+pg_xdigits pg_xdigits_carve(void *base, size_t rows, size_t k);
+pg_status pg_launch_x_to_digits(pg_ctx *ctx, const float *x_dev, size_t rows, size_t k,
+                                int ggml_type, const pg_xdigits &xd);
+// A batch of independent M = 1 products: item i uses activation row i / x_row_div and,
+// when a table is given, the weights of expert expert_of[i].
+struct pg_gemv_batch {
+    int count;
+    const uint8_t *const *qs_table;
+    const uint16_t *const *d_table;
+    const int *expert_of;
+    int x_row_div;
+};
+pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in,
+                              const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
+                              const pg_xdigits &xd, float *y);
+// y[m, n_out] = x[m, k_in] . dequant(w)^T on device pointers (uses the scratch arena).
+pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
+                              float *y_dev);

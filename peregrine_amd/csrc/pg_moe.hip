@@ -1,0 +1,173 @@
+// Grouped MoE expert FFN over block-quantised (Q8_0 / Q4_0) experts, entirely
+// stream-ordered on the device (no host round trip for the routing):
+//   1. route: softmax over the E router logits of each token, top-k by stable
+//      descending order (ties -> lower expert index)   examples/grok1/moe.rs:76-89
+//   2. gate / up products of every (token, k) pair against its expert's weights
+//   3. h = act(g) * u                                   grok1/moe.rs:27-34, deepseek/moe.rs:55-59
+//   4. down product of every pair
+//   5. out[t] = 0 + p_0 * y_0 + p_1 * y_1 ... in k order, multiply then add
+//      (examples/grok1/moe.rs:99-104), raw softmax probabilities.
+#include "pg_internal.h"
+
+namespace {
+
+inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
+
+constexpr int MAX_EXPERTS = 256;
+
+// One thread per token.
+__global__ void route_topk_kernel(const float *__restrict__ logits, int T, int E, int top_k,
+                                  int *__restrict__ topk_idx, float *__restrict__ topk_p) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= T) return;
+    const float *x = logits + (size_t)t * E;
+    float mx = -INFINITY;
+    for (int e = 0; e < E; ++e)
+        if (x[e] > mx) mx = x[e];
+    float sum = 0.0f;
+    for (int e = 0; e < E; ++e) sum += expf(x[e] - mx);
+    // k passes of "largest remaining, lowest index on ties" == stable descending sort
+    unsigned taken[MAX_EXPERTS / 32];
+    for (int i = 0; i < MAX_EXPERTS / 32; ++i) taken[i] = 0u;
+    for (int k = 0; k < top_k; ++k) {
+        int best = -1;
+        float bp = 0.0f;
+        for (int e = 0; e < E; ++e) {
+            if (taken[e >> 5] & (1u << (e & 31))) continue;
+            const float p = expf(x[e] - mx) / sum;
+            if (best < 0 || p > bp) { best = e; bp = p; }
+        }
+        taken[best >> 5] |= 1u << (best & 31);
+        topk_idx[(size_t)t * top_k + k] = best;
+        topk_p[(size_t)t * top_k + k] = bp;
+    }
+}
+
+__device__ __forceinline__ float act_silu(float x) {
+    const float sig = 1.0f / (1.0f + expf(-x));
+    return x * sig;
+}
+__device__ __forceinline__ float act_gelu_tanh(float x) {
+    const float c = sqrtf(2.0f / 3.14159265358979323846f);
+    const float inner = c * (x + 0.044715f * x * x * x);
+    return 0.5f * x * (1.0f + tanhf(inner));
+}
+
+__global__ void act_mul_kernel(const float *__restrict__ g, const float *__restrict__ u, size_t n,
+                               int act, float *__restrict__ h) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float a = (act == PG_ACT_GELU_TANH) ? act_gelu_tanh(g[i]) : act_silu(g[i]);
+    h[i] = a * u[i];
+}
+
+__global__ void combine_kernel(const float *__restrict__ yb, const float *__restrict__ topk_p, int T,
+                               int d, int top_k, float *__restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)T * d) return;
+    const size_t t = i / d, c = i - t * d;
+    float acc = 0.0f;
+    for (int k = 0; k < top_k; ++k) {
+        const float prod = topk_p[t * top_k + k] * yb[(t * top_k + k) * d + c];
+        acc = acc + prod;
+    }
+    out[i] = acc;
+}
+
+}  // namespace
+
+PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
+                                const float *router_logits_dev, size_t E, size_t top_k,
+                                const pg_gguf_tensor *const *gate, const pg_gguf_tensor *const *up,
+                                const pg_gguf_tensor *const *down, int act, float *out_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(E >= 1 && E <= MAX_EXPERTS, "pg_moe_ffn: %zu experts (1..%d supported)", E, MAX_EXPERTS);
+    PG_CHECK_ARG(top_k >= 1 && top_k <= E, "pg_moe_ffn: top_k %zu of %zu experts", top_k, E);
+    PG_CHECK_ARG(act == PG_ACT_SILU || act == PG_ACT_GELU_TANH, "pg_moe_ffn: unknown activation %d", act);
+    PG_CHECK_ARG(gate && up && down && gate[0] && up[0] && down[0], "pg_moe_ffn: null expert table");
+    const size_t d = gate[0]->k_in, ffn = gate[0]->n_out;
+    const int type = gate[0]->ggml_type;
+    for (size_t e = 0; e < E; ++e) {
+        PG_CHECK_ARG(gate[e] && up[e] && down[e], "pg_moe_ffn: expert %zu has a null tensor", e);
+        PG_CHECK_ARG(gate[e]->k_in == d && gate[e]->n_out == ffn && up[e]->k_in == d &&
+                         up[e]->n_out == ffn && down[e]->k_in == ffn && down[e]->n_out == d,
+                     "pg_moe_ffn: expert %zu shapes do not match [ffn=%zu, d=%zu]", e, ffn, d);
+        PG_CHECK_ARG(gate[e]->ggml_type == type && up[e]->ggml_type == type && down[e]->ggml_type == type,
+                     "pg_moe_ffn: expert %zu mixes block types", e);
+    }
+    if (T == 0) return PG_OK;
+    PG_CHECK_ARG(x_dev && router_logits_dev && out_dev, "pg_moe_ffn: null pointer");
+    PG_CHECK_ARG((uintptr_t)x_dev % 16 == 0, "pg_moe_ffn: x must be 16-byte aligned");
+    PG_CHECK_ARG(T * top_k < (1ull << 20), "pg_moe_ffn: too many (token, expert) pairs");
+    const size_t P = T * top_k;
+
+    // Arena layout.
+    const size_t sz_tab = pg_round_up(6 * E * sizeof(void *), 256);
+    const size_t sz_idx = pg_round_up(P * sizeof(int), 256);
+    const size_t sz_p = pg_round_up(P * sizeof(float), 256);
+    const size_t sz_act = pg_round_up(P * ffn * sizeof(float), 256);
+    const size_t sz_y = pg_round_up(P * d * sizeof(float), 256);
+    const size_t sz_xd = pg_xdigits_bytes(T, d), sz_hd = pg_xdigits_bytes(P, ffn);
+    void *ws = nullptr;
+    PG_TRY(pg_workspace(ctx, sz_tab + sz_idx + sz_p + 3 * sz_act + sz_y + sz_xd + sz_hd, &ws));
+    char *p = static_cast<char *>(ws);
+    const void **tab = reinterpret_cast<const void **>(p); p += sz_tab;
+    int *topk_idx = reinterpret_cast<int *>(p); p += sz_idx;
+    float *topk_p = reinterpret_cast<float *>(p); p += sz_p;
+    float *g = reinterpret_cast<float *>(p); p += sz_act;
+    float *u = reinterpret_cast<float *>(p); p += sz_act;
+    float *h = reinterpret_cast<float *>(p); p += sz_act;
+    float *yb = reinterpret_cast<float *>(p); p += sz_y;
+    const pg_xdigits xd = pg_xdigits_carve(p, T, d); p += sz_xd;
+    const pg_xdigits hd = pg_xdigits_carve(p, P, ffn);
+
+    // Expert pointer tables: [gate qs | gate d | up qs | up d | down qs | down d], E each.
+    const void *host_tab[6 * MAX_EXPERTS];
+    for (size_t e = 0; e < E; ++e) {
+        host_tab[0 * E + e] = gate[e]->qs; host_tab[1 * E + e] = gate[e]->d;
+        host_tab[2 * E + e] = up[e]->qs;   host_tab[3 * E + e] = up[e]->d;
+        host_tab[4 * E + e] = down[e]->qs; host_tab[5 * E + e] = down[e]->d;
+    }
+    PG_HIP(hipMemcpyAsync(tab, host_tab, 6 * E * sizeof(void *), hipMemcpyHostToDevice, ctx->stream));
+    // host_tab lives on this stack frame: the copy must have left it before we return.
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+
+    route_topk_kernel<<<grid_for(T, 64), 64, 0, ctx->stream>>>(router_logits_dev, (int)T, (int)E, (int)top_k,
+                                                             topk_idx, topk_p);
+    PG_TRY(pg_launch_check("route_topk"));
+    PG_TRY(pg_launch_x_to_digits(ctx, x_dev, T, d, type, xd));
+    auto table = [&](int which) { return reinterpret_cast<const uint8_t *const *>(tab + which * E); };
+    auto dtable = [&](int which) { return reinterpret_cast<const uint16_t *const *>(tab + which * E); };
+    pg_gemv_batch bg = {(int)P, table(0), dtable(1), topk_idx, (int)top_k};
+    PG_TRY(pg_launch_gguf_gemv(ctx, type, ffn, d, nullptr, nullptr, bg, xd, g));
+    pg_gemv_batch bu = {(int)P, table(2), dtable(3), topk_idx, (int)top_k};
+    PG_TRY(pg_launch_gguf_gemv(ctx, type, ffn, d, nullptr, nullptr, bu, xd, u));
+    act_mul_kernel<<<grid_for(P * ffn, 256), 256, 0, ctx->stream>>>(g, u, P * ffn, act, h);
+    PG_TRY(pg_launch_check("act_mul"));
+    PG_TRY(pg_launch_x_to_digits(ctx, h, P, ffn, type, hd));
+    pg_gemv_batch bd = {(int)P, table(4), dtable(5), topk_idx, 1};
+    PG_TRY(pg_launch_gguf_gemv(ctx, type, d, ffn, nullptr, nullptr, bd, hd, yb));
+    combine_kernel<<<grid_for(T * d, 256), 256, 0, ctx->stream>>>(yb, topk_p, (int)T, (int)d, (int)top_k, out_dev);
+    return pg_launch_check("moe_combine");
+}
+
+PG_API pg_status pg_moe_ffn(pg_ctx *ctx, const float *x, size_t T, const float *router_logits,
+                            size_t E, size_t top_k, const pg_gguf_tensor *const *gate,
+                            const pg_gguf_tensor *const *up, const pg_gguf_tensor *const *down,
+                            int act, float *out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(gate && gate[0], "pg_moe_ffn: null expert table");
+    if (T == 0) return PG_OK;
+    PG_CHECK_ARG(x && router_logits && out, "pg_moe_ffn: null pointer");
+    const size_t d = gate[0]->k_in;
+    pg_tmp dx, dl, dout;
+    PG_TRY(dx.alloc(T * d * sizeof(float)));
+    PG_TRY(dl.alloc(T * E * sizeof(float)));
+    PG_TRY(dout.alloc(T * d * sizeof(float)));
+    PG_HIP(hipMemcpyAsync(dx.p, x, T * d * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(dl.p, router_logits, T * E * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_moe_ffn_dev(ctx, dx.as<float>(), T, dl.as<float>(), E, top_k, gate, up, down, act, dout.as<float>()));
+    PG_HIP(hipMemcpyAsync(out, dout.p, T * d * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}

@@ -1,0 +1,475 @@
+// quant::* entry points: weight / activation quantisation, dequantise, device
+// residency of QuantizedTensor, and the W8A8 matmul dispatcher.
+//
+// Bit-exactness notes (all checked against the CPU oracle by the GPU tests):
+//  - rounding is roundf (half away from zero), never rintf;
+//  - weights divide by the scale (IEEE divide), activations multiply by the
+//    reciprocal 1.0f/scale: two different roundings, kept as the reference has them;
+//  - this file is compiled with -ffp-contract=off, f32 denormals stay enabled
+//    and hipcc's default correctly-rounded f32 divide is relied on.
+#include <new>
+#include "pg_internal.h"
+
+namespace {
+
+constexpr int QA_THREADS = 256;
+
+// round -> clamp(-127,127) -> `as i8` (NaN -> 0), returned as int.
+__device__ __forceinline__ int quant_to_i8(float v) {
+    float r = roundf(v);
+    r = fminf(fmaxf(r, -127.0f), 127.0f);
+    return (r != r || v != v) ? 0 : (int)r;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+__device__ __forceinline__ float block_max_256(float v, float *red) {
+    v = wave_max(v);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    v = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    return v;
+}
+
+// One workgroup per row.  The row is read once into registers (up to
+// 4*256*MAXV floats), reduced to its absmax, then rounded to i8 and written as
+// packed dwords.  Columns [cols, q_stride) of the output row are zero-filled.
+template <int MAXV>
+__global__ __launch_bounds__(QA_THREADS) void quantize_rows_vec4_kernel(
+    const float *__restrict__ a, size_t cols, int8_t *__restrict__ q, size_t q_stride,
+    float *__restrict__ row_scales) {
+    __shared__ float red[4];
+    const size_t row = blockIdx.x;
+    const float4 *ar = reinterpret_cast<const float4 *>(a + row * cols);
+    const int nvec = (int)(cols >> 2);
+    float4 v[MAXV];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+        const int idx = threadIdx.x + i * QA_THREADS;
+        if (idx < nvec) {
+            v[i] = ar[idx];
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)),
+                                     fmaxf(fabsf(v[i].z), fabsf(v[i].w))));
+        }
+    }
+    amax = block_max_256(amax, red);
+    const float scale = (amax == 0.0f) ? 1.0f : amax / 127.0f;
+    const float inv_scale = 1.0f / scale;
+    if (threadIdx.x == 0) row_scales[row] = scale;
+    int *qr = reinterpret_cast<int *>(q + row * q_stride);
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+        const int idx = threadIdx.x + i * QA_THREADS;
+        if (idx < nvec) {
+            const int b0 = quant_to_i8(v[i].x * inv_scale) & 0xFF;
+            const int b1 = quant_to_i8(v[i].y * inv_scale) & 0xFF;
+            const int b2 = quant_to_i8(v[i].z * inv_scale) & 0xFF;
+            const int b3 = quant_to_i8(v[i].w * inv_scale) & 0xFF;
+            qr[idx] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+        }
+    }
+    const int npad = (int)(q_stride >> 2);
+    for (int idx = nvec + threadIdx.x; idx < npad; idx += QA_THREADS) qr[idx] = 0;
+}
+
+// Any shape: two passes over the row (the second one hits L2), scalar accesses.
+__global__ __launch_bounds__(QA_THREADS) void quantize_rows_generic_kernel(
+    const float *__restrict__ a, size_t cols, int8_t *__restrict__ q, size_t q_stride,
+    float *__restrict__ row_scales) {
+    __shared__ float red[4];
+    const size_t row = blockIdx.x;
+    const float *ar = a + row * cols;
+    float amax = 0.0f;
+    for (size_t k = threadIdx.x; k < cols; k += QA_THREADS) amax = fmaxf(amax, fabsf(ar[k]));
+    amax = block_max_256(amax, red);
+    const float scale = (amax == 0.0f) ? 1.0f : amax / 127.0f;
+    const float inv_scale = 1.0f / scale;
+    if (threadIdx.x == 0) row_scales[row] = scale;
+    int8_t *qr = q + row * q_stride;
+    for (size_t k = threadIdx.x; k < cols; k += QA_THREADS)
+        qr[k] = (int8_t)quant_to_i8(ar[k] * inv_scale);
+    for (size_t k = cols + threadIdx.x; k < q_stride; k += QA_THREADS) qr[k] = 0;
+}
+
+// ---- weight quantisation -----------------------------------------------------
+
+__global__ void fill_u32_kernel(uint32_t *p, size_t n, uint32_t v) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// Per-column absmax with the reference's strict `>` (NaN never wins).  One
+// thread per column, rows split over blockIdx.y; partial maxima are merged with
+// an unsigned atomicMax on the bit pattern (order-independent for values >= 0).
+constexpr int CM_ROWS_PER_BLOCK = 128;
+__global__ __launch_bounds__(256) void col_absmax_kernel(const float *__restrict__ w, size_t rows,
+                                                         size_t cols,
+                                                         uint32_t *__restrict__ amax_bits) {
+    const size_t n = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (n >= cols) return;
+    const size_t r0 = (size_t)blockIdx.y * CM_ROWS_PER_BLOCK;
+    const size_t r1 = r0 + CM_ROWS_PER_BLOCK < rows ? r0 + CM_ROWS_PER_BLOCK : rows;
+    float cur = 0.0f;
+    for (size_t r = r0; r < r1; ++r) {
+        const float v = fabsf(w[r * cols + n]);
+        if (v > cur) cur = v;
+    }
+    if (cur > 0.0f) atomicMax(amax_bits + n, __float_as_uint(cur));
+}
+
+__global__ void scales_from_amax_kernel(const uint32_t *__restrict__ amax_bits, size_t cols,
+                                        size_t cols_pad, float *__restrict__ scales) {
+    const size_t n = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= cols_pad) return;
+    float s = 1.0f;
+    if (n < cols) {
+        const float amax = __uint_as_float(amax_bits[n]);
+        s = (amax == 0.0f) ? 1.0f : amax / 127.0f;
+    }
+    scales[n] = s;
+}
+
+// 64x64 tile: q[k, n] = round(w[k, n] / scale[n]); optional dense q [rows, cols]
+// and the K-contiguous transpose q_t[n * t_stride + k], staged through LDS so
+// both global writes are row-contiguous.
+__global__ __launch_bounds__(256) void quantize_weights_tile_kernel(
+    const float *__restrict__ w, size_t rows, size_t cols, const float *__restrict__ scales,
+    int8_t *__restrict__ q, int8_t *__restrict__ q_t, size_t t_stride) {
+    __shared__ int8_t tile[64][65];
+    const size_t k0 = (size_t)blockIdx.y * 64, n0 = (size_t)blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // ty in 0..3
+    const size_t n = n0 + tx;
+    const float scale = (n < cols) ? scales[n] : 1.0f;
+    for (int r = ty; r < 64; r += 4) {
+        const size_t k = k0 + r;
+        int8_t v = 0;
+        if (k < rows && n < cols) {
+            v = (int8_t)quant_to_i8(w[k * cols + n] / scale);
+            if (q) q[k * cols + n] = v;
+        }
+        tile[r][tx] = v;
+    }
+    __syncthreads();
+    if (q_t) {
+        for (int c = ty; c < 64; c += 4) {
+            const size_t nn = n0 + c, kk = k0 + tx;
+            if (nn < cols && kk < rows) q_t[nn * t_stride + kk] = tile[tx][c];
+        }
+    }
+}
+
+// dst[c * dst_stride + r] = src[r * src_stride + c] for r < rows, c < cols.
+__global__ __launch_bounds__(256) void transpose_i8_kernel(const int8_t *__restrict__ src,
+                                                           size_t rows, size_t cols,
+                                                           size_t src_stride,
+                                                           int8_t *__restrict__ dst,
+                                                           size_t dst_stride) {
+    __shared__ int8_t tile[64][65];
+    const size_t r0 = (size_t)blockIdx.y * 64, c0 = (size_t)blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < 64; r += 4)
+        tile[r][tx] = (r0 + r < rows && c0 + tx < cols) ? src[(r0 + r) * src_stride + c0 + tx] : 0;
+    __syncthreads();
+    for (int c = ty; c < 64; c += 4)
+        if (c0 + c < cols && r0 + tx < rows) dst[(c0 + c) * dst_stride + r0 + tx] = tile[tx][c];
+}
+
+__global__ void dequantize_kernel(const int8_t *__restrict__ q, const float *__restrict__ scales,
+                                  size_t rows, size_t cols, float *__restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * cols) return;
+    out[i] = (float)q[i] * scales[i % cols];
+}
+
+inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
+
+// amax -> scales, quantise, write q (optional) and q_t with the given stride.
+pg_status quantize_weights_on_device(pg_ctx *ctx, const float *w_dev, size_t rows, size_t cols,
+                                     int8_t *q_dev, int8_t *q_t_dev, size_t t_stride,
+                                     float *scales_dev, size_t cols_pad) {
+    pg_tmp amax;
+    PG_TRY(amax.alloc(cols * sizeof(uint32_t)));
+    fill_u32_kernel<<<grid_for(cols, 256), 256, 0, ctx->stream>>>(amax.as<uint32_t>(), cols, 0u);
+    PG_TRY(pg_launch_check("fill_u32"));
+    dim3 g1(grid_for(cols, 256), grid_for(rows, CM_ROWS_PER_BLOCK));
+    col_absmax_kernel<<<g1, 256, 0, ctx->stream>>>(w_dev, rows, cols, amax.as<uint32_t>());
+    PG_TRY(pg_launch_check("col_absmax"));
+    scales_from_amax_kernel<<<grid_for(cols_pad, 256), 256, 0, ctx->stream>>>(
+        amax.as<uint32_t>(), cols, cols_pad, scales_dev);
+    PG_TRY(pg_launch_check("scales_from_amax"));
+    dim3 g2(grid_for(cols, 64), grid_for(rows, 64));
+    quantize_weights_tile_kernel<<<g2, 256, 0, ctx->stream>>>(w_dev, rows, cols, scales_dev, q_dev,
+                                                              q_t_dev, t_stride);
+    PG_TRY(pg_launch_check("quantize_weights_tile"));
+    PG_HIP(hipStreamSynchronize(ctx->stream));  // amax is freed on return
+    return PG_OK;
+}
+
+pg_status qtensor_alloc(pg_ctx *ctx, size_t rows, size_t cols, pg_qtensor **out) {
+    pg_qtensor *t = new (std::nothrow) pg_qtensor();
+    if (!t) return pg_fail(PG_ENOMEM, "host allocation failed");
+    t->rows = rows;
+    t->cols = cols;
+    t->k_pad = pg_round_up(rows, PG_KPAD);
+    t->n_pad = pg_round_up(cols, PG_NPAD);
+    t->w_t = nullptr;
+    t->scales = nullptr;
+    const size_t bytes = t->k_pad * t->n_pad;
+    hipError_t e = hipMalloc((void **)&t->w_t, bytes);
+    if (e == hipSuccess) e = hipMalloc((void **)&t->scales, t->n_pad * sizeof(float));
+    if (e == hipSuccess) e = hipMemsetAsync(t->w_t, 0, bytes, ctx->stream);
+    if (e != hipSuccess) {
+        if (t->w_t) (void)hipFree(t->w_t);
+        if (t->scales) (void)hipFree(t->scales);
+        delete t;
+        return pg_fail(e == hipErrorOutOfMemory ? PG_ENOMEM : PG_EDEVICE,
+                       "allocating a %zu x %zu quantised tensor failed: %s", rows, cols,
+                       hipGetErrorString(e));
+    }
+    *out = t;
+    return PG_OK;
+}
+
+}  // namespace
+
+pg_status pg_launch_quantize_activations(pg_ctx *ctx, const float *a, size_t rows, size_t cols,
+                                         int8_t *q, size_t q_stride, float *row_scales) {
+    if (rows == 0) return PG_OK;
+    const bool vec_ok = (cols % 4 == 0) && (q_stride % 4 == 0) &&
+                        ((uintptr_t)a % 16 == 0) && ((uintptr_t)q % 4 == 0) && cols > 0;
+    const size_t nvec = cols / 4;
+    const dim3 grid((unsigned)rows);
+    if (vec_ok && nvec <= 4 * QA_THREADS)
+        quantize_rows_vec4_kernel<4><<<grid, QA_THREADS, 0, ctx->stream>>>(a, cols, q, q_stride, row_scales);
+    else if (vec_ok && nvec <= 16 * QA_THREADS)
+        quantize_rows_vec4_kernel<16><<<grid, QA_THREADS, 0, ctx->stream>>>(a, cols, q, q_stride, row_scales);
+    else
+        quantize_rows_generic_kernel<<<grid, QA_THREADS, 0, ctx->stream>>>(a, cols, q, q_stride, row_scales);
+    return pg_launch_check("quantize_rows");
+}
+
+PG_API pg_status pg_quantize_activations_dev(pg_ctx *ctx, const float *a_dev, size_t rows,
+                                             size_t cols, int8_t *q_dev, float *row_scales_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(rows == 0 || (a_dev && q_dev && row_scales_dev) || cols == 0,
+                 "pg_quantize_activations_dev: null pointer");
+    PG_CHECK_ARG(rows == 0 || (row_scales_dev != nullptr), "pg_quantize_activations_dev: null scales");
+    PG_CHECK_ARG(rows < (1ull << 31), "pg_quantize_activations_dev: too many rows");
+    return pg_launch_quantize_activations(ctx, a_dev, rows, cols, q_dev, cols, row_scales_dev);
+}
+
+PG_API pg_status pg_quantize_activations(pg_ctx *ctx, const float *a, size_t rows, size_t cols,
+                                         int8_t *q, float *row_scales) {
+    PG_TRY(pg_use(ctx));
+    if (rows == 0) return PG_OK;
+    PG_CHECK_ARG(row_scales && (cols == 0 || (a && q)), "pg_quantize_activations: null pointer");
+    PG_CHECK_ARG(rows < (1ull << 31), "pg_quantize_activations: too many rows");
+    const size_t n = rows * cols;
+    pg_tmp da, dq, ds;
+    PG_TRY(da.alloc(n * sizeof(float)));
+    PG_TRY(dq.alloc(n));
+    PG_TRY(ds.alloc(rows * sizeof(float)));
+    if (n) PG_HIP(hipMemcpyAsync(da.p, a, n * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_launch_quantize_activations(ctx, da.as<float>(), rows, cols, dq.as<int8_t>(), cols,
+                                          ds.as<float>()));
+    if (n) PG_HIP(hipMemcpyAsync(q, dq.p, n, hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipMemcpyAsync(row_scales, ds.p, rows * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+PG_API pg_status pg_quantize_weights(pg_ctx *ctx, const float *w, size_t rows, size_t cols,
+                                     int8_t *q, int8_t *q_t, float *scales) {
+    PG_TRY(pg_use(ctx));
+    const size_t n = rows * cols;
+    if (cols == 0) return PG_OK;
+    PG_CHECK_ARG(scales != nullptr, "pg_quantize_weights: scales is null");
+    PG_CHECK_ARG(n == 0 || (w && q), "pg_quantize_weights: null pointer");
+    pg_tmp dw, dq, dqt, ds;
+    PG_TRY(dw.alloc(n * sizeof(float)));
+    PG_TRY(dq.alloc(n));
+    if (q_t) PG_TRY(dqt.alloc(n));
+    PG_TRY(ds.alloc(cols * sizeof(float)));
+    if (n) PG_HIP(hipMemcpyAsync(dw.p, w, n * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(quantize_weights_on_device(ctx, dw.as<float>(), rows, cols, dq.as<int8_t>(),
+                                      q_t ? dqt.as<int8_t>() : nullptr, rows, ds.as<float>(), cols));
+    if (n) PG_HIP(hipMemcpyAsync(q, dq.p, n, hipMemcpyDeviceToHost, ctx->stream));
+    if (n && q_t) PG_HIP(hipMemcpyAsync(q_t, dqt.p, n, hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipMemcpyAsync(scales, ds.p, cols * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+PG_API pg_status pg_dequantize(pg_ctx *ctx, const int8_t *q, const float *scales, size_t rows,
+                               size_t cols, float *out) {
+    PG_TRY(pg_use(ctx));
+    const size_t n = rows * cols;
+    if (n == 0) return PG_OK;
+    PG_CHECK_ARG(q && scales && out, "pg_dequantize: null pointer");
+    pg_tmp dq, ds, dout;
+    PG_TRY(dq.alloc(n));
+    PG_TRY(ds.alloc(cols * sizeof(float)));
+    PG_TRY(dout.alloc(n * sizeof(float)));
+    PG_HIP(hipMemcpyAsync(dq.p, q, n, hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(ds.p, scales, cols * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    dequantize_kernel<<<grid_for(n, 256), 256, 0, ctx->stream>>>(dq.as<int8_t>(), ds.as<float>(), rows,
+                                                               cols, dout.as<float>());
+    PG_TRY(pg_launch_check("dequantize"));
+    PG_HIP(hipMemcpyAsync(out, dout.p, n * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+PG_API pg_status pg_qtensor_upload(pg_ctx *ctx, const int8_t *q, const float *scales, size_t rows,
+                                   size_t cols, pg_qtensor **out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(out != nullptr, "pg_qtensor_upload: out is null");
+    *out = nullptr;
+    PG_CHECK_ARG(rows > 0 && cols > 0, "pg_qtensor_upload: empty tensor %zu x %zu", rows, cols);
+    PG_CHECK_ARG(q && scales, "pg_qtensor_upload: null pointer");
+    PG_CHECK_ARG(rows < (1ull << 31) && cols < (1ull << 31), "pg_qtensor_upload: shape too large");
+    pg_qtensor *t = nullptr;
+    PG_TRY(qtensor_alloc(ctx, rows, cols, &t));
+    pg_tmp dq;
+    pg_status st = dq.alloc(rows * cols);
+    if (st == PG_OK) {
+        hipError_t e = hipMemcpyAsync(dq.p, q, rows * cols, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) {
+            fill_u32_kernel<<<grid_for(t->n_pad, 256), 256, 0, ctx->stream>>>(
+                reinterpret_cast<uint32_t *>(t->scales), t->n_pad, 0x3F800000u);
+            e = hipMemcpyAsync(t->scales, scales, cols * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
+        }
+        if (e == hipSuccess) {
+            dim3 g(grid_for(cols, 64), grid_for(rows, 64));
+            transpose_i8_kernel<<<g, 256, 0, ctx->stream>>>(dq.as<int8_t>(), rows, cols, cols, t->w_t, t->k_pad);
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) st = pg_fail(PG_EDEVICE, "pg_qtensor_upload: %s", hipGetErrorString(e));
+    }
+    if (st != PG_OK) { pg_qtensor_free(ctx, t); return st; }
+    *out = t;
+    return PG_OK;
+}
+
+PG_API pg_status pg_qtensor_from_f32_dev(pg_ctx *ctx, const float *w_dev, size_t rows, size_t cols,
+                                         pg_qtensor **out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(out != nullptr, "pg_qtensor_from_f32: out is null");
+    *out = nullptr;
+    PG_CHECK_ARG(rows > 0 && cols > 0, "pg_qtensor_from_f32: empty tensor %zu x %zu", rows, cols);
+    PG_CHECK_ARG(w_dev != nullptr, "pg_qtensor_from_f32: null pointer");
+    PG_CHECK_ARG(rows < (1ull << 31) && cols < (1ull << 31), "pg_qtensor_from_f32: shape too large");
+    pg_qtensor *t = nullptr;
+    PG_TRY(qtensor_alloc(ctx, rows, cols, &t));
+    pg_status st = quantize_weights_on_device(ctx, w_dev, rows, cols, nullptr, t->w_t, t->k_pad,
+                                              t->scales, t->n_pad);
+    if (st != PG_OK) { pg_qtensor_free(ctx, t); return st; }
+    *out = t;
+    return PG_OK;
+}
+
+PG_API pg_status pg_qtensor_from_f32(pg_ctx *ctx, const float *w, size_t rows, size_t cols,
+                                     pg_qtensor **out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(out != nullptr, "pg_qtensor_from_f32: out is null");
+    *out = nullptr;
+    PG_CHECK_ARG(rows > 0 && cols > 0 && w, "pg_qtensor_from_f32: empty tensor or null pointer");
+    pg_tmp dw;
+    PG_TRY(dw.alloc(rows * cols * sizeof(float)));
+    PG_HIP(hipMemcpyAsync(dw.p, w, rows * cols * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    return pg_qtensor_from_f32_dev(ctx, dw.as<float>(), rows, cols, out);
+}
+
+PG_API pg_status pg_qtensor_download(pg_ctx *ctx, const pg_qtensor *t, int8_t *q, int8_t *q_t,
+                                     float *scales) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(t != nullptr, "pg_qtensor_download: null tensor");
+    const size_t rows = t->rows, cols = t->cols;
+    if (q) {
+        pg_tmp dq;
+        PG_TRY(dq.alloc(rows * cols));
+        dim3 g(grid_for(rows, 64), grid_for(cols, 64));
+        // w_t is [cols, rows] with stride k_pad; transpose back to [rows, cols].
+        transpose_i8_kernel<<<g, 256, 0, ctx->stream>>>(t->w_t, cols, rows, t->k_pad, dq.as<int8_t>(), cols);
+        PG_TRY(pg_launch_check("transpose_i8"));
+        PG_HIP(hipMemcpyAsync(q, dq.p, rows * cols, hipMemcpyDeviceToHost, ctx->stream));
+        PG_HIP(hipStreamSynchronize(ctx->stream));
+    }
+    if (q_t)
+        PG_HIP(hipMemcpy2DAsync(q_t, rows, t->w_t, t->k_pad, rows, cols, hipMemcpyDeviceToHost, ctx->stream));
+    if (scales)
+        PG_HIP(hipMemcpyAsync(scales, t->scales, cols * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+PG_API pg_status pg_qtensor_shape(const pg_qtensor *t, size_t *rows, size_t *cols) {
+    PG_CHECK_ARG(t != nullptr, "pg_qtensor_shape: null tensor");
+    if (rows) *rows = t->rows;
+    if (cols) *cols = t->cols;
+    return PG_OK;
+}
+
+PG_API void pg_qtensor_free(pg_ctx *ctx, pg_qtensor *t) {
+    if (!t) return;
+    if (ctx) {
+        (void)hipSetDevice(ctx->device);
+        (void)hipStreamSynchronize(ctx->stream);
+    }
+    if (t->w_t) (void)hipFree(t->w_t);
+    if (t->scales) (void)hipFree(t->scales);
+    delete t;
+}
+
+// ---- the W8A8 matmul -----------------------------------------------------------
+
+// Rows of the quantised-activation scratch are padded to this many so the GEMM
+// tiles never read past the arena.
+constexpr size_t PG_MPAD = 256;
+// At or below this many activation rows the weight stream, not the matrix cores,
+// bounds the product: use the dot-product GEMV kernel.
+constexpr size_t PG_GEMV_MAX_M = 4;
+
+PG_API pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
+                                         const pg_qtensor *w, float *out_dev, int32_t *acc_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(w != nullptr, "pg_matmul_quantized: null weights");
+    PG_CHECK_ARG(w->rows == k, "pg_matmul_quantized: a has k = %zu but w has %zu rows", k, w->rows);
+    if (m == 0) return PG_OK;
+    PG_CHECK_ARG(a_dev && out_dev, "pg_matmul_quantized: null pointer");
+    PG_CHECK_ARG(m < (1ull << 24), "pg_matmul_quantized: m = %zu too large", m);
+    const size_t m_pad = pg_round_up(m, PG_MPAD);
+    const size_t a_bytes = m_pad * w->k_pad;
+    void *ws = nullptr;
+    PG_TRY(pg_workspace(ctx, a_bytes + m_pad * sizeof(float), &ws));
+    int8_t *a_i8 = static_cast<int8_t *>(ws);
+    float *a_scales = reinterpret_cast<float *>(a_i8 + a_bytes);
+    PG_TRY(pg_launch_quantize_activations(ctx, a_dev, m, k, a_i8, w->k_pad, a_scales));
+    if (m <= PG_GEMV_MAX_M)
+        return pg_launch_gemv_w8a8(ctx, a_i8, w->k_pad, a_scales, w, m, out_dev, acc_dev);
+    return pg_launch_gemm_w8a8(ctx, a_i8, w->k_pad, a_scales, w, m, out_dev, acc_dev);
+}
+
+PG_API pg_status pg_matmul_quantized(pg_ctx *ctx, const float *a, size_t m, size_t k,
+                                     const pg_qtensor *w, float *out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(w != nullptr, "pg_matmul_quantized: null weights");
+    PG_CHECK_ARG(w->rows == k, "pg_matmul_quantized: a has k = %zu but w has %zu rows", k, w->rows);
+    if (m == 0) return PG_OK;
+    PG_CHECK_ARG(a && out, "pg_matmul_quantized: null pointer");
+    pg_tmp da, dout;
+    PG_TRY(da.alloc(m * k * sizeof(float)));
+    PG_TRY(dout.alloc(m * w->cols * sizeof(float)));
+    PG_HIP(hipMemcpyAsync(da.p, a, m * k * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_matmul_quantized_dev(ctx, da.as<float>(), m, k, w, dout.as<float>(), nullptr));
+    PG_HIP(hipMemcpyAsync(out, dout.p, m * w->cols * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}

@@ -1,0 +1,44 @@
+"""Host-side mirror of the MoE expert FFN (reference: examples/grok1/moe.rs:27-109,
+expert body with SiLU: examples/deepseek/moe.rs:55-59) over block-quantised experts."""
+import ctypes as C
+
+import numpy as np
+
+from . import _ffi
+from .context import default_context
+from .quant import _ptr
+
+SILU, GELU_TANH = _ffi.ACT_SILU, _ffi.ACT_GELU_TANH
+
+
+class MoEExperts:
+    """E experts, each (gate [ffn, d], up [ffn, d], down [d, ffn]) as GgufWeight."""
+
+    def __init__(self, gate, up, down, top_k, act=SILU, ctx=None):
+        if not (len(gate) == len(up) == len(down)) or not gate:
+            raise ValueError("MoEExperts: gate/up/down must be equally long, non-empty lists")
+        self.ctx = ctx or default_context()
+        self.gate, self.up, self.down = list(gate), list(up), list(down)
+        self.top_k, self.act = int(top_k), int(act)
+        self.d, self.ffn = gate[0].k_in, gate[0].n_out
+
+    def _table(self, ws):
+        arr = (C.c_void_p * len(ws))(*[w._h for w in ws])
+        return C.cast(arr, C.POINTER(C.c_void_p)), arr
+
+    def forward(self, x, router_logits):
+        """MoELayer::forward after `logits = x.matmul(&router)` (examples/grok1/moe.rs:76-109):
+        x [T, d], router_logits [T, E] -> out [T, d]."""
+        E = len(self.gate)
+        x = np.ascontiguousarray(x, np.float32).reshape(-1)
+        T = x.size // self.d
+        if x.size != T * self.d:
+            raise ValueError("MoEExperts.forward: x is not [T, d]")
+        logits = np.ascontiguousarray(router_logits, np.float32).reshape(-1)
+        if logits.size != T * E:
+            raise ValueError("MoEExperts.forward: router_logits is not [T, E]")
+        out = np.empty(T * self.d, np.float32)
+        (g, _g), (u, _u), (dn, _d) = self._table(self.gate), self._table(self.up), self._table(self.down)
+        _ffi.check(_ffi.lib.pg_moe_ffn(self.ctx.handle, _ptr(x), T, _ptr(logits), E, self.top_k,
+                                       g, u, dn, self.act, _ptr(out)))
+        return out.reshape(T, self.d)

@@ -1,0 +1,152 @@
+"""ctypes/NumPy front end of the CPU oracle (oracle/peregrine_oracle.c).  Test infrastructure:
+only tests, the smoke check and the benchmark's cpu_baseline leg import this."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SO = os.path.join(ROOT, "oracle", "_build", "libperegrine_oracle.so")
+
+
+def _load():
+    if not os.path.exists(SO):
+        subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle")], stdout=subprocess.DEVNULL)
+    return C.CDLL(SO)
+
+
+lib = _load()
+_vp, _sz = C.c_void_p, C.c_size_t
+lib.orc_f16_to_f32_bits.restype = C.c_uint32
+lib.orc_f16_to_f32_bits.argtypes = [C.c_uint16]
+lib.orc_rng_next_u64.restype = C.c_uint64
+lib.orc_rng_next_u64.argtypes = [_vp]
+lib.orc_rng_seed.argtypes = [_vp, C.c_uint64]
+lib.orc_rng_normal.argtypes = [C.c_uint64, _sz, C.c_float, C.c_float, _vp]
+for _n in ("orc_quantize_weights", "orc_quantize_activations", "orc_dequantize", "orc_gemm_i8",
+           "orc_matmul_f32", "orc_softmax_rows", "orc_silu", "orc_gelu_tanh", "orc_swiglu_llama"):
+    getattr(lib, _n).restype = None
+
+
+def _p(a):
+    return C.c_void_p(a.ctypes.data) if a is not None else C.c_void_p(None)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, np.float32)
+
+
+def quantize_weights(w, rows, cols):
+    w = _f32(w).reshape(-1)
+    q = np.empty(rows * cols, np.int8)
+    qt = np.empty(rows * cols, np.int8)
+    s = np.empty(cols, np.float32)
+    lib.orc_quantize_weights(_p(w), _sz(rows), _sz(cols), _p(q), _p(qt), _p(s))
+    return q, qt, s
+
+
+def quantize_activations(a, rows, cols):
+    a = _f32(a).reshape(-1)
+    q = np.empty(rows * cols, np.int8)
+    s = np.empty(rows, np.float32)
+    lib.orc_quantize_activations(_p(a), _sz(rows), _sz(cols), _p(q), _p(s))
+    return q, s
+
+
+def dequantize(q, scales, rows, cols):
+    out = np.empty(rows * cols, np.float32)
+    lib.orc_dequantize(_p(np.ascontiguousarray(q, np.int8)), _p(_f32(scales)), _sz(rows), _sz(cols), _p(out))
+    return out
+
+
+def gemm_i8(a_i8, a_scales, b_t, w_scales, m, n, k):
+    out = np.empty(m * n, np.float32)
+    acc = np.empty(m * n, np.int32)
+    lib.orc_gemm_i8(_p(np.ascontiguousarray(a_i8, np.int8)), _p(_f32(a_scales)),
+                    _p(np.ascontiguousarray(b_t, np.int8)), _p(_f32(w_scales)),
+                    _sz(m), _sz(n), _sz(k), _p(out), _p(acc))
+    return out, acc
+
+
+def matmul_quantized(a, m, k, q_t, w_scales, n):
+    a = _f32(a).reshape(-1)
+    out = np.empty(m * n, np.float32)
+    acc = np.empty(m * n, np.int32)
+    rc = lib.orc_matmul_quantized(_p(a), _sz(m), _sz(k), _p(np.ascontiguousarray(q_t, np.int8)),
+                                  _p(_f32(w_scales)), _sz(n), _p(out), _p(acc))
+    assert rc == 0
+    return out, acc
+
+
+def f16_to_f32_bits(bits):
+    return np.array([lib.orc_f16_to_f32_bits(int(b)) for b in np.asarray(bits).reshape(-1)], np.uint32)
+
+
+def _dequant(fn, data, n):
+    buf = np.frombuffer(bytes(data), np.uint8).copy()
+    out = np.empty(n, np.float32)
+    rc = fn(_p(buf), _sz(n), _p(out))
+    if rc != 0:
+        raise ValueError("num_elements must be a multiple of 32")
+    return out
+
+
+def dequant_q8_0(data, n):
+    return _dequant(lib.orc_dequant_q8_0, data, n)
+
+
+def dequant_q4_0(data, n):
+    return _dequant(lib.orc_dequant_q4_0, data, n)
+
+
+def dequant_q4_1(data, n):
+    return _dequant(lib.orc_dequant_q4_1, data, n)
+
+
+def matmul_f32(a, b, m, k, n):
+    out = np.empty(m * n, np.float32)
+    lib.orc_matmul_f32(_p(_f32(a).reshape(-1)), _p(_f32(b).reshape(-1)), _sz(m), _sz(k), _sz(n), _p(out))
+    return out
+
+
+def gguf_matmul(x, m, blocks, ggml_type, n_out, k_in):
+    buf = np.frombuffer(bytes(blocks), np.uint8).copy()
+    y = np.empty(m * n_out, np.float32)
+    rc = lib.orc_gguf_matmul(_p(_f32(x).reshape(-1)), _sz(m), _p(buf), C.c_int(ggml_type), _sz(n_out), _sz(k_in), _p(y))
+    assert rc == 0, rc
+    return y
+
+
+def softmax_rows(x, rows, cols):
+    out = np.empty(rows * cols, np.float32)
+    lib.orc_softmax_rows(_p(_f32(x).reshape(-1)), _sz(rows), _sz(cols), _p(out))
+    return out
+
+
+def unary(name, x):
+    x = _f32(x).reshape(-1)
+    out = np.empty_like(x)
+    getattr(lib, name)(_p(x), _sz(x.size), _p(out))
+    return out
+
+
+def moe_ffn(x, T, d, ffn, E, top_k, logits, gate, up, down, ggml_type, act):
+    """gate/up/down: lists of E raw block byte strings."""
+    keep = [np.frombuffer(bytes(b), np.uint8).copy() for b in list(gate) + list(up) + list(down)]
+    mk = lambda arrs: (C.c_void_p * E)(*[a.ctypes.data for a in arrs])
+    g, u, dn = mk(keep[:E]), mk(keep[E:2 * E]), mk(keep[2 * E:])
+    out = np.empty(T * d, np.float32)
+    idx = np.empty(T * top_k, np.int32)
+    prob = np.empty(T * top_k, np.float32)
+    rc = lib.orc_moe_ffn(_p(_f32(x).reshape(-1)), _sz(T), _sz(d), _sz(ffn), _sz(E), _sz(top_k),
+                         _p(_f32(logits).reshape(-1)), g, u, dn, C.c_int(ggml_type), C.c_int(act),
+                         _p(out), _p(idx), _p(prob))
+    assert rc == 0, rc
+    return out.reshape(T, d), idx.reshape(T, top_k), prob.reshape(T, top_k)
+
+
+def rng_normal(seed, n, mean=0.0, std=1.0):
+    out = np.empty(n, np.float32)
+    lib.orc_rng_normal(C.c_uint64(seed), _sz(n), C.c_float(mean), C.c_float(std), _p(out))
+    return out

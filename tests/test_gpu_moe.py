@@ -1,0 +1,84 @@
+"""GPU parity of the grouped MoE expert FFN against the CPU oracle, through the C ABI.
+
+Bar: routing (expert indices, order, tie-breaks) identical; outputs within 1e-3 relative
+(block-dequant path; H.assert_close_rel), asserted at 1e-4 (GPU expf/tanhf differ from
+glibc's in the last ulp, which is all that separates the two)."""
+import sys
+
+import numpy as np
+import pytest
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def build(orc, seed, d, ffn, E, typ):
+    pack = H.pack_q4_0 if typ == 2 else H.pack_q8_0
+    raws = []
+    for i, (n_out, k_in) in enumerate(((ffn, d), (ffn, d), (d, ffn))):
+        raws.append([pack(orc.rng_normal(seed + 100 * i + e, n_out * k_in, 0.0, 0.05)) for e in range(E)])
+    return raws
+
+
+@pytest.mark.parametrize("typ", [8, 2])
+@pytest.mark.parametrize("act", [0, 1])
+def test_moe_small_vs_oracle(ctx, orc, typ, act):
+    from peregrine_amd import gguf, moe
+    T, d, ffn, E, top_k = 6, 64, 96, 4, 2
+    say(f"moe small typ={typ} act={act}")
+    raws = build(orc, 50, d, ffn, E, typ)
+    x = orc.rng_normal(1, T * d)
+    logits = orc.rng_normal(2, T * E).reshape(T, E)
+    logits[0] = 0.5                    # full tie -> experts 0, 1
+    logits[1] = [0.1, 0.9, 0.9, 0.2]   # tie for first -> 1 then 2
+    mk = lambda rs, n_out, k_in: [gguf.GgufWeight(r, typ, n_out, k_in, ctx) for r in rs]
+    ex = moe.MoEExperts(mk(raws[0], ffn, d), mk(raws[1], ffn, d), mk(raws[2], d, ffn), top_k, act, ctx)
+    got = ex.forward(x, logits)
+    want, idx, prob = orc.moe_ffn(x, T, d, ffn, E, top_k, logits, raws[0], raws[1], raws[2], typ, act)
+    assert list(idx[0]) == [0, 1] and list(idx[1]) == [1, 2]
+    for t in range(T):
+        H.assert_close_rel(got[t], want[t], 1e-4, f"token {t}")
+
+
+def test_moe_grok_shaped_reduced(ctx, orc):
+    """BASELINE config 5's structure (8 experts, top-2, 64 tokens, Q8_0, SiLU) at reduced
+    width (d 512, ffn 1024) so the oracle finishes in seconds."""
+    from peregrine_amd import gguf, moe
+    T, d, ffn, E, top_k = 64, 512, 1024, 8, 2
+    say("moe grok-shaped reduced")
+    raws = build(orc, 70, d, ffn, E, 8)
+    x = orc.rng_normal(3, T * d)
+    logits = orc.rng_normal(4, T * E).reshape(T, E)
+    mk = lambda rs, n_out, k_in: [gguf.GgufWeight(r, 8, n_out, k_in, ctx) for r in rs]
+    ex = moe.MoEExperts(mk(raws[0], ffn, d), mk(raws[1], ffn, d), mk(raws[2], d, ffn), top_k, moe.SILU, ctx)
+    got = ex.forward(x, logits)
+    want, idx, prob = orc.moe_ffn(x, T, d, ffn, E, top_k, logits, raws[0], raws[1], raws[2], 8, 0)
+    for t in range(T):
+        H.assert_close_rel(got[t], want[t], 1e-4, f"token {t}")
+    # top_k = E with one expert: the layer reduces to p * expert(x) with p = 1
+    ex1 = moe.MoEExperts(ex.gate[:1], ex.up[:1], ex.down[:1], 1, moe.SILU, ctx)
+    got1 = ex1.forward(x[: 2 * d], np.zeros((2, 1), np.float32))
+    want1, _, p1 = orc.moe_ffn(x[: 2 * d], 2, d, ffn, 1, 1, np.zeros((2, 1), np.float32),
+                               raws[0][:1], raws[1][:1], raws[2][:1], 8, 0)
+    assert (p1 == 1.0).all()
+    H.assert_close_rel(got1, want1, 1e-4, "single expert")
+
+
+def test_moe_argument_errors(ctx, orc):
+    from peregrine_amd import gguf, moe, _ffi
+    d, ffn = 64, 96
+    raws = build(orc, 90, d, ffn, 2, 8)
+    mk = lambda rs, n_out, k_in: [gguf.GgufWeight(r, 8, n_out, k_in, ctx) for r in rs]
+    g, u, dn = mk(raws[0], ffn, d), mk(raws[1], ffn, d), mk(raws[2], d, ffn)
+    with pytest.raises(_ffi.PeregrineError):
+        moe.MoEExperts(g, u, dn, 3, moe.SILU, ctx).forward(np.zeros(d, np.float32), np.zeros((1, 2), np.float32))  # top_k > E
+    with pytest.raises(_ffi.PeregrineError):
+        moe.MoEExperts(g, u, [g[0], dn[1]], 1, moe.SILU, ctx).forward(np.zeros(d, np.float32), np.zeros((1, 2), np.float32))
+    out = moe.MoEExperts(g, u, dn, 1, moe.SILU, ctx).forward(np.zeros((0, d), np.float32), np.zeros((0, 2), np.float32))
+    assert out.shape == (0, d)

@@ -1,0 +1,235 @@
+"""GPU parity of the quant::* path against the CPU oracle, through the C ABI.
+
+Bar: quantised i8 values, f32 scales, i32 accumulators and the f32 outputs of the W8A8
+product are all BIT-EXACT (the epilogue keeps the reference's multiplication order, so
+even the f32 result has a single correct bit pattern).
+"""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+
+import helpers as H
+from devbuf import DevBuf
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def edge_rows(cols):
+    """Rows the reference's arithmetic treats specially (ties, zero, NaN, inf, subnormal)."""
+    r = np.zeros((6, cols), np.float32)
+    r[0, :8] = [127, -127, 0.5, -0.5, 1.5, 2.5, -2.5, 0]
+    r[2, :] = 4.0
+    r[2, 1::2] = -4.0
+    r[3, :8] = [np.nan, 1, -2, 0.5, 0, 0, 0, 2]
+    r[4, :8] = [np.inf, 1, -1, 0, 0, 0, 0, -np.inf]
+    r[5, :8] = [1e-42, -1e-42, 0, 0, 0, 0, 0, 5e-43]
+    return r
+
+
+@pytest.mark.parametrize("rows,cols", [(32, 4096), (1, 4096), (1, 14336), (7, 100), (5, 4100),
+                                       (3, 20000), (2, 16384), (9, 33), (4, 1)])
+def test_quantize_activations_bit_exact(ctx, orc, rows, cols):
+    from peregrine_amd import quant
+    say(f"quantize_activations rows={rows} cols={cols}")
+    a = orc.rng_normal(1000 + rows * 7 + cols, rows * cols).reshape(rows, cols)
+    a[:, :: max(1, cols // 40)] *= 20  # outlier channels
+    q, s = quant.quantize_activations(a, rows, cols, ctx)
+    qo, so = orc.quantize_activations(a, rows, cols)
+    assert (bits(s) == bits(so)).all()
+    assert (q == qo).all()
+
+
+def test_quantize_activations_edge_rows_and_empty(ctx, orc):
+    from peregrine_amd import quant
+    for cols in (8, 64, 4096):
+        say(f"quantize_activations edge rows cols={cols}")
+        a = edge_rows(cols)
+        q, s = quant.quantize_activations(a, a.shape[0], cols, ctx)
+        qo, so = orc.quantize_activations(a, a.shape[0], cols)
+        assert (bits(s) == bits(so)).all() and (q == qo).all()
+    # constructed near-tie rows that separate x*(1/s) from x/s
+    fh = float.fromhex
+    tie = np.array([[fh("0x1.13c502p-4"), fh("0x1.e6658ep-10"), fh("-0x1.09ff8ap-4"), fh("-0x1.f9f07ep-5")],
+                    [fh("0x1.18d40ep-5"), fh("0x1.1b0a2p-13"), fh("-0x1.1116c6p-5"), fh("-0x1.134cdap-5")]], np.float32)
+    q, s = quant.quantize_activations(tie, 2, 4, ctx)
+    qo, so = orc.quantize_activations(tie, 2, 4)
+    assert (q == qo).all() and (bits(s) == bits(so)).all()
+    q, s = quant.quantize_activations(np.zeros(0, np.float32), 0, 16, ctx)  # empty input
+    assert q.size == 0 and s.size == 0
+    with pytest.raises(ValueError):
+        quant.quantize_activations(np.zeros(5, np.float32), 2, 3, ctx)
+
+
+@pytest.mark.parametrize("rows,cols", [(128, 96), (100, 70), (4096, 64), (64, 1000), (1, 5), (300, 1)])
+def test_quantize_weights_bit_exact(ctx, orc, rows, cols):
+    from peregrine_amd import quant
+    say(f"quantize_weights rows={rows} cols={cols}")
+    w = orc.rng_normal(5678 + rows + cols, rows * cols, 0.0, 0.02)
+    qt = quant.quantize_weights(w, rows, cols, ctx)
+    q, q_t, s = orc.quantize_weights(w, rows, cols)
+    assert (bits(qt.scales) == bits(s)).all()
+    assert (qt.data_i8 == q).all()
+    assert (qt.data_i8_t == q_t).all()
+    assert (bits(quant.dequantize(qt, ctx)) == bits(orc.dequantize(q, s, rows, cols))).all()
+
+
+def test_quantize_weights_edge_columns(ctx, orc):
+    from peregrine_amd import quant
+    say("quantize_weights edge columns")
+    fh = float.fromhex
+    w = np.zeros((6, 7), np.float32)
+    w[:, 0] = [127, -127, 2.5, -2.5, 0.5, 1.5]
+    w[:, 2] = [3, 3, -3, 3, -3, 3]
+    w[:, 3] = [np.nan, 1, -2, 0.25, 0, 2]
+    w[:, 4] = [np.inf, 1, -1, 0, 5, -np.inf]
+    w[:4, 5] = [fh("0x1.13c502p-4"), fh("0x1.e6658ep-10"), fh("-0x1.09ff8ap-4"), fh("-0x1.f9f07ep-5")]
+    w[:4, 6] = [fh("0x1.18d40ep-5"), fh("0x1.1b0a2p-13"), fh("-0x1.1116c6p-5"), fh("-0x1.134cdap-5")]
+    qt = quant.quantize_weights(w, 6, 7, ctx)
+    q, q_t, s = orc.quantize_weights(w, 6, 7)
+    assert (bits(qt.scales) == bits(s)).all() and (qt.data_i8 == q).all() and (qt.data_i8_t == q_t).all()
+
+
+def test_reference_roundtrip_property(ctx):
+    # tests/quant_parity.rs:6-32 run against the GPU path
+    from peregrine_amd import quant
+    rows, cols = 64, 128
+    data = H.mod_pattern(rows * cols, 17, 5, 400, 100.0, 2.0)
+    qt = quant.quantize_weights(data, rows, cols, ctx)
+    rec = quant.dequantize(qt, ctx).reshape(rows, cols)
+    d = data.reshape(rows, cols)
+    amax = np.abs(d).max(axis=0)
+    scale = np.where(amax == 0, 1.0, amax / np.float32(127)).astype(np.float32)
+    assert (np.abs(d - rec) <= scale[None, :] + 1e-7).all()
+
+
+def test_to_gpu_from_gpu_roundtrip(ctx, orc):
+    # QuantizedTensor::to_gpu / from_gpu (src/quant.rs:173-191); upload is idempotent
+    from peregrine_amd import quant
+    rows, cols = 200, 130
+    w = orc.rng_normal(77, rows * cols, 0.0, 0.02)
+    qt = quant.quantize_weights(w, rows, cols, ctx)
+    q0, qt0, s0 = qt.data_i8.copy(), qt.data_i8_t.copy(), qt.scales.copy()
+    qt.to_gpu(ctx)
+    h = qt._gpu
+    qt.to_gpu(ctx)
+    assert qt._gpu is h
+    qt.data_i8[:] = 0
+    qt.from_gpu(ctx)
+    assert (qt.data_i8 == q0).all() and (qt.data_i8_t == qt0).all() and (bits(qt.scales) == bits(s0)).all()
+    with pytest.raises(RuntimeError):
+        quant.matmul_quantized_gpu(ctx, np.zeros(rows, np.float32), 1, rows,
+                                   quant.QuantizedTensor(q0, qt0, s0, rows, cols))  # "weights not on GPU"
+
+
+def run_matmul_dev(ctx, a, m, k, qt):
+    """pg_matmul_quantized_dev with the accumulator dump; returns (out, acc)."""
+    from peregrine_amd import _ffi
+    qt.to_gpu(ctx)
+    n = qt.cols
+    da = DevBuf(ctx, host=np.ascontiguousarray(a, np.float32))
+    dout, dacc = DevBuf(ctx, m * n * 4), DevBuf(ctx, m * n * 4)
+    _ffi.check(_ffi.lib.pg_matmul_quantized_dev(ctx.handle, da.ptr, m, k, qt._gpu, dout.ptr, dacc.ptr))
+    ctx.sync()
+    return dout.to_host(np.float32), dacc.to_host(np.int32)
+
+
+# (m, k, n): reference test shapes, decode GEMV shapes, every GEMM tile config, ragged edges
+MATMUL_SHAPES = [
+    (32, 128, 64), (16, 64, 32),                       # tests/quant_parity.rs:35, src/quant.rs:252
+    (8, 32, 16), (1, 64, 1), (16, 256, 32),            # tests/huffman_parity.rs:25
+    (1, 4096, 14336), (1, 14336, 4096),                # BASELINE config 2 (decode GEMV)
+    (2, 4096, 1024), (3, 1000, 77), (4, 4096, 300),    # GEMV with m = 2..4, ragged k and n
+    (32, 4096, 4096),                                  # BASELINE config 1
+    (5, 96, 40), (64, 200, 130), (65, 384, 129),       # 64x64 and 128x128 tiles, ragged
+    (196, 768, 3072),                                  # benches/wallclock.rs:758-786
+    (300, 512, 1000),                                  # 128x128 tiles, ragged m and n
+    (2048, 128, 4096),                                 # 256x128 tiles
+    (2050, 192, 4100),                                 # 256x128 tiles, ragged m and n
+]
+
+
+@pytest.mark.parametrize("m,k,n", MATMUL_SHAPES)
+def test_matmul_quantized_bit_exact(ctx, orc, m, k, n):
+    from peregrine_amd import quant
+    say(f"matmul_quantized m={m} k={k} n={n}")
+    a = orc.rng_normal(1234 + m, m * k)
+    if k >= 100:
+        a.reshape(m, k)[:, :: k // 50] *= 20  # outlier channels
+    w = orc.rng_normal(5678 + n, k * n, 0.0, 0.02)
+    qt = quant.quantize_weights(w, k, n, ctx)
+    q, q_t, s = orc.quantize_weights(w, k, n)
+    assert (qt.data_i8_t == q_t).all()
+    want, want_acc = orc.matmul_quantized(a, m, k, q_t, s, n)
+    got, got_acc = run_matmul_dev(ctx, a, m, k, qt)
+    assert (got_acc == want_acc).all(), "i32 accumulators differ"
+    assert (bits(got) == bits(want)).all(), "f32 outputs differ"
+    # the host-pointer entry point gives the same answer
+    got2 = quant.matmul_quantized(a, m, k, qt, ctx)
+    assert (bits(got2) == bits(want)).all()
+
+
+def test_matmul_quantized_extreme_integers(ctx, orc):
+    # every product is (-127)*(-127) or 127*(-127): the largest accumulators the path can see
+    from peregrine_amd import quant
+    m, k, n = 70, 14336, 130
+    say(f"matmul_quantized extremes m={m} k={k} n={n}")
+    a = np.full((m, k), -3.0, np.float32)
+    a[::2] = 3.0
+    w = np.full((k, n), -0.5, np.float32)
+    qt = quant.quantize_weights(w, k, n, ctx)
+    got, acc = run_matmul_dev(ctx, a, m, k, qt)
+    want_acc = np.where((np.arange(m) % 2 == 0)[:, None], -127 * 127 * k, 127 * 127 * k) * np.ones((1, n), np.int64)
+    assert (acc.reshape(m, n) == want_acc).all()
+    q, q_t, s = orc.quantize_weights(w, k, n)
+    want, _ = orc.matmul_quantized(a, m, k, q_t, s, n)
+    assert (bits(got) == bits(want)).all()
+
+
+def test_matmul_quantized_shape_mismatch_is_an_error(ctx, orc):
+    from peregrine_amd import quant, _ffi
+    qt = quant.quantize_weights(np.ones(64 * 8, np.float32), 64, 8, ctx)
+    with pytest.raises(ValueError):
+        quant.matmul_quantized(np.zeros(2 * 32, np.float32), 2, 32, qt, ctx)  # assert_eq!(w.rows, k)
+    qt.to_gpu(ctx)
+    out = np.zeros(16, np.float32)
+    st = _ffi.lib.pg_matmul_quantized(ctx.handle, C.c_void_p(out.ctypes.data), 2, 32, qt._gpu, C.c_void_p(out.ctypes.data))
+    assert st == _ffi.PG_EINVAL and b"rows" in _ffi.lib.pg_last_error()
+    assert quant.matmul_quantized(np.zeros(0, np.float32), 0, 64, qt, ctx).size == 0  # m = 0
+
+
+def test_prefill_shape_full_size_properties(ctx, orc):
+    """BASELINE config 3 shape (M = 2048, q_proj 4096 -> 4096) at full size: the oracle would
+    need 3.4e10 scalar MACs, so check (a) 48 sampled rows bit-exactly against the oracle and
+    (b) the sum over ALL accumulators against the exact identity
+        sum_{m,n} acc[m,n] = sum_k (sum_m a_i8[m,k]) * (sum_n w_t[n,k])   (int64)."""
+    from peregrine_amd import quant
+    m, k, n = 2048, 4096, 4096
+    say(f"prefill full size m={m} k={k} n={n}")
+    a = orc.rng_normal(4321, m * k).reshape(m, k)
+    chan = np.random.default_rng(1).choice(k, k // 100, replace=False)
+    a[:, chan] *= 20  # 1 % outlier channels
+    w = orc.rng_normal(8765, k * n, 0.0, 0.02)
+    qt = quant.quantize_weights(w, k, n, ctx)
+    q, q_t, s = orc.quantize_weights(w, k, n)
+    assert (qt.data_i8_t == q_t).all() and (bits(qt.scales) == bits(s)).all()
+    got, acc = run_matmul_dev(ctx, a, m, k, qt)
+    got, acc = got.reshape(m, n), acc.reshape(m, n)
+    a_i8, a_s = orc.quantize_activations(a, m, k)
+    col = a_i8.reshape(m, k).astype(np.int64).sum(axis=0)
+    wsum = q_t.reshape(n, k).astype(np.int64).sum(axis=0)
+    assert int(acc.astype(np.int64).sum()) == int((col * wsum).sum())
+    rows = np.random.default_rng(2).choice(m, 48, replace=False)
+    want, want_acc = orc.matmul_quantized(a[rows], len(rows), k, q_t, s, n)
+    assert (acc[rows] == want_acc.reshape(len(rows), n)).all()
+    assert (bits(got[rows]) == bits(want.reshape(len(rows), n))).all()
