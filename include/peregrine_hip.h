@@ -68,6 +68,16 @@ void *pg_ctx_stream(pg_ctx *ctx);
 const char *pg_last_error(void);
 const char *pg_status_string(pg_status st);
 
+/* Per-kernel timing.  No counterpart in the reference (it times whole calls with
+ * Instant::now(), benches/wallclock.rs:28-41): between pg_profile_begin and
+ * pg_profile_end every kernel the library launches on this context is bracketed by
+ * HIP events recorded on the context's stream; pg_profile_end waits for the stream
+ * and aggregates elapsed time per kernel name, read back with pg_profile_get. */
+pg_status pg_profile_begin(pg_ctx *ctx);
+pg_status pg_profile_end(pg_ctx *ctx, size_t *num_kernels);
+pg_status pg_profile_get(pg_ctx *ctx, size_t i, const char **name, double *total_ms,
+                         size_t *launches);
+
 /* Device memory for callers that have no HIP binding of their own
  * (GpuContext::alloc / upload / GpuBuffer::read, src/metal/buffer.rs). */
 pg_status pg_dev_alloc(pg_ctx *ctx, size_t bytes, void **dptr);

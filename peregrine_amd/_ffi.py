@@ -28,6 +28,9 @@ SIGNATURES = {
     "pg_ctx_stream": [_vp],
     "pg_last_error": [],
     "pg_status_string": [_int],
+    "pg_profile_begin": [_vp],
+    "pg_profile_end": [_vp, C.POINTER(_sz)],
+    "pg_profile_get": [_vp, _sz, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(_sz)],
     "pg_dev_alloc": [_vp, _sz, _pp],
     "pg_dev_free": [_vp, _vp],
     "pg_memcpy_h2d": [_vp, _vp, _vp, _sz],

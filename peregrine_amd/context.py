@@ -26,6 +26,21 @@ class Context:
     def sync(self):
         _ffi.check(_ffi.lib.pg_sync(self.handle))
 
+    def profile_begin(self):
+        """Start bracketing every kernel launch on this context with HIP events."""
+        _ffi.check(_ffi.lib.pg_profile_begin(self.handle))
+
+    def profile_end(self):
+        """Stop profiling; returns {kernel name: (total_ms, launches)}."""
+        n = C.c_size_t()
+        _ffi.check(_ffi.lib.pg_profile_end(self.handle, C.byref(n)))
+        out = {}
+        for i in range(n.value):
+            name, ms, cnt = C.c_char_p(), C.c_double(), C.c_size_t()
+            _ffi.check(_ffi.lib.pg_profile_get(self.handle, i, C.byref(name), C.byref(ms), C.byref(cnt)))
+            out[name.value.decode()] = (ms.value, cnt.value)
+        return out
+
     def close(self):
         if self._h:
             _ffi.lib.pg_ctx_destroy(self._h)

@@ -72,6 +72,7 @@ PG_API pg_status pg_ctx_create(int device, void *hip_stream, pg_ctx **out) {
     ctx->ws = nullptr;
     ctx->ws_bytes = 0;
     ctx->num_cu = prop.multiProcessorCount;
+    ctx->profiling = false;
     if (hip_stream) {
         ctx->stream = static_cast<hipStream_t>(hip_stream);
         ctx->owns_stream = false;
@@ -87,11 +88,14 @@ PG_API pg_status pg_ctx_create(int device, void *hip_stream, pg_ctx **out) {
     return PG_OK;
 }
 
+static void prof_drop(pg_ctx *ctx);
+
 PG_API void pg_ctx_destroy(pg_ctx *ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void)hipFree(ctx->ws);
+    prof_drop(ctx);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -134,5 +138,57 @@ PG_API pg_status pg_memcpy_d2h(pg_ctx *ctx, void *dst_host, const void *src_dev,
     PG_CHECK_ARG(dst_host && src_dev, "pg_memcpy_d2h: null pointer");
     PG_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+// ---- per-kernel timing with HIP events ------------------------------------------
+
+static void prof_drop(pg_ctx *ctx) {
+    for (auto &r : ctx->prof) {
+        (void)hipEventDestroy(r.start);
+        (void)hipEventDestroy(r.stop);
+    }
+    ctx->prof.clear();
+}
+
+PG_API pg_status pg_profile_begin(pg_ctx *ctx) {
+    PG_TRY(pg_use(ctx));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    prof_drop(ctx);
+    ctx->totals.clear();
+    ctx->profiling = true;
+    return PG_OK;
+}
+
+PG_API pg_status pg_profile_end(pg_ctx *ctx, size_t *num_kernels) {
+    PG_TRY(pg_use(ctx));
+    ctx->profiling = false;
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    ctx->totals.clear();
+    for (auto &r : ctx->prof) {
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, r.start, r.stop) != hipSuccess) continue;
+        pg_prof_total *t = nullptr;
+        for (auto &x : ctx->totals)
+            if (x.name == r.name) t = &x;
+        if (!t) {
+            ctx->totals.push_back({r.name, 0.0, 0});
+            t = &ctx->totals.back();
+        }
+        t->total_ms += ms;
+        t->launches += 1;
+    }
+    prof_drop(ctx);
+    if (num_kernels) *num_kernels = ctx->totals.size();
+    return PG_OK;
+}
+
+PG_API pg_status pg_profile_get(pg_ctx *ctx, size_t i, const char **name, double *total_ms,
+                                size_t *launches) {
+    PG_CHECK_ARG(ctx != nullptr, "null context");
+    PG_CHECK_ARG(i < ctx->totals.size(), "pg_profile_get: index %zu of %zu", i, ctx->totals.size());
+    if (name) *name = ctx->totals[i].name.c_str();
+    if (total_ms) *total_ms = ctx->totals[i].total_ms;
+    if (launches) *launches = ctx->totals[i].launches;
     return PG_OK;
 }

@@ -95,8 +95,11 @@ pg_status launch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *
         if (e != hipSuccess) return pg_fail(PG_EDEVICE, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     }
     const unsigned grid = (unsigned)(w->n_pad / (4 * R));
-    gemv_w8a8_kernel<R, M><<<grid, 256, lds, ctx->stream>>>(w->w_t, (int)w->k_pad, w->scales, a_i8,
-                                                          (int)a_stride, a_scales, (int)w->cols, out, acc);
+    {
+        pg_prof_scope ps(ctx, "gemv_w8a8");
+        gemv_w8a8_kernel<R, M><<<grid, 256, lds, ctx->stream>>>(w->w_t, (int)w->k_pad, w->scales, a_i8,
+                                                              (int)a_stride, a_scales, (int)w->cols, out, acc);
+    }
     return pg_launch_check("gemv_w8a8");
 }
 

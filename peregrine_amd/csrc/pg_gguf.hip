@@ -358,6 +358,7 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
 #define PG_GGUF_GEMV_LAUNCH(RR)                                                                    \
     do {                                                                                           \
         const dim3 grid((unsigned)batch.count, grid_for(n_out, 4 * RR));                           \
+        pg_prof_scope ps(ctx, QT == 4 ? "gguf_gemv_q4_0" : "gguf_gemv_q8_0");                      \
         gguf_gemv_kernel<QT, BPL, RR><<<grid, 256, lds, ctx->stream>>>(                            \
             qs, d, batch, (int)n_out, nb, xd.digits, dps, xd.bsum, bps, xd.xs, y);                 \
     } while (0)
@@ -411,6 +412,7 @@ pg_xdigits pg_xdigits_carve(void *base, size_t rows, size_t k) {
 pg_status pg_launch_x_to_digits(pg_ctx *ctx, const float *x_dev, size_t rows, size_t k,
                                 int ggml_type, const pg_xdigits &xd) {
     if (rows == 0) return PG_OK;
+    pg_prof_scope ps(ctx, "x_to_digits");
     x_to_digits_kernel<<<(unsigned)rows, 256, 0, ctx->stream>>>(
         x_dev, k, ggml_type == PG_GGML_Q4_0 ? 1 : 0, rows, xd.digits, xd.xs, xd.bsum);
     return pg_launch_check("x_to_digits");

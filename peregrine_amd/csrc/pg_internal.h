@@ -4,9 +4,21 @@
 #include <stddef.h>
 #include <stdint.h>
 #include <string.h>
+#include <string>
+#include <vector>
 #include "peregrine_hip.h"
 
 #define PG_API extern "C" __attribute__((visibility("default")))
+
+struct pg_prof_rec {
+    const char *name;
+    hipEvent_t start, stop;
+};
+struct pg_prof_total {
+    std::string name;
+    double total_ms;
+    size_t launches;
+};
 
 // One device + one stream + one growable scratch arena.
 struct pg_ctx {
@@ -16,6 +28,26 @@ struct pg_ctx {
     void *ws;        // scratch arena (quantised activations, partial results)
     size_t ws_bytes;
     int num_cu;
+    bool profiling;                     // per-kernel HIP events (pg_profile_begin/end)
+    std::vector<pg_prof_rec> prof;      // one record per launch while profiling
+    std::vector<pg_prof_total> totals;  // aggregated by pg_profile_end
+};
+
+// Brackets one kernel launch with HIP events on the context's stream while profiling.
+struct pg_prof_scope {
+    pg_ctx *ctx;
+    hipEvent_t stop = nullptr;
+    pg_prof_scope(pg_ctx *c, const char *name) : ctx(c) {
+        if (!c->profiling) return;
+        hipEvent_t start = nullptr;
+        if (hipEventCreate(&start) != hipSuccess) return;
+        if (hipEventCreate(&stop) != hipSuccess) { (void)hipEventDestroy(start); stop = nullptr; return; }
+        (void)hipEventRecord(start, c->stream);
+        c->prof.push_back({name, start, stop});
+    }
+    ~pg_prof_scope() {
+        if (stop) (void)hipEventRecord(stop, ctx->stream);
+    }
 };
 
 // Device-resident quantised weight, K-contiguous and zero-padded:

@@ -132,8 +132,9 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     // host_tab lives on this stack frame: the copy must have left it before we return.
     PG_HIP(hipStreamSynchronize(ctx->stream));
 
+    { pg_prof_scope ps(ctx, "moe_route_topk");
     route_topk_kernel<<<grid_for(T, 64), 64, 0, ctx->stream>>>(router_logits_dev, (int)T, (int)E, (int)top_k,
-                                                             topk_idx, topk_p);
+                                                             topk_idx, topk_p); }
     PG_TRY(pg_launch_check("route_topk"));
     PG_TRY(pg_launch_x_to_digits(ctx, x_dev, T, d, type, xd));
     auto table = [&](int which) { return reinterpret_cast<const uint8_t *const *>(tab + which * E); };
@@ -142,12 +143,14 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     PG_TRY(pg_launch_gguf_gemv(ctx, type, ffn, d, nullptr, nullptr, bg, xd, g));
     pg_gemv_batch bu = {(int)P, table(2), dtable(3), topk_idx, (int)top_k};
     PG_TRY(pg_launch_gguf_gemv(ctx, type, ffn, d, nullptr, nullptr, bu, xd, u));
-    act_mul_kernel<<<grid_for(P * ffn, 256), 256, 0, ctx->stream>>>(g, u, P * ffn, act, h);
+    { pg_prof_scope ps(ctx, "moe_act_mul");
+    act_mul_kernel<<<grid_for(P * ffn, 256), 256, 0, ctx->stream>>>(g, u, P * ffn, act, h); }
     PG_TRY(pg_launch_check("act_mul"));
     PG_TRY(pg_launch_x_to_digits(ctx, h, P, ffn, type, hd));
     pg_gemv_batch bd = {(int)P, table(4), dtable(5), topk_idx, 1};
     PG_TRY(pg_launch_gguf_gemv(ctx, type, d, ffn, nullptr, nullptr, bd, hd, yb));
-    combine_kernel<<<grid_for(T * d, 256), 256, 0, ctx->stream>>>(yb, topk_p, (int)T, (int)d, (int)top_k, out_dev);
+    { pg_prof_scope ps(ctx, "moe_combine");
+    combine_kernel<<<grid_for(T * d, 256), 256, 0, ctx->stream>>>(yb, topk_p, (int)T, (int)d, (int)top_k, out_dev); }
     return pg_launch_check("moe_combine");
 }
 
