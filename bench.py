@@ -61,8 +61,13 @@ def main():
         sys.exit("bench.py: no GPU visible; peregrine_amd has no CPU path to measure")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    stream = torch.cuda.current_stream()
-    ctx = Context(0, stream=stream.cuda_stream)  # library launches on torch's current stream
+    # A dedicated (non-null) stream shared by torch and the library, so the torch events
+    # that bracket the timed region see the library's kernels.
+    stream = torch.cuda.Stream(device=dev)
+    torch.cuda.set_stream(stream)
+    assert stream.cuda_stream != 0
+    ctx = Context(0, stream=stream.cuda_stream)
+    assert ctx.stream == stream.cuda_stream
     lib, check = _ffi.lib, _ffi.check
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)

@@ -2,16 +2,20 @@
 // dequantise-matmul over GGUF Q4_0 / Q8_0 weights kept quantised in HBM.
 //
 // Fused product, y[m, n] = sum_k x[m, k] * (q[n, k] * d[n, k/32]):
-//  * each activation row is first rewritten as 24-bit fixed point,
-//    x[k] = s * X[k] with s a power of two and |X| < 2^22 (absolute error
-//    <= 2^-23 * max|x| per element, the rounding an f32 accumulation of the row
-//    would commit anyway), and X split into three signed byte digits
-//    X = 65536*a0 + 256*a1 + a2;
-//  * the inner sums over one block of 32, sum_k q*a_j, are then exact integer
-//    dot products (v_dot4_i32_i8 on the packed bytes, no per-element int->float
-//    conversion), recombined and scaled by d in f32 once per block.
-// The result differs from the reference's dequantise-then-f32-matmul only by
-// f32 rounding noise (relative tolerance 1e-3 is the contract; observed ~1e-6).
+//  * each block of 32 activations is first rewritten as fixed point, x[k] = s * X[k] with s
+//    a power of two taken from the block's absmax (absolute error <= 2^-19 (Q4_0) or 2^-23
+//    (Q8_0) of the block's max|x| per element, at or below what an f32 accumulation commits
+//    anyway), and X is split into signed digits: five 4-bit digits for Q4_0, three bytes
+//    for Q8_0;
+//  * the inner sums over one block, sum_k q * digit_j, are then exact integer dot products
+//    on packed data with no per-element unpack or int->float conversion: Q4_0 nibbles are
+//    stored with their top bit flipped at upload, which makes each nibble the two's
+//    complement of (q - 8), so v_dot8_i32_i4 multiplies 8 weights by 8 activation digits per
+//    instruction straight from the packed bytes; Q8_0 uses v_dot4_i32_i8;
+//  * the digit sums are recombined exactly in integers, converted once and scaled by
+//    d * s in f32 once per block.
+// The result differs from the reference's dequantise-then-f32-matmul only by rounding noise
+// (relative tolerance 1e-3 is the contract; the tests hold this path to 2e-5).
 #include <new>
 #include "pg_internal.h"
 
@@ -86,153 +90,147 @@ __global__ void dequant_q4_1_kernel(const uint8_t *__restrict__ data, size_t nbl
 }
 
 // ---- upload: split raw blocks into planes ---------------------------------------
-// Q4_0: qs[(n*nb + b)*16 .. +16] = the block's 16 nibble bytes.
+// Q4_0: qs[(n*nb + b)*16 .. +16] = the block's 16 nibble bytes, each nibble's top bit flipped.
 // Q8_0: qs[((n*2 + h)*nb + b)*16 .. +16] = bytes 16h..16h+15 of the block's 32 i8.
-// d[n*nb + b] = the block's f16 scale.
+// d[((n/8)*nb + b)*8 + n%8] = the block's f16 scale: tiles of 8 rows, so one 128-bit load
+// gives a lane the scales of its block for 8 consecutive weight rows (rows past n_out: 0).
 __global__ void split_blocks_kernel(const uint8_t *__restrict__ raw, size_t n_out, size_t nb,
                                     int ggml_type, uint8_t *__restrict__ qs,
                                     uint16_t *__restrict__ d) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n_out * nb) return;
+    const size_t n_pad = (n_out + 7) / 8 * 8;
+    if (i >= n_pad * nb) return;
     const size_t n = i / nb, b = i - n * nb;
+    uint16_t *dd = d + ((n / 8) * nb + b) * 8 + (n % 8);
+    if (n >= n_out) { *dd = 0; return; }
     if (ggml_type == PG_GGML_Q4_0) {
         const uint8_t *blk = raw + i * 18;
-        d[i] = ld_u16(blk);
-        for (int j = 0; j < 16; ++j) qs[i * 16 + j] = blk[2 + j];
+        *dd = ld_u16(blk);
+        for (int j = 0; j < 16; ++j) qs[i * 16 + j] = blk[2 + j] ^ 0x88;  // nibble -> (q - 8) in two's complement
     } else {
         const uint8_t *blk = raw + i * 34;
-        d[i] = ld_u16(blk);
+        *dd = ld_u16(blk);
         for (int h = 0; h < 2; ++h)
             for (int j = 0; j < 16; ++j) qs[((n * 2 + h) * nb + b) * 16 + j] = blk[2 + 16 * h + j];
     }
 }
 
-// ---- activation rows -> 24-bit fixed point, three byte digits -------------------
-// Output for row m (all of it in the scratch arena):
-//   digits[j][m][k']  j = 0..2, k' = k for Q8_0; for Q4_0 each block of 32 is stored
-//                     as its 16 even-indexed elements followed by its 16 odd-indexed
-//                     ones, matching (byte & 15) / (byte >> 4) unpacked as dwords;
-//   xs[m]             the power-of-two scale (NaN if the row holds a NaN or inf);
-//   bsum[j][m][b]     sum of digit j over block b (Q4_0's -8 offset needs it).
-__device__ __forceinline__ void split_digits(int X, int &a0, int &a1, int &a2) {
-    a2 = ((X + 128) & 255) - 128;
-    const int X1 = (X - a2) >> 8;
-    a1 = ((X1 + 128) & 255) - 128;
-    a0 = (X1 - a1) >> 8;
-}
-
-__global__ __launch_bounds__(256) void x_to_digits_kernel(const float *__restrict__ x, size_t k,
-                                                          int deinterleave, size_t rows,
+// ---- activation blocks -> fixed point digits ------------------------------------------
+// For every block of 32 activations: x[k] = s * X[k] with s a power of two chosen from the
+// block's absmax.  Output for activation row m (all of it in the scratch arena):
+//   xs[m][b]            the block's scale s (NaN if the block holds a NaN or inf)
+//   digits[m][j][b]     16 bytes per (plane j, block b); lanes that own consecutive blocks
+//                       read consecutive 16-byte chunks.
+//     Q4_0 (NIB): |X| < 2^18, X = sum_j 16^j n_j with five signed 4-bit digits; plane j holds
+//                 n_j of the block's 32 elements, element e in nibble e (the order the
+//                 weight bytes pack them: byte i = elements 2i (low) and 2i+1 (high)).
+//     Q8_0:       |X| < 2^22, X = 65536 a0 + 256 a1 + a2 with signed byte digits; plane
+//                 2j+h holds a_j of elements 16h..16h+15.
+// 8 consecutive threads own one block (4 elements each); a workgroup covers 32 blocks.
+template <bool NIB>
+__global__ __launch_bounds__(256) void x_to_digits_kernel(const float *__restrict__ x, int nb,
                                                           int8_t *__restrict__ digits,
-                                                          float *__restrict__ xs,
-                                                          int *__restrict__ bsum) {
-    __shared__ float red[4];
-    __shared__ int bad[4];
-    const size_t row = blockIdx.x;
-    const float *xr = x + row * k;
-    float amax = 0.0f;
-    int nan_seen = 0;
-    for (size_t i = threadIdx.x; i < k; i += 256) {
-        const float v = xr[i];
-        nan_seen |= (v != v);
-        amax = fmaxf(amax, fabsf(v));
-    }
+                                                          float *__restrict__ xs) {
+    const size_t row = blockIdx.y;
+    const int b = blockIdx.x * 32 + (threadIdx.x >> 3), sub = threadIdx.x & 7;
+    if (b >= nb) return;  // whole 8-thread groups leave together
+    const float4 v = reinterpret_cast<const float4 *>(x + (row * nb + b) * 32)[sub];
+    const float f[4] = {v.x, v.y, v.z, v.w};
+    float amax = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3])));
+    int bad = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]);
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
+    for (int off = 1; off < 8; off <<= 1) {
         amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-        nan_seen |= __shfl_xor(nan_seen, off, 64);
+        bad |= __shfl_xor(bad, off, 64);
     }
-    if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = amax; bad[threadIdx.x >> 6] = nan_seen; }
-    __syncthreads();
-    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    nan_seen = bad[0] | bad[1] | bad[2] | bad[3];
+    constexpr int BITS = NIB ? 18 : 22;
     float s = 1.0f, inv = 1.0f;
-    if (nan_seen || !(amax <= 3.4028234663852886e38f)) {
+    if (bad || !(amax <= 3.4028234663852886e38f)) {
         s = __uint_as_float(0x7FC00000u);
         inv = 0.0f;
     } else if (amax > 0.0f) {
         int ex;
         (void)frexpf(amax, &ex);  // amax = f * 2^ex, f in [0.5, 1)
-        int se = ex - 22;         // |x| / 2^se < 2^22
+        int se = ex - BITS;       // |x| / 2^se < 2^BITS
         if (se < -126) se = -126;
         s = ldexpf(1.0f, se);
         inv = ldexpf(1.0f, -se);
     }
-    if (threadIdx.x == 0) xs[row] = s;
-    const size_t nb = k / 32;
-    // 8 consecutive threads cover one block of 32 (4 elements each).
-    for (size_t g = threadIdx.x; g < k / 4; g += 256) {
-        const float4 v = reinterpret_cast<const float4 *>(xr)[g];
-        const float f[4] = {v.x, v.y, v.z, v.w};
+    int X[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float t = f[e] * inv;
+        X[e] = (t != t) ? 0 : (int)rintf(t);
+    }
+    int8_t *drow = digits + row * (size_t)nb * 96;
+    if (NIB) {
+#pragma unroll
+        for (int j = 0; j < 5; ++j) {
+            unsigned packed = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = ((X[e] + 8) & 15) - 8;  // signed 4-bit digit
+                X[e] = (X[e] - n) >> 4;
+                packed |= (unsigned)(n & 15) << (4 * e);
+            }
+            // this thread's elements 4*sub .. 4*sub+3 are nibbles 4*sub.. of the block: bytes 2*sub, 2*sub+1
+            *reinterpret_cast<uint16_t *>(drow + ((size_t)j * nb + b) * 16 + 2 * sub) = (uint16_t)packed;
+        }
+    } else {
         int a[3][4];
-        int sum[3] = {0, 0, 0};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const float t = f[e] * inv;
-            const int X = (t != t) ? 0 : (int)rintf(t);
-            split_digits(X, a[0][e], a[1][e], a[2][e]);
-#pragma unroll
-            for (int j = 0; j < 3; ++j) sum[j] += a[j][e];
+            a[2][e] = ((X[e] + 128) & 255) - 128;
+            const int X1 = (X[e] - a[2][e]) >> 8;
+            a[1][e] = ((X1 + 128) & 255) - 128;
+            a[0][e] = (X1 - a[1][e]) >> 8;
         }
-        const size_t b = g / 8;
-        const int e0 = (int)(g & 7) * 4;  // first element of this thread within the block
+        const int e0 = sub * 4, h = e0 >> 4;
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
-            int8_t *dst = digits + ((size_t)j * rows + row) * k + b * 32;
-            if (deinterleave) {
-                dst[e0 / 2] = (int8_t)a[j][0];
-                dst[e0 / 2 + 1] = (int8_t)a[j][2];
-                dst[16 + e0 / 2] = (int8_t)a[j][1];
-                dst[16 + e0 / 2 + 1] = (int8_t)a[j][3];
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) dst[e0 + e] = (int8_t)a[j][e];
-            }
-            int t = sum[j];
-            t += __shfl_xor(t, 1, 64);
-            t += __shfl_xor(t, 2, 64);
-            t += __shfl_xor(t, 4, 64);
-            if ((g & 7) == 0) bsum[((size_t)j * rows + row) * nb + b] = t;
+            const unsigned packed = (unsigned)(a[j][0] & 255) | ((unsigned)(a[j][1] & 255) << 8) |
+                                    ((unsigned)(a[j][2] & 255) << 16) | ((unsigned)(a[j][3] & 255) << 24);
+            *reinterpret_cast<unsigned *>(drow + ((size_t)(2 * j + h) * nb + b) * 16 + (e0 & 15)) = packed;
         }
     }
+    if (sub == 0) xs[row * (size_t)nb + b] = s;
 }
 
 // ---- M = 1 fused dequant-GEMV ------------------------------------------------------
-// Workgroup = 4 wavefronts; wavefront w owns R consecutive weight rows.  Lane l
-// owns blocks l, l+64, ... (BPL of them per K segment of 64*BPL blocks): its
-// activation digits for those blocks sit in registers for all R rows, and one
-// wavefront load of weights covers 64 consecutive blocks (1 KiB) of one row.
-// The workgroup first stages the row's digits in LDS as [digit][16B-half][block]
-// so the per-lane 128-bit LDS reads are conflict-free.
-template <int QT>  // 4 = Q4_0, 8 = Q8_0
-struct BlockDot;
-
-template <>
-struct BlockDot<4> {
-    // w: 16 nibble bytes; xe/xo: even/odd element digits (4 dwords each).
-    static __device__ __forceinline__ int dot(const v4i w, const v4i xe, const v4i xo, int acc) {
+// One wavefront per workgroup, no LDS, no barrier.  Lane l owns blocks l, l+64, ... (BPL
+// of them per K segment of 64*BPL blocks): its activation digits, block sums and block
+// scales for those blocks sit in registers while the wavefront walks R*NG weight rows, R at
+// a time, requesting the next R rows before it consumes the current ones.  One wavefront
+// load of weights covers 64 consecutive blocks (1 KiB) of one row.
+// sum over one block of (weight) * (activation fixed-point value X), exact, as an i32.
+// Q4_0: w = 16 bytes of biased nibbles, xn[j] = plane j (32 signed nibbles).
+__device__ __forceinline__ int block_dot_q4(const v4i w, const v4i (&xn)[5]) {
+    int acc = 0;
+#pragma unroll
+    for (int j = 4; j >= 0; --j) {  // Horner over the 4-bit digits: acc = 16*acc + I_j
+        int ij = 0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) ij = __builtin_amdgcn_sdot8(w[t], xn[j][t], ij, false);
+        acc = acc * 16 + ij;
+    }
+    return acc;  // |acc| <= 32 * 8 * 2^18 = 2^26
+}
+// Q8_0: w0/w1 = the block's 32 i8, x[j][h] = byte digit j of half h.  Returns the high and
+// low parts separately (65536 * i0 would overflow i32 when added to the rest).
+__device__ __forceinline__ void block_dot_q8(const v4i w0, const v4i w1, const v4i (&x)[6], int &hi, int &lo) {
+    int i[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        i[j] = 0;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            const int lo = w[t] & 0x0F0F0F0F;
-            const int hi = (w[t] >> 4) & 0x0F0F0F0F;
-            acc = __builtin_amdgcn_sdot4(lo, xe[t], acc, false);
-            acc = __builtin_amdgcn_sdot4(hi, xo[t], acc, false);
+            i[j] = __builtin_amdgcn_sdot4(w0[t], x[2 * j][t], i[j], false);
+            i[j] = __builtin_amdgcn_sdot4(w1[t], x[2 * j + 1][t], i[j], false);
         }
-        return acc;
     }
-};
-
-template <>
-struct BlockDot<8> {
-    static __device__ __forceinline__ int dot(const v4i w0, const v4i w1, const v4i x0, const v4i x1, int acc) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            acc = __builtin_amdgcn_sdot4(w0[t], x0[t], acc, false);
-            acc = __builtin_amdgcn_sdot4(w1[t], x1[t], acc, false);
-        }
-        return acc;
-    }
-};
+    hi = i[0];
+    lo = i[1] * 256 + i[2];
+}
 
 // Hardware f16 -> f32 (exact for every non-NaN input).
 __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
@@ -241,130 +239,142 @@ __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
     return (float)v;
 }
 
-__device__ __forceinline__ float wave_sum_f32(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
+__device__ __forceinline__ float wave_sum_f32(float v) { return pg_wave_sum_f32(v); }
 
-// blockIdx.x = batch item (activation row / MoE pair), blockIdx.y = group of 4*R
-// weight rows.  With a table, item i multiplies by expert table[expert_of[i]] and
-// reads activation row i / x_row_div; without one, every item uses (qs0, d0).
+typedef const v4i __attribute__((address_space(1))) *gv4i_ptr;  // loads known to be global, not flat
+
 template <int QT, int BPL, int R>
-__global__ __launch_bounds__(256) void gguf_gemv_kernel(
+struct RowLoads {
+    v4i w[R][BPL][QT == 8 ? 2 : 1];
+};
+
+// blockIdx.x = group of RW consecutive weight rows (RW divides 8: one scale tile),
+// blockIdx.y = batch item (activation row / MoE pair).  With a table, item i multiplies by
+// expert table[expert_of[i]] and reads activation row i / x_row_div; without one, every item
+// uses (qs0, d0).  R rows are in flight at a time (NG = RW / R groups, double-buffered).
+template <int QT, int BPL, int RW, int R>
+__global__ __launch_bounds__(64) void gguf_gemv_kernel(
     const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0, pg_gemv_batch batch,
-    int n_out, int nb, const int8_t *__restrict__ digits_base, size_t digit_plane_stride,
-    const int *__restrict__ bsum_base, size_t bsum_plane_stride, const float *__restrict__ xs_base,
+    int n_out, int nb, const int8_t *__restrict__ digits_base, const float *__restrict__ xs_base,
     float *__restrict__ y_base) {
-    extern __shared__ v4i xl[];  // [3][2][seg_blocks] 16-byte halves
     constexpr int SEG = 64 * BPL;  // blocks per K segment
-    const int item = blockIdx.x;
-    const uint8_t *__restrict__ qs = qs0;
-    const uint16_t *__restrict__ dsc = d0;
+    constexpr int NG = RW / R;
+    constexpr int NH = QT == 8 ? 2 : 1;
+    constexpr int NP = QT == 8 ? 6 : 5;  // digit planes
+    const int item = blockIdx.y;
+    const uint8_t *qs_any = qs0;
+    const uint16_t *d_any = d0;
     if (batch.qs_table) {
         const int e = batch.expert_of[item];
-        qs = batch.qs_table[e];
-        dsc = batch.d_table[e];
+        qs_any = batch.qs_table[e];
+        d_any = batch.d_table[e];
     }
+    const gv4i_ptr qs = (gv4i_ptr)(uintptr_t)qs_any;
+    const gv4i_ptr dsc = (gv4i_ptr)(uintptr_t)d_any;
     const size_t xrow = (size_t)(item / batch.x_row_div);
-    const int8_t *__restrict__ digits = digits_base + xrow * (size_t)nb * 32;
-    const int *__restrict__ bsum = bsum_base + xrow * (size_t)nb;
-    const float *__restrict__ xs = xs_base + xrow;
+    const gv4i_ptr digits = (gv4i_ptr)(uintptr_t)(digits_base + xrow * (size_t)nb * 96);
+    const float *__restrict__ xs = xs_base + xrow * (size_t)nb;
     float *__restrict__ y = y_base + (size_t)item * n_out;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int row0 = (blockIdx.y * 4 + wave) * R;
-    float acc[R];
+    const int lane = threadIdx.x;
+    const int row0 = blockIdx.x * RW;
+    float acc[NG][R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[g][r] = 0.0f;
 
     for (int seg0 = 0; seg0 < nb; seg0 += SEG) {
         const int seg_n = (nb - seg0 < SEG) ? nb - seg0 : SEG;
-        __syncthreads();  // previous segment fully consumed
-        for (int i = threadIdx.x; i < 3 * 2 * seg_n; i += 256) {
-            const int j = i / (2 * seg_n), rem = i - j * 2 * seg_n;
-            const int b = rem >> 1, h = rem & 1;
-            const v4i v = *reinterpret_cast<const v4i *>(digits + (size_t)j * digit_plane_stride +
-                                                         (size_t)(seg0 + b) * 32 + h * 16);
-            xl[(j * 2 + h) * SEG + b] = v;
-        }
-        __syncthreads();
-        // this lane's digits and block sums for the segment
-        v4i xd[BPL][3][2];
-        int off8[BPL][3];
+        int blk[BPL];  // this lane's blocks; lanes past the segment end re-read block seg0 with a zero scale
 #pragma unroll
-        for (int p = 0; p < BPL; ++p) {
-            const int bl = lane + 64 * p;
-            const bool live = bl < seg_n;
-#pragma unroll
-            for (int j = 0; j < 3; ++j) {
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    v4i v = xl[(j * 2 + h) * SEG + (live ? bl : 0)];
-                    if (!live) v = (v4i){0, 0, 0, 0};
-                    xd[p][j][h] = v;
-                }
-                off8[p][j] = (QT == 4 && live) ? -8 * bsum[(size_t)j * bsum_plane_stride + seg0 + bl] : 0;
-            }
-        }
-        if (row0 < n_out) {
+        for (int p = 0; p < BPL; ++p) blk[p] = seg0 + (lane + 64 * p < seg_n ? lane + 64 * p : 0);
+        auto load_rows = [&](RowLoads<QT, BPL, R> &L, int g) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const int row = (row0 + r < n_out) ? row0 + r : n_out - 1;  // clamp, masked at the store
+                int row = row0 + g * R + r;
+                row = row < n_out ? row : n_out - 1;  // clamped; masked at the store
+#pragma unroll
+                for (int p = 0; p < BPL; ++p)
+#pragma unroll
+                    for (int h = 0; h < NH; ++h)
+                        L.w[r][p][h] = __builtin_nontemporal_load(qs + ((size_t)row * NH + h) * nb + blk[p]);
+            }
+        };
+        // Loads return in issue order, so the (L2 / L1 resident) digits, block sums and scales
+        // of this lane's blocks are requested first and the HBM weight rows right behind them:
+        // the arithmetic on row r can then start as soon as row r lands, while later rows are
+        // still in flight.
+        v4i xd[BPL][NP];
+        float sb[BPL];
+        v4i dtile[BPL];  // f16 scales of this lane's blocks for the 8 rows of the tile
+#pragma unroll
+        for (int p = 0; p < BPL; ++p) {
+#pragma unroll
+            for (int j = 0; j < NP; ++j) xd[p][j] = digits[(size_t)j * nb + blk[p]];
+            sb[p] = xs[blk[p]];
+            dtile[p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        RowLoads<QT, BPL, R> L[2];
+        load_rows(L[0], 0);
+        __builtin_amdgcn_sched_barrier(0);  // every load is issued before any arithmetic
+#pragma unroll
+        for (int p = 0; p < BPL; ++p) sb[p] *= (lane + 64 * p < seg_n ? 1.0f : 0.0f);
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            if (g + 1 < NG) {
+                load_rows(L[(g + 1) & 1], g + 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            const RowLoads<QT, BPL, R> &C = L[g & 1];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int tr = (row0 & 7) + g * R + r;  // row within the scale tile
 #pragma unroll
                 for (int p = 0; p < BPL; ++p) {
-                    const int bl = lane + 64 * p;
-                    const int b = seg0 + ((bl < seg_n) ? bl : 0);
-                    int i0 = off8[p][0], i1 = off8[p][1], i2 = off8[p][2];
-                    if (QT == 4) {
-                        const v4i w = __builtin_nontemporal_load(
-                            reinterpret_cast<const v4i *>(qs + ((size_t)row * nb + b) * 16));
-                        i0 = BlockDot<4>::dot(w, xd[p][0][0], xd[p][0][1], i0);
-                        i1 = BlockDot<4>::dot(w, xd[p][1][0], xd[p][1][1], i1);
-                        i2 = BlockDot<4>::dot(w, xd[p][2][0], xd[p][2][1], i2);
+                    float f;  // sum_k (weight) * X over the block
+                    if constexpr (QT == 4) {
+                        f = (float)block_dot_q4(C.w[r][p][0], reinterpret_cast<const v4i(&)[5]>(xd[p]));
                     } else {
-                        const v4i w0 = __builtin_nontemporal_load(
-                            reinterpret_cast<const v4i *>(qs + (((size_t)row * 2 + 0) * nb + b) * 16));
-                        const v4i w1 = __builtin_nontemporal_load(
-                            reinterpret_cast<const v4i *>(qs + (((size_t)row * 2 + 1) * nb + b) * 16));
-                        i0 = BlockDot<8>::dot(w0, w1, xd[p][0][0], xd[p][0][1], i0);
-                        i1 = BlockDot<8>::dot(w0, w1, xd[p][1][0], xd[p][1][1], i1);
-                        i2 = BlockDot<8>::dot(w0, w1, xd[p][2][0], xd[p][2][1], i2);
+                        int hi, lo;
+                        block_dot_q8(C.w[r][p][0], C.w[r][p][NH - 1], reinterpret_cast<const v4i(&)[6]>(xd[p]), hi, lo);
+                        f = fmaf((float)hi, 65536.0f, (float)lo);  // both terms exact in f32
                     }
-                    const float d = half_bits_to_float(dsc[(size_t)row * nb + b]);
-                    // X-weighted block sum: 65536*i0 + 256*i1 + i2 (each term exact in f32)
-                    const float f = fmaf((float)i0, 65536.0f, (float)(i1 * 256 + i2));
-                    acc[r] = fmaf(d, f, acc[r]);
+                    const uint32_t pair = (uint32_t)dtile[p][tr >> 1];
+                    const float ds = half_bits_to_float((uint16_t)((tr & 1) ? pair >> 16 : pair & 0xFFFFu)) * sb[p];
+                    acc[g][r] = fmaf(ds, f, acc[g][r]);
                 }
             }
         }
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = wave_sum_f32(acc[r]);
-    if (lane == 0) {
-        const float s = xs[0];
+    for (int g = 0; g < NG; ++g)
 #pragma unroll
-        for (int r = 0; r < R; ++r)
-            if (row0 + r < n_out) y[row0 + r] = acc[r] * s;
-    }
+        for (int r = 0; r < R; ++r) {
+            const float v = wave_sum_f32(acc[g][r]);
+            const int row = row0 + g * R + r;
+            if (lane == 0 && row < n_out) y[row] = v;
+        }
 }
 
 template <int QT, int BPL>
 pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
                           const pg_gemv_batch &batch, const pg_xdigits &xd, float *y) {
     const int nb = (int)(k_in / 32);
-    const size_t lds = (size_t)3 * 2 * 64 * BPL * 16;
-    const size_t want_waves = (size_t)ctx->num_cu * 8;
-    const size_t dps = xd.rows * xd.k, bps = xd.rows * (size_t)nb;
-#define PG_GGUF_GEMV_LAUNCH(RR)                                                                    \
+    // rows in flight per wavefront: bounded by registers (16 B of weights per row and block)
+    constexpr int NH = QT == 8 ? 2 : 1;
+    constexpr int R8 = BPL * NH <= 2 ? 8 : (BPL * NH <= 4 ? 4 : 2);
+    pg_prof_scope ps(ctx, QT == 4 ? "gguf_gemv_q4_0" : "gguf_gemv_q8_0");
+    const size_t want = (size_t)ctx->num_cu * 6;  // wavefronts wanted in the grid
+#define PG_GGUF_GEMV_LAUNCH(RWW, RR)                                                               \
     do {                                                                                           \
-        const dim3 grid((unsigned)batch.count, grid_for(n_out, 4 * RR));                           \
-        pg_prof_scope ps(ctx, QT == 4 ? "gguf_gemv_q4_0" : "gguf_gemv_q8_0");                      \
-        gguf_gemv_kernel<QT, BPL, RR><<<grid, 256, lds, ctx->stream>>>(                            \
-            qs, d, batch, (int)n_out, nb, xd.digits, dps, xd.bsum, bps, xd.xs, y);                 \
+        const dim3 grid(grid_for(n_out, RWW), (unsigned)batch.count);                              \
+        gguf_gemv_kernel<QT, BPL, RWW, RR><<<grid, 64, 0, ctx->stream>>>(                          \
+            qs, d, batch, (int)n_out, nb, xd.digits, xd.xs, y);                           \
     } while (0)
-    if (n_out / 4 * batch.count >= want_waves) PG_GGUF_GEMV_LAUNCH(4);
-    else if (n_out / 2 * batch.count >= want_waves) PG_GGUF_GEMV_LAUNCH(2);
-    else PG_GGUF_GEMV_LAUNCH(1);
+    if (n_out / 8 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(8, R8);
+    else if (n_out / 4 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(4, (R8 < 4 ? R8 : 4));
+    else PG_GGUF_GEMV_LAUNCH(2, 2);
 #undef PG_GGUF_GEMV_LAUNCH
     return pg_launch_check("gguf_gemv");
 }
@@ -374,16 +384,12 @@ pg_status launch_gemv(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs,
                       const pg_gemv_batch &batch, const pg_xdigits &xd, float *y) {
     const size_t nb = k_in / 32;
     size_t bpl = (nb + 63) / 64;
-    if (bpl > 8) bpl = 8;  // longer rows run as several K segments
+    if (bpl > 4) bpl = 4;  // longer rows run as several K segments of 256 blocks
     switch (bpl) {
         case 1: return launch_gemv_bpl<QT, 1>(ctx, n_out, k_in, qs, d, batch, xd, y);
         case 2: return launch_gemv_bpl<QT, 2>(ctx, n_out, k_in, qs, d, batch, xd, y);
         case 3: return launch_gemv_bpl<QT, 3>(ctx, n_out, k_in, qs, d, batch, xd, y);
-        case 4: return launch_gemv_bpl<QT, 4>(ctx, n_out, k_in, qs, d, batch, xd, y);
-        case 5: return launch_gemv_bpl<QT, 5>(ctx, n_out, k_in, qs, d, batch, xd, y);
-        case 6: return launch_gemv_bpl<QT, 6>(ctx, n_out, k_in, qs, d, batch, xd, y);
-        case 7: return launch_gemv_bpl<QT, 7>(ctx, n_out, k_in, qs, d, batch, xd, y);
-        default: return launch_gemv_bpl<QT, 8>(ctx, n_out, k_in, qs, d, batch, xd, y);
+        default: return launch_gemv_bpl<QT, 4>(ctx, n_out, k_in, qs, d, batch, xd, y);
     }
 }
 
@@ -391,8 +397,7 @@ pg_status launch_gemv(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs,
 
 size_t pg_xdigits_bytes(size_t rows, size_t k) {
     const size_t nb = k / 32;
-    return pg_round_up(3 * rows * k, 256) + pg_round_up(3 * rows * nb * sizeof(int), 256) +
-           pg_round_up(rows * sizeof(float), 256);
+    return pg_round_up(3 * rows * k, 256) + pg_round_up(rows * nb * sizeof(float), 256);
 }
 
 pg_xdigits pg_xdigits_carve(void *base, size_t rows, size_t k) {
@@ -401,9 +406,8 @@ pg_xdigits pg_xdigits_carve(void *base, size_t rows, size_t k) {
     char *p = static_cast<char *>(base);
     xd.digits = reinterpret_cast<int8_t *>(p);
     p += pg_round_up(3 * rows * k, 256);
-    xd.bsum = reinterpret_cast<int *>(p);
-    p += pg_round_up(3 * rows * nb * sizeof(int), 256);
     xd.xs = reinterpret_cast<float *>(p);
+    (void)nb;
     xd.rows = rows;
     xd.k = k;
     return xd;
@@ -412,9 +416,14 @@ pg_xdigits pg_xdigits_carve(void *base, size_t rows, size_t k) {
 pg_status pg_launch_x_to_digits(pg_ctx *ctx, const float *x_dev, size_t rows, size_t k,
                                 int ggml_type, const pg_xdigits &xd) {
     if (rows == 0) return PG_OK;
+    if (rows > 65535) return pg_fail(PG_EUNSUPPORTED, "x_to_digits: more than 65535 activation rows");
+    const int nb = (int)(k / 32);
     pg_prof_scope ps(ctx, "x_to_digits");
-    x_to_digits_kernel<<<(unsigned)rows, 256, 0, ctx->stream>>>(
-        x_dev, k, ggml_type == PG_GGML_Q4_0 ? 1 : 0, rows, xd.digits, xd.xs, xd.bsum);
+    const dim3 grid(grid_for(nb, 32), (unsigned)rows);
+    if (ggml_type == PG_GGML_Q4_0)
+        x_to_digits_kernel<true><<<grid, 256, 0, ctx->stream>>>(x_dev, nb, xd.digits, xd.xs);
+    else
+        x_to_digits_kernel<false><<<grid, 256, 0, ctx->stream>>>(x_dev, nb, xd.digits, xd.xs);
     return pg_launch_check("x_to_digits");
 }
 
@@ -422,6 +431,7 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
                               const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
                               const pg_xdigits &xd, float *y) {
     if (batch.count == 0) return PG_OK;
+    if (batch.count > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_gemv: more than 65535 batch items");
     if (ggml_type == PG_GGML_Q4_0) return launch_gemv<4>(ctx, n_out, k_in, qs, d, batch, xd, y);
     return launch_gemv<8>(ctx, n_out, k_in, qs, d, batch, xd, y);
 }
@@ -513,10 +523,10 @@ PG_API pg_status pg_gguf_upload(pg_ctx *ctx, const void *blocks, int ggml_type, 
     hipError_t e = hipSuccess;
     if (st == PG_OK) {
         e = hipMalloc((void **)&t->qs, nblocks * qb);
-        if (e == hipSuccess) e = hipMalloc((void **)&t->d, nblocks * sizeof(uint16_t));
+        if (e == hipSuccess) e = hipMalloc((void **)&t->d, (n_out + 7) / 8 * 8 * nb * sizeof(uint16_t));
         if (e == hipSuccess) e = hipMemcpyAsync(raw.p, blocks, nblocks * bb, hipMemcpyHostToDevice, ctx->stream);
         if (e == hipSuccess) {
-            split_blocks_kernel<<<grid_for(nblocks, 256), 256, 0, ctx->stream>>>(raw.as<uint8_t>(), n_out, nb,
+            split_blocks_kernel<<<grid_for((n_out + 7) / 8 * 8 * nb, 256), 256, 0, ctx->stream>>>(raw.as<uint8_t>(), n_out, nb,
                                                                                ggml_type, t->qs, t->d);
             e = hipGetLastError();
         }

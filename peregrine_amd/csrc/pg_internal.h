@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <string.h>
 #include <string>
+#include <type_traits>
 #include <vector>
 #include "peregrine_hip.h"
 
@@ -62,7 +63,7 @@ struct pg_qtensor {
 
 // GGUF block tensor split into planes at upload:
 //   qs     [n_out, k_in/32, QB] quant bytes (QB = 16 for Q4_0, 32 for Q8_0)
-//   d      [n_out, k_in/32]     f16 block scales
+//   d      [ceil(n_out/8), k_in/32, 8]  f16 block scales, tiled by 8 weight rows
 struct pg_gguf_tensor {
     uint8_t *qs;
     uint16_t *d;
@@ -128,11 +129,37 @@ pg_status pg_launch_gemv_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
                               float *out, int32_t *acc);
 // Activation rows rewritten as three byte-digit planes (see pg_gguf.hip).
 struct pg_xdigits {
-    int8_t *digits;  // [3][rows][k]
-    float *xs;       // [rows] power-of-two scale
-    int *bsum;       // [3][rows][k/32] per-block digit sums
+    int8_t *digits;  // [rows][6 planes][k/32 blocks][16 bytes] (Q4_0 uses 5 planes, Q8_0 all 6)
+    float *xs;       // [rows][k/32] power-of-two block scales
     size_t rows, k;
 };
+
+// Sum over the 64 lanes of a wavefront, returned in every lane (DPP within rows of 16
+// lanes, then the four row totals through scalar registers).
+__device__ __forceinline__ float pg_wave_sum_f32(float v) {
+    auto dpp_add = [](float x, auto ctrl) {
+        const int y = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, false);
+        return x + __builtin_bit_cast(float, y);
+    };
+    v = dpp_add(v, std::integral_constant<int, 0xB1>{});   // quad_perm [1,0,3,2]
+    v = dpp_add(v, std::integral_constant<int, 0x4E>{});   // quad_perm [2,3,0,1]
+    v = dpp_add(v, std::integral_constant<int, 0x141>{});  // row_half_mirror
+    v = dpp_add(v, std::integral_constant<int, 0x140>{});  // row_mirror
+    const int b = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16)) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+}
+
+__device__ __forceinline__ int pg_wave_sum_i32(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, false);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xf, 0xf, false);
+    return __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) +
+           __builtin_amdgcn_readlane(v, 32) + __builtin_amdgcn_readlane(v, 48);
+}
 size_t pg_xdigits_bytes(size_t rows, size_t k);
 pg_xdigits pg_xdigits_carve(void *base, size_t rows, size_t k);
 pg_status pg_launch_x_to_digits(pg_ctx *ctx, const float *x_dev, size_t rows, size_t k,

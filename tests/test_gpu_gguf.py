@@ -3,7 +3,8 @@
 Bars: f16 conversion and whole-tensor dequantisation are BIT-EXACT; the fused
 dequantise-matmul matches the oracle's dequantise -> transpose -> f32 matmul within
 1e-3 relative (H.assert_close_rel: relative to max(|ref|, rms(ref))); the tests also
-assert the much tighter 2e-5 the integer-digit kernel actually achieves.
+assert the tighter bound the fixed-point kernels actually achieve: 1e-4 for Q4_0
+(18-bit activation blocks) and 2e-5 for Q8_0 (22-bit), with x20 outlier channels present.
 """
 import sys
 
@@ -14,8 +15,8 @@ import helpers as H
 
 pytestmark = pytest.mark.gpu
 
-RTOL_CONTRACT = 1e-3   # BASELINE: Q4_0/Q8_0 block-dequant paths
-RTOL_ACHIEVED = 2e-5   # what this implementation is held to
+RTOL_CONTRACT = 1e-3                 # BASELINE: Q4_0/Q8_0 block-dequant paths
+RTOL_ACHIEVED = {2: 1e-4, 8: 2e-5}   # what this implementation is held to, per ggml type
 
 
 def say(msg):
@@ -108,7 +109,7 @@ def test_gguf_matmul_vs_oracle(ctx, orc, typ, n_out, k_in, m):
     for r in range(m):
         sl = slice(r * n_out, (r + 1) * n_out)
         H.assert_close_rel(got[sl], want[sl], RTOL_CONTRACT, f"row {r} (contract)")
-        H.assert_close_rel(got[sl], want[sl], RTOL_ACHIEVED, f"row {r} (achieved)")
+        H.assert_close_rel(got[sl], want[sl], RTOL_ACHIEVED[typ], f"row {r} (achieved)")
     gw.free()
 
 
@@ -125,10 +126,10 @@ def test_gguf_matmul_full_size_m16_and_linearity(ctx, orc):
     got = gw.matmul(x, m).reshape(m, n_out)
     want = orc.gguf_matmul(x, m, raw, 2, n_out, k_in).reshape(m, n_out)
     for r in range(m):
-        H.assert_close_rel(got[r], want[r], RTOL_ACHIEVED, f"row {r}")
+        H.assert_close_rel(got[r], want[r], RTOL_ACHIEVED[2], f"row {r}")
     xs = x.reshape(m, k_in)
     y12 = gw.matmul(xs[0] + xs[1], 1)
-    H.assert_close_rel(y12, got[0].astype(np.float64) + got[1], 1e-5, "linearity")
+    H.assert_close_rel(y12, got[0].astype(np.float64) + got[1], 1e-4, "linearity")
     gw.free()
 
 
@@ -140,9 +141,9 @@ def test_gguf_matmul_special_inputs(ctx, orc):
     gw = gguf.GgufWeight(raw, 2, n_out, k_in, ctx)
     assert (gw.matmul(np.zeros(k_in, np.float32), 1) == 0).all()           # zero row
     tiny = np.full(k_in, 1e-30, np.float32)
-    H.assert_close_rel(gw.matmul(tiny, 1), orc.gguf_matmul(tiny, 1, raw, 2, n_out, k_in), RTOL_ACHIEVED, "tiny")
+    H.assert_close_rel(gw.matmul(tiny, 1), orc.gguf_matmul(tiny, 1, raw, 2, n_out, k_in), RTOL_ACHIEVED[2], "tiny")
     big = orc.rng_normal(6, k_in) * np.float32(1e30)
-    H.assert_close_rel(gw.matmul(big, 1), orc.gguf_matmul(big, 1, raw, 2, n_out, k_in), RTOL_ACHIEVED, "huge")
+    H.assert_close_rel(gw.matmul(big, 1), orc.gguf_matmul(big, 1, raw, 2, n_out, k_in), RTOL_ACHIEVED[2], "huge")
     bad = np.ones(k_in, np.float32)
     bad[3] = np.nan
     assert np.isnan(gw.matmul(bad, 1)).all() and np.isnan(orc.gguf_matmul(bad, 1, raw, 2, n_out, k_in)).all()
