@@ -37,6 +37,20 @@ LAYER = [("q_proj", 4096, 4096), ("k_proj", 4096, 1024), ("v_proj", 4096, 1024),
 LAYER_OPS = sum(2 * M_PREFILL * k * n for _, k, n in LAYER)  # 893 353 197 568
 
 
+def load_traffic():
+    """profiles/hbm_traffic.json: per-kernel HBM bytes per launch derived from rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE runs of this benchmark, scaled by a plain copy of known size
+    (the file names the commands).  Absent file -> traffic is reported as null."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            return json.load(f).get("bytes_per_launch", {})
+    except (OSError, ValueError):
+        return {}
+
+
+TRAFFIC = load_traffic()
+
+
 def gemv_bytes(k, n):
     """Algorithmic bytes of one M = 1 W8A8 product: i8 weights + w scales + f32 x + f32 out."""
     return k * n + 4 * n + 4 * k + 4 * n
@@ -48,6 +62,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run plain 512 MiB device copies (counter calibration under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; every kernel here runs at its real "
@@ -101,10 +117,18 @@ def main():
         return e0.elapsed_time(e1) / steps  # ms per step
 
     def profiled(fn, steps):
+        """Per-kernel durations from the library's HIP events: each dispatch carries a start
+        and a stop event stamped with the kernel's own begin/end on the stream it runs on
+        (hipExtLaunchKernel), so the figures are comparable with a rocprofv3 kernel trace.
+        Returns {name: (avg_ms, launches)}."""
         ctx.profile_begin()
         for _ in range(steps):
             fn()
-        return ctx.profile_end()
+        return {name: (total / n, n) for name, (total, n) in ctx.profile_end().items()}
+
+    def traffic_for(kernel):
+        """HBM bytes per launch from the committed rocprofv3 --pmc measurement, or None."""
+        return TRAFFIC.get(kernel)
 
     # ------------------------------------------------------------------ prefill (headline)
     weights = {name: make_weight(k, n) for name, k, n in LAYER}
@@ -119,19 +143,20 @@ def main():
     ms_step = timed(prefill_step, args.steps, args.warmup)
     tops = LAYER_OPS / (ms_step * 1e-3) / 1e12
     prof = profiled(prefill_step, args.steps)
-    g_ms, g_n = prof["gemm_w8a8"]
-    q_ms, q_n = prof["quantize_rows"]
-    gemm_avg_ms = g_ms / g_n
+    gemm_avg_ms, g_n = prof["gemm_w8a8"]
+    q_avg_ms, q_n = prof["quantize_rows"]
     gemm_tops = (LAYER_OPS / len(LAYER)) / (gemm_avg_ms * 1e-3) / 1e12
     quant_bytes = sum(M_PREFILL * k * 4 + M_PREFILL * k + M_PREFILL * 4 for _, k, _ in LAYER)
     roofline = {"kernel": "gemm_w8a8_kernel (i8 MFMA 32x32x32, all 7 shapes)", "bound": "mfma",
                 "achieved": round(gemm_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
-                "frac": round(gemm_tops / PEAK_INT8_TOPS, 4), "traffic": None,
+                "frac": round(gemm_tops / PEAK_INT8_TOPS, 4), "traffic": traffic_for("gemm_w8a8"),
                 "ops_per_launch": LAYER_OPS // len(LAYER), "avg_launch_ms": round(gemm_avg_ms, 4),
-                "note": "unit counts int8 multiply-adds as 2 ops (TOP/s); duration from HIP events per launch"}
+                "note": "unit counts int8 multiply-adds as 2 ops (TOP/s); duration from the HIP events "
+                        "attached to each dispatch"}
     act_quant = {"kernel": "quantize_rows_vec4_kernel", "bound": "hbm",
-                 "achieved": round(quant_bytes / len(LAYER) / (q_ms / q_n * 1e-3) / 1e9, 1),
-                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "avg_launch_ms": round(q_ms / q_n, 4)}
+                 "achieved": round(quant_bytes / len(LAYER) / (q_avg_ms * 1e-3) / 1e9, 1),
+                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "avg_launch_ms": round(q_avg_ms, 4),
+                 "traffic": traffic_for("quantize_rows")}
     act_quant["frac"] = round(act_quant["achieved"] / PEAK_HBM_GBS, 4)
 
     # keep one set of device-quantised weights on the host for the CPU baseline, then free
@@ -168,8 +193,7 @@ def main():
     dsteps = max(args.steps * 10, 100)
     dec_ms = timed(decode_step, dsteps, max(args.warmup, 8))
     prof = profiled(decode_step, dsteps)
-    v_ms, v_n = prof["gemv_w8a8"]
-    gemv_avg_ms = v_ms / v_n
+    gemv_avg_ms, v_n = prof["gemv_w8a8"]
     gemv_gbs = (dec_bytes / 3) / (gemv_avg_ms * 1e-3) / 1e9
     decode = {"workload": "cfg2: M=1 int8 GEMV, x[4096]->gate,up[14336], x[14336]->down[4096]; "
                           f"{LAYERS_ROT} layers of weights rotated ({LAYERS_ROT * 3 * 58.7:.0f} MB, HBM-resident reads)",
@@ -177,7 +201,7 @@ def main():
               "ms_per_step": round(dec_ms, 5), "steps": dsteps, "bytes_per_step": dec_bytes,
               "roofline": {"kernel": "gemv_w8a8_kernel", "bound": "hbm", "achieved": round(gemv_gbs, 1),
                            "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gemv_gbs / PEAK_HBM_GBS, 4),
-                           "traffic": None, "bytes_per_launch": dec_bytes // 3,
+                           "traffic": traffic_for("gemv_w8a8"), "bytes_per_launch": dec_bytes // 3,
                            "avg_launch_ms": round(gemv_avg_ms, 5)}}
     for trio in dec_w:
         for h in trio:
@@ -205,15 +229,24 @@ def main():
     q4_bytes = n_out * (k_in // 32) * 18 + 4 * k_in + 4 * n_out  # 33 103 872
     q4_ms = timed(q4_step, dsteps, max(args.warmup, 8))
     prof = profiled(q4_step, dsteps)
-    k_ms, k_n = prof["gguf_gemv_q4_0"]
-    q4_gbs = q4_bytes / (k_ms / k_n * 1e-3) / 1e9
+    q4_avg_ms, k_n = prof["gguf_gemv_q4_0"]
+    q4_gbs = q4_bytes / (q4_avg_ms * 1e-3) / 1e9
     gguf = {"workload": f"cfg4: M=1 Q4_0 dequant-GEMV [4096]->[14336]; {Q4_ROT} tensors rotated (330 MB)",
             "value": round(q4_bytes / (q4_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "ms_per_step": round(q4_ms, 5),
             "roofline": {"kernel": "gguf_gemv_kernel<Q4_0>", "bound": "hbm", "achieved": round(q4_gbs, 1),
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(q4_gbs / PEAK_HBM_GBS, 4),
-                         "traffic": None, "bytes_per_launch": q4_bytes, "avg_launch_ms": round(k_ms / k_n, 5)}}
+                         "traffic": traffic_for("gguf_gemv_q4_0"), "bytes_per_launch": q4_bytes,
+                         "avg_launch_ms": round(q4_avg_ms, 5)}}
     for h in q4:
         lib.pg_gguf_free(ctx.handle, h)
+
+    if args.calibrate_copy:  # a plain copy of known size: 512 MiB read + 512 MiB written per launch
+        src = torch.empty(128 << 20, device=dev, dtype=torch.float32).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ------------------------------------------------------------------ CPU baseline (oracle)
     cpu = None

@@ -70,9 +70,10 @@ const char *pg_status_string(pg_status st);
 
 /* Per-kernel timing.  No counterpart in the reference (it times whole calls with
  * Instant::now(), benches/wallclock.rs:28-41): between pg_profile_begin and
- * pg_profile_end every kernel the library launches on this context is bracketed by
- * HIP events recorded on the context's stream; pg_profile_end waits for the stream
- * and aggregates elapsed time per kernel name, read back with pg_profile_get. */
+ * pg_profile_end every hot-path kernel the library launches on this context carries a
+ * start and a stop HIP event stamped with the dispatch's own begin and end times
+ * (hipExtLaunchKernel) on the context's stream; pg_profile_end waits for the stream and
+ * aggregates elapsed time per kernel name, read back with pg_profile_get. */
 pg_status pg_profile_begin(pg_ctx *ctx);
 pg_status pg_profile_end(pg_ctx *ctx, size_t *num_kernels);
 pg_status pg_profile_get(pg_ctx *ctx, size_t i, const char **name, double *total_ms,

@@ -27,7 +27,7 @@ class Context:
         _ffi.check(_ffi.lib.pg_sync(self.handle))
 
     def profile_begin(self):
-        """Start bracketing every kernel launch on this context with HIP events."""
+        """Start stamping every hot-path kernel launch on this context with HIP events."""
         _ffi.check(_ffi.lib.pg_profile_begin(self.handle))
 
     def profile_end(self):

@@ -167,7 +167,8 @@ PG_API pg_status pg_profile_end(pg_ctx *ctx, size_t *num_kernels) {
     ctx->totals.clear();
     for (auto &r : ctx->prof) {
         float ms = 0.0f;
-        if (hipEventElapsedTime(&ms, r.start, r.stop) != hipSuccess) continue;
+        const hipError_t ee = hipEventElapsedTime(&ms, r.start, r.stop);
+        if (ee != hipSuccess) { (void)pg_fail(PG_EDEVICE, "hipEventElapsedTime(%s): %s", r.name, hipGetErrorString(ee)); continue; }
         pg_prof_total *t = nullptr;
         for (auto &x : ctx->totals)
             if (x.name == r.name) t = &x;

@@ -231,12 +231,9 @@ pg_status launch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *
         attr_done = true;
     }
     const unsigned grid = (unsigned)(((ntiles + 7) / 8) * 8);
-    {
-        pg_prof_scope ps(ctx, "gemm_w8a8");
-        kern<<<grid, 64 * NWM * NWN, lds, ctx->stream>>>(a_i8, (int)a_stride, w->w_t, (int)w->k_pad, a_scales,
-                                                          w->scales, out, acc, (int)m, (int)w->cols,
-                                                          (int)w->k_pad, tiles_m, ntiles);
-    }
+    PG_TRY(pg_launch(ctx, "gemm_w8a8", kern, dim3(grid), dim3(64 * NWM * NWN), lds, a_i8, (int)a_stride, w->w_t,
+                     (int)w->k_pad, a_scales, w->scales, out, acc, (int)m, (int)w->cols, (int)w->k_pad, tiles_m,
+                     ntiles));
     return pg_launch_check("gemm_w8a8");
 }
 

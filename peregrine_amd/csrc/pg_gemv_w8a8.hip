@@ -127,11 +127,8 @@ template <int NCH, int RPW>
 pg_status launch_m1(pg_ctx *ctx, const int8_t *a_i8, const float *a_scales, const pg_qtensor *w,
                     float *out, int32_t *acc) {
     const unsigned grid = (unsigned)(w->n_pad / (4 * RPW));
-    {
-        pg_prof_scope ps(ctx, "gemv_w8a8");
-        gemv_w8a8_m1_kernel<NCH, RPW><<<grid, 256, 0, ctx->stream>>>(w->w_t, (int)w->k_pad, w->scales, a_i8,
-                                                                   a_scales, (int)w->cols, out, acc);
-    }
+    PG_TRY(pg_launch(ctx, "gemv_w8a8", gemv_w8a8_m1_kernel<NCH, RPW>, dim3(grid), dim3(256), 0, w->w_t,
+                     (int)w->k_pad, w->scales, a_i8, a_scales, (int)w->cols, out, acc));
     return pg_launch_check("gemv_w8a8_m1");
 }
 
@@ -153,11 +150,8 @@ pg_status launch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *
         if (e != hipSuccess) return pg_fail(PG_EDEVICE, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     }
     const unsigned grid = (unsigned)(w->n_pad / (4 * R));
-    {
-        pg_prof_scope ps(ctx, "gemv_w8a8");
-        gemv_w8a8_kernel<R, M><<<grid, 256, lds, ctx->stream>>>(w->w_t, (int)w->k_pad, w->scales, a_i8,
-                                                              (int)a_stride, a_scales, (int)w->cols, out, acc);
-    }
+    PG_TRY(pg_launch(ctx, "gemv_w8a8", gemv_w8a8_kernel<R, M>, dim3(grid), dim3(256), lds, w->w_t, (int)w->k_pad,
+                     w->scales, a_i8, (int)a_stride, a_scales, (int)w->cols, out, acc));
     return pg_launch_check("gemv_w8a8");
 }
 

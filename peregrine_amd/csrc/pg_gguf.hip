@@ -364,19 +364,19 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
     // rows in flight per wavefront: bounded by registers (16 B of weights per row and block)
     constexpr int NH = QT == 8 ? 2 : 1;
     constexpr int R8 = BPL * NH <= 2 ? 8 : (BPL * NH <= 4 ? 4 : 2);
-    pg_prof_scope ps(ctx, QT == 4 ? "gguf_gemv_q4_0" : "gguf_gemv_q8_0");
     const size_t want = (size_t)ctx->num_cu * 6;  // wavefronts wanted in the grid
 #define PG_GGUF_GEMV_LAUNCH(RWW, RR)                                                               \
     do {                                                                                           \
         const dim3 grid(grid_for(n_out, RWW), (unsigned)batch.count);                              \
-        gguf_gemv_kernel<QT, BPL, RWW, RR><<<grid, 64, 0, ctx->stream>>>(                          \
-            qs, d, batch, (int)n_out, nb, xd.digits, xd.xs, y);                           \
+        PG_TRY(pg_launch(ctx, QT == 4 ? "gguf_gemv_q4_0" : "gguf_gemv_q8_0",                       \
+                         gguf_gemv_kernel<QT, BPL, RWW, RR>, grid, dim3(64), 0, qs, d, batch,      \
+                         (int)n_out, nb, xd.digits, xd.xs, y));                                    \
     } while (0)
     if (n_out / 8 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(8, R8);
     else if (n_out / 4 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(4, (R8 < 4 ? R8 : 4));
     else PG_GGUF_GEMV_LAUNCH(2, 2);
 #undef PG_GGUF_GEMV_LAUNCH
-    return pg_launch_check("gguf_gemv");
+    return PG_OK;
 }
 
 template <int QT>
@@ -418,12 +418,11 @@ pg_status pg_launch_x_to_digits(pg_ctx *ctx, const float *x_dev, size_t rows, si
     if (rows == 0) return PG_OK;
     if (rows > 65535) return pg_fail(PG_EUNSUPPORTED, "x_to_digits: more than 65535 activation rows");
     const int nb = (int)(k / 32);
-    pg_prof_scope ps(ctx, "x_to_digits");
     const dim3 grid(grid_for(nb, 32), (unsigned)rows);
     if (ggml_type == PG_GGML_Q4_0)
-        x_to_digits_kernel<true><<<grid, 256, 0, ctx->stream>>>(x_dev, nb, xd.digits, xd.xs);
+        PG_TRY(pg_launch(ctx, "x_to_digits", x_to_digits_kernel<true>, grid, dim3(256), 0, x_dev, nb, xd.digits, xd.xs));
     else
-        x_to_digits_kernel<false><<<grid, 256, 0, ctx->stream>>>(x_dev, nb, xd.digits, xd.xs);
+        PG_TRY(pg_launch(ctx, "x_to_digits", x_to_digits_kernel<false>, grid, dim3(256), 0, x_dev, nb, xd.digits, xd.xs));
     return pg_launch_check("x_to_digits");
 }
 

@@ -1,11 +1,14 @@
 // Internal definitions shared by the HIP translation units of libperegrine_hip.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stddef.h>
 #include <stdint.h>
 #include <string.h>
 #include <string>
+#include <tuple>
 #include <type_traits>
+#include <utility>
 #include <vector>
 #include "peregrine_hip.h"
 
@@ -32,23 +35,6 @@ struct pg_ctx {
     bool profiling;                     // per-kernel HIP events (pg_profile_begin/end)
     std::vector<pg_prof_rec> prof;      // one record per launch while profiling
     std::vector<pg_prof_total> totals;  // aggregated by pg_profile_end
-};
-
-// Brackets one kernel launch with HIP events on the context's stream while profiling.
-struct pg_prof_scope {
-    pg_ctx *ctx;
-    hipEvent_t stop = nullptr;
-    pg_prof_scope(pg_ctx *c, const char *name) : ctx(c) {
-        if (!c->profiling) return;
-        hipEvent_t start = nullptr;
-        if (hipEventCreate(&start) != hipSuccess) return;
-        if (hipEventCreate(&stop) != hipSuccess) { (void)hipEventDestroy(start); stop = nullptr; return; }
-        (void)hipEventRecord(start, c->stream);
-        c->prof.push_back({name, start, stop});
-    }
-    ~pg_prof_scope() {
-        if (stop) (void)hipEventRecord(stop, ctx->stream);
-    }
 };
 
 // Device-resident quantised weight, K-contiguous and zero-padded:
@@ -105,6 +91,33 @@ pg_status pg_use(pg_ctx *ctx);
 pg_status pg_workspace(pg_ctx *ctx, size_t bytes, void **out);
 // Check the launch just made.
 pg_status pg_launch_check(const char *what);
+
+// Launch `kernel` on the context's stream.  While profiling (pg_profile_begin/end) the
+// dispatch carries a start and a stop event: hipExtLaunchKernel stamps them with the
+// kernel's own begin and end times (what a kernel trace reports), not with the time the
+// stream reaches a separately recorded event.
+template <typename... KArgs, size_t... I>
+inline void pg_arg_ptrs(std::tuple<KArgs...> &t, void **out, std::index_sequence<I...>) {
+    ((out[I] = static_cast<void *>(&std::get<I>(t))), ...);
+}
+template <typename... KArgs, typename... Args>
+inline pg_status pg_launch(pg_ctx *ctx, const char *name, void (*kernel)(KArgs...), dim3 grid, dim3 block,
+                           size_t lds, Args &&...args) {
+    static_assert(sizeof...(KArgs) == sizeof...(Args), "argument count differs from the kernel's");
+    hipEvent_t start = nullptr, stop = nullptr;
+    if (ctx->profiling) {
+        if (hipEventCreate(&start) != hipSuccess) start = nullptr;
+        if (start && hipEventCreate(&stop) != hipSuccess) { (void)hipEventDestroy(start); start = stop = nullptr; }
+        if (start) ctx->prof.push_back({name, start, stop});
+    }
+    std::tuple<KArgs...> tup{static_cast<KArgs>(args)...};
+    void *ptrs[sizeof...(KArgs) ? sizeof...(KArgs) : 1];
+    pg_arg_ptrs(tup, ptrs, std::index_sequence_for<KArgs...>{});
+    const hipError_t e = hipExtLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, ptrs, lds,
+                                            ctx->stream, start, stop, 0);
+    if (e != hipSuccess) return pg_fail(PG_EDEVICE, "launch of %s failed: %s", name, hipGetErrorString(e));
+    return PG_OK;
+}
 
 // RAII device temporary for the host-pointer entry points.
 struct pg_tmp {

@@ -132,10 +132,8 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     // host_tab lives on this stack frame: the copy must have left it before we return.
     PG_HIP(hipStreamSynchronize(ctx->stream));
 
-    { pg_prof_scope ps(ctx, "moe_route_topk");
-    route_topk_kernel<<<grid_for(T, 64), 64, 0, ctx->stream>>>(router_logits_dev, (int)T, (int)E, (int)top_k,
-                                                             topk_idx, topk_p); }
-    PG_TRY(pg_launch_check("route_topk"));
+    PG_TRY(pg_launch(ctx, "moe_route_topk", route_topk_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
+                     router_logits_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
     PG_TRY(pg_launch_x_to_digits(ctx, x_dev, T, d, type, xd));
     auto table = [&](int which) { return reinterpret_cast<const uint8_t *const *>(tab + which * E); };
     auto dtable = [&](int which) { return reinterpret_cast<const uint16_t *const *>(tab + which * E); };
@@ -143,15 +141,13 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     PG_TRY(pg_launch_gguf_gemv(ctx, type, ffn, d, nullptr, nullptr, bg, xd, g));
     pg_gemv_batch bu = {(int)P, table(2), dtable(3), topk_idx, (int)top_k};
     PG_TRY(pg_launch_gguf_gemv(ctx, type, ffn, d, nullptr, nullptr, bu, xd, u));
-    { pg_prof_scope ps(ctx, "moe_act_mul");
-    act_mul_kernel<<<grid_for(P * ffn, 256), 256, 0, ctx->stream>>>(g, u, P * ffn, act, h); }
-    PG_TRY(pg_launch_check("act_mul"));
+    PG_TRY(pg_launch(ctx, "moe_act_mul", act_mul_kernel, dim3(grid_for(P * ffn, 256)), dim3(256), 0, g, u, P * ffn,
+                     act, h));
     PG_TRY(pg_launch_x_to_digits(ctx, h, P, ffn, type, hd));
     pg_gemv_batch bd = {(int)P, table(4), dtable(5), topk_idx, 1};
     PG_TRY(pg_launch_gguf_gemv(ctx, type, d, ffn, nullptr, nullptr, bd, hd, yb));
-    { pg_prof_scope ps(ctx, "moe_combine");
-    combine_kernel<<<grid_for(T * d, 256), 256, 0, ctx->stream>>>(yb, topk_p, (int)T, (int)d, (int)top_k, out_dev); }
-    return pg_launch_check("moe_combine");
+    return pg_launch(ctx, "moe_combine", combine_kernel, dim3(grid_for(T * d, 256)), dim3(256), 0, yb, topk_p, (int)T,
+                     (int)d, (int)top_k, out_dev);
 }
 
 PG_API pg_status pg_moe_ffn(pg_ctx *ctx, const float *x, size_t T, const float *router_logits,

@@ -245,13 +245,15 @@ pg_status pg_launch_quantize_activations(pg_ctx *ctx, const float *a, size_t row
                         ((uintptr_t)a % 16 == 0) && ((uintptr_t)q % 4 == 0) && cols > 0;
     const size_t nvec = cols / 4;
     const dim3 grid((unsigned)rows);
-    pg_prof_scope ps(ctx, "quantize_rows");
     if (vec_ok && nvec <= 4 * QA_THREADS)
-        quantize_rows_vec4_kernel<4><<<grid, QA_THREADS, 0, ctx->stream>>>(a, cols, q, q_stride, row_scales);
+        PG_TRY(pg_launch(ctx, "quantize_rows", quantize_rows_vec4_kernel<4>, grid, dim3(QA_THREADS), 0, a, cols, q,
+                         q_stride, row_scales));
     else if (vec_ok && nvec <= 16 * QA_THREADS)
-        quantize_rows_vec4_kernel<16><<<grid, QA_THREADS, 0, ctx->stream>>>(a, cols, q, q_stride, row_scales);
+        PG_TRY(pg_launch(ctx, "quantize_rows", quantize_rows_vec4_kernel<16>, grid, dim3(QA_THREADS), 0, a, cols, q,
+                         q_stride, row_scales));
     else
-        quantize_rows_generic_kernel<<<grid, QA_THREADS, 0, ctx->stream>>>(a, cols, q, q_stride, row_scales);
+        PG_TRY(pg_launch(ctx, "quantize_rows", quantize_rows_generic_kernel, grid, dim3(QA_THREADS), 0, a, cols, q,
+                         q_stride, row_scales));
     return pg_launch_check("quantize_rows");
 }
 
