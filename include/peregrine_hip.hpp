@@ -1,0 +1,248 @@
+// peregrine_hip.hpp -- C++ host-side mirror of peregrine's quantized-inference API
+// on top of the C ABI in peregrine_hip.h.
+//
+// Names, argument order and meaning follow the reference's Rust surface:
+//   peregrine::quant::{QuantizedTensor, quantize_weights, quantize_activations,
+//                      dequantize, matmul_quantized, matmul_quantized_gpu}   src/quant.rs:12-218
+//   peregrine::gguf::{f16_to_f32, dequant_q8_0, dequant_q4_0, dequant_q4_1,
+//                     load_tensor_q8_as_quantized}                           src/gguf.rs:286-401
+// The reference panics (assert!/expect) on shape mismatch; here the same
+// conditions throw peregrine::Panic carrying the library's message.  Outputs
+// are freshly allocated vectors owned by the caller, like the reference's Vec.
+// Header-only; link with -lperegrine_hip.
+#ifndef PEREGRINE_HIP_HPP
+#define PEREGRINE_HIP_HPP
+
+#include <cstdint>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "peregrine_hip.h"
+
+namespace peregrine {
+
+// Stands in for a Rust panic crossing the API.
+struct Panic : std::runtime_error {
+    pg_status status;
+    Panic(pg_status st, const std::string &what) : std::runtime_error(what), status(st) {}
+};
+
+inline void check(pg_status st, const char *what) {
+    if (st != PG_OK)
+        throw Panic(st, std::string(what) + ": " + pg_status_string(st) + ": " + pg_last_error());
+}
+
+// GpuContext (src/metal/context.rs:2472-2510): one device, one stream.
+class GpuContext {
+public:
+    explicit GpuContext(int device = 0, void *hip_stream = nullptr) {
+        check(pg_ctx_create(device, hip_stream, &ctx_), "GpuContext::new");
+    }
+    ~GpuContext() { pg_ctx_destroy(ctx_); }
+    GpuContext(const GpuContext &) = delete;
+    GpuContext &operator=(const GpuContext &) = delete;
+    void sync() const { check(pg_sync(ctx_), "GpuContext::sync"); }
+    pg_ctx *raw() const { return ctx_; }
+
+private:
+    pg_ctx *ctx_ = nullptr;
+};
+
+// GpuBuffer<T> (src/metal/buffer.rs): device memory owned by the object.
+template <typename T>
+class GpuBuffer {
+public:
+    GpuBuffer(const GpuContext &gpu, size_t len) : gpu_(&gpu), len_(len) {
+        check(pg_dev_alloc(gpu.raw(), len * sizeof(T), &ptr_), "GpuBuffer::alloc");
+    }
+    ~GpuBuffer() { if (ptr_) pg_dev_free(gpu_->raw(), ptr_); }
+    GpuBuffer(GpuBuffer &&o) noexcept : gpu_(o.gpu_), ptr_(o.ptr_), len_(o.len_) { o.ptr_ = nullptr; }
+    GpuBuffer(const GpuBuffer &) = delete;
+    GpuBuffer &operator=(const GpuBuffer &) = delete;
+    size_t len() const { return len_; }
+    T *device_ptr() const { return static_cast<T *>(ptr_); }
+    void upload(const T *src) { check(pg_memcpy_h2d(gpu_->raw(), ptr_, src, len_ * sizeof(T)), "GpuBuffer::upload"); }
+    // GpuBuffer::read: the caller syncs first (tests/quant_parity.rs:102-107); the copy itself is synchronous.
+    std::vector<T> read() const {
+        std::vector<T> out(len_);
+        check(pg_memcpy_d2h(gpu_->raw(), out.data(), ptr_, len_ * sizeof(T)), "GpuBuffer::read");
+        return out;
+    }
+
+private:
+    const GpuContext *gpu_;
+    void *ptr_ = nullptr;
+    size_t len_;
+};
+
+namespace quant {
+
+// quant::QuantizedTensor  src/quant.rs:12-23
+struct QuantizedTensor {
+    std::vector<int8_t> data_i8;    // [rows, cols] row-major
+    std::vector<int8_t> data_i8_t;  // [cols, rows]
+    std::vector<float> scales;      // [cols]
+    size_t rows = 0, cols = 0;
+
+    // QuantizedTensor::to_gpu  src/quant.rs:174-181 (idempotent)
+    void to_gpu(const GpuContext &gpu) {
+        if (gpu_) return;
+        pg_qtensor *h = nullptr;
+        check(pg_qtensor_upload(gpu.raw(), data_i8.data(), scales.data(), rows, cols, &h), "QuantizedTensor::to_gpu");
+        pg_ctx *c = gpu.raw();
+        gpu_ = std::shared_ptr<pg_qtensor>(h, [c](pg_qtensor *t) { pg_qtensor_free(c, t); });
+    }
+    // QuantizedTensor::from_gpu  src/quant.rs:183-190
+    void from_gpu(const GpuContext &gpu) {
+        if (!gpu_) return;
+        check(pg_qtensor_download(gpu.raw(), gpu_.get(), data_i8.data(), data_i8_t.data(), scales.data()),
+              "QuantizedTensor::from_gpu");
+    }
+    bool on_gpu() const { return (bool)gpu_; }
+    const pg_qtensor *gpu_handle() const { return gpu_.get(); }
+
+private:
+    std::shared_ptr<pg_qtensor> gpu_;
+};
+
+// quant::quantize_weights  src/quant.rs:27-75
+inline QuantizedTensor quantize_weights(const GpuContext &gpu, const std::vector<float> &data, size_t rows, size_t cols) {
+    if (data.size() != rows * cols) throw Panic(PG_EINVAL, "quantize_weights: data.len() != rows * cols");
+    QuantizedTensor qt;
+    qt.rows = rows; qt.cols = cols;
+    qt.data_i8.resize(rows * cols); qt.data_i8_t.resize(rows * cols); qt.scales.resize(cols);
+    check(pg_quantize_weights(gpu.raw(), data.data(), rows, cols, qt.data_i8.data(), qt.data_i8_t.data(), qt.scales.data()),
+          "quantize_weights");
+    return qt;
+}
+
+// quant::quantize_activations  src/quant.rs:79-112
+inline std::pair<std::vector<int8_t>, std::vector<float>> quantize_activations(const GpuContext &gpu, const std::vector<float> &data,
+                                                                                size_t rows, size_t cols) {
+    if (data.size() != rows * cols) throw Panic(PG_EINVAL, "quantize_activations: data.len() != rows * cols");
+    std::vector<int8_t> q(rows * cols);
+    std::vector<float> s(rows);
+    check(pg_quantize_activations(gpu.raw(), data.data(), rows, cols, q.data(), s.data()), "quantize_activations");
+    return {std::move(q), std::move(s)};
+}
+
+// quant::dequantize  src/quant.rs:115-123
+inline std::vector<float> dequantize(const GpuContext &gpu, const QuantizedTensor &qt) {
+    std::vector<float> out(qt.rows * qt.cols);
+    check(pg_dequantize(gpu.raw(), qt.data_i8.data(), qt.scales.data(), qt.rows, qt.cols, out.data()), "dequantize");
+    return out;
+}
+
+// quant::matmul_quantized  src/quant.rs:129-169.  The reference computes this on the CPU; here the
+// weights are uploaded on first use and the product runs on the device with identical results.
+inline std::vector<float> matmul_quantized(const GpuContext &gpu, const std::vector<float> &a, size_t m, size_t k, QuantizedTensor &w) {
+    if (w.rows != k) throw Panic(PG_EINVAL, "matmul_quantized: weight rows must equal k");
+    if (a.size() != m * k) throw Panic(PG_EINVAL, "matmul_quantized: a.len() != m * k");
+    w.to_gpu(gpu);
+    std::vector<float> out(m * w.cols);
+    check(pg_matmul_quantized(gpu.raw(), a.data(), m, k, w.gpu_handle(), out.data()), "matmul_quantized");
+    return out;
+}
+
+// quant::matmul_quantized_gpu  src/quant.rs:196-218: uploads a, returns an UNSYNCED device buffer.
+inline GpuBuffer<float> matmul_quantized_gpu(const GpuContext &gpu, const std::vector<float> &a, size_t m, size_t k,
+                                             const QuantizedTensor &w) {
+    if (w.rows != k) throw Panic(PG_EINVAL, "matmul_quantized_gpu: weight rows must equal k");
+    if (a.size() != m * k) throw Panic(PG_EINVAL, "matmul_quantized_gpu: a.len() != m * k");
+    if (!w.on_gpu()) throw Panic(PG_EINVAL, "weights not on GPU");  // .expect() at src/quant.rs:208-209
+    GpuBuffer<float> a_buf(gpu, m * k), out(gpu, m * w.cols);
+    a_buf.upload(a.data());
+    check(pg_matmul_quantized_dev(gpu.raw(), a_buf.device_ptr(), m, k, w.gpu_handle(), out.device_ptr(), nullptr),
+          "matmul_quantized_gpu");
+    gpu.sync();  // a_buf is released on return; the product must have consumed it
+    return out;
+}
+
+}  // namespace quant
+
+namespace gguf {
+
+// GGML block sizes  src/gguf.rs:47-55
+constexpr size_t Q8_0_BLOCK_BYTES = 34, Q4_0_BLOCK_BYTES = 18, Q4_1_BLOCK_BYTES = 20, BLOCK_ELEMS = 32;
+
+// gguf::f16_to_f32  src/gguf.rs:354-382
+inline float f16_to_f32(const GpuContext &gpu, uint16_t bits) {
+    float out;
+    check(pg_f16_to_f32(gpu.raw(), &bits, 1, &out), "f16_to_f32");
+    return out;
+}
+
+#define PEREGRINE_DEQUANT(name, bytes)                                                                        \
+    inline std::vector<float> name(const GpuContext &gpu, const std::vector<uint8_t> &data, size_t n) {      \
+        if (n % BLOCK_ELEMS != 0) throw Panic(PG_EINVAL, #name ": num_elements must be a multiple of 32");   \
+        if (data.size() < n / BLOCK_ELEMS * (bytes)) throw Panic(PG_EINVAL, #name ": data too short");       \
+        std::vector<float> out(n);                                                                            \
+        check(pg_##name(gpu.raw(), data.data(), n, out.data()), #name);                                       \
+        return out;                                                                                           \
+    }
+PEREGRINE_DEQUANT(dequant_q8_0, Q8_0_BLOCK_BYTES)  // src/gguf.rs:286-302
+PEREGRINE_DEQUANT(dequant_q4_0, Q4_0_BLOCK_BYTES)  // src/gguf.rs:307-326
+PEREGRINE_DEQUANT(dequant_q4_1, Q4_1_BLOCK_BYTES)  // src/gguf.rs:331-351
+#undef PEREGRINE_DEQUANT
+
+// gguf::load_tensor_q8_as_quantized  src/gguf.rs:386-401: Q8_0 -> f32 -> quantize_weights.
+inline quant::QuantizedTensor load_tensor_q8_as_quantized(const GpuContext &gpu, const std::vector<uint8_t> &data, size_t rows,
+                                                          size_t cols) {
+    return quant::quantize_weights(gpu, dequant_q8_0(gpu, data, rows * cols), rows, cols);
+}
+
+// A GGUF weight kept block-quantised on the device; matmul() is the fused form of
+// dequantise + transpose + Tensor::matmul (src/models/llama/model.rs:243-257, src/tensor.rs:1342-1353).
+class BlockWeight {
+public:
+    BlockWeight(const GpuContext &gpu, const std::vector<uint8_t> &blocks, int ggml_type, size_t n_out, size_t k_in) : gpu_(&gpu) {
+        check(pg_gguf_upload(gpu.raw(), blocks.data(), ggml_type, n_out, k_in, &h_), "BlockWeight::upload");
+        n_out_ = n_out; k_in_ = k_in;
+    }
+    ~BlockWeight() { if (h_) pg_gguf_free(gpu_->raw(), h_); }
+    BlockWeight(const BlockWeight &) = delete;
+    BlockWeight &operator=(const BlockWeight &) = delete;
+    std::vector<float> matmul(const std::vector<float> &x, size_t m) const {
+        if (x.size() != m * k_in_) throw Panic(PG_EINVAL, "BlockWeight::matmul: x.len() != m * k_in");
+        std::vector<float> y(m * n_out_);
+        check(pg_gguf_matmul(gpu_->raw(), x.data(), m, h_, y.data()), "BlockWeight::matmul");
+        return y;
+    }
+    const pg_gguf_tensor *handle() const { return h_; }
+    size_t n_out() const { return n_out_; }
+    size_t k_in() const { return k_in_; }
+
+private:
+    const GpuContext *gpu_;
+    pg_gguf_tensor *h_ = nullptr;
+    size_t n_out_ = 0, k_in_ = 0;
+};
+
+}  // namespace gguf
+
+namespace moe {
+
+// MoELayer::forward after the router matmul  examples/grok1/moe.rs:70-109.
+inline std::vector<float> expert_ffn(const GpuContext &gpu, const std::vector<float> &x, size_t tokens,
+                                     const std::vector<float> &router_logits, size_t top_k,
+                                     const std::vector<const gguf::BlockWeight *> &gate,
+                                     const std::vector<const gguf::BlockWeight *> &up,
+                                     const std::vector<const gguf::BlockWeight *> &down, int act) {
+    const size_t E = gate.size();
+    if (E == 0 || up.size() != E || down.size() != E) throw Panic(PG_EINVAL, "expert_ffn: expert tables differ in length");
+    std::vector<const pg_gguf_tensor *> g(E), u(E), d(E);
+    for (size_t e = 0; e < E; ++e) { g[e] = gate[e]->handle(); u[e] = up[e]->handle(); d[e] = down[e]->handle(); }
+    const size_t dm = gate[0]->k_in();
+    if (x.size() != tokens * dm || router_logits.size() != tokens * E) throw Panic(PG_EINVAL, "expert_ffn: input sizes");
+    std::vector<float> out(tokens * dm);
+    check(pg_moe_ffn(gpu.raw(), x.data(), tokens, router_logits.data(), E, top_k, g.data(), u.data(), d.data(), act, out.data()),
+          "expert_ffn");
+    return out;
+}
+
+}  // namespace moe
+}  // namespace peregrine
+#endif  // PEREGRINE_HIP_HPP

@@ -1,0 +1,206 @@
+// C++ parity program for the host mirror (include/peregrine_hip.hpp).
+// The cases follow the reference's own tests: tests/quant_parity.rs:6-77,149-173,
+// src/quant.rs:225-291, tests/gguf_parity.rs:7-76, src/gguf.rs:574-631, and then
+// tighten them: where the reference only bounds the error, the device result is
+// compared bit-for-bit with the CPU oracle (which is test infrastructure only).
+// Needs a GPU; prints one line per case and exits non-zero on the first failure.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "peregrine_hip.hpp"
+
+extern "C" {
+void orc_quantize_weights(const float *, size_t, size_t, int8_t *, int8_t *, float *);
+void orc_quantize_activations(const float *, size_t, size_t, int8_t *, float *);
+int orc_matmul_quantized(const float *, size_t, size_t, const int8_t *, const float *, size_t, float *, int32_t *);
+int orc_gguf_matmul(const float *, size_t, const uint8_t *, int, size_t, size_t, float *);
+}
+
+using namespace peregrine;
+
+static int failures = 0;
+#define EXPECT(cond, ...)                                     \
+    do {                                                      \
+        if (!(cond)) {                                        \
+            std::printf("  FAIL %s:%d: ", __FILE__, __LINE__); \
+            std::printf(__VA_ARGS__);                         \
+            std::printf("\n");                                \
+            ++failures;                                       \
+        }                                                     \
+    } while (0)
+
+static bool same_bits(const std::vector<float> &a, const std::vector<float> &b) {
+    return a.size() == b.size() && std::memcmp(a.data(), b.data(), a.size() * sizeof(float)) == 0;
+}
+
+// tests/quant_parity.rs:6-32
+static void test_quantize_dequantize_roundtrip(const GpuContext &gpu) {
+    std::printf("test_quantize_dequantize_roundtrip\n");
+    const size_t rows = 64, cols = 128;
+    std::vector<float> data(rows * cols);
+    for (size_t i = 0; i < data.size(); ++i) data[i] = (float)((i * 17 + 5) % 400) / 100.0f - 2.0f;
+    auto qt = quant::quantize_weights(gpu, data, rows, cols);
+    auto recovered = quant::dequantize(gpu, qt);
+    EXPECT(recovered.size() == data.size(), "length");
+    for (size_t i = 0; i < data.size(); ++i) {
+        const float scale = qt.scales[i % cols];
+        EXPECT(std::fabs(data[i] - recovered[i]) <= scale + 1e-7f, "element %zu: %g vs %g (scale %g)", i, data[i], recovered[i], scale);
+    }
+    // beyond the reference's bound: integers, transpose and scales equal the CPU path's exactly
+    std::vector<int8_t> q(rows * cols), qt_t(rows * cols);
+    std::vector<float> sc(cols);
+    orc_quantize_weights(data.data(), rows, cols, q.data(), qt_t.data(), sc.data());
+    EXPECT(q == qt.data_i8, "data_i8 differs from the CPU path");
+    EXPECT(qt_t == qt.data_i8_t, "data_i8_t differs from the CPU path");
+    EXPECT(same_bits(sc, qt.scales), "scales differ from the CPU path");
+}
+
+// tests/quant_parity.rs:35-77 and src/quant.rs:252-291
+static void test_quantized_matmul_accuracy(const GpuContext &gpu, size_t m, size_t k, size_t n, int mod) {
+    std::printf("test_quantized_matmul_accuracy m=%zu k=%zu n=%zu\n", m, k, n);
+    std::vector<float> a(m * k), w(k * n);
+    for (size_t i = 0; i < a.size(); ++i) a[i] = (float)((i * 7 + 3) % mod) / (float)mod - 0.5f;
+    for (size_t i = 0; i < w.size(); ++i) w[i] = (float)((i * 13 + 7) % mod) / (float)mod - 0.5f;
+    auto qt = quant::quantize_weights(gpu, w, k, n);
+    auto out = quant::matmul_quantized(gpu, a, m, k, qt);
+    // the reference's own check: against the f32 product, loose tolerance
+    for (size_t i = 0; i < m; ++i)
+        for (size_t j = 0; j < n; ++j) {
+            float ref = 0.0f;
+            for (size_t p = 0; p < k; ++p) ref += a[i * k + p] * w[p * n + j];
+            const float diff = std::fabs(out[i * n + j] - ref);
+            EXPECT(diff / std::fmax(std::fabs(ref), 1e-6f) < 0.15f || diff < 0.05f, "(%zu,%zu): %g vs f32 %g", i, j, out[i * n + j], ref);
+        }
+    // and bit-for-bit against the CPU path
+    std::vector<float> cpu(m * n);
+    orc_matmul_quantized(a.data(), m, k, qt.data_i8_t.data(), qt.scales.data(), n, cpu.data(), nullptr);
+    EXPECT(same_bits(cpu, out), "matmul_quantized differs from the CPU path");
+    // GPU entry point: unsynced buffer, sync, read  (tests/quant_parity.rs:95-107)
+    auto buf = quant::matmul_quantized_gpu(gpu, a, m, k, qt);
+    gpu.sync();
+    EXPECT(same_bits(cpu, buf.read()), "matmul_quantized_gpu differs from the CPU path");
+}
+
+// quantize_activations: closed forms and CPU-path equality
+static void test_quantize_activations(const GpuContext &gpu) {
+    std::printf("test_quantize_activations\n");
+    const size_t rows = 5, cols = 96;
+    std::vector<float> x(rows * cols);
+    for (size_t i = 0; i < x.size(); ++i) x[i] = std::sin(0.37f * (float)i) * (float)(1 + i % 7);
+    for (size_t c = 0; c < cols; ++c) { x[1 * cols + c] = 0.0f; x[2 * cols + c] = (c % 2) ? 3.5f : -3.5f; }
+    auto [q, s] = quant::quantize_activations(gpu, x, rows, cols);
+    EXPECT(s[1] == 1.0f, "zero row must get scale 1.0, got %g", s[1]);
+    EXPECT(s[2] == 3.5f / 127.0f, "constant row scale");
+    for (size_t c = 0; c < cols; ++c) {
+        EXPECT(q[1 * cols + c] == 0, "zero row");
+        EXPECT(q[2 * cols + c] == ((c % 2) ? 127 : -127), "constant row -> +-127");
+    }
+    std::vector<int8_t> cq(rows * cols);
+    std::vector<float> cs(rows);
+    orc_quantize_activations(x.data(), rows, cols, cq.data(), cs.data());
+    EXPECT(cq == q, "integers differ from the CPU path");
+    EXPECT(same_bits(cs, s), "row scales differ from the CPU path");
+}
+
+// the reference panics on shape mismatch (src/quant.rs:28,80,135,137,208)
+static void test_shape_panics(const GpuContext &gpu) {
+    std::printf("test_shape_panics\n");
+    std::vector<float> w(8 * 4, 0.5f), a(3 * 7, 1.0f);
+    auto qt = quant::quantize_weights(gpu, w, 8, 4);
+    bool threw = false;
+    try { quant::matmul_quantized(gpu, a, 3, 7, qt); } catch (const Panic &) { threw = true; }
+    EXPECT(threw, "k != weight rows must panic");
+    threw = false;
+    try { quant::quantize_weights(gpu, w, 8, 5); } catch (const Panic &) { threw = true; }
+    EXPECT(threw, "data.len() != rows*cols must panic");
+    threw = false;
+    quant::QuantizedTensor cold = qt;  // copy shares no upload unless to_gpu ran
+    try { if (!cold.on_gpu()) quant::matmul_quantized_gpu(gpu, std::vector<float>(3 * 8, 1.0f), 3, 8, cold); } catch (const Panic &) { threw = true; }
+    EXPECT(threw || cold.on_gpu(), "weights not on GPU must panic");
+}
+
+// src/gguf.rs:574-631, tests/gguf_parity.rs:7-76
+static void test_gguf_known_answers(const GpuContext &gpu) {
+    std::printf("test_gguf_known_answers\n");
+    const uint16_t bits[] = {0x0000, 0x3C00, 0xBC00, 0x3800, 0x4000, 0x4900};
+    const float want[] = {0.0f, 1.0f, -1.0f, 0.5f, 2.0f, 10.0f};
+    for (int i = 0; i < 6; ++i) EXPECT(gguf::f16_to_f32(gpu, bits[i]) == want[i], "f16 0x%04x", bits[i]);
+    EXPECT(std::signbit(gguf::f16_to_f32(gpu, 0x8000)), "f16 -0.0 keeps its sign");
+    {   // Q8_0: d = 0.5, q = 1..32  -> (i+1)/2
+        std::vector<uint8_t> blk(34);
+        blk[0] = 0x00; blk[1] = 0x38;
+        for (int i = 0; i < 32; ++i) blk[2 + i] = (uint8_t)(int8_t)(i + 1);
+        auto out = gguf::dequant_q8_0(gpu, blk, 32);
+        for (int i = 0; i < 32; ++i) EXPECT(out[i] == (float)(i + 1) * 0.5f, "q8_0[%d] = %g", i, out[i]);
+    }
+    {   // Q4_0: d = 1.0, byte0 = 0x98 -> out[0] = 0, out[1] = 1 (interleaved order)
+        std::vector<uint8_t> blk(18, 0x88);
+        blk[0] = 0x00; blk[1] = 0x3C; blk[2] = 0x98;
+        auto out = gguf::dequant_q4_0(gpu, blk, 32);
+        EXPECT(out[0] == 0.0f && out[1] == 1.0f, "q4_0 interleave: %g %g", out[0], out[1]);
+        for (int i = 2; i < 32; ++i) EXPECT(out[i] == 0.0f, "q4_0[%d] = %g", i, out[i]);
+    }
+    {   // Q4_1: d = 1.0, m = 10.0, byte0 = 0x53 -> 13, 15 ; rest (0x00) -> 10
+        std::vector<uint8_t> blk(20, 0x00);
+        blk[0] = 0x00; blk[1] = 0x3C; blk[2] = 0x00; blk[3] = 0x49; blk[4] = 0x53;
+        auto out = gguf::dequant_q4_1(gpu, blk, 32);
+        EXPECT(out[0] == 13.0f && out[1] == 15.0f && out[2] == 10.0f, "q4_1: %g %g %g", out[0], out[1], out[2]);
+    }
+    bool threw = false;
+    try { gguf::dequant_q8_0(gpu, std::vector<uint8_t>(34), 33); } catch (const Panic &) { threw = true; }
+    EXPECT(threw, "num_elements %% 32 != 0 must panic (src/gguf.rs:287)");
+}
+
+// dequantise-then-matmul against the CPU composition, Q4_0 and Q8_0, M = 1 and 3
+static void test_block_weight_matmul(const GpuContext &gpu) {
+    std::printf("test_block_weight_matmul\n");
+    const size_t n_out = 48, k_in = 256, nb = n_out * k_in / 32;
+    uint32_t s = 42;
+    auto lcg = [&]() { s = s * 1103515245u + 12345u; return (float)s / 4294967295.0f * 2.0f - 1.0f; };  // tests/huffman_parity.rs:7-14
+    for (int type : {PG_GGML_Q4_0, PG_GGML_Q8_0}) {
+        const size_t bb = type == PG_GGML_Q4_0 ? 18 : 34;
+        std::vector<uint8_t> blocks(nb * bb);
+        for (size_t b = 0; b < nb; ++b) {
+            const uint16_t d = (uint16_t)(0x2000 + (b * 37) % 0x0C00);  // positive normal halves around 1e-2
+            blocks[b * bb] = (uint8_t)(d & 0xFF); blocks[b * bb + 1] = (uint8_t)(d >> 8);
+            for (size_t i = 2; i < bb; ++i) { s = s * 1103515245u + 12345u; blocks[b * bb + i] = (uint8_t)(s >> 16); }
+        }
+        for (size_t m : {(size_t)1, (size_t)3}) {
+            std::vector<float> x(m * k_in);
+            for (auto &v : x) v = lcg();
+            gguf::BlockWeight w(gpu, blocks, type, n_out, k_in);
+            auto y = w.matmul(x, m);
+            std::vector<float> ref(m * n_out);
+            orc_gguf_matmul(x.data(), m, blocks.data(), type, n_out, k_in, ref.data());
+            double rms = 0;
+            for (float v : ref) rms += (double)v * v;
+            rms = std::sqrt(rms / ref.size());
+            for (size_t i = 0; i < ref.size(); ++i) {
+                const double tol = 1e-3 * std::fmax(std::fabs((double)ref[i]), rms);  // the block-dequant contract
+                EXPECT(std::fabs((double)y[i] - ref[i]) <= tol, "type %d m %zu [%zu]: %g vs %g", type, m, i, y[i], ref[i]);
+            }
+        }
+    }
+}
+
+int main() {
+    try {
+        GpuContext gpu(0);
+        test_quantize_dequantize_roundtrip(gpu);
+        test_quantized_matmul_accuracy(gpu, 32, 128, 64, 200);
+        test_quantized_matmul_accuracy(gpu, 16, 64, 32, 100);
+        test_quantized_matmul_accuracy(gpu, 1, 64, 1, 200);
+        test_quantize_activations(gpu);
+        test_shape_panics(gpu);
+        test_gguf_known_answers(gpu);
+        test_block_weight_matmul(gpu);
+    } catch (const std::exception &e) {
+        std::printf("FAIL: uncaught %s\n", e.what());
+        return 2;
+    }
+    std::printf(failures ? "FAILED: %d check(s)\n" : "OK: all checks passed\n", failures);
+    return failures ? 1 : 0;
+}
