@@ -435,15 +435,27 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
     return launch_gemv<8>(ctx, n_out, k_in, qs, d, batch, xd, y);
 }
 
-// Quantise `m` activation rows (device) into the arena and run the fused product.
+// Quantise `m` activation rows (device) into the arena and run the fused product: the
+// streaming GEMV for one row, the matrix-core kernel (weights read once) for more.
 pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
                               float *y_dev) {
     void *ws = nullptr;
-    PG_TRY(pg_workspace(ctx, pg_xdigits_bytes(m, w->k_in), &ws));
-    const pg_xdigits xd = pg_xdigits_carve(ws, m, w->k_in);
-    PG_TRY(pg_launch_x_to_digits(ctx, x_dev, m, w->k_in, w->ggml_type, xd));
-    pg_gemv_batch batch = {(int)m, nullptr, nullptr, nullptr, 1};
-    return pg_launch_gguf_gemv(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, batch, xd, y_dev);
+    if (m == 1) {
+        PG_TRY(pg_workspace(ctx, pg_xdigits_bytes(m, w->k_in), &ws));
+        const pg_xdigits xd = pg_xdigits_carve(ws, m, w->k_in);
+        PG_TRY(pg_launch_x_to_digits(ctx, x_dev, m, w->k_in, w->ggml_type, xd));
+        pg_gemv_batch batch = {(int)m, nullptr, nullptr, nullptr, 1};
+        return pg_launch_gguf_gemv(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, batch, xd, y_dev);
+    }
+    const int ks = pg_gguf_mm_splitk(ctx, w->n_out, w->k_in, 1, nullptr);
+    const size_t sz_d = pg_mmdigits_bytes(m, w->k_in);
+    const size_t sz_part = ks > 1 ? pg_round_up((size_t)ks * m * w->n_out * sizeof(float), 256) : 0;
+    PG_TRY(pg_workspace(ctx, sz_d + sz_part, &ws));
+    const pg_mmdigits md = pg_mmdigits_carve(ws, m, w->k_in);
+    float *part = ks > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + sz_d) : nullptr;
+    PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, m, w->k_in, w->ggml_type, md));
+    pg_mm_group grp = {1, nullptr, nullptr, nullptr, nullptr, 0, (int)((m + 31) / 32), (int)m, 1};
+    return pg_launch_gguf_mm(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, grp, m, md, y_dev, part);
 }
 
 PG_API pg_status pg_f16_to_f32(pg_ctx *ctx, const uint16_t *bits, size_t n, float *out) {

@@ -1,0 +1,368 @@
+// Skinny / grouped product over GGUF block-quantised weights on the int8 matrix cores:
+//   y[pair, n] = sum_b  d[n, b] * xs[tok, b] * sum_{k in block b} q[n, k] * X[tok, k]
+// for up to 32 activation rows ("tokens") per workgroup, so the weights are read from HBM
+// once per group of tokens instead of once per token (M > 1 dequant-matmul of models::llama,
+// src/models/llama/model.rs:243-257 + src/tensor.rs:1342-1353, and the per-expert products
+// of the MoE FFN, examples/grok1/moe.rs:91-104).
+//
+// A GGUF block is 32 consecutive k, exactly the K of one v_mfma_i32_32x32x32_i8: per block
+// and 32x32 (weight rows x tokens) tile, two MFMAs give the exact integer dots of the
+// weights with the high and the low byte digit of the fixed-point activations
+// X = 256 * hi + lo (|X| <= 32639, per-block scale xs = absmax / 32639), and the tile is scaled by
+// d[n, b] * xs[tok, b] and accumulated in f32.  Weight rows sit on the accumulator
+// registers, tokens on lanes.
+//
+// Workgroup = 4 wavefronts = 128 weight rows x 32 tokens x one K chunk.  Everything is
+// staged through LDS with direct global->LDS loads, two stages of 4 blocks ahead of the one
+// being consumed: each wavefront's own 32 weight rows and their f16 block scales, and the
+// token digits and scales of the stage, which the four wavefronts share.
+#include "pg_internal.h"
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef const void __attribute__((address_space(1))) *gptr_t;
+typedef void __attribute__((address_space(3))) *lptr_t;
+typedef const v4i __attribute__((address_space(1))) *gv4i_ptr;
+
+inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
+
+constexpr int NBU = 4;                              // blocks per stage
+constexpr int RING = 3;                             // LDS stages (two in flight beyond the one consumed)
+constexpr int DIG_STAGE = NBU * 2 * 2 * 32 * 16;    // [j][plane][half][token][16 B]            8 KiB
+constexpr int D_STAGE = 4 * 256;                    // [wave][row group of 8][j][8 f16]          1 KiB
+constexpr int XS_STAGE = 64 * 16;                   // [token][4 block scales] (upper half idle) 1 KiB
+constexpr int W_STAGE = 4 * NBU * 1024;             // [wave][j][lane][16 B]                    16 KiB
+constexpr int OFF_D = DIG_STAGE, OFF_XS = OFF_D + D_STAGE, OFF_W = OFF_XS + XS_STAGE;
+constexpr int STAGE = OFF_W + W_STAGE;
+constexpr int LPS = 8;  // LDS fills per wavefront and stage: 2 digit, 1 scale, 1 xs, 4 weight
+
+// ---- activation rows -> two byte-digit planes -------------------------------------------
+// digits[row][plane][b][half][16]: plane 0 = high digit, 1 = low digit of X[k] = round(x[k] / xs[b]).
+// The 16 bytes of (b, half) follow the order in which the weight operand presents its k:
+//   Q8_0: half h holds elements 16h .. 16h+15;
+//   Q4_0: half h holds elements 2i + h (i = 0..15): the low (h = 0) or high (h = 1) nibbles
+//         of the block's 16 bytes (byte i = elements 2i, 2i+1, src/gguf.rs:316-323).
+// xs[row][nbp]: block scales absmax / 32639 (NaN for a block holding NaN or inf), nbp = nb
+// rounded up to 4.  8 consecutive threads own one block (4 elements each).
+template <bool NIB>
+__global__ __launch_bounds__(256) void x_to_mm_digits_kernel(const float *__restrict__ x, int nb, int nbp,
+                                                             int8_t *__restrict__ digits, float *__restrict__ xs) {
+    const size_t row = blockIdx.y;
+    const int b = blockIdx.x * 32 + (threadIdx.x >> 3), sub = threadIdx.x & 7;
+    if (b >= nb) return;  // whole 8-thread groups leave together
+    const float4 v = reinterpret_cast<const float4 *>(x + (row * nb + b) * 32)[sub];
+    const float f[4] = {v.x, v.y, v.z, v.w};
+    float amax = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3])));
+    int bad = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]);
+#pragma unroll
+    for (int off = 1; off < 8; off <<= 1) {
+        amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+        bad |= __shfl_xor(bad, off, 64);
+    }
+    float s = 1.0f, inv = 1.0f;
+    if (bad || !(amax <= 3.4028234663852886e38f)) {
+        s = __uint_as_float(0x7FC00000u);
+        inv = 0.0f;
+    } else if (amax > 0.0f) {
+        // the two signed byte digits reach 127 * 256 + 127: map the block's absmax onto that
+        s = fmaxf(amax / 32639.0f, 1.17549435e-38f);
+        inv = 1.0f / s;
+    }
+    int hi[4], lo[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float t = f[e] * inv;
+        const int X = (t != t) ? 0 : (int)rintf(t);
+        lo[e] = ((X + 128) & 255) - 128;
+        hi[e] = (X - lo[e]) >> 8;
+    }
+    int8_t *d0 = digits + ((row * 2 + 0) * (size_t)nb + b) * 32;  // plane 0, block b: [half][16]
+    int8_t *d1 = digits + ((row * 2 + 1) * (size_t)nb + b) * 32;
+    if (NIB) {
+        // elements 4*sub + {0, 2} -> half 0 positions 2*sub, 2*sub+1;  {1, 3} -> half 1, same positions
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            *reinterpret_cast<uint16_t *>(d0 + h * 16 + 2 * sub) = (uint16_t)((hi[h] & 255) | ((hi[h + 2] & 255) << 8));
+            *reinterpret_cast<uint16_t *>(d1 + h * 16 + 2 * sub) = (uint16_t)((lo[h] & 255) | ((lo[h + 2] & 255) << 8));
+        }
+    } else {
+        const int h = sub >> 2, pos = (sub & 3) * 4;
+        *reinterpret_cast<unsigned *>(d0 + h * 16 + pos) = (unsigned)(hi[0] & 255) | ((unsigned)(hi[1] & 255) << 8) |
+                                                          ((unsigned)(hi[2] & 255) << 16) | ((unsigned)(hi[3] & 255) << 24);
+        *reinterpret_cast<unsigned *>(d1 + h * 16 + pos) = (unsigned)(lo[0] & 255) | ((unsigned)(lo[1] & 255) << 8) |
+                                                          ((unsigned)(lo[2] & 255) << 16) | ((unsigned)(lo[3] & 255) << 24);
+    }
+    if (sub == 0) xs[row * (size_t)nbp + b] = s;
+}
+
+// Two's-complement nibbles (as stored at upload) of one dword -> four signed bytes: half h
+// takes the low (h = 0) or high (h = 1) nibble of every byte.  Per byte, with n the nibble:
+// ((n ^ 8) | 0x80) - 8 never borrows from the next byte; flipping bit 7 afterwards leaves n
+// sign-extended.
+__device__ __forceinline__ int nibbles_to_i8(int v, int shift) {
+    const unsigned y = ((unsigned)v >> shift) & 0x0F0F0F0Fu;
+    return (int)((((y ^ 0x08080808u) | 0x80808080u) - 0x08080808u) ^ 0x80808080u);
+}
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t h) {
+    _Float16 v;
+    const uint16_t hb = (uint16_t)h;
+    __builtin_memcpy(&v, &hb, 2);
+    return (float)v;
+}
+
+// grid: x = tiles of 128 weight rows, y = expert * tiles_per_expert + token tile, z = K chunk.
+// `chunk` (blocks per K chunk) is a multiple of NBU and no chunk is empty.
+// out: [gridDim.z][total pairs][n_out] (plain y when gridDim.z == 1).
+// (Two wavefronts per SIMD: with at most 256 registers per lane the MFMA results are written
+// to ordinary VGPRs, not to accumulation registers that would have to be copied out first.)
+template <int QT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gguf_mm_kernel(const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0,
+                                                      pg_mm_group grp, int n_out, int nb, int nbp, int chunk,
+                                                      const int8_t *__restrict__ digits, const float *__restrict__ xs,
+                                                      float *__restrict__ out, size_t part_stride) {
+    extern __shared__ __attribute__((aligned(1024))) char lds[];  // RING * STAGE bytes
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int l31 = lane & 31, hh = lane >> 5;
+
+    int e = 0, tt = blockIdx.y;
+    if (grp.counts) {
+        e = blockIdx.y / grp.tiles_per_expert;
+        tt = blockIdx.y - e * grp.tiles_per_expert;
+    }
+    const int count = grp.counts ? grp.counts[e] : grp.max_count;
+    if (tt * 32 >= count) return;  // the same for every thread of the workgroup
+    const uint8_t *qs_any = grp.qs_table ? grp.qs_table[e] : qs0;
+    const uint16_t *d_any = grp.d_table ? grp.d_table[e] : d0;
+
+    // this lane's token
+    const int slot = tt * 32 + l31;
+    const bool tok_ok = slot < count;
+    const int slot_c = tok_ok ? slot : tt * 32;  // spare lanes shadow the tile's first token
+    const int pair = grp.lists ? grp.lists[(size_t)e * grp.list_stride + slot_c] : slot_c;
+    const size_t xrow = (size_t)(pair / grp.x_row_div);
+    const int8_t *dig_row = digits + xrow * (size_t)nb * 64;
+    const float *xs_row = xs + xrow * (size_t)nbp;
+
+    // this lane's weight row (clamped; masked at the store) and this wavefront's scale groups
+    const int row0 = blockIdx.x * 128 + wave * 32;
+    const int wrow = row0 + l31 < n_out ? row0 + l31 : n_out - 1;
+    const int8_t *w_row = reinterpret_cast<const int8_t *>(qs_any) +
+                          (QT == 8 ? ((size_t)wrow * 2 + hh) * nb * 16 : (size_t)wrow * nb * 16);
+    const int ngroups = (n_out + 7) / 8;
+    int dg = (row0 >> 3) + (lane >> 4);
+    dg = dg < ngroups ? dg : ngroups - 1;
+    const char *d_grp = reinterpret_cast<const char *>(d_any) + (size_t)dg * nb * 16 + (lane & 3) * 4;
+    const int d_jb = (lane >> 2) & 3;  // the block of the stage this lane fetches scales of
+
+    const int b_begin = blockIdx.z * chunk;
+    const int b_end = b_begin + chunk < nb ? b_begin + chunk : nb;
+    const int nst = (b_end - b_begin + NBU - 1) / NBU;
+
+    // Every load of the K loop is a direct global->LDS fill, so the only memory waits in the
+    // loop are the explicit ones below (two stages stay in flight across the barrier).
+    // (The ring slot is a compile-time constant everywhere so that the compiler can tell the
+    // stage being filled from the stage being read and adds no waits of its own.)
+    auto issue = [&](auto ring_slot, int s) {
+        const int b0 = b_begin + s * NBU;
+        char *base = lds + decltype(ring_slot)::value * STAGE;
+        {   // token digits of blocks b0 .. b0+3: this wavefront fills block j = wave, both planes
+            const int b = b0 + wave < b_end ? b0 + wave : b_end - 1;
+#pragma unroll
+            for (int p = 0; p < 2; ++p)
+                __builtin_amdgcn_global_load_lds((gptr_t)(dig_row + (((size_t)p * nb + b) * 2 + hh) * 16),
+                                                 (lptr_t)(base + (wave * 2 + p) * 1024), 16, 0, 0);
+        }
+        {   // f16 scales of this wavefront's 32 rows: lane -> (group lane/16, block (lane/4)%4, dword lane%4)
+            const int b = b0 + d_jb < b_end ? b0 + d_jb : b_end - 1;
+            __builtin_amdgcn_global_load_lds((gptr_t)(d_grp + (size_t)b * 16), (lptr_t)(base + OFF_D + wave * 256), 4, 0, 0);
+        }
+        // xs[token][b0 .. b0+3]; the four wavefronts write the same bytes to the same place
+        __builtin_amdgcn_global_load_lds((gptr_t)(xs_row + b0), (lptr_t)(base + OFF_XS), 16, 0, 0);
+#pragma unroll
+        for (int j = 0; j < NBU; ++j) {
+            const int b = b0 + j < b_end ? b0 + j : b_end - 1;
+            __builtin_amdgcn_global_load_lds((gptr_t)(w_row + (size_t)b * 16), (lptr_t)(base + OFF_W + (wave * NBU + j) * 1024),
+                                             16, 0, 0);
+        }
+    };
+
+    float acc[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+
+    auto block_step = [&](const char *base, int j, float sj) {
+        const v4i bhi = *reinterpret_cast<const v4i *>(base + (j * 2 + 0) * 1024 + lane * 16);
+        const v4i blo = *reinterpret_cast<const v4i *>(base + (j * 2 + 1) * 1024 + lane * 16);
+        v4i a = *reinterpret_cast<const v4i *>(base + OFF_W + (wave * NBU + j) * 1024 + lane * 16);
+        if constexpr (QT == 4) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) a[t] = nibbles_to_i8(a[t], 4 * hh);
+        }
+        v16i zero;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) zero[r] = 0;
+        const v16i ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi, zero, 0, 0, 0);
+        const v16i ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo, zero, 0, 0, 0);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            // rows 8g + 4*hh + {0..3}  <->  accumulator registers 4g .. 4g+3
+            const v2i dd = *reinterpret_cast<const v2i *>(base + OFF_D + wave * 256 + (g * 4 + j) * 16 + hh * 8);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int r = 4 * g + q;
+                const uint32_t pairbits = (uint32_t)dd[q >> 1];
+                const float dv = half_bits_to_float((q & 1) ? pairbits >> 16 : pairbits & 0xFFFFu);
+                // |integer| < 2^28: rounded to 24 bits, then scaled (two roundings of 2^-24, far below the digit step)
+                const float fx = (float)(ihi[r] * 256 + ilo[r]) * sj;
+                acc[r] = fmaf(dv, fx, acc[r]);
+            }
+        }
+    };
+    auto compute = [&](auto ring_slot, int s) {
+        const int b0 = b_begin + s * NBU;
+        const char *base = lds + decltype(ring_slot)::value * STAGE;
+        // Read as integers: a float-typed LDS read makes the compiler wait for every LDS fill in
+        // flight (it cannot tell the stages apart), an int-typed one leaves the waits to us.
+        const v4i sxi = *reinterpret_cast<const v4i *>(base + OFF_XS + l31 * 16);
+        // (element -> named int -> float: a bit cast applied directly to a vector element
+        // expression was compiled as a cast of element 0)
+        const int sx0 = sxi[0], sx1 = sxi[1], sx2 = sxi[2], sx3 = sxi[3];
+        const float4 sx = make_float4(__int_as_float(sx0), __int_as_float(sx1), __int_as_float(sx2), __int_as_float(sx3));
+        if (b0 + NBU <= b_end) {  // full stage (wavefront-uniform)
+            block_step(base, 0, sx.x);
+            block_step(base, 1, sx.y);
+            block_step(base, 2, sx.z);
+            block_step(base, 3, sx.w);
+        } else {
+            block_step(base, 0, sx.x);
+            if (b0 + 1 < b_end) block_step(base, 1, sx.y);
+            if (b0 + 2 < b_end) block_step(base, 2, sx.z);
+        }
+    };
+
+    auto wait_barrier = [&](bool one_ahead) {
+        if (one_ahead) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n s_barrier" ::"n"(LPS) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n s_barrier" ::: "memory");
+    };
+
+    issue(std::integral_constant<int, 0>{}, 0);
+    if (nst > 1) issue(std::integral_constant<int, 1>{}, 1);
+    for (int s0 = 0; s0 < nst; s0 += RING) {
+#define PG_MM_STEP(U)                                                                     \
+        if (s0 + U < nst) {                                                               \
+            const int s = s0 + U;                                                         \
+            wait_barrier(s + 1 < nst);                                                    \
+            if (s + 2 < nst) issue(std::integral_constant<int, (U + 2) % RING>{}, s + 2); \
+            compute(std::integral_constant<int, U>{}, s);                                 \
+        }
+        PG_MM_STEP(0)
+        PG_MM_STEP(1)
+        PG_MM_STEP(2)
+#undef PG_MM_STEP
+    }
+
+    if (!tok_ok) return;
+    float *y = out + blockIdx.z * part_stride + (size_t)pair * n_out;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const int r0 = row0 + 8 * g + 4 * hh;
+        if (r0 + 3 < n_out && (n_out & 3) == 0) {
+            *reinterpret_cast<float4 *>(y + r0) = make_float4(acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]);
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (r0 + q < n_out) y[r0 + q] = acc[4 * g + q];
+        }
+    }
+}
+
+// y[i] = part[0][i] + part[1][i] + ... in a fixed order.
+__global__ void sum_parts_kernel(const float *__restrict__ part, size_t n, int ks, size_t stride, float *__restrict__ y) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float acc = part[i];
+    for (int s = 1; s < ks; ++s) acc += part[(size_t)s * stride + i];
+    y[i] = acc;
+}
+
+}  // namespace
+
+size_t pg_mmdigits_bytes(size_t rows, size_t k) {
+    const size_t nb = k / 32, nbp = pg_round_up(nb, 4);
+    return pg_round_up(rows * nb * 64, 256) + pg_round_up(rows * nbp * sizeof(float), 256);
+}
+
+pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k) {
+    const size_t nb = k / 32;
+    pg_mmdigits md;
+    char *p = static_cast<char *>(base);
+    md.digits = reinterpret_cast<int8_t *>(p);
+    p += pg_round_up(rows * nb * 64, 256);
+    md.xs = reinterpret_cast<float *>(p);
+    md.rows = rows;
+    md.k = k;
+    return md;
+}
+
+pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows, size_t k, int ggml_type,
+                                   const pg_mmdigits &md) {
+    if (rows == 0) return PG_OK;
+    if (rows > 65535) return pg_fail(PG_EUNSUPPORTED, "x_to_mm_digits: more than 65535 activation rows");
+    const int nb = (int)(k / 32), nbp = (int)pg_round_up(nb, 4);
+    const dim3 grid(grid_for(nb, 32), (unsigned)rows);
+    if (ggml_type == PG_GGML_Q4_0)
+        return pg_launch(ctx, "x_to_mm_digits", x_to_mm_digits_kernel<true>, grid, dim3(256), 0, x_dev, nb, nbp, md.digits, md.xs);
+    return pg_launch(ctx, "x_to_mm_digits", x_to_mm_digits_kernel<false>, grid, dim3(256), 0, x_dev, nb, nbp, md.digits, md.xs);
+}
+
+int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t groups, int *chunk_out) {
+    const size_t nb = k_in / 32;
+    const size_t wgs = ((n_out + 127) / 128) * (groups ? groups : 1);
+    size_t ks = (2 * (size_t)ctx->num_cu + wgs - 1) / wgs;
+    if (ks > 8) ks = 8;
+    if (ks < 1) ks = 1;
+    size_t chunk = pg_round_up((nb + ks - 1) / ks, NBU);
+    if (chunk < 2 * NBU) chunk = 2 * NBU;
+    ks = (nb + chunk - 1) / chunk;
+    if (chunk_out) *chunk_out = (int)chunk;
+    return (int)ks;
+}
+
+pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,
+                            const uint16_t *d, const pg_mm_group &grp, size_t total_pairs, const pg_mmdigits &md,
+                            float *y, float *part) {
+    if (total_pairs == 0) return PG_OK;
+    const int nb = (int)(k_in / 32), nbp = (int)pg_round_up(nb, 4);
+    const size_t experts = grp.counts ? (size_t)grp.num_experts : 1;
+    int chunk = 0;
+    const int ks = pg_gguf_mm_splitk(ctx, n_out, k_in, experts, &chunk);
+    if (ks > 1 && !part) return pg_fail(PG_EINVAL, "gguf_mm: split-K needs a partial-sum buffer");
+    const size_t gy = experts * (size_t)grp.tiles_per_expert;
+    if (gy > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_mm: too many token tiles");
+    const dim3 grid(grid_for(n_out, 128), (unsigned)gy, (unsigned)ks);
+    float *dst = ks > 1 ? part : y;
+    const size_t stride = total_pairs * n_out;
+    constexpr size_t lds = (size_t)RING * STAGE;
+    static bool attr_set[2] = {false, false};  // per kernel instantiation
+    auto launch = [&](auto kern, const char *name) -> pg_status {
+        bool &attr_done = attr_set[ggml_type == PG_GGML_Q4_0 ? 0 : 1];
+        if (!attr_done) {
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return pg_fail(PG_EDEVICE, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+            attr_done = true;
+        }
+        return pg_launch(ctx, name, kern, grid, dim3(256), lds, qs, d, grp, (int)n_out, nb, nbp, chunk, md.digits, md.xs, dst,
+                         stride);
+    };
+    if (ggml_type == PG_GGML_Q4_0) PG_TRY(launch(gguf_mm_kernel<4>, "gguf_mm_q4_0"));
+    else PG_TRY(launch(gguf_mm_kernel<8>, "gguf_mm_q8_0"));
+    if (ks > 1)
+        PG_TRY(pg_launch(ctx, "gguf_mm_sum_parts", sum_parts_kernel, dim3(grid_for(stride, 256)), dim3(256), 0, part, stride, ks,
+                         stride, y));
+    return PG_OK;
+}

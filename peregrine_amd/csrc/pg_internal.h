@@ -189,6 +189,36 @@ struct pg_gemv_batch {
 pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in,
                               const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
                               const pg_xdigits &xd, float *y);
+// Activation rows as two byte-digit planes for the matrix-core product (see pg_gguf_mm.hip).
+struct pg_mmdigits {
+    int8_t *digits;  // [rows][2 planes][k/32 blocks][2 halves][16 bytes]
+    float *xs;       // [rows][k/32 rounded up to 4] block scales
+    size_t rows, k;
+};
+size_t pg_mmdigits_bytes(size_t rows, size_t k);
+pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k);
+pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows, size_t k, int ggml_type,
+                                   const pg_mmdigits &md);
+// Which activation rows multiply which weights.  Without `counts`: one weight tensor and pairs
+// 0 .. max_count-1.  With `counts`: expert e owns counts[e] pairs, listed (in ascending order) in
+// lists[e * list_stride ..]; its weights are qs_table[e] / d_table[e].  Pair p reads activation
+// row p / x_row_div and writes output row p.  tiles_per_expert = ceil(max pairs per expert / 32).
+struct pg_mm_group {
+    int num_experts;
+    const uint8_t *const *qs_table;
+    const uint16_t *const *d_table;
+    const int *lists;
+    const int *counts;
+    int list_stride;
+    int tiles_per_expert;
+    int max_count;
+    int x_row_div;
+};
+// Number of K chunks the product is split into (partial sums: [chunks][pairs][n_out] floats).
+int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t groups, int *chunk_out);
+pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,
+                            const uint16_t *d, const pg_mm_group &grp, size_t total_pairs, const pg_mmdigits &md,
+                            float *y, float *part);
 // y[m, n_out] = x[m, k_in] . dequant(w)^T on device pointers (uses the scratch arena).
 pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
                               float *y_dev);

@@ -8,6 +8,7 @@
 //   5. out[t] = 0 + p_0 * y_0 + p_1 * y_1 ... in k order, multiply then add
 //      (examples/grok1/moe.rs:99-104), raw softmax probabilities.
 #include "pg_internal.h"
+#include <algorithm>
 
 namespace {
 
@@ -41,6 +42,22 @@ __global__ void route_topk_kernel(const float *__restrict__ logits, int T, int E
         topk_idx[(size_t)t * top_k + k] = best;
         topk_p[(size_t)t * top_k + k] = bp;
     }
+}
+
+// Per expert, the (token, k) pairs routed to it, in ascending pair order.  One wavefront per
+// expert: ballot + prefix count over 64 pairs at a time.
+__global__ __launch_bounds__(64) void expert_lists_kernel(const int *__restrict__ topk_idx, int P, int stride,
+                                                          int *__restrict__ lists, int *__restrict__ counts) {
+    const int e = blockIdx.x, lane = threadIdx.x;
+    int base = 0;
+    for (int p0 = 0; p0 < P; p0 += 64) {
+        const int p = p0 + lane;
+        const bool mine = p < P && topk_idx[p] == e;
+        const unsigned long long mask = __ballot(mine);
+        if (mine) lists[(size_t)e * stride + base + __popcll(mask & ((1ull << lane) - 1ull))] = p;
+        base += __popcll(mask);
+    }
+    if (lane == 0) counts[e] = base;
 }
 
 __device__ __forceinline__ float act_silu(float x) {
@@ -102,24 +119,31 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     const size_t P = T * top_k;
 
     // Arena layout.
+    const int ks_up = pg_gguf_mm_splitk(ctx, ffn, d, E, nullptr), ks_down = pg_gguf_mm_splitk(ctx, d, ffn, E, nullptr);
+    const size_t part_floats = std::max(ks_up > 1 ? (size_t)ks_up * P * ffn : 0, ks_down > 1 ? (size_t)ks_down * P * d : 0);
     const size_t sz_tab = pg_round_up(6 * E * sizeof(void *), 256);
     const size_t sz_idx = pg_round_up(P * sizeof(int), 256);
     const size_t sz_p = pg_round_up(P * sizeof(float), 256);
+    const size_t sz_lists = pg_round_up(E * T * sizeof(int), 256), sz_counts = pg_round_up(E * sizeof(int), 256);
     const size_t sz_act = pg_round_up(P * ffn * sizeof(float), 256);
     const size_t sz_y = pg_round_up(P * d * sizeof(float), 256);
-    const size_t sz_xd = pg_xdigits_bytes(T, d), sz_hd = pg_xdigits_bytes(P, ffn);
+    const size_t sz_part = pg_round_up(part_floats * sizeof(float), 256);
+    const size_t sz_xd = pg_mmdigits_bytes(T, d), sz_hd = pg_mmdigits_bytes(P, ffn);
     void *ws = nullptr;
-    PG_TRY(pg_workspace(ctx, sz_tab + sz_idx + sz_p + 3 * sz_act + sz_y + sz_xd + sz_hd, &ws));
+    PG_TRY(pg_workspace(ctx, sz_tab + sz_idx + sz_p + sz_lists + sz_counts + 3 * sz_act + sz_y + sz_part + sz_xd + sz_hd, &ws));
     char *p = static_cast<char *>(ws);
     const void **tab = reinterpret_cast<const void **>(p); p += sz_tab;
     int *topk_idx = reinterpret_cast<int *>(p); p += sz_idx;
     float *topk_p = reinterpret_cast<float *>(p); p += sz_p;
+    int *lists = reinterpret_cast<int *>(p); p += sz_lists;
+    int *counts = reinterpret_cast<int *>(p); p += sz_counts;
     float *g = reinterpret_cast<float *>(p); p += sz_act;
     float *u = reinterpret_cast<float *>(p); p += sz_act;
     float *h = reinterpret_cast<float *>(p); p += sz_act;
     float *yb = reinterpret_cast<float *>(p); p += sz_y;
-    const pg_xdigits xd = pg_xdigits_carve(p, T, d); p += sz_xd;
-    const pg_xdigits hd = pg_xdigits_carve(p, P, ffn);
+    float *part = sz_part ? reinterpret_cast<float *>(p) : nullptr; p += sz_part;
+    const pg_mmdigits xd = pg_mmdigits_carve(p, T, d); p += sz_xd;
+    const pg_mmdigits hd = pg_mmdigits_carve(p, P, ffn);
 
     // Expert pointer tables: [gate qs | gate d | up qs | up d | down qs | down d], E each.
     const void *host_tab[6 * MAX_EXPERTS];
@@ -134,18 +158,22 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
 
     PG_TRY(pg_launch(ctx, "moe_route_topk", route_topk_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
                      router_logits_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
-    PG_TRY(pg_launch_x_to_digits(ctx, x_dev, T, d, type, xd));
+    PG_TRY(pg_launch(ctx, "moe_expert_lists", expert_lists_kernel, dim3((unsigned)E), dim3(64), 0, topk_idx, (int)P, (int)T,
+                     lists, counts));
+    PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, T, d, type, xd));
     auto table = [&](int which) { return reinterpret_cast<const uint8_t *const *>(tab + which * E); };
     auto dtable = [&](int which) { return reinterpret_cast<const uint16_t *const *>(tab + which * E); };
-    pg_gemv_batch bg = {(int)P, table(0), dtable(1), topk_idx, (int)top_k};
-    PG_TRY(pg_launch_gguf_gemv(ctx, type, ffn, d, nullptr, nullptr, bg, xd, g));
-    pg_gemv_batch bu = {(int)P, table(2), dtable(3), topk_idx, (int)top_k};
-    PG_TRY(pg_launch_gguf_gemv(ctx, type, ffn, d, nullptr, nullptr, bu, xd, u));
+    // Each token reaches an expert at most once, so an expert owns at most T pairs.
+    const int tiles = (int)((T + 31) / 32);
+    const pg_mm_group gg = {(int)E, table(0), dtable(1), lists, counts, (int)T, tiles, (int)T, (int)top_k};
+    PG_TRY(pg_launch_gguf_mm(ctx, type, ffn, d, nullptr, nullptr, gg, P, xd, g, part));
+    const pg_mm_group gu = {(int)E, table(2), dtable(3), lists, counts, (int)T, tiles, (int)T, (int)top_k};
+    PG_TRY(pg_launch_gguf_mm(ctx, type, ffn, d, nullptr, nullptr, gu, P, xd, u, part));
     PG_TRY(pg_launch(ctx, "moe_act_mul", act_mul_kernel, dim3(grid_for(P * ffn, 256)), dim3(256), 0, g, u, P * ffn,
                      act, h));
-    PG_TRY(pg_launch_x_to_digits(ctx, h, P, ffn, type, hd));
-    pg_gemv_batch bd = {(int)P, table(4), dtable(5), topk_idx, 1};
-    PG_TRY(pg_launch_gguf_gemv(ctx, type, d, ffn, nullptr, nullptr, bd, hd, yb));
+    PG_TRY(pg_launch_x_to_mm_digits(ctx, h, P, ffn, type, hd));
+    const pg_mm_group gd = {(int)E, table(4), dtable(5), lists, counts, (int)T, tiles, (int)T, 1};
+    PG_TRY(pg_launch_gguf_mm(ctx, type, d, ffn, nullptr, nullptr, gd, P, hd, yb, part));
     return pg_launch(ctx, "moe_combine", combine_kernel, dim3(grid_for(T * d, 256)), dim3(256), 0, yb, topk_p, (int)T,
                      (int)d, (int)top_k, out_dev);
 }

@@ -16,7 +16,8 @@ import helpers as H
 pytestmark = pytest.mark.gpu
 
 RTOL_CONTRACT = 1e-3                 # BASELINE: Q4_0/Q8_0 block-dequant paths
-RTOL_ACHIEVED = {2: 1e-4, 8: 2e-5}   # what this implementation is held to, per ggml type
+RTOL_ACHIEVED = {2: 1e-4, 8: 2e-5}   # what the one-row (GEMV) path is held to, per ggml type
+RTOL_ACHIEVED_MM = 4e-4              # several rows: 16-bit fixed-point activations per block
 
 
 def say(msg):
@@ -92,6 +93,8 @@ GGUF_SHAPES = [
     (8, 256, 4096, 1), (8, 77, 96, 3), (8, 96, 6144, 4), (8, 64, 32768, 2),
     (2, 14336, 4096, 1),                                        # BASELINE config 4, full size
     (8, 6144, 4096, 1),
+    # more than one row: matrix-core path (token tiles of 32, row tiles of 128, split K)
+    (2, 130, 224, 33), (8, 131, 160, 40), (2, 515, 4096, 64), (8, 257, 6144, 35), (2, 14336, 4096, 4), (8, 4096, 14336, 16),
 ]
 
 
@@ -109,7 +112,7 @@ def test_gguf_matmul_vs_oracle(ctx, orc, typ, n_out, k_in, m):
     for r in range(m):
         sl = slice(r * n_out, (r + 1) * n_out)
         H.assert_close_rel(got[sl], want[sl], RTOL_CONTRACT, f"row {r} (contract)")
-        H.assert_close_rel(got[sl], want[sl], RTOL_ACHIEVED[typ], f"row {r} (achieved)")
+        H.assert_close_rel(got[sl], want[sl], RTOL_ACHIEVED[typ] if m == 1 else RTOL_ACHIEVED_MM, f"row {r} (achieved)")
     gw.free()
 
 
@@ -126,10 +129,10 @@ def test_gguf_matmul_full_size_m16_and_linearity(ctx, orc):
     got = gw.matmul(x, m).reshape(m, n_out)
     want = orc.gguf_matmul(x, m, raw, 2, n_out, k_in).reshape(m, n_out)
     for r in range(m):
-        H.assert_close_rel(got[r], want[r], RTOL_ACHIEVED[2], f"row {r}")
+        H.assert_close_rel(got[r], want[r], RTOL_ACHIEVED_MM, f"row {r}")
     xs = x.reshape(m, k_in)
     y12 = gw.matmul(xs[0] + xs[1], 1)
-    H.assert_close_rel(y12, got[0].astype(np.float64) + got[1], 1e-4, "linearity")
+    H.assert_close_rel(y12, got[0].astype(np.float64) + got[1], RTOL_ACHIEVED_MM, "linearity")
     gw.free()
 
 
