@@ -208,6 +208,26 @@ def main():
             lib.pg_qtensor_free(ctx.handle, h)
     torch.cuda.empty_cache()
 
+    # ------------------------------------------------------------------ cfg1: one W8A8 linear, M = 32
+    w1 = [make_weight(4096, 4096) for _ in range(8)]  # 8 x 16.8 MB rotated
+    a1 = torch.randn(32, 4096, device=dev, generator=gen, dtype=torch.float32)
+    o1 = torch.empty(32, 4096, device=dev)
+
+    def lin_step():
+        h = w1[state["i"] % len(w1)]
+        state["i"] += 1
+        check(lib.pg_matmul_quantized_dev(ctx.handle, ptr(a1), 32, 4096, h, ptr(o1), None))
+
+    lin_ms = timed(lin_step, dsteps, max(args.warmup, 8))
+    prof = profiled(lin_step, dsteps)
+    lin_bytes = 17842176
+    linear_m32 = {"workload": "cfg1: W8A8 linear [32x4096] x [4096x4096] (the reference's CPU-runnable case); 8 weights rotated",
+                  "value": round(2 * 32 * 4096 * 4096 / (lin_ms * 1e-3) / 1e12, 2), "unit": "TOP/s",
+                  "gbs": round(lin_bytes / (lin_ms * 1e-3) / 1e9, 1), "ms_per_step": round(lin_ms, 5),
+                  "kernels_ms": {k: round(v[0], 5) for k, v in prof.items()}}
+    for h in w1:
+        lib.pg_qtensor_free(ctx.handle, h)
+
     # ------------------------------------------------------------------ decode GEMV (GGUF Q4_0)
     from peregrine_amd import synth
     n_out, k_in = 14336, 4096
@@ -237,8 +257,77 @@ def main():
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(q4_gbs / PEAK_HBM_GBS, 4),
                          "traffic": traffic_for("gguf_gemv_q4_0"), "bytes_per_launch": q4_bytes,
                          "avg_launch_ms": round(q4_avg_ms, 5)}}
+    # ------------------------------------------------------------------ cfg4 at M = 4 and 16 (matrix-core path)
+    skinny = []
+    for m_q in (4, 16):
+        x_m = torch.randn(m_q, k_in, device=dev, generator=gen, dtype=torch.float32)
+        y_m = torch.empty(m_q, n_out, device=dev)
+
+        def mm_step():
+            h = q4[state["i"] % Q4_ROT]
+            state["i"] += 1
+            check(lib.pg_gguf_matmul_dev(ctx.handle, ptr(x_m), m_q, h, ptr(y_m)))
+
+        mm_bytes = n_out * (k_in // 32) * 18 + 4 * m_q * k_in + 4 * m_q * n_out
+        mm_ms = timed(mm_step, dsteps, max(args.warmup, 8))
+        prof = profiled(mm_step, dsteps)
+        k_ms = prof["gguf_mm_q4_0"][0]
+        skinny.append({"workload": f"cfg4: M={m_q} Q4_0 dequant-matmul [{m_q}x4096]->[{m_q}x14336], weights read once",
+                       "value": round(mm_bytes / (mm_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "ms_per_step": round(mm_ms, 5),
+                       "gflops": round(2 * m_q * n_out * k_in / (mm_ms * 1e-3) / 1e9, 1),
+                       "kernels_ms": {k: round(v[0], 5) for k, v in prof.items()},
+                       "roofline": {"kernel": "gguf_mm_kernel<Q4_0>", "bound": "hbm",
+                                    "achieved": round(mm_bytes / (k_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                    "frac": round(mm_bytes / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None,
+                                    "bytes_per_launch": mm_bytes, "avg_launch_ms": round(k_ms, 5)}})
     for h in q4:
         lib.pg_gguf_free(ctx.handle, h)
+    del raw, wq
+
+    # ------------------------------------------------------------------ cfg5: Grok-1-shaped MoE expert FFN, Q8_0
+    T_moe, d_moe, ffn_moe, E_moe, topk_moe = 64, 6144, 32768, 8, 2
+    nblk = ffn_moe * d_moe // 32
+    rng = np.random.default_rng(5)
+    blocks = np.empty((nblk, 34), np.uint8)
+    blocks[:, 2:] = rng.integers(0, 256, size=(nblk, 32), dtype=np.uint8)      # i8 quants
+    blocks[:, :2] = np.frombuffer(np.float16(0.02 / 127).tobytes(), np.uint8)  # d
+    experts = [[], [], []]
+    for which, (no, ki) in enumerate(((ffn_moe, d_moe), (ffn_moe, d_moe), (d_moe, ffn_moe))):
+        for e in range(E_moe):
+            blocks[:, 2] = e + 8 * which  # make the tensors differ
+            h = C.c_void_p()
+            check(lib.pg_gguf_upload(ctx.handle, C.c_void_p(blocks.ctypes.data), _ffi.GGML_Q8_0, no, ki, C.byref(h)))
+            experts[which].append(h)
+    del blocks
+    tabs = [(C.c_void_p * E_moe)(*[h.value for h in experts[w]]) for w in range(3)]
+    x_moe = torch.randn(T_moe, d_moe, device=dev, generator=gen, dtype=torch.float32)
+    lg_moe = torch.randn(T_moe, E_moe, device=dev, generator=gen, dtype=torch.float32)
+    out_moe = torch.empty(T_moe, d_moe, device=dev)
+
+    def moe_step():
+        check(lib.pg_moe_ffn_dev(ctx.handle, ptr(x_moe), T_moe, ptr(lg_moe), E_moe, topk_moe, tabs[0], tabs[1], tabs[2],
+                                 _ffi.ACT_SILU, ptr(out_moe)))
+
+    moe_bytes = 3 * E_moe * nblk * 34 + 2 * 4 * T_moe * d_moe  # every expert is hit at T=64, k=2 (checked below)
+    hit = int(torch.unique(torch.topk(lg_moe, topk_moe, dim=1).indices).numel())
+    moe_ms = timed(moe_step, 5, 2)
+    prof = profiled(moe_step, 5)
+    mm_total = prof["gguf_mm_q8_0"][0] * prof["gguf_mm_q8_0"][1] / 5  # three launches per step
+    moe = {"workload": "cfg5: Grok-1-shaped MoE FFN, Q8_0 experts (d 6144, ffn 32768, 8 experts, top-2, 64 tokens, SiLU); "
+                       "5.13 GB of expert weights, read once per step",
+           "experts_hit": hit, "value": round(moe_bytes / (moe_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+           "ms_per_step": round(moe_ms, 4),
+           "tflops": round(2 * T_moe * topk_moe * 3 * ffn_moe * d_moe / (moe_ms * 1e-3) / 1e12, 2),
+           "kernels_ms": {k: round(v[0], 5) for k, v in prof.items()},
+           "roofline": {"kernel": "gguf_mm_kernel<Q8_0> (gate, up, down)", "bound": "hbm",
+                        "achieved": round(3 * E_moe * nblk * 34 / (mm_total * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                        "unit": "GB/s", "frac": round(3 * E_moe * nblk * 34 / (mm_total * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                        "traffic": None, "bytes_per_launch": E_moe * nblk * 34,
+                        "avg_launch_ms": round(prof["gguf_mm_q8_0"][0], 5)}}
+    for w3 in experts:
+        for h in w3:
+            lib.pg_gguf_free(ctx.handle, h)
+    torch.cuda.empty_cache()
 
     if args.calibrate_copy:  # a plain copy of known size: 512 MiB read + 512 MiB written per launch
         src = torch.empty(128 << 20, device=dev, dtype=torch.float32).normal_()
@@ -263,7 +352,7 @@ def main():
                                "each product = per-row activation quantisation + i8 GEMM + f32 rescale",
                    "m": M_PREFILL, "ops_per_step": LAYER_OPS},
         "pct_int8_mfma_peak": round(100 * tops / PEAK_INT8_TOPS, 2),
-        "roofline": roofline, "activation_quant": act_quant, "decode_gemv": decode, "gguf_q4_0_gemv": gguf,
+        "roofline": roofline, "activation_quant": act_quant, "linear_m32": linear_m32, "decode_gemv": decode, "gguf_q4_0_gemv": gguf, "gguf_q4_0_skinny": skinny, "moe_q8_0": moe,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line), flush=True)

@@ -95,6 +95,7 @@ PG_API void pg_ctx_destroy(pg_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void)hipFree(ctx->ws);
+    if (ctx->moe_tab_dev) (void)hipFree(ctx->moe_tab_dev);
     prof_drop(ctx);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;

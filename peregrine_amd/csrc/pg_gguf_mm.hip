@@ -31,13 +31,20 @@ inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + bloc
 
 constexpr int NBU = 4;                              // blocks per stage
 constexpr int RING = 3;                             // LDS stages (two in flight beyond the one consumed)
-constexpr int DIG_STAGE = NBU * 2 * 2 * 32 * 16;    // [j][plane][half][token][16 B]            8 KiB
-constexpr int D_STAGE = 4 * 256;                    // [wave][row group of 8][j][8 f16]          1 KiB
-constexpr int XS_STAGE = 64 * 16;                   // [token][4 block scales] (upper half idle) 1 KiB
-constexpr int W_STAGE = 4 * NBU * 1024;             // [wave][j][lane][16 B]                    16 KiB
+// LDS stage layout.  Every fill is arranged so that neighbouring lanes fetch neighbouring
+// 16-byte chunks of global memory (whole 64- or 128-byte runs per request); the chunk order
+// inside a run is XOR-swizzled so that the 128-bit LDS reads of 8 neighbouring lanes fall
+// into 8 different 16-byte bank groups.
+constexpr int DIG_STAGE = 64 * 128;                 // [token][plane] units of 128 B: 4 blocks x 2 halves  8 KiB
+constexpr int D_STAGE = 4 * 256;                    // [wave][row group of 8][j][8 f16]                     1 KiB
+constexpr int XS_STAGE = 32 * 16;                   // [token][4 block scales]                              512 B
 constexpr int OFF_D = DIG_STAGE, OFF_XS = OFF_D + D_STAGE, OFF_W = OFF_XS + XS_STAGE;
-constexpr int STAGE = OFF_W + W_STAGE;
-constexpr int LPS = 8;  // LDS fills per wavefront and stage: 2 digit, 1 scale, 1 xs, 4 weight
+template <int QT> struct MMCfg {
+    static constexpr int W_WAVE = QT == 8 ? 64 * 64 : 32 * 64;  // per wavefront: [stream][4 blocks][16 B]
+    static constexpr int W_FILLS = W_WAVE / 1024;               // weight fills per wavefront and stage
+    static constexpr int STAGE = OFF_W + 4 * W_WAVE;            // 25.5 KiB (Q8_0) / 17.5 KiB (Q4_0)
+    static constexpr int LPS = 2 + 1 + 1 + W_FILLS;             // LDS fills per wavefront and stage
+};
 
 // ---- activation rows -> two byte-digit planes -------------------------------------------
 // digits[row][plane][b][half][16]: plane 0 = high digit, 1 = low digit of X[k] = round(x[k] / xs[b]).
@@ -98,13 +105,11 @@ __global__ __launch_bounds__(256) void x_to_mm_digits_kernel(const float *__rest
     if (sub == 0) xs[row * (size_t)nbp + b] = s;
 }
 
-// Two's-complement nibbles (as stored at upload) of one dword -> four signed bytes: half h
-// takes the low (h = 0) or high (h = 1) nibble of every byte.  Per byte, with n the nibble:
-// ((n ^ 8) | 0x80) - 8 never borrows from the next byte; flipping bit 7 afterwards leaves n
-// sign-extended.
-__device__ __forceinline__ int nibbles_to_i8(int v, int shift) {
-    const unsigned y = ((unsigned)v >> shift) & 0x0F0F0F0Fu;
-    return (int)((((y ^ 0x08080808u) | 0x80808080u) - 0x08080808u) ^ 0x80808080u);
+// Two's-complement nibbles (as stored at upload) of one dword -> four signed bytes holding
+// 16 * (q - 8): a nibble moved to the top of its byte IS that value, no sign extension
+// needed.  left = 4 takes the low nibble of every byte, left = 0 the high one.
+__device__ __forceinline__ int nibbles_to_i8x16(int v, int left) {
+    return (int)(((unsigned)v << left) & 0xF0F0F0F0u);
 }
 
 __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
@@ -139,25 +144,50 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint8_t *qs_any = grp.qs_table ? grp.qs_table[e] : qs0;
     const uint16_t *d_any = grp.d_table ? grp.d_table[e] : d0;
 
-    // this lane's token
-    const int slot = tt * 32 + l31;
-    const bool tok_ok = slot < count;
-    const int slot_c = tok_ok ? slot : tt * 32;  // spare lanes shadow the tile's first token
-    const int pair = grp.lists ? grp.lists[(size_t)e * grp.list_stride + slot_c] : slot_c;
-    const size_t xrow = (size_t)(pair / grp.x_row_div);
-    const int8_t *dig_row = digits + xrow * (size_t)nb * 64;
-    const float *xs_row = xs + xrow * (size_t)nbp;
+    constexpr int STAGE = MMCfg<QT>::STAGE, W_WAVE = MMCfg<QT>::W_WAVE, W_FILLS = MMCfg<QT>::W_FILLS;
+    // Activation row of a token slot of this tile (spare slots shadow the tile's first token).
+    auto xrow_of = [&](int tok) -> size_t {
+        const int slot = tt * 32 + tok;
+        const int slot_c = slot < count ? slot : tt * 32;
+        const int pr = grp.lists ? grp.lists[(size_t)e * grp.list_stride + slot_c] : slot_c;
+        return (size_t)(pr / grp.x_row_div);
+    };
+    // the token whose outputs this lane accumulates
+    const bool tok_ok = tt * 32 + l31 < count;
+    const int pair = tok_ok ? (grp.lists ? grp.lists[(size_t)e * grp.list_stride + tt * 32 + l31] : tt * 32 + l31) : 0;
 
-    // this lane's weight row (clamped; masked at the store) and this wavefront's scale groups
+    // Fill duties of this lane.
+    // digits: fill n = 2*wave + u covers units 8n .. 8n+7, unit = 2*token + plane; the lane
+    // fetches chunk (lane & 7) ^ (token & 7) of the unit's 128 bytes, chunk = 2*block + half.
+    const int8_t *dig_src[2];
+    int dig_jb[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int unit = (2 * wave + u) * 8 + (lane >> 3), tok = unit >> 1, pl = unit & 1;
+        const int ch = (lane & 7) ^ (tok & 7);
+        dig_jb[u] = ch >> 1;
+        dig_src[u] = digits + xrow_of(tok) * (size_t)nb * 64 + (size_t)pl * nb * 32 + (ch & 1) * 16;
+    }
+    // xs: lanes 0..7 of wavefront w fetch the 4 block scales of tokens 8w .. 8w+7
+    const float *xs_src = xs + xrow_of(8 * wave + (lane & 7)) * (size_t)nbp;
+    // weights: fill q covers streams 16q .. 16q+15 (Q8_0: stream = 32*half + row, Q4_0: stream = row);
+    // the lane fetches block (lane & 3) ^ swizzle of the stream's 4 blocks.
     const int row0 = blockIdx.x * 128 + wave * 32;
-    const int wrow = row0 + l31 < n_out ? row0 + l31 : n_out - 1;
-    const int8_t *w_row = reinterpret_cast<const int8_t *>(qs_any) +
-                          (QT == 8 ? ((size_t)wrow * 2 + hh) * nb * 16 : (size_t)wrow * nb * 16);
+    const int w_jb = (lane & 3) ^ ((lane >> 3) & 3);  // stream >> 1 = 8q + (lane >> 3)
+    const int8_t *w_src[W_FILLS];
+#pragma unroll
+    for (int q = 0; q < W_FILLS; ++q) {
+        const int st = 16 * q + (lane >> 2);
+        const int wrow = row0 + (st & 31) < n_out ? row0 + (st & 31) : n_out - 1;  // clamped; masked at the store
+        w_src[q] = reinterpret_cast<const int8_t *>(qs_any) +
+                   (QT == 8 ? ((size_t)wrow * 2 + (st >> 5)) * nb * 16 : (size_t)wrow * nb * 16);
+    }
+    // f16 scales of this wavefront's 32 rows: lane -> (group lane/16, block (lane/4)%4, dword lane%4)
     const int ngroups = (n_out + 7) / 8;
     int dg = (row0 >> 3) + (lane >> 4);
     dg = dg < ngroups ? dg : ngroups - 1;
     const char *d_grp = reinterpret_cast<const char *>(d_any) + (size_t)dg * nb * 16 + (lane & 3) * 4;
-    const int d_jb = (lane >> 2) & 3;  // the block of the stage this lane fetches scales of
+    const int d_jb = (lane >> 2) & 3;
 
     const int b_begin = blockIdx.z * chunk;
     const int b_end = b_begin + chunk < nb ? b_begin + chunk : nb;
@@ -170,58 +200,61 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     auto issue = [&](auto ring_slot, int s) {
         const int b0 = b_begin + s * NBU;
         char *base = lds + decltype(ring_slot)::value * STAGE;
-        {   // token digits of blocks b0 .. b0+3: this wavefront fills block j = wave, both planes
-            const int b = b0 + wave < b_end ? b0 + wave : b_end - 1;
+        auto blk = [&](int j) { return (size_t)(b0 + j < b_end ? b0 + j : b_end - 1); };  // past the end: a valid, unused block
 #pragma unroll
-            for (int p = 0; p < 2; ++p)
-                __builtin_amdgcn_global_load_lds((gptr_t)(dig_row + (((size_t)p * nb + b) * 2 + hh) * 16),
-                                                 (lptr_t)(base + (wave * 2 + p) * 1024), 16, 0, 0);
-        }
-        {   // f16 scales of this wavefront's 32 rows: lane -> (group lane/16, block (lane/4)%4, dword lane%4)
-            const int b = b0 + d_jb < b_end ? b0 + d_jb : b_end - 1;
-            __builtin_amdgcn_global_load_lds((gptr_t)(d_grp + (size_t)b * 16), (lptr_t)(base + OFF_D + wave * 256), 4, 0, 0);
-        }
-        // xs[token][b0 .. b0+3]; the four wavefronts write the same bytes to the same place
-        __builtin_amdgcn_global_load_lds((gptr_t)(xs_row + b0), (lptr_t)(base + OFF_XS), 16, 0, 0);
+        for (int u = 0; u < 2; ++u)
+            __builtin_amdgcn_global_load_lds((gptr_t)(dig_src[u] + blk(dig_jb[u]) * 32), (lptr_t)(base + (2 * wave + u) * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(d_grp + blk(d_jb) * 16), (lptr_t)(base + OFF_D + wave * 256), 4, 0, 0);
+        if (lane < 8)
+            __builtin_amdgcn_global_load_lds((gptr_t)(xs_src + b0), (lptr_t)(base + OFF_XS + wave * 128), 16, 0, 0);
 #pragma unroll
-        for (int j = 0; j < NBU; ++j) {
-            const int b = b0 + j < b_end ? b0 + j : b_end - 1;
-            __builtin_amdgcn_global_load_lds((gptr_t)(w_row + (size_t)b * 16), (lptr_t)(base + OFF_W + (wave * NBU + j) * 1024),
-                                             16, 0, 0);
-        }
+        for (int q = 0; q < W_FILLS; ++q)
+            __builtin_amdgcn_global_load_lds((gptr_t)(w_src[q] + blk(w_jb) * 16), (lptr_t)(base + OFF_W + wave * W_WAVE + q * 1024), 16, 0, 0);
     };
 
     float acc[16];
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
 
-    auto block_step = [&](const char *base, int j, float sj) {
-        const v4i bhi = *reinterpret_cast<const v4i *>(base + (j * 2 + 0) * 1024 + lane * 16);
-        const v4i blo = *reinterpret_cast<const v4i *>(base + (j * 2 + 1) * 1024 + lane * 16);
-        v4i a = *reinterpret_cast<const v4i *>(base + OFF_W + (wave * NBU + j) * 1024 + lane * 16);
+    // One block of the stage at `base`: operands from LDS, two MFMAs, scale-and-accumulate.
+    // Split into three phases so that the full-stage path can overlap them across blocks.
+    const int w_rd = OFF_W + wave * W_WAVE + (QT == 8 ? lane : l31) * 64, w_sw = ((QT == 8 ? lane : l31) >> 1) & 3;
+    const int dig_rd = l31 * 256, dig_sw = l31 & 7;
+    auto read_ab = [&](const char *base, int j, v4i (&ab)[3]) {
+        ab[0] = *reinterpret_cast<const v4i *>(base + w_rd + ((j ^ w_sw) * 16));
+        ab[1] = *reinterpret_cast<const v4i *>(base + dig_rd + (((2 * j + hh) ^ dig_sw) * 16));
+        ab[2] = *reinterpret_cast<const v4i *>(base + dig_rd + 128 + (((2 * j + hh) ^ dig_sw) * 16));
+    };
+    auto read_d = [&](const char *base, int j, v2i (&dd)[4]) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)  // rows 8g + 4*hh + {0..3}  <->  accumulator registers 4g .. 4g+3
+            dd[g] = *reinterpret_cast<const v2i *>(base + OFF_D + wave * 256 + (g * 4 + j) * 16 + hh * 8);
+    };
+    auto mfmas = [&](const v4i (&ab)[3], v16i &ihi, v16i &ilo) {
+        v4i a = ab[0];
         if constexpr (QT == 4) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) a[t] = nibbles_to_i8(a[t], 4 * hh);
+            for (int t = 0; t < 4; ++t) a[t] = nibbles_to_i8x16(a[t], 4 - 4 * hh);
         }
         v16i zero;
 #pragma unroll
         for (int r = 0; r < 16; ++r) zero[r] = 0;
-        const v16i ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi, zero, 0, 0, 0);
-        const v16i ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo, zero, 0, 0, 0);
+        ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, ab[1], zero, 0, 0, 0);
+        ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, ab[2], zero, 0, 0, 0);
+    };
+    auto scale_acc = [&](const v16i &ihi, const v16i &ilo, const v2i (&dd)[4], float sj) {
+        if constexpr (QT == 4) sj *= 0.0625f;  // the weight operand was 16 * (q - 8)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            // rows 8g + 4*hh + {0..3}  <->  accumulator registers 4g .. 4g+3
-            const v2i dd = *reinterpret_cast<const v2i *>(base + OFF_D + wave * 256 + (g * 4 + j) * 16 + hh * 8);
+        for (int g = 0; g < 4; ++g)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int r = 4 * g + q;
-                const uint32_t pairbits = (uint32_t)dd[q >> 1];
+                const uint32_t pairbits = (uint32_t)dd[g][q >> 1];
                 const float dv = half_bits_to_float((q & 1) ? pairbits >> 16 : pairbits & 0xFFFFu);
-                // |integer| < 2^28: rounded to 24 bits, then scaled (two roundings of 2^-24, far below the digit step)
+                // |integer| < 2^31: rounded to 24 bits, then scaled (two roundings of 2^-24, far below the digit step)
                 const float fx = (float)(ihi[r] * 256 + ilo[r]) * sj;
                 acc[r] = fmaf(dv, fx, acc[r]);
             }
-        }
     };
     auto compute = [&](auto ring_slot, int s) {
         const int b0 = b_begin + s * NBU;
@@ -232,21 +265,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         // (element -> named int -> float: a bit cast applied directly to a vector element
         // expression was compiled as a cast of element 0)
         const int sx0 = sxi[0], sx1 = sxi[1], sx2 = sxi[2], sx3 = sxi[3];
-        const float4 sx = make_float4(__int_as_float(sx0), __int_as_float(sx1), __int_as_float(sx2), __int_as_float(sx3));
+        const float sx[4] = {__int_as_float(sx0), __int_as_float(sx1), __int_as_float(sx2), __int_as_float(sx3)};
+        v4i ab[2][3];
+        v2i dd[2][4];
+        v16i ihi[2], ilo[2];
         if (b0 + NBU <= b_end) {  // full stage (wavefront-uniform)
-            block_step(base, 0, sx.x);
-            block_step(base, 1, sx.y);
-            block_step(base, 2, sx.z);
-            block_step(base, 3, sx.w);
+            // Software pipeline over the 4 blocks: while block j is scaled and accumulated on
+            // the vector ALU, the MFMAs of block j+1 run and the LDS reads of block j+2 return.
+            read_ab(base, 0, ab[0]);
+            read_d(base, 0, dd[0]);
+            read_ab(base, 1, ab[1]);
+            mfmas(ab[0], ihi[0], ilo[0]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < NBU; ++j) {
+                if (j + 1 < NBU) {
+                    mfmas(ab[(j + 1) & 1], ihi[(j + 1) & 1], ilo[(j + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);  // younger LDS reads must not be waited for here
+                    read_d(base, j + 1, dd[(j + 1) & 1]);
+                }
+                if (j + 2 < NBU) read_ab(base, j + 2, ab[j & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                scale_acc(ihi[j & 1], ilo[j & 1], dd[j & 1], sx[j]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         } else {
-            block_step(base, 0, sx.x);
-            if (b0 + 1 < b_end) block_step(base, 1, sx.y);
-            if (b0 + 2 < b_end) block_step(base, 2, sx.z);
+#pragma unroll
+            for (int j = 0; j < NBU - 1; ++j)
+                if (b0 + j < b_end) {
+                    read_ab(base, j, ab[0]);
+                    read_d(base, j, dd[0]);
+                    mfmas(ab[0], ihi[0], ilo[0]);
+                    scale_acc(ihi[0], ilo[0], dd[0], sx[j]);
+                }
         }
     };
 
     auto wait_barrier = [&](bool one_ahead) {
-        if (one_ahead) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n s_barrier" ::"n"(LPS) : "memory");
+        if (one_ahead) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n s_barrier" ::"n"(MMCfg<QT>::LPS) : "memory");
         else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n s_barrier" ::: "memory");
     };
 
@@ -347,7 +403,7 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
     const dim3 grid(grid_for(n_out, 128), (unsigned)gy, (unsigned)ks);
     float *dst = ks > 1 ? part : y;
     const size_t stride = total_pairs * n_out;
-    constexpr size_t lds = (size_t)RING * STAGE;
+    const size_t lds = (size_t)RING * (ggml_type == PG_GGML_Q4_0 ? MMCfg<4>::STAGE : MMCfg<8>::STAGE);
     static bool attr_set[2] = {false, false};  // per kernel instantiation
     auto launch = [&](auto kern, const char *name) -> pg_status {
         bool &attr_done = attr_set[ggml_type == PG_GGML_Q4_0 ? 0 : 1];

@@ -35,6 +35,11 @@ struct pg_ctx {
     bool profiling;                     // per-kernel HIP events (pg_profile_begin/end)
     std::vector<pg_prof_rec> prof;      // one record per launch while profiling
     std::vector<pg_prof_total> totals;  // aggregated by pg_profile_end
+    // MoE expert pointer tables: the last set uploaded, kept so that repeated calls with the
+    // same experts neither copy nor synchronise.
+    std::vector<const void *> moe_tab_host;
+    void *moe_tab_dev = nullptr;
+    size_t moe_tab_cap = 0;
 };
 
 // Device-resident quantised weight, K-contiguous and zero-padded:

@@ -121,7 +121,6 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     // Arena layout.
     const int ks_up = pg_gguf_mm_splitk(ctx, ffn, d, E, nullptr), ks_down = pg_gguf_mm_splitk(ctx, d, ffn, E, nullptr);
     const size_t part_floats = std::max(ks_up > 1 ? (size_t)ks_up * P * ffn : 0, ks_down > 1 ? (size_t)ks_down * P * d : 0);
-    const size_t sz_tab = pg_round_up(6 * E * sizeof(void *), 256);
     const size_t sz_idx = pg_round_up(P * sizeof(int), 256);
     const size_t sz_p = pg_round_up(P * sizeof(float), 256);
     const size_t sz_lists = pg_round_up(E * T * sizeof(int), 256), sz_counts = pg_round_up(E * sizeof(int), 256);
@@ -130,9 +129,8 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     const size_t sz_part = pg_round_up(part_floats * sizeof(float), 256);
     const size_t sz_xd = pg_mmdigits_bytes(T, d), sz_hd = pg_mmdigits_bytes(P, ffn);
     void *ws = nullptr;
-    PG_TRY(pg_workspace(ctx, sz_tab + sz_idx + sz_p + sz_lists + sz_counts + 3 * sz_act + sz_y + sz_part + sz_xd + sz_hd, &ws));
+    PG_TRY(pg_workspace(ctx, sz_idx + sz_p + sz_lists + sz_counts + 3 * sz_act + sz_y + sz_part + sz_xd + sz_hd, &ws));
     char *p = static_cast<char *>(ws);
-    const void **tab = reinterpret_cast<const void **>(p); p += sz_tab;
     int *topk_idx = reinterpret_cast<int *>(p); p += sz_idx;
     float *topk_p = reinterpret_cast<float *>(p); p += sz_p;
     int *lists = reinterpret_cast<int *>(p); p += sz_lists;
@@ -145,16 +143,30 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     const pg_mmdigits xd = pg_mmdigits_carve(p, T, d); p += sz_xd;
     const pg_mmdigits hd = pg_mmdigits_carve(p, P, ffn);
 
-    // Expert pointer tables: [gate qs | gate d | up qs | up d | down qs | down d], E each.
+    // Expert pointer tables: [gate qs | gate d | up qs | up d | down qs | down d], E each, in a
+    // device buffer the context keeps; uploaded (with a wait, the source is this stack frame)
+    // only when the set of experts differs from the previous call's.
     const void *host_tab[6 * MAX_EXPERTS];
     for (size_t e = 0; e < E; ++e) {
         host_tab[0 * E + e] = gate[e]->qs; host_tab[1 * E + e] = gate[e]->d;
         host_tab[2 * E + e] = up[e]->qs;   host_tab[3 * E + e] = up[e]->d;
         host_tab[4 * E + e] = down[e]->qs; host_tab[5 * E + e] = down[e]->d;
     }
-    PG_HIP(hipMemcpyAsync(tab, host_tab, 6 * E * sizeof(void *), hipMemcpyHostToDevice, ctx->stream));
-    // host_tab lives on this stack frame: the copy must have left it before we return.
-    PG_HIP(hipStreamSynchronize(ctx->stream));
+    if (ctx->moe_tab_host.size() != 6 * E || memcmp(ctx->moe_tab_host.data(), host_tab, 6 * E * sizeof(void *)) != 0) {
+        PG_HIP(hipStreamSynchronize(ctx->stream));  // earlier calls may still read the old table
+        if (ctx->moe_tab_cap < 6 * E * sizeof(void *)) {
+            if (ctx->moe_tab_dev) PG_HIP(hipFree(ctx->moe_tab_dev));
+            ctx->moe_tab_dev = nullptr;
+            ctx->moe_tab_cap = 0;
+            PG_HIP(hipMalloc(&ctx->moe_tab_dev, 6 * MAX_EXPERTS * sizeof(void *)));
+            ctx->moe_tab_cap = 6 * MAX_EXPERTS * sizeof(void *);
+        }
+        ctx->moe_tab_host.clear();
+        PG_HIP(hipMemcpyAsync(ctx->moe_tab_dev, host_tab, 6 * E * sizeof(void *), hipMemcpyHostToDevice, ctx->stream));
+        PG_HIP(hipStreamSynchronize(ctx->stream));
+        ctx->moe_tab_host.assign(host_tab, host_tab + 6 * E);
+    }
+    const void **tab = static_cast<const void **>(ctx->moe_tab_dev);
 
     PG_TRY(pg_launch(ctx, "moe_route_topk", route_topk_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
                      router_logits_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
