@@ -59,7 +59,7 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__res
     constexpr int STAGE = (BM + BN) * BK;            // bytes per LDS stage
     constexpr int KS = BK / 32;                      // k-steps per stage
     constexpr int NF = TM + TN, NMFMA = TM * TN;
-    static_assert(LA >= 1 && LB >= 1 && KS % 2 == 0, "unsupported tile configuration");
+    static_assert(LA >= 1 && LB >= 1 && KS % 2 == 0 && BM <= 64 * NW && BN <= 64 * NW, "unsupported tile configuration");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
     // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous
@@ -100,6 +100,15 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__res
         b_off[ks] = BM * BK + rb * BK + (((2 * ks + half) ^ swz<BK>(rb)) * 16);
     }
 
+    // The scales of this tile's rows and columns go to LDS (behind the stages) now, so that
+    // the epilogue does not start with dependent global round trips.
+    float *lds_as = reinterpret_cast<float *>(lds + NST * STAGE), *lds_ws = lds_as + BM;
+    {
+        const int t = threadIdx.x;
+        if (t < BM) lds_as[t] = a_scales[m0 + t < M ? m0 + t : M - 1];
+        if (t < BN) lds_ws[t] = w_scales[n0 + t < N ? n0 + t : N - 1];
+    }
+
     v16i acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -136,11 +145,17 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__res
     // `ahead` of its youngest stage fills have landed (vmcnt).  After it, every wavefront's
     // share of the awaited stage is in LDS and the stage just consumed may be refilled.
     auto wait_barrier = [&](int ahead) {
-        if (ahead <= 0) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n s_barrier" ::: "memory");
-        else if (ahead == 1) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n s_barrier" ::"n"(LPS) : "memory");
-        else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n s_barrier" ::"n"(2 * LPS > 63 ? 63 : 2 * LPS) : "memory");
+#define PG_WB(N) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n s_barrier" ::"n"((N) * LPS > 63 ? 63 : (N) * LPS) : "memory")
+        switch (ahead) {
+            case 1: PG_WB(1); break;
+            case 2: PG_WB(2); break;
+            case 3: PG_WB(3); break;
+            case 4: PG_WB(4); break;
+            default: asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n s_barrier" ::: "memory"); break;
+        }
+#undef PG_WB
     };
-    static_assert(NST >= 2 && NST <= 4, "wait_barrier covers up to 2 stages in flight beyond the awaited one");
+    static_assert(NST >= 2 && NST <= 6, "wait_barrier covers up to 4 stages in flight beyond the awaited one");
 
     const int KT = K / BK;
 #pragma unroll
@@ -187,26 +202,21 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__res
     }
 
     // ---- epilogue.  Accumulator register r of a 32x32 tile holds
-    // row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
+    // row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.  (The scales were requested before the
+    // K loop: loading them here would put several dependent memory round trips on every tile.)
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        float as[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = m0 + wm * WM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
-            as[r] = a_scales[m < M ? m : M - 1];
-        }
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const int n = n0 + wn * WN + 32 * j + l31;
             if (n < N) {
-                const float ws = w_scales[n];
+                const float ws = lds_ws[wn * WN + 32 * j + l31];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int m = m0 + wm * WM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
                     if (m < M) {
                         const int a = acc[i][j][r];
-                        out[(size_t)m * N + n] = (float)a * as[r] * ws;
+                        out[(size_t)m * N + n] = (float)a * lds_as[wm * WM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3)] * ws;
                         if (acc_out) acc_out[(size_t)m * N + n] = a;
                     }
                 }
@@ -222,7 +232,7 @@ pg_status launch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *
     const int tiles_m = (int)((m + BM - 1) / BM);
     const int tiles_n = (int)((w->cols + BN - 1) / BN);
     const int ntiles = tiles_m * tiles_n;
-    const size_t lds = (size_t)NST * (BM + BN) * BK;
+    const size_t lds = (size_t)NST * (BM + BN) * BK + (BM + BN) * sizeof(float);
     auto kern = gemm_w8a8_kernel<BM, BN, BK, NST, NWM, NWN, OCC>;
     static bool attr_done = false;  // per instantiation
     if (!attr_done) {

@@ -312,9 +312,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #define PG_MM_STEP(U)                                                                     \
         if (s0 + U < nst) {                                                               \
             const int s = s0 + U;                                                         \
-            wait_barrier(s + 1 < nst);                                                    \
+            wait_barrier(s + 1 < nst);                       \
             if (s + 2 < nst) issue(std::integral_constant<int, (U + 2) % RING>{}, s + 2); \
-            compute(std::integral_constant<int, U>{}, s);                                 \
+            compute(std::integral_constant<int, U>{}, s);          \
         }
         PG_MM_STEP(0)
         PG_MM_STEP(1)
@@ -379,7 +379,9 @@ pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows,
 int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t groups, int *chunk_out) {
     const size_t nb = k_in / 32;
     const size_t wgs = ((n_out + 127) / 128) * (groups ? groups : 1);
-    size_t ks = (2 * (size_t)ctx->num_cu + wgs - 1) / wgs;
+    // Two workgroups fit on a CU.  Split K only as far as every workgroup is still resident
+    // at once: a second round of workgroups would pay the start-up latency again.
+    size_t ks = 2 * (size_t)ctx->num_cu / wgs;
     if (ks > 8) ks = 8;
     if (ks < 1) ks = 1;
     size_t chunk = pg_round_up((nb + ks - 1) / ks, NBU);
