@@ -47,16 +47,22 @@ __global__ __launch_bounds__(QA_THREADS) void quantize_rows_vec4_kernel(
     const size_t row = blockIdx.x;
     const float4 *ar = reinterpret_cast<const float4 *>(a + row * cols);
     const int nvec = (int)(cols >> 2);
+    // Every load is issued before anything waits: vectors past the end of the row re-read
+    // the last one (no branch between the loads) and are left out of the maximum.
     float4 v[MAXV];
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+        const int idx = threadIdx.x + i * QA_THREADS;
+        typedef float f4v __attribute__((ext_vector_type(4)));
+        const f4v t = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(ar) + (idx < nvec ? idx : nvec - 1));
+        v[i] = make_float4(t.x, t.y, t.z, t.w);
+    }
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < MAXV; ++i) {
         const int idx = threadIdx.x + i * QA_THREADS;
-        if (idx < nvec) {
-            v[i] = ar[idx];
-            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)),
-                                     fmaxf(fabsf(v[i].z), fabsf(v[i].w))));
-        }
+        const float m4 = fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)), fmaxf(fabsf(v[i].z), fabsf(v[i].w)));
+        amax = fmaxf(amax, idx < nvec ? m4 : 0.0f);
     }
     amax = block_max_256(amax, red);
     const float scale = (amax == 0.0f) ? 1.0f : amax / 127.0f;
@@ -245,12 +251,14 @@ pg_status pg_launch_quantize_activations(pg_ctx *ctx, const float *a, size_t row
                         ((uintptr_t)a % 16 == 0) && ((uintptr_t)q % 4 == 0) && cols > 0;
     const size_t nvec = cols / 4;
     const dim3 grid((unsigned)rows);
-    if (vec_ok && nvec <= 4 * QA_THREADS)
-        PG_TRY(pg_launch(ctx, "quantize_rows", quantize_rows_vec4_kernel<4>, grid, dim3(QA_THREADS), 0, a, cols, q,
+#define PG_QROWS(V)                                                                                      \
+    else if (vec_ok && nvec <= (V) * QA_THREADS)                                                         \
+        PG_TRY(pg_launch(ctx, "quantize_rows", quantize_rows_vec4_kernel<V>, grid, dim3(QA_THREADS), 0, a, cols, q, \
                          q_stride, row_scales));
-    else if (vec_ok && nvec <= 16 * QA_THREADS)
-        PG_TRY(pg_launch(ctx, "quantize_rows", quantize_rows_vec4_kernel<16>, grid, dim3(QA_THREADS), 0, a, cols, q,
-                         q_stride, row_scales));
+    if (cols == 0) PG_TRY(pg_launch(ctx, "quantize_rows", quantize_rows_generic_kernel, grid, dim3(QA_THREADS), 0, a, cols, q,
+                                    q_stride, row_scales));
+    PG_QROWS(2) PG_QROWS(4) PG_QROWS(6) PG_QROWS(8) PG_QROWS(11) PG_QROWS(14) PG_QROWS(16)
+#undef PG_QROWS
     else
         PG_TRY(pg_launch(ctx, "quantize_rows", quantize_rows_generic_kernel, grid, dim3(QA_THREADS), 0, a, cols, q,
                          q_stride, row_scales));
