@@ -145,12 +145,13 @@ def main():
     prof = profiled(prefill_step, args.steps)
     gemm_avg_ms, g_n = prof["gemm_w8a8"]
     q_avg_ms, q_n = prof["quantize_rows"]
-    gemm_tops = (LAYER_OPS / len(LAYER)) / (gemm_avg_ms * 1e-3) / 1e12
+    gemm_lps = g_n / args.steps  # GEMM launches per step (a product may run as two column panels)
+    gemm_tops = (LAYER_OPS / gemm_lps) / (gemm_avg_ms * 1e-3) / 1e12
     quant_bytes = sum(M_PREFILL * k * 4 + M_PREFILL * k + M_PREFILL * 4 for _, k, _ in LAYER)
-    roofline = {"kernel": "gemm_w8a8_kernel (i8 MFMA 32x32x32, all 7 shapes)", "bound": "mfma",
+    roofline = {"kernel": "gemm_w8a8_kernel (i8 MFMA 32x32x32, all 7 products)", "bound": "mfma",
                 "achieved": round(gemm_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
                 "frac": round(gemm_tops / PEAK_INT8_TOPS, 4), "traffic": traffic_for("gemm_w8a8"),
-                "ops_per_launch": LAYER_OPS // len(LAYER), "avg_launch_ms": round(gemm_avg_ms, 4),
+                "ops_per_launch": int(LAYER_OPS / gemm_lps), "launches_per_step": gemm_lps, "avg_launch_ms": round(gemm_avg_ms, 4),
                 "note": "unit counts int8 multiply-adds as 2 ops (TOP/s); duration from the HIP events "
                         "attached to each dispatch"}
     act_quant = {"kernel": "quantize_rows_vec4_kernel", "bound": "hbm",
