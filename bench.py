@@ -279,7 +279,7 @@ def main():
                        "kernels_ms": {k: round(v[0], 5) for k, v in prof.items()},
                        "roofline": {"kernel": "gguf_mm_kernel<Q4_0>", "bound": "hbm",
                                     "achieved": round(mm_bytes / (k_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                    "frac": round(mm_bytes / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None,
+                                    "frac": round(mm_bytes / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": traffic_for("gguf_mm_q4_0"),
                                     "bytes_per_launch": mm_bytes, "avg_launch_ms": round(k_ms, 5)}})
     for h in q4:
         lib.pg_gguf_free(ctx.handle, h)
@@ -323,7 +323,7 @@ def main():
            "roofline": {"kernel": "gguf_mm_kernel<Q8_0> (gate, up, down)", "bound": "hbm",
                         "achieved": round(3 * E_moe * nblk * 34 / (mm_total * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                         "unit": "GB/s", "frac": round(3 * E_moe * nblk * 34 / (mm_total * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                        "traffic": None, "bytes_per_launch": E_moe * nblk * 34,
+                        "traffic": traffic_for("gguf_mm_q8_0"), "bytes_per_launch": E_moe * nblk * 34,
                         "avg_launch_ms": round(prof["gguf_mm_q8_0"][0], 5)}}
     for w3 in experts:
         for h in w3:
