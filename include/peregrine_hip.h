@@ -163,6 +163,44 @@ pg_status pg_gguf_matmul(pg_ctx *ctx, const float *x, size_t m, const pg_gguf_te
 pg_status pg_gguf_matmul_dev(pg_ctx *ctx, const float *x_dev, size_t m,
                              const pg_gguf_tensor *w, float *y_dev);
 
+/* ---- GGUF container (gguf::GgufFile, src/gguf.rs:403-561) ---------------------
+ * Parsing needs no device.  A malformed or truncated file is PG_EINVAL (the reference
+ * returns io::Error for a bad magic/version and panics on the rest). */
+typedef struct pg_gguf_file pg_gguf_file;
+/* GgufFile::parse  src/gguf.rs:411-483.  `data` is borrowed and must outlive the handle. */
+pg_status pg_gguf_file_parse(const void *data, size_t len, pg_gguf_file **out);
+/* GgufFile::load  src/gguf.rs:405-408 (the file is memory-mapped, not read). */
+pg_status pg_gguf_file_open(const char *path, pg_gguf_file **out);
+void pg_gguf_file_close(pg_gguf_file *f);
+/* metadata.len(), tensors.len(), header version, offset of the data section. */
+pg_status pg_gguf_file_counts(const pg_gguf_file *f, size_t *n_tensors, size_t *n_metadata,
+                              uint32_t *version, uint64_t *data_start);
+/* GgufFile::tensor_names  src/gguf.rs:559-561 (file order). */
+pg_status pg_gguf_file_tensor_name(const pg_gguf_file *f, size_t index, const char **name);
+/* GgufTensor {dtype, shape, data_offset} + data_size()  src/gguf.rs:143-164.  shape is in
+ * GGUF order (innermost first; tensor_shape() reverses it, src/gguf.rs:551-556);
+ * data points into the parsed buffer.  Any output may be NULL. */
+pg_status pg_gguf_file_tensor_info(const pg_gguf_file *f, const char *name, int *ggml_type,
+                                   size_t *n_dims, uint64_t *shape, size_t shape_cap,
+                                   uint64_t *data_offset, size_t *data_size, const void **data);
+/* GgufFile::get_u32 / get_f32  src/gguf.rs:541-548, MetadataValue::as_str / arrays
+ * src/gguf.rs:95-139.  *found = 0 (or *value = NULL, *count = (size_t)-1) when the key is
+ * absent or of another type. */
+pg_status pg_gguf_file_get_u32(const pg_gguf_file *f, const char *key, uint32_t *value, int *found);
+pg_status pg_gguf_file_get_f32(const pg_gguf_file *f, const char *key, float *value, int *found);
+pg_status pg_gguf_file_get_str(const pg_gguf_file *f, const char *key, const char **value, size_t *len);
+pg_status pg_gguf_file_get_array(const pg_gguf_file *f, const char *key, uint32_t *elem_type, size_t *count);
+pg_status pg_gguf_file_get_array_str(const pg_gguf_file *f, const char *key, size_t index, const char **value);
+pg_status pg_gguf_file_get_array_f64(const pg_gguf_file *f, const char *key, double *values, size_t cap);
+/* GgufFile::load_tensor_f32  src/gguf.rs:485-517 (F32, F16, Q8_0, Q4_0, Q4_1 -> f32). */
+pg_status pg_gguf_file_load_tensor_f32(pg_ctx *ctx, const pg_gguf_file *f, const char *name,
+                                       float *out, size_t out_cap);
+/* The keep-quantised route: a 1-D or 2-D Q4_0 / Q8_0 tensor goes to the device as it is
+ * (pg_gguf_upload with n_out = shape[1], k_in = shape[0]) instead of through
+ * load_tensor_f32 + transpose  src/models/llama/model.rs:243-257. */
+pg_status pg_gguf_file_upload_tensor(pg_ctx *ctx, const pg_gguf_file *f, const char *name,
+                                     pg_gguf_tensor **out);
+
 /* ---- grouped MoE expert FFN ------------------------------------------------- */
 
 /* MoELayer::forward after the router matmul  examples/grok1/moe.rs:70-109

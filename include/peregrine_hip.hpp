@@ -221,6 +221,74 @@ private:
     size_t n_out_ = 0, k_in_ = 0;
 };
 
+// gguf::GgufFile  src/gguf.rs:166-171, 403-561.  parse() borrows the buffer; load() maps the file.
+class GgufFile {
+public:
+    static GgufFile parse(const std::vector<uint8_t> &data) {
+        pg_gguf_file *f = nullptr;
+        check(pg_gguf_file_parse(data.data(), data.size(), &f), "GgufFile::parse");
+        return GgufFile(f);
+    }
+    static GgufFile load(const std::string &path) {
+        pg_gguf_file *f = nullptr;
+        check(pg_gguf_file_open(path.c_str(), &f), "GgufFile::load");
+        return GgufFile(f);
+    }
+    ~GgufFile() { pg_gguf_file_close(f_); }
+    GgufFile(GgufFile &&o) noexcept : f_(o.f_) { o.f_ = nullptr; }
+    GgufFile(const GgufFile &) = delete;
+    GgufFile &operator=(const GgufFile &) = delete;
+
+    std::vector<std::string> tensor_names() const {  // src/gguf.rs:559-561
+        size_t n = 0;
+        check(pg_gguf_file_counts(f_, &n, nullptr, nullptr, nullptr), "GgufFile::tensor_names");
+        std::vector<std::string> out;
+        for (size_t i = 0; i < n; ++i) {
+            const char *nm = nullptr;
+            check(pg_gguf_file_tensor_name(f_, i, &nm), "GgufFile::tensor_names");
+            out.emplace_back(nm);
+        }
+        return out;
+    }
+    // Peregrine order: GGUF's shape reversed  src/gguf.rs:551-556
+    std::vector<size_t> tensor_shape(const std::string &name) const {
+        uint64_t shape[8];
+        size_t nd = 0;
+        check(pg_gguf_file_tensor_info(f_, name.c_str(), nullptr, &nd, shape, 8, nullptr, nullptr, nullptr), "GgufFile::tensor_shape");
+        std::vector<size_t> out;
+        for (size_t i = nd; i-- > 0;) out.push_back((size_t)shape[i]);
+        return out;
+    }
+    bool get_u32(const std::string &key, uint32_t *v) const {  // src/gguf.rs:541-543
+        int found = 0;
+        check(pg_gguf_file_get_u32(f_, key.c_str(), v, &found), "GgufFile::get_u32");
+        return found != 0;
+    }
+    bool get_f32(const std::string &key, float *v) const {  // src/gguf.rs:546-548
+        int found = 0;
+        check(pg_gguf_file_get_f32(f_, key.c_str(), v, &found), "GgufFile::get_f32");
+        return found != 0;
+    }
+    std::vector<float> load_tensor_f32(const GpuContext &gpu, const std::string &name) const {  // src/gguf.rs:485-517
+        size_t n = 1;
+        for (size_t d : tensor_shape(name)) n *= d;
+        std::vector<float> out(n);
+        check(pg_gguf_file_load_tensor_f32(gpu.raw(), f_, name.c_str(), out.data(), n), "GgufFile::load_tensor_f32");
+        return out;
+    }
+    quant::QuantizedTensor load_tensor_q8(const GpuContext &gpu, const std::string &name) const {  // src/gguf.rs:521-537
+        const std::vector<size_t> shape = tensor_shape(name);  // [rows, cols] after the reversal
+        if (shape.size() != 1 && shape.size() != 2) throw Panic(PG_EINVAL, "expected 1D or 2D tensor for q8 load");
+        const size_t rows = shape.size() == 2 ? shape[0] : 1, cols = shape.back();
+        return quant::quantize_weights(gpu, load_tensor_f32(gpu, name), rows, cols);
+    }
+    const pg_gguf_file *raw() const { return f_; }
+
+private:
+    explicit GgufFile(pg_gguf_file *f) : f_(f) {}
+    pg_gguf_file *f_;
+};
+
 }  // namespace gguf
 
 namespace moe {

@@ -56,6 +56,21 @@ SIGNATURES = {
     "pg_gguf_free": [_vp, _vp],
     "pg_gguf_matmul": [_vp, _vp, _sz, _vp, _vp],
     "pg_gguf_matmul_dev": [_vp, _vp, _sz, _vp, _vp],
+    "pg_gguf_file_parse": [_vp, _sz, _pp],
+    "pg_gguf_file_open": [C.c_char_p, _pp],
+    "pg_gguf_file_close": [_vp],
+    "pg_gguf_file_counts": [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(C.c_uint32), C.POINTER(C.c_uint64)],
+    "pg_gguf_file_tensor_name": [_vp, _sz, C.POINTER(C.c_char_p)],
+    "pg_gguf_file_tensor_info": [_vp, C.c_char_p, C.POINTER(_int), C.POINTER(_sz), C.POINTER(C.c_uint64), _sz,
+                                 C.POINTER(C.c_uint64), C.POINTER(_sz), _pp],
+    "pg_gguf_file_get_u32": [_vp, C.c_char_p, C.POINTER(C.c_uint32), C.POINTER(_int)],
+    "pg_gguf_file_get_f32": [_vp, C.c_char_p, C.POINTER(C.c_float), C.POINTER(_int)],
+    "pg_gguf_file_get_str": [_vp, C.c_char_p, C.POINTER(C.c_char_p), C.POINTER(_sz)],
+    "pg_gguf_file_get_array": [_vp, C.c_char_p, C.POINTER(C.c_uint32), C.POINTER(_sz)],
+    "pg_gguf_file_get_array_str": [_vp, C.c_char_p, _sz, C.POINTER(C.c_char_p)],
+    "pg_gguf_file_get_array_f64": [_vp, C.c_char_p, C.POINTER(C.c_double), _sz],
+    "pg_gguf_file_load_tensor_f32": [_vp, _vp, C.c_char_p, _vp, _sz],
+    "pg_gguf_file_upload_tensor": [_vp, _vp, C.c_char_p, _pp],
     "pg_moe_ffn": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
     "pg_moe_ffn_dev": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
 }
@@ -63,6 +78,7 @@ _OTHER_RESTYPE = {
     "pg_ctx_destroy": None,
     "pg_qtensor_free": None,
     "pg_gguf_free": None,
+    "pg_gguf_file_close": None,
     "pg_ctx_stream": _vp,
     "pg_last_error": C.c_char_p,
     "pg_status_string": C.c_char_p,

@@ -69,3 +69,50 @@ def assert_close_rel(got, ref, rtol, what=""):
     worst = int(np.argmax(err - bound)) if ref.size else 0
     assert (err <= bound).all(), (
         f"{what}: element {worst}: got {got[worst]!r}, want {ref[worst]!r}, err {err[worst]:.3e} > {bound[worst]:.3e}")
+
+
+# ---- a GGUF writer for the container tests (format: reference src/gguf.rs:411-483) ----
+GGUF_TYPE_CODES = {"u8": 0, "i8": 1, "u16": 2, "i16": 3, "u32": 4, "i32": 5, "f32": 6, "bool": 7, "str": 8,
+                   "arr": 9, "u64": 10, "i64": 11, "f64": 12}
+_GGUF_FMT = {"u8": "<B", "i8": "<b", "u16": "<H", "i16": "<h", "u32": "<I", "i32": "<i", "f32": "<f", "bool": "<B",
+             "u64": "<Q", "i64": "<q", "f64": "<d"}
+
+
+def _gguf_str(s):
+    import struct
+    b = s.encode()
+    return struct.pack("<Q", len(b)) + b
+
+
+def _gguf_value(kind, v):
+    import struct
+    if kind == "str":
+        return _gguf_str(v)
+    if kind == "arr":  # v = (element kind, [elements])
+        ek, items = v
+        return struct.pack("<IQ", GGUF_TYPE_CODES[ek], len(items)) + b"".join(_gguf_value(ek, x) for x in items)
+    return struct.pack(_GGUF_FMT[kind], v)
+
+
+def build_gguf(metadata, tensors, version=3, magic=0x46554747):
+    """metadata: list of (key, kind, value); tensors: list of (name, ggml_type, shape_gguf_order, raw_bytes).
+    Returns (file bytes, data_start, {name: offset in data section})."""
+    import struct
+    align = 32
+    for key, kind, v in metadata:
+        if key == "general.alignment":
+            align = int(v)
+    head = struct.pack("<IIQQ", magic, version, len(tensors), len(metadata))
+    for key, kind, v in metadata:
+        head += _gguf_str(key) + struct.pack("<I", GGUF_TYPE_CODES[kind]) + _gguf_value(kind, v)
+    offsets, off = {}, 0
+    for name, typ, shape, raw in tensors:
+        offsets[name] = off
+        head += _gguf_str(name) + struct.pack("<I", len(shape)) + b"".join(struct.pack("<Q", d) for d in shape)
+        head += struct.pack("<IQ", typ, off)
+        off = (off + len(raw) + align - 1) // align * align
+    data_start = (len(head) + align - 1) // align * align
+    body = bytearray(off)
+    for name, typ, shape, raw in tensors:
+        body[offsets[name]: offsets[name] + len(raw)] = raw
+    return head + b"\0" * (data_start - len(head)) + bytes(body), data_start, offsets
