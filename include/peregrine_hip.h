@@ -201,6 +201,24 @@ pg_status pg_gguf_file_load_tensor_f32(pg_ctx *ctx, const pg_gguf_file *f, const
 pg_status pg_gguf_file_upload_tensor(pg_ctx *ctx, const pg_gguf_file *f, const char *name,
                                      pg_gguf_tensor **out);
 
+/* ---- int8 wire record (src/serial.rs:124-222) -------------------------------------
+ * [name_len u32][name][dtype u8 = 1][ndim u32 = 2][rows u32][cols u32][rows*cols i8][cols f32],
+ * little-endian.  Host code, no device needed except for pg_qtensor_from_record. */
+pg_status pg_quantized_record_size(size_t name_len, size_t rows, size_t cols, size_t *bytes);
+/* serial::write_quantized_tensor  src/serial.rs:126-157 into a caller buffer. */
+pg_status pg_write_quantized_tensor(void *buf, size_t cap, const char *name, size_t name_len,
+                                    const int8_t *q, const float *scales, size_t rows, size_t cols,
+                                    size_t *written);
+/* serial::read_quantized_tensor  src/serial.rs:161-222: the outputs point into buf (scales
+ * possibly unaligned); a wrong dtype tag or ndim (the reference's assert_eq!s) and a short
+ * buffer (its read_exact error) are PG_EINVAL. */
+pg_status pg_read_quantized_tensor(const void *buf, size_t len, const char **name, size_t *name_len,
+                                   size_t *rows, size_t *cols, const int8_t **q, const void **scales,
+                                   size_t *consumed);
+/* read_quantized_tensor followed by QuantizedTensor::to_gpu. */
+pg_status pg_qtensor_from_record(pg_ctx *ctx, const void *buf, size_t len, pg_qtensor **out,
+                                 size_t *consumed);
+
 /* ---- grouped MoE expert FFN ------------------------------------------------- */
 
 /* MoELayer::forward after the router matmul  examples/grok1/moe.rs:70-109

@@ -71,6 +71,10 @@ SIGNATURES = {
     "pg_gguf_file_get_array_f64": [_vp, C.c_char_p, C.POINTER(C.c_double), _sz],
     "pg_gguf_file_load_tensor_f32": [_vp, _vp, C.c_char_p, _vp, _sz],
     "pg_gguf_file_upload_tensor": [_vp, _vp, C.c_char_p, _pp],
+    "pg_quantized_record_size": [_sz, _sz, _sz, C.POINTER(_sz)],
+    "pg_write_quantized_tensor": [_vp, _sz, C.c_char_p, _sz, _vp, _vp, _sz, _sz, C.POINTER(_sz)],
+    "pg_read_quantized_tensor": [_vp, _sz, _pp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz), _pp, _pp, C.POINTER(_sz)],
+    "pg_qtensor_from_record": [_vp, _vp, _sz, _pp, C.POINTER(_sz)],
     "pg_moe_ffn": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
     "pg_moe_ffn_dev": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
 }

@@ -233,3 +233,26 @@ def test_prefill_shape_full_size_properties(ctx, orc):
     want, want_acc = orc.matmul_quantized(a[rows], len(rows), k, q_t, s, n)
     assert (acc[rows] == want_acc.reshape(len(rows), n)).all()
     assert (bits(got[rows]) == bits(want.reshape(len(rows), n))).all()
+
+
+def test_wire_record_straight_to_device(ctx, orc):
+    """read_quantized_tensor + to_gpu in one call (reference src/serial.rs:161-222,
+    src/quant.rs:174-181): the device tensor multiplies exactly like the original."""
+    import io
+    import ctypes as C
+    from peregrine_amd import serial, _ffi
+    from peregrine_amd.quant import QuantizedTensor
+    say("wire record -> device tensor")
+    rows, cols, m = 96, 40, 3
+    w = orc.rng_normal(31, rows * cols, 0.0, 0.02)
+    q, q_t, s = orc.quantize_weights(w, rows, cols)
+    buf = io.BytesIO()
+    serial.write_quantized_tensor(buf, "odd", QuantizedTensor(q, q_t, s, rows, cols))  # 3-byte name: unaligned payload
+    h, used = serial.quantized_tensor_to_gpu(buf.getvalue() + b"trailing", ctx)
+    assert used == len(buf.getvalue())
+    a = orc.rng_normal(32, m * rows)
+    out = np.empty(m * cols, np.float32)
+    _ffi.check(_ffi.lib.pg_matmul_quantized(ctx.handle, C.c_void_p(a.ctypes.data), m, rows, h, C.c_void_p(out.ctypes.data)))
+    want, _ = orc.matmul_quantized(a, m, rows, q_t, s, cols)
+    assert (out.view(np.uint32) == want.view(np.uint32)).all()
+    _ffi.lib.pg_qtensor_free(ctx.handle, h)
