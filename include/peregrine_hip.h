@@ -134,6 +134,17 @@ pg_status pg_matmul_quantized(pg_ctx *ctx, const float *a, size_t m, size_t k,
 pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
                                   const pg_qtensor *w, float *out_dev, int32_t *acc_dev);
 
+/* The reference's GPU numerics for the same call (W8A32): f32 activations, weights
+ * dequantised to f32, f32 accumulate, no activation quantisation --
+ * GpuContext::dispatch_matmul_dequant_i8  src/metal/context.rs:2226-2306, shader
+ * matmul_dequant_i8  src/metal/shaders.rs:2329-2375, reached through
+ * quant::matmul_quantized_gpu  src/quant.rs:196-218.
+ * out[m, n] = sum_k a[m, k] * ((w_i8[k, n] as f32) * scale[n]), within 1e-5 relative. */
+pg_status pg_matmul_dequant_i8(pg_ctx *ctx, const float *a, size_t m, size_t k,
+                               const pg_qtensor *w, float *out);
+pg_status pg_matmul_dequant_i8_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
+                                   const pg_qtensor *w, float *out_dev);
+
 /* ---- gguf::* (src/gguf.rs) -------------------------------------------------- */
 
 /* gguf::f16_to_f32  src/gguf.rs:354-382, applied to n values (bit-exact, NaN payloads

@@ -161,6 +161,17 @@ inline GpuBuffer<float> matmul_quantized_gpu(const GpuContext &gpu, const std::v
     return out;
 }
 
+// The reference's GPU numerics (W8A32) for the same product: f32 activations, dequantised
+// weights, f32 accumulate (dispatch_matmul_dequant_i8, src/metal/context.rs:2226-2306).
+inline std::vector<float> matmul_dequant_i8(const GpuContext &gpu, const std::vector<float> &a, size_t m, size_t k, QuantizedTensor &w) {
+    if (w.rows != k) throw Panic(PG_EINVAL, "matmul_dequant_i8: weight rows must equal k");
+    if (a.size() != m * k) throw Panic(PG_EINVAL, "matmul_dequant_i8: a.len() != m * k");
+    w.to_gpu(gpu);
+    std::vector<float> out(m * w.cols);
+    check(pg_matmul_dequant_i8(gpu.raw(), a.data(), m, k, w.gpu_handle(), out.data()), "matmul_dequant_i8");
+    return out;
+}
+
 }  // namespace quant
 
 namespace gguf {

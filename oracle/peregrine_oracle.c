@@ -142,6 +142,28 @@ ORC_API int orc_matmul_quantized(const float *a, size_t m, size_t k,
     return 0;
 }
 
+/* Metal kernel matmul_dequant_i8     reference: src/metal/shaders.rs:2329-2375
+ *   (the numerics behind quant::matmul_quantized_gpu, src/quant.rs:196-218)
+ *   a [m, k] f32; q [k, n] i8 row-major; scales [n]; out [m, n].
+ *   Per output: w = (float)q * scale (one rounding), sum += a * w for k ascending,
+ *   multiply and add rounded separately (tiles of 16 do not change the order).
+ *   Pinned by equality with orc_matmul_f32(a, orc_dequantize(q)), whose two halves
+ *   are pinned on their own. */
+ORC_API void orc_matmul_dequant_i8(const float *a, size_t m, size_t k, const int8_t *q,
+                                   const float *scales, size_t n, float *out) {
+    for (size_t mi = 0; mi < m; ++mi)
+        for (size_t ni = 0; ni < n; ++ni) {
+            const float w_scale = scales[ni];
+            float sum = 0.0f;
+            for (size_t ki = 0; ki < k; ++ki) {
+                const float w = (float)q[ki * n + ni] * w_scale;
+                const float prod = a[mi * k + ki] * w;
+                sum = sum + prod;
+            }
+            out[mi * n + ni] = sum;
+        }
+}
+
 /* ------------------------------------------------------------------------
  * gguf::f16_to_f32                   reference: src/gguf.rs:354-382
  *   Bit-level IEEE half -> single, including the subnormal normalise loop

@@ -47,6 +47,8 @@ SIGNATURES = {
     "pg_qtensor_free": [_vp, _vp],
     "pg_matmul_quantized": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_matmul_quantized_dev": [_vp, _vp, _sz, _sz, _vp, _vp, _vp],
+    "pg_matmul_dequant_i8": [_vp, _vp, _sz, _sz, _vp, _vp],
+    "pg_matmul_dequant_i8_dev": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_f16_to_f32": [_vp, _vp, _sz, _vp],
     "pg_dequant_q8_0": [_vp, _vp, _sz, _vp],
     "pg_dequant_q4_0": [_vp, _vp, _sz, _vp],

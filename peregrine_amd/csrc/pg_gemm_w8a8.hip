@@ -216,7 +216,7 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__res
                     const int m = m0 + wm * WM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
                     if (m < M) {
                         const int a = acc[i][j][r];
-                        out[(size_t)m * N + n] = (float)a * lds_as[wm * WM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3)] * ws;
+                        if (out) out[(size_t)m * N + n] = (float)a * lds_as[wm * WM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3)] * ws;
                         if (acc_out) acc_out[(size_t)m * N + n] = a;
                     }
                 }

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void gemv_w8a8_kernel(
                 const float ws = w_scales[col];
 #pragma unroll
                 for (int m = 0; m < M; ++m) {
-                    out[(size_t)m * n + col] = (float)acc[r][m] * a_scales[m] * ws;
+                    if (out) out[(size_t)m * n + col] = (float)acc[r][m] * a_scales[m] * ws;
                     if (acc_out) acc_out[(size_t)m * n + col] = acc[r][m];
                 }
             }
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_kernel(
         for (int j = 0; j < NCH; ++j) acc = dot16(w[j], x[j], acc);  // x is zero beyond nchunk
         acc = wave_sum_i32(acc);
         if (lane == 0 && row < n) {
-            out[row] = (float)acc * a_scale * w_scales[row];
+            if (out) out[row] = (float)acc * a_scale * w_scales[row];
             if (acc_out) acc_out[row] = acc;
         }
     }

@@ -103,6 +103,70 @@ __global__ __launch_bounds__(QA_THREADS) void quantize_rows_generic_kernel(
     for (size_t k = cols + threadIdx.x; k < q_stride; k += QA_THREADS) qr[k] = 0;
 }
 
+// ---- f32 rows as three signed byte digits ---------------------------------------------
+// x[k] ~= s * X[k], X = 65536 d2 + 256 d1 + d0 with signed byte digits, |X| <= 8355711, s a power of two:
+// 23 to 24 bits of fixed point per row, exact integer arithmetic on the matrix cores afterwards.
+// planes[p][row][k] (p = 0: d0 .. 2: d2), rows of q_stride bytes, pad columns zero.
+constexpr float DIG3_MAX = 8355711.0f;  // 127 * (65536 + 256 + 1)
+__global__ __launch_bounds__(QA_THREADS) void rows_to_digits3_kernel(const float *__restrict__ a, size_t cols,
+                                                                     int8_t *__restrict__ planes, size_t q_stride,
+                                                                     size_t plane_bytes, float *__restrict__ row_scales) {
+    __shared__ float red[4];
+    const size_t row = blockIdx.x;
+    const float *ar = a + row * cols;
+    float amax = 0.0f;
+    int bad = 0;
+    for (size_t k = threadIdx.x; k < cols; k += QA_THREADS) {
+        const float v = ar[k];
+        amax = fmaxf(amax, fabsf(v));
+        bad |= (v != v);
+    }
+    amax = block_max_256(amax, red);
+    bad = __syncthreads_or(bad);
+    const bool finite = !bad && amax <= 3.4028234663852886e38f;
+    // power-of-two scale, so x -> X is exact whenever x has no bits below s
+    // (integers stay integers), and s * X is exact again on the way back
+    float s = 1.0f, inv = 1.0f;
+    if (!finite) {
+        s = __uint_as_float(0x7FC00000u);
+        inv = 0.0f;
+    } else if (amax > 0.0f) {
+        int ex;
+        (void)frexpf(amax, &ex);  // amax = f * 2^ex, f in [0.5, 1)
+        int se = ex - 23;         // |x| / 2^se < 2^23 ...
+        if (se < -126) se = -126;
+        if (rintf(amax * ldexpf(1.0f, -se)) > DIG3_MAX) se += 1;  // ... but three signed bytes stop at 127 * 65793
+        s = ldexpf(1.0f, se);
+        inv = ldexpf(1.0f, -se);
+    }
+    if (threadIdx.x == 0) row_scales[row] = s;
+    int8_t *p0 = planes + row * q_stride;
+    for (size_t k = threadIdx.x; k < q_stride; k += QA_THREADS) {
+        int X = 0;
+        if (k < cols && finite) {
+            const float t = fminf(fmaxf(rintf(ar[k] * inv), -DIG3_MAX), DIG3_MAX);
+            X = (int)t;
+        }
+        const int d0 = ((X + 128) & 255) - 128;
+        const int X1 = (X - d0) >> 8;
+        const int d1 = ((X1 + 128) & 255) - 128;
+        const int d2 = (X1 - d1) >> 8;
+        p0[k] = (int8_t)d0;
+        p0[plane_bytes + k] = (int8_t)d1;
+        p0[2 * plane_bytes + k] = (int8_t)d2;
+    }
+}
+
+// out[m, n] = (65536 I2 + 256 I1 + I0) * s[m] * w_scale[n], the integer exactly in f64.
+__global__ void combine_digits3_kernel(const int32_t *__restrict__ acc, size_t plane_elems, const float *__restrict__ row_scales,
+                                       const float *__restrict__ w_scales, size_t m, size_t n, float *__restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= m * n) return;
+    const size_t r = i / n, c = i - r * n;
+    const double v = 65536.0 * (double)acc[2 * plane_elems + i] + 256.0 * (double)acc[plane_elems + i] + (double)acc[i];
+    out[i] = (float)(v * (double)row_scales[r] * (double)w_scales[c]);
+}
+
 // ---- weight quantisation -----------------------------------------------------
 
 __global__ void fill_u32_kernel(uint32_t *p, size_t n, uint32_t v) {
@@ -466,6 +530,56 @@ PG_API pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t
     if (m <= PG_GEMV_MAX_M)
         return pg_launch_gemv_w8a8(ctx, a_i8, w->k_pad, a_scales, w, m, out_dev, acc_dev);
     return pg_launch_gemm_w8a8(ctx, a_i8, w->k_pad, a_scales, w, m, out_dev, acc_dev);
+}
+
+// The reference's GPU numerics for the same call: f32 activations times dequantised weights,
+// f32 accumulate (matmul_dequant_i8, src/metal/shaders.rs:2329-2375).  Here the activations
+// become 23/24-bit fixed point per row (power-of-two scale) and the product runs three times on the int8 matrix
+// cores (one pass per byte digit), exact in integers; the only roundings are the
+// activation step (at most 2^-23 of the row's absmax, none for values that are multiples of the scale) and the final f64 -> f32.
+PG_API pg_status pg_matmul_dequant_i8_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
+                                          const pg_qtensor *w, float *out_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(w != nullptr, "pg_matmul_dequant_i8: null weights");
+    PG_CHECK_ARG(w->rows == k, "pg_matmul_dequant_i8: a has k = %zu but w has %zu rows", k, w->rows);  // src/quant.rs:204
+    if (m == 0) return PG_OK;
+    PG_CHECK_ARG(a_dev && out_dev, "pg_matmul_dequant_i8: null pointer");
+    PG_CHECK_ARG(m < (1ull << 24), "pg_matmul_dequant_i8: m = %zu too large", m);
+    PG_CHECK_ARG(k <= 133000, "pg_matmul_dequant_i8: k = %zu would overflow the i32 digit sums", k);  // 127 * 127 * k < 2^31
+    const size_t m_pad = pg_round_up(m, PG_MPAD), n = w->cols;
+    const size_t plane_bytes = m_pad * w->k_pad, plane_elems = m * n;
+    const size_t sz_planes = pg_round_up(3 * plane_bytes, 256), sz_scales = pg_round_up(m_pad * sizeof(float), 256);
+    void *ws = nullptr;
+    PG_TRY(pg_workspace(ctx, sz_planes + sz_scales + 3 * plane_elems * sizeof(int32_t), &ws));
+    int8_t *planes = static_cast<int8_t *>(ws);
+    float *row_scales = reinterpret_cast<float *>(planes + sz_planes);
+    int32_t *acc = reinterpret_cast<int32_t *>(planes + sz_planes + sz_scales);
+    PG_TRY(pg_launch(ctx, "rows_to_digits3", rows_to_digits3_kernel, dim3((unsigned)m), dim3(QA_THREADS), 0, a_dev, k, planes,
+                     w->k_pad, plane_bytes, row_scales));
+    for (int p = 0; p < 3; ++p) {
+        if (m <= PG_GEMV_MAX_M)
+            PG_TRY(pg_launch_gemv_w8a8(ctx, planes + p * plane_bytes, w->k_pad, row_scales, w, m, nullptr, acc + p * plane_elems));
+        else
+            PG_TRY(pg_launch_gemm_w8a8(ctx, planes + p * plane_bytes, w->k_pad, row_scales, w, m, nullptr, acc + p * plane_elems));
+    }
+    return pg_launch(ctx, "combine_digits3", combine_digits3_kernel, dim3(grid_for(plane_elems, 256)), dim3(256), 0, acc, plane_elems,
+                     row_scales, w->scales, m, n, out_dev);
+}
+
+PG_API pg_status pg_matmul_dequant_i8(pg_ctx *ctx, const float *a, size_t m, size_t k, const pg_qtensor *w, float *out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(w != nullptr, "pg_matmul_dequant_i8: null weights");
+    PG_CHECK_ARG(w->rows == k, "pg_matmul_dequant_i8: a has k = %zu but w has %zu rows", k, w->rows);
+    if (m == 0) return PG_OK;
+    PG_CHECK_ARG(a && out, "pg_matmul_dequant_i8: null pointer");
+    pg_tmp da, dout;
+    PG_TRY(da.alloc(m * k * sizeof(float)));
+    PG_TRY(dout.alloc(m * w->cols * sizeof(float)));
+    PG_HIP(hipMemcpyAsync(da.p, a, m * k * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_matmul_dequant_i8_dev(ctx, da.as<float>(), m, k, w, dout.as<float>()));
+    PG_HIP(hipMemcpyAsync(out, dout.p, m * w->cols * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
 }
 
 PG_API pg_status pg_matmul_quantized(pg_ctx *ctx, const float *a, size_t m, size_t k,

@@ -117,3 +117,17 @@ def matmul_quantized_gpu(ctx, a_data, m, k, w):
     if not w.on_gpu:
         raise RuntimeError("weights not on GPU")
     return matmul_quantized(a_data, m, k, w, ctx)
+
+
+def matmul_dequant_i8(a_data, m, k, w, ctx=None):
+    """The reference's GPU numerics (W8A32) for `matmul_quantized_gpu`: f32 activations times
+    dequantised weights, f32 accumulate (`dispatch_matmul_dequant_i8` src/metal/context.rs:2226-2306,
+    shader src/metal/shaders.rs:2329-2375)."""
+    ctx = ctx or default_context()
+    if w.rows != k:  # assert_eq!(w.rows, k)  src/quant.rs:204
+        raise ValueError(f"weight rows ({w.rows}) must equal k ({k})")
+    a = _f32(a_data, m * k, "matmul_dequant_i8")
+    w.to_gpu(ctx)
+    out = np.empty(m * w.cols, np.float32)
+    _ffi.check(_ffi.lib.pg_matmul_dequant_i8(ctx.handle, _ptr(a), m, k, w._gpu, _ptr(out)))
+    return out

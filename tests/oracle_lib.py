@@ -79,6 +79,13 @@ def matmul_quantized(a, m, k, q_t, w_scales, n):
     return out, acc
 
 
+def matmul_dequant_i8(a, m, k, q, w_scales, n):
+    out = np.empty(m * n, np.float32)
+    lib.orc_matmul_dequant_i8(_p(_f32(a).reshape(-1)), _sz(m), _sz(k), _p(np.ascontiguousarray(q, np.int8)),
+                              _p(_f32(w_scales)), _sz(n), _p(out))
+    return out
+
+
 def f16_to_f32_bits(bits):
     return np.array([lib.orc_f16_to_f32_bits(int(b)) for b in np.asarray(bits).reshape(-1)], np.uint32)
 

@@ -256,3 +256,56 @@ def test_wire_record_straight_to_device(ctx, orc):
     want, _ = orc.matmul_quantized(a, m, rows, q_t, s, cols)
     assert (out.view(np.uint32) == want.view(np.uint32)).all()
     _ffi.lib.pg_qtensor_free(ctx.handle, h)
+
+
+W8A32_SHAPES = [(32, 128, 64), (1, 4096, 1024), (3, 200, 77), (70, 4096, 300), (300, 1000, 520)]
+
+
+@pytest.mark.parametrize("m,k,n", W8A32_SHAPES)
+def test_matmul_dequant_i8_vs_oracle(ctx, orc, m, k, n):
+    """W8A32, the reference's GPU numerics (src/metal/shaders.rs:2329-2375).  Two bars: against
+    the exact (float64) product of the same f32 activations and dequantised weights, 1e-5 of
+    max(|ref|, rms(ref)) -- this implementation's own error (23/24-bit fixed point per row, so a
+    row with x20 outlier channels loses ~6 bits on its ordinary elements; exact integer sums);
+    against the oracle's K-sequential f32 sum, 2e-5 -- at K = 4096 that sum itself carries up to
+    ~1e-5 of rounding error."""
+    from peregrine_amd import quant
+    say(f"matmul_dequant_i8 m={m} k={k} n={n}")
+    a = orc.rng_normal(11 + m, m * k)
+    a.reshape(m, k)[:, :: max(1, k // 37)] *= 20
+    w = orc.rng_normal(12 + n, k * n, 0.0, 0.02)
+    q, q_t, s = orc.quantize_weights(w, k, n)
+    qt = quant.QuantizedTensor(q, q_t, s, k, n)
+    got = quant.matmul_dequant_i8(a, m, k, qt, ctx).reshape(m, n)
+    want = orc.matmul_dequant_i8(a, m, k, q, s, n).reshape(m, n)
+    exact = a.reshape(m, k).astype(np.float64) @ orc.dequantize(q, s, k, n).reshape(k, n).astype(np.float64)
+    for r in range(m):
+        H.assert_close_rel(got[r], exact[r], 1e-5, f"row {r} vs exact")
+        H.assert_close_rel(got[r], want[r], 2e-5, f"row {r} vs f32 oracle")
+    qt.free_gpu()
+
+
+def test_matmul_dequant_i8_reference_tolerance_and_closed_form(ctx, orc):
+    """tests/quant_parity.rs:79-146 restated: the W8A32 result is within 10 % / 0.02 of the f32
+    product of the unquantised weights; plus integer inputs with unit scales give exact integers,
+    zero rows give zeros and a NaN poisons exactly its row."""
+    from peregrine_amd import quant
+    m, k, n = 32, 128, 64
+    a = H.mod_pattern(m * k, 7, 3, 200, 200, 0.5)
+    w = H.mod_pattern(k * n, 13, 7, 200, 200, 0.5)
+    qt = quant.quantize_weights(w, k, n, ctx)
+    got = quant.matmul_dequant_i8(a, m, k, qt, ctx)
+    ref = orc.matmul_f32(a, w, m, k, n)
+    diff = np.abs(got - ref)
+    assert ((diff / np.maximum(np.abs(ref), 1e-6) < 0.10) | (diff < 0.02)).all()
+    ai = (np.arange(m * k, dtype=np.float32) % 9 - 4).reshape(m, k)
+    ai[3] = 0
+    qi = (np.arange(k * n).reshape(k, n) % 13 - 6).astype(np.int8)
+    qt2 = quant.QuantizedTensor(qi.reshape(-1), np.ascontiguousarray(qi.T).reshape(-1), np.ones(n, np.float32), k, n)
+    got = quant.matmul_dequant_i8(ai, m, k, qt2, ctx).reshape(m, n)
+    assert (got == ai.astype(np.int64) @ qi.astype(np.int64)).all() and (got[3] == 0).all()
+    ai[5, 17] = np.nan
+    got = quant.matmul_dequant_i8(ai, m, k, qt2, ctx).reshape(m, n)
+    assert np.isnan(got[5]).all() and np.isfinite(np.delete(got, 5, axis=0)).all()
+    with pytest.raises(ValueError):
+        quant.matmul_dequant_i8(ai, m, k + 1, qt2, ctx)

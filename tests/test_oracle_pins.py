@@ -382,3 +382,22 @@ def test_normal_statistics(orc):
     assert (orc.rng_normal(1234, 10, 0.0, 0.02) == x[:10]).all()  # deterministic, prefix-stable
     y = orc.rng_normal(1234, 7, 1.0, 0.0)
     assert (y == 1.0).all()
+
+
+def test_matmul_dequant_i8_is_dequantize_then_f32_matmul(orc):
+    """The Metal kernel's arithmetic (src/metal/shaders.rs:2329-2375) equals the composition
+    of two functions pinned above -- dequantize (one rounding per weight) then the
+    K-sequential f32 matmul -- bit for bit, and a closed form: integer activations with
+    unit scales give exact integers."""
+    m, k, n = 5, 70, 9
+    a = H.lcg_data(m * k, 42)
+    w = H.lcg_data(k * n, 123)
+    q, q_t, s = orc.quantize_weights(w, k, n)
+    got = orc.matmul_dequant_i8(a, m, k, q, s, n)
+    want = orc.matmul_f32(a, orc.dequantize(q, s, k, n), m, k, n)
+    assert (got.view(np.uint32) == want.view(np.uint32)).all()
+    ai = np.arange(m * k, dtype=np.float32).reshape(m, k) % 7 - 3
+    qi = (np.arange(k * n).reshape(k, n) % 11 - 5).astype(np.int8)
+    exact = ai.astype(np.int64) @ qi.astype(np.int64)
+    got = orc.matmul_dequant_i8(ai, m, k, qi, np.ones(n, np.float32), n).reshape(m, n)
+    assert (got == exact).all()
