@@ -160,6 +160,17 @@ def main():
                  "traffic": traffic_for("quantize_rows")}
     act_quant["frac"] = round(act_quant["achieved"] / PEAK_HBM_GBS, 4)
 
+    # ------------------------------------------------------------------ W8A32 (the reference's GPU numerics), gate product
+    def w8a32_step():
+        check(lib.pg_matmul_dequant_i8_dev(ctx.handle, ptr(acts[4096]), M_PREFILL, 4096, weights["gate_proj"], ptr(outs[14336])))
+
+    w32_ms = timed(w8a32_step, args.steps, args.warmup)
+    prof32 = profiled(w8a32_step, args.steps)
+    w8a32 = {"workload": "W8A32 product [2048x4096] x [4096x14336] (f32 activations, dequantised i8 weights, f32 accumulate): "
+                         "three int8 matrix-core passes over 24-bit fixed-point activations",
+             "value": round(2 * M_PREFILL * 4096 * 14336 / (w32_ms * 1e-3) / 1e12, 1), "unit": "TFLOP/s",
+             "ms_per_step": round(w32_ms, 4), "kernels_ms": {k: round(v[0], 5) for k, v in prof32.items()}}
+
     # keep one set of device-quantised weights on the host for the CPU baseline, then free
     cpu_w = {}
     if not args.skip_cpu:
@@ -353,7 +364,7 @@ def main():
                                "each product = per-row activation quantisation + i8 GEMM + f32 rescale",
                    "m": M_PREFILL, "ops_per_step": LAYER_OPS},
         "pct_int8_mfma_peak": round(100 * tops / PEAK_INT8_TOPS, 2),
-        "roofline": roofline, "activation_quant": act_quant, "linear_m32": linear_m32, "decode_gemv": decode, "gguf_q4_0_gemv": gguf, "gguf_q4_0_skinny": skinny, "moe_q8_0": moe,
+        "roofline": roofline, "activation_quant": act_quant, "w8a32_gate": w8a32, "linear_m32": linear_m32, "decode_gemv": decode, "gguf_q4_0_gemv": gguf, "gguf_q4_0_skinny": skinny, "moe_q8_0": moe,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line), flush=True)

@@ -15,7 +15,7 @@ import helpers as H
 
 pytestmark = pytest.mark.gpu
 
-RTOL_CONTRACT = 1e-3                 # BASELINE: Q4_0/Q8_0 block-dequant paths
+RTOL_CONTRACT = 1e-3                 # the stated tolerance for Q4_0/Q8_0 block-dequant paths
 RTOL_ACHIEVED = {2: 1e-4, 8: 2e-5}   # what the one-row (GEMV) path is held to, per ggml type
 RTOL_ACHIEVED_MM = 4e-4              # several rows: 16-bit fixed-point activations per block
 
@@ -86,12 +86,12 @@ def test_load_tensor_q8_as_quantized(ctx, orc):
 
 # (type, n_out, k_in, m)
 GGUF_SHAPES = [
-    (2, 256, 4096, 1), (2, 256, 4096, 4), (2, 256, 4096, 16),   # BASELINE config 4 row counts
+    (2, 256, 4096, 1), (2, 256, 4096, 4), (2, 256, 4096, 16),   # benchmark configuration 4 row counts
     (2, 77, 96, 3), (2, 1000, 2048, 2), (2, 128, 14336, 1),     # ragged n, 1 / 7 blocks per lane
     (2, 64, 32768, 2),                                          # two K segments
     (2, 50, 11008, 1),                                          # partial last lane group
     (8, 256, 4096, 1), (8, 77, 96, 3), (8, 96, 6144, 4), (8, 64, 32768, 2),
-    (2, 14336, 4096, 1),                                        # BASELINE config 4, full size
+    (2, 14336, 4096, 1),                                        # benchmark configuration 4, full size
     (8, 6144, 4096, 1),
     # more than one row: matrix-core path (token tiles of 32, row tiles of 128, split K)
     (2, 130, 224, 33), (8, 131, 160, 40), (2, 515, 4096, 64), (8, 257, 6144, 35), (2, 14336, 4096, 4), (8, 4096, 14336, 16),
@@ -117,7 +117,7 @@ def test_gguf_matmul_vs_oracle(ctx, orc, typ, n_out, k_in, m):
 
 
 def test_gguf_matmul_full_size_m16_and_linearity(ctx, orc):
-    """BASELINE config 4 at M = 16, full size, plus a size-independent property: the product
+    """benchmark configuration 4 at M = 16, full size, plus a size-independent property: the product
     is linear in x, so y(x1 + x2) - y(x1) - y(x2) is zero up to rounding."""
     from peregrine_amd import gguf
     n_out, k_in, m = 14336, 4096, 16

@@ -49,7 +49,7 @@ def test_moe_small_vs_oracle(ctx, orc, typ, act):
 
 
 def test_moe_grok_shaped_reduced(ctx, orc):
-    """BASELINE config 5's structure (8 experts, top-2, 64 tokens, Q8_0, SiLU) at reduced
+    """benchmark configuration 5's structure (8 experts, top-2, 64 tokens, Q8_0, SiLU) at reduced
     width (d 512, ffn 1024) so the oracle finishes in seconds."""
     from peregrine_amd import gguf, moe
     T, d, ffn, E, top_k = 64, 512, 1024, 8, 2

@@ -148,9 +148,9 @@ def run_matmul_dev(ctx, a, m, k, qt):
 MATMUL_SHAPES = [
     (32, 128, 64), (16, 64, 32),                       # tests/quant_parity.rs:35, src/quant.rs:252
     (8, 32, 16), (1, 64, 1), (16, 256, 32),            # tests/huffman_parity.rs:25
-    (1, 4096, 14336), (1, 14336, 4096),                # BASELINE config 2 (decode GEMV)
+    (1, 4096, 14336), (1, 14336, 4096),                # benchmark configuration 2 (decode GEMV)
     (2, 4096, 1024), (3, 1000, 77), (4, 4096, 300),    # GEMV with m = 2..4, ragged k and n
-    (32, 4096, 4096),                                  # BASELINE config 1
+    (32, 4096, 4096),                                  # benchmark configuration 1
     (5, 96, 40), (64, 200, 130), (65, 384, 129),       # 64x64 and 128x128 tiles, ragged
     (196, 768, 3072),                                  # benches/wallclock.rs:758-786
     (300, 512, 1000),                                  # 128x128 tiles, ragged m and n
@@ -209,7 +209,7 @@ def test_matmul_quantized_shape_mismatch_is_an_error(ctx, orc):
 
 
 def test_prefill_shape_full_size_properties(ctx, orc):
-    """BASELINE config 3 shape (M = 2048, q_proj 4096 -> 4096) at full size: the oracle would
+    """benchmark configuration 3 shape (M = 2048, q_proj 4096 -> 4096) at full size: the oracle would
     need 3.4e10 scalar MACs, so check (a) 48 sampled rows bit-exactly against the oracle and
     (b) the sum over ALL accumulators against the exact identity
         sum_{m,n} acc[m,n] = sum_k (sum_m a_i8[m,k]) * (sum_n w_t[n,k])   (int64)."""
