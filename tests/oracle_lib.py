@@ -157,3 +157,51 @@ def rng_normal(seed, n, mean=0.0, std=1.0):
     out = np.empty(n, np.float32)
     lib.orc_rng_normal(C.c_uint64(seed), _sz(n), C.c_float(mean), C.c_float(std), _p(out))
     return out
+
+
+# ---- Llama block glue (oracle/peregrine_oracle_llama.c) ----
+for _n in ("orc_rmsnorm", "orc_rope_tables", "orc_rope_apply", "orc_gqa_attention"):
+    getattr(lib, _n).restype = None
+
+
+def rmsnorm(x, rows, dim, w, eps):
+    out = np.empty(rows * dim, np.float32)
+    lib.orc_rmsnorm(_p(_f32(x).reshape(-1)), _sz(rows), _sz(dim), _p(_f32(w)), C.c_float(eps), _p(out))
+    return out
+
+
+def rope_tables(head_dim, max_seq_len, base):
+    cos = np.empty((max_seq_len, head_dim), np.float32)
+    sin = np.empty((max_seq_len, head_dim), np.float32)
+    lib.orc_rope_tables(_sz(head_dim), _sz(max_seq_len), C.c_float(base), _p(cos), _p(sin))
+    return cos, sin
+
+
+def rope_apply(x, seq_len, head_dim, offset, cos, sin):
+    out = np.empty(seq_len * head_dim, np.float32)
+    lib.orc_rope_apply(_p(_f32(x).reshape(-1)), _sz(seq_len), _sz(head_dim), _sz(offset), _p(cos), _p(sin), _p(out))
+    return out
+
+
+def gqa_attention(q, k, v, length, capacity, nqh, nkvh, seq_q, hd, scale, mask_kind=0, offset=0, window=0, sink=0,
+                  logit_cap=0.0):
+    """q [nqh, seq_q, hd]; k, v [nkvh, capacity, hd]; returns [seq_q, nqh*hd]."""
+    out = np.zeros(seq_q * nqh * hd, np.float32)
+    lib.orc_gqa_attention(_p(_f32(q).reshape(-1)), _p(_f32(k).reshape(-1)), _p(_f32(v).reshape(-1)), _sz(length),
+                          _sz(capacity), _sz(nqh), _sz(nkvh), _sz(seq_q), _sz(hd), C.c_float(scale), C.c_int(mask_kind),
+                          _sz(offset), _sz(window), _sz(sink), C.c_float(logit_cap), _p(out))
+    return out
+
+
+def llama_block_forward(h, seq, d, nqh, nkvh, hd, ffn, ggml_type, weights, attn_norm_w, ffn_norm_w, eps, cos, sin,
+                        k_cache, v_cache, cache_len, capacity):
+    """weights: 7 raw block byte strings (q, k, v, o, gate, up, down).  k_cache / v_cache are
+    updated in place ([nkvh, capacity, hd] float32 arrays).  Returns out [seq, d]."""
+    keep = [np.frombuffer(bytes(b), np.uint8).copy() for b in weights]
+    out = np.empty(seq * d, np.float32)
+    rc = lib.orc_llama_block_forward(_p(_f32(h).reshape(-1)), _sz(seq), _sz(d), _sz(nqh), _sz(nkvh), _sz(hd), _sz(ffn),
+                                     C.c_int(ggml_type), *[_p(a) for a in keep], _p(_f32(attn_norm_w)),
+                                     _p(_f32(ffn_norm_w)), C.c_float(eps), _p(cos), _p(sin), _p(k_cache), _p(v_cache),
+                                     _sz(cache_len), _sz(capacity), _p(out))
+    assert rc == 0, rc
+    return out.reshape(seq, d)
