@@ -247,6 +247,89 @@ pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
                          const pg_gguf_tensor *const *gate, const pg_gguf_tensor *const *up,
                          const pg_gguf_tensor *const *down, int act, float *out_dev);
 
+/* ---- Llama decoder block: the glue around the quantised products -------------- */
+
+typedef struct pg_rope pg_rope;               /* nn::RoPE                  src/nn.rs:1250-1256 */
+typedef struct pg_kv_cache pg_kv_cache;       /* attention::StandardKVCache src/attention.rs:8-15 */
+typedef struct pg_llama_block pg_llama_block; /* LlamaBlock                src/models/llama/decoder.rs:7-16 */
+
+/* attention::AttentionMask  src/attention.rs:102-120 (LocalGlobal is not offered). */
+#define PG_MASK_NONE 0
+#define PG_MASK_CAUSAL 1                 /* Causal { offset } */
+#define PG_MASK_CAUSAL_SLIDING_WINDOW 2  /* CausalSlidingWindow { offset, window, sink_tokens } */
+
+/* nn::RMSNorm::forward, inference path  src/nn.rs:577-652:
+ *   out[r, i] = x[r, i] / sqrt(mean_i(x[r]^2) + eps) * w[i];  x, out [rows, dim]; w [dim]. */
+pg_status pg_rmsnorm(pg_ctx *ctx, const float *x, size_t rows, size_t dim, const float *w, float eps,
+                     float *out);
+pg_status pg_rmsnorm_dev(pg_ctx *ctx, const float *x_dev, size_t rows, size_t dim, const float *w_dev,
+                         float eps, float *out_dev);
+
+/* nn::RoPE::new  src/nn.rs:1258-1282: cos/sin tables [max_seq_len, head_dim] (f32 libm
+ * values computed on the host, then resident on the device).  head_dim must be even. */
+pg_status pg_rope_create(pg_ctx *ctx, size_t head_dim, size_t max_seq_len, float base, pg_rope **out);
+void pg_rope_free(pg_ctx *ctx, pg_rope *rope);
+/* nn::RoPE::apply  src/nn.rs:1286-1338: x, out [seq_len, head_dim], positions
+ * offset..offset+seq_len, pairs (i, i + head_dim/2).  A position past max_seq_len (the
+ * reference's slice panic) is PG_EINVAL. */
+pg_status pg_rope_apply(pg_ctx *ctx, const pg_rope *rope, const float *x, size_t seq_len, size_t offset,
+                        float *out);
+pg_status pg_rope_apply_dev(pg_ctx *ctx, const pg_rope *rope, const float *x_dev, size_t seq_len,
+                            size_t offset, float *out_dev);
+
+/* StandardKVCache::new  src/attention.rs:18-27: empty, capacity 0; head_dim <= 256. */
+pg_status pg_kv_cache_create(pg_ctx *ctx, size_t num_kv_heads, size_t head_dim, pg_kv_cache **out);
+void pg_kv_cache_free(pg_ctx *ctx, pg_kv_cache *cache);
+/* StandardKVCache::append  src/attention.rs:65-83 (growth as ensure_capacity, :31-62:
+ * at least double, from 16): new_k, new_v [num_kv_heads, seq_len, head_dim]. */
+pg_status pg_kv_cache_append(pg_ctx *ctx, pg_kv_cache *cache, const float *new_k, const float *new_v,
+                             size_t seq_len);
+pg_status pg_kv_cache_append_dev(pg_ctx *ctx, pg_kv_cache *cache, const float *new_k_dev,
+                                 const float *new_v_dev, size_t seq_len);
+/* StandardKVCache::rollback_to  src/attention.rs:87-91; new_len > len (its assert!) is PG_EINVAL. */
+pg_status pg_kv_cache_rollback_to(pg_kv_cache *cache, size_t new_len);
+size_t pg_kv_cache_len(const pg_kv_cache *cache);      /* the `len` field */
+size_t pg_kv_cache_capacity(const pg_kv_cache *cache); /* head_stride() / head_dim  src/attention.rs:96-98 */
+/* The `k` and `v` fields without the capacity padding: [num_kv_heads, len, head_dim] each. */
+pg_status pg_kv_cache_download(pg_ctx *ctx, const pg_kv_cache *cache, float *k, float *v);
+
+/* attention::gqa_attention_cpu  src/attention.rs:141-265 (masks :269-300):
+ *   q [num_q_heads, seq_q, head_dim]; keys from k_cache, values from v_cache (same shape
+ *   and length); out [seq_q, num_q_heads * head_dim] is ADDED TO, as the reference adds
+ *   into `output` (callers pass zeros).  logit_cap > 0 applies cap * tanh(score / cap)
+ *   (PostScoreTransform::LogitCap), 0 = PostScoreTransform::None.  offset / window /
+ *   sink_tokens are read as the mask kind needs them. */
+pg_status pg_gqa_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *k_cache,
+                           const pg_kv_cache *v_cache, size_t num_q_heads, size_t seq_q, float scale,
+                           int mask_kind, size_t offset, size_t window, size_t sink_tokens,
+                           float logit_cap, float *out);
+pg_status pg_gqa_attention_dev(pg_ctx *ctx, const float *q_dev, const pg_kv_cache *k_cache,
+                               const pg_kv_cache *v_cache, size_t num_q_heads, size_t seq_q, float scale,
+                               int mask_kind, size_t offset, size_t window, size_t sink_tokens,
+                               float logit_cap, float *out_dev);
+
+/* LlamaBlock::new  src/models/llama/decoder.rs:19-47 (with LlamaAttention::new,
+ * src/models/llama/attention.rs:25-48). */
+pg_status pg_llama_block_create(pg_ctx *ctx, size_t model_dim, size_t num_q_heads, size_t num_kv_heads,
+                                size_t head_dim, size_t ffn_dim, size_t max_seq_len, float rope_base,
+                                float rms_eps, pg_llama_block **out);
+void pg_llama_block_free(pg_ctx *ctx, pg_llama_block *block);
+/* The block's seven projections as GGUF block tensors [out, in] (borrowed: they must
+ * outlive the block) and its two norm weights [model_dim] (copied).  The reference holds
+ * the projections dequantised and transposed (src/models/llama/model.rs:243-257). */
+pg_status pg_llama_block_set_weights(pg_ctx *ctx, pg_llama_block *block, const pg_gguf_tensor *q_proj,
+                                     const pg_gguf_tensor *k_proj, const pg_gguf_tensor *v_proj,
+                                     const pg_gguf_tensor *o_proj, const pg_gguf_tensor *gate_proj,
+                                     const pg_gguf_tensor *up_proj, const pg_gguf_tensor *down_proj,
+                                     const float *attn_norm_w, const float *ffn_norm_w);
+/* LlamaBlock::forward  src/models/llama/decoder.rs:69-155 with LlamaAttention::forward
+ * (src/models/llama/attention.rs:73-212), unfused projections: h, out [seq, model_dim];
+ * the cache gains seq positions (causal mask at offset = its length on entry). */
+pg_status pg_llama_block_forward(pg_ctx *ctx, pg_llama_block *block, const float *h, size_t seq,
+                                 pg_kv_cache *cache, float *out);
+pg_status pg_llama_block_forward_dev(pg_ctx *ctx, pg_llama_block *block, const float *h_dev, size_t seq,
+                                     pg_kv_cache *cache, float *out_dev);
+
 #ifdef __cplusplus
 }
 #endif

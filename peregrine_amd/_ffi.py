@@ -16,6 +16,7 @@ lib = C.CDLL(LIB_PATH)
 PG_OK, PG_EINVAL, PG_EDEVICE, PG_ENOMEM, PG_EUNSUPPORTED = 0, 1, 2, 3, 4
 GGML_Q4_0, GGML_Q4_1, GGML_Q8_0 = 2, 3, 8
 ACT_SILU, ACT_GELU_TANH = 0, 1
+MASK_NONE, MASK_CAUSAL, MASK_CAUSAL_SLIDING_WINDOW = 0, 1, 2
 
 _vp, _sz, _int = C.c_void_p, C.c_size_t, C.c_int
 _pp = C.POINTER(C.c_void_p)
@@ -79,12 +80,38 @@ SIGNATURES = {
     "pg_qtensor_from_record": [_vp, _vp, _sz, _pp, C.POINTER(_sz)],
     "pg_moe_ffn": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
     "pg_moe_ffn_dev": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
+    "pg_rmsnorm": [_vp, _vp, _sz, _sz, _vp, C.c_float, _vp],
+    "pg_rmsnorm_dev": [_vp, _vp, _sz, _sz, _vp, C.c_float, _vp],
+    "pg_rope_create": [_vp, _sz, _sz, C.c_float, _pp],
+    "pg_rope_free": [_vp, _vp],
+    "pg_rope_apply": [_vp, _vp, _vp, _sz, _sz, _vp],
+    "pg_rope_apply_dev": [_vp, _vp, _vp, _sz, _sz, _vp],
+    "pg_kv_cache_create": [_vp, _sz, _sz, _pp],
+    "pg_kv_cache_free": [_vp, _vp],
+    "pg_kv_cache_append": [_vp, _vp, _vp, _vp, _sz],
+    "pg_kv_cache_append_dev": [_vp, _vp, _vp, _vp, _sz],
+    "pg_kv_cache_rollback_to": [_vp, _sz],
+    "pg_kv_cache_len": [_vp],
+    "pg_kv_cache_capacity": [_vp],
+    "pg_kv_cache_download": [_vp, _vp, _vp, _vp],
+    "pg_gqa_attention": [_vp, _vp, _vp, _vp, _sz, _sz, C.c_float, _int, _sz, _sz, _sz, C.c_float, _vp],
+    "pg_gqa_attention_dev": [_vp, _vp, _vp, _vp, _sz, _sz, C.c_float, _int, _sz, _sz, _sz, C.c_float, _vp],
+    "pg_llama_block_create": [_vp, _sz, _sz, _sz, _sz, _sz, _sz, C.c_float, C.c_float, _pp],
+    "pg_llama_block_free": [_vp, _vp],
+    "pg_llama_block_set_weights": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
+    "pg_llama_block_forward": [_vp, _vp, _vp, _sz, _vp, _vp],
+    "pg_llama_block_forward_dev": [_vp, _vp, _vp, _sz, _vp, _vp],
 }
 _OTHER_RESTYPE = {
     "pg_ctx_destroy": None,
     "pg_qtensor_free": None,
     "pg_gguf_free": None,
     "pg_gguf_file_close": None,
+    "pg_rope_free": None,
+    "pg_kv_cache_free": None,
+    "pg_llama_block_free": None,
+    "pg_kv_cache_len": _sz,
+    "pg_kv_cache_capacity": _sz,
     "pg_ctx_stream": _vp,
     "pg_last_error": C.c_char_p,
     "pg_status_string": C.c_char_p,

@@ -1,0 +1,704 @@
+// The glue of peregrine's Llama decoder block around the quantised products: RMSNorm, RoPE,
+// the KV cache, grouped-query attention and the block itself, all on the device so that a
+// block step is one chain of stream-ordered launches with no host round trip.
+//
+//   nn::RMSNorm::forward            reference: src/nn.rs:577-652
+//   nn::RoPE::{new, apply}          reference: src/nn.rs:1250-1345
+//   attention::StandardKVCache      reference: src/attention.rs:8-100
+//   attention::gqa_attention_cpu    reference: src/attention.rs:141-300
+//   LlamaAttention::forward         reference: src/models/llama/attention.rs:73-212
+//   LlamaBlock::forward             reference: src/models/llama/decoder.rs:69-155
+//
+// Layouts (all f32, row-major):
+//   KV cache   k, v [num_kv_heads][capacity][head_dim], `len` positions valid per head
+//   RoPE       cos, sin [max_seq_len][head_dim] (the half-row repeated, as the reference holds it)
+//   q          [num_q_heads][seq_q][head_dim]; attention output [seq_q][num_q_heads * head_dim]
+#include <math.h>
+#include <new>
+#include "pg_internal.h"
+
+struct pg_rope {
+    float *cos_t, *sin_t;
+    size_t head_dim, max_seq_len;
+};
+
+struct pg_kv_cache {
+    float *k, *v;
+    size_t len, capacity, num_kv_heads, head_dim;
+};
+
+struct pg_llama_block {
+    size_t d, nqh, nkvh, hd, ffn;
+    float eps;
+    pg_rope *rope;
+    const pg_gguf_tensor *w[7];  // q, k, v, o, gate, up, down (borrowed)
+    float *attn_norm_w, *ffn_norm_w;
+    float *arena;  // activations for seq_cap tokens
+    size_t seq_cap;
+};
+
+namespace {
+
+__device__ __forceinline__ float block_sum(float v, float *red) {
+    v = pg_wave_sum_f32(v);
+    const int wave = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) t += red[i];
+    return t;
+}
+
+__device__ __forceinline__ float block_max(float v, float *red) {
+    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
+    const int wave = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    float t = red[0];
+    for (int i = 1; i < (int)(blockDim.x >> 6); ++i) t = fmaxf(t, red[i]);
+    return t;
+}
+
+// One workgroup per row: s = a (+ b), optionally stored, then out = s / rms(s) * w.
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(const float *a, const float *__restrict__ b, float *sum_out,
+                                                          const float *__restrict__ w,
+                                                          float eps, int dim, float *__restrict__ out) {
+    __shared__ float red[4];
+    const size_t row = (size_t)blockIdx.x * dim;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        float s = a[row + i];
+        if (b) {
+            s = s + b[row + i];
+            sum_out[row + i] = s;
+        }
+        ss += s * s;
+    }
+    ss = block_sum(ss, red);
+    const float inv_rms = 1.0f / sqrtf(ss * (1.0f / (float)dim) + eps);
+    const float *src = b ? sum_out : a;  // a thread re-reads only what it wrote itself
+    for (int i = threadIdx.x; i < dim; i += 256) out[row + i] = src[row + i] * inv_rms * w[i];
+}
+
+// Up to three [seq][heads*hd] sources re-laid head-major, rotated or copied.
+struct rope_seg {
+    const float *src;  // token t, head h at src + t*src_tstride + h*hd
+    float *dst;        // at dst + h*dst_hstride + t*hd
+    size_t src_tstride, dst_hstride;
+    int heads, rotate;
+};
+struct rope_args {
+    rope_seg seg[3];
+    const float *cos_t, *sin_t;
+    int hd, pos0, nseg;
+};
+
+__global__ __launch_bounds__(128) void rope_kernel(rope_args ra) {
+    const int t = blockIdx.x;
+    int h = blockIdx.y, s = 0;
+    while (s < ra.nseg - 1 && h >= ra.seg[s].heads) h -= ra.seg[s++].heads;
+    const rope_seg sg = ra.seg[s];
+    const float *src = sg.src + (size_t)t * sg.src_tstride + (size_t)h * ra.hd;
+    float *dst = sg.dst + (size_t)h * sg.dst_hstride + (size_t)t * ra.hd;
+    const int half = ra.hd / 2;
+    if (!sg.rotate) {
+        for (int i = threadIdx.x; i < ra.hd; i += 128) dst[i] = src[i];
+        return;
+    }
+    const float *c = ra.cos_t + (size_t)(ra.pos0 + t) * ra.hd, *sn = ra.sin_t + (size_t)(ra.pos0 + t) * ra.hd;
+    for (int i = threadIdx.x; i < half; i += 128) {
+        const float x0 = src[i], x1 = src[half + i];
+        dst[i] = x0 * c[i] - x1 * sn[i];
+        dst[half + i] = x0 * sn[i] + x1 * c[i];
+    }
+}
+
+__device__ __forceinline__ bool attn_masked(int mask_kind, int offset, int window, int sink, int qt, int kt) {
+    if (mask_kind == 0) return false;
+    const int query_pos = offset + qt;
+    if (kt > query_pos) return true;
+    if (mask_kind == 1) return false;
+    if (kt < sink) return false;
+    return query_pos - kt > window;
+}
+
+struct attn_args {
+    const float *q, *kc, *vc;
+    float *scores_g, *out;
+    size_t k_stride, v_stride;  // per kv head
+    int len, nqh, group, seq_q, hd, lanes;  // lanes = power of two >= hd/4, <= 64
+    float scale, logit_cap;
+    int mask_kind, offset, window, sink, accumulate;
+};
+
+constexpr int ATT_RED = 1024;  // partial output rows: (256 / lanes) slices x (lanes * 4) dims
+
+// One workgroup per (query token, query head).  Scores: `lanes` lanes share one key, four
+// dims each, so that a key row is one contiguous read; softmax over the scores held in LDS
+// (or in global memory for very long caches); then P.V with the same lane-to-dim mapping,
+// the key range cut into 256/lanes slices whose partial rows are summed in a fixed order.
+__global__ __launch_bounds__(256) void gqa_attention_kernel(attn_args aa) {
+    extern __shared__ float lds[];
+    __shared__ float red[4];
+    const int tid = threadIdx.x, qt = blockIdx.x, qh = blockIdx.y, kvh = qh / aa.group;
+    const int L = aa.lanes, hd = aa.hd, len = aa.len;
+    float *qs = lds, *part = lds + 256, *sc = aa.scores_g ? aa.scores_g + ((size_t)qh * aa.seq_q + qt) * len : lds + 256 + ATT_RED;
+    const float *qsrc = aa.q + ((size_t)qh * aa.seq_q + qt) * hd;
+    for (int i = tid; i < 4 * L; i += 256) qs[i] = i < hd ? qsrc[i] : 0.f;
+    __syncthreads();
+    const int sub = tid / L, within = tid % L, nsub = 256 / L, d0 = within * 4;
+    const bool vec = (hd & 3) == 0;
+    const float *kbase = aa.kc + (size_t)kvh * aa.k_stride, *vbase = aa.vc + (size_t)kvh * aa.v_stride;
+    float q4[4];
+    for (int j = 0; j < 4; ++j) q4[j] = qs[d0 + j];
+
+    float mx = -INFINITY;
+    const int rounds = (len + nsub - 1) / nsub;
+    for (int r = 0; r < rounds; ++r) {  // every lane runs every round: the shuffles need the whole wave
+        const int kt = r * nsub + sub;
+        float dot = 0.f;
+        const bool live = kt < len && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, qt, kt);
+        if (live && d0 < hd) {
+            const float *kr = kbase + (size_t)kt * hd + d0;
+            if (vec) {
+                const float4 kv = *reinterpret_cast<const float4 *>(kr);
+                dot = q4[0] * kv.x + q4[1] * kv.y + q4[2] * kv.z + q4[3] * kv.w;
+            } else {
+                for (int j = 0; j < 4; ++j)
+                    if (d0 + j < hd) dot += q4[j] * kr[j];
+            }
+        }
+        for (int m = 1; m < L; m <<= 1) dot += __shfl_xor(dot, m);
+        if (kt < len) {
+            float s = -INFINITY;
+            if (live) {
+                s = dot * aa.scale;
+                if (aa.logit_cap > 0.f) s = aa.logit_cap * tanhf(s / aa.logit_cap);
+            }
+            if (within == 0) sc[kt] = s;
+            mx = fmaxf(mx, s);
+        }
+    }
+    mx = block_max(mx, red);  // the barriers inside also publish sc[]
+    float sum = 0.f;
+    for (int kt = tid; kt < len; kt += 256) {
+        const float s = sc[kt];
+        const float e = s == -INFINITY ? 0.f : expf(s - mx);
+        sc[kt] = e;
+        sum += e;
+    }
+    sum = block_sum(sum, red);
+    const float inv_sum = sum > 0.f ? 1.0f / sum : 0.f;
+
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    if (d0 < hd) {
+        for (int kt = sub; kt < len; kt += nsub) {
+            const float p = sc[kt] * inv_sum;
+            if (p > 0.f) {
+                const float *vr = vbase + (size_t)kt * hd + d0;
+                if (vec) {
+                    const float4 vv = *reinterpret_cast<const float4 *>(vr);
+                    acc[0] += p * vv.x; acc[1] += p * vv.y; acc[2] += p * vv.z; acc[3] += p * vv.w;
+                } else {
+                    for (int j = 0; j < 4; ++j)
+                        if (d0 + j < hd) acc[j] += p * vr[j];
+                }
+            }
+        }
+    }
+    for (int j = 0; j < 4; ++j) part[sub * (4 * L) + d0 + j] = acc[j];
+    __syncthreads();
+    for (int i = tid; i < hd; i += 256) {
+        float o = 0.f;
+        for (int s = 0; s < nsub; ++s) o += part[s * (4 * L) + i];
+        float *dst = aa.out + ((size_t)qt * aa.nqh + qh) * hd + i;
+        *dst = aa.accumulate ? *dst + o : o;
+    }
+}
+
+__global__ __launch_bounds__(256) void swiglu_kernel(float *__restrict__ g, const float *__restrict__ u, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        const float gi = g[i];
+        g[i] = gi / (1.0f + expf(-gi)) * u[i];
+    }
+}
+
+__global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                  float *__restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = a[i] + b[i];
+}
+
+inline unsigned blocks_for(size_t n) { return (unsigned)((n + 255) / 256); }
+
+pg_status launch_rmsnorm(pg_ctx *ctx, const float *a, const float *b, float *sum_out, const float *w, float eps,
+                         size_t rows, size_t dim, float *out) {
+    if (rows == 0) return PG_OK;
+    return pg_launch(ctx, "add_rmsnorm", add_rmsnorm_kernel, dim3((unsigned)rows), dim3(256), 0, a, b, sum_out, w, eps,
+                     (int)dim, out);
+}
+
+constexpr size_t ATT_LDS_KEYS = 36864;  // scores kept in LDS up to this cache length (147 KB + fixed part)
+
+pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, const pg_kv_cache *vc, size_t nqh,
+                           size_t seq_q, float scale, int mask_kind, size_t offset, size_t window, size_t sink,
+                           float logit_cap, float *out, int accumulate) {
+    const size_t len = kc->len, hd = kc->head_dim;
+    if (seq_q == 0 || nqh == 0) return PG_OK;
+    if (len == 0) {  // nothing to attend to: the reference adds nothing to `output`
+        if (!accumulate) PG_HIP(hipMemsetAsync(out, 0, seq_q * nqh * hd * sizeof(float), ctx->stream));
+        return PG_OK;
+    }
+    attn_args aa;
+    aa.q = q; aa.kc = kc->k; aa.vc = vc->v; aa.out = out; aa.scores_g = nullptr;
+    aa.k_stride = kc->capacity * hd; aa.v_stride = vc->capacity * hd;
+    aa.len = (int)len; aa.nqh = (int)nqh; aa.group = (int)(nqh / kc->num_kv_heads); aa.seq_q = (int)seq_q; aa.hd = (int)hd;
+    int lanes = 1;
+    while ((size_t)lanes * 4 < hd) lanes <<= 1;
+    aa.lanes = lanes;
+    aa.scale = scale; aa.logit_cap = logit_cap;
+    aa.mask_kind = mask_kind; aa.offset = (int)offset;
+    aa.window = (int)(window > 0x7fffffffu ? 0x7fffffffu : window);
+    aa.sink = (int)(sink > 0x7fffffffu ? 0x7fffffffu : sink);
+    aa.accumulate = accumulate;
+    size_t lds = (256 + ATT_RED) * sizeof(float);
+    if (len <= ATT_LDS_KEYS) {
+        lds += len * sizeof(float);
+    } else {
+        void *ws = nullptr;
+        PG_TRY(pg_workspace(ctx, nqh * seq_q * len * sizeof(float), &ws));
+        aa.scores_g = static_cast<float *>(ws);
+    }
+    static bool attr_done = false;
+    if (!attr_done) {
+        PG_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gqa_attention_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)((256 + ATT_RED + ATT_LDS_KEYS) * sizeof(float))));
+        attr_done = true;
+    }
+    return pg_launch(ctx, "gqa_attention", gqa_attention_kernel, dim3((unsigned)seq_q, (unsigned)nqh), dim3(256), lds, aa);
+}
+
+pg_status check_attention_args(const char *fn, const pg_kv_cache *kc, const pg_kv_cache *vc, size_t nqh, size_t seq_q,
+                               int mask_kind, size_t offset) {
+    PG_CHECK_ARG(kc && vc, "%s: null cache", fn);
+    PG_CHECK_ARG(kc->num_kv_heads == vc->num_kv_heads && kc->head_dim == vc->head_dim && kc->len == vc->len,
+                 "%s: the key and value caches differ in shape or length", fn);
+    PG_CHECK_ARG(kc->num_kv_heads > 0 && nqh % kc->num_kv_heads == 0,
+                 "%s: num_q_heads %zu is not a multiple of num_kv_heads %zu", fn, nqh, kc->num_kv_heads);
+    PG_CHECK_ARG(mask_kind >= PG_MASK_NONE && mask_kind <= PG_MASK_CAUSAL_SLIDING_WINDOW, "%s: unknown mask kind %d", fn,
+                 mask_kind);
+    PG_CHECK_ARG(nqh <= 65535, "%s: more than 65535 query heads", fn);
+    PG_CHECK_ARG(offset + seq_q < (1ull << 31) && kc->len < (1ull << 31), "%s: positions beyond 2^31", fn);
+    return PG_OK;
+}
+
+// Room for `needed` positions per head; grows like the reference (at least double, from 16).
+pg_status cache_reserve(pg_ctx *ctx, pg_kv_cache *c, size_t needed) {
+    if (needed <= c->capacity) return PG_OK;
+    const size_t grown = (c->capacity > 16 ? c->capacity : 16) * 2;
+    const size_t new_cap = needed > grown ? needed : grown;
+    const size_t hd = c->head_dim, total = c->num_kv_heads * new_cap * hd * sizeof(float);
+    float *nk = nullptr, *nv = nullptr;
+    PG_HIP(hipMalloc(reinterpret_cast<void **>(&nk), total));
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&nv), total);
+    if (e != hipSuccess) {
+        (void)hipFree(nk);
+        return pg_fail(PG_ENOMEM, "hipMalloc(%zu) failed: %s", total, hipGetErrorString(e));
+    }
+    e = hipMemsetAsync(nk, 0, total, ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(nv, 0, total, ctx->stream);
+    if (e == hipSuccess && c->len > 0) {
+        const size_t width = c->len * hd * sizeof(float);
+        e = hipMemcpy2DAsync(nk, new_cap * hd * sizeof(float), c->k, c->capacity * hd * sizeof(float), width,
+                             c->num_kv_heads, hipMemcpyDeviceToDevice, ctx->stream);
+        if (e == hipSuccess)
+            e = hipMemcpy2DAsync(nv, new_cap * hd * sizeof(float), c->v, c->capacity * hd * sizeof(float), width,
+                                 c->num_kv_heads, hipMemcpyDeviceToDevice, ctx->stream);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);  // the old planes are freed next
+    if (e != hipSuccess) {
+        (void)hipFree(nk);
+        (void)hipFree(nv);
+        return pg_fail(PG_EDEVICE, "KV cache growth failed: %s", hipGetErrorString(e));
+    }
+    if (c->k) (void)hipFree(c->k);
+    if (c->v) (void)hipFree(c->v);
+    c->k = nk;
+    c->v = nv;
+    c->capacity = new_cap;
+    return PG_OK;
+}
+
+pg_status launch_rope(pg_ctx *ctx, const rope_args &ra, size_t seq, size_t heads) {
+    if (seq == 0 || heads == 0) return PG_OK;
+    return pg_launch(ctx, "rope", rope_kernel, dim3((unsigned)seq, (unsigned)heads), dim3(128), 0, ra);
+}
+
+}  // namespace
+
+// ---- RMSNorm ----------------------------------------------------------------------------------
+
+PG_API pg_status pg_rmsnorm_dev(pg_ctx *ctx, const float *x_dev, size_t rows, size_t dim, const float *w_dev, float eps,
+                                float *out_dev) {
+    PG_TRY(pg_use(ctx));
+    if (rows == 0 || dim == 0) return PG_OK;
+    PG_CHECK_ARG(x_dev && w_dev && out_dev, "pg_rmsnorm: null pointer");
+    PG_CHECK_ARG(dim < (1ull << 31) && rows < (1ull << 31), "pg_rmsnorm: shape too large");
+    return launch_rmsnorm(ctx, x_dev, nullptr, nullptr, w_dev, eps, rows, dim, out_dev);
+}
+
+PG_API pg_status pg_rmsnorm(pg_ctx *ctx, const float *x, size_t rows, size_t dim, const float *w, float eps, float *out) {
+    PG_TRY(pg_use(ctx));
+    if (rows == 0 || dim == 0) return PG_OK;
+    PG_CHECK_ARG(x && w && out, "pg_rmsnorm: null pointer");
+    pg_tmp dx, dw, dout;
+    PG_TRY(dx.alloc(rows * dim * sizeof(float)));
+    PG_TRY(dw.alloc(dim * sizeof(float)));
+    PG_TRY(dout.alloc(rows * dim * sizeof(float)));
+    PG_HIP(hipMemcpyAsync(dx.p, x, rows * dim * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(dw.p, w, dim * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_rmsnorm_dev(ctx, dx.as<float>(), rows, dim, dw.as<float>(), eps, dout.as<float>()));
+    PG_HIP(hipMemcpyAsync(out, dout.p, rows * dim * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+// ---- RoPE -------------------------------------------------------------------------------------
+
+PG_API pg_status pg_rope_create(pg_ctx *ctx, size_t head_dim, size_t max_seq_len, float base, pg_rope **out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(out != nullptr, "pg_rope_create: null output");
+    *out = nullptr;
+    PG_CHECK_ARG(head_dim > 0 && head_dim % 2 == 0, "pg_rope_create: head_dim %zu must be even and positive", head_dim);
+    PG_CHECK_ARG(max_seq_len > 0 && max_seq_len < (1ull << 31) && head_dim < (1ull << 16), "pg_rope_create: shape out of range");
+    // The tables are f32 libm values, as the reference computes them (src/nn.rs:1258-1282).
+    const size_t half = head_dim / 2, n = max_seq_len * head_dim;
+    std::vector<float> freq(half), c(n), s(n);
+    for (size_t i = 0; i < half; ++i) freq[i] = powf(base, 2.0f * (float)i / (float)head_dim);
+    for (size_t pos = 0; pos < max_seq_len; ++pos)
+        for (size_t i = 0; i < half; ++i) {
+            const float theta = (float)pos / freq[i];
+            const float cv = cosf(theta), sv = sinf(theta);
+            c[pos * head_dim + i] = cv; c[pos * head_dim + half + i] = cv;
+            s[pos * head_dim + i] = sv; s[pos * head_dim + half + i] = sv;
+        }
+    pg_rope *r = new (std::nothrow) pg_rope{nullptr, nullptr, head_dim, max_seq_len};
+    if (!r) return pg_fail(PG_ENOMEM, "pg_rope_create: out of host memory");
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&r->cos_t), n * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&r->sin_t), n * sizeof(float));
+    if (e == hipSuccess) e = hipMemcpyAsync(r->cos_t, c.data(), n * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(r->sin_t, s.data(), n * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        if (r->cos_t) (void)hipFree(r->cos_t);
+        if (r->sin_t) (void)hipFree(r->sin_t);
+        delete r;
+        return pg_fail(e == hipErrorOutOfMemory ? PG_ENOMEM : PG_EDEVICE, "pg_rope_create: %s", hipGetErrorString(e));
+    }
+    *out = r;
+    return PG_OK;
+}
+
+PG_API void pg_rope_free(pg_ctx *ctx, pg_rope *r) {
+    if (!r) return;
+    if (ctx) (void)pg_use(ctx);
+    if (r->cos_t) (void)hipFree(r->cos_t);
+    if (r->sin_t) (void)hipFree(r->sin_t);
+    delete r;
+}
+
+PG_API pg_status pg_rope_apply_dev(pg_ctx *ctx, const pg_rope *r, const float *x_dev, size_t seq_len, size_t offset,
+                                   float *out_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(r != nullptr, "pg_rope_apply: null table");
+    if (seq_len == 0) return PG_OK;
+    PG_CHECK_ARG(x_dev && out_dev, "pg_rope_apply: null pointer");
+    PG_CHECK_ARG(offset + seq_len <= r->max_seq_len, "pg_rope_apply: positions %zu..%zu exceed max_seq_len %zu", offset,
+                 offset + seq_len, r->max_seq_len);
+    rope_args ra = {};
+    ra.seg[0] = {x_dev, out_dev, r->head_dim, 0, 1, 1};
+    ra.cos_t = r->cos_t; ra.sin_t = r->sin_t; ra.hd = (int)r->head_dim; ra.pos0 = (int)offset; ra.nseg = 1;
+    return launch_rope(ctx, ra, seq_len, 1);
+}
+
+PG_API pg_status pg_rope_apply(pg_ctx *ctx, const pg_rope *r, const float *x, size_t seq_len, size_t offset, float *out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(r != nullptr, "pg_rope_apply: null table");
+    if (seq_len == 0) return PG_OK;
+    PG_CHECK_ARG(x && out, "pg_rope_apply: null pointer");
+    const size_t bytes = seq_len * r->head_dim * sizeof(float);
+    pg_tmp dx, dout;
+    PG_TRY(dx.alloc(bytes));
+    PG_TRY(dout.alloc(bytes));
+    PG_HIP(hipMemcpyAsync(dx.p, x, bytes, hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_rope_apply_dev(ctx, r, dx.as<float>(), seq_len, offset, dout.as<float>()));
+    PG_HIP(hipMemcpyAsync(out, dout.p, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+// ---- KV cache ---------------------------------------------------------------------------------
+
+PG_API pg_status pg_kv_cache_create(pg_ctx *ctx, size_t num_kv_heads, size_t head_dim, pg_kv_cache **out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(out != nullptr, "pg_kv_cache_create: null output");
+    *out = nullptr;
+    PG_CHECK_ARG(num_kv_heads > 0 && head_dim > 0 && head_dim <= 256 && num_kv_heads < 65536,
+                 "pg_kv_cache_create: num_kv_heads %zu / head_dim %zu out of range (head_dim <= 256)", num_kv_heads, head_dim);
+    pg_kv_cache *c = new (std::nothrow) pg_kv_cache{nullptr, nullptr, 0, 0, num_kv_heads, head_dim};
+    if (!c) return pg_fail(PG_ENOMEM, "pg_kv_cache_create: out of host memory");
+    *out = c;
+    return PG_OK;
+}
+
+PG_API void pg_kv_cache_free(pg_ctx *ctx, pg_kv_cache *c) {
+    if (!c) return;
+    if (ctx) {
+        (void)pg_use(ctx);
+        (void)hipStreamSynchronize(ctx->stream);
+    }
+    if (c->k) (void)hipFree(c->k);
+    if (c->v) (void)hipFree(c->v);
+    delete c;
+}
+
+PG_API size_t pg_kv_cache_len(const pg_kv_cache *c) { return c ? c->len : 0; }
+PG_API size_t pg_kv_cache_capacity(const pg_kv_cache *c) { return c ? c->capacity : 0; }
+
+PG_API pg_status pg_kv_cache_rollback_to(pg_kv_cache *c, size_t new_len) {
+    PG_CHECK_ARG(c != nullptr, "pg_kv_cache_rollback_to: null cache");
+    PG_CHECK_ARG(new_len <= c->len, "rollback_to: new_len %zu > current len %zu", new_len, c->len);
+    c->len = new_len;
+    return PG_OK;
+}
+
+PG_API pg_status pg_kv_cache_append_dev(pg_ctx *ctx, pg_kv_cache *c, const float *new_k_dev, const float *new_v_dev,
+                                        size_t seq_len) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(c != nullptr, "pg_kv_cache_append: null cache");
+    if (seq_len == 0) return PG_OK;
+    PG_CHECK_ARG(new_k_dev && new_v_dev, "pg_kv_cache_append: null pointer");
+    PG_CHECK_ARG(c->len + seq_len < (1ull << 31), "pg_kv_cache_append: length beyond 2^31");
+    PG_TRY(cache_reserve(ctx, c, c->len + seq_len));
+    const size_t hd = c->head_dim, width = seq_len * hd * sizeof(float);
+    PG_HIP(hipMemcpy2DAsync(c->k + c->len * hd, c->capacity * hd * sizeof(float), new_k_dev, width, width,
+                            c->num_kv_heads, hipMemcpyDeviceToDevice, ctx->stream));
+    PG_HIP(hipMemcpy2DAsync(c->v + c->len * hd, c->capacity * hd * sizeof(float), new_v_dev, width, width,
+                            c->num_kv_heads, hipMemcpyDeviceToDevice, ctx->stream));
+    c->len += seq_len;
+    return PG_OK;
+}
+
+PG_API pg_status pg_kv_cache_append(pg_ctx *ctx, pg_kv_cache *c, const float *new_k, const float *new_v, size_t seq_len) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(c != nullptr, "pg_kv_cache_append: null cache");
+    if (seq_len == 0) return PG_OK;
+    PG_CHECK_ARG(new_k && new_v, "pg_kv_cache_append: null pointer");
+    const size_t bytes = c->num_kv_heads * seq_len * c->head_dim * sizeof(float);
+    pg_tmp dk, dv;
+    PG_TRY(dk.alloc(bytes));
+    PG_TRY(dv.alloc(bytes));
+    PG_HIP(hipMemcpyAsync(dk.p, new_k, bytes, hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(dv.p, new_v, bytes, hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_kv_cache_append_dev(ctx, c, dk.as<float>(), dv.as<float>(), seq_len));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+PG_API pg_status pg_kv_cache_download(pg_ctx *ctx, const pg_kv_cache *c, float *k, float *v) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(c != nullptr, "pg_kv_cache_download: null cache");
+    if (c->len == 0) return PG_OK;
+    PG_CHECK_ARG(k && v, "pg_kv_cache_download: null pointer");
+    const size_t hd = c->head_dim, width = c->len * hd * sizeof(float);
+    PG_HIP(hipMemcpy2DAsync(k, width, c->k, c->capacity * hd * sizeof(float), width, c->num_kv_heads,
+                            hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipMemcpy2DAsync(v, width, c->v, c->capacity * hd * sizeof(float), width, c->num_kv_heads,
+                            hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+// ---- grouped-query attention ------------------------------------------------------------------
+
+PG_API pg_status pg_gqa_attention_dev(pg_ctx *ctx, const float *q_dev, const pg_kv_cache *k_cache,
+                                      const pg_kv_cache *v_cache, size_t num_q_heads, size_t seq_q, float scale,
+                                      int mask_kind, size_t offset, size_t window, size_t sink_tokens, float logit_cap,
+                                      float *out_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_TRY(check_attention_args("pg_gqa_attention", k_cache, v_cache, num_q_heads, seq_q, mask_kind, offset));
+    if (seq_q == 0 || num_q_heads == 0) return PG_OK;
+    PG_CHECK_ARG(q_dev && out_dev, "pg_gqa_attention: null pointer");
+    return launch_attention(ctx, q_dev, k_cache, v_cache, num_q_heads, seq_q, scale, mask_kind, offset, window,
+                            sink_tokens, logit_cap, out_dev, 1);
+}
+
+PG_API pg_status pg_gqa_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *k_cache, const pg_kv_cache *v_cache,
+                                  size_t num_q_heads, size_t seq_q, float scale, int mask_kind, size_t offset,
+                                  size_t window, size_t sink_tokens, float logit_cap, float *out) {
+    PG_TRY(pg_use(ctx));
+    PG_TRY(check_attention_args("pg_gqa_attention", k_cache, v_cache, num_q_heads, seq_q, mask_kind, offset));
+    if (seq_q == 0 || num_q_heads == 0) return PG_OK;
+    PG_CHECK_ARG(q && out, "pg_gqa_attention: null pointer");
+    const size_t bytes = num_q_heads * seq_q * k_cache->head_dim * sizeof(float);
+    pg_tmp dq, dout;
+    PG_TRY(dq.alloc(bytes));
+    PG_TRY(dout.alloc(bytes));
+    PG_HIP(hipMemcpyAsync(dq.p, q, bytes, hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(dout.p, out, bytes, hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(launch_attention(ctx, dq.as<float>(), k_cache, v_cache, num_q_heads, seq_q, scale, mask_kind, offset, window,
+                            sink_tokens, logit_cap, dout.as<float>(), 1));
+    PG_HIP(hipMemcpyAsync(out, dout.p, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+// ---- the decoder block ------------------------------------------------------------------------
+
+PG_API pg_status pg_llama_block_create(pg_ctx *ctx, size_t model_dim, size_t num_q_heads, size_t num_kv_heads,
+                                       size_t head_dim, size_t ffn_dim, size_t max_seq_len, float rope_base,
+                                       float rms_eps, pg_llama_block **out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(out != nullptr, "pg_llama_block_create: null output");
+    *out = nullptr;
+    PG_CHECK_ARG(model_dim > 0 && ffn_dim > 0 && num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0,
+                 "pg_llama_block_create: bad shape (d %zu, ffn %zu, heads %zu/%zu)", model_dim, ffn_dim, num_q_heads,
+                 num_kv_heads);
+    PG_CHECK_ARG(head_dim <= 256 && num_q_heads < 65536, "pg_llama_block_create: head_dim %zu > 256 or too many heads", head_dim);
+    PG_CHECK_ARG(model_dim % 32 == 0 && ffn_dim % 32 == 0 && (num_q_heads * head_dim) % 32 == 0,
+                 "pg_llama_block_create: model_dim, ffn_dim and num_q_heads*head_dim must be multiples of the 32-value GGUF block");
+    pg_llama_block *b = new (std::nothrow) pg_llama_block{};
+    if (!b) return pg_fail(PG_ENOMEM, "pg_llama_block_create: out of host memory");
+    b->d = model_dim; b->nqh = num_q_heads; b->nkvh = num_kv_heads; b->hd = head_dim; b->ffn = ffn_dim; b->eps = rms_eps;
+    pg_status st = pg_rope_create(ctx, head_dim, max_seq_len, rope_base, &b->rope);
+    if (st == PG_OK) {
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&b->attn_norm_w), 2 * model_dim * sizeof(float));
+        if (e != hipSuccess) st = pg_fail(PG_ENOMEM, "pg_llama_block_create: %s", hipGetErrorString(e));
+    }
+    if (st != PG_OK) {
+        pg_rope_free(ctx, b->rope);
+        delete b;
+        return st;
+    }
+    b->ffn_norm_w = b->attn_norm_w + model_dim;
+    *out = b;
+    return PG_OK;
+}
+
+PG_API void pg_llama_block_free(pg_ctx *ctx, pg_llama_block *b) {
+    if (!b) return;
+    if (ctx) {
+        (void)pg_use(ctx);
+        (void)hipStreamSynchronize(ctx->stream);
+    }
+    pg_rope_free(ctx, b->rope);
+    if (b->attn_norm_w) (void)hipFree(b->attn_norm_w);
+    if (b->arena) (void)hipFree(b->arena);
+    delete b;
+}
+
+PG_API pg_status pg_llama_block_set_weights(pg_ctx *ctx, pg_llama_block *b, const pg_gguf_tensor *q_proj,
+                                            const pg_gguf_tensor *k_proj, const pg_gguf_tensor *v_proj,
+                                            const pg_gguf_tensor *o_proj, const pg_gguf_tensor *gate_proj,
+                                            const pg_gguf_tensor *up_proj, const pg_gguf_tensor *down_proj,
+                                            const float *attn_norm_w, const float *ffn_norm_w) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(b != nullptr, "pg_llama_block_set_weights: null block");
+    const pg_gguf_tensor *w[7] = {q_proj, k_proj, v_proj, o_proj, gate_proj, up_proj, down_proj};
+    const size_t q_dim = b->nqh * b->hd, kv_dim = b->nkvh * b->hd;
+    const size_t want[7][2] = {{q_dim, b->d}, {kv_dim, b->d}, {kv_dim, b->d}, {b->d, q_dim},
+                               {b->ffn, b->d}, {b->ffn, b->d}, {b->d, b->ffn}};
+    static const char *names[7] = {"q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"};
+    for (int i = 0; i < 7; ++i) {
+        PG_CHECK_ARG(w[i] != nullptr, "pg_llama_block_set_weights: %s is null", names[i]);
+        PG_CHECK_ARG(w[i]->n_out == want[i][0] && w[i]->k_in == want[i][1],
+                     "pg_llama_block_set_weights: %s is [%zu, %zu], expected [%zu, %zu] (out, in)", names[i], w[i]->n_out,
+                     w[i]->k_in, want[i][0], want[i][1]);
+    }
+    PG_CHECK_ARG(attn_norm_w && ffn_norm_w, "pg_llama_block_set_weights: null norm weights");
+    PG_HIP(hipMemcpyAsync(b->attn_norm_w, attn_norm_w, b->d * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(b->ffn_norm_w, ffn_norm_w, b->d * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    for (int i = 0; i < 7; ++i) b->w[i] = w[i];
+    return PG_OK;
+}
+
+PG_API pg_status pg_llama_block_forward_dev(pg_ctx *ctx, pg_llama_block *b, const float *h_dev, size_t seq,
+                                            pg_kv_cache *cache, float *out_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(b && cache, "pg_llama_block_forward: null block or cache");
+    PG_CHECK_ARG(b->w[0] != nullptr, "pg_llama_block_forward: weights not set");
+    PG_CHECK_ARG(cache->num_kv_heads == b->nkvh && cache->head_dim == b->hd,
+                 "pg_llama_block_forward: cache is %zu heads x %zu, block is %zu x %zu", cache->num_kv_heads,
+                 cache->head_dim, b->nkvh, b->hd);
+    if (seq == 0) return PG_OK;
+    PG_CHECK_ARG(h_dev && out_dev, "pg_llama_block_forward: null pointer");
+    PG_CHECK_ARG(seq < (1ull << 24), "pg_llama_block_forward: seq %zu too large", seq);
+    const size_t offset = cache->len;
+    PG_CHECK_ARG(offset + seq <= b->rope->max_seq_len, "pg_llama_block_forward: positions %zu..%zu exceed max_seq_len %zu",
+                 offset, offset + seq, b->rope->max_seq_len);
+    const size_t d = b->d, hd = b->hd, q_dim = b->nqh * hd, kv_dim = b->nkvh * hd, ffn = b->ffn;
+    // activation arena: every slice a multiple of 64 floats so that each stays 256-byte aligned
+    auto slot = [](size_t n) { return pg_round_up(n, 64); };
+    if (seq > b->seq_cap) {
+        const size_t cap = seq > 2 * b->seq_cap ? seq : 2 * b->seq_cap;
+        const size_t floats = 3 * slot(cap * d) + 3 * slot(cap * q_dim) + 2 * slot(cap * kv_dim) + 2 * slot(cap * ffn);
+        PG_HIP(hipStreamSynchronize(ctx->stream));
+        if (b->arena) (void)hipFree(b->arena);
+        b->arena = nullptr;
+        b->seq_cap = 0;
+        PG_HIP(hipMalloc(reinterpret_cast<void **>(&b->arena), floats * sizeof(float)));
+        b->seq_cap = cap;
+    }
+    const size_t cap = b->seq_cap;
+    float *p = b->arena;
+    auto take = [&](size_t n) { float *r = p; p += slot(n); return r; };
+    float *normed = take(cap * d), *h1 = take(cap * d), *proj = take(cap * d);
+    float *qd = take(cap * q_dim), *q_rope = take(cap * q_dim), *attn = take(cap * q_dim);
+    float *kd = take(cap * kv_dim), *vd = take(cap * kv_dim);
+    float *g = take(cap * ffn), *u = take(cap * ffn);
+
+    PG_TRY(launch_rmsnorm(ctx, h_dev, nullptr, nullptr, b->attn_norm_w, b->eps, seq, d, normed));
+    PG_TRY(pg_gguf_matmul_rows(ctx, normed, seq, b->w[0], qd));
+    PG_TRY(pg_gguf_matmul_rows(ctx, normed, seq, b->w[1], kd));
+    PG_TRY(pg_gguf_matmul_rows(ctx, normed, seq, b->w[2], vd));
+    PG_TRY(cache_reserve(ctx, cache, offset + seq));
+    rope_args ra = {};
+    ra.seg[0] = {qd, q_rope, q_dim, seq * hd, (int)b->nqh, 1};
+    ra.seg[1] = {kd, cache->k + offset * hd, kv_dim, cache->capacity * hd, (int)b->nkvh, 1};
+    ra.seg[2] = {vd, cache->v + offset * hd, kv_dim, cache->capacity * hd, (int)b->nkvh, 0};
+    ra.cos_t = b->rope->cos_t; ra.sin_t = b->rope->sin_t; ra.hd = (int)hd; ra.pos0 = (int)offset; ra.nseg = 3;
+    PG_TRY(launch_rope(ctx, ra, seq, b->nqh + 2 * b->nkvh));
+    cache->len = offset + seq;
+    PG_TRY(launch_attention(ctx, q_rope, cache, cache, b->nqh, seq, 1.0f / sqrtf((float)hd), PG_MASK_CAUSAL, offset, 0, 0,
+                            0.0f, attn, 0));
+    PG_TRY(pg_gguf_matmul_rows(ctx, attn, seq, b->w[3], proj));
+    PG_TRY(launch_rmsnorm(ctx, h_dev, proj, h1, b->ffn_norm_w, b->eps, seq, d, normed));
+    PG_TRY(pg_gguf_matmul_rows(ctx, normed, seq, b->w[4], g));
+    PG_TRY(pg_gguf_matmul_rows(ctx, normed, seq, b->w[5], u));
+    PG_TRY(pg_launch(ctx, "swiglu", swiglu_kernel, dim3(blocks_for(seq * ffn)), dim3(256), 0, g, (const float *)u, seq * ffn));
+    PG_TRY(pg_gguf_matmul_rows(ctx, g, seq, b->w[6], proj));
+    return pg_launch(ctx, "residual_add", add_kernel, dim3(blocks_for(seq * d)), dim3(256), 0, (const float *)h1,
+                     (const float *)proj, out_dev, seq * d);
+}
+
+PG_API pg_status pg_llama_block_forward(pg_ctx *ctx, pg_llama_block *b, const float *h, size_t seq, pg_kv_cache *cache,
+                                        float *out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(b != nullptr, "pg_llama_block_forward: null block");
+    if (seq == 0) return PG_OK;
+    PG_CHECK_ARG(h && out, "pg_llama_block_forward: null pointer");
+    const size_t bytes = seq * b->d * sizeof(float);
+    pg_tmp dh, dout;
+    PG_TRY(dh.alloc(bytes));
+    PG_TRY(dout.alloc(bytes));
+    PG_HIP(hipMemcpyAsync(dh.p, h, bytes, hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_llama_block_forward_dev(ctx, b, dh.as<float>(), seq, cache, dout.as<float>()));
+    PG_HIP(hipMemcpyAsync(out, dout.p, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}

@@ -1,0 +1,234 @@
+"""GPU parity of the Llama decoder-block glue against the CPU oracle, through the C ABI.
+
+Bars: RMSNorm, RoPE and attention are f32 ports with a different (tree / sliced) summation
+order: 1e-5 relative (H.assert_close_rel).  The KV cache is a byte copy: bit-exact.  The
+whole block chains seven block-dequant products, each inside the 1e-3 contract for
+Q4_0/Q8_0 paths; the block is held to that same 1e-3 against the oracle's block.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+RTOL_F32 = 1e-5
+RTOL_BLOCK = 1e-3
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 4096), (5, 96), (3, 257), (64, 4096), (2, 1)])
+def test_rmsnorm(ctx, orc, rows, dim):
+    from peregrine_amd import llama
+    say(f"rmsnorm rows={rows} dim={dim}")
+    x = orc.rng_normal(rows * 7 + dim, rows * dim)
+    x[:dim] *= 50.0                                   # one loud row
+    norm = llama.RMSNorm(dim, 1e-5, ctx)
+    norm.weight = (1 + 0.1 * orc.rng_normal(3, dim)).astype(np.float32)
+    got = norm.forward(x.reshape(rows, dim))
+    H.assert_close_rel(got, orc.rmsnorm(x, rows, dim, norm.weight, 1e-5), RTOL_F32, "rmsnorm")
+    assert norm.forward(np.zeros((0, dim), np.float32)).shape == (0, dim)
+    with pytest.raises(ValueError):
+        norm.forward(np.zeros((2, dim + 1), np.float32))
+
+
+def test_rmsnorm_closed_form(ctx):
+    from peregrine_amd import llama
+    norm = llama.RMSNorm(64, 0.0, ctx)
+    norm.weight = np.arange(64, dtype=np.float32) / 8
+    got = norm.forward(np.full((1, 64), -3.0, np.float32))          # x / rms(x) = -1 for a constant row
+    assert np.allclose(got[0], -norm.weight, rtol=0, atol=1e-6 * 8)
+    assert (llama.RMSNorm(64, 1e-5, ctx).forward(np.zeros((1, 64), np.float32)) == 0).all()
+
+
+@pytest.mark.parametrize("hd,seq,offset", [(8, 5, 3), (128, 7, 0), (64, 1, 100), (2, 4, 1)])
+def test_rope(ctx, orc, hd, seq, offset):
+    from peregrine_amd import llama, _ffi
+    say(f"rope hd={hd} seq={seq} offset={offset}")
+    n = 128
+    rope = llama.RoPE(hd, n, 10000.0, ctx)
+    cos, sin = orc.rope_tables(hd, n, 10000.0)
+    x = orc.rng_normal(hd + seq, seq * hd).reshape(seq, hd)
+    got = rope.apply(x, offset)
+    want = orc.rope_apply(x, seq, hd, offset, cos, sin).reshape(seq, hd)
+    # same f32 expression per element; only libm's cos/sin/pow may differ in the last bit
+    H.assert_close_rel(got, want, 1e-6, "rope")
+    assert (rope.apply(x[:1], 0) == x[:1]).all()                    # position 0 is the identity
+    with pytest.raises(_ffi.PeregrineError):
+        rope.apply(x, n - seq + 1)                                    # past max_seq_len: the reference's slice panic
+    with pytest.raises(_ffi.PeregrineError):
+        llama.RoPE(7, 16, 10000.0, ctx)
+
+
+def test_kv_cache_append_growth_rollback(ctx, orc):
+    """StandardKVCache semantics (src/attention.rs:18-98): growth keeps old rows, capacity at
+    least doubles from 16, rollback truncates logically, appends after rollback overwrite."""
+    from peregrine_amd import llama, _ffi
+    nkv, hd = 3, 8
+    cache = llama.StandardKVCache(nkv, hd, ctx)
+    assert cache.len == 0 and cache.head_stride() == 0
+    mirror_k = np.zeros((nkv, 0, hd), np.float32)
+    mirror_v = np.zeros((nkv, 0, hd), np.float32)
+    caps = []
+    for step, seq in enumerate((1, 5, 30, 1, 40)):
+        k = orc.rng_normal(10 + step, nkv * seq * hd).reshape(nkv, seq, hd)
+        v = orc.rng_normal(20 + step, nkv * seq * hd).reshape(nkv, seq, hd)
+        cache.append(k, v, seq)
+        mirror_k = np.concatenate([mirror_k, k], 1)
+        mirror_v = np.concatenate([mirror_v, v], 1)
+        gk, gv = cache.to_host()
+        assert cache.len == mirror_k.shape[1]
+        assert (gk == mirror_k).all() and (gv == mirror_v).all()
+        caps.append(cache.head_stride() // hd)
+    assert caps == [32, 32, 64, 64, 128]            # needed.max(capacity.max(16) * 2)
+    cache.rollback_to(10)
+    assert cache.len == 10 and cache.head_stride() == 128 * hd
+    with pytest.raises(_ffi.PeregrineError):
+        cache.rollback_to(11)
+    k = orc.rng_normal(31, nkv * 2 * hd).reshape(nkv, 2, hd)
+    cache.append(k, k, 2)
+    gk, gv = cache.to_host()
+    assert (gk[:, :10] == mirror_k[:, :10]).all() and (gk[:, 10:] == k).all() and (gv[:, 10:] == k).all()
+    with pytest.raises(ValueError):
+        cache.append(k, k, 3)
+
+
+def _attention_case(ctx, orc, nqh, nkvh, hd, seq_q, length, mask, logit_cap, seed, appends=None):
+    from peregrine_amd import llama
+    cache = llama.StandardKVCache(nkvh, hd, ctx)
+    k = orc.rng_normal(seed, nkvh * length * hd).reshape(nkvh, length, hd)
+    v = orc.rng_normal(seed + 1, nkvh * length * hd).reshape(nkvh, length, hd)
+    pos = 0
+    for n in appends or (length,):                   # several appends: capacity > len, strides matter
+        cache.append(k[:, pos:pos + n], v[:, pos:pos + n], n)
+        pos += n
+    assert pos == length
+    q = orc.rng_normal(seed + 2, nqh * seq_q * hd).reshape(nqh, seq_q, hd)
+    scale = 1 / np.sqrt(hd)
+    base = orc.rng_normal(seed + 3, seq_q * nqh * hd)            # the output is added to, not overwritten
+    got = base.copy()
+    llama.gqa_attention(q, cache, cache, nqh, nkvh, seq_q, hd, scale, mask, logit_cap, got, ctx)
+    want = orc.gqa_attention(q, k, v, length, length, nqh, nkvh, seq_q, hd, scale, mask.kind, mask.offset, mask.window,
+                             mask.sink_tokens, logit_cap or 0.0)
+    H.assert_close_rel(got - base, want, RTOL_F32 * 4, "gqa_attention")   # (base + o) - base rounds once more
+    return got
+
+
+@pytest.mark.parametrize("nqh,nkvh,hd,seq_q,length", [
+    (2, 2, 4, 2, 3),          # tests/attention.rs MHA shape
+    (4, 2, 4, 2, 3),          # GQA ratio 2
+    (4, 1, 4, 2, 3),          # MQA
+    (32, 8, 128, 1, 1000),    # Llama-3-8B decode step
+    (8, 2, 64, 5, 77),
+    (6, 3, 20, 3, 40),        # head_dim not a power of two
+    (2, 1, 6, 2, 9),          # head_dim not a multiple of 4: the scalar path
+    (2, 2, 256, 1, 300),
+])
+def test_gqa_attention_unmasked(ctx, orc, nqh, nkvh, hd, seq_q, length):
+    from peregrine_amd import llama
+    say(f"attention nqh={nqh} nkvh={nkvh} hd={hd} seq_q={seq_q} len={length}")
+    _attention_case(ctx, orc, nqh, nkvh, hd, seq_q, length, llama.AttentionMask.none(), None, 100 + hd,
+                    appends=(1, length - 1) if length > 1 else None)
+
+
+def test_gqa_attention_masks_and_logit_cap(ctx, orc):
+    from peregrine_amd import llama
+    M = llama.AttentionMask
+    for mask, cap in ((M.causal(0), None), (M.causal(20), None), (M.causal_sliding_window(27, 5, 2), None),
+                      (M.causal_sliding_window(27, 0, 0), None), (M.none(), 1.5), (M.causal(27), 30.0)):
+        say(f"attention mask={mask} cap={cap}")
+        _attention_case(ctx, orc, 8, 2, 32, 4, 31, mask, cap, 7)
+    # causal, offset 0, first query row sees only position 0: the output row is v[0] exactly
+    cache = llama.StandardKVCache(1, 8, ctx)
+    k = orc.rng_normal(1, 5 * 8).reshape(1, 5, 8)
+    v = orc.rng_normal(2, 5 * 8).reshape(1, 5, 8)
+    cache.append(k, v, 5)
+    out = np.zeros(2 * 8, np.float32)
+    llama.gqa_attention(orc.rng_normal(3, 2 * 8), cache, cache, 1, 1, 2, 8, 0.35, M.causal(0), None, out, ctx)
+    assert (out[:8] == v[0, 0]).all()
+
+
+def test_gqa_attention_long_cache_uses_global_scores(ctx, orc):
+    """Beyond 36864 positions the scores live in global memory instead of LDS."""
+    from peregrine_amd import llama
+    say("attention len=40000")
+    _attention_case(ctx, orc, 2, 1, 16, 1, 40000, llama.AttentionMask.causal(39999), None, 55)
+
+
+def test_gqa_attention_edges(ctx, orc):
+    from peregrine_amd import llama, _ffi
+    cache = llama.StandardKVCache(2, 8, ctx)
+    out = np.full(2 * 4 * 8, 3.0, np.float32)
+    llama.gqa_attention(np.ones(4 * 2 * 8, np.float32), cache, cache, 4, 2, 2, 8, 1.0, llama.AttentionMask.none(), None, out, ctx)
+    assert (out == 3.0).all()                         # empty cache: nothing is added
+    with pytest.raises(_ffi.PeregrineError):
+        llama.gqa_attention(np.ones(3 * 8, np.float32), cache, cache, 3, 2, 1, 8, 1.0, llama.AttentionMask.none(), None,
+                            np.zeros(3 * 8, np.float32), ctx)    # 3 query heads over 2 kv heads
+    with pytest.raises(ValueError):
+        llama.gqa_attention(np.ones(5, np.float32), cache, cache, 4, 2, 2, 8, 1.0, llama.AttentionMask.none(), None, out, ctx)
+
+
+def _block_case(ctx, orc, d, nqh, nkvh, hd, ffn, typ, steps, max_seq=64, seed=0):
+    from peregrine_amd import gguf, llama
+    shapes = [(nqh * hd, d), (nkvh * hd, d), (nkvh * hd, d), (d, nqh * hd), (ffn, d), (ffn, d), (d, ffn)]
+    pack = H.pack_q4_0 if typ == 2 else H.pack_q8_0
+    raws = [bytes(pack(orc.rng_normal(seed + 40 + i, n * k, 0.0, 1.0 / np.sqrt(k)))) for i, (n, k) in enumerate(shapes)]
+    ws = [gguf.GgufWeight(r, typ, n, k, ctx) for r, (n, k) in zip(raws, shapes)]
+    wa = (1 + 0.1 * orc.rng_normal(seed + 1, d)).astype(np.float32)
+    wf = (1 + 0.1 * orc.rng_normal(seed + 2, d)).astype(np.float32)
+    eps = 1e-5
+    blk = llama.LlamaBlock(d, nqh, nkvh, hd, ffn, max_seq, 10000.0, eps, ctx)
+    blk.set_weights(*ws, wa, wf)
+    cache = blk.new_cache()
+    cos, sin = orc.rope_tables(hd, max_seq, 10000.0)
+    kc = np.zeros((nkvh, max_seq, hd), np.float32)
+    vc = np.zeros((nkvh, max_seq, hd), np.float32)
+    pos = 0
+    for i, seq in enumerate(steps):
+        say(f"llama block d={d} heads={nqh}/{nkvh} hd={hd} ffn={ffn} type={typ} step {i}: seq={seq} at {pos}")
+        h = orc.rng_normal(seed + 90 + i, seq * d).reshape(seq, d)
+        got = blk.forward(h, cache)
+        want = orc.llama_block_forward(h, seq, d, nqh, nkvh, hd, ffn, typ, raws, wa, wf, eps, cos, sin, kc, vc, pos, max_seq)
+        pos += seq
+        assert cache.len == pos
+        H.assert_close_rel(got, want, RTOL_BLOCK, f"llama block step {i}")
+        gk, gv = cache.to_host()
+        H.assert_close_rel(gk, kc[:, :pos], RTOL_BLOCK, "k cache")
+        H.assert_close_rel(gv, vc[:, :pos], RTOL_BLOCK, "v cache")
+    return blk, cache
+
+
+@pytest.mark.parametrize("typ", [8, 2])
+def test_llama_block_prefill_then_decode(ctx, orc, typ):
+    """Prefill (matrix-core products), two decode steps (streaming GEMV), another prefill chunk."""
+    _block_case(ctx, orc, 256, 8, 2, 32, 512, typ, (5, 1, 1, 33))
+
+
+def test_llama_block_mha_and_odd_shapes(ctx, orc):
+    _block_case(ctx, orc, 96, 3, 3, 32, 160, 8, (1, 2, 1), seed=5)
+
+
+def test_llama_block_rollback_and_errors(ctx, orc):
+    from peregrine_amd import _ffi, llama
+    blk, cache = _block_case(ctx, orc, 128, 4, 2, 32, 256, 8, (4,), max_seq=8, seed=9)
+    h = orc.rng_normal(1, 2 * 128).reshape(2, 128)
+    a = blk.forward(h, cache)
+    cache.rollback_to(4)                               # speculative decoding: reject, replay
+    b = blk.forward(h, cache)
+    assert (a == b).all() and cache.len == 6
+    with pytest.raises(_ffi.PeregrineError):
+        blk.forward(orc.rng_normal(2, 3 * 128).reshape(3, 128), cache)   # 6 + 3 > max_seq_len 8
+    assert cache.len == 6
+    with pytest.raises(_ffi.PeregrineError):
+        blk.forward(h[:1], llama.StandardKVCache(3, 32, ctx))            # cache of another shape
+    with pytest.raises(_ffi.PeregrineError):
+        llama.LlamaBlock(128, 4, 2, 32, 256, 8, 10000.0, 1e-5, ctx).forward(h[:1], blk.new_cache())   # weights not set
+    with pytest.raises(_ffi.PeregrineError):
+        llama.LlamaBlock(128, 4, 3, 32, 256, 8, 10000.0, 1e-5, ctx)      # 4 query heads over 3 kv heads
+    assert blk.forward(np.zeros((0, 128), np.float32), cache).shape == (0, 128)
