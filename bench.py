@@ -341,6 +341,76 @@ def main():
             lib.pg_gguf_free(ctx.handle, h)
     torch.cuda.empty_cache()
 
+    # ------------------------------------------------------------------ one Llama-3-8B decoder block, Q4_0 weights
+    d_l, nqh_l, nkv_l, hd_l, ffn_l, ctx_len = 4096, 32, 8, 128, 14336, 1024
+    shapes_l = [(nqh_l * hd_l, d_l), (nkv_l * hd_l, d_l), (nkv_l * hd_l, d_l), (d_l, nqh_l * hd_l),
+                (ffn_l, d_l), (ffn_l, d_l), (d_l, ffn_l)]
+    L_ROT = 4  # 4 x 123 MB of block weights rotated: more than the 256 MB last-level cache
+    rng = np.random.default_rng(8)
+    blocks_l, keep_l = [], []
+    for r in range(L_ROT):
+        hs = []
+        for no, ki in shapes_l:
+            nb = no * ki // 32
+            rawb = np.empty((nb, 18), np.uint8)
+            rawb[:, 2:] = rng.integers(0, 256, size=(nb, 16), dtype=np.uint8)
+            rawb[:, :2] = np.frombuffer(np.float16(0.02 / 7 * 64 / np.sqrt(ki)).tobytes(), np.uint8)
+            h = C.c_void_p()
+            check(lib.pg_gguf_upload(ctx.handle, C.c_void_p(rawb.ctypes.data), _ffi.GGML_Q4_0, no, ki, C.byref(h)))
+            hs.append(h)
+        b = C.c_void_p()
+        check(lib.pg_llama_block_create(ctx.handle, d_l, nqh_l, nkv_l, hd_l, ffn_l, 4096, 500000.0, 1e-5, C.byref(b)))
+        ones = np.ones(d_l, np.float32)
+        check(lib.pg_llama_block_set_weights(ctx.handle, b, *hs, C.c_void_p(ones.ctypes.data), C.c_void_p(ones.ctypes.data)))
+        kv = C.c_void_p()
+        check(lib.pg_kv_cache_create(ctx.handle, nkv_l, hd_l, C.byref(kv)))
+        blocks_l.append((b, kv))
+        keep_l.append(hs)
+    w_bytes_l = sum(no * ki // 32 * 18 for no, ki in shapes_l)
+    h_pre = torch.randn(ctx_len, d_l, device=dev, generator=gen, dtype=torch.float32)
+    o_pre = torch.empty_like(h_pre)
+    h_dec = torch.randn(1, d_l, device=dev, generator=gen, dtype=torch.float32)
+    o_dec = torch.empty_like(h_dec)
+
+    def block_prefill():
+        b, kv = blocks_l[state["i"] % L_ROT]
+        state["i"] += 1
+        check(lib.pg_kv_cache_rollback_to(kv, 0))
+        check(lib.pg_llama_block_forward_dev(ctx.handle, b, ptr(h_pre), ctx_len, kv, ptr(o_pre)))
+
+    def block_decode():  # position ctx_len on top of the prefilled cache, then rolled back
+        b, kv = blocks_l[state["i"] % L_ROT]
+        state["i"] += 1
+        check(lib.pg_kv_cache_rollback_to(kv, ctx_len))
+        check(lib.pg_llama_block_forward_dev(ctx.handle, b, ptr(h_dec), 1, kv, ptr(o_dec)))
+
+    pre_ms = timed(block_prefill, 8, 4)  # leaves every cache filled to ctx_len
+    pre_prof = profiled(block_prefill, 8)
+    dec_ms = timed(block_decode, dsteps, max(args.warmup, 8))
+    dec_prof = profiled(block_decode, dsteps)
+    kv_bytes_l = 2 * nkv_l * (ctx_len + 1) * hd_l * 4
+    dec_bytes = w_bytes_l + kv_bytes_l
+    pre_flops = 2 * ctx_len * sum(no * ki for no, ki in shapes_l) + 4 * nqh_l * hd_l * ctx_len * (ctx_len + 1) // 2
+    llama_block = {
+        "workload": f"one Llama-3-8B decoder block (d 4096, 32/8 heads x 128, ffn 14336), Q4_0 projections ({w_bytes_l / 1e6:.0f} MB), "
+                    f"f32 KV cache; {L_ROT} blocks rotated",
+        "decode": {"what": f"seq 1 at position {ctx_len}", "ms_per_step": round(dec_ms, 5),
+                   "value": round(dec_bytes / (dec_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                   "frac_of_hbm_peak": round(dec_bytes / (dec_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                   "bytes_per_step": dec_bytes,
+                   "kernels_ms_x_launches": {k: [round(v[0], 5), round(v[1] / dsteps, 2)] for k, v in dec_prof.items()}},
+        "prefill": {"what": f"seq {ctx_len} into an empty cache", "ms_per_step": round(pre_ms, 4),
+                    "tflops": round(pre_flops / (pre_ms * 1e-3) / 1e12, 1),
+                    "tokens_per_s": round(ctx_len / (pre_ms * 1e-3), 0),
+                    "kernels_ms_x_launches": {k: [round(v[0], 5), round(v[1] / 8, 2)] for k, v in pre_prof.items()}},
+    }
+    for (b, kv), hs in zip(blocks_l, keep_l):
+        lib.pg_llama_block_free(ctx.handle, b)
+        lib.pg_kv_cache_free(ctx.handle, kv)
+        for h in hs:
+            lib.pg_gguf_free(ctx.handle, h)
+    torch.cuda.empty_cache()
+
     if args.calibrate_copy:  # a plain copy of known size: 512 MiB read + 512 MiB written per launch
         src = torch.empty(128 << 20, device=dev, dtype=torch.float32).normal_()
         dst = torch.empty_like(src)
@@ -364,7 +434,7 @@ def main():
                                "each product = per-row activation quantisation + i8 GEMM + f32 rescale",
                    "m": M_PREFILL, "ops_per_step": LAYER_OPS},
         "pct_int8_mfma_peak": round(100 * tops / PEAK_INT8_TOPS, 2),
-        "roofline": roofline, "activation_quant": act_quant, "w8a32_gate": w8a32, "linear_m32": linear_m32, "decode_gemv": decode, "gguf_q4_0_gemv": gguf, "gguf_q4_0_skinny": skinny, "moe_q8_0": moe,
+        "roofline": roofline, "activation_quant": act_quant, "w8a32_gate": w8a32, "linear_m32": linear_m32, "decode_gemv": decode, "gguf_q4_0_gemv": gguf, "gguf_q4_0_skinny": skinny, "moe_q8_0": moe, "llama_block_q4_0": llama_block,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line), flush=True)

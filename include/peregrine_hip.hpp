@@ -323,5 +323,139 @@ inline std::vector<float> expert_ffn(const GpuContext &gpu, const std::vector<fl
 }
 
 }  // namespace moe
+
+namespace llama {
+
+// nn::RMSNorm  src/nn.rs:560-652.
+class RMSNorm {
+public:
+    RMSNorm(const GpuContext &gpu, size_t dim, float eps) : weight(dim, 1.0f), gpu_(&gpu), eps_(eps) {}
+    std::vector<float> forward(const std::vector<float> &x) const {
+        if (weight.empty() || x.size() % weight.size()) throw Panic(PG_EINVAL, "RMSNorm::forward: x.len() % dim != 0");
+        std::vector<float> out(x.size());
+        check(pg_rmsnorm(gpu_->raw(), x.data(), x.size() / weight.size(), weight.size(), weight.data(), eps_, out.data()),
+              "RMSNorm::forward");
+        return out;
+    }
+    std::vector<float> weight;
+
+private:
+    const GpuContext *gpu_;
+    float eps_;
+};
+
+// nn::RoPE  src/nn.rs:1250-1345.
+class RoPE {
+public:
+    RoPE(const GpuContext &gpu, size_t head_dim, size_t max_seq_len, float base) : gpu_(&gpu), head_dim_(head_dim) {
+        check(pg_rope_create(gpu.raw(), head_dim, max_seq_len, base, &h_), "RoPE::new");
+    }
+    ~RoPE() { pg_rope_free(gpu_->raw(), h_); }
+    RoPE(const RoPE &) = delete;
+    RoPE &operator=(const RoPE &) = delete;
+    std::vector<float> apply(const std::vector<float> &x, size_t seq_len, size_t offset) const {
+        if (x.size() != seq_len * head_dim_) throw Panic(PG_EINVAL, "RoPE::apply: x.len() != seq_len * head_dim");
+        std::vector<float> out(x.size());
+        check(pg_rope_apply(gpu_->raw(), h_, x.data(), seq_len, offset, out.data()), "RoPE::apply");
+        return out;
+    }
+
+private:
+    const GpuContext *gpu_;
+    pg_rope *h_ = nullptr;
+    size_t head_dim_;
+};
+
+// attention::StandardKVCache  src/attention.rs:8-100.
+class StandardKVCache {
+public:
+    StandardKVCache(const GpuContext &gpu, size_t num_kv_heads, size_t head_dim)
+        : num_kv_heads(num_kv_heads), head_dim(head_dim), gpu_(&gpu) {
+        check(pg_kv_cache_create(gpu.raw(), num_kv_heads, head_dim, &h_), "StandardKVCache::new");
+    }
+    ~StandardKVCache() { pg_kv_cache_free(gpu_->raw(), h_); }
+    StandardKVCache(const StandardKVCache &) = delete;
+    StandardKVCache &operator=(const StandardKVCache &) = delete;
+    size_t len() const { return pg_kv_cache_len(h_); }
+    size_t head_stride() const { return pg_kv_cache_capacity(h_) * head_dim; }
+    void append(const std::vector<float> &new_k, const std::vector<float> &new_v, size_t seq_len) {
+        const size_t n = num_kv_heads * seq_len * head_dim;
+        if (new_k.size() != n || new_v.size() != n) throw Panic(PG_EINVAL, "StandardKVCache::append: slice lengths");
+        check(pg_kv_cache_append(gpu_->raw(), h_, new_k.data(), new_v.data(), seq_len), "StandardKVCache::append");
+    }
+    void rollback_to(size_t new_len) { check(pg_kv_cache_rollback_to(h_, new_len), "StandardKVCache::rollback_to"); }
+    pg_kv_cache *handle() const { return h_; }
+    const size_t num_kv_heads, head_dim;
+
+private:
+    const GpuContext *gpu_;
+    pg_kv_cache *h_ = nullptr;
+};
+using KVCache = StandardKVCache;  // src/models/llama/attention.rs:7
+
+// attention::AttentionMask  src/attention.rs:102-120 (no LocalGlobal).
+struct AttentionMask {
+    int kind = PG_MASK_NONE;
+    size_t offset = 0, window = 0, sink_tokens = 0;
+    static AttentionMask None() { return {}; }
+    static AttentionMask Causal(size_t offset) { return {PG_MASK_CAUSAL, offset, 0, 0}; }
+    static AttentionMask CausalSlidingWindow(size_t offset, size_t window, size_t sink_tokens) {
+        return {PG_MASK_CAUSAL_SLIDING_WINDOW, offset, window, sink_tokens};
+    }
+};
+
+// attention::gqa_attention_cpu  src/attention.rs:141-265; `output` is added to.
+inline void gqa_attention(const GpuContext &gpu, const std::vector<float> &q, const StandardKVCache &k_cache,
+                          const StandardKVCache &v_cache, size_t num_q_heads, size_t num_kv_heads, size_t seq_q,
+                          size_t head_dim, float scale, const AttentionMask &mask, float logit_cap,
+                          std::vector<float> &output) {
+    if (num_kv_heads != k_cache.num_kv_heads || head_dim != k_cache.head_dim)
+        throw Panic(PG_EINVAL, "gqa_attention: num_kv_heads / head_dim differ from the cache's");
+    if (q.size() != num_q_heads * seq_q * head_dim || output.size() != q.size())
+        throw Panic(PG_EINVAL, "gqa_attention: q / output lengths");
+    check(pg_gqa_attention(gpu.raw(), q.data(), k_cache.handle(), v_cache.handle(), num_q_heads, seq_q, scale, mask.kind,
+                           mask.offset, mask.window, mask.sink_tokens, logit_cap, output.data()),
+          "gqa_attention");
+}
+
+// LlamaBlock  src/models/llama/decoder.rs:7-155 over block-quantised projections.
+class LlamaBlock {
+public:
+    LlamaBlock(const GpuContext &gpu, size_t model_dim, size_t num_q_heads, size_t num_kv_heads, size_t head_dim,
+               size_t ffn_dim, size_t max_seq_len, float rope_base, float rms_eps)
+        : gpu_(&gpu), model_dim_(model_dim) {
+        check(pg_llama_block_create(gpu.raw(), model_dim, num_q_heads, num_kv_heads, head_dim, ffn_dim, max_seq_len,
+                                    rope_base, rms_eps, &h_),
+              "LlamaBlock::new");
+    }
+    ~LlamaBlock() { pg_llama_block_free(gpu_->raw(), h_); }
+    LlamaBlock(const LlamaBlock &) = delete;
+    LlamaBlock &operator=(const LlamaBlock &) = delete;
+    // The block borrows the weights: they must outlive it.
+    void set_weights(const gguf::BlockWeight &q_proj, const gguf::BlockWeight &k_proj, const gguf::BlockWeight &v_proj,
+                     const gguf::BlockWeight &o_proj, const gguf::BlockWeight &gate_proj, const gguf::BlockWeight &up_proj,
+                     const gguf::BlockWeight &down_proj, const std::vector<float> &attn_norm_w,
+                     const std::vector<float> &ffn_norm_w) {
+        if (attn_norm_w.size() != model_dim_ || ffn_norm_w.size() != model_dim_)
+            throw Panic(PG_EINVAL, "LlamaBlock::set_weights: norm weights are not [model_dim]");
+        check(pg_llama_block_set_weights(gpu_->raw(), h_, q_proj.handle(), k_proj.handle(), v_proj.handle(), o_proj.handle(),
+                                         gate_proj.handle(), up_proj.handle(), down_proj.handle(), attn_norm_w.data(),
+                                         ffn_norm_w.data()),
+              "LlamaBlock::set_weights");
+    }
+    std::vector<float> forward(const std::vector<float> &h, size_t seq, KVCache &kv_cache) const {
+        if (h.size() != seq * model_dim_) throw Panic(PG_EINVAL, "LlamaBlock::forward: h.len() != seq * model_dim");
+        std::vector<float> out(h.size());
+        check(pg_llama_block_forward(gpu_->raw(), h_, h.data(), seq, kv_cache.handle(), out.data()), "LlamaBlock::forward");
+        return out;
+    }
+
+private:
+    const GpuContext *gpu_;
+    pg_llama_block *h_ = nullptr;
+    size_t model_dim_;
+};
+
+}  // namespace llama
 }  // namespace peregrine
 #endif  // PEREGRINE_HIP_HPP

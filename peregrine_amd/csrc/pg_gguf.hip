@@ -458,6 +458,52 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
     return pg_launch_gguf_mm(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, grp, m, md, y_dev, part);
 }
 
+// Several products over the same activation rows (q/k/v, gate/up): the rows are rewritten
+// as digits once per ggml type in use instead of once per product.  All k_in are equal.
+pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *const *w,
+                                    float *const *y_dev, int count) {
+    if (count <= 0 || m == 0) return PG_OK;
+    const size_t k_in = w[0]->k_in;
+    for (int i = 1; i < count; ++i)
+        if (w[i]->k_in != k_in) return pg_fail(PG_EINVAL, "gguf_matmul_multi: the products differ in k_in");
+    void *ws = nullptr;
+    int digits_type = -1;
+    if (m == 1) {
+        PG_TRY(pg_workspace(ctx, pg_xdigits_bytes(m, k_in), &ws));
+        const pg_xdigits xd = pg_xdigits_carve(ws, m, k_in);
+        const pg_gemv_batch batch = {1, nullptr, nullptr, nullptr, 1};
+        for (int i = 0; i < count; ++i) {
+            if (w[i]->ggml_type != digits_type) {
+                PG_TRY(pg_launch_x_to_digits(ctx, x_dev, m, k_in, w[i]->ggml_type, xd));
+                digits_type = w[i]->ggml_type;
+            }
+            PG_TRY(pg_launch_gguf_gemv(ctx, w[i]->ggml_type, w[i]->n_out, k_in, w[i]->qs, w[i]->d, batch, xd, y_dev[i]));
+        }
+        return PG_OK;
+    }
+    const size_t sz_d = pg_mmdigits_bytes(m, k_in);
+    size_t sz_part = 0;
+    for (int i = 0; i < count; ++i) {
+        const int ks = pg_gguf_mm_splitk(ctx, w[i]->n_out, k_in, 1, nullptr);
+        const size_t sz = ks > 1 ? pg_round_up((size_t)ks * m * w[i]->n_out * sizeof(float), 256) : 0;
+        if (sz > sz_part) sz_part = sz;
+    }
+    PG_TRY(pg_workspace(ctx, sz_d + sz_part, &ws));
+    const pg_mmdigits md = pg_mmdigits_carve(ws, m, k_in);
+    float *part_base = reinterpret_cast<float *>(static_cast<char *>(ws) + sz_d);
+    const pg_mm_group grp = {1, nullptr, nullptr, nullptr, nullptr, 0, (int)((m + 31) / 32), (int)m, 1};
+    for (int i = 0; i < count; ++i) {
+        if (w[i]->ggml_type != digits_type) {
+            PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, m, k_in, w[i]->ggml_type, md));
+            digits_type = w[i]->ggml_type;
+        }
+        const int ks = pg_gguf_mm_splitk(ctx, w[i]->n_out, k_in, 1, nullptr);
+        PG_TRY(pg_launch_gguf_mm(ctx, w[i]->ggml_type, w[i]->n_out, k_in, w[i]->qs, w[i]->d, grp, m, md, y_dev[i],
+                                 ks > 1 ? part_base : nullptr));
+    }
+    return PG_OK;
+}
+
 PG_API pg_status pg_f16_to_f32(pg_ctx *ctx, const uint16_t *bits, size_t n, float *out) {
     PG_TRY(pg_use(ctx));
     if (n == 0) return PG_OK;

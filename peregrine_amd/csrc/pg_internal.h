@@ -227,3 +227,6 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
 // y[m, n_out] = x[m, k_in] . dequant(w)^T on device pointers (uses the scratch arena).
 pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
                               float *y_dev);
+// `count` such products over the same rows (equal k_in), the rows rewritten as digits once.
+pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *const *w,
+                                    float *const *y_dev, int count);

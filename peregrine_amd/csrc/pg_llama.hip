@@ -62,9 +62,10 @@ __device__ __forceinline__ float block_max(float v, float *red) {
 }
 
 // One workgroup per row: s = a (+ b), optionally stored, then out = s / rms(s) * w.
+// Generic two-pass form for any dim.
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(const float *a, const float *__restrict__ b, float *sum_out,
-                                                          const float *__restrict__ w,
-                                                          float eps, int dim, float *__restrict__ out) {
+                                                          const float *__restrict__ w, float eps, int dim,
+                                                          float *__restrict__ out) {
     __shared__ float red[4];
     const size_t row = (size_t)blockIdx.x * dim;
     float ss = 0.f;
@@ -80,6 +81,50 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(const float *a, const 
     const float inv_rms = 1.0f / sqrtf(ss * (1.0f / (float)dim) + eps);
     const float *src = b ? sum_out : a;  // a thread re-reads only what it wrote itself
     for (int i = threadIdx.x; i < dim; i += 256) out[row + i] = src[row + i] * inv_rms * w[i];
+}
+
+// The same with the row held in registers: dim % 4 == 0 and dim <= 1024 * MAXV, so that every
+// load of the row is issued before the first is needed.
+template <int MAXV>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(const float4 *__restrict__ a, const float4 *__restrict__ b,
+                                                              float4 *__restrict__ sum_out, const float4 *__restrict__ w,
+                                                              float eps, int dim4, float4 *__restrict__ out) {
+    __shared__ float red[4];
+    const size_t row = (size_t)blockIdx.x * dim4;
+    float4 v[MAXV], wv[MAXV];
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        v[j] = i < dim4 ? a[row + i] : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (b) {
+#pragma unroll
+        for (int j = 0; j < MAXV; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            if (i < dim4) {
+                const float4 t = b[row + i];
+                v[j].x += t.x; v[j].y += t.y; v[j].z += t.z; v[j].w += t.w;
+                sum_out[row + i] = v[j];
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        wv[j] = i < dim4 ? w[i] : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+    ss = block_sum(ss, red);
+    const float inv_rms = 1.0f / sqrtf(ss * (1.0f / (float)(dim4 * 4)) + eps);
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        if (i < dim4)
+            out[row + i] = float4{v[j].x * inv_rms * wv[j].x, v[j].y * inv_rms * wv[j].y, v[j].z * inv_rms * wv[j].z,
+                                  v[j].w * inv_rms * wv[j].w};
+    }
 }
 
 // Up to three [seq][heads*hd] sources re-laid head-major, rotated or copied.
@@ -126,40 +171,50 @@ __device__ __forceinline__ bool attn_masked(int mask_kind, int offset, int windo
 
 struct attn_args {
     const float *q, *kc, *vc;
-    float *scores_g, *out;
+    float *part, *out;          // part: [row][split][hd + 2] = (max, exp-sum, unnormalised P.V) when splits > 1
     size_t k_stride, v_stride;  // per kv head
     int len, nqh, group, seq_q, hd, lanes;  // lanes = power of two >= hd/4, <= 64
+    int chunk, splits;                       // keys per split (the LDS score buffer holds one chunk)
     float scale, logit_cap;
     int mask_kind, offset, window, sink, accumulate;
 };
 
-constexpr int ATT_RED = 1024;  // partial output rows: (256 / lanes) slices x (lanes * 4) dims
+constexpr int ATT_RED = 1024;     // partial output rows: (256 / lanes) slices x (lanes * 4) dims
+constexpr int ATT_CHUNK_MAX = 8192;  // keys per workgroup: 32 KB of scores in LDS
 
-// One workgroup per (query token, query head).  Scores: `lanes` lanes share one key, four
-// dims each, so that a key row is one contiguous read; softmax over the scores held in LDS
-// (or in global memory for very long caches); then P.V with the same lane-to-dim mapping,
-// the key range cut into 256/lanes slices whose partial rows are summed in a fixed order.
+// One workgroup per (query token, query head, key split).  Scores: `lanes` lanes share one
+// key, four dims each, so that a key row is one contiguous read; softmax over the split's
+// scores held in LDS; then P.V with the same lane-to-dim mapping, the keys cut into
+// 256/lanes slices whose partial rows are summed in a fixed order.  With one split the
+// result is normalised and written (or added) here; with several, each split leaves its
+// maximum, exp-sum and unnormalised row for gqa_combine_kernel.  Causal masks also cut the
+// key range at the query position, so that a prefill does not visit keys it cannot see.
 __global__ __launch_bounds__(256) void gqa_attention_kernel(attn_args aa) {
     extern __shared__ float lds[];
     __shared__ float red[4];
-    const int tid = threadIdx.x, qt = blockIdx.x, qh = blockIdx.y, kvh = qh / aa.group;
-    const int L = aa.lanes, hd = aa.hd, len = aa.len;
-    float *qs = lds, *part = lds + 256, *sc = aa.scores_g ? aa.scores_g + ((size_t)qh * aa.seq_q + qt) * len : lds + 256 + ATT_RED;
+    const int tid = threadIdx.x, qt = blockIdx.x, qh = blockIdx.y, split = blockIdx.z, kvh = qh / aa.group;
+    const int L = aa.lanes, hd = aa.hd;
+    const int k0 = split * aa.chunk;
+    int k1 = min(aa.len, k0 + aa.chunk);
+    if (aa.mask_kind != 0) k1 = min(k1, aa.offset + qt + 1);
+    const int n = max(k1 - k0, 0);  // keys of this split, uniform over the workgroup
+    float *qs = lds, *part = lds + 256, *sc = lds + 256 + ATT_RED;
     const float *qsrc = aa.q + ((size_t)qh * aa.seq_q + qt) * hd;
     for (int i = tid; i < 4 * L; i += 256) qs[i] = i < hd ? qsrc[i] : 0.f;
     __syncthreads();
     const int sub = tid / L, within = tid % L, nsub = 256 / L, d0 = within * 4;
     const bool vec = (hd & 3) == 0;
-    const float *kbase = aa.kc + (size_t)kvh * aa.k_stride, *vbase = aa.vc + (size_t)kvh * aa.v_stride;
+    const float *kbase = aa.kc + (size_t)kvh * aa.k_stride + (size_t)k0 * hd;
+    const float *vbase = aa.vc + (size_t)kvh * aa.v_stride + (size_t)k0 * hd;
     float q4[4];
     for (int j = 0; j < 4; ++j) q4[j] = qs[d0 + j];
 
     float mx = -INFINITY;
-    const int rounds = (len + nsub - 1) / nsub;
+    const int rounds = (n + nsub - 1) / nsub;
     for (int r = 0; r < rounds; ++r) {  // every lane runs every round: the shuffles need the whole wave
         const int kt = r * nsub + sub;
         float dot = 0.f;
-        const bool live = kt < len && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, qt, kt);
+        const bool live = kt < n && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, qt, k0 + kt);
         if (live && d0 < hd) {
             const float *kr = kbase + (size_t)kt * hd + d0;
             if (vec) {
@@ -171,7 +226,7 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(attn_args aa) {
             }
         }
         for (int m = 1; m < L; m <<= 1) dot += __shfl_xor(dot, m);
-        if (kt < len) {
+        if (kt < n) {
             float s = -INFINITY;
             if (live) {
                 s = dot * aa.scale;
@@ -183,18 +238,19 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(attn_args aa) {
     }
     mx = block_max(mx, red);  // the barriers inside also publish sc[]
     float sum = 0.f;
-    for (int kt = tid; kt < len; kt += 256) {
+    for (int kt = tid; kt < n; kt += 256) {
         const float s = sc[kt];
         const float e = s == -INFINITY ? 0.f : expf(s - mx);
         sc[kt] = e;
         sum += e;
     }
     sum = block_sum(sum, red);
-    const float inv_sum = sum > 0.f ? 1.0f / sum : 0.f;
+    const bool final_pass = aa.splits == 1;
+    const float inv_sum = !final_pass ? 1.0f : (sum > 0.f ? 1.0f / sum : 0.f);
 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     if (d0 < hd) {
-        for (int kt = sub; kt < len; kt += nsub) {
+        for (int kt = sub; kt < n; kt += nsub) {
             const float p = sc[kt] * inv_sum;
             if (p > 0.f) {
                 const float *vr = vbase + (size_t)kt * hd + d0;
@@ -210,11 +266,51 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(attn_args aa) {
     }
     for (int j = 0; j < 4; ++j) part[sub * (4 * L) + d0 + j] = acc[j];
     __syncthreads();
+    const size_t rowi = (size_t)qt * aa.nqh + qh;
+    float *pdst = final_pass ? nullptr : aa.part + (rowi * aa.splits + split) * (size_t)(hd + 2);
+    if (!final_pass && tid == 0) {
+        pdst[0] = mx;
+        pdst[1] = sum;
+    }
     for (int i = tid; i < hd; i += 256) {
         float o = 0.f;
         for (int s = 0; s < nsub; ++s) o += part[s * (4 * L) + i];
-        float *dst = aa.out + ((size_t)qt * aa.nqh + qh) * hd + i;
-        *dst = aa.accumulate ? *dst + o : o;
+        if (final_pass) {
+            float *dst = aa.out + rowi * hd + i;
+            *dst = aa.accumulate ? *dst + o : o;
+        } else {
+            pdst[2 + i] = o;
+        }
+    }
+}
+
+constexpr int ATT_SPLITS_MAX = 2048;
+
+// Merge the splits of one (query token, query head) row: with M = max of the split maxima and
+// w_s = exp(m_s - M), out = sum_s w_s o_s / sum_s w_s l_s, splits in ascending order.
+__global__ __launch_bounds__(128) void gqa_combine_kernel(const float *__restrict__ part, int splits, int hd,
+                                                          float *__restrict__ out, int accumulate) {
+    __shared__ float wts[ATT_SPLITS_MAX];
+    __shared__ float red[2];
+    const float *p = part + (size_t)blockIdx.x * splits * (hd + 2);
+    const int tid = threadIdx.x;
+    float M = -INFINITY;
+    for (int s = tid; s < splits; s += 128) M = fmaxf(M, p[(size_t)s * (hd + 2)]);
+    M = block_max(M, red);
+    float l = 0.f;
+    for (int s = tid; s < splits; s += 128) {
+        const float m = p[(size_t)s * (hd + 2)];
+        const float w = m == -INFINITY ? 0.f : expf(m - M);
+        wts[s] = w;
+        l += w * p[(size_t)s * (hd + 2) + 1];
+    }
+    l = block_sum(l, red);  // its barriers publish wts[]
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    for (int i = tid; i < hd; i += 128) {
+        float o = 0.f;
+        for (int s = 0; s < splits; ++s) o += wts[s] * p[(size_t)s * (hd + 2) + 2 + i];
+        float *dst = out + (size_t)blockIdx.x * hd + i;
+        *dst = accumulate ? *dst + o * inv : o * inv;
     }
 }
 
@@ -237,11 +333,15 @@ inline unsigned blocks_for(size_t n) { return (unsigned)((n + 255) / 256); }
 pg_status launch_rmsnorm(pg_ctx *ctx, const float *a, const float *b, float *sum_out, const float *w, float eps,
                          size_t rows, size_t dim, float *out) {
     if (rows == 0) return PG_OK;
+    const uintptr_t align = (uintptr_t)a | (uintptr_t)b | (uintptr_t)sum_out | (uintptr_t)w | (uintptr_t)out;
+    if (dim % 4 == 0 && dim <= 8192 && align % 16 == 0) {
+        auto *kern = dim <= 4096 ? add_rmsnorm_vec_kernel<4> : add_rmsnorm_vec_kernel<8>;
+        return pg_launch(ctx, "add_rmsnorm", kern, dim3((unsigned)rows), dim3(256), 0, (const float4 *)a, (const float4 *)b,
+                         (float4 *)sum_out, (const float4 *)w, eps, (int)(dim / 4), (float4 *)out);
+    }
     return pg_launch(ctx, "add_rmsnorm", add_rmsnorm_kernel, dim3((unsigned)rows), dim3(256), 0, a, b, sum_out, w, eps,
                      (int)dim, out);
 }
-
-constexpr size_t ATT_LDS_KEYS = 36864;  // scores kept in LDS up to this cache length (147 KB + fixed part)
 
 pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, const pg_kv_cache *vc, size_t nqh,
                            size_t seq_q, float scale, int mask_kind, size_t offset, size_t window, size_t sink,
@@ -253,7 +353,7 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
         return PG_OK;
     }
     attn_args aa;
-    aa.q = q; aa.kc = kc->k; aa.vc = vc->v; aa.out = out; aa.scores_g = nullptr;
+    aa.q = q; aa.kc = kc->k; aa.vc = vc->v; aa.out = out; aa.part = nullptr;
     aa.k_stride = kc->capacity * hd; aa.v_stride = vc->capacity * hd;
     aa.len = (int)len; aa.nqh = (int)nqh; aa.group = (int)(nqh / kc->num_kv_heads); aa.seq_q = (int)seq_q; aa.hd = (int)hd;
     int lanes = 1;
@@ -264,22 +364,31 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     aa.window = (int)(window > 0x7fffffffu ? 0x7fffffffu : window);
     aa.sink = (int)(sink > 0x7fffffffu ? 0x7fffffffu : sink);
     aa.accumulate = accumulate;
-    size_t lds = (256 + ATT_RED) * sizeof(float);
-    if (len <= ATT_LDS_KEYS) {
-        lds += len * sizeof(float);
-    } else {
+    // Split the keys when the rows alone cannot fill the chip (decode) or a chunk would not
+    // fit the LDS score buffer; at least 4 rounds of keys per split.
+    const size_t rows = seq_q * nqh, keys_per_round = 256 / (size_t)lanes;
+    size_t splits = rows >= 2 * (size_t)ctx->num_cu ? 1 : (2 * (size_t)ctx->num_cu + rows - 1) / rows;
+    const size_t max_splits = (len + 4 * keys_per_round - 1) / (4 * keys_per_round);
+    if (splits > max_splits) splits = max_splits;
+    const size_t min_splits = (len + ATT_CHUNK_MAX - 1) / ATT_CHUNK_MAX;
+    if (splits < min_splits) splits = min_splits;
+    size_t chunk = (len + splits - 1) / splits;
+    chunk = pg_round_up(chunk, keys_per_round);
+    splits = (len + chunk - 1) / chunk;
+    if (splits > (size_t)ATT_SPLITS_MAX) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: cache of %zu positions is too long", len);
+    aa.chunk = (int)chunk; aa.splits = (int)splits;
+    if (splits > 1) {
         void *ws = nullptr;
-        PG_TRY(pg_workspace(ctx, nqh * seq_q * len * sizeof(float), &ws));
-        aa.scores_g = static_cast<float *>(ws);
+        PG_TRY(pg_workspace(ctx, rows * splits * (hd + 2) * sizeof(float), &ws));
+        aa.part = static_cast<float *>(ws);
     }
-    static bool attr_done = false;
-    if (!attr_done) {
-        PG_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gqa_attention_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)((256 + ATT_RED + ATT_LDS_KEYS) * sizeof(float))));
-        attr_done = true;
-    }
-    return pg_launch(ctx, "gqa_attention", gqa_attention_kernel, dim3((unsigned)seq_q, (unsigned)nqh), dim3(256), lds, aa);
+    const size_t lds = (256 + ATT_RED + chunk) * sizeof(float);
+    PG_TRY(pg_launch(ctx, "gqa_attention", gqa_attention_kernel, dim3((unsigned)seq_q, (unsigned)nqh, (unsigned)splits),
+                     dim3(256), lds, aa));
+    if (splits > 1)
+        PG_TRY(pg_launch(ctx, "gqa_combine", gqa_combine_kernel, dim3((unsigned)rows), dim3(128), 0, (const float *)aa.part,
+                         (int)splits, (int)hd, out, accumulate));
+    return PG_OK;
 }
 
 pg_status check_attention_args(const char *fn, const pg_kv_cache *kc, const pg_kv_cache *vc, size_t nqh, size_t seq_q,
@@ -663,9 +772,8 @@ PG_API pg_status pg_llama_block_forward_dev(pg_ctx *ctx, pg_llama_block *b, cons
     float *g = take(cap * ffn), *u = take(cap * ffn);
 
     PG_TRY(launch_rmsnorm(ctx, h_dev, nullptr, nullptr, b->attn_norm_w, b->eps, seq, d, normed));
-    PG_TRY(pg_gguf_matmul_rows(ctx, normed, seq, b->w[0], qd));
-    PG_TRY(pg_gguf_matmul_rows(ctx, normed, seq, b->w[1], kd));
-    PG_TRY(pg_gguf_matmul_rows(ctx, normed, seq, b->w[2], vd));
+    float *const qkv[3] = {qd, kd, vd};
+    PG_TRY(pg_gguf_matmul_rows_multi(ctx, normed, seq, b->w, qkv, 3));
     PG_TRY(cache_reserve(ctx, cache, offset + seq));
     rope_args ra = {};
     ra.seg[0] = {qd, q_rope, q_dim, seq * hd, (int)b->nqh, 1};
@@ -678,8 +786,8 @@ PG_API pg_status pg_llama_block_forward_dev(pg_ctx *ctx, pg_llama_block *b, cons
                             0.0f, attn, 0));
     PG_TRY(pg_gguf_matmul_rows(ctx, attn, seq, b->w[3], proj));
     PG_TRY(launch_rmsnorm(ctx, h_dev, proj, h1, b->ffn_norm_w, b->eps, seq, d, normed));
-    PG_TRY(pg_gguf_matmul_rows(ctx, normed, seq, b->w[4], g));
-    PG_TRY(pg_gguf_matmul_rows(ctx, normed, seq, b->w[5], u));
+    float *const gu[2] = {g, u};
+    PG_TRY(pg_gguf_matmul_rows_multi(ctx, normed, seq, b->w + 4, gu, 2));
     PG_TRY(pg_launch(ctx, "swiglu", swiglu_kernel, dim3(blocks_for(seq * ffn)), dim3(256), 0, g, (const float *)u, seq * ffn));
     PG_TRY(pg_gguf_matmul_rows(ctx, g, seq, b->w[6], proj));
     return pg_launch(ctx, "residual_add", add_kernel, dim3(blocks_for(seq * d)), dim3(256), 0, (const float *)h1,

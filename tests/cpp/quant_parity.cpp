@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <vector>
 
 #include "peregrine_hip.hpp"
@@ -17,6 +18,13 @@ void orc_quantize_weights(const float *, size_t, size_t, int8_t *, int8_t *, flo
 void orc_quantize_activations(const float *, size_t, size_t, int8_t *, float *);
 int orc_matmul_quantized(const float *, size_t, size_t, const int8_t *, const float *, size_t, float *, int32_t *);
 int orc_gguf_matmul(const float *, size_t, const uint8_t *, int, size_t, size_t, float *);
+void orc_rope_tables(size_t, size_t, float, float *, float *);
+void orc_gqa_attention(const float *, const float *, const float *, size_t, size_t, size_t, size_t, size_t, size_t, float,
+                       int, size_t, size_t, size_t, float, float *);
+int orc_llama_block_forward(const float *, size_t, size_t, size_t, size_t, size_t, size_t, int, const uint8_t *,
+                            const uint8_t *, const uint8_t *, const uint8_t *, const uint8_t *, const uint8_t *,
+                            const uint8_t *, const float *, const float *, float, const float *, const float *, float *,
+                            float *, size_t, size_t, float *);
 }
 
 using namespace peregrine;
@@ -186,6 +194,79 @@ static void test_block_weight_matmul(const GpuContext &gpu) {
     }
 }
 
+// tests/attention.rs:59-133 (MHA against the naive per-head form) with the reference's sin/cos
+// inputs, then the same through a cache whose capacity exceeds its length
+static void test_gqa_attention(const GpuContext &gpu) {
+    std::printf("test_gqa_attention\n");
+    const size_t nqh = 4, nkvh = 2, seq_q = 2, seq_kv = 3, hd = 4;
+    std::vector<float> q(nqh * seq_q * hd), k(nkvh * seq_kv * hd), v(nkvh * seq_kv * hd);
+    for (size_t i = 0; i < q.size(); ++i) q[i] = std::sin((float)i * 0.1f);
+    for (size_t i = 0; i < k.size(); ++i) { k[i] = std::cos((float)i * 0.2f); v[i] = std::sin((float)i * 0.15f); }
+    llama::StandardKVCache cache(gpu, nkvh, hd);
+    cache.append(k, v, seq_kv);
+    EXPECT(cache.len() == seq_kv && cache.head_stride() == 32 * hd, "len %zu stride %zu", cache.len(), cache.head_stride());
+    const float scale = 1.0f / std::sqrt((float)hd);
+    for (const auto &mask : {llama::AttentionMask::None(), llama::AttentionMask::Causal(1)}) {
+        std::vector<float> out(seq_q * nqh * hd, 0.0f), ref(out.size(), 0.0f);
+        llama::gqa_attention(gpu, q, cache, cache, nqh, nkvh, seq_q, hd, scale, mask, 0.0f, out);
+        orc_gqa_attention(q.data(), k.data(), v.data(), seq_kv, seq_kv, nqh, nkvh, seq_q, hd, scale, mask.kind, mask.offset, 0, 0,
+                          0.0f, ref.data());
+        for (size_t i = 0; i < ref.size(); ++i)
+            EXPECT(std::fabs(out[i] - ref[i]) <= 1e-5f, "mask %d [%zu]: %g vs %g", mask.kind, i, out[i], ref[i]);
+    }
+    bool threw = false;
+    try { cache.rollback_to(4); } catch (const Panic &) { threw = true; }
+    EXPECT(threw, "rollback_to beyond len must panic (src/attention.rs:88)");
+}
+
+// LlamaBlock::forward: a prefill of 3 then a decode step against the CPU composition
+static void test_llama_block(const GpuContext &gpu) {
+    std::printf("test_llama_block\n");
+    const size_t d = 128, nqh = 4, nkvh = 2, hd = 32, ffn = 256, cap = 16;
+    const size_t shp[7][2] = {{nqh * hd, d}, {nkvh * hd, d}, {nkvh * hd, d}, {d, nqh * hd}, {ffn, d}, {ffn, d}, {d, ffn}};
+    uint32_t s = 7;
+    auto next = [&]() { s = s * 1103515245u + 12345u; return s; };
+    std::vector<std::vector<uint8_t>> raw(7);
+    std::vector<std::unique_ptr<gguf::BlockWeight>> w;
+    for (int i = 0; i < 7; ++i) {
+        const size_t nb = shp[i][0] * shp[i][1] / 32;
+        raw[i].resize(nb * 34);
+        for (size_t b = 0; b < nb; ++b) {
+            const uint16_t dd = (uint16_t)(0x1400 + (b * 37) % 0x0400);  // halves near 1e-3: products stay O(1)
+            raw[i][b * 34] = (uint8_t)(dd & 0xFF); raw[i][b * 34 + 1] = (uint8_t)(dd >> 8);
+            for (size_t j = 2; j < 34; ++j) raw[i][b * 34 + j] = (uint8_t)(next() >> 16);
+        }
+        w.emplace_back(new gguf::BlockWeight(gpu, raw[i], PG_GGML_Q8_0, shp[i][0], shp[i][1]));
+    }
+    std::vector<float> wa(d), wf(d);
+    for (size_t i = 0; i < d; ++i) { wa[i] = 1.0f + 0.01f * (float)(i % 7); wf[i] = 1.0f - 0.01f * (float)(i % 5); }
+    llama::LlamaBlock blk(gpu, d, nqh, nkvh, hd, ffn, cap, 10000.0f, 1e-5f);
+    blk.set_weights(*w[0], *w[1], *w[2], *w[3], *w[4], *w[5], *w[6], wa, wf);
+    llama::KVCache cache(gpu, nkvh, hd);
+    std::vector<float> cos_t(cap * hd), sin_t(cap * hd), kc(nkvh * cap * hd, 0.0f), vc(nkvh * cap * hd, 0.0f);
+    orc_rope_tables(hd, cap, 10000.0f, cos_t.data(), sin_t.data());
+    size_t pos = 0;
+    for (size_t seq : {(size_t)3, (size_t)1}) {
+        std::vector<float> h(seq * d), ref(seq * d);
+        for (auto &x : h) x = (float)next() / 4294967295.0f * 2.0f - 1.0f;
+        auto out = blk.forward(h, seq, cache);
+        const int rc = orc_llama_block_forward(h.data(), seq, d, nqh, nkvh, hd, ffn, PG_GGML_Q8_0, raw[0].data(), raw[1].data(),
+                                               raw[2].data(), raw[3].data(), raw[4].data(), raw[5].data(), raw[6].data(),
+                                               wa.data(), wf.data(), 1e-5f, cos_t.data(), sin_t.data(), kc.data(), vc.data(),
+                                               pos, cap, ref.data());
+        EXPECT(rc == 0, "oracle rc %d", rc);
+        pos += seq;
+        EXPECT(cache.len() == pos, "cache len %zu", cache.len());
+        double rms = 0;
+        for (float x : ref) rms += (double)x * x;
+        rms = std::sqrt(rms / ref.size());
+        for (size_t i = 0; i < ref.size(); ++i) {
+            const double tol = 1e-3 * std::fmax(std::fabs((double)ref[i]), rms);
+            EXPECT(std::fabs((double)out[i] - ref[i]) <= tol, "seq %zu [%zu]: %g vs %g", seq, i, out[i], ref[i]);
+        }
+    }
+}
+
 int main() {
     try {
         GpuContext gpu(0);
@@ -197,6 +278,8 @@ int main() {
         test_shape_panics(gpu);
         test_gguf_known_answers(gpu);
         test_block_weight_matmul(gpu);
+        test_gqa_attention(gpu);
+        test_llama_block(gpu);
     } catch (const std::exception &e) {
         std::printf("FAIL: uncaught %s\n", e.what());
         return 2;

@@ -154,8 +154,8 @@ def test_gqa_attention_masks_and_logit_cap(ctx, orc):
     assert (out[:8] == v[0, 0]).all()
 
 
-def test_gqa_attention_long_cache_uses_global_scores(ctx, orc):
-    """Beyond 36864 positions the scores live in global memory instead of LDS."""
+def test_gqa_attention_long_cache_splits_keys(ctx, orc):
+    """A long cache under one query row: the keys are cut into many splits and merged."""
     from peregrine_amd import llama
     say("attention len=40000")
     _attention_case(ctx, orc, 2, 1, 16, 1, 40000, llama.AttentionMask.causal(39999), None, 55)
