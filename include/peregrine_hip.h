@@ -41,6 +41,9 @@ enum {
 
 /* GGML block types, numbered as src/gguf.rs:14-33 does. */
 enum { PG_GGML_Q4_0 = 2, PG_GGML_Q4_1 = 3, PG_GGML_Q8_0 = 8 };
+/* Type tag reported by pg_gguf_shape for a tensor made by pg_mxfp4_upload (ggml's own number
+ * for MXFP4; the reference's GGUF enum stops before it). */
+enum { PG_MXFP4 = 39 };
 
 /* Expert activation of the grouped MoE FFN. */
 enum {
@@ -173,6 +176,35 @@ pg_status pg_gguf_matmul(pg_ctx *ctx, const float *x, size_t m, const pg_gguf_te
                          float *y);
 pg_status pg_gguf_matmul_dev(pg_ctx *ctx, const float *x_dev, size_t m,
                              const pg_gguf_tensor *w, float *y_dev);
+
+/* ---- MXFP4 (the gpt_oss experts' format) ------------------------------------------ */
+
+/* mxfp4_matmul  examples/gpt_oss/moe.rs:16-53: weight [out_dim, in_dim] as 16-byte blocks of
+ * FP4 codes (byte k = elements 2k low nibble, 2k+1 high) in `blocks` [out_dim * in_dim/32 * 16]
+ * and one E8M0 scale byte per block in `scales` [out_dim * in_dim/32];
+ * output[r] = sum_b ( sum_k LUT[code] * input[32b + k] ) * 2^(scale - 127). */
+pg_status pg_mxfp4_matmul(pg_ctx *ctx, const float *input, const uint8_t *blocks, const uint8_t *scales,
+                          size_t out_dim, size_t in_dim, float *output);
+/* The same weight kept on the device: a pg_gguf_tensor (type PG_MXFP4) for pg_gguf_matmul(_dev),
+ * each row of x being one mxfp4_matmul. */
+pg_status pg_mxfp4_upload(pg_ctx *ctx, const uint8_t *blocks, const uint8_t *scales, size_t out_dim,
+                          size_t in_dim, pg_gguf_tensor **out);
+
+/* Mxfp4Expert  examples/gpt_oss/moe.rs:55-117: mlp1 [2*intermediate, hidden] + bias, the
+ * gpt-oss SwiGLU over interleaved (gate, linear) pairs (examples/gpt_oss/moe.rs:145-154),
+ * mlp2 [hidden, intermediate] + bias. */
+typedef struct pg_mxfp4_expert pg_mxfp4_expert;
+pg_status pg_mxfp4_expert_create(pg_ctx *ctx, size_t hidden, size_t intermediate, float alpha, float clamp,
+                                 const uint8_t *mlp1_blocks, const uint8_t *mlp1_scales,
+                                 const uint8_t *mlp2_blocks, const uint8_t *mlp2_scales,
+                                 const float *mlp1_bias, const float *mlp2_bias, pg_mxfp4_expert **out);
+void pg_mxfp4_expert_free(pg_ctx *ctx, pg_mxfp4_expert *expert);
+/* Mxfp4Expert::forward  examples/gpt_oss/moe.rs:84-115 on m rows: x, out [m, hidden]. */
+pg_status pg_mxfp4_expert_forward(pg_ctx *ctx, const pg_mxfp4_expert *expert, const float *x, size_t m,
+                                  float *out);
+/* scratch_dev: m * 3 * intermediate floats, 16-byte aligned. */
+pg_status pg_mxfp4_expert_forward_dev(pg_ctx *ctx, const pg_mxfp4_expert *expert, const float *x_dev, size_t m,
+                                      float *scratch_dev, float *out_dev);
 
 /* ---- GGUF container (gguf::GgufFile, src/gguf.rs:403-561) ---------------------
  * Parsing needs no device.  A malformed or truncated file is PG_EINVAL (the reference

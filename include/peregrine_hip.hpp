@@ -457,5 +457,51 @@ private:
 };
 
 }  // namespace llama
+
+namespace mxfp4 {
+
+// mxfp4_matmul  examples/gpt_oss/moe.rs:16-53.
+inline std::vector<float> mxfp4_matmul(const GpuContext &gpu, const std::vector<float> &input, const std::vector<uint8_t> &blocks,
+                                       const std::vector<uint8_t> &scales, size_t out_dim, size_t in_dim) {
+    if (in_dim % 32 || input.size() != in_dim || blocks.size() != out_dim * in_dim / 2 || scales.size() != out_dim * in_dim / 32)
+        throw Panic(PG_EINVAL, "mxfp4_matmul: slice lengths do not match [out_dim, in_dim]");
+    std::vector<float> out(out_dim);
+    check(pg_mxfp4_matmul(gpu.raw(), input.data(), blocks.data(), scales.data(), out_dim, in_dim, out.data()), "mxfp4_matmul");
+    return out;
+}
+
+// Mxfp4Expert  examples/gpt_oss/moe.rs:55-117.
+class Mxfp4Expert {
+public:
+    Mxfp4Expert(const GpuContext &gpu, size_t hidden, size_t intermediate, float alpha, float clamp,
+                const std::vector<uint8_t> &mlp1_blocks, const std::vector<uint8_t> &mlp1_scales,
+                const std::vector<uint8_t> &mlp2_blocks, const std::vector<uint8_t> &mlp2_scales,
+                const std::vector<float> &mlp1_bias, const std::vector<float> &mlp2_bias)
+        : gpu_(&gpu), hidden_(hidden) {
+        if (hidden % 32 || intermediate % 32 || mlp1_blocks.size() != intermediate * hidden || mlp1_scales.size() != intermediate * hidden / 16 ||
+            mlp2_blocks.size() != hidden * intermediate / 2 || mlp2_scales.size() != hidden * intermediate / 32 ||
+            mlp1_bias.size() != 2 * intermediate || mlp2_bias.size() != hidden)
+            throw Panic(PG_EINVAL, "Mxfp4Expert: slice lengths do not match (hidden, intermediate)");
+        check(pg_mxfp4_expert_create(gpu.raw(), hidden, intermediate, alpha, clamp, mlp1_blocks.data(), mlp1_scales.data(),
+                                     mlp2_blocks.data(), mlp2_scales.data(), mlp1_bias.data(), mlp2_bias.data(), &h_),
+              "Mxfp4Expert::new");
+    }
+    ~Mxfp4Expert() { pg_mxfp4_expert_free(gpu_->raw(), h_); }
+    Mxfp4Expert(const Mxfp4Expert &) = delete;
+    Mxfp4Expert &operator=(const Mxfp4Expert &) = delete;
+    std::vector<float> forward(const std::vector<float> &x) const {
+        if (x.size() != hidden_) throw Panic(PG_EINVAL, "Mxfp4Expert::forward: x.len() != hidden");
+        std::vector<float> out(hidden_);
+        check(pg_mxfp4_expert_forward(gpu_->raw(), h_, x.data(), 1, out.data()), "Mxfp4Expert::forward");
+        return out;
+    }
+
+private:
+    const GpuContext *gpu_;
+    pg_mxfp4_expert *h_ = nullptr;
+    size_t hidden_;
+};
+
+}  // namespace mxfp4
 }  // namespace peregrine
 #endif  // PEREGRINE_HIP_HPP

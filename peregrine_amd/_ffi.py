@@ -15,6 +15,7 @@ lib = C.CDLL(LIB_PATH)
 
 PG_OK, PG_EINVAL, PG_EDEVICE, PG_ENOMEM, PG_EUNSUPPORTED = 0, 1, 2, 3, 4
 GGML_Q4_0, GGML_Q4_1, GGML_Q8_0 = 2, 3, 8
+MXFP4 = 39
 ACT_SILU, ACT_GELU_TANH = 0, 1
 MASK_NONE, MASK_CAUSAL, MASK_CAUSAL_SLIDING_WINDOW = 0, 1, 2
 
@@ -80,6 +81,12 @@ SIGNATURES = {
     "pg_qtensor_from_record": [_vp, _vp, _sz, _pp, C.POINTER(_sz)],
     "pg_moe_ffn": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
     "pg_moe_ffn_dev": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
+    "pg_mxfp4_matmul": [_vp, _vp, _vp, _vp, _sz, _sz, _vp],
+    "pg_mxfp4_upload": [_vp, _vp, _vp, _sz, _sz, _pp],
+    "pg_mxfp4_expert_create": [_vp, _sz, _sz, C.c_float, C.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _pp],
+    "pg_mxfp4_expert_free": [_vp, _vp],
+    "pg_mxfp4_expert_forward": [_vp, _vp, _vp, _sz, _vp],
+    "pg_mxfp4_expert_forward_dev": [_vp, _vp, _vp, _sz, _vp, _vp],
     "pg_rmsnorm": [_vp, _vp, _sz, _sz, _vp, C.c_float, _vp],
     "pg_rmsnorm_dev": [_vp, _vp, _sz, _sz, _vp, C.c_float, _vp],
     "pg_rope_create": [_vp, _sz, _sz, C.c_float, _pp],
@@ -108,6 +115,7 @@ _OTHER_RESTYPE = {
     "pg_gguf_free": None,
     "pg_gguf_file_close": None,
     "pg_rope_free": None,
+    "pg_mxfp4_expert_free": None,
     "pg_kv_cache_free": None,
     "pg_llama_block_free": None,
     "pg_kv_cache_len": _sz,

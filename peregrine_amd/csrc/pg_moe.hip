@@ -104,6 +104,7 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     PG_CHECK_ARG(gate && up && down && gate[0] && up[0] && down[0], "pg_moe_ffn: null expert table");
     const size_t d = gate[0]->k_in, ffn = gate[0]->n_out;
     const int type = gate[0]->ggml_type;
+    PG_CHECK_ARG(type == PG_GGML_Q4_0 || type == PG_GGML_Q8_0, "pg_moe_ffn: experts must be Q4_0 or Q8_0 block tensors");
     for (size_t e = 0; e < E; ++e) {
         PG_CHECK_ARG(gate[e] && up[e] && down[e], "pg_moe_ffn: expert %zu has a null tensor", e);
         PG_CHECK_ARG(gate[e]->k_in == d && gate[e]->n_out == ffn && up[e]->k_in == d &&

@@ -29,8 +29,11 @@ class RMSNorm:
         if x.size % self.dim or (x.ndim and x.shape[-1] != self.dim):
             raise ValueError(f"RMSNorm.forward: last dimension is not {self.dim}")
         out = np.empty(x.size, np.float32)
+        w = _f32(self.weight)
+        if w.size != self.dim:
+            raise ValueError(f"RMSNorm.forward: weight is not [{self.dim}]")
         _ffi.check(_ffi.lib.pg_rmsnorm(self.ctx.handle, _ptr(x.reshape(-1)), x.size // self.dim, self.dim,
-                                       _ptr(_f32(self.weight)), self.eps, _ptr(out)))
+                                       _ptr(w), self.eps, _ptr(out)))
         return out.reshape(x.shape)
 
 
@@ -170,8 +173,10 @@ class LlamaBlock:
 
     def set_weights(self, q_proj, k_proj, v_proj, o_proj, gate_proj, up_proj, down_proj, attn_norm_w, ffn_norm_w):
         ws = (q_proj, k_proj, v_proj, o_proj, gate_proj, up_proj, down_proj)
-        _ffi.check(_ffi.lib.pg_llama_block_set_weights(self.ctx.handle, self._h, *[w._h for w in ws],
-                                                       _ptr(_f32(attn_norm_w)), _ptr(_f32(ffn_norm_w))))
+        wa, wf = _f32(attn_norm_w), _f32(ffn_norm_w)
+        if wa.size != self.model_dim or wf.size != self.model_dim:
+            raise ValueError("LlamaBlock.set_weights: norm weights are not [model_dim]")
+        _ffi.check(_ffi.lib.pg_llama_block_set_weights(self.ctx.handle, self._h, *[w._h for w in ws], _ptr(wa), _ptr(wf)))
         self._weights = ws  # the block borrows the handles: keep them alive
 
     def new_cache(self):

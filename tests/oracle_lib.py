@@ -29,8 +29,16 @@ for _n in ("orc_quantize_weights", "orc_quantize_activations", "orc_dequantize",
     getattr(lib, _n).restype = None
 
 
+class _KeptPtr(C.c_void_p):
+    """A void pointer that keeps the array it points into alive for as long as it lives."""
+
+
 def _p(a):
-    return C.c_void_p(a.ctypes.data) if a is not None else C.c_void_p(None)
+    if a is None:
+        return C.c_void_p(None)
+    p = _KeptPtr(a.ctypes.data)
+    p._keep = a
+    return p
 
 
 def _f32(a):
@@ -205,3 +213,28 @@ def llama_block_forward(h, seq, d, nqh, nkvh, hd, ffn, ggml_type, weights, attn_
                                      _sz(cache_len), _sz(capacity), _p(out))
     assert rc == 0, rc
     return out.reshape(seq, d)
+
+
+# ---- sibling formats (oracle/peregrine_oracle_formats.c) ----
+lib.orc_mxfp4_matmul.restype = None
+
+
+def _u8(b):
+    return np.frombuffer(bytes(b), np.uint8).copy() if not isinstance(b, np.ndarray) else np.ascontiguousarray(b, np.uint8).reshape(-1)
+
+
+def mxfp4_matmul(x, blocks, scales, out_dim, in_dim):
+    blocks, scales = _u8(blocks), _u8(scales)
+    assert blocks.size == out_dim * in_dim // 2 and scales.size == out_dim * in_dim // 32
+    out = np.empty(out_dim, np.float32)
+    lib.orc_mxfp4_matmul(_p(_f32(x).reshape(-1)), _p(blocks), _p(scales), _sz(out_dim), _sz(in_dim), _p(out))
+    return out
+
+
+def mxfp4_expert_forward(x, hidden, intermediate, alpha, clamp, b1, s1, b2, s2, bias1, bias2):
+    out = np.empty(hidden, np.float32)
+    rc = lib.orc_mxfp4_expert_forward(_p(_f32(x).reshape(-1)), _sz(hidden), _sz(intermediate), C.c_float(alpha),
+                                      C.c_float(clamp), _p(_u8(b1)), _p(_u8(s1)), _p(_u8(b2)), _p(_u8(s2)),
+                                      _p(_f32(bias1)), _p(_f32(bias2)), _p(out))
+    assert rc == 0
+    return out

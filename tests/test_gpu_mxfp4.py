@@ -1,0 +1,97 @@
+"""GPU parity of the MXFP4 path (examples/gpt_oss/moe.rs) against the CPU oracle, through the
+C ABI.  Bar: the block-dequant contract, 1e-3 relative (H.assert_close_rel); the fixed-point
+kernel is exact up to the final f32 roundings, so the tests also hold it to 2e-5."""
+import sys
+
+import numpy as np
+import pytest
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+RTOL_CONTRACT, RTOL_ACHIEVED = 1e-3, 2e-5
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def _weights(rng, n, k, lo=118, hi=124):
+    return (rng.integers(0, 256, n * k // 2, dtype=np.uint8), rng.integers(lo, hi, n * k // 32, dtype=np.uint8))
+
+
+def test_mxfp4_codes_scales_and_order_exact(ctx, orc):
+    """One-hot inputs read single weights back: every code, both nibbles, a spread of scale bytes."""
+    from peregrine_amd import mxfp4
+    in_dim, out_dim = 64, 16
+    blocks = np.zeros((out_dim, 2, 16), np.uint8)
+    for r in range(out_dim):
+        blocks[r, 0, 0] = r                    # code r in the low nibble of element 0
+        blocks[r, 1, 5] = r << 4               # code r in the high nibble of element 32 + 11
+    scales = np.full((out_dim, 2), 127, np.uint8)
+    for pos in (0, 1, 43, 42):
+        x = np.zeros(in_dim, np.float32)
+        x[pos] = 3.0
+        got = mxfp4.mxfp4_matmul(x, blocks, scales, out_dim, in_dim, ctx)
+        assert (got == orc.mxfp4_matmul(x, blocks, scales, out_dim, in_dim)).all(), pos
+    x = np.zeros(in_dim, np.float32)
+    x[0] = 1.0
+    one = np.zeros((1, 2, 16), np.uint8)
+    one[0, 0, 0] = 2
+    for e in (0, 1, 2, 60, 126, 127, 128, 200, 253, 254):
+        s = np.array([[e, 127]], np.uint8)
+        got = mxfp4.mxfp4_matmul(x, one, s, 1, in_dim, ctx)[0]
+        want = orc.mxfp4_matmul(x, one, s, 1, in_dim)[0]
+        assert got == want, (e, got, want)
+
+
+@pytest.mark.parametrize("out_dim,in_dim", [(5760, 2880), (2880, 2880), (33, 96), (1, 32), (257, 8192 + 32)])
+def test_mxfp4_matmul(ctx, orc, out_dim, in_dim):
+    """gpt-oss shapes (hidden 2880, mlp1 rows 2 x 2880) and ragged ones."""
+    from peregrine_amd import mxfp4
+    say(f"mxfp4 matmul [{in_dim}] -> [{out_dim}]")
+    rng = np.random.default_rng(out_dim + in_dim)
+    b, s = _weights(rng, out_dim, in_dim)
+    x = orc.rng_normal(out_dim, in_dim)
+    x[::97] *= 20.0
+    got = mxfp4.mxfp4_matmul(x, b, s, out_dim, in_dim, ctx)
+    want = orc.mxfp4_matmul(x, b, s, out_dim, in_dim)
+    H.assert_close_rel(got, want, RTOL_CONTRACT, "mxfp4 contract")
+    H.assert_close_rel(got, want, RTOL_ACHIEVED, "mxfp4 achieved")
+
+
+def test_mxfp4_resident_weight_rows_and_errors(ctx, orc):
+    from peregrine_amd import mxfp4, _ffi
+    rng = np.random.default_rng(5)
+    out_dim, in_dim, m = 200, 256, 7
+    b, s = _weights(rng, out_dim, in_dim, 100, 150)
+    w = mxfp4.upload(b, s, out_dim, in_dim, ctx)
+    assert (w.n_out, w.k_in, w.ggml_type) == (out_dim, in_dim, _ffi.MXFP4)
+    x = orc.rng_normal(3, m * in_dim).reshape(m, in_dim)
+    got = w.matmul(x, m).reshape(m, out_dim)
+    for i in range(m):
+        H.assert_close_rel(got[i], orc.mxfp4_matmul(x[i], b, s, out_dim, in_dim), RTOL_ACHIEVED, f"row {i}")
+    with pytest.raises(ValueError):
+        mxfp4.mxfp4_matmul(x[0], b, s, out_dim, in_dim + 1, ctx)
+    with pytest.raises(ValueError):
+        mxfp4.mxfp4_matmul(x[0], b[:-1], s, out_dim, in_dim, ctx)
+
+
+@pytest.mark.parametrize("m", [1, 3])
+def test_mxfp4_expert_forward(ctx, orc, m):
+    from peregrine_amd import mxfp4
+    hidden, inter, alpha, clamp = 2880, 2880, 1.702, 7.0
+    say(f"mxfp4 expert hidden={hidden} intermediate={inter} m={m}")
+    rng = np.random.default_rng(21)
+    b1, s1 = _weights(rng, 2 * inter, hidden, 116, 120)
+    b2, s2 = _weights(rng, hidden, inter, 116, 120)
+    bias1 = orc.rng_normal(1, 2 * inter)
+    bias2 = orc.rng_normal(2, hidden)
+    ex = mxfp4.Mxfp4Expert(hidden, inter, alpha, clamp, b1, s1, b2, s2, bias1, bias2, ctx)
+    x = orc.rng_normal(4, m * hidden).reshape(m, hidden)
+    got = ex.forward(x if m > 1 else x[0]).reshape(m, hidden)
+    for i in range(m):
+        want = orc.mxfp4_expert_forward(x[i], hidden, inter, alpha, clamp, b1, s1, b2, s2, bias1, bias2)
+        H.assert_close_rel(got[i], want, RTOL_CONTRACT, f"mxfp4 expert row {i}")
+        H.assert_close_rel(got[i], want, 1e-4, f"mxfp4 expert row {i} (achieved)")
