@@ -262,6 +262,49 @@ pg_status pg_read_quantized_tensor(const void *buf, size_t len, const char **nam
 pg_status pg_qtensor_from_record(pg_ctx *ctx, const void *buf, size_t len, pg_qtensor **out,
                                  size_t *consumed);
 
+/* ---- Huffman-coded int8 weights (src/huffman.rs) ------------------------------------
+ * Symbols are i8 values, index = value + 128.  The table builder, the encoder and the
+ * HuffmanTensor container are host code (no device needed); decoding runs on the device. */
+typedef struct pg_huffman_tensor pg_huffman_tensor;
+/* HuffmanTable::from_frequencies  src/huffman.rs:35-150: freqs[256] -> bit_lengths[256]
+ * (0 = unused, at most 12) and, if codes is not NULL, the canonical codes[256]. */
+pg_status pg_huffman_table_from_frequencies(const uint64_t *freqs, uint8_t *bit_lengths, uint32_t *codes);
+/* HuffmanTable::canonical_codes  src/huffman.rs:152-186 (what from_bytes, :292-306, rebuilds). */
+pg_status pg_huffman_canonical_codes(const uint8_t *bit_lengths, uint32_t *codes);
+/* HuffmanTable::encode  src/huffman.rs:216-251: MSB first, last byte zero-padded.  *bytes is
+ * the size needed; out may be NULL to ask for it.  A symbol without a code is PG_EINVAL. */
+pg_status pg_huffman_encode(const uint8_t *bit_lengths, const int8_t *data, size_t n, uint8_t *out, size_t cap,
+                            size_t *bytes);
+/* HuffmanTable::decode  src/huffman.rs:254-284 on the device (host pointers in and out).  A
+ * stream that ends before num_symbols codes, or an unassigned code (the reference's
+ * debug_assert), is PG_EINVAL. */
+pg_status pg_huffman_decode(pg_ctx *ctx, const uint8_t *bit_lengths, const uint8_t *bitstream, size_t len,
+                            size_t num_symbols, int8_t *out);
+/* HuffmanTensor::from_quantized  src/huffman.rs:332-372: q [rows, cols] row-major, scales [cols]. */
+pg_status pg_huffman_tensor_from_quantized(const int8_t *q, const float *scales, size_t rows, size_t cols,
+                                           size_t num_streams, pg_huffman_tensor **out);
+/* The struct literal of serial::read_huffman_tensor  src/serial.rs:367-445: a tensor from
+ * its stored parts (everything is copied). */
+pg_status pg_huffman_tensor_from_parts(const uint8_t *bit_lengths, const uint8_t *const *streams,
+                                       const size_t *stream_bytes, const size_t *stream_lengths, size_t num_streams,
+                                       const float *scales, size_t rows, size_t cols, pg_huffman_tensor **out);
+void pg_huffman_tensor_free(pg_huffman_tensor *t);
+/* rows, cols, num_streams fields and compressed_size()  src/huffman.rs:407-412. */
+pg_status pg_huffman_tensor_info(const pg_huffman_tensor *t, size_t *rows, size_t *cols, size_t *num_streams,
+                                 size_t *compressed_size);
+/* streams[index], its byte length and stream_lengths[index]. */
+pg_status pg_huffman_tensor_stream(const pg_huffman_tensor *t, size_t index, const uint8_t **data, size_t *bytes,
+                                   size_t *symbols);
+/* table.bit_lengths [256] and scales [cols]. */
+pg_status pg_huffman_tensor_table(const pg_huffman_tensor *t, const uint8_t **bit_lengths, const float **scales);
+/* HuffmanTensor::decode_to_quantized  src/huffman.rs:374-404: q, q_t [rows*cols], scales [cols]. */
+pg_status pg_huffman_tensor_decode_to_quantized(pg_ctx *ctx, const pg_huffman_tensor *t, int8_t *q, int8_t *q_t,
+                                                float *scales);
+/* HuffmanTensor::to_gpu  src/huffman.rs:430-435, decoding on the device. */
+pg_status pg_huffman_tensor_to_gpu(pg_ctx *ctx, const pg_huffman_tensor *t, pg_qtensor **out);
+/* matmul_huffman  src/huffman.rs:465-474: decode, then pg_matmul_quantized. */
+pg_status pg_matmul_huffman(pg_ctx *ctx, const float *a, size_t m, size_t k, const pg_huffman_tensor *t, float *out);
+
 /* ---- grouped MoE expert FFN ------------------------------------------------- */
 
 /* MoELayer::forward after the router matmul  examples/grok1/moe.rs:70-109

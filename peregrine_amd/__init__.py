@@ -8,6 +8,6 @@ library raises, and every call needs a GPU.
 """
 from . import _ffi  # noqa: F401  (fails loudly if the library is missing)
 from .context import Context, default_context
-from . import quant, gguf, moe, llama, mxfp4
+from . import quant, gguf, moe, llama, mxfp4, huffman
 
-__all__ = ["Context", "default_context", "quant", "gguf", "moe", "llama", "mxfp4"]
+__all__ = ["Context", "default_context", "quant", "gguf", "moe", "llama", "mxfp4", "huffman"]

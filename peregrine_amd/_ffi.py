@@ -81,6 +81,19 @@ SIGNATURES = {
     "pg_qtensor_from_record": [_vp, _vp, _sz, _pp, C.POINTER(_sz)],
     "pg_moe_ffn": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
     "pg_moe_ffn_dev": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
+    "pg_huffman_table_from_frequencies": [_vp, _vp, _vp],
+    "pg_huffman_canonical_codes": [_vp, _vp],
+    "pg_huffman_encode": [_vp, _vp, _sz, _vp, _sz, C.POINTER(_sz)],
+    "pg_huffman_decode": [_vp, _vp, _vp, _sz, _sz, _vp],
+    "pg_huffman_tensor_from_quantized": [_vp, _vp, _sz, _sz, _sz, _pp],
+    "pg_huffman_tensor_from_parts": [_vp, _pp, C.POINTER(_sz), C.POINTER(_sz), _sz, _vp, _sz, _sz, _pp],
+    "pg_huffman_tensor_free": [_vp],
+    "pg_huffman_tensor_info": [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)],
+    "pg_huffman_tensor_stream": [_vp, _sz, _pp, C.POINTER(_sz), C.POINTER(_sz)],
+    "pg_huffman_tensor_table": [_vp, _pp, _pp],
+    "pg_huffman_tensor_decode_to_quantized": [_vp, _vp, _vp, _vp, _vp],
+    "pg_huffman_tensor_to_gpu": [_vp, _vp, _pp],
+    "pg_matmul_huffman": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_mxfp4_matmul": [_vp, _vp, _vp, _vp, _sz, _sz, _vp],
     "pg_mxfp4_upload": [_vp, _vp, _vp, _sz, _sz, _pp],
     "pg_mxfp4_expert_create": [_vp, _sz, _sz, C.c_float, C.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _pp],
@@ -115,6 +128,7 @@ _OTHER_RESTYPE = {
     "pg_gguf_free": None,
     "pg_gguf_file_close": None,
     "pg_rope_free": None,
+    "pg_huffman_tensor_free": None,
     "pg_mxfp4_expert_free": None,
     "pg_kv_cache_free": None,
     "pg_llama_block_free": None,

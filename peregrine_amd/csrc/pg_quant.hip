@@ -401,6 +401,29 @@ PG_API pg_status pg_dequantize(pg_ctx *ctx, const int8_t *q, const float *scales
     return PG_OK;
 }
 
+// A quantised weight from its row-major [rows, cols] integers already on the device.
+pg_status pg_qtensor_from_device_q(pg_ctx *ctx, const int8_t *q_dev, const float *scales_host, size_t rows, size_t cols,
+                                   pg_qtensor **out) {
+    *out = nullptr;
+    pg_qtensor *t = nullptr;
+    PG_TRY(qtensor_alloc(ctx, rows, cols, &t));
+    fill_u32_kernel<<<grid_for(t->n_pad, 256), 256, 0, ctx->stream>>>(reinterpret_cast<uint32_t *>(t->scales), t->n_pad,
+                                                                    0x3F800000u);
+    hipError_t e = hipMemcpyAsync(t->scales, scales_host, cols * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) {
+        dim3 g(grid_for(cols, 64), grid_for(rows, 64));
+        transpose_i8_kernel<<<g, 256, 0, ctx->stream>>>(q_dev, rows, cols, cols, t->w_t, t->k_pad);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        pg_qtensor_free(ctx, t);
+        return pg_fail(PG_EDEVICE, "qtensor from device integers: %s", hipGetErrorString(e));
+    }
+    *out = t;
+    return PG_OK;
+}
+
 PG_API pg_status pg_qtensor_upload(pg_ctx *ctx, const int8_t *q, const float *scales, size_t rows,
                                    size_t cols, pg_qtensor **out) {
     PG_TRY(pg_use(ctx));
@@ -409,28 +432,10 @@ PG_API pg_status pg_qtensor_upload(pg_ctx *ctx, const int8_t *q, const float *sc
     PG_CHECK_ARG(rows > 0 && cols > 0, "pg_qtensor_upload: empty tensor %zu x %zu", rows, cols);
     PG_CHECK_ARG(q && scales, "pg_qtensor_upload: null pointer");
     PG_CHECK_ARG(rows < (1ull << 31) && cols < (1ull << 31), "pg_qtensor_upload: shape too large");
-    pg_qtensor *t = nullptr;
-    PG_TRY(qtensor_alloc(ctx, rows, cols, &t));
     pg_tmp dq;
-    pg_status st = dq.alloc(rows * cols);
-    if (st == PG_OK) {
-        hipError_t e = hipMemcpyAsync(dq.p, q, rows * cols, hipMemcpyHostToDevice, ctx->stream);
-        if (e == hipSuccess) {
-            fill_u32_kernel<<<grid_for(t->n_pad, 256), 256, 0, ctx->stream>>>(
-                reinterpret_cast<uint32_t *>(t->scales), t->n_pad, 0x3F800000u);
-            e = hipMemcpyAsync(t->scales, scales, cols * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
-        }
-        if (e == hipSuccess) {
-            dim3 g(grid_for(cols, 64), grid_for(rows, 64));
-            transpose_i8_kernel<<<g, 256, 0, ctx->stream>>>(dq.as<int8_t>(), rows, cols, cols, t->w_t, t->k_pad);
-            e = hipGetLastError();
-        }
-        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
-        if (e != hipSuccess) st = pg_fail(PG_EDEVICE, "pg_qtensor_upload: %s", hipGetErrorString(e));
-    }
-    if (st != PG_OK) { pg_qtensor_free(ctx, t); return st; }
-    *out = t;
-    return PG_OK;
+    PG_TRY(dq.alloc(rows * cols));
+    PG_HIP(hipMemcpyAsync(dq.p, q, rows * cols, hipMemcpyHostToDevice, ctx->stream));
+    return pg_qtensor_from_device_q(ctx, dq.as<int8_t>(), scales, rows, cols, out);
 }
 
 PG_API pg_status pg_qtensor_from_f32_dev(pg_ctx *ctx, const float *w_dev, size_t rows, size_t cols,

@@ -238,3 +238,42 @@ def mxfp4_expert_forward(x, hidden, intermediate, alpha, clamp, b1, s1, b2, s2, 
                                       _p(_f32(bias1)), _p(_f32(bias2)), _p(out))
     assert rc == 0
     return out
+
+
+lib.orc_huffman_table.restype = None
+lib.orc_huffman_canonical_codes.restype = None
+lib.orc_huffman_encode.restype = C.c_size_t
+
+
+def huffman_table(freqs):
+    """(bit_lengths[256] u8, codes[256] u32) from 256 frequencies."""
+    f = np.ascontiguousarray(freqs, np.uint64)
+    bl, codes = np.zeros(256, np.uint8), np.zeros(256, np.uint32)
+    lib.orc_huffman_table(_p(f), _p(bl), _p(codes))
+    return bl, codes
+
+
+def huffman_codes(bl):
+    bl = np.ascontiguousarray(bl, np.uint8)
+    codes = np.zeros(256, np.uint32)
+    lib.orc_huffman_canonical_codes(_p(bl), _p(codes))
+    return codes
+
+
+def huffman_encode(bl, data):
+    bl = np.ascontiguousarray(bl, np.uint8)
+    codes = huffman_codes(bl)
+    d = np.ascontiguousarray(data, np.int8).reshape(-1)
+    n = lib.orc_huffman_encode(_p(bl), _p(codes), _p(d), _sz(d.size), None)
+    out = np.zeros(n, np.uint8)
+    lib.orc_huffman_encode(_p(bl), _p(codes), _p(d), _sz(d.size), _p(out))
+    return out.tobytes()
+
+
+def huffman_decode(bl, stream, num_symbols):
+    bl = np.ascontiguousarray(bl, np.uint8)
+    b = np.frombuffer(bytes(stream), np.uint8)
+    out = np.empty(num_symbols, np.int8)
+    rc = lib.orc_huffman_decode(_p(bl), _p(b), _sz(b.size), _sz(num_symbols), _p(out))
+    assert rc == 0, "a code does not fit the 12-bit table"
+    return out

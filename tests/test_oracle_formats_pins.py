@@ -104,3 +104,103 @@ def test_mxfp4_expert_closed_forms_and_float64(orc):
     want = mx_dequant(b2, s2, hidden, inter) @ act + bias2
     got = orc.mxfp4_expert_forward(x, hidden, inter, alpha, clamp, b1, s1, b2, s2, bias1, bias2)
     assert np.abs(got - want).max() <= 5e-6 * np.abs(want).max()
+
+
+# ---- canonical Huffman ------------------------------------------------------------------
+
+def biased_i8(n, seed):
+    """random_i8 of the reference's unit tests (src/huffman.rs:743-754)."""
+    out, state = np.empty(n, np.int8), seed
+    for i in range(n):
+        state = (state * 1103515245 + 12345) & 0xFFFFFFFF
+        raw = ((state >> 16) % 256 - 128)
+        raw = raw - 256 if raw > 127 else raw
+        v = raw if (state >> 8) % 4 == 0 else int(raw / 4)      # Rust integer division truncates
+        out[i] = v
+    return out
+
+
+def heap_huffman_cost(freqs):
+    import heapq
+    h = [int(f) for f in freqs if f > 0]
+    if len(h) == 1:
+        return h[0]
+    heapq.heapify(h)
+    cost = 0
+    while len(h) > 1:
+        a, b = heapq.heappop(h), heapq.heappop(h)
+        cost += a + b
+        heapq.heappush(h, a + b)
+    return cost
+
+
+def test_huffman_table_hand_worked_tie_breaking(orc):
+    """Leaves [1,1,1,1,2] (symbols -128..-124).  Stable order a b c d e; a+b -> I1(2); c+d -> I2(2);
+    then e(2), I1(2), I2(2) tie and the LEAF goes first: e+I1 -> I3(4); I2+I3 -> root.  Depths:
+    a,b = 3; c,d = 2; e = 2.  (Taking internal nodes first would give e = 1 and a..d = 3.)"""
+    f = np.zeros(256, np.uint64)
+    f[:5] = [1, 1, 1, 1, 2]
+    bl, codes = orc.huffman_table(f)
+    assert bl[:5].tolist() == [3, 3, 2, 2, 2] and not bl[5:].any()
+    # canonical: lengths ascending, symbol order within a length: c=00 d=01 e=10 a=110 b=111
+    assert codes[:5].tolist() == [0b110, 0b111, 0b00, 0b01, 0b10]
+    # the reference's own table test (src/huffman.rs:801-815) and the one-symbol rule (:52-64)
+    f = np.zeros(256, np.uint64)
+    f[128], f[129] = 100, 50
+    bl, codes = orc.huffman_table(f)
+    assert bl[128] == 1 and bl[129] == 1 and codes[128] == 0 and codes[129] == 1
+    f = np.zeros(256, np.uint64)
+    f[170] = 512
+    bl, codes = orc.huffman_table(f)
+    assert bl[170] == 1 and codes[170] == 0 and bl.sum() == 1
+    assert not orc.huffman_table(np.zeros(256, np.uint64))[0].any()
+
+
+def test_huffman_table_is_optimal_and_complete(orc):
+    rng = np.random.default_rng(2)
+    for trial in range(6):
+        f = np.zeros(256, np.uint64)
+        k = [2, 3, 17, 100, 256, 256][trial]
+        f[rng.choice(256, k, replace=False)] = rng.integers(1, 50 if trial < 5 else 4, k)
+        bl, codes = orc.huffman_table(f)
+        assert ((bl > 0) == (f > 0)).all()
+        assert bl.max() <= 12                                     # a clamped depth would break the cost equality below
+        assert int((f * bl).sum()) == heap_huffman_cost(f)        # any Huffman tree has the optimal cost
+        assert sum(2.0 ** -int(l) for l in bl if l) == 1.0        # Kraft equality: a complete prefix code
+        used = [(int(bl[s]), int(codes[s])) for s in range(256) if bl[s]]
+        strs = sorted(format(c, "b").zfill(l) for l, c in used)
+        assert all(not strs[i + 1].startswith(strs[i]) for i in range(len(strs) - 1))   # prefix-free
+
+
+def test_huffman_depth_clamp_is_the_reference_s(orc):
+    """Fibonacci frequencies make a path deeper than 12; the reference clamps the depths and
+    keeps going (src/huffman.rs:128-134), which over-subscribes the code."""
+    fib = [1, 1]
+    while len(fib) < 20:
+        fib.append(fib[-1] + fib[-2])
+    f = np.zeros(256, np.uint64)
+    f[:20] = fib
+    bl, _ = orc.huffman_table(f)
+    assert bl[:20].max() == 12 and (bl[:8] == 12).all()
+    assert sum(2.0 ** -int(l) for l in bl if l) > 1.0
+
+
+def test_huffman_encode_hand_packed_and_reference_round_trips(orc):
+    f = np.zeros(256, np.uint64)
+    f[:5] = [1, 1, 1, 1, 2]
+    bl, _ = orc.huffman_table(f)                                  # a=110 b=111 c=00 d=01 e=10
+    data = np.array([-128, -124, -126, -127, -125], np.int8)      # a e c b d -> 110 10 00 111 01 -> 11010001 1101(0000)
+    assert orc.huffman_encode(bl, data) == bytes([0b11010001, 0b11010000])
+    assert (orc.huffman_decode(bl, bytes([0b11010001, 0b11010000]), 5) == data).all()
+    assert orc.huffman_encode(bl, np.zeros(0, np.int8)) == b""    # src/huffman.rs:771-778
+    # src/huffman.rs:756-768: round trip on the biased generator
+    data = biased_i8(1024, 42)
+    bl, _ = orc.huffman_table(np.bincount(data.astype(np.int16) + 128, minlength=256))
+    enc = orc.huffman_encode(bl, data)
+    assert (orc.huffman_decode(bl, enc, data.size) == data).all()
+    assert len(enc) < data.size                                    # it does compress
+    # src/huffman.rs:780-797: 512 equal symbols in at most 65 bytes
+    same = np.full(512, 42, np.int8)
+    bl, _ = orc.huffman_table(np.bincount(same.astype(np.int16) + 128, minlength=256))
+    enc = orc.huffman_encode(bl, same)
+    assert len(enc) <= 65 and (orc.huffman_decode(bl, enc, 512) == same).all()
