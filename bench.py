@@ -411,6 +411,37 @@ def main():
             lib.pg_gguf_free(ctx.handle, h)
     torch.cuda.empty_cache()
 
+    # ------------------------------------------------------------------ Huffman-coded weight -> device tensor
+    hk, hn, hstreams = 4096, 4096, 16
+    hq = np.clip(np.rint(np.random.default_rng(21).standard_normal(hk * hn) * 9.0), -24, 24).astype(np.int8)
+    hscales = np.full(hn, 0.01, np.float32)
+    ht = C.c_void_p()
+    check(lib.pg_huffman_tensor_from_quantized(C.c_void_p(hq.ctypes.data), C.c_void_p(hscales.ctypes.data), hk, hn, hstreams,
+                                               C.byref(ht)))
+    hsz = C.c_size_t()
+    check(lib.pg_huffman_tensor_info(ht, None, None, None, C.byref(hsz)))
+
+    def huff_step():
+        h = C.c_void_p()
+        check(lib.pg_huffman_tensor_to_gpu(ctx.handle, ht, C.byref(h)))
+        lib.pg_qtensor_free(ctx.handle, h)
+
+    for _ in range(2):
+        huff_step()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        huff_step()
+    huff_ms = (time.perf_counter() - t0) / 5 * 1e3
+    hprof = profiled(huff_step, 5)
+    huff_kernels_ms = sum(v[0] * v[1] for k, v in hprof.items() if k.startswith("huffman")) / 5
+    huffman = {"workload": f"HuffmanTensor::to_gpu of a [{hk}x{hn}] int8 weight in {hstreams} streams "
+                           f"({hsz.value / 1e6:.1f} MB compressed, ratio {(hk * hn + 4 * hn) / hsz.value:.2f}); host streams in, device tensor out",
+               "ms_per_call_wall": round(huff_ms, 3), "decode_kernels_ms": round(huff_kernels_ms, 3),
+               "symbols_per_s_kernels": round(hk * hn / (huff_kernels_ms * 1e-3), 0),
+               "kernels_ms_x_launches": {k: [round(v[0], 4), round(v[1] / 5, 1)] for k, v in hprof.items()}}
+    lib.pg_huffman_tensor_free(ht)
+    del hq
+
     if args.calibrate_copy:  # a plain copy of known size: 512 MiB read + 512 MiB written per launch
         src = torch.empty(128 << 20, device=dev, dtype=torch.float32).normal_()
         dst = torch.empty_like(src)
@@ -434,7 +465,7 @@ def main():
                                "each product = per-row activation quantisation + i8 GEMM + f32 rescale",
                    "m": M_PREFILL, "ops_per_step": LAYER_OPS},
         "pct_int8_mfma_peak": round(100 * tops / PEAK_INT8_TOPS, 2),
-        "roofline": roofline, "activation_quant": act_quant, "w8a32_gate": w8a32, "linear_m32": linear_m32, "decode_gemv": decode, "gguf_q4_0_gemv": gguf, "gguf_q4_0_skinny": skinny, "moe_q8_0": moe, "llama_block_q4_0": llama_block,
+        "roofline": roofline, "activation_quant": act_quant, "w8a32_gate": w8a32, "linear_m32": linear_m32, "decode_gemv": decode, "gguf_q4_0_gemv": gguf, "gguf_q4_0_skinny": skinny, "moe_q8_0": moe, "llama_block_q4_0": llama_block, "huffman_to_gpu": huffman,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line), flush=True)

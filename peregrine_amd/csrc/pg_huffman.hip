@@ -213,7 +213,15 @@ __global__ __launch_bounds__(WG) void huff_sync_kernel(const uint8_t *__restrict
     for (int round = 0; round < WG + 1; ++round) {  // settles in at most WG rounds given the first start
         __syncthreads();
         unsigned long long want = start;
-        if (live && local > 0) want = threadIdx.x == 0 ? end_g[g - 1] : s_end[threadIdx.x - 1];
+        if (live && local > 0) {
+            // The neighbouring workgroup's last end is only there from the second round on.
+            if (threadIdx.x > 0) want = s_end[threadIdx.x - 1];
+            else if (!first_round) want = end_g[g - 1];
+            // A predecessor ends on the first code boundary at or past this subsequence's first
+            // bit; anything else is not an end it can have reported.
+            const unsigned long long lo = (unsigned long long)local * SUBSEQ_BITS;
+            if (want < lo || want >= lo + MAX_LUT_BITS) want = start;
+        }
         __syncthreads();
         const bool redo = live && want != start;
         if (redo) {
