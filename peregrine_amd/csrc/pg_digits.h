@@ -1,0 +1,77 @@
+// Activation blocks -> fixed-point digits for the streaming (one-row) block-dequant product:
+// the step every producer of a GEMV input ends with, so that the f32 row need not be written
+// and read back by a separate kernel.
+#pragma once
+#include "pg_internal.h"
+
+// Eight consecutive lanes hold one block of 32 activations, four each (`sub` = lane within the
+// group, f = its elements 4*sub .. 4*sub+3 of block b of activation row `row`); all eight
+// must call together.  Writes the block's digit planes and its power-of-two scale:
+//   xs[row][b]          the scale s (NaN if the block holds a NaN or inf)
+//   digits[row][j][b]   16 bytes per (plane j, block b)
+//     NIB (Q4_0):  |X| < 2^18, X = sum_j 16^j n_j with five signed 4-bit digits; plane j holds
+//                  n_j of the block's 32 elements, element e in nibble e.
+//     bytes (Q8_0, MXFP4): |X| < 2^22, X = 65536 a0 + 256 a1 + a2 with signed byte digits;
+//                  plane 2j+h holds a_j of elements 16h..16h+15.
+template <bool NIB>
+__device__ __forceinline__ void pg_emit_digits(const float (&f)[4], size_t row, int b, int sub, int nb,
+                                               int8_t *__restrict__ digits, float *__restrict__ xs) {
+    float amax = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3])));
+    int bad = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]);
+#pragma unroll
+    for (int off = 1; off < 8; off <<= 1) {
+        amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+        bad |= __shfl_xor(bad, off, 64);
+    }
+    constexpr int BITS = NIB ? 18 : 22;
+    float s = 1.0f, inv = 1.0f;
+    if (bad || !(amax <= 3.4028234663852886e38f)) {
+        s = __uint_as_float(0x7FC00000u);
+        inv = 0.0f;
+    } else if (amax > 0.0f) {
+        int ex;
+        (void)frexpf(amax, &ex);  // amax = f * 2^ex, f in [0.5, 1)
+        int se = ex - BITS;       // |x| / 2^se < 2^BITS
+        if (se < -126) se = -126;
+        s = ldexpf(1.0f, se);
+        inv = ldexpf(1.0f, -se);
+    }
+    int X[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float t = f[e] * inv;
+        X[e] = (t != t) ? 0 : (int)rintf(t);
+    }
+    int8_t *drow = digits + row * (size_t)nb * 96;
+    if (NIB) {
+#pragma unroll
+        for (int j = 0; j < 5; ++j) {
+            unsigned packed = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = ((X[e] + 8) & 15) - 8;  // signed 4-bit digit
+                X[e] = (X[e] - n) >> 4;
+                packed |= (unsigned)(n & 15) << (4 * e);
+            }
+            // this thread's elements 4*sub .. 4*sub+3 are nibbles 4*sub.. of the block: bytes 2*sub, 2*sub+1
+            *reinterpret_cast<uint16_t *>(drow + ((size_t)j * nb + b) * 16 + 2 * sub) = (uint16_t)packed;
+        }
+    } else {
+        int a[3][4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            a[2][e] = ((X[e] + 128) & 255) - 128;
+            const int X1 = (X[e] - a[2][e]) >> 8;
+            a[1][e] = ((X1 + 128) & 255) - 128;
+            a[0][e] = (X1 - a[1][e]) >> 8;
+        }
+        const int e0 = sub * 4, h = e0 >> 4;
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const unsigned packed = (unsigned)(a[j][0] & 255) | ((unsigned)(a[j][1] & 255) << 8) |
+                                    ((unsigned)(a[j][2] & 255) << 16) | ((unsigned)(a[j][3] & 255) << 24);
+            *reinterpret_cast<unsigned *>(drow + ((size_t)(2 * j + h) * nb + b) * 16 + (e0 & 15)) = packed;
+        }
+    }
+    if (sub == 0) xs[row * (size_t)nb + b] = s;
+}

@@ -18,6 +18,7 @@
 // (relative tolerance 1e-3 is the contract; the tests hold this path to 2e-5).
 #include <new>
 #include "pg_internal.h"
+#include "pg_digits.h"
 
 namespace {
 
@@ -136,64 +137,7 @@ __global__ __launch_bounds__(256) void x_to_digits_kernel(const float *__restric
     if (b >= nb) return;  // whole 8-thread groups leave together
     const float4 v = reinterpret_cast<const float4 *>(x + (row * nb + b) * 32)[sub];
     const float f[4] = {v.x, v.y, v.z, v.w};
-    float amax = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3])));
-    int bad = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]);
-#pragma unroll
-    for (int off = 1; off < 8; off <<= 1) {
-        amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-        bad |= __shfl_xor(bad, off, 64);
-    }
-    constexpr int BITS = NIB ? 18 : 22;
-    float s = 1.0f, inv = 1.0f;
-    if (bad || !(amax <= 3.4028234663852886e38f)) {
-        s = __uint_as_float(0x7FC00000u);
-        inv = 0.0f;
-    } else if (amax > 0.0f) {
-        int ex;
-        (void)frexpf(amax, &ex);  // amax = f * 2^ex, f in [0.5, 1)
-        int se = ex - BITS;       // |x| / 2^se < 2^BITS
-        if (se < -126) se = -126;
-        s = ldexpf(1.0f, se);
-        inv = ldexpf(1.0f, -se);
-    }
-    int X[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const float t = f[e] * inv;
-        X[e] = (t != t) ? 0 : (int)rintf(t);
-    }
-    int8_t *drow = digits + row * (size_t)nb * 96;
-    if (NIB) {
-#pragma unroll
-        for (int j = 0; j < 5; ++j) {
-            unsigned packed = 0;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int n = ((X[e] + 8) & 15) - 8;  // signed 4-bit digit
-                X[e] = (X[e] - n) >> 4;
-                packed |= (unsigned)(n & 15) << (4 * e);
-            }
-            // this thread's elements 4*sub .. 4*sub+3 are nibbles 4*sub.. of the block: bytes 2*sub, 2*sub+1
-            *reinterpret_cast<uint16_t *>(drow + ((size_t)j * nb + b) * 16 + 2 * sub) = (uint16_t)packed;
-        }
-    } else {
-        int a[3][4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            a[2][e] = ((X[e] + 128) & 255) - 128;
-            const int X1 = (X[e] - a[2][e]) >> 8;
-            a[1][e] = ((X1 + 128) & 255) - 128;
-            a[0][e] = (X1 - a[1][e]) >> 8;
-        }
-        const int e0 = sub * 4, h = e0 >> 4;
-#pragma unroll
-        for (int j = 0; j < 3; ++j) {
-            const unsigned packed = (unsigned)(a[j][0] & 255) | ((unsigned)(a[j][1] & 255) << 8) |
-                                    ((unsigned)(a[j][2] & 255) << 16) | ((unsigned)(a[j][3] & 255) << 24);
-            *reinterpret_cast<unsigned *>(drow + ((size_t)(2 * j + h) * nb + b) * 16 + (e0 & 15)) = packed;
-        }
-    }
-    if (sub == 0) xs[row * (size_t)nb + b] = s;
+    pg_emit_digits<NIB>(f, row, b, sub, nb, digits, xs);
 }
 
 // ---- M = 1 fused dequant-GEMV ------------------------------------------------------
@@ -258,7 +202,7 @@ template <int QT, int BPL, int RW, int R, bool BF = false>
 __global__ __launch_bounds__(64) void gguf_gemv_kernel(
     const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0, pg_gemv_batch batch,
     int n_out, int nb, const int8_t *__restrict__ digits_base, const float *__restrict__ xs_base,
-    float *__restrict__ y_base) {
+    float *__restrict__ y_base, const float *__restrict__ residual_base) {
     constexpr int SEG = 64 * BPL;  // blocks per K segment
     constexpr int NG = RW / R;
     constexpr int NH = QT == 8 ? 2 : 1;
@@ -357,13 +301,13 @@ __global__ __launch_bounds__(64) void gguf_gemv_kernel(
         for (int r = 0; r < R; ++r) {
             const float v = wave_sum_f32(acc[g][r]);
             const int row = row0 + g * R + r;
-            if (lane == 0 && row < n_out) y[row] = v;
+            if (lane == 0 && row < n_out) y[row] = residual_base ? residual_base[(size_t)item * n_out + row] + v : v;
         }
 }
 
 template <int QT, int BPL, bool BF>
 pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
-                          const pg_gemv_batch &batch, const pg_xdigits &xd, float *y) {
+                          const pg_gemv_batch &batch, const pg_xdigits &xd, float *y, const float *residual) {
     const int nb = (int)(k_in / 32);
     // rows in flight per wavefront: bounded by registers (16 B of weights per row and block)
     constexpr int NH = QT == 8 ? 2 : 1;
@@ -374,7 +318,7 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
         const dim3 grid(grid_for(n_out, RWW), (unsigned)batch.count);                              \
         PG_TRY(pg_launch(ctx, QT == 4 ? "gguf_gemv_q4_0" : (BF ? "gguf_gemv_mxfp4" : "gguf_gemv_q8_0"), \
                          gguf_gemv_kernel<QT, BPL, RWW, RR, BF>, grid, dim3(64), 0, qs, d, batch,  \
-                         (int)n_out, nb, xd.digits, xd.xs, y));                                    \
+                         (int)n_out, nb, xd.digits, xd.xs, y, residual));                          \
     } while (0)
     if (n_out / 8 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(8, R8);
     else if (n_out / 4 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(4, (R8 < 4 ? R8 : 4));
@@ -385,15 +329,15 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
 
 template <int QT, bool BF = false>
 pg_status launch_gemv(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
-                      const pg_gemv_batch &batch, const pg_xdigits &xd, float *y) {
+                      const pg_gemv_batch &batch, const pg_xdigits &xd, float *y, const float *residual) {
     const size_t nb = k_in / 32;
     size_t bpl = (nb + 63) / 64;
     if (bpl > 4) bpl = 4;  // longer rows run as several K segments of 256 blocks
     switch (bpl) {
-        case 1: return launch_gemv_bpl<QT, 1, BF>(ctx, n_out, k_in, qs, d, batch, xd, y);
-        case 2: return launch_gemv_bpl<QT, 2, BF>(ctx, n_out, k_in, qs, d, batch, xd, y);
-        case 3: return launch_gemv_bpl<QT, 3, BF>(ctx, n_out, k_in, qs, d, batch, xd, y);
-        default: return launch_gemv_bpl<QT, 4, BF>(ctx, n_out, k_in, qs, d, batch, xd, y);
+        case 1: return launch_gemv_bpl<QT, 1, BF>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
+        case 2: return launch_gemv_bpl<QT, 2, BF>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
+        case 3: return launch_gemv_bpl<QT, 3, BF>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
+        default: return launch_gemv_bpl<QT, 4, BF>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
     }
 }
 
@@ -432,12 +376,12 @@ pg_status pg_launch_x_to_digits(pg_ctx *ctx, const float *x_dev, size_t rows, si
 
 pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in,
                               const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
-                              const pg_xdigits &xd, float *y) {
+                              const pg_xdigits &xd, float *y, const float *residual) {
     if (batch.count == 0) return PG_OK;
     if (batch.count > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_gemv: more than 65535 batch items");
-    if (ggml_type == PG_GGML_Q4_0) return launch_gemv<4>(ctx, n_out, k_in, qs, d, batch, xd, y);
-    if (ggml_type == PG_MXFP4) return launch_gemv<8, true>(ctx, n_out, k_in, qs, d, batch, xd, y);
-    return launch_gemv<8>(ctx, n_out, k_in, qs, d, batch, xd, y);
+    if (ggml_type == PG_GGML_Q4_0) return launch_gemv<4>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
+    if (ggml_type == PG_MXFP4) return launch_gemv<8, true>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
+    return launch_gemv<8>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
 }
 
 // Quantise `m` activation rows (device) into the arena and run the fused product: the

@@ -191,9 +191,10 @@ struct pg_gemv_batch {
     const int *expert_of;
     int x_row_div;
 };
+// y[item][row] = product (+ residual[item][row] when `residual` is given).
 pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in,
                               const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
-                              const pg_xdigits &xd, float *y);
+                              const pg_xdigits &xd, float *y, const float *residual = nullptr);
 // Activation rows as two byte-digit planes for the matrix-core product (see pg_gguf_mm.hip).
 struct pg_mmdigits {
     int8_t *digits;  // [rows][2 planes][k/32 blocks][2 halves][16 bytes]

@@ -16,6 +16,7 @@
 #include <math.h>
 #include <new>
 #include "pg_internal.h"
+#include "pg_digits.h"
 
 struct pg_rope {
     float *cos_t, *sin_t;
@@ -35,6 +36,14 @@ struct pg_llama_block {
     float *attn_norm_w, *ffn_norm_w;
     float *arena;  // activations for seq_cap tokens
     size_t seq_cap;
+    // One-token step: digit buffers for the three GEMV inputs (model_dim, q_dim, ffn) and the
+    // device tables that let k/v and gate/up each run as one two-item launch.
+    void *dec;                        // one allocation
+    pg_xdigits xd_d, xd_q, xd_f;
+    const uint8_t *const *qs_kv, *const *qs_gu;
+    const uint16_t *const *d_kv, *const *d_gu;
+    const int *item_ids;              // {0, 1}
+    int digit_kind;                   // PG_GGML_Q4_0 (nibble digits), PG_GGML_Q8_0 (byte digits), 0 = mixed: no fused step
 };
 
 namespace {
@@ -85,10 +94,13 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(const float *a, const 
 
 // The same with the row held in registers: dim % 4 == 0 and dim <= 1024 * MAXV, so that every
 // load of the row is issued before the first is needed.
-template <int MAXV>
+// DIG: 0 = write the normalised row as f32; 1 / 2 = write it as nibble / byte digits for the
+// streaming product instead (dim a multiple of 32, so that 8-lane groups hold whole blocks).
+template <int MAXV, int DIG>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(const float4 *__restrict__ a, const float4 *__restrict__ b,
                                                               float4 *__restrict__ sum_out, const float4 *__restrict__ w,
-                                                              float eps, int dim4, float4 *__restrict__ out) {
+                                                              float eps, int dim4, float4 *__restrict__ out,
+                                                              int8_t *__restrict__ digits, float *__restrict__ xs) {
     __shared__ float red[4];
     const size_t row = (size_t)blockIdx.x * dim4;
     float4 v[MAXV], wv[MAXV];
@@ -121,9 +133,12 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(const float4 *__re
 #pragma unroll
     for (int j = 0; j < MAXV; ++j) {
         const int i = threadIdx.x + 256 * j;
-        if (i < dim4)
-            out[row + i] = float4{v[j].x * inv_rms * wv[j].x, v[j].y * inv_rms * wv[j].y, v[j].z * inv_rms * wv[j].z,
-                                  v[j].w * inv_rms * wv[j].w};
+        if (i < dim4) {
+            const float o[4] = {v[j].x * inv_rms * wv[j].x, v[j].y * inv_rms * wv[j].y, v[j].z * inv_rms * wv[j].z,
+                                v[j].w * inv_rms * wv[j].w};
+            if constexpr (DIG == 0) out[row + i] = float4{o[0], o[1], o[2], o[3]};
+            else pg_emit_digits<DIG == 1>(o, blockIdx.x, i >> 3, i & 7, dim4 >> 3, digits, xs);
+        }
     }
 }
 
@@ -284,12 +299,117 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(attn_args aa) {
     }
 }
 
+// The same for a split of at most 8 rounds of keys (the one-token step): q, the split's K rows
+// and its V rows are all requested at once, scores stay in registers, and the only exchanges
+// are the two block reductions and the sum over key slices.
+constexpr int ATT_SHORT_ROUNDS = 8;
+__global__ __launch_bounds__(256) void gqa_attention_short_kernel(attn_args aa) {
+    __shared__ float part[ATT_RED];
+    __shared__ float red[4];
+    // Workgroups go to the 8 XCDs round-robin.  All query rows that read the same keys (the
+    // heads of one kv group, every query token) are given to ONE XCD, one after the other, so
+    // that its L2 fetches that split's K and V rows once: workgroup id = 8 * j + xcd, the
+    // j-th workgroup of an XCD being member j % members of key set (j / members) * 8 + xcd.
+    const int members = aa.group * aa.seq_q, nkv = aa.nqh / aa.group;
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int member = j % members, set = (j / members) * 8 + xcd;
+    if (set >= nkv * aa.splits) return;  // the grid is rounded up to whole rounds of 8 key sets
+    const int kvh = set % nkv, split = set / nkv, qh = kvh * aa.group + member % aa.group, qt = member / aa.group;
+    const int tid = threadIdx.x;
+    const int L = aa.lanes, hd = aa.hd;
+    const int k0 = split * aa.chunk;
+    int k1 = min(aa.len, k0 + aa.chunk);
+    if (aa.mask_kind != 0) k1 = min(k1, aa.offset + qt + 1);
+    const int n = max(k1 - k0, 0);
+    const int sub = tid / L, within = tid % L, nsub = 256 / L, d0 = within * 4;
+    const bool vec = (hd & 3) == 0, have = d0 < hd;
+    const float *qsrc = aa.q + ((size_t)qh * aa.seq_q + qt) * hd + d0;
+    const float *kbase = aa.kc + (size_t)kvh * aa.k_stride + (size_t)k0 * hd + d0;
+    const float *vbase = aa.vc + (size_t)kvh * aa.v_stride + (size_t)k0 * hd + d0;
+    auto load4 = [&](const float *p) {
+        float4 r = {0.f, 0.f, 0.f, 0.f};
+        if (vec) {
+            r = *reinterpret_cast<const float4 *>(p);
+        } else {
+            r.x = p[0];
+            if (d0 + 1 < hd) r.y = p[1];
+            if (d0 + 2 < hd) r.z = p[2];
+            if (d0 + 3 < hd) r.w = p[3];
+        }
+        return r;
+    };
+    float4 q4 = {0.f, 0.f, 0.f, 0.f}, kv[ATT_SHORT_ROUNDS], vv[ATT_SHORT_ROUNDS];
+    bool live[ATT_SHORT_ROUNDS];
+    if (have) q4 = load4(qsrc);
+#pragma unroll
+    for (int u = 0; u < ATT_SHORT_ROUNDS; ++u) {
+        const int kt = u * nsub + sub;
+        live[u] = kt < n && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, qt, k0 + kt);
+        kv[u] = float4{0.f, 0.f, 0.f, 0.f};
+        vv[u] = float4{0.f, 0.f, 0.f, 0.f};
+        if (live[u] && have) {
+            kv[u] = load4(kbase + (size_t)kt * hd);
+            vv[u] = load4(vbase + (size_t)kt * hd);
+        }
+    }
+    float s[ATT_SHORT_ROUNDS], mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < ATT_SHORT_ROUNDS; ++u) {
+        float dot = q4.x * kv[u].x + q4.y * kv[u].y + q4.z * kv[u].z + q4.w * kv[u].w;
+        for (int m = 1; m < L; m <<= 1) dot += __shfl_xor(dot, m);
+        s[u] = -INFINITY;
+        if (live[u]) {
+            s[u] = dot * aa.scale;
+            if (aa.logit_cap > 0.f) s[u] = aa.logit_cap * tanhf(s[u] / aa.logit_cap);
+        }
+        mx = fmaxf(mx, s[u]);
+    }
+    mx = block_max(mx, red);
+    float sum = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < ATT_SHORT_ROUNDS; ++u) {
+        const float e = s[u] == -INFINITY ? 0.f : expf(s[u] - mx);
+        if (within == 0) sum += e;  // one lane per key
+        s[u] = e;
+    }
+    sum = block_sum(sum, red);
+    const bool final_pass = aa.splits == 1;
+    const float inv_sum = !final_pass ? 1.0f : (sum > 0.f ? 1.0f / sum : 0.f);
+#pragma unroll
+    for (int u = 0; u < ATT_SHORT_ROUNDS; ++u) {
+        const float p = s[u] * inv_sum;
+        if (p > 0.f) { acc[0] += p * vv[u].x; acc[1] += p * vv[u].y; acc[2] += p * vv[u].z; acc[3] += p * vv[u].w; }
+    }
+    for (int j = 0; j < 4; ++j) part[sub * (4 * L) + d0 + j] = acc[j];
+    __syncthreads();
+    const size_t rowi = (size_t)qt * aa.nqh + qh;
+    float *pdst = final_pass ? nullptr : aa.part + (rowi * aa.splits + split) * (size_t)(hd + 2);
+    if (!final_pass && tid == 0) {
+        pdst[0] = mx;
+        pdst[1] = sum;
+    }
+    for (int i = tid; i < hd; i += 256) {
+        float o = 0.f;
+        for (int ss = 0; ss < nsub; ++ss) o += part[ss * (4 * L) + i];
+        if (final_pass) {
+            float *dst = aa.out + rowi * hd + i;
+            *dst = aa.accumulate ? *dst + o : o;
+        } else {
+            pdst[2 + i] = o;
+        }
+    }
+}
+
 constexpr int ATT_SPLITS_MAX = 2048;
 
 // Merge the splits of one (query token, query head) row: with M = max of the split maxima and
 // w_s = exp(m_s - M), out = sum_s w_s o_s / sum_s w_s l_s, splits in ascending order.
+// DIG 1 / 2: the merged row is written as nibble / byte digits of the [seq_q, num_q_heads * hd]
+// matrix that o_proj multiplies (hd a multiple of 32; workgroup = row qt * nqh + qh), not as f32.
+template <int DIG>
 __global__ __launch_bounds__(128) void gqa_combine_kernel(const float *__restrict__ part, int splits, int hd,
-                                                          float *__restrict__ out, int accumulate) {
+                                                          float *__restrict__ out, int accumulate, int nqh,
+                                                          int8_t *__restrict__ digits, float *__restrict__ xs) {
     __shared__ float wts[ATT_SPLITS_MAX];
     __shared__ float red[2];
     const float *p = part + (size_t)blockIdx.x * splits * (hd + 2);
@@ -306,11 +426,26 @@ __global__ __launch_bounds__(128) void gqa_combine_kernel(const float *__restric
     }
     l = block_sum(l, red);  // its barriers publish wts[]
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    for (int i = tid; i < hd; i += 128) {
-        float o = 0.f;
-        for (int s = 0; s < splits; ++s) o += wts[s] * p[(size_t)s * (hd + 2) + 2 + i];
-        float *dst = out + (size_t)blockIdx.x * hd + i;
-        *dst = accumulate ? *dst + o * inv : o * inv;
+    if constexpr (DIG == 0) {
+        for (int i = tid; i < hd; i += 128) {
+            float o = 0.f;
+            for (int s = 0; s < splits; ++s) o += wts[s] * p[(size_t)s * (hd + 2) + 2 + i];
+            float *dst = out + (size_t)blockIdx.x * hd + i;
+            *dst = accumulate ? *dst + o * inv : o * inv;
+        }
+    } else {
+        const int qt = blockIdx.x / nqh, qh = blockIdx.x - qt * nqh;
+        for (int i4 = tid; i4 < hd / 4; i4 += 128) {  // whole 8-lane groups: hd / 4 is a multiple of 8
+            float o[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int s = 0; s < splits; ++s) {
+                const float wv = wts[s];
+                const float *src = p + (size_t)s * (hd + 2) + 2 + 4 * i4;
+                o[0] += wv * src[0]; o[1] += wv * src[1]; o[2] += wv * src[2]; o[3] += wv * src[3];
+            }
+            for (int j = 0; j < 4; ++j) o[j] *= inv;
+            const int e4 = qh * (hd / 4) + i4;  // float4 index within the row
+            pg_emit_digits<DIG == 1>(o, qt, e4 >> 3, e4 & 7, nqh * hd / 32, digits, xs);
+        }
     }
 }
 
@@ -322,6 +457,18 @@ __global__ __launch_bounds__(256) void swiglu_kernel(float *__restrict__ g, cons
     }
 }
 
+// One row: silu(g) * u written as GEMV digits (n a multiple of 32).
+template <bool NIB>
+__global__ __launch_bounds__(256) void swiglu_digits_kernel(const float4 *__restrict__ g, const float4 *__restrict__ u, int n4,
+                                                            int8_t *__restrict__ digits, float *__restrict__ xs) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;  // whole 8-lane groups leave together
+    const float4 gv = g[i], uv = u[i];
+    const float o[4] = {gv.x / (1.0f + expf(-gv.x)) * uv.x, gv.y / (1.0f + expf(-gv.y)) * uv.y,
+                        gv.z / (1.0f + expf(-gv.z)) * uv.z, gv.w / (1.0f + expf(-gv.w)) * uv.w};
+    pg_emit_digits<NIB>(o, 0, i >> 3, i & 7, n4 >> 3, digits, xs);
+}
+
 __global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, const float *__restrict__ b,
                                                   float *__restrict__ out, size_t n) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -330,14 +477,29 @@ __global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, c
 
 inline unsigned blocks_for(size_t n) { return (unsigned)((n + 255) / 256); }
 
+bool rmsnorm_vec_ok(const float *a, const float *b, float *sum_out, const float *w, float *out, size_t dim) {
+    const uintptr_t align = (uintptr_t)a | (uintptr_t)b | (uintptr_t)sum_out | (uintptr_t)w | (uintptr_t)out;
+    return dim % 4 == 0 && dim <= 8192 && align % 16 == 0;
+}
+
+// RMSNorm whose output goes straight to GEMV digits (kind: PG_GGML_Q4_0 nibbles, else bytes).
+pg_status launch_rmsnorm_digits(pg_ctx *ctx, const float *a, const float *b, float *sum_out, const float *w, float eps,
+                                size_t rows, size_t dim, int kind, const pg_xdigits &xd) {
+    const bool nib = kind == PG_GGML_Q4_0;
+    auto *kern = dim <= 4096 ? (nib ? add_rmsnorm_vec_kernel<4, 1> : add_rmsnorm_vec_kernel<4, 2>)
+                             : (nib ? add_rmsnorm_vec_kernel<8, 1> : add_rmsnorm_vec_kernel<8, 2>);
+    return pg_launch(ctx, "add_rmsnorm_digits", kern, dim3((unsigned)rows), dim3(256), 0, (const float4 *)a, (const float4 *)b,
+                     (float4 *)sum_out, (const float4 *)w, eps, (int)(dim / 4), (float4 *)nullptr, xd.digits, xd.xs);
+}
+
 pg_status launch_rmsnorm(pg_ctx *ctx, const float *a, const float *b, float *sum_out, const float *w, float eps,
                          size_t rows, size_t dim, float *out) {
     if (rows == 0) return PG_OK;
-    const uintptr_t align = (uintptr_t)a | (uintptr_t)b | (uintptr_t)sum_out | (uintptr_t)w | (uintptr_t)out;
-    if (dim % 4 == 0 && dim <= 8192 && align % 16 == 0) {
-        auto *kern = dim <= 4096 ? add_rmsnorm_vec_kernel<4> : add_rmsnorm_vec_kernel<8>;
+    if (rmsnorm_vec_ok(a, b, sum_out, w, out, dim)) {
+        auto *kern = dim <= 4096 ? add_rmsnorm_vec_kernel<4, 0> : add_rmsnorm_vec_kernel<8, 0>;
         return pg_launch(ctx, "add_rmsnorm", kern, dim3((unsigned)rows), dim3(256), 0, (const float4 *)a, (const float4 *)b,
-                         (float4 *)sum_out, (const float4 *)w, eps, (int)(dim / 4), (float4 *)out);
+                         (float4 *)sum_out, (const float4 *)w, eps, (int)(dim / 4), (float4 *)out, (int8_t *)nullptr,
+                         (float *)nullptr);
     }
     return pg_launch(ctx, "add_rmsnorm", add_rmsnorm_kernel, dim3((unsigned)rows), dim3(256), 0, a, b, sum_out, w, eps,
                      (int)dim, out);
@@ -345,7 +507,9 @@ pg_status launch_rmsnorm(pg_ctx *ctx, const float *a, const float *b, float *sum
 
 pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, const pg_kv_cache *vc, size_t nqh,
                            size_t seq_q, float scale, int mask_kind, size_t offset, size_t window, size_t sink,
-                           float logit_cap, float *out, int accumulate) {
+                           float logit_cap, float *out, int accumulate, const pg_xdigits *xd = nullptr, int digit_kind = 0) {
+    // With `xd` (one-token step, accumulate == 0, head_dim % 32 == 0) the rows also, or only,
+    // leave as GEMV digits of kind `digit_kind`; `out` must still be a valid buffer.
     const size_t len = kc->len, hd = kc->head_dim;
     if (seq_q == 0 || nqh == 0) return PG_OK;
     if (len == 0) {  // nothing to attend to: the reference adds nothing to `output`
@@ -364,17 +528,21 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     aa.window = (int)(window > 0x7fffffffu ? 0x7fffffffu : window);
     aa.sink = (int)(sink > 0x7fffffffu ? 0x7fffffffu : sink);
     aa.accumulate = accumulate;
-    // Split the keys when the rows alone cannot fill the chip (decode) or a chunk would not
-    // fit the LDS score buffer; at least 4 rounds of keys per split.
+    // Split the keys when the rows alone cannot fill the chip (the one-token step) or a chunk
+    // would not fit the LDS score buffer.  Few rows: splits of 8 rounds of keys, which the
+    // short kernel handles with every load in flight at once.
     const size_t rows = seq_q * nqh, keys_per_round = 256 / (size_t)lanes;
-    size_t splits = rows >= 2 * (size_t)ctx->num_cu ? 1 : (2 * (size_t)ctx->num_cu + rows - 1) / rows;
-    const size_t max_splits = (len + 4 * keys_per_round - 1) / (4 * keys_per_round);
-    if (splits > max_splits) splits = max_splits;
-    const size_t min_splits = (len + ATT_CHUNK_MAX - 1) / ATT_CHUNK_MAX;
-    if (splits < min_splits) splits = min_splits;
-    size_t chunk = (len + splits - 1) / splits;
-    chunk = pg_round_up(chunk, keys_per_round);
-    splits = (len + chunk - 1) / chunk;
+    size_t chunk, splits;
+    bool short_kernel = false;
+    if (rows < 2 * (size_t)ctx->num_cu && (len + ATT_SHORT_ROUNDS * keys_per_round - 1) / (ATT_SHORT_ROUNDS * keys_per_round) <= (size_t)ATT_SPLITS_MAX) {
+        chunk = ATT_SHORT_ROUNDS * keys_per_round;
+        splits = (len + chunk - 1) / chunk;
+        short_kernel = true;
+    } else {
+        splits = (len + ATT_CHUNK_MAX - 1) / ATT_CHUNK_MAX;
+        chunk = pg_round_up((len + splits - 1) / splits, keys_per_round);
+        splits = (len + chunk - 1) / chunk;
+    }
     if (splits > (size_t)ATT_SPLITS_MAX) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: cache of %zu positions is too long", len);
     aa.chunk = (int)chunk; aa.splits = (int)splits;
     if (splits > 1) {
@@ -382,12 +550,23 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
         PG_TRY(pg_workspace(ctx, rows * splits * (hd + 2) * sizeof(float), &ws));
         aa.part = static_cast<float *>(ws);
     }
-    const size_t lds = (256 + ATT_RED + chunk) * sizeof(float);
-    PG_TRY(pg_launch(ctx, "gqa_attention", gqa_attention_kernel, dim3((unsigned)seq_q, (unsigned)nqh, (unsigned)splits),
-                     dim3(256), lds, aa));
-    if (splits > 1)
-        PG_TRY(pg_launch(ctx, "gqa_combine", gqa_combine_kernel, dim3((unsigned)rows), dim3(128), 0, (const float *)aa.part,
-                         (int)splits, (int)hd, out, accumulate));
+    const dim3 grid((unsigned)seq_q, (unsigned)nqh, (unsigned)splits);
+    if (short_kernel) {
+        const size_t sets = kc->num_kv_heads * splits, members = (nqh / kc->num_kv_heads) * seq_q;
+        const size_t wgs = (sets + 7) / 8 * 8 * members;
+        if (wgs >= (1ull << 31)) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: grid too large");
+        PG_TRY(pg_launch(ctx, "gqa_attention_short", gqa_attention_short_kernel, dim3((unsigned)wgs), dim3(256), 0, aa));
+    }
+    else
+        PG_TRY(pg_launch(ctx, "gqa_attention", gqa_attention_kernel, grid, dim3(256), (256 + ATT_RED + chunk) * sizeof(float), aa));
+    if (splits > 1) {
+        auto *kern = !xd ? gqa_combine_kernel<0> : (digit_kind == PG_GGML_Q4_0 ? gqa_combine_kernel<1> : gqa_combine_kernel<2>);
+        PG_TRY(pg_launch(ctx, xd ? "gqa_combine_digits" : "gqa_combine", kern, dim3((unsigned)rows), dim3(128), 0,
+                         (const float *)aa.part, (int)splits, (int)hd, out, accumulate, (int)nqh, xd ? xd->digits : nullptr,
+                         xd ? xd->xs : nullptr));
+    } else if (xd) {
+        PG_TRY(pg_launch_x_to_digits(ctx, out, seq_q, nqh * hd, digit_kind, *xd));
+    }
     return PG_OK;
 }
 
@@ -694,6 +873,26 @@ PG_API pg_status pg_llama_block_create(pg_ctx *ctx, size_t model_dim, size_t num
         return st;
     }
     b->ffn_norm_w = b->attn_norm_w + model_dim;
+    // one-token step buffers: three digit sets, then the pointer tables and the item ids
+    const size_t q_dim = num_q_heads * head_dim;
+    const size_t o_q = pg_xdigits_bytes(1, model_dim), o_f = o_q + pg_xdigits_bytes(1, q_dim);
+    const size_t o_tab = o_f + pg_xdigits_bytes(1, ffn_dim);
+    hipError_t e = hipMalloc(&b->dec, o_tab + 256);
+    if (e != hipSuccess) {
+        st = pg_fail(PG_ENOMEM, "pg_llama_block_create: %s", hipGetErrorString(e));
+        pg_llama_block_free(ctx, b);
+        return st;
+    }
+    char *base = static_cast<char *>(b->dec);
+    b->xd_d = pg_xdigits_carve(base, 1, model_dim);
+    b->xd_q = pg_xdigits_carve(base + o_q, 1, q_dim);
+    b->xd_f = pg_xdigits_carve(base + o_f, 1, ffn_dim);
+    const void **tab = reinterpret_cast<const void **>(base + o_tab);
+    b->qs_kv = reinterpret_cast<const uint8_t *const *>(tab);
+    b->d_kv = reinterpret_cast<const uint16_t *const *>(tab + 2);
+    b->qs_gu = reinterpret_cast<const uint8_t *const *>(tab + 4);
+    b->d_gu = reinterpret_cast<const uint16_t *const *>(tab + 6);
+    b->item_ids = reinterpret_cast<const int *>(tab + 8);
     *out = b;
     return PG_OK;
 }
@@ -707,6 +906,7 @@ PG_API void pg_llama_block_free(pg_ctx *ctx, pg_llama_block *b) {
     pg_rope_free(ctx, b->rope);
     if (b->attn_norm_w) (void)hipFree(b->attn_norm_w);
     if (b->arena) (void)hipFree(b->arena);
+    if (b->dec) (void)hipFree(b->dec);
     delete b;
 }
 
@@ -731,9 +931,71 @@ PG_API pg_status pg_llama_block_set_weights(pg_ctx *ctx, pg_llama_block *b, cons
     PG_CHECK_ARG(attn_norm_w && ffn_norm_w, "pg_llama_block_set_weights: null norm weights");
     PG_HIP(hipMemcpyAsync(b->attn_norm_w, attn_norm_w, b->d * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
     PG_HIP(hipMemcpyAsync(b->ffn_norm_w, ffn_norm_w, b->d * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    // tables for the two-item launches: {k, v} and {gate, up}, then the item ids {0, 1}
+    struct { const void *p[8]; int ids[2]; } tab = {{w[1]->qs, w[2]->qs, w[1]->d, w[2]->d, w[4]->qs, w[5]->qs, w[4]->d, w[5]->d}, {0, 1}};
+    PG_HIP(hipMemcpyAsync(const_cast<uint8_t **>(b->qs_kv), &tab, sizeof(tab), hipMemcpyHostToDevice, ctx->stream));
     PG_HIP(hipStreamSynchronize(ctx->stream));
     for (int i = 0; i < 7; ++i) b->w[i] = w[i];
+    auto kind = [](const pg_gguf_tensor *t) { return t->ggml_type == PG_GGML_Q4_0 ? PG_GGML_Q4_0 : PG_GGML_Q8_0; };
+    b->digit_kind = kind(w[0]);
+    for (int i = 1; i < 7; ++i)
+        if (kind(w[i]) != b->digit_kind) b->digit_kind = 0;
     return PG_OK;
+}
+
+// The one-token step: every producer of a GEMV input writes digits instead of f32 (RMSNorm,
+// the attention merge, SiLU·up), k/v and gate/up each run as one two-item launch, and the
+// second residual add is the down projection's epilogue: 11 launches instead of 18.
+static pg_status block_forward_one_token(pg_ctx *ctx, pg_llama_block *b, const float *h_dev, pg_kv_cache *cache,
+                                         float *out_dev) {
+    const size_t d = b->d, hd = b->hd, q_dim = b->nqh * hd, kv_dim = b->nkvh * hd, ffn = b->ffn, offset = cache->len;
+    auto slot = [](size_t n) { return pg_round_up(n, 64); };
+    const size_t cap = b->seq_cap;
+    float *p = b->arena;
+    auto take = [&](size_t n) { float *r = p; p += slot(n); return r; };
+    float *normed = take(cap * d), *h1 = take(cap * d), *proj = take(cap * d);
+    float *qd = take(cap * q_dim), *q_rope = take(cap * q_dim), *attn = take(cap * q_dim);
+    (void)normed; (void)proj;
+    // k|v and g|u as adjacent rows: item i of a two-item launch writes y + i * n_out
+    float *kd = take(2 * cap * kv_dim), *vd = kd + kv_dim;
+    float *g = take(2 * cap * ffn), *u = g + ffn;
+    const int kind = b->digit_kind;
+    const pg_gemv_batch one = {1, nullptr, nullptr, nullptr, 1};
+    const pg_gemv_batch kv2 = {2, b->qs_kv, b->d_kv, b->item_ids, 2}, gu2 = {2, b->qs_gu, b->d_gu, b->item_ids, 2};
+    const bool kv_same = b->w[1]->ggml_type == b->w[2]->ggml_type, gu_same = b->w[4]->ggml_type == b->w[5]->ggml_type;
+
+    PG_TRY(launch_rmsnorm_digits(ctx, h_dev, nullptr, nullptr, b->attn_norm_w, b->eps, 1, d, kind, b->xd_d));
+    PG_TRY(pg_launch_gguf_gemv(ctx, b->w[0]->ggml_type, q_dim, d, b->w[0]->qs, b->w[0]->d, one, b->xd_d, qd));
+    if (kv_same) {
+        PG_TRY(pg_launch_gguf_gemv(ctx, b->w[1]->ggml_type, kv_dim, d, nullptr, nullptr, kv2, b->xd_d, kd));
+    } else {
+        PG_TRY(pg_launch_gguf_gemv(ctx, b->w[1]->ggml_type, kv_dim, d, b->w[1]->qs, b->w[1]->d, one, b->xd_d, kd));
+        PG_TRY(pg_launch_gguf_gemv(ctx, b->w[2]->ggml_type, kv_dim, d, b->w[2]->qs, b->w[2]->d, one, b->xd_d, vd));
+    }
+    PG_TRY(cache_reserve(ctx, cache, offset + 1));
+    rope_args ra = {};
+    ra.seg[0] = {qd, q_rope, q_dim, hd, (int)b->nqh, 1};
+    ra.seg[1] = {kd, cache->k + offset * hd, kv_dim, cache->capacity * hd, (int)b->nkvh, 1};
+    ra.seg[2] = {vd, cache->v + offset * hd, kv_dim, cache->capacity * hd, (int)b->nkvh, 0};
+    ra.cos_t = b->rope->cos_t; ra.sin_t = b->rope->sin_t; ra.hd = (int)hd; ra.pos0 = (int)offset; ra.nseg = 3;
+    PG_TRY(launch_rope(ctx, ra, 1, b->nqh + 2 * b->nkvh));
+    cache->len = offset + 1;
+    PG_TRY(launch_attention(ctx, q_rope, cache, cache, b->nqh, 1, 1.0f / sqrtf((float)hd), PG_MASK_CAUSAL, offset, 0, 0, 0.0f,
+                            attn, 0, &b->xd_q, kind));
+    // h1 = h + attn . Wo
+    PG_TRY(pg_launch_gguf_gemv(ctx, b->w[3]->ggml_type, d, q_dim, b->w[3]->qs, b->w[3]->d, one, b->xd_q, h1, h_dev));
+    PG_TRY(launch_rmsnorm_digits(ctx, h1, nullptr, nullptr, b->ffn_norm_w, b->eps, 1, d, kind, b->xd_d));
+    if (gu_same) {
+        PG_TRY(pg_launch_gguf_gemv(ctx, b->w[4]->ggml_type, ffn, d, nullptr, nullptr, gu2, b->xd_d, g));
+    } else {
+        PG_TRY(pg_launch_gguf_gemv(ctx, b->w[4]->ggml_type, ffn, d, b->w[4]->qs, b->w[4]->d, one, b->xd_d, g));
+        PG_TRY(pg_launch_gguf_gemv(ctx, b->w[5]->ggml_type, ffn, d, b->w[5]->qs, b->w[5]->d, one, b->xd_d, u));
+    }
+    auto *sw = kind == PG_GGML_Q4_0 ? swiglu_digits_kernel<true> : swiglu_digits_kernel<false>;
+    PG_TRY(pg_launch(ctx, "swiglu_digits", sw, dim3(blocks_for(ffn / 4)), dim3(256), 0, (const float4 *)g, (const float4 *)u,
+                     (int)(ffn / 4), b->xd_f.digits, b->xd_f.xs));
+    // out = h1 + act . Wd
+    return pg_launch_gguf_gemv(ctx, b->w[6]->ggml_type, d, ffn, b->w[6]->qs, b->w[6]->d, one, b->xd_f, out_dev, h1);
 }
 
 PG_API pg_status pg_llama_block_forward_dev(pg_ctx *ctx, pg_llama_block *b, const float *h_dev, size_t seq,
@@ -764,12 +1026,14 @@ PG_API pg_status pg_llama_block_forward_dev(pg_ctx *ctx, pg_llama_block *b, cons
         b->seq_cap = cap;
     }
     const size_t cap = b->seq_cap;
+    if (seq == 1 && b->digit_kind != 0 && hd % 32 == 0 && d <= 8192 && (uintptr_t)h_dev % 16 == 0)
+        return block_forward_one_token(ctx, b, h_dev, cache, out_dev);
     float *p = b->arena;
     auto take = [&](size_t n) { float *r = p; p += slot(n); return r; };
     float *normed = take(cap * d), *h1 = take(cap * d), *proj = take(cap * d);
     float *qd = take(cap * q_dim), *q_rope = take(cap * q_dim), *attn = take(cap * q_dim);
     float *kd = take(cap * kv_dim), *vd = take(cap * kv_dim);
-    float *g = take(cap * ffn), *u = take(cap * ffn);
+    float *g = take(cap * ffn), *u = take(cap * ffn);  // the one-token step relies on this order (k, v and g, u adjacent)
 
     PG_TRY(launch_rmsnorm(ctx, h_dev, nullptr, nullptr, b->attn_norm_w, b->eps, seq, d, normed));
     float *const qkv[3] = {qd, kd, vd};

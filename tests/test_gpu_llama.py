@@ -154,6 +154,16 @@ def test_gqa_attention_masks_and_logit_cap(ctx, orc):
     assert (out[:8] == v[0, 0]).all()
 
 
+def test_gqa_attention_many_rows(ctx, orc):
+    """Enough (token, head) rows to fill the chip without key splits: the long-chunk kernel, with
+    and without the causal cut of the key range."""
+    from peregrine_amd import llama
+    say("attention 8 heads x 70 tokens")
+    _attention_case(ctx, orc, 8, 2, 64, 70, 90, llama.AttentionMask.none(), None, 61)
+    _attention_case(ctx, orc, 8, 2, 64, 70, 90, llama.AttentionMask.causal(20), None, 62)
+    _attention_case(ctx, orc, 8, 4, 32, 70, 90, llama.AttentionMask.causal_sliding_window(20, 7, 3), 2.0, 63)
+
+
 def test_gqa_attention_long_cache_splits_keys(ctx, orc):
     """A long cache under one query row: the keys are cut into many splits and merged."""
     from peregrine_amd import llama
