@@ -40,9 +40,11 @@ struct pg_llama_block {
     // device tables that let k/v and gate/up each run as one two-item launch.
     void *dec;                        // one allocation
     pg_xdigits xd_d, xd_q, xd_f;
-    const uint8_t *const *qs_kv, *const *qs_gu;
-    const uint16_t *const *d_kv, *const *d_gu;
-    const int *item_ids;              // {0, 1}
+    const uint8_t *const *qs_qkv, *const *qs_gu;   // q cut into kv_dim-row items, then k, v; gate, up
+    const uint16_t *const *d_qkv, *const *d_gu;
+    const int *item_ids;              // 0, 1, 2, ...
+    int qkv_items;                    // num_q_heads / num_kv_heads + 2
+    unsigned *tickets;                // one arrival counter per query head, zero between launches
     int digit_kind;                   // PG_GGML_Q4_0 (nibble digits), PG_GGML_Q8_0 (byte digits), 0 = mixed: no fused step
 };
 
@@ -873,11 +875,17 @@ PG_API pg_status pg_llama_block_create(pg_ctx *ctx, size_t model_dim, size_t num
         return st;
     }
     b->ffn_norm_w = b->attn_norm_w + model_dim;
-    // one-token step buffers: three digit sets, then the pointer tables and the item ids
+    // one-token step buffers: three digit sets, then the pointer tables, the item ids and the
+    // attention arrival counters
     const size_t q_dim = num_q_heads * head_dim;
+    const size_t items = num_q_heads / num_kv_heads + 2;
     const size_t o_q = pg_xdigits_bytes(1, model_dim), o_f = o_q + pg_xdigits_bytes(1, q_dim);
     const size_t o_tab = o_f + pg_xdigits_bytes(1, ffn_dim);
-    hipError_t e = hipMalloc(&b->dec, o_tab + 256);
+    const size_t tab_bytes = pg_round_up((2 * items + 4) * sizeof(void *) + items * sizeof(int), 256);
+    const size_t total = o_tab + tab_bytes + pg_round_up(num_q_heads * sizeof(unsigned), 256);
+    hipError_t e = hipMalloc(&b->dec, total);
+    if (e == hipSuccess) e = hipMemsetAsync(b->dec, 0, total, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
         st = pg_fail(PG_ENOMEM, "pg_llama_block_create: %s", hipGetErrorString(e));
         pg_llama_block_free(ctx, b);
@@ -888,11 +896,13 @@ PG_API pg_status pg_llama_block_create(pg_ctx *ctx, size_t model_dim, size_t num
     b->xd_q = pg_xdigits_carve(base + o_q, 1, q_dim);
     b->xd_f = pg_xdigits_carve(base + o_f, 1, ffn_dim);
     const void **tab = reinterpret_cast<const void **>(base + o_tab);
-    b->qs_kv = reinterpret_cast<const uint8_t *const *>(tab);
-    b->d_kv = reinterpret_cast<const uint16_t *const *>(tab + 2);
-    b->qs_gu = reinterpret_cast<const uint8_t *const *>(tab + 4);
-    b->d_gu = reinterpret_cast<const uint16_t *const *>(tab + 6);
-    b->item_ids = reinterpret_cast<const int *>(tab + 8);
+    b->qkv_items = (int)items;
+    b->qs_qkv = reinterpret_cast<const uint8_t *const *>(tab);
+    b->d_qkv = reinterpret_cast<const uint16_t *const *>(tab + items);
+    b->qs_gu = reinterpret_cast<const uint8_t *const *>(tab + 2 * items);
+    b->d_gu = reinterpret_cast<const uint16_t *const *>(tab + 2 * items + 2);
+    b->item_ids = reinterpret_cast<const int *>(tab + 2 * items + 4);
+    b->tickets = reinterpret_cast<unsigned *>(base + o_tab + tab_bytes);
     *out = b;
     return PG_OK;
 }
@@ -931,9 +941,28 @@ PG_API pg_status pg_llama_block_set_weights(pg_ctx *ctx, pg_llama_block *b, cons
     PG_CHECK_ARG(attn_norm_w && ffn_norm_w, "pg_llama_block_set_weights: null norm weights");
     PG_HIP(hipMemcpyAsync(b->attn_norm_w, attn_norm_w, b->d * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
     PG_HIP(hipMemcpyAsync(b->ffn_norm_w, ffn_norm_w, b->d * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
-    // tables for the two-item launches: {k, v} and {gate, up}, then the item ids {0, 1}
-    struct { const void *p[8]; int ids[2]; } tab = {{w[1]->qs, w[2]->qs, w[1]->d, w[2]->d, w[4]->qs, w[5]->qs, w[4]->d, w[5]->d}, {0, 1}};
-    PG_HIP(hipMemcpyAsync(const_cast<uint8_t **>(b->qs_kv), &tab, sizeof(tab), hipMemcpyHostToDevice, ctx->stream));
+    // Tables for the multi-item launches.  An item is kv_dim weight rows: q contributes
+    // num_q_heads / num_kv_heads of them (row offsets into its planes: 16 or 32 quant bytes and
+    // one scale per block, scales in tiles of 8 rows), then k, then v; gate and up are one each.
+    {
+        const size_t items = (size_t)b->qkv_items, nb = b->d / 32;
+        const size_t qb = w[0]->ggml_type == PG_GGML_Q4_0 ? 16 : 32;
+        std::vector<const void *> ptrs(2 * items + 4);
+        for (size_t i = 0; i + 2 < items; ++i) {
+            ptrs[i] = w[0]->qs + i * kv_dim * nb * qb;
+            ptrs[items + i] = w[0]->d + i * kv_dim * nb;  // (kv_dim / 8) tiles x nb blocks x 8 scales
+        }
+        ptrs[items - 2] = w[1]->qs; ptrs[items - 1] = w[2]->qs;
+        ptrs[2 * items - 2] = w[1]->d; ptrs[2 * items - 1] = w[2]->d;
+        ptrs[2 * items] = w[4]->qs; ptrs[2 * items + 1] = w[5]->qs;
+        ptrs[2 * items + 2] = w[4]->d; ptrs[2 * items + 3] = w[5]->d;
+        std::vector<int> ids(items);
+        for (size_t i = 0; i < items; ++i) ids[i] = (int)i;
+        PG_HIP(hipMemcpyAsync(const_cast<uint8_t **>(b->qs_qkv), ptrs.data(), ptrs.size() * sizeof(void *), hipMemcpyHostToDevice,
+                              ctx->stream));
+        PG_HIP(hipMemcpyAsync(const_cast<int *>(b->item_ids), ids.data(), items * sizeof(int), hipMemcpyHostToDevice, ctx->stream));
+        PG_HIP(hipStreamSynchronize(ctx->stream));  // the vectors die with this scope
+    }
     PG_HIP(hipStreamSynchronize(ctx->stream));
     for (int i = 0; i < 7; ++i) b->w[i] = w[i];
     auto kind = [](const pg_gguf_tensor *t) { return t->ggml_type == PG_GGML_Q4_0 ? PG_GGML_Q4_0 : PG_GGML_Q8_0; };
@@ -954,21 +983,25 @@ static pg_status block_forward_one_token(pg_ctx *ctx, pg_llama_block *b, const f
     float *p = b->arena;
     auto take = [&](size_t n) { float *r = p; p += slot(n); return r; };
     float *normed = take(cap * d), *h1 = take(cap * d), *proj = take(cap * d);
-    float *qd = take(cap * q_dim), *q_rope = take(cap * q_dim), *attn = take(cap * q_dim);
-    (void)normed; (void)proj;
-    // k|v and g|u as adjacent rows: item i of a two-item launch writes y + i * n_out
-    float *kd = take(2 * cap * kv_dim), *vd = kd + kv_dim;
+    float *unused_q = take(cap * q_dim), *q_rope = take(cap * q_dim), *attn = take(cap * q_dim);
+    (void)normed; (void)proj; (void)unused_q;
+    float *kv_gap = take(cap * kv_dim), *kv_gap2 = take(cap * kv_dim);
+    (void)kv_gap; (void)kv_gap2;
     float *g = take(2 * cap * ffn), *u = g + ffn;
+    // q|k|v and g|u as adjacent rows: item i of a multi-item launch writes y + i * n_out
+    float *qkv = take(cap * (q_dim + 2 * kv_dim) + 128), *qd = qkv, *kd = qkv + q_dim, *vd = kd + kv_dim;
     const int kind = b->digit_kind;
     const pg_gemv_batch one = {1, nullptr, nullptr, nullptr, 1};
-    const pg_gemv_batch kv2 = {2, b->qs_kv, b->d_kv, b->item_ids, 2}, gu2 = {2, b->qs_gu, b->d_gu, b->item_ids, 2};
-    const bool kv_same = b->w[1]->ggml_type == b->w[2]->ggml_type, gu_same = b->w[4]->ggml_type == b->w[5]->ggml_type;
+    const pg_gemv_batch qkv_n = {b->qkv_items, b->qs_qkv, b->d_qkv, b->item_ids, b->qkv_items};
+    const pg_gemv_batch gu2 = {2, b->qs_gu, b->d_gu, b->item_ids, 2};
+    const bool qkv_same = b->w[0]->ggml_type == b->w[1]->ggml_type && b->w[1]->ggml_type == b->w[2]->ggml_type && kv_dim % 8 == 0;
+    const bool gu_same = b->w[4]->ggml_type == b->w[5]->ggml_type;
 
     PG_TRY(launch_rmsnorm_digits(ctx, h_dev, nullptr, nullptr, b->attn_norm_w, b->eps, 1, d, kind, b->xd_d));
-    PG_TRY(pg_launch_gguf_gemv(ctx, b->w[0]->ggml_type, q_dim, d, b->w[0]->qs, b->w[0]->d, one, b->xd_d, qd));
-    if (kv_same) {
-        PG_TRY(pg_launch_gguf_gemv(ctx, b->w[1]->ggml_type, kv_dim, d, nullptr, nullptr, kv2, b->xd_d, kd));
+    if (qkv_same) {
+        PG_TRY(pg_launch_gguf_gemv(ctx, b->w[0]->ggml_type, kv_dim, d, nullptr, nullptr, qkv_n, b->xd_d, qkv));
     } else {
+        PG_TRY(pg_launch_gguf_gemv(ctx, b->w[0]->ggml_type, q_dim, d, b->w[0]->qs, b->w[0]->d, one, b->xd_d, qd));
         PG_TRY(pg_launch_gguf_gemv(ctx, b->w[1]->ggml_type, kv_dim, d, b->w[1]->qs, b->w[1]->d, one, b->xd_d, kd));
         PG_TRY(pg_launch_gguf_gemv(ctx, b->w[2]->ggml_type, kv_dim, d, b->w[2]->qs, b->w[2]->d, one, b->xd_d, vd));
     }
@@ -1017,7 +1050,8 @@ PG_API pg_status pg_llama_block_forward_dev(pg_ctx *ctx, pg_llama_block *b, cons
     auto slot = [](size_t n) { return pg_round_up(n, 64); };
     if (seq > b->seq_cap) {
         const size_t cap = seq > 2 * b->seq_cap ? seq : 2 * b->seq_cap;
-        const size_t floats = 3 * slot(cap * d) + 3 * slot(cap * q_dim) + 2 * slot(cap * kv_dim) + 2 * slot(cap * ffn);
+        const size_t floats = 3 * slot(cap * d) + 3 * slot(cap * q_dim) + 2 * slot(cap * kv_dim) + 2 * slot(cap * ffn) +
+                              slot(cap * (q_dim + 2 * kv_dim) + 128);  // the last term: q|k|v adjacent for the one-token step
         PG_HIP(hipStreamSynchronize(ctx->stream));
         if (b->arena) (void)hipFree(b->arena);
         b->arena = nullptr;
