@@ -149,12 +149,41 @@ ORC_API void orc_gqa_attention(const float *q, const float *k, const float *v, s
  *   [nkv, capacity, hd] holding cache_len positions on entry, cache_len + seq on return
  *   (the caller owns capacity >= cache_len + seq).  out [seq, d].  Returns 0, or -1 on
  *   allocation failure. */
+static int block_forward_types(const float *h, size_t seq, size_t d, size_t nqh, size_t nkvh, size_t hd, size_t ffn,
+                               const int *ggml_types, const uint8_t *wq, const uint8_t *wk, const uint8_t *wv,
+                               const uint8_t *wo, const uint8_t *wg, const uint8_t *wu, const uint8_t *wd,
+                               const float *attn_norm_w, const float *ffn_norm_w, float rms_eps, const float *cos_t,
+                               const float *sin_t, float *k_cache, float *v_cache, size_t cache_len, size_t capacity,
+                               float *out);
+
 ORC_API int orc_llama_block_forward(const float *h, size_t seq, size_t d, size_t nqh, size_t nkvh, size_t hd, size_t ffn,
                                     int ggml_type, const uint8_t *wq, const uint8_t *wk, const uint8_t *wv,
                                     const uint8_t *wo, const uint8_t *wg, const uint8_t *wu, const uint8_t *wd,
                                     const float *attn_norm_w, const float *ffn_norm_w, float rms_eps,
                                     const float *cos_t, const float *sin_t, float *k_cache, float *v_cache,
                                     size_t cache_len, size_t capacity, float *out) {
+    const int types[7] = {ggml_type, ggml_type, ggml_type, ggml_type, ggml_type, ggml_type, ggml_type};
+    return block_forward_types(h, seq, d, nqh, nkvh, hd, ffn, types, wq, wk, wv, wo, wg, wu, wd, attn_norm_w, ffn_norm_w, rms_eps,
+                               cos_t, sin_t, k_cache, v_cache, cache_len, capacity, out);
+}
+
+/* The same with one GGML type per projection (q, k, v, o, gate, up, down). */
+ORC_API int orc_llama_block_forward_types(const float *h, size_t seq, size_t d, size_t nqh, size_t nkvh, size_t hd,
+                                          size_t ffn, const int *ggml_types, const uint8_t *wq, const uint8_t *wk,
+                                          const uint8_t *wv, const uint8_t *wo, const uint8_t *wg, const uint8_t *wu,
+                                          const uint8_t *wd, const float *attn_norm_w, const float *ffn_norm_w,
+                                          float rms_eps, const float *cos_t, const float *sin_t, float *k_cache,
+                                          float *v_cache, size_t cache_len, size_t capacity, float *out) {
+    return block_forward_types(h, seq, d, nqh, nkvh, hd, ffn, ggml_types, wq, wk, wv, wo, wg, wu, wd, attn_norm_w, ffn_norm_w,
+                               rms_eps, cos_t, sin_t, k_cache, v_cache, cache_len, capacity, out);
+}
+
+static int block_forward_types(const float *h, size_t seq, size_t d, size_t nqh, size_t nkvh, size_t hd, size_t ffn,
+                               const int *ty, const uint8_t *wq, const uint8_t *wk, const uint8_t *wv,
+                               const uint8_t *wo, const uint8_t *wg, const uint8_t *wu, const uint8_t *wd,
+                               const float *attn_norm_w, const float *ffn_norm_w, float rms_eps, const float *cos_t,
+                               const float *sin_t, float *k_cache, float *v_cache, size_t cache_len, size_t capacity,
+                               float *out) {
     const size_t q_dim = nqh * hd, kv_dim = nkvh * hd;
     float *normed = (float *)malloc(seq * d * sizeof(float));
     float *qd = (float *)malloc(seq * q_dim * sizeof(float)), *kd = (float *)malloc(seq * kv_dim * sizeof(float));
@@ -165,9 +194,9 @@ ORC_API int orc_llama_block_forward(const float *h, size_t seq, size_t d, size_t
     int rc = -1;
     if (normed && qd && kd && vd && q_rope && attn && proj && h1 && g && u) {
         orc_rmsnorm(h, seq, d, attn_norm_w, rms_eps, normed);
-        rc = orc_gguf_matmul(normed, seq, wq, ggml_type, q_dim, d, qd);
-        if (!rc) rc = orc_gguf_matmul(normed, seq, wk, ggml_type, kv_dim, d, kd);
-        if (!rc) rc = orc_gguf_matmul(normed, seq, wv, ggml_type, kv_dim, d, vd);
+        rc = orc_gguf_matmul(normed, seq, wq, ty[0], q_dim, d, qd);
+        if (!rc) rc = orc_gguf_matmul(normed, seq, wk, ty[1], kv_dim, d, kd);
+        if (!rc) rc = orc_gguf_matmul(normed, seq, wv, ty[2], kv_dim, d, vd);
         if (!rc) {
             /* RoPE into head-major [heads, seq, hd]; K and V straight into the cache rows */
             for (size_t hh = 0; hh < nqh; ++hh)
@@ -182,13 +211,13 @@ ORC_API int orc_llama_block_forward(const float *h, size_t seq, size_t d, size_t
                 }
             orc_gqa_attention(q_rope, k_cache, v_cache, cache_len + seq, capacity, nqh, nkvh, seq, hd,
                               1.0f / sqrtf((float)hd), 1, cache_len, 0, 0, 0.0f, attn);
-            rc = orc_gguf_matmul(attn, seq, wo, ggml_type, d, q_dim, proj);
+            rc = orc_gguf_matmul(attn, seq, wo, ty[3], d, q_dim, proj);
         }
         if (!rc) {
             for (size_t i = 0; i < seq * d; ++i) h1[i] = h[i] + proj[i];
             orc_rmsnorm(h1, seq, d, ffn_norm_w, rms_eps, normed);
-            rc = orc_gguf_matmul(normed, seq, wg, ggml_type, ffn, d, g);
-            if (!rc) rc = orc_gguf_matmul(normed, seq, wu, ggml_type, ffn, d, u);
+            rc = orc_gguf_matmul(normed, seq, wg, ty[4], ffn, d, g);
+            if (!rc) rc = orc_gguf_matmul(normed, seq, wu, ty[5], ffn, d, u);
         }
         if (!rc) {
             for (size_t i = 0; i < seq * ffn; ++i) {
@@ -196,7 +225,7 @@ ORC_API int orc_llama_block_forward(const float *h, size_t seq, size_t d, size_t
                 const float silu = gi / (1.0f + expf(-gi));
                 g[i] = silu * u[i];
             }
-            rc = orc_gguf_matmul(g, seq, wd, ggml_type, d, ffn, proj);
+            rc = orc_gguf_matmul(g, seq, wd, ty[6], d, ffn, proj);
         }
         if (!rc)
             for (size_t i = 0; i < seq * d; ++i) out[i] = h1[i] + proj[i];

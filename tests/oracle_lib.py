@@ -207,8 +207,9 @@ def llama_block_forward(h, seq, d, nqh, nkvh, hd, ffn, ggml_type, weights, attn_
     updated in place ([nkvh, capacity, hd] float32 arrays).  Returns out [seq, d]."""
     keep = [np.frombuffer(bytes(b), np.uint8).copy() for b in weights]
     out = np.empty(seq * d, np.float32)
-    rc = lib.orc_llama_block_forward(_p(_f32(h).reshape(-1)), _sz(seq), _sz(d), _sz(nqh), _sz(nkvh), _sz(hd), _sz(ffn),
-                                     C.c_int(ggml_type), *[_p(a) for a in keep], _p(_f32(attn_norm_w)),
+    types = np.asarray([ggml_type] * 7 if np.isscalar(ggml_type) else ggml_type, np.int32)   # one type, or one per projection
+    rc = lib.orc_llama_block_forward_types(_p(_f32(h).reshape(-1)), _sz(seq), _sz(d), _sz(nqh), _sz(nkvh), _sz(hd), _sz(ffn),
+                                     _p(types), *[_p(a) for a in keep], _p(_f32(attn_norm_w)),
                                      _p(_f32(ffn_norm_w)), C.c_float(eps), _p(cos), _p(sin), _p(k_cache), _p(v_cache),
                                      _sz(cache_len), _sz(capacity), _p(out))
     assert rc == 0, rc
