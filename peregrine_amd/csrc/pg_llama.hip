@@ -402,6 +402,159 @@ __global__ __launch_bounds__(256) void gqa_attention_short_kernel(attn_args aa) 
     }
 }
 
+// ---- many query rows (prefill): tiled, online softmax ----------------------------------------
+// One (token, head) row per workgroup makes every row stream all of its keys and values again
+// and spends most instructions on cross-lane sums.  Here a workgroup owns 32 query rows that
+// read the SAME kv head (the heads of a group, then consecutive tokens), eight per wavefront,
+// and walks the keys in blocks of 64 staged through LDS:
+//   scores   lane = key: the lane walks its key row (LDS, row stride HD + 4 floats: conflict
+//            free 128-bit reads) against the eight query rows (LDS broadcast reads): no
+//            cross-lane traffic at all, 32 FMAs per 9 LDS reads;
+//   softmax  online (running maximum and sum per row, accumulators rescaled), the only
+//            cross-lane work: two wavefront reductions per row and block;
+//   P.V      lane = HD/64 output dims: probabilities read back four keys at a time as
+//            broadcasts, value rows as coalesced LDS reads.
+// K and V share one LDS buffer (K staged, scores, V staged, P.V); the next tile is fetched into
+// registers while the current one is used.  Any cache length, no key splits.
+__device__ __forceinline__ float wave_max_f32(float v) {
+    auto dpp_max = [](float x, auto ctrl) {
+        const int y = __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, false);
+        return fmaxf(x, __builtin_bit_cast(float, y));
+    };
+    v = dpp_max(v, std::integral_constant<int, 0xB1>{});
+    v = dpp_max(v, std::integral_constant<int, 0x4E>{});
+    v = dpp_max(v, std::integral_constant<int, 0x141>{});
+    v = dpp_max(v, std::integral_constant<int, 0x140>{});
+    const int b = __builtin_bit_cast(int, v);
+    return fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)), __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16))),
+                 fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)), __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48))));
+}
+
+constexpr int ATT_T_ROWS = 32, ATT_T_RW = 8, ATT_T_KB = 64;
+template <int HD> constexpr size_t att_tiled_lds() { return (size_t)(ATT_T_ROWS * HD + ATT_T_KB * (HD + 4) + 4 * ATT_T_RW * ATT_T_KB) * sizeof(float); }
+
+template <int HD>
+__global__ __launch_bounds__(256) void gqa_attention_tiled_kernel(attn_args aa) {
+    constexpr int ROWS = ATT_T_ROWS, RW = ATT_T_RW, KB = ATT_T_KB, KS = HD + 4, DPL = HD / 64, C4 = HD / 4;
+    constexpr int TPT = KB * C4 / 256;  // float4 of a staged tile per thread
+    extern __shared__ float lds[];
+    float *q_l = lds, *kv_l = q_l + ROWS * HD, *p_l = kv_l + KB * KS;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kvh = blockIdx.y, G = aa.group, row0 = blockIdx.x * ROWS, nrows = G * aa.seq_q;  // row index = qt * G + g
+    auto row_qt = [&](int row) { return min(row, nrows - 1) / G; };
+    auto row_qh = [&](int row) { return kvh * G + min(row, nrows - 1) % G; };
+    // query rows -> LDS (rows past the end repeat the last one and are not stored)
+    for (int idx = tid; idx < ROWS * C4; idx += 256) {
+        const int i = idx / C4, c = idx - i * C4, row = row0 + i;
+        reinterpret_cast<float4 *>(q_l)[idx] =
+            *reinterpret_cast<const float4 *>(aa.q + ((size_t)row_qh(row) * aa.seq_q + row_qt(row)) * HD + 4 * c);
+    }
+    int qt_of[RW];
+#pragma unroll
+    for (int r = 0; r < RW; ++r) qt_of[r] = row_qt(row0 + wave * RW + r);
+    int kend = aa.len;
+    if (aa.mask_kind != 0) kend = min(kend, aa.offset + row_qt(row0 + ROWS - 1) + 1);
+    const int nblocks = (kend + KB - 1) / KB;
+    const float *kg = aa.kc + (size_t)kvh * aa.k_stride, *vg = aa.vc + (size_t)kvh * aa.v_stride;
+    auto fetch = [&](const float *base, int k0, float4 (&reg)[TPT]) {  // tile rows k0 .. k0+63, zeros past kend
+#pragma unroll
+        for (int i = 0; i < TPT; ++i) {
+            const int idx = tid + 256 * i, key = idx / C4, c = idx - key * C4;
+            reg[i] = float4{0.f, 0.f, 0.f, 0.f};
+            if (k0 + key < kend) reg[i] = *reinterpret_cast<const float4 *>(base + (size_t)(k0 + key) * HD + 4 * c);
+        }
+    };
+    auto stage = [&](const float4 (&reg)[TPT], int stride) {
+#pragma unroll
+        for (int i = 0; i < TPT; ++i) {
+            const int idx = tid + 256 * i, key = idx / C4, c = idx - key * C4;
+            *reinterpret_cast<float4 *>(kv_l + key * stride + 4 * c) = reg[i];
+        }
+    };
+    float m[RW], l[RW], o[RW][DPL];
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+        m[r] = -INFINITY;
+        l[r] = 0.f;
+#pragma unroll
+        for (int d = 0; d < DPL; ++d) o[r][d] = 0.f;
+    }
+    float4 kreg[TPT], vreg[TPT];
+    if (nblocks > 0) fetch(kg, 0, kreg);
+    for (int kb = 0; kb < nblocks; ++kb) {
+        const int k0 = kb * KB;
+        __syncthreads();  // the previous block's P.V has finished with kv_l (and, first time, q_l is written)
+        stage(kreg, KS);
+        fetch(vg, k0, vreg);
+        __syncthreads();
+        // scores of key k0 + lane against this wavefront's rows
+        float s[RW];
+#pragma unroll
+        for (int r = 0; r < RW; ++r) s[r] = 0.f;
+        const float *krow = kv_l + lane * KS, *qrow = q_l + wave * RW * HD;
+#pragma unroll 4
+        for (int c = 0; c < C4; ++c) {
+            const float4 k4 = *reinterpret_cast<const float4 *>(krow + 4 * c);
+#pragma unroll
+            for (int r = 0; r < RW; ++r) {
+                const float4 q4 = *reinterpret_cast<const float4 *>(qrow + r * HD + 4 * c);
+                s[r] += q4.x * k4.x + q4.y * k4.y + q4.z * k4.z + q4.w * k4.w;
+            }
+        }
+        __syncthreads();  // every wavefront has read K
+        stage(vreg, HD);
+        if (kb + 1 < nblocks) fetch(kg, k0 + KB, kreg);
+        // online softmax
+#pragma unroll
+        for (int r = 0; r < RW; ++r) {
+            float sv = -INFINITY;
+            if (k0 + lane < kend && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, qt_of[r], k0 + lane)) {
+                sv = s[r] * aa.scale;
+                if (aa.logit_cap > 0.f) sv = aa.logit_cap * tanhf(sv / aa.logit_cap);
+            }
+            const float m_new = fmaxf(m[r], wave_max_f32(sv));
+            const float alpha = m[r] == -INFINITY ? 1.0f : expf(m[r] - m_new);  // nothing accumulated yet: any factor
+            const float pv = sv == -INFINITY ? 0.f : expf(sv - m_new);
+            l[r] = l[r] * alpha + pg_wave_sum_f32(pv);
+#pragma unroll
+            for (int d = 0; d < DPL; ++d) o[r][d] *= alpha;
+            m[r] = m_new;
+            p_l[(wave * RW + r) * KB + lane] = pv;
+        }
+        __syncthreads();  // V is staged, the probabilities are written
+        const float *prow = p_l + wave * RW * KB;
+#pragma unroll 2
+        for (int k4 = 0; k4 < KB; k4 += 4) {
+            float4 p4[RW];
+#pragma unroll
+            for (int r = 0; r < RW; ++r) p4[r] = *reinterpret_cast<const float4 *>(prow + r * KB + k4);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float v[DPL];
+                const float *vrow = kv_l + (k4 + j) * HD + DPL * lane;
+                if constexpr (DPL == 1) v[0] = vrow[0];
+                else if constexpr (DPL == 2) { const float2 t = *reinterpret_cast<const float2 *>(vrow); v[0] = t.x; v[1] = t.y; }
+                else { const float4 t = *reinterpret_cast<const float4 *>(vrow); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+#pragma unroll
+                for (int r = 0; r < RW; ++r) {
+                    const float pj = j == 0 ? p4[r].x : (j == 1 ? p4[r].y : (j == 2 ? p4[r].z : p4[r].w));
+#pragma unroll
+                    for (int d = 0; d < DPL; ++d) o[r][d] += pj * v[d];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+        const int row = row0 + wave * RW + r;
+        if (row >= nrows) continue;
+        const float inv = l[r] > 0.f ? 1.0f / l[r] : 0.f;
+        float *dst = aa.out + ((size_t)(row / G) * aa.nqh + kvh * G + row % G) * HD + DPL * lane;
+#pragma unroll
+        for (int d = 0; d < DPL; ++d) dst[d] = aa.accumulate ? dst[d] + o[r][d] * inv : o[r][d] * inv;
+    }
+}
+
 constexpr int ATT_SPLITS_MAX = 2048;
 
 // Merge the splits of one (query token, query head) row: with M = max of the split maxima and
@@ -535,11 +688,15 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     // short kernel handles with every load in flight at once.
     const size_t rows = seq_q * nqh, keys_per_round = 256 / (size_t)lanes;
     size_t chunk, splits;
-    bool short_kernel = false;
+    bool short_kernel = false, tiled_kernel = false;
     if (rows < 2 * (size_t)ctx->num_cu && (len + ATT_SHORT_ROUNDS * keys_per_round - 1) / (ATT_SHORT_ROUNDS * keys_per_round) <= (size_t)ATT_SPLITS_MAX) {
         chunk = ATT_SHORT_ROUNDS * keys_per_round;
         splits = (len + chunk - 1) / chunk;
         short_kernel = true;
+    } else if (hd == 64 || hd == 128 || hd == 256) {
+        tiled_kernel = true;  // online softmax over key blocks: any length in one pass
+        splits = 1;
+        chunk = len;
     } else {
         splits = (len + ATT_CHUNK_MAX - 1) / ATT_CHUNK_MAX;
         chunk = pg_round_up((len + splits - 1) / splits, keys_per_round);
@@ -559,7 +716,19 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
         if (wgs >= (1ull << 31)) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: grid too large");
         PG_TRY(pg_launch(ctx, "gqa_attention_short", gqa_attention_short_kernel, dim3((unsigned)wgs), dim3(256), 0, aa));
     }
-    else
+    else if (tiled_kernel) {
+        const size_t G = nqh / kc->num_kv_heads, row_sets = (G * seq_q + ATT_T_ROWS - 1) / ATT_T_ROWS;
+        const dim3 grid_t((unsigned)row_sets, (unsigned)kc->num_kv_heads);
+        auto *kern = hd == 64 ? gqa_attention_tiled_kernel<64> : (hd == 128 ? gqa_attention_tiled_kernel<128> : gqa_attention_tiled_kernel<256>);
+        const size_t lds_t = hd == 64 ? att_tiled_lds<64>() : (hd == 128 ? att_tiled_lds<128>() : att_tiled_lds<256>());
+        static bool attr_done[3] = {false, false, false};
+        bool &done = attr_done[hd == 64 ? 0 : (hd == 128 ? 1 : 2)];
+        if (!done) {
+            PG_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_t));
+            done = true;
+        }
+        PG_TRY(pg_launch(ctx, "gqa_attention_tiled", kern, grid_t, dim3(256), lds_t, aa));
+    } else
         PG_TRY(pg_launch(ctx, "gqa_attention", gqa_attention_kernel, grid, dim3(256), (256 + ATT_RED + chunk) * sizeof(float), aa));
     if (splits > 1) {
         auto *kern = !xd ? gqa_combine_kernel<0> : (digit_kind == PG_GGML_Q4_0 ? gqa_combine_kernel<1> : gqa_combine_kernel<2>);
