@@ -408,8 +408,9 @@ __global__ __launch_bounds__(256) void gqa_attention_short_kernel(attn_args aa) 
 // read the SAME kv head (the heads of a group, then consecutive tokens), eight per wavefront,
 // and walks the keys in blocks of 64 staged through LDS:
 //   scores   lane = key: the lane walks its key row (LDS, row stride HD + 4 floats: conflict
-//            free 128-bit reads) against the eight query rows (LDS broadcast reads): no
-//            cross-lane traffic at all, 32 FMAs per 9 LDS reads;
+//            free 128-bit reads) against the eight query rows, which are wavefront-uniform
+//            and come in through scalar loads as FMA operands: no cross-lane traffic at all,
+//            32 FMAs per LDS read;
 //   softmax  online (running maximum and sum per row, accumulators rescaled), the only
 //            cross-lane work: two wavefront reductions per row and block;
 //   P.V      lane = HD/64 output dims: probabilities read back four keys at a time as
@@ -431,27 +432,28 @@ __device__ __forceinline__ float wave_max_f32(float v) {
 }
 
 constexpr int ATT_T_ROWS = 32, ATT_T_RW = 8, ATT_T_KB = 64;
-template <int HD> constexpr size_t att_tiled_lds() { return (size_t)(ATT_T_ROWS * HD + ATT_T_KB * (HD + 4) + 4 * ATT_T_RW * ATT_T_KB) * sizeof(float); }
+template <int HD> constexpr size_t att_tiled_lds() { return (size_t)(ATT_T_KB * (HD + 4) + 4 * ATT_T_RW * ATT_T_KB) * sizeof(float); }
 
 template <int HD>
 __global__ __launch_bounds__(256) void gqa_attention_tiled_kernel(attn_args aa) {
     constexpr int ROWS = ATT_T_ROWS, RW = ATT_T_RW, KB = ATT_T_KB, KS = HD + 4, DPL = HD / 64, C4 = HD / 4;
     constexpr int TPT = KB * C4 / 256;  // float4 of a staged tile per thread
     extern __shared__ float lds[];
-    float *q_l = lds, *kv_l = q_l + ROWS * HD, *p_l = kv_l + KB * KS;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float *kv_l = lds, *p_l = kv_l + KB * KS;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kvh = blockIdx.y, G = aa.group, row0 = blockIdx.x * ROWS, nrows = G * aa.seq_q;  // row index = qt * G + g
     auto row_qt = [&](int row) { return min(row, nrows - 1) / G; };
     auto row_qh = [&](int row) { return kvh * G + min(row, nrows - 1) % G; };
-    // query rows -> LDS (rows past the end repeat the last one and are not stored)
-    for (int idx = tid; idx < ROWS * C4; idx += 256) {
-        const int i = idx / C4, c = idx - i * C4, row = row0 + i;
-        reinterpret_cast<float4 *>(q_l)[idx] =
-            *reinterpret_cast<const float4 *>(aa.q + ((size_t)row_qh(row) * aa.seq_q + row_qt(row)) * HD + 4 * c);
-    }
+    // The eight query rows of this wavefront are the same for all of its lanes: they are read
+    // through wavefront-uniform addresses (scalar loads), not staged (rows past the end repeat
+    // the last one and are not stored).
     int qt_of[RW];
+    const float *qrow[RW];
 #pragma unroll
-    for (int r = 0; r < RW; ++r) qt_of[r] = row_qt(row0 + wave * RW + r);
+    for (int r = 0; r < RW; ++r) {
+        qt_of[r] = row_qt(row0 + wave * RW + r);
+        qrow[r] = aa.q + ((size_t)row_qh(row0 + wave * RW + r) * aa.seq_q + qt_of[r]) * HD;
+    }
     int kend = aa.len;
     if (aa.mask_kind != 0) kend = min(kend, aa.offset + row_qt(row0 + ROWS - 1) + 1);
     const int nblocks = (kend + KB - 1) / KB;
@@ -483,7 +485,7 @@ __global__ __launch_bounds__(256) void gqa_attention_tiled_kernel(attn_args aa) 
     if (nblocks > 0) fetch(kg, 0, kreg);
     for (int kb = 0; kb < nblocks; ++kb) {
         const int k0 = kb * KB;
-        __syncthreads();  // the previous block's P.V has finished with kv_l (and, first time, q_l is written)
+        __syncthreads();  // the previous block's P.V has finished with kv_l
         stage(kreg, KS);
         fetch(vg, k0, vreg);
         __syncthreads();
@@ -491,14 +493,14 @@ __global__ __launch_bounds__(256) void gqa_attention_tiled_kernel(attn_args aa) 
         float s[RW];
 #pragma unroll
         for (int r = 0; r < RW; ++r) s[r] = 0.f;
-        const float *krow = kv_l + lane * KS, *qrow = q_l + wave * RW * HD;
+        const float *krow = kv_l + lane * KS;
 #pragma unroll 4
         for (int c = 0; c < C4; ++c) {
             const float4 k4 = *reinterpret_cast<const float4 *>(krow + 4 * c);
 #pragma unroll
             for (int r = 0; r < RW; ++r) {
-                const float4 q4 = *reinterpret_cast<const float4 *>(qrow + r * HD + 4 * c);
-                s[r] += q4.x * k4.x + q4.y * k4.y + q4.z * k4.z + q4.w * k4.w;
+                const float4 q4 = *reinterpret_cast<const float4 *>(qrow[r] + 4 * c);
+                s[r] = fmaf(q4.w, k4.w, fmaf(q4.z, k4.z, fmaf(q4.y, k4.y, fmaf(q4.x, k4.x, s[r]))));  // the build does not contract a*b+c
             }
         }
         __syncthreads();  // every wavefront has read K
@@ -539,7 +541,7 @@ __global__ __launch_bounds__(256) void gqa_attention_tiled_kernel(attn_args aa) 
                 for (int r = 0; r < RW; ++r) {
                     const float pj = j == 0 ? p4[r].x : (j == 1 ? p4[r].y : (j == 2 ? p4[r].z : p4[r].w));
 #pragma unroll
-                    for (int d = 0; d < DPL; ++d) o[r][d] += pj * v[d];
+                    for (int d = 0; d < DPL; ++d) o[r][d] = fmaf(pj, v[d], o[r][d]);
                 }
             }
         }
