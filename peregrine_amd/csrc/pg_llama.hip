@@ -481,13 +481,12 @@ __global__ __launch_bounds__(256) void gqa_attention_tiled_kernel(attn_args aa) 
 #pragma unroll
         for (int d = 0; d < DPL; ++d) o[r][d] = 0.f;
     }
-    float4 kreg[TPT], vreg[TPT];
-    if (nblocks > 0) fetch(kg, 0, kreg);
+    float4 treg[TPT];
     for (int kb = 0; kb < nblocks; ++kb) {
         const int k0 = kb * KB;
         __syncthreads();  // the previous block's P.V has finished with kv_l
-        stage(kreg, KS);
-        fetch(vg, k0, vreg);
+        fetch(kg, k0, treg);
+        stage(treg, KS);
         __syncthreads();
         // scores of key k0 + lane against this wavefront's rows
         float s[RW];
@@ -504,8 +503,8 @@ __global__ __launch_bounds__(256) void gqa_attention_tiled_kernel(attn_args aa) 
             }
         }
         __syncthreads();  // every wavefront has read K
-        stage(vreg, HD);
-        if (kb + 1 < nblocks) fetch(kg, k0 + KB, kreg);
+        fetch(vg, k0, treg);
+        stage(treg, HD);
         // online softmax
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
