@@ -397,7 +397,7 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
         pg_gemv_batch batch = {(int)m, nullptr, nullptr, nullptr, 1};
         return pg_launch_gguf_gemv(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, batch, xd, y_dev);
     }
-    const int ks = pg_gguf_mm_splitk(ctx, w->n_out, w->k_in, 1, nullptr);
+    const int ks = pg_gguf_mm_splitk(ctx, w->n_out, w->k_in, (m + 31) / 32, nullptr);
     const size_t sz_d = pg_mmdigits_bytes(m, w->k_in);
     const size_t sz_part = ks > 1 ? pg_round_up((size_t)ks * m * w->n_out * sizeof(float), 256) : 0;
     PG_TRY(pg_workspace(ctx, sz_d + sz_part, &ws));
@@ -441,7 +441,7 @@ pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, c
     const size_t sz_d = pg_mmdigits_bytes(m, k_in);
     size_t sz_part = 0;
     for (int i = 0; i < count; ++i) {
-        const int ks = pg_gguf_mm_splitk(ctx, w[i]->n_out, k_in, 1, nullptr);
+        const int ks = pg_gguf_mm_splitk(ctx, w[i]->n_out, k_in, (m + 31) / 32, nullptr);
         const size_t sz = ks > 1 ? pg_round_up((size_t)ks * m * w[i]->n_out * sizeof(float), 256) : 0;
         if (sz > sz_part) sz_part = sz;
     }
@@ -454,7 +454,7 @@ pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, c
             PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, m, k_in, w[i]->ggml_type, md));
             digits_type = w[i]->ggml_type;
         }
-        const int ks = pg_gguf_mm_splitk(ctx, w[i]->n_out, k_in, 1, nullptr);
+        const int ks = pg_gguf_mm_splitk(ctx, w[i]->n_out, k_in, (m + 31) / 32, nullptr);
         PG_TRY(pg_launch_gguf_mm(ctx, w[i]->ggml_type, w[i]->n_out, k_in, w[i]->qs, w[i]->d, grp, m, md, y_dev[i],
                                  ks > 1 ? part_base : nullptr));
     }

@@ -134,10 +134,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l31 = lane & 31, hh = lane >> 5;
 
-    int e = 0, tt = blockIdx.y;
+    // Which 128 weight rows (bx) and which token tile (by).  With many token tiles (a prefill)
+    // the launch is one-dimensional and XCD-aware: workgroup id = 8 * j + xcd, and the j-th
+    // workgroup of an XCD is member j % 32 of super-tile (j / 32) * 8 + xcd, a super-tile being
+    // 4 row groups x 8 token tiles whose weights and digits (about 3 MB) stay in that XCD's L2
+    // while its 32 workgroups run: each weight row group is fetched once per 8 token tiles
+    // instead of once per tile.
+    int bx = blockIdx.x, by = blockIdx.y;
+    if (grp.remap_rg) {
+        const int nrgb = (grp.remap_rg + 3) / 4, ntb = (grp.remap_tiles + 7) / 8;
+        const int jj = blockIdx.x >> 3, st = (jj >> 5) * 8 + (blockIdx.x & 7), w = jj & 31;
+        if (st >= nrgb * ntb) return;
+        bx = (st % nrgb) * 4 + (w & 3);
+        by = (st / nrgb) * 8 + (w >> 2);
+        if (bx >= grp.remap_rg || by >= grp.remap_tiles) return;
+    }
+    int e = 0, tt = by;
     if (grp.counts) {
-        e = blockIdx.y / grp.tiles_per_expert;
-        tt = blockIdx.y - e * grp.tiles_per_expert;
+        e = by / grp.tiles_per_expert;
+        tt = by - e * grp.tiles_per_expert;
     }
     const int count = grp.counts ? grp.counts[e] : grp.max_count;
     if (tt * 32 >= count) return;  // the same for every thread of the workgroup
@@ -172,7 +187,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const float *xs_src = xs + xrow_of(8 * wave + (lane & 7)) * (size_t)nbp;
     // weights: fill q covers streams 16q .. 16q+15 (Q8_0: stream = 32*half + row, Q4_0: stream = row);
     // the lane fetches block (lane & 3) ^ swizzle of the stream's 4 blocks.
-    const int row0 = blockIdx.x * 128 + wave * 32;
+    const int row0 = bx * 128 + wave * 32;
     const int w_jb = (lane & 3) ^ ((lane >> 3) & 3);  // stream >> 1 = 8q + (lane >> 3)
     const int8_t *w_src[W_FILLS];
 #pragma unroll
@@ -398,11 +413,20 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
     const int nb = (int)(k_in / 32), nbp = (int)pg_round_up(nb, 4);
     const size_t experts = grp.counts ? (size_t)grp.num_experts : 1;
     int chunk = 0;
-    const int ks = pg_gguf_mm_splitk(ctx, n_out, k_in, experts, &chunk);
-    if (ks > 1 && !part) return pg_fail(PG_EINVAL, "gguf_mm: split-K needs a partial-sum buffer");
     const size_t gy = experts * (size_t)grp.tiles_per_expert;
+    // token tiles that certainly hold work: all of them without expert lists, one per expert with
+    const int ks = pg_gguf_mm_splitk(ctx, n_out, k_in, grp.counts ? experts : gy, &chunk);
+    if (ks > 1 && !part) return pg_fail(PG_EINVAL, "gguf_mm: split-K needs a partial-sum buffer");
     if (gy > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_mm: too many token tiles");
-    const dim3 grid(grid_for(n_out, 128), (unsigned)gy, (unsigned)ks);
+    dim3 grid(grid_for(n_out, 128), (unsigned)gy, (unsigned)ks);
+    pg_mm_group g2 = grp;
+    g2.remap_rg = g2.remap_tiles = 0;
+    if (!grp.counts && ks == 1 && gy >= 16) {  // a plain product over many token tiles: see the kernel
+        g2.remap_rg = (int)grid.x;
+        g2.remap_tiles = (int)gy;
+        const size_t supertiles = (size_t)((grid.x + 3) / 4) * ((gy + 7) / 8);
+        grid = dim3((unsigned)((supertiles + 7) / 8 * 8 * 32), 1, 1);
+    }
     float *dst = ks > 1 ? part : y;
     const size_t stride = total_pairs * n_out;
     const size_t lds = (size_t)RING * (ggml_type == PG_GGML_Q4_0 ? MMCfg<4>::STAGE : MMCfg<8>::STAGE);
@@ -414,7 +438,7 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
             if (e != hipSuccess) return pg_fail(PG_EDEVICE, "hipFuncSetAttribute: %s", hipGetErrorString(e));
             attr_done = true;
         }
-        return pg_launch(ctx, name, kern, grid, dim3(256), lds, qs, d, grp, (int)n_out, nb, nbp, chunk, md.digits, md.xs, dst,
+        return pg_launch(ctx, name, kern, grid, dim3(256), lds, qs, d, g2, (int)n_out, nb, nbp, chunk, md.digits, md.xs, dst,
                          stride);
     };
     if (ggml_type == PG_GGML_Q4_0) PG_TRY(launch(gguf_mm_kernel<4>, "gguf_mm_q4_0"));

@@ -219,8 +219,10 @@ struct pg_mm_group {
     int tiles_per_expert;
     int max_count;
     int x_row_div;
+    int remap_rg, remap_tiles;  // set by the launcher (row groups and token tiles of an XCD-aware 1-D launch), else 0
 };
-// Number of K chunks the product is split into (partial sums: [chunks][pairs][n_out] floats).
+// Number of K chunks the product is split into (partial sums: [chunks][pairs][n_out] floats);
+// `groups` = token tiles that certainly hold work (all tiles of a plain product, one per expert).
 int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t groups, int *chunk_out);
 pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,
                             const uint16_t *d, const pg_mm_group &grp, size_t total_pairs, const pg_mmdigits &md,

@@ -95,6 +95,8 @@ GGUF_SHAPES = [
     (8, 6144, 4096, 1),
     # more than one row: matrix-core path (token tiles of 32, row tiles of 128, split K)
     (2, 130, 224, 33), (8, 131, 160, 40), (2, 515, 4096, 64), (8, 257, 6144, 35), (2, 14336, 4096, 4), (8, 4096, 14336, 16),
+    # 16 token tiles and more: no split K, XCD-aware super-tiles of 4 row groups x 8 token tiles (ragged on both sides)
+    (2, 600, 256, 545), (8, 1100, 128, 700), (2, 128, 512, 512),
 ]
 
 
