@@ -503,5 +503,83 @@ private:
 };
 
 }  // namespace mxfp4
+
+namespace huffman {
+
+// HuffmanTable  src/huffman.rs:19-306 (index = value + 128).
+struct HuffmanTable {
+    std::vector<uint8_t> bit_lengths = std::vector<uint8_t>(256, 0);
+    std::vector<uint32_t> codes = std::vector<uint32_t>(256, 0);
+    static HuffmanTable from_frequencies(const std::vector<uint64_t> &freqs) {
+        if (freqs.size() != 256) throw Panic(PG_EINVAL, "HuffmanTable::from_frequencies: 256 frequencies expected");
+        HuffmanTable t;
+        check(pg_huffman_table_from_frequencies(freqs.data(), t.bit_lengths.data(), t.codes.data()), "HuffmanTable::from_frequencies");
+        return t;
+    }
+    static HuffmanTable from_bytes(const std::vector<uint8_t> &data) {
+        if (data.size() < 256) throw Panic(PG_EINVAL, "codebook too short");
+        HuffmanTable t;
+        t.bit_lengths.assign(data.begin(), data.begin() + 256);
+        check(pg_huffman_canonical_codes(t.bit_lengths.data(), t.codes.data()), "HuffmanTable::from_bytes");
+        return t;
+    }
+    std::vector<uint8_t> to_bytes() const { return bit_lengths; }
+    std::vector<uint8_t> encode(const std::vector<int8_t> &data) const {
+        size_t need = 0;
+        check(pg_huffman_encode(bit_lengths.data(), data.data(), data.size(), nullptr, 0, &need), "HuffmanTable::encode");
+        std::vector<uint8_t> out(need);
+        check(pg_huffman_encode(bit_lengths.data(), data.data(), data.size(), out.data(), out.size(), &need), "HuffmanTable::encode");
+        return out;
+    }
+    std::vector<int8_t> decode(const GpuContext &gpu, const std::vector<uint8_t> &bitstream, size_t num_symbols) const {
+        std::vector<int8_t> out(num_symbols);
+        check(pg_huffman_decode(gpu.raw(), bit_lengths.data(), bitstream.data(), bitstream.size(), num_symbols, out.data()),
+              "HuffmanTable::decode");
+        return out;
+    }
+};
+
+// HuffmanTensor  src/huffman.rs:311-435.
+class HuffmanTensor {
+public:
+    static HuffmanTensor from_quantized(const quant::QuantizedTensor &qt, size_t num_streams) {
+        pg_huffman_tensor *h = nullptr;
+        check(pg_huffman_tensor_from_quantized(qt.data_i8.data(), qt.scales.data(), qt.rows, qt.cols, num_streams, &h),
+              "HuffmanTensor::from_quantized");
+        return HuffmanTensor(h);
+    }
+    ~HuffmanTensor() { pg_huffman_tensor_free(h_); }
+    HuffmanTensor(HuffmanTensor &&o) noexcept : h_(o.h_) { o.h_ = nullptr; }
+    HuffmanTensor(const HuffmanTensor &) = delete;
+    HuffmanTensor &operator=(const HuffmanTensor &) = delete;
+    size_t rows() const { size_t r = 0; check(pg_huffman_tensor_info(h_, &r, nullptr, nullptr, nullptr), "HuffmanTensor"); return r; }
+    size_t cols() const { size_t c = 0; check(pg_huffman_tensor_info(h_, nullptr, &c, nullptr, nullptr), "HuffmanTensor"); return c; }
+    size_t compressed_size() const { size_t z = 0; check(pg_huffman_tensor_info(h_, nullptr, nullptr, nullptr, &z), "HuffmanTensor"); return z; }
+    size_t uncompressed_size() const { return rows() * cols() + cols() * 4; }
+    float compression_ratio() const { return (float)uncompressed_size() / (float)compressed_size(); }
+    quant::QuantizedTensor decode_to_quantized(const GpuContext &gpu) const {
+        quant::QuantizedTensor qt;
+        qt.rows = rows(); qt.cols = cols();
+        qt.data_i8.resize(qt.rows * qt.cols); qt.data_i8_t.resize(qt.rows * qt.cols); qt.scales.resize(qt.cols);
+        check(pg_huffman_tensor_decode_to_quantized(gpu.raw(), h_, qt.data_i8.data(), qt.data_i8_t.data(), qt.scales.data()),
+              "HuffmanTensor::decode_to_quantized");
+        return qt;
+    }
+    const pg_huffman_tensor *handle() const { return h_; }
+
+private:
+    explicit HuffmanTensor(pg_huffman_tensor *h) : h_(h) {}
+    pg_huffman_tensor *h_;
+};
+
+// matmul_huffman  src/huffman.rs:465-474.
+inline std::vector<float> matmul_huffman(const GpuContext &gpu, const std::vector<float> &a, size_t m, size_t k, const HuffmanTensor &ht) {
+    if (a.size() != m * k) throw Panic(PG_EINVAL, "matmul_huffman: a.len() != m * k");
+    std::vector<float> out(m * ht.cols());
+    check(pg_matmul_huffman(gpu.raw(), a.data(), m, k, ht.handle(), out.data()), "matmul_huffman");
+    return out;
+}
+
+}  // namespace huffman
 }  // namespace peregrine
 #endif  // PEREGRINE_HIP_HPP

@@ -267,6 +267,36 @@ static void test_llama_block(const GpuContext &gpu) {
     }
 }
 
+// tests/huffman_parity.rs:23-42: Huffman-coded weights give the same product as the plain
+// quantised ones (here: bit for bit), through a round trip of the coded tensor
+static void test_huffman_matmul(const GpuContext &gpu) {
+    std::printf("test_huffman_matmul\n");
+    const size_t shapes[4][3] = {{8, 32, 16}, {1, 64, 1}, {32, 128, 64}, {16, 256, 32}};
+    for (const auto &sh : shapes) {
+        const size_t m = sh[0], k = sh[1], n = sh[2];
+        uint32_t sa = 42, sw = 123;
+        auto lcg = [](uint32_t &st) { st = st * 1103515245u + 12345u; return (float)st / 4294967295.0f * 2.0f - 1.0f; };
+        std::vector<float> a(m * k), w(k * n);
+        for (auto &v : a) v = lcg(sa);
+        for (auto &v : w) v = lcg(sw);
+        auto qt = quant::quantize_weights(gpu, w, k, n);
+        auto ht = huffman::HuffmanTensor::from_quantized(qt, 4);
+        auto back = ht.decode_to_quantized(gpu);
+        EXPECT(back.data_i8 == qt.data_i8 && back.data_i8_t == qt.data_i8_t && same_bits(back.scales, qt.scales), "round trip m=%zu", m);
+        auto ref = quant::matmul_quantized(gpu, a, m, k, qt);
+        auto got = huffman::matmul_huffman(gpu, a, m, k, ht);
+        EXPECT(same_bits(ref, got), "matmul_huffman differs from matmul_quantized at M=%zu K=%zu N=%zu", m, k, n);
+    }
+    // src/huffman.rs:780-797: one symbol, 512 times, in at most 65 bytes
+    std::vector<uint64_t> freqs(256, 0);
+    freqs[42 + 128] = 512;
+    auto table = huffman::HuffmanTable::from_frequencies(freqs);
+    std::vector<int8_t> same(512, 42);
+    auto enc = table.encode(same);
+    EXPECT(enc.size() <= 65, "encoded %zu bytes", enc.size());
+    EXPECT(table.decode(gpu, enc, 512) == same, "one-symbol round trip");
+}
+
 int main() {
     try {
         GpuContext gpu(0);
@@ -280,6 +310,7 @@ int main() {
         test_block_weight_matmul(gpu);
         test_gqa_attention(gpu);
         test_llama_block(gpu);
+        test_huffman_matmul(gpu);
     } catch (const std::exception &e) {
         std::printf("FAIL: uncaught %s\n", e.what());
         return 2;
