@@ -72,6 +72,40 @@ def test_moe_grok_shaped_reduced(ctx, orc):
     H.assert_close_rel(got1, want1, MOE_RTOL, "single expert")
 
 
+def test_moe_full_size_equal_experts_property(ctx, orc):
+    """Benchmark configuration 5 at full width (d 6144, ffn 32768, 8 experts, top-2, 64 tokens,
+    Q8_0, SiLU), where the scalar oracle would run for minutes.  With all eight experts holding
+    the same weights the layer collapses to  out[t] = (p_1 + p_2) * expert(x[t]),  so routing,
+    pair lists, grouped products and the combine can be checked against three plain products
+    over the same tensors (the un-grouped path, itself held to the oracle at smaller sizes) and
+    the oracle's own softmax / top-k."""
+    from peregrine_amd import gguf, moe
+    T, d, ffn, E, top_k = 64, 6144, 32768, 8, 2
+    say("moe full size, equal experts")
+    rng = np.random.default_rng(50)
+    def blocks(n_out, k_in, scale):
+        b = np.empty((n_out * k_in // 32, 34), np.uint8)
+        b[:, 2:] = rng.integers(0, 256, size=(b.shape[0], 32), dtype=np.uint8)
+        b[:, :2] = np.frombuffer(np.float16(scale).tobytes(), np.uint8)
+        return b
+    wg = gguf.GgufWeight(blocks(ffn, d, 0.02 / 127).tobytes(), 8, ffn, d, ctx)
+    wu = gguf.GgufWeight(blocks(ffn, d, 0.02 / 127).tobytes(), 8, ffn, d, ctx)
+    wd = gguf.GgufWeight(blocks(d, ffn, 0.02 / 127).tobytes(), 8, d, ffn, ctx)
+    x = orc.rng_normal(6, T * d)
+    logits = orc.rng_normal(7, T * E).reshape(T, E)
+    ex = moe.MoEExperts([wg] * E, [wu] * E, [wd] * E, top_k, moe.SILU, ctx)
+    got = ex.forward(x, logits)
+    g = wg.matmul(x, T).reshape(T, ffn)
+    u = wu.matmul(x, T).reshape(T, ffn)
+    h = (g / (np.float32(1) + np.exp(-g)) * u).astype(np.float32)
+    y = wd.matmul(h, T).reshape(T, d)
+    probs = orc.softmax_rows(logits, T, E).reshape(T, E)            # the two largest, whichever experts they are
+    top = np.sort(probs, axis=1)[:, ::-1][:, :top_k]
+    want = top[:, :1] * y + top[:, 1:2] * y                           # out[t] += p * y in k order (examples/grok1/moe.rs:98-105)
+    for t in range(T):
+        H.assert_close_rel(got[t], want[t], 1e-3, f"token {t}")
+
+
 def test_moe_many_tokens_per_expert(ctx, orc):
     """More than 32 tokens reach one expert (two token tiles), another expert gets none, and the
     widths are not multiples of the kernel's 128-row / 4-block tiles."""
