@@ -167,9 +167,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int pr = grp.lists ? grp.lists[(size_t)e * grp.list_stride + slot_c] : slot_c;
         return (size_t)(pr / grp.x_row_div);
     };
-    // the token whose outputs this lane accumulates
-    const bool tok_ok = tt * 32 + l31 < count;
-    const int pair = tok_ok ? (grp.lists ? grp.lists[(size_t)e * grp.list_stride + tt * 32 + l31] : tt * 32 + l31) : 0;
+    // Orientation of the 32x32 result tile: TOKENS on the accumulator-register axis (register r
+    // of lanes with hh = lane/32 holds token slot 8*(r/4) + 4*hh + r%4), WEIGHT ROWS on the lanes.
+    // A tile with few tokens then needs only the first NR registers scaled and accumulated:
+    // NR = 4 covers 8 token slots, 8 covers 16, 16 all 32.
+    const int ntok = count - tt * 32 < 32 ? count - tt * 32 : 32;
 
     // Fill duties of this lane.
     // digits: fill n = 2*wave + u covers units 8n .. 8n+7, unit = 2*token + plane; the lane
@@ -235,15 +237,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // Split into three phases so that the full-stage path can overlap them across blocks.
     const int w_rd = OFF_W + wave * W_WAVE + (QT == 8 ? lane : l31) * 64, w_sw = ((QT == 8 ? lane : l31) >> 1) & 3;
     const int dig_rd = l31 * 256, dig_sw = l31 & 7;
+    const int d_rd = OFF_D + wave * 256 + (l31 >> 3) * 64 + (l31 & 7) * 2;  // this lane's weight row: [group of 8][j][8 f16]
     auto read_ab = [&](const char *base, int j, v4i (&ab)[3]) {
         ab[0] = *reinterpret_cast<const v4i *>(base + w_rd + ((j ^ w_sw) * 16));
         ab[1] = *reinterpret_cast<const v4i *>(base + dig_rd + (((2 * j + hh) ^ dig_sw) * 16));
         ab[2] = *reinterpret_cast<const v4i *>(base + dig_rd + 128 + (((2 * j + hh) ^ dig_sw) * 16));
     };
-    auto read_d = [&](const char *base, int j, v2i (&dd)[4]) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g)  // rows 8g + 4*hh + {0..3}  <->  accumulator registers 4g .. 4g+3
-            dd[g] = *reinterpret_cast<const v2i *>(base + OFF_D + wave * 256 + (g * 4 + j) * 16 + hh * 8);
+    // the block's weight scale of this lane's row
+    // (read as integers: a float-typed LDS read makes the compiler wait for every fill in flight)
+    auto read_d = [&](const char *base, int j, unsigned &dbits) {
+        dbits = *reinterpret_cast<const unsigned short *>(base + d_rd + j * 16);
     };
     auto mfmas = [&](const v4i (&ab)[3], v16i &ihi, v16i &ilo) {
         v4i a = ab[0];
@@ -254,35 +257,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         v16i zero;
 #pragma unroll
         for (int r = 0; r < 16; ++r) zero[r] = 0;
-        ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, ab[1], zero, 0, 0, 0);
-        ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, ab[2], zero, 0, 0, 0);
+        ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(ab[1], a, zero, 0, 0, 0);  // rows = tokens, columns = weight rows
+        ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(ab[2], a, zero, 0, 0, 0);
     };
-    auto scale_acc = [&](const v16i &ihi, const v16i &ilo, const v2i (&dd)[4], float sj) {
-        if constexpr (QT == 4) sj *= 0.0625f;  // the weight operand was 16 * (q - 8)
+    auto scale_acc = [&](auto nr, const v16i &ihi, const v16i &ilo, unsigned dbits, const int (&sx)[16][4], int j) {
+        float dv = half_bits_to_float(dbits);
+        if constexpr (QT == 4) dv *= 0.0625f;  // the weight operand was 16 * (q - 8)
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int r = 4 * g + q;
-                const uint32_t pairbits = (uint32_t)dd[g][q >> 1];
-                const float dv = half_bits_to_float((q & 1) ? pairbits >> 16 : pairbits & 0xFFFFu);
-                // |integer| < 2^31: rounded to 24 bits, then scaled (two roundings of 2^-24, far below the digit step)
-                const float fx = (float)(ihi[r] * 256 + ilo[r]) * sj;
-                acc[r] = fmaf(dv, fx, acc[r]);
-            }
+        for (int r = 0; r < decltype(nr)::value; ++r) {
+            // |integer| < 2^31: rounded to 24 bits, then scaled (two roundings of 2^-24, far below the digit step)
+            const float fx = (float)(ihi[r] * 256 + ilo[r]) * __int_as_float(sx[r][j]);
+            acc[r] = fmaf(dv, fx, acc[r]);
+        }
     };
-    auto compute = [&](auto ring_slot, int s) {
+    auto compute = [&](auto nr, auto ring_slot, int s) {
         const int b0 = b_begin + s * NBU;
         const char *base = lds + decltype(ring_slot)::value * STAGE;
-        // Read as integers: a float-typed LDS read makes the compiler wait for every LDS fill in
-        // flight (it cannot tell the stages apart), an int-typed one leaves the waits to us.
-        const v4i sxi = *reinterpret_cast<const v4i *>(base + OFF_XS + l31 * 16);
-        // (element -> named int -> float: a bit cast applied directly to a vector element
+        // activation scales of this lane's NR token slots for the stage's four blocks
+        // (vector element -> named int: a bit cast applied directly to a vector element
         // expression was compiled as a cast of element 0)
-        const int sx0 = sxi[0], sx1 = sxi[1], sx2 = sxi[2], sx3 = sxi[3];
-        const float sx[4] = {__int_as_float(sx0), __int_as_float(sx1), __int_as_float(sx2), __int_as_float(sx3)};
+        int sx[16][4];
+#pragma unroll
+        for (int r = 0; r < decltype(nr)::value; ++r) {
+            const v4i t = *reinterpret_cast<const v4i *>(base + OFF_XS + (8 * (r >> 2) + 4 * hh + (r & 3)) * 16);
+            const int t0 = t[0], t1 = t[1], t2 = t[2], t3 = t[3];
+            sx[r][0] = t0; sx[r][1] = t1; sx[r][2] = t2; sx[r][3] = t3;
+        }
         v4i ab[2][3];
-        v2i dd[2][4];
+        unsigned dd[2];
         v16i ihi[2], ilo[2];
         if (b0 + NBU <= b_end) {  // full stage (wavefront-uniform)
             // Software pipeline over the 4 blocks: while block j is scaled and accumulated on
@@ -301,7 +303,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 }
                 if (j + 2 < NBU) read_ab(base, j + 2, ab[j & 1]);
                 __builtin_amdgcn_sched_barrier(0);
-                scale_acc(ihi[j & 1], ilo[j & 1], dd[j & 1], sx[j]);
+                scale_acc(nr, ihi[j & 1], ilo[j & 1], dd[j & 1], sx, j);
                 __builtin_amdgcn_sched_barrier(0);
             }
         } else {
@@ -311,7 +313,87 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     read_ab(base, j, ab[0]);
                     read_d(base, j, dd[0]);
                     mfmas(ab[0], ihi[0], ilo[0]);
-                    scale_acc(ihi[0], ilo[0], dd[0], sx[j]);
+                    scale_acc(nr, ihi[0], ilo[0], dd[0], sx, j);
+                }
+        }
+    };
+
+    // ---- the other orientation, for tiles with more than 16 tokens: weight rows on the
+    // accumulator-register axis (register r <-> row 8*(r/4) + 4*hh + r%4), tokens on the lanes.
+    // All 16 registers are needed either way, and this way round the activation scales are one
+    // LDS read per stage instead of sixteen.
+    auto read_d_rows = [&](const char *base, int j, v2i (&dd)[4]) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)  // rows 8g + 4*hh + {0..3}  <->  accumulator registers 4g .. 4g+3
+            dd[g] = *reinterpret_cast<const v2i *>(base + OFF_D + wave * 256 + (g * 4 + j) * 16 + hh * 8);
+    };
+    auto mfmas_rows = [&](const v4i (&ab)[3], v16i &ihi, v16i &ilo) {  // rows = weight rows, columns = tokens
+        v4i a = ab[0];
+        if constexpr (QT == 4) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) a[t] = nibbles_to_i8x16(a[t], 4 - 4 * hh);
+        }
+        v16i zero;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) zero[r] = 0;
+        ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, ab[1], zero, 0, 0, 0);
+        ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, ab[2], zero, 0, 0, 0);
+    };
+    auto scale_acc_rows = [&](const v16i &ihi, const v16i &ilo, const v2i (&dd)[4], float sj) {
+        if constexpr (QT == 4) sj *= 0.0625f;  // the weight operand was 16 * (q - 8)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int r = 4 * g + q;
+                const uint32_t pairbits = (uint32_t)dd[g][q >> 1];
+                const float dv = half_bits_to_float((q & 1) ? pairbits >> 16 : pairbits & 0xFFFFu);
+                // |integer| < 2^31: rounded to 24 bits, then scaled (two roundings of 2^-24, far below the digit step)
+                const float fx = (float)(ihi[r] * 256 + ilo[r]) * sj;
+                acc[r] = fmaf(dv, fx, acc[r]);
+            }
+    };
+    auto compute_rows = [&](auto ring_slot, int s) {
+        const int b0 = b_begin + s * NBU;
+        const char *base = lds + decltype(ring_slot)::value * STAGE;
+        // Read as integers: a float-typed LDS read makes the compiler wait for every LDS fill in
+        // flight (it cannot tell the stages apart), an int-typed one leaves the waits to us.
+        const v4i sxi = *reinterpret_cast<const v4i *>(base + OFF_XS + l31 * 16);
+        // (element -> named int -> float: a bit cast applied directly to a vector element
+        // expression was compiled as a cast of element 0)
+        const int sx0 = sxi[0], sx1 = sxi[1], sx2 = sxi[2], sx3 = sxi[3];
+        const float sx[4] = {__int_as_float(sx0), __int_as_float(sx1), __int_as_float(sx2), __int_as_float(sx3)};
+        v4i ab[2][3];
+        v2i dd[2][4];
+        v16i ihi[2], ilo[2];
+        if (b0 + NBU <= b_end) {  // full stage (wavefront-uniform)
+            // Software pipeline over the 4 blocks: while block j is scaled and accumulated on
+            // the vector ALU, the MFMAs of block j+1 run and the LDS reads of block j+2 return.
+            read_ab(base, 0, ab[0]);
+            read_d_rows(base, 0, dd[0]);
+            read_ab(base, 1, ab[1]);
+            mfmas_rows(ab[0], ihi[0], ilo[0]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < NBU; ++j) {
+                if (j + 1 < NBU) {
+                    mfmas_rows(ab[(j + 1) & 1], ihi[(j + 1) & 1], ilo[(j + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);  // younger LDS reads must not be waited for here
+                    read_d_rows(base, j + 1, dd[(j + 1) & 1]);
+                }
+                if (j + 2 < NBU) read_ab(base, j + 2, ab[j & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                scale_acc_rows(ihi[j & 1], ilo[j & 1], dd[j & 1], sx[j]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NBU - 1; ++j)
+                if (b0 + j < b_end) {
+                    read_ab(base, j, ab[0]);
+                    read_d_rows(base, j, dd[0]);
+                    mfmas_rows(ab[0], ihi[0], ilo[0]);
+                    scale_acc_rows(ihi[0], ilo[0], dd[0], sx[j]);
                 }
         }
     };
@@ -323,31 +405,66 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     issue(std::integral_constant<int, 0>{}, 0);
     if (nst > 1) issue(std::integral_constant<int, 1>{}, 1);
-    for (int s0 = 0; s0 < nst; s0 += RING) {
+    auto k_loop = [&](auto nr) {
+        for (int s0 = 0; s0 < nst; s0 += RING) {
 #define PG_MM_STEP(U)                                                                     \
-        if (s0 + U < nst) {                                                               \
-            const int s = s0 + U;                                                         \
-            wait_barrier(s + 1 < nst);                       \
-            if (s + 2 < nst) issue(std::integral_constant<int, (U + 2) % RING>{}, s + 2); \
-            compute(std::integral_constant<int, U>{}, s);          \
-        }
-        PG_MM_STEP(0)
-        PG_MM_STEP(1)
-        PG_MM_STEP(2)
+            if (s0 + U < nst) {                                                           \
+                const int s = s0 + U;                                                     \
+                wait_barrier(s + 1 < nst);                                                \
+                if (s + 2 < nst) issue(std::integral_constant<int, (U + 2) % RING>{}, s + 2); \
+                compute(nr, std::integral_constant<int, U>{}, s);                         \
+            }
+            PG_MM_STEP(0)
+            PG_MM_STEP(1)
+            PG_MM_STEP(2)
 #undef PG_MM_STEP
+        }
+    };
+    if (ntok > 16) {  // the same choice for the whole workgroup
+        for (int s0 = 0; s0 < nst; s0 += RING) {
+#define PG_MM_STEP(U)                                                                     \
+            if (s0 + U < nst) {                                                           \
+                const int s = s0 + U;                                                     \
+                wait_barrier(s + 1 < nst);                                                \
+                if (s + 2 < nst) issue(std::integral_constant<int, (U + 2) % RING>{}, s + 2); \
+                compute_rows(std::integral_constant<int, U>{}, s);                        \
+            }
+            PG_MM_STEP(0)
+            PG_MM_STEP(1)
+            PG_MM_STEP(2)
+#undef PG_MM_STEP
+        }
+        const bool tok_ok = tt * 32 + l31 < count;  // the token whose outputs this lane accumulated
+        if (!tok_ok) return;
+        const int pair = grp.lists ? grp.lists[(size_t)e * grp.list_stride + tt * 32 + l31] : tt * 32 + l31;
+        float *y = out + blockIdx.z * part_stride + (size_t)pair * n_out;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int r0 = row0 + 8 * g + 4 * hh;
+            if (r0 + 3 < n_out && (n_out & 3) == 0) {
+                *reinterpret_cast<float4 *>(y + r0) = make_float4(acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]);
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (r0 + q < n_out) y[r0 + q] = acc[4 * g + q];
+            }
+        }
+        return;
     }
+    if (ntok <= 8) k_loop(std::integral_constant<int, 4>{});
+    else k_loop(std::integral_constant<int, 8>{});
 
-    if (!tok_ok) return;
-    float *y = out + blockIdx.z * part_stride + (size_t)pair * n_out;
+    // lanes hold consecutive weight rows: each token's 32 outputs leave as one 128-byte run
+    const int row = row0 + l31;
+    if (row >= n_out) return;
+    float *ybase = out + blockIdx.z * part_stride + row;
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-        const int r0 = row0 + 8 * g + 4 * hh;
-        if (r0 + 3 < n_out && (n_out & 3) == 0) {
-            *reinterpret_cast<float4 *>(y + r0) = make_float4(acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]);
-        } else {
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                if (r0 + q < n_out) y[r0 + q] = acc[4 * g + q];
+    for (int r = 0; r < 16; ++r) {
+        const int tok = 8 * (r >> 2) + 4 * hh + (r & 3);
+        if (tok < ntok) {
+            const int slot = tt * 32 + tok;
+            const int pair = grp.lists ? grp.lists[(size_t)e * grp.list_stride + slot] : slot;
+            ybase[(size_t)pair * n_out] = acc[r];
         }
     }
 }
