@@ -163,7 +163,8 @@ pg_status pg_dequant_q4_1(pg_ctx *ctx, const uint8_t *data, size_t num_elements,
 /* Keep a GGUF weight quantised on the device instead of materialising f32 as
  * GgufFile::load_tensor_f32 + load_transposed_weight do
  * (src/gguf.rs:485-517, src/models/llama/model.rs:243-257).
- * blocks: the tensor's raw block bytes, [n_out, k_in] with blocks of 32 along k_in. */
+ * blocks: the tensor's raw block bytes, [n_out, k_in] with blocks of 32 along k_in; Q4_0,
+ * Q4_1 or Q8_0 (18 / 20 / 34 bytes per block, src/gguf.rs:47-55). */
 pg_status pg_gguf_upload(pg_ctx *ctx, const void *blocks, int ggml_type, size_t n_out,
                          size_t k_in, pg_gguf_tensor **out);
 pg_status pg_gguf_shape(const pg_gguf_tensor *t, size_t *n_out, size_t *k_in, int *ggml_type);

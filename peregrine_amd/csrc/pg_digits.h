@@ -13,9 +13,12 @@
 //                  n_j of the block's 32 elements, element e in nibble e.
 //     bytes (Q8_0, MXFP4): |X| < 2^22, X = 65536 a0 + 256 a1 + a2 with signed byte digits;
 //                  plane 2j+h holds a_j of elements 16h..16h+15.
+// With `xsum` (Q4_1, whose blocks carry an offset m: sum_k (q d + m) x = d sum q x + m sum x) the
+// block's sum of fixed-point values, sum_k X[k], is stored too: xsum[row][b] (exact: < 2^23).
 template <bool NIB>
 __device__ __forceinline__ void pg_emit_digits(const float (&f)[4], size_t row, int b, int sub, int nb,
-                                               int8_t *__restrict__ digits, float *__restrict__ xs) {
+                                               int8_t *__restrict__ digits, float *__restrict__ xs,
+                                               float *__restrict__ xsum = nullptr) {
     float amax = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3])));
     int bad = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]);
 #pragma unroll
@@ -41,6 +44,12 @@ __device__ __forceinline__ void pg_emit_digits(const float (&f)[4], size_t row, 
     for (int e = 0; e < 4; ++e) {
         const float t = f[e] * inv;
         X[e] = (t != t) ? 0 : (int)rintf(t);
+    }
+    if (xsum) {  // the same for all lanes
+        int part = X[0] + X[1] + X[2] + X[3];
+#pragma unroll
+        for (int off = 1; off < 8; off <<= 1) part += __shfl_xor(part, off, 64);
+        if (sub == 0) xsum[row * (size_t)nb + b] = (float)part;
     }
     int8_t *drow = digits + row * (size_t)nb * 96;
     if (NIB) {

@@ -95,16 +95,27 @@ __global__ void dequant_q4_1_kernel(const uint8_t *__restrict__ data, size_t nbl
 // Q8_0: qs[((n*2 + h)*nb + b)*16 .. +16] = bytes 16h..16h+15 of the block's 32 i8.
 // d[((n/8)*nb + b)*8 + n%8] = the block's f16 scale: tiles of 8 rows, so one 128-bit load
 // gives a lane the scales of its block for 8 consecutive weight rows (rows past n_out: 0).
+// Q4_1: as Q4_0, plus the block's f16 offset in m[] (tiled like d); q - 8 goes to the dot
+// product and the 8 is folded into the offset term at run time.
 __global__ void split_blocks_kernel(const uint8_t *__restrict__ raw, size_t n_out, size_t nb,
                                     int ggml_type, uint8_t *__restrict__ qs,
-                                    uint16_t *__restrict__ d) {
+                                    uint16_t *__restrict__ d, uint16_t *__restrict__ m) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t n_pad = (n_out + 7) / 8 * 8;
     if (i >= n_pad * nb) return;
     const size_t n = i / nb, b = i - n * nb;
     uint16_t *dd = d + ((n / 8) * nb + b) * 8 + (n % 8);
-    if (n >= n_out) { *dd = 0; return; }
-    if (ggml_type == PG_GGML_Q4_0) {
+    if (n >= n_out) {
+        *dd = 0;
+        if (m) m[((n / 8) * nb + b) * 8 + (n % 8)] = 0;
+        return;
+    }
+    if (ggml_type == PG_GGML_Q4_1) {
+        const uint8_t *blk = raw + i * 20;
+        *dd = ld_u16(blk);
+        m[((n / 8) * nb + b) * 8 + (n % 8)] = ld_u16(blk + 2);
+        for (int j = 0; j < 16; ++j) qs[i * 16 + j] = blk[4 + j] ^ 0x88;
+    } else if (ggml_type == PG_GGML_Q4_0) {
         const uint8_t *blk = raw + i * 18;
         *dd = ld_u16(blk);
         for (int j = 0; j < 16; ++j) qs[i * 16 + j] = blk[2 + j] ^ 0x88;  // nibble -> (q - 8) in two's complement
@@ -131,13 +142,13 @@ __global__ void split_blocks_kernel(const uint8_t *__restrict__ raw, size_t n_ou
 template <bool NIB>
 __global__ __launch_bounds__(256) void x_to_digits_kernel(const float *__restrict__ x, int nb,
                                                           int8_t *__restrict__ digits,
-                                                          float *__restrict__ xs) {
+                                                          float *__restrict__ xs, float *__restrict__ xsum) {
     const size_t row = blockIdx.y;
     const int b = blockIdx.x * 32 + (threadIdx.x >> 3), sub = threadIdx.x & 7;
     if (b >= nb) return;  // whole 8-thread groups leave together
     const float4 v = reinterpret_cast<const float4 *>(x + (row * nb + b) * 32)[sub];
     const float f[4] = {v.x, v.y, v.z, v.w};
-    pg_emit_digits<NIB>(f, row, b, sub, nb, digits, xs);
+    pg_emit_digits<NIB>(f, row, b, sub, nb, digits, xs, xsum);
 }
 
 // ---- M = 1 fused dequant-GEMV ------------------------------------------------------
@@ -198,11 +209,14 @@ struct RowLoads {
 // uses (qs0, d0).  R rows are in flight at a time (NG = RW / R groups, double-buffered).
 // BF: the 16-bit block scales are the top halves of f32 values (the power-of-two scales of
 // MXFP4 blocks, whose range f16 cannot hold) instead of f16.
-template <int QT, int BPL, int RW, int R, bool BF = false>
+// Q41 (with QT = 4): every block also has an offset m; its term (8 d + m) * sum_k x_k uses the
+// block sums written with the digits.
+template <int QT, int BPL, int RW, int R, bool BF = false, bool Q41 = false>
 __global__ __launch_bounds__(64) void gguf_gemv_kernel(
     const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0, pg_gemv_batch batch,
     int n_out, int nb, const int8_t *__restrict__ digits_base, const float *__restrict__ xs_base,
-    float *__restrict__ y_base, const float *__restrict__ residual_base) {
+    float *__restrict__ y_base, const float *__restrict__ residual_base, const uint16_t *__restrict__ m0,
+    const float *__restrict__ xsum_base) {
     constexpr int SEG = 64 * BPL;  // blocks per K segment
     constexpr int NG = RW / R;
     constexpr int NH = QT == 8 ? 2 : 1;
@@ -220,6 +234,8 @@ __global__ __launch_bounds__(64) void gguf_gemv_kernel(
     const size_t xrow = (size_t)(item / batch.x_row_div);
     const gv4i_ptr digits = (gv4i_ptr)(uintptr_t)(digits_base + xrow * (size_t)nb * 96);
     const float *__restrict__ xs = xs_base + xrow * (size_t)nb;
+    const gv4i_ptr msc = (gv4i_ptr)(uintptr_t)m0;
+    const float *__restrict__ xsum = Q41 ? xsum_base + xrow * (size_t)nb : nullptr;
     float *__restrict__ y = y_base + (size_t)item * n_out;
     const int lane = threadIdx.x;
     const int row0 = blockIdx.x * RW;
@@ -253,19 +269,28 @@ __global__ __launch_bounds__(64) void gguf_gemv_kernel(
         v4i xd[BPL][NP];
         float sb[BPL];
         v4i dtile[BPL];  // f16 scales of this lane's blocks for the 8 rows of the tile
+        v4i mtile[BPL];  // Q4_1: their f16 offsets
+        float sxs[BPL];  // Q4_1: scale * block sum of the activation block
 #pragma unroll
         for (int p = 0; p < BPL; ++p) {
 #pragma unroll
             for (int j = 0; j < NP; ++j) xd[p][j] = digits[(size_t)j * nb + blk[p]];
             sb[p] = xs[blk[p]];
             dtile[p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+            if constexpr (Q41) {
+                mtile[p] = msc[(size_t)(row0 >> 3) * nb + blk[p]];
+                sxs[p] = xsum[blk[p]];
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         RowLoads<QT, BPL, R> L[2];
         load_rows(L[0], 0);
         __builtin_amdgcn_sched_barrier(0);  // every load is issued before any arithmetic
 #pragma unroll
-        for (int p = 0; p < BPL; ++p) sb[p] *= (lane + 64 * p < seg_n ? 1.0f : 0.0f);
+        for (int p = 0; p < BPL; ++p) {
+            sb[p] *= (lane + 64 * p < seg_n ? 1.0f : 0.0f);
+            if constexpr (Q41) sxs[p] *= sb[p];
+        }
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
             if (g + 1 < NG) {
@@ -291,6 +316,11 @@ __global__ __launch_bounds__(64) void gguf_gemv_kernel(
                                         : half_bits_to_float((uint16_t)((tr & 1) ? pair >> 16 : pair & 0xFFFFu));
                     const float ds = dv * sb[p];
                     acc[g][r] = fmaf(ds, f, acc[g][r]);
+                    if constexpr (Q41) {
+                        const uint32_t mp = (uint32_t)mtile[p][tr >> 1];
+                        const float mv = half_bits_to_float((uint16_t)((tr & 1) ? mp >> 16 : mp & 0xFFFFu));
+                        acc[g][r] = fmaf(fmaf(8.0f, dv, mv), sxs[p], acc[g][r]);  // q = (q - 8) + 8
+                    }
                 }
             }
         }
@@ -305,9 +335,10 @@ __global__ __launch_bounds__(64) void gguf_gemv_kernel(
         }
 }
 
-template <int QT, int BPL, bool BF>
+template <int QT, int BPL, bool BF, bool Q41>
 pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
-                          const pg_gemv_batch &batch, const pg_xdigits &xd, float *y, const float *residual) {
+                          const pg_gemv_batch &batch, const pg_xdigits &xd, float *y, const float *residual,
+                          const uint16_t *m) {
     const int nb = (int)(k_in / 32);
     // rows in flight per wavefront: bounded by registers (16 B of weights per row and block)
     constexpr int NH = QT == 8 ? 2 : 1;
@@ -316,9 +347,9 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
 #define PG_GGUF_GEMV_LAUNCH(RWW, RR)                                                               \
     do {                                                                                           \
         const dim3 grid(grid_for(n_out, RWW), (unsigned)batch.count);                              \
-        PG_TRY(pg_launch(ctx, QT == 4 ? "gguf_gemv_q4_0" : (BF ? "gguf_gemv_mxfp4" : "gguf_gemv_q8_0"), \
-                         gguf_gemv_kernel<QT, BPL, RWW, RR, BF>, grid, dim3(64), 0, qs, d, batch,  \
-                         (int)n_out, nb, xd.digits, xd.xs, y, residual));                          \
+        PG_TRY(pg_launch(ctx, QT == 4 ? (Q41 ? "gguf_gemv_q4_1" : "gguf_gemv_q4_0") : (BF ? "gguf_gemv_mxfp4" : "gguf_gemv_q8_0"), \
+                         gguf_gemv_kernel<QT, BPL, RWW, RR, BF, Q41>, grid, dim3(64), 0, qs, d, batch, \
+                         (int)n_out, nb, xd.digits, xd.xs, y, residual, m, (const float *)xd.xsum)); \
     } while (0)
     if (n_out / 8 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(8, R8);
     else if (n_out / 4 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(4, (R8 < 4 ? R8 : 4));
@@ -327,17 +358,18 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
     return PG_OK;
 }
 
-template <int QT, bool BF = false>
+template <int QT, bool BF = false, bool Q41 = false>
 pg_status launch_gemv(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
-                      const pg_gemv_batch &batch, const pg_xdigits &xd, float *y, const float *residual) {
+                      const pg_gemv_batch &batch, const pg_xdigits &xd, float *y, const float *residual,
+                      const uint16_t *m) {
     const size_t nb = k_in / 32;
     size_t bpl = (nb + 63) / 64;
     if (bpl > 4) bpl = 4;  // longer rows run as several K segments of 256 blocks
     switch (bpl) {
-        case 1: return launch_gemv_bpl<QT, 1, BF>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
-        case 2: return launch_gemv_bpl<QT, 2, BF>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
-        case 3: return launch_gemv_bpl<QT, 3, BF>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
-        default: return launch_gemv_bpl<QT, 4, BF>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
+        case 1: return launch_gemv_bpl<QT, 1, BF, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
+        case 2: return launch_gemv_bpl<QT, 2, BF, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
+        case 3: return launch_gemv_bpl<QT, 3, BF, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
+        default: return launch_gemv_bpl<QT, 4, BF, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
     }
 }
 
@@ -345,7 +377,7 @@ pg_status launch_gemv(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs,
 
 size_t pg_xdigits_bytes(size_t rows, size_t k) {
     const size_t nb = k / 32;
-    return pg_round_up(3 * rows * k, 256) + pg_round_up(rows * nb * sizeof(float), 256);
+    return pg_round_up(3 * rows * k, 256) + 2 * pg_round_up(rows * nb * sizeof(float), 256);
 }
 
 pg_xdigits pg_xdigits_carve(void *base, size_t rows, size_t k) {
@@ -355,7 +387,8 @@ pg_xdigits pg_xdigits_carve(void *base, size_t rows, size_t k) {
     xd.digits = reinterpret_cast<int8_t *>(p);
     p += pg_round_up(3 * rows * k, 256);
     xd.xs = reinterpret_cast<float *>(p);
-    (void)nb;
+    p += pg_round_up(rows * nb * sizeof(float), 256);
+    xd.xsum = reinterpret_cast<float *>(p);
     xd.rows = rows;
     xd.k = k;
     return xd;
@@ -367,21 +400,27 @@ pg_status pg_launch_x_to_digits(pg_ctx *ctx, const float *x_dev, size_t rows, si
     if (rows > 65535) return pg_fail(PG_EUNSUPPORTED, "x_to_digits: more than 65535 activation rows");
     const int nb = (int)(k / 32);
     const dim3 grid(grid_for(nb, 32), (unsigned)rows);
-    if (ggml_type == PG_GGML_Q4_0)
-        PG_TRY(pg_launch(ctx, "x_to_digits", x_to_digits_kernel<true>, grid, dim3(256), 0, x_dev, nb, xd.digits, xd.xs));
+    if (ggml_type == PG_GGML_Q4_0 || ggml_type == PG_GGML_Q4_1)
+        PG_TRY(pg_launch(ctx, "x_to_digits", x_to_digits_kernel<true>, grid, dim3(256), 0, x_dev, nb, xd.digits, xd.xs,
+                         ggml_type == PG_GGML_Q4_1 ? xd.xsum : (float *)nullptr));
     else
-        PG_TRY(pg_launch(ctx, "x_to_digits", x_to_digits_kernel<false>, grid, dim3(256), 0, x_dev, nb, xd.digits, xd.xs));
+        PG_TRY(pg_launch(ctx, "x_to_digits", x_to_digits_kernel<false>, grid, dim3(256), 0, x_dev, nb, xd.digits, xd.xs,
+                         (float *)nullptr));
     return pg_launch_check("x_to_digits");
 }
 
 pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in,
                               const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
-                              const pg_xdigits &xd, float *y, const float *residual) {
+                              const pg_xdigits &xd, float *y, const float *residual, const uint16_t *m) {
     if (batch.count == 0) return PG_OK;
     if (batch.count > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_gemv: more than 65535 batch items");
-    if (ggml_type == PG_GGML_Q4_0) return launch_gemv<4>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
-    if (ggml_type == PG_MXFP4) return launch_gemv<8, true>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
-    return launch_gemv<8>(ctx, n_out, k_in, qs, d, batch, xd, y, residual);
+    if (ggml_type == PG_GGML_Q4_1) {
+        if (!m || batch.qs_table) return pg_fail(PG_EINVAL, "gguf_gemv: Q4_1 needs its offsets and runs without expert tables");
+        return launch_gemv<4, false, true>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
+    }
+    if (ggml_type == PG_GGML_Q4_0) return launch_gemv<4>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, nullptr);
+    if (ggml_type == PG_MXFP4) return launch_gemv<8, true>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, nullptr);
+    return launch_gemv<8>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, nullptr);
 }
 
 // Quantise `m` activation rows (device) into the arena and run the fused product: the
@@ -389,13 +428,13 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
 pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
                               float *y_dev) {
     void *ws = nullptr;
-    if (m == 1 || w->ggml_type == PG_MXFP4) {  // MXFP4 has the streaming kernel only: one item per row
-        if (m > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_matmul: more than 65535 rows against an MXFP4 tensor");
+    if (m == 1 || w->ggml_type == PG_MXFP4 || w->ggml_type == PG_GGML_Q4_1) {  // these two have the streaming kernel only: one item per row
+        if (m > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_matmul: more than 65535 rows against an MXFP4 or Q4_1 tensor");
         PG_TRY(pg_workspace(ctx, pg_xdigits_bytes(m, w->k_in), &ws));
         const pg_xdigits xd = pg_xdigits_carve(ws, m, w->k_in);
         PG_TRY(pg_launch_x_to_digits(ctx, x_dev, m, w->k_in, w->ggml_type, xd));
         pg_gemv_batch batch = {(int)m, nullptr, nullptr, nullptr, 1};
-        return pg_launch_gguf_gemv(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, batch, xd, y_dev);
+        return pg_launch_gguf_gemv(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, batch, xd, y_dev, nullptr, w->m);
     }
     const int ks = pg_gguf_mm_splitk(ctx, w->n_out, w->k_in, (m + 31) / 32, nullptr);
     const size_t sz_d = pg_mmdigits_bytes(m, w->k_in);
@@ -418,9 +457,12 @@ pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, c
         if (w[i]->k_in != k_in) return pg_fail(PG_EINVAL, "gguf_matmul_multi: the products differ in k_in");
     void *ws = nullptr;
     int digits_type = -1;
-    bool any_mxfp4 = false;
-    for (int i = 0; i < count; ++i) any_mxfp4 |= w[i]->ggml_type == PG_MXFP4;
-    if (any_mxfp4 && m > 1) {  // no shared matrix-core route: product by product
+    bool any_mxfp4 = false, any_q41 = false;
+    for (int i = 0; i < count; ++i) {
+        any_mxfp4 |= w[i]->ggml_type == PG_MXFP4;
+        any_q41 |= w[i]->ggml_type == PG_GGML_Q4_1;
+    }
+    if ((any_mxfp4 && m > 1) || any_q41) {  // no shared route: product by product
         for (int i = 0; i < count; ++i) PG_TRY(pg_gguf_matmul_rows(ctx, x_dev, m, w[i], y_dev[i]));
         return PG_OK;
     }
@@ -515,20 +557,19 @@ PG_API pg_status pg_gguf_upload(pg_ctx *ctx, const void *blocks, int ggml_type, 
     PG_TRY(pg_use(ctx));
     PG_CHECK_ARG(out != nullptr, "pg_gguf_upload: out is null");
     *out = nullptr;
-    if (ggml_type == PG_GGML_Q4_1)
-        return pg_fail(PG_EUNSUPPORTED, "pg_gguf_upload: Q4_1 has a dequantise kernel only");
-    PG_CHECK_ARG(ggml_type == PG_GGML_Q4_0 || ggml_type == PG_GGML_Q8_0,
+    PG_CHECK_ARG(ggml_type == PG_GGML_Q4_0 || ggml_type == PG_GGML_Q4_1 || ggml_type == PG_GGML_Q8_0,
                  "pg_gguf_upload: ggml type %d is not a block-quantised type", ggml_type);
     PG_CHECK_ARG(n_out > 0 && k_in > 0 && blocks, "pg_gguf_upload: empty tensor or null pointer");
     PG_CHECK_ARG(k_in % 32 == 0, "pg_gguf_upload: k_in %zu is not a multiple of 32", k_in);
     PG_CHECK_ARG(n_out < (1ull << 31) && k_in < (1ull << 31) && n_out * (k_in / 32) < (1ull << 31),
                  "pg_gguf_upload: shape too large");
     const size_t nb = k_in / 32, nblocks = n_out * nb;
-    const size_t bb = ggml_type == PG_GGML_Q4_0 ? 18 : 34, qb = bb - 2;
+    const size_t bb = ggml_type == PG_GGML_Q4_0 ? 18 : (ggml_type == PG_GGML_Q4_1 ? 20 : 34), qb = ggml_type == PG_GGML_Q8_0 ? 32 : 16;
     pg_gguf_tensor *t = new (std::nothrow) pg_gguf_tensor();
     if (!t) return pg_fail(PG_ENOMEM, "host allocation failed");
     t->qs = nullptr;
     t->d = nullptr;
+    t->m = nullptr;
     t->ggml_type = ggml_type;
     t->n_out = n_out;
     t->k_in = k_in;
@@ -538,10 +579,11 @@ PG_API pg_status pg_gguf_upload(pg_ctx *ctx, const void *blocks, int ggml_type, 
     if (st == PG_OK) {
         e = hipMalloc((void **)&t->qs, nblocks * qb);
         if (e == hipSuccess) e = hipMalloc((void **)&t->d, (n_out + 7) / 8 * 8 * nb * sizeof(uint16_t));
+        if (e == hipSuccess && ggml_type == PG_GGML_Q4_1) e = hipMalloc((void **)&t->m, (n_out + 7) / 8 * 8 * nb * sizeof(uint16_t));
         if (e == hipSuccess) e = hipMemcpyAsync(raw.p, blocks, nblocks * bb, hipMemcpyHostToDevice, ctx->stream);
         if (e == hipSuccess) {
             split_blocks_kernel<<<grid_for((n_out + 7) / 8 * 8 * nb, 256), 256, 0, ctx->stream>>>(raw.as<uint8_t>(), n_out, nb,
-                                                                               ggml_type, t->qs, t->d);
+                                                                               ggml_type, t->qs, t->d, t->m);
             e = hipGetLastError();
         }
         if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
@@ -593,6 +635,7 @@ PG_API pg_status pg_mxfp4_upload(pg_ctx *ctx, const uint8_t *blocks, const uint8
     if (!t) return pg_fail(PG_ENOMEM, "host allocation failed");
     t->qs = nullptr;
     t->d = nullptr;
+    t->m = nullptr;
     t->ggml_type = PG_MXFP4;
     t->n_out = out_dim;
     t->k_in = in_dim;
@@ -751,6 +794,7 @@ PG_API void pg_gguf_free(pg_ctx *ctx, pg_gguf_tensor *t) {
     }
     if (t->qs) (void)hipFree(t->qs);
     if (t->d) (void)hipFree(t->d);
+    if (t->m) (void)hipFree(t->m);
     delete t;
 }
 

@@ -58,6 +58,7 @@ struct pg_qtensor {
 struct pg_gguf_tensor {
     uint8_t *qs;
     uint16_t *d;
+    uint16_t *m;  // Q4_1 only: the blocks' f16 offsets, tiled like d; else null
     int ggml_type;
     size_t n_out, k_in;
 };
@@ -149,6 +150,7 @@ pg_status pg_launch_gemv_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
 struct pg_xdigits {
     int8_t *digits;  // [rows][6 planes][k/32 blocks][16 bytes] (Q4_0 uses 5 planes, Q8_0 all 6)
     float *xs;       // [rows][k/32] power-of-two block scales
+    float *xsum;     // [rows][k/32] sum of each block's fixed-point values (written for Q4_1 only)
     size_t rows, k;
 };
 
@@ -194,7 +196,8 @@ struct pg_gemv_batch {
 // y[item][row] = product (+ residual[item][row] when `residual` is given).
 pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in,
                               const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
-                              const pg_xdigits &xd, float *y, const float *residual = nullptr);
+                              const pg_xdigits &xd, float *y, const float *residual = nullptr,
+                              const uint16_t *m = nullptr);
 // Activation rows as two byte-digit planes for the matrix-core product (see pg_gguf_mm.hip).
 struct pg_mmdigits {
     int8_t *digits;  // [rows][2 planes][k/32 blocks][2 halves][16 bytes]

@@ -1,4 +1,4 @@
-"""Synthetic GGUF block data: quantise f32 matrices into Q8_0 / Q4_0 blocks on the host.
+"""Synthetic GGUF block data: quantise f32 matrices into Q8_0 / Q4_0 / Q4_1 blocks on the host.
 
 Input synthesis for tests and the benchmark (there are no real .gguf files offline); any
 packer will do, because parity is always judged against the dequantisation of the same bytes.
@@ -34,4 +34,21 @@ def pack_q4_0(w):
     out = np.empty((w.shape[0], 18), np.uint8)
     out[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
     out[:, 2:] = q[:, 0::2] | (q[:, 1::2] << 4)
+    return out.tobytes()
+
+
+def pack_q4_1(w):
+    """Quantise f32 into GGUF Q4_1 blocks (d = f16((max - min) / 15), m = f16(min), q = 0..15,
+    value = q * d + m; same nibble order as Q4_0, src/gguf.rs:331-351)."""
+    w = np.ascontiguousarray(w, np.float32).reshape(-1, 32)
+    lo, hi = w.min(axis=1), w.max(axis=1)
+    d = ((hi - lo) / 15.0).astype(np.float16)
+    m = lo.astype(np.float16)
+    df, mf = d.astype(np.float32), m.astype(np.float32)
+    inv = np.where(df != 0, 1.0 / np.where(df != 0, df, 1), 0).astype(np.float32)
+    q = np.clip(np.rint((w - mf[:, None]) * inv[:, None]), 0, 15).astype(np.uint8)
+    out = np.empty((w.shape[0], 20), np.uint8)
+    out[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
+    out[:, 2:4] = m.view(np.uint8).reshape(-1, 2)
+    out[:, 4:] = q[:, 0::2] | (q[:, 1::2] << 4)
     return out.tobytes()

@@ -34,7 +34,7 @@ def mod_pattern(n, mul, add, mod, div, sub):
     return (((i * mul + add) % mod).astype(np.float32) / np.float32(div) - np.float32(sub)).astype(np.float32)
 
 
-from peregrine_amd.synth import pack_q4_0, pack_q8_0  # noqa: E402,F401
+from peregrine_amd.synth import pack_q4_0, pack_q4_1, pack_q8_0  # noqa: E402,F401
 
 
 def np_dequant_q4_0(raw, n):

@@ -16,7 +16,7 @@ import helpers as H
 pytestmark = pytest.mark.gpu
 
 RTOL_CONTRACT = 1e-3                 # the stated tolerance for Q4_0/Q8_0 block-dequant paths
-RTOL_ACHIEVED = {2: 1e-4, 8: 2e-5}   # what the one-row (GEMV) path is held to, per ggml type
+RTOL_ACHIEVED = {2: 1e-4, 3: 1e-4, 8: 2e-5}   # what the one-row (GEMV) path is held to, per ggml type
 RTOL_ACHIEVED_MM = 4e-4              # several rows: 16-bit fixed-point activations per block
 
 
@@ -95,6 +95,8 @@ GGUF_SHAPES = [
     (8, 6144, 4096, 1),
     # more than one row: matrix-core path (token tiles of 32, row tiles of 128, split K)
     (2, 130, 224, 33), (8, 131, 160, 40), (2, 515, 4096, 64), (8, 257, 6144, 35), (2, 14336, 4096, 4), (8, 4096, 14336, 16),
+    # Q4_1 (offset blocks): the streaming kernel with the block-sum term, one item per row
+    (3, 256, 4096, 1), (3, 77, 96, 3), (3, 1000, 2048, 2), (3, 50, 11008, 1), (3, 64, 32768, 2), (3, 14336, 4096, 1), (3, 130, 224, 33),
     # 16 token tiles and more: no split K, XCD-aware super-tiles of 4 row groups x 8 token tiles (ragged on both sides)
     (2, 600, 256, 545), (8, 1100, 128, 700), (2, 128, 512, 512),
 ]
@@ -105,7 +107,9 @@ def test_gguf_matmul_vs_oracle(ctx, orc, typ, n_out, k_in, m):
     from peregrine_amd import gguf
     say(f"gguf_matmul type={typ} n_out={n_out} k_in={k_in} m={m}")
     w = orc.rng_normal(900 + n_out + typ, n_out * k_in, 0.0, 0.02)
-    raw = (H.pack_q4_0 if typ == 2 else H.pack_q8_0)(w)
+    if typ == 3:
+        w = w + np.float32(0.03)                      # off-centre, so that the block offsets matter
+    raw = {2: H.pack_q4_0, 3: H.pack_q4_1, 8: H.pack_q8_0}[typ](w)
     x = orc.rng_normal(17 + m, m * k_in)
     x.reshape(m, k_in)[:, :: max(1, k_in // 40)] *= 20
     gw = gguf.GgufWeight(raw, typ, n_out, k_in, ctx)
@@ -114,7 +118,7 @@ def test_gguf_matmul_vs_oracle(ctx, orc, typ, n_out, k_in, m):
     for r in range(m):
         sl = slice(r * n_out, (r + 1) * n_out)
         H.assert_close_rel(got[sl], want[sl], RTOL_CONTRACT, f"row {r} (contract)")
-        H.assert_close_rel(got[sl], want[sl], RTOL_ACHIEVED[typ] if m == 1 else RTOL_ACHIEVED_MM, f"row {r} (achieved)")
+        H.assert_close_rel(got[sl], want[sl], RTOL_ACHIEVED[typ] if (m == 1 or typ == 3) else RTOL_ACHIEVED_MM, f"row {r} (achieved)")
     gw.free()
 
 

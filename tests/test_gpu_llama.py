@@ -188,7 +188,7 @@ def _block_case(ctx, orc, d, nqh, nkvh, hd, ffn, typ, steps, max_seq=64, seed=0)
     from peregrine_amd import gguf, llama
     shapes = [(nqh * hd, d), (nkvh * hd, d), (nkvh * hd, d), (d, nqh * hd), (ffn, d), (ffn, d), (d, ffn)]
     types = [typ] * 7 if np.isscalar(typ) else list(typ)
-    raws = [bytes((H.pack_q4_0 if t == 2 else H.pack_q8_0)(orc.rng_normal(seed + 40 + i, n * k, 0.0, 1.0 / np.sqrt(k))))
+    raws = [bytes({2: H.pack_q4_0, 3: H.pack_q4_1, 8: H.pack_q8_0}[t](orc.rng_normal(seed + 40 + i, n * k, 0.0, 1.0 / np.sqrt(k))))
             for i, ((n, k), t) in enumerate(zip(shapes, types))]
     ws = [gguf.GgufWeight(r, t, n, k, ctx) for r, (n, k), t in zip(raws, shapes, types)]
     wa = (1 + 0.1 * orc.rng_normal(seed + 1, d)).astype(np.float32)
@@ -225,6 +225,11 @@ def test_llama_block_mixed_block_types(ctx, orc):
     """Q4_0 and Q8_0 projections in one block: their activation digits differ in kind, so the
     one-token step cannot share them and takes the product-by-product route."""
     _block_case(ctx, orc, 128, 4, 2, 32, 256, (8, 2, 8, 2, 2, 8, 8), (3, 1, 1), seed=3)
+
+
+def test_llama_block_q4_1_weights(ctx, orc):
+    """Offset blocks (Q4_1) run on the streaming kernel only, one item per row."""
+    _block_case(ctx, orc, 128, 4, 2, 32, 256, 3, (3, 1), seed=13)
 
 
 def test_llama_block_mha_and_odd_shapes(ctx, orc):
