@@ -162,6 +162,13 @@ def test_gqa_attention_many_rows(ctx, orc):
     _attention_case(ctx, orc, 8, 2, 64, 70, 90, llama.AttentionMask.none(), None, 61)
     _attention_case(ctx, orc, 8, 2, 64, 70, 90, llama.AttentionMask.causal(20), None, 62)
     _attention_case(ctx, orc, 8, 4, 32, 70, 90, llama.AttentionMask.causal_sliding_window(20, 7, 3), 2.0, 63)
+    # head sizes of the tiled kernel (64, 128, 256), key counts that are not multiples of its 64-key blocks,
+    # row counts that are not multiples of its 32-row workgroups, several appends (capacity > length)
+    say("attention, tiled kernel shapes")
+    _attention_case(ctx, orc, 8, 2, 128, 67, 150, llama.AttentionMask.causal(83), None, 64, appends=(100, 50))
+    _attention_case(ctx, orc, 8, 2, 128, 67, 150, llama.AttentionMask.none(), 3.0, 65)
+    _attention_case(ctx, orc, 4, 4, 256, 131, 131, llama.AttentionMask.causal(0), None, 66)
+    _attention_case(ctx, orc, 16, 2, 64, 33, 200, llama.AttentionMask.causal_sliding_window(167, 40, 4), None, 67)
 
 
 def test_gqa_attention_long_cache_splits_keys(ctx, orc):
@@ -225,6 +232,12 @@ def test_llama_block_mixed_block_types(ctx, orc):
     """Q4_0 and Q8_0 projections in one block: their activation digits differ in kind, so the
     one-token step cannot share them and takes the product-by-product route."""
     _block_case(ctx, orc, 128, 4, 2, 32, 256, (8, 2, 8, 2, 2, 8, 8), (3, 1, 1), seed=3)
+
+
+def test_llama_block_long_prefill_head_128(ctx, orc):
+    """A prefill long enough for the tiled attention kernel and the many-token-tile product
+    order (140 tokens x 4 heads of 128), then a decode step on top of it."""
+    _block_case(ctx, orc, 512, 4, 2, 128, 768, 2, (140, 1), max_seq=160, seed=21)
 
 
 def test_llama_block_q4_1_weights(ctx, orc):
