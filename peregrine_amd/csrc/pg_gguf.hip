@@ -423,6 +423,47 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
     return launch_gemv<8>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, nullptr);
 }
 
+// The tile-major copy of a tensor's quant plane that gguf_mm_kernel fetches: 16-byte chunks in
+// the order [group of 128 rows][group of 4 blocks][wavefront][fill][lane], where the lane of a
+// fill stands for (stream 16*fill + lane/4, block (lane%4) ^ ((lane/8)%4)) exactly as in the
+// kernel's fill duties; rows past n_out and blocks past k_in/32 are zeros.
+template <int QT>
+__global__ void tile_weights_kernel(const uint8_t *__restrict__ qs, int n_out, int nb, uint4 *__restrict__ tiled, size_t chunks) {
+    constexpr int CH = (QT == 8 ? 4096 : 2048) / 16, FILLS = CH / 64;  // chunks and fills per wavefront and stage
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= chunks) return;
+    const int lane = (int)(i & 63), q = (int)((i >> 6) % FILLS), wave = (int)((i / CH) & 3);
+    const size_t t = i / (4 * CH);
+    const int nsg = (nb + 3) / 4, sg = (int)(t % nsg), rg = (int)(t / nsg);
+    const int st = 16 * q + (lane >> 2), j = (lane & 3) ^ ((lane >> 3) & 3);
+    const int row = rg * 128 + wave * 32 + (st & 31), half = st >> 5, block = sg * 4 + j;
+    uint4 v = {0, 0, 0, 0};
+    if (row < n_out && block < nb)
+        v = *reinterpret_cast<const uint4 *>(qs + (QT == 8 ? ((size_t)row * 2 + half) * nb + block : (size_t)row * nb + block) * 16);
+    tiled[i] = v;
+}
+
+pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w) {
+    if (w->qs_tiled) return PG_OK;
+    if (w->ggml_type != PG_GGML_Q4_0 && w->ggml_type != PG_GGML_Q8_0)
+        return pg_fail(PG_EUNSUPPORTED, "gguf: no tile-major copy for ggml type %d", w->ggml_type);
+    const int nb = (int)(w->k_in / 32);
+    const size_t per_stage = 4 * (size_t)(w->ggml_type == PG_GGML_Q8_0 ? 4096 : 2048);
+    const size_t bytes = (w->n_out + 127) / 128 * (size_t)((nb + 3) / 4) * per_stage, chunks = bytes / 16;
+    uint8_t *p = nullptr;
+    hipError_t e = hipMalloc((void **)&p, bytes);
+    if (e != hipSuccess)
+        return pg_fail(e == hipErrorOutOfMemory ? PG_ENOMEM : PG_EDEVICE, "gguf tile-major copy (%zu bytes): %s", bytes, hipGetErrorString(e));
+    pg_status st = w->ggml_type == PG_GGML_Q8_0
+                       ? pg_launch(ctx, "gguf_tile_weights", tile_weights_kernel<8>, dim3(grid_for(chunks, 256)), dim3(256), 0,
+                                   (const uint8_t *)w->qs, (int)w->n_out, nb, reinterpret_cast<uint4 *>(p), chunks)
+                       : pg_launch(ctx, "gguf_tile_weights", tile_weights_kernel<4>, dim3(grid_for(chunks, 256)), dim3(256), 0,
+                                   (const uint8_t *)w->qs, (int)w->n_out, nb, reinterpret_cast<uint4 *>(p), chunks);
+    if (st != PG_OK) { (void)hipFree(p); return st; }
+    w->qs_tiled = p;
+    return PG_OK;
+}
+
 // Quantise `m` activation rows (device) into the arena and run the fused product: the
 // streaming GEMV for one row, the matrix-core kernel (weights read once) for more.
 pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
@@ -444,7 +485,9 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
     float *part = ks > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + sz_d) : nullptr;
     PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, m, w->k_in, w->ggml_type, md));
     pg_mm_group grp = {1, nullptr, nullptr, nullptr, nullptr, 0, (int)((m + 31) / 32), (int)m, 1};
-    return pg_launch_gguf_mm(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, grp, m, md, y_dev, part);
+    PG_TRY(pg_gguf_ensure_tiled(ctx, w));
+    grp.tiled = 1;
+    return pg_launch_gguf_mm(ctx, w->ggml_type, w->n_out, w->k_in, w->qs_tiled, w->d, grp, m, md, y_dev, part);
 }
 
 // Several products over the same activation rows (q/k/v, gate/up): the rows are rewritten
@@ -490,14 +533,16 @@ pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, c
     PG_TRY(pg_workspace(ctx, sz_d + sz_part, &ws));
     const pg_mmdigits md = pg_mmdigits_carve(ws, m, k_in);
     float *part_base = reinterpret_cast<float *>(static_cast<char *>(ws) + sz_d);
-    const pg_mm_group grp = {1, nullptr, nullptr, nullptr, nullptr, 0, (int)((m + 31) / 32), (int)m, 1};
+    pg_mm_group grp = {1, nullptr, nullptr, nullptr, nullptr, 0, (int)((m + 31) / 32), (int)m, 1};
+    grp.tiled = 1;
     for (int i = 0; i < count; ++i) {
+        PG_TRY(pg_gguf_ensure_tiled(ctx, w[i]));
         if (w[i]->ggml_type != digits_type) {
             PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, m, k_in, w[i]->ggml_type, md));
             digits_type = w[i]->ggml_type;
         }
         const int ks = pg_gguf_mm_splitk(ctx, w[i]->n_out, k_in, (m + 31) / 32, nullptr);
-        PG_TRY(pg_launch_gguf_mm(ctx, w[i]->ggml_type, w[i]->n_out, k_in, w[i]->qs, w[i]->d, grp, m, md, y_dev[i],
+        PG_TRY(pg_launch_gguf_mm(ctx, w[i]->ggml_type, w[i]->n_out, k_in, w[i]->qs_tiled, w[i]->d, grp, m, md, y_dev[i],
                                  ks > 1 ? part_base : nullptr));
     }
     return PG_OK;
@@ -570,6 +615,7 @@ PG_API pg_status pg_gguf_upload(pg_ctx *ctx, const void *blocks, int ggml_type, 
     t->qs = nullptr;
     t->d = nullptr;
     t->m = nullptr;
+    t->qs_tiled = nullptr;
     t->ggml_type = ggml_type;
     t->n_out = n_out;
     t->k_in = k_in;
@@ -636,6 +682,7 @@ PG_API pg_status pg_mxfp4_upload(pg_ctx *ctx, const uint8_t *blocks, const uint8
     t->qs = nullptr;
     t->d = nullptr;
     t->m = nullptr;
+    t->qs_tiled = nullptr;
     t->ggml_type = PG_MXFP4;
     t->n_out = out_dim;
     t->k_in = in_dim;
@@ -795,6 +842,7 @@ PG_API void pg_gguf_free(pg_ctx *ctx, pg_gguf_tensor *t) {
     if (t->qs) (void)hipFree(t->qs);
     if (t->d) (void)hipFree(t->d);
     if (t->m) (void)hipFree(t->m);
+    if (t->qs_tiled) (void)hipFree(t->qs_tiled);
     delete t;
 }
 

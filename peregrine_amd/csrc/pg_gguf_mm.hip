@@ -198,6 +198,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int wrow = row0 + (st & 31) < n_out ? row0 + (st & 31) : n_out - 1;  // clamped; masked at the store
         w_src[q] = reinterpret_cast<const int8_t *>(qs_any) +
                    (QT == 8 ? ((size_t)wrow * 2 + (st >> 5)) * nb * 16 : (size_t)wrow * nb * 16);
+        // Tile-major copy: [row group][4 blocks][wavefront][fill][lane] 16-byte chunks, the very
+        // order of the fills below, padded with zero rows and blocks: a stage of a workgroup is
+        // 4 * W_WAVE contiguous bytes.
+        if (grp.tiled)
+            w_src[q] = reinterpret_cast<const int8_t *>(qs_any) +
+                       ((size_t)bx * ((nb + 3) / 4) * 4 + wave) * W_WAVE + q * 1024 + lane * 16;
     }
     // f16 scales of this wavefront's 32 rows: lane -> (group lane/16, block (lane/4)%4, dword lane%4)
     const int ngroups = (n_out + 7) / 8;
@@ -224,9 +230,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         __builtin_amdgcn_global_load_lds((gptr_t)(d_grp + blk(d_jb) * 16), (lptr_t)(base + OFF_D + wave * 256), 4, 0, 0);
         if (lane < 8)
             __builtin_amdgcn_global_load_lds((gptr_t)(xs_src + b0), (lptr_t)(base + OFF_XS + wave * 128), 16, 0, 0);
+        const size_t w_off = grp.tiled ? (size_t)(b0 >> 2) * (4 * W_WAVE) : blk(w_jb) * 16;
 #pragma unroll
         for (int q = 0; q < W_FILLS; ++q)
-            __builtin_amdgcn_global_load_lds((gptr_t)(w_src[q] + blk(w_jb) * 16), (lptr_t)(base + OFF_W + wave * W_WAVE + q * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(w_src[q] + w_off), (lptr_t)(base + OFF_W + wave * W_WAVE + q * 1024), 16, 0, 0);
     };
 
     float acc[16];

@@ -59,6 +59,9 @@ struct pg_gguf_tensor {
     uint8_t *qs;
     uint16_t *d;
     uint16_t *m;  // Q4_1 only: the blocks' f16 offsets, tiled like d; else null
+    // Q4_0 / Q8_0: a second copy of qs in the order gguf_mm_kernel's workgroups fetch it
+    // (pg_gguf_ensure_tiled makes it on the tensor's first product over more than one row).
+    mutable uint8_t *qs_tiled;
     int ggml_type;
     size_t n_out, k_in;
 };
@@ -223,7 +226,10 @@ struct pg_mm_group {
     int max_count;
     int x_row_div;
     int remap_rg, remap_tiles;  // set by the launcher (row groups and token tiles of an XCD-aware 1-D launch), else 0
+    int tiled;                  // the qs pointers are tile-major copies (pg_gguf_tensor::qs_tiled)
 };
+// Makes w->qs_tiled if it is missing (one allocation and one kernel on the context's stream).
+pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w);
 // Number of K chunks the product is split into (partial sums: [chunks][pairs][n_out] floats);
 // `groups` = token tiles that certainly hold work (all tiles of a plain product, one per expert).
 int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t groups, int *chunk_out);

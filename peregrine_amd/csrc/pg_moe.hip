@@ -147,11 +147,15 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     // Expert pointer tables: [gate qs | gate d | up qs | up d | down qs | down d], E each, in a
     // device buffer the context keeps; uploaded (with a wait, the source is this stack frame)
     // only when the set of experts differs from the previous call's.
+    // (The quant planes are the tile-major copies, made on an expert's first use.)
     const void *host_tab[6 * MAX_EXPERTS];
     for (size_t e = 0; e < E; ++e) {
-        host_tab[0 * E + e] = gate[e]->qs; host_tab[1 * E + e] = gate[e]->d;
-        host_tab[2 * E + e] = up[e]->qs;   host_tab[3 * E + e] = up[e]->d;
-        host_tab[4 * E + e] = down[e]->qs; host_tab[5 * E + e] = down[e]->d;
+        PG_TRY(pg_gguf_ensure_tiled(ctx, gate[e]));
+        PG_TRY(pg_gguf_ensure_tiled(ctx, up[e]));
+        PG_TRY(pg_gguf_ensure_tiled(ctx, down[e]));
+        host_tab[0 * E + e] = gate[e]->qs_tiled; host_tab[1 * E + e] = gate[e]->d;
+        host_tab[2 * E + e] = up[e]->qs_tiled;   host_tab[3 * E + e] = up[e]->d;
+        host_tab[4 * E + e] = down[e]->qs_tiled; host_tab[5 * E + e] = down[e]->d;
     }
     if (ctx->moe_tab_host.size() != 6 * E || memcmp(ctx->moe_tab_host.data(), host_tab, 6 * E * sizeof(void *)) != 0) {
         PG_HIP(hipStreamSynchronize(ctx->stream));  // earlier calls may still read the old table
@@ -178,14 +182,14 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     auto dtable = [&](int which) { return reinterpret_cast<const uint16_t *const *>(tab + which * E); };
     // Each token reaches an expert at most once, so an expert owns at most T pairs.
     const int tiles = (int)((T + 31) / 32);
-    const pg_mm_group gg = {(int)E, table(0), dtable(1), lists, counts, (int)T, tiles, (int)T, (int)top_k};
+    const pg_mm_group gg = {(int)E, table(0), dtable(1), lists, counts, (int)T, tiles, (int)T, (int)top_k, 0, 0, 1};
     PG_TRY(pg_launch_gguf_mm(ctx, type, ffn, d, nullptr, nullptr, gg, P, xd, g, part));
-    const pg_mm_group gu = {(int)E, table(2), dtable(3), lists, counts, (int)T, tiles, (int)T, (int)top_k};
+    const pg_mm_group gu = {(int)E, table(2), dtable(3), lists, counts, (int)T, tiles, (int)T, (int)top_k, 0, 0, 1};
     PG_TRY(pg_launch_gguf_mm(ctx, type, ffn, d, nullptr, nullptr, gu, P, xd, u, part));
     PG_TRY(pg_launch(ctx, "moe_act_mul", act_mul_kernel, dim3(grid_for(P * ffn, 256)), dim3(256), 0, g, u, P * ffn,
                      act, h));
     PG_TRY(pg_launch_x_to_mm_digits(ctx, h, P, ffn, type, hd));
-    const pg_mm_group gd = {(int)E, table(4), dtable(5), lists, counts, (int)T, tiles, (int)T, 1};
+    const pg_mm_group gd = {(int)E, table(4), dtable(5), lists, counts, (int)T, tiles, (int)T, 1, 0, 0, 1};
     PG_TRY(pg_launch_gguf_mm(ctx, type, d, ffn, nullptr, nullptr, gd, P, hd, yb, part));
     return pg_launch(ctx, "moe_combine", combine_kernel, dim3(grid_for(T * d, 256)), dim3(256), 0, yb, topk_p, (int)T,
                      (int)d, (int)top_k, out_dev);
