@@ -428,19 +428,18 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
 // fill stands for (stream 16*fill + lane/4, block (lane%4) ^ ((lane/8)%4)) exactly as in the
 // kernel's fill duties; rows past n_out and blocks past k_in/32 are zeros.
 template <int QT>
-__global__ void tile_weights_kernel(const uint8_t *__restrict__ qs, int n_out, int nb, uint4 *__restrict__ tiled, size_t chunks) {
+__global__ void tile_weights_kernel(const uint8_t *__restrict__ qs, int n_out, int nb, uint8_t *__restrict__ tiled) {
     constexpr int CH = (QT == 8 ? 4096 : 2048) / 16, FILLS = CH / 64;  // chunks and fills per wavefront and stage
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= chunks) return;
-    const int lane = (int)(i & 63), q = (int)((i >> 6) % FILLS), wave = (int)((i / CH) & 3);
-    const size_t t = i / (4 * CH);
-    const int nsg = (nb + 3) / 4, sg = (int)(t % nsg), rg = (int)(t / nsg);
+    const int nsg = (nb + 3) / 4, rg = blockIdx.y;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;    // chunk within the row group
+    if (i >= (size_t)nsg * 4 * CH) return;
+    const int lane = (int)(i & 63), q = (int)((i >> 6) % FILLS), wave = (int)((i / CH) & 3), sg = (int)(i / (4 * CH));
     const int st = 16 * q + (lane >> 2), j = (lane & 3) ^ ((lane >> 3) & 3);
     const int row = rg * 128 + wave * 32 + (st & 31), half = st >> 5, block = sg * 4 + j;
     uint4 v = {0, 0, 0, 0};
     if (row < n_out && block < nb)
         v = *reinterpret_cast<const uint4 *>(qs + (QT == 8 ? ((size_t)row * 2 + half) * nb + block : (size_t)row * nb + block) * 16);
-    tiled[i] = v;
+    *reinterpret_cast<uint4 *>(tiled + rg * pg_tiled_group_bytes(nb, QT == 8) + i * 16) = v;
 }
 
 pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w) {
@@ -448,17 +447,19 @@ pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w) {
     if (w->ggml_type != PG_GGML_Q4_0 && w->ggml_type != PG_GGML_Q8_0)
         return pg_fail(PG_EUNSUPPORTED, "gguf: no tile-major copy for ggml type %d", w->ggml_type);
     const int nb = (int)(w->k_in / 32);
-    const size_t per_stage = 4 * (size_t)(w->ggml_type == PG_GGML_Q8_0 ? 4096 : 2048);
-    const size_t bytes = (w->n_out + 127) / 128 * (size_t)((nb + 3) / 4) * per_stage, chunks = bytes / 16;
+    const bool q8 = w->ggml_type == PG_GGML_Q8_0;
+    const size_t groups = (w->n_out + 127) / 128, group_bytes = pg_tiled_group_bytes(nb, q8);
+    const size_t bytes = groups * group_bytes, chunks = (group_bytes - 4352) / 16;
+    if (groups > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf: too many weight rows for a tile-major copy");
     uint8_t *p = nullptr;
     hipError_t e = hipMalloc((void **)&p, bytes);
     if (e != hipSuccess)
         return pg_fail(e == hipErrorOutOfMemory ? PG_ENOMEM : PG_EDEVICE, "gguf tile-major copy (%zu bytes): %s", bytes, hipGetErrorString(e));
-    pg_status st = w->ggml_type == PG_GGML_Q8_0
-                       ? pg_launch(ctx, "gguf_tile_weights", tile_weights_kernel<8>, dim3(grid_for(chunks, 256)), dim3(256), 0,
-                                   (const uint8_t *)w->qs, (int)w->n_out, nb, reinterpret_cast<uint4 *>(p), chunks)
-                       : pg_launch(ctx, "gguf_tile_weights", tile_weights_kernel<4>, dim3(grid_for(chunks, 256)), dim3(256), 0,
-                                   (const uint8_t *)w->qs, (int)w->n_out, nb, reinterpret_cast<uint4 *>(p), chunks);
+    const dim3 grid(grid_for(chunks, 256), (unsigned)groups);
+    pg_status st = q8 ? pg_launch(ctx, "gguf_tile_weights", tile_weights_kernel<8>, grid, dim3(256), 0, (const uint8_t *)w->qs,
+                                  (int)w->n_out, nb, p)
+                      : pg_launch(ctx, "gguf_tile_weights", tile_weights_kernel<4>, grid, dim3(256), 0, (const uint8_t *)w->qs,
+                                  (int)w->n_out, nb, p);
     if (st != PG_OK) { (void)hipFree(p); return st; }
     w->qs_tiled = p;
     return PG_OK;
@@ -477,7 +478,7 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
         pg_gemv_batch batch = {(int)m, nullptr, nullptr, nullptr, 1};
         return pg_launch_gguf_gemv(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, batch, xd, y_dev, nullptr, w->m);
     }
-    const int ks = pg_gguf_mm_splitk(ctx, w->n_out, w->k_in, (m + 31) / 32, nullptr);
+    const int ks = pg_gguf_mm_splitk(ctx, w->n_out, w->k_in, (m + 31) / 32, m, false, nullptr);
     const size_t sz_d = pg_mmdigits_bytes(m, w->k_in);
     const size_t sz_part = ks > 1 ? pg_round_up((size_t)ks * m * w->n_out * sizeof(float), 256) : 0;
     PG_TRY(pg_workspace(ctx, sz_d + sz_part, &ws));
@@ -526,7 +527,7 @@ pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, c
     const size_t sz_d = pg_mmdigits_bytes(m, k_in);
     size_t sz_part = 0;
     for (int i = 0; i < count; ++i) {
-        const int ks = pg_gguf_mm_splitk(ctx, w[i]->n_out, k_in, (m + 31) / 32, nullptr);
+        const int ks = pg_gguf_mm_splitk(ctx, w[i]->n_out, k_in, (m + 31) / 32, m, false, nullptr);
         const size_t sz = ks > 1 ? pg_round_up((size_t)ks * m * w[i]->n_out * sizeof(float), 256) : 0;
         if (sz > sz_part) sz_part = sz;
     }
@@ -541,7 +542,7 @@ pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, c
             PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, m, k_in, w[i]->ggml_type, md));
             digits_type = w[i]->ggml_type;
         }
-        const int ks = pg_gguf_mm_splitk(ctx, w[i]->n_out, k_in, (m + 31) / 32, nullptr);
+        const int ks = pg_gguf_mm_splitk(ctx, w[i]->n_out, k_in, (m + 31) / 32, m, false, nullptr);
         PG_TRY(pg_launch_gguf_mm(ctx, w[i]->ggml_type, w[i]->n_out, k_in, w[i]->qs_tiled, w[i]->d, grp, m, md, y_dev[i],
                                  ks > 1 ? part_base : nullptr));
     }

@@ -54,6 +54,15 @@ template <int QT> struct MMCfg {
 //         of the block's 16 bytes (byte i = elements 2i, 2i+1, src/gguf.rs:316-323).
 // xs[row][nbp]: block scales absmax / 32639 (NaN for a block holding NaN or inf), nbp = nb
 // rounded up to 4.  8 consecutive threads own one block (4 elements each).
+// Bytes from one activation row's digits to the next: the two planes (nb * 64 bytes) padded to
+// an odd number of 256-byte lines.  The 32 token rows of a tile are fetched at the same K
+// offset at the same time; an even (worst: power-of-two, 64 KiB at K = 32768) stride sends
+// all of them to the same memory channels.
+__host__ __device__ static inline size_t mm_row_bytes(size_t nb) {
+    const size_t lines = (nb * 64 + 255) / 256;
+    return (lines | 1) * 256;
+}
+
 template <bool NIB>
 __global__ __launch_bounds__(256) void x_to_mm_digits_kernel(const float *__restrict__ x, int nb, int nbp,
                                                              int8_t *__restrict__ digits, float *__restrict__ xs) {
@@ -86,8 +95,8 @@ __global__ __launch_bounds__(256) void x_to_mm_digits_kernel(const float *__rest
         lo[e] = ((X + 128) & 255) - 128;
         hi[e] = (X - lo[e]) >> 8;
     }
-    int8_t *d0 = digits + ((row * 2 + 0) * (size_t)nb + b) * 32;  // plane 0, block b: [half][16]
-    int8_t *d1 = digits + ((row * 2 + 1) * (size_t)nb + b) * 32;
+    int8_t *d0 = digits + row * mm_row_bytes(nb) + (size_t)b * 32;  // plane 0, block b: [half][16]
+    int8_t *d1 = d0 + (size_t)nb * 32;
     if (NIB) {
         // elements 4*sub + {0, 2} -> half 0 positions 2*sub, 2*sub+1;  {1, 3} -> half 1, same positions
 #pragma unroll
@@ -121,7 +130,7 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
 
 // grid: x = tiles of 128 weight rows, y = expert * tiles_per_expert + token tile, z = K chunk.
 // `chunk` (blocks per K chunk) is a multiple of NBU and no chunk is empty.
-// out: [gridDim.z][total pairs][n_out] (plain y when gridDim.z == 1).
+// out: [K chunks][total pairs][n_out] (plain y with one chunk).
 // (Two wavefronts per SIMD: with at most 256 registers per lane the MFMA results are written
 // to ordinary VGPRs, not to accumulation registers that would have to be copied out first.)
 template <int QT>
@@ -140,8 +149,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // 4 row groups x 8 token tiles whose weights and digits (about 3 MB) stay in that XCD's L2
     // while its 32 workgroups run: each weight row group is fetched once per 8 token tiles
     // instead of once per tile.
-    int bx = blockIdx.x, by = blockIdx.y;
-    if (grp.remap_rg) {
+    int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+    if (grp.xcd_ks) {
+        // K chunks dealt to XCDs (workgroup id % 8 = XCD): chunk z runs on the 8 / ks XCDs with
+        // id % ks == z, so an XCD's L2 holds only its chunk of the activation digits, and the
+        // workgroups of an XCD walk the row groups of one token tile after another.
+        const int xcd = blockIdx.x & 7, per = 8 / grp.xcd_ks;
+        const int j = (blockIdx.x >> 3) * per + xcd / grp.xcd_ks;
+        if (j >= grp.remap_rg * grp.remap_tiles) return;
+        bz = xcd % grp.xcd_ks;
+        bx = j % grp.remap_rg;
+        by = j / grp.remap_rg;
+    } else if (grp.remap_rg) {
         const int nrgb = (grp.remap_rg + 3) / 4, ntb = (grp.remap_tiles + 7) / 8;
         const int jj = blockIdx.x >> 3, st = (jj >> 5) * 8 + (blockIdx.x & 7), w = jj & 31;
         if (st >= nrgb * ntb) return;
@@ -183,7 +202,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int unit = (2 * wave + u) * 8 + (lane >> 3), tok = unit >> 1, pl = unit & 1;
         const int ch = (lane & 7) ^ (tok & 7);
         dig_jb[u] = ch >> 1;
-        dig_src[u] = digits + xrow_of(tok) * (size_t)nb * 64 + (size_t)pl * nb * 32 + (ch & 1) * 16;
+        dig_src[u] = digits + xrow_of(tok) * mm_row_bytes(nb) + (size_t)pl * nb * 32 + (ch & 1) * 16;
     }
     // xs: lanes 0..7 of wavefront w fetch the 4 block scales of tokens 8w .. 8w+7
     const float *xs_src = xs + xrow_of(8 * wave + (lane & 7)) * (size_t)nbp;
@@ -200,10 +219,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                    (QT == 8 ? ((size_t)wrow * 2 + (st >> 5)) * nb * 16 : (size_t)wrow * nb * 16);
         // Tile-major copy: [row group][4 blocks][wavefront][fill][lane] 16-byte chunks, the very
         // order of the fills below, padded with zero rows and blocks: a stage of a workgroup is
-        // 4 * W_WAVE contiguous bytes.
+        // 4 * W_WAVE contiguous bytes (row groups pg_tiled_group_bytes apart).
         if (grp.tiled)
             w_src[q] = reinterpret_cast<const int8_t *>(qs_any) +
-                       ((size_t)bx * ((nb + 3) / 4) * 4 + wave) * W_WAVE + q * 1024 + lane * 16;
+                       (size_t)bx * pg_tiled_group_bytes(nb, QT == 8) + wave * W_WAVE + q * 1024 + lane * 16;
     }
     // f16 scales of this wavefront's 32 rows: lane -> (group lane/16, block (lane/4)%4, dword lane%4)
     const int ngroups = (n_out + 7) / 8;
@@ -212,7 +231,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const char *d_grp = reinterpret_cast<const char *>(d_any) + (size_t)dg * nb * 16 + (lane & 3) * 4;
     const int d_jb = (lane >> 2) & 3;
 
-    const int b_begin = blockIdx.z * chunk;
+    const int b_begin = bz * chunk;
     const int b_end = b_begin + chunk < nb ? b_begin + chunk : nb;
     const int nst = (b_end - b_begin + NBU - 1) / NBU;
 
@@ -444,7 +463,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const bool tok_ok = tt * 32 + l31 < count;  // the token whose outputs this lane accumulated
         if (!tok_ok) return;
         const int pair = grp.lists ? grp.lists[(size_t)e * grp.list_stride + tt * 32 + l31] : tt * 32 + l31;
-        float *y = out + blockIdx.z * part_stride + (size_t)pair * n_out;
+        float *y = out + bz * part_stride + (size_t)pair * n_out;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const int r0 = row0 + 8 * g + 4 * hh;
@@ -464,7 +483,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // lanes hold consecutive weight rows: each token's 32 outputs leave as one 128-byte run
     const int row = row0 + l31;
     if (row >= n_out) return;
-    float *ybase = out + blockIdx.z * part_stride + row;
+    float *ybase = out + bz * part_stride + row;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int tok = 8 * (r >> 2) + 4 * hh + (r & 3);
@@ -489,7 +508,7 @@ __global__ void sum_parts_kernel(const float *__restrict__ part, size_t n, int k
 
 size_t pg_mmdigits_bytes(size_t rows, size_t k) {
     const size_t nb = k / 32, nbp = pg_round_up(nb, 4);
-    return pg_round_up(rows * nb * 64, 256) + pg_round_up(rows * nbp * sizeof(float), 256);
+    return rows * mm_row_bytes(nb) + pg_round_up(rows * nbp * sizeof(float), 256);
 }
 
 pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k) {
@@ -497,7 +516,7 @@ pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k) {
     pg_mmdigits md;
     char *p = static_cast<char *>(base);
     md.digits = reinterpret_cast<int8_t *>(p);
-    p += pg_round_up(rows * nb * 64, 256);
+    p += rows * mm_row_bytes(nb);
     md.xs = reinterpret_cast<float *>(p);
     md.rows = rows;
     md.k = k;
@@ -515,19 +534,41 @@ pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows,
     return pg_launch(ctx, "x_to_mm_digits", x_to_mm_digits_kernel<false>, grid, dim3(256), 0, x_dev, nb, nbp, md.digits, md.xs);
 }
 
-int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t groups, int *chunk_out) {
+// Digits of `act_rows` activation rows that no XCD's L2 (4 MiB) can keep while every workgroup
+// of a token tile reads them: then K is split so that a chunk's share does fit, and the chunks
+// are dealt to XCDs (see the kernel).  Without the split a K = 32768 product over 128 rows
+// fetches its 8 MiB of digits once per 128-row group: 1.2x the weight bytes in total.
+static bool digits_exceed_l2(size_t act_rows, size_t nb) { return act_rows * mm_row_bytes(nb) > (2u << 20); }
+
+int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t groups, size_t act_rows, bool grouped,
+                      int *chunk_out, bool *xcd_chunks) {
     const size_t nb = k_in / 32;
     const size_t wgs = ((n_out + 127) / 128) * (groups ? groups : 1);
-    // Two workgroups fit on a CU.  Split K only as far as every workgroup is still resident
-    // at once: a second round of workgroups would pay the start-up latency again.
-    size_t ks = 2 * (size_t)ctx->num_cu / wgs;
+    // Two workgroups fit on a CU.  A short K is split only as far as every workgroup is still
+    // resident at once: a second round of workgroups would pay the start-up latency again.
+    const size_t slots = 2 * (size_t)ctx->num_cu;
+    size_t ks = slots / wgs;
     if (ks > 8) ks = 8;
     if (ks < 1) ks = 1;
+    bool by_xcd = false;
+    // (Plain products over 16 token tiles and more are not split: they run as super-tiles.)
+    if ((grouped || groups < 16) && digits_exceed_l2(act_rows, nb)) {
+        size_t c = 2;
+        while (c < 8 && act_rows * mm_row_bytes(nb) > c * (size_t)(2u << 20)) c *= 2;
+        // worth it while the partial sums (written and read back) stay under a tenth of the weights
+        const bool cheap = c * act_rows * 8 * 10 <= nb * 34 * (grouped ? groups : 1);  // per weight row
+        if (c >= ks && nb / c >= 8 * NBU && cheap) {
+            ks = c;
+            by_xcd = true;
+        }
+    }
     size_t chunk = pg_round_up((nb + ks - 1) / ks, NBU);
     if (chunk < 2 * NBU) chunk = 2 * NBU;
-    ks = (nb + chunk - 1) / chunk;
+    const size_t ks_real = (nb + chunk - 1) / chunk;
+    if (ks_real != ks) by_xcd = false;  // the deal needs 2, 4 or 8 chunks exactly
     if (chunk_out) *chunk_out = (int)chunk;
-    return (int)ks;
+    if (xcd_chunks) *xcd_chunks = by_xcd;
+    return (int)ks_real;
 }
 
 pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,
@@ -539,7 +580,8 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
     int chunk = 0;
     const size_t gy = experts * (size_t)grp.tiles_per_expert;
     // token tiles that certainly hold work: all of them without expert lists, one per expert with
-    const int ks = pg_gguf_mm_splitk(ctx, n_out, k_in, grp.counts ? experts : gy, &chunk);
+    bool by_xcd = false;
+    const int ks = pg_gguf_mm_splitk(ctx, n_out, k_in, grp.counts ? experts : gy, md.rows, grp.counts != nullptr, &chunk, &by_xcd);
     if (ks > 1 && !part) return pg_fail(PG_EINVAL, "gguf_mm: split-K needs a partial-sum buffer");
     if (gy > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_mm: too many token tiles");
     dim3 grid(grid_for(n_out, 128), (unsigned)gy, (unsigned)ks);
@@ -550,6 +592,14 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
         g2.remap_tiles = (int)gy;
         const size_t supertiles = (size_t)((grid.x + 3) / 4) * ((gy + 7) / 8);
         grid = dim3((unsigned)((supertiles + 7) / 8 * 8 * 32), 1, 1);
+    }
+    g2.xcd_ks = 0;
+    if (by_xcd) {
+        g2.xcd_ks = ks;
+        g2.remap_rg = (int)grid.x;
+        g2.remap_tiles = (int)gy;
+        const size_t per = 8 / (size_t)ks, tiles = (size_t)grid.x * gy;
+        grid = dim3((unsigned)((tiles + per - 1) / per * 8), 1, 1);
     }
     float *dst = ks > 1 ? part : y;
     const size_t stride = total_pairs * n_out;

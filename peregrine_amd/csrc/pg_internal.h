@@ -203,7 +203,7 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
                               const uint16_t *m = nullptr);
 // Activation rows as two byte-digit planes for the matrix-core product (see pg_gguf_mm.hip).
 struct pg_mmdigits {
-    int8_t *digits;  // [rows][2 planes][k/32 blocks][2 halves][16 bytes]
+    int8_t *digits;  // [rows][2 planes][k/32 blocks][2 halves][16 bytes], rows padded to an odd number of 256-byte lines
     float *xs;       // [rows][k/32 rounded up to 4] block scales
     size_t rows, k;
 };
@@ -227,12 +227,21 @@ struct pg_mm_group {
     int x_row_div;
     int remap_rg, remap_tiles;  // set by the launcher (row groups and token tiles of an XCD-aware 1-D launch), else 0
     int tiled;                  // the qs pointers are tile-major copies (pg_gguf_tensor::qs_tiled)
+    int xcd_ks;                 // set by the launcher: K chunks dealt to XCDs (2, 4 or 8), else 0
 };
+// Bytes from one 128-row group of a tile-major copy to the next: the group's stages (16 KiB
+// each for Q8_0, 8 KiB for Q4_0) plus 4352 bytes, so that workgroups walking their groups in
+// step do not all address the same memory channels (a bare power-of-two stride would).
+__host__ __device__ static inline size_t pg_tiled_group_bytes(int nb, bool q8) {
+    return (size_t)((nb + 3) / 4) * (q8 ? 16384 : 8192) + 4352;
+}
 // Makes w->qs_tiled if it is missing (one allocation and one kernel on the context's stream).
 pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w);
 // Number of K chunks the product is split into (partial sums: [chunks][pairs][n_out] floats);
 // `groups` = token tiles that certainly hold work (all tiles of a plain product, one per expert).
-int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t groups, int *chunk_out);
+// `act_rows` = activation rows the product reads, `grouped` = with expert lists.
+int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t groups, size_t act_rows, bool grouped,
+                      int *chunk_out, bool *xcd_chunks = nullptr);
 pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,
                             const uint16_t *d, const pg_mm_group &grp, size_t total_pairs, const pg_mmdigits &md,
                             float *y, float *part);

@@ -120,7 +120,7 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     const size_t P = T * top_k;
 
     // Arena layout.
-    const int ks_up = pg_gguf_mm_splitk(ctx, ffn, d, E, nullptr), ks_down = pg_gguf_mm_splitk(ctx, d, ffn, E, nullptr);
+    const int ks_up = pg_gguf_mm_splitk(ctx, ffn, d, E, T, true, nullptr), ks_down = pg_gguf_mm_splitk(ctx, d, ffn, E, P, true, nullptr);
     const size_t part_floats = std::max(ks_up > 1 ? (size_t)ks_up * P * ffn : 0, ks_down > 1 ? (size_t)ks_down * P * d : 0);
     const size_t sz_idx = pg_round_up(P * sizeof(int), 256);
     const size_t sz_p = pg_round_up(P * sizeof(float), 256);
