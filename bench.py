@@ -160,6 +160,34 @@ def main():
                  "traffic": traffic_for("quantize_rows")}
     act_quant["frac"] = round(act_quant["achieved"] / PEAK_HBM_GBS, 4)
 
+    # Per product shape: this library's GEMM kernel beside the vendor library's int8 GEMM
+    # (torch._int_mm = hipBLASLt; same operand layouts, i32 output without the rescale) on
+    # random int8 operands.  A calibration of what int8 matrix-core code reaches on this
+    # part at these sizes, not a figure of this library.
+    vendor = []
+    for name, k, n in (("q/o_proj", 4096, 4096), ("gate/up_proj", 4096, 14336), ("down_proj", 14336, 4096)):
+        wname = {"q/o_proj": "q_proj", "gate/up_proj": "gate_proj", "down_proj": "down_proj"}[name]
+
+        def one_product():
+            check(lib.pg_matmul_quantized_dev(ctx.handle, ptr(acts[k]), M_PREFILL, k, weights[wname], ptr(outs[n]), None))
+
+        for _ in range(3):
+            one_product()
+        ours_ms = profiled(one_product, 10)["gemm_w8a8"]
+        ours_ms = ours_ms[0] * ours_ms[1] / 10  # per product (a product may run as two launches)
+        entry = {"shape": f"{name}: [{M_PREFILL}x{k}] x [{k}x{n}]", "gemm_w8a8_ms": round(ours_ms, 4),
+                 "gemm_w8a8_tops": round(2 * M_PREFILL * k * n / (ours_ms * 1e-3) / 1e12, 1)}
+        try:
+            va = torch.randint(-127, 128, (M_PREFILL, k), dtype=torch.int8, device=dev)
+            vb = torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev).t()
+            v_ms = timed(lambda: torch._int_mm(va, vb), 20, 5)
+            entry["vendor_int_mm_ms"] = round(v_ms, 4)
+            entry["vendor_int_mm_tops"] = round(2 * M_PREFILL * k * n / (v_ms * 1e-3) / 1e12, 1)
+            del va, vb
+        except Exception as exc:  # the calibration is optional
+            entry["vendor_int_mm_error"] = repr(exc)[:120]
+        vendor.append(entry)
+
     # ------------------------------------------------------------------ W8A32 (the reference's GPU numerics), gate product
     def w8a32_step():
         check(lib.pg_matmul_dequant_i8_dev(ctx.handle, ptr(acts[4096]), M_PREFILL, 4096, weights["gate_proj"], ptr(outs[14336])))
@@ -465,7 +493,7 @@ def main():
                                "each product = per-row activation quantisation + i8 GEMM + f32 rescale",
                    "m": M_PREFILL, "ops_per_step": LAYER_OPS},
         "pct_int8_mfma_peak": round(100 * tops / PEAK_INT8_TOPS, 2),
-        "roofline": roofline, "activation_quant": act_quant, "w8a32_gate": w8a32, "linear_m32": linear_m32, "decode_gemv": decode, "gguf_q4_0_gemv": gguf, "gguf_q4_0_skinny": skinny, "moe_q8_0": moe, "llama_block_q4_0": llama_block, "huffman_to_gpu": huffman,
+        "roofline": roofline, "gemm_vs_vendor_library": vendor, "activation_quant": act_quant, "w8a32_gate": w8a32, "linear_m32": linear_m32, "decode_gemv": decode, "gguf_q4_0_gemv": gguf, "gguf_q4_0_skinny": skinny, "moe_q8_0": moe, "llama_block_q4_0": llama_block, "huffman_to_gpu": huffman,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line), flush=True)
