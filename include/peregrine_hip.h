@@ -333,6 +333,7 @@ typedef struct pg_llama_block pg_llama_block; /* LlamaBlock                src/m
 #define PG_MASK_NONE 0
 #define PG_MASK_CAUSAL 1                 /* Causal { offset } */
 #define PG_MASK_CAUSAL_SLIDING_WINDOW 2  /* CausalSlidingWindow { offset, window, sink_tokens } */
+#define PG_MASK_LOCAL_GLOBAL 3           /* LocalGlobal: through pg_gqa_attention_local_global only */
 
 /* nn::RMSNorm::forward, inference path  src/nn.rs:577-652:
  *   out[r, i] = x[r, i] / sqrt(mean_i(x[r]^2) + eps) * w[i];  x, out [rows, dim]; w [dim]. */
@@ -383,6 +384,21 @@ pg_status pg_gqa_attention_dev(pg_ctx *ctx, const float *q_dev, const pg_kv_cach
                                const pg_kv_cache *v_cache, size_t num_q_heads, size_t seq_q, float scale,
                                int mask_kind, size_t offset, size_t window, size_t sink_tokens,
                                float logit_cap, float *out_dev);
+/* The same with AttentionMask::LocalGlobal { offset, local_window, global_positions }
+ * src/attention.rs:115-119, 287-299: a key is visible when it is not after the query and is
+ * either within local_window positions of it or one of the global positions (a host array
+ * in both variants; entries past the cache length never match).  The _dev variant waits
+ * for the stream once, while the positions are uploaded. */
+pg_status pg_gqa_attention_local_global(pg_ctx *ctx, const float *q, const pg_kv_cache *k_cache,
+                                        const pg_kv_cache *v_cache, size_t num_q_heads, size_t seq_q,
+                                        float scale, size_t offset, size_t local_window,
+                                        const size_t *global_positions, size_t num_global,
+                                        float logit_cap, float *out);
+pg_status pg_gqa_attention_local_global_dev(pg_ctx *ctx, const float *q_dev, const pg_kv_cache *k_cache,
+                                            const pg_kv_cache *v_cache, size_t num_q_heads, size_t seq_q,
+                                            float scale, size_t offset, size_t local_window,
+                                            const size_t *global_positions, size_t num_global,
+                                            float logit_cap, float *out_dev);
 
 /* LlamaBlock::new  src/models/llama/decoder.rs:19-47 (with LlamaAttention::new,
  * src/models/llama/attention.rs:25-48). */

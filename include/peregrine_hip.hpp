@@ -393,14 +393,18 @@ private:
 };
 using KVCache = StandardKVCache;  // src/models/llama/attention.rs:7
 
-// attention::AttentionMask  src/attention.rs:102-120 (no LocalGlobal).
+// attention::AttentionMask  src/attention.rs:102-120.
 struct AttentionMask {
     int kind = PG_MASK_NONE;
     size_t offset = 0, window = 0, sink_tokens = 0;
+    std::vector<size_t> global_positions;
     static AttentionMask None() { return {}; }
-    static AttentionMask Causal(size_t offset) { return {PG_MASK_CAUSAL, offset, 0, 0}; }
+    static AttentionMask Causal(size_t offset) { return {PG_MASK_CAUSAL, offset, 0, 0, {}}; }
     static AttentionMask CausalSlidingWindow(size_t offset, size_t window, size_t sink_tokens) {
-        return {PG_MASK_CAUSAL_SLIDING_WINDOW, offset, window, sink_tokens};
+        return {PG_MASK_CAUSAL_SLIDING_WINDOW, offset, window, sink_tokens, {}};
+    }
+    static AttentionMask LocalGlobal(size_t offset, size_t local_window, std::vector<size_t> global_positions) {
+        return {PG_MASK_LOCAL_GLOBAL, offset, local_window, 0, std::move(global_positions)};
     }
 };
 
@@ -413,6 +417,13 @@ inline void gqa_attention(const GpuContext &gpu, const std::vector<float> &q, co
         throw Panic(PG_EINVAL, "gqa_attention: num_kv_heads / head_dim differ from the cache's");
     if (q.size() != num_q_heads * seq_q * head_dim || output.size() != q.size())
         throw Panic(PG_EINVAL, "gqa_attention: q / output lengths");
+    if (mask.kind == PG_MASK_LOCAL_GLOBAL) {
+        check(pg_gqa_attention_local_global(gpu.raw(), q.data(), k_cache.handle(), v_cache.handle(), num_q_heads, seq_q, scale,
+                                            mask.offset, mask.window, mask.global_positions.data(),
+                                            mask.global_positions.size(), logit_cap, output.data()),
+              "gqa_attention");
+        return;
+    }
     check(pg_gqa_attention(gpu.raw(), q.data(), k_cache.handle(), v_cache.handle(), num_q_heads, seq_q, scale, mask.kind,
                            mask.offset, mask.window, mask.sink_tokens, logit_cap, output.data()),
           "gqa_attention");

@@ -75,14 +75,22 @@ ORC_API void orc_rope_apply(const float *x, size_t seq_len, size_t head_dim, siz
 }
 
 /* attention::is_masked                              reference: src/attention.rs:269-300
- *   mask_kind 0 None, 1 Causal{offset}, 2 CausalSlidingWindow{offset, window, sink_tokens}. */
-static int is_masked(int mask_kind, size_t offset, size_t window, size_t sink, size_t qt, size_t kt) {
+ *   mask_kind 0 None, 1 Causal{offset}, 2 CausalSlidingWindow{offset, window, sink_tokens},
+ *   3 LocalGlobal{offset, local_window = window, global_positions = gpos[0..ngpos)}. */
+static int is_masked(int mask_kind, size_t offset, size_t window, size_t sink, const size_t *gpos, size_t ngpos,
+                     size_t qt, size_t kt) {
     if (mask_kind == 0) return 0;
     const size_t query_pos = offset + qt;
     if (kt > query_pos) return 1;
     if (mask_kind == 1) return 0;
+    if (mask_kind == 3) {
+        if (query_pos - kt <= window) return 0; /* saturating_sub: kt <= query_pos here */
+        for (size_t i = 0; i < ngpos; ++i)
+            if (gpos[i] == kt) return 0;        /* global_positions.contains(&kt) */
+        return 1;
+    }
     if (kt < sink) return 0;
-    return query_pos - kt > window; /* saturating_sub: kt <= query_pos here */
+    return query_pos - kt > window;
 }
 
 /* attention::gqa_attention_cpu, non-aarch64          reference: src/attention.rs:141-265
@@ -90,9 +98,33 @@ static int is_masked(int mask_kind, size_t offset, size_t window, size_t sink, s
  *   `len` valid positions; out [seq_q, num_q_heads * head_dim], ACCUMULATED INTO (the
  *   reference adds into `output`; callers pass zeros).  logit_cap > 0 applies
  *   cap * tanh(score / cap) (PostScoreTransform::LogitCap), 0 = none. */
+static void attention_masked(const float *q, const float *k, const float *v, size_t len, size_t capacity,
+                             size_t num_q_heads, size_t num_kv_heads, size_t seq_q, size_t head_dim, float scale,
+                             int mask_kind, size_t offset, size_t window, size_t sink, const size_t *gpos, size_t ngpos,
+                             float logit_cap, float *out);
+
 ORC_API void orc_gqa_attention(const float *q, const float *k, const float *v, size_t len, size_t capacity,
                                size_t num_q_heads, size_t num_kv_heads, size_t seq_q, size_t head_dim, float scale,
                                int mask_kind, size_t offset, size_t window, size_t sink, float logit_cap, float *out) {
+    attention_masked(q, k, v, len, capacity, num_q_heads, num_kv_heads, seq_q, head_dim, scale, mask_kind, offset, window,
+                     sink, NULL, 0, logit_cap, out);
+}
+
+/* The same with AttentionMask::LocalGlobal { offset, local_window, global_positions }
+ *                                                   reference: src/attention.rs:115-119, 287-299 */
+ORC_API void orc_gqa_attention_local_global(const float *q, const float *k, const float *v, size_t len, size_t capacity,
+                                            size_t num_q_heads, size_t num_kv_heads, size_t seq_q, size_t head_dim,
+                                            float scale, size_t offset, size_t local_window,
+                                            const size_t *global_positions, size_t num_global, float logit_cap,
+                                            float *out) {
+    attention_masked(q, k, v, len, capacity, num_q_heads, num_kv_heads, seq_q, head_dim, scale, 3, offset, local_window, 0,
+                     global_positions, num_global, logit_cap, out);
+}
+
+static void attention_masked(const float *q, const float *k, const float *v, size_t len, size_t capacity,
+                             size_t num_q_heads, size_t num_kv_heads, size_t seq_q, size_t head_dim, float scale,
+                             int mask_kind, size_t offset, size_t window, size_t sink, const size_t *gpos, size_t ngpos,
+                             float logit_cap, float *out) {
     const size_t group = num_q_heads / num_kv_heads, stride = capacity * head_dim;
     float *scores = (float *)malloc((len ? len : 1) * sizeof(float));
     for (size_t qh = 0; qh < num_q_heads; ++qh) {
@@ -100,7 +132,7 @@ ORC_API void orc_gqa_attention(const float *q, const float *k, const float *v, s
         for (size_t qt = 0; qt < seq_q; ++qt) {
             const float *qs = q + qh * seq_q * head_dim + qt * head_dim;
             for (size_t kt = 0; kt < len; ++kt) {
-                if (is_masked(mask_kind, offset, window, sink, qt, kt)) {
+                if (is_masked(mask_kind, offset, window, sink, gpos, ngpos, qt, kt)) {
                     scores[kt] = -INFINITY;
                 } else {
                     const float *ks = k + kvh * stride + kt * head_dim;

@@ -17,7 +17,7 @@ PG_OK, PG_EINVAL, PG_EDEVICE, PG_ENOMEM, PG_EUNSUPPORTED = 0, 1, 2, 3, 4
 GGML_Q4_0, GGML_Q4_1, GGML_Q8_0 = 2, 3, 8
 MXFP4 = 39
 ACT_SILU, ACT_GELU_TANH = 0, 1
-MASK_NONE, MASK_CAUSAL, MASK_CAUSAL_SLIDING_WINDOW = 0, 1, 2
+MASK_NONE, MASK_CAUSAL, MASK_CAUSAL_SLIDING_WINDOW, MASK_LOCAL_GLOBAL = 0, 1, 2, 3
 
 _vp, _sz, _int = C.c_void_p, C.c_size_t, C.c_int
 _pp = C.POINTER(C.c_void_p)
@@ -116,6 +116,8 @@ SIGNATURES = {
     "pg_kv_cache_download": [_vp, _vp, _vp, _vp],
     "pg_gqa_attention": [_vp, _vp, _vp, _vp, _sz, _sz, C.c_float, _int, _sz, _sz, _sz, C.c_float, _vp],
     "pg_gqa_attention_dev": [_vp, _vp, _vp, _vp, _sz, _sz, C.c_float, _int, _sz, _sz, _sz, C.c_float, _vp],
+    "pg_gqa_attention_local_global": [_vp, _vp, _vp, _vp, _sz, _sz, C.c_float, _sz, _sz, _vp, _sz, C.c_float, _vp],
+    "pg_gqa_attention_local_global_dev": [_vp, _vp, _vp, _vp, _sz, _sz, C.c_float, _sz, _sz, _vp, _sz, C.c_float, _vp],
     "pg_llama_block_create": [_vp, _sz, _sz, _sz, _sz, _sz, _sz, C.c_float, C.c_float, _pp],
     "pg_llama_block_free": [_vp, _vp],
     "pg_llama_block_set_weights": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],

@@ -15,6 +15,7 @@
 //   q          [num_q_heads][seq_q][head_dim]; attention output [seq_q][num_q_heads * head_dim]
 #include <math.h>
 #include <new>
+#include <vector>
 #include "pg_internal.h"
 #include "pg_digits.h"
 
@@ -177,11 +178,18 @@ __global__ __launch_bounds__(128) void rope_kernel(rope_args ra) {
     }
 }
 
-__device__ __forceinline__ bool attn_masked(int mask_kind, int offset, int window, int sink, int qt, int kt) {
+// Mask kinds 0..2 as in the header; 3 = LocalGlobal (src/attention.rs:287-299): `window` is the
+// local window and bit kt of `gbits` says that key position kt is a global one.
+__device__ __forceinline__ bool attn_masked(int mask_kind, int offset, int window, int sink, const uint32_t *gbits, int qt,
+                                            int kt) {
     if (mask_kind == 0) return false;
     const int query_pos = offset + qt;
     if (kt > query_pos) return true;
     if (mask_kind == 1) return false;
+    if (mask_kind == 3) {
+        if (query_pos - kt <= window) return false;
+        return !((gbits[kt >> 5] >> (kt & 31)) & 1u);
+    }
     if (kt < sink) return false;
     return query_pos - kt > window;
 }
@@ -194,6 +202,7 @@ struct attn_args {
     int chunk, splits;                       // keys per split (the LDS score buffer holds one chunk)
     float scale, logit_cap;
     int mask_kind, offset, window, sink, accumulate;
+    const uint32_t *gbits;      // mask kind 3: one bit per key position
 };
 
 constexpr int ATT_RED = 1024;     // partial output rows: (256 / lanes) slices x (lanes * 4) dims
@@ -231,7 +240,7 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(attn_args aa) {
     for (int r = 0; r < rounds; ++r) {  // every lane runs every round: the shuffles need the whole wave
         const int kt = r * nsub + sub;
         float dot = 0.f;
-        const bool live = kt < n && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, qt, k0 + kt);
+        const bool live = kt < n && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, aa.gbits, qt, k0 + kt);
         if (live && d0 < hd) {
             const float *kr = kbase + (size_t)kt * hd + d0;
             if (vec) {
@@ -346,7 +355,7 @@ __global__ __launch_bounds__(256) void gqa_attention_short_kernel(attn_args aa) 
 #pragma unroll
     for (int u = 0; u < ATT_SHORT_ROUNDS; ++u) {
         const int kt = u * nsub + sub;
-        live[u] = kt < n && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, qt, k0 + kt);
+        live[u] = kt < n && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, aa.gbits, qt, k0 + kt);
         kv[u] = float4{0.f, 0.f, 0.f, 0.f};
         vv[u] = float4{0.f, 0.f, 0.f, 0.f};
         if (live[u] && have) {
@@ -509,7 +518,7 @@ __global__ __launch_bounds__(256) void gqa_attention_tiled_kernel(attn_args aa) 
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
             float sv = -INFINITY;
-            if (k0 + lane < kend && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, qt_of[r], k0 + lane)) {
+            if (k0 + lane < kend && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, aa.gbits, qt_of[r], k0 + lane)) {
                 sv = s[r] * aa.scale;
                 if (aa.logit_cap > 0.f) sv = aa.logit_cap * tanhf(sv / aa.logit_cap);
             }
@@ -663,7 +672,8 @@ pg_status launch_rmsnorm(pg_ctx *ctx, const float *a, const float *b, float *sum
 
 pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, const pg_kv_cache *vc, size_t nqh,
                            size_t seq_q, float scale, int mask_kind, size_t offset, size_t window, size_t sink,
-                           float logit_cap, float *out, int accumulate, const pg_xdigits *xd = nullptr, int digit_kind = 0) {
+                           float logit_cap, float *out, int accumulate, const pg_xdigits *xd = nullptr, int digit_kind = 0,
+                           const size_t *global_positions = nullptr, size_t num_global = 0) {
     // With `xd` (one-token step, accumulate == 0, head_dim % 32 == 0) the rows also, or only,
     // leave as GEMV digits of kind `digit_kind`; `out` must still be a valid buffer.
     const size_t len = kc->len, hd = kc->head_dim;
@@ -684,6 +694,7 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     aa.window = (int)(window > 0x7fffffffu ? 0x7fffffffu : window);
     aa.sink = (int)(sink > 0x7fffffffu ? 0x7fffffffu : sink);
     aa.accumulate = accumulate;
+    aa.gbits = nullptr;
     // Split the keys when the rows alone cannot fill the chip (the one-token step) or a chunk
     // would not fit the LDS score buffer.  Few rows: splits of 8 rounds of keys, which the
     // short kernel handles with every load in flight at once.
@@ -705,10 +716,23 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     }
     if (splits > (size_t)ATT_SPLITS_MAX) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: cache of %zu positions is too long", len);
     aa.chunk = (int)chunk; aa.splits = (int)splits;
-    if (splits > 1) {
+    const size_t part_bytes = splits > 1 ? pg_round_up(rows * splits * (hd + 2) * sizeof(float), 256) : 0;
+    const size_t bits_words = mask_kind == PG_MASK_LOCAL_GLOBAL ? (len + 31) / 32 : 0;
+    if (part_bytes + bits_words) {
         void *ws = nullptr;
-        PG_TRY(pg_workspace(ctx, rows * splits * (hd + 2) * sizeof(float), &ws));
-        aa.part = static_cast<float *>(ws);
+        PG_TRY(pg_workspace(ctx, part_bytes + bits_words * sizeof(uint32_t), &ws));
+        if (part_bytes) aa.part = static_cast<float *>(ws);
+        if (bits_words) {
+            // The global positions become one bit per key position (positions past the cache
+            // can never be a key).  The words are copied from this frame, hence the wait.
+            std::vector<uint32_t> bits(bits_words, 0u);
+            for (size_t i = 0; i < num_global; ++i)
+                if (global_positions[i] < len) bits[global_positions[i] >> 5] |= 1u << (global_positions[i] & 31);
+            uint32_t *dev_bits = reinterpret_cast<uint32_t *>(static_cast<char *>(ws) + part_bytes);
+            PG_HIP(hipMemcpyAsync(dev_bits, bits.data(), bits_words * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
+            PG_HIP(hipStreamSynchronize(ctx->stream));
+            aa.gbits = dev_bits;
+        }
     }
     const dim3 grid((unsigned)seq_q, (unsigned)nqh, (unsigned)splits);
     if (short_kernel) {
@@ -1012,6 +1036,42 @@ PG_API pg_status pg_gqa_attention(pg_ctx *ctx, const float *q, const pg_kv_cache
     PG_HIP(hipMemcpyAsync(dout.p, out, bytes, hipMemcpyHostToDevice, ctx->stream));
     PG_TRY(launch_attention(ctx, dq.as<float>(), k_cache, v_cache, num_q_heads, seq_q, scale, mask_kind, offset, window,
                             sink_tokens, logit_cap, dout.as<float>(), 1));
+    PG_HIP(hipMemcpyAsync(out, dout.p, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+
+PG_API pg_status pg_gqa_attention_local_global_dev(pg_ctx *ctx, const float *q_dev, const pg_kv_cache *k_cache,
+                                                   const pg_kv_cache *v_cache, size_t num_q_heads, size_t seq_q,
+                                                   float scale, size_t offset, size_t local_window,
+                                                   const size_t *global_positions, size_t num_global, float logit_cap,
+                                                   float *out_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_TRY(check_attention_args("pg_gqa_attention_local_global", k_cache, v_cache, num_q_heads, seq_q, PG_MASK_CAUSAL, offset));
+    PG_CHECK_ARG(global_positions || num_global == 0, "pg_gqa_attention_local_global: null position list");
+    if (seq_q == 0 || num_q_heads == 0) return PG_OK;
+    PG_CHECK_ARG(q_dev && out_dev, "pg_gqa_attention_local_global: null pointer");
+    return launch_attention(ctx, q_dev, k_cache, v_cache, num_q_heads, seq_q, scale, PG_MASK_LOCAL_GLOBAL, offset,
+                            local_window, 0, logit_cap, out_dev, 1, nullptr, 0, global_positions, num_global);
+}
+
+PG_API pg_status pg_gqa_attention_local_global(pg_ctx *ctx, const float *q, const pg_kv_cache *k_cache,
+                                               const pg_kv_cache *v_cache, size_t num_q_heads, size_t seq_q, float scale,
+                                               size_t offset, size_t local_window, const size_t *global_positions,
+                                               size_t num_global, float logit_cap, float *out) {
+    PG_TRY(pg_use(ctx));
+    PG_TRY(check_attention_args("pg_gqa_attention_local_global", k_cache, v_cache, num_q_heads, seq_q, PG_MASK_CAUSAL, offset));
+    PG_CHECK_ARG(global_positions || num_global == 0, "pg_gqa_attention_local_global: null position list");
+    if (seq_q == 0 || num_q_heads == 0) return PG_OK;
+    PG_CHECK_ARG(q && out, "pg_gqa_attention_local_global: null pointer");
+    const size_t bytes = num_q_heads * seq_q * k_cache->head_dim * sizeof(float);
+    pg_tmp dq, dout;
+    PG_TRY(dq.alloc(bytes));
+    PG_TRY(dout.alloc(bytes));
+    PG_HIP(hipMemcpyAsync(dq.p, q, bytes, hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(dout.p, out, bytes, hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(launch_attention(ctx, dq.as<float>(), k_cache, v_cache, num_q_heads, seq_q, scale, PG_MASK_LOCAL_GLOBAL, offset,
+                            local_window, 0, logit_cap, dout.as<float>(), 1, nullptr, 0, global_positions, num_global));
     PG_HIP(hipMemcpyAsync(out, dout.p, bytes, hipMemcpyDeviceToHost, ctx->stream));
     PG_HIP(hipStreamSynchronize(ctx->stream));
     return PG_OK;

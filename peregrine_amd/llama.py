@@ -121,11 +121,12 @@ KVCache = StandardKVCache  # src/models/llama/attention.rs:7
 
 @dataclass
 class AttentionMask:
-    """`attention::AttentionMask` (src/attention.rs:102-120) without LocalGlobal."""
+    """`attention::AttentionMask` (src/attention.rs:102-120)."""
     kind: int = _ffi.MASK_NONE
     offset: int = 0
     window: int = 0
     sink_tokens: int = 0
+    global_positions: tuple = ()
 
     @classmethod
     def none(cls):
@@ -138,6 +139,10 @@ class AttentionMask:
     @classmethod
     def causal_sliding_window(cls, offset, window, sink_tokens):
         return cls(_ffi.MASK_CAUSAL_SLIDING_WINDOW, int(offset), int(window), int(sink_tokens))
+
+    @classmethod
+    def local_global(cls, offset, local_window, global_positions):
+        return cls(_ffi.MASK_LOCAL_GLOBAL, int(offset), int(local_window), 0, tuple(int(p) for p in global_positions))
 
 
 def gqa_attention(q, k_cache, v_cache, num_q_heads, num_kv_heads, seq_q, head_dim, scale, mask, logit_cap, output, ctx=None):
@@ -153,6 +158,12 @@ def gqa_attention(q, k_cache, v_cache, num_q_heads, num_kv_heads, seq_q, head_di
     if not (isinstance(output, np.ndarray) and output.dtype == np.float32 and output.flags.c_contiguous
             and output.size == q.size):
         raise ValueError("gqa_attention: output must be a contiguous float32 array of seq_q * num_q_heads * head_dim")
+    if mask.kind == _ffi.MASK_LOCAL_GLOBAL:
+        gp = np.asarray(mask.global_positions, np.uint64)
+        _ffi.check(_ffi.lib.pg_gqa_attention_local_global(ctx.handle, _ptr(q), k_cache._h, v_cache._h, num_q_heads, seq_q,
+                                                          float(scale), mask.offset, mask.window, _ptr(gp), gp.size,
+                                                          float(logit_cap or 0.0), _ptr(output)))
+        return output
     _ffi.check(_ffi.lib.pg_gqa_attention(ctx.handle, _ptr(q), k_cache._h, v_cache._h, num_q_heads, seq_q, float(scale),
                                          mask.kind, mask.offset, mask.window, mask.sink_tokens, float(logit_cap or 0.0),
                                          _ptr(output)))

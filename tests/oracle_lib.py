@@ -168,7 +168,7 @@ def rng_normal(seed, n, mean=0.0, std=1.0):
 
 
 # ---- Llama block glue (oracle/peregrine_oracle_llama.c) ----
-for _n in ("orc_rmsnorm", "orc_rope_tables", "orc_rope_apply", "orc_gqa_attention"):
+for _n in ("orc_rmsnorm", "orc_rope_tables", "orc_rope_apply", "orc_gqa_attention", "orc_gqa_attention_local_global"):
     getattr(lib, _n).restype = None
 
 
@@ -198,6 +198,18 @@ def gqa_attention(q, k, v, length, capacity, nqh, nkvh, seq_q, hd, scale, mask_k
     lib.orc_gqa_attention(_p(_f32(q).reshape(-1)), _p(_f32(k).reshape(-1)), _p(_f32(v).reshape(-1)), _sz(length),
                           _sz(capacity), _sz(nqh), _sz(nkvh), _sz(seq_q), _sz(hd), C.c_float(scale), C.c_int(mask_kind),
                           _sz(offset), _sz(window), _sz(sink), C.c_float(logit_cap), _p(out))
+    return out
+
+
+def gqa_attention_local_global(q, k, v, length, capacity, nqh, nkvh, seq_q, hd, scale, offset, local_window,
+                               global_positions, logit_cap=0.0):
+    """AttentionMask::LocalGlobal; shapes as gqa_attention."""
+    out = np.zeros(seq_q * nqh * hd, np.float32)
+    gp = np.asarray(list(global_positions), np.uint64)
+    lib.orc_gqa_attention_local_global(_p(_f32(q).reshape(-1)), _p(_f32(k).reshape(-1)), _p(_f32(v).reshape(-1)),
+                                       _sz(length), _sz(capacity), _sz(nqh), _sz(nkvh), _sz(seq_q), _sz(hd),
+                                       C.c_float(scale), _sz(offset), _sz(local_window), _p(gp), _sz(gp.size),
+                                       C.c_float(logit_cap), _p(out))
     return out
 
 

@@ -114,8 +114,12 @@ def _attention_case(ctx, orc, nqh, nkvh, hd, seq_q, length, mask, logit_cap, see
     base = orc.rng_normal(seed + 3, seq_q * nqh * hd)            # the output is added to, not overwritten
     got = base.copy()
     llama.gqa_attention(q, cache, cache, nqh, nkvh, seq_q, hd, scale, mask, logit_cap, got, ctx)
-    want = orc.gqa_attention(q, k, v, length, length, nqh, nkvh, seq_q, hd, scale, mask.kind, mask.offset, mask.window,
-                             mask.sink_tokens, logit_cap or 0.0)
+    if mask.kind == 3:
+        want = orc.gqa_attention_local_global(q, k, v, length, length, nqh, nkvh, seq_q, hd, scale, mask.offset, mask.window,
+                                              mask.global_positions, logit_cap or 0.0)
+    else:
+        want = orc.gqa_attention(q, k, v, length, length, nqh, nkvh, seq_q, hd, scale, mask.kind, mask.offset, mask.window,
+                                 mask.sink_tokens, logit_cap or 0.0)
     H.assert_close_rel(got - base, want, RTOL_F32 * 4, "gqa_attention")   # (base + o) - base rounds once more
     return got
 
@@ -169,6 +173,23 @@ def test_gqa_attention_many_rows(ctx, orc):
     _attention_case(ctx, orc, 8, 2, 128, 67, 150, llama.AttentionMask.none(), 3.0, 65)
     _attention_case(ctx, orc, 4, 4, 256, 131, 131, llama.AttentionMask.causal(0), None, 66)
     _attention_case(ctx, orc, 16, 2, 64, 33, 200, llama.AttentionMask.causal_sliding_window(167, 40, 4), None, 67)
+
+
+def test_gqa_attention_local_global(ctx, orc):
+    """AttentionMask::LocalGlobal through each of the three kernels (few rows with key splits, the
+    generic one, the tiled one), global positions in no order, repeated and past the cache."""
+    from peregrine_amd import llama
+    M = llama.AttentionMask
+    say("attention, local + global mask")
+    _attention_case(ctx, orc, 8, 2, 32, 4, 31, M.local_global(27, 3, [0, 9, 9, 17, 400]), None, 71)
+    _attention_case(ctx, orc, 8, 2, 32, 4, 31, M.local_global(27, 0, []), 2.0, 72)
+    _attention_case(ctx, orc, 32, 8, 128, 1, 1000, M.local_global(999, 64, [0, 1, 2, 500, 731]), None, 73)
+    _attention_case(ctx, orc, 6, 3, 20, 90, 120, M.local_global(30, 5, [119, 64, 3]), None, 74)
+    _attention_case(ctx, orc, 8, 2, 128, 67, 150, M.local_global(83, 10, [149, 0, 31, 32, 33, 95]), None, 75, appends=(100, 50))
+    _attention_case(ctx, orc, 16, 2, 64, 33, 200, M.local_global(167, 1, list(range(0, 200, 7))), 3.0, 76)
+    # every position global = the causal mask, bit for bit (same kernels, same order of operations)
+    got = _attention_case(ctx, orc, 8, 2, 64, 40, 90, M.local_global(50, 0, range(90)), None, 77)
+    assert (got == _attention_case(ctx, orc, 8, 2, 64, 40, 90, M.causal(50), None, 77)).all()
 
 
 def test_gqa_attention_long_cache_splits_keys(ctx, orc):

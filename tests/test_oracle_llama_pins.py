@@ -108,6 +108,33 @@ def test_causal_masks_and_window_and_cap(orc):
         assert np.abs(out[qh] - (p / p.sum()) @ v[0, :5]).max() < 1e-5
 
 
+def test_local_global_mask(orc):
+    """AttentionMask::LocalGlobal (src/attention.rs:287-299) against an explicit visibility set
+    in float64, and its reductions: every position global, or a window as long as the cache,
+    is the causal mask; no global positions is the sliding window without sinks."""
+    hd, nqh, nkvh, cap, n = 4, 2, 1, 16, 9
+    scale = 0.5
+    q, k, v = _qkv(nqh, nkvh, 3, n, hd, cap)
+    offset, window, glob = 6, 1, [0, 3, 12]            # position 12 is past the cache: never a key
+    out = orc.gqa_attention_local_global(q, k, v, n, cap, nqh, nkvh, 3, hd, scale, offset, window, glob).reshape(3, nqh, hd)
+    for qt in range(3):
+        pos = offset + qt
+        visible = [kt for kt in range(n) if kt <= pos and (pos - kt <= window or kt in glob)]
+        assert visible == [0, 3, pos - 1, pos]
+        for qh in range(nqh):
+            s = (k[0, :n].astype(np.float64) @ q[qh, qt]) * scale
+            hidden = np.ones(n, bool)
+            hidden[visible] = False
+            s[hidden] = -np.inf
+            p = np.exp(s - s.max())
+            assert np.abs(out[qt, qh] - (p / p.sum()) @ v[0, :n]).max() < 1e-5
+    causal = orc.gqa_attention(q, k, v, n, cap, nqh, nkvh, 3, hd, scale, mask_kind=1, offset=offset)
+    assert (orc.gqa_attention_local_global(q, k, v, n, cap, nqh, nkvh, 3, hd, scale, offset, 0, range(n)) == causal).all()
+    assert (orc.gqa_attention_local_global(q, k, v, n, cap, nqh, nkvh, 3, hd, scale, offset, n, []) == causal).all()
+    window_only = orc.gqa_attention(q, k, v, n, cap, nqh, nkvh, 3, hd, scale, mask_kind=2, offset=offset, window=2, sink=0)
+    assert (orc.gqa_attention_local_global(q, k, v, n, cap, nqh, nkvh, 3, hd, scale, offset, 2, []) == window_only).all()
+
+
 def test_llama_block_against_float64_numpy(orc):
     """The block composition (decoder.rs:69-155 + attention.rs:74-212) recomputed in float64
     from the same dequantised weights: residuals, norms, RoPE positions, cache append and
