@@ -1,0 +1,111 @@
+"""Seeded random shapes through the C ABI against the CPU oracle: ragged rows, columns and
+block counts around the kernels' tile sizes (32 / 64 / 128 / 256), which the fixed shapes of
+the other files only sample.  Same bars as there: the W8A8 product bit-exact, block-dequant
+products within 1e-3, attention within 4e-5."""
+import sys
+
+import numpy as np
+import pytest
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def _pick(rng, *choices):
+    return int(rng.choice(choices))
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_w8a8_random_shapes_bit_exact(ctx, orc, seed):
+    from peregrine_amd import quant
+    rng = np.random.default_rng(seed)
+    for case in range(40):
+        m = _pick(rng, 1, 2, 3, 17, 31, 33, 63, 64, 65, 100, 129, 255, 257, 300)
+        k = _pick(rng, 1, 3, 16, 31, 64, 100, 127, 128, 129, 255, 256, 384, 500, 1000, 1024, 2050)
+        n = _pick(rng, 1, 2, 7, 31, 32, 33, 64, 100, 127, 128, 129, 255, 256, 257, 300, 511, 513)
+        say(f"w8a8 random case {case}: m={m} k={k} n={n}")
+        a = orc.rng_normal(seed * 1000 + case, m * k)
+        if rng.random() < 0.3:
+            a.reshape(m, k)[rng.integers(m)] = 0.0          # a zero row: scale 1.0
+        w = orc.rng_normal(seed * 1000 + 500 + case, k * n, 0.0, 0.02)
+        if rng.random() < 0.3:
+            w.reshape(k, n)[:, rng.integers(n)] = 0.0       # a zero column: scale 1.0
+        qt = quant.quantize_weights(w, k, n, ctx)
+        q, q_t, s = orc.quantize_weights(w, k, n)
+        assert (qt.data_i8_t == q_t).all() and (bits(qt.scales) == bits(s)).all()
+        want, _ = orc.matmul_quantized(a, m, k, q_t, s, n)
+        got = quant.matmul_quantized(a, m, k, qt, ctx)
+        assert (bits(got) == bits(want)).all()
+        qt.free_gpu()
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_gguf_matmul_random_shapes(ctx, orc, seed):
+    from peregrine_amd import gguf
+    rng = np.random.default_rng(seed)
+    for case in range(40):
+        typ = _pick(rng, 2, 8, 2, 8, 3)
+        m = _pick(rng, 1, 2, 5, 8, 9, 16, 17, 31, 32, 33, 47, 64, 65, 100)
+        nb = _pick(rng, 1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 33, 63, 64, 65, 100, 129)
+        n_out = _pick(rng, 16, 31, 64, 100, 127, 128, 129, 255, 256, 257, 300, 520)
+        k_in = nb * 32
+        say(f"gguf random case {case}: type={typ} m={m} n_out={n_out} k_in={k_in}")
+        w = orc.rng_normal(seed * 1000 + case, n_out * k_in, 0.0, 0.02)
+        if typ == 3:
+            w = w + np.float32(0.03)
+        raw = {2: H.pack_q4_0, 3: H.pack_q4_1, 8: H.pack_q8_0}[typ](w)
+        x = orc.rng_normal(seed * 1000 + 500 + case, m * k_in)
+        gw = gguf.GgufWeight(raw, typ, n_out, k_in, ctx)
+        got = gw.matmul(x, m)
+        want = orc.gguf_matmul(x, m, raw, typ, n_out, k_in)
+        for r in range(m):
+            sl = slice(r * n_out, (r + 1) * n_out)
+            H.assert_close_rel(got[sl], want[sl], 1e-3, f"row {r}")
+        gw.free()
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_attention_random_shapes_and_masks(ctx, orc, seed):
+    from peregrine_amd import llama
+    rng = np.random.default_rng(seed)
+    M = llama.AttentionMask
+    for case in range(40):
+        nkvh = _pick(rng, 1, 2, 3, 4)
+        nqh = nkvh * _pick(rng, 1, 2, 4, 8)
+        hd = _pick(rng, 4, 6, 8, 20, 32, 64, 64, 128, 128, 256)
+        seq_q = _pick(rng, 1, 1, 2, 5, 31, 32, 33, 70)
+        extra = _pick(rng, 0, 1, 7, 63, 64, 65, 200, 700)
+        length = seq_q + extra
+        kind = _pick(rng, 0, 1, 1, 2, 3)
+        offset = extra if kind else 0
+        window, sink, cap = _pick(rng, 0, 1, 5, 64, 1000), _pick(rng, 0, 1, 4), _pick(rng, 0, 0, 2)
+        glob = [int(v) for v in rng.integers(0, length + 5, size=_pick(rng, 0, 1, 5, 40))]
+        say(f"attention random case {case}: heads={nqh}/{nkvh} hd={hd} seq_q={seq_q} len={length} mask={kind} "
+            f"window={window} sink={sink} cap={cap}")
+        mask = [M.none(), M.causal(offset), M.causal_sliding_window(offset, window, sink),
+                M.local_global(offset, window, glob)][kind]
+        cache = llama.StandardKVCache(nkvh, hd, ctx)
+        k = orc.rng_normal(seed * 1000 + case, nkvh * length * hd).reshape(nkvh, length, hd)
+        v = orc.rng_normal(seed * 1000 + 300 + case, nkvh * length * hd).reshape(nkvh, length, hd)
+        cache.append(k, v, length)
+        q = orc.rng_normal(seed * 1000 + 600 + case, nqh * seq_q * hd).reshape(nqh, seq_q, hd)
+        scale = 1 / np.sqrt(hd)
+        got = np.zeros(seq_q * nqh * hd, np.float32)
+        llama.gqa_attention(q, cache, cache, nqh, nkvh, seq_q, hd, scale, mask, cap, got, ctx)
+        if kind == 3:
+            want = orc.gqa_attention_local_global(q, k, v, length, length, nqh, nkvh, seq_q, hd, scale, offset, window,
+                                                  glob, float(cap))
+        else:
+            want = orc.gqa_attention(q, k, v, length, length, nqh, nkvh, seq_q, hd, scale, kind, offset, window, sink,
+                                     float(cap))
+        H.assert_close_rel(got, want, 4e-5, "attention")
