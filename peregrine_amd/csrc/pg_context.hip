@@ -39,6 +39,15 @@ pg_status pg_launch_check(const char *what) {
     return PG_OK;
 }
 
+pg_status pg_allow_dynamic_lds(pg_ctx *ctx, const void *kernel, size_t bytes) {
+    for (const void *k : ctx->lds_raised)
+        if (k == kernel) return PG_OK;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return pg_fail(PG_EDEVICE, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    ctx->lds_raised.push_back(kernel);
+    return PG_OK;
+}
+
 pg_status pg_workspace(pg_ctx *ctx, size_t bytes, void **out) {
     if (bytes > ctx->ws_bytes) {
         // Work already queued may still use the old arena: drain before replacing it.

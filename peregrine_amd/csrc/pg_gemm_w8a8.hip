@@ -234,12 +234,7 @@ pg_status launch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *
     const int ntiles = tiles_m * tiles_n;
     const size_t lds = (size_t)NST * (BM + BN) * BK + (BM + BN) * sizeof(float);
     auto kern = gemm_w8a8_kernel<BM, BN, BK, NST, NWM, NWN, OCC>;
-    static bool attr_done = false;  // per instantiation
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return pg_fail(PG_EDEVICE, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-        attr_done = true;
-    }
+    PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
     const unsigned grid = (unsigned)(((ntiles + 7) / 8) * 8);
     PG_TRY(pg_launch(ctx, "gemm_w8a8", kern, dim3(grid), dim3(64 * NWM * NWN), lds, a_i8, (int)a_stride, w->w_t,
                      (int)w->k_pad, a_scales, w->scales, out, acc, (int)m, (int)w->cols, (int)w->k_pad, tiles_m,

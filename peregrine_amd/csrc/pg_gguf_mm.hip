@@ -604,14 +604,8 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
     float *dst = ks > 1 ? part : y;
     const size_t stride = total_pairs * n_out;
     const size_t lds = (size_t)RING * (ggml_type == PG_GGML_Q4_0 ? MMCfg<4>::STAGE : MMCfg<8>::STAGE);
-    static bool attr_set[2] = {false, false};  // per kernel instantiation
     auto launch = [&](auto kern, const char *name) -> pg_status {
-        bool &attr_done = attr_set[ggml_type == PG_GGML_Q4_0 ? 0 : 1];
-        if (!attr_done) {
-            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return pg_fail(PG_EDEVICE, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-            attr_done = true;
-        }
+        PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
         return pg_launch(ctx, name, kern, grid, dim3(256), lds, qs, d, g2, (int)n_out, nb, nbp, chunk, md.digits, md.xs, dst,
                          stride);
     };

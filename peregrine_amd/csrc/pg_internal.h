@@ -40,6 +40,8 @@ struct pg_ctx {
     std::vector<const void *> moe_tab_host;
     void *moe_tab_dev = nullptr;
     size_t moe_tab_cap = 0;
+    // Kernels whose dynamic LDS limit was raised on this context's device (pg_allow_dynamic_lds).
+    std::vector<const void *> lds_raised;
 };
 
 // Device-resident quantised weight, K-contiguous and zero-padded:
@@ -100,6 +102,9 @@ pg_status pg_use(pg_ctx *ctx);
 pg_status pg_workspace(pg_ctx *ctx, size_t bytes, void **out);
 // Check the launch just made.
 pg_status pg_launch_check(const char *what);
+// Let `kernel` use `bytes` of dynamic LDS on this context's device (the attribute is set once
+// per context: it belongs to the device's copy of the kernel).
+pg_status pg_allow_dynamic_lds(pg_ctx *ctx, const void *kernel, size_t bytes);
 
 // Launch `kernel` on the context's stream.  While profiling (pg_profile_begin/end) the
 // dispatch carries a start and a stop event: hipExtLaunchKernel stamps them with the

@@ -746,12 +746,7 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
         const dim3 grid_t((unsigned)row_sets, (unsigned)kc->num_kv_heads);
         auto *kern = hd == 64 ? gqa_attention_tiled_kernel<64> : (hd == 128 ? gqa_attention_tiled_kernel<128> : gqa_attention_tiled_kernel<256>);
         const size_t lds_t = hd == 64 ? att_tiled_lds<64>() : (hd == 128 ? att_tiled_lds<128>() : att_tiled_lds<256>());
-        static bool attr_done[3] = {false, false, false};
-        bool &done = attr_done[hd == 64 ? 0 : (hd == 128 ? 1 : 2)];
-        if (!done) {
-            PG_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_t));
-            done = true;
-        }
+        PG_TRY(pg_allow_dynamic_lds(ctx, reinterpret_cast<const void *>(kern), lds_t));
         PG_TRY(pg_launch(ctx, "gqa_attention_tiled", kern, grid_t, dim3(256), lds_t, aa));
     } else
         PG_TRY(pg_launch(ctx, "gqa_attention", gqa_attention_kernel, grid, dim3(256), (256 + ATT_RED + chunk) * sizeof(float), aa));
