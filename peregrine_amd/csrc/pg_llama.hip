@@ -203,6 +203,12 @@ struct attn_args {
     float scale, logit_cap;
     int mask_kind, offset, window, sink, accumulate;
     const uint32_t *gbits;      // mask kind 3: one bit per key position
+    // One-token step with RoPE and the cache append folded in (short kernel only; null raw_q =
+    // off): q, k, v as the projections left them ([heads, hd] each), the cos / sin rows of the
+    // new position, and where its rotated key and its value belong in the caches.
+    const float *raw_q, *raw_k, *raw_v, *rope_c, *rope_s;
+    float *k_new, *v_new;       // cache rows of position new_pos, kv head 0
+    int new_pos;
 };
 
 constexpr int ATT_RED = 1024;     // partial output rows: (256 / lanes) slices x (lanes * 4) dims
@@ -349,9 +355,26 @@ __global__ __launch_bounds__(256) void gqa_attention_short_kernel(attn_args aa) 
         }
         return r;
     };
+    // This lane's four dims of a head row after RoPE (pairs (i, i + hd/2), the operations of
+    // rope_kernel in the same order); hd is a multiple of 8 on this route.
+    const bool fused = aa.raw_q != nullptr;
+    auto rot4 = [&](const float *row) {
+        const int half = hd >> 1, i0 = d0 < half ? d0 : d0 - half;
+        const float4 x0 = *reinterpret_cast<const float4 *>(row + i0), x1 = *reinterpret_cast<const float4 *>(row + half + i0);
+        const float4 c = *reinterpret_cast<const float4 *>(aa.rope_c + i0), sn = *reinterpret_cast<const float4 *>(aa.rope_s + i0);
+        float4 r;
+        if (d0 < half) {
+            r.x = x0.x * c.x - x1.x * sn.x; r.y = x0.y * c.y - x1.y * sn.y;
+            r.z = x0.z * c.z - x1.z * sn.z; r.w = x0.w * c.w - x1.w * sn.w;
+        } else {
+            r.x = x0.x * sn.x + x1.x * c.x; r.y = x0.y * sn.y + x1.y * c.y;
+            r.z = x0.z * sn.z + x1.z * c.z; r.w = x0.w * sn.w + x1.w * c.w;
+        }
+        return r;
+    };
     float4 q4 = {0.f, 0.f, 0.f, 0.f}, kv[ATT_SHORT_ROUNDS], vv[ATT_SHORT_ROUNDS];
     bool live[ATT_SHORT_ROUNDS];
-    if (have) q4 = load4(qsrc);
+    if (have) q4 = fused ? rot4(aa.raw_q + (size_t)qh * hd) : load4(qsrc);
 #pragma unroll
     for (int u = 0; u < ATT_SHORT_ROUNDS; ++u) {
         const int kt = u * nsub + sub;
@@ -359,8 +382,19 @@ __global__ __launch_bounds__(256) void gqa_attention_short_kernel(attn_args aa) 
         kv[u] = float4{0.f, 0.f, 0.f, 0.f};
         vv[u] = float4{0.f, 0.f, 0.f, 0.f};
         if (live[u] && have) {
-            kv[u] = load4(kbase + (size_t)kt * hd);
-            vv[u] = load4(vbase + (size_t)kt * hd);
+            if (fused && k0 + kt == aa.new_pos) {
+                // The new position is not in the cache yet: every workgroup that needs it makes
+                // it from the projections, and the first member of the key set also stores it.
+                kv[u] = rot4(aa.raw_k + (size_t)kvh * hd);
+                vv[u] = *reinterpret_cast<const float4 *>(aa.raw_v + (size_t)kvh * hd + d0);
+                if (member == 0) {
+                    *reinterpret_cast<float4 *>(aa.k_new + (size_t)kvh * aa.k_stride + d0) = kv[u];
+                    *reinterpret_cast<float4 *>(aa.v_new + (size_t)kvh * aa.v_stride + d0) = vv[u];
+                }
+            } else {
+                kv[u] = load4(kbase + (size_t)kt * hd);
+                vv[u] = load4(vbase + (size_t)kt * hd);
+            }
         }
     }
     float s[ATT_SHORT_ROUNDS], mx = -INFINITY;
@@ -670,10 +704,20 @@ pg_status launch_rmsnorm(pg_ctx *ctx, const float *a, const float *b, float *sum
                      (int)dim, out);
 }
 
+// Whether launch_attention takes the one-token kernel for `rows` (token, head) rows over `len` keys.
+bool attention_is_short(const pg_ctx *ctx, size_t rows, size_t len, size_t hd) {
+    size_t lanes = 1;
+    while (lanes * 4 < hd) lanes <<= 1;
+    const size_t keys_per_round = 256 / lanes;
+    return rows < 2 * (size_t)ctx->num_cu &&
+           (len + ATT_SHORT_ROUNDS * keys_per_round - 1) / (ATT_SHORT_ROUNDS * keys_per_round) <= (size_t)ATT_SPLITS_MAX;
+}
+
 pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, const pg_kv_cache *vc, size_t nqh,
                            size_t seq_q, float scale, int mask_kind, size_t offset, size_t window, size_t sink,
                            float logit_cap, float *out, int accumulate, const pg_xdigits *xd = nullptr, int digit_kind = 0,
-                           const size_t *global_positions = nullptr, size_t num_global = 0) {
+                           const size_t *global_positions = nullptr, size_t num_global = 0,
+                           const attn_args *rope_fusion = nullptr) {
     // With `xd` (one-token step, accumulate == 0, head_dim % 32 == 0) the rows also, or only,
     // leave as GEMV digits of kind `digit_kind`; `out` must still be a valid buffer.
     const size_t len = kc->len, hd = kc->head_dim;
@@ -695,13 +739,16 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     aa.sink = (int)(sink > 0x7fffffffu ? 0x7fffffffu : sink);
     aa.accumulate = accumulate;
     aa.gbits = nullptr;
+    aa.raw_q = aa.raw_k = aa.raw_v = aa.rope_c = aa.rope_s = nullptr;
+    aa.k_new = aa.v_new = nullptr;
+    aa.new_pos = -1;
     // Split the keys when the rows alone cannot fill the chip (the one-token step) or a chunk
     // would not fit the LDS score buffer.  Few rows: splits of 8 rounds of keys, which the
     // short kernel handles with every load in flight at once.
     const size_t rows = seq_q * nqh, keys_per_round = 256 / (size_t)lanes;
     size_t chunk, splits;
     bool short_kernel = false, tiled_kernel = false;
-    if (rows < 2 * (size_t)ctx->num_cu && (len + ATT_SHORT_ROUNDS * keys_per_round - 1) / (ATT_SHORT_ROUNDS * keys_per_round) <= (size_t)ATT_SPLITS_MAX) {
+    if (attention_is_short(ctx, rows, len, hd)) {
         chunk = ATT_SHORT_ROUNDS * keys_per_round;
         splits = (len + chunk - 1) / chunk;
         short_kernel = true;
@@ -735,6 +782,13 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
         }
     }
     const dim3 grid((unsigned)seq_q, (unsigned)nqh, (unsigned)splits);
+    if (rope_fusion) {
+        if (!short_kernel || seq_q != 1 || hd % 8 != 0) return pg_fail(PG_EINVAL, "gqa_attention: RoPE fusion needs the one-token kernel");
+        aa.raw_q = rope_fusion->raw_q; aa.raw_k = rope_fusion->raw_k; aa.raw_v = rope_fusion->raw_v;
+        aa.rope_c = rope_fusion->rope_c; aa.rope_s = rope_fusion->rope_s;
+        aa.k_new = rope_fusion->k_new; aa.v_new = rope_fusion->v_new;
+        aa.new_pos = rope_fusion->new_pos;
+    }
     if (short_kernel) {
         const size_t sets = kc->num_kv_heads * splits, members = (nqh / kc->num_kv_heads) * seq_q;
         const size_t wgs = (sets + 7) / 8 * 8 * members;
@@ -1204,7 +1258,8 @@ PG_API pg_status pg_llama_block_set_weights(pg_ctx *ctx, pg_llama_block *b, cons
 
 // The one-token step: every producer of a GEMV input writes digits instead of f32 (RMSNorm,
 // the attention merge, SiLU·up), k/v and gate/up each run as one two-item launch, and the
-// second residual add is the down projection's epilogue: 11 launches instead of 18.
+// second residual add is the down projection's epilogue, RoPE and the cache append ride in the
+// attention kernel: 9 launches instead of 18.
 static pg_status block_forward_one_token(pg_ctx *ctx, pg_llama_block *b, const float *h_dev, pg_kv_cache *cache,
                                          float *out_dev) {
     const size_t d = b->d, hd = b->hd, q_dim = b->nqh * hd, kv_dim = b->nkvh * hd, ffn = b->ffn, offset = cache->len;
@@ -1236,15 +1291,28 @@ static pg_status block_forward_one_token(pg_ctx *ctx, pg_llama_block *b, const f
         PG_TRY(pg_launch_gguf_gemv(ctx, b->w[2]->ggml_type, kv_dim, d, b->w[2]->qs, b->w[2]->d, one, b->xd_d, vd));
     }
     PG_TRY(cache_reserve(ctx, cache, offset + 1));
-    rope_args ra = {};
-    ra.seg[0] = {qd, q_rope, q_dim, hd, (int)b->nqh, 1};
-    ra.seg[1] = {kd, cache->k + offset * hd, kv_dim, cache->capacity * hd, (int)b->nkvh, 1};
-    ra.seg[2] = {vd, cache->v + offset * hd, kv_dim, cache->capacity * hd, (int)b->nkvh, 0};
-    ra.cos_t = b->rope->cos_t; ra.sin_t = b->rope->sin_t; ra.hd = (int)hd; ra.pos0 = (int)offset; ra.nseg = 3;
-    PG_TRY(launch_rope(ctx, ra, 1, b->nqh + 2 * b->nkvh));
-    cache->len = offset + 1;
-    PG_TRY(launch_attention(ctx, q_rope, cache, cache, b->nqh, 1, 1.0f / sqrtf((float)hd), PG_MASK_CAUSAL, offset, 0, 0, 0.0f,
-                            attn, 0, &b->xd_q, kind));
+    if (attention_is_short(ctx, b->nqh, offset + 1, hd)) {
+        // RoPE of q and of the new key, and the append of the new key and value, happen inside
+        // the attention kernel: one launch less.
+        attn_args fuse = {};
+        fuse.raw_q = qd; fuse.raw_k = kd; fuse.raw_v = vd;
+        fuse.rope_c = b->rope->cos_t + offset * hd; fuse.rope_s = b->rope->sin_t + offset * hd;
+        fuse.k_new = cache->k + offset * hd; fuse.v_new = cache->v + offset * hd;
+        fuse.new_pos = (int)offset;
+        cache->len = offset + 1;
+        PG_TRY(launch_attention(ctx, qd, cache, cache, b->nqh, 1, 1.0f / sqrtf((float)hd), PG_MASK_CAUSAL, offset, 0, 0, 0.0f,
+                                attn, 0, &b->xd_q, kind, nullptr, 0, &fuse));
+    } else {
+        rope_args ra = {};
+        ra.seg[0] = {qd, q_rope, q_dim, hd, (int)b->nqh, 1};
+        ra.seg[1] = {kd, cache->k + offset * hd, kv_dim, cache->capacity * hd, (int)b->nkvh, 1};
+        ra.seg[2] = {vd, cache->v + offset * hd, kv_dim, cache->capacity * hd, (int)b->nkvh, 0};
+        ra.cos_t = b->rope->cos_t; ra.sin_t = b->rope->sin_t; ra.hd = (int)hd; ra.pos0 = (int)offset; ra.nseg = 3;
+        PG_TRY(launch_rope(ctx, ra, 1, b->nqh + 2 * b->nkvh));
+        cache->len = offset + 1;
+        PG_TRY(launch_attention(ctx, q_rope, cache, cache, b->nqh, 1, 1.0f / sqrtf((float)hd), PG_MASK_CAUSAL, offset, 0, 0, 0.0f,
+                                attn, 0, &b->xd_q, kind));
+    }
     // h1 = h + attn . Wo
     PG_TRY(pg_launch_gguf_gemv(ctx, b->w[3]->ggml_type, d, q_dim, b->w[3]->qs, b->w[3]->d, one, b->xd_q, h1, h_dev));
     PG_TRY(launch_rmsnorm_digits(ctx, h1, nullptr, nullptr, b->ffn_norm_w, b->eps, 1, d, kind, b->xd_d));
