@@ -204,6 +204,29 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__res
     // ---- epilogue.  Accumulator register r of a 32x32 tile holds
     // row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.  (The scales were requested before the
     // K loop: loading them here would put several dependent memory round trips on every tile.)
+    if (out && !acc_out && m0 + BM <= M && n0 + BN <= N) {
+        // A whole tile inside the matrix, f32 output only (every tile of the prefill shapes):
+        // straight-line code, the 16 row scales of a 32-row tile as four 128-bit LDS reads.
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            float as[16];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 v = *reinterpret_cast<const float4 *>(lds_as + wm * WM + 32 * i + 8 * g + 4 * half);
+                as[4 * g] = v.x; as[4 * g + 1] = v.y; as[4 * g + 2] = v.z; as[4 * g + 3] = v.w;
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const float ws = lds_ws[wn * WN + 32 * j + l31];
+                float *dst = out + (size_t)(m0 + wm * WM + 32 * i + 4 * half) * N + (n0 + wn * WN + 32 * j + l31);
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    dst[(size_t)(8 * (r >> 2) + (r & 3)) * N] = (float)acc[i][j][r] * as[r] * ws;
+                __builtin_amdgcn_sched_barrier(0);  // one tile's stores at a time: bounded live ranges
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
