@@ -285,5 +285,8 @@ pg_status pg_launch_gemm_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
     if (m <= 64) return launch<64, 64, 128, 2, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
     if (tiles(256, 256) * 2 >= 3 * cus) return launch<256, 256, 128, 2, 2, 4, 2>(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
     if (tiles(128, 256) >= cus) return launch<128, 256, 128, 2, 2, 4, 2>(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
+    // Too few 128x128 tiles for the CUs (k/v projections, N = 1024): halve the tile instead of leaving
+    // half of the chip idle (21.2 -> 16.5 us at 2048 x 4096 -> 1024).
+    if (tiles(128, 128) < cus) return launch<128, 64, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
     return launch<128, 128, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
 }
