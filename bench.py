@@ -35,6 +35,7 @@ M_PREFILL = 2048
 LAYER = [("q_proj", 4096, 4096), ("k_proj", 4096, 1024), ("v_proj", 4096, 1024), ("o_proj", 4096, 4096),
          ("gate_proj", 4096, 14336), ("up_proj", 4096, 14336), ("down_proj", 14336, 4096)]
 LAYER_OPS = sum(2 * M_PREFILL * k * n for _, k, n in LAYER)  # 893 353 197 568
+SETTLE_S = 0.2  # untimed run of the headline step before its warm-up, seconds
 
 
 def load_traffic():
@@ -131,15 +132,30 @@ def main():
         return TRAFFIC.get(kernel)
 
     # ------------------------------------------------------------------ prefill (headline)
-    weights = {name: make_weight(k, n) for name, k, n in LAYER}
+    # Two layers' worth of weights (436 MB), used alternately: more than the 256 MB Infinity Cache
+    # holds, so every step streams its weights from HBM as a model with many layers would
+    # (with one set reused every step the layer runs about 3 % faster).
+    weight_sets = [{name: make_weight(k, n) for name, k, n in LAYER} for _ in range(2)]
+    weights = weight_sets[0]
+    prefill_state = {"i": 0}
     acts = {4096: make_acts(M_PREFILL, 4096), 14336: make_acts(M_PREFILL, 14336)}
     outs = {n: torch.empty(M_PREFILL, n, device=dev, dtype=torch.float32) for n in (4096, 1024, 14336)}
 
     def prefill_step():
+        ws = weight_sets[prefill_state["i"] % len(weight_sets)]
+        prefill_state["i"] += 1
         for name, k, n in LAYER:
-            check(lib.pg_matmul_quantized_dev(ctx.handle, ptr(acts[k]), M_PREFILL, k, weights[name],
+            check(lib.pg_matmul_quantized_dev(ctx.handle, ptr(acts[k]), M_PREFILL, k, ws[name],
                                               ptr(outs[n]), None))
 
+    # Clocks and caches need tens of milliseconds of this work to settle (a 3 ms warm-up leaves
+    # the layer about 8 % slower than its steady state): run it untimed for SETTLE_S first, then
+    # the W warm-up steps and the K timed ones as asked.
+    t_settle = time.time()
+    while time.time() - t_settle < SETTLE_S:
+        for _ in range(10):
+            prefill_step()
+        torch.cuda.synchronize()
     ms_step = timed(prefill_step, args.steps, args.warmup)
     tops = LAYER_OPS / (ms_step * 1e-3) / 1e12
     prof = profiled(prefill_step, args.steps)
@@ -209,8 +225,9 @@ def main():
                                           C.c_void_p(sc.ctypes.data)))
             cpu_w[name] = (qt, sc)
         cpu_a = {k: acts[k].cpu().numpy().copy() for k in acts}
-    for h in weights.values():
-        lib.pg_qtensor_free(ctx.handle, h)
+    for ws in weight_sets:
+        for h in ws.values():
+            lib.pg_qtensor_free(ctx.handle, h)
     del acts, outs
     torch.cuda.empty_cache()
 
@@ -489,9 +506,9 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": "cfg3: W8A8 prefill GEMMs of one Llama-3-8B layer at M=2048 "
                                "(q 4096->4096, k/v 4096->1024, o 4096->4096, gate/up 4096->14336, down 14336->4096), "
-                               "activations N(0,1) with 1% channels x20, weights N(0,0.02), "
+                               "activations N(0,1) with 1% channels x20, weights N(0,0.02), two weight sets (436 MB) alternated so that they stream from HBM, "
                                "each product = per-row activation quantisation + i8 GEMM + f32 rescale",
-                   "m": M_PREFILL, "ops_per_step": LAYER_OPS},
+                   "m": M_PREFILL, "ops_per_step": LAYER_OPS, "untimed_settle_s": SETTLE_S},
         "pct_int8_mfma_peak": round(100 * tops / PEAK_INT8_TOPS, 2),
         "roofline": roofline, "gemm_vs_vendor_library": vendor, "activation_quant": act_quant, "w8a32_gate": w8a32, "linear_m32": linear_m32, "decode_gemv": decode, "gguf_q4_0_gemv": gguf, "gguf_q4_0_skinny": skinny, "moe_q8_0": moe, "llama_block_q4_0": llama_block, "huffman_to_gpu": huffman,
         "cpu_baseline": cpu,
