@@ -6,7 +6,9 @@
 Prints ONE JSON line.  Headline (`value`): W8A8 prefill GEMM throughput, in TOP/s, over the
 seven projections of one Llama-3-8B layer at M = 2048 tokens (q, k, v, o, gate, up, down;
 893 353 197 568 integer ops per step), each through `pg_matmul_quantized_dev` (per-row
-activation quantisation + i8 MFMA GEMM + f32 rescale), inputs resident in HBM.
+activation quantisation + i8 MFMA GEMM + f32 rescale), inputs resident in HBM: two sets of
+layer weights (436 MB, more than the Infinity Cache) are used alternately, and the step runs
+untimed for 0.2 s before the W warm-up steps so that clocks and caches have settled.
 The same line carries the decode leg of the metric (`decode_gemv`: M = 1 int8 GEMV GB/s at
 the 8B FFN shapes, weights rotated through more distinct buffers than the 256 MB Infinity
 Cache holds), the Q4_0 decode GEMV (`gguf_q4_0_gemv`), a `roofline` object per dominant
