@@ -54,7 +54,10 @@ __global__ __launch_bounds__(QA_THREADS) void quantize_rows_vec4_kernel(
     for (int i = 0; i < MAXV; ++i) {
         const int idx = threadIdx.x + i * QA_THREADS;
         typedef float f4v __attribute__((ext_vector_type(4)));
-        const f4v t = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(ar) + (idx < nvec ? idx : nvec - 1));
+        // (a plain load: the activations of a layer are read by several products in a row and
+        // are usually still in the Infinity Cache; a non-temporal load would fetch them from HBM
+        // every time)
+        const f4v t = *(reinterpret_cast<const f4v *>(ar) + (idx < nvec ? idx : nvec - 1));
         v[i] = make_float4(t.x, t.y, t.z, t.w);
     }
     float amax = 0.0f;
