@@ -369,7 +369,7 @@ def main():
 
     moe_bytes = 3 * E_moe * nblk * 34 + 2 * 4 * T_moe * d_moe  # every expert is hit at T=64, k=2 (checked below)
     hit = int(torch.unique(torch.topk(lg_moe, topk_moe, dim=1).indices).numel())
-    moe_ms = timed(moe_step, 5, 2)
+    moe_ms = timed(moe_step, 20, 10)  # 5 GB of weights: the first passes also warm the TLBs
     prof = profiled(moe_step, 5)
     mm_total = prof["gguf_mm_q8_0"][0] * prof["gguf_mm_q8_0"][1] / 5  # three launches per step
     moe = {"workload": "cfg5: Grok-1-shaped MoE FFN, Q8_0 experts (d 6144, ffn 32768, 8 experts, top-2, 64 tokens, SiLU); "
@@ -431,7 +431,7 @@ def main():
         check(lib.pg_kv_cache_rollback_to(kv, ctx_len))
         check(lib.pg_llama_block_forward_dev(ctx.handle, b, ptr(h_dec), 1, kv, ptr(o_dec)))
 
-    pre_ms = timed(block_prefill, 8, 4)  # leaves every cache filled to ctx_len
+    pre_ms = timed(block_prefill, 16, 8)  # leaves every cache filled to ctx_len
     pre_prof = profiled(block_prefill, 8)
     dec_ms = timed(block_decode, dsteps, max(args.warmup, 8))
     dec_prof = profiled(block_decode, dsteps)
