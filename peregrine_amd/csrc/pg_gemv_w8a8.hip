@@ -8,6 +8,7 @@
 // Integer sums are exact, so the lane/chunk order does not matter; the f32
 // epilogue keeps the reference's multiplication order (src/quant.rs:163).
 #include "pg_internal.h"
+#include "pg_quant_dev.h"
 
 namespace {
 
@@ -123,6 +124,92 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_kernel(
     }
 }
 
+// The same with the activation row still in f32 (quant::quantize_activations for one row,
+// src/quant.rs:79-112, folded in): the workgroup requests its first weight rows, then finds the
+// row's absmax, rounds the row to i8 into LDS with the arithmetic of quantize_rows_vec4_kernel
+// (same scale, same reciprocal, same rounding: bit-identical integers), and every lane takes its
+// chunks from there.  One launch per product instead of two: the separate one-row quantisation
+// kernel costs about 4 us, as much as a third of the product itself.  k % 4 == 0.
+template <int NCH, int RPW>
+__global__ __launch_bounds__(256) void gemv_w8a8_m1_f32x_kernel(
+    const int8_t *__restrict__ w_t, int k_pad, const float *__restrict__ w_scales,
+    const float *__restrict__ x_f32, int k, int n, float *__restrict__ out, int32_t *__restrict__ acc_out) {
+    __shared__ int xq[NCH * 256];  // the quantised row, zero beyond k: NCH KiB >= k_pad bytes
+    __shared__ float red[4];
+    const int nchunk = k_pad >> 4;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row0 = (blockIdx.x * 4 + wave) * RPW;
+    auto load_row = [&](int row, v4i (&w)[NCH]) {
+        const v4i *wp = reinterpret_cast<const v4i *>(w_t + (size_t)row * k_pad);
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            const int c = lane + 64 * j;
+            w[j] = __builtin_nontemporal_load(wp + (c < nchunk ? c : lane));
+        }
+    };
+    v4i w[NCH];
+    load_row(row0, w);  // in flight while the activations are prepared
+
+    const int nvec = k >> 2;
+    const float4 *x4 = reinterpret_cast<const float4 *>(x_f32);
+    float4 v[NCH];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int idx = threadIdx.x + 256 * i;
+        v[i] = x4[idx < nvec ? idx : nvec - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int idx = threadIdx.x + 256 * i;
+        const float m4 = fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)), fmaxf(fabsf(v[i].z), fabsf(v[i].w)));
+        amax = fmaxf(amax, idx < nvec ? m4 : 0.0f);
+    }
+    amax = pg_block_max_256(amax, red);
+    const float a_scale = (amax == 0.0f) ? 1.0f : amax / 127.0f;
+    const float inv_scale = 1.0f / a_scale;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int idx = threadIdx.x + 256 * i;
+        const int b0 = pg_quant_to_i8(v[i].x * inv_scale) & 0xFF;
+        const int b1 = pg_quant_to_i8(v[i].y * inv_scale) & 0xFF;
+        const int b2 = pg_quant_to_i8(v[i].z * inv_scale) & 0xFF;
+        const int b3 = pg_quant_to_i8(v[i].w * inv_scale) & 0xFF;
+        xq[idx] = idx < nvec ? (b0 | (b1 << 8) | (b2 << 16) | (b3 << 24)) : 0;
+    }
+    __syncthreads();
+    v4i x[NCH];
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) x[j] = reinterpret_cast<const v4i *>(xq)[lane + 64 * j];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+        const int row = row0 + r;  // < n_pad by construction of the grid
+        if (r > 0) load_row(row, w);
+        int acc = 0;
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) acc = dot16(w[j], x[j], acc);  // x is zero beyond k
+        acc = wave_sum_i32(acc);
+        if (lane == 0 && row < n) {
+            if (out) out[row] = (float)acc * a_scale * w_scales[row];
+            if (acc_out) acc_out[row] = acc;
+        }
+    }
+}
+
+template <int NCH, int RPW>
+pg_status launch_m1_f32x(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *w, float *out, int32_t *acc) {
+    const unsigned grid = (unsigned)(w->n_pad / (4 * RPW));
+    PG_TRY(pg_launch(ctx, "gemv_w8a8", gemv_w8a8_m1_f32x_kernel<NCH, RPW>, dim3(grid), dim3(256), 0, w->w_t,
+                     (int)w->k_pad, w->scales, x_f32, (int)k, (int)w->cols, out, acc));
+    return pg_launch_check("gemv_w8a8_m1_f32x");
+}
+
+template <int NCH>
+pg_status launch_m1_f32x_rows(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *w, float *out, int32_t *acc) {
+    if (w->n_pad / 2 >= (size_t)ctx->num_cu * 8) return launch_m1_f32x<NCH, 2>(ctx, x_f32, k, w, out, acc);
+    return launch_m1_f32x<NCH, 1>(ctx, x_f32, k, w, out, acc);
+}
+
 template <int NCH, int RPW>
 pg_status launch_m1(pg_ctx *ctx, const int8_t *a_i8, const float *a_scales, const pg_qtensor *w,
                     float *out, int32_t *acc) {
@@ -166,6 +253,19 @@ pg_status launch_m(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float
 }
 
 }  // namespace
+
+bool pg_gemv_w8a8_takes_f32_row(const pg_qtensor *w, size_t m, size_t k, const float *x_f32) {
+    return m == 1 && w->k_pad <= 16384 && k % 4 == 0 && k > 0 && (uintptr_t)x_f32 % 16 == 0;  // 128-bit loads of the row
+}
+
+pg_status pg_launch_gemv_w8a8_f32_row(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *w, float *out,
+                                      int32_t *acc) {
+    const size_t nch = (w->k_pad / 16 + 63) / 64;
+    if (nch <= 4) return launch_m1_f32x_rows<4>(ctx, x_f32, k, w, out, acc);
+    if (nch <= 8) return launch_m1_f32x_rows<8>(ctx, x_f32, k, w, out, acc);
+    if (nch <= 14) return launch_m1_f32x_rows<14>(ctx, x_f32, k, w, out, acc);
+    return launch_m1_f32x_rows<16>(ctx, x_f32, k, w, out, acc);
+}
 
 pg_status pg_launch_gemv_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
                               const float *a_scales, const pg_qtensor *w, size_t m, float *out,

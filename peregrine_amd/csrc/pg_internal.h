@@ -154,6 +154,11 @@ pg_status pg_launch_gemm_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
 pg_status pg_launch_gemv_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
                               const float *a_scales, const pg_qtensor *w, size_t m,
                               float *out, int32_t *acc);
+// One activation row still in f32: quantised inside the product's own launch (same integers and
+// scale as pg_launch_quantize_activations would give).  Only where the predicate holds.
+bool pg_gemv_w8a8_takes_f32_row(const pg_qtensor *w, size_t m, size_t k, const float *x_f32);
+pg_status pg_launch_gemv_w8a8_f32_row(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *w, float *out,
+                                      int32_t *acc);
 // Activation rows rewritten as three byte-digit planes (see pg_gguf.hip).
 struct pg_xdigits {
     int8_t *digits;  // [rows][6 planes][k/32 blocks][16 bytes] (Q4_0 uses 5 planes, Q8_0 all 6)

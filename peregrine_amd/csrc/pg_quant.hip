@@ -9,32 +9,15 @@
 //    and hipcc's default correctly-rounded f32 divide is relied on.
 #include <new>
 #include "pg_internal.h"
+#include "pg_quant_dev.h"
 
 namespace {
 
 constexpr int QA_THREADS = 256;
 
-// round -> clamp(-127,127) -> `as i8` (NaN -> 0), returned as int.
-__device__ __forceinline__ int quant_to_i8(float v) {
-    float r = roundf(v);
-    r = fminf(fmaxf(r, -127.0f), 127.0f);
-    return (r != r || v != v) ? 0 : (int)r;
-}
-
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
-}
-
-__device__ __forceinline__ float block_max_256(float v, float *red) {
-    v = wave_max(v);
-    const int wave = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) red[wave] = v;
-    __syncthreads();
-    v = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    return v;
-}
+__device__ __forceinline__ int quant_to_i8(float v) { return pg_quant_to_i8(v); }
+__device__ __forceinline__ float wave_max(float v) { return pg_wave_max_f32(v); }
+__device__ __forceinline__ float block_max_256(float v, float *red) { return pg_block_max_256(v, red); }
 
 // One workgroup per row.  The row is read once into registers (up to
 // 4*256*MAXV floats), reduced to its absmax, then rounded to i8 and written as
@@ -528,6 +511,7 @@ PG_API pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t
     if (m == 0) return PG_OK;
     PG_CHECK_ARG(a_dev && out_dev, "pg_matmul_quantized: null pointer");
     PG_CHECK_ARG(m < (1ull << 24), "pg_matmul_quantized: m = %zu too large", m);
+    if (pg_gemv_w8a8_takes_f32_row(w, m, k, a_dev)) return pg_launch_gemv_w8a8_f32_row(ctx, a_dev, k, w, out_dev, acc_dev);
     const size_t m_pad = pg_round_up(m, PG_MPAD);
     const size_t a_bytes = m_pad * w->k_pad;
     void *ws = nullptr;

@@ -179,6 +179,29 @@ def test_matmul_quantized_bit_exact(ctx, orc, m, k, n):
     assert (bits(got2) == bits(want)).all()
 
 
+@pytest.mark.parametrize("k,n", [(8, 5), (64, 33), (4096, 300), (4100, 64), (14336, 128), (16384, 16), (16400, 16)])
+def test_matmul_quantized_one_row_quantised_inside_the_product(ctx, orc, k, n):
+    """m = 1 with k % 4 == 0 and k <= 16384 runs as ONE launch that quantises the activation row
+    itself: the accumulators (hence the row's integers) and the f32 output must be those of the
+    two-step path bit for bit, on ordinary rows and on the rows the arithmetic treats specially
+    (ties, zero row, NaN, inf, subnormals).  k = 4100 and 16400 are past that route's limits."""
+    from peregrine_amd import quant
+    say(f"matmul_quantized one row k={k} n={n}")
+    w = orc.rng_normal(321 + n, k * n, 0.0, 0.02)
+    qt = quant.quantize_weights(w, k, n, ctx)
+    q, q_t, s = orc.quantize_weights(w, k, n)
+    rows = [orc.rng_normal(77 + k, k)]
+    rows[0][:: max(1, k // 40)] *= 20
+    rows += list(edge_rows(k))
+    for i, a in enumerate(rows):
+        want, want_acc = orc.matmul_quantized(a, 1, k, q_t, s, n)
+        got, got_acc = run_matmul_dev(ctx, a, 1, k, qt)
+        assert (got_acc == want_acc).all(), f"row {i}: i32 accumulators differ"
+        finite = np.isfinite(want)
+        assert (np.isfinite(got) == finite).all() and (bits(got[finite]) == bits(want[finite])).all(), f"row {i}: f32 outputs differ"
+    qt.free_gpu()
+
+
 def test_matmul_quantized_extreme_integers(ctx, orc):
     # every product is (-127)*(-127) or 127*(-127): the largest accumulators the path can see
     from peregrine_amd import quant
