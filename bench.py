@@ -258,7 +258,7 @@ def main():
                           f"{LAYERS_ROT} layers of weights rotated ({LAYERS_ROT * 3 * 58.7:.0f} MB, HBM-resident reads)",
               "value": round(dec_bytes / (dec_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
               "ms_per_step": round(dec_ms, 5), "steps": dsteps, "bytes_per_step": dec_bytes,
-              "roofline": {"kernel": "gemv_w8a8_kernel", "bound": "hbm", "achieved": round(gemv_gbs, 1),
+              "roofline": {"kernel": "gemv_w8a8_m1_f32x_kernel (quantises its activation row, then streams the weights)", "bound": "hbm", "achieved": round(gemv_gbs, 1),
                            "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gemv_gbs / PEAK_HBM_GBS, 4),
                            "traffic": traffic_for("gemv_w8a8"), "bytes_per_launch": dec_bytes // 3,
                            "avg_launch_ms": round(gemv_avg_ms, 5)}}
