@@ -199,6 +199,15 @@ def test_matmul_quantized_one_row_quantised_inside_the_product(ctx, orc, k, n):
         assert (got_acc == want_acc).all(), f"row {i}: i32 accumulators differ"
         finite = np.isfinite(want)
         assert (np.isfinite(got) == finite).all() and (bits(got[finite]) == bits(want[finite])).all(), f"row {i}: f32 outputs differ"
+    # a row that does not start on a 16-byte boundary takes the two-launch path: same answer
+    from peregrine_amd import _ffi
+    a = rows[0]
+    want, _ = orc.matmul_quantized(a, 1, k, q_t, s, n)
+    shifted = DevBuf(ctx, host=np.concatenate([np.zeros(1, np.float32), a]))
+    dout = DevBuf(ctx, n * 4)
+    _ffi.check(_ffi.lib.pg_matmul_quantized_dev(ctx.handle, C.c_void_p(shifted.ptr.value + 4), 1, k, qt._gpu, dout.ptr, None))
+    ctx.sync()
+    assert (bits(dout.to_host(np.float32)) == bits(want)).all()
     qt.free_gpu()
 
 
