@@ -51,7 +51,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) __attribute__((amdgpu_waves_per_eu(
 void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__restrict__ Bw, int ldb,
                       const float *__restrict__ a_scales, const float *__restrict__ w_scales,
                       float *__restrict__ out, int32_t *__restrict__ acc_out, int M, int N, int K,
-                      int tiles_m, int ntiles) {
+                      int tiles_m, int ntiles, int kt_per_split) {
     constexpr int NW = NWM * NWN;
     constexpr int WM = BM / NWM, WN = BN / NWN;      // wavefront tile
     constexpr int TM = WM / 32, TN = WN / 32;        // 32x32 MFMA tiles per wavefront
@@ -88,8 +88,12 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__res
         const int row = RPL * (wave + NW * i) + lr;
         b_goff[i] = row * ldb + 16 * (pc ^ swz<BK>(row));
     }
-    const int8_t *a_base = A + (size_t)m0 * lda;
-    const int8_t *b_base = Bw + (size_t)n0 * ldb;
+    // A split product (few activation rows): blockIdx.y owns kt_per_split k-tiles of BK bytes and
+    // writes its i32 partial sums to plane blockIdx.y of acc_out.  Otherwise gridDim.y == 1.
+    const int kt0_split = blockIdx.y * kt_per_split;
+    const int8_t *a_base = A + (size_t)m0 * lda + (size_t)kt0_split * BK;
+    const int8_t *b_base = Bw + (size_t)n0 * ldb + (size_t)kt0_split * BK;
+    if (acc_out) acc_out += (size_t)blockIdx.y * M * N;
 
     // ---- LDS fragment offsets (bytes) for each k-step of a stage.
     const int l31 = lane & 31, half = lane >> 5;
@@ -158,7 +162,7 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__res
     };
     static_assert(NST >= 2 && NST <= 6, "wait_barrier covers up to 4 stages in flight beyond the awaited one");
 
-    const int KT = K / BK;
+    const int KT = (K / BK - kt0_split < kt_per_split) ? K / BK - kt0_split : kt_per_split;
 #pragma unroll
     for (int s = 0; s < NST - 1; ++s)
         if (s < KT) issue(s, s * BK);
@@ -269,7 +273,7 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__res
 
 template <int BM, int BN, int BK, int NST, int NWM, int NWN, int OCC>
 pg_status launch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
-                 const pg_qtensor *w, size_t m, float *out, int32_t *acc) {
+                 const pg_qtensor *w, size_t m, float *out, int32_t *acc, int splits = 1, int kt_per_split = 0) {
     const int tiles_m = (int)((m + BM - 1) / BM);
     const int tiles_n = (int)((w->cols + BN - 1) / BN);
     const int ntiles = tiles_m * tiles_n;
@@ -277,13 +281,62 @@ pg_status launch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *
     auto kern = gemm_w8a8_kernel<BM, BN, BK, NST, NWM, NWN, OCC>;
     PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
     const unsigned grid = (unsigned)(((ntiles + 7) / 8) * 8);
-    PG_TRY(pg_launch(ctx, "gemm_w8a8", kern, dim3(grid), dim3(64 * NWM * NWN), lds, a_i8, (int)a_stride, w->w_t,
+    if (splits == 1) kt_per_split = (int)(w->k_pad / BK);
+    PG_TRY(pg_launch(ctx, "gemm_w8a8", kern, dim3(grid, (unsigned)splits), dim3(64 * NWM * NWN), lds, a_i8, (int)a_stride, w->w_t,
                      (int)w->k_pad, a_scales, w->scales, out, acc, (int)m, (int)w->cols, (int)w->k_pad, tiles_m,
-                     ntiles));
+                     ntiles, kt_per_split));
     return pg_launch_check("gemm_w8a8");
 }
 
+// out[m, n] = (float)(sum over the K splits of part[s][m, n]) * a_scale[m] * w_scale[n]: the integer sum is
+// exact and order-free, the f32 epilogue is the one of the unsplit product (src/quant.rs:163).
+__global__ __launch_bounds__(256) void splitk_finish_kernel(const int32_t *__restrict__ part, int splits, size_t plane,
+                                                             const float *__restrict__ a_scales,
+                                                             const float *__restrict__ w_scales, int n,
+                                                             float *__restrict__ out, int32_t *__restrict__ acc_out) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= plane) return;
+    int acc = 0, s = 0;
+    for (; s + 8 <= splits; s += 8) {  // eight independent loads in flight
+        int v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(part + (size_t)(s + u) * plane + i);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += v[u];
+    }
+    for (; s < splits; ++s) acc += __builtin_nontemporal_load(part + (size_t)s * plane + i);
+    const size_t r = i / n, c = i - r * n;
+    if (out) out[i] = (float)acc * a_scales[r] * w_scales[c];
+    if (acc_out) acc_out[i] = acc;
+}
+
 }  // namespace
+
+// Few activation rows (5 .. 64: batched decode): one 32- or 64-row tile of activations against
+// every weight row is far too few workgroups to stream the weights (64 on 256 CUs at N = 4096),
+// so K is split until about two workgroups per CU exist; the partial i32 sums go to `part`
+// ([splits][m][n]) and a second launch adds them and applies the scales.  Returns the number of
+// splits through *splits_out when called with part == nullptr (sizing), else runs.
+pg_status pg_launch_gemm_w8a8_few_rows(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                                       const pg_qtensor *w, size_t m, float *out, int32_t *acc, int32_t *part,
+                                       int *splits_out) {
+    const size_t n = w->cols, kt = w->k_pad / 128, n_tiles = (n + 127) / 128;
+    size_t splits = (2 * (size_t)ctx->num_cu + n_tiles - 1) / n_tiles;
+    if (splits > kt / 2) splits = kt / 2;  // at least two k-tiles per workgroup
+    if (splits < 1) splits = 1;
+    const size_t kt_per = (kt + splits - 1) / splits;
+    splits = (kt + kt_per - 1) / kt_per;   // no empty split
+    if (splits_out) *splits_out = (int)splits;
+    if (!part) return PG_OK;
+    if (a_stride != w->k_pad) return pg_fail(PG_EINVAL, "gemm_w8a8: activation stride %zu != k_pad %zu", a_stride, w->k_pad);
+    if (m <= 32)
+        PG_TRY((launch<32, 128, 128, 3, 1, 4, 2>(ctx, a_i8, a_stride, a_scales, w, m, nullptr, part, (int)splits, (int)kt_per)));
+    else
+        PG_TRY((launch<64, 128, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, m, nullptr, part, (int)splits, (int)kt_per)));
+    const size_t plane = m * n;
+    return pg_launch(ctx, "gemm_w8a8_finish", splitk_finish_kernel, dim3((unsigned)((plane + 255) / 256)), dim3(256), 0,
+                     (const int32_t *)part, (int)splits, plane, a_scales, (const float *)w->scales, (int)n, out, acc);
+}
 
 // a_i8 must have at least round_up(m, 256) rows of a_stride bytes (rows >= m may
 // hold anything: they only feed accumulators that are never stored), a_stride ==

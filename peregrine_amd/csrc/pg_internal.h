@@ -151,6 +151,11 @@ pg_status pg_launch_quantize_activations(pg_ctx *ctx, const float *a, size_t row
 pg_status pg_launch_gemm_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
                               const float *a_scales, const pg_qtensor *w, size_t m,
                               float *out, int32_t *acc);
+// 5 .. 64 activation rows: K split over workgroups, i32 partial sums in `part`, then one finishing
+// launch.  With part == nullptr only reports the number of splits (for sizing `part`).
+pg_status pg_launch_gemm_w8a8_few_rows(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                                       const pg_qtensor *w, size_t m, float *out, int32_t *acc, int32_t *part,
+                                       int *splits_out);
 pg_status pg_launch_gemv_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
                               const float *a_scales, const pg_qtensor *w, size_t m,
                               float *out, int32_t *acc);

@@ -514,13 +514,22 @@ PG_API pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t
     if (pg_gemv_w8a8_takes_f32_row(w, m, k, a_dev)) return pg_launch_gemv_w8a8_f32_row(ctx, a_dev, k, w, out_dev, acc_dev);
     const size_t m_pad = pg_round_up(m, PG_MPAD);
     const size_t a_bytes = m_pad * w->k_pad;
+    // 5 .. 64 rows (batched decode): split-K product with i32 partial planes behind the scales
+    int splits = 1;
+    if (m > PG_GEMV_MAX_M && m <= 64)
+        PG_TRY(pg_launch_gemm_w8a8_few_rows(ctx, nullptr, w->k_pad, nullptr, w, m, nullptr, nullptr, nullptr, &splits));
+    const size_t sz_scales = pg_round_up(m_pad * sizeof(float), 256);
+    const size_t part_bytes = splits > 1 ? (size_t)splits * m * w->cols * sizeof(int32_t) : 0;
     void *ws = nullptr;
-    PG_TRY(pg_workspace(ctx, a_bytes + m_pad * sizeof(float), &ws));
+    PG_TRY(pg_workspace(ctx, a_bytes + sz_scales + part_bytes, &ws));
     int8_t *a_i8 = static_cast<int8_t *>(ws);
     float *a_scales = reinterpret_cast<float *>(a_i8 + a_bytes);
     PG_TRY(pg_launch_quantize_activations(ctx, a_dev, m, k, a_i8, w->k_pad, a_scales));
     if (m <= PG_GEMV_MAX_M)
         return pg_launch_gemv_w8a8(ctx, a_i8, w->k_pad, a_scales, w, m, out_dev, acc_dev);
+    if (splits > 1)
+        return pg_launch_gemm_w8a8_few_rows(ctx, a_i8, w->k_pad, a_scales, w, m, out_dev, acc_dev,
+                                            reinterpret_cast<int32_t *>(a_i8 + a_bytes + sz_scales), nullptr);
     return pg_launch_gemm_w8a8(ctx, a_i8, w->k_pad, a_scales, w, m, out_dev, acc_dev);
 }
 
