@@ -156,6 +156,8 @@ MATMUL_SHAPES = [
     (300, 512, 1000),                                  # 128x128 tiles, ragged m and n
     (2048, 128, 4096),                                 # 256x128 tiles
     (2050, 192, 4100),                                 # 256x128 tiles, ragged m and n
+    # 5 .. 64 rows: K split over workgroups, i32 partial planes, finishing pass (ragged everywhere)
+    (5, 4096, 1000), (17, 4224, 520), (33, 1024, 4100), (40, 1024, 14336), (64, 14336, 300), (31, 512, 77),
 ]
 
 
