@@ -312,7 +312,7 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const int32_t *__res
 
 }  // namespace
 
-// Few activation rows (5 .. 64: batched decode): one 32- or 64-row tile of activations against
+// Few activation rows (5 .. 256: batched decode, short prefill chunks): one or two tiles of activations against
 // every weight row is far too few workgroups to stream the weights (64 on 256 CUs at N = 4096),
 // so K is split until about two workgroups per CU exist; the partial i32 sums go to `part`
 // ([splits][m][n]) and a second launch adds them and applies the scales.  Returns the number of
@@ -320,19 +320,24 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const int32_t *__res
 pg_status pg_launch_gemm_w8a8_few_rows(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
                                        const pg_qtensor *w, size_t m, float *out, int32_t *acc, int32_t *part,
                                        int *splits_out) {
-    const size_t n = w->cols, kt = w->k_pad / 128, n_tiles = (n + 127) / 128;
-    size_t splits = (2 * (size_t)ctx->num_cu + n_tiles - 1) / n_tiles;
+    const size_t n = w->cols, kt = w->k_pad / 128;
+    const size_t bm = m <= 32 ? 32 : (m <= 64 ? 64 : 128);
+    const size_t tiles = ((m + bm - 1) / bm) * ((n + 127) / 128);
+    size_t splits = (2 * (size_t)ctx->num_cu + tiles - 1) / tiles;
     if (splits > kt / 2) splits = kt / 2;  // at least two k-tiles per workgroup
+    if (splits > 16) splits = 16;
     if (splits < 1) splits = 1;
     const size_t kt_per = (kt + splits - 1) / splits;
     splits = (kt + kt_per - 1) / kt_per;   // no empty split
     if (splits_out) *splits_out = (int)splits;
     if (!part) return PG_OK;
     if (a_stride != w->k_pad) return pg_fail(PG_EINVAL, "gemm_w8a8: activation stride %zu != k_pad %zu", a_stride, w->k_pad);
-    if (m <= 32)
+    if (bm == 32)
         PG_TRY((launch<32, 128, 128, 3, 1, 4, 2>(ctx, a_i8, a_stride, a_scales, w, m, nullptr, part, (int)splits, (int)kt_per)));
-    else
+    else if (bm == 64)
         PG_TRY((launch<64, 128, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, m, nullptr, part, (int)splits, (int)kt_per)));
+    else
+        PG_TRY((launch<128, 128, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, m, nullptr, part, (int)splits, (int)kt_per)));
     const size_t plane = m * n;
     return pg_launch(ctx, "gemm_w8a8_finish", splitk_finish_kernel, dim3((unsigned)((plane + 255) / 256)), dim3(256), 0,
                      (const int32_t *)part, (int)splits, plane, a_scales, (const float *)w->scales, (int)n, out, acc);

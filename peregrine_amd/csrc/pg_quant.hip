@@ -514,9 +514,12 @@ PG_API pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t
     if (pg_gemv_w8a8_takes_f32_row(w, m, k, a_dev)) return pg_launch_gemv_w8a8_f32_row(ctx, a_dev, k, w, out_dev, acc_dev);
     const size_t m_pad = pg_round_up(m, PG_MPAD);
     const size_t a_bytes = m_pad * w->k_pad;
-    // 5 .. 64 rows (batched decode): split-K product with i32 partial planes behind the scales
+    // 5 .. 256 rows (batched decode, short prefill chunks): split-K product with i32 partial planes
+    // behind the scales, where the unsplit tiles would leave most CUs idle
+    // (up to 64 rows always; up to 256 only for long-K, narrow-N products like a down projection --
+    // measured at 128 rows: 14336 -> 4096 35 -> 25 us split, but 4096 -> 4096 12.6 -> 19 us)
     int splits = 1;
-    if (m > PG_GEMV_MAX_M && m <= 64)
+    if (m > PG_GEMV_MAX_M && (m <= 64 || (m <= 256 && w->k_pad >= 2 * w->cols)))
         PG_TRY(pg_launch_gemm_w8a8_few_rows(ctx, nullptr, w->k_pad, nullptr, w, m, nullptr, nullptr, nullptr, &splits));
     const size_t sz_scales = pg_round_up(m_pad * sizeof(float), 256);
     const size_t part_bytes = splits > 1 ? (size_t)splits * m * w->cols * sizeof(int32_t) : 0;

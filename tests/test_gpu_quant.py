@@ -158,6 +158,7 @@ MATMUL_SHAPES = [
     (2050, 192, 4100),                                 # 256x128 tiles, ragged m and n
     # 5 .. 64 rows: K split over workgroups, i32 partial planes, finishing pass (ragged everywhere)
     (5, 4096, 1000), (17, 4224, 520), (33, 1024, 4100), (40, 1024, 14336), (64, 14336, 300), (31, 512, 77),
+    (100, 8192, 300), (130, 4096, 257), (256, 2048, 1000),   # up to 256 rows when K >= 2 N: 128-row tiles
 ]
 
 
