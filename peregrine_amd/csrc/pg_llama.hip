@@ -45,7 +45,6 @@ struct pg_llama_block {
     const uint16_t *const *d_qkv, *const *d_gu;
     const int *item_ids;              // 0, 1, 2, ...
     int qkv_items;                    // num_q_heads / num_kv_heads + 2
-    unsigned *tickets;                // one arrival counter per query head, zero between launches
     int digit_kind;                   // PG_GGML_Q4_0 (nibble digits), PG_GGML_Q8_0 (byte digits), 0 = mixed: no fused step
 };
 
@@ -1154,14 +1153,13 @@ PG_API pg_status pg_llama_block_create(pg_ctx *ctx, size_t model_dim, size_t num
         return st;
     }
     b->ffn_norm_w = b->attn_norm_w + model_dim;
-    // one-token step buffers: three digit sets, then the pointer tables, the item ids and the
-    // attention arrival counters
+    // one-token step buffers: three digit sets, then the pointer tables and the item ids
     const size_t q_dim = num_q_heads * head_dim;
     const size_t items = num_q_heads / num_kv_heads + 2;
     const size_t o_q = pg_xdigits_bytes(1, model_dim), o_f = o_q + pg_xdigits_bytes(1, q_dim);
     const size_t o_tab = o_f + pg_xdigits_bytes(1, ffn_dim);
     const size_t tab_bytes = pg_round_up((2 * items + 4) * sizeof(void *) + items * sizeof(int), 256);
-    const size_t total = o_tab + tab_bytes + pg_round_up(num_q_heads * sizeof(unsigned), 256);
+    const size_t total = o_tab + tab_bytes;
     hipError_t e = hipMalloc(&b->dec, total);
     if (e == hipSuccess) e = hipMemsetAsync(b->dec, 0, total, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
@@ -1181,7 +1179,6 @@ PG_API pg_status pg_llama_block_create(pg_ctx *ctx, size_t model_dim, size_t num
     b->qs_gu = reinterpret_cast<const uint8_t *const *>(tab + 2 * items);
     b->d_gu = reinterpret_cast<const uint16_t *const *>(tab + 2 * items + 2);
     b->item_ids = reinterpret_cast<const int *>(tab + 2 * items + 4);
-    b->tickets = reinterpret_cast<unsigned *>(base + o_tab + tab_bytes);
     *out = b;
     return PG_OK;
 }
@@ -1267,11 +1264,15 @@ static pg_status block_forward_one_token(pg_ctx *ctx, pg_llama_block *b, const f
     const size_t cap = b->seq_cap;
     float *p = b->arena;
     auto take = [&](size_t n) { float *r = p; p += slot(n); return r; };
-    float *normed = take(cap * d), *h1 = take(cap * d), *proj = take(cap * d);
-    float *unused_q = take(cap * q_dim), *q_rope = take(cap * q_dim), *attn = take(cap * q_dim);
-    (void)normed; (void)proj; (void)unused_q;
-    float *kv_gap = take(cap * kv_dim), *kv_gap2 = take(cap * kv_dim);
-    (void)kv_gap; (void)kv_gap2;
+    // the arena is laid out for the many-token route (normed, h1, proj | q, q_rope, attn | k, v | g, u | q|k|v);
+    // this step uses h1, q_rope, attn, g|u and the adjacent q|k|v rows
+    (void)take(cap * d);
+    float *h1 = take(cap * d);
+    (void)take(cap * d);
+    (void)take(cap * q_dim);
+    float *q_rope = take(cap * q_dim), *attn = take(cap * q_dim);
+    (void)take(cap * kv_dim);
+    (void)take(cap * kv_dim);
     float *g = take(2 * cap * ffn), *u = g + ffn;
     // q|k|v and g|u as adjacent rows: item i of a multi-item launch writes y + i * n_out
     float *qkv = take(cap * (q_dim + 2 * kv_dim) + 128), *qd = qkv, *kd = qkv + q_dim, *vd = kd + kv_dim;
