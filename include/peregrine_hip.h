@@ -172,7 +172,10 @@ void pg_gguf_free(pg_ctx *ctx, pg_gguf_tensor *t);
 
 /* The dequantise-then-matmul of models::llama, fused:
  * y [m, n_out] = x [m, k_in] . dequant(w)^T, i.e. Tensor::matmul
- * (src/tensor.rs:1342-1353) applied to the transposed dequantised weight. */
+ * (src/tensor.rs:1342-1353) applied to the transposed dequantised weight.
+ * The first call with m > 1 on a Q4_0 / Q8_0 tensor (and an expert's first pg_moe_ffn) adds a
+ * second, tile-major copy of the quant payload to the handle (freed by pg_gguf_free): a
+ * handle must not see its first such call from two threads at once. */
 pg_status pg_gguf_matmul(pg_ctx *ctx, const float *x, size_t m, const pg_gguf_tensor *w,
                          float *y);
 pg_status pg_gguf_matmul_dev(pg_ctx *ctx, const float *x_dev, size_t m,
