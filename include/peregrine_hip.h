@@ -137,6 +137,25 @@ pg_status pg_matmul_quantized(pg_ctx *ctx, const float *a, size_t m, size_t k,
 pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
                                   const pg_qtensor *w, float *out_dev, int32_t *acc_dev);
 
+/* The fused products of models::llama: `x.matmul(qkv_fused)` / `normed.matmul(gate_up_fused)`
+ * over column-concatenated weights (fuse_qkv  src/models/llama/attention.rs:51-71, used :84;
+ * fuse_gate_up  src/models/llama/decoder.rs:49-67, used :78), here without a fused copy:
+ * `count` (1 .. 4) weights with the same number of rows k, the activation rows quantised once,
+ * one launch for more than 256 rows.  out_dev[i] is [m, cols of w[i]] and equals
+ * pg_matmul_quantized_dev(a, w[i]) bit for bit (scales are per row and per column). */
+pg_status pg_matmul_quantized_multi_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
+                                        const pg_qtensor *const *w, size_t count,
+                                        float *const *out_dev);
+
+/* Diagnostics of the matrix-core product.  No counterpart in the reference (its Metal
+ * dispatcher picks between two shaders by size, src/metal/context.rs:2243, without a query):
+ * the output tile (rows x columns) and the number of K splits of the most recent W8A8 GEMM
+ * launch on this context, and an override of the dispatcher's tile choice (0 = automatic,
+ * 1 = 64x64, 2 = 256x256, 3 = 128x256, 4 = 128x64, 5 = 128x128).  Every tile gives the same
+ * bits; tests use the pair to prove each kernel instantiation ran. */
+pg_status pg_gemm_w8a8_last_tile(const pg_ctx *ctx, int *bm, int *bn, int *k_splits);
+pg_status pg_gemm_w8a8_force_tile(pg_ctx *ctx, int tile);
+
 /* The reference's GPU numerics for the same call (W8A32): f32 activations, weights
  * dequantised to f32, f32 accumulate, no activation quantisation --
  * GpuContext::dispatch_matmul_dequant_i8  src/metal/context.rs:2226-2306, shader

@@ -49,6 +49,9 @@ SIGNATURES = {
     "pg_qtensor_free": [_vp, _vp],
     "pg_matmul_quantized": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_matmul_quantized_dev": [_vp, _vp, _sz, _sz, _vp, _vp, _vp],
+    "pg_matmul_quantized_multi_dev": [_vp, _vp, _sz, _sz, _pp, _sz, _pp],
+    "pg_gemm_w8a8_last_tile": [_vp, C.POINTER(_int), C.POINTER(_int), C.POINTER(_int)],
+    "pg_gemm_w8a8_force_tile": [_vp, _int],
     "pg_matmul_dequant_i8": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_matmul_dequant_i8_dev": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_f16_to_f32": [_vp, _vp, _sz, _vp],

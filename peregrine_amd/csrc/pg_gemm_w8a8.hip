@@ -26,6 +26,7 @@
 // of __syncthreads would drain every outstanding prefetch), refills the stage it
 // just finished and reads the next stage's first fragments under the remaining
 // MFMAs.
+#include <limits.h>
 #include "pg_internal.h"
 
 namespace {
@@ -46,11 +47,21 @@ template <int BK> __device__ __forceinline__ int swz(int r);
 template <> __device__ __forceinline__ int swz<64>(int r) { return ((r >> 1) + (r >> 3)) & 3; }
 template <> __device__ __forceinline__ int swz<128>(int r) { return ((r >> 1) & 7) ^ ((r & 1) << 2); }
 
+// The weights of one launch: up to PG_GEMM_MAX_GROUP tensors of equal K whose column panels are
+// laid end to end in the launch's tile space (weight g owns the n-panels panel0[g] .. panel0[g+1]-1;
+// unused slots hold INT_MAX).  One weight is a group of one.
+struct gemm_wgroup {
+    const int8_t *w[PG_GEMM_MAX_GROUP];
+    const float *ws[PG_GEMM_MAX_GROUP];
+    float *out[PG_GEMM_MAX_GROUP];
+    int n[PG_GEMM_MAX_GROUP];
+    int panel0[PG_GEMM_MAX_GROUP];
+};
+
 template <int BM, int BN, int BK, int NST, int NWM, int NWN, int OCC>
 __global__ __launch_bounds__(64 * NWM * NWN) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
-void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__restrict__ Bw, int ldb,
-                      const float *__restrict__ a_scales, const float *__restrict__ w_scales,
-                      float *__restrict__ out, int32_t *__restrict__ acc_out, int M, int N, int K,
+void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const gemm_wgroup grp, int ldb,
+                      const float *__restrict__ a_scales, int32_t *__restrict__ acc_out, int M, int K,
                       int tiles_m, int ntiles, int kt_per_split) {
     constexpr int NW = NWM * NWN;
     constexpr int WM = BM / NWM, WN = BN / NWN;      // wavefront tile
@@ -68,7 +79,15 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__res
     const int chunk = (ntiles + 7) / 8;
     const int t = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
     if (t >= ntiles) return;
-    const int m0 = (t % tiles_m) * BM, n0 = (t / tiles_m) * BN;
+    const int np = t / tiles_m;  // n-panel of the launch; which weight owns it (uniform: scalar code)
+    int g = 0;
+#pragma unroll
+    for (int i = 1; i < PG_GEMM_MAX_GROUP; ++i) g = np >= grp.panel0[i] ? i : g;
+    const int8_t *__restrict__ Bw = grp.w[g];
+    const float *__restrict__ w_scales = grp.ws[g];
+    float *__restrict__ out = grp.out[g];
+    const int N = grp.n[g];
+    const int m0 = (t % tiles_m) * BM, n0 = (np - grp.panel0[g]) * BN;
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -272,20 +291,41 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const int8_t *__res
 }
 
 template <int BM, int BN, int BK, int NST, int NWM, int NWN, int OCC>
-pg_status launch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
-                 const pg_qtensor *w, size_t m, float *out, int32_t *acc, int splits = 1, int kt_per_split = 0) {
+pg_status launch_group(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                       const pg_qtensor *const *w, float *const *out, int count, size_t m, int32_t *acc,
+                       int splits = 1, int kt_per_split = 0) {
     const int tiles_m = (int)((m + BM - 1) / BM);
-    const int tiles_n = (int)((w->cols + BN - 1) / BN);
-    const int ntiles = tiles_m * tiles_n;
+    gemm_wgroup grp;
+    int panels = 0;
+    for (int i = 0; i < PG_GEMM_MAX_GROUP; ++i) {
+        const bool used = i < count;
+        grp.w[i] = used ? w[i]->w_t : nullptr;
+        grp.ws[i] = used ? w[i]->scales : nullptr;
+        grp.out[i] = used && out ? out[i] : nullptr;
+        grp.n[i] = used ? (int)w[i]->cols : 0;
+        grp.panel0[i] = used ? panels : INT_MAX;
+        if (used) panels += (int)((w[i]->cols + BN - 1) / BN);
+    }
+    const int ntiles = tiles_m * panels;
     const size_t lds = (size_t)NST * (BM + BN) * BK + (BM + BN) * sizeof(float);
     auto kern = gemm_w8a8_kernel<BM, BN, BK, NST, NWM, NWN, OCC>;
     PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
     const unsigned grid = (unsigned)(((ntiles + 7) / 8) * 8);
-    if (splits == 1) kt_per_split = (int)(w->k_pad / BK);
-    PG_TRY(pg_launch(ctx, "gemm_w8a8", kern, dim3(grid, (unsigned)splits), dim3(64 * NWM * NWN), lds, a_i8, (int)a_stride, w->w_t,
-                     (int)w->k_pad, a_scales, w->scales, out, acc, (int)m, (int)w->cols, (int)w->k_pad, tiles_m,
-                     ntiles, kt_per_split));
+    const size_t k_pad = w[0]->k_pad;
+    if (splits == 1) kt_per_split = (int)(k_pad / BK);
+    ctx->gemm_last_bm = BM;
+    ctx->gemm_last_bn = BN;
+    ctx->gemm_last_splits = splits;
+    PG_TRY(pg_launch(ctx, "gemm_w8a8", kern, dim3(grid, (unsigned)splits), dim3(64 * NWM * NWN), lds, a_i8, (int)a_stride, grp,
+                     (int)k_pad, a_scales, acc, (int)m, (int)k_pad, tiles_m, ntiles, kt_per_split));
     return pg_launch_check("gemm_w8a8");
+}
+
+template <int BM, int BN, int BK, int NST, int NWM, int NWN, int OCC>
+pg_status launch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                 const pg_qtensor *w, size_t m, float *out, int32_t *acc, int splits = 1, int kt_per_split = 0) {
+    return launch_group<BM, BN, BK, NST, NWM, NWN, OCC>(ctx, a_i8, a_stride, a_scales, &w, &out, 1, m, acc, splits,
+                                                        kt_per_split);
 }
 
 // out[m, n] = (float)(sum over the K splits of part[s][m, n]) * a_scale[m] * w_scale[n]: the integer sum is
@@ -308,6 +348,39 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const int32_t *__res
     const size_t r = i / n, c = i - r * n;
     if (out) out[i] = (float)acc * a_scales[r] * w_scales[c];
     if (acc_out) acc_out[i] = acc;
+}
+
+// Tile choice (measured on MI355X at M = 2048): the larger the tile the fewer bytes each
+// CU pulls from L2 per MFMA, but every CU needs a tile.  8 wavefronts per workgroup also
+// double the rate at which one CU can stream from L2 (about 9 GB/s per wavefront).
+// ctx->gemm_force_tile (pg_gemm_w8a8_force_tile) overrides the choice: 1 = 64x64, 2 = 256x256,
+// 3 = 128x256, 4 = 128x64, 5 = 128x128.
+pg_status gemm_dispatch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                        const pg_qtensor *const *w, float *const *out, int count, size_t m, int32_t *acc) {
+    const size_t cus = (size_t)ctx->num_cu;
+    auto tiles = [&](size_t bm, size_t bn) {
+        size_t panels = 0;
+        for (int i = 0; i < count; ++i) panels += (w[i]->cols + bn - 1) / bn;
+        return ((m + bm - 1) / bm) * panels;
+    };
+    int pick = ctx->gemm_force_tile;
+    if (pick == 0) {
+        if (m <= 64) pick = 1;
+        else if (tiles(256, 256) * 2 >= 3 * cus) pick = 2;
+        else if (tiles(128, 256) >= cus) pick = 3;
+        // Too few 128x128 tiles for the CUs (k/v projections, N = 1024): halve the tile instead of
+        // leaving half of the chip idle (21.2 -> 16.5 us at 2048 x 4096 -> 1024).
+        else if (tiles(128, 128) < cus) pick = 4;
+        else pick = 5;
+    }
+    switch (pick) {
+        case 1: return launch_group<64, 64, 128, 2, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
+        case 2: return launch_group<256, 256, 128, 2, 2, 4, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
+        case 3: return launch_group<128, 256, 128, 2, 2, 4, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
+        case 4: return launch_group<128, 64, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
+        case 5: return launch_group<128, 128, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
+        default: return pg_fail(PG_EINVAL, "gemm_w8a8: unknown tile override %d", pick);
+    }
 }
 
 }  // namespace
@@ -346,23 +419,22 @@ pg_status pg_launch_gemm_w8a8_few_rows(pg_ctx *ctx, const int8_t *a_i8, size_t a
 // a_i8 must have at least round_up(m, 256) rows of a_stride bytes (rows >= m may
 // hold anything: they only feed accumulators that are never stored), a_stride ==
 // w->k_pad with the K padding zero-filled.
+pg_status pg_launch_gemm_w8a8_group(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                                    const pg_qtensor *const *w, float *const *out, int count, size_t m) {
+    if (count < 1 || count > PG_GEMM_MAX_GROUP) return pg_fail(PG_EINVAL, "gemm_w8a8: %d weights in one launch (1 .. %d)", count, PG_GEMM_MAX_GROUP);
+    for (int i = 0; i < count; ++i) {
+        if (a_stride != w[i]->k_pad) return pg_fail(PG_EINVAL, "gemm_w8a8: activation stride %zu != k_pad %zu", a_stride, w[i]->k_pad);
+        if (w[i]->k_pad >= (1ull << 22) || m >= (1ull << 24) || w[i]->cols >= (1ull << 30))
+            return pg_fail(PG_EUNSUPPORTED, "gemm_w8a8: shape exceeds the kernel's 32-bit tile offsets");
+    }
+    return gemm_dispatch(ctx, a_i8, a_stride, a_scales, w, out, count, m, nullptr);
+}
+
 pg_status pg_launch_gemm_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
                               const float *a_scales, const pg_qtensor *w, size_t m, float *out,
                               int32_t *acc) {
     if (a_stride != w->k_pad) return pg_fail(PG_EINVAL, "gemm_w8a8: activation stride %zu != k_pad %zu", a_stride, w->k_pad);
     if (w->k_pad >= (1ull << 22) || m >= (1ull << 24) || w->cols >= (1ull << 30))
         return pg_fail(PG_EUNSUPPORTED, "gemm_w8a8: shape exceeds the kernel's 32-bit tile offsets");
-    const size_t n = w->cols;
-    const size_t cus = (size_t)ctx->num_cu;
-    auto tiles = [&](size_t bm, size_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-    // Tile choice (measured on MI355X at M = 2048): the larger the tile the fewer bytes each
-    // CU pulls from L2 per MFMA, but every CU needs a tile.  8 wavefronts per workgroup also
-    // double the rate at which one CU can stream from L2 (about 9 GB/s per wavefront).
-    if (m <= 64) return launch<64, 64, 128, 2, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
-    if (tiles(256, 256) * 2 >= 3 * cus) return launch<256, 256, 128, 2, 2, 4, 2>(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
-    if (tiles(128, 256) >= cus) return launch<128, 256, 128, 2, 2, 4, 2>(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
-    // Too few 128x128 tiles for the CUs (k/v projections, N = 1024): halve the tile instead of leaving
-    // half of the chip idle (21.2 -> 16.5 us at 2048 x 4096 -> 1024).
-    if (tiles(128, 128) < cus) return launch<128, 64, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
-    return launch<128, 128, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, m, out, acc);
+    return gemm_dispatch(ctx, a_i8, a_stride, a_scales, &w, &out, 1, m, acc);
 }

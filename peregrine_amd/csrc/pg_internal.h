@@ -42,6 +42,10 @@ struct pg_ctx {
     size_t moe_tab_cap = 0;
     // Kernels whose dynamic LDS limit was raised on this context's device (pg_allow_dynamic_lds).
     std::vector<const void *> lds_raised;
+    // W8A8 GEMM dispatch: the tile of the most recent launch (pg_gemm_w8a8_last_tile) and an
+    // optional override of the dispatcher's choice (pg_gemm_w8a8_force_tile; 0 = automatic).
+    int gemm_last_bm = 0, gemm_last_bn = 0, gemm_last_splits = 0;
+    int gemm_force_tile = 0;
 };
 
 // Device-resident quantised weight, K-contiguous and zero-padded:
@@ -151,6 +155,12 @@ pg_status pg_launch_quantize_activations(pg_ctx *ctx, const float *a, size_t row
 pg_status pg_launch_gemm_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
                               const float *a_scales, const pg_qtensor *w, size_t m,
                               float *out, int32_t *acc);
+// The same activation rows against up to PG_GEMM_MAX_GROUP weights of equal K in ONE launch: the
+// weights' column panels form one tile space (a fused QKV or gate|up product without a fused
+// copy of the weights).  out[i] is [m, w[i]->cols].
+constexpr int PG_GEMM_MAX_GROUP = 4;
+pg_status pg_launch_gemm_w8a8_group(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                                    const pg_qtensor *const *w, float *const *out, int count, size_t m);
 // 5 .. 64 activation rows: K split over workgroups, i32 partial sums in `part`, then one finishing
 // launch.  With part == nullptr only reports the number of splits (for sizing `part`).
 pg_status pg_launch_gemm_w8a8_few_rows(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,

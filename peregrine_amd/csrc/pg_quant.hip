@@ -503,14 +503,11 @@ constexpr size_t PG_MPAD = 256;
 // bounds the product: use the dot-product GEMV kernel.
 constexpr size_t PG_GEMV_MAX_M = 4;
 
-PG_API pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
-                                         const pg_qtensor *w, float *out_dev, int32_t *acc_dev) {
-    PG_TRY(pg_use(ctx));
-    PG_CHECK_ARG(w != nullptr, "pg_matmul_quantized: null weights");
-    PG_CHECK_ARG(w->rows == k, "pg_matmul_quantized: a has k = %zu but w has %zu rows", k, w->rows);
-    if (m == 0) return PG_OK;
-    PG_CHECK_ARG(a_dev && out_dev, "pg_matmul_quantized: null pointer");
-    PG_CHECK_ARG(m < (1ull << 24), "pg_matmul_quantized: m = %zu too large", m);
+// The product over device pointers.  Scratch (quantised rows, row scales, split-K partial planes)
+// comes from the context's arena, or from `fixed` (of fixed_cap bytes) when that is given: then
+// nothing is allocated and a request that does not fit is an error.
+static pg_status matmul_quantized_on(pg_ctx *ctx, const float *a_dev, size_t m, size_t k, const pg_qtensor *w,
+                                     float *out_dev, int32_t *acc_dev, void *fixed, size_t fixed_cap) {
     if (pg_gemv_w8a8_takes_f32_row(w, m, k, a_dev)) return pg_launch_gemv_w8a8_f32_row(ctx, a_dev, k, w, out_dev, acc_dev);
     const size_t m_pad = pg_round_up(m, PG_MPAD);
     const size_t a_bytes = m_pad * w->k_pad;
@@ -523,8 +520,15 @@ PG_API pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t
         PG_TRY(pg_launch_gemm_w8a8_few_rows(ctx, nullptr, w->k_pad, nullptr, w, m, nullptr, nullptr, nullptr, &splits));
     const size_t sz_scales = pg_round_up(m_pad * sizeof(float), 256);
     const size_t part_bytes = splits > 1 ? (size_t)splits * m * w->cols * sizeof(int32_t) : 0;
-    void *ws = nullptr;
-    PG_TRY(pg_workspace(ctx, a_bytes + sz_scales + part_bytes, &ws));
+    const size_t need = a_bytes + sz_scales + part_bytes;
+    void *ws = fixed;
+    if (fixed) {
+        if (need > fixed_cap)
+            return pg_fail(PG_EINVAL, "this product needs %zu bytes of scratch (m = %zu, k = %zu, n = %zu); the fixed scratch holds %zu",
+                           need, m, k, w->cols, fixed_cap);
+    } else {
+        PG_TRY(pg_workspace(ctx, need, &ws));
+    }
     int8_t *a_i8 = static_cast<int8_t *>(ws);
     float *a_scales = reinterpret_cast<float *>(a_i8 + a_bytes);
     PG_TRY(pg_launch_quantize_activations(ctx, a_dev, m, k, a_i8, w->k_pad, a_scales));
@@ -534,6 +538,70 @@ PG_API pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t
         return pg_launch_gemm_w8a8_few_rows(ctx, a_i8, w->k_pad, a_scales, w, m, out_dev, acc_dev,
                                             reinterpret_cast<int32_t *>(a_i8 + a_bytes + sz_scales), nullptr);
     return pg_launch_gemm_w8a8(ctx, a_i8, w->k_pad, a_scales, w, m, out_dev, acc_dev);
+}
+
+PG_API pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
+                                         const pg_qtensor *w, float *out_dev, int32_t *acc_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(w != nullptr, "pg_matmul_quantized: null weights");
+    PG_CHECK_ARG(w->rows == k, "pg_matmul_quantized: a has k = %zu but w has %zu rows", k, w->rows);
+    if (m == 0) return PG_OK;
+    PG_CHECK_ARG(a_dev && out_dev, "pg_matmul_quantized: null pointer");
+    PG_CHECK_ARG(m < (1ull << 24), "pg_matmul_quantized: m = %zu too large", m);
+    return matmul_quantized_on(ctx, a_dev, m, k, w, out_dev, acc_dev, nullptr, 0);
+}
+
+// One activation matrix against several weights of equal K: the reference multiplies by
+// column-concatenated weights (fuse_qkv src/models/llama/attention.rs:51-71, fuse_gate_up
+// src/models/llama/decoder.rs:49-67) and slices the result; per-column weight scales and per-row
+// activation scales make every output column independent of its neighbours, so the separate
+// outputs here are bit for bit those of the single products.  The rows are quantised ONCE and,
+// for more than 64 rows, the products share one launch (the weights' column panels side by side
+// in one tile space).
+PG_API pg_status pg_matmul_quantized_multi_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
+                                               const pg_qtensor *const *w, size_t count, float *const *out_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(count >= 1 && count <= (size_t)PG_GEMM_MAX_GROUP, "pg_matmul_quantized_multi: %zu weights (1 .. %d)", count,
+                 PG_GEMM_MAX_GROUP);
+    PG_CHECK_ARG(w != nullptr && out_dev != nullptr, "pg_matmul_quantized_multi: null table");
+    for (size_t i = 0; i < count; ++i) {
+        PG_CHECK_ARG(w[i] != nullptr, "pg_matmul_quantized_multi: weight %zu is null", i);
+        PG_CHECK_ARG(w[i]->rows == k, "pg_matmul_quantized_multi: a has k = %zu but weight %zu has %zu rows", k, i, w[i]->rows);
+        PG_CHECK_ARG(m == 0 || out_dev[i] != nullptr, "pg_matmul_quantized_multi: output %zu is null", i);
+    }
+    if (m == 0) return PG_OK;
+    PG_CHECK_ARG(a_dev != nullptr, "pg_matmul_quantized_multi: null pointer");
+    PG_CHECK_ARG(m < (1ull << 24), "pg_matmul_quantized_multi: m = %zu too large", m);
+    if (count == 1 || m <= 256) {  // few rows: the single products pick their own route (GEMV, split K)
+        for (size_t i = 0; i < count; ++i) PG_TRY(pg_matmul_quantized_dev(ctx, a_dev, m, k, w[i], out_dev[i], nullptr));
+        return PG_OK;
+    }
+    const size_t k_pad = w[0]->k_pad, m_pad = pg_round_up(m, PG_MPAD);
+    const size_t a_bytes = m_pad * k_pad;
+    void *ws = nullptr;
+    PG_TRY(pg_workspace(ctx, a_bytes + pg_round_up(m_pad * sizeof(float), 256), &ws));
+    int8_t *a_i8 = static_cast<int8_t *>(ws);
+    float *a_scales = reinterpret_cast<float *>(a_i8 + a_bytes);
+    PG_TRY(pg_launch_quantize_activations(ctx, a_dev, m, k, a_i8, k_pad, a_scales));
+    return pg_launch_gemm_w8a8_group(ctx, a_i8, k_pad, a_scales, w, out_dev, (int)count, m);
+}
+
+// Which tile the W8A8 matrix-core product last ran with on this context, and an override of the
+// dispatcher's choice (0 = automatic; 1 = 64x64, 2 = 256x256, 3 = 128x256, 4 = 128x64,
+// 5 = 128x128 output tiles).  For tests and tuning runs: every tile shape gives the same bits.
+PG_API pg_status pg_gemm_w8a8_last_tile(const pg_ctx *ctx, int *bm, int *bn, int *k_splits) {
+    PG_CHECK_ARG(ctx != nullptr, "null context");
+    if (bm) *bm = ctx->gemm_last_bm;
+    if (bn) *bn = ctx->gemm_last_bn;
+    if (k_splits) *k_splits = ctx->gemm_last_splits;
+    return PG_OK;
+}
+
+PG_API pg_status pg_gemm_w8a8_force_tile(pg_ctx *ctx, int tile) {
+    PG_CHECK_ARG(ctx != nullptr, "null context");
+    PG_CHECK_ARG(tile >= 0 && tile <= 5, "pg_gemm_w8a8_force_tile: tile %d (0 .. 5)", tile);
+    ctx->gemm_force_tile = tile;
+    return PG_OK;
 }
 
 // The reference's GPU numerics for the same call: f32 activations times dequantised weights,

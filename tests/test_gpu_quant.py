@@ -154,8 +154,10 @@ MATMUL_SHAPES = [
     (5, 96, 40), (64, 200, 130), (65, 384, 129),       # 64x64 and 128x128 tiles, ragged
     (196, 768, 3072),                                  # benches/wallclock.rs:758-786
     (300, 512, 1000),                                  # 128x128 tiles, ragged m and n
-    (2048, 128, 4096),                                 # 256x128 tiles
-    (2050, 192, 4100),                                 # 256x128 tiles, ragged m and n
+    (2048, 128, 4096),                                 # 128x256 tiles
+    (2050, 192, 4100),                                 # 128x256 tiles, ragged m and n
+    (2049, 128, 12300),                                # 256x256 tiles, ragged m and n
+    (1030, 256, 4000),                                 # 128x128 tiles unsplit, ragged m and n
     # 5 .. 64 rows: K split over workgroups, i32 partial planes, finishing pass (ragged everywhere)
     (5, 4096, 1000), (17, 4224, 520), (33, 1024, 4100), (40, 1024, 14336), (64, 14336, 300), (31, 512, 77),
     (100, 8192, 300), (130, 4096, 257), (256, 2048, 1000),   # up to 256 rows when K >= 2 N: 128-row tiles
@@ -243,31 +245,171 @@ def test_matmul_quantized_shape_mismatch_is_an_error(ctx, orc):
     assert quant.matmul_quantized(np.zeros(0, np.float32), 0, 64, qt, ctx).size == 0  # m = 0
 
 
-def test_prefill_shape_full_size_properties(ctx, orc):
-    """benchmark configuration 3 shape (M = 2048, q_proj 4096 -> 4096) at full size: the oracle would
-    need 3.4e10 scalar MACs, so check (a) 48 sampled rows bit-exactly against the oracle and
-    (b) the sum over ALL accumulators against the exact identity
-        sum_{m,n} acc[m,n] = sum_k (sum_m a_i8[m,k]) * (sum_n w_t[n,k])   (int64)."""
-    from peregrine_amd import quant
-    m, k, n = 2048, 4096, 4096
-    say(f"prefill full size m={m} k={k} n={n}")
-    a = orc.rng_normal(4321, m * k).reshape(m, k)
-    chan = np.random.default_rng(1).choice(k, k // 100, replace=False)
-    a[:, chan] *= 20  # 1 % outlier channels
-    w = orc.rng_normal(8765, k * n, 0.0, 0.02)
-    qt = quant.quantize_weights(w, k, n, ctx)
+def last_tile(ctx):
+    """(rows, columns, K splits) of the most recent W8A8 matrix-core launch on this context."""
+    from peregrine_amd import _ffi
+    bm, bn, sp = C.c_int(), C.c_int(), C.c_int()
+    _ffi.check(_ffi.lib.pg_gemm_w8a8_last_tile(ctx.handle, C.byref(bm), C.byref(bn), C.byref(sp)))
+    return bm.value, bn.value, sp.value
+
+
+def outlier_acts(orc, seed, m, k):
+    """N(0,1) activations with 1 % of the channels scaled x20 (benchmark configuration 3)."""
+    a = orc.rng_normal(seed, m * k).reshape(m, k)
+    chan = np.random.default_rng(seed).choice(k, max(1, k // 100), replace=False)
+    a[:, chan] *= 20
+    return a
+
+
+def np_epilogue(acc, a_s, w_s):
+    """((acc as f32) * a_scale[m]) * w_scale[n] in IEEE single, the order of src/quant.rs:163."""
+    return (acc.astype(np.float32) * a_s.astype(np.float32)[:, None]) * w_s.astype(np.float32)[None, :]
+
+
+# benchmark configuration 3: the seven products of one Llama-3-8B layer at M = 2048 are these four shapes;
+# the last column is the output tile the dispatcher must pick (so a dispatcher change cannot
+# silently leave a tile shape without a test)
+PREFILL_SHAPES = [
+    ("q/o_proj", 2048, 4096, 4096, (128, 256)),
+    ("k/v_proj", 2048, 4096, 1024, (128, 64)),
+    ("gate/up_proj", 2048, 4096, 14336, (256, 256)),
+    ("down_proj", 2048, 14336, 4096, (128, 256)),
+    ("unsplit 128x128", 1024, 256, 4096, (128, 128)),
+]
+
+
+@pytest.mark.parametrize("name,m,k,n,tile", PREFILL_SHAPES, ids=[p[0] for p in PREFILL_SHAPES])
+def test_prefill_shape_full_size_properties(ctx, orc, name, m, k, n, tile):
+    """Every product shape of benchmark configuration 3 at full size (the oracle would need up to
+    1.2e11 scalar MACs for one of them), checked through:
+      (a) one row out of every 32-row band of the output (64 rows at M = 2048: every MFMA row tile
+          of every workgroup tile, all columns) bit-exactly against the oracle, accumulators and f32;
+      (b) 96 sampled columns over ALL rows against an int32 NumPy product of the oracle's
+          quantised operands and the IEEE-single epilogue in the reference's order;
+      (c) the sum over ALL accumulators against the exact identity
+            sum_{m,n} acc[m,n] = sum_k (sum_m a_i8[m,k]) * (sum_n w_t[n,k])   (int64);
+      (d) the f32-only call (no accumulator dump: the straight-line, non-temporal epilogue the
+          benchmark runs) against the f32 output of the dumping call, every element;
+      (e) the tile shape the dispatcher chose."""
+    from peregrine_amd import quant, _ffi
+    say(f"prefill full size {name}: m={m} k={k} n={n}")
+    a = outlier_acts(orc, 4321 + n, m, k)
+    w = orc.rng_normal(8765 + k, k * n, 0.0, 0.02)
     q, q_t, s = orc.quantize_weights(w, k, n)
-    assert (qt.data_i8_t == q_t).all() and (bits(qt.scales) == bits(s)).all()
+    qt = quant.QuantizedTensor(q, q_t, s, k, n)
+    del w
     got, acc = run_matmul_dev(ctx, a, m, k, qt)
+    assert last_tile(ctx) == tile + (1,), f"dispatcher picked {last_tile(ctx)}, the test expects {tile}"
     got, acc = got.reshape(m, n), acc.reshape(m, n)
     a_i8, a_s = orc.quantize_activations(a, m, k)
-    col = a_i8.reshape(m, k).astype(np.int64).sum(axis=0)
+    a_i8 = a_i8.reshape(m, k)
+    # (c)
+    col = a_i8.astype(np.int64).sum(axis=0)
     wsum = q_t.reshape(n, k).astype(np.int64).sum(axis=0)
     assert int(acc.astype(np.int64).sum()) == int((col * wsum).sum())
-    rows = np.random.default_rng(2).choice(m, 48, replace=False)
+    # (a)
+    rng = np.random.default_rng(2)
+    rows = np.arange(0, m, 32) + rng.integers(0, 32, size=(m + 31) // 32)
+    rows = rows[rows < m]
     want, want_acc = orc.matmul_quantized(a[rows], len(rows), k, q_t, s, n)
     assert (acc[rows] == want_acc.reshape(len(rows), n)).all()
     assert (bits(got[rows]) == bits(want.reshape(len(rows), n))).all()
+    # (b)
+    cols = np.unique(np.concatenate([rng.choice(n, 90, replace=False), [0, 31, 32, n - 33, n - 32, n - 1]]))
+    wc = q_t.reshape(n, k)[cols].astype(np.float64)          # [cols, k]
+    acc_c = (a_i8.astype(np.float64) @ wc.T).astype(np.int32)  # exact: every partial sum is an integer below 2^53
+    assert (acc[:, cols] == acc_c).all()
+    assert (bits(got[:, cols]) == bits(np_epilogue(acc_c, a_s, s[cols]))).all()
+    # (d)
+    da = DevBuf(ctx, host=a)
+    dout = DevBuf(ctx, m * n * 4)
+    _ffi.check(_ffi.lib.pg_matmul_quantized_dev(ctx.handle, da.ptr, m, k, qt._gpu, dout.ptr, None))
+    ctx.sync()
+    assert last_tile(ctx) == tile + (1,)
+    assert (bits(dout.to_host(np.float32)) == bits(got).reshape(-1)).all(), "f32-only epilogue differs"
+    qt.free_gpu()
+
+
+# pg_gemm_w8a8_force_tile codes -> output tile
+TILES = {1: (64, 64), 2: (256, 256), 3: (128, 256), 4: (128, 64), 5: (128, 128)}
+
+
+@pytest.mark.parametrize("m,k,n", [(300, 512, 1000), (512, 384, 768), (70, 128, 257)])
+def test_every_gemm_tile_gives_the_same_bits(ctx, orc, m, k, n):
+    """Each instantiation of the matrix-core kernel, forced in turn on ragged and whole-tile
+    shapes, with and without the accumulator dump, against the oracle."""
+    from peregrine_amd import quant, _ffi
+    a = outlier_acts(orc, 99 + m, m, k)
+    w = orc.rng_normal(55 + n, k * n, 0.0, 0.02)
+    q, q_t, s = orc.quantize_weights(w, k, n)
+    qt = quant.QuantizedTensor(q, q_t, s, k, n).to_gpu(ctx)
+    want, want_acc = orc.matmul_quantized(a, m, k, q_t, s, n)
+    da = DevBuf(ctx, host=a)
+    dout, dacc = DevBuf(ctx, m * n * 4), DevBuf(ctx, m * n * 4)
+    try:
+        for code, tile in TILES.items():
+            say(f"gemm tile {tile} on m={m} k={k} n={n}")
+            _ffi.check(_ffi.lib.pg_gemm_w8a8_force_tile(ctx.handle, code))
+            for acc_ptr in (dacc.ptr, None):
+                _ffi.check(_ffi.lib.pg_matmul_quantized_dev(ctx.handle, da.ptr, m, k, qt._gpu, dout.ptr, acc_ptr))
+                ctx.sync()
+                bm, bn, sp = last_tile(ctx)
+                if sp == 1:  # (a split product keeps its own row tile)
+                    assert (bm, bn) == tile
+                assert (bits(dout.to_host(np.float32)) == bits(want)).all(), f"tile {tile}: f32 outputs differ"
+            assert (dacc.to_host(np.int32) == want_acc).all(), f"tile {tile}: accumulators differ"
+    finally:
+        _ffi.check(_ffi.lib.pg_gemm_w8a8_force_tile(ctx.handle, 0))
+    assert _ffi.lib.pg_gemm_w8a8_force_tile(ctx.handle, 9) == _ffi.PG_EINVAL
+    qt.free_gpu()
+
+
+def run_multi(ctx, da, m, k, qts, douts):
+    from peregrine_amd import _ffi
+    wtab = (C.c_void_p * len(qts))(*[q._gpu.value for q in qts])
+    otab = (C.c_void_p * len(qts))(*[d.ptr.value for d in douts])
+    _ffi.check(_ffi.lib.pg_matmul_quantized_multi_dev(ctx.handle, da.ptr, m, k, wtab, len(qts), otab))
+    ctx.sync()
+
+
+@pytest.mark.parametrize("m,k,ns", [(300, 512, (1000, 130, 257)), (257, 128, (64, 64, 64, 64)), (40, 1024, (300, 77)),
+                                     (1, 4096, (1024, 512)), (3, 200, (33,)), (2048, 4096, (4096, 1024, 1024)),
+                                     (2048, 4096, (14336, 14336))],
+                         ids=["ragged3", "four", "few-rows", "one-row", "single", "qkv", "gate-up"])
+def test_matmul_quantized_multi_equals_the_single_products(ctx, orc, m, k, ns):
+    """Several weights against one activation matrix (the reference's fused QKV / gate|up
+    products): every output equals the single product bit for bit, and sampled rows equal the
+    oracle."""
+    from peregrine_amd import quant, _ffi
+    say(f"matmul_quantized_multi m={m} k={k} ns={ns}")
+    a = outlier_acts(orc, 7 + m, m, k)
+    da = DevBuf(ctx, host=a)
+    qts, parts = [], []
+    for i, n in enumerate(ns):
+        w = orc.rng_normal(100 + 13 * i + n, k * n, 0.0, 0.02)
+        q, q_t, s = orc.quantize_weights(w, k, n)
+        parts.append((q_t, s))
+        qts.append(quant.QuantizedTensor(q, q_t, s, k, n).to_gpu(ctx))
+    douts = [DevBuf(ctx, m * n * 4) for n in ns]
+    run_multi(ctx, da, m, k, qts, douts)
+    if m == 2048 and len(ns) == 2:
+        assert last_tile(ctx)[:2] == (256, 256)
+    rows = np.unique(np.random.default_rng(3).choice(m, min(m, 24), replace=False))
+    single = DevBuf(ctx, m * max(ns) * 4)
+    for i, n in enumerate(ns):
+        got = douts[i].to_host(np.float32)
+        _ffi.check(_ffi.lib.pg_matmul_quantized_dev(ctx.handle, da.ptr, m, k, qts[i]._gpu, single.ptr, None))
+        ctx.sync()
+        assert (bits(got) == bits(single.to_host(np.float32, m * n))).all(), f"weight {i}: differs from the single product"
+        want, _ = orc.matmul_quantized(a[rows], len(rows), k, parts[i][0], parts[i][1], n)
+        assert (bits(got.reshape(m, n)[rows]) == bits(want.reshape(len(rows), n))).all(), f"weight {i}: differs from the oracle"
+    # argument errors: too many weights, a weight with another k
+    five = (C.c_void_p * 5)(*[qts[0]._gpu.value] * 5)
+    outs5 = (C.c_void_p * 5)(*[douts[0].ptr.value] * 5)
+    assert _ffi.lib.pg_matmul_quantized_multi_dev(ctx.handle, da.ptr, m, k, five, 5, outs5) == _ffi.PG_EINVAL
+    assert _ffi.lib.pg_matmul_quantized_multi_dev(ctx.handle, da.ptr, m, k + 1, five, 1, outs5) == _ffi.PG_EINVAL
+    for qt in qts:
+        qt.free_gpu()
 
 
 def test_wire_record_straight_to_device(ctx, orc):
