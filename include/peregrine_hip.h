@@ -137,6 +137,19 @@ pg_status pg_matmul_quantized(pg_ctx *ctx, const float *a, size_t m, size_t k,
 pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
                                   const pg_qtensor *w, float *out_dev, int32_t *acc_dev);
 
+/* pg_matmul_quantized_dev for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same result, bit for bit; the scratch the product needs (quantised rows, row
+ * scales, split-K partial sums) is a fixed 32 MiB array inside the library instead of the
+ * context's growable arena, so the call allocates and frees nothing.  A product that needs more
+ * than pg_fixed_scratch_bytes() -- about round_up(m, 256) * round_up(k, 128) + 4 * round_up(m, 256)
+ * bytes, plus up to 16 * m * n * 4 for 5 .. 256 rows -- is PG_EINVAL (2048 x 14336 rows fit).
+ * Every call on one GPU shares that GPU's array: calls that overlap on one GPU (two contexts,
+ * two streams) race; calls on one context are stream-ordered and safe. */
+pg_status pg_matmul_quantized_fixed_scratch_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
+                                                const pg_qtensor *w, float *out_dev);
+size_t pg_fixed_scratch_bytes(void);
+
 /* The fused products of models::llama: `x.matmul(qkv_fused)` / `normed.matmul(gate_up_fused)`
  * over column-concatenated weights (fuse_qkv  src/models/llama/attention.rs:51-71, used :84;
  * fuse_gate_up  src/models/llama/decoder.rs:49-67, used :78), here without a fused copy:

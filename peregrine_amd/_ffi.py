@@ -50,6 +50,8 @@ SIGNATURES = {
     "pg_matmul_quantized": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_matmul_quantized_dev": [_vp, _vp, _sz, _sz, _vp, _vp, _vp],
     "pg_matmul_quantized_multi_dev": [_vp, _vp, _sz, _sz, _pp, _sz, _pp],
+    "pg_matmul_quantized_fixed_scratch_dev": [_vp, _vp, _sz, _sz, _vp, _vp],
+    "pg_fixed_scratch_bytes": [],
     "pg_gemm_w8a8_last_tile": [_vp, C.POINTER(_int), C.POINTER(_int), C.POINTER(_int)],
     "pg_gemm_w8a8_force_tile": [_vp, _int],
     "pg_matmul_dequant_i8": [_vp, _vp, _sz, _sz, _vp, _vp],
@@ -138,6 +140,7 @@ _OTHER_RESTYPE = {
     "pg_kv_cache_free": None,
     "pg_llama_block_free": None,
     "pg_kv_cache_len": _sz,
+    "pg_fixed_scratch_bytes": _sz,
     "pg_kv_cache_capacity": _sz,
     "pg_ctx_stream": _vp,
     "pg_last_error": C.c_char_p,

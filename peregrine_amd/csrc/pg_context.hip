@@ -82,6 +82,7 @@ PG_API pg_status pg_ctx_create(int device, void *hip_stream, pg_ctx **out) {
     ctx->ws_bytes = 0;
     ctx->num_cu = prop.multiProcessorCount;
     ctx->profiling = false;
+    ctx->lds_raised.reserve(64);  // so that noting a kernel's raised LDS limit never allocates later
     if (hip_stream) {
         ctx->stream = static_cast<hipStream_t>(hip_stream);
         ctx->owns_stream = false;

@@ -551,6 +551,46 @@ PG_API pg_status pg_matmul_quantized_dev(pg_ctx *ctx, const float *a_dev, size_t
     return matmul_quantized_on(ctx, a_dev, m, k, w, out_dev, acc_dev, nullptr, 0);
 }
 
+// ---- the same product for callers that cannot allocate ------------------------------------
+// The scratch of pg_matmul_quantized_dev (quantised rows, row scales, split-K partial planes)
+// lives in a file-scope device array instead of the context's growable arena.  Each GPU the
+// library runs on holds its own copy of the array, at its own address, until the process ends;
+// host code never passes the array's name to a kernel (on the host the name is only a stand-in
+// for hipGetSymbolAddress), only the per-device address resolved below.
+constexpr size_t PG_FIXED_SCRATCH_BYTES = 32u << 20;
+static __device__ __align__(256) unsigned char scratch[PG_FIXED_SCRATCH_BYTES];
+constexpr int PG_MAX_DEVICES = 64;
+static void *g_fixed_scratch[PG_MAX_DEVICES];  // device address of `scratch` per device, null until resolved
+
+// With ctx's device current: the address of this device's copy of the array.
+static pg_status fixed_scratch_for(pg_ctx *ctx, void **out) {
+    PG_CHECK_ARG(ctx->device >= 0 && ctx->device < PG_MAX_DEVICES, "device %d: the fixed scratch covers devices 0 .. %d", ctx->device,
+                 PG_MAX_DEVICES - 1);
+    void *p = g_fixed_scratch[ctx->device];
+    if (!p) {
+        PG_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return pg_fail(PG_EDEVICE, "hipGetSymbolAddress returned a null address for the fixed scratch");
+        g_fixed_scratch[ctx->device] = p;
+    }
+    *out = p;
+    return PG_OK;
+}
+
+PG_API pg_status pg_matmul_quantized_fixed_scratch_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
+                                                       const pg_qtensor *w, float *out_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(w != nullptr, "pg_matmul_quantized_fixed_scratch: null weights");
+    PG_CHECK_ARG(w->rows == k, "pg_matmul_quantized_fixed_scratch: a has k = %zu but w has %zu rows", k, w->rows);
+    if (m == 0) return PG_OK;
+    PG_CHECK_ARG(a_dev && out_dev, "pg_matmul_quantized_fixed_scratch: null pointer");
+    PG_CHECK_ARG(m < (1ull << 24), "pg_matmul_quantized_fixed_scratch: m = %zu too large", m);
+    void *fixed = nullptr;
+    PG_TRY(fixed_scratch_for(ctx, &fixed));
+    return matmul_quantized_on(ctx, a_dev, m, k, w, out_dev, nullptr, fixed, PG_FIXED_SCRATCH_BYTES);
+}
+
+PG_API size_t pg_fixed_scratch_bytes(void) { return PG_FIXED_SCRATCH_BYTES; }
+
 // One activation matrix against several weights of equal K: the reference multiplies by
 // column-concatenated weights (fuse_qkv src/models/llama/attention.rs:51-71, fuse_gate_up
 // src/models/llama/decoder.rs:49-67) and slices the result; per-column weight scales and per-row
