@@ -81,6 +81,26 @@ pg_status pg_profile_begin(pg_ctx *ctx);
 pg_status pg_profile_end(pg_ctx *ctx, size_t *num_kernels);
 pg_status pg_profile_get(pg_ctx *ctx, size_t i, const char **name, double *total_ms,
                          size_t *launches);
+/* The distinct launch sizes (work-items = grid x workgroup, as a kernel trace lists them) behind
+ * entry i and how many launches had each: up to `cap` pairs are written, *count gets their number.
+ * Lets a benchmark check that a stored counter summary still describes the launches it makes. */
+pg_status pg_profile_get_grids(pg_ctx *ctx, size_t i, size_t *work_items, size_t *launches, size_t cap,
+                               size_t *count);
+
+/* Ceilings of the part, measured (no counterpart in the reference; a benchmark reports them
+ * beside the published peaks):
+ *   pg_probe_mfma_i8    int8 matrix-core rate with every operand in registers, in TOP/s (2 ops
+ *                       per multiply-add), one workgroup of 8 wavefronts per CU for `iters` x 8
+ *                       MFMAs per wavefront, and the shader clock the loop ran at;
+ *   pg_probe_hbm_read   a pure 128-bit read stream: `passes` kernels, each reading
+ *                       bytes_per_pass from one of `buffers` distinct buffers in turn (make
+ *                       buffers x bytes_per_pass exceed the 256 MB last-level cache), in GB/s;
+ *   pg_probe_gemm_clock the shader clock inside the K loop of the W8A8 GEMM's 256x256 tile on an
+ *                       [m x k] . [k x n] product, and the mean duration of a workgroup's loop.
+ * Each allocates its own buffers and waits for completion. */
+pg_status pg_probe_mfma_i8(pg_ctx *ctx, int iters, double *tops, double *clock_ghz);
+pg_status pg_probe_hbm_read(pg_ctx *ctx, size_t bytes_per_pass, int buffers, int passes, double *gbs);
+pg_status pg_probe_gemm_clock(pg_ctx *ctx, size_t m, size_t k, size_t n, double *clock_ghz, double *loop_us);
 
 /* Device memory for callers that have no HIP binding of their own
  * (GpuContext::alloc / upload / GpuBuffer::read, src/metal/buffer.rs). */

@@ -403,8 +403,8 @@ done:
 /* ------------------------------------------------------------------------
  * Input synthesis: SplitMix64-seeded Xoshiro256++ and Box-Muller normals
  *                                    reference: src/random.rs:16-53, 311-380
- *   (the sequential generator; the reference switches to a Philox path above
- *   a size threshold, which is not restated).
+ *   (the sequential generator; at 200 000 elements and more the reference
+ *   switches to the counter-based Philox path restated further down).
  * ---------------------------------------------------------------------- */
 typedef struct { uint64_t s[4]; } orc_rng;
 
@@ -451,5 +451,73 @@ ORC_API void orc_rng_normal(uint64_t seed, size_t n, float mean, float std, floa
         float theta = 2.0f * 3.14159265358979323846f * u2;
         out[2 * i] = mean + std * rad * cosf(theta);
         if (2 * i + 1 < n) out[2 * i + 1] = mean + std * rad * sinf(theta);
+    }
+}
+
+/* ------------------------------------------------------------------------
+ * Input synthesis, large tensors: Philox 4x32-10 counter-based generator and
+ * the normal() front end that chooses between the two generators
+ *                         reference: src/random.rs:72-103, 147-270, 273-380
+ * ---------------------------------------------------------------------- */
+#define ORC_PHILOX_THRESHOLD 200000u /* src/random.rs:79 */
+
+/* philox_4x32_10  src/random.rs:88-103 */
+ORC_API void orc_philox_4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]) {
+    uint32_t c[4] = {counter[0], counter[1], counter[2], counter[3]};
+    uint32_t k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; ++r) {
+        uint64_t p0 = (uint64_t)0xD2511F53u * c[0], p1 = (uint64_t)0xCD9E8D57u * c[2];
+        uint32_t lo0 = (uint32_t)p0, hi0 = (uint32_t)(p0 >> 32), lo1 = (uint32_t)p1, hi1 = (uint32_t)(p1 >> 32);
+        uint32_t n0 = hi1 ^ c[1] ^ k0, n2 = hi0 ^ c[3] ^ k1;
+        c[0] = n0; c[1] = lo1; c[2] = n2; c[3] = lo0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c[0]; out[1] = c[1]; out[2] = c[2]; out[3] = c[3];
+}
+
+/* random::seed + the two pieces of global state  src/random.rs:11-14, 273-278 */
+typedef struct { orc_rng xo; uint64_t philox_counter; } orc_random;
+
+ORC_API void orc_random_seed(orc_random *st, uint64_t seed) {
+    orc_rng_seed(&st->xo, seed);
+    st->philox_counter = seed;
+}
+
+/* philox_normal_parallel  src/random.rs:147-270 (non-macOS transform :248-258) */
+static void philox_normal(orc_random *st, size_t n, float mean, float std, float *out) {
+    const size_t alloc_n = n + (n & 1), pairs = alloc_n / 2, calls = (pairs + 3) / 4;
+    const uint64_t base = st->philox_counter;
+    st->philox_counter += (uint64_t)calls * 2;
+    const uint32_t key_u1[2] = {0xDEADBEEFu, 0xCAFEBABEu}, key_u2[2] = {0xFEEDFACEu, 0xBAADF00Du};
+    const float scale = 1.0f / (float)(1ull << 32), two_pi = 2.0f * 3.14159265358979323846f;
+    for (size_t call = 0; call < calls; ++call) {
+        const uint64_t c1 = base + call, c2 = base + calls + call;
+        const uint32_t ctr1[4] = {(uint32_t)c1, (uint32_t)(c1 >> 32), 0, 0}, ctr2[4] = {(uint32_t)c2, (uint32_t)(c2 >> 32), 0, 0};
+        uint32_t o1[4], o2[4];
+        orc_philox_4x32_10(ctr1, key_u1, o1);
+        orc_philox_4x32_10(ctr2, key_u2, o2);
+        for (size_t j = 0; j < 4 && 4 * call + j < pairs; ++j) {
+            const size_t i = 4 * call + j;
+            const float u1 = fmaxf((float)o1[j] * scale, 1e-10f), u2 = (float)o2[j] * scale;
+            const float r = sqrtf(-2.0f * logf(u1)), theta = two_pi * u2;
+            if (2 * i < n) out[2 * i] = mean + std * r * cosf(theta);
+            if (2 * i + 1 < n) out[2 * i + 1] = mean + std * r * sinf(theta);
+        }
+    }
+}
+
+/* random::normal  src/random.rs:311-380 (non-macOS branch :364-378) */
+ORC_API void orc_random_normal(orc_random *st, size_t n, float mean, float std, float *out) {
+    if (n >= ORC_PHILOX_THRESHOLD) {
+        philox_normal(st, n, mean, std, out);
+        return;
+    }
+    const size_t pairs = (n + 1) / 2;
+    for (size_t i = 0; i < pairs; ++i) {  /* pair by pair: the stream is consumed in the reference's order */
+        const float u1 = fmaxf(rng_next_f32(&st->xo), 1e-10f), u2 = rng_next_f32(&st->xo);
+        const float r = sqrtf(-2.0f * logf(u1)), theta = 2.0f * 3.14159265358979323846f * u2;
+        out[2 * i] = mean + std * r * cosf(theta);
+        if (2 * i + 1 < n) out[2 * i + 1] = mean + std * r * sinf(theta);
     }
 }

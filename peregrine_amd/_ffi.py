@@ -33,6 +33,10 @@ SIGNATURES = {
     "pg_profile_begin": [_vp],
     "pg_profile_end": [_vp, C.POINTER(_sz)],
     "pg_profile_get": [_vp, _sz, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(_sz)],
+    "pg_probe_mfma_i8": [_vp, _int, C.POINTER(C.c_double), C.POINTER(C.c_double)],
+    "pg_probe_hbm_read": [_vp, _sz, _int, _int, C.POINTER(C.c_double)],
+    "pg_probe_gemm_clock": [_vp, _sz, _sz, _sz, C.POINTER(C.c_double), C.POINTER(C.c_double)],
+    "pg_profile_get_grids": [_vp, _sz, C.POINTER(_sz), C.POINTER(_sz), _sz, C.POINTER(_sz)],
     "pg_dev_alloc": [_vp, _sz, _pp],
     "pg_dev_free": [_vp, _vp],
     "pg_memcpy_h2d": [_vp, _vp, _vp, _sz],

@@ -41,6 +41,20 @@ class Context:
             out[name.value.decode()] = (ms.value, cnt.value)
         return out
 
+    def profile_grids(self):
+        """After profile_end(): {kernel name: {work-items of a launch: launches}}."""
+        out = {}
+        i = 0
+        while True:
+            name = C.c_char_p()
+            if _ffi.lib.pg_profile_get(self.handle, i, C.byref(name), None, None) != _ffi.PG_OK:
+                break
+            w, n, cnt = (C.c_size_t * 16)(), (C.c_size_t * 16)(), C.c_size_t()
+            _ffi.check(_ffi.lib.pg_profile_get_grids(self.handle, i, w, n, 16, C.byref(cnt)))
+            out[name.value.decode()] = {int(w[j]): int(n[j]) for j in range(min(cnt.value, 16))}
+            i += 1
+        return out
+
     def close(self):
         if self._h:
             _ffi.lib.pg_ctx_destroy(self._h)

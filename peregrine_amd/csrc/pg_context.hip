@@ -105,7 +105,8 @@ PG_API void pg_ctx_destroy(pg_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void)hipFree(ctx->ws);
-    if (ctx->moe_tab_dev) (void)hipFree(ctx->moe_tab_dev);
+    for (auto &t : ctx->moe_tabs)
+        if (t.dev) (void)hipFree(t.dev);
     prof_drop(ctx);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
@@ -184,11 +185,15 @@ PG_API pg_status pg_profile_end(pg_ctx *ctx, size_t *num_kernels) {
         for (auto &x : ctx->totals)
             if (x.name == r.name) t = &x;
         if (!t) {
-            ctx->totals.push_back({r.name, 0.0, 0});
+            ctx->totals.push_back({r.name, 0.0, 0, {}});
             t = &ctx->totals.back();
         }
         t->total_ms += ms;
         t->launches += 1;
+        bool seen = false;
+        for (auto &g : t->grids)
+            if (g.first == r.threads) { g.second += 1; seen = true; }
+        if (!seen) t->grids.push_back({r.threads, 1});
     }
     prof_drop(ctx);
     if (num_kernels) *num_kernels = ctx->totals.size();
@@ -202,5 +207,17 @@ PG_API pg_status pg_profile_get(pg_ctx *ctx, size_t i, const char **name, double
     if (name) *name = ctx->totals[i].name.c_str();
     if (total_ms) *total_ms = ctx->totals[i].total_ms;
     if (launches) *launches = ctx->totals[i].launches;
+    return PG_OK;
+}
+
+PG_API pg_status pg_profile_get_grids(pg_ctx *ctx, size_t i, size_t *work_items, size_t *launches, size_t cap, size_t *count) {
+    PG_CHECK_ARG(ctx != nullptr, "null context");
+    PG_CHECK_ARG(i < ctx->totals.size(), "pg_profile_get_grids: index %zu of %zu", i, ctx->totals.size());
+    const auto &g = ctx->totals[i].grids;
+    if (count) *count = g.size();
+    for (size_t j = 0; j < g.size() && j < cap; ++j) {
+        if (work_items) work_items[j] = g[j].first;
+        if (launches) launches[j] = g[j].second;
+    }
     return PG_OK;
 }

@@ -58,11 +58,13 @@ struct gemm_wgroup {
     int panel0[PG_GEMM_MAX_GROUP];
 };
 
-template <int BM, int BN, int BK, int NST, int NWM, int NWN, int OCC>
+// CLK (the clock probe only): thread 0 of every workgroup also stores the shader cycles and the
+// wall-clock ticks its K loop took, clk[2 * blockIdx.x] and clk[2 * blockIdx.x + 1].
+template <int BM, int BN, int BK, int NST, int NWM, int NWN, int OCC, bool CLK = false>
 __global__ __launch_bounds__(64 * NWM * NWN) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const gemm_wgroup grp, int ldb,
                       const float *__restrict__ a_scales, int32_t *__restrict__ acc_out, int M, int K,
-                      int tiles_m, int ntiles, int kt_per_split) {
+                      int tiles_m, int ntiles, int kt_per_split, long long *__restrict__ clk) {
     constexpr int NW = NWM * NWN;
     constexpr int WM = BM / NWM, WN = BN / NWN;      // wavefront tile
     constexpr int TM = WM / 32, TN = WN / 32;        // 32x32 MFMA tiles per wavefront
@@ -182,6 +184,8 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const gemm_wgroup g
     static_assert(NST >= 2 && NST <= 6, "wait_barrier covers up to 4 stages in flight beyond the awaited one");
 
     const int KT = (K / BK - kt0_split < kt_per_split) ? K / BK - kt0_split : kt_per_split;
+    long long clk_c0 = 0, clk_w0 = 0;
+    if constexpr (CLK) { clk_c0 = clock64(); clk_w0 = wall_clock64(); }
 #pragma unroll
     for (int s = 0; s < NST - 1; ++s)
         if (s < KT) issue(s, s * BK);
@@ -225,6 +229,12 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const gemm_wgroup g
         }
     }
 
+    if constexpr (CLK) {
+        if (threadIdx.x == 0) {
+            clk[2 * blockIdx.x] = clock64() - clk_c0;
+            clk[2 * blockIdx.x + 1] = wall_clock64() - clk_w0;
+        }
+    }
     // ---- epilogue.  Accumulator register r of a 32x32 tile holds
     // row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.  (The scales were requested before the
     // K loop: loading them here would put several dependent memory round trips on every tile.)
@@ -317,7 +327,7 @@ pg_status launch_group(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const f
     ctx->gemm_last_bn = BN;
     ctx->gemm_last_splits = splits;
     PG_TRY(pg_launch(ctx, "gemm_w8a8", kern, dim3(grid, (unsigned)splits), dim3(64 * NWM * NWN), lds, a_i8, (int)a_stride, grp,
-                     (int)k_pad, a_scales, acc, (int)m, (int)k_pad, tiles_m, ntiles, kt_per_split));
+                     (int)k_pad, a_scales, acc, (int)m, (int)k_pad, tiles_m, ntiles, kt_per_split, (long long *)nullptr));
     return pg_launch_check("gemm_w8a8");
 }
 
@@ -365,8 +375,12 @@ pg_status gemm_dispatch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const 
     };
     int pick = ctx->gemm_force_tile;
     if (pick == 0) {
+        const size_t t256 = tiles(256, 256);
         if (m <= 64) pick = 1;
-        else if (tiles(256, 256) * 2 >= 3 * cus) pick = 2;
+        // one and a half rounds of the largest tile or more -- or a single round that fills at least 70 %
+        // of the CUs: the fused q|k|v product (192 tiles on 256 CUs) runs 56 us so against 65 us as
+        // 384 half-size tiles (the CUs left idle let the busy ones clock higher)
+        else if (t256 * 2 >= 3 * cus || (t256 <= cus && t256 * 10 >= 7 * cus)) pick = 2;
         else if (tiles(128, 256) >= cus) pick = 3;
         // Too few 128x128 tiles for the CUs (k/v projections, N = 1024): halve the tile instead of
         // leaving half of the chip idle (21.2 -> 16.5 us at 2048 x 4096 -> 1024).
@@ -437,4 +451,52 @@ pg_status pg_launch_gemm_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
     if (w->k_pad >= (1ull << 22) || m >= (1ull << 24) || w->cols >= (1ull << 30))
         return pg_fail(PG_EUNSUPPORTED, "gemm_w8a8: shape exceeds the kernel's 32-bit tile offsets");
     return gemm_dispatch(ctx, a_i8, a_stride, a_scales, &w, &out, 1, m, acc);
+}
+
+// The shader clock inside the K loop of the 256x256 tile (the gate|up product's kernel): the
+// product [m x k] . [k x n] on pseudo-random operands, every workgroup timing its own loop with
+// the shader cycle counter and the constant-rate wall clock.
+PG_API pg_status pg_probe_gemm_clock(pg_ctx *ctx, size_t m, size_t k, size_t n, double *clock_ghz, double *loop_us) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(m >= 256 && m <= 8192 && k >= 256 && k <= 32768 && n >= 256 && n <= 65536 && m % 256 == 0 && k % 128 == 0 && n % 256 == 0,
+                 "pg_probe_gemm_clock: m %zu, n %zu must be multiples of 256 and k %zu of 128, within 8192 x 32768 x 65536", m, n, k);
+    constexpr int BM = 256, BN = 256, BK = 128, NST = 2;
+    const int tiles_m = (int)(m / BM), ntiles = tiles_m * (int)(n / BN);
+    const unsigned grid = (unsigned)(((ntiles + 7) / 8) * 8);
+    pg_tmp a, b, sc, out, clk;
+    PG_TRY(a.alloc(m * k));
+    PG_TRY(b.alloc(n * k));
+    PG_TRY(sc.alloc((m > n ? m : n) * sizeof(float)));
+    PG_TRY(out.alloc(m * n * sizeof(float)));
+    PG_TRY(clk.alloc((size_t)grid * 2 * sizeof(long long)));
+    PG_TRY(pg_probe_fill_random(ctx, a.p, m * k));
+    PG_TRY(pg_probe_fill_random(ctx, b.p, n * k));
+    PG_HIP(hipMemsetAsync(sc.p, 0, (m > n ? m : n) * sizeof(float), ctx->stream));
+    PG_HIP(hipMemsetAsync(clk.p, 0, (size_t)grid * 2 * sizeof(long long), ctx->stream));
+    gemm_wgroup grp;
+    for (int i = 0; i < PG_GEMM_MAX_GROUP; ++i) {
+        grp.w[i] = nullptr;
+        grp.ws[i] = nullptr; grp.out[i] = nullptr; grp.n[i] = 0; grp.panel0[i] = INT_MAX;
+    }
+    grp.w[0] = b.as<int8_t>(); grp.ws[0] = sc.as<float>(); grp.out[0] = out.as<float>(); grp.n[0] = (int)n; grp.panel0[0] = 0;
+    const size_t lds = (size_t)NST * (BM + BN) * BK + (BM + BN) * sizeof(float);
+    auto kern = gemm_w8a8_kernel<BM, BN, BK, NST, 2, 4, 2, true>;
+    PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
+    for (int rep = 0; rep < 20; ++rep)  // the clock settles over the first launches; the last one is read
+        PG_TRY(pg_launch(ctx, "gemm_w8a8_clock_probe", kern, dim3(grid), dim3(512), lds, a.as<int8_t>(), (int)k, grp, (int)k, sc.as<float>(),
+                         (int32_t *)nullptr, (int)m, (int)k, tiles_m, ntiles, (int)(k / BK), clk.as<long long>()));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    std::vector<long long> h((size_t)grid * 2);
+    PG_HIP(hipMemcpy(h.data(), clk.p, h.size() * sizeof(long long), hipMemcpyDeviceToHost));
+    int wall_khz = 0;
+    PG_HIP(hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, ctx->device));
+    double cyc = 0.0, wall = 0.0;
+    int used = 0;
+    for (unsigned i = 0; i < grid; ++i)
+        if (h[2 * i + 1] > 0) { cyc += (double)h[2 * i]; wall += (double)h[2 * i + 1]; ++used; }
+    PG_CHECK_ARG(used > 0 && wall_khz > 0, "pg_probe_gemm_clock: no workgroup reported");
+    const double secs = wall / (wall_khz * 1e3);
+    if (clock_ghz) *clock_ghz = cyc / secs / 1e9;
+    if (loop_us) *loop_us = secs / used * 1e6;
+    return PG_OK;
 }

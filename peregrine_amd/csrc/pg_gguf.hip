@@ -16,6 +16,7 @@
 //    d * s in f32 once per block.
 // The result differs from the reference's dequantise-then-f32-matmul only by rounding noise
 // (relative tolerance 1e-3 is the contract; the tests hold this path to 2e-5).
+#include <mutex>
 #include <new>
 #include "pg_internal.h"
 #include "pg_digits.h"
@@ -442,7 +443,12 @@ __global__ void tile_weights_kernel(const uint8_t *__restrict__ qs, int n_out, i
     *reinterpret_cast<uint4 *>(tiled + rg * pg_tiled_group_bytes(nb, QT == 8) + i * 16) = v;
 }
 
+static std::mutex g_tiled_mutex;
+
 pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w) {
+    // One maker at a time, and the pointer is published only once the copy is complete, so another
+    // context, stream or thread that finds it set may read it at once.
+    std::lock_guard<std::mutex> lock(g_tiled_mutex);
     if (w->qs_tiled) return PG_OK;
     if (w->ggml_type != PG_GGML_Q4_0 && w->ggml_type != PG_GGML_Q8_0)
         return pg_fail(PG_EUNSUPPORTED, "gguf: no tile-major copy for ggml type %d", w->ggml_type);
@@ -460,6 +466,7 @@ pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w) {
                                   (int)w->n_out, nb, p)
                       : pg_launch(ctx, "gguf_tile_weights", tile_weights_kernel<4>, grid, dim3(256), 0, (const uint8_t *)w->qs,
                                   (int)w->n_out, nb, p);
+    if (st == PG_OK && hipStreamSynchronize(ctx->stream) != hipSuccess) st = pg_fail(PG_EDEVICE, "gguf tile-major copy: the stream failed");
     if (st != PG_OK) { (void)hipFree(p); return st; }
     w->qs_tiled = p;
     return PG_OK;
@@ -470,8 +477,9 @@ pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w) {
 pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
                               float *y_dev) {
     void *ws = nullptr;
-    if (m == 1 || w->ggml_type == PG_MXFP4 || w->ggml_type == PG_GGML_Q4_1) {  // these two have the streaming kernel only: one item per row
-        if (m > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_matmul: more than 65535 rows against an MXFP4 or Q4_1 tensor");
+    // MXFP4 and Q4_1 have the streaming kernel only; a K of a few blocks needs its finer fixed point
+    if (m == 1 || w->ggml_type == PG_MXFP4 || w->ggml_type == PG_GGML_Q4_1 || w->k_in / 32 < PG_MM_MIN_BLOCKS) {
+        if (m > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_matmul: more than 65535 rows through the streaming kernel (MXFP4, Q4_1 or k_in < %zu)", PG_MM_MIN_BLOCKS * 32);
         PG_TRY(pg_workspace(ctx, pg_xdigits_bytes(m, w->k_in), &ws));
         const pg_xdigits xd = pg_xdigits_carve(ws, m, w->k_in);
         PG_TRY(pg_launch_x_to_digits(ctx, x_dev, m, w->k_in, w->ggml_type, xd));
@@ -506,7 +514,7 @@ pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, c
         any_mxfp4 |= w[i]->ggml_type == PG_MXFP4;
         any_q41 |= w[i]->ggml_type == PG_GGML_Q4_1;
     }
-    if ((any_mxfp4 && m > 1) || any_q41) {  // no shared route: product by product
+    if ((any_mxfp4 && m > 1) || any_q41 || (m > 1 && k_in / 32 < PG_MM_MIN_BLOCKS)) {  // no shared route: product by product
         for (int i = 0; i < count; ++i) PG_TRY(pg_gguf_matmul_rows(ctx, x_dev, m, w[i], y_dev[i]));
         return PG_OK;
     }

@@ -17,11 +17,13 @@
 struct pg_prof_rec {
     const char *name;
     hipEvent_t start, stop;
+    size_t threads;  // work-items of the launch (grid x block)
 };
 struct pg_prof_total {
     std::string name;
     double total_ms;
     size_t launches;
+    std::vector<std::pair<size_t, size_t>> grids;  // distinct launch sizes (work-items) and how many launches had each
 };
 
 // One device + one stream + one growable scratch arena.
@@ -35,11 +37,13 @@ struct pg_ctx {
     bool profiling;                     // per-kernel HIP events (pg_profile_begin/end)
     std::vector<pg_prof_rec> prof;      // one record per launch while profiling
     std::vector<pg_prof_total> totals;  // aggregated by pg_profile_end
-    // MoE expert pointer tables: the last set uploaded, kept so that repeated calls with the
-    // same experts neither copy nor synchronise.
-    std::vector<const void *> moe_tab_host;
-    void *moe_tab_dev = nullptr;
-    size_t moe_tab_cap = 0;
+    // MoE expert pointer tables, one per distinct set of experts seen (a model's MoE layers
+    // alternate): a repeated call with a known set neither copies nor synchronises.
+    struct moe_table {
+        std::vector<const void *> host;
+        void *dev;
+    };
+    std::vector<moe_table> moe_tabs;
     // Kernels whose dynamic LDS limit was raised on this context's device (pg_allow_dynamic_lds).
     std::vector<const void *> lds_raised;
     // W8A8 GEMM dispatch: the tile of the most recent launch (pg_gemm_w8a8_last_tile) and an
@@ -72,6 +76,12 @@ struct pg_gguf_tensor {
     size_t n_out, k_in;
 };
 
+// The matrix-core block product carries 16-bit fixed-point activations per block: fine when a
+// dot product averages over many blocks, too coarse when one or two blocks make the whole sum
+// (an outlier in the block then costs every other element ~2^-16 of the outlier).  Products
+// whose K spans fewer blocks than this run the streaming kernel (18 / 22-bit activations),
+// one item per activation row.
+constexpr size_t PG_MM_MIN_BLOCKS = 5;
 constexpr size_t PG_KPAD = 128;  // device K stride is a multiple of this
 constexpr size_t PG_NPAD = 256;  // device weight rows are padded to this
 
@@ -126,7 +136,8 @@ inline pg_status pg_launch(pg_ctx *ctx, const char *name, void (*kernel)(KArgs..
     if (ctx->profiling) {
         if (hipEventCreate(&start) != hipSuccess) start = nullptr;
         if (start && hipEventCreate(&stop) != hipSuccess) { (void)hipEventDestroy(start); start = stop = nullptr; }
-        if (start) ctx->prof.push_back({name, start, stop});
+        if (start)
+            ctx->prof.push_back({name, start, stop, (size_t)grid.x * grid.y * grid.z * block.x * block.y * block.z});
     }
     std::tuple<KArgs...> tup{static_cast<KArgs>(args)...};
     void *ptrs[sizeof...(KArgs) ? sizeof...(KArgs) : 1];
@@ -148,6 +159,9 @@ struct pg_tmp {
     }
     template <class T> T *as() const { return static_cast<T *>(p); }
 };
+
+// Fills device memory with pseudo-random bytes (the probes' operands), stream ordered.
+pg_status pg_probe_fill_random(pg_ctx *ctx, void *dev, size_t bytes);
 
 // Kernel launchers implemented per translation unit (device pointers, stream ordered).
 pg_status pg_launch_quantize_activations(pg_ctx *ctx, const float *a, size_t rows, size_t cols,

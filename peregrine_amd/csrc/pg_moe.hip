@@ -119,8 +119,22 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     PG_CHECK_ARG(T * top_k < (1ull << 20), "pg_moe_ffn: too many (token, expert) pairs");
     const size_t P = T * top_k;
 
+    // Which products take the streaming kernel (18 / 22-bit activations, one item per pair) instead
+    // of the matrix-core one (16-bit activations per block):
+    //  * a product whose own K spans only a few blocks (as everywhere);
+    //  * all three when the experts are narrow (ffn < 512).  An error of 2^-16 of a block's
+    //    absmax in g or u is multiplied by the partner factor in h = act(g) * u; where that factor
+    //    is an outlier (|g| of 10 and more happens) the one h element carries an absolute error far
+    //    above the others', and the down product only averages it away over many terms: its share
+    //    of an output's error falls as 1 / sqrt(ffn) (measured 1.4e-3 of the row rms at ffn 64,
+    //    below 2e-4 from ffn 2048 up).  Narrow experts are tiny products; the price is nil.
+    const bool narrow = ffn < 512 && P <= 65535;
+    const bool up_stream = narrow || d / 32 < PG_MM_MIN_BLOCKS, down_stream = narrow || ffn / 32 < PG_MM_MIN_BLOCKS;
+    PG_CHECK_ARG(!(up_stream || down_stream) || P <= 65535, "pg_moe_ffn: too many pairs for experts this small");
+
     // Arena layout.
-    const int ks_up = pg_gguf_mm_splitk(ctx, ffn, d, E, T, true, nullptr), ks_down = pg_gguf_mm_splitk(ctx, d, ffn, E, P, true, nullptr);
+    const int ks_up = up_stream ? 1 : pg_gguf_mm_splitk(ctx, ffn, d, E, T, true, nullptr);
+    const int ks_down = down_stream ? 1 : pg_gguf_mm_splitk(ctx, d, ffn, E, P, true, nullptr);
     const size_t part_floats = std::max(ks_up > 1 ? (size_t)ks_up * P * ffn : 0, ks_down > 1 ? (size_t)ks_down * P * d : 0);
     const size_t sz_idx = pg_round_up(P * sizeof(int), 256);
     const size_t sz_p = pg_round_up(P * sizeof(float), 256);
@@ -128,7 +142,8 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     const size_t sz_act = pg_round_up(P * ffn * sizeof(float), 256);
     const size_t sz_y = pg_round_up(P * d * sizeof(float), 256);
     const size_t sz_part = pg_round_up(part_floats * sizeof(float), 256);
-    const size_t sz_xd = pg_mmdigits_bytes(T, d), sz_hd = pg_mmdigits_bytes(P, ffn);
+    const size_t sz_xd = up_stream ? pg_xdigits_bytes(T, d) : pg_mmdigits_bytes(T, d);
+    const size_t sz_hd = down_stream ? pg_xdigits_bytes(P, ffn) : pg_mmdigits_bytes(P, ffn);
     void *ws = nullptr;
     PG_TRY(pg_workspace(ctx, sz_idx + sz_p + sz_lists + sz_counts + 3 * sz_act + sz_y + sz_part + sz_xd + sz_hd, &ws));
     char *p = static_cast<char *>(ws);
@@ -141,56 +156,81 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     float *h = reinterpret_cast<float *>(p); p += sz_act;
     float *yb = reinterpret_cast<float *>(p); p += sz_y;
     float *part = sz_part ? reinterpret_cast<float *>(p) : nullptr; p += sz_part;
-    const pg_mmdigits xd = pg_mmdigits_carve(p, T, d); p += sz_xd;
-    const pg_mmdigits hd = pg_mmdigits_carve(p, P, ffn);
+    char *xd_base = p; p += sz_xd;
+    char *hd_base = p;
 
     // Expert pointer tables: [gate qs | gate d | up qs | up d | down qs | down d], E each, in a
-    // device buffer the context keeps; uploaded (with a wait, the source is this stack frame)
-    // only when the set of experts differs from the previous call's.
-    // (The quant planes are the tile-major copies, made on an expert's first use.)
+    // device buffer kept with the context, one per distinct set of experts (a model's layers
+    // alternate); uploaded (blocking: the source is this stack frame) only on a set's first use.
+    // The quant planes are the tile-major copies (made on an expert's first use) for the
+    // matrix-core kernel, the row-major planes for the streaming one.
     const void *host_tab[6 * MAX_EXPERTS];
     for (size_t e = 0; e < E; ++e) {
-        PG_TRY(pg_gguf_ensure_tiled(ctx, gate[e]));
-        PG_TRY(pg_gguf_ensure_tiled(ctx, up[e]));
-        PG_TRY(pg_gguf_ensure_tiled(ctx, down[e]));
-        host_tab[0 * E + e] = gate[e]->qs_tiled; host_tab[1 * E + e] = gate[e]->d;
-        host_tab[2 * E + e] = up[e]->qs_tiled;   host_tab[3 * E + e] = up[e]->d;
-        host_tab[4 * E + e] = down[e]->qs_tiled; host_tab[5 * E + e] = down[e]->d;
-    }
-    if (ctx->moe_tab_host.size() != 6 * E || memcmp(ctx->moe_tab_host.data(), host_tab, 6 * E * sizeof(void *)) != 0) {
-        PG_HIP(hipStreamSynchronize(ctx->stream));  // earlier calls may still read the old table
-        if (ctx->moe_tab_cap < 6 * E * sizeof(void *)) {
-            if (ctx->moe_tab_dev) PG_HIP(hipFree(ctx->moe_tab_dev));
-            ctx->moe_tab_dev = nullptr;
-            ctx->moe_tab_cap = 0;
-            PG_HIP(hipMalloc(&ctx->moe_tab_dev, 6 * MAX_EXPERTS * sizeof(void *)));
-            ctx->moe_tab_cap = 6 * MAX_EXPERTS * sizeof(void *);
+        if (!up_stream) {
+            PG_TRY(pg_gguf_ensure_tiled(ctx, gate[e]));
+            PG_TRY(pg_gguf_ensure_tiled(ctx, up[e]));
         }
-        ctx->moe_tab_host.clear();
-        PG_HIP(hipMemcpyAsync(ctx->moe_tab_dev, host_tab, 6 * E * sizeof(void *), hipMemcpyHostToDevice, ctx->stream));
-        PG_HIP(hipStreamSynchronize(ctx->stream));
-        ctx->moe_tab_host.assign(host_tab, host_tab + 6 * E);
+        if (!down_stream) PG_TRY(pg_gguf_ensure_tiled(ctx, down[e]));
+        host_tab[0 * E + e] = up_stream ? gate[e]->qs : gate[e]->qs_tiled; host_tab[1 * E + e] = gate[e]->d;
+        host_tab[2 * E + e] = up_stream ? up[e]->qs : up[e]->qs_tiled;     host_tab[3 * E + e] = up[e]->d;
+        host_tab[4 * E + e] = down_stream ? down[e]->qs : down[e]->qs_tiled; host_tab[5 * E + e] = down[e]->d;
     }
-    const void **tab = static_cast<const void **>(ctx->moe_tab_dev);
+    const void **tab = nullptr;
+    for (const auto &t : ctx->moe_tabs)
+        if (t.host.size() == 6 * E && memcmp(t.host.data(), host_tab, 6 * E * sizeof(void *)) == 0) tab = static_cast<const void **>(t.dev);
+    if (!tab) {
+        if (ctx->moe_tabs.size() >= 64) {  // a bounded cache: drop the oldest set once nothing can still read it
+            PG_HIP(hipStreamSynchronize(ctx->stream));
+            (void)hipFree(ctx->moe_tabs.front().dev);
+            ctx->moe_tabs.erase(ctx->moe_tabs.begin());
+        }
+        void *dev = nullptr;
+        PG_HIP(hipMalloc(&dev, 6 * E * sizeof(void *)));
+        const hipError_t ce = hipMemcpy(dev, host_tab, 6 * E * sizeof(void *), hipMemcpyHostToDevice);
+        if (ce != hipSuccess) {
+            (void)hipFree(dev);
+            return pg_fail(PG_EDEVICE, "pg_moe_ffn: uploading the expert table: %s", hipGetErrorString(ce));
+        }
+        ctx->moe_tabs.push_back({std::vector<const void *>(host_tab, host_tab + 6 * E), dev});
+        tab = static_cast<const void **>(dev);
+    }
 
     PG_TRY(pg_launch(ctx, "moe_route_topk", route_topk_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
                      router_logits_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
     PG_TRY(pg_launch(ctx, "moe_expert_lists", expert_lists_kernel, dim3((unsigned)E), dim3(64), 0, topk_idx, (int)P, (int)T,
                      lists, counts));
-    PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, T, d, type, xd));
     auto table = [&](int which) { return reinterpret_cast<const uint8_t *const *>(tab + which * E); };
     auto dtable = [&](int which) { return reinterpret_cast<const uint16_t *const *>(tab + which * E); };
     // Each token reaches an expert at most once, so an expert owns at most T pairs.
     const int tiles = (int)((T + 31) / 32);
-    const pg_mm_group gg = {(int)E, table(0), dtable(1), lists, counts, (int)T, tiles, (int)T, (int)top_k, 0, 0, 1};
-    PG_TRY(pg_launch_gguf_mm(ctx, type, ffn, d, nullptr, nullptr, gg, P, xd, g, part));
-    const pg_mm_group gu = {(int)E, table(2), dtable(3), lists, counts, (int)T, tiles, (int)T, (int)top_k, 0, 0, 1};
-    PG_TRY(pg_launch_gguf_mm(ctx, type, ffn, d, nullptr, nullptr, gu, P, xd, u, part));
+    if (up_stream) {  // pair p: activation row p / top_k against expert topk_idx[p]
+        const pg_xdigits xd = pg_xdigits_carve(xd_base, T, d);
+        PG_TRY(pg_launch_x_to_digits(ctx, x_dev, T, d, type, xd));
+        const pg_gemv_batch bg = {(int)P, table(0), dtable(1), topk_idx, (int)top_k};
+        PG_TRY(pg_launch_gguf_gemv(ctx, type, ffn, d, nullptr, nullptr, bg, xd, g));
+        const pg_gemv_batch bu = {(int)P, table(2), dtable(3), topk_idx, (int)top_k};
+        PG_TRY(pg_launch_gguf_gemv(ctx, type, ffn, d, nullptr, nullptr, bu, xd, u));
+    } else {
+        const pg_mmdigits xd = pg_mmdigits_carve(xd_base, T, d);
+        PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, T, d, type, xd));
+        const pg_mm_group gg = {(int)E, table(0), dtable(1), lists, counts, (int)T, tiles, (int)T, (int)top_k, 0, 0, 1};
+        PG_TRY(pg_launch_gguf_mm(ctx, type, ffn, d, nullptr, nullptr, gg, P, xd, g, part));
+        const pg_mm_group gu = {(int)E, table(2), dtable(3), lists, counts, (int)T, tiles, (int)T, (int)top_k, 0, 0, 1};
+        PG_TRY(pg_launch_gguf_mm(ctx, type, ffn, d, nullptr, nullptr, gu, P, xd, u, part));
+    }
     PG_TRY(pg_launch(ctx, "moe_act_mul", act_mul_kernel, dim3(grid_for(P * ffn, 256)), dim3(256), 0, g, u, P * ffn,
                      act, h));
-    PG_TRY(pg_launch_x_to_mm_digits(ctx, h, P, ffn, type, hd));
-    const pg_mm_group gd = {(int)E, table(4), dtable(5), lists, counts, (int)T, tiles, (int)T, 1, 0, 0, 1};
-    PG_TRY(pg_launch_gguf_mm(ctx, type, d, ffn, nullptr, nullptr, gd, P, hd, yb, part));
+    if (down_stream) {
+        const pg_xdigits hd = pg_xdigits_carve(hd_base, P, ffn);
+        PG_TRY(pg_launch_x_to_digits(ctx, h, P, ffn, type, hd));
+        const pg_gemv_batch bd = {(int)P, table(4), dtable(5), topk_idx, 1};
+        PG_TRY(pg_launch_gguf_gemv(ctx, type, d, ffn, nullptr, nullptr, bd, hd, yb));
+    } else {
+        const pg_mmdigits hd = pg_mmdigits_carve(hd_base, P, ffn);
+        PG_TRY(pg_launch_x_to_mm_digits(ctx, h, P, ffn, type, hd));
+        const pg_mm_group gd = {(int)E, table(4), dtable(5), lists, counts, (int)T, tiles, (int)T, 1, 0, 0, 1};
+        PG_TRY(pg_launch_gguf_mm(ctx, type, d, ffn, nullptr, nullptr, gd, P, hd, yb, part));
+    }
     return pg_launch(ctx, "moe_combine", combine_kernel, dim3(grid_for(T * d, 256)), dim3(256), 0, yb, topk_p, (int)T,
                      (int)d, (int)top_k, out_dev);
 }

@@ -596,8 +596,8 @@ PG_API size_t pg_fixed_scratch_bytes(void) { return PG_FIXED_SCRATCH_BYTES; }
 // src/models/llama/decoder.rs:49-67) and slices the result; per-column weight scales and per-row
 // activation scales make every output column independent of its neighbours, so the separate
 // outputs here are bit for bit those of the single products.  The rows are quantised ONCE and,
-// for more than 64 rows, the products share one launch (the weights' column panels side by side
-// in one tile space).
+// for more than 256 rows, the narrow products share one launch (the weights' column panels side
+// by side in one tile space).
 PG_API pg_status pg_matmul_quantized_multi_dev(pg_ctx *ctx, const float *a_dev, size_t m, size_t k,
                                                const pg_qtensor *const *w, size_t count, float *const *out_dev) {
     PG_TRY(pg_use(ctx));
@@ -623,7 +623,23 @@ PG_API pg_status pg_matmul_quantized_multi_dev(pg_ctx *ctx, const float *a_dev, 
     int8_t *a_i8 = static_cast<int8_t *>(ws);
     float *a_scales = reinterpret_cast<float *>(a_i8 + a_bytes);
     PG_TRY(pg_launch_quantize_activations(ctx, a_dev, m, k, a_i8, k_pad, a_scales));
-    return pg_launch_gemm_w8a8_group(ctx, a_i8, k_pad, a_scales, w, out_dev, (int)count, m);
+    // Weights that fill the chip with 256x256 tiles on their own run on their own (measured: gate and up
+    // as two launches 2 x 112 us, as one launch of 896 tiles 242 us: the rounds that leave CUs idle run
+    // faster); the narrow ones (q, k, v) share one launch, where k and v alone would leave most CUs idle.
+    const pg_qtensor *small_w[PG_GEMM_MAX_GROUP];
+    float *small_out[PG_GEMM_MAX_GROUP];
+    int n_small = 0;
+    for (size_t i = 0; i < count; ++i) {
+        const size_t t256 = ((m + 255) / 256) * ((w[i]->cols + 255) / 256);
+        if (t256 >= (size_t)ctx->num_cu) {
+            PG_TRY(pg_launch_gemm_w8a8(ctx, a_i8, k_pad, a_scales, w[i], m, out_dev[i], nullptr));
+        } else {
+            small_w[n_small] = w[i];
+            small_out[n_small++] = out_dev[i];
+        }
+    }
+    if (n_small) PG_TRY(pg_launch_gemm_w8a8_group(ctx, a_i8, k_pad, a_scales, small_w, small_out, n_small, m));
+    return PG_OK;
 }
 
 // Which tile the W8A8 matrix-core product last ran with on this context, and an override of the

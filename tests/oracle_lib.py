@@ -24,6 +24,12 @@ lib.orc_rng_next_u64.restype = C.c_uint64
 lib.orc_rng_next_u64.argtypes = [_vp]
 lib.orc_rng_seed.argtypes = [_vp, C.c_uint64]
 lib.orc_rng_normal.argtypes = [C.c_uint64, _sz, C.c_float, C.c_float, _vp]
+lib.orc_philox_4x32_10.argtypes = [_vp, _vp, _vp]
+lib.orc_philox_4x32_10.restype = None
+lib.orc_random_seed.argtypes = [_vp, C.c_uint64]
+lib.orc_random_seed.restype = None
+lib.orc_random_normal.argtypes = [_vp, _sz, C.c_float, C.c_float, _vp]
+lib.orc_random_normal.restype = None
 for _n in ("orc_quantize_weights", "orc_quantize_activations", "orc_dequantize", "orc_gemm_i8",
            "orc_matmul_f32", "orc_softmax_rows", "orc_silu", "orc_gelu_tanh", "orc_swiglu_llama"):
     getattr(lib, _n).restype = None
@@ -159,6 +165,31 @@ def moe_ffn(x, T, d, ffn, E, top_k, logits, gate, up, down, ggml_type, act):
                          _p(out), _p(idx), _p(prob))
     assert rc == 0, rc
     return out.reshape(T, d), idx.reshape(T, top_k), prob.reshape(T, top_k)
+
+
+def philox_4x32_10(counter, key):
+    """orc_philox_4x32_10 on one (counter[4], key[2]); returns the four u32 outputs."""
+    c = (C.c_uint32 * 4)(*counter)
+    k = (C.c_uint32 * 2)(*key)
+    o = (C.c_uint32 * 4)()
+    lib.orc_philox_4x32_10(c, k, o)
+    return list(o)
+
+
+class Random:
+    """The oracle's restatement of random::seed / random::normal (both generators)."""
+
+    def __init__(self, seed):
+        self._st = (C.c_uint64 * 5)()
+        lib.orc_random_seed(self._st, C.c_uint64(seed))
+
+    def normal(self, n, mean=0.0, std=1.0):
+        out = np.empty(n, np.float32)
+        lib.orc_random_normal(self._st, _sz(n), C.c_float(mean), C.c_float(std), _p(out))
+        return out
+
+    def next_u64(self):
+        return lib.orc_rng_next_u64(self._st)
 
 
 def rng_normal(seed, n, mean=0.0, std=1.0):

@@ -126,6 +126,34 @@ def test_moe_many_tokens_per_expert(ctx, orc):
         H.assert_close_rel(got[t], want[t], MOE_RTOL, f"token {t}")
 
 
+@pytest.mark.parametrize("typ", [8, 2])
+@pytest.mark.parametrize("d,ffn", [(256, 64), (256, 32), (64, 32), (32, 96), (128, 128), (256, 480), (96, 512)])
+def test_moe_products_over_one_or_two_blocks(ctx, orc, typ, d, ffn):
+    """Narrow experts, down to products whose K spans one block.  The matrix-core route carries
+    16-bit fixed-point activations per block; its error in g and u (4e-5 of their rms) is
+    multiplied by the partner factor in h = silu(g) * u, and a down product over only 32 - 128
+    terms does not average an outlier's error away.  Seed 937967 is such a case (33 tokens, d 256,
+    ffn 64, two experts both chosen; expert 1's gate rows come from the very stream the activation
+    rows come from, so one g per token sits near 0.05 |x|^2 = 13): it missed the 1e-3 bar by 40 %.
+    Narrow experts and short-K products therefore run the streaming kernel (18 / 22-bit
+    activations); that case and a sweep of seeds with x20 outlier channels hold the contract."""
+    from peregrine_amd import gguf, moe
+    E, top_k, T = 2, 2, 33
+    for seed in (937967, 11, 12, 13, 14, 15):
+        say(f"moe narrow experts typ={typ} d={d} ffn={ffn} seed={seed}")
+        raws = build(orc, seed, d, ffn, E, typ)
+        x = orc.rng_normal(seed + 1, T * d).reshape(T, d)
+        if seed != 937967:
+            x[:, :: max(1, d // 3)] *= 20   # outlier channels -> outliers in h as well
+        logits = orc.rng_normal(seed + 2, T * E).reshape(T, E)
+        mk = lambda rs, n_out, k_in: [gguf.GgufWeight(r, typ, n_out, k_in, ctx) for r in rs]
+        ex = moe.MoEExperts(mk(raws[0], ffn, d), mk(raws[1], ffn, d), mk(raws[2], d, ffn), top_k, moe.SILU, ctx)
+        got = ex.forward(x.reshape(-1), logits)
+        want, idx, prob = orc.moe_ffn(x.reshape(-1), T, d, ffn, E, top_k, logits, raws[0], raws[1], raws[2], typ, 0)
+        for t in range(T):
+            H.assert_close_rel(got[t], want[t], 1e-3, f"seed {seed} token {t}")
+
+
 def test_moe_argument_errors(ctx, orc):
     from peregrine_amd import gguf, moe, _ffi
     d, ffn = 64, 96
