@@ -52,19 +52,19 @@ SETTLE_S = 0.2  # untimed run of the headline step before its warm-up, seconds
 
 
 def load_traffic():
-    """profiles/hbm_traffic.json: per-kernel HBM bytes per launch derived from rocprofv3 --pmc
-    FETCH_SIZE / WRITE_SIZE runs of this benchmark, scaled by a plain copy of known size
-    (the file names the commands), and the launch sizes (work-items) those averages were taken
-    over.  Absent file -> traffic is reported as null."""
+    """profiles/hbm_traffic.json: HBM bytes per launch, per kernel family and launch size
+    (work-items), derived from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this benchmark and
+    scaled by a plain copy of known size (the file names the commands).  Absent file -> traffic is
+    reported as null."""
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-            d = json.load(f)
-            return d.get("bytes_per_launch", {}), d.get("launch_work_items", {})
+            return json.load(f).get("bytes_per_launch_by_size", {})
     except (OSError, ValueError):
-        return {}, {}
+        return {}
 
 
-TRAFFIC, TRAFFIC_GRIDS = load_traffic()
+TRAFFIC = load_traffic()
+LAUNCHES_SEEN = {}  # kernel family -> launch sizes (work-items) of this run, reported as `launch_work_items`
 
 
 def gemv_bytes(k, n):
@@ -168,14 +168,16 @@ class Bench:
 
     @staticmethod
     def traffic_for(kernel, grids):
-        """HBM bytes per launch from the committed rocprofv3 --pmc measurement -- but only while the
-        launches this run made of that kernel have the sizes the counters were averaged over;
-        otherwise None (the kernel or its dispatch changed since: the summary is stale)."""
-        if kernel not in TRAFFIC:
+        """HBM bytes per launch of a kernel family: the committed rocprofv3 --pmc figures per launch
+        size, weighted by the launches this run made of each size -- but only while those sizes are
+        exactly the ones the counters were taken on; otherwise None (the kernel or its dispatch
+        changed since: the summary is stale)."""
+        got = grids.get(kernel, {})
+        LAUNCHES_SEEN[kernel] = sorted(got)
+        have = TRAFFIC.get(kernel)
+        if not have or sorted(int(g) for g in have) != sorted(got):
             return None
-        want = sorted(int(g) for g in TRAFFIC_GRIDS.get(kernel, []))
-        got = sorted(grids.get(kernel, {}))
-        return TRAFFIC[kernel] if want and want == got else None
+        return int(sum(n * have[str(g)] for g, n in got.items()) / sum(got.values()))
 
     def ceilings(self):
         """What the part delivers on three probes, measured now (fractions stay against the published peaks)."""
@@ -274,7 +276,7 @@ def main():
                  "peak": PEAK_HBM_GBS, "unit": "GB/s", "avg_launch_ms": round(q_avg_ms, 4),
                  "traffic": B.traffic_for("quantize_rows", grids)}
     act_quant["frac"] = round(act_quant["achieved"] / PEAK_HBM_GBS, 4)
-    ceil = B.ceilings()
+    ceil = None if args.calibrate_copy else B.ceilings()  # (counter runs measure traffic only)
 
     # Per product shape: this library's GEMM kernel beside the vendor library's int8 GEMM
     # (torch._int_mm = hipBLASLt; same operand layouts, i32 output without the rescale) on
@@ -291,7 +293,7 @@ def main():
             torch.cuda.synchronize()
 
     vendor = []
-    for name, k, n in (("q/o_proj", 4096, 4096), ("gate/up_proj", 4096, 14336), ("down_proj", 14336, 4096)):
+    for name, k, n in (() if args.calibrate_copy else (("q/o_proj", 4096, 4096), ("gate/up_proj", 4096, 14336), ("down_proj", 14336, 4096))):
         wname = {"q/o_proj": "q_proj", "gate/up_proj": "gate_proj", "down_proj": "down_proj"}[name]
 
         def one_product():
@@ -380,6 +382,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    line["launch_work_items"] = LAUNCHES_SEEN
     line["cpu_baseline"] = cpu_baseline(B.orc, cpu_w, cpu_a) if B.cpu else None
     print(json.dumps(line), flush=True)
     B.ctx.close()
@@ -398,27 +401,31 @@ def section_decode_and_linear(B, line):
     x_d, x_f = B.make_acts(1, 4096, 1240), B.make_acts(1, 14336, 1242)
     y_f, y_u, y_d = torch.empty(1, 14336, device=dev), torch.empty(1, 14336, device=dev), torch.empty(1, 4096, device=dev)
 
-    def decode_step():
-        g, u, d = dec_w[B.i % LAYERS_ROT]
+    VP2 = C.c_void_p * 2
+    gu_tabs = [VP2(g.value, u.value) for g, u, _ in dec_w]
+    gu_out = VP2(y_f.data_ptr(), y_u.data_ptr())
+
+    def decode_step():  # gate|up as the fused product of models::llama (one launch), then down
+        r = B.i % LAYERS_ROT
         B.i += 1
-        check(lib.pg_matmul_quantized_dev(B.h, ptr(x_d), 1, 4096, g, ptr(y_f), None))
-        check(lib.pg_matmul_quantized_dev(B.h, ptr(x_d), 1, 4096, u, ptr(y_u), None))
-        check(lib.pg_matmul_quantized_dev(B.h, ptr(x_f), 1, 14336, d, ptr(y_d), None))
+        check(lib.pg_matmul_quantized_multi_dev(B.h, ptr(x_d), 1, 4096, gu_tabs[r], 2, gu_out))
+        check(lib.pg_matmul_quantized_dev(B.h, ptr(x_f), 1, 14336, dec_w[r][2], ptr(y_d), None))
 
     dec_bytes = 2 * gemv_bytes(4096, 14336) + gemv_bytes(14336, 4096)
     t_dec = B.timed(decode_step, B.dsteps, max(args.warmup, 8))
     prof, grids = B.profiled(decode_step, B.dsteps)
     gemv_avg_ms, v_n = prof["gemv_w8a8"]
-    gemv_gbs = (dec_bytes / 3) / (gemv_avg_ms * 1e-3) / 1e9
-    decode = {"workload": "cfg2: M=1 int8 GEMV, x[4096]->gate,up[14336], x[14336]->down[4096]; "
+    gemv_lps = v_n / B.dsteps  # launches per step: gate|up together, down
+    gemv_gbs = (dec_bytes / gemv_lps) / (gemv_avg_ms * 1e-3) / 1e9
+    decode = {"workload": "cfg2: M=1 int8 GEMV, x[4096]->gate|up[14336+14336] (one launch), x[14336]->down[4096]; "
                           f"{LAYERS_ROT} layers of weights rotated ({LAYERS_ROT * 3 * 58.7:.0f} MB, HBM-resident reads)",
               "value": round(dec_bytes / (t_dec["ms_per_step"] * 1e-3) / 1e9, 1), "unit": "GB/s",
               "frac_of_hbm_peak": round(dec_bytes / (t_dec["ms_per_step"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
               **B.stats(t_dec), "steps": B.dsteps, "bytes_per_step": dec_bytes,
               "roofline": {"kernel": "gemv_w8a8_m1_f32x_kernel (quantises its activation row, then streams the weights)", "bound": "hbm",
                            "achieved": round(gemv_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gemv_gbs / PEAK_HBM_GBS, 4),
-                           "traffic": B.traffic_for("gemv_w8a8", grids), "bytes_per_launch": dec_bytes // 3,
-                           "avg_launch_ms": round(gemv_avg_ms, 5)}}
+                           "traffic": B.traffic_for("gemv_w8a8", grids), "bytes_per_launch": int(dec_bytes / gemv_lps),
+                           "launches_per_step": gemv_lps, "avg_launch_ms": round(gemv_avg_ms, 5)}}
     if B.cpu:
         decode["cpu_baseline"] = cpu_decode(B.orc, kept, x_d.cpu().numpy(), x_f.cpu().numpy(), dec_bytes)
     line["decode_gemv"] = decode

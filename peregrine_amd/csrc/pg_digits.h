@@ -15,17 +15,27 @@
 //                  plane 2j+h holds a_j of elements 16h..16h+15.
 // With `xsum` (Q4_1, whose blocks carry an offset m: sum_k (q d + m) x = d sum q x + m sum x) the
 // block's sum of fixed-point values, sum_k X[k], is stored too: xsum[row][b] (exact: < 2^23).
+// A DPP move within groups of 8 lanes: 0xB1 = quad_perm [1,0,3,2], 0x4E = quad_perm [2,3,0,1],
+// 0x141 = row_half_mirror (lane i of the 8 takes lane 7 - i).
+template <int CTRL>
+__device__ __forceinline__ int pg_dpp8(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+
 template <bool NIB>
 __device__ __forceinline__ void pg_emit_digits(const float (&f)[4], size_t row, int b, int sub, int nb,
                                                int8_t *__restrict__ digits, float *__restrict__ xs,
                                                float *__restrict__ xsum = nullptr) {
     float amax = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3])));
     int bad = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]);
-#pragma unroll
-    for (int off = 1; off < 8; off <<= 1) {
-        amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-        bad |= __shfl_xor(bad, off, 64);
-    }
+    // over the 8 lanes of the group with DPP moves (no LDS round trips): neighbour, other pair, then the
+    // mirror image within the 8 lanes, which pairs the two quads (max, or and + are symmetric)
+    amax = fmaxf(amax, __builtin_bit_cast(float, pg_dpp8<0xB1>(__builtin_bit_cast(int, amax))));
+    bad |= pg_dpp8<0xB1>(bad);
+    amax = fmaxf(amax, __builtin_bit_cast(float, pg_dpp8<0x4E>(__builtin_bit_cast(int, amax))));
+    bad |= pg_dpp8<0x4E>(bad);
+    amax = fmaxf(amax, __builtin_bit_cast(float, pg_dpp8<0x141>(__builtin_bit_cast(int, amax))));
+    bad |= pg_dpp8<0x141>(bad);
     constexpr int BITS = NIB ? 18 : 22;
     float s = 1.0f, inv = 1.0f;
     if (bad || !(amax <= 3.4028234663852886e38f)) {
@@ -47,38 +57,37 @@ __device__ __forceinline__ void pg_emit_digits(const float (&f)[4], size_t row, 
     }
     if (xsum) {  // the same for all lanes
         int part = X[0] + X[1] + X[2] + X[3];
-#pragma unroll
-        for (int off = 1; off < 8; off <<= 1) part += __shfl_xor(part, off, 64);
+        part += pg_dpp8<0xB1>(part);
+        part += pg_dpp8<0x4E>(part);
+        part += pg_dpp8<0x141>(part);
         if (sub == 0) xsum[row * (size_t)nb + b] = (float)part;
     }
     int8_t *drow = digits + row * (size_t)nb * 96;
     if (NIB) {
+        // Balanced base-16 digits n_j in [-8, 7] without a carry loop: X + 0x88888 = sum_j 16^j (n_j + 8),
+        // and n_j + 8 with its top bit flipped is n_j in 4-bit two's complement, so nibble j of
+        // (X + 0x88888) ^ 0x88888 is digit j as stored (|X| < 2^18 lies well inside the range).
+        unsigned W[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) W[e] = (unsigned)(X[e] + 0x88888) ^ 0x88888u;
 #pragma unroll
         for (int j = 0; j < 5; ++j) {
-            unsigned packed = 0;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int n = ((X[e] + 8) & 15) - 8;  // signed 4-bit digit
-                X[e] = (X[e] - n) >> 4;
-                packed |= (unsigned)(n & 15) << (4 * e);
-            }
+            const unsigned packed = __builtin_amdgcn_ubfe(W[0], 4 * j, 4) | (__builtin_amdgcn_ubfe(W[1], 4 * j, 4) << 4) |
+                                    (__builtin_amdgcn_ubfe(W[2], 4 * j, 4) << 8) | (__builtin_amdgcn_ubfe(W[3], 4 * j, 4) << 12);
             // this thread's elements 4*sub .. 4*sub+3 are nibbles 4*sub.. of the block: bytes 2*sub, 2*sub+1
             *reinterpret_cast<uint16_t *>(drow + ((size_t)j * nb + b) * 16 + 2 * sub) = (uint16_t)packed;
         }
     } else {
-        int a[3][4];
+        // The same in base 256: byte k of (X + 0x808080) ^ 0x808080 is the signed byte digit of weight 256^k.
+        unsigned W[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            a[2][e] = ((X[e] + 128) & 255) - 128;
-            const int X1 = (X[e] - a[2][e]) >> 8;
-            a[1][e] = ((X1 + 128) & 255) - 128;
-            a[0][e] = (X1 - a[1][e]) >> 8;
-        }
+        for (int e = 0; e < 4; ++e) W[e] = (unsigned)(X[e] + 0x808080) ^ 0x808080u;
         const int e0 = sub * 4, h = e0 >> 4;
 #pragma unroll
-        for (int j = 0; j < 3; ++j) {
-            const unsigned packed = (unsigned)(a[j][0] & 255) | ((unsigned)(a[j][1] & 255) << 8) |
-                                    ((unsigned)(a[j][2] & 255) << 16) | ((unsigned)(a[j][3] & 255) << 24);
+        for (int j = 0; j < 3; ++j) {  // plane pair j holds the digit of weight 256^(2-j)
+            const int k = 2 - j;
+            const unsigned packed = ((W[0] >> (8 * k)) & 255u) | (((W[1] >> (8 * k)) & 255u) << 8) |
+                                    (((W[2] >> (8 * k)) & 255u) << 16) | (((W[3] >> (8 * k)) & 255u) << 24);
             *reinterpret_cast<unsigned *>(drow + ((size_t)(2 * j + h) * nb + b) * 16 + (e0 & 15)) = packed;
         }
     }

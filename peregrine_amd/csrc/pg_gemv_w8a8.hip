@@ -7,6 +7,7 @@
 //
 // Integer sums are exact, so the lane/chunk order does not matter; the f32
 // epilogue keeps the reference's multiplication order (src/quant.rs:163).
+#include <limits.h>
 #include "pg_internal.h"
 #include "pg_quant_dev.h"
 
@@ -130,15 +131,32 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_kernel(
 // (same scale, same reciprocal, same rounding: bit-identical integers), and every lane takes its
 // chunks from there.  One launch per product instead of two: the separate one-row quantisation
 // kernel costs about 4 us, as much as a third of the product itself.  k % 4 == 0.
+// Up to PG_GEMM_MAX_GROUP weights of equal K against the same row in one launch (the reference's
+// fused gate|up and q|k|v products at one token): weight g owns the workgroups wg0[g] .. wg0[g+1]-1
+// (unused slots hold INT_MAX).  One weight is a group of one.
+struct gemv_wgroup {
+    const int8_t *w[PG_GEMM_MAX_GROUP];
+    const float *ws[PG_GEMM_MAX_GROUP];
+    float *out[PG_GEMM_MAX_GROUP];
+    int n[PG_GEMM_MAX_GROUP];
+    int wg0[PG_GEMM_MAX_GROUP];
+};
+
 template <int NCH, int RPW>
 __global__ __launch_bounds__(256) void gemv_w8a8_m1_f32x_kernel(
-    const int8_t *__restrict__ w_t, int k_pad, const float *__restrict__ w_scales,
-    const float *__restrict__ x_f32, int k, int n, float *__restrict__ out, int32_t *__restrict__ acc_out) {
+    const gemv_wgroup grp, int k_pad, const float *__restrict__ x_f32, int k, int32_t *__restrict__ acc_out) {
     __shared__ int xq[NCH * 256];  // the quantised row, zero beyond k: NCH KiB >= k_pad bytes
     __shared__ float red[4];
+    int g = 0;
+#pragma unroll
+    for (int i = 1; i < PG_GEMM_MAX_GROUP; ++i) g = (int)blockIdx.x >= grp.wg0[i] ? i : g;
+    const int8_t *__restrict__ w_t = grp.w[g];
+    const float *__restrict__ w_scales = grp.ws[g];
+    float *__restrict__ out = grp.out[g];
+    const int n = grp.n[g];
     const int nchunk = k_pad >> 4;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int row0 = (blockIdx.x * 4 + wave) * RPW;
+    const int row0 = (((int)blockIdx.x - grp.wg0[g]) * 4 + wave) * RPW;
     auto load_row = [&](int row, v4i (&w)[NCH]) {
         const v4i *wp = reinterpret_cast<const v4i *>(w_t + (size_t)row * k_pad);
 #pragma unroll
@@ -147,9 +165,9 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_f32x_kernel(
             w[j] = __builtin_nontemporal_load(wp + (c < nchunk ? c : lane));
         }
     };
-    v4i w[NCH];
-    load_row(row0, w);  // in flight while the activations are prepared
-
+    // Loads return in issue order: the activation row (from L2) is requested first, so that its
+    // quantisation can start as soon as it is there; every weight row of this wavefront (from HBM)
+    // right behind it, all in flight together.
     const int nvec = k >> 2;
     const float4 *x4 = reinterpret_cast<const float4 *>(x_f32);
     float4 v[NCH];
@@ -159,13 +177,17 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_f32x_kernel(
         const int idx = threadIdx.x + 256 * i;
         v[i] = x4[idx < nvec ? idx : nvec - 1];
     }
+    v4i w[RPW][NCH];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) load_row(row0 + r, w[r]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
         const int idx = threadIdx.x + 256 * i;
         const float m4 = fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)), fmaxf(fabsf(v[i].z), fabsf(v[i].w)));
         amax = fmaxf(amax, idx < nvec ? m4 : 0.0f);
     }
-    amax = pg_block_max_256(amax, red);
+    amax = pg_block_max_256_keep_loads(amax, red);
     const float a_scale = (amax == 0.0f) ? 1.0f : amax / 127.0f;
     const float inv_scale = 1.0f / a_scale;
 #pragma unroll
@@ -177,17 +199,17 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_f32x_kernel(
         const int b3 = pg_quant_to_i8(v[i].w * inv_scale) & 0xFF;
         xq[idx] = idx < nvec ? (b0 | (b1 << 8) | (b2 << 16) | (b3 << 24)) : 0;
     }
-    __syncthreads();
+    // (not __syncthreads(): that would also wait for every weight row in flight)
+    asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier" ::: "memory");
     v4i x[NCH];
 #pragma unroll
     for (int j = 0; j < NCH; ++j) x[j] = reinterpret_cast<const v4i *>(xq)[lane + 64 * j];
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
         const int row = row0 + r;  // < n_pad by construction of the grid
-        if (r > 0) load_row(row, w);
         int acc = 0;
 #pragma unroll
-        for (int j = 0; j < NCH; ++j) acc = dot16(w[j], x[j], acc);  // x is zero beyond k
+        for (int j = 0; j < NCH; ++j) acc = dot16(w[r][j], x[j], acc);  // x is zero beyond k
         acc = wave_sum_i32(acc);
         if (lane == 0 && row < n) {
             if (out) out[row] = (float)acc * a_scale * w_scales[row];
@@ -197,17 +219,31 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_f32x_kernel(
 }
 
 template <int NCH, int RPW>
-pg_status launch_m1_f32x(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *w, float *out, int32_t *acc) {
-    const unsigned grid = (unsigned)(w->n_pad / (4 * RPW));
-    PG_TRY(pg_launch(ctx, "gemv_w8a8", gemv_w8a8_m1_f32x_kernel<NCH, RPW>, dim3(grid), dim3(256), 0, w->w_t,
-                     (int)w->k_pad, w->scales, x_f32, (int)k, (int)w->cols, out, acc));
+pg_status launch_m1_f32x(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *const *w, float *const *out, int count,
+                         int32_t *acc) {
+    gemv_wgroup grp;
+    int wgs = 0;
+    for (int i = 0; i < PG_GEMM_MAX_GROUP; ++i) {
+        const bool used = i < count;
+        grp.w[i] = used ? w[i]->w_t : nullptr;
+        grp.ws[i] = used ? w[i]->scales : nullptr;
+        grp.out[i] = used && out ? out[i] : nullptr;
+        grp.n[i] = used ? (int)w[i]->cols : 0;
+        grp.wg0[i] = used ? wgs : INT_MAX;
+        if (used) wgs += (int)(w[i]->n_pad / (4 * RPW));
+    }
+    PG_TRY(pg_launch(ctx, "gemv_w8a8", gemv_w8a8_m1_f32x_kernel<NCH, RPW>, dim3((unsigned)wgs), dim3(256), 0, grp,
+                     (int)w[0]->k_pad, x_f32, (int)k, acc));
     return pg_launch_check("gemv_w8a8_m1_f32x");
 }
 
 template <int NCH>
-pg_status launch_m1_f32x_rows(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *w, float *out, int32_t *acc) {
-    if (w->n_pad / 2 >= (size_t)ctx->num_cu * 8) return launch_m1_f32x<NCH, 2>(ctx, x_f32, k, w, out, acc);
-    return launch_m1_f32x<NCH, 1>(ctx, x_f32, k, w, out, acc);
+pg_status launch_m1_f32x_rows(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *const *w, float *const *out, int count,
+                              int32_t *acc) {
+    size_t rows = 0;
+    for (int i = 0; i < count; ++i) rows += w[i]->n_pad;
+    if (rows / 2 >= (size_t)ctx->num_cu * 8) return launch_m1_f32x<NCH, 2>(ctx, x_f32, k, w, out, count, acc);
+    return launch_m1_f32x<NCH, 1>(ctx, x_f32, k, w, out, count, acc);
 }
 
 template <int NCH, int RPW>
@@ -258,13 +294,21 @@ bool pg_gemv_w8a8_takes_f32_row(const pg_qtensor *w, size_t m, size_t k, const f
     return m == 1 && w->k_pad <= 16384 && k % 4 == 0 && k > 0 && (uintptr_t)x_f32 % 16 == 0;  // 128-bit loads of the row
 }
 
+pg_status pg_launch_gemv_w8a8_f32_row_group(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *const *w,
+                                            float *const *out, int count, int32_t *acc) {
+    if (count < 1 || count > PG_GEMM_MAX_GROUP) return pg_fail(PG_EINVAL, "gemv_w8a8: %d weights in one launch (1 .. %d)", count, PG_GEMM_MAX_GROUP);
+    for (int i = 1; i < count; ++i)
+        if (w[i]->k_pad != w[0]->k_pad) return pg_fail(PG_EINVAL, "gemv_w8a8: the weights of one launch differ in K");
+    const size_t nch = (w[0]->k_pad / 16 + 63) / 64;
+    if (nch <= 4) return launch_m1_f32x_rows<4>(ctx, x_f32, k, w, out, count, acc);
+    if (nch <= 8) return launch_m1_f32x_rows<8>(ctx, x_f32, k, w, out, count, acc);
+    if (nch <= 14) return launch_m1_f32x_rows<14>(ctx, x_f32, k, w, out, count, acc);
+    return launch_m1_f32x_rows<16>(ctx, x_f32, k, w, out, count, acc);
+}
+
 pg_status pg_launch_gemv_w8a8_f32_row(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *w, float *out,
                                       int32_t *acc) {
-    const size_t nch = (w->k_pad / 16 + 63) / 64;
-    if (nch <= 4) return launch_m1_f32x_rows<4>(ctx, x_f32, k, w, out, acc);
-    if (nch <= 8) return launch_m1_f32x_rows<8>(ctx, x_f32, k, w, out, acc);
-    if (nch <= 14) return launch_m1_f32x_rows<14>(ctx, x_f32, k, w, out, acc);
-    return launch_m1_f32x_rows<16>(ctx, x_f32, k, w, out, acc);
+    return pg_launch_gemv_w8a8_f32_row_group(ctx, x_f32, k, &w, &out, 1, acc);
 }
 
 pg_status pg_launch_gemv_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,

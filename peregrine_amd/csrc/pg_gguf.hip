@@ -212,16 +212,24 @@ struct RowLoads {
 // MXFP4 blocks, whose range f16 cannot hold) instead of f16.
 // Q41 (with QT = 4): every block also has an offset m; its term (8 d + m) * sum_k x_k uses the
 // block sums written with the digits.
-template <int QT, int BPL, int RW, int R, bool BF = false, bool Q41 = false>
-__global__ __launch_bounds__(64) void gguf_gemv_kernel(
+// XF32 (one item, no tables): the activation row arrives in f32 (x_f32) and the workgroup -- NW
+// wavefronts, each with its own RW rows -- rewrites it as digits into LDS itself, after every
+// wavefront has requested its first weight rows: the product is one launch instead of two, and
+// the digit arithmetic (18 vector operations per element, shared by NW wavefronts) runs while
+// those first loads are in flight.
+template <int QT, int BPL, int RW, int R, bool BF = false, bool Q41 = false, bool XF32 = false, int NW = 1>
+__global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
     const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0, pg_gemv_batch batch,
     int n_out, int nb, const int8_t *__restrict__ digits_base, const float *__restrict__ xs_base,
     float *__restrict__ y_base, const float *__restrict__ residual_base, const uint16_t *__restrict__ m0,
-    const float *__restrict__ xsum_base) {
+    const float *__restrict__ xsum_base, const float *__restrict__ x_f32) {
     constexpr int SEG = 64 * BPL;  // blocks per K segment
     constexpr int NG = RW / R;
     constexpr int NH = QT == 8 ? 2 : 1;
     constexpr int NP = QT == 8 ? 6 : 5;  // digit planes
+    static_assert(!XF32 || !Q41, "the one-launch form has no block sums");
+    static_assert(XF32 || NW == 1, "several wavefronts per workgroup only where they share the digits");
+    extern __shared__ __attribute__((aligned(16))) char lds_digits[];  // XF32: [6 planes][nb][16 B], then nb scales
     const int item = blockIdx.y;
     const uint8_t *qs_any = qs0;
     const uint16_t *d_any = d0;
@@ -238,8 +246,10 @@ __global__ __launch_bounds__(64) void gguf_gemv_kernel(
     const gv4i_ptr msc = (gv4i_ptr)(uintptr_t)m0;
     const float *__restrict__ xsum = Q41 ? xsum_base + xrow * (size_t)nb : nullptr;
     float *__restrict__ y = y_base + (size_t)item * n_out;
-    const int lane = threadIdx.x;
-    const int row0 = blockIdx.x * RW;
+    const int lane = threadIdx.x & 63;
+    const int row0 = (blockIdx.x * NW + (threadIdx.x >> 6)) * RW;
+    int8_t *const ldig = reinterpret_cast<int8_t *>(lds_digits);
+    float *const lxs = reinterpret_cast<float *>(lds_digits + (size_t)nb * 96);
     float acc[NG][R];
 #pragma unroll
     for (int g = 0; g < NG; ++g)
@@ -272,20 +282,73 @@ __global__ __launch_bounds__(64) void gguf_gemv_kernel(
         v4i dtile[BPL];  // f16 scales of this lane's blocks for the 8 rows of the tile
         v4i mtile[BPL];  // Q4_1: their f16 offsets
         float sxs[BPL];  // Q4_1: scale * block sum of the activation block
-#pragma unroll
-        for (int p = 0; p < BPL; ++p) {
-#pragma unroll
-            for (int j = 0; j < NP; ++j) xd[p][j] = digits[(size_t)j * nb + blk[p]];
-            sb[p] = xs[blk[p]];
-            dtile[p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
-            if constexpr (Q41) {
-                mtile[p] = msc[(size_t)(row0 >> 3) * nb + blk[p]];
-                sxs[p] = xsum[blk[p]];
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
         RowLoads<QT, BPL, R> L[2];
-        load_rows(L[0], 0);
+        if constexpr (XF32) {
+            // weights first: they come from HBM and take longest (a wavefront whose rows all lie past
+            // n_out -- the last workgroup's spare ones -- only helps with the digits)
+            // Loads return in issue order: the row (a few KiB, from L2) is requested first so that the digit
+            // arithmetic can start as soon as it is there, the weight rows (from HBM) right behind it so
+            // that they fly meanwhile.  (A wavefront whose rows all lie past n_out -- the last workgroup's
+            // spare ones -- only helps with the digits.)
+            const bool live = row0 < n_out;
+            const int sub = threadIdx.x & 7, bfirst = (int)threadIdx.x >> 3;
+            float4 xv[4];
+            if (seg0 == 0) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int b = bfirst + u * 8 * NW;
+                    xv[u] = reinterpret_cast<const float4 *>(x_f32)[(size_t)(b < nb ? b : 0) * 8 + sub];
+                }
+            }
+            if (live) {
+#pragma unroll
+                for (int p = 0; p < BPL; ++p) dtile[p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+                load_rows(L[0], 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (seg0 == 0) {  // the row as digits, once per workgroup: 8 threads per block of 32, 4 elements each
+                for (int b0 = bfirst; b0 < nb; b0 += 32 * NW) {  // four blocks per thread and round
+                    if (b0 != bfirst) {
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int b = b0 + u * 8 * NW;
+                            xv[u] = reinterpret_cast<const float4 *>(x_f32)[(size_t)(b < nb ? b : 0) * 8 + sub];
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int b = b0 + u * 8 * NW;
+                        if (b < nb) {  // whole 8-thread groups together
+                            const float f[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+                            pg_emit_digits<QT == 4>(f, 0, b, sub, nb, ldig, lxs);
+                        }
+                    }
+                }
+                // (not __syncthreads(): that would also wait for every weight load in flight)
+                asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier" ::: "memory");
+            }
+            if (!live) return;  // after the workgroup's only barrier
+#pragma unroll
+            for (int p = 0; p < BPL; ++p) {
+#pragma unroll
+                for (int j = 0; j < NP; ++j) xd[p][j] = *reinterpret_cast<const v4i *>(ldig + ((size_t)j * nb + blk[p]) * 16);
+                sb[p] = lxs[blk[p]];
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < BPL; ++p) {
+#pragma unroll
+                for (int j = 0; j < NP; ++j) xd[p][j] = digits[(size_t)j * nb + blk[p]];
+                sb[p] = xs[blk[p]];
+                dtile[p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+                if constexpr (Q41) {
+                    mtile[p] = msc[(size_t)(row0 >> 3) * nb + blk[p]];
+                    sxs[p] = xsum[blk[p]];
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            load_rows(L[0], 0);
+        }
         __builtin_amdgcn_sched_barrier(0);  // every load is issued before any arithmetic
 #pragma unroll
         for (int p = 0; p < BPL; ++p) {
@@ -350,13 +413,54 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
         const dim3 grid(grid_for(n_out, RWW), (unsigned)batch.count);                              \
         PG_TRY(pg_launch(ctx, QT == 4 ? (Q41 ? "gguf_gemv_q4_1" : "gguf_gemv_q4_0") : (BF ? "gguf_gemv_mxfp4" : "gguf_gemv_q8_0"), \
                          gguf_gemv_kernel<QT, BPL, RWW, RR, BF, Q41>, grid, dim3(64), 0, qs, d, batch, \
-                         (int)n_out, nb, xd.digits, xd.xs, y, residual, m, (const float *)xd.xsum)); \
+                         (int)n_out, nb, xd.digits, xd.xs, y, residual, m, (const float *)xd.xsum, (const float *)nullptr)); \
     } while (0)
     if (n_out / 8 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(8, R8);
     else if (n_out / 4 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(4, (R8 < 4 ? R8 : 4));
     else PG_GGUF_GEMV_LAUNCH(2, 2);
 #undef PG_GGUF_GEMV_LAUNCH
     return PG_OK;
+}
+
+// One row still in f32: the one-launch form (four or eight wavefronts per workgroup share the digits).
+template <int QT, int BPL, bool BF, int NW>
+pg_status launch_gemv_f32x_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const float *x_f32,
+                               float *y) {
+    constexpr int NH = QT == 8 ? 2 : 1;
+    constexpr int R8 = BPL * NH <= 2 ? 8 : (BPL * NH <= 4 ? 4 : 2);
+    const int nb = (int)(k_in / 32);
+    const size_t lds = (size_t)nb * 96 + (size_t)nb * sizeof(float);
+    const pg_gemv_batch one = {1, nullptr, nullptr, nullptr, 1};
+    const size_t want = (size_t)ctx->num_cu * 6;
+    const char *name = QT == 4 ? "gguf_gemv_q4_0" : (BF ? "gguf_gemv_mxfp4" : "gguf_gemv_q8_0");
+#define PG_GGUF_GEMV_X_LAUNCH(RWW, RR)                                                                             \
+    do {                                                                                                           \
+        auto kern = gguf_gemv_kernel<QT, BPL, RWW, RR, BF, false, true, NW>;                                       \
+        PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                \
+        PG_TRY(pg_launch(ctx, name, kern, dim3(grid_for(n_out, RWW * NW)), dim3(64 * NW), lds, qs, d, one, (int)n_out, nb, \
+                         (const int8_t *)nullptr, (const float *)nullptr, y, (const float *)nullptr,               \
+                         (const uint16_t *)nullptr, (const float *)nullptr, x_f32));                               \
+    } while (0)
+    if (n_out / 8 >= want) PG_GGUF_GEMV_X_LAUNCH(8, R8);
+    else if (n_out / 4 >= want) PG_GGUF_GEMV_X_LAUNCH(4, (R8 < 4 ? R8 : 4));
+    else PG_GGUF_GEMV_X_LAUNCH(2, 2);
+#undef PG_GGUF_GEMV_X_LAUNCH
+    return PG_OK;
+}
+
+template <int QT, bool BF = false>
+pg_status launch_gemv_f32x(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const float *x_f32, float *y) {
+    size_t bpl = (k_in / 32 + 63) / 64;
+    if (bpl > 4) bpl = 4;
+    // Every workgroup makes the whole row's digits: the fewer, larger workgroups the less of that work
+    // in total -- eight wavefronts each where that still leaves a workgroup for a good part of the CUs.
+    const bool wide = n_out / 64 >= (size_t)ctx->num_cu / 6;
+    switch (bpl) {
+        case 1: return wide ? launch_gemv_f32x_bpl<QT, 1, BF, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 1, BF, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
+        case 2: return wide ? launch_gemv_f32x_bpl<QT, 2, BF, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 2, BF, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
+        case 3: return wide ? launch_gemv_f32x_bpl<QT, 3, BF, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 3, BF, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
+        default: return wide ? launch_gemv_f32x_bpl<QT, 4, BF, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 4, BF, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
+    }
 }
 
 template <int QT, bool BF = false, bool Q41 = false>
@@ -424,6 +528,22 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
     return launch_gemv<8>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, nullptr);
 }
 
+// y[row] = product over one activation row given in f32 (16-byte aligned): one launch, digits made inside.
+// Every workgroup repeats the digit arithmetic for the whole row, so the form pays where there are few
+// workgroups and the separate digit launch (2.4 us in a chain of launches) weighs most: Q4_0 with up to
+// 8192 weight rows (measured one launch against two: 4096 -> 4096 5.5 against 6.7 us, 14336 -> 4096 11.5
+// against 12.8 us; but 4096 -> 14336 10.9 against 10.3 us, and Q8_0 there 19.3 against 14.6 us).
+// k_in up to 32768 (the row's digits live in LDS).
+bool pg_gguf_gemv_takes_f32_row(int ggml_type, size_t n_out, size_t k_in, const float *x_f32) {
+    return ggml_type == PG_GGML_Q4_0 && n_out <= 8192 && k_in >= 32 && k_in <= 32768 && (uintptr_t)x_f32 % 16 == 0;
+}
+
+pg_status pg_launch_gguf_gemv_f32_row(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,
+                                      const uint16_t *d, const float *x_f32, float *y) {
+    if (ggml_type != PG_GGML_Q4_0) return pg_fail(PG_EUNSUPPORTED, "gguf_gemv: the one-launch row product holds Q4_0 code only");
+    return launch_gemv_f32x<4>(ctx, n_out, k_in, qs, d, x_f32, y);
+}
+
 // The tile-major copy of a tensor's quant plane that gguf_mm_kernel fetches: 16-byte chunks in
 // the order [group of 128 rows][group of 4 blocks][wavefront][fill][lane], where the lane of a
 // fill stands for (stream 16*fill + lane/4, block (lane%4) ^ ((lane/8)%4)) exactly as in the
@@ -478,6 +598,8 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
                               float *y_dev) {
     void *ws = nullptr;
     // MXFP4 and Q4_1 have the streaming kernel only; a K of a few blocks needs its finer fixed point
+    if (m == 1 && pg_gguf_gemv_takes_f32_row(w->ggml_type, w->n_out, w->k_in, x_dev))
+        return pg_launch_gguf_gemv_f32_row(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, x_dev, y_dev);
     if (m == 1 || w->ggml_type == PG_MXFP4 || w->ggml_type == PG_GGML_Q4_1 || w->k_in / 32 < PG_MM_MIN_BLOCKS) {
         if (m > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_matmul: more than 65535 rows through the streaming kernel (MXFP4, Q4_1 or k_in < %zu)", PG_MM_MIN_BLOCKS * 32);
         PG_TRY(pg_workspace(ctx, pg_xdigits_bytes(m, w->k_in), &ws));

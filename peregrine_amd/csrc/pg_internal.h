@@ -82,6 +82,7 @@ struct pg_gguf_tensor {
 // whose K spans fewer blocks than this run the streaming kernel (18 / 22-bit activations),
 // one item per activation row.
 constexpr size_t PG_MM_MIN_BLOCKS = 5;
+constexpr int PG_GEMM_MAX_GROUP = 4;  // weights one W8A8 launch can carry (fused q|k|v, gate|up)
 constexpr size_t PG_KPAD = 128;  // device K stride is a multiple of this
 constexpr size_t PG_NPAD = 256;  // device weight rows are padded to this
 
@@ -172,7 +173,6 @@ pg_status pg_launch_gemm_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
 // The same activation rows against up to PG_GEMM_MAX_GROUP weights of equal K in ONE launch: the
 // weights' column panels form one tile space (a fused QKV or gate|up product without a fused
 // copy of the weights).  out[i] is [m, w[i]->cols].
-constexpr int PG_GEMM_MAX_GROUP = 4;
 pg_status pg_launch_gemm_w8a8_group(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
                                     const pg_qtensor *const *w, float *const *out, int count, size_t m);
 // 5 .. 64 activation rows: K split over workgroups, i32 partial sums in `part`, then one finishing
@@ -188,6 +188,9 @@ pg_status pg_launch_gemv_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
 bool pg_gemv_w8a8_takes_f32_row(const pg_qtensor *w, size_t m, size_t k, const float *x_f32);
 pg_status pg_launch_gemv_w8a8_f32_row(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *w, float *out,
                                       int32_t *acc);
+// The same row against up to PG_GEMM_MAX_GROUP weights of equal K in one launch.
+pg_status pg_launch_gemv_w8a8_f32_row_group(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *const *w,
+                                            float *const *out, int count, int32_t *acc);
 // Activation rows rewritten as three byte-digit planes (see pg_gguf.hip).
 struct pg_xdigits {
     int8_t *digits;  // [rows][6 planes][k/32 blocks][16 bytes] (Q4_0 uses 5 planes, Q8_0 all 6)
@@ -240,6 +243,10 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
                               const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
                               const pg_xdigits &xd, float *y, const float *residual = nullptr,
                               const uint16_t *m = nullptr);
+// One activation row still in f32: digits made inside the product's own launch.  Only where the predicate holds.
+bool pg_gguf_gemv_takes_f32_row(int ggml_type, size_t n_out, size_t k_in, const float *x_f32);
+pg_status pg_launch_gguf_gemv_f32_row(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,
+                                      const uint16_t *d, const float *x_f32, float *y);
 // Activation rows as two byte-digit planes for the matrix-core product (see pg_gguf_mm.hip).
 struct pg_mmdigits {
     int8_t *digits;  // [rows][2 planes][k/32 blocks][2 halves][16 bytes], rows padded to an odd number of 256-byte lines

@@ -612,6 +612,10 @@ PG_API pg_status pg_matmul_quantized_multi_dev(pg_ctx *ctx, const float *a_dev, 
     if (m == 0) return PG_OK;
     PG_CHECK_ARG(a_dev != nullptr, "pg_matmul_quantized_multi: null pointer");
     PG_CHECK_ARG(m < (1ull << 24), "pg_matmul_quantized_multi: m = %zu too large", m);
+    bool one_row_group = m == 1 && count > 1;
+    for (size_t i = 0; i < count && one_row_group; ++i) one_row_group = pg_gemv_w8a8_takes_f32_row(w[i], m, k, a_dev);
+    if (one_row_group)  // one token: every weight's rows in one streaming launch that quantises the row itself
+        return pg_launch_gemv_w8a8_f32_row_group(ctx, a_dev, k, w, out_dev, (int)count, nullptr);
     if (count == 1 || m <= 256) {  // few rows: the single products pick their own route (GEMV, split K)
         for (size_t i = 0; i < count; ++i) PG_TRY(pg_matmul_quantized_dev(ctx, a_dev, m, k, w[i], out_dev[i], nullptr));
         return PG_OK;

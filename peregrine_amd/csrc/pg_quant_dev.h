@@ -25,3 +25,14 @@ __device__ __forceinline__ float pg_block_max_256(float v, float *red) {
     v = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     return v;
 }
+
+// The same without draining the wavefront's outstanding global loads (__syncthreads() waits for
+// vmcnt(0) as well): for kernels that keep weight rows in flight across the reduction.
+__device__ __forceinline__ float pg_block_max_256_keep_loads(float v, float *red) {
+    v = pg_wave_max_f32(v);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier" ::: "memory");
+    v = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    return v;
+}

@@ -91,6 +91,8 @@ GGUF_SHAPES = [
     (2, 64, 32768, 2),                                          # two K segments
     (2, 50, 11008, 1),                                          # partial last lane group
     (8, 256, 4096, 1), (8, 77, 96, 3), (8, 96, 6144, 4), (8, 64, 32768, 2),
+    (2, 100, 32768, 1), (2, 40, 64, 1), (2, 9, 32, 1), (2, 8192, 512, 1), (2, 4096, 4096, 1),   # Q4_0 one-launch row product: longest K, spare wavefronts, most rows
+    (2, 64, 32800, 1), (2, 8200, 256, 1), (8, 33, 32768, 1), (8, 9, 32, 1),   # past its limits (K, rows) and Q8_0: digits by a launch of their own
     (2, 14336, 4096, 1),                                        # benchmark configuration 4, full size
     (8, 6144, 4096, 1),
     # more than one row: matrix-core path (token tiles of 32, row tiles of 128, split K)
@@ -156,6 +158,13 @@ def test_gguf_matmul_special_inputs(ctx, orc):
     bad = np.ones(k_in, np.float32)
     bad[3] = np.nan
     assert np.isnan(gw.matmul(bad, 1)).all() and np.isnan(orc.gguf_matmul(bad, 1, raw, 2, n_out, k_in)).all()
+    # a device row that does not start on a 16-byte boundary is an argument error (128-bit loads)
+    from devbuf import DevBuf
+    from peregrine_amd import _ffi
+    import ctypes as C
+    shifted = DevBuf(ctx, host=np.zeros(k_in + 1, np.float32))
+    dy = DevBuf(ctx, n_out * 4)
+    assert _ffi.lib.pg_gguf_matmul_dev(ctx.handle, C.c_void_p(shifted.ptr.value + 4), 1, gw._h, dy.ptr) == _ffi.PG_EINVAL
     assert gw.matmul(np.zeros(0, np.float32), 0).size == 0                  # m = 0
     with pytest.raises(ValueError):
         gw.matmul(np.zeros(k_in + 1, np.float32), 1)

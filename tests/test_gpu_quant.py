@@ -373,9 +373,9 @@ def run_multi(ctx, da, m, k, qts, douts):
 
 
 @pytest.mark.parametrize("m,k,ns", [(300, 512, (1000, 130, 257)), (257, 128, (64, 64, 64, 64)), (40, 1024, (300, 77)),
-                                     (1, 4096, (1024, 512)), (3, 200, (33,)), (2048, 4096, (4096, 1024, 1024)),
+                                     (1, 4096, (1024, 512)), (1, 14336, (300, 77, 4096)), (3, 200, (33,)), (2048, 4096, (4096, 1024, 1024)),
                                      (2048, 4096, (14336, 14336))],
-                         ids=["ragged3", "four", "few-rows", "one-row", "single", "qkv", "gate-up"])
+                         ids=["ragged3", "four", "few-rows", "one-row", "one-row-long-k", "single", "qkv", "gate-up"])
 def test_matmul_quantized_multi_equals_the_single_products(ctx, orc, m, k, ns):
     """Several weights against one activation matrix (the reference's fused QKV / gate|up
     products): every output equals the single product bit for bit, and sampled rows equal the
