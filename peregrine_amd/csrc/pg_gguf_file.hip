@@ -14,6 +14,8 @@
 #include <map>
 #include <new>
 
+#include <exception>
+#include <new>
 #include "pg_internal.h"
 
 namespace {
@@ -73,7 +75,8 @@ struct Reader {
                 v.arr_type = rd<uint32_t>();
                 const uint64_t n = rd<uint64_t>();
                 if (depth > 4 || n > len - pos) { ok = false; break; }  // every element takes >= 1 byte
-                v.arr.reserve((size_t)n);
+                // (no reserve of n: a forged count would ask for ~100 bytes per claimed element; growth
+                // by push_back is bounded by what the file can really hold)
                 for (uint64_t i = 0; ok && i < n; ++i) v.arr.push_back(value(v.arr_type, depth + 1));
                 break;
             }
@@ -165,7 +168,14 @@ PG_API pg_status pg_gguf_file_parse(const void *data, size_t len, pg_gguf_file *
     if (!f) return pg_fail(PG_ENOMEM, "host allocation failed");
     f->data = static_cast<const uint8_t *>(data);
     f->len = len;
-    const pg_status st = parse_into(f);
+    pg_status st;
+    try {  // the containers can throw (bad_alloc, length_error): nothing may unwind across the ABI
+        st = parse_into(f);
+    } catch (const std::bad_alloc &) {
+        st = pg_fail(PG_ENOMEM, "out of host memory while parsing the GGUF header");
+    } catch (const std::exception &e) {
+        st = pg_fail(PG_EINVAL, "GGUF header is corrupt (%s)", e.what());
+    }
     if (st != PG_OK) { delete f; return st; }
     *out = f;
     return PG_OK;
@@ -215,7 +225,10 @@ static pg_status tensor_extent(const pg_gguf_file *f, const TensorInfo &t, size_
     size_t be = 1, bb = 1;
     (void)type_geometry(t.ggml_type, &be, &bb);
     unsigned __int128 n = 1;
-    for (uint64_t d : t.shape) { n *= d; if (n > ((unsigned __int128)1 << 62)) return pg_fail(PG_EINVAL, "tensor '%s' is too large", t.name.c_str()); }
+    // no tensor holds more elements than 32 per byte of the file (Q4_0 packs 32 into 18 bytes): a
+    // larger count is corrupt, and bounding it here keeps every product below in range
+    const unsigned __int128 max_elems = (unsigned __int128)f->len * 32 + 32;
+    for (uint64_t d : t.shape) { n *= d; if (n > max_elems) return pg_fail(PG_EINVAL, "tensor '%s' is larger than the file", t.name.c_str()); }
     const size_t ne = (size_t)n;
     PG_CHECK_ARG(ne % be == 0, "tensor elements %zu not divisible by block size %zu", ne, be);  // src/gguf.rs:160
     const size_t nbytes = ne / be * bb;

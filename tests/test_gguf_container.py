@@ -130,6 +130,19 @@ def test_gguf_malformed_files_are_errors_not_crashes(G):
     huge_arr = struct.pack("<IIQQ", 0x46554747, 3, 0, 1) + struct.pack("<Q", 1) + b"k" + struct.pack("<IIQ", 9, 0, 1 << 60)
     with pytest.raises(PeregrineError):  # array length far beyond the file
         G.GgufFile.parse(huge_arr)
+    # a large but honest array (1 M empty strings = 8 MB of length fields) parses; the same count with the
+    # last length field cut, or a count the file cannot hold, is an error -- and neither reserves
+    # room for the claimed count up front
+    big = struct.pack("<IIQQ", 0x46554747, 3, 0, 1) + struct.pack("<Q", 1) + b"k" + struct.pack("<IIQ", 9, 8, 1 << 20) + bytes(8 << 20)
+    G.GgufFile.parse(big)
+    forged = big[:-1]
+    with pytest.raises(PeregrineError):
+        G.GgufFile.parse(forged)
+    # an F32 tensor whose element count times 4 wraps 64 bits: larger than the file, not "0 bytes"
+    wrap, _, _ = H.build_gguf([], [("w", 0, [1 << 62], bytes(64))])
+    gw = G.GgufFile.parse(wrap)
+    assert _ffi.lib.pg_gguf_file_tensor_info(gw._h, b"w", None, None, None, 0, None, C.byref(size), None) != 0
+    assert "larger than the file" in _ffi.lib.pg_last_error().decode()
     not_div, _, _ = H.build_gguf([], [("x", 8, [33], bytes(68))])
     g = G.GgufFile.parse(not_div)
     assert _ffi.lib.pg_gguf_file_tensor_info(g._h, b"x", None, None, None, 0, None, C.byref(size), None) != 0
