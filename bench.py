@@ -370,6 +370,7 @@ def main():
     if not args.only_headline:
         section_decode_and_linear(B, line)
         section_gguf(B, line)
+        section_mxfp4(B, line)
         section_moe(B, line)
         section_llama_block(B, line)
         section_huffman(B, line)
@@ -530,6 +531,48 @@ def section_gguf(B, line):
     line["gguf_q4_0_skinny"] = skinny
     for h in q4:
         lib.pg_gguf_free(B.h, h)
+    torch.cuda.empty_cache()
+
+
+def section_mxfp4(B, line):
+    """MXFP4 one-row products (examples/gpt_oss/moe.rs mxfp4_matmul): the gpt-oss expert shapes and cfg4's shape."""
+    import numpy as np
+
+    torch, lib, check, ptr, dev, args = B.torch, B.lib, B.check, B.ptr, B.dev, B.args
+    out = []
+    rng = np.random.default_rng(7400)
+    for n_out, k_in, rot in ((14336, 4096, 10), (5760, 2880, 40), (2880, 2880, 80)):
+        codes = rng.integers(0, 256, size=n_out * k_in // 2, dtype=np.uint8)
+        scales = rng.integers(118, 124, size=n_out * k_in // 32, dtype=np.uint8)
+        hs = []
+        for r in range(rot):  # rot x 17 B per block of distinct tensors: more than the 256 MB last-level cache
+            codes[0] = r
+            h = C.c_void_p()
+            check(lib.pg_mxfp4_upload(B.h, C.c_void_p(codes.ctypes.data), C.c_void_p(scales.ctypes.data), n_out, k_in, C.byref(h)))
+            hs.append(h)
+        x = B.make_acts(1, k_in, 7410)
+        y = torch.empty(1, n_out, device=dev)
+
+        def step():
+            h = hs[B.i % rot]
+            B.i += 1
+            check(lib.pg_gguf_matmul_dev(B.h, ptr(x), 1, h, ptr(y)))
+
+        nbytes = n_out * (k_in // 32) * 17 + 4 * k_in + 4 * n_out
+        t = B.timed(step, B.dsteps, max(args.warmup, 8))
+        prof, grids = B.profiled(step, B.dsteps)
+        k_ms = prof["mxfp4_rows"][0]
+        out.append({"workload": f"M=1 MXFP4 [{k_in}]->[{n_out}], one launch (FP4 codes and E8M0 scales straight into the scaled "
+                                f"matrix-core instruction); {rot} tensors rotated",
+                    "value": round(nbytes / (t["ms_per_step"] * 1e-3) / 1e9, 1), "unit": "GB/s",
+                    "frac_of_hbm_peak": round(nbytes / (t["ms_per_step"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), **B.stats(t),
+                    "roofline": {"kernel": "mxfp4_rows_kernel", "bound": "hbm", "achieved": round(nbytes / (k_ms * 1e-3) / 1e9, 1),
+                                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(nbytes / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                                 "traffic": B.traffic_for("mxfp4_rows", grids), "bytes_per_launch": nbytes,
+                                 "avg_launch_ms": round(k_ms, 5)}})
+        for h in hs:
+            lib.pg_gguf_free(B.h, h)
+    line["mxfp4_gemv"] = out
     torch.cuda.empty_cache()
 
 

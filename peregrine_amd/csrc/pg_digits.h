@@ -11,7 +11,7 @@
 //   digits[row][j][b]   16 bytes per (plane j, block b)
 //     NIB (Q4_0):  |X| < 2^18, X = sum_j 16^j n_j with five signed 4-bit digits; plane j holds
 //                  n_j of the block's 32 elements, element e in nibble e.
-//     bytes (Q8_0, MXFP4): |X| < 2^22, X = 65536 a0 + 256 a1 + a2 with signed byte digits;
+//     bytes (Q8_0): |X| < 2^22, X = 65536 a0 + 256 a1 + a2 with signed byte digits;
 //                  plane 2j+h holds a_j of elements 16h..16h+15.
 // With `xsum` (Q4_1, whose blocks carry an offset m: sum_k (q d + m) x = d sum q x + m sum x) the
 // block's sum of fixed-point values, sum_k X[k], is stored too: xsum[row][b] (exact: < 2^23).

@@ -208,8 +208,6 @@ struct RowLoads {
 // blockIdx.y = batch item (activation row / MoE pair).  With a table, item i multiplies by
 // expert table[expert_of[i]] and reads activation row i / x_row_div; without one, every item
 // uses (qs0, d0).  R rows are in flight at a time (NG = RW / R groups, double-buffered).
-// BF: the 16-bit block scales are the top halves of f32 values (the power-of-two scales of
-// MXFP4 blocks, whose range f16 cannot hold) instead of f16.
 // Q41 (with QT = 4): every block also has an offset m; its term (8 d + m) * sum_k x_k uses the
 // block sums written with the digits.
 // XF32 (one item, no tables): the activation row arrives in f32 (x_f32) and the workgroup -- NW
@@ -217,7 +215,7 @@ struct RowLoads {
 // wavefront has requested its first weight rows: the product is one launch instead of two, and
 // the digit arithmetic (18 vector operations per element, shared by NW wavefronts) runs while
 // those first loads are in flight.
-template <int QT, int BPL, int RW, int R, bool BF = false, bool Q41 = false, bool XF32 = false, int NW = 1>
+template <int QT, int BPL, int RW, int R, bool Q41 = false, bool XF32 = false, int NW = 1>
 __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
     const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0, pg_gemv_batch batch,
     int n_out, int nb, const int8_t *__restrict__ digits_base, const float *__restrict__ xs_base,
@@ -376,8 +374,7 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
                         f = fmaf((float)hi, 65536.0f, (float)lo);  // both terms exact in f32
                     }
                     const uint32_t pair = (uint32_t)dtile[p][tr >> 1];
-                    const float dv = BF ? __uint_as_float((tr & 1) ? pair & 0xFFFF0000u : pair << 16)
-                                        : half_bits_to_float((uint16_t)((tr & 1) ? pair >> 16 : pair & 0xFFFFu));
+                    const float dv = half_bits_to_float((uint16_t)((tr & 1) ? pair >> 16 : pair & 0xFFFFu));
                     const float ds = dv * sb[p];
                     acc[g][r] = fmaf(ds, f, acc[g][r]);
                     if constexpr (Q41) {
@@ -399,7 +396,7 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
         }
 }
 
-template <int QT, int BPL, bool BF, bool Q41>
+template <int QT, int BPL, bool Q41>
 pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
                           const pg_gemv_batch &batch, const pg_xdigits &xd, float *y, const float *residual,
                           const uint16_t *m) {
@@ -411,8 +408,8 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
 #define PG_GGUF_GEMV_LAUNCH(RWW, RR)                                                               \
     do {                                                                                           \
         const dim3 grid(grid_for(n_out, RWW), (unsigned)batch.count);                              \
-        PG_TRY(pg_launch(ctx, QT == 4 ? (Q41 ? "gguf_gemv_q4_1" : "gguf_gemv_q4_0") : (BF ? "gguf_gemv_mxfp4" : "gguf_gemv_q8_0"), \
-                         gguf_gemv_kernel<QT, BPL, RWW, RR, BF, Q41>, grid, dim3(64), 0, qs, d, batch, \
+        PG_TRY(pg_launch(ctx, QT == 4 ? (Q41 ? "gguf_gemv_q4_1" : "gguf_gemv_q4_0") : "gguf_gemv_q8_0", \
+                         gguf_gemv_kernel<QT, BPL, RWW, RR, Q41>, grid, dim3(64), 0, qs, d, batch, \
                          (int)n_out, nb, xd.digits, xd.xs, y, residual, m, (const float *)xd.xsum, (const float *)nullptr)); \
     } while (0)
     if (n_out / 8 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(8, R8);
@@ -423,7 +420,7 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
 }
 
 // One row still in f32: the one-launch form (four or eight wavefronts per workgroup share the digits).
-template <int QT, int BPL, bool BF, int NW>
+template <int QT, int BPL, int NW>
 pg_status launch_gemv_f32x_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const float *x_f32,
                                float *y) {
     constexpr int NH = QT == 8 ? 2 : 1;
@@ -432,10 +429,10 @@ pg_status launch_gemv_f32x_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uin
     const size_t lds = (size_t)nb * 96 + (size_t)nb * sizeof(float);
     const pg_gemv_batch one = {1, nullptr, nullptr, nullptr, 1};
     const size_t want = (size_t)ctx->num_cu * 6;
-    const char *name = QT == 4 ? "gguf_gemv_q4_0" : (BF ? "gguf_gemv_mxfp4" : "gguf_gemv_q8_0");
+    const char *name = QT == 4 ? "gguf_gemv_q4_0" : "gguf_gemv_q8_0";
 #define PG_GGUF_GEMV_X_LAUNCH(RWW, RR)                                                                             \
     do {                                                                                                           \
-        auto kern = gguf_gemv_kernel<QT, BPL, RWW, RR, BF, false, true, NW>;                                       \
+        auto kern = gguf_gemv_kernel<QT, BPL, RWW, RR, false, true, NW>;                                       \
         PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                \
         PG_TRY(pg_launch(ctx, name, kern, dim3(grid_for(n_out, RWW * NW)), dim3(64 * NW), lds, qs, d, one, (int)n_out, nb, \
                          (const int8_t *)nullptr, (const float *)nullptr, y, (const float *)nullptr,               \
@@ -448,7 +445,7 @@ pg_status launch_gemv_f32x_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uin
     return PG_OK;
 }
 
-template <int QT, bool BF = false>
+template <int QT>
 pg_status launch_gemv_f32x(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const float *x_f32, float *y) {
     size_t bpl = (k_in / 32 + 63) / 64;
     if (bpl > 4) bpl = 4;
@@ -456,14 +453,14 @@ pg_status launch_gemv_f32x(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t
     // in total -- eight wavefronts each where that still leaves a workgroup for a good part of the CUs.
     const bool wide = n_out / 64 >= (size_t)ctx->num_cu / 6;
     switch (bpl) {
-        case 1: return wide ? launch_gemv_f32x_bpl<QT, 1, BF, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 1, BF, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
-        case 2: return wide ? launch_gemv_f32x_bpl<QT, 2, BF, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 2, BF, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
-        case 3: return wide ? launch_gemv_f32x_bpl<QT, 3, BF, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 3, BF, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
-        default: return wide ? launch_gemv_f32x_bpl<QT, 4, BF, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 4, BF, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
+        case 1: return wide ? launch_gemv_f32x_bpl<QT, 1, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 1, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
+        case 2: return wide ? launch_gemv_f32x_bpl<QT, 2, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 2, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
+        case 3: return wide ? launch_gemv_f32x_bpl<QT, 3, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 3, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
+        default: return wide ? launch_gemv_f32x_bpl<QT, 4, 8>(ctx, n_out, k_in, qs, d, x_f32, y) : launch_gemv_f32x_bpl<QT, 4, 4>(ctx, n_out, k_in, qs, d, x_f32, y);
     }
 }
 
-template <int QT, bool BF = false, bool Q41 = false>
+template <int QT, bool Q41 = false>
 pg_status launch_gemv(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
                       const pg_gemv_batch &batch, const pg_xdigits &xd, float *y, const float *residual,
                       const uint16_t *m) {
@@ -471,10 +468,10 @@ pg_status launch_gemv(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs,
     size_t bpl = (nb + 63) / 64;
     if (bpl > 4) bpl = 4;  // longer rows run as several K segments of 256 blocks
     switch (bpl) {
-        case 1: return launch_gemv_bpl<QT, 1, BF, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
-        case 2: return launch_gemv_bpl<QT, 2, BF, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
-        case 3: return launch_gemv_bpl<QT, 3, BF, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
-        default: return launch_gemv_bpl<QT, 4, BF, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
+        case 1: return launch_gemv_bpl<QT, 1, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
+        case 2: return launch_gemv_bpl<QT, 2, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
+        case 3: return launch_gemv_bpl<QT, 3, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
+        default: return launch_gemv_bpl<QT, 4, Q41>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
     }
 }
 
@@ -521,10 +518,10 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
     if (batch.count > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_gemv: more than 65535 batch items");
     if (ggml_type == PG_GGML_Q4_1) {
         if (!m || batch.qs_table) return pg_fail(PG_EINVAL, "gguf_gemv: Q4_1 needs its offsets and runs without expert tables");
-        return launch_gemv<4, false, true>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
+        return launch_gemv<4, true>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, m);
     }
     if (ggml_type == PG_GGML_Q4_0) return launch_gemv<4>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, nullptr);
-    if (ggml_type == PG_MXFP4) return launch_gemv<8, true>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, nullptr);
+    if (ggml_type == PG_MXFP4) return pg_fail(PG_EUNSUPPORTED, "gguf_gemv: MXFP4 tensors have their own kernel");
     return launch_gemv<8>(ctx, n_out, k_in, qs, d, batch, xd, y, residual, nullptr);
 }
 
@@ -597,11 +594,12 @@ pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w) {
 pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
                               float *y_dev) {
     void *ws = nullptr;
-    // MXFP4 and Q4_1 have the streaming kernel only; a K of a few blocks needs its finer fixed point
+    if (w->ggml_type == PG_MXFP4) return pg_launch_mxfp4_rows(ctx, x_dev, m, w, y_dev);
+    // Q4_1 has the streaming kernel only; a K of a few blocks needs its finer fixed point
     if (m == 1 && pg_gguf_gemv_takes_f32_row(w->ggml_type, w->n_out, w->k_in, x_dev))
         return pg_launch_gguf_gemv_f32_row(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, x_dev, y_dev);
-    if (m == 1 || w->ggml_type == PG_MXFP4 || w->ggml_type == PG_GGML_Q4_1 || w->k_in / 32 < PG_MM_MIN_BLOCKS) {
-        if (m > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_matmul: more than 65535 rows through the streaming kernel (MXFP4, Q4_1 or k_in < %zu)", PG_MM_MIN_BLOCKS * 32);
+    if (m == 1 || w->ggml_type == PG_GGML_Q4_1 || w->k_in / 32 < PG_MM_MIN_BLOCKS) {
+        if (m > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_matmul: more than 65535 rows through the streaming kernel (Q4_1 or k_in < %zu)", PG_MM_MIN_BLOCKS * 32);
         PG_TRY(pg_workspace(ctx, pg_xdigits_bytes(m, w->k_in), &ws));
         const pg_xdigits xd = pg_xdigits_carve(ws, m, w->k_in);
         PG_TRY(pg_launch_x_to_digits(ctx, x_dev, m, w->k_in, w->ggml_type, xd));
@@ -636,7 +634,7 @@ pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, c
         any_mxfp4 |= w[i]->ggml_type == PG_MXFP4;
         any_q41 |= w[i]->ggml_type == PG_GGML_Q4_1;
     }
-    if ((any_mxfp4 && m > 1) || any_q41 || (m > 1 && k_in / 32 < PG_MM_MIN_BLOCKS)) {  // no shared route: product by product
+    if (any_mxfp4 || any_q41 || (m > 1 && k_in / 32 < PG_MM_MIN_BLOCKS)) {  // no shared route: product by product
         for (int i = 0; i < count; ++i) PG_TRY(pg_gguf_matmul_rows(ctx, x_dev, m, w[i], y_dev[i]));
         return PG_OK;
     }
@@ -769,190 +767,6 @@ PG_API pg_status pg_gguf_upload(pg_ctx *ctx, const void *blocks, int ggml_type, 
     }
     if (st != PG_OK) { pg_gguf_free(ctx, t); return st; }
     *out = t;
-    return PG_OK;
-}
-
-// ---- MXFP4 (gpt_oss experts) ----------------------------------------------------------
-// A block is 16 bytes of FP4 (E2M1) codes, byte k = elements 2k (low nibble) and 2k+1, plus
-// one E8M0 scale byte: value = LUT[code] * 2^(scale - 127)   (examples/gpt_oss/moe.rs:5-53).
-// Twice the LUT is an integer in [-12, 12], so the tensor is kept as i8 planes (the Q8_0
-// device layout) with the block scale 2^(scale - 128) stored as the top half of its f32.
-__global__ void mxfp4_split_kernel(const uint8_t *__restrict__ blocks, const uint8_t *__restrict__ scales, size_t n_out,
-                                   size_t nb, uint8_t *__restrict__ qs, uint16_t *__restrict__ d) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t n_pad = (n_out + 7) / 8 * 8;
-    if (i >= n_pad * nb) return;
-    const size_t n = i / nb, b = i - n * nb;
-    uint16_t *dd = d + ((n / 8) * nb + b) * 8 + (n % 8);
-    if (n >= n_out) { *dd = 0; return; }
-    const unsigned e = scales[i];
-    // f32::from_bits(e << 23) / 2: zero for e = 0, the subnormal 2^-127 for e = 1, inf for e = 255
-    *dd = (uint16_t)(e == 0 ? 0u : (e == 1 ? 0x0040u : (e == 255 ? 0x7F80u : (e - 1) << 7)));
-    const int8_t twice[8] = {0, 1, 2, 3, 4, 6, 8, 12};
-    for (int k = 0; k < 16; ++k) {
-        const unsigned byte = blocks[i * 16 + k];
-        const int lo = twice[byte & 7], hi = twice[(byte >> 4) & 7];
-        const int e0 = 2 * k, e1 = 2 * k + 1;
-        qs[((n * 2 + (e0 >> 4)) * nb + b) * 16 + (e0 & 15)] = (uint8_t)(int8_t)((byte & 8) ? -lo : lo);
-        qs[((n * 2 + (e1 >> 4)) * nb + b) * 16 + (e1 & 15)] = (uint8_t)(int8_t)((byte & 0x80) ? -hi : hi);
-    }
-}
-
-PG_API pg_status pg_mxfp4_upload(pg_ctx *ctx, const uint8_t *blocks, const uint8_t *scales, size_t out_dim,
-                                 size_t in_dim, pg_gguf_tensor **out) {
-    PG_TRY(pg_use(ctx));
-    PG_CHECK_ARG(out != nullptr, "pg_mxfp4_upload: out is null");
-    *out = nullptr;
-    PG_CHECK_ARG(out_dim > 0 && in_dim > 0 && blocks && scales, "pg_mxfp4_upload: empty tensor or null pointer");
-    PG_CHECK_ARG(in_dim % 32 == 0, "pg_mxfp4_upload: in_dim %zu is not a multiple of 32", in_dim);
-    PG_CHECK_ARG(out_dim < (1ull << 31) && in_dim < (1ull << 31) && out_dim * (in_dim / 32) < (1ull << 31),
-                 "pg_mxfp4_upload: shape too large");
-    const size_t nb = in_dim / 32, nblocks = out_dim * nb;
-    pg_gguf_tensor *t = new (std::nothrow) pg_gguf_tensor();
-    if (!t) return pg_fail(PG_ENOMEM, "host allocation failed");
-    t->qs = nullptr;
-    t->d = nullptr;
-    t->m = nullptr;
-    t->qs_tiled = nullptr;
-    t->ggml_type = PG_MXFP4;
-    t->n_out = out_dim;
-    t->k_in = in_dim;
-    pg_tmp rb, rs;
-    pg_status st = rb.alloc(nblocks * 16);
-    if (st == PG_OK) st = rs.alloc(nblocks);
-    hipError_t e = hipSuccess;
-    if (st == PG_OK) {
-        e = hipMalloc((void **)&t->qs, nblocks * 32);
-        if (e == hipSuccess) e = hipMalloc((void **)&t->d, (out_dim + 7) / 8 * 8 * nb * sizeof(uint16_t));
-        if (e == hipSuccess) e = hipMemcpyAsync(rb.p, blocks, nblocks * 16, hipMemcpyHostToDevice, ctx->stream);
-        if (e == hipSuccess) e = hipMemcpyAsync(rs.p, scales, nblocks, hipMemcpyHostToDevice, ctx->stream);
-        if (e == hipSuccess) {
-            mxfp4_split_kernel<<<grid_for((out_dim + 7) / 8 * 8 * nb, 256), 256, 0, ctx->stream>>>(
-                rb.as<uint8_t>(), rs.as<uint8_t>(), out_dim, nb, t->qs, t->d);
-            e = hipGetLastError();
-        }
-        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
-        if (e != hipSuccess)
-            st = pg_fail(e == hipErrorOutOfMemory ? PG_ENOMEM : PG_EDEVICE, "pg_mxfp4_upload: %s", hipGetErrorString(e));
-    }
-    if (st != PG_OK) { pg_gguf_free(ctx, t); return st; }
-    *out = t;
-    return PG_OK;
-}
-
-PG_API pg_status pg_mxfp4_matmul(pg_ctx *ctx, const float *input, const uint8_t *blocks, const uint8_t *scales,
-                                 size_t out_dim, size_t in_dim, float *output) {
-    pg_gguf_tensor *t = nullptr;
-    PG_TRY(pg_mxfp4_upload(ctx, blocks, scales, out_dim, in_dim, &t));
-    const pg_status st = pg_gguf_matmul(ctx, input, 1, t, output);
-    pg_gguf_free(ctx, t);
-    return st;
-}
-
-// Mxfp4Expert  examples/gpt_oss/moe.rs:55-117, swiglu :145-154.
-struct pg_mxfp4_expert {
-    pg_gguf_tensor *mlp1, *mlp2;  // [2 * intermediate, hidden], [hidden, intermediate]
-    float *bias1, *bias2;         // [2 * intermediate], [hidden] (one allocation)
-    size_t hidden, intermediate;
-    float alpha, clamp;
-};
-
-namespace {
-// biased = h + bias1; gate = biased[2i].min(clamp); linear = biased[2i+1].clamp(-clamp, clamp);
-// out[i] = gate * (1 / (1 + exp(-alpha * gate))) * (linear + 1)
-__global__ __launch_bounds__(256) void mxfp4_bias_swiglu_kernel(const float *__restrict__ h, const float *__restrict__ bias,
-                                                                size_t rows, size_t inter, float alpha, float clamp,
-                                                                float *__restrict__ out) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= rows * inter) return;
-    const size_t r = i / inter, c = i - r * inter;
-    const float g0 = h[r * 2 * inter + 2 * c] + bias[2 * c], l0 = h[r * 2 * inter + 2 * c + 1] + bias[2 * c + 1];
-    const float gate = fminf(g0, clamp);                                     // f32::min: a NaN operand loses
-    const float linear = l0 != l0 ? l0 : fminf(fmaxf(l0, -clamp), clamp);    // f32::clamp keeps NaN
-    const float activated = gate * (1.0f / (1.0f + expf(-alpha * gate)));
-    out[i] = activated * (linear + 1.0f);
-}
-
-__global__ __launch_bounds__(256) void bias_add_kernel(const float *__restrict__ a, const float *__restrict__ bias,
-                                                       size_t rows, size_t cols, float *__restrict__ out) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < rows * cols) out[i] = a[i] + bias[i % cols];
-}
-}  // namespace
-
-PG_API void pg_mxfp4_expert_free(pg_ctx *ctx, pg_mxfp4_expert *e) {
-    if (!e) return;
-    if (ctx) {
-        (void)pg_use(ctx);
-        (void)hipStreamSynchronize(ctx->stream);
-    }
-    pg_gguf_free(ctx, e->mlp1);
-    pg_gguf_free(ctx, e->mlp2);
-    if (e->bias1) (void)hipFree(e->bias1);
-    delete e;
-}
-
-PG_API pg_status pg_mxfp4_expert_create(pg_ctx *ctx, size_t hidden, size_t intermediate, float alpha, float clamp,
-                                        const uint8_t *mlp1_blocks, const uint8_t *mlp1_scales,
-                                        const uint8_t *mlp2_blocks, const uint8_t *mlp2_scales, const float *mlp1_bias,
-                                        const float *mlp2_bias, pg_mxfp4_expert **out) {
-    PG_TRY(pg_use(ctx));
-    PG_CHECK_ARG(out != nullptr, "pg_mxfp4_expert_create: out is null");
-    *out = nullptr;
-    PG_CHECK_ARG(mlp1_bias && mlp2_bias, "pg_mxfp4_expert_create: null bias");
-    pg_mxfp4_expert *e = new (std::nothrow) pg_mxfp4_expert{nullptr, nullptr, nullptr, nullptr, hidden, intermediate, alpha, clamp};
-    if (!e) return pg_fail(PG_ENOMEM, "host allocation failed");
-    pg_status st = pg_mxfp4_upload(ctx, mlp1_blocks, mlp1_scales, 2 * intermediate, hidden, &e->mlp1);
-    if (st == PG_OK) st = pg_mxfp4_upload(ctx, mlp2_blocks, mlp2_scales, hidden, intermediate, &e->mlp2);
-    if (st == PG_OK) {
-        hipError_t he = hipMalloc((void **)&e->bias1, (2 * intermediate + hidden) * sizeof(float));
-        if (he == hipSuccess) {
-            e->bias2 = e->bias1 + 2 * intermediate;
-            he = hipMemcpyAsync(e->bias1, mlp1_bias, 2 * intermediate * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
-        }
-        if (he == hipSuccess) he = hipMemcpyAsync(e->bias2, mlp2_bias, hidden * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
-        if (he == hipSuccess) he = hipStreamSynchronize(ctx->stream);
-        if (he != hipSuccess)
-            st = pg_fail(he == hipErrorOutOfMemory ? PG_ENOMEM : PG_EDEVICE, "pg_mxfp4_expert_create: %s", hipGetErrorString(he));
-    }
-    if (st != PG_OK) { pg_mxfp4_expert_free(ctx, e); return st; }
-    *out = e;
-    return PG_OK;
-}
-
-// scratch_dev: [m, 3 * intermediate] floats (the mlp1 output, then the activated rows).
-PG_API pg_status pg_mxfp4_expert_forward_dev(pg_ctx *ctx, const pg_mxfp4_expert *e, const float *x_dev, size_t m,
-                                             float *scratch_dev, float *out_dev) {
-    PG_TRY(pg_use(ctx));
-    PG_CHECK_ARG(e != nullptr, "pg_mxfp4_expert_forward: null expert");
-    if (m == 0) return PG_OK;
-    PG_CHECK_ARG(x_dev && scratch_dev && out_dev, "pg_mxfp4_expert_forward: null pointer");
-    PG_CHECK_ARG((uintptr_t)x_dev % 16 == 0 && (uintptr_t)scratch_dev % 16 == 0,
-                 "pg_mxfp4_expert_forward: x and scratch must be 16-byte aligned");
-    PG_CHECK_ARG(m <= 65535, "pg_mxfp4_expert_forward: more than 65535 rows");
-    const size_t inter = e->intermediate, hid = e->hidden;
-    float *h = scratch_dev, *act = scratch_dev + m * 2 * inter;
-    PG_TRY(pg_gguf_matmul_rows(ctx, x_dev, m, e->mlp1, h));
-    PG_TRY(pg_launch(ctx, "mxfp4_bias_swiglu", mxfp4_bias_swiglu_kernel, dim3(grid_for(m * inter, 256)), dim3(256), 0,
-                     (const float *)h, (const float *)e->bias1, m, inter, e->alpha, e->clamp, act));
-    PG_TRY(pg_gguf_matmul_rows(ctx, act, m, e->mlp2, out_dev));
-    return pg_launch(ctx, "bias_add", bias_add_kernel, dim3(grid_for(m * hid, 256)), dim3(256), 0, (const float *)out_dev,
-                     (const float *)e->bias2, m, hid, out_dev);
-}
-
-PG_API pg_status pg_mxfp4_expert_forward(pg_ctx *ctx, const pg_mxfp4_expert *e, const float *x, size_t m, float *out) {
-    PG_TRY(pg_use(ctx));
-    PG_CHECK_ARG(e != nullptr, "pg_mxfp4_expert_forward: null expert");
-    if (m == 0) return PG_OK;
-    PG_CHECK_ARG(x && out, "pg_mxfp4_expert_forward: null pointer");
-    pg_tmp dx, ds, dout;
-    PG_TRY(dx.alloc(m * e->hidden * sizeof(float)));
-    PG_TRY(ds.alloc(m * 3 * e->intermediate * sizeof(float)));
-    PG_TRY(dout.alloc(m * e->hidden * sizeof(float)));
-    PG_HIP(hipMemcpyAsync(dx.p, x, m * e->hidden * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
-    PG_TRY(pg_mxfp4_expert_forward_dev(ctx, e, dx.as<float>(), m, ds.as<float>(), dout.as<float>()));
-    PG_HIP(hipMemcpyAsync(out, dout.p, m * e->hidden * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
-    PG_HIP(hipStreamSynchronize(ctx->stream));
     return PG_OK;
 }
 

@@ -292,6 +292,9 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
                             const uint16_t *d, const pg_mm_group &grp, size_t total_pairs, const pg_mmdigits &md,
                             float *y, float *part);
 // y[m, n_out] = x[m, k_in] . dequant(w)^T on device pointers (uses the scratch arena).
+// MXFP4 tensors (pg_mxfp4.hip): qs holds the code bytes in matrix-core fragment order, d the E8M0 scale
+// bytes (four per dword); every product over them runs pg_launch_mxfp4_rows.
+pg_status pg_launch_mxfp4_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w, float *y_dev);
 pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
                               float *y_dev);
 // `count` such products over the same rows (equal k_in), the rows rewritten as digits once.

@@ -1241,10 +1241,10 @@ PG_API pg_status pg_llama_block_set_weights(pg_ctx *ctx, pg_llama_block *b, cons
     }
     PG_HIP(hipStreamSynchronize(ctx->stream));
     for (int i = 0; i < 7; ++i) b->w[i] = w[i];
-    // nibble digits (Q4_0) or byte digits (Q8_0, MXFP4); Q4_1 also needs block sums, which only
-    // the separate digit kernel writes: such a block takes the product-by-product route
+    // nibble digits (Q4_0) or byte digits (Q8_0); Q4_1 also needs block sums and MXFP4 its own digit
+    // order, which only the separate digit kernel writes: such a block takes the product-by-product route
     auto kind = [](const pg_gguf_tensor *t) {
-        return t->ggml_type == PG_GGML_Q4_1 ? -1 : (t->ggml_type == PG_GGML_Q4_0 ? PG_GGML_Q4_0 : PG_GGML_Q8_0);
+        return t->ggml_type == PG_GGML_Q4_0 ? PG_GGML_Q4_0 : (t->ggml_type == PG_GGML_Q8_0 ? PG_GGML_Q8_0 : -1);
     };
     b->digit_kind = kind(w[0]);
     for (int i = 1; i < 7; ++i)

@@ -1,0 +1,463 @@
+// MXFP4 weights (gpt_oss experts, examples/gpt_oss/moe.rs:5-117) on the scaled matrix-core
+// instruction of gfx950, which takes FP4 (E2M1) codes and E8M0 block scales as they sit in the file.
+//
+// v_mfma_scale_f32_16x16x128_f8f6f4, D[16 x 16] += A[16 x 128] * B[128 x 16], with A in FP4 and B in
+// FP8 (E4M3), every 32 consecutive k of a row of A / column of B scaled by 2^(byte - 127):
+//   A  lane l holds row l % 16, k = 32 (l / 16) .. + 31: the 16 code bytes of one MXFP4 block, element e
+//      in nibble e -- exactly the file's packing (byte i = elements 2i low, 2i + 1 high);
+//   B  lane l holds column l % 16; its first 16 bytes are k = 16 (l / 16) .. + 15, its last 16 bytes
+//      k = 64 + 16 (l / 16) .. + 15;
+//   scale operands: one byte per lane (selected by op_sel), lane l = row or column l % 16, k block l / 16;
+//   D  lane l holds column l % 16, rows 4 (l / 16) .. + 3.
+// (Layouts read off the hardware with one-hot operands.)
+//
+// The weights are rows of A: 17 bytes per block are all the product reads.  An activation row is not
+// representable in FP8, but a fixed-point rewriting of it is: per block x[k] = 2^se X[k], |X| < 2^23, and
+// X = sum_j 32^j n_j with five balanced base-32 digits n_j in [-16, 16], each exact in E4M3.  Digit plane
+// j of a row is one column of B with block scale byte 127 + se + 5 j, so the instruction itself applies
+// both block scales and sums over K; the five columns of a row are added at the end.  Three activation
+// rows (15 columns) share one pass over the weights.
+#include "pg_internal.h"
+#include "pg_digits.h"
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef const v4i __attribute__((address_space(1))) *gv4i_ptr;
+
+constexpr int MX_PLANES = 5;  // digit planes per activation row
+constexpr int MX_U = 8;       // chunks (of 4 blocks) per batch of weight loads in flight
+constexpr int MX_MAX_T = 3;   // activation rows per pass over the weights
+
+inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
+// chunks of 4 blocks per row, rounded up to whole scale dwords (4 chunks)
+inline size_t mx_chunks(size_t nb) { return ((nb + 3) / 4 + 3) & ~(size_t)3; }
+
+// ---- device layout of a tensor ------------------------------------------------------
+// Fragment-major: for every group of 16 rows and every chunk of 4 blocks (128 k), the 64 lanes' 16 code
+// bytes in lane order (one fully coalesced 1 KiB load per instruction), and per 4 chunks one dword per
+// lane with the 4 scale bytes.  Rows and blocks past the tensor's end hold zero codes; blocks whose
+// scale byte is 0 (the reference's f32::from_bits(0) = 0.0, the hardware's 2^-127) also get zero codes.
+__global__ void mxfp4_fragments_kernel(const uint8_t *__restrict__ blocks, const uint8_t *__restrict__ scales, int n_out,
+                                       int nb, int ncp, uint4 *__restrict__ qs, uint8_t *__restrict__ sc) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // (row group, chunk, lane)
+    const size_t nrg = ((size_t)n_out + 15) / 16;
+    if (i >= nrg * ncp * 64) return;
+    const int lane = (int)(i & 63), c = (int)((i >> 6) % ncp);
+    const size_t rg = (i >> 6) / ncp;
+    const size_t row = rg * 16 + (lane & 15);
+    const int blk = 4 * c + (lane >> 4);
+    uint4 v = {0, 0, 0, 0};
+    unsigned e = 127;
+    if (row < (size_t)n_out && blk < nb) {
+        e = scales[row * nb + blk];
+        if (e != 0) {
+            const uint8_t *src = blocks + (row * nb + blk) * 16;  // any alignment
+            unsigned wv[4];
+            for (int t = 0; t < 4; ++t) wv[t] = src[4 * t] | (src[4 * t + 1] << 8) | (src[4 * t + 2] << 16) | ((unsigned)src[4 * t + 3] << 24);
+            v = make_uint4(wv[0], wv[1], wv[2], wv[3]);
+        }
+    }
+    qs[i] = v;
+    sc[((rg * (ncp / 4) + c / 4) * 64 + lane) * 4 + (c & 3)] = (uint8_t)e;
+}
+
+// ---- one activation block -> five E4M3 digit planes in LDS ---------------------------
+// Eight consecutive lanes hold one block (f = elements 4 sub .. 4 sub + 3); all eight call together.
+// dig: the row's first plane, planes `stride` bytes apart, k-th element of plane j at dig[j * stride + k];
+// sb:  scale bytes, plane j / block b at sb[(j * 4 + b % 4) * ncp + b / 4].
+__device__ __forceinline__ void mx_emit_digits(const float (&f)[4], int b, int sub, char *dig, int stride, uint8_t *sb, int ncp) {
+    float amax = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3])));
+    int bad = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]);
+    amax = fmaxf(amax, __builtin_bit_cast(float, pg_dpp8<0xB1>(__builtin_bit_cast(int, amax))));
+    bad |= pg_dpp8<0xB1>(bad);
+    amax = fmaxf(amax, __builtin_bit_cast(float, pg_dpp8<0x4E>(__builtin_bit_cast(int, amax))));
+    bad |= pg_dpp8<0x4E>(bad);
+    amax = fmaxf(amax, __builtin_bit_cast(float, pg_dpp8<0x141>(__builtin_bit_cast(int, amax))));
+    bad |= pg_dpp8<0x141>(bad);
+    int se = 0;
+    float inv = 1.0f;
+    if (bad || !(amax <= 3.4028234663852886e38f)) {
+        bad = 1;
+        inv = 0.0f;
+    } else if (amax > 0.0f) {
+        int ex;
+        (void)frexpf(amax, &ex);  // amax = f * 2^ex, f in [0.5, 1)
+        se = ex - 23;             // |x| / 2^se < 2^23
+        if (se < -126) se = -126;
+        inv = ldexpf(1.0f, -se);
+    }
+    // Balanced base-32 digits, top down and all in f32 (every value is a small integer times a power of two,
+    // so each step is exact): n_j = round(r / 32^j), r -= n_j 32^j; |n_j| <= 16.
+    float r[4], d[MX_PLANES][4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float t = f[e] * inv;
+        r[e] = (t != t) ? 0.0f : rintf(t);
+    }
+#pragma unroll
+    for (int j = MX_PLANES - 1; j >= 1; --j) {
+        const float down = __builtin_bit_cast(float, (127 - 5 * j) << 23), up = -__builtin_bit_cast(float, (127 + 5 * j) << 23);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            d[j][e] = rintf(r[e] * down);
+            r[e] = fmaf(d[j][e], up, r[e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) d[0][e] = r[e];
+#pragma unroll
+    for (int j = 0; j < MX_PLANES; ++j) {  // integers in [-16, 16] are exact in E4M3: the conversion's rounding never acts
+        int packed = __builtin_amdgcn_cvt_pk_fp8_f32(d[j][0], d[j][1], 0, false);
+        packed = __builtin_amdgcn_cvt_pk_fp8_f32(d[j][2], d[j][3], packed, true);
+        *reinterpret_cast<int *>(dig + (size_t)j * stride + b * 32 + 4 * sub) = packed;
+    }
+    if (sub < MX_PLANES)  // a NaN / inf block poisons every product it enters: scale byte 255 is NaN
+        sb[(sub * 4 + (b & 3)) * ncp + (b >> 2)] = (uint8_t)(bad ? 255 : 127 + se + 5 * sub);
+}
+
+// ---- the product ----------------------------------------------------------------------
+// A workgroup of NW wavefronts = RG groups of 16 weight rows x KS = NW / RG slices of K, against T
+// activation rows (blockIdx.y picks which); it first rewrites those rows (all of K) as digit planes in
+// LDS while its first weight loads are in flight.  Each wavefront then walks its K slice in batches of
+// MX_U chunks, the next batch requested before the current one is consumed, and the partial tiles of
+// the KS slices and the 5 planes are added through LDS in a fixed order.
+template <int T, int RG, int NW>
+__global__ __launch_bounds__(64 * NW) void mxfp4_rows_kernel(const uint8_t *__restrict__ qs_frag, const uint32_t *__restrict__ sc_frag,
+                                                                  const float *__restrict__ x, float *__restrict__ y,
+                                                                  int n_out, int nb, int ncp, int m) {
+    constexpr int KS = NW / RG, COLS = MX_PLANES * T;
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int kp = ncp * 128, stride = kp + 64;  // plane stride: not a multiple of the LDS bank span
+    char *const dig = lds;
+    uint8_t *const sb = reinterpret_cast<uint8_t *>(lds + (size_t)COLS * stride);
+    float *const part = reinterpret_cast<float *>(lds + (size_t)COLS * stride + (((size_t)COLS * 4 * ncp + 15) & ~(size_t)15));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int rgi = wave / KS, ksi = wave % KS;
+    const int nrg = (n_out + 15) / 16;
+    int rg = blockIdx.x * RG + rgi;
+    rg = rg < nrg ? rg : nrg - 1;  // a spare wavefront repeats the last group; its result is not stored
+    const int cps = ((ncp + KS - 1) / KS + 3) & ~3;  // chunks per K slice, whole scale dwords
+    const int c0 = ksi * cps, c1 = (c0 + cps < ncp) ? c0 + cps : ncp;
+    const gv4i_ptr qa = (gv4i_ptr)(uintptr_t)qs_frag + (size_t)rg * ncp * 64 + lane;
+    const uint32_t *__restrict__ sa = sc_frag + (size_t)rg * (ncp / 4) * 64 + lane;
+
+    v4i abuf[2][MX_U];
+    uint32_t sabuf[2][MX_U / 4];
+    auto load_batch = [&](v4i (&a)[MX_U], uint32_t (&s)[MX_U / 4], int cb) {
+#pragma unroll
+        for (int u = 0; u < MX_U; ++u) {
+            const int c = cb + u;
+            a[u] = __builtin_nontemporal_load(qa + (size_t)(c < ncp ? c : ncp - 1) * 64);
+        }
+#pragma unroll
+        for (int g = 0; g < MX_U / 4; ++g) {
+            const int c = cb + 4 * g;
+            s[g] = sa[(size_t)((c < ncp ? c : ncp - 4) >> 2) * 64];
+        }
+    };
+    // Loads return in issue order: the activation blocks of the first rounds (from L2) are requested
+    // before the weights (from HBM), so that the digit arithmetic runs while the weights are in flight.
+    const int sub = threadIdx.x & 7, nblk = 4 * ncp;
+    // (No branch around a load: behind one the compiler waits for every load in flight, the weights too.
+    // Block ids past the end load the last block again.)
+    const int last = T * nblk - 1;
+    auto row_of = [&](int id) { return T == 1 ? 0 : (id >= nblk) + (T > 2 && id >= 2 * nblk); };  // id / nblk
+    auto x_valid = [&](int id) {
+        const int t = row_of(id), b = id - t * nblk;
+        return b < nb && (size_t)blockIdx.y * T + t < (size_t)m;  // blocks nb .. 4 ncp - 1 and rows past m are zeros
+    };
+    auto load_x = [&](int id) {
+        const int t = row_of(id), b = id - t * nblk;
+        const size_t at = x_valid(id) ? (((size_t)blockIdx.y * T + t) * nb + b) * 8 + sub : 0;
+        return reinterpret_cast<const float4 *>(x)[at];
+    };
+    auto emit = [&](int id, const float4 v) {
+        const int t = row_of(id), b = id - t * nblk;
+        const bool keep = x_valid(id);
+        const float f[4] = {keep ? v.x : 0.0f, keep ? v.y : 0.0f, keep ? v.z : 0.0f, keep ? v.w : 0.0f};
+        mx_emit_digits(f, b, sub, dig + (size_t)t * MX_PLANES * stride, stride, sb + (size_t)t * MX_PLANES * 4 * ncp, ncp);
+    };
+    constexpr int PER_ROUND = 8 * NW;  // blocks per round: 8 threads each
+    constexpr int NPRE = 4;                  // rounds whose activation blocks are requested ahead of the weights
+    const int g0 = threadIdx.x >> 3;
+    float4 xv[NPRE];
+#pragma unroll
+    for (int r = 0; r < NPRE; ++r) {
+        const int id = g0 + r * PER_ROUND;
+        xv[r] = load_x(id < last ? id : last);
+    }
+    asm volatile("" ::: "memory");  // (keeps the compiler from moving these loads down to their uses)
+    __builtin_amdgcn_sched_barrier(0);
+    load_batch(abuf[0], sabuf[0], c0 < ncp ? c0 : 0);  // (an empty slice consumes nothing)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < NPRE; ++r) {
+        const int id = g0 + r * PER_ROUND;
+        if (id <= last) emit(id, xv[r]);  // whole 8-thread groups together
+    }
+    for (int id = g0 + NPRE * PER_ROUND; id <= last; id += PER_ROUND) emit(id, load_x(id));
+    asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier" ::: "memory");  // (not __syncthreads(): the weight loads stay in flight)
+
+    // B side of this lane: column min(lane % 16, COLS - 1) (the spare columns repeat the last one and are dropped)
+    const int col = (lane & 15) < COLS ? (lane & 15) : COLS - 1, q = lane >> 4;
+    const char *const bcol = dig + (size_t)col * stride + 16 * q;
+    const uint8_t *const sbl = sb + (size_t)(col * 4 + q) * ncp;
+    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto consume = [&](const v4i (&a)[MX_U], const uint32_t (&s)[MX_U / 4], int cb) {
+#pragma unroll
+        for (int g = 0; g < MX_U / 4; ++g) {
+            if (cb + 4 * g < c1) {  // the same for the whole wavefront
+                const int sbv = *reinterpret_cast<const int *>(sbl + cb + 4 * g);
+                const char *bp = bcol + (size_t)(cb + 4 * g) * 128;
+                // (the byte selectors of the two scale operands are immediates)
+#define PG_MX_STEP(U)                                                                                                   \
+    do {                                                                                                                \
+        const v4i b0 = *reinterpret_cast<const v4i *>(bp + (U) * 128), b1 = *reinterpret_cast<const v4i *>(bp + (U) * 128 + 64); \
+        const v4i aw = a[4 * g + (U)];                                                                                  \
+        const v8i A = {aw[0], aw[1], aw[2], aw[3], 0, 0, 0, 0};                                                         \
+        const v8i B = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};                                         \
+        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, acc, 4, 0, (U), (int)s[g], (U), sbv);              \
+    } while (0)
+                PG_MX_STEP(0);
+                PG_MX_STEP(1);
+                PG_MX_STEP(2);
+                PG_MX_STEP(3);
+#undef PG_MX_STEP
+            }
+        }
+    };
+    for (int cb = c0; cb < c1; cb += 2 * MX_U) {
+        if (cb + MX_U < c1) load_batch(abuf[1], sabuf[1], cb + MX_U);
+        __builtin_amdgcn_sched_barrier(0);
+        consume(abuf[0], sabuf[0], cb);
+        if (cb + 2 * MX_U < c1) load_batch(abuf[0], sabuf[0], cb + 2 * MX_U);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cb + MX_U < c1) consume(abuf[1], sabuf[1], cb + MX_U);
+    }
+
+    // part[wave][lane][r]: column lane % 16, row 4 (lane / 16) + r of this wavefront's tile
+    *reinterpret_cast<v4f *>(part + ((size_t)wave * 64 + lane) * 4) = acc;
+    __syncthreads();
+    if (threadIdx.x < RG * 16 * T) {
+        const int t = threadIdx.x / (RG * 16), rr = threadIdx.x % (RG * 16), g = rr / 16, i = rr % 16;
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = MX_PLANES - 1; j >= 0; --j)
+#pragma unroll
+            for (int k = 0; k < KS; ++k)
+                sum += part[((size_t)(g * KS + k) * 64 + 16 * (i >> 2) + t * MX_PLANES + j) * 4 + (i & 3)];
+        const size_t row = ((size_t)blockIdx.x * RG + g) * 16 + i, item = (size_t)blockIdx.y * T + t;
+        if (row < (size_t)n_out && item < (size_t)m) y[item * n_out + row] = sum;
+    }
+}
+
+size_t mx_lds_bytes(int t, int ncp, int nw = 16) {
+    const size_t cols = (size_t)MX_PLANES * t;
+    return cols * ((size_t)ncp * 128 + 64) + ((cols * 4 * ncp + 15) & ~(size_t)15) + (size_t)nw * 64 * 4 * sizeof(float);
+}
+
+template <int T, int RG, int NW>
+pg_status launch_rows(pg_ctx *ctx, const pg_gguf_tensor *w, const float *x, float *y, size_t m, int ncp) {
+    const size_t lds = mx_lds_bytes(T, ncp, NW);
+    auto kern = mxfp4_rows_kernel<T, RG, NW>;
+    PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
+    const dim3 grid(grid_for((w->n_out + 15) / 16, RG), grid_for(m, T));
+    return pg_launch(ctx, "mxfp4_rows", kern, grid, dim3(64 * NW), lds, (const uint8_t *)w->qs,
+                     reinterpret_cast<const uint32_t *>(w->d), x, y, (int)w->n_out, (int)(w->k_in / 32), ncp, (int)m);
+}
+
+}  // namespace
+
+// y[m, n_out] = x[m, k_in] . W^T for an MXFP4 tensor; x 16-byte aligned.
+pg_status pg_launch_mxfp4_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w, float *y_dev) {
+    if (m == 0) return PG_OK;
+    const int nb = (int)(w->k_in / 32), ncp = (int)mx_chunks((size_t)nb);
+    int t = m < (size_t)MX_MAX_T ? (int)m : MX_MAX_T;
+    while (t > 1 && mx_lds_bytes(t, ncp) > (96u << 10)) --t;  // room for a second workgroup per CU
+    if (mx_lds_bytes(t, ncp) > (160u << 10))
+        return pg_fail(PG_EUNSUPPORTED, "mxfp4: k_in %zu does not fit the digit planes in LDS (up to 28160)", w->k_in);
+    if ((m + t - 1) / t > 65535) return pg_fail(PG_EUNSUPPORTED, "mxfp4: more than %d activation rows", 65535 * t);
+    // Every workgroup rewrites the activation rows as digits, so the fewer workgroups the less of that work.
+    // Up to one group of 16 weight rows per CU: 16 wavefronts on it, K in 16 slices.  Beyond: 8 wavefronts
+    // with the fewest row groups per workgroup (1, 2 or 4; K in 8, 4 or 2 slices) with which all
+    // workgroups are resident at once (two per CU), four past that.
+    const size_t groups = (w->n_out + 15) / 16 * ((m + t - 1) / t), slots = (size_t)ctx->num_cu * 2;
+    const int shape = groups <= (size_t)ctx->num_cu ? 0 : (groups <= slots ? 1 : ((groups + 1) / 2 <= slots ? 2 : 4));
+#define PG_MX_LAUNCH(TT)                                                                                              \
+    (shape == 0 ? launch_rows<TT, 1, 16>(ctx, w, x_dev, y_dev, m, ncp)                                                \
+     : shape == 1 ? launch_rows<TT, 1, 8>(ctx, w, x_dev, y_dev, m, ncp)                                               \
+     : shape == 2 ? launch_rows<TT, 2, 8>(ctx, w, x_dev, y_dev, m, ncp) : launch_rows<TT, 4, 8>(ctx, w, x_dev, y_dev, m, ncp))
+    switch (t) {
+        case 1: return PG_MX_LAUNCH(1);
+        case 2: return PG_MX_LAUNCH(2);
+        default: return PG_MX_LAUNCH(3);
+    }
+#undef PG_MX_LAUNCH
+}
+
+// ---- ABI --------------------------------------------------------------------------------
+// A block is 16 bytes of FP4 (E2M1) codes, byte k = elements 2k (low nibble) and 2k+1, plus
+// one E8M0 scale byte: value = LUT[code] * 2^(scale - 127)   (examples/gpt_oss/moe.rs:5-53).
+PG_API pg_status pg_mxfp4_upload(pg_ctx *ctx, const uint8_t *blocks, const uint8_t *scales, size_t out_dim,
+                                 size_t in_dim, pg_gguf_tensor **out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(out != nullptr, "pg_mxfp4_upload: out is null");
+    *out = nullptr;
+    PG_CHECK_ARG(out_dim > 0 && in_dim > 0 && blocks && scales, "pg_mxfp4_upload: empty tensor or null pointer");
+    PG_CHECK_ARG(in_dim % 32 == 0, "pg_mxfp4_upload: in_dim %zu is not a multiple of 32", in_dim);
+    PG_CHECK_ARG(out_dim < (1ull << 31) && in_dim < (1ull << 31) && out_dim * (in_dim / 32) < (1ull << 31),
+                 "pg_mxfp4_upload: shape too large");
+    const size_t nb = in_dim / 32, nblocks = out_dim * nb;
+    const size_t ncp = mx_chunks(nb), nrg = (out_dim + 15) / 16;
+    pg_gguf_tensor *t = new (std::nothrow) pg_gguf_tensor();
+    if (!t) return pg_fail(PG_ENOMEM, "host allocation failed");
+    t->qs = nullptr;
+    t->d = nullptr;
+    t->m = nullptr;
+    t->qs_tiled = nullptr;
+    t->ggml_type = PG_MXFP4;
+    t->n_out = out_dim;
+    t->k_in = in_dim;
+    pg_tmp rb, rs;
+    pg_status st = rb.alloc(nblocks * 16);
+    if (st == PG_OK) st = rs.alloc(nblocks);
+    hipError_t e = hipSuccess;
+    if (st == PG_OK) {
+        e = hipMalloc((void **)&t->qs, nrg * ncp * 64 * 16);
+        if (e == hipSuccess) e = hipMalloc((void **)&t->d, nrg * (ncp / 4) * 64 * 4);
+        if (e == hipSuccess) e = hipMemcpyAsync(rb.p, blocks, nblocks * 16, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipMemcpyAsync(rs.p, scales, nblocks, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) {
+            mxfp4_fragments_kernel<<<grid_for(nrg * ncp * 64, 256), 256, 0, ctx->stream>>>(
+                rb.as<uint8_t>(), rs.as<uint8_t>(), (int)out_dim, (int)nb, (int)ncp, reinterpret_cast<uint4 *>(t->qs),
+                reinterpret_cast<uint8_t *>(t->d));
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess)
+            st = pg_fail(e == hipErrorOutOfMemory ? PG_ENOMEM : PG_EDEVICE, "pg_mxfp4_upload: %s", hipGetErrorString(e));
+    }
+    if (st != PG_OK) { pg_gguf_free(ctx, t); return st; }
+    *out = t;
+    return PG_OK;
+}
+
+PG_API pg_status pg_mxfp4_matmul(pg_ctx *ctx, const float *input, const uint8_t *blocks, const uint8_t *scales,
+                                 size_t out_dim, size_t in_dim, float *output) {
+    pg_gguf_tensor *t = nullptr;
+    PG_TRY(pg_mxfp4_upload(ctx, blocks, scales, out_dim, in_dim, &t));
+    const pg_status st = pg_gguf_matmul(ctx, input, 1, t, output);
+    pg_gguf_free(ctx, t);
+    return st;
+}
+
+// Mxfp4Expert  examples/gpt_oss/moe.rs:55-117, swiglu :145-154.
+struct pg_mxfp4_expert {
+    pg_gguf_tensor *mlp1, *mlp2;  // [2 * intermediate, hidden], [hidden, intermediate]
+    float *bias1, *bias2;         // [2 * intermediate], [hidden] (one allocation)
+    size_t hidden, intermediate;
+    float alpha, clamp;
+};
+
+namespace {
+// biased = h + bias1; gate = biased[2i].min(clamp); linear = biased[2i+1].clamp(-clamp, clamp);
+// out[i] = gate * (1 / (1 + exp(-alpha * gate))) * (linear + 1)
+__global__ __launch_bounds__(256) void mxfp4_bias_swiglu_kernel(const float *__restrict__ h, const float *__restrict__ bias,
+                                                                size_t rows, size_t inter, float alpha, float clamp,
+                                                                float *__restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * inter) return;
+    const size_t r = i / inter, c = i - r * inter;
+    const float g0 = h[r * 2 * inter + 2 * c] + bias[2 * c], l0 = h[r * 2 * inter + 2 * c + 1] + bias[2 * c + 1];
+    const float gate = fminf(g0, clamp);                                     // f32::min: a NaN operand loses
+    const float linear = l0 != l0 ? l0 : fminf(fmaxf(l0, -clamp), clamp);    // f32::clamp keeps NaN
+    const float activated = gate * (1.0f / (1.0f + expf(-alpha * gate)));
+    out[i] = activated * (linear + 1.0f);
+}
+
+__global__ __launch_bounds__(256) void bias_add_kernel(const float *__restrict__ a, const float *__restrict__ bias,
+                                                       size_t rows, size_t cols, float *__restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < rows * cols) out[i] = a[i] + bias[i % cols];
+}
+}  // namespace
+
+PG_API void pg_mxfp4_expert_free(pg_ctx *ctx, pg_mxfp4_expert *e) {
+    if (!e) return;
+    if (ctx) {
+        (void)pg_use(ctx);
+        (void)hipStreamSynchronize(ctx->stream);
+    }
+    pg_gguf_free(ctx, e->mlp1);
+    pg_gguf_free(ctx, e->mlp2);
+    if (e->bias1) (void)hipFree(e->bias1);
+    delete e;
+}
+
+PG_API pg_status pg_mxfp4_expert_create(pg_ctx *ctx, size_t hidden, size_t intermediate, float alpha, float clamp,
+                                        const uint8_t *mlp1_blocks, const uint8_t *mlp1_scales,
+                                        const uint8_t *mlp2_blocks, const uint8_t *mlp2_scales, const float *mlp1_bias,
+                                        const float *mlp2_bias, pg_mxfp4_expert **out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(out != nullptr, "pg_mxfp4_expert_create: out is null");
+    *out = nullptr;
+    PG_CHECK_ARG(mlp1_bias && mlp2_bias, "pg_mxfp4_expert_create: null bias");
+    pg_mxfp4_expert *e = new (std::nothrow) pg_mxfp4_expert{nullptr, nullptr, nullptr, nullptr, hidden, intermediate, alpha, clamp};
+    if (!e) return pg_fail(PG_ENOMEM, "host allocation failed");
+    pg_status st = pg_mxfp4_upload(ctx, mlp1_blocks, mlp1_scales, 2 * intermediate, hidden, &e->mlp1);
+    if (st == PG_OK) st = pg_mxfp4_upload(ctx, mlp2_blocks, mlp2_scales, hidden, intermediate, &e->mlp2);
+    if (st == PG_OK) {
+        hipError_t he = hipMalloc((void **)&e->bias1, (2 * intermediate + hidden) * sizeof(float));
+        if (he == hipSuccess) {
+            e->bias2 = e->bias1 + 2 * intermediate;
+            he = hipMemcpyAsync(e->bias1, mlp1_bias, 2 * intermediate * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
+        }
+        if (he == hipSuccess) he = hipMemcpyAsync(e->bias2, mlp2_bias, hidden * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
+        if (he == hipSuccess) he = hipStreamSynchronize(ctx->stream);
+        if (he != hipSuccess)
+            st = pg_fail(he == hipErrorOutOfMemory ? PG_ENOMEM : PG_EDEVICE, "pg_mxfp4_expert_create: %s", hipGetErrorString(he));
+    }
+    if (st != PG_OK) { pg_mxfp4_expert_free(ctx, e); return st; }
+    *out = e;
+    return PG_OK;
+}
+
+// scratch_dev: [m, 3 * intermediate] floats (the mlp1 output, then the activated rows).
+PG_API pg_status pg_mxfp4_expert_forward_dev(pg_ctx *ctx, const pg_mxfp4_expert *e, const float *x_dev, size_t m,
+                                             float *scratch_dev, float *out_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(e != nullptr, "pg_mxfp4_expert_forward: null expert");
+    if (m == 0) return PG_OK;
+    PG_CHECK_ARG(x_dev && scratch_dev && out_dev, "pg_mxfp4_expert_forward: null pointer");
+    PG_CHECK_ARG((uintptr_t)x_dev % 16 == 0 && (uintptr_t)scratch_dev % 16 == 0,
+                 "pg_mxfp4_expert_forward: x and scratch must be 16-byte aligned");
+    PG_CHECK_ARG(m <= 65535, "pg_mxfp4_expert_forward: more than 65535 rows");
+    const size_t inter = e->intermediate, hid = e->hidden;
+    float *h = scratch_dev, *act = scratch_dev + m * 2 * inter;
+    PG_TRY(pg_gguf_matmul_rows(ctx, x_dev, m, e->mlp1, h));
+    PG_TRY(pg_launch(ctx, "mxfp4_bias_swiglu", mxfp4_bias_swiglu_kernel, dim3(grid_for(m * inter, 256)), dim3(256), 0,
+                     (const float *)h, (const float *)e->bias1, m, inter, e->alpha, e->clamp, act));
+    PG_TRY(pg_gguf_matmul_rows(ctx, act, m, e->mlp2, out_dev));
+    return pg_launch(ctx, "bias_add", bias_add_kernel, dim3(grid_for(m * hid, 256)), dim3(256), 0, (const float *)out_dev,
+                     (const float *)e->bias2, m, hid, out_dev);
+}
+
+PG_API pg_status pg_mxfp4_expert_forward(pg_ctx *ctx, const pg_mxfp4_expert *e, const float *x, size_t m, float *out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(e != nullptr, "pg_mxfp4_expert_forward: null expert");
+    if (m == 0) return PG_OK;
+    PG_CHECK_ARG(x && out, "pg_mxfp4_expert_forward: null pointer");
+    pg_tmp dx, ds, dout;
+    PG_TRY(dx.alloc(m * e->hidden * sizeof(float)));
+    PG_TRY(ds.alloc(m * 3 * e->intermediate * sizeof(float)));
+    PG_TRY(dout.alloc(m * e->hidden * sizeof(float)));
+    PG_HIP(hipMemcpyAsync(dx.p, x, m * e->hidden * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_mxfp4_expert_forward_dev(ctx, e, dx.as<float>(), m, ds.as<float>(), dout.as<float>()));
+    PG_HIP(hipMemcpyAsync(out, dout.p, m * e->hidden * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}
+

@@ -95,3 +95,54 @@ def test_mxfp4_expert_forward(ctx, orc, m):
         want = orc.mxfp4_expert_forward(x[i], hidden, inter, alpha, clamp, b1, s1, b2, s2, bias1, bias2)
         H.assert_close_rel(got[i], want, RTOL_CONTRACT, f"mxfp4 expert row {i}")
         H.assert_close_rel(got[i], want, 1e-4, f"mxfp4 expert row {i} (achieved)")
+
+
+@pytest.mark.parametrize("out_dim,in_dim,m", [(4096, 14336, 1), (14336, 4096, 2), (600, 512, 5), (48, 28160, 1), (8200, 1024, 3)])
+def test_mxfp4_workgroup_shapes(ctx, orc, out_dim, in_dim, m):
+    """One case per launch shape of the product kernel: 16 wavefronts on one row group (few row groups),
+    8 wavefronts on 1, 2 or 4 row groups, one to three activation rows per pass, several passes (m = 5),
+    and K at the upper limit of what the digit planes in LDS hold."""
+    from peregrine_amd import mxfp4
+    say(f"mxfp4 shapes [{m} x {in_dim}] -> [{out_dim}]")
+    rng = np.random.default_rng(out_dim * 7 + in_dim + m)
+    b, s = _weights(rng, out_dim, in_dim)
+    w = mxfp4.upload(b, s, out_dim, in_dim, ctx)
+    x = orc.rng_normal(m + 11, m * in_dim).reshape(m, in_dim)
+    x[:, ::89] *= 30.0
+    got = w.matmul(x, m).reshape(m, out_dim)
+    rows = rng.choice(out_dim, size=min(out_dim, 256), replace=False)   # the oracle on a sample of the weight rows
+    bb = b.reshape(out_dim, -1)[rows].reshape(-1)
+    ss = s.reshape(out_dim, -1)[rows].reshape(-1)
+    for i in range(m):
+        want = orc.mxfp4_matmul(x[i], bb, ss, len(rows), in_dim)
+        H.assert_close_rel(got[i][rows], want, RTOL_ACHIEVED, f"row {i}")
+    w.free()
+
+
+def test_mxfp4_limits_and_non_finite(ctx, orc):
+    from peregrine_amd import mxfp4, _ffi
+    rng = np.random.default_rng(9)
+    b, s = _weights(rng, 16, 28672)
+    with pytest.raises(_ffi.PeregrineError):   # the row's digit planes no longer fit in LDS
+        mxfp4.mxfp4_matmul(np.zeros(28672, np.float32), b, s, 16, 28672, ctx)
+    out_dim, in_dim = 40, 128
+    b, s = _weights(rng, out_dim, in_dim)
+    x = orc.rng_normal(1, in_dim)
+    base = mxfp4.mxfp4_matmul(x, b, s, out_dim, in_dim, ctx)
+    assert np.isfinite(base).all()
+    for bad in (np.nan, np.inf, -np.inf):       # the reference's f32 sum turns inf or NaN in every row as well
+        xb = x.copy()
+        xb[37] = bad
+        got = mxfp4.mxfp4_matmul(xb, b, s, out_dim, in_dim, ctx)
+        want = orc.mxfp4_matmul(xb, b, s, out_dim, in_dim)
+        assert not np.isfinite(got).any() and not np.isfinite(want).any()
+    s2 = s.copy().reshape(out_dim, -1)
+    s2[3, 1] = 255                              # f32::from_bits(255 << 23) = inf: that row is lost, the others are not
+    got = mxfp4.mxfp4_matmul(x, b, s2.reshape(-1), out_dim, in_dim, ctx)
+    assert not np.isfinite(got[3]) and not np.isfinite(orc.mxfp4_matmul(x, b, s2.reshape(-1), out_dim, in_dim)[3])
+    keep = np.arange(out_dim) != 3
+    assert (got[keep] == base[keep]).all()
+    s3 = s.copy().reshape(out_dim, -1)
+    s3[5, :] = 0                                # f32::from_bits(0) = 0.0: the row is exactly zero
+    got = mxfp4.mxfp4_matmul(x, b, s3.reshape(-1), out_dim, in_dim, ctx)
+    assert got[5] == 0.0 and orc.mxfp4_matmul(x, b, s3.reshape(-1), out_dim, in_dim)[5] == 0.0
