@@ -238,7 +238,10 @@ pg_status pg_gguf_matmul_dev(pg_ctx *ctx, const float *x_dev, size_t m,
 /* mxfp4_matmul  examples/gpt_oss/moe.rs:16-53: weight [out_dim, in_dim] as 16-byte blocks of
  * FP4 codes (byte k = elements 2k low nibble, 2k+1 high) in `blocks` [out_dim * in_dim/32 * 16]
  * and one E8M0 scale byte per block in `scales` [out_dim * in_dim/32];
- * output[r] = sum_b ( sum_k LUT[code] * input[32b + k] ) * 2^(scale - 127). */
+ * output[r] = sum_b ( sum_k LUT[code] * input[32b + k] ) * 2^(scale - 127).
+ * in_dim is a multiple of 32, at most 28160 (a row's fixed-point planes live in on-chip memory; larger:
+ * PG_EUNSUPPORTED).  Scale byte 0 is the reference's f32::from_bits(0) = 0.0; scale byte 255 (inf there)
+ * makes the row's result NaN, as does an inf or NaN anywhere in the input. */
 pg_status pg_mxfp4_matmul(pg_ctx *ctx, const float *input, const uint8_t *blocks, const uint8_t *scales,
                           size_t out_dim, size_t in_dim, float *output);
 /* The same weight kept on the device: a pg_gguf_tensor (type PG_MXFP4) for pg_gguf_matmul(_dev),
