@@ -185,7 +185,12 @@ class Bench:
         self.check(self.lib.pg_probe_mfma_i8(self.h, 20000, C.byref(tops), C.byref(ghz)))
         self.check(self.lib.pg_probe_hbm_read(self.h, 256 << 20, 3, 30, C.byref(gbs)))
         self.check(self.lib.pg_probe_gemm_clock(self.h, 2048, 4096, 14336, C.byref(g_ghz), C.byref(loop_us)))
-        return {"int8_mfma_registers_only_tops": round(tops.value, 1), "its_shader_clock_ghz": round(ghz.value, 3),
+        small = {}
+        for label, nbytes, bufs in (("33MB", 33103872, 10), ("59MB", 58851328, 6)):  # cfg4's and cfg2's largest launches
+            g = C.c_double()
+            self.check(self.lib.pg_probe_hbm_read(self.h, nbytes, bufs, 300, C.byref(g)))
+            small[label] = round(g.value, 1)
+        return {"hbm_read_stream_per_launch_size_gbs": small,"int8_mfma_registers_only_tops": round(tops.value, 1), "its_shader_clock_ghz": round(ghz.value, 3),
                 "hbm_read_stream_gbs": round(gbs.value, 1), "gemm_tile_shader_clock_ghz": round(g_ghz.value, 3),
                 "gemm_tile_k_loop_us": round(loop_us.value, 2),
                 "int8_peak_at_gemm_clock_tops": round(256 * 8192 * g_ghz.value / 1e3, 1),
