@@ -598,6 +598,262 @@ __global__ __launch_bounds__(256) void gqa_attention_tiled_kernel(attn_args aa) 
     }
 }
 
+// ---- many query rows on the matrix cores -------------------------------------------------------
+// v_mfma_f32_32x32x2_f32 runs f32 multiply-adds at twice the rate the vector unit reaches without
+// packed operations, and keeps its 32x32 tile in registers.  A wavefront owns 32 query rows of
+// one kv head (row index = token * group + head in group, as above) and walks the keys 32 at a
+// time, with both products transposed so that nothing has to change lanes in between:
+//   S^T[key][row] = sum_d K[key][d] Q[row][d]     A = K tile (lane: key, half h), B = Q (lane: row, h)
+//   O^T[d][row]  += sum_key V[key][d] P^T[key][row]   A = V tile, B = the probabilities
+// The tile a lane holds after the first product (column = row l%32, register r = key
+// 8(r/4) + 4h + r%4) is exactly a B operand of the second, register by register: summation
+// indices may be visited in any order, so step j of the second product takes key 8(j/4) + 4h + j%4
+// from half h, and the V operand is loaded in that order.  The same freedom makes every load
+// 128 bits wide: step 4i+c of the first product takes d = 8i + 4h + c, and output row i of d-tile
+// dt stands for d = (HD/32) i + dt.  K, V and Q go from L2 straight into operand registers; no LDS,
+// no barrier inside the key loop.  Softmax is online per column; a column's two halves exchange
+// only their maxima (lane ^ 32), the sums are joined at the end.
+// Causal work is uneven (row block i sees i + 1 key tiles), so a workgroup of two wavefronts takes
+// the pair (i, n - 1 - i) and cuts the pair's tiles in two equal parts: wavefront 0 the first part
+// of the long item, wavefront 1 the short item and the rest of the long one, whose partial
+// (maximum, sum, rows) it hands over through LDS.
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+template <int HD>
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gqa_attention_mfma_kernel(attn_args aa, int n_items, int nkvh) {
+    constexpr int NDT = HD / 32, QR = HD / 2;
+    typedef float vdt __attribute__((ext_vector_type(NDT)));
+    __shared__ float part_l[(NDT * 16 + 2) * 64];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int col = lane & 31, h = lane >> 5;
+    const int kvh = blockIdx.x % nkvh, pair = blockIdx.x / nkvh;
+    const int G = aa.group, nrows = G * aa.seq_q;
+    const int item_a = pair, item_b = n_items - 1 - pair;  // the short and the long one (equal: one item)
+    auto kend_of = [&](int item) {
+        const int last_qt = min(item * 32 + 31, nrows - 1) / G;
+        return aa.mask_kind != 0 ? min(aa.len, aa.offset + last_qt + 1) : aa.len;
+    };
+    const int tb = (kend_of(item_b) + 31) / 32, ta = item_a != item_b ? (kend_of(item_a) + 31) / 32 : 0;
+    const int cut = min(tb, (ta + tb + 1) / 2);
+    const float *kg = aa.kc + (size_t)kvh * aa.k_stride, *vg = aa.vc + (size_t)kvh * aa.v_stride;
+
+    float m = -INFINITY, l = 0.f;
+    v16f o[NDT];
+    int row = 0, qt = 0, qh = 0;
+    for (int seg = 0; seg < 2; ++seg) {
+        // wavefront 0: (long item, tiles [0, cut)), nothing; wavefront 1: (short item, all), (long item, [cut, tb))
+        const int item = (wave == 0 || seg == 1) ? item_b : item_a;
+        const int t0 = wave == 0 ? 0 : (seg == 0 ? 0 : cut);
+        const int t1 = wave == 0 ? (seg == 0 ? cut : 0) : (seg == 0 ? ta : tb);
+        if (t1 <= t0) continue;
+        const int kend = kend_of(item);
+        row = item * 32 + col;
+        const int rowc = min(row, nrows - 1);
+        qt = rowc / G;
+        qh = kvh * G + rowc % G;
+        const int qt_min = (item * 32) / G;
+        m = -INFINITY;
+        l = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
+        float qreg[QR];
+        {
+            const float *qp = aa.q + ((size_t)qh * aa.seq_q + qt) * HD + 4 * h;
+#pragma unroll
+            for (int i = 0; i < HD / 8; ++i) {
+                const float4 v = *reinterpret_cast<const float4 *>(qp + 8 * i);
+                qreg[4 * i] = v.x; qreg[4 * i + 1] = v.y; qreg[4 * i + 2] = v.z; qreg[4 * i + 3] = v.w;
+            }
+        }
+        float4 kreg[HD / 8];
+        vdt vreg[16];
+        auto load_k = [&](int t) {
+            const float *kp = kg + (size_t)min(32 * t + col, kend - 1) * HD + 4 * h;
+#pragma unroll
+            for (int i = 0; i < HD / 8; ++i) kreg[i] = *reinterpret_cast<const float4 *>(kp + 8 * i);
+        };
+        auto load_v = [&](int t) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int key = min(32 * t + 8 * (j >> 2) + 4 * h + (j & 3), kend - 1);
+                vreg[j] = *reinterpret_cast<const vdt *>(vg + (size_t)key * HD + NDT * col);
+            }
+        };
+        auto scores = [&](v16f &s) {  // S^T of the tile in kreg
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+            for (int i = 0; i < HD / 8; ++i) {
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[i].x, qreg[4 * i], s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[i].y, qreg[4 * i + 1], s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[i].z, qreg[4 * i + 2], s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[i].w, qreg[4 * i + 3], s, 0, 0, 0);
+            }
+        };
+        // scale, cap and mask the raw scores of tile t (the branches are wavefront-uniform and kept out of
+        // the straight-line part below, which the scheduler interleaves with the next tile's products)
+        auto finish_scores = [&](v16f &s, int t) {
+            const int k0 = 32 * t;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[r] *= aa.scale;
+            if (aa.logit_cap > 0.f) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[r] = aa.logit_cap * tanhf(s[r] / aa.logit_cap);
+            }
+            const bool all_visible = k0 + 31 < kend && (aa.mask_kind == 0 || (aa.mask_kind == 1 && k0 + 31 <= aa.offset + qt_min));
+            if (!all_visible) {
+                // attn_masked() as plain bit arithmetic (selects, no lane-dependent branches); a tile's 32 keys
+                // share one word of the global-position bits
+                const int mk = aa.mask_kind, qp = aa.offset + qt;
+                const uint32_t gw = mk == 3 ? aa.gbits[t] : 0u;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int kin = 8 * (r >> 2) + 4 * h + (r & 3), key = k0 + kin;
+                    const bool far = qp - key > aa.window;
+                    const bool hide = (key >= kend) | ((mk != 0) & (key > qp)) | ((mk == 2) & (key >= aa.sink) & far) |
+                                      ((mk == 3) & far & !((gw >> kin) & 1u));
+                    s[r] = hide ? -INFINITY : s[r];
+                }
+            }
+        };
+        // online softmax of this lane's column (16 of its 32 keys here, the rest in lane ^ 32): s becomes p
+        auto softmax = [&](v16f &s) {
+            float mt = s[0];
+#pragma unroll
+            for (int r = 1; r < 16; ++r) mt = fmaxf(mt, s[r]);
+            mt = fmaxf(mt, __shfl_xor(mt, 32));
+            const float m_new = fmaxf(m, mt);
+            const float alpha = m == -INFINITY ? 1.0f : expf(m - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float p = s[r] == -INFINITY ? 0.f : expf(s[r] - m_new);
+                s[r] = p;
+                psum += p;
+            }
+            l = l * alpha + psum;
+            m = m_new;
+            return alpha;
+        };
+        auto rescale = [&](float alpha) {
+            if (__any(alpha != 1.0f)) {
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+            }
+        };
+        auto weighted_values = [&](const v16f &p) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vreg[j][dt], p[j], o[dt], 0, 0, 0);
+        };
+        // Software pipeline: while the vector unit turns tile t's scores into probabilities, the matrix
+        // unit already forms tile t+1's scores; K is requested two tiles ahead, V one.
+        v16f s_cur, s_next;
+        load_k(t0);
+        load_v(t0);
+        scores(s_cur);
+        if (t0 + 1 < t1) load_k(t0 + 1);
+        for (int t = t0; t + 1 < t1; ++t) {
+            finish_scores(s_cur, t);
+            __builtin_amdgcn_sched_barrier(0);
+            // column maximum first, then four matrix instructions of tile t+1 for every probability of tile t:
+            // the order is pinned so that the vector work runs while the matrix unit is busy
+            float mt = s_cur[0];
+#pragma unroll
+            for (int r = 1; r < 16; ++r) mt = fmaxf(mt, s_cur[r]);
+            mt = fmaxf(mt, __shfl_xor(mt, 32));
+            const float m_new = fmaxf(m, mt);
+            const float alpha = m == -INFINITY ? 1.0f : expf(m - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_next[r] = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = r * (HD / 8) / 16; i < (r + 1) * (HD / 8) / 16; ++i) {
+                    s_next = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[i].x, qreg[4 * i], s_next, 0, 0, 0);
+                    s_next = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[i].y, qreg[4 * i + 1], s_next, 0, 0, 0);
+                    s_next = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[i].z, qreg[4 * i + 2], s_next, 0, 0, 0);
+                    s_next = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[i].w, qreg[4 * i + 3], s_next, 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                const float p = s_cur[r] == -INFINITY ? 0.f : expf(s_cur[r] - m_new);
+                s_cur[r] = p;
+                psum += p;
+            }
+            l = l * alpha + psum;
+            m = m_new;
+            // the probabilities are pinned to this block (a use with side effects): left alone, the compiler moves
+            // their computation past the matrix instructions, next to its first use
+            asm volatile("" ::"v"(s_cur), "v"(l));
+            __builtin_amdgcn_sched_barrier(0);
+            load_k(min(t + 2, t1 - 1));  // unconditional (the last one repeats a tile): no branch splits the block
+            rescale(alpha);
+            weighted_values(s_cur);
+            __builtin_amdgcn_sched_barrier(0);
+            load_v(t + 1);
+            s_cur = s_next;
+        }
+        finish_scores(s_cur, t1 - 1);
+        rescale(softmax(s_cur));
+        weighted_values(s_cur);
+        if (wave == 1 && seg == 0) {  // the short item is complete
+            const float lt = l + __shfl_xor(l, 32);
+            const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+            if (row < nrows) {
+                float *dst = aa.out + ((size_t)qt * aa.nqh + qh) * HD;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    vdt v;
+#pragma unroll
+                    for (int dt = 0; dt < NDT; ++dt) v[dt] = o[dt][r] * inv;
+                    vdt *p = reinterpret_cast<vdt *>(dst + NDT * (8 * (r >> 2) + 4 * h + (r & 3)));
+                    *p = aa.accumulate ? *p + v : v;
+                }
+            }
+        } else if (wave == 1) {  // the rest of the long item: hand it to wavefront 0
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) part_l[(dt * 16 + r) * 64 + lane] = o[dt][r];
+            part_l[NDT * 16 * 64 + lane] = m;
+            part_l[(NDT * 16 + 1) * 64 + lane] = l;
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    if (cut < tb) {  // join the two parts of the long item
+        const float m1 = part_l[NDT * 16 * 64 + lane], l1 = part_l[(NDT * 16 + 1) * 64 + lane];
+        const float mm = fmaxf(m, m1);
+        const float w0 = m == -INFINITY ? 0.f : expf(m - mm), w1 = m1 == -INFINITY ? 0.f : expf(m1 - mm);
+        l = l * w0 + l1 * w1;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[dt][r] = o[dt][r] * w0 + part_l[(dt * 16 + r) * 64 + lane] * w1;
+    }
+    const float lt = l + __shfl_xor(l, 32);
+    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    if (row < nrows) {
+        float *dst = aa.out + ((size_t)qt * aa.nqh + qh) * HD;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            vdt v;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) v[dt] = o[dt][r] * inv;
+            vdt *p = reinterpret_cast<vdt *>(dst + NDT * (8 * (r >> 2) + 4 * h + (r & 3)));
+            *p = aa.accumulate ? *p + v : v;
+        }
+    }
+}
+
 constexpr int ATT_SPLITS_MAX = 2048;
 
 // Merge the splits of one (query token, query head) row: with M = max of the split maxima and
@@ -794,7 +1050,15 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
         if (wgs >= (1ull << 31)) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: grid too large");
         PG_TRY(pg_launch(ctx, "gqa_attention_short", gqa_attention_short_kernel, dim3((unsigned)wgs), dim3(256), 0, aa));
     }
-    else if (tiled_kernel) {
+    else if (tiled_kernel && (hd == 64 || hd == 128)) {
+        // matrix-core kernel: one workgroup per kv head and pair of 32-row items (first with last, ...);
+        // the kv head varies fastest, so with eight kv heads each XCD's L2 keeps one head's keys and values
+        const size_t G = nqh / kc->num_kv_heads, n_items = (G * seq_q + 31) / 32, pairs = (n_items + 1) / 2;
+        if (pairs * kc->num_kv_heads >= (1ull << 31)) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: grid too large");
+        auto *kern = hd == 64 ? gqa_attention_mfma_kernel<64> : gqa_attention_mfma_kernel<128>;
+        PG_TRY(pg_launch(ctx, "gqa_attention_mfma", kern, dim3((unsigned)(pairs * kc->num_kv_heads)), dim3(128), 0, aa, (int)n_items,
+                         (int)kc->num_kv_heads));
+    } else if (tiled_kernel) {
         const size_t G = nqh / kc->num_kv_heads, row_sets = (G * seq_q + ATT_T_ROWS - 1) / ATT_T_ROWS;
         const dim3 grid_t((unsigned)row_sets, (unsigned)kc->num_kv_heads);
         auto *kern = hd == 64 ? gqa_attention_tiled_kernel<64> : (hd == 128 ? gqa_attention_tiled_kernel<128> : gqa_attention_tiled_kernel<256>);

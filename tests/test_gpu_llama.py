@@ -175,6 +175,23 @@ def test_gqa_attention_many_rows(ctx, orc):
     _attention_case(ctx, orc, 16, 2, 64, 33, 200, llama.AttentionMask.causal_sliding_window(167, 40, 4), None, 67)
 
 
+def test_gqa_attention_matrix_core_kernel_pairs_and_masks(ctx, orc):
+    """Head sizes 64 and 128 with many rows run on the matrix cores: 32-row items, paired first with last, the
+    long item of a pair cut between two wavefronts and joined through LDS.  Shapes with an odd and an even
+    number of items, a last item that is not full, every mask kind (tiles that are wholly hidden included),
+    a logit cap, and a cache longer than the rows can see."""
+    from peregrine_amd import llama
+    M = llama.AttentionMask
+    say("attention, matrix-core kernel")
+    _attention_case(ctx, orc, 8, 2, 128, 150, 150, M.causal(0), None, 81)                       # 19 items: 9 pairs + the middle one
+    _attention_case(ctx, orc, 8, 2, 64, 128, 200, M.causal(72), None, 82, appends=(72, 128))    # 16 items, all full
+    _attention_case(ctx, orc, 16, 4, 64, 90, 230, M.causal_sliding_window(140, 24, 3), None, 83)  # early tiles wholly hidden
+    _attention_case(ctx, orc, 16, 4, 64, 90, 230, M.causal_sliding_window(140, 0, 0), 5.0, 84)
+    _attention_case(ctx, orc, 8, 2, 128, 97, 160, M.local_global(63, 9, [0, 5, 31, 32, 64, 65, 159, 1000]), None, 85)
+    _attention_case(ctx, orc, 8, 8, 128, 80, 100, M.none(), 2.5, 86)                            # MHA: one head per kv head
+    _attention_case(ctx, orc, 12, 2, 64, 75, 75, M.causal(0), None, 87)                         # group of 6: items straddle tokens
+
+
 def test_gqa_attention_local_global(ctx, orc):
     """AttentionMask::LocalGlobal through each of the three kernels (few rows with key splits, the
     generic one, the tiled one), global positions in no order, repeated and past the cache."""
