@@ -142,11 +142,17 @@ struct gemv_wgroup {
     int wg0[PG_GEMM_MAX_GROUP];
 };
 
-template <int NCH, int RPW>
-__global__ __launch_bounds__(256) void gemv_w8a8_m1_f32x_kernel(
+// NW wavefronts per workgroup share one quantisation of the row: every workgroup repeats that
+// arithmetic (about 14 vector instructions per element), so a long row is spread over more
+// threads (K = 14336 on 256 threads is 56 elements each and 512 such workgroups: the vector
+// units, not the weight stream, then set the pace; on 1024 threads it is 14 each and 256
+// workgroups).
+template <int NCH, int RPW, int NW>
+__global__ __launch_bounds__(64 * NW) void gemv_w8a8_m1_f32x_kernel(
     const gemv_wgroup grp, int k_pad, const float *__restrict__ x_f32, int k, int32_t *__restrict__ acc_out) {
+    constexpr int NT = 64 * NW, NV = (NCH * 256 + NT - 1) / NT;  // float4 of the row per thread
     __shared__ int xq[NCH * 256];  // the quantised row, zero beyond k: NCH KiB >= k_pad bytes
-    __shared__ float red[4];
+    __shared__ float red[NW];
     int g = 0;
 #pragma unroll
     for (int i = 1; i < PG_GEMM_MAX_GROUP; ++i) g = (int)blockIdx.x >= grp.wg0[i] ? i : g;
@@ -156,7 +162,7 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_f32x_kernel(
     const int n = grp.n[g];
     const int nchunk = k_pad >> 4;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int row0 = (((int)blockIdx.x - grp.wg0[g]) * 4 + wave) * RPW;
+    const int row0 = (((int)blockIdx.x - grp.wg0[g]) * NW + wave) * RPW;
     auto load_row = [&](int row, v4i (&w)[NCH]) {
         const v4i *wp = reinterpret_cast<const v4i *>(w_t + (size_t)row * k_pad);
 #pragma unroll
@@ -170,11 +176,11 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_f32x_kernel(
     // right behind it, all in flight together.
     const int nvec = k >> 2;
     const float4 *x4 = reinterpret_cast<const float4 *>(x_f32);
-    float4 v[NCH];
+    float4 v[NV];
     float amax = 0.0f;
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        const int idx = threadIdx.x + 256 * i;
+    for (int i = 0; i < NV; ++i) {
+        const int idx = threadIdx.x + NT * i;
         v[i] = x4[idx < nvec ? idx : nvec - 1];
     }
     v4i w[RPW][NCH];
@@ -182,43 +188,52 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_f32x_kernel(
     for (int r = 0; r < RPW; ++r) load_row(row0 + r, w[r]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        const int idx = threadIdx.x + 256 * i;
+    for (int i = 0; i < NV; ++i) {
+        const int idx = threadIdx.x + NT * i;
         const float m4 = fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)), fmaxf(fabsf(v[i].z), fabsf(v[i].w)));
         amax = fmaxf(amax, idx < nvec ? m4 : 0.0f);
     }
-    amax = pg_block_max_256_keep_loads(amax, red);
+    // maximum over the workgroup; the barriers wait for LDS only (not __syncthreads(): that would
+    // also wait for every weight row in flight)
+    amax = pg_wave_max_f32(amax);
+    if (lane == 0) red[wave] = amax;
+    asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier" ::: "memory");
+    amax = red[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) amax = fmaxf(amax, red[i]);
     const float a_scale = (amax == 0.0f) ? 1.0f : amax / 127.0f;
     const float inv_scale = 1.0f / a_scale;
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        const int idx = threadIdx.x + 256 * i;
+    for (int i = 0; i < NV; ++i) {
+        const int idx = threadIdx.x + NT * i;
         const int b0 = pg_quant_to_i8(v[i].x * inv_scale) & 0xFF;
         const int b1 = pg_quant_to_i8(v[i].y * inv_scale) & 0xFF;
         const int b2 = pg_quant_to_i8(v[i].z * inv_scale) & 0xFF;
         const int b3 = pg_quant_to_i8(v[i].w * inv_scale) & 0xFF;
-        xq[idx] = idx < nvec ? (b0 | (b1 << 8) | (b2 << 16) | (b3 << 24)) : 0;
+        if (NV * NT == NCH * 256 || idx < NCH * 256) xq[idx] = idx < nvec ? (b0 | (b1 << 8) | (b2 << 16) | (b3 << 24)) : 0;
     }
-    // (not __syncthreads(): that would also wait for every weight row in flight)
     asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier" ::: "memory");
-    v4i x[NCH];
+    int acc[RPW];
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) x[j] = reinterpret_cast<const v4i *>(xq)[lane + 64 * j];
+    for (int r = 0; r < RPW; ++r) acc[r] = 0;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        const v4i x = reinterpret_cast<const v4i *>(xq)[lane + 64 * j];  // zero beyond k
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) acc[r] = dot16(w[r][j], x, acc[r]);
+    }
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
         const int row = row0 + r;  // < n_pad by construction of the grid
-        int acc = 0;
-#pragma unroll
-        for (int j = 0; j < NCH; ++j) acc = dot16(w[r][j], x[j], acc);  // x is zero beyond k
-        acc = wave_sum_i32(acc);
+        const int sum = wave_sum_i32(acc[r]);
         if (lane == 0 && row < n) {
-            if (out) out[row] = (float)acc * a_scale * w_scales[row];
-            if (acc_out) acc_out[row] = acc;
+            if (out) out[row] = (float)sum * a_scale * w_scales[row];
+            if (acc_out) acc_out[row] = sum;
         }
     }
 }
 
-template <int NCH, int RPW>
+template <int NCH, int RPW, int NW>
 pg_status launch_m1_f32x(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *const *w, float *const *out, int count,
                          int32_t *acc) {
     gemv_wgroup grp;
@@ -230,20 +245,26 @@ pg_status launch_m1_f32x(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qte
         grp.out[i] = used && out ? out[i] : nullptr;
         grp.n[i] = used ? (int)w[i]->cols : 0;
         grp.wg0[i] = used ? wgs : INT_MAX;
-        if (used) wgs += (int)(w[i]->n_pad / (4 * RPW));
+        if (used) wgs += (int)(w[i]->n_pad / (NW * RPW));  // n_pad is a multiple of 256
     }
-    PG_TRY(pg_launch(ctx, "gemv_w8a8", gemv_w8a8_m1_f32x_kernel<NCH, RPW>, dim3((unsigned)wgs), dim3(256), 0, grp,
+    PG_TRY(pg_launch(ctx, "gemv_w8a8", gemv_w8a8_m1_f32x_kernel<NCH, RPW, NW>, dim3((unsigned)wgs), dim3(64 * NW), 0, grp,
                      (int)w[0]->k_pad, x_f32, (int)k, acc));
     return pg_launch_check("gemv_w8a8_m1_f32x");
 }
 
+// Wavefronts per workgroup by row length (16 elements of the row per thread or fewer); two weight
+// rows per wavefront where that still leaves eight wavefronts per CU and the registers allow it
+// (sixteen wavefronts per workgroup have 128 registers each: one row of up to 16 KiB in flight).
 template <int NCH>
 pg_status launch_m1_f32x_rows(pg_ctx *ctx, const float *x_f32, size_t k, const pg_qtensor *const *w, float *const *out, int count,
                               int32_t *acc) {
     size_t rows = 0;
     for (int i = 0; i < count; ++i) rows += w[i]->n_pad;
-    if (rows / 2 >= (size_t)ctx->num_cu * 8) return launch_m1_f32x<NCH, 2>(ctx, x_f32, k, w, out, count, acc);
-    return launch_m1_f32x<NCH, 1>(ctx, x_f32, k, w, out, count, acc);
+    constexpr int NW = NCH <= 4 ? 4 : (NCH <= 8 ? 8 : 16);
+    if constexpr (NW < 16) {
+        if (rows / 2 >= (size_t)ctx->num_cu * 8) return launch_m1_f32x<NCH, 2, NW>(ctx, x_f32, k, w, out, count, acc);
+    }
+    return launch_m1_f32x<NCH, 1, NW>(ctx, x_f32, k, w, out, count, acc);
 }
 
 template <int NCH, int RPW>
