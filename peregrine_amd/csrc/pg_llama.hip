@@ -444,7 +444,8 @@ __global__ __launch_bounds__(256) void gqa_attention_short_kernel(attn_args aa) 
     }
 }
 
-// ---- many query rows (prefill): tiled, online softmax ----------------------------------------
+// ---- many query rows (prefill), head size 256: tiled, online softmax -------------------------
+// (head sizes 64 and 128 run on the matrix cores, further down; the template is kept general)
 // One (token, head) row per workgroup makes every row stream all of its keys and values again
 // and spends most instructions on cross-lane sums.  Here a workgroup owns 32 query rows that
 // read the SAME kv head (the heads of a group, then consecutive tokens), eight per wavefront,
@@ -1061,8 +1062,8 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     } else if (tiled_kernel) {
         const size_t G = nqh / kc->num_kv_heads, row_sets = (G * seq_q + ATT_T_ROWS - 1) / ATT_T_ROWS;
         const dim3 grid_t((unsigned)row_sets, (unsigned)kc->num_kv_heads);
-        auto *kern = hd == 64 ? gqa_attention_tiled_kernel<64> : (hd == 128 ? gqa_attention_tiled_kernel<128> : gqa_attention_tiled_kernel<256>);
-        const size_t lds_t = hd == 64 ? att_tiled_lds<64>() : (hd == 128 ? att_tiled_lds<128>() : att_tiled_lds<256>());
+        auto *kern = gqa_attention_tiled_kernel<256>;  // head sizes 64 and 128 took the matrix-core kernel above
+        const size_t lds_t = att_tiled_lds<256>();
         PG_TRY(pg_allow_dynamic_lds(ctx, reinterpret_cast<const void *>(kern), lds_t));
         PG_TRY(pg_launch(ctx, "gqa_attention_tiled", kern, grid_t, dim3(256), lds_t, aa));
     } else
