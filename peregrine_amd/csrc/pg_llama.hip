@@ -924,6 +924,12 @@ __global__ __launch_bounds__(256) void swiglu_digits_kernel(const float4 *__rest
     pg_emit_digits<NIB>(o, 0, i >> 3, i & 7, n4 >> 3, digits, xs);
 }
 
+// (a fill kernel rather than hipMemsetAsync: a caller may capture the stream-ordered entry points in a graph)
+__global__ __launch_bounds__(256) void zero_f32_kernel(float *__restrict__ p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0.0f;
+}
+
 __global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, const float *__restrict__ b,
                                                   float *__restrict__ out, size_t n) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -979,7 +985,10 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     const size_t len = kc->len, hd = kc->head_dim;
     if (seq_q == 0 || nqh == 0) return PG_OK;
     if (len == 0) {  // nothing to attend to: the reference adds nothing to `output`
-        if (!accumulate) PG_HIP(hipMemsetAsync(out, 0, seq_q * nqh * hd * sizeof(float), ctx->stream));
+        if (!accumulate) {
+            const size_t n = seq_q * nqh * hd;
+            PG_TRY(pg_launch(ctx, "zero_f32", zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, out, n));
+        }
         return PG_OK;
     }
     attn_args aa;
