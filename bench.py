@@ -208,6 +208,9 @@ def main():
     ap.add_argument("--only-headline", action="store_true", help="cfg3 (and the ceilings) only")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain 512 MiB device copies (counter calibration under rocprofv3 --pmc)")
+    ap.add_argument("--cache-residency", action="store_true",
+                    help="instead of the benchmark: the one-row products timed with 1 .. 12 tensors rotated "
+                         "(weights served by the L2s, the Infinity Cache, HBM), one JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; every kernel here runs at its real "
@@ -217,6 +220,9 @@ def main():
 
     B = Bench(args)
     torch, lib, check, ptr, dev = B.torch, B.lib, B.check, B.ptr, B.dev
+    if args.cache_residency:
+        print(json.dumps(cache_residency(B)), flush=True)
+        return
 
     # ------------------------------------------------------------------ prefill (headline)
     # Two layers' worth of weights (436 MB), used alternately: more than the 256 MB Infinity Cache
@@ -392,6 +398,56 @@ def main():
     line["cpu_baseline"] = cpu_baseline(B.orc, cpu_w, cpu_a) if B.cpu else None
     print(json.dumps(line), flush=True)
     B.ctx.close()
+
+
+def cache_residency(B):
+    """How much of a one-row product's time is the weight stream?  The same product over 1, 2, 3, 4, 6 and 12
+    tensors used in turn: one 33 MB tensor is served by the eight L2s (4 MB each), 66 - 198 MB by the 256 MB
+    Infinity Cache, 396 MB and more by HBM.  us per product (stream time over 240 products, launches included)."""
+    import numpy as np
+
+    torch, lib, check, ptr, dev, _ffi = B.torch, B.lib, B.check, B.ptr, B.dev, B.ffi
+    rots = (1, 2, 3, 4, 6, 12)
+    out = {"what": cache_residency.__doc__.split("  us per")[0].replace("\n   ", ""), "unit": "us per product", "tensors_rotated": list(rots)}
+
+    def sweep(step_for):
+        row = []
+        for rot in rots:
+            B.i = 0
+            t = B.timed(step_for(rot), 240, 48)
+            row.append(round(t["ms_per_step"] * 1e3, 2))
+        return row
+
+    for n_out, k_in in ((14336, 4096), (4096, 14336), (28672, 4096)):
+        raw = np.frombuffer(B.synth.pack_q4_0(B.normal(7300 + n_out % 97, (n_out, k_in), 0.02).cpu().numpy()), np.uint8)
+        hs = []
+        for _ in range(max(rots)):
+            h = C.c_void_p()
+            check(lib.pg_gguf_upload(B.h, C.c_void_p(raw.ctypes.data), _ffi.GGML_Q4_0, n_out, k_in, C.byref(h)))
+            hs.append(h)
+        x, y = B.make_acts(1, k_in, 1250), torch.empty(1, n_out, device=dev)
+
+        def step_for(rot):
+            def step():
+                check(lib.pg_gguf_matmul_dev(B.h, ptr(x), 1, hs[B.i % rot], ptr(y)))
+                B.i += 1
+            return step
+        out[f"q4_0 [{k_in}]->[{n_out}] ({raw.size / 1e6:.0f} MB each)"] = sweep(step_for)
+        for h in hs:
+            lib.pg_gguf_free(B.h, h)
+    for k, n in ((4096, 14336), (14336, 4096)):
+        ws = [B.make_weight(k, n, 7400 + i) for i in range(max(rots))]
+        x, y = B.make_acts(1, k, 1251), torch.empty(1, n, device=dev)
+
+        def step_for(rot):
+            def step():
+                check(lib.pg_matmul_quantized_dev(B.h, ptr(x), 1, k, ws[B.i % rot], ptr(y), None))
+                B.i += 1
+            return step
+        out[f"int8 [{k}]->[{n}] ({k * n / 1e6:.0f} MB each)"] = sweep(step_for)
+        for h in ws:
+            lib.pg_qtensor_free(B.h, h)
+    return out
 
 
 def section_decode_and_linear(B, line):
