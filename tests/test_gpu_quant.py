@@ -435,7 +435,9 @@ def test_wire_record_straight_to_device(ctx, orc):
     _ffi.lib.pg_qtensor_free(ctx.handle, h)
 
 
-W8A32_SHAPES = [(32, 128, 64), (1, 4096, 1024), (3, 200, 77), (70, 4096, 300), (300, 1000, 520)]
+W8A32_SHAPES = [(32, 128, 64), (1, 4096, 1024), (3, 200, 77), (70, 4096, 300), (191, 256, 130),
+                # from 192 rows the three digit planes run as one product over the stacked planes
+                (192, 512, 300), (256, 384, 256), (300, 1000, 520), (700, 256, 1000)]
 
 
 @pytest.mark.parametrize("m,k,n", W8A32_SHAPES)
