@@ -192,6 +192,14 @@ def test_gqa_attention_matrix_core_kernel_pairs_and_masks(ctx, orc):
     _attention_case(ctx, orc, 12, 2, 64, 75, 75, M.causal(0), None, 87)                         # group of 6: items straddle tokens
 
 
+def test_gqa_attention_prefill_at_llama_8b_size(ctx, orc):
+    """The benchmark's prefill attention at full size (32 query heads over 8 kv heads of 128, 1024 tokens into
+    an empty cache, causal): 64 pairs of 32-row items per kv head, up to 32 key tiles per item."""
+    from peregrine_amd import llama
+    say("attention 32/8 heads x 128, 1024 tokens, causal")
+    _attention_case(ctx, orc, 32, 8, 128, 1024, 1024, llama.AttentionMask.causal(0), None, 91)
+
+
 def test_gqa_attention_local_global(ctx, orc):
     """AttentionMask::LocalGlobal through each of the three kernels (few rows with key splits, the
     generic one, the tiled one), global positions in no order, repeated and past the cache."""
