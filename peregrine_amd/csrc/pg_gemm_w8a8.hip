@@ -56,11 +56,16 @@ struct gemm_wgroup {
     float *out[PG_GEMM_MAX_GROUP];
     int n[PG_GEMM_MAX_GROUP];
     int panel0[PG_GEMM_MAX_GROUP];
+    // The last pass of the W8A32 product (one weight): with `comb` the accumulator is the digit of weight 65536
+    // and the output is (65536 acc + 256 comb[comb_plane + i] + comb[i]) * a_scale * w_scale, the integer exact
+    // and the scaling done in f64 (what combine_digits3_kernel computes from three stored planes).
+    const int32_t *comb;
+    long long comb_plane;
 };
 
 // CLK (the clock probe only): thread 0 of every workgroup also stores the shader cycles and the
 // wall-clock ticks its K loop took, clk[2 * blockIdx.x] and clk[2 * blockIdx.x + 1].
-template <int BM, int BN, int BK, int NST, int NWM, int NWN, int OCC, bool CLK = false>
+template <int BM, int BN, int BK, int NST, int NWM, int NWN, int OCC, bool CLK = false, bool COMB = false>
 __global__ __launch_bounds__(64 * NWM * NWN) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const gemm_wgroup grp, int ldb,
                       const float *__restrict__ a_scales, int32_t *__restrict__ acc_out, int M, int K,
@@ -238,7 +243,7 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const gemm_wgroup g
     // ---- epilogue.  Accumulator register r of a 32x32 tile holds
     // row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.  (The scales were requested before the
     // K loop: loading them here would put several dependent memory round trips on every tile.)
-    if (out && !acc_out && m0 + BM <= M && n0 + BN <= N) {
+    if (!COMB && out && !acc_out && m0 + BM <= M && n0 + BN <= N) {
         // A whole tile inside the matrix, f32 output only (every tile of the prefill shapes):
         // straight-line code, the 16 row scales of a 32-row tile as four 128-bit LDS reads.
         // The stores are non-temporal: this kernel never reads the output back, and 117 MB of
@@ -261,6 +266,43 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const gemm_wgroup g
                 for (int r = 0; r < 16; ++r)
                     __builtin_nontemporal_store((float)acc[i][j][r] * as[r] * ws, dst + (size_t)(8 * (r >> 2) + (r & 3)) * N);
                 __builtin_amdgcn_sched_barrier(0);  // one tile's stores at a time: bounded live ranges
+            }
+        }
+        return;
+    }
+    if (COMB && out && !acc_out && m0 + BM <= M && n0 + BN <= N) {
+        // The W8A32 product's last pass on a whole tile: the two other digits' accumulators are fetched in the
+        // order the stores go out (a lane's rows of one column, four at a time).
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            float as[16];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 v = *reinterpret_cast<const float4 *>(lds_as + wm * WM + 32 * i + 8 * g + 4 * half);
+                as[4 * g] = v.x; as[4 * g + 1] = v.y; as[4 * g + 2] = v.z; as[4 * g + 3] = v.w;
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const double ws = (double)lds_ws[wn * WN + 32 * j + l31];
+                const size_t base = (size_t)(m0 + wm * WM + 32 * i + 4 * half) * N + (n0 + wn * WN + 32 * j + l31);
+#pragma unroll
+                for (int r0 = 0; r0 < 16; r0 += 4) {  // four rows at a time (the 256x256 tile has no registers to spare)
+                    int c0[4], c1[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const size_t idx = base + (size_t)(8 * ((r0 + r) >> 2) + ((r0 + r) & 3)) * N;
+                        c0[r] = __builtin_nontemporal_load(grp.comb + idx);
+                        c1[r] = __builtin_nontemporal_load(grp.comb + grp.comb_plane + idx);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const double v = 65536.0 * (double)acc[i][j][r0 + r] + 256.0 * (double)c1[r] + (double)c0[r];
+                        __builtin_nontemporal_store((float)(v * (double)as[r0 + r] * ws),
+                                                    out + base + (size_t)(8 * ((r0 + r) >> 2) + ((r0 + r) & 3)) * N);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                __builtin_amdgcn_sched_barrier(0);  // one tile at a time: bounded live ranges
             }
         }
         return;
@@ -290,7 +332,14 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const gemm_wgroup g
                     const int m = m0 + wm * WM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
                     if (m < M) {
                         const int a = acc[i][j][r];
-                        if (out) out[(size_t)m * N + n] = (float)a * lds_as[wm * WM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3)] * ws;
+                        const float as = lds_as[wm * WM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3)];
+                        if (COMB && out) {
+                            const size_t idx = (size_t)m * N + n;
+                            const double v = 65536.0 * (double)a + 256.0 * (double)grp.comb[grp.comb_plane + idx] + (double)grp.comb[idx];
+                            out[idx] = (float)(v * (double)as * (double)ws);
+                        } else if (out) {
+                            out[(size_t)m * N + n] = (float)a * as * ws;
+                        }
                         if (acc_out) acc_out[(size_t)m * N + n] = a;
                     }
                 }
@@ -300,10 +349,10 @@ void gemm_w8a8_kernel(const int8_t *__restrict__ A, int lda, const gemm_wgroup g
     }
 }
 
-template <int BM, int BN, int BK, int NST, int NWM, int NWN, int OCC>
+template <int BM, int BN, int BK, int NST, int NWM, int NWN, int OCC, bool COMB = false>
 pg_status launch_group(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
                        const pg_qtensor *const *w, float *const *out, int count, size_t m, int32_t *acc,
-                       int splits = 1, int kt_per_split = 0) {
+                       int splits = 1, int kt_per_split = 0, const int32_t *comb = nullptr, size_t comb_plane = 0) {
     const int tiles_m = (int)((m + BM - 1) / BM);
     gemm_wgroup grp;
     int panels = 0;
@@ -316,9 +365,11 @@ pg_status launch_group(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const f
         grp.panel0[i] = used ? panels : INT_MAX;
         if (used) panels += (int)((w[i]->cols + BN - 1) / BN);
     }
+    grp.comb = comb;
+    grp.comb_plane = (long long)comb_plane;
     const int ntiles = tiles_m * panels;
     const size_t lds = (size_t)NST * (BM + BN) * BK + (BM + BN) * sizeof(float);
-    auto kern = gemm_w8a8_kernel<BM, BN, BK, NST, NWM, NWN, OCC>;
+    auto kern = gemm_w8a8_kernel<BM, BN, BK, NST, NWM, NWN, OCC, false, COMB>;
     PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
     const unsigned grid = (unsigned)(((ntiles + 7) / 8) * 8);
     const size_t k_pad = w[0]->k_pad;
@@ -366,7 +417,8 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const int32_t *__res
 // ctx->gemm_force_tile (pg_gemm_w8a8_force_tile) overrides the choice: 1 = 64x64, 2 = 256x256,
 // 3 = 128x256, 4 = 128x64, 5 = 128x128.
 pg_status gemm_dispatch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
-                        const pg_qtensor *const *w, float *const *out, int count, size_t m, int32_t *acc) {
+                        const pg_qtensor *const *w, float *const *out, int count, size_t m, int32_t *acc,
+                        const int32_t *comb = nullptr, size_t comb_plane = 0) {
     const size_t cus = (size_t)ctx->num_cu;
     auto tiles = [&](size_t bm, size_t bn) {
         size_t panels = 0;
@@ -388,11 +440,21 @@ pg_status gemm_dispatch(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const 
         else pick = 5;
     }
     switch (pick) {
-        case 1: return launch_group<64, 64, 128, 2, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
-        case 2: return launch_group<256, 256, 128, 2, 2, 4, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
-        case 3: return launch_group<128, 256, 128, 2, 2, 4, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
-        case 4: return launch_group<128, 64, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
-        case 5: return launch_group<128, 128, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
+        case 1:
+            if (comb) return launch_group<64, 64, 128, 2, 2, 2, 2, true>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc, 1, 0, comb, comb_plane);
+            return launch_group<64, 64, 128, 2, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
+        case 2:
+            if (comb) return launch_group<256, 256, 128, 2, 2, 4, 2, true>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc, 1, 0, comb, comb_plane);
+            return launch_group<256, 256, 128, 2, 2, 4, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
+        case 3:
+            if (comb) return launch_group<128, 256, 128, 2, 2, 4, 2, true>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc, 1, 0, comb, comb_plane);
+            return launch_group<128, 256, 128, 2, 2, 4, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
+        case 4:
+            if (comb) return launch_group<128, 64, 128, 3, 2, 2, 2, true>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc, 1, 0, comb, comb_plane);
+            return launch_group<128, 64, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
+        case 5:
+            if (comb) return launch_group<128, 128, 128, 3, 2, 2, 2, true>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc, 1, 0, comb, comb_plane);
+            return launch_group<128, 128, 128, 3, 2, 2, 2>(ctx, a_i8, a_stride, a_scales, w, out, count, m, acc);
         default: return pg_fail(PG_EINVAL, "gemm_w8a8: unknown tile override %d", pick);
     }
 }
@@ -453,6 +515,16 @@ pg_status pg_launch_gemm_w8a8(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride,
     return gemm_dispatch(ctx, a_i8, a_stride, a_scales, &w, &out, 1, m, acc);
 }
 
+// The W8A32 product's last pass: `a_i8` is the digit plane of weight 65536, `comb` holds the accumulators of
+// the other two ([2][comb_plane], the plane of weight 256 second); writes the finished f32 product.
+pg_status pg_launch_gemm_w8a8_combine(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                                      const pg_qtensor *w, size_t m, float *out, const int32_t *comb, size_t comb_plane) {
+    if (a_stride != w->k_pad) return pg_fail(PG_EINVAL, "gemm_w8a8: activation stride %zu != k_pad %zu", a_stride, w->k_pad);
+    if (w->k_pad >= (1ull << 22) || m >= (1ull << 24) || w->cols >= (1ull << 30))
+        return pg_fail(PG_EUNSUPPORTED, "gemm_w8a8: shape exceeds the kernel's 32-bit tile offsets");
+    return gemm_dispatch(ctx, a_i8, a_stride, a_scales, &w, &out, 1, m, nullptr, comb, comb_plane);
+}
+
 // The shader clock inside the K loop of the 256x256 tile (the gate|up product's kernel): the
 // product [m x k] . [k x n] on pseudo-random operands, every workgroup timing its own loop with
 // the shader cycle counter and the constant-rate wall clock.
@@ -478,6 +550,8 @@ PG_API pg_status pg_probe_gemm_clock(pg_ctx *ctx, size_t m, size_t k, size_t n, 
         grp.w[i] = nullptr;
         grp.ws[i] = nullptr; grp.out[i] = nullptr; grp.n[i] = 0; grp.panel0[i] = INT_MAX;
     }
+    grp.comb = nullptr;
+    grp.comb_plane = 0;
     grp.w[0] = b.as<int8_t>(); grp.ws[0] = sc.as<float>(); grp.out[0] = out.as<float>(); grp.n[0] = (int)n; grp.panel0[0] = 0;
     const size_t lds = (size_t)NST * (BM + BN) * BK + (BM + BN) * sizeof(float);
     auto kern = gemm_w8a8_kernel<BM, BN, BK, NST, 2, 4, 2, true>;

@@ -177,6 +177,8 @@ pg_status pg_launch_gemm_w8a8_group(pg_ctx *ctx, const int8_t *a_i8, size_t a_st
                                     const pg_qtensor *const *w, float *const *out, int count, size_t m);
 // 5 .. 64 activation rows: K split over workgroups, i32 partial sums in `part`, then one finishing
 // launch.  With part == nullptr only reports the number of splits (for sizing `part`).
+pg_status pg_launch_gemm_w8a8_combine(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                                      const pg_qtensor *w, size_t m, float *out, const int32_t *comb, size_t comb_plane);
 pg_status pg_launch_gemm_w8a8_few_rows(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
                                        const pg_qtensor *w, size_t m, float *out, int32_t *acc, int32_t *part,
                                        int *splits_out);

@@ -679,9 +679,9 @@ PG_API pg_status pg_matmul_dequant_i8_dev(pg_ctx *ctx, const float *a_dev, size_
     PG_CHECK_ARG(m < (1ull << 24), "pg_matmul_dequant_i8: m = %zu too large", m);
     PG_CHECK_ARG(k <= 133000, "pg_matmul_dequant_i8: k = %zu would overflow the i32 digit sums", k);  // 127 * 127 * k < 2^31
     const size_t m_pad = pg_round_up(m, PG_MPAD), n = w->cols;
-    // With enough rows the three digit planes run as ONE product over the planes stacked row-wise (they lie
-    // back to back in the scratch, each m_pad rows): one launch, one tile space of three times the
-    // rows, the accumulator planes then m_pad rows apart.
+    // With enough rows the two low digit planes run as ONE product over the planes stacked row-wise (they lie
+    // back to back in the scratch, each m_pad rows; the accumulator planes are then m_pad rows apart) and
+    // the third plane's product finishes the sum in its epilogue.
     const bool stacked = m >= 192;
     const size_t plane_bytes = m_pad * w->k_pad, plane_elems = (stacked ? m_pad : m) * n;
     // (the product's prologue reads a scale per stacked row, whether or not it writes f32: three planes' worth)
@@ -693,9 +693,13 @@ PG_API pg_status pg_matmul_dequant_i8_dev(pg_ctx *ctx, const float *a_dev, size_
     int32_t *acc = reinterpret_cast<int32_t *>(planes + sz_planes + sz_scales);
     PG_TRY(pg_launch(ctx, "rows_to_digits3", rows_to_digits3_kernel, dim3((unsigned)m), dim3(QA_THREADS), 0, a_dev, k, planes,
                      w->k_pad, plane_bytes, row_scales));
-    if (stacked)
-        PG_TRY(pg_launch_gemm_w8a8(ctx, planes, w->k_pad, row_scales, w, 2 * m_pad + m, nullptr, acc));
-    for (int p = 0; p < 3 && !stacked; ++p) {
+    if (stacked) {
+        // the two low planes as one product, then the plane of weight 65536, whose epilogue joins the three
+        // accumulators and scales them: no third accumulator plane and no combining launch
+        PG_TRY(pg_launch_gemm_w8a8(ctx, planes, w->k_pad, row_scales, w, m_pad + m, nullptr, acc));
+        return pg_launch_gemm_w8a8_combine(ctx, planes + 2 * plane_bytes, w->k_pad, row_scales, w, m, out_dev, acc, plane_elems);
+    }
+    for (int p = 0; p < 3; ++p) {
         if (m <= PG_GEMV_MAX_M)
             PG_TRY(pg_launch_gemv_w8a8(ctx, planes + p * plane_bytes, w->k_pad, row_scales, w, m, nullptr, acc + p * plane_elems));
         else

@@ -464,6 +464,41 @@ def test_matmul_dequant_i8_vs_oracle(ctx, orc, m, k, n):
     qt.free_gpu()
 
 
+def test_matmul_dequant_i8_combining_epilogue_on_every_tile(ctx, orc):
+    """From 192 rows the product of the plane of weight 65536 finishes the sum in its epilogue (it reads the other
+    two planes' accumulators).  Every tile shape of the matrix-core kernel in turn, on a ragged shape (the
+    bounds-checked epilogue at the edges, the straight-line one inside), and two shapes that the dispatcher
+    itself gives 256x256 tiles (whole tiles only, and ragged): exact small integers in, exact integers out, and
+    the float64 product as the bar for random data."""
+    from peregrine_amd import quant, _ffi
+    for m, k, n, force in [(300, 256, 520, c) for c in TILES] + [(2048, 128, 5888, 0), (2050, 128, 5900, 0)]:
+        say(f"matmul_dequant_i8 m={m} k={k} n={n} tile override {force}")
+        a = orc.rng_normal(21 + m, m * k)
+        a.reshape(m, k)[:, :: max(1, k // 37)] *= 20
+        w = orc.rng_normal(22 + n, k * n, 0.0, 0.02)
+        q, q_t, s = orc.quantize_weights(w, k, n)
+        qt = quant.QuantizedTensor(q, q_t, s, k, n)
+        ai = (np.arange(m * k, dtype=np.float32) % 9 - 4).reshape(m, k)
+        qi = (np.arange(k * n).reshape(k, n) % 13 - 6).astype(np.int8)
+        qt_int = quant.QuantizedTensor(qi.reshape(-1), np.ascontiguousarray(qi.T).reshape(-1), np.ones(n, np.float32), k, n)
+        try:
+            _ffi.check(_ffi.lib.pg_gemm_w8a8_force_tile(ctx.handle, force))
+            got = quant.matmul_dequant_i8(a, m, k, qt, ctx).reshape(m, n)
+            if force:
+                assert last_tile(ctx)[:2] == TILES[force]
+            else:
+                assert last_tile(ctx)[:2] == (256, 256)
+            got_int = quant.matmul_dequant_i8(ai, m, k, qt_int, ctx).reshape(m, n)
+        finally:
+            _ffi.check(_ffi.lib.pg_gemm_w8a8_force_tile(ctx.handle, 0))
+        assert (got_int == (ai.astype(np.int64) @ qi.astype(np.int64))).all(), "integer inputs: the product is not exact"
+        exact = a.reshape(m, k).astype(np.float64) @ orc.dequantize(q, s, k, n).reshape(k, n).astype(np.float64)
+        for r in range(m):
+            H.assert_close_rel(got[r], exact[r], 1e-5, f"row {r} vs exact")
+        qt.free_gpu()
+        qt_int.free_gpu()
+
+
 def test_matmul_dequant_i8_reference_tolerance_and_closed_form(ctx, orc):
     """tests/quant_parity.rs:79-146 restated: the W8A32 result is within 10 % / 0.02 of the f32
     product of the unquantised weights; plus integer inputs with unit scales give exact integers,
