@@ -215,18 +215,28 @@ struct RowLoads {
 // wavefront has requested its first weight rows: the product is one launch instead of two, and
 // the digit arithmetic (18 vector operations per element, shared by NW wavefronts) runs while
 // those first loads are in flight.
-template <int QT, int BPL, int RW, int R, bool Q41 = false, bool XF32 = false, int NW = 1>
+// EPI (one item, NW * RW = 32: a workgroup owns one block of 32 output rows) makes the output the digit
+// input of the NEXT product, so that the one-token step of models::llama needs no launch in between:
+//   1  y (+ residual) is stored as usual, and also as digits of y * gamma (the RMSNorm weights,
+//      src/nn.rs:560-652) with the block's sum of y^2 in ss_out[block]: the normalisation factor is a
+//      scalar, which the next product applies to its result (POST);
+//   2  the workgroup multiplies by two tensors (gate, then up = epi.qs1 / d1) and leaves only the digits
+//      of silu(gate) * up (src/models/llama/decoder.rs:143-150).
+// POST: the product is multiplied by 1 / sqrt(sum(ss_in[0 .. ss_n)) * ss_inv_dim + eps) before anything else.
+template <int QT, int BPL, int RW, int R, bool Q41 = false, bool XF32 = false, int NW = 1, int EPI = 0, bool POST = false>
 __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
     const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0, pg_gemv_batch batch,
     int n_out, int nb, const int8_t *__restrict__ digits_base, const float *__restrict__ xs_base,
     float *__restrict__ y_base, const float *__restrict__ residual_base, const uint16_t *__restrict__ m0,
-    const float *__restrict__ xsum_base, const float *__restrict__ x_f32) {
+    const float *__restrict__ xsum_base, const float *__restrict__ x_f32, pg_gemv_epi epi) {
     constexpr int SEG = 64 * BPL;  // blocks per K segment
-    constexpr int NG = RW / R;
+    constexpr int NT = EPI == 2 ? 2 : 1;  // tensors per workgroup
+    constexpr int NG = RW / R, NGT = NG * NT;
+    static_assert(EPI == 0 || (!XF32 && !Q41 && NW * RW == 32), "an output block of 32 rows per workgroup");
+    static_assert(EPI != 0 || XF32 || NW == 1, "several wavefronts per workgroup only where they share something");
     constexpr int NH = QT == 8 ? 2 : 1;
     constexpr int NP = QT == 8 ? 6 : 5;  // digit planes
     static_assert(!XF32 || !Q41, "the one-launch form has no block sums");
-    static_assert(XF32 || NW == 1, "several wavefronts per workgroup only where they share the digits");
     extern __shared__ __attribute__((aligned(16))) char lds_digits[];  // XF32: [6 planes][nb][16 B], then nb scales
     const int item = blockIdx.y;
     const uint8_t *qs_any = qs0;
@@ -238,6 +248,8 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
     }
     const gv4i_ptr qs = (gv4i_ptr)(uintptr_t)qs_any;
     const gv4i_ptr dsc = (gv4i_ptr)(uintptr_t)d_any;
+    const gv4i_ptr qs_t[2] = {qs, (gv4i_ptr)(uintptr_t)epi.qs1};
+    const gv4i_ptr dsc_t[2] = {dsc, (gv4i_ptr)(uintptr_t)epi.d1};
     const size_t xrow = (size_t)(item / batch.x_row_div);
     const gv4i_ptr digits = (gv4i_ptr)(uintptr_t)(digits_base + xrow * (size_t)nb * 96);
     const float *__restrict__ xs = xs_base + xrow * (size_t)nb;
@@ -248,11 +260,17 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
     const int row0 = (blockIdx.x * NW + (threadIdx.x >> 6)) * RW;
     int8_t *const ldig = reinterpret_cast<int8_t *>(lds_digits);
     float *const lxs = reinterpret_cast<float *>(lds_digits + (size_t)nb * 96);
-    float acc[NG][R];
+    float acc[NGT][R];  // group g: tensor g / NG, rows (g % NG) * R ..
 #pragma unroll
-    for (int g = 0; g < NG; ++g)
+    for (int g = 0; g < NGT; ++g)
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[g][r] = 0.0f;
+    float post = 1.0f;
+    if constexpr (POST) {  // requested first, needed last
+        float ss = 0.0f;
+        for (int i = lane; i < epi.ss_n; i += 64) ss += epi.ss_in[i];
+        post = 1.0f / sqrtf(wave_sum_f32(ss) * epi.ss_inv_dim + epi.eps);
+    }
 
     for (int seg0 = 0; seg0 < nb; seg0 += SEG) {
         const int seg_n = (nb - seg0 < SEG) ? nb - seg0 : SEG;
@@ -262,13 +280,13 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
         auto load_rows = [&](RowLoads<QT, BPL, R> &L, int g) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                int row = row0 + g * R + r;
+                int row = row0 + (g % NG) * R + r;
                 row = row < n_out ? row : n_out - 1;  // clamped; masked at the store
 #pragma unroll
                 for (int p = 0; p < BPL; ++p)
 #pragma unroll
                     for (int h = 0; h < NH; ++h)
-                        L.w[r][p][h] = __builtin_nontemporal_load(qs + ((size_t)row * NH + h) * nb + blk[p]);
+                        L.w[r][p][h] = __builtin_nontemporal_load(qs_t[NT == 1 ? 0 : g / NG] + ((size_t)row * NH + h) * nb + blk[p]);
             }
         };
         // Loads return in issue order, so the (L2 / L1 resident) digits, block sums and scales
@@ -277,7 +295,7 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
         // still in flight.
         v4i xd[BPL][NP];
         float sb[BPL];
-        v4i dtile[BPL];  // f16 scales of this lane's blocks for the 8 rows of the tile
+        v4i dtile[NT][BPL];  // f16 scales of this lane's blocks for the 8 rows of the tile
         v4i mtile[BPL];  // Q4_1: their f16 offsets
         float sxs[BPL];  // Q4_1: scale * block sum of the activation block
         RowLoads<QT, BPL, R> L[2];
@@ -300,7 +318,7 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
             }
             if (live) {
 #pragma unroll
-                for (int p = 0; p < BPL; ++p) dtile[p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+                for (int p = 0; p < BPL; ++p) dtile[0][p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
                 load_rows(L[0], 0);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -338,7 +356,8 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
 #pragma unroll
                 for (int j = 0; j < NP; ++j) xd[p][j] = digits[(size_t)j * nb + blk[p]];
                 sb[p] = xs[blk[p]];
-                dtile[p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+#pragma unroll
+                for (int t = 0; t < NT; ++t) dtile[t][p] = dsc_t[t][(size_t)(row0 >> 3) * nb + blk[p]];
                 if constexpr (Q41) {
                     mtile[p] = msc[(size_t)(row0 >> 3) * nb + blk[p]];
                     sxs[p] = xsum[blk[p]];
@@ -354,15 +373,15 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
             if constexpr (Q41) sxs[p] *= sb[p];
         }
 #pragma unroll
-        for (int g = 0; g < NG; ++g) {
-            if (g + 1 < NG) {
+        for (int g = 0; g < NGT; ++g) {
+            if (g + 1 < NGT) {
                 load_rows(L[(g + 1) & 1], g + 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
             const RowLoads<QT, BPL, R> &C = L[g & 1];
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const int tr = (row0 & 7) + g * R + r;  // row within the scale tile
+                const int tr = (row0 & 7) + (g % NG) * R + r;  // row within the scale tile
 #pragma unroll
                 for (int p = 0; p < BPL; ++p) {
                     float f;  // sum_k (weight) * X over the block
@@ -373,7 +392,7 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
                         block_dot_q8(C.w[r][p][0], C.w[r][p][NH - 1], reinterpret_cast<const v4i(&)[6]>(xd[p]), hi, lo);
                         f = fmaf((float)hi, 65536.0f, (float)lo);  // both terms exact in f32
                     }
-                    const uint32_t pair = (uint32_t)dtile[p][tr >> 1];
+                    const uint32_t pair = (uint32_t)dtile[g / NG][p][tr >> 1];
                     const float dv = half_bits_to_float((uint16_t)((tr & 1) ? pair >> 16 : pair & 0xFFFFu));
                     const float ds = dv * sb[p];
                     acc[g][r] = fmaf(ds, f, acc[g][r]);
@@ -386,14 +405,48 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
             }
         }
     }
+    __shared__ float res[NT][EPI != 0 ? 32 : 1];  // EPI: the workgroup's 32 outputs (per tensor)
 #pragma unroll
-    for (int g = 0; g < NG; ++g)
+    for (int g = 0; g < NGT; ++g)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const float v = wave_sum_f32(acc[g][r]);
-            const int row = row0 + g * R + r;
-            if (lane == 0 && row < n_out) y[row] = residual_base ? residual_base[(size_t)item * n_out + row] + v : v;
+            float v = wave_sum_f32(acc[g][r]);
+            if constexpr (POST) v *= post;
+            const int row = row0 + (g % NG) * R + r;
+            if constexpr (EPI != 2) {
+                if (lane == 0 && row < n_out) {
+                    if (residual_base) v = residual_base[(size_t)item * n_out + row] + v;
+                    y[row] = v;
+                }
+            }
+            if constexpr (EPI != 0) {
+                if (lane == 0) res[g / NG][row - blockIdx.x * 32] = v;
+            }
         }
+    if constexpr (EPI != 0) {  // n_out is a multiple of 32 here
+        __syncthreads();
+        if (threadIdx.x < 8) {  // one block of 32: eight lanes, four elements each
+            const int sub = threadIdx.x, e0 = sub * 4;
+            float f[4];
+            if constexpr (EPI == 1) {
+                const float4 gm = reinterpret_cast<const float4 *>(epi.gamma)[blockIdx.x * 8 + sub];
+                const float h[4] = {res[0][e0], res[0][e0 + 1], res[0][e0 + 2], res[0][e0 + 3]};
+                f[0] = h[0] * gm.x; f[1] = h[1] * gm.y; f[2] = h[2] * gm.z; f[3] = h[3] * gm.w;
+                float ss = h[0] * h[0] + h[1] * h[1] + h[2] * h[2] + h[3] * h[3];
+                ss += __builtin_bit_cast(float, pg_dpp8<0xB1>(__builtin_bit_cast(int, ss)));
+                ss += __builtin_bit_cast(float, pg_dpp8<0x4E>(__builtin_bit_cast(int, ss)));
+                ss += __builtin_bit_cast(float, pg_dpp8<0x141>(__builtin_bit_cast(int, ss)));
+                if (sub == 0) epi.ss_out[blockIdx.x] = ss;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float gv = res[0][e0 + e];
+                    f[e] = gv / (1.0f + expf(-gv)) * res[NT - 1][e0 + e];
+                }
+            }
+            pg_emit_digits<QT == 4>(f, 0, blockIdx.x, sub, n_out / 32, epi.out_digits, epi.out_xs);
+        }
+    }
 }
 
 template <int QT, int BPL, bool Q41>
@@ -410,13 +463,48 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
         const dim3 grid(grid_for(n_out, RWW), (unsigned)batch.count);                              \
         PG_TRY(pg_launch(ctx, QT == 4 ? (Q41 ? "gguf_gemv_q4_1" : "gguf_gemv_q4_0") : "gguf_gemv_q8_0", \
                          gguf_gemv_kernel<QT, BPL, RWW, RR, Q41>, grid, dim3(64), 0, qs, d, batch, \
-                         (int)n_out, nb, xd.digits, xd.xs, y, residual, m, (const float *)xd.xsum, (const float *)nullptr)); \
+                         (int)n_out, nb, xd.digits, xd.xs, y, residual, m, (const float *)xd.xsum, (const float *)nullptr, pg_gemv_epi{})); \
     } while (0)
     if (n_out / 8 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(8, R8);
     else if (n_out / 4 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(4, (R8 < 4 ? R8 : 4));
     else PG_GGUF_GEMV_LAUNCH(2, 2);
 #undef PG_GGUF_GEMV_LAUNCH
     return PG_OK;
+}
+
+// Q4_0 products whose output is the next product's digit input (see EPI at the kernel): a workgroup owns
+// 32 output rows as 32 / RW wavefronts.
+template <int BPL, int EPI, bool POST>
+pg_status launch_gemv_epi_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const pg_xdigits &xd,
+                              float *y, const float *residual, const pg_gemv_epi &epi) {
+    const int nb = (int)(k_in / 32);
+    const pg_gemv_batch one = {1, nullptr, nullptr, nullptr, 1};
+    constexpr int R8 = BPL <= 2 ? 8 : (BPL <= 4 ? 4 : 2);
+    const size_t want = (size_t)ctx->num_cu * 6;  // wavefronts wanted in the grid
+    const size_t rows = n_out * (EPI == 2 ? 2 : 1);
+#define PG_GGUF_GEMV_E_LAUNCH(RWW, RR)                                                                                            \
+    PG_TRY(pg_launch(ctx, EPI == 1 ? "gguf_gemv_q4_0_norm_digits" : "gguf_gemv_q4_0_swiglu_digits",                              \
+                     gguf_gemv_kernel<4, BPL, RWW, RR, false, false, 32 / RWW, EPI, POST>, dim3((unsigned)(n_out / 32)),          \
+                     dim3(64 * (32 / RWW)), 0, qs, d, one, (int)n_out, nb, xd.digits, xd.xs, y, residual, (const uint16_t *)nullptr, \
+                     (const float *)nullptr, (const float *)nullptr, epi))
+    if (rows / 8 >= want && EPI != 2) PG_GGUF_GEMV_E_LAUNCH(8, R8);
+    else if (rows / 4 >= want || BPL > 2) PG_GGUF_GEMV_E_LAUNCH(4, (R8 < 4 ? R8 : 4));  // (16 wavefronts leave 128 registers each)
+    else PG_GGUF_GEMV_E_LAUNCH(2, 2);
+#undef PG_GGUF_GEMV_E_LAUNCH
+    return PG_OK;
+}
+
+template <int EPI, bool POST>
+pg_status launch_gemv_epi(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const pg_xdigits &xd, float *y,
+                          const float *residual, const pg_gemv_epi &epi) {
+    size_t bpl = (k_in / 32 + 63) / 64;
+    if (bpl > 4) bpl = 4;
+    switch (bpl) {
+        case 1: return launch_gemv_epi_bpl<1, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
+        case 2: return launch_gemv_epi_bpl<2, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
+        case 3: return launch_gemv_epi_bpl<3, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
+        default: return launch_gemv_epi_bpl<4, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
+    }
 }
 
 // One row still in f32: the one-launch form (four or eight wavefronts per workgroup share the digits).
@@ -436,7 +524,7 @@ pg_status launch_gemv_f32x_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uin
         PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                \
         PG_TRY(pg_launch(ctx, name, kern, dim3(grid_for(n_out, RWW * NW)), dim3(64 * NW), lds, qs, d, one, (int)n_out, nb, \
                          (const int8_t *)nullptr, (const float *)nullptr, y, (const float *)nullptr,               \
-                         (const uint16_t *)nullptr, (const float *)nullptr, x_f32));                               \
+                         (const uint16_t *)nullptr, (const float *)nullptr, x_f32, pg_gemv_epi{}));                    \
     } while (0)
     if (n_out / 8 >= want) PG_GGUF_GEMV_X_LAUNCH(8, R8);
     else if (n_out / 4 >= want) PG_GGUF_GEMV_X_LAUNCH(4, (R8 < 4 ? R8 : 4));
@@ -509,6 +597,27 @@ pg_status pg_launch_x_to_digits(pg_ctx *ctx, const float *x_dev, size_t rows, si
         PG_TRY(pg_launch(ctx, "x_to_digits", x_to_digits_kernel<false>, grid, dim3(256), 0, x_dev, nb, xd.digits, xd.xs,
                          (float *)nullptr));
     return pg_launch_check("x_to_digits");
+}
+
+pg_status pg_launch_gguf_gemv_norm_digits(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
+                                          const pg_xdigits &xd, float *y, const float *residual, const float *gamma,
+                                          const pg_xdigits &out, float *ss_out) {
+    if (n_out % 32 != 0 || k_in % 32 != 0 || !gamma || (uintptr_t)gamma % 16 != 0 || !ss_out || !y)
+        return pg_fail(PG_EINVAL, "gguf_gemv (digits of the normalised output): [%zu, %zu] or an argument does not fit", n_out, k_in);
+    pg_gemv_epi epi = {};
+    epi.gamma = gamma; epi.out_digits = out.digits; epi.out_xs = out.xs; epi.ss_out = ss_out;
+    return launch_gemv_epi<1, false>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
+}
+
+pg_status pg_launch_gguf_gemv_swiglu_digits(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs_gate, const uint16_t *d_gate,
+                                            const uint8_t *qs_up, const uint16_t *d_up, const pg_xdigits &xd, const float *ss_in,
+                                            size_t ss_n, size_t ss_dim, float eps, const pg_xdigits &out) {
+    if (n_out % 32 != 0 || k_in % 32 != 0 || !ss_in || ss_n == 0 || ss_dim == 0)
+        return pg_fail(PG_EINVAL, "gguf_gemv (digits of SiLU(gate) * up): [%zu, %zu] or an argument does not fit", n_out, k_in);
+    pg_gemv_epi epi = {};
+    epi.qs1 = qs_up; epi.d1 = d_up; epi.out_digits = out.digits; epi.out_xs = out.xs;
+    epi.ss_in = ss_in; epi.ss_n = (int)ss_n; epi.ss_inv_dim = 1.0f / (float)ss_dim; epi.eps = eps;
+    return launch_gemv_epi<2, true>(ctx, n_out, k_in, qs_gate, d_gate, xd, nullptr, nullptr, epi);
 }
 
 pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in,

@@ -240,11 +240,34 @@ struct pg_gemv_batch {
     const int *expert_of;
     int x_row_div;
 };
+// What a product whose output feeds the next product does besides (see gguf_gemv_kernel).
+struct pg_gemv_epi {
+    const float *gamma;      // RMSNorm weights of the output row
+    int8_t *out_digits;      // the output (times gamma, or SiLU(gate) * up) as digits
+    float *out_xs;
+    float *ss_out;           // [n_out / 32] sums of squares of the output, one per block
+    const float *ss_in;      // the input row's sums of squares: the product is divided by its RMS
+    int ss_n;
+    float ss_inv_dim, eps;
+    const uint8_t *qs1;      // the second tensor (up) of the SiLU(gate) * up form
+    const uint16_t *d1;
+};
 // y[item][row] = product (+ residual[item][row] when `residual` is given).
 pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in,
                               const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
                               const pg_xdigits &xd, float *y, const float *residual = nullptr,
                               const uint16_t *m = nullptr);
+// Q4_0, one row: y = product (+ residual) as usual, and besides `out` = the digits of y * gamma and
+// ss_out[n_out / 32] = the sums of squares of y by block: RMSNorm(y) without a launch, its scalar factor
+// left to the consumer.  n_out a multiple of 32.
+pg_status pg_launch_gguf_gemv_norm_digits(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
+                                          const pg_xdigits &xd, float *y, const float *residual, const float *gamma,
+                                          const pg_xdigits &out, float *ss_out);
+// Q4_0, one row: out = digits of SiLU(g) * u with g, u = the products by gate and up, both divided by the
+// RMS of the input row (ss_in: ss_n partial sums of squares over ss_dim elements, eps).
+pg_status pg_launch_gguf_gemv_swiglu_digits(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs_gate, const uint16_t *d_gate,
+                                            const uint8_t *qs_up, const uint16_t *d_up, const pg_xdigits &xd, const float *ss_in,
+                                            size_t ss_n, size_t ss_dim, float eps, const pg_xdigits &out);
 // One activation row still in f32: digits made inside the product's own launch.  Only where the predicate holds.
 bool pg_gguf_gemv_takes_f32_row(int ggml_type, size_t n_out, size_t k_in, const float *x_f32);
 pg_status pg_launch_gguf_gemv_f32_row(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,

@@ -35,6 +35,7 @@ struct pg_llama_block {
     pg_rope *rope;
     const pg_gguf_tensor *w[7];  // q, k, v, o, gate, up, down (borrowed)
     float *attn_norm_w, *ffn_norm_w;
+    float *ss_part;  // one-token step: sums of squares of the attention output row, by block of 32
     float *arena;  // activations for seq_cap tokens
     size_t seq_cap;
     // One-token step: digit buffers for the three GEMV inputs (model_dim, q_dim, ffn) and the
@@ -855,6 +856,187 @@ void gqa_attention_mfma_kernel(attn_args aa, int n_items, int nkvh) {
     }
 }
 
+// ---- one query token, head size 64 or 128: the heads of a kv group together ----
+// A workgroup owns (kv head, split of the keys) and serves every query head of the group from one read
+// of the split's keys and values.  HD / 8 lanes share a key, eight dims each -- i .. i+3 and HD/2 + i ..
+// HD/2 + i+3, the pairs RoPE rotates, so that the raw projections of the new position are rotated in
+// registers.  A score is a sum over those lanes by DPP moves, and each such group of lanes runs its own
+// online softmax (running maximum, sum and row per head) over the keys it meets: no exchange at all until
+// the 64 (HD 128) or 128 (HD 64) groups of the workgroup meet once, in LDS.  Wavefront instructions, not
+// bytes, bound this kernel (a wavefront instruction takes four cycles and there are one or two wavefronts
+// per SIMD): fused multiply-adds, v_exp_f32 on base-2 arguments, U as a template parameter.  A split is
+// `tps` tiles of U rounds of 2048 / HD keys; every workgroup leaves (maximum, exp-sum, row) per head for
+// gqa_combine_kernel.
+constexpr int ATT_DEC_GC = 4;  // query heads per pass over the keys
+
+template <int LPK>
+__device__ __forceinline__ float lanes_sum_f32(float v) {  // over aligned groups of LPK = 8 or 16 lanes, in every lane
+    auto mv = [](float x, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, false));
+    };
+    v += mv(v, std::integral_constant<int, 0xB1>{});
+    v += mv(v, std::integral_constant<int, 0x4E>{});
+    v += mv(v, std::integral_constant<int, 0x141>{});
+    if constexpr (LPK == 16) v += mv(v, std::integral_constant<int, 0x140>{});
+    return v;
+}
+
+// e^x for x <= 0 (or -inf -> 0) in two instructions
+__device__ __forceinline__ float exp_neg(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896341f); }
+
+template <int HD, int U>
+__global__ __launch_bounds__(256) void gqa_decode_kernel(attn_args aa, int nkv, int tps) {
+    constexpr int LPK = HD / 8, KPW = 64 / LPK, ROWS = 4 * KPW, GC = ATT_DEC_GC, HALF = HD / 2, TK = U * ROWS;
+    __shared__ __attribute__((aligned(16))) float xch[GC][ROWS][HD];  // 32 KB: each key row's partial output rows
+    __shared__ float wm[GC][ROWS], wl[GC][ROWS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kvh = blockIdx.x % nkv, split = blockIdx.x / nkv;
+    const int li = lane % LPK, krow = lane / LPK;
+    const int G = aa.group, splits = aa.splits;
+    int kend = aa.len;
+    if (aa.mask_kind != 0) kend = min(kend, aa.offset + 1);
+    const bool fused = aa.raw_q != nullptr;
+    const float *kbase = aa.kc + (size_t)kvh * aa.k_stride + 4 * li;
+    const float *vbase = aa.vc + (size_t)kvh * aa.v_stride + 4 * li;
+    // the lane's eight dims of a head row after RoPE (the operations of rope_kernel in the same order)
+    auto rot = [&](const float *row, float4 &lo, float4 &hi) {
+        const float4 x0 = *reinterpret_cast<const float4 *>(row + 4 * li), x1 = *reinterpret_cast<const float4 *>(row + HALF + 4 * li);
+        const float4 c = *reinterpret_cast<const float4 *>(aa.rope_c + 4 * li), sn = *reinterpret_cast<const float4 *>(aa.rope_s + 4 * li);
+        lo.x = x0.x * c.x - x1.x * sn.x; lo.y = x0.y * c.y - x1.y * sn.y; lo.z = x0.z * c.z - x1.z * sn.z; lo.w = x0.w * c.w - x1.w * sn.w;
+        hi.x = x0.x * sn.x + x1.x * c.x; hi.y = x0.y * sn.y + x1.y * c.y; hi.z = x0.z * sn.z + x1.z * c.z; hi.w = x0.w * sn.w + x1.w * c.w;
+    };
+    for (int hc = 0; hc < G; hc += GC) {
+        float4 q0[GC], q1[GC];
+#pragma unroll
+        for (int h = 0; h < GC; ++h) {
+            q0[h] = q1[h] = float4{0.f, 0.f, 0.f, 0.f};
+            if (hc + h < G) {
+                const size_t qh = (size_t)kvh * G + hc + h;
+                if (fused) {
+                    rot(aa.raw_q + qh * HD, q0[h], q1[h]);
+                } else {
+                    q0[h] = *reinterpret_cast<const float4 *>(aa.q + qh * HD + 4 * li);
+                    q1[h] = *reinterpret_cast<const float4 *>(aa.q + qh * HD + HALF + 4 * li);
+                }
+            }
+        }
+        float m_run[GC], l_run[GC], acc[GC][8];
+#pragma unroll
+        for (int h = 0; h < GC; ++h) {
+            m_run[h] = -INFINITY;
+            l_run[h] = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[h][j] = 0.f;
+        }
+        for (int t = 0; t < tps; ++t) {
+            const int kb = (split * tps + t) * TK;
+            if (kb >= kend) break;
+            float4 k0[U], k1[U], v0[U], v1[U];
+            bool live[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                k0[u] = k1[u] = v0[u] = v1[u] = float4{0.f, 0.f, 0.f, 0.f};
+                const int kt = kb + (u * 4 + wave) * KPW + krow;
+                live[u] = kt < kend && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, aa.gbits, 0, kt);
+                if (live[u]) {
+                    if (fused && kt == aa.new_pos) {
+                        // not in the cache yet: made from the projections, and stored by this workgroup, the only
+                        // one of its kv head that meets the position
+                        rot(aa.raw_k + (size_t)kvh * HD, k0[u], k1[u]);
+                        v0[u] = *reinterpret_cast<const float4 *>(aa.raw_v + (size_t)kvh * HD + 4 * li);
+                        v1[u] = *reinterpret_cast<const float4 *>(aa.raw_v + (size_t)kvh * HD + HALF + 4 * li);
+                        if (hc == 0) {
+                            float *kn = aa.k_new + (size_t)kvh * aa.k_stride + 4 * li, *vn = aa.v_new + (size_t)kvh * aa.v_stride + 4 * li;
+                            *reinterpret_cast<float4 *>(kn) = k0[u]; *reinterpret_cast<float4 *>(kn + HALF) = k1[u];
+                            *reinterpret_cast<float4 *>(vn) = v0[u]; *reinterpret_cast<float4 *>(vn + HALF) = v1[u];
+                        }
+                    } else {
+                        typedef float f4v __attribute__((ext_vector_type(4)));
+                        const f4v *kr = reinterpret_cast<const f4v *>(kbase + (size_t)kt * HD);
+                        const f4v *vr = reinterpret_cast<const f4v *>(vbase + (size_t)kt * HD);
+                        const f4v a = __builtin_nontemporal_load(kr), b = __builtin_nontemporal_load(kr + HALF / 4);
+                        const f4v c = __builtin_nontemporal_load(vr), d = __builtin_nontemporal_load(vr + HALF / 4);
+                        k0[u] = float4{a.x, a.y, a.z, a.w}; k1[u] = float4{b.x, b.y, b.z, b.w};
+                        v0[u] = float4{c.x, c.y, c.z, c.w}; v1[u] = float4{d.x, d.y, d.z, d.w};
+                    }
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < GC; ++h) {
+                float sc[U], tmax = -INFINITY;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    float dot = q0[h].x * k0[u].x;
+                    dot = fmaf(q0[h].y, k0[u].y, dot); dot = fmaf(q0[h].z, k0[u].z, dot); dot = fmaf(q0[h].w, k0[u].w, dot);
+                    dot = fmaf(q1[h].x, k1[u].x, dot); dot = fmaf(q1[h].y, k1[u].y, dot);
+                    dot = fmaf(q1[h].z, k1[u].z, dot); dot = fmaf(q1[h].w, k1[u].w, dot);
+                    dot = lanes_sum_f32<LPK>(dot);
+                    float sv = dot * aa.scale;
+                    if (aa.logit_cap > 0.f) sv = aa.logit_cap * tanhf(sv / aa.logit_cap);
+                    sc[u] = live[u] ? sv : -INFINITY;
+                    tmax = fmaxf(tmax, sc[u]);
+                }
+                // this group of lanes' own running maximum: nothing crosses to the other keys' lanes
+                const float m_new = fmaxf(m_run[h], tmax);
+                const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // (all hidden so far: every term below is e^-inf = 0)
+                const float alpha = exp_neg(m_run[h] - m_ref);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[h][j] *= alpha;
+                l_run[h] *= alpha;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const float pv = exp_neg(sc[u] - m_ref);
+                    l_run[h] += pv;
+                    acc[h][0] = fmaf(pv, v0[u].x, acc[h][0]); acc[h][1] = fmaf(pv, v0[u].y, acc[h][1]);
+                    acc[h][2] = fmaf(pv, v0[u].z, acc[h][2]); acc[h][3] = fmaf(pv, v0[u].w, acc[h][3]);
+                    acc[h][4] = fmaf(pv, v1[u].x, acc[h][4]); acc[h][5] = fmaf(pv, v1[u].y, acc[h][5]);
+                    acc[h][6] = fmaf(pv, v1[u].z, acc[h][6]); acc[h][7] = fmaf(pv, v1[u].w, acc[h][7]);
+                }
+                m_run[h] = m_new;
+            }
+        }
+        // the groups' partial rows, maxima and sums meet in LDS
+        const int row = wave * KPW + krow;
+#pragma unroll
+        for (int h = 0; h < GC; ++h) {
+            float *dst = &xch[h][row][4 * li];
+            *reinterpret_cast<float4 *>(dst) = float4{acc[h][0], acc[h][1], acc[h][2], acc[h][3]};
+            *reinterpret_cast<float4 *>(dst + HALF) = float4{acc[h][4], acc[h][5], acc[h][6], acc[h][7]};
+            if (li == 0) {
+                wm[h][row] = m_run[h];
+                wl[h][row] = l_run[h];
+            }
+        }
+        __syncthreads();
+        if (tid < GC * HD / 4) {
+            const int h = tid / (HD / 4), i4 = tid % (HD / 4);
+            if (hc + h < G) {
+                float M = -INFINITY;
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) M = fmaxf(M, wm[h][r]);
+                const float m_ref = M == -INFINITY ? 0.f : M;
+                float L = 0.f;
+                float4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    const float w = exp_neg(wm[h][r] - m_ref);
+                    const float4 a = *reinterpret_cast<const float4 *>(&xch[h][r][4 * i4]);
+                    L = fmaf(w, wl[h][r], L);
+                    o.x = fmaf(w, a.x, o.x); o.y = fmaf(w, a.y, o.y); o.z = fmaf(w, a.z, o.z); o.w = fmaf(w, a.w, o.w);
+                }
+                float *dst = aa.part + (((size_t)kvh * G + hc + h) * splits + split) * (size_t)(HD + 2);
+                if (i4 == 0) {
+                    dst[0] = M;
+                    dst[1] = L;
+                }
+                *reinterpret_cast<float2 *>(dst + 2 + 4 * i4) = float2{o.x, o.y};
+                *reinterpret_cast<float2 *>(dst + 4 + 4 * i4) = float2{o.z, o.w};
+            }
+        }
+        if (hc + GC < G) __syncthreads();  // the next pass of heads writes xch again
+    }
+}
+
 constexpr int ATT_SPLITS_MAX = 2048;
 
 // Merge the splits of one (query token, query head) row: with M = max of the split maxima and
@@ -901,6 +1083,73 @@ __global__ __launch_bounds__(128) void gqa_combine_kernel(const float *__restric
             const int e4 = qh * (hd / 4) + i4;  // float4 index within the row
             pg_emit_digits<DIG == 1>(o, qt, e4 >> 3, e4 & 7, nqh * hd / 32, digits, xs);
         }
+    }
+}
+
+// The same merge for head sizes 64 and 128 and at most 64 splits, every load in flight at once: thread =
+// (float4 of the row, slice of the splits), the slices' sums meet in LDS.  Splits are still added in
+// ascending order within a slice and the slices in ascending order: the result does not depend on timing.
+template <int HD, int DIG>
+__global__ __launch_bounds__(256) void gqa_combine_few_kernel(const float *__restrict__ part, int splits, float *__restrict__ out,
+                                                              int accumulate, int nqh, int8_t *__restrict__ digits,
+                                                              float *__restrict__ xs) {
+    constexpr int UNITS = HD / 4, SLICES = 256 / UNITS, NS = 64 / SLICES;  // 8 slices x 8 splits, or 16 x 4
+    __shared__ float sm[64], sl[64];
+    __shared__ float ex[SLICES][UNITS][5];
+    const float *p = part + (size_t)blockIdx.x * splits * (HD + 2);
+    const int tid = threadIdx.x, i4 = tid % UNITS, slice = tid / UNITS;
+    float2 ra[NS], rb[NS];
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {  // this thread's splits: slice * NS + j
+        const int sp = slice * NS + j;
+        ra[j] = rb[j] = float2{0.f, 0.f};
+        if (sp < splits) {
+            ra[j] = *reinterpret_cast<const float2 *>(p + (size_t)sp * (HD + 2) + 2 + 4 * i4);
+            rb[j] = *reinterpret_cast<const float2 *>(p + (size_t)sp * (HD + 2) + 4 + 4 * i4);
+        }
+    }
+    if (tid < 64) {
+        const float2 ml = tid < splits ? *reinterpret_cast<const float2 *>(p + (size_t)tid * (HD + 2)) : float2{-INFINITY, 0.f};
+        sm[tid] = ml.x;
+        sl[tid] = ml.y;
+    }
+    __syncthreads();
+    const float M = wave_max_f32(sm[tid & 63]);
+    const float m_ref = M == -INFINITY ? 0.f : M;
+    float L = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {
+        const int sp = slice * NS + j;
+        const float w = exp_neg(sm[sp] - m_ref);  // (splits past the last: e^-inf = 0)
+        L = fmaf(w, sl[sp], L);
+        o[0] = fmaf(w, ra[j].x, o[0]); o[1] = fmaf(w, ra[j].y, o[1]); o[2] = fmaf(w, rb[j].x, o[2]); o[3] = fmaf(w, rb[j].y, o[3]);
+    }
+    float *mine = ex[slice][i4];
+    mine[0] = L; mine[1] = o[0]; mine[2] = o[1]; mine[3] = o[2]; mine[4] = o[3];
+    __syncthreads();
+    if (tid >= UNITS) return;  // whole 8-lane groups stay: UNITS is a multiple of 8
+    L = 0.f;
+    o[0] = o[1] = o[2] = o[3] = 0.f;
+#pragma unroll
+    for (int sx = 0; sx < SLICES; ++sx) {
+        const float *e = ex[sx][i4];
+        L += e[0]; o[0] += e[1]; o[1] += e[2]; o[2] += e[3]; o[3] += e[4];
+    }
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] *= inv;
+    if constexpr (DIG == 0) {
+        float4 *dst = reinterpret_cast<float4 *>(out + (size_t)blockIdx.x * HD) + i4;
+        float4 r = {o[0], o[1], o[2], o[3]};
+        if (accumulate) {
+            const float4 old = *dst;
+            r.x += old.x; r.y += old.y; r.z += old.z; r.w += old.w;
+        }
+        *dst = r;
+    } else {
+        const int qt = blockIdx.x / nqh, qh = blockIdx.x - qt * nqh;
+        const int e4 = qh * UNITS + i4;  // float4 index within the row
+        pg_emit_digits<DIG == 1>(o, qt, e4 >> 3, e4 & 7, nqh * HD / 32, digits, xs);
     }
 }
 
@@ -1012,8 +1261,27 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     // short kernel handles with every load in flight at once.
     const size_t rows = seq_q * nqh, keys_per_round = 256 / (size_t)lanes;
     size_t chunk, splits;
-    bool short_kernel = false, tiled_kernel = false;
-    if (attention_is_short(ctx, rows, len, hd)) {
+    bool short_kernel = false, tiled_kernel = false, decode_kernel = false;
+    int dec_u = 1, dec_tps = 1;
+    const uintptr_t align_all = (uintptr_t)q | (uintptr_t)out | (uintptr_t)kc->k | (uintptr_t)vc->v |
+                                (rope_fusion ? (uintptr_t)rope_fusion->raw_q | (uintptr_t)rope_fusion->raw_k | (uintptr_t)rope_fusion->raw_v |
+                                                   (uintptr_t)rope_fusion->rope_c | (uintptr_t)rope_fusion->rope_s
+                                             : 0);
+    if (seq_q == 1 && (hd == 64 || hd == 128) && align_all % 16 == 0 && attention_is_short(ctx, rows, len, hd)) {
+        // one token: the heads of a kv group share a workgroup
+        const size_t nkv = kc->num_kv_heads, tile_rows = 2048 / hd;
+        const size_t kend = mask_kind != 0 && offset + 1 < len ? offset + 1 : len;
+        auto tiles_of = [&](size_t u) { return (kend + u * tile_rows - 1) / (u * tile_rows); };
+        size_t u = 4;
+        while (u > 1 && nkv * tiles_of(u) < (size_t)ctx->num_cu) u >>= 1;  // fewer rounds per tile, more workgroups
+        const size_t tiles = tiles_of(u);
+        size_t tps = nkv * tiles > 2 * (size_t)ctx->num_cu ? (nkv * tiles + 2 * ctx->num_cu - 1) / (2 * ctx->num_cu) : 1;
+        if ((tiles + tps - 1) / tps > (size_t)ATT_SPLITS_MAX) tps = (tiles + ATT_SPLITS_MAX - 1) / ATT_SPLITS_MAX;
+        splits = (tiles + tps - 1) / tps;
+        chunk = tps * u * tile_rows;
+        dec_u = (int)u; dec_tps = (int)tps;
+        decode_kernel = true;
+    } else if (attention_is_short(ctx, rows, len, hd)) {
         chunk = ATT_SHORT_ROUNDS * keys_per_round;
         splits = (len + chunk - 1) / chunk;
         short_kernel = true;
@@ -1028,7 +1296,7 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     }
     if (splits > (size_t)ATT_SPLITS_MAX) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: cache of %zu positions is too long", len);
     aa.chunk = (int)chunk; aa.splits = (int)splits;
-    const size_t part_bytes = splits > 1 ? pg_round_up(rows * splits * (hd + 2) * sizeof(float), 256) : 0;
+    const size_t part_bytes = splits > 1 || decode_kernel ? pg_round_up(rows * splits * (hd + 2) * sizeof(float), 256) : 0;
     const size_t bits_words = mask_kind == PG_MASK_LOCAL_GLOBAL ? (len + 31) / 32 : 0;
     if (part_bytes + bits_words) {
         void *ws = nullptr;
@@ -1048,13 +1316,20 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     }
     const dim3 grid((unsigned)seq_q, (unsigned)nqh, (unsigned)splits);
     if (rope_fusion) {
-        if (!short_kernel || seq_q != 1 || hd % 8 != 0) return pg_fail(PG_EINVAL, "gqa_attention: RoPE fusion needs the one-token kernel");
+        if (!(short_kernel || decode_kernel) || seq_q != 1 || hd % 8 != 0)
+            return pg_fail(PG_EINVAL, "gqa_attention: RoPE fusion needs a one-token kernel");
         aa.raw_q = rope_fusion->raw_q; aa.raw_k = rope_fusion->raw_k; aa.raw_v = rope_fusion->raw_v;
         aa.rope_c = rope_fusion->rope_c; aa.rope_s = rope_fusion->rope_s;
         aa.k_new = rope_fusion->k_new; aa.v_new = rope_fusion->v_new;
         aa.new_pos = rope_fusion->new_pos;
     }
-    if (short_kernel) {
+    if (decode_kernel) {
+        if (kc->num_kv_heads * splits >= (1ull << 31)) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: grid too large");
+        auto *kern = hd == 64 ? (dec_u == 4 ? gqa_decode_kernel<64, 4> : (dec_u == 2 ? gqa_decode_kernel<64, 2> : gqa_decode_kernel<64, 1>))
+                              : (dec_u == 4 ? gqa_decode_kernel<128, 4> : (dec_u == 2 ? gqa_decode_kernel<128, 2> : gqa_decode_kernel<128, 1>));
+        PG_TRY(pg_launch(ctx, "gqa_decode", kern, dim3((unsigned)(kc->num_kv_heads * splits)), dim3(256), 0, aa, (int)kc->num_kv_heads,
+                         dec_tps));
+    } else if (short_kernel) {
         const size_t sets = kc->num_kv_heads * splits, members = (nqh / kc->num_kv_heads) * seq_q;
         const size_t wgs = (sets + 7) / 8 * 8 * members;
         if (wgs >= (1ull << 31)) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: grid too large");
@@ -1077,7 +1352,13 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
         PG_TRY(pg_launch(ctx, "gqa_attention_tiled", kern, grid_t, dim3(256), lds_t, aa));
     } else
         PG_TRY(pg_launch(ctx, "gqa_attention", gqa_attention_kernel, grid, dim3(256), (256 + ATT_RED + chunk) * sizeof(float), aa));
-    if (splits > 1) {
+    if (decode_kernel && splits <= 64) {  // (decode_kernel: `out` is 16-byte aligned)
+        const int dg = !xd ? 0 : (digit_kind == PG_GGML_Q4_0 ? 1 : 2);
+        auto *kern = hd == 64 ? (dg == 0 ? gqa_combine_few_kernel<64, 0> : (dg == 1 ? gqa_combine_few_kernel<64, 1> : gqa_combine_few_kernel<64, 2>))
+                              : (dg == 0 ? gqa_combine_few_kernel<128, 0> : (dg == 1 ? gqa_combine_few_kernel<128, 1> : gqa_combine_few_kernel<128, 2>));
+        PG_TRY(pg_launch(ctx, xd ? "gqa_combine_digits" : "gqa_combine", kern, dim3((unsigned)rows), dim3(256), 0, (const float *)aa.part,
+                         (int)splits, out, accumulate, (int)nqh, xd ? xd->digits : (int8_t *)nullptr, xd ? xd->xs : (float *)nullptr));
+    } else if (splits > 1 || decode_kernel) {
         auto *kern = !xd ? gqa_combine_kernel<0> : (digit_kind == PG_GGML_Q4_0 ? gqa_combine_kernel<1> : gqa_combine_kernel<2>);
         PG_TRY(pg_launch(ctx, xd ? "gqa_combine_digits" : "gqa_combine", kern, dim3((unsigned)rows), dim3(128), 0,
                          (const float *)aa.part, (int)splits, (int)hd, out, accumulate, (int)nqh, xd ? xd->digits : nullptr,
@@ -1433,7 +1714,7 @@ PG_API pg_status pg_llama_block_create(pg_ctx *ctx, size_t model_dim, size_t num
     const size_t o_q = pg_xdigits_bytes(1, model_dim), o_f = o_q + pg_xdigits_bytes(1, q_dim);
     const size_t o_tab = o_f + pg_xdigits_bytes(1, ffn_dim);
     const size_t tab_bytes = pg_round_up((2 * items + 4) * sizeof(void *) + items * sizeof(int), 256);
-    const size_t total = o_tab + tab_bytes;
+    const size_t total = o_tab + tab_bytes + pg_round_up(model_dim / 32 * sizeof(float), 256);
     hipError_t e = hipMalloc(&b->dec, total);
     if (e == hipSuccess) e = hipMemsetAsync(b->dec, 0, total, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
@@ -1453,6 +1734,7 @@ PG_API pg_status pg_llama_block_create(pg_ctx *ctx, size_t model_dim, size_t num
     b->qs_gu = reinterpret_cast<const uint8_t *const *>(tab + 2 * items);
     b->d_gu = reinterpret_cast<const uint16_t *const *>(tab + 2 * items + 2);
     b->item_ids = reinterpret_cast<const int *>(tab + 2 * items + 4);
+    b->ss_part = reinterpret_cast<float *>(base + o_tab + tab_bytes);
     *out = b;
     return PG_OK;
 }
@@ -1587,6 +1869,16 @@ static pg_status block_forward_one_token(pg_ctx *ctx, pg_llama_block *b, const f
         cache->len = offset + 1;
         PG_TRY(launch_attention(ctx, q_rope, cache, cache, b->nqh, 1, 1.0f / sqrtf((float)hd), PG_MASK_CAUSAL, offset, 0, 0, 0.0f,
                                 attn, 0, &b->xd_q, kind));
+    }
+    if (kind == PG_GGML_Q4_0 && d % 32 == 0 && ffn % 32 == 0) {
+        // h1 = h + attn . Wo, stored, and also left as the digits of h1 * (norm weights) with its sums of
+        // squares; gate and up divide by the RMS themselves and leave the digits of SiLU(g) * u: two
+        // launches (RMSNorm, SiLU.up) fewer
+        PG_TRY(pg_launch_gguf_gemv_norm_digits(ctx, d, q_dim, b->w[3]->qs, b->w[3]->d, b->xd_q, h1, h_dev, b->ffn_norm_w, b->xd_d,
+                                               b->ss_part));
+        PG_TRY(pg_launch_gguf_gemv_swiglu_digits(ctx, ffn, d, b->w[4]->qs, b->w[4]->d, b->w[5]->qs, b->w[5]->d, b->xd_d, b->ss_part,
+                                                 d / 32, d, b->eps, b->xd_f));
+        return pg_launch_gguf_gemv(ctx, PG_GGML_Q4_0, d, ffn, b->w[6]->qs, b->w[6]->d, one, b->xd_f, out_dev, h1);
     }
     // h1 = h + attn . Wo
     PG_TRY(pg_launch_gguf_gemv(ctx, b->w[3]->ggml_type, d, q_dim, b->w[3]->qs, b->w[3]->d, one, b->xd_q, h1, h_dev));

@@ -217,6 +217,40 @@ def test_gqa_attention_local_global(ctx, orc):
     assert (got == _attention_case(ctx, orc, 8, 2, 64, 40, 90, M.causal(50), None, 77)).all()
 
 
+def test_gqa_attention_one_token_heads_of_a_group_together(ctx, orc):
+    """One query token with head size 64 or 128: a workgroup serves all query heads of a kv group (in passes of
+    four) over one split of the keys, and the last workgroup of a kv head to finish merges the splits.  Lengths
+    around the tile sizes (16 / 32 keys a round, up to four rounds a tile), one tile and several per split,
+    groups of 1, 2, 4, 5 and 8 heads, every mask kind, a cache longer than the token may see, a logit cap, and
+    the same call twice in a row (the arrival counters must be back at zero)."""
+    from peregrine_amd import llama
+    M = llama.AttentionMask
+    seed = 300
+    for hd in (128, 64):
+        for length in (1, 15, 16, 17, 63, 64, 65, 300):
+            say(f"one-token attention hd={hd} len={length}")
+            _attention_case(ctx, orc, 8, 2, hd, 1, length, M.none(), None, seed)
+            _attention_case(ctx, orc, 8, 2, hd, 1, length, M.causal(length - 1), None, seed + 1,
+                            appends=(1, length - 1) if length > 1 else None)
+            seed += 2
+    for nqh, nkvh in ((4, 4), (4, 2), (10, 2), (16, 2), (5, 1)):
+        say(f"one-token attention heads {nqh}/{nkvh}")
+        _attention_case(ctx, orc, nqh, nkvh, 128, 1, 200, M.causal(199), None, seed)
+        _attention_case(ctx, orc, nqh, nkvh, 64, 1, 333, M.causal(332), 4.0, seed + 1)
+        seed += 2
+    say("one-token attention, masks")
+    _attention_case(ctx, orc, 8, 2, 128, 1, 500, M.causal(250), None, seed)                       # half of the cache is ahead
+    _attention_case(ctx, orc, 8, 2, 128, 1, 500, M.causal_sliding_window(499, 100, 4), None, seed + 1)  # whole tiles hidden
+    _attention_case(ctx, orc, 8, 2, 64, 1, 500, M.causal_sliding_window(450, 0, 0), None, seed + 2)      # sees itself only
+    _attention_case(ctx, orc, 8, 2, 64, 1, 700, M.local_global(699, 37, [0, 5, 64, 65, 300, 698, 5000]), 2.0, seed + 3)
+    _attention_case(ctx, orc, 32, 8, 128, 1, 1025, M.causal(1024), None, seed + 4)              # the benchmark's step
+    say("one-token attention, several tiles per split")
+    _attention_case(ctx, orc, 32, 8, 128, 1, 5000, M.causal(4999), None, seed + 5, appends=(4096, 904))
+    _attention_case(ctx, orc, 64, 16, 64, 1, 6001, M.none(), None, seed + 6)
+    a = _attention_case(ctx, orc, 8, 1, 128, 1, 9000, M.causal(8999), None, seed + 7)
+    assert (a == _attention_case(ctx, orc, 8, 1, 128, 1, 9000, M.causal(8999), None, seed + 7)).all()
+
+
 def test_gqa_attention_long_cache_splits_keys(ctx, orc):
     """A long cache under one query row: the keys are cut into many splits and merged."""
     from peregrine_amd import llama
@@ -284,6 +318,13 @@ def test_llama_block_long_prefill_head_128(ctx, orc):
     """A prefill long enough for the tiled attention kernel and the many-token-tile product
     order (140 tokens x 4 heads of 128), then a decode step on top of it."""
     _block_case(ctx, orc, 512, 4, 2, 128, 768, 2, (140, 1), max_seq=160, seed=21)
+
+
+@pytest.mark.parametrize("typ", [2, 8])
+def test_llama_block_decode_steps_head_64_group_of_3(ctx, orc, typ):
+    """Several one-token steps in a row with the grouped one-token attention (head size 64, three query heads per
+    kv head) and, for Q4_0, the products that leave their output as the next product's digits."""
+    _block_case(ctx, orc, 384, 6, 2, 64, 640, typ, (7, 1, 1, 1, 20, 1), seed=31)
 
 
 def test_llama_block_q4_1_weights(ctx, orc):
