@@ -199,6 +199,8 @@ __device__ __forceinline__ float wave_sum_f32(float v) { return pg_wave_sum_f32(
 
 typedef const v4i __attribute__((address_space(1))) *gv4i_ptr;  // loads known to be global, not flat
 
+constexpr int GGUF_LDSX_CPT = 6;  // XM 2: 16-byte units of digits and scales each thread carries into LDS
+
 template <int QT, int BPL, int R>
 struct RowLoads {
     v4i w[R][BPL][QT == 8 ? 2 : 1];
@@ -223,21 +225,29 @@ struct RowLoads {
 //   2  the workgroup multiplies by two tensors (gate, then up = epi.qs1 / d1) and leaves only the digits
 //      of silu(gate) * up (src/models/llama/decoder.rs:143-150).
 // POST: the product is multiplied by 1 / sqrt(sum(ss_in[0 .. ss_n)) * ss_inv_dim + eps) before anything else.
-template <int QT, int BPL, int RW, int R, bool Q41 = false, bool XF32 = false, int NW = 1, int EPI = 0, bool POST = false>
+// XM 2: the row's digits are read as usual, but once per workgroup, into LDS, for its NW wavefronts: with
+// few rows per wavefront and a long row (K = 14336 is 36 KB of digits, more than the CU's vector cache)
+// every wavefront would otherwise pull the whole of them through L2 again.
+// NORM (with XM 1): the row is RMSNorm(x_f32) with the weights epi.gamma (src/nn.rs:560-652): the digits are
+// those of x * gamma, the sum of squares rides on the digits' barrier, and the scalar factor is applied to
+// the product: the norm costs no launch and no extra barrier.
+template <int QT, int BPL, int RW, int R, bool Q41 = false, int XM = 0, int NW = 1, int EPI = 0, bool POST = false, bool NORM = false>
 __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
     const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0, pg_gemv_batch batch,
     int n_out, int nb, const int8_t *__restrict__ digits_base, const float *__restrict__ xs_base,
     float *__restrict__ y_base, const float *__restrict__ residual_base, const uint16_t *__restrict__ m0,
     const float *__restrict__ xsum_base, const float *__restrict__ x_f32, pg_gemv_epi epi) {
     constexpr int SEG = 64 * BPL;  // blocks per K segment
+    constexpr bool XF32 = XM == 1, LDSX = XM == 2;
     constexpr int NT = EPI == 2 ? 2 : 1;  // tensors per workgroup
     constexpr int NG = RW / R, NGT = NG * NT;
-    static_assert(EPI == 0 || (!XF32 && !Q41 && NW * RW == 32), "an output block of 32 rows per workgroup");
-    static_assert(EPI != 0 || XF32 || NW == 1, "several wavefronts per workgroup only where they share something");
+    static_assert(EPI == 0 || (XM == 0 && !Q41 && NW * RW == 32), "an output block of 32 rows per workgroup");
+    static_assert(EPI != 0 || XM != 0 || NW == 1, "several wavefronts per workgroup only where they share something");
     constexpr int NH = QT == 8 ? 2 : 1;
     constexpr int NP = QT == 8 ? 6 : 5;  // digit planes
-    static_assert(!XF32 || !Q41, "the one-launch form has no block sums");
-    extern __shared__ __attribute__((aligned(16))) char lds_digits[];  // XF32: [6 planes][nb][16 B], then nb scales
+    static_assert(XM == 0 || !Q41, "the LDS forms hold no block sums");
+    static_assert(!NORM || (XM == 1 && !POST), "the norm is folded in where the row arrives in f32");
+    extern __shared__ __attribute__((aligned(16))) char lds_digits[];  // XM 1, 2: [6 planes][nb][16 B], then nb scales
     const int item = blockIdx.y;
     const uint8_t *qs_any = qs0;
     const uint16_t *d_any = d0;
@@ -299,21 +309,18 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
         v4i mtile[BPL];  // Q4_1: their f16 offsets
         float sxs[BPL];  // Q4_1: scale * block sum of the activation block
         RowLoads<QT, BPL, R> L[2];
-        if constexpr (XF32) {
-            // weights first: they come from HBM and take longest (a wavefront whose rows all lie past
-            // n_out -- the last workgroup's spare ones -- only helps with the digits)
-            // Loads return in issue order: the row (a few KiB, from L2) is requested first so that the digit
-            // arithmetic can start as soon as it is there, the weight rows (from HBM) right behind it so
-            // that they fly meanwhile.  (A wavefront whose rows all lie past n_out -- the last workgroup's
-            // spare ones -- only helps with the digits.)
+        if constexpr (LDSX) {
+            // Loads return in issue order: the digits (from L2) are requested first, the weight rows (from HBM)
+            // right behind them, and only the digits are waited for before the workgroup's one barrier.
+            constexpr int CPT = GGUF_LDSX_CPT;  // 16-byte units per thread: digit planes, then the block scales
             const bool live = row0 < n_out;
-            const int sub = threadIdx.x & 7, bfirst = (int)threadIdx.x >> 3;
-            float4 xv[4];
+            const int nd = NP * nb, nu = nd + (nb >> 2);
+            v4i cp[CPT];
             if (seg0 == 0) {
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int b = bfirst + u * 8 * NW;
-                    xv[u] = reinterpret_cast<const float4 *>(x_f32)[(size_t)(b < nb ? b : 0) * 8 + sub];
+                for (int c = 0; c < CPT; ++c) {
+                    const int u = (int)threadIdx.x + c * 64 * NW;
+                    cp[c] = u < nd ? digits[u] : ((gv4i_ptr)(uintptr_t)xs)[u < nu ? u - nd : 0];
                 }
             }
             if (live) {
@@ -322,26 +329,75 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
                 load_rows(L[0], 0);
             }
             __builtin_amdgcn_sched_barrier(0);
+            if (seg0 == 0) {
+#pragma unroll
+                for (int c = 0; c < CPT; ++c) {
+                    const int u = (int)threadIdx.x + c * 64 * NW;
+                    if (u < nd) *reinterpret_cast<v4i *>(ldig + (size_t)u * 16) = cp[c];
+                    else if (u < nu) *reinterpret_cast<v4i *>(reinterpret_cast<char *>(lxs) + (size_t)(u - nd) * 16) = cp[c];
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier" ::: "memory");  // (the weight loads stay in flight)
+            }
+            if (!live) return;  // after the workgroup's only barrier
+#pragma unroll
+            for (int p = 0; p < BPL; ++p) {
+#pragma unroll
+                for (int j = 0; j < NP; ++j) xd[p][j] = *reinterpret_cast<const v4i *>(ldig + ((size_t)j * nb + blk[p]) * 16);
+                sb[p] = lxs[blk[p]];
+            }
+        } else if constexpr (XF32) {
+            // Loads return in issue order: the row (a few KiB, from L2) is requested first so that the digit
+            // arithmetic can start as soon as it is there, the weight rows (from HBM) right behind it so
+            // that they fly meanwhile.  (A wavefront whose rows all lie past n_out -- the last workgroup's
+            // spare ones -- only helps with the digits.)
+            const bool live = row0 < n_out;
+            const int sub = threadIdx.x & 7, bfirst = (int)threadIdx.x >> 3;
+            float4 xv[4], gv[4];
+            float ssq = 0.0f;
+            auto fetch = [&](int b0) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int b = b0 + u * 8 * NW;
+                    xv[u] = reinterpret_cast<const float4 *>(x_f32)[(size_t)(b < nb ? b : 0) * 8 + sub];
+                    if constexpr (NORM) gv[u] = reinterpret_cast<const float4 *>(epi.gamma)[(size_t)(b < nb ? b : 0) * 8 + sub];
+                }
+            };
+            if (seg0 == 0) fetch(bfirst);
+            if (live) {
+#pragma unroll
+                for (int p = 0; p < BPL; ++p) dtile[0][p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+                load_rows(L[0], 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
             if (seg0 == 0) {  // the row as digits, once per workgroup: 8 threads per block of 32, 4 elements each
                 for (int b0 = bfirst; b0 < nb; b0 += 32 * NW) {  // four blocks per thread and round
-                    if (b0 != bfirst) {
-#pragma unroll
-                        for (int u = 0; u < 4; ++u) {
-                            const int b = b0 + u * 8 * NW;
-                            xv[u] = reinterpret_cast<const float4 *>(x_f32)[(size_t)(b < nb ? b : 0) * 8 + sub];
-                        }
-                    }
+                    if (b0 != bfirst) fetch(b0);
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
                         const int b = b0 + u * 8 * NW;
                         if (b < nb) {  // whole 8-thread groups together
-                            const float f[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+                            float f[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+                            if constexpr (NORM) {
+                                ssq += f[0] * f[0] + f[1] * f[1] + f[2] * f[2] + f[3] * f[3];
+                                f[0] *= gv[u].x; f[1] *= gv[u].y; f[2] *= gv[u].z; f[3] *= gv[u].w;
+                            }
                             pg_emit_digits<QT == 4>(f, 0, b, sub, nb, ldig, lxs);
                         }
                     }
                 }
+                float *red = lxs + nb;  // NORM: the wavefronts' sums of squares, behind the block scales
+                if constexpr (NORM) {
+                    ssq = wave_sum_f32(ssq);
+                    if (lane == 0) red[threadIdx.x >> 6] = ssq;
+                }
                 // (not __syncthreads(): that would also wait for every weight load in flight)
                 asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier" ::: "memory");
+                if constexpr (NORM) {
+                    float ss = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < NW; ++w) ss += red[w];
+                    post = 1.0f / sqrtf(ss * epi.ss_inv_dim + epi.eps);
+                }
             }
             if (!live) return;  // after the workgroup's only barrier
 #pragma unroll
@@ -411,7 +467,7 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             float v = wave_sum_f32(acc[g][r]);
-            if constexpr (POST) v *= post;
+            if constexpr (POST || NORM) v *= post;
             const int row = row0 + (g % NG) * R + r;
             if constexpr (EPI != 2) {
                 if (lane == 0 && row < n_out) {
@@ -467,7 +523,15 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
     } while (0)
     if (n_out / 8 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(8, R8);
     else if (n_out / 4 * batch.count >= want) PG_GGUF_GEMV_LAUNCH(4, (R8 < 4 ? R8 : 4));
-    else PG_GGUF_GEMV_LAUNCH(2, 2);
+    else if (!Q41 && BPL == 4 && nb % 4 == 0 && (size_t)nb * (QT == 8 ? 6 : 5) + nb / 4 <= (size_t)GGUF_LDSX_CPT * 512) {
+        // two rows per wavefront under a long row: eight wavefronts share one copy of the digits in LDS
+        auto kern = gguf_gemv_kernel<QT, BPL, 2, 2, false, 2, 8>;
+        const size_t lds = (size_t)nb * 96 + (size_t)nb * sizeof(float);
+        PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
+        PG_TRY(pg_launch(ctx, QT == 4 ? "gguf_gemv_q4_0" : "gguf_gemv_q8_0", kern, dim3(grid_for(n_out, 16), (unsigned)batch.count), dim3(512),
+                         lds, qs, d, batch, (int)n_out, nb, xd.digits, xd.xs, y, residual, m, (const float *)nullptr, (const float *)nullptr,
+                         pg_gemv_epi{}));
+    } else PG_GGUF_GEMV_LAUNCH(2, 2);
 #undef PG_GGUF_GEMV_LAUNCH
     return PG_OK;
 }
@@ -530,6 +594,29 @@ pg_status launch_gemv_f32x_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uin
     else if (n_out / 4 >= want) PG_GGUF_GEMV_X_LAUNCH(4, (R8 < 4 ? R8 : 4));
     else PG_GGUF_GEMV_X_LAUNCH(2, 2);
 #undef PG_GGUF_GEMV_X_LAUNCH
+    return PG_OK;
+}
+
+// The same over any number of items (all multiply the one row), with RMSNorm folded in.
+template <int BPL>
+pg_status launch_gemv_norm_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
+                               const float *x_f32, const pg_gemv_epi &epi, float *y) {
+    constexpr int NW = 8, R8 = BPL <= 2 ? 8 : (BPL <= 4 ? 4 : 2);
+    const int nb = (int)(k_in / 32);
+    const size_t lds = (size_t)nb * 96 + (size_t)nb * sizeof(float) + NW * sizeof(float);
+    const size_t want = (size_t)ctx->num_cu * 6;
+#define PG_GGUF_GEMV_N_LAUNCH(RWW, RR)                                                                                           \
+    do {                                                                                                                         \
+        auto kern = gguf_gemv_kernel<4, BPL, RWW, RR, false, 1, NW, 0, false, true>;                                             \
+        PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                              \
+        PG_TRY(pg_launch(ctx, "gguf_gemv_q4_0_rmsnorm", kern, dim3(grid_for(n_out, RWW * NW), (unsigned)batch.count), dim3(64 * NW), lds, \
+                         qs, d, batch, (int)n_out, nb, (const int8_t *)nullptr, (const float *)nullptr, y, (const float *)nullptr, \
+                         (const uint16_t *)nullptr, (const float *)nullptr, x_f32, epi));                                        \
+    } while (0)
+    if (n_out / 8 * batch.count >= want) PG_GGUF_GEMV_N_LAUNCH(8, R8);
+    else if (n_out / 4 * batch.count >= want) PG_GGUF_GEMV_N_LAUNCH(4, (R8 < 4 ? R8 : 4));
+    else PG_GGUF_GEMV_N_LAUNCH(2, 2);
+#undef PG_GGUF_GEMV_N_LAUNCH
     return PG_OK;
 }
 
@@ -597,6 +684,22 @@ pg_status pg_launch_x_to_digits(pg_ctx *ctx, const float *x_dev, size_t rows, si
         PG_TRY(pg_launch(ctx, "x_to_digits", x_to_digits_kernel<false>, grid, dim3(256), 0, x_dev, nb, xd.digits, xd.xs,
                          (float *)nullptr));
     return pg_launch_check("x_to_digits");
+}
+
+pg_status pg_launch_gguf_gemv_rmsnorm(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
+                                      const pg_gemv_batch &batch, const float *x_f32, const float *gamma, float eps, float *y) {
+    if (batch.count == 0) return PG_OK;
+    if (batch.count > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_gemv: more than 65535 batch items");
+    if (k_in % 32 != 0 || k_in > 8192 || !gamma || (((uintptr_t)gamma | (uintptr_t)x_f32) % 16) != 0)
+        return pg_fail(PG_EINVAL, "gguf_gemv (RMSNorm folded in): k_in %zu (a multiple of 32, at most 8192) or an argument does not fit", k_in);
+    pg_gemv_epi epi = {};
+    epi.gamma = gamma; epi.eps = eps; epi.ss_inv_dim = 1.0f / (float)k_in;
+    switch ((k_in / 32 + 63) / 64) {
+        case 1: return launch_gemv_norm_bpl<1>(ctx, n_out, k_in, qs, d, batch, x_f32, epi, y);
+        case 2: return launch_gemv_norm_bpl<2>(ctx, n_out, k_in, qs, d, batch, x_f32, epi, y);
+        case 3: return launch_gemv_norm_bpl<3>(ctx, n_out, k_in, qs, d, batch, x_f32, epi, y);
+        default: return launch_gemv_norm_bpl<4>(ctx, n_out, k_in, qs, d, batch, x_f32, epi, y);
+    }
 }
 
 pg_status pg_launch_gguf_gemv_norm_digits(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,

@@ -257,6 +257,10 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
                               const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
                               const pg_xdigits &xd, float *y, const float *residual = nullptr,
                               const uint16_t *m = nullptr);
+// Q4_0, one f32 row shared by every item: y[item] = W[item] . RMSNorm(x_f32; gamma, eps), the norm folded
+// into the product's launch.  k_in at most 8192; x_f32 and gamma 16-byte aligned.
+pg_status pg_launch_gguf_gemv_rmsnorm(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
+                                      const pg_gemv_batch &batch, const float *x_f32, const float *gamma, float eps, float *y);
 // Q4_0, one row: y = product (+ residual) as usual, and besides `out` = the digits of y * gamma and
 // ss_out[n_out / 32] = the sums of squares of y by block: RMSNorm(y) without a launch, its scalar factor
 // left to the consumer.  n_out a multiple of 32.

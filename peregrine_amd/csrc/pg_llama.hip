@@ -905,19 +905,65 @@ __global__ __launch_bounds__(256) void gqa_decode_kernel(attn_args aa, int nkv, 
         lo.x = x0.x * c.x - x1.x * sn.x; lo.y = x0.y * c.y - x1.y * sn.y; lo.z = x0.z * c.z - x1.z * sn.z; lo.w = x0.w * c.w - x1.w * sn.w;
         hi.x = x0.x * sn.x + x1.x * c.x; hi.y = x0.y * sn.y + x1.y * c.y; hi.z = x0.z * sn.z + x1.z * c.z; hi.w = x0.w * sn.w + x1.w * c.w;
     };
+    float4 k0[U], k1[U], v0[U], v1[U];
+    bool live[U];
+    auto load_tile = [&](int kb, bool store_new) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            k0[u] = k1[u] = v0[u] = v1[u] = float4{0.f, 0.f, 0.f, 0.f};
+            const int kt = kb + (u * 4 + wave) * KPW + krow;
+            live[u] = kt < kend && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, aa.gbits, 0, kt);
+            if (live[u]) {
+                if (fused && kt == aa.new_pos) {
+                    // not in the cache yet: made from the projections, and stored by this workgroup, the only
+                    // one of its kv head that meets the position
+                    rot(aa.raw_k + (size_t)kvh * HD, k0[u], k1[u]);
+                    v0[u] = *reinterpret_cast<const float4 *>(aa.raw_v + (size_t)kvh * HD + 4 * li);
+                    v1[u] = *reinterpret_cast<const float4 *>(aa.raw_v + (size_t)kvh * HD + HALF + 4 * li);
+                    if (store_new) {
+                        float *kn = aa.k_new + (size_t)kvh * aa.k_stride + 4 * li, *vn = aa.v_new + (size_t)kvh * aa.v_stride + 4 * li;
+                        *reinterpret_cast<float4 *>(kn) = k0[u]; *reinterpret_cast<float4 *>(kn + HALF) = k1[u];
+                        *reinterpret_cast<float4 *>(vn) = v0[u]; *reinterpret_cast<float4 *>(vn + HALF) = v1[u];
+                    }
+                } else {
+                    typedef float f4v __attribute__((ext_vector_type(4)));
+                    const f4v *kr = reinterpret_cast<const f4v *>(kbase + (size_t)kt * HD);
+                    const f4v *vr = reinterpret_cast<const f4v *>(vbase + (size_t)kt * HD);
+                    const f4v a = __builtin_nontemporal_load(kr), b = __builtin_nontemporal_load(kr + HALF / 4);
+                    const f4v c = __builtin_nontemporal_load(vr), d = __builtin_nontemporal_load(vr + HALF / 4);
+                    k0[u] = float4{a.x, a.y, a.z, a.w}; k1[u] = float4{b.x, b.y, b.z, b.w};
+                    v0[u] = float4{c.x, c.y, c.z, c.w}; v1[u] = float4{d.x, d.y, d.z, d.w};
+                }
+            }
+        }
+    };
+    // Loads return in issue order: the query rows (from L2) are requested first and the first tile's keys and
+    // values (from HBM) right behind them, all before the first use, so that the two trips overlap.
     for (int hc = 0; hc < G; hc += GC) {
-        float4 q0[GC], q1[GC];
+        float4 q0[GC], q1[GC], qc = {0.f, 0.f, 0.f, 0.f}, qs = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int h = 0; h < GC; ++h) {
             q0[h] = q1[h] = float4{0.f, 0.f, 0.f, 0.f};
             if (hc + h < G) {
-                const size_t qh = (size_t)kvh * G + hc + h;
-                if (fused) {
-                    rot(aa.raw_q + qh * HD, q0[h], q1[h]);
-                } else {
-                    q0[h] = *reinterpret_cast<const float4 *>(aa.q + qh * HD + 4 * li);
-                    q1[h] = *reinterpret_cast<const float4 *>(aa.q + qh * HD + HALF + 4 * li);
-                }
+                const float *qrow = (fused ? aa.raw_q : aa.q) + ((size_t)kvh * G + hc + h) * HD;
+                q0[h] = *reinterpret_cast<const float4 *>(qrow + 4 * li);
+                q1[h] = *reinterpret_cast<const float4 *>(qrow + HALF + 4 * li);
+            }
+        }
+        if (fused) {
+            qc = *reinterpret_cast<const float4 *>(aa.rope_c + 4 * li);
+            qs = *reinterpret_cast<const float4 *>(aa.rope_s + 4 * li);
+        }
+        load_tile(split * tps * TK, hc == 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (fused) {  // the operations of rope_kernel in the same order
+#pragma unroll
+            for (int h = 0; h < GC; ++h) {
+                const float4 x0 = q0[h], x1 = q1[h];
+                q0[h].x = x0.x * qc.x - x1.x * qs.x; q0[h].y = x0.y * qc.y - x1.y * qs.y;
+                q0[h].z = x0.z * qc.z - x1.z * qs.z; q0[h].w = x0.w * qc.w - x1.w * qs.w;
+                q1[h].x = x0.x * qs.x + x1.x * qc.x; q1[h].y = x0.y * qs.y + x1.y * qc.y;
+                q1[h].z = x0.z * qs.z + x1.z * qc.z; q1[h].w = x0.w * qs.w + x1.w * qc.w;
             }
         }
         float m_run[GC], l_run[GC], acc[GC][8];
@@ -929,37 +975,10 @@ __global__ __launch_bounds__(256) void gqa_decode_kernel(attn_args aa, int nkv, 
             for (int j = 0; j < 8; ++j) acc[h][j] = 0.f;
         }
         for (int t = 0; t < tps; ++t) {
-            const int kb = (split * tps + t) * TK;
-            if (kb >= kend) break;
-            float4 k0[U], k1[U], v0[U], v1[U];
-            bool live[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                k0[u] = k1[u] = v0[u] = v1[u] = float4{0.f, 0.f, 0.f, 0.f};
-                const int kt = kb + (u * 4 + wave) * KPW + krow;
-                live[u] = kt < kend && !attn_masked(aa.mask_kind, aa.offset, aa.window, aa.sink, aa.gbits, 0, kt);
-                if (live[u]) {
-                    if (fused && kt == aa.new_pos) {
-                        // not in the cache yet: made from the projections, and stored by this workgroup, the only
-                        // one of its kv head that meets the position
-                        rot(aa.raw_k + (size_t)kvh * HD, k0[u], k1[u]);
-                        v0[u] = *reinterpret_cast<const float4 *>(aa.raw_v + (size_t)kvh * HD + 4 * li);
-                        v1[u] = *reinterpret_cast<const float4 *>(aa.raw_v + (size_t)kvh * HD + HALF + 4 * li);
-                        if (hc == 0) {
-                            float *kn = aa.k_new + (size_t)kvh * aa.k_stride + 4 * li, *vn = aa.v_new + (size_t)kvh * aa.v_stride + 4 * li;
-                            *reinterpret_cast<float4 *>(kn) = k0[u]; *reinterpret_cast<float4 *>(kn + HALF) = k1[u];
-                            *reinterpret_cast<float4 *>(vn) = v0[u]; *reinterpret_cast<float4 *>(vn + HALF) = v1[u];
-                        }
-                    } else {
-                        typedef float f4v __attribute__((ext_vector_type(4)));
-                        const f4v *kr = reinterpret_cast<const f4v *>(kbase + (size_t)kt * HD);
-                        const f4v *vr = reinterpret_cast<const f4v *>(vbase + (size_t)kt * HD);
-                        const f4v a = __builtin_nontemporal_load(kr), b = __builtin_nontemporal_load(kr + HALF / 4);
-                        const f4v c = __builtin_nontemporal_load(vr), d = __builtin_nontemporal_load(vr + HALF / 4);
-                        k0[u] = float4{a.x, a.y, a.z, a.w}; k1[u] = float4{b.x, b.y, b.z, b.w};
-                        v0[u] = float4{c.x, c.y, c.z, c.w}; v1[u] = float4{d.x, d.y, d.z, d.w};
-                    }
-                }
+            if (t > 0) {
+                const int kb = (split * tps + t) * TK;
+                if (kb >= kend) break;
+                load_tile(kb, hc == 0);
             }
 #pragma unroll
             for (int h = 0; h < GC; ++h) {
@@ -1839,10 +1858,14 @@ static pg_status block_forward_one_token(pg_ctx *ctx, pg_llama_block *b, const f
     const bool qkv_same = b->w[0]->ggml_type == b->w[1]->ggml_type && b->w[1]->ggml_type == b->w[2]->ggml_type && kv_dim % 8 == 0;
     const bool gu_same = b->w[4]->ggml_type == b->w[5]->ggml_type;
 
-    PG_TRY(launch_rmsnorm_digits(ctx, h_dev, nullptr, nullptr, b->attn_norm_w, b->eps, 1, d, kind, b->xd_d));
-    if (qkv_same) {
+    if (kind == PG_GGML_Q4_0 && qkv_same && d <= 8192) {
+        // the norm rides in the products' launch: digits of h * (norm weights) per workgroup, the scalar factor at the end
+        PG_TRY(pg_launch_gguf_gemv_rmsnorm(ctx, kv_dim, d, nullptr, nullptr, qkv_n, h_dev, b->attn_norm_w, b->eps, qkv));
+    } else if (qkv_same) {
+        PG_TRY(launch_rmsnorm_digits(ctx, h_dev, nullptr, nullptr, b->attn_norm_w, b->eps, 1, d, kind, b->xd_d));
         PG_TRY(pg_launch_gguf_gemv(ctx, b->w[0]->ggml_type, kv_dim, d, nullptr, nullptr, qkv_n, b->xd_d, qkv));
     } else {
+        PG_TRY(launch_rmsnorm_digits(ctx, h_dev, nullptr, nullptr, b->attn_norm_w, b->eps, 1, d, kind, b->xd_d));
         PG_TRY(pg_launch_gguf_gemv(ctx, b->w[0]->ggml_type, q_dim, d, b->w[0]->qs, b->w[0]->d, one, b->xd_d, qd));
         PG_TRY(pg_launch_gguf_gemv(ctx, b->w[1]->ggml_type, kv_dim, d, b->w[1]->qs, b->w[1]->d, one, b->xd_d, kd));
         PG_TRY(pg_launch_gguf_gemv(ctx, b->w[2]->ggml_type, kv_dim, d, b->w[2]->qs, b->w[2]->d, one, b->xd_d, vd));

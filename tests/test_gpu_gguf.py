@@ -95,6 +95,7 @@ GGUF_SHAPES = [
     (2, 64, 32800, 1), (2, 8200, 256, 1), (8, 33, 32768, 1), (8, 9, 32, 1),   # past its limits (K, rows) and Q8_0: digits by a launch of their own
     (2, 14336, 4096, 1),                                        # benchmark configuration 4, full size
     (8, 6144, 4096, 1),
+    (8, 4096, 14336, 1), (8, 300, 8192, 1), (8, 24, 16384, 1),  # two rows a wavefront under a long row: the digits shared through LDS (ragged last workgroups)
     # more than one row: matrix-core path (token tiles of 32, row tiles of 128, split K)
     (2, 130, 224, 33), (8, 131, 160, 40), (2, 515, 4096, 64), (8, 257, 6144, 35), (2, 14336, 4096, 4), (8, 4096, 14336, 16),
     # Q4_1 (offset blocks): the streaming kernel with the block-sum term, one item per row

@@ -327,6 +327,13 @@ def test_llama_block_decode_steps_head_64_group_of_3(ctx, orc, typ):
     _block_case(ctx, orc, 384, 6, 2, 64, 640, typ, (7, 1, 1, 1, 20, 1), seed=31)
 
 
+@pytest.mark.parametrize("typ", [2, 8])
+def test_llama_block_decode_long_ffn_rows(ctx, orc, typ):
+    """A down projection with few output rows under a long input row (ffn 8192): its one-token product shares
+    one copy of the input digits per workgroup through LDS."""
+    _block_case(ctx, orc, 256, 8, 2, 32, 8192, typ, (3, 1, 1), seed=37)
+
+
 def test_llama_block_q4_1_weights(ctx, orc):
     """Offset blocks (Q4_1) run on the streaming kernel only, one item per row."""
     _block_case(ctx, orc, 128, 4, 2, 32, 256, 3, (3, 1), seed=13)
