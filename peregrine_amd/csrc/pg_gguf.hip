@@ -276,10 +276,15 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[g][r] = 0.0f;
     float post = 1.0f;
-    if constexpr (POST) {  // requested first, needed last
-        float ss = 0.0f;
-        for (int i = lane; i < epi.ss_n; i += 64) ss += epi.ss_in[i];
-        post = 1.0f / sqrtf(wave_sum_f32(ss) * epi.ss_inv_dim + epi.eps);
+    float ssv[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // POST: requested first, needed last (ss_n <= 256)
+    if constexpr (POST) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (lane + 64 * i < epi.ss_n) ssv[i] = epi.ss_in[lane + 64 * i];
+    }
+    float4 gm = {0.0f, 0.0f, 0.0f, 0.0f};     // EPI 1: the norm weights of the workgroup's block, likewise
+    if constexpr (EPI == 1) {
+        if (threadIdx.x < 8) gm = reinterpret_cast<const float4 *>(epi.gamma)[blockIdx.x * 8 + threadIdx.x];
     }
 
     for (int seg0 = 0; seg0 < nb; seg0 += SEG) {
@@ -462,6 +467,7 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
         }
     }
     __shared__ float res[NT][EPI != 0 ? 32 : 1];  // EPI: the workgroup's 32 outputs (per tensor)
+    if constexpr (POST) post = 1.0f / sqrtf(wave_sum_f32((ssv[0] + ssv[1]) + (ssv[2] + ssv[3])) * epi.ss_inv_dim + epi.eps);
 #pragma unroll
     for (int g = 0; g < NGT; ++g)
 #pragma unroll
@@ -485,7 +491,6 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
             const int sub = threadIdx.x, e0 = sub * 4;
             float f[4];
             if constexpr (EPI == 1) {
-                const float4 gm = reinterpret_cast<const float4 *>(epi.gamma)[blockIdx.x * 8 + sub];
                 const float h[4] = {res[0][e0], res[0][e0 + 1], res[0][e0 + 2], res[0][e0 + 3]};
                 f[0] = h[0] * gm.x; f[1] = h[1] * gm.y; f[2] = h[2] * gm.z; f[3] = h[3] * gm.w;
                 float ss = h[0] * h[0] + h[1] * h[1] + h[2] * h[2] + h[3] * h[3];
@@ -536,38 +541,51 @@ pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t 
     return PG_OK;
 }
 
-// Q4_0 products whose output is the next product's digit input (see EPI at the kernel): a workgroup owns
+// Products whose output is the next product's digit input (see EPI at the kernel): a workgroup owns
 // 32 output rows as 32 / RW wavefronts.
-template <int BPL, int EPI, bool POST>
+template <int QT, int BPL, int EPI, bool POST>
 pg_status launch_gemv_epi_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const pg_xdigits &xd,
                               float *y, const float *residual, const pg_gemv_epi &epi) {
     const int nb = (int)(k_in / 32);
     const pg_gemv_batch one = {1, nullptr, nullptr, nullptr, 1};
-    constexpr int R8 = BPL <= 2 ? 8 : (BPL <= 4 ? 4 : 2);
+    constexpr int NH = QT == 8 ? 2 : 1;
+    constexpr int R8 = BPL * NH <= 2 ? 8 : (BPL * NH <= 4 ? 4 : 2);
     const size_t want = (size_t)ctx->num_cu * 6;  // wavefronts wanted in the grid
     const size_t rows = n_out * (EPI == 2 ? 2 : 1);
 #define PG_GGUF_GEMV_E_LAUNCH(RWW, RR)                                                                                            \
-    PG_TRY(pg_launch(ctx, EPI == 1 ? "gguf_gemv_q4_0_norm_digits" : "gguf_gemv_q4_0_swiglu_digits",                              \
-                     gguf_gemv_kernel<4, BPL, RWW, RR, false, false, 32 / RWW, EPI, POST>, dim3((unsigned)(n_out / 32)),          \
+    PG_TRY(pg_launch(ctx, EPI == 1 ? (QT == 4 ? "gguf_gemv_q4_0_norm_digits" : "gguf_gemv_q8_0_norm_digits")                      \
+                              : (QT == 4 ? "gguf_gemv_q4_0_swiglu_digits" : "gguf_gemv_q8_0_swiglu_digits"),                      \
+                     gguf_gemv_kernel<QT, BPL, RWW, RR, false, 0, 32 / RWW, EPI, POST>, dim3((unsigned)(n_out / 32)),             \
                      dim3(64 * (32 / RWW)), 0, qs, d, one, (int)n_out, nb, xd.digits, xd.xs, y, residual, (const uint16_t *)nullptr, \
                      (const float *)nullptr, (const float *)nullptr, epi))
-    if (rows / 8 >= want && EPI != 2) PG_GGUF_GEMV_E_LAUNCH(8, R8);
-    else if (rows / 4 >= want || BPL > 2) PG_GGUF_GEMV_E_LAUNCH(4, (R8 < 4 ? R8 : 4));  // (16 wavefronts leave 128 registers each)
-    else PG_GGUF_GEMV_E_LAUNCH(2, 2);
+    if constexpr (BPL * NH > 2) {  // (8 or 16 wavefronts would leave too few registers each for rows this long)
+        PG_GGUF_GEMV_E_LAUNCH(8, R8);
+    } else {
+        if (rows / 8 >= want) PG_GGUF_GEMV_E_LAUNCH(8, R8);
+        else if (rows / 4 >= want) PG_GGUF_GEMV_E_LAUNCH(4, (R8 < 4 ? R8 : 4));
+        else PG_GGUF_GEMV_E_LAUNCH(2, 2);
+    }
 #undef PG_GGUF_GEMV_E_LAUNCH
     return PG_OK;
 }
 
 template <int EPI, bool POST>
-pg_status launch_gemv_epi(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const pg_xdigits &xd, float *y,
-                          const float *residual, const pg_gemv_epi &epi) {
+pg_status launch_gemv_epi(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const pg_xdigits &xd,
+                          float *y, const float *residual, const pg_gemv_epi &epi) {
     size_t bpl = (k_in / 32 + 63) / 64;
     if (bpl > 4) bpl = 4;
+    if (ggml_type != PG_GGML_Q4_0 && ggml_type != PG_GGML_Q8_0)
+        return pg_fail(PG_EUNSUPPORTED, "gguf_gemv: only Q4_0 and Q8_0 products leave their output as digits");
+    const bool q4 = ggml_type == PG_GGML_Q4_0;
     switch (bpl) {
-        case 1: return launch_gemv_epi_bpl<1, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
-        case 2: return launch_gemv_epi_bpl<2, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
-        case 3: return launch_gemv_epi_bpl<3, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
-        default: return launch_gemv_epi_bpl<4, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
+        case 1: return q4 ? launch_gemv_epi_bpl<4, 1, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi)
+                          : launch_gemv_epi_bpl<8, 1, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
+        case 2: return q4 ? launch_gemv_epi_bpl<4, 2, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi)
+                          : launch_gemv_epi_bpl<8, 2, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
+        case 3: return q4 ? launch_gemv_epi_bpl<4, 3, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi)
+                          : launch_gemv_epi_bpl<8, 3, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
+        default: return q4 ? launch_gemv_epi_bpl<4, 4, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi)
+                           : launch_gemv_epi_bpl<8, 4, EPI, POST>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
     }
 }
 
@@ -601,7 +619,7 @@ pg_status launch_gemv_f32x_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uin
 template <int BPL>
 pg_status launch_gemv_norm_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const pg_gemv_batch &batch,
                                const float *x_f32, const pg_gemv_epi &epi, float *y) {
-    constexpr int NW = 8, R8 = BPL <= 2 ? 8 : (BPL <= 4 ? 4 : 2);
+    constexpr int NW = 8, R8 = BPL <= 2 ? 8 : (BPL <= 4 ? 4 : 2);  // (measured on 6 x 1024 rows of 4096: 7.6 us; four wavefronts 8.2)
     const int nb = (int)(k_in / 32);
     const size_t lds = (size_t)nb * 96 + (size_t)nb * sizeof(float) + NW * sizeof(float);
     const size_t want = (size_t)ctx->num_cu * 6;
@@ -613,9 +631,13 @@ pg_status launch_gemv_norm_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uin
                          qs, d, batch, (int)n_out, nb, (const int8_t *)nullptr, (const float *)nullptr, y, (const float *)nullptr, \
                          (const uint16_t *)nullptr, (const float *)nullptr, x_f32, epi));                                        \
     } while (0)
-    if (n_out / 8 * batch.count >= want) PG_GGUF_GEMV_N_LAUNCH(8, R8);
-    else if (n_out / 4 * batch.count >= want) PG_GGUF_GEMV_N_LAUNCH(4, (R8 < 4 ? R8 : 4));
-    else PG_GGUF_GEMV_N_LAUNCH(2, 2);
+    if constexpr (BPL > 2) {  // (more rows in flight would spill registers)
+        PG_GGUF_GEMV_N_LAUNCH(2, 2);
+    } else {
+        if (n_out / 8 * batch.count >= want) PG_GGUF_GEMV_N_LAUNCH(8, R8);
+        else if (n_out / 4 * batch.count >= want) PG_GGUF_GEMV_N_LAUNCH(4, (R8 < 4 ? R8 : 4));
+        else PG_GGUF_GEMV_N_LAUNCH(2, 2);
+    }
 #undef PG_GGUF_GEMV_N_LAUNCH
     return PG_OK;
 }
@@ -702,25 +724,26 @@ pg_status pg_launch_gguf_gemv_rmsnorm(pg_ctx *ctx, size_t n_out, size_t k_in, co
     }
 }
 
-pg_status pg_launch_gguf_gemv_norm_digits(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
+pg_status pg_launch_gguf_gemv_norm_digits(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
                                           const pg_xdigits &xd, float *y, const float *residual, const float *gamma,
                                           const pg_xdigits &out, float *ss_out) {
     if (n_out % 32 != 0 || k_in % 32 != 0 || !gamma || (uintptr_t)gamma % 16 != 0 || !ss_out || !y)
         return pg_fail(PG_EINVAL, "gguf_gemv (digits of the normalised output): [%zu, %zu] or an argument does not fit", n_out, k_in);
     pg_gemv_epi epi = {};
     epi.gamma = gamma; epi.out_digits = out.digits; epi.out_xs = out.xs; epi.ss_out = ss_out;
-    return launch_gemv_epi<1, false>(ctx, n_out, k_in, qs, d, xd, y, residual, epi);
+    return launch_gemv_epi<1, false>(ctx, ggml_type, n_out, k_in, qs, d, xd, y, residual, epi);
 }
 
-pg_status pg_launch_gguf_gemv_swiglu_digits(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs_gate, const uint16_t *d_gate,
+pg_status pg_launch_gguf_gemv_swiglu_digits(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs_gate, const uint16_t *d_gate,
                                             const uint8_t *qs_up, const uint16_t *d_up, const pg_xdigits &xd, const float *ss_in,
                                             size_t ss_n, size_t ss_dim, float eps, const pg_xdigits &out) {
     if (n_out % 32 != 0 || k_in % 32 != 0 || !ss_in || ss_n == 0 || ss_dim == 0)
         return pg_fail(PG_EINVAL, "gguf_gemv (digits of SiLU(gate) * up): [%zu, %zu] or an argument does not fit", n_out, k_in);
     pg_gemv_epi epi = {};
     epi.qs1 = qs_up; epi.d1 = d_up; epi.out_digits = out.digits; epi.out_xs = out.xs;
+    if (ss_n > 256) return pg_fail(PG_EUNSUPPORTED, "gguf_gemv (digits of SiLU(gate) * up): more than 256 partial sums");
     epi.ss_in = ss_in; epi.ss_n = (int)ss_n; epi.ss_inv_dim = 1.0f / (float)ss_dim; epi.eps = eps;
-    return launch_gemv_epi<2, true>(ctx, n_out, k_in, qs_gate, d_gate, xd, nullptr, nullptr, epi);
+    return launch_gemv_epi<2, true>(ctx, ggml_type, n_out, k_in, qs_gate, d_gate, xd, nullptr, nullptr, epi);
 }
 
 pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in,

@@ -261,15 +261,15 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
 // into the product's launch.  k_in at most 8192; x_f32 and gamma 16-byte aligned.
 pg_status pg_launch_gguf_gemv_rmsnorm(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
                                       const pg_gemv_batch &batch, const float *x_f32, const float *gamma, float eps, float *y);
-// Q4_0, one row: y = product (+ residual) as usual, and besides `out` = the digits of y * gamma and
+// Q4_0 or Q8_0, one row: y = product (+ residual) as usual, and besides `out` = the digits of y * gamma and
 // ss_out[n_out / 32] = the sums of squares of y by block: RMSNorm(y) without a launch, its scalar factor
 // left to the consumer.  n_out a multiple of 32.
-pg_status pg_launch_gguf_gemv_norm_digits(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
+pg_status pg_launch_gguf_gemv_norm_digits(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
                                           const pg_xdigits &xd, float *y, const float *residual, const float *gamma,
                                           const pg_xdigits &out, float *ss_out);
-// Q4_0, one row: out = digits of SiLU(g) * u with g, u = the products by gate and up, both divided by the
+// Q4_0 or Q8_0 (gate and up alike), one row: out = digits of SiLU(g) * u with g, u = the products by gate and up, both divided by the
 // RMS of the input row (ss_in: ss_n partial sums of squares over ss_dim elements, eps).
-pg_status pg_launch_gguf_gemv_swiglu_digits(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs_gate, const uint16_t *d_gate,
+pg_status pg_launch_gguf_gemv_swiglu_digits(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs_gate, const uint16_t *d_gate,
                                             const uint8_t *qs_up, const uint16_t *d_up, const pg_xdigits &xd, const float *ss_in,
                                             size_t ss_n, size_t ss_dim, float eps, const pg_xdigits &out);
 // One activation row still in f32: digits made inside the product's own launch.  Only where the predicate holds.

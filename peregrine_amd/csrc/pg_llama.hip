@@ -1893,15 +1893,15 @@ static pg_status block_forward_one_token(pg_ctx *ctx, pg_llama_block *b, const f
         PG_TRY(launch_attention(ctx, q_rope, cache, cache, b->nqh, 1, 1.0f / sqrtf((float)hd), PG_MASK_CAUSAL, offset, 0, 0, 0.0f,
                                 attn, 0, &b->xd_q, kind));
     }
-    if (kind == PG_GGML_Q4_0 && d % 32 == 0 && ffn % 32 == 0) {
+    if (d % 32 == 0 && ffn % 32 == 0 && d <= 8192) {  // (kind: all seven tensors Q4_0, or all Q8_0)
         // h1 = h + attn . Wo, stored, and also left as the digits of h1 * (norm weights) with its sums of
         // squares; gate and up divide by the RMS themselves and leave the digits of SiLU(g) * u: two
         // launches (RMSNorm, SiLU.up) fewer
-        PG_TRY(pg_launch_gguf_gemv_norm_digits(ctx, d, q_dim, b->w[3]->qs, b->w[3]->d, b->xd_q, h1, h_dev, b->ffn_norm_w, b->xd_d,
+        PG_TRY(pg_launch_gguf_gemv_norm_digits(ctx, kind, d, q_dim, b->w[3]->qs, b->w[3]->d, b->xd_q, h1, h_dev, b->ffn_norm_w, b->xd_d,
                                                b->ss_part));
-        PG_TRY(pg_launch_gguf_gemv_swiglu_digits(ctx, ffn, d, b->w[4]->qs, b->w[4]->d, b->w[5]->qs, b->w[5]->d, b->xd_d, b->ss_part,
+        PG_TRY(pg_launch_gguf_gemv_swiglu_digits(ctx, kind, ffn, d, b->w[4]->qs, b->w[4]->d, b->w[5]->qs, b->w[5]->d, b->xd_d, b->ss_part,
                                                  d / 32, d, b->eps, b->xd_f));
-        return pg_launch_gguf_gemv(ctx, PG_GGML_Q4_0, d, ffn, b->w[6]->qs, b->w[6]->d, one, b->xd_f, out_dev, h1);
+        return pg_launch_gguf_gemv(ctx, kind, d, ffn, b->w[6]->qs, b->w[6]->d, one, b->xd_f, out_dev, h1);
     }
     // h1 = h + attn . Wo
     PG_TRY(pg_launch_gguf_gemv(ctx, b->w[3]->ggml_type, d, q_dim, b->w[3]->qs, b->w[3]->d, one, b->xd_q, h1, h_dev));

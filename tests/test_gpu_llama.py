@@ -334,6 +334,15 @@ def test_llama_block_decode_long_ffn_rows(ctx, orc, typ):
     _block_case(ctx, orc, 256, 8, 2, 32, 8192, typ, (3, 1, 1), seed=37)
 
 
+@pytest.mark.parametrize("typ", [2, 8])
+def test_llama_block_decode_wide_rows(ctx, orc, typ):
+    """One-token steps whose folded products meet long rows: a model dim of 6144 under the norm-folding q|k|v
+    product and the gate|up pair (three 64-block groups per lane), and 48 heads of 128 under the o-projection
+    that leaves its output as digits."""
+    _block_case(ctx, orc, 6144, 8, 2, 64, 256, typ, (2, 1, 1), seed=41)
+    _block_case(ctx, orc, 256, 48, 8, 128, 320, typ, (2, 1, 1), seed=43)
+
+
 def test_llama_block_q4_1_weights(ctx, orc):
     """Offset blocks (Q4_1) run on the streaming kernel only, one item per row."""
     _block_case(ctx, orc, 128, 4, 2, 32, 256, 3, (3, 1), seed=13)
