@@ -1828,10 +1828,12 @@ PG_API pg_status pg_llama_block_set_weights(pg_ctx *ctx, pg_llama_block *b, cons
     return PG_OK;
 }
 
-// The one-token step: every producer of a GEMV input writes digits instead of f32 (RMSNorm,
-// the attention merge, SiLU·up), k/v and gate/up each run as one two-item launch, and the
-// second residual add is the down projection's epilogue, RoPE and the cache append ride in the
-// attention kernel: 9 launches instead of 18.
+// The one-token step: every producer of a GEMV input writes digits instead of f32, and where the producer
+// is a product its workgroups do so themselves (the o-projection leaves h1 * norm weights, gate|up leave
+// SiLU(g) * u; the first RMSNorm rides in the q|k|v launch), q/k/v run as one multi-item launch, the
+// residual adds are GEMV epilogues, RoPE and the cache append ride in the attention kernel: with Q4_0
+// tensors 6 launches (q|k|v, attention, merge of its key splits, o, gate|up, down) instead of 18; Q8_0
+// tensors keep the first RMSNorm as a launch (7).
 static pg_status block_forward_one_token(pg_ctx *ctx, pg_llama_block *b, const float *h_dev, pg_kv_cache *cache,
                                          float *out_dev) {
     const size_t d = b->d, hd = b->hd, q_dim = b->nqh * hd, kv_dim = b->nkvh * hd, ffn = b->ffn, offset = cache->len;
