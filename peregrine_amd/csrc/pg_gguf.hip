@@ -212,11 +212,18 @@ struct RowLoads {
 // uses (qs0, d0).  R rows are in flight at a time (NG = RW / R groups, double-buffered).
 // Q41 (with QT = 4): every block also has an offset m; its term (8 d + m) * sum_k x_k uses the
 // block sums written with the digits.
-// XF32 (one item, no tables): the activation row arrives in f32 (x_f32) and the workgroup -- NW
-// wavefronts, each with its own RW rows -- rewrites it as digits into LDS itself, after every
-// wavefront has requested its first weight rows: the product is one launch instead of two, and
-// the digit arithmetic (18 vector operations per element, shared by NW wavefronts) runs while
-// those first loads are in flight.
+// XM, where the activation digits come from:
+//   0  from memory, every wavefront its own reads (the rows come as digits, one row per item / x_row_div);
+//   1  the one activation row, the same for every item, arrives in f32 (x_f32) and the workgroup -- NW
+//      wavefronts, each with its own RW rows -- rewrites it as digits into LDS itself, after every
+//      wavefront has requested its first weight rows: one launch instead of two, and the digit arithmetic
+//      (18 vector operations per element, shared by NW wavefronts) runs while those first loads are in
+//      flight.  NORM: that row is RMSNorm(x_f32) with the weights epi.gamma (src/nn.rs:560-652): the digits
+//      are those of x * gamma, the sum of squares rides on the digits' barrier, and the scalar factor
+//      multiplies the product: the norm costs no launch and no extra barrier;
+//   2  from memory, but once per workgroup, into LDS, for its NW wavefronts: with few rows per wavefront
+//      under a long row (K = 14336 is 36 KB of digits, more than the CU's vector cache) every wavefront
+//      would otherwise pull the whole of them through L2 again.
 // EPI (one item, NW * RW = 32: a workgroup owns one block of 32 output rows) makes the output the digit
 // input of the NEXT product, so that the one-token step of models::llama needs no launch in between:
 //   1  y (+ residual) is stored as usual, and also as digits of y * gamma (the RMSNorm weights,
@@ -225,12 +232,6 @@ struct RowLoads {
 //   2  the workgroup multiplies by two tensors (gate, then up = epi.qs1 / d1) and leaves only the digits
 //      of silu(gate) * up (src/models/llama/decoder.rs:143-150).
 // POST: the product is multiplied by 1 / sqrt(sum(ss_in[0 .. ss_n)) * ss_inv_dim + eps) before anything else.
-// XM 2: the row's digits are read as usual, but once per workgroup, into LDS, for its NW wavefronts: with
-// few rows per wavefront and a long row (K = 14336 is 36 KB of digits, more than the CU's vector cache)
-// every wavefront would otherwise pull the whole of them through L2 again.
-// NORM (with XM 1): the row is RMSNorm(x_f32) with the weights epi.gamma (src/nn.rs:560-652): the digits are
-// those of x * gamma, the sum of squares rides on the digits' barrier, and the scalar factor is applied to
-// the product: the norm costs no launch and no extra barrier.
 template <int QT, int BPL, int RW, int R, bool Q41 = false, int XM = 0, int NW = 1, int EPI = 0, bool POST = false, bool NORM = false>
 __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
     const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0, pg_gemv_batch batch,
