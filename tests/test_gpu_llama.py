@@ -271,12 +271,13 @@ def test_gqa_attention_edges(ctx, orc):
         llama.gqa_attention(np.ones(5, np.float32), cache, cache, 4, 2, 2, 8, 1.0, llama.AttentionMask.none(), None, out, ctx)
 
 
-def _block_case(ctx, orc, d, nqh, nkvh, hd, ffn, typ, steps, max_seq=64, seed=0):
+def _block_case(ctx, orc, d, nqh, nkvh, hd, ffn, typ, steps, max_seq=64, seed=0, raws=None):
     from peregrine_amd import gguf, llama
     shapes = [(nqh * hd, d), (nkvh * hd, d), (nkvh * hd, d), (d, nqh * hd), (ffn, d), (ffn, d), (d, ffn)]
     types = [typ] * 7 if np.isscalar(typ) else list(typ)
-    raws = [bytes({2: H.pack_q4_0, 3: H.pack_q4_1, 8: H.pack_q8_0}[t](orc.rng_normal(seed + 40 + i, n * k, 0.0, 1.0 / np.sqrt(k))))
-            for i, ((n, k), t) in enumerate(zip(shapes, types))]
+    if raws is None:
+        raws = [bytes({2: H.pack_q4_0, 3: H.pack_q4_1, 8: H.pack_q8_0}[t](orc.rng_normal(seed + 40 + i, n * k, 0.0, 1.0 / np.sqrt(k))))
+                for i, ((n, k), t) in enumerate(zip(shapes, types))]
     ws = [gguf.GgufWeight(r, t, n, k, ctx) for r, (n, k), t in zip(raws, shapes, types)]
     wa = (1 + 0.1 * orc.rng_normal(seed + 1, d)).astype(np.float32)
     wf = (1 + 0.1 * orc.rng_normal(seed + 2, d)).astype(np.float32)
@@ -341,6 +342,23 @@ def test_llama_block_decode_wide_rows(ctx, orc, typ):
     that leaves its output as digits."""
     _block_case(ctx, orc, 6144, 8, 2, 64, 256, typ, (2, 1, 1), seed=41)
     _block_case(ctx, orc, 256, 48, 8, 128, 320, typ, (2, 1, 1), seed=43)
+
+
+def test_llama_block_one_token_steps_at_llama_8b_size(ctx, orc):
+    """The benchmark's block at full size (d 4096, 32 / 8 heads of 128, ffn 14336, Q4_0): a three-token prefill and
+    two one-token steps against the oracle.  The tensors are written as Q4_0 blocks directly (random nibbles, block
+    scales drawn from eight f16 values around 1 / (4 sqrt(K))): packing 218 M normal weights would take minutes."""
+    d, nqh, nkvh, hd, ffn = 4096, 32, 8, 128, 14336
+    rng = np.random.default_rng(2024)
+    raws = []
+    for n, k in [(nqh * hd, d), (nkvh * hd, d), (nkvh * hd, d), (d, nqh * hd), (ffn, d), (ffn, d), (d, ffn)]:
+        nb = n * k // 32
+        raw = np.empty((nb, 18), np.uint8)
+        raw[:, 2:] = rng.integers(0, 256, size=(nb, 16), dtype=np.uint8)
+        scales = (np.float16(0.25 / np.sqrt(k)) * np.arange(5, 13, dtype=np.float16) / np.float16(8)).astype(np.float16)
+        raw[:, :2] = scales.view(np.uint8).reshape(8, 2)[rng.integers(0, 8, size=nb)]
+        raws.append(raw.tobytes())
+    _block_case(ctx, orc, d, nqh, nkvh, hd, ffn, 2, (3, 1, 1), max_seq=16, seed=51, raws=raws)
 
 
 def test_llama_block_q4_1_weights(ctx, orc):
