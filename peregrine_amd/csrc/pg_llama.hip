@@ -621,15 +621,22 @@ __global__ __launch_bounds__(256) void gqa_attention_tiled_kernel(attn_args aa) 
 // (maximum, sum, rows) it hands over through LDS.
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-template <int HD>
+// SPLIT (few rows under a long cache: a chunk of a prefill, a handful of draft tokens): the keys are cut
+// into aa.splits runs of aa.chunk tiles as well, workgroup = (kv head, two adjacent items, run), one item per
+// wavefront and no hand-over; every wavefront leaves (maximum, exp-sum, unnormalised rows) for
+// gqa_combine_kernel in rows of HD + 4 floats, or an empty record where its rows see none of the run's keys.
+template <int HD, bool SPLIT = false>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void gqa_attention_mfma_kernel(attn_args aa, int n_items, int nkvh) {
     constexpr int NDT = HD / 32, QR = HD / 2;
     typedef float vdt __attribute__((ext_vector_type(NDT)));
-    __shared__ float part_l[(NDT * 16 + 2) * 64];
+    __shared__ float part_l[SPLIT ? 1 : (NDT * 16 + 2) * 64];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int col = lane & 31, h = lane >> 5;
-    const int kvh = blockIdx.x % nkvh, pair = blockIdx.x / nkvh;
+    const int kvh = blockIdx.x % nkvh;
+    const int n_pairs = (n_items + 1) / 2;
+    const int pair = SPLIT ? (blockIdx.x / nkvh) % n_pairs : blockIdx.x / nkvh;
+    const int run = SPLIT ? (blockIdx.x / nkvh) / n_pairs : 0;
     const int G = aa.group, nrows = G * aa.seq_q;
     const int item_a = pair, item_b = n_items - 1 - pair;  // the short and the long one (equal: one item)
     auto kend_of = [&](int item) {
@@ -643,18 +650,41 @@ void gqa_attention_mfma_kernel(attn_args aa, int n_items, int nkvh) {
     float m = -INFINITY, l = 0.f;
     v16f o[NDT];
     int row = 0, qt = 0, qh = 0;
-    for (int seg = 0; seg < 2; ++seg) {
+    for (int seg = 0; seg < (SPLIT ? 1 : 2); ++seg) {
         // wavefront 0: (long item, tiles [0, cut)), nothing; wavefront 1: (short item, all), (long item, [cut, tb))
-        const int item = (wave == 0 || seg == 1) ? item_b : item_a;
-        const int t0 = wave == 0 ? 0 : (seg == 0 ? 0 : cut);
-        const int t1 = wave == 0 ? (seg == 0 ? cut : 0) : (seg == 0 ? ta : tb);
-        if (t1 <= t0) continue;
+        int item = (wave == 0 || seg == 1) ? item_b : item_a;
+        int t0 = wave == 0 ? 0 : (seg == 0 ? 0 : cut);
+        int t1 = wave == 0 ? (seg == 0 ? cut : 0) : (seg == 0 ? ta : tb);
+        if constexpr (SPLIT) {
+            item = 2 * pair + wave;
+            if (item >= n_items) return;  // (no barrier on this path)
+            t0 = run * aa.chunk;
+            t1 = min((kend_of(item) + 31) / 32, t0 + aa.chunk);
+        } else {
+            if (t1 <= t0) continue;
+        }
         const int kend = kend_of(item);
         row = item * 32 + col;
         const int rowc = min(row, nrows - 1);
         qt = rowc / G;
         qh = kvh * G + rowc % G;
         const int qt_min = (item * 32) / G;
+        float *const rec = SPLIT ? aa.part + (((size_t)qt * aa.nqh + qh) * aa.splits + run) * (size_t)(HD + 4) : nullptr;
+        if constexpr (SPLIT) {
+            if (t1 <= t0) {  // none of the run's keys are before these rows
+                if (row < nrows) {
+                    if (h == 0) *reinterpret_cast<float2 *>(rec) = float2{-INFINITY, 0.f};
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        vdt z;
+#pragma unroll
+                        for (int dt = 0; dt < NDT; ++dt) z[dt] = 0.f;
+                        *reinterpret_cast<vdt *>(rec + 4 + NDT * (8 * (r >> 2) + 4 * h + (r & 3))) = z;
+                    }
+                }
+                return;
+            }
+        }
         m = -INFINITY;
         l = 0.f;
 #pragma unroll
@@ -806,6 +836,20 @@ void gqa_attention_mfma_kernel(attn_args aa, int n_items, int nkvh) {
         finish_scores(s_cur, t1 - 1);
         rescale(softmax(s_cur));
         weighted_values(s_cur);
+        if constexpr (SPLIT) {
+            const float lt = l + __shfl_xor(l, 32);
+            if (row < nrows) {
+                if (h == 0) *reinterpret_cast<float2 *>(rec) = float2{m, lt};
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    vdt v;
+#pragma unroll
+                    for (int dt = 0; dt < NDT; ++dt) v[dt] = o[dt][r];
+                    *reinterpret_cast<vdt *>(rec + 4 + NDT * (8 * (r >> 2) + 4 * h + (r & 3))) = v;
+                }
+            }
+            return;
+        }
         if (wave == 1 && seg == 0) {  // the short item is complete
             const float lt = l + __shfl_xor(l, 32);
             const float inv = lt > 0.f ? 1.0f / lt : 0.f;
@@ -1062,30 +1106,32 @@ constexpr int ATT_SPLITS_MAX = 2048;
 // w_s = exp(m_s - M), out = sum_s w_s o_s / sum_s w_s l_s, splits in ascending order.
 // DIG 1 / 2: the merged row is written as nibble / byte digits of the [seq_q, num_q_heads * hd]
 // matrix that o_proj multiplies (hd a multiple of 32; workgroup = row qt * nqh + qh), not as f32.
+// A record is hdr floats (maximum, exp-sum, padding) followed by the row.
 template <int DIG>
-__global__ __launch_bounds__(128) void gqa_combine_kernel(const float *__restrict__ part, int splits, int hd,
+__global__ __launch_bounds__(128) void gqa_combine_kernel(const float *__restrict__ part, int splits, int hd, int hdr,
                                                           float *__restrict__ out, int accumulate, int nqh,
                                                           int8_t *__restrict__ digits, float *__restrict__ xs) {
     __shared__ float wts[ATT_SPLITS_MAX];
     __shared__ float red[2];
-    const float *p = part + (size_t)blockIdx.x * splits * (hd + 2);
+    const size_t rec = (size_t)(hd + hdr);
+    const float *p = part + (size_t)blockIdx.x * splits * rec;
     const int tid = threadIdx.x;
     float M = -INFINITY;
-    for (int s = tid; s < splits; s += 128) M = fmaxf(M, p[(size_t)s * (hd + 2)]);
+    for (int s = tid; s < splits; s += 128) M = fmaxf(M, p[s * rec]);
     M = block_max(M, red);
     float l = 0.f;
     for (int s = tid; s < splits; s += 128) {
-        const float m = p[(size_t)s * (hd + 2)];
+        const float m = p[s * rec];
         const float w = m == -INFINITY ? 0.f : expf(m - M);
         wts[s] = w;
-        l += w * p[(size_t)s * (hd + 2) + 1];
+        l += w * p[s * rec + 1];
     }
     l = block_sum(l, red);  // its barriers publish wts[]
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     if constexpr (DIG == 0) {
         for (int i = tid; i < hd; i += 128) {
             float o = 0.f;
-            for (int s = 0; s < splits; ++s) o += wts[s] * p[(size_t)s * (hd + 2) + 2 + i];
+            for (int s = 0; s < splits; ++s) o += wts[s] * p[s * rec + hdr + i];
             float *dst = out + (size_t)blockIdx.x * hd + i;
             *dst = accumulate ? *dst + o * inv : o * inv;
         }
@@ -1095,7 +1141,7 @@ __global__ __launch_bounds__(128) void gqa_combine_kernel(const float *__restric
             float o[4] = {0.f, 0.f, 0.f, 0.f};
             for (int s = 0; s < splits; ++s) {
                 const float wv = wts[s];
-                const float *src = p + (size_t)s * (hd + 2) + 2 + 4 * i4;
+                const float *src = p + s * rec + hdr + 4 * i4;
                 o[0] += wv * src[0]; o[1] += wv * src[1]; o[2] += wv * src[2]; o[3] += wv * src[3];
             }
             for (int j = 0; j < 4; ++j) o[j] *= inv;
@@ -1243,6 +1289,25 @@ bool attention_is_short(const pg_ctx *ctx, size_t rows, size_t len, size_t hd) {
            (len + ATT_SHORT_ROUNDS * keys_per_round - 1) / (ATT_SHORT_ROUNDS * keys_per_round) <= (size_t)ATT_SPLITS_MAX;
 }
 
+// Whether a call with several query tokens should cut its keys into runs for the matrix-core kernel (its
+// workgroups, one per kv head and pair of 32-row items, would leave most CUs idle while each walks a long
+// cache), and how: *chunk tiles of 32 keys per run, *splits runs.
+bool split_mfma_tiles(const pg_ctx *ctx, size_t group, size_t seq_q, size_t nkv, int mask_kind, size_t offset, size_t len,
+                      size_t *chunk, size_t *splits) {
+    const size_t n_items = (group * seq_q + 31) / 32, wgs = (n_items + 1) / 2 * nkv;
+    const size_t kend = mask_kind != 0 && offset + seq_q < len ? offset + seq_q : len;
+    const size_t tiles = (kend + 31) / 32;
+    if (wgs * 2 > (size_t)ctx->num_cu || tiles < 8) return false;
+    // A tile costs a wavefront about 5 us whatever the number of live rows (128 matrix instructions of 16 passes,
+    // one wavefront per SIMD), so the runs are as short as two workgroups per CU allow
+    size_t want = (2 * (size_t)ctx->num_cu + wgs - 1) / wgs;
+    if (want > tiles) want = tiles;
+    if (want > (size_t)ATT_SPLITS_MAX) want = ATT_SPLITS_MAX;
+    *chunk = (tiles + want - 1) / want;
+    *splits = (tiles + *chunk - 1) / *chunk;
+    return *splits > 1;
+}
+
 pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, const pg_kv_cache *vc, size_t nqh,
                            size_t seq_q, float scale, int mask_kind, size_t offset, size_t window, size_t sink,
                            float logit_cap, float *out, int accumulate, const pg_xdigits *xd = nullptr, int digit_kind = 0,
@@ -1280,7 +1345,7 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     // short kernel handles with every load in flight at once.
     const size_t rows = seq_q * nqh, keys_per_round = 256 / (size_t)lanes;
     size_t chunk, splits;
-    bool short_kernel = false, tiled_kernel = false, decode_kernel = false;
+    bool short_kernel = false, tiled_kernel = false, decode_kernel = false, split_kernel = false;
     int dec_u = 1, dec_tps = 1;
     const uintptr_t align_all = (uintptr_t)q | (uintptr_t)out | (uintptr_t)kc->k | (uintptr_t)vc->v |
                                 (rope_fusion ? (uintptr_t)rope_fusion->raw_q | (uintptr_t)rope_fusion->raw_k | (uintptr_t)rope_fusion->raw_v |
@@ -1300,6 +1365,10 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
         chunk = tps * u * tile_rows;
         dec_u = (int)u; dec_tps = (int)tps;
         decode_kernel = true;
+    } else if (seq_q > 1 && (hd == 64 || hd == 128) && align_all % 16 == 0 && split_mfma_tiles(ctx, nqh / kc->num_kv_heads, seq_q,
+                                                                                                 kc->num_kv_heads, mask_kind, offset, len, &chunk, &splits)) {
+        // few rows under a long cache: the matrix-core kernel over runs of key tiles, then the merge
+        tiled_kernel = split_kernel = true;
     } else if (attention_is_short(ctx, rows, len, hd)) {
         chunk = ATT_SHORT_ROUNDS * keys_per_round;
         splits = (len + chunk - 1) / chunk;
@@ -1315,7 +1384,8 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     }
     if (splits > (size_t)ATT_SPLITS_MAX) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: cache of %zu positions is too long", len);
     aa.chunk = (int)chunk; aa.splits = (int)splits;
-    const size_t part_bytes = splits > 1 || decode_kernel ? pg_round_up(rows * splits * (hd + 2) * sizeof(float), 256) : 0;
+    const size_t part_hdr = split_kernel ? 4 : 2;  // floats ahead of a partial row (maximum, exp-sum, padding)
+    const size_t part_bytes = splits > 1 || decode_kernel ? pg_round_up(rows * splits * (hd + part_hdr) * sizeof(float), 256) : 0;
     const size_t bits_words = mask_kind == PG_MASK_LOCAL_GLOBAL ? (len + 31) / 32 : 0;
     if (part_bytes + bits_words) {
         void *ws = nullptr;
@@ -1358,9 +1428,11 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
         // matrix-core kernel: one workgroup per kv head and pair of 32-row items (first with last, ...);
         // the kv head varies fastest, so with eight kv heads each XCD's L2 keeps one head's keys and values
         const size_t G = nqh / kc->num_kv_heads, n_items = (G * seq_q + 31) / 32, pairs = (n_items + 1) / 2;
-        if (pairs * kc->num_kv_heads >= (1ull << 31)) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: grid too large");
-        auto *kern = hd == 64 ? gqa_attention_mfma_kernel<64> : gqa_attention_mfma_kernel<128>;
-        PG_TRY(pg_launch(ctx, "gqa_attention_mfma", kern, dim3((unsigned)(pairs * kc->num_kv_heads)), dim3(128), 0, aa, (int)n_items,
+        if (pairs * kc->num_kv_heads * splits >= (1ull << 31)) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: grid too large");
+        auto *kern = split_kernel ? (hd == 64 ? gqa_attention_mfma_kernel<64, true> : gqa_attention_mfma_kernel<128, true>)
+                                  : (hd == 64 ? gqa_attention_mfma_kernel<64> : gqa_attention_mfma_kernel<128>);
+        PG_TRY(pg_launch(ctx, split_kernel ? "gqa_attention_mfma_split" : "gqa_attention_mfma", kern,
+                         dim3((unsigned)(pairs * kc->num_kv_heads * (split_kernel ? splits : 1))), dim3(128), 0, aa, (int)n_items,
                          (int)kc->num_kv_heads));
     } else if (tiled_kernel) {
         const size_t G = nqh / kc->num_kv_heads, row_sets = (G * seq_q + ATT_T_ROWS - 1) / ATT_T_ROWS;
@@ -1380,8 +1452,8 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
     } else if (splits > 1 || decode_kernel) {
         auto *kern = !xd ? gqa_combine_kernel<0> : (digit_kind == PG_GGML_Q4_0 ? gqa_combine_kernel<1> : gqa_combine_kernel<2>);
         PG_TRY(pg_launch(ctx, xd ? "gqa_combine_digits" : "gqa_combine", kern, dim3((unsigned)rows), dim3(128), 0,
-                         (const float *)aa.part, (int)splits, (int)hd, out, accumulate, (int)nqh, xd ? xd->digits : nullptr,
-                         xd ? xd->xs : nullptr));
+                         (const float *)aa.part, (int)splits, (int)hd, (int)part_hdr, out, accumulate, (int)nqh,
+                         xd ? xd->digits : nullptr, xd ? xd->xs : nullptr));
     } else if (xd) {
         PG_TRY(pg_launch_x_to_digits(ctx, out, seq_q, nqh * hd, digit_kind, *xd));
     }

@@ -251,6 +251,27 @@ def test_gqa_attention_one_token_heads_of_a_group_together(ctx, orc):
     assert (a == _attention_case(ctx, orc, 8, 1, 128, 1, 9000, M.causal(8999), None, seed + 7)).all()
 
 
+def test_gqa_attention_few_rows_under_a_long_cache(ctx, orc):
+    """Several query tokens, but too few rows to fill the chip, over a long cache (a chunk of a prefill, draft
+    tokens being verified): the matrix-core kernel runs over runs of key tiles and the runs are merged.  Rows
+    that fill less than one 32-row item, an odd number of items (a wavefront without work), runs that some rows
+    cannot see at all (causal, the chunk at the end of the cache or in its middle), every mask kind, a logit cap."""
+    from peregrine_amd import llama
+    M = llama.AttentionMask
+    say("attention, few rows under a long cache")
+    _attention_case(ctx, orc, 32, 8, 128, 2, 1026, M.causal(1024), None, 401)
+    _attention_case(ctx, orc, 32, 8, 128, 8, 1032, M.causal(1024), None, 402, appends=(1024, 8))
+    _attention_case(ctx, orc, 32, 8, 128, 16, 1040, M.causal(1024), None, 403)
+    _attention_case(ctx, orc, 32, 8, 128, 32, 2080, M.none(), None, 404)
+    _attention_case(ctx, orc, 6, 2, 64, 30, 700, M.causal(670), 3.0, 405)                        # 90 rows: three items
+    _attention_case(ctx, orc, 6, 2, 64, 30, 700, M.causal(200), None, 406)                       # most of the cache is ahead
+    _attention_case(ctx, orc, 8, 2, 64, 5, 900, M.causal_sliding_window(895, 100, 4), None, 407)  # whole runs hidden
+    _attention_case(ctx, orc, 8, 2, 128, 12, 600, M.local_global(588, 40, [0, 7, 64, 300, 301, 599, 9999]), None, 408)
+    _attention_case(ctx, orc, 4, 4, 128, 3, 5000, M.causal(4997), None, 409)                     # one head per kv head
+    a = _attention_case(ctx, orc, 16, 2, 128, 9, 3000, M.causal(2991), None, 410)
+    assert (a == _attention_case(ctx, orc, 16, 2, 128, 9, 3000, M.causal(2991), None, 410)).all()
+
+
 def test_gqa_attention_long_cache_splits_keys(ctx, orc):
     """A long cache under one query row: the keys are cut into many splits and merged."""
     from peregrine_amd import llama
