@@ -744,10 +744,21 @@ def section_llama_block(B, line):
         check(lib.pg_kv_cache_rollback_to(kv, ctx_len))
         check(lib.pg_llama_block_forward_dev(B.h, b, ptr(h_dec), 1, kv, ptr(o_dec)))
 
+    h_few = B.normal(1282, (4, d_l))
+    o_few = torch.empty_like(h_few)
+
+    def block_few():  # four tokens at once on top of the prefilled cache (draft tokens being verified), then rolled back
+        b, kv = blocks_l[B.i % L_ROT]
+        B.i += 1
+        check(lib.pg_kv_cache_rollback_to(kv, ctx_len))
+        check(lib.pg_llama_block_forward_dev(B.h, b, ptr(h_few), 4, kv, ptr(o_few)))
+
     t_pre = B.timed(block_prefill, 16, 8)  # leaves every cache filled to ctx_len
     pre_prof, _ = B.profiled(block_prefill, 8)
     t_bd = B.timed(block_decode, B.dsteps, max(args.warmup, 8))
     dec_prof, _ = B.profiled(block_decode, B.dsteps)
+    t_few = B.timed(block_few, B.dsteps, max(args.warmup, 8))
+    few_prof, _ = B.profiled(block_few, B.dsteps)
     kv_bytes_l = 2 * nkv_l * (ctx_len + 1) * hd_l * 4
     dec_bytes_l = w_bytes_l + kv_bytes_l
     pre_flops = 2 * ctx_len * sum(no * ki for no, ki in shapes_l) + 4 * nqh_l * hd_l * ctx_len * (ctx_len + 1) // 2
@@ -759,6 +770,9 @@ def section_llama_block(B, line):
                    "frac_of_hbm_peak": round(dec_bytes_l / (t_bd["ms_per_step"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                    "bytes_per_step": dec_bytes_l, "launches_per_step": round(sum(v[1] for v in dec_prof.values()) / B.dsteps, 2),
                    "kernels_ms_x_launches": {k: [round(v[0], 5), round(v[1] / B.dsteps, 2)] for k, v in dec_prof.items()}},
+        "four_tokens": {"what": f"seq 4 at positions {ctx_len}..{ctx_len + 3}", **B.stats(t_few),
+                        "launches_per_step": round(sum(v[1] for v in few_prof.values()) / B.dsteps, 2),
+                        "kernels_ms_x_launches": {k: [round(v[0], 5), round(v[1] / B.dsteps, 2)] for k, v in few_prof.items()}},
         "prefill": {"what": f"seq {ctx_len} into an empty cache", **B.stats(t_pre, 4),
                     "tflops": round(pre_flops / (t_pre["ms_per_step"] * 1e-3) / 1e12, 1),
                     "tokens_per_s": round(ctx_len / (t_pre["ms_per_step"] * 1e-3), 0),

@@ -93,3 +93,69 @@ __device__ __forceinline__ void pg_emit_digits(const float (&f)[4], size_t row, 
     }
     if (sub == 0) xs[row * (size_t)nb + b] = s;
 }
+
+// ---- activation blocks -> two byte-digit planes for the matrix-core block product (gguf_mm_kernel) ----
+// digits[row][plane][b][half][16]: plane 0 = high digit, 1 = low digit of X[k] = round(x[k] / xs[b]).
+// The 16 bytes of (b, half) follow the order in which the weight operand presents its k:
+//   Q8_0: half h holds elements 16h .. 16h+15;
+//   Q4_0: half h holds elements 2i + h (i = 0..15): the low (h = 0) or high (h = 1) nibbles
+//         of the block's 16 bytes (byte i = elements 2i, 2i+1, src/gguf.rs:316-323).
+// xs[row][nbp]: block scales absmax / 32639 (NaN for a block holding NaN or inf), nbp = nb
+// rounded up to 4.
+// Bytes from one activation row's digits to the next: the two planes (nb * 64 bytes) padded to
+// an odd number of 256-byte lines.  The 32 token rows of a tile are fetched at the same K
+// offset at the same time; an even (worst: power-of-two, 64 KiB at K = 32768) stride sends
+// all of them to the same memory channels.
+__host__ __device__ static inline size_t pg_mm_row_bytes(size_t nb) {
+    const size_t lines = (nb * 64 + 255) / 256;
+    return (lines | 1) * 256;
+}
+
+// Eight consecutive lanes hold block b of activation row `row`, four elements each (as for pg_emit_digits);
+// all eight must call together.
+template <bool NIB>
+__device__ __forceinline__ void pg_emit_mm_digits(const float (&f)[4], size_t row, int b, int sub, int nb, int nbp,
+                                                  int8_t *__restrict__ digits, float *__restrict__ xs) {
+    float amax = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3])));
+    int bad = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]);
+    amax = fmaxf(amax, __builtin_bit_cast(float, pg_dpp8<0xB1>(__builtin_bit_cast(int, amax))));
+    bad |= pg_dpp8<0xB1>(bad);
+    amax = fmaxf(amax, __builtin_bit_cast(float, pg_dpp8<0x4E>(__builtin_bit_cast(int, amax))));
+    bad |= pg_dpp8<0x4E>(bad);
+    amax = fmaxf(amax, __builtin_bit_cast(float, pg_dpp8<0x141>(__builtin_bit_cast(int, amax))));
+    bad |= pg_dpp8<0x141>(bad);
+    float s = 1.0f, inv = 1.0f;
+    if (bad || !(amax <= 3.4028234663852886e38f)) {
+        s = __uint_as_float(0x7FC00000u);
+        inv = 0.0f;
+    } else if (amax > 0.0f) {
+        // the two signed byte digits reach 127 * 256 + 127: map the block's absmax onto that
+        s = fmaxf(amax / 32639.0f, 1.17549435e-38f);
+        inv = 1.0f / s;
+    }
+    int hi[4], lo[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float t = f[e] * inv;
+        const int X = (t != t) ? 0 : (int)rintf(t);
+        lo[e] = ((X + 128) & 255) - 128;
+        hi[e] = (X - lo[e]) >> 8;
+    }
+    int8_t *d0 = digits + row * pg_mm_row_bytes(nb) + (size_t)b * 32;  // plane 0, block b: [half][16]
+    int8_t *d1 = d0 + (size_t)nb * 32;
+    if (NIB) {
+        // elements 4*sub + {0, 2} -> half 0 positions 2*sub, 2*sub+1;  {1, 3} -> half 1, same positions
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            *reinterpret_cast<uint16_t *>(d0 + h * 16 + 2 * sub) = (uint16_t)((hi[h] & 255) | ((hi[h + 2] & 255) << 8));
+            *reinterpret_cast<uint16_t *>(d1 + h * 16 + 2 * sub) = (uint16_t)((lo[h] & 255) | ((lo[h + 2] & 255) << 8));
+        }
+    } else {
+        const int h = sub >> 2, pos = (sub & 3) * 4;
+        *reinterpret_cast<unsigned *>(d0 + h * 16 + pos) = (unsigned)(hi[0] & 255) | ((unsigned)(hi[1] & 255) << 8) |
+                                                          ((unsigned)(hi[2] & 255) << 16) | ((unsigned)(hi[3] & 255) << 24);
+        *reinterpret_cast<unsigned *>(d1 + h * 16 + pos) = (unsigned)(lo[0] & 255) | ((unsigned)(lo[1] & 255) << 8) |
+                                                          ((unsigned)(lo[2] & 255) << 16) | ((unsigned)(lo[3] & 255) << 24);
+    }
+    if (sub == 0) xs[row * (size_t)nbp + b] = s;
+}

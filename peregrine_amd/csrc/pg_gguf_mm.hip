@@ -17,6 +17,7 @@
 // being consumed: each wavefront's own 32 weight rows and their f16 block scales, and the
 // token digits and scales of the stage, which the four wavefronts share.
 #include "pg_internal.h"
+#include "pg_digits.h"
 
 namespace {
 
@@ -46,23 +47,7 @@ template <int QT> struct MMCfg {
     static constexpr int LPS = 2 + 1 + 1 + W_FILLS;             // LDS fills per wavefront and stage
 };
 
-// ---- activation rows -> two byte-digit planes -------------------------------------------
-// digits[row][plane][b][half][16]: plane 0 = high digit, 1 = low digit of X[k] = round(x[k] / xs[b]).
-// The 16 bytes of (b, half) follow the order in which the weight operand presents its k:
-//   Q8_0: half h holds elements 16h .. 16h+15;
-//   Q4_0: half h holds elements 2i + h (i = 0..15): the low (h = 0) or high (h = 1) nibbles
-//         of the block's 16 bytes (byte i = elements 2i, 2i+1, src/gguf.rs:316-323).
-// xs[row][nbp]: block scales absmax / 32639 (NaN for a block holding NaN or inf), nbp = nb
-// rounded up to 4.  8 consecutive threads own one block (4 elements each).
-// Bytes from one activation row's digits to the next: the two planes (nb * 64 bytes) padded to
-// an odd number of 256-byte lines.  The 32 token rows of a tile are fetched at the same K
-// offset at the same time; an even (worst: power-of-two, 64 KiB at K = 32768) stride sends
-// all of them to the same memory channels.
-__host__ __device__ static inline size_t mm_row_bytes(size_t nb) {
-    const size_t lines = (nb * 64 + 255) / 256;
-    return (lines | 1) * 256;
-}
-
+// ---- activation rows -> two byte-digit planes (pg_emit_mm_digits, pg_digits.h) ----------
 template <bool NIB>
 __global__ __launch_bounds__(256) void x_to_mm_digits_kernel(const float *__restrict__ x, int nb, int nbp,
                                                              int8_t *__restrict__ digits, float *__restrict__ xs) {
@@ -71,47 +56,7 @@ __global__ __launch_bounds__(256) void x_to_mm_digits_kernel(const float *__rest
     if (b >= nb) return;  // whole 8-thread groups leave together
     const float4 v = reinterpret_cast<const float4 *>(x + (row * nb + b) * 32)[sub];
     const float f[4] = {v.x, v.y, v.z, v.w};
-    float amax = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3])));
-    int bad = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]);
-#pragma unroll
-    for (int off = 1; off < 8; off <<= 1) {
-        amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-        bad |= __shfl_xor(bad, off, 64);
-    }
-    float s = 1.0f, inv = 1.0f;
-    if (bad || !(amax <= 3.4028234663852886e38f)) {
-        s = __uint_as_float(0x7FC00000u);
-        inv = 0.0f;
-    } else if (amax > 0.0f) {
-        // the two signed byte digits reach 127 * 256 + 127: map the block's absmax onto that
-        s = fmaxf(amax / 32639.0f, 1.17549435e-38f);
-        inv = 1.0f / s;
-    }
-    int hi[4], lo[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const float t = f[e] * inv;
-        const int X = (t != t) ? 0 : (int)rintf(t);
-        lo[e] = ((X + 128) & 255) - 128;
-        hi[e] = (X - lo[e]) >> 8;
-    }
-    int8_t *d0 = digits + row * mm_row_bytes(nb) + (size_t)b * 32;  // plane 0, block b: [half][16]
-    int8_t *d1 = d0 + (size_t)nb * 32;
-    if (NIB) {
-        // elements 4*sub + {0, 2} -> half 0 positions 2*sub, 2*sub+1;  {1, 3} -> half 1, same positions
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            *reinterpret_cast<uint16_t *>(d0 + h * 16 + 2 * sub) = (uint16_t)((hi[h] & 255) | ((hi[h + 2] & 255) << 8));
-            *reinterpret_cast<uint16_t *>(d1 + h * 16 + 2 * sub) = (uint16_t)((lo[h] & 255) | ((lo[h + 2] & 255) << 8));
-        }
-    } else {
-        const int h = sub >> 2, pos = (sub & 3) * 4;
-        *reinterpret_cast<unsigned *>(d0 + h * 16 + pos) = (unsigned)(hi[0] & 255) | ((unsigned)(hi[1] & 255) << 8) |
-                                                          ((unsigned)(hi[2] & 255) << 16) | ((unsigned)(hi[3] & 255) << 24);
-        *reinterpret_cast<unsigned *>(d1 + h * 16 + pos) = (unsigned)(lo[0] & 255) | ((unsigned)(lo[1] & 255) << 8) |
-                                                          ((unsigned)(lo[2] & 255) << 16) | ((unsigned)(lo[3] & 255) << 24);
-    }
-    if (sub == 0) xs[row * (size_t)nbp + b] = s;
+    pg_emit_mm_digits<NIB>(f, row, b, sub, nb, nbp, digits, xs);
 }
 
 // Two's-complement nibbles (as stored at upload) of one dword -> four signed bytes holding
@@ -206,7 +151,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int unit = (2 * wave + u) * 8 + (lane >> 3), tok = unit >> 1, pl = unit & 1;
         const int ch = (lane & 7) ^ (tok & 7);
         dig_jb[u] = ch >> 1;
-        dig_src[u] = digits + xrow_of(tok) * mm_row_bytes(nb) + (size_t)pl * nb * 32 + (ch & 1) * 16;
+        dig_src[u] = digits + xrow_of(tok) * pg_mm_row_bytes(nb) + (size_t)pl * nb * 32 + (ch & 1) * 16;
     }
     // xs: lanes 0..7 of wavefront w fetch the 4 block scales of tokens 8w .. 8w+7
     const float *xs_src = xs + xrow_of(8 * wave + (lane & 7)) * (size_t)nbp;
@@ -512,7 +457,7 @@ __global__ void sum_parts_kernel(const float *__restrict__ part, size_t n, int k
 
 size_t pg_mmdigits_bytes(size_t rows, size_t k) {
     const size_t nb = k / 32, nbp = pg_round_up(nb, 4);
-    return rows * mm_row_bytes(nb) + pg_round_up(rows * nbp * sizeof(float), 256);
+    return rows * pg_mm_row_bytes(nb) + pg_round_up(rows * nbp * sizeof(float), 256);
 }
 
 pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k) {
@@ -520,7 +465,7 @@ pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k) {
     pg_mmdigits md;
     char *p = static_cast<char *>(base);
     md.digits = reinterpret_cast<int8_t *>(p);
-    p += rows * mm_row_bytes(nb);
+    p += rows * pg_mm_row_bytes(nb);
     md.xs = reinterpret_cast<float *>(p);
     md.rows = rows;
     md.k = k;
@@ -542,7 +487,7 @@ pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows,
 // of a token tile reads them: then K is split so that a chunk's share does fit, and the chunks
 // are dealt to XCDs (see the kernel).  Without the split a K = 32768 product over 128 rows
 // fetches its 8 MiB of digits once per 128-row group: 1.2x the weight bytes in total.
-static bool digits_exceed_l2(size_t act_rows, size_t nb) { return act_rows * mm_row_bytes(nb) > (2u << 20); }
+static bool digits_exceed_l2(size_t act_rows, size_t nb) { return act_rows * pg_mm_row_bytes(nb) > (2u << 20); }
 
 int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t groups, size_t act_rows, bool grouped,
                       int *chunk_out, bool *xcd_chunks) {
@@ -558,7 +503,7 @@ int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t group
     // (Plain products over 16 token tiles and more are not split: they run as super-tiles.)
     if ((grouped || groups < 16) && digits_exceed_l2(act_rows, nb)) {
         size_t c = 2;
-        while (c < 8 && act_rows * mm_row_bytes(nb) > c * (size_t)(2u << 20)) c *= 2;
+        while (c < 8 && act_rows * pg_mm_row_bytes(nb) > c * (size_t)(2u << 20)) c *= 2;
         // worth it while the partial sums (written and read back) stay under a tenth of the weights
         const bool cheap = c * act_rows * 8 * 10 <= nb * 34 * (grouped ? groups : 1);  // per weight row
         if (c >= ks && nb / c >= 8 * NBU && cheap) {
@@ -577,7 +522,7 @@ int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t group
 
 pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,
                             const uint16_t *d, const pg_mm_group &grp, size_t total_pairs, const pg_mmdigits &md,
-                            float *y, float *part) {
+                            float *y, float *part, bool keep_parts) {
     if (total_pairs == 0) return PG_OK;
     const int nb = (int)(k_in / 32), nbp = (int)pg_round_up(nb, 4);
     const size_t experts = grp.counts ? (size_t)grp.num_experts : 1;
@@ -616,7 +561,7 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
     const bool nt = grp.counts != nullptr;
     if (ggml_type == PG_GGML_Q4_0) PG_TRY(nt ? launch(gguf_mm_kernel<4, true>, "gguf_mm_q4_0") : launch(gguf_mm_kernel<4, false>, "gguf_mm_q4_0"));
     else PG_TRY(nt ? launch(gguf_mm_kernel<8, true>, "gguf_mm_q8_0") : launch(gguf_mm_kernel<8, false>, "gguf_mm_q8_0"));
-    if (ks > 1)
+    if (ks > 1 && !keep_parts)
         PG_TRY(pg_launch(ctx, "gguf_mm_sum_parts", sum_parts_kernel, dim3(grid_for(stride, 256)), dim3(256), 0, part, stride, ks,
                          stride, y));
     return PG_OK;

@@ -319,7 +319,7 @@ int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t group
                       int *chunk_out, bool *xcd_chunks = nullptr);
 pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,
                             const uint16_t *d, const pg_mm_group &grp, size_t total_pairs, const pg_mmdigits &md,
-                            float *y, float *part);
+                            float *y, float *part, bool keep_parts = false);  // keep_parts: the K chunks' planes are left in `part` unsummed
 // y[m, n_out] = x[m, k_in] . dequant(w)^T on device pointers (uses the scratch arena).
 // MXFP4 tensors (pg_mxfp4.hip): qs holds the code bytes in matrix-core fragment order, d the E8M0 scale
 // bytes (four per dword); every product over them runs pg_launch_mxfp4_rows.

@@ -38,6 +38,8 @@ struct pg_llama_block {
     float *ss_part;  // one-token step: sums of squares of the attention output row, by block of 32
     float *arena;  // activations for seq_cap tokens
     size_t seq_cap;
+    void *chain;   // many-token step: digit planes of the three product inputs and the products' K-chunk planes
+    size_t chain_bytes;
     // One-token step: digit buffers for the three GEMV inputs (model_dim, q_dim, ffn) and the
     // device tables that let k/v and gate/up each run as one two-item launch.
     void *dec;                        // one allocation
@@ -98,12 +100,16 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(const float *a, const 
 // The same with the row held in registers: dim % 4 == 0 and dim <= 1024 * MAXV, so that every
 // load of the row is issued before the first is needed.
 // DIG: 0 = write the normalised row as f32; 1 / 2 = write it as nibble / byte digits for the
-// streaming product instead (dim a multiple of 32, so that 8-lane groups hold whole blocks).
+// streaming product instead (dim a multiple of 32, so that 8-lane groups hold whole blocks); 3 / 4 = as the
+// two byte-digit planes of the matrix-core block product (Q4_0 / Q8_0 element order).
+// The second input may come as b_planes planes, b_stride4 float4 apart (the K chunks of a split product,
+// summed here in ascending order before the addition, as gguf_mm's own summing pass would).
 template <int MAXV, int DIG>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(const float4 *__restrict__ a, const float4 *__restrict__ b,
                                                               float4 *__restrict__ sum_out, const float4 *__restrict__ w,
                                                               float eps, int dim4, float4 *__restrict__ out,
-                                                              int8_t *__restrict__ digits, float *__restrict__ xs) {
+                                                              int8_t *__restrict__ digits, float *__restrict__ xs,
+                                                              int b_planes, size_t b_stride4) {
     __shared__ float red[4];
     const size_t row = (size_t)blockIdx.x * dim4;
     float4 v[MAXV], wv[MAXV];
@@ -117,7 +123,11 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(const float4 *__re
         for (int j = 0; j < MAXV; ++j) {
             const int i = threadIdx.x + 256 * j;
             if (i < dim4) {
-                const float4 t = b[row + i];
+                float4 t = b[row + i];
+                for (int pl = 1; pl < b_planes; ++pl) {
+                    const float4 t2 = b[pl * b_stride4 + row + i];
+                    t.x += t2.x; t.y += t2.y; t.z += t2.z; t.w += t2.w;
+                }
                 v[j].x += t.x; v[j].y += t.y; v[j].z += t.z; v[j].w += t.w;
                 sum_out[row + i] = v[j];
             }
@@ -140,7 +150,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(const float4 *__re
             const float o[4] = {v[j].x * inv_rms * wv[j].x, v[j].y * inv_rms * wv[j].y, v[j].z * inv_rms * wv[j].z,
                                 v[j].w * inv_rms * wv[j].w};
             if constexpr (DIG == 0) out[row + i] = float4{o[0], o[1], o[2], o[3]};
-            else pg_emit_digits<DIG == 1>(o, blockIdx.x, i >> 3, i & 7, dim4 >> 3, digits, xs);
+            else if constexpr (DIG <= 2) pg_emit_digits<DIG == 1>(o, blockIdx.x, i >> 3, i & 7, dim4 >> 3, digits, xs);
+            else pg_emit_mm_digits<DIG == 3>(o, blockIdx.x, i >> 3, i & 7, dim4 >> 3, ((dim4 >> 3) + 3) & ~3, digits, xs);
         }
     }
 }
@@ -151,6 +162,8 @@ struct rope_seg {
     float *dst;        // at dst + h*dst_hstride + t*hd
     size_t src_tstride, dst_hstride;
     int heads, rotate;
+    int planes = 1;          // src as the sum of this many planes (the K chunks of a split product), in ascending order
+    size_t plane_stride = 0;
 };
 struct rope_args {
     rope_seg seg[3];
@@ -166,13 +179,18 @@ __global__ __launch_bounds__(128) void rope_kernel(rope_args ra) {
     const float *src = sg.src + (size_t)t * sg.src_tstride + (size_t)h * ra.hd;
     float *dst = sg.dst + (size_t)h * sg.dst_hstride + (size_t)t * ra.hd;
     const int half = ra.hd / 2;
+    auto at = [&](int i) {
+        float x = src[i];
+        for (int pl = 1; pl < sg.planes; ++pl) x += src[pl * sg.plane_stride + i];
+        return x;
+    };
     if (!sg.rotate) {
-        for (int i = threadIdx.x; i < ra.hd; i += 128) dst[i] = src[i];
+        for (int i = threadIdx.x; i < ra.hd; i += 128) dst[i] = at(i);
         return;
     }
     const float *c = ra.cos_t + (size_t)(ra.pos0 + t) * ra.hd, *sn = ra.sin_t + (size_t)(ra.pos0 + t) * ra.hd;
     for (int i = threadIdx.x; i < half; i += 128) {
-        const float x0 = src[i], x1 = src[half + i];
+        const float x0 = at(i), x1 = at(half + i);
         dst[i] = x0 * c[i] - x1 * sn[i];
         dst[half + i] = x0 * sn[i] + x1 * c[i];
     }
@@ -1238,6 +1256,37 @@ __global__ __launch_bounds__(256) void swiglu_digits_kernel(const float4 *__rest
     pg_emit_digits<NIB>(o, 0, i >> 3, i & 7, n4 >> 3, digits, xs);
 }
 
+// Rows of silu(g) * u written as the matrix-core product's digit planes (n a multiple of 32 per row); g and u
+// each the sum of `planes` planes, `stride` floats apart, in ascending order.
+template <bool NIB>
+__global__ __launch_bounds__(256) void swiglu_mm_digits_kernel(const float *__restrict__ g, const float *__restrict__ u, int planes,
+                                                               size_t stride, int nb, int nbp, int8_t *__restrict__ digits,
+                                                               float *__restrict__ xs) {
+    const size_t row = blockIdx.y;
+    const int b = blockIdx.x * 32 + (threadIdx.x >> 3), sub = threadIdx.x & 7;
+    if (b >= nb) return;  // whole 8-thread groups leave together
+    const size_t at = (row * nb + b) * 8 + sub;  // float4 index
+    float4 gv = reinterpret_cast<const float4 *>(g)[at], uv = reinterpret_cast<const float4 *>(u)[at];
+    for (int pl = 1; pl < planes; ++pl) {
+        const float4 g2 = reinterpret_cast<const float4 *>(g + pl * stride)[at], u2 = reinterpret_cast<const float4 *>(u + pl * stride)[at];
+        gv.x += g2.x; gv.y += g2.y; gv.z += g2.z; gv.w += g2.w;
+        uv.x += u2.x; uv.y += u2.y; uv.z += u2.z; uv.w += u2.w;
+    }
+    const float o[4] = {gv.x / (1.0f + expf(-gv.x)) * uv.x, gv.y / (1.0f + expf(-gv.y)) * uv.y,
+                        gv.z / (1.0f + expf(-gv.z)) * uv.z, gv.w / (1.0f + expf(-gv.w)) * uv.w};
+    pg_emit_mm_digits<NIB>(o, row, b, sub, nb, nbp, digits, xs);
+}
+
+// out = a + (b as the sum of `planes` planes, in ascending order)
+__global__ __launch_bounds__(256) void add_planes_kernel(const float *__restrict__ a, const float *__restrict__ b, int planes,
+                                                         size_t stride, float *__restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float t = b[i];
+    for (int pl = 1; pl < planes; ++pl) t += b[pl * stride + i];
+    out[i] = a[i] + t;
+}
+
 // (a fill kernel rather than hipMemsetAsync: a caller may capture the stream-ordered entry points in a graph)
 __global__ __launch_bounds__(256) void zero_f32_kernel(float *__restrict__ p, size_t n) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -1264,7 +1313,7 @@ pg_status launch_rmsnorm_digits(pg_ctx *ctx, const float *a, const float *b, flo
     auto *kern = dim <= 4096 ? (nib ? add_rmsnorm_vec_kernel<4, 1> : add_rmsnorm_vec_kernel<4, 2>)
                              : (nib ? add_rmsnorm_vec_kernel<8, 1> : add_rmsnorm_vec_kernel<8, 2>);
     return pg_launch(ctx, "add_rmsnorm_digits", kern, dim3((unsigned)rows), dim3(256), 0, (const float4 *)a, (const float4 *)b,
-                     (float4 *)sum_out, (const float4 *)w, eps, (int)(dim / 4), (float4 *)nullptr, xd.digits, xd.xs);
+                     (float4 *)sum_out, (const float4 *)w, eps, (int)(dim / 4), (float4 *)nullptr, xd.digits, xd.xs, 1, (size_t)0);
 }
 
 pg_status launch_rmsnorm(pg_ctx *ctx, const float *a, const float *b, float *sum_out, const float *w, float eps,
@@ -1274,7 +1323,7 @@ pg_status launch_rmsnorm(pg_ctx *ctx, const float *a, const float *b, float *sum
         auto *kern = dim <= 4096 ? add_rmsnorm_vec_kernel<4, 0> : add_rmsnorm_vec_kernel<8, 0>;
         return pg_launch(ctx, "add_rmsnorm", kern, dim3((unsigned)rows), dim3(256), 0, (const float4 *)a, (const float4 *)b,
                          (float4 *)sum_out, (const float4 *)w, eps, (int)(dim / 4), (float4 *)out, (int8_t *)nullptr,
-                         (float *)nullptr);
+                         (float *)nullptr, 1, (size_t)0);
     }
     return pg_launch(ctx, "add_rmsnorm", add_rmsnorm_kernel, dim3((unsigned)rows), dim3(256), 0, a, b, sum_out, w, eps,
                      (int)dim, out);
@@ -1839,6 +1888,7 @@ PG_API void pg_llama_block_free(pg_ctx *ctx, pg_llama_block *b) {
     pg_rope_free(ctx, b->rope);
     if (b->attn_norm_w) (void)hipFree(b->attn_norm_w);
     if (b->arena) (void)hipFree(b->arena);
+    if (b->chain) (void)hipFree(b->chain);
     if (b->dec) (void)hipFree(b->dec);
     delete b;
 }
@@ -1993,6 +2043,84 @@ static pg_status block_forward_one_token(pg_ctx *ctx, pg_llama_block *b, const f
     return pg_launch_gguf_gemv(ctx, b->w[6]->ggml_type, d, ffn, b->w[6]->qs, b->w[6]->d, one, b->xd_f, out_dev, h1);
 }
 
+// The many-token step with all seven tensors Q4_0 (or all Q8_0): every product's input reaches it as the two
+// digit planes its producer wrote (RMSNorm, SiLU.up), and a product whose K was cut into chunks leaves the
+// chunks' planes to its consumer, which adds them up as it reads (RoPE, the residual add inside the second
+// RMSNorm, SiLU.up, the last residual add).  The same arithmetic in the same order as the product-by-product
+// route, 15 launches instead of 25 when every product is split (a few tokens: each launch is 4 us there).
+static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const float *h_dev, size_t seq, pg_kv_cache *cache,
+                                       float *out_dev, float *h1, float *q_rope, float *attn) {
+    const size_t d = b->d, hd = b->hd, q_dim = b->nqh * hd, kv_dim = b->nkvh * hd, ffn = b->ffn, offset = cache->len;
+    const int type = b->digit_kind;
+    const bool nib = type == PG_GGML_Q4_0;
+    const size_t tiles = (seq + 31) / 32;
+    const size_t n_of[7] = {q_dim, kv_dim, kv_dim, d, ffn, ffn, d}, k_of[7] = {d, d, d, q_dim, d, d, ffn};
+    int ks[7];
+    size_t part_off[7], floats = 0;
+    for (int i = 0; i < 7; ++i) {
+        ks[i] = pg_gguf_mm_splitk(ctx, n_of[i], k_of[i], tiles, seq, false, nullptr);
+        part_off[i] = floats;
+        floats += pg_round_up((size_t)ks[i] * seq * n_of[i], 64);
+    }
+    const size_t sz_d = pg_mmdigits_bytes(seq, d), sz_q = pg_mmdigits_bytes(seq, q_dim), sz_f = pg_mmdigits_bytes(seq, ffn);
+    const size_t need = sz_d + sz_q + sz_f + floats * sizeof(float);
+    if (need > b->chain_bytes) {
+        PG_HIP(hipStreamSynchronize(ctx->stream));
+        if (b->chain) (void)hipFree(b->chain);
+        b->chain = nullptr;
+        b->chain_bytes = 0;
+        const size_t want = need + need / 4;
+        PG_HIP(hipMalloc(&b->chain, want));
+        b->chain_bytes = want;
+    }
+    char *base = static_cast<char *>(b->chain);
+    const pg_mmdigits md_d = pg_mmdigits_carve(base, seq, d), md_q = pg_mmdigits_carve(base + sz_d, seq, q_dim),
+                      md_f = pg_mmdigits_carve(base + sz_d + sz_q, seq, ffn);
+    float *parts = reinterpret_cast<float *>(base + sz_d + sz_q + sz_f);
+    auto part = [&](int i) { return parts + part_off[i]; };
+    pg_mm_group grp = {1, nullptr, nullptr, nullptr, nullptr, 0, (int)tiles, (int)seq, 1};
+    grp.tiled = 1;
+    auto product = [&](int i, const pg_mmdigits &md) -> pg_status {
+        PG_TRY(pg_gguf_ensure_tiled(ctx, b->w[i]));
+        return pg_launch_gguf_mm(ctx, type, n_of[i], k_of[i], b->w[i]->qs_tiled, b->w[i]->d, grp, seq, md, part(i), part(i), true);
+    };
+    auto norm_digits = [&](const float *a, int bi, float *sum_out, const float *w) -> pg_status {
+        auto *kern = d <= 4096 ? (nib ? add_rmsnorm_vec_kernel<4, 3> : add_rmsnorm_vec_kernel<4, 4>)
+                               : (nib ? add_rmsnorm_vec_kernel<8, 3> : add_rmsnorm_vec_kernel<8, 4>);
+        return pg_launch(ctx, "add_rmsnorm_mm_digits", kern, dim3((unsigned)seq), dim3(256), 0, (const float4 *)a,
+                         (const float4 *)(bi >= 0 ? part(bi) : nullptr), (float4 *)sum_out, (const float4 *)w, b->eps, (int)(d / 4),
+                         (float4 *)nullptr, md_d.digits, md_d.xs, bi >= 0 ? ks[bi] : 1, seq * d / 4);
+    };
+    const int nbf = (int)(ffn / 32);
+
+    PG_TRY(norm_digits(h_dev, -1, nullptr, b->attn_norm_w));
+    for (int i = 0; i < 3; ++i) PG_TRY(product(i, md_d));
+    PG_TRY(cache_reserve(ctx, cache, offset + seq));
+    rope_args ra = {};
+    ra.seg[0] = {part(0), q_rope, q_dim, seq * hd, (int)b->nqh, 1, ks[0], seq * q_dim};
+    ra.seg[1] = {part(1), cache->k + offset * hd, kv_dim, cache->capacity * hd, (int)b->nkvh, 1, ks[1], seq * kv_dim};
+    ra.seg[2] = {part(2), cache->v + offset * hd, kv_dim, cache->capacity * hd, (int)b->nkvh, 0, ks[2], seq * kv_dim};
+    ra.cos_t = b->rope->cos_t; ra.sin_t = b->rope->sin_t; ra.hd = (int)hd; ra.pos0 = (int)offset; ra.nseg = 3;
+    PG_TRY(launch_rope(ctx, ra, seq, b->nqh + 2 * b->nkvh));
+    cache->len = offset + seq;
+    PG_TRY(launch_attention(ctx, q_rope, cache, cache, b->nqh, seq, 1.0f / sqrtf((float)hd), PG_MASK_CAUSAL, offset, 0, 0,
+                            0.0f, attn, 0));
+    PG_TRY(pg_launch_x_to_mm_digits(ctx, attn, seq, q_dim, type, md_q));
+    PG_TRY(product(3, md_q));
+    PG_TRY(norm_digits(h_dev, 3, h1, b->ffn_norm_w));  // h1 = h + attn . Wo, and its norm as digits
+    PG_TRY(product(4, md_d));
+    PG_TRY(product(5, md_d));
+    {
+        auto *kern = nib ? swiglu_mm_digits_kernel<true> : swiglu_mm_digits_kernel<false>;
+        PG_TRY(pg_launch(ctx, "swiglu_mm_digits", kern, dim3((unsigned)((nbf + 31) / 32), (unsigned)seq), dim3(256), 0,
+                         (const float *)part(4), (const float *)part(5), ks[4], seq * ffn, nbf, (int)pg_round_up(nbf, 4),
+                         md_f.digits, md_f.xs));
+    }
+    PG_TRY(product(6, md_f));
+    return pg_launch(ctx, "residual_add", add_planes_kernel, dim3(blocks_for(seq * d)), dim3(256), 0, (const float *)h1,
+                     (const float *)part(6), ks[6], seq * d, out_dev, seq * d);
+}
+
 PG_API pg_status pg_llama_block_forward_dev(pg_ctx *ctx, pg_llama_block *b, const float *h_dev, size_t seq,
                                             pg_kv_cache *cache, float *out_dev) {
     PG_TRY(pg_use(ctx));
@@ -2030,6 +2158,10 @@ PG_API pg_status pg_llama_block_forward_dev(pg_ctx *ctx, pg_llama_block *b, cons
     float *qd = take(cap * q_dim), *q_rope = take(cap * q_dim), *attn = take(cap * q_dim);
     float *kd = take(cap * kv_dim), *vd = take(cap * kv_dim);
     float *g = take(cap * ffn), *u = take(cap * ffn);  // the one-token step relies on this order (k, v and g, u adjacent)
+    const size_t min_k = PG_MM_MIN_BLOCKS * 32;
+    if (b->digit_kind != 0 && seq <= 65535 && d >= min_k && q_dim >= min_k && ffn >= min_k && d <= 8192 &&
+        ((uintptr_t)h_dev | (uintptr_t)out_dev) % 16 == 0)
+        return block_forward_chained(ctx, b, h_dev, seq, cache, out_dev, h1, q_rope, attn);
 
     PG_TRY(launch_rmsnorm(ctx, h_dev, nullptr, nullptr, b->attn_norm_w, b->eps, seq, d, normed));
     float *const qkv[3] = {qd, kd, vd};
