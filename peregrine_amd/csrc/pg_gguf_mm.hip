@@ -84,9 +84,9 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
 // (MoE step 1.22 -> 1.17 ms); wrong for a prefill, where 32 token tiles re-read every weight.
 template <int QT, bool NT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gguf_mm_kernel(const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0,
-                                                      pg_mm_group grp, int n_out, int nb, int nbp, int chunk,
+                                                      pg_mm_group grp, int n_out_arg, int nb, int nbp, int chunk,
                                                       const int8_t *__restrict__ digits, const float *__restrict__ xs,
-                                                      float *__restrict__ out, size_t part_stride) {
+                                                      float *__restrict__ out_arg, size_t part_stride_arg) {
     extern __shared__ __attribute__((aligned(1024))) char lds[];  // RING * STAGE bytes
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -126,6 +126,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (tt * 32 >= count) return;  // the same for every thread of the workgroup
     const uint8_t *qs_any = grp.qs_table ? grp.qs_table[e] : qs0;
     const uint16_t *d_any = grp.d_table ? grp.d_table[e] : d0;
+    int n_out = n_out_arg;
+    float *__restrict__ out = out_arg;
+    size_t part_stride = part_stride_arg;
+    if (grp.nseg) {  // which tensor of the launch this row group belongs to
+        int t = 0;
+        while (t + 1 < grp.nseg && bx >= grp.seg_first[t + 1]) ++t;
+        bx -= grp.seg_first[t];
+        qs_any = grp.seg_qs[t];
+        d_any = grp.seg_d[t];
+        n_out = grp.seg_n[t];
+        out = grp.seg_out[t];
+        part_stride = grp.seg_stride[t];
+    }
 
     constexpr int STAGE = MMCfg<QT>::STAGE, W_WAVE = MMCfg<QT>::W_WAVE, W_FILLS = MMCfg<QT>::W_FILLS;
     // Activation row of a token slot of this tile (spare slots shadow the tile's first token).
@@ -532,6 +545,8 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
     bool by_xcd = false;
     const int ks = pg_gguf_mm_splitk(ctx, n_out, k_in, grp.counts ? experts : gy, md.rows, grp.counts != nullptr, &chunk, &by_xcd);
     if (ks > 1 && !part) return pg_fail(PG_EINVAL, "gguf_mm: split-K needs a partial-sum buffer");
+    if (grp.nseg && ((ks > 1 && !keep_parts) || grp.counts || !grp.tiled))
+        return pg_fail(PG_EINVAL, "gguf_mm: several tensors in one launch leave their K chunks unsummed, take no expert lists and read tile-major copies");
     if (gy > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_mm: too many token tiles");
     dim3 grid(grid_for(n_out, 128), (unsigned)gy, (unsigned)ks);
     pg_mm_group g2 = grp;

@@ -303,6 +303,15 @@ struct pg_mm_group {
     int remap_rg, remap_tiles;  // set by the launcher (row groups and token tiles of an XCD-aware 1-D launch), else 0
     int tiled;                  // the qs pointers are tile-major copies (pg_gguf_tensor::qs_tiled)
     int xcd_ks;                 // set by the launcher: K chunks dealt to XCDs (2, 4 or 8), else 0
+    // Several tensors of equal K in one launch (q|k|v, gate|up): the launch's 128-row groups are the tensors'
+    // groups one after the other; tensor t starts at group seg_first[t], has seg_n[t] rows, its own tile-major
+    // copy, scales and output (planes seg_stride[t] floats apart).  nseg = 0: the one tensor of the arguments.
+    int nseg;
+    int seg_first[3], seg_n[3];
+    const uint8_t *seg_qs[3];
+    const uint16_t *seg_d[3];
+    float *seg_out[3];
+    size_t seg_stride[3];
 };
 // Bytes from one 128-row group of a tile-major copy to the next: the group's stages (16 KiB
 // each for Q8_0, 8 KiB for Q4_0) plus 4352 bytes, so that workgroups walking their groups in

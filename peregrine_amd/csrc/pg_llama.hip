@@ -2047,7 +2047,8 @@ static pg_status block_forward_one_token(pg_ctx *ctx, pg_llama_block *b, const f
 // digit planes its producer wrote (RMSNorm, SiLU.up), and a product whose K was cut into chunks leaves the
 // chunks' planes to its consumer, which adds them up as it reads (RoPE, the residual add inside the second
 // RMSNorm, SiLU.up, the last residual add).  The same arithmetic in the same order as the product-by-product
-// route, 15 launches instead of 25 when every product is split (a few tokens: each launch is 4 us there).
+// route, with q|k|v and gate|up as one launch each: 12 launches instead of 25 when every product is split (a few
+// tokens: each launch is 4 us there).
 static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const float *h_dev, size_t seq, pg_kv_cache *cache,
                                        float *out_dev, float *h1, float *q_rope, float *attn) {
     const size_t d = b->d, hd = b->hd, q_dim = b->nqh * hd, kv_dim = b->nkvh * hd, ffn = b->ffn, offset = cache->len;
@@ -2055,10 +2056,14 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     const bool nib = type == PG_GGML_Q4_0;
     const size_t tiles = (seq + 31) / 32;
     const size_t n_of[7] = {q_dim, kv_dim, kv_dim, d, ffn, ffn, d}, k_of[7] = {d, d, d, q_dim, d, d, ffn};
+    // q|k|v and gate|up are one launch each (the tensors' 128-row groups one after the other): one K split for the launch
+    const int first_of[7] = {0, 0, 0, 3, 4, 4, 6}, count_of[7] = {3, 3, 3, 1, 2, 2, 1};
     int ks[7];
     size_t part_off[7], floats = 0;
     for (int i = 0; i < 7; ++i) {
-        ks[i] = pg_gguf_mm_splitk(ctx, n_of[i], k_of[i], tiles, seq, false, nullptr);
+        size_t groups = 0;
+        for (int j = first_of[i]; j < first_of[i] + count_of[i]; ++j) groups += (n_of[j] + 127) / 128;
+        ks[i] = pg_gguf_mm_splitk(ctx, groups * 128, k_of[i], tiles, seq, false, nullptr);
         part_off[i] = floats;
         floats += pg_round_up((size_t)ks[i] * seq * n_of[i], 64);
     }
@@ -2080,9 +2085,20 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     auto part = [&](int i) { return parts + part_off[i]; };
     pg_mm_group grp = {1, nullptr, nullptr, nullptr, nullptr, 0, (int)tiles, (int)seq, 1};
     grp.tiled = 1;
-    auto product = [&](int i, const pg_mmdigits &md) -> pg_status {
-        PG_TRY(pg_gguf_ensure_tiled(ctx, b->w[i]));
-        return pg_launch_gguf_mm(ctx, type, n_of[i], k_of[i], b->w[i]->qs_tiled, b->w[i]->d, grp, seq, md, part(i), part(i), true);
+    auto product = [&](int i, const pg_mmdigits &md) -> pg_status {  // tensors i .. i + count_of[i] - 1
+        pg_mm_group g = grp;
+        size_t groups = 0;
+        g.nseg = count_of[i] > 1 ? count_of[i] : 0;
+        for (int j = 0; j < count_of[i]; ++j) {
+            PG_TRY(pg_gguf_ensure_tiled(ctx, b->w[i + j]));
+            g.seg_first[j] = (int)groups; g.seg_n[j] = (int)n_of[i + j];
+            g.seg_qs[j] = b->w[i + j]->qs_tiled; g.seg_d[j] = b->w[i + j]->d;
+            g.seg_out[j] = part(i + j); g.seg_stride[j] = seq * n_of[i + j];
+            groups += (n_of[i + j] + 127) / 128;
+        }
+        if (count_of[i] == 1)
+            return pg_launch_gguf_mm(ctx, type, n_of[i], k_of[i], b->w[i]->qs_tiled, b->w[i]->d, g, seq, md, part(i), part(i), true);
+        return pg_launch_gguf_mm(ctx, type, groups * 128, k_of[i], nullptr, nullptr, g, seq, md, part(i), part(i), true);
     };
     auto norm_digits = [&](const float *a, int bi, float *sum_out, const float *w) -> pg_status {
         auto *kern = d <= 4096 ? (nib ? add_rmsnorm_vec_kernel<4, 3> : add_rmsnorm_vec_kernel<4, 4>)
@@ -2094,7 +2110,7 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     const int nbf = (int)(ffn / 32);
 
     PG_TRY(norm_digits(h_dev, -1, nullptr, b->attn_norm_w));
-    for (int i = 0; i < 3; ++i) PG_TRY(product(i, md_d));
+    PG_TRY(product(0, md_d));
     PG_TRY(cache_reserve(ctx, cache, offset + seq));
     rope_args ra = {};
     ra.seg[0] = {part(0), q_rope, q_dim, seq * hd, (int)b->nqh, 1, ks[0], seq * q_dim};
@@ -2109,7 +2125,6 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     PG_TRY(product(3, md_q));
     PG_TRY(norm_digits(h_dev, 3, h1, b->ffn_norm_w));  // h1 = h + attn . Wo, and its norm as digits
     PG_TRY(product(4, md_d));
-    PG_TRY(product(5, md_d));
     {
         auto *kern = nib ? swiglu_mm_digits_kernel<true> : swiglu_mm_digits_kernel<false>;
         PG_TRY(pg_launch(ctx, "swiglu_mm_digits", kern, dim3((unsigned)((nbf + 31) / 32), (unsigned)seq), dim3(256), 0,
