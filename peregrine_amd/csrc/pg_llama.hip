@@ -53,6 +53,8 @@ struct pg_llama_block {
 
 namespace {
 
+constexpr int PG_MAX_PLANES = 8;  // K chunks of a split block product (pg_gguf_mm_splitk never makes more)
+
 __device__ __forceinline__ float block_sum(float v, float *red) {
     v = pg_wave_sum_f32(v);
     const int wave = threadIdx.x >> 6;
@@ -123,11 +125,14 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(const float4 *__re
         for (int j = 0; j < MAXV; ++j) {
             const int i = threadIdx.x + 256 * j;
             if (i < dim4) {
-                float4 t = b[row + i];
-                for (int pl = 1; pl < b_planes; ++pl) {
-                    const float4 t2 = b[pl * b_stride4 + row + i];
-                    t.x += t2.x; t.y += t2.y; t.z += t2.z; t.w += t2.w;
-                }
+                float4 tp[PG_MAX_PLANES];  // every plane requested before the first is used
+#pragma unroll
+                for (int pl = 0; pl < PG_MAX_PLANES; ++pl)
+                    tp[pl] = pl < b_planes ? b[pl * b_stride4 + row + i] : float4{0.f, 0.f, 0.f, 0.f};
+                float4 t = tp[0];
+#pragma unroll
+                for (int pl = 1; pl < PG_MAX_PLANES; ++pl)
+                    if (pl < b_planes) { t.x += tp[pl].x; t.y += tp[pl].y; t.z += tp[pl].z; t.w += tp[pl].w; }
                 v[j].x += t.x; v[j].y += t.y; v[j].z += t.z; v[j].w += t.w;
                 sum_out[row + i] = v[j];
             }
@@ -180,8 +185,13 @@ __global__ __launch_bounds__(128) void rope_kernel(rope_args ra) {
     float *dst = sg.dst + (size_t)h * sg.dst_hstride + (size_t)t * ra.hd;
     const int half = ra.hd / 2;
     auto at = [&](int i) {
-        float x = src[i];
-        for (int pl = 1; pl < sg.planes; ++pl) x += src[pl * sg.plane_stride + i];
+        float xp[PG_MAX_PLANES];
+#pragma unroll
+        for (int pl = 0; pl < PG_MAX_PLANES; ++pl) xp[pl] = pl < sg.planes ? src[pl * sg.plane_stride + i] : 0.f;
+        float x = xp[0];
+#pragma unroll
+        for (int pl = 1; pl < PG_MAX_PLANES; ++pl)
+            if (pl < sg.planes) x += xp[pl];
         return x;
     };
     if (!sg.rotate) {
@@ -1164,7 +1174,9 @@ __global__ __launch_bounds__(128) void gqa_combine_kernel(const float *__restric
             }
             for (int j = 0; j < 4; ++j) o[j] *= inv;
             const int e4 = qh * (hd / 4) + i4;  // float4 index within the row
-            pg_emit_digits<DIG == 1>(o, qt, e4 >> 3, e4 & 7, nqh * hd / 32, digits, xs);
+            const int nb = nqh * hd / 32;
+            if constexpr (DIG <= 2) pg_emit_digits<DIG == 1>(o, qt, e4 >> 3, e4 & 7, nb, digits, xs);
+            else pg_emit_mm_digits<DIG == 3>(o, qt, e4 >> 3, e4 & 7, nb, (nb + 3) & ~3, digits, xs);  // the matrix-core product's planes
         }
     }
 }
@@ -1266,11 +1278,20 @@ __global__ __launch_bounds__(256) void swiglu_mm_digits_kernel(const float *__re
     const int b = blockIdx.x * 32 + (threadIdx.x >> 3), sub = threadIdx.x & 7;
     if (b >= nb) return;  // whole 8-thread groups leave together
     const size_t at = (row * nb + b) * 8 + sub;  // float4 index
-    float4 gv = reinterpret_cast<const float4 *>(g)[at], uv = reinterpret_cast<const float4 *>(u)[at];
-    for (int pl = 1; pl < planes; ++pl) {
-        const float4 g2 = reinterpret_cast<const float4 *>(g + pl * stride)[at], u2 = reinterpret_cast<const float4 *>(u + pl * stride)[at];
-        gv.x += g2.x; gv.y += g2.y; gv.z += g2.z; gv.w += g2.w;
-        uv.x += u2.x; uv.y += u2.y; uv.z += u2.z; uv.w += u2.w;
+    float4 gp[PG_MAX_PLANES], up[PG_MAX_PLANES];
+#pragma unroll
+    for (int pl = 0; pl < PG_MAX_PLANES; ++pl) {
+        const bool have = pl < planes;
+        gp[pl] = have ? reinterpret_cast<const float4 *>(g + pl * stride)[at] : float4{0.f, 0.f, 0.f, 0.f};
+        up[pl] = have ? reinterpret_cast<const float4 *>(u + pl * stride)[at] : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    float4 gv = gp[0], uv = up[0];
+#pragma unroll
+    for (int pl = 1; pl < PG_MAX_PLANES; ++pl) {
+        if (pl < planes) {
+            gv.x += gp[pl].x; gv.y += gp[pl].y; gv.z += gp[pl].z; gv.w += gp[pl].w;
+            uv.x += up[pl].x; uv.y += up[pl].y; uv.z += up[pl].z; uv.w += up[pl].w;
+        }
     }
     const float o[4] = {gv.x / (1.0f + expf(-gv.x)) * uv.x, gv.y / (1.0f + expf(-gv.y)) * uv.y,
                         gv.z / (1.0f + expf(-gv.z)) * uv.z, gv.w / (1.0f + expf(-gv.w)) * uv.w};
@@ -1282,8 +1303,13 @@ __global__ __launch_bounds__(256) void add_planes_kernel(const float *__restrict
                                                          size_t stride, float *__restrict__ out, size_t n) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
-    float t = b[i];
-    for (int pl = 1; pl < planes; ++pl) t += b[pl * stride + i];
+    float tp[PG_MAX_PLANES];
+#pragma unroll
+    for (int pl = 0; pl < PG_MAX_PLANES; ++pl) tp[pl] = pl < planes ? b[pl * stride + i] : 0.f;
+    float t = tp[0];
+#pragma unroll
+    for (int pl = 1; pl < PG_MAX_PLANES; ++pl)
+        if (pl < planes) t += tp[pl];
     out[i] = a[i] + t;
 }
 
@@ -1361,7 +1387,9 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
                            size_t seq_q, float scale, int mask_kind, size_t offset, size_t window, size_t sink,
                            float logit_cap, float *out, int accumulate, const pg_xdigits *xd = nullptr, int digit_kind = 0,
                            const size_t *global_positions = nullptr, size_t num_global = 0,
-                           const attn_args *rope_fusion = nullptr) {
+                           const attn_args *rope_fusion = nullptr, const pg_mmdigits *md = nullptr, bool *md_written = nullptr) {
+    // With `md` (digit_kind names the tensor type) a merge of key runs writes the rows as the matrix-core
+    // product's digit planes instead of f32 and sets *md_written; a kernel that needs no merge writes `out`.
     // With `xd` (one-token step, accumulate == 0, head_dim % 32 == 0) the rows also, or only,
     // leave as GEMV digits of kind `digit_kind`; `out` must still be a valid buffer.
     const size_t len = kc->len, hd = kc->head_dim;
@@ -1498,6 +1526,11 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
                               : (dg == 0 ? gqa_combine_few_kernel<128, 0> : (dg == 1 ? gqa_combine_few_kernel<128, 1> : gqa_combine_few_kernel<128, 2>));
         PG_TRY(pg_launch(ctx, xd ? "gqa_combine_digits" : "gqa_combine", kern, dim3((unsigned)rows), dim3(256), 0, (const float *)aa.part,
                          (int)splits, out, accumulate, (int)nqh, xd ? xd->digits : (int8_t *)nullptr, xd ? xd->xs : (float *)nullptr));
+    } else if ((splits > 1 || decode_kernel) && md && !xd && !accumulate && hd % 32 == 0) {
+        auto *kern = digit_kind == PG_GGML_Q4_0 ? gqa_combine_kernel<3> : gqa_combine_kernel<4>;
+        PG_TRY(pg_launch(ctx, "gqa_combine_mm_digits", kern, dim3((unsigned)rows), dim3(128), 0, (const float *)aa.part, (int)splits,
+                         (int)hd, (int)part_hdr, out, accumulate, (int)nqh, md->digits, md->xs));
+        if (md_written) *md_written = true;
     } else if (splits > 1 || decode_kernel) {
         auto *kern = !xd ? gqa_combine_kernel<0> : (digit_kind == PG_GGML_Q4_0 ? gqa_combine_kernel<1> : gqa_combine_kernel<2>);
         PG_TRY(pg_launch(ctx, xd ? "gqa_combine_digits" : "gqa_combine", kern, dim3((unsigned)rows), dim3(128), 0,
@@ -2064,6 +2097,7 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
         size_t groups = 0;
         for (int j = first_of[i]; j < first_of[i] + count_of[i]; ++j) groups += (n_of[j] + 127) / 128;
         ks[i] = pg_gguf_mm_splitk(ctx, groups * 128, k_of[i], tiles, seq, false, nullptr);
+        if (ks[i] > PG_MAX_PLANES) return pg_fail(PG_EUNSUPPORTED, "llama block: a product in %d K chunks", ks[i]);
         part_off[i] = floats;
         floats += pg_round_up((size_t)ks[i] * seq * n_of[i], 64);
     }
@@ -2119,9 +2153,10 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     ra.cos_t = b->rope->cos_t; ra.sin_t = b->rope->sin_t; ra.hd = (int)hd; ra.pos0 = (int)offset; ra.nseg = 3;
     PG_TRY(launch_rope(ctx, ra, seq, b->nqh + 2 * b->nkvh));
     cache->len = offset + seq;
+    bool md_written = false;  // (a merge of key runs writes the o-projection's digit planes itself)
     PG_TRY(launch_attention(ctx, q_rope, cache, cache, b->nqh, seq, 1.0f / sqrtf((float)hd), PG_MASK_CAUSAL, offset, 0, 0,
-                            0.0f, attn, 0));
-    PG_TRY(pg_launch_x_to_mm_digits(ctx, attn, seq, q_dim, type, md_q));
+                            0.0f, attn, 0, nullptr, type, nullptr, 0, nullptr, hd % 32 == 0 ? &md_q : nullptr, &md_written));
+    if (!md_written) PG_TRY(pg_launch_x_to_mm_digits(ctx, attn, seq, q_dim, type, md_q));
     PG_TRY(product(3, md_q));
     PG_TRY(norm_digits(h_dev, 3, h1, b->ffn_norm_w));  // h1 = h + attn . Wo, and its norm as digits
     PG_TRY(product(4, md_d));
