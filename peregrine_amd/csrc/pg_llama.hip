@@ -1428,7 +1428,7 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
                                 (rope_fusion ? (uintptr_t)rope_fusion->raw_q | (uintptr_t)rope_fusion->raw_k | (uintptr_t)rope_fusion->raw_v |
                                                    (uintptr_t)rope_fusion->rope_c | (uintptr_t)rope_fusion->rope_s
                                              : 0);
-    if (seq_q == 1 && (hd == 64 || hd == 128) && align_all % 16 == 0 && attention_is_short(ctx, rows, len, hd)) {
+    if (seq_q == 1 && (hd == 64 || hd == 128) && align_all % 16 == 0 && rows < 2 * (size_t)ctx->num_cu) {  // (any cache length)
         // one token: the heads of a kv group share a workgroup
         const size_t nkv = kc->num_kv_heads, tile_rows = 2048 / hd;
         const size_t kend = mask_kind != 0 && offset + 1 < len ? offset + 1 : len;

@@ -273,10 +273,14 @@ def test_gqa_attention_few_rows_under_a_long_cache(ctx, orc):
 
 
 def test_gqa_attention_long_cache_splits_keys(ctx, orc):
-    """A long cache under one query row: the keys are cut into many splits and merged."""
+    """A long cache under one query row: the keys are cut into many splits and merged.  Head size 16 takes the
+    general kernels; head size 128 at 140 000 keys the one-token kernel with 35 tiles per split (a length at
+    which 64-key splits would exceed the merge's limit of 2048)."""
     from peregrine_amd import llama
     say("attention len=40000")
     _attention_case(ctx, orc, 2, 1, 16, 1, 40000, llama.AttentionMask.causal(39999), None, 55)
+    say("attention len=140000")
+    _attention_case(ctx, orc, 4, 1, 128, 1, 140000, llama.AttentionMask.causal(139999), None, 56)
 
 
 def test_gqa_attention_edges(ctx, orc):
