@@ -384,6 +384,7 @@ def main():
         section_mxfp4(B, line)
         section_moe(B, line)
         section_llama_block(B, line)
+        section_decode_attention(B, line)
         section_huffman(B, line)
 
     if args.calibrate_copy:  # a plain copy of known size: 512 MiB read + 512 MiB written per launch
@@ -695,6 +696,46 @@ def section_moe(B, line):
         for h in w3:
             lib.pg_gguf_free(B.h, h)
     torch.cuda.empty_cache()
+
+
+def section_decode_attention(B, line):
+    """GQA attention of one query token (32 query heads over 8 kv heads of 128, causal) over f32 caches of 1 025 to
+    32 769 positions: the bytes are the keys and values, read once."""
+    torch, lib, check, ptr, dev = B.torch, B.lib, B.check, B.ptr, B.dev
+    nqh, nkv, hd = 32, 8, 128
+    out_rows = []
+    for ctx_len in (1025, 8193, 32769):
+        caches = []
+        for r in range(3):  # three caches rotated (0.8 GB at the longest: more than the Infinity Cache)
+            kv = C.c_void_p()
+            check(lib.pg_kv_cache_create(B.h, nkv, hd, C.byref(kv)))
+            k = B.normal(1400 + r, (nkv, ctx_len, hd))
+            check(lib.pg_kv_cache_append_dev(B.h, kv, ptr(k), ptr(k), ctx_len))
+            caches.append(kv)
+            del k
+        q = B.normal(1410, (nqh, 1, hd))
+        out = torch.zeros(1, nqh * hd, device=dev)
+
+        def step():
+            kv = caches[B.i % 3]
+            B.i += 1
+            check(lib.pg_gqa_attention_dev(B.h, ptr(q), kv, kv, nqh, 1, C.c_float(hd ** -0.5), 1, ctx_len - 1, 0, 0,
+                                           C.c_float(0.0), ptr(out)))
+
+        t = B.timed(step, B.dsteps, max(B.args.warmup, 8))
+        prof, _ = B.profiled(step, B.dsteps)
+        nbytes = 2 * nkv * ctx_len * hd * 4
+        k_ms = prof["gqa_decode"][0]
+        out_rows.append({"positions": ctx_len, **B.stats(t), "bytes_per_step": nbytes,
+                         "value": round(nbytes / (t["ms_per_step"] * 1e-3) / 1e9, 1), "unit": "GB/s",
+                         "kernels_ms": {k: round(v[0], 5) for k, v in prof.items()},
+                         "roofline": {"kernel": "gqa_decode_kernel<128, U>", "bound": "hbm", "achieved": round(nbytes / (k_ms * 1e-3) / 1e9, 1),
+                                      "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(nbytes / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                                      "traffic": None, "bytes_per_launch": nbytes, "avg_launch_ms": round(k_ms, 5)}})
+        for kv in caches:
+            lib.pg_kv_cache_free(B.h, kv)
+        torch.cuda.empty_cache()
+    line["decode_attention"] = {"workload": "one query token, 32 / 8 heads of 128, causal, f32 caches; 3 caches rotated", "by_length": out_rows}
 
 
 def section_llama_block(B, line):
