@@ -650,9 +650,9 @@ __global__ __launch_bounds__(256) void gqa_attention_tiled_kernel(attn_args aa) 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 // SPLIT (few rows under a long cache: a chunk of a prefill, a handful of draft tokens): the keys are cut
-// into aa.splits runs of aa.chunk tiles as well, workgroup = (kv head, two adjacent items, run), one item per
-// wavefront and no hand-over; every wavefront leaves (maximum, exp-sum, unnormalised rows) for
-// gqa_combine_kernel in rows of HD + 4 floats, or an empty record where its rows see none of the run's keys.
+// into aa.splits runs of aa.chunk tiles as well, workgroup = one wavefront = (kv head, item, run), no
+// hand-over; every wavefront leaves (maximum, exp-sum, unnormalised rows) for gqa_combine_kernel in rows of
+// HD + 4 floats, or an empty record where its rows see none of the run's keys.
 template <int HD, bool SPLIT = false>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void gqa_attention_mfma_kernel(attn_args aa, int n_items, int nkvh) {
@@ -662,9 +662,8 @@ void gqa_attention_mfma_kernel(attn_args aa, int n_items, int nkvh) {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int col = lane & 31, h = lane >> 5;
     const int kvh = blockIdx.x % nkvh;
-    const int n_pairs = (n_items + 1) / 2;
-    const int pair = SPLIT ? (blockIdx.x / nkvh) % n_pairs : blockIdx.x / nkvh;
-    const int run = SPLIT ? (blockIdx.x / nkvh) / n_pairs : 0;
+    const int pair = SPLIT ? (blockIdx.x / nkvh) % n_items : blockIdx.x / nkvh;  // SPLIT: the item itself
+    const int run = SPLIT ? (blockIdx.x / nkvh) / n_items : 0;
     const int G = aa.group, nrows = G * aa.seq_q;
     const int item_a = pair, item_b = n_items - 1 - pair;  // the short and the long one (equal: one item)
     auto kend_of = [&](int item) {
@@ -684,8 +683,7 @@ void gqa_attention_mfma_kernel(attn_args aa, int n_items, int nkvh) {
         int t0 = wave == 0 ? 0 : (seg == 0 ? 0 : cut);
         int t1 = wave == 0 ? (seg == 0 ? cut : 0) : (seg == 0 ? ta : tb);
         if constexpr (SPLIT) {
-            item = 2 * pair + wave;
-            if (item >= n_items) return;  // (no barrier on this path)
+            item = pair;
             t0 = run * aa.chunk;
             t1 = min((kend_of(item) + 31) / 32, t0 + aa.chunk);
         } else {
@@ -1369,13 +1367,13 @@ bool attention_is_short(const pg_ctx *ctx, size_t rows, size_t len, size_t hd) {
 // cache), and how: *chunk tiles of 32 keys per run, *splits runs.
 bool split_mfma_tiles(const pg_ctx *ctx, size_t group, size_t seq_q, size_t nkv, int mask_kind, size_t offset, size_t len,
                       size_t *chunk, size_t *splits) {
-    const size_t n_items = (group * seq_q + 31) / 32, wgs = (n_items + 1) / 2 * nkv;
+    const size_t n_items = (group * seq_q + 31) / 32, wgs = n_items * nkv;  // one wavefront each
     const size_t kend = mask_kind != 0 && offset + seq_q < len ? offset + seq_q : len;
     const size_t tiles = (kend + 31) / 32;
     if (wgs * 2 > (size_t)ctx->num_cu || tiles < 8) return false;
     // A tile costs a wavefront about 5 us whatever the number of live rows (128 matrix instructions of 16 passes,
-    // one wavefront per SIMD), so the runs are as short as two workgroups per CU allow
-    size_t want = (2 * (size_t)ctx->num_cu + wgs - 1) / wgs;
+    // one wavefront per SIMD), so the runs are as short as one wavefront per SIMD allows
+    size_t want = (4 * (size_t)ctx->num_cu + wgs - 1) / wgs;
     if (want > tiles) want = tiles;
     if (want > (size_t)ATT_SPLITS_MAX) want = ATT_SPLITS_MAX;
     *chunk = (tiles + want - 1) / want;
@@ -1505,12 +1503,15 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
         // matrix-core kernel: one workgroup per kv head and pair of 32-row items (first with last, ...);
         // the kv head varies fastest, so with eight kv heads each XCD's L2 keeps one head's keys and values
         const size_t G = nqh / kc->num_kv_heads, n_items = (G * seq_q + 31) / 32, pairs = (n_items + 1) / 2;
-        if (pairs * kc->num_kv_heads * splits >= (1ull << 31)) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: grid too large");
+        if (n_items * kc->num_kv_heads * splits >= (1ull << 31)) return pg_fail(PG_EUNSUPPORTED, "gqa_attention: grid too large");
         auto *kern = split_kernel ? (hd == 64 ? gqa_attention_mfma_kernel<64, true> : gqa_attention_mfma_kernel<128, true>)
                                   : (hd == 64 ? gqa_attention_mfma_kernel<64> : gqa_attention_mfma_kernel<128>);
-        PG_TRY(pg_launch(ctx, split_kernel ? "gqa_attention_mfma_split" : "gqa_attention_mfma", kern,
-                         dim3((unsigned)(pairs * kc->num_kv_heads * (split_kernel ? splits : 1))), dim3(128), 0, aa, (int)n_items,
-                         (int)kc->num_kv_heads));
+        if (split_kernel)  // one wavefront per workgroup: (kv head, item, run)
+            PG_TRY(pg_launch(ctx, "gqa_attention_mfma_split", kern, dim3((unsigned)(n_items * kc->num_kv_heads * splits)), dim3(64), 0, aa,
+                             (int)n_items, (int)kc->num_kv_heads));
+        else
+            PG_TRY(pg_launch(ctx, "gqa_attention_mfma", kern, dim3((unsigned)(pairs * kc->num_kv_heads)), dim3(128), 0, aa, (int)n_items,
+                             (int)kc->num_kv_heads));
     } else if (tiled_kernel) {
         const size_t G = nqh / kc->num_kv_heads, row_sets = (G * seq_q + ATT_T_ROWS - 1) / ATT_T_ROWS;
         const dim3 grid_t((unsigned)row_sets, (unsigned)kc->num_kv_heads);
