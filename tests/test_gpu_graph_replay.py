@@ -1,0 +1,98 @@
+"""The block step under stream capture: pg_llama_block_forward_dev, once its buffers exist, only launches
+kernels on the context's stream, so a caller may capture a step into a hipGraph and replay it.
+
+A replay must give what the eager step gives, every time: each graph is replayed several times with eager
+work of the library on the same stream in between, and each replay is compared bit for bit with the eager
+result for the input the buffer holds at that moment (the graph reads its input where the eager call did)."""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+
+import helpers as H
+from devbuf import DevBuf
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+class Hip:
+    """The four runtime calls a capture needs, from the HIP runtime the library itself is linked with."""
+
+    def __init__(self):
+        self.lib = C.CDLL("libamdhip64.so")
+        for name, args in (("hipStreamBeginCapture", [C.c_void_p, C.c_int]), ("hipStreamEndCapture", [C.c_void_p, C.POINTER(C.c_void_p)]),
+                           ("hipGraphInstantiate", [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
+                           ("hipGraphLaunch", [C.c_void_p, C.c_void_p]), ("hipGraphExecDestroy", [C.c_void_p]),
+                           ("hipGraphDestroy", [C.c_void_p]), ("hipStreamSynchronize", [C.c_void_p])):
+            fn = getattr(self.lib, name)
+            fn.argtypes, fn.restype = args, C.c_int
+
+    def ok(self, rc, what):
+        assert rc == 0, f"{what}: hipError {rc}"
+
+    def capture(self, stream, fn):
+        graph, ex = C.c_void_p(), C.c_void_p()
+        self.ok(self.lib.hipStreamBeginCapture(stream, 1), "hipStreamBeginCapture")   # thread-local: a forbidden call fails the capture
+        try:
+            fn()
+        finally:
+            rc = self.lib.hipStreamEndCapture(stream, C.byref(graph))
+        self.ok(rc, "hipStreamEndCapture")
+        self.ok(self.lib.hipGraphInstantiate(C.byref(ex), graph, None, None, 0), "hipGraphInstantiate")
+        return graph, ex
+
+
+@pytest.mark.parametrize("typ,seq", [(2, 1), (8, 1), (2, 4)])
+def test_block_step_replayed_from_a_graph(ctx, orc, typ, seq):
+    from peregrine_amd import _ffi, gguf, llama
+    hip = Hip()
+    d, nqh, nkvh, hd, ffn, pre = 256, 8, 2, 64, 512, 300     # 300 positions: the keys are cut into splits / runs
+    shapes = [(nqh * hd, d), (nkvh * hd, d), (nkvh * hd, d), (d, nqh * hd), (ffn, d), (ffn, d), (d, ffn)]
+    pack = {2: H.pack_q4_0, 8: H.pack_q8_0}[typ]
+    ws = [gguf.GgufWeight(bytes(pack(orc.rng_normal(70 + i, n * k, 0.0, 1.0 / np.sqrt(k)))), typ, n, k, ctx)
+          for i, (n, k) in enumerate(shapes)]
+    blk = llama.LlamaBlock(d, nqh, nkvh, hd, ffn, 512, 10000.0, 1e-5, ctx)
+    blk.set_weights(*ws, (1 + 0.1 * orc.rng_normal(1, d)).astype(np.float32), (1 + 0.1 * orc.rng_normal(2, d)).astype(np.float32))
+    cache = blk.new_cache()
+    blk.forward(orc.rng_normal(3, pre * d).reshape(pre, d), cache)
+    inputs = [orc.rng_normal(10 + i, seq * d) for i in range(4)]
+    h_dev, o_dev = DevBuf(ctx, host=inputs[0]), DevBuf(ctx, seq * d * 4)
+    other_in, other_out = DevBuf(ctx, host=orc.rng_normal(20, 9 * d)), DevBuf(ctx, 9 * d * 4)
+    other_cache = blk.new_cache()
+
+    def step():
+        _ffi.check(_ffi.lib.pg_kv_cache_rollback_to(cache._h, pre))
+        _ffi.check(_ffi.lib.pg_llama_block_forward_dev(ctx.handle, blk._h, h_dev.ptr, seq, cache._h, o_dev.ptr))
+
+    def eager(x):
+        _ffi.check(_ffi.lib.pg_memcpy_h2d(ctx.handle, h_dev.ptr, C.c_void_p(x.ctypes.data), x.nbytes))
+        step()
+        ctx.sync()
+        return o_dev.to_host(np.float32)
+
+    want = [eager(x) for x in inputs]        # (also the warm-up: every buffer the step needs exists now)
+    say(f"capturing a {seq}-token step, type {typ}")
+    graph, ex = hip.capture(ctx.stream, step)
+    try:
+        for i, x in enumerate(inputs):
+            # other work of the library on the stream, and a synchronisation, between the replays
+            _ffi.check(_ffi.lib.pg_kv_cache_rollback_to(other_cache._h, 0))
+            _ffi.check(_ffi.lib.pg_llama_block_forward_dev(ctx.handle, blk._h, other_in.ptr, 9, other_cache._h, other_out.ptr))
+            _ffi.check(_ffi.lib.pg_memcpy_h2d(ctx.handle, h_dev.ptr, C.c_void_p(x.ctypes.data), x.nbytes))
+            _ffi.check(_ffi.lib.pg_memcpy_h2d(ctx.handle, o_dev.ptr, C.c_void_p(np.full(seq * d, np.nan, np.float32).ctypes.data), seq * d * 4))
+            ctx.sync()
+            hip.ok(hip.lib.hipGraphLaunch(ex, ctx.stream), "hipGraphLaunch")
+            ctx.sync()
+            got = o_dev.to_host(np.float32)
+            assert (got.view(np.uint32) == want[i].view(np.uint32)).all(), f"replay {i} differs from the eager step"
+    finally:
+        hip.lib.hipGraphExecDestroy(ex)
+        hip.lib.hipGraphDestroy(graph)
+    for w in ws:
+        w.free()
