@@ -1179,17 +1179,18 @@ __global__ __launch_bounds__(128) void gqa_combine_kernel(const float *__restric
     }
 }
 
-// The same merge for head sizes 64 and 128 and at most 64 splits, every load in flight at once: thread =
-// (float4 of the row, slice of the splits), the slices' sums meet in LDS.  Splits are still added in
+// The same merge for head sizes 64 and 128 and at most MAXS (64 or 128) splits, every load in flight at once:
+// thread = (float4 of the row, slice of the splits), the slices' sums meet in LDS.  Splits are still added in
 // ascending order within a slice and the slices in ascending order: the result does not depend on timing.
-template <int HD, int DIG>
+// A record is HDR floats (maximum, exp-sum, padding) followed by the row.  DIG as in gqa_combine_kernel.
+template <int HD, int DIG, int HDR, int MAXS>
 __global__ __launch_bounds__(256) void gqa_combine_few_kernel(const float *__restrict__ part, int splits, float *__restrict__ out,
                                                               int accumulate, int nqh, int8_t *__restrict__ digits,
                                                               float *__restrict__ xs) {
-    constexpr int UNITS = HD / 4, SLICES = 256 / UNITS, NS = 64 / SLICES;  // 8 slices x 8 splits, or 16 x 4
-    __shared__ float sm[64], sl[64];
+    constexpr int UNITS = HD / 4, SLICES = 256 / UNITS, NS = MAXS / SLICES, REC = HD + HDR;
+    __shared__ float sm[MAXS], sl[MAXS];
     __shared__ float ex[SLICES][UNITS][5];
-    const float *p = part + (size_t)blockIdx.x * splits * (HD + 2);
+    const float *p = part + (size_t)blockIdx.x * splits * REC;
     const int tid = threadIdx.x, i4 = tid % UNITS, slice = tid / UNITS;
     float2 ra[NS], rb[NS];
 #pragma unroll
@@ -1197,17 +1198,19 @@ __global__ __launch_bounds__(256) void gqa_combine_few_kernel(const float *__res
         const int sp = slice * NS + j;
         ra[j] = rb[j] = float2{0.f, 0.f};
         if (sp < splits) {
-            ra[j] = *reinterpret_cast<const float2 *>(p + (size_t)sp * (HD + 2) + 2 + 4 * i4);
-            rb[j] = *reinterpret_cast<const float2 *>(p + (size_t)sp * (HD + 2) + 4 + 4 * i4);
+            ra[j] = *reinterpret_cast<const float2 *>(p + (size_t)sp * REC + HDR + 4 * i4);
+            rb[j] = *reinterpret_cast<const float2 *>(p + (size_t)sp * REC + HDR + 2 + 4 * i4);
         }
     }
-    if (tid < 64) {
-        const float2 ml = tid < splits ? *reinterpret_cast<const float2 *>(p + (size_t)tid * (HD + 2)) : float2{-INFINITY, 0.f};
+    if (tid < MAXS) {
+        const float2 ml = tid < splits ? *reinterpret_cast<const float2 *>(p + (size_t)tid * REC) : float2{-INFINITY, 0.f};
         sm[tid] = ml.x;
         sl[tid] = ml.y;
     }
     __syncthreads();
-    const float M = wave_max_f32(sm[tid & 63]);
+    float mine_m = sm[tid & 63];
+    if constexpr (MAXS > 64) mine_m = fmaxf(mine_m, sm[64 + (tid & 63)]);
+    const float M = wave_max_f32(mine_m);
     const float m_ref = M == -INFINITY ? 0.f : M;
     float L = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -1241,8 +1244,9 @@ __global__ __launch_bounds__(256) void gqa_combine_few_kernel(const float *__res
         *dst = r;
     } else {
         const int qt = blockIdx.x / nqh, qh = blockIdx.x - qt * nqh;
-        const int e4 = qh * UNITS + i4;  // float4 index within the row
-        pg_emit_digits<DIG == 1>(o, qt, e4 >> 3, e4 & 7, nqh * HD / 32, digits, xs);
+        const int e4 = qh * UNITS + i4, nb = nqh * HD / 32;  // float4 index within the row
+        if constexpr (DIG <= 2) pg_emit_digits<DIG == 1>(o, qt, e4 >> 3, e4 & 7, nb, digits, xs);
+        else pg_emit_mm_digits<DIG == 3>(o, qt, e4 >> 3, e4 & 7, nb, (nb + 3) & ~3, digits, xs);
     }
 }
 
@@ -1521,12 +1525,24 @@ pg_status launch_attention(pg_ctx *ctx, const float *q, const pg_kv_cache *kc, c
         PG_TRY(pg_launch(ctx, "gqa_attention_tiled", kern, grid_t, dim3(256), lds_t, aa));
     } else
         PG_TRY(pg_launch(ctx, "gqa_attention", gqa_attention_kernel, grid, dim3(256), (256 + ATT_RED + chunk) * sizeof(float), aa));
-    if (decode_kernel && splits <= 64) {  // (decode_kernel: `out` is 16-byte aligned)
-        const int dg = !xd ? 0 : (digit_kind == PG_GGML_Q4_0 ? 1 : 2);
-        auto *kern = hd == 64 ? (dg == 0 ? gqa_combine_few_kernel<64, 0> : (dg == 1 ? gqa_combine_few_kernel<64, 1> : gqa_combine_few_kernel<64, 2>))
-                              : (dg == 0 ? gqa_combine_few_kernel<128, 0> : (dg == 1 ? gqa_combine_few_kernel<128, 1> : gqa_combine_few_kernel<128, 2>));
-        PG_TRY(pg_launch(ctx, xd ? "gqa_combine_digits" : "gqa_combine", kern, dim3((unsigned)rows), dim3(256), 0, (const float *)aa.part,
-                         (int)splits, out, accumulate, (int)nqh, xd ? xd->digits : (int8_t *)nullptr, xd ? xd->xs : (float *)nullptr));
+    if ((decode_kernel || split_kernel) && splits <= 128) {  // (these kernels: `out` is 16-byte aligned, hd is 64 or 128)
+        // what the merged rows leave as: f32, the streaming product's digits (one-token step), or -- a merge of key
+        // runs under a many-token block step -- the matrix-core product's digit planes
+        const bool planes = md && !xd && !accumulate;
+        const int dg = xd ? (digit_kind == PG_GGML_Q4_0 ? 1 : 2) : (planes ? (digit_kind == PG_GGML_Q4_0 ? 3 : 4) : 0);
+        int8_t *dig = xd ? xd->digits : (planes ? md->digits : nullptr);
+        float *dxs = xd ? xd->xs : (planes ? md->xs : nullptr);
+        const char *name = xd ? "gqa_combine_digits" : (planes ? "gqa_combine_mm_digits" : "gqa_combine");
+#define PG_COMBINE_FEW(HD_, DG_)                                                                                                   \
+    (split_kernel ? (splits <= 64 ? gqa_combine_few_kernel<HD_, DG_, 4, 64> : gqa_combine_few_kernel<HD_, DG_, 4, 128>)              \
+                  : (splits <= 64 ? gqa_combine_few_kernel<HD_, DG_, 2, 64> : gqa_combine_few_kernel<HD_, DG_, 2, 128>))
+#define PG_COMBINE_FEW_HD(DG_) (hd == 64 ? PG_COMBINE_FEW(64, DG_) : PG_COMBINE_FEW(128, DG_))
+        auto *kern = dg == 0 ? PG_COMBINE_FEW_HD(0) : (dg == 1 ? PG_COMBINE_FEW_HD(1) : (dg == 2 ? PG_COMBINE_FEW_HD(2) : (dg == 3 ? PG_COMBINE_FEW_HD(3) : PG_COMBINE_FEW_HD(4))));
+#undef PG_COMBINE_FEW_HD
+#undef PG_COMBINE_FEW
+        PG_TRY(pg_launch(ctx, name, kern, dim3((unsigned)rows), dim3(256), 0, (const float *)aa.part, (int)splits, out, accumulate, (int)nqh,
+                         dig, dxs));
+        if (planes && md_written) *md_written = true;
     } else if ((splits > 1 || decode_kernel) && md && !xd && !accumulate && hd % 32 == 0) {
         auto *kern = digit_kind == PG_GGML_Q4_0 ? gqa_combine_kernel<3> : gqa_combine_kernel<4>;
         PG_TRY(pg_launch(ctx, "gqa_combine_mm_digits", kern, dim3((unsigned)rows), dim3(128), 0, (const float *)aa.part, (int)splits,
