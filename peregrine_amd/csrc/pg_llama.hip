@@ -1374,7 +1374,10 @@ bool split_mfma_tiles(const pg_ctx *ctx, size_t group, size_t seq_q, size_t nkv,
     const size_t n_items = (group * seq_q + 31) / 32, wgs = n_items * nkv;  // one wavefront each
     const size_t kend = mask_kind != 0 && offset + seq_q < len ? offset + seq_q : len;
     const size_t tiles = (kend + 31) / 32;
-    if (wgs * 2 > (size_t)ctx->num_cu || tiles < 8) return false;
+    // few wavefronts: worth it from 8 tiles on; up to three per CU (a chunk of a few hundred tokens appended to a long
+    // cache): only when every wavefront would otherwise walk 64 tiles and more while SIMDs stand idle
+    const bool few = wgs * 2 <= (size_t)ctx->num_cu;
+    if (!(few ? tiles >= 8 : (wgs < 3 * (size_t)ctx->num_cu && tiles >= 64))) return false;
     // A tile costs a wavefront about 5 us whatever the number of live rows (128 matrix instructions of 16 passes,
     // one wavefront per SIMD), so the runs are as short as one wavefront per SIMD allows
     size_t want = (4 * (size_t)ctx->num_cu + wgs - 1) / wgs;

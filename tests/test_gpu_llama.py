@@ -268,6 +268,9 @@ def test_gqa_attention_few_rows_under_a_long_cache(ctx, orc):
     _attention_case(ctx, orc, 8, 2, 64, 5, 900, M.causal_sliding_window(895, 100, 4), None, 407)  # whole runs hidden
     _attention_case(ctx, orc, 8, 2, 128, 12, 600, M.local_global(588, 40, [0, 7, 64, 300, 301, 599, 9999]), None, 408)
     _attention_case(ctx, orc, 4, 4, 128, 3, 5000, M.causal(4997), None, 409)                     # one head per kv head
+    say("attention, a chunk of a prefill appended to a long cache")
+    _attention_case(ctx, orc, 32, 8, 128, 136, 2100, M.causal(1964), None, 411)                  # 17 items per kv head, 66 key tiles
+    _attention_case(ctx, orc, 16, 8, 64, 300, 2300, M.causal_sliding_window(2000, 700, 8), None, 412)
     a = _attention_case(ctx, orc, 16, 2, 128, 9, 3000, M.causal(2991), None, 410)
     assert (a == _attention_case(ctx, orc, 16, 2, 128, 9, 3000, M.causal(2991), None, 410)).all()
 
