@@ -1380,7 +1380,8 @@ bool split_mfma_tiles(const pg_ctx *ctx, size_t group, size_t seq_q, size_t nkv,
     if (!(few ? tiles >= 8 : (wgs < 3 * (size_t)ctx->num_cu && tiles >= 64))) return false;
     // A tile costs a wavefront about 5 us whatever the number of live rows (128 matrix instructions of 16 passes,
     // one wavefront per SIMD), so the runs are as short as one wavefront per SIMD allows
-    size_t want = (4 * (size_t)ctx->num_cu + wgs - 1) / wgs;
+    size_t want = 4 * (size_t)ctx->num_cu / wgs;  // (rounded down: a few wavefronts past one per SIMD would cost a second round)
+    if (want < 2) return false;
     if (want > tiles) want = tiles;
     if (want > (size_t)ATT_SPLITS_MAX) want = ATT_SPLITS_MAX;
     *chunk = (tiles + want - 1) / want;
