@@ -113,9 +113,19 @@ __host__ __device__ static inline size_t pg_mm_row_bytes(size_t nb) {
 
 // Eight consecutive lanes hold block b of activation row `row`, four elements each (as for pg_emit_digits);
 // all eight must call together.
+// With `xsum` (Q4_1: sum_k (q d + m) x = d sum q x + m sum x) the block's plain f32 sum of x is stored too, in
+// xsum[row][nbp] (lanes' partial sums added pairwise, fixed order).
 template <bool NIB>
 __device__ __forceinline__ void pg_emit_mm_digits(const float (&f)[4], size_t row, int b, int sub, int nb, int nbp,
-                                                  int8_t *__restrict__ digits, float *__restrict__ xs) {
+                                                  int8_t *__restrict__ digits, float *__restrict__ xs,
+                                                  float *__restrict__ xsum = nullptr) {
+    if (xsum) {  // the same for all lanes
+        float t = (f[0] + f[1]) + (f[2] + f[3]);
+        t += __builtin_bit_cast(float, pg_dpp8<0xB1>(__builtin_bit_cast(int, t)));
+        t += __builtin_bit_cast(float, pg_dpp8<0x4E>(__builtin_bit_cast(int, t)));
+        t += __builtin_bit_cast(float, pg_dpp8<0x141>(__builtin_bit_cast(int, t)));
+        if (sub == 0) xsum[row * (size_t)nbp + b] = t;
+    }
     float amax = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3])));
     int bad = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]);
     amax = fmaxf(amax, __builtin_bit_cast(float, pg_dpp8<0xB1>(__builtin_bit_cast(int, amax))));

@@ -803,7 +803,7 @@ pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w) {
     // context, stream or thread that finds it set may read it at once.
     std::lock_guard<std::mutex> lock(g_tiled_mutex);
     if (w->qs_tiled) return PG_OK;
-    if (w->ggml_type != PG_GGML_Q4_0 && w->ggml_type != PG_GGML_Q8_0)
+    if (w->ggml_type != PG_GGML_Q4_0 && w->ggml_type != PG_GGML_Q8_0 && w->ggml_type != PG_GGML_Q4_1)
         return pg_fail(PG_EUNSUPPORTED, "gguf: no tile-major copy for ggml type %d", w->ggml_type);
     const int nb = (int)(w->k_in / 32);
     const bool q8 = w->ggml_type == PG_GGML_Q8_0;
@@ -831,10 +831,13 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
                               float *y_dev) {
     void *ws = nullptr;
     if (w->ggml_type == PG_MXFP4) return pg_launch_mxfp4_rows(ctx, x_dev, m, w, y_dev);
-    // Q4_1 has the streaming kernel only; a K of a few blocks needs its finer fixed point
+    // a K of a few blocks needs the streaming kernel's finer fixed point; so do up to seven rows of Q4_1 (its
+    // matrix-core route is three launches more than the streaming one: 27 against 19 us at four rows of 4096 ->
+    // 14336, 35 against 59 at sixteen) and Q4_1 rows too long for the offset kernel
     if (m == 1 && pg_gguf_gemv_takes_f32_row(w->ggml_type, w->n_out, w->k_in, x_dev))
         return pg_launch_gguf_gemv_f32_row(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, x_dev, y_dev);
-    if (m == 1 || w->ggml_type == PG_GGML_Q4_1 || w->k_in / 32 < PG_MM_MIN_BLOCKS) {
+    const bool q41 = w->ggml_type == PG_GGML_Q4_1;
+    if (m == 1 || (q41 && (m < 8 || w->k_in > 32768)) || w->k_in / 32 < PG_MM_MIN_BLOCKS) {
         if (m > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_matmul: more than 65535 rows through the streaming kernel (Q4_1 or k_in < %zu)", PG_MM_MIN_BLOCKS * 32);
         PG_TRY(pg_workspace(ctx, pg_xdigits_bytes(m, w->k_in), &ws));
         const pg_xdigits xd = pg_xdigits_carve(ws, m, w->k_in);
@@ -852,7 +855,9 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
     pg_mm_group grp = {1, nullptr, nullptr, nullptr, nullptr, 0, (int)((m + 31) / 32), (int)m, 1};
     PG_TRY(pg_gguf_ensure_tiled(ctx, w));
     grp.tiled = 1;
-    return pg_launch_gguf_mm(ctx, w->ggml_type, w->n_out, w->k_in, w->qs_tiled, w->d, grp, m, md, y_dev, part);
+    // Q4_1: the Q4_0 product on the same nibbles and scales, then the blocks' offsets times the rows' block sums
+    PG_TRY(pg_launch_gguf_mm(ctx, q41 ? PG_GGML_Q4_0 : w->ggml_type, w->n_out, w->k_in, w->qs_tiled, w->d, grp, m, md, y_dev, part));
+    return q41 ? pg_launch_q41_offset(ctx, w, md, m, y_dev) : PG_OK;
 }
 
 // Several products over the same activation rows (q/k/v, gate/up): the rows are rewritten

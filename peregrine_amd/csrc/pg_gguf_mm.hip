@@ -50,13 +50,71 @@ template <int QT> struct MMCfg {
 // ---- activation rows -> two byte-digit planes (pg_emit_mm_digits, pg_digits.h) ----------
 template <bool NIB>
 __global__ __launch_bounds__(256) void x_to_mm_digits_kernel(const float *__restrict__ x, int nb, int nbp,
-                                                             int8_t *__restrict__ digits, float *__restrict__ xs) {
+                                                             int8_t *__restrict__ digits, float *__restrict__ xs,
+                                                             float *__restrict__ xsum) {
     const size_t row = blockIdx.y;
     const int b = blockIdx.x * 32 + (threadIdx.x >> 3), sub = threadIdx.x & 7;
     if (b >= nb) return;  // whole 8-thread groups leave together
     const float4 v = reinterpret_cast<const float4 *>(x + (row * nb + b) * 32)[sub];
     const float f[4] = {v.x, v.y, v.z, v.w};
-    pg_emit_mm_digits<NIB>(f, row, b, sub, nb, nbp, digits, xs);
+    pg_emit_mm_digits<NIB>(f, row, b, sub, nb, nbp, digits, xs, xsum);
+}
+
+// Q4_1's second term on many rows: y[t][n] += sum_b (8 d[n][b] + m[n][b]) * xsum[t][b] (the first, d sum (q - 8) x,
+// is the Q4_0 product on the same nibbles).  Workgroup = 256 / NQ weight rows x 16 tokens; thread = (row, one of NQ
+// runs of blocks), 16 tokens in registers; the tokens' block sums wait in LDS as [b][16]; the runs are added in
+// ascending order.  NQ = 4 for few tokens (more workgroups, shorter loops), 1 for many (the block sums staged once
+// per 256 rows).
+constexpr int Q41_TT = 16;
+template <int NQ>
+__global__ __launch_bounds__(256) void q41_offset_kernel(const uint16_t *__restrict__ d, const uint16_t *__restrict__ m, int n_out,
+                                                         int nb, const float *__restrict__ xsum, int nbp, int rows,
+                                                         float *__restrict__ y) {
+    constexpr int RPW = 256 / NQ;
+    extern __shared__ __attribute__((aligned(16))) float s_tile[];  // [nb][Q41_TT], then [NQ - 1][RPW][Q41_TT] partial sums
+    const int t0 = blockIdx.y * Q41_TT, lrow = threadIdx.x % RPW, quarter = threadIdx.x / RPW;
+    const int n = blockIdx.x * RPW + lrow;
+    for (int i = threadIdx.x; i < nb * Q41_TT; i += 256) {
+        const int t = i / nb, b = i - t * nb;  // (consecutive threads: consecutive blocks of one token)
+        s_tile[b * Q41_TT + t] = t0 + t < rows ? xsum[(size_t)(t0 + t) * nbp + b] : 0.0f;
+    }
+    __syncthreads();
+    float acc[Q41_TT];
+#pragma unroll
+    for (int t = 0; t < Q41_TT; ++t) acc[t] = 0.0f;
+    const int nc = n < n_out ? n : n_out - 1;
+    const size_t tile = (size_t)(nc >> 3) * nb * 8 + (nc & 7);
+    const int per = (nb + NQ - 1) / NQ, b_lo = quarter * per, b_hi = b_lo + per < nb ? b_lo + per : nb;
+    for (int b = b_lo; b < b_hi; ++b) {
+        _Float16 dh, mh;
+        const uint16_t db = d[tile + (size_t)b * 8], mb = m[tile + (size_t)b * 8];
+        __builtin_memcpy(&dh, &db, 2);
+        __builtin_memcpy(&mh, &mb, 2);
+        const float c = fmaf(8.0f, (float)dh, (float)mh);
+#pragma unroll
+        for (int t4 = 0; t4 < Q41_TT / 4; ++t4) {
+            const float4 sv = *reinterpret_cast<const float4 *>(s_tile + b * Q41_TT + 4 * t4);
+            acc[4 * t4] = fmaf(c, sv.x, acc[4 * t4]); acc[4 * t4 + 1] = fmaf(c, sv.y, acc[4 * t4 + 1]);
+            acc[4 * t4 + 2] = fmaf(c, sv.z, acc[4 * t4 + 2]); acc[4 * t4 + 3] = fmaf(c, sv.w, acc[4 * t4 + 3]);
+        }
+    }
+    if constexpr (NQ > 1) {
+        float *part = s_tile + nb * Q41_TT;
+        if (quarter > 0) {
+#pragma unroll
+            for (int t = 0; t < Q41_TT; ++t) part[((quarter - 1) * RPW + lrow) * Q41_TT + t] = acc[t];
+        }
+        __syncthreads();
+        if (quarter > 0) return;
+#pragma unroll
+        for (int qv = 0; qv < NQ - 1; ++qv)
+#pragma unroll
+            for (int t = 0; t < Q41_TT; ++t) acc[t] += part[(qv * RPW + lrow) * Q41_TT + t];
+    }
+    if (n >= n_out) return;
+#pragma unroll
+    for (int t = 0; t < Q41_TT; ++t)
+        if (t0 + t < rows) y[(size_t)(t0 + t) * n_out + n] += acc[t];
 }
 
 // Two's-complement nibbles (as stored at upload) of one dword -> four signed bytes holding
@@ -470,7 +528,7 @@ __global__ void sum_parts_kernel(const float *__restrict__ part, size_t n, int k
 
 size_t pg_mmdigits_bytes(size_t rows, size_t k) {
     const size_t nb = k / 32, nbp = pg_round_up(nb, 4);
-    return rows * pg_mm_row_bytes(nb) + pg_round_up(rows * nbp * sizeof(float), 256);
+    return rows * pg_mm_row_bytes(nb) + 2 * pg_round_up(rows * nbp * sizeof(float), 256);
 }
 
 pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k) {
@@ -480,6 +538,8 @@ pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k) {
     md.digits = reinterpret_cast<int8_t *>(p);
     p += rows * pg_mm_row_bytes(nb);
     md.xs = reinterpret_cast<float *>(p);
+    p += pg_round_up(rows * pg_round_up(nb, 4) * sizeof(float), 256);
+    md.xsum = reinterpret_cast<float *>(p);
     md.rows = rows;
     md.k = k;
     return md;
@@ -491,9 +551,26 @@ pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows,
     if (rows > 65535) return pg_fail(PG_EUNSUPPORTED, "x_to_mm_digits: more than 65535 activation rows");
     const int nb = (int)(k / 32), nbp = (int)pg_round_up(nb, 4);
     const dim3 grid(grid_for(nb, 32), (unsigned)rows);
-    if (ggml_type == PG_GGML_Q4_0)
-        return pg_launch(ctx, "x_to_mm_digits", x_to_mm_digits_kernel<true>, grid, dim3(256), 0, x_dev, nb, nbp, md.digits, md.xs);
-    return pg_launch(ctx, "x_to_mm_digits", x_to_mm_digits_kernel<false>, grid, dim3(256), 0, x_dev, nb, nbp, md.digits, md.xs);
+    if (ggml_type == PG_GGML_Q4_0 || ggml_type == PG_GGML_Q4_1)
+        return pg_launch(ctx, "x_to_mm_digits", x_to_mm_digits_kernel<true>, grid, dim3(256), 0, x_dev, nb, nbp, md.digits, md.xs,
+                         ggml_type == PG_GGML_Q4_1 ? md.xsum : (float *)nullptr);
+    return pg_launch(ctx, "x_to_mm_digits", x_to_mm_digits_kernel<false>, grid, dim3(256), 0, x_dev, nb, nbp, md.digits, md.xs,
+                     (float *)nullptr);
+}
+
+pg_status pg_launch_q41_offset(pg_ctx *ctx, const pg_gguf_tensor *w, const pg_mmdigits &md, size_t rows, float *y) {
+    const int nb = (int)(w->k_in / 32), nbp = (int)pg_round_up(nb, 4);
+    const bool few = rows <= 64;
+    const size_t lds = ((size_t)nb + (few ? 3 * 64 : 0)) * Q41_TT * sizeof(float);
+    if (lds > 128 * 1024) return pg_fail(PG_EUNSUPPORTED, "gguf_matmul: Q4_1 rows of %zu on the matrix-core route", w->k_in);
+    PG_TRY(pg_allow_dynamic_lds(ctx, few ? (const void *)q41_offset_kernel<4> : (const void *)q41_offset_kernel<1>, 128 * 1024));
+    if ((rows + Q41_TT - 1) / Q41_TT > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_matmul: too many activation rows");
+    const dim3 grid(grid_for(w->n_out, few ? 64 : 256), (unsigned)((rows + Q41_TT - 1) / Q41_TT));
+    if (few)
+        return pg_launch(ctx, "gguf_q4_1_offsets", q41_offset_kernel<4>, grid, dim3(256), lds, (const uint16_t *)w->d,
+                         (const uint16_t *)w->m, (int)w->n_out, nb, (const float *)md.xsum, nbp, (int)rows, y);
+    return pg_launch(ctx, "gguf_q4_1_offsets", q41_offset_kernel<1>, grid, dim3(256), lds, (const uint16_t *)w->d,
+                     (const uint16_t *)w->m, (int)w->n_out, nb, (const float *)md.xsum, nbp, (int)rows, y);
 }
 
 // Digits of `act_rows` activation rows that no XCD's L2 (4 MiB) can keep while every workgroup

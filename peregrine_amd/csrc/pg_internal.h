@@ -280,12 +280,17 @@ pg_status pg_launch_gguf_gemv_f32_row(pg_ctx *ctx, int ggml_type, size_t n_out, 
 struct pg_mmdigits {
     int8_t *digits;  // [rows][2 planes][k/32 blocks][2 halves][16 bytes], rows padded to an odd number of 256-byte lines
     float *xs;       // [rows][k/32 rounded up to 4] block scales
+    float *xsum;     // [rows][k/32 rounded up to 4] plain block sums of x (written for Q4_1 products only)
     size_t rows, k;
 };
 size_t pg_mmdigits_bytes(size_t rows, size_t k);
 pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k);
 pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows, size_t k, int ggml_type,
                                    const pg_mmdigits &md);
+// Q4_1 on the matrix-core route: the product is the Q4_0 product on the same nibbles and scales plus
+// y[t][n] += sum_b (8 d + m)[n][b] * (sum of x over block b of row t); this adds the second term (md.xsum
+// as pg_launch_x_to_mm_digits leaves it for PG_GGML_Q4_1).  k_in up to 32768.
+pg_status pg_launch_q41_offset(pg_ctx *ctx, const pg_gguf_tensor *w, const pg_mmdigits &md, size_t rows, float *y);
 // Which activation rows multiply which weights.  Without `counts`: one weight tensor and pairs
 // 0 .. max_count-1.  With `counts`: expert e owns counts[e] pairs, listed (in ascending order) in
 // lists[e * list_stride ..]; its weights are qs_table[e] / d_table[e].  Pair p reads activation

@@ -100,6 +100,8 @@ GGUF_SHAPES = [
     (2, 130, 224, 33), (8, 131, 160, 40), (2, 515, 4096, 64), (8, 257, 6144, 35), (2, 14336, 4096, 4), (8, 4096, 14336, 16),
     # Q4_1 (offset blocks): the streaming kernel with the block-sum term, one item per row
     (3, 256, 4096, 1), (3, 77, 96, 3), (3, 1000, 2048, 2), (3, 50, 11008, 1), (3, 64, 32768, 2), (3, 14336, 4096, 1), (3, 130, 224, 33),
+    # Q4_1 from four rows on: the Q4_0 matrix-core product on the same nibbles plus the offsets times the rows' block sums
+    (3, 256, 4096, 8), (3, 515, 4096, 64), (3, 14336, 4096, 16), (3, 600, 256, 545), (3, 100, 32768, 9), (3, 40, 32800, 8), (3, 256, 4096, 7),
     # 16 token tiles and more: no split K, XCD-aware super-tiles of 4 row groups x 8 token tiles (ragged on both sides)
     (2, 600, 256, 545), (8, 1100, 128, 700), (2, 128, 512, 512),
 ]
@@ -121,7 +123,8 @@ def test_gguf_matmul_vs_oracle(ctx, orc, typ, n_out, k_in, m):
     for r in range(m):
         sl = slice(r * n_out, (r + 1) * n_out)
         H.assert_close_rel(got[sl], want[sl], RTOL_CONTRACT, f"row {r} (contract)")
-        H.assert_close_rel(got[sl], want[sl], RTOL_ACHIEVED[typ] if (m == 1 or typ == 3) else RTOL_ACHIEVED_MM, f"row {r} (achieved)")
+        streaming = m == 1 or (typ == 3 and (m < 8 or k_in > 32768)) or k_in < 160
+        H.assert_close_rel(got[sl], want[sl], RTOL_ACHIEVED[typ] if streaming else RTOL_ACHIEVED_MM, f"row {r} (achieved)")
     gw.free()
 
 

@@ -390,8 +390,10 @@ def test_llama_block_one_token_steps_at_llama_8b_size(ctx, orc):
 
 
 def test_llama_block_q4_1_weights(ctx, orc):
-    """Offset blocks (Q4_1) run on the streaming kernel only, one item per row."""
+    """Offset blocks (Q4_1): the streaming kernel, one item per row, up to seven rows; more rows take the Q4_0
+    matrix-core product on the same nibbles plus a launch that adds the offsets times the rows' block sums."""
     _block_case(ctx, orc, 128, 4, 2, 32, 256, 3, (3, 1), seed=13)
+    _block_case(ctx, orc, 256, 4, 2, 32, 512, 3, (40, 1, 9), seed=14)   # from eight rows: the matrix-core product plus the offsets' launch
 
 
 def test_llama_block_mha_and_odd_shapes(ctx, orc):
