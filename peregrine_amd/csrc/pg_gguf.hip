@@ -830,7 +830,17 @@ pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w) {
 pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
                               float *y_dev) {
     void *ws = nullptr;
-    if (w->ggml_type == PG_MXFP4) return pg_launch_mxfp4_rows(ctx, x_dev, m, w, y_dev);
+    if (w->ggml_type == PG_MXFP4) {
+        // The MXFP4 kernel is a decode kernel (three rows per pass over the weights).  From 16 rows on (24 for a
+        // tensor under 2^25 weights, where the passes are short) the tensor's Q8_0 twin takes the matrix-core block
+        // product, which reads the weights once per 32 rows and tile.
+        if (m >= (w->n_out * w->k_in >= ((size_t)1 << 25) ? 16u : 24u) && w->k_in / 32 >= PG_MM_MIN_BLOCKS) {
+            const pg_gguf_tensor *twin = nullptr;
+            PG_TRY(pg_mxfp4_q8_twin(ctx, w, &twin));
+            if (twin) return pg_gguf_matmul_rows(ctx, x_dev, m, twin, y_dev);
+        }
+        return pg_launch_mxfp4_rows(ctx, x_dev, m, w, y_dev);
+    }
     // a K of a few blocks needs the streaming kernel's finer fixed point; so do up to seven rows of Q4_1 (its
     // matrix-core route is three launches more than the streaming one: 27 against 19 us at four rows of 4096 ->
     // 14336, 35 against 59 at sixteen) and Q4_1 rows too long for the offset kernel
@@ -1029,6 +1039,7 @@ PG_API void pg_gguf_free(pg_ctx *ctx, pg_gguf_tensor *t) {
     if (t->d) (void)hipFree(t->d);
     if (t->m) (void)hipFree(t->m);
     if (t->qs_tiled) (void)hipFree(t->qs_tiled);
+    if (t->twin) pg_gguf_free(nullptr, t->twin);  // (the stream was drained above)
     delete t;
 }
 

@@ -74,6 +74,11 @@ struct pg_gguf_tensor {
     mutable uint8_t *qs_tiled;
     int ggml_type;
     size_t n_out, k_in;
+    // MXFP4 only: the same tensor as Q8_0 blocks (i8 = twice the FP4 value, f16 scale 2^(e - 128): exact), made on
+    // the tensor's first product over many rows for the matrix-core block product; twin_state 0 = not tried,
+    // 1 = made, -1 = a block scale is not an f16 (the tensor keeps to its own kernel).
+    mutable pg_gguf_tensor *twin;
+    mutable int twin_state;
 };
 
 // The matrix-core block product carries 16-bit fixed-point activations per block: fine when a
@@ -290,6 +295,7 @@ pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows,
 // Q4_1 on the matrix-core route: the product is the Q4_0 product on the same nibbles and scales plus
 // y[t][n] += sum_b (8 d + m)[n][b] * (sum of x over block b of row t); this adds the second term (md.xsum
 // as pg_launch_x_to_mm_digits leaves it for PG_GGML_Q4_1).  k_in up to 32768.
+pg_status pg_mxfp4_q8_twin(pg_ctx *ctx, const pg_gguf_tensor *w, const pg_gguf_tensor **twin);  // *twin null: not representable
 pg_status pg_launch_q41_offset(pg_ctx *ctx, const pg_gguf_tensor *w, const pg_mmdigits &md, size_t rows, float *y);
 // Which activation rows multiply which weights.  Without `counts`: one weight tensor and pairs
 // 0 .. max_count-1.  With `counts`: expert e owns counts[e] pairs, listed (in ascending order) in

@@ -17,6 +17,8 @@
 // j of a row is one column of B with block scale byte 127 + se + 5 j, so the instruction itself applies
 // both block scales and sums over K; the five columns of a row are added at the end.  Three activation
 // rows (15 columns) share one pass over the weights.
+#include <mutex>
+
 #include "pg_internal.h"
 #include "pg_digits.h"
 
@@ -301,6 +303,87 @@ pg_status pg_launch_mxfp4_rows(pg_ctx *ctx, const float *x_dev, size_t m, const 
 // ---- ABI --------------------------------------------------------------------------------
 // A block is 16 bytes of FP4 (E2M1) codes, byte k = elements 2k (low nibble) and 2k+1, plus
 // one E8M0 scale byte: value = LUT[code] * 2^(scale - 127)   (examples/gpt_oss/moe.rs:5-53).
+// ---- the tensor as Q8_0 blocks (for products over many rows) ---------------------------------
+// Twice an FP4 (E2M1) value is an integer: 0, 1, 2, 3, 4, 6, 8, 12; with the block scale 2^(e - 128) as an f16 the
+// block is a Q8_0 block holding exactly the same numbers.  Planes as split_blocks_kernel lays Q8_0 out:
+// qs8[((n * 2 + h) * nb + b) * 16 + j] = element 16 h + j, d8 in tiles of 8 rows.  *bad is set when a scale has no
+// f16 (e above 143 or, for a block with nonzero codes, below 104).
+__global__ void mxfp4_to_q8_kernel(const uint4 *__restrict__ qs_frag, const uint8_t *__restrict__ sc_frag, int n_out, int nb, int ncp,
+                                   uint8_t *__restrict__ qs8, uint16_t *__restrict__ d8, int *__restrict__ bad) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t n_pad = ((size_t)n_out + 7) / 8 * 8;
+    if (i >= n_pad * nb) return;
+    const size_t n = i / nb, b = i - n * nb;
+    uint16_t *dd = d8 + ((n / 8) * nb + b) * 8 + (n % 8);
+    if (n >= (size_t)n_out) {
+        *dd = 0;
+        return;
+    }
+    const size_t rg = n / 16, c = b / 4;
+    const int lane = (int)(n % 16) + 16 * (int)(b % 4);
+    const uint4 v = qs_frag[(rg * ncp + c) * 64 + lane];
+    const int e = sc_frag[((rg * (ncp / 4) + c / 4) * 64 + lane) * 4 + (c & 3)];
+    const unsigned wv[4] = {v.x, v.y, v.z, v.w};
+    const bool zero = (v.x | v.y | v.z | v.w) == 0u;  // (an all-zero block, or one whose scale byte was 0)
+    const int ex = e - 128;
+    uint16_t bits = 0;
+    if (ex >= -14 && ex <= 15) bits = (uint16_t)((ex + 15) << 10);
+    else if (ex >= -24 && ex < -14) bits = (uint16_t)(1u << (ex + 24));  // subnormal f16: still a power of two
+    else if (!zero || ex > 15) atomicOr(bad, 1);  // (a huge scale times zero codes is not zero where the scale is inf / NaN)
+    *dd = bits;
+#pragma unroll
+    for (int el = 0; el < 32; ++el) {
+        const unsigned code = (wv[el >> 3] >> (4 * (el & 7))) & 15u;   // element el in nibble el
+        const int mag = (int)((0x0C08060403020100ull >> (8 * (code & 7u))) & 255u);  // 2 x {0, .5, 1, 1.5, 2, 3, 4, 6}
+        qs8[((n * 2 + (el >> 4)) * nb + b) * 16 + (el & 15)] = (uint8_t)(int8_t)((code & 8u) ? -mag : mag);
+    }
+}
+
+static std::mutex g_twin_mutex;
+
+pg_status pg_mxfp4_q8_twin(pg_ctx *ctx, const pg_gguf_tensor *w, const pg_gguf_tensor **twin) {
+    // One maker at a time; the pointer is published once the planes are complete.
+    std::lock_guard<std::mutex> lock(g_twin_mutex);
+    *twin = nullptr;
+    if (w->twin_state != 0) {
+        *twin = w->twin_state > 0 ? w->twin : nullptr;
+        return PG_OK;
+    }
+    const size_t nb = w->k_in / 32, ncp = mx_chunks(nb), n_pad = (w->n_out + 7) / 8 * 8;
+    pg_gguf_tensor *t = new (std::nothrow) pg_gguf_tensor();
+    if (!t) return pg_fail(PG_ENOMEM, "host allocation failed");
+    t->ggml_type = PG_GGML_Q8_0;
+    t->n_out = w->n_out;
+    t->k_in = w->k_in;
+    int *bad_dev = nullptr, bad = 0;
+    hipError_t e = hipMalloc((void **)&t->qs, w->n_out * nb * 32);
+    if (e == hipSuccess) e = hipMalloc((void **)&t->d, n_pad * nb * sizeof(uint16_t));
+    if (e == hipSuccess) e = hipMalloc((void **)&bad_dev, sizeof(int));
+    if (e == hipSuccess) e = hipMemsetAsync(bad_dev, 0, sizeof(int), ctx->stream);  // (set-up, once per tensor: not a capturable path)
+    if (e == hipSuccess) {
+        mxfp4_to_q8_kernel<<<grid_for(n_pad * nb, 256), 256, 0, ctx->stream>>>(reinterpret_cast<const uint4 *>(w->qs),
+                                                                               reinterpret_cast<const uint8_t *>(w->d), (int)w->n_out,
+                                                                               (int)nb, (int)ncp, t->qs, t->d, bad_dev);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(&bad, bad_dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (bad_dev) (void)hipFree(bad_dev);
+    if (e != hipSuccess) {
+        pg_gguf_free(nullptr, t);
+        return pg_fail(e == hipErrorOutOfMemory ? PG_ENOMEM : PG_EDEVICE, "mxfp4 Q8_0 twin: %s", hipGetErrorString(e));
+    }
+    if (bad) {
+        pg_gguf_free(nullptr, t);
+        w->twin_state = -1;
+        return PG_OK;
+    }
+    w->twin = t;
+    w->twin_state = 1;
+    *twin = t;
+    return PG_OK;
+}
+
 PG_API pg_status pg_mxfp4_upload(pg_ctx *ctx, const uint8_t *blocks, const uint8_t *scales, size_t out_dim,
                                  size_t in_dim, pg_gguf_tensor **out) {
     PG_TRY(pg_use(ctx));
