@@ -511,6 +511,132 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
     }
 }
 
+// Two to four activation rows in f32 over one Q4_0 tensor, in ONE launch and one pass over the weights
+// (src/tensor.rs:1342-1353 on dequantised weights, M of 2 to 4): the workgroup -- NW wavefronts with RW weight rows
+// each -- rewrites all the rows as digits into LDS (per row the planes, then the block scales) while
+// its first weight rows are in flight (row a at a * nb * 100 bytes rounded up to 16); a weight row then meets every activation row from registers, the digits
+// of one activation row at a time coming back from LDS (10 reads of 16 bytes per row and BPL blocks against
+// 20 R BPL dot instructions).  The matrix-core route for these counts is three launches (digits, product over four
+// K chunks, their sum): 17 to 20 us on 4096 -> 14336 where the weights stream in 8.  Same digits, same integer
+// dots and the same order of sums as the one-row kernel: a row's result equals that kernel's bit for bit.
+template <int BPL, int RW, int R, int NW, int AR>
+__global__ __launch_bounds__(64 * NW) void gguf_gemv_fewrows_kernel(const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0,
+                                                                     int n_out, int nb, const float *__restrict__ x_f32,
+                                                                     float *__restrict__ y) {
+    constexpr int SEG = 64 * BPL, NG = RW / R, MAXA = AR, ar = AR;
+    extern __shared__ __attribute__((aligned(16))) char lds_digits[];
+    const gv4i_ptr qs = (gv4i_ptr)(uintptr_t)qs0;
+    const gv4i_ptr dsc = (gv4i_ptr)(uintptr_t)d0;
+    const int lane = threadIdx.x & 63;
+    const int row0 = (blockIdx.x * NW + (threadIdx.x >> 6)) * RW;
+    const bool live = row0 < n_out;
+    const size_t row_bytes = ((size_t)nb * 100 + 15) & ~(size_t)15;
+    float acc[MAXA][RW];
+#pragma unroll
+    for (int a = 0; a < MAXA; ++a)
+#pragma unroll
+        for (int r = 0; r < RW; ++r) acc[a][r] = 0.0f;
+
+    for (int seg0 = 0; seg0 < nb; seg0 += SEG) {
+        const int seg_n = (nb - seg0 < SEG) ? nb - seg0 : SEG;
+        int blk[BPL];  // this lane's blocks; lanes past the segment end re-read block seg0 with a zero scale
+#pragma unroll
+        for (int p = 0; p < BPL; ++p) blk[p] = seg0 + (lane + 64 * p < seg_n ? lane + 64 * p : 0);
+        auto load_rows = [&](RowLoads<4, BPL, R> &L, int g) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                int row = row0 + g * R + r;
+                row = row < n_out ? row : n_out - 1;  // clamped; masked at the store
+#pragma unroll
+                for (int p = 0; p < BPL; ++p) L.w[r][p][0] = __builtin_nontemporal_load(qs + (size_t)row * nb + blk[p]);
+            }
+        };
+        v4i dtile[BPL];
+        RowLoads<4, BPL, R> L[2];
+        if (seg0 == 0) {
+            // Loads return in issue order: the first activation blocks (from L2) are requested first, the weight
+            // rows (from HBM) right behind them, so that the digit arithmetic runs while the weights fly.
+            const int sub = threadIdx.x & 7, bfirst = (int)threadIdx.x >> 3, total = ar * nb;  // (row, block) pairs, row-major
+            float4 xv[4];
+            auto fetch = [&](int i0) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int i = i0 + u * 8 * NW;
+                    xv[u] = reinterpret_cast<const float4 *>(x_f32)[(size_t)(i < total ? i : 0) * 8 + sub];
+                }
+            };
+            fetch(bfirst);
+            if (live) {
+#pragma unroll
+                for (int p = 0; p < BPL; ++p) dtile[p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+                load_rows(L[0], 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            for (int i0 = bfirst; i0 < total; i0 += 32 * NW) {
+                if (i0 != bfirst) fetch(i0);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int i = i0 + u * 8 * NW;
+                    if (i < total) {  // whole 8-thread groups together
+                        const int a = i / nb, b = i - a * nb;
+                        const float f[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+                        // block-major in LDS: a block's five planes side by side (80 bytes), its scale at float 5 b behind
+                        // them -- the plane-major writer with one block per plane and block index 5 b
+                        int8_t *base = reinterpret_cast<int8_t *>(lds_digits + a * row_bytes);
+                        pg_emit_digits<true>(f, 0, 5 * b, sub, 1, base, reinterpret_cast<float *>(base + (size_t)nb * 80));
+                    }
+                }
+            }
+            // (not __syncthreads(): that would also wait for every weight load in flight)
+            asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier" ::: "memory");
+            if (!live) return;  // after the workgroup's only barrier
+        } else {
+#pragma unroll
+            for (int p = 0; p < BPL; ++p) dtile[p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+            load_rows(L[0], 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            if (g + 1 < NG) {
+                load_rows(L[(g + 1) & 1], g + 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            const RowLoads<4, BPL, R> &C = L[g & 1];
+#pragma unroll
+            for (int a = 0; a < MAXA; ++a) {
+                {
+                    __builtin_amdgcn_sched_barrier(0);  // (one activation row's reads at a time: registers)
+                    const char *base = lds_digits + a * row_bytes;
+#pragma unroll
+                    for (int p = 0; p < BPL; ++p) {  // (one block's digits at a time: 20 registers, not 20 BPL)
+                        v4i xd[5];
+#pragma unroll
+                        for (int j = 0; j < 5; ++j) xd[j] = *reinterpret_cast<const v4i *>(base + blk[p] * 80 + j * 16);
+                        const float sb = reinterpret_cast<const float *>(base + nb * 80)[5 * blk[p]] * (lane + 64 * p < seg_n ? 1.0f : 0.0f);
+#pragma unroll
+                        for (int r = 0; r < R; ++r) {
+                            const int tr = (row0 & 7) + g * R + r;  // row within the scale tile
+                            const float f = (float)block_dot_q4(C.w[r][p][0], xd);
+                            const uint32_t pair = (uint32_t)dtile[p][tr >> 1];
+                            const float dv = half_bits_to_float((uint16_t)((tr & 1) ? pair >> 16 : pair & 0xFFFFu));
+                            acc[a][g * R + r] = fmaf(dv * sb, f, acc[a][g * R + r]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < MAXA; ++a) {
+#pragma unroll
+            for (int r = 0; r < RW; ++r) {
+                const float v = wave_sum_f32(acc[a][r]);
+                if (lane == 0 && row0 + r < n_out) y[(size_t)a * n_out + row0 + r] = v;
+            }
+        }
+}
+
 template <int QT, int BPL, bool Q41>
 pg_status launch_gemv_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
                           const pg_gemv_batch &batch, const pg_xdigits &xd, float *y, const float *residual,
@@ -658,6 +784,35 @@ pg_status launch_gemv_f32x(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t
     }
 }
 
+// Bytes of LDS the few-rows kernel needs; its launch shapes follow the one-row form's.
+inline size_t fewrows_lds(size_t m, size_t k_in) { return m * pg_round_up((k_in / 32) * 100, 16); }
+
+template <int BPL, int AR>
+pg_status launch_gemv_fewrows_bpl(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const float *x_f32,
+                                  float *y) {
+    constexpr size_t m = AR;
+    constexpr int NW = 8, R8 = BPL <= 1 ? 8 : 4;  // rows in flight: bounded by registers
+    const int nb = (int)(k_in / 32);
+    const size_t lds = fewrows_lds(m, k_in), want = (size_t)ctx->num_cu * 6;
+#define PG_GGUF_FEWROWS_LAUNCH(RWW, RR)                                                                                          \
+    do {                                                                                                                         \
+        auto kern = gguf_gemv_fewrows_kernel<BPL, RWW, RR, NW, AR>;                                                              \
+        PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                              \
+        PG_TRY(pg_launch(ctx, "gguf_gemv_q4_0_few_rows", kern, dim3(grid_for(n_out, RWW * NW)), dim3(64 * NW), lds, qs, d,     \
+                         (int)n_out, nb, x_f32, y));                                                                             \
+    } while (0)
+    if constexpr (BPL <= 2) {
+        if (n_out / 8 >= want) {
+            PG_GGUF_FEWROWS_LAUNCH(8, R8);
+            return PG_OK;
+        }
+    }
+    if (n_out / 4 >= want) PG_GGUF_FEWROWS_LAUNCH(4, 4);
+    else PG_GGUF_FEWROWS_LAUNCH(2, 2);
+#undef PG_GGUF_FEWROWS_LAUNCH
+    return PG_OK;
+}
+
 template <int QT, bool Q41 = false>
 pg_status launch_gemv(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d,
                       const pg_gemv_batch &batch, const pg_xdigits &xd, float *y, const float *residual,
@@ -767,6 +922,31 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
 // 8192 weight rows (measured one launch against two: 4096 -> 4096 5.5 against 6.7 us, 14336 -> 4096 11.5
 // against 12.8 us; but 4096 -> 14336 10.9 against 10.3 us, and Q8_0 there 19.3 against 14.6 us).
 // k_in up to 32768 (the row's digits live in LDS).
+// Two rows at once, three or four over a small tensor (Q4_0; all their digits fit in LDS).  The kernel's time grows
+// by the arithmetic of every further row, the matrix-core route's hardly at all, but that one is three launches:
+// 4096 -> 14336 in us, rows 2 / 3 / 4: 12.2 / 16.2 / 19.9 against 17.5 / 17.5 / 17.7; 4096 -> 4096: 6.7 / 8.6 / 10.4
+// against 13.4; 14336 -> 4096: 17.8 / 24.1 against 21.4.
+bool pg_gguf_gemv_takes_few_rows(int ggml_type, size_t m, size_t n_out, size_t k_in, const float *x_f32) {
+    return ggml_type == PG_GGML_Q4_0 && (m == 2 || ((m == 3 || m == 4) && n_out * k_in <= ((size_t)1 << 25))) && k_in >= 32 &&
+           fewrows_lds(m, k_in) <= 150 * 1024 && (uintptr_t)x_f32 % 16 == 0;
+}
+
+pg_status pg_launch_gguf_gemv_few_rows(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const float *x_f32,
+                                       size_t m, float *y) {
+#define PG_FEWROWS_BPL(B)                                                                   \
+    (m == 2 ? launch_gemv_fewrows_bpl<B, 2>(ctx, n_out, k_in, qs, d, x_f32, y)                  \
+            : m == 3 ? launch_gemv_fewrows_bpl<B, 3>(ctx, n_out, k_in, qs, d, x_f32, y)         \
+                     : launch_gemv_fewrows_bpl<B, 4>(ctx, n_out, k_in, qs, d, x_f32, y))
+    if (m < 2 || m > 4) return pg_fail(PG_EINVAL, "gguf_gemv (few rows): %zu rows", m);
+    switch ((k_in / 32 + 63) / 64) {
+        case 1: return PG_FEWROWS_BPL(1);
+        case 2: return PG_FEWROWS_BPL(2);
+        case 3: return PG_FEWROWS_BPL(3);
+        default: return PG_FEWROWS_BPL(4);
+    }
+#undef PG_FEWROWS_BPL
+}
+
 bool pg_gguf_gemv_takes_f32_row(int ggml_type, size_t n_out, size_t k_in, const float *x_f32) {
     return ggml_type == PG_GGML_Q4_0 && n_out <= 8192 && k_in >= 32 && k_in <= 32768 && (uintptr_t)x_f32 % 16 == 0;
 }
@@ -846,6 +1026,8 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
     // 14336, 35 against 59 at sixteen) and Q4_1 rows too long for the offset kernel
     if (m == 1 && pg_gguf_gemv_takes_f32_row(w->ggml_type, w->n_out, w->k_in, x_dev))
         return pg_launch_gguf_gemv_f32_row(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, x_dev, y_dev);
+    if (pg_gguf_gemv_takes_few_rows(w->ggml_type, m, w->n_out, w->k_in, x_dev))
+        return pg_launch_gguf_gemv_few_rows(ctx, w->n_out, w->k_in, w->qs, w->d, x_dev, m, y_dev);
     const bool q41 = w->ggml_type == PG_GGML_Q4_1;
     if (m == 1 || (q41 && (m < 8 || w->k_in > 32768)) || w->k_in / 32 < PG_MM_MIN_BLOCKS) {
         if (m > 65535) return pg_fail(PG_EUNSUPPORTED, "gguf_matmul: more than 65535 rows through the streaming kernel (Q4_1 or k_in < %zu)", PG_MM_MIN_BLOCKS * 32);

@@ -281,6 +281,9 @@ pg_status pg_launch_gguf_gemv_swiglu_digits(pg_ctx *ctx, int ggml_type, size_t n
 bool pg_gguf_gemv_takes_f32_row(int ggml_type, size_t n_out, size_t k_in, const float *x_f32);
 pg_status pg_launch_gguf_gemv_f32_row(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,
                                       const uint16_t *d, const float *x_f32, float *y);
+bool pg_gguf_gemv_takes_few_rows(int ggml_type, size_t m, size_t n_out, size_t k_in, const float *x_f32);
+pg_status pg_launch_gguf_gemv_few_rows(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const float *x_f32,
+                                       size_t m, float *y);
 // Activation rows as two byte-digit planes for the matrix-core product (see pg_gguf_mm.hip).
 struct pg_mmdigits {
     int8_t *digits;  // [rows][2 planes][k/32 blocks][2 halves][16 bytes], rows padded to an odd number of 256-byte lines
