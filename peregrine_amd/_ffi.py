@@ -11,6 +11,14 @@ if not os.path.exists(LIB_PATH):
         "or `make -C peregrine_amd/csrc`. peregrine_amd has no CPU fallback."
     )
 
+# A process that also uses PyTorch-ROCm must load torch's bundled HIP runtime first: the library then binds to
+# that copy.  Loaded the other way round the process holds two runtimes, and the second to initialise finds no
+# device ("no ROCm-capable device is detected" from pg_ctx_create).
+try:
+    import torch  # noqa: F401
+except ImportError:
+    pass
+
 lib = C.CDLL(LIB_PATH)
 
 PG_OK, PG_EINVAL, PG_EDEVICE, PG_ENOMEM, PG_EUNSUPPORTED = 0, 1, 2, 3, 4
