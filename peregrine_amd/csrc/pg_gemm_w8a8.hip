@@ -411,6 +411,133 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const int32_t *__res
     if (acc_out) acc_out[i] = acc;
 }
 
+// ---- 2 .. 32 activation rows: one pass over the weights, no K split between workgroups -------------
+// A workgroup owns 16 weight rows (output columns) and all of K: its NW wavefronts take one K run each and add
+// their 16 x 16 i32 tiles through LDS at the end, so nothing is left for a second launch.  Operands of
+// v_mfma_i32_16x16x64_i8 want lane -> (row lane % 16, 16 k at lane / 16): loaded that way from row-major memory,
+// one instruction touches 64 cache lines a quarter at a time and the CU's vector cache, not HBM, sets the pace
+// (19 us for 58.7 MB).  So every wavefront keeps a ring of its own in LDS, filled by direct global -> LDS loads in
+// units of 128 k: one instruction brings 8 rows x 128 B (whole lines), chunk position p of row r holding the row's
+// 16-byte chunk p ^ ((r >> 1) & 7), so that the fragment reads (16 rows, one chunk) fall into 16 different bank
+// groups.  A unit of the ring holds the weight tile and MB tiles of quantised activation rows (from L2); NST - 1
+// units are in flight while one is consumed.  No barrier in the loop: a wavefront reads only what it has loaded
+// itself.  (The activations in fragment order straight into registers, with a deeper ring for the weights alone,
+// measured slower: 13.0 against 11.8 us.)
+// Every weight row is k_pad bytes from the next, so workgroups that all walked K from the start of their runs would
+// ask the same memory channels at the same time: each starts at its own unit and wraps round its run (integer
+// sums do not depend on the order).  The epilogue is the reference's (acc as f32) * a_scale[m] * w_scale[n]
+// (src/quant.rs:163).  a_i8 has at least 16 MB rows of a_stride bytes (rows >= m feed accumulators never stored).
+// NB: tiles of 16 weight rows per workgroup (2 for more than 16 activation rows: every activation fragment then
+// meets two weight tiles, which halves what the CUs pull from L2).
+template <int MB, int NB, int NW, int NST>
+__global__ __launch_bounds__(64 * NW) void gemm_w8a8_skinny_kernel(const int8_t *__restrict__ a_i8, const int8_t *__restrict__ w_t,
+                                                                    int k_pad, int m, int n, const float *__restrict__ a_scales,
+                                                                    const float *__restrict__ w_scales, float *__restrict__ out,
+                                                                    int32_t *__restrict__ acc_out) {
+    constexpr int TILE = 2048, UNIT = (NB + MB) * TILE, LPS = 2 * (NB + MB);  // bytes per tile and unit; fills per unit
+    static_assert((NST - 1) * LPS < 64 && NST <= 6, "the wait counter holds 63");
+    extern __shared__ __attribute__((aligned(1024))) char lds[];  // NW rings of NST units; afterwards the wavefronts' tiles
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n0 = blockIdx.x * 16 * NB;
+    const int units = k_pad / 128, per = (units + NW - 1) / NW;
+    const int u_begin = wave * per, u_end = u_begin + per < units ? u_begin + per : units;
+    const int cnt = u_end - u_begin;
+    char *ring = lds + (size_t)wave * NST * UNIT;
+    // fill duty of this lane: rows 8 j + lane / 8 (j = 0, 1) of every tile, chunk (lane % 8) ^ ((row >> 1) & 7)
+    const int8_t *src[NB + MB][2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int r = 8 * j + (lane >> 3), ch = (lane & 7) ^ ((r >> 1) & 7);
+#pragma unroll
+        for (int c = 0; c < NB; ++c) src[c][j] = w_t + (size_t)(n0 + 16 * c + r) * k_pad + ch * 16;  // (weight rows are padded to 256)
+#pragma unroll
+        for (int b = 0; b < MB; ++b) src[NB + b][j] = a_i8 + (size_t)(16 * b + r) * k_pad + ch * 16;
+    }
+    // fragment reads: row lane % 16, chunk 4 s + lane / 16 of k-step s
+    const int fr = lane & 15, fsw = (fr >> 1) & 7;
+    int rd[2];
+#pragma unroll
+    for (int st = 0; st < 2; ++st) rd[st] = fr * 128 + (((4 * st + (lane >> 4)) ^ fsw) * 16);
+    const int rot = cnt > 0 ? (int)((blockIdx.x * 5u) % (unsigned)cnt) : 0;
+    auto issue = [&](auto slot, int t) {  // t-th unit of the walk into ring slot `slot`
+        const int r = t + rot;
+        const size_t kb = (size_t)(u_begin + (r >= cnt ? r - cnt : r)) * 128;
+        char *base = ring + decltype(slot)::value * UNIT;
+#pragma unroll
+        for (int q = 0; q < NB; ++q)  // the weights: used once, non-temporal
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                __builtin_amdgcn_global_load_lds((gptr_t)(src[q][j] + kb), (lptr_t)(base + q * TILE + j * 1024), 16, 0, 2);
+#pragma unroll
+        for (int q = NB; q < NB + MB; ++q)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                __builtin_amdgcn_global_load_lds((gptr_t)(src[q][j] + kb), (lptr_t)(base + q * TILE + j * 1024), 16, 0, 0);
+    };
+    v4i acc[NB][MB];
+#pragma unroll
+    for (int c = 0; c < NB; ++c)
+#pragma unroll
+        for (int b = 0; b < MB; ++b) acc[c][b] = v4i{0, 0, 0, 0};
+    auto consume = [&](auto slot) {
+        const char *base = ring + decltype(slot)::value * UNIT;
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+            v4i wf[NB];
+#pragma unroll
+            for (int c = 0; c < NB; ++c) wf[c] = *reinterpret_cast<const v4i *>(base + c * TILE + rd[st]);
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+                const v4i af = *reinterpret_cast<const v4i *>(base + (NB + b) * TILE + rd[st]);
+#pragma unroll
+                for (int c = 0; c < NB; ++c) acc[c][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf[c], acc[c][b], 0, 0, 0);
+            }
+        }
+    };
+    if (cnt > 0) {
+        // prologue: NST - 1 units requested (fewer if the run is shorter)
+#define PG_SK_PRO(U) if (U < NST - 1 && U < cnt) issue(std::integral_constant<int, (U < NST ? U : 0)>{}, U);
+        PG_SK_PRO(0) PG_SK_PRO(1) PG_SK_PRO(2) PG_SK_PRO(3) PG_SK_PRO(4)
+#undef PG_SK_PRO
+        for (int t0 = 0; t0 < cnt; t0 += NST) {
+#define PG_SK_STEP(U)                                                                                          \
+            if (U < NST && t0 + U < cnt) {                                                                     \
+                const int t = t0 + U;                                                                          \
+                /* unit t is the oldest of those in flight: all but the NST - 2 younger ones have landed */   \
+                if (t + NST - 2 < cnt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 2) * LPS) : "memory");  \
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                          \
+                if (t + NST - 1 < cnt) issue(std::integral_constant<int, (U + NST - 1) % NST>{}, t + NST - 1); \
+                __builtin_amdgcn_sched_barrier(0);                                                             \
+                consume(std::integral_constant<int, (U < NST ? U : 0)>{});                                     \
+                __builtin_amdgcn_sched_barrier(0);                                                             \
+            }
+            PG_SK_STEP(0) PG_SK_STEP(1) PG_SK_STEP(2) PG_SK_STEP(3) PG_SK_STEP(4) PG_SK_STEP(5)
+#undef PG_SK_STEP
+        }
+    }
+    __syncthreads();  // the rings are done with: their space takes the wavefronts' tiles
+    int *red = reinterpret_cast<int *>(lds);  // [NW][NB * MB][4][64]
+#pragma unroll
+    for (int c = 0; c < NB; ++c)
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[((wave * NB * MB + c * MB + b) * 4 + i) * 64 + lane] = acc[c][b][i];
+    __syncthreads();
+    for (int e = threadIdx.x; e < NB * MB * 4 * 64; e += 64 * NW) {
+        const int l = e & 63, i = (e >> 6) & 3, cb = e >> 8, c = cb / MB, b = cb - c * MB;
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += red[((w * NB * MB + cb) * 4 + i) * 64 + l];
+        const int row = b * 16 + 4 * (l >> 4) + i, col = n0 + 16 * c + (l & 15);
+        if (row < m && col < n) {
+            const size_t o = (size_t)row * n + col;
+            if (out) out[o] = (float)sum * a_scales[row] * w_scales[col];
+            if (acc_out) acc_out[o] = sum;
+        }
+    }
+}
+
 // Tile choice (measured on MI355X at M = 2048): the larger the tile the fewer bytes each
 // CU pulls from L2 per MFMA, but every CU needs a tile.  8 wavefronts per workgroup also
 // double the rate at which one CU can stream from L2 (about 9 GB/s per wavefront).
@@ -490,6 +617,45 @@ pg_status pg_launch_gemm_w8a8_few_rows(pg_ctx *ctx, const int8_t *a_i8, size_t a
     const size_t plane = m * n;
     return pg_launch(ctx, "gemm_w8a8_finish", splitk_finish_kernel, dim3((unsigned)((plane + 255) / 256)), dim3(256), 0,
                      (const int32_t *)part, (int)splits, plane, a_scales, (const float *)w->scales, (int)n, out, acc);
+}
+
+// 2 .. 32 rows in one launch (see gemm_w8a8_skinny_kernel).
+bool pg_gemm_w8a8_takes_skinny(const pg_qtensor *w, size_t m) { return m >= 2 && m <= 32 && w->k_pad < (1ull << 30) && w->cols < (1ull << 30); }
+
+pg_status pg_launch_gemm_w8a8_skinny(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                                     const pg_qtensor *w, size_t m, float *out, int32_t *acc) {
+    if (a_stride != w->k_pad) return pg_fail(PG_EINVAL, "gemm_w8a8: activation stride %zu != k_pad %zu", a_stride, w->k_pad);
+    if (!pg_gemm_w8a8_takes_skinny(w, m)) return pg_fail(PG_EINVAL, "gemm_w8a8 (few rows in one launch): m = %zu", m);
+    // Wavefronts per workgroup (K runs): as many as keep every workgroup resident at once -- a second round of
+    // workgroups would stream its weights after the first has drained.  The rings fill the CU's LDS: eight
+    // wavefronts a CU with 16 to 18 KiB each, or four with 32 KiB where more than 16 rows meet two weight tiles at
+    // a time -- which pays while that still gives every CU a workgroup (32 rows, us: 4096 -> 14336 14.7 against
+    // 16.0, but 14336 -> 4096 20.0 against 16.0).
+    const int nb_tiles = (m > 16 && w->cols / 32 >= (size_t)ctx->num_cu) ? 2 : 1;
+    const dim3 grid((unsigned)((w->cols + 16 * nb_tiles - 1) / (16 * nb_tiles)));
+    const size_t slots = (size_t)ctx->num_cu * (nb_tiles == 1 ? 8 : 4), units = w->k_pad / 128;
+    int nw = nb_tiles == 1 ? 8 : 4;
+    while (nw > 1 && ((size_t)grid.x * nw > slots || units / nw < 4)) nw >>= 1;
+#define PG_SKINNY_LAUNCH(MBB, NBB, NWW, NSTT)                                                                                \
+    do {                                                                                                                     \
+        auto kern = gemm_w8a8_skinny_kernel<MBB, NBB, NWW, NSTT>;                                                            \
+        const size_t lds = (size_t)NWW * NSTT * (NBB + MBB) * 2048;                                                          \
+        PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                          \
+        return pg_launch(ctx, "gemm_w8a8_few_rows", kern, grid, dim3(64 * NWW), lds, a_i8, (const int8_t *)w->w_t,         \
+                         (int)w->k_pad, (int)m, (int)w->cols, a_scales, (const float *)w->scales, out, acc);                 \
+    } while (0)
+#define PG_SKINNY_NW(MBB, NBB, NSTT)                        \
+    switch (nw) {                                           \
+        case 8: PG_SKINNY_LAUNCH(MBB, NBB, 8, NSTT);        \
+        case 4: PG_SKINNY_LAUNCH(MBB, NBB, 4, NSTT);        \
+        case 2: PG_SKINNY_LAUNCH(MBB, NBB, 2, NSTT);        \
+        default: PG_SKINNY_LAUNCH(MBB, NBB, 1, NSTT);       \
+    }
+    if (m <= 16) PG_SKINNY_NW(1, 1, 4)
+    if (nb_tiles == 1) PG_SKINNY_NW(2, 1, 3)
+    PG_SKINNY_NW(2, 2, 4)
+#undef PG_SKINNY_NW
+#undef PG_SKINNY_LAUNCH
 }
 
 // a_i8 must have at least round_up(m, 256) rows of a_stride bytes (rows >= m may

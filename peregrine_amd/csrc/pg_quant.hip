@@ -516,7 +516,8 @@ static pg_status matmul_quantized_on(pg_ctx *ctx, const float *a_dev, size_t m, 
     // (up to 64 rows always; up to 256 only for long-K, narrow-N products like a down projection --
     // measured at 128 rows: 14336 -> 4096 35 -> 25 us split, but 4096 -> 4096 12.6 -> 19 us)
     int splits = 1;
-    if (m > PG_GEMV_MAX_M && (m <= 64 || (m <= 256 && w->k_pad >= 2 * w->cols)))
+    const bool skinny = pg_gemm_w8a8_takes_skinny(w, m);
+    if (!skinny && m > PG_GEMV_MAX_M && (m <= 64 || (m <= 256 && w->k_pad >= 2 * w->cols)))
         PG_TRY(pg_launch_gemm_w8a8_few_rows(ctx, nullptr, w->k_pad, nullptr, w, m, nullptr, nullptr, nullptr, &splits));
     const size_t sz_scales = pg_round_up(m_pad * sizeof(float), 256);
     const size_t part_bytes = splits > 1 ? (size_t)splits * m * w->cols * sizeof(int32_t) : 0;
@@ -532,6 +533,7 @@ static pg_status matmul_quantized_on(pg_ctx *ctx, const float *a_dev, size_t m, 
     int8_t *a_i8 = static_cast<int8_t *>(ws);
     float *a_scales = reinterpret_cast<float *>(a_i8 + a_bytes);
     PG_TRY(pg_launch_quantize_activations(ctx, a_dev, m, k, a_i8, w->k_pad, a_scales));
+    if (skinny) return pg_launch_gemm_w8a8_skinny(ctx, a_i8, w->k_pad, a_scales, w, m, out_dev, acc_dev);
     if (m <= PG_GEMV_MAX_M)
         return pg_launch_gemv_w8a8(ctx, a_i8, w->k_pad, a_scales, w, m, out_dev, acc_dev);
     if (splits > 1)
@@ -616,6 +618,18 @@ PG_API pg_status pg_matmul_quantized_multi_dev(pg_ctx *ctx, const float *a_dev, 
     for (size_t i = 0; i < count && one_row_group; ++i) one_row_group = pg_gemv_w8a8_takes_f32_row(w[i], m, k, a_dev);
     if (one_row_group)  // one token: every weight's rows in one streaming launch that quantises the row itself
         return pg_launch_gemv_w8a8_f32_row_group(ctx, a_dev, k, w, out_dev, (int)count, nullptr);
+    bool skinny_group = count > 1;
+    for (size_t i = 0; i < count && skinny_group; ++i) skinny_group = pg_gemm_w8a8_takes_skinny(w[i], m) && w[i]->k_pad == w[0]->k_pad;
+    if (skinny_group) {  // 2 .. 32 rows: quantised once, then one launch per weight
+        const size_t k_pad = w[0]->k_pad, a_bytes = pg_round_up(m, PG_MPAD) * k_pad;
+        void *ws = nullptr;
+        PG_TRY(pg_workspace(ctx, a_bytes + pg_round_up(PG_MPAD * sizeof(float), 256), &ws));
+        int8_t *a_i8 = static_cast<int8_t *>(ws);
+        float *a_scales = reinterpret_cast<float *>(a_i8 + a_bytes);
+        PG_TRY(pg_launch_quantize_activations(ctx, a_dev, m, k, a_i8, k_pad, a_scales));
+        for (size_t i = 0; i < count; ++i) PG_TRY(pg_launch_gemm_w8a8_skinny(ctx, a_i8, k_pad, a_scales, w[i], m, out_dev[i], nullptr));
+        return PG_OK;
+    }
     if (count == 1 || m <= 256) {  // few rows: the single products pick their own route (GEMV, split K)
         for (size_t i = 0; i < count; ++i) PG_TRY(pg_matmul_quantized_dev(ctx, a_dev, m, k, w[i], out_dev[i], nullptr));
         return PG_OK;

@@ -158,8 +158,12 @@ MATMUL_SHAPES = [
     (2050, 192, 4100),                                 # 128x256 tiles, ragged m and n
     (2049, 128, 12300),                                # 256x256 tiles, ragged m and n
     (1030, 256, 4000),                                 # 128x128 tiles unsplit, ragged m and n
-    # 5 .. 64 rows: K split over workgroups, i32 partial planes, finishing pass (ragged everywhere)
-    (5, 4096, 1000), (17, 4224, 520), (33, 1024, 4100), (40, 1024, 14336), (64, 14336, 300), (31, 512, 77),
+    # 2 .. 32 rows: one launch, a workgroup per 16 (or 32) weight rows with its wavefronts on runs of K (ragged everywhere;
+    # K of one unit of 128; more than 16 rows on a wide tensor: two weight tiles per workgroup)
+    (5, 4096, 1000), (17, 4224, 520), (31, 512, 77), (2, 128, 16), (16, 130, 5), (9, 2000, 33), (20, 1024, 8200),
+    (32, 4096, 14336), (17, 384, 8208), (24, 14336, 4096), (3, 14336, 4100),
+    # 33 .. 64 rows: K split over workgroups, i32 partial planes, finishing pass
+    (33, 1024, 4100), (40, 1024, 14336), (64, 14336, 300),
     (100, 8192, 300), (130, 4096, 257), (256, 2048, 1000),   # up to 256 rows when K >= 2 N: 128-row tiles
 ]
 
@@ -374,8 +378,9 @@ def run_multi(ctx, da, m, k, qts, douts):
 
 @pytest.mark.parametrize("m,k,ns", [(300, 512, (1000, 130, 257)), (257, 128, (64, 64, 64, 64)), (40, 1024, (300, 77)),
                                      (1, 4096, (1024, 512)), (1, 14336, (300, 77, 4096)), (3, 200, (33,)), (2048, 4096, (4096, 1024, 1024)),
-                                     (2048, 4096, (14336, 14336))],
-                         ids=["ragged3", "four", "few-rows", "one-row", "one-row-long-k", "single", "qkv", "gate-up"])
+                                     (2048, 4096, (14336, 14336)), (8, 4096, (4096, 1024, 1030)), (32, 1000, (8200, 520))],
+                         ids=["ragged3", "four", "few-rows", "one-row", "one-row-long-k", "single", "qkv", "gate-up",
+                              "qkv-8-rows-quantised-once", "32-rows-quantised-once"])
 def test_matmul_quantized_multi_equals_the_single_products(ctx, orc, m, k, ns):
     """Several weights against one activation matrix (the reference's fused QKV / gate|up
     products): every output equals the single product bit for bit, and sampled rows equal the
