@@ -411,7 +411,7 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const int32_t *__res
     if (acc_out) acc_out[i] = acc;
 }
 
-// ---- 2 .. 32 activation rows: one pass over the weights, no K split between workgroups -------------
+// ---- 2 .. 64 activation rows: one pass over the weights, no K split between workgroups -------------
 // A workgroup owns 16 weight rows (output columns) and all of K: its NW wavefronts take one K run each and add
 // their 16 x 16 i32 tiles through LDS at the end, so nothing is left for a second launch.  Operands of
 // v_mfma_i32_16x16x64_i8 want lane -> (row lane % 16, 16 k at lane / 16): loaded that way from row-major memory,
@@ -619,8 +619,10 @@ pg_status pg_launch_gemm_w8a8_few_rows(pg_ctx *ctx, const int8_t *a_i8, size_t a
                      (const int32_t *)part, (int)splits, plane, a_scales, (const float *)w->scales, (int)n, out, acc);
 }
 
-// 2 .. 32 rows in one launch (see gemm_w8a8_skinny_kernel).
-bool pg_gemm_w8a8_takes_skinny(const pg_qtensor *w, size_t m) { return m >= 2 && m <= 32 && w->k_pad < (1ull << 30) && w->cols < (1ull << 30); }
+// 2 .. 64 rows in one launch (see gemm_w8a8_skinny_kernel).
+// (33 .. 64 rows, us with the quantisation launch: 4096 -> 14336 24.7 against 30.3 split over K with a finishing pass,
+// 4096 -> 4096 11.1 against 15.8, but 14336 -> 4096 27.8 against 26.2: long, narrow products keep the split.)
+bool pg_gemm_w8a8_takes_skinny(const pg_qtensor *w, size_t m) { return m >= 2 && (m <= 32 || (m <= 64 && w->cols >= w->k_pad)) && w->k_pad < (1ull << 30) && w->cols < (1ull << 30); }
 
 pg_status pg_launch_gemm_w8a8_skinny(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
                                      const pg_qtensor *w, size_t m, float *out, int32_t *acc) {
@@ -628,13 +630,18 @@ pg_status pg_launch_gemm_w8a8_skinny(pg_ctx *ctx, const int8_t *a_i8, size_t a_s
     if (!pg_gemm_w8a8_takes_skinny(w, m)) return pg_fail(PG_EINVAL, "gemm_w8a8 (few rows in one launch): m = %zu", m);
     // Wavefronts per workgroup (K runs): as many as keep every workgroup resident at once -- a second round of
     // workgroups would stream its weights after the first has drained.  The rings fill the CU's LDS: eight
-    // wavefronts a CU with 16 to 18 KiB each, or four with 32 KiB where more than 16 rows meet two weight tiles at
-    // a time -- which pays while that still gives every CU a workgroup (32 rows, us: 4096 -> 14336 14.7 against
-    // 16.0, but 14336 -> 4096 20.0 against 16.0).
+    // wavefronts a CU with 16 to 18 KiB each up to 32 rows, four with 30 to 36 KiB where four activation tiles or
+    // two weight tiles share a unit.  Two weight tiles a workgroup (more than 16 rows: halves what the CUs pull
+    // from L2 for the activations) pay while that still gives every CU a workgroup (32 rows, us: 4096 -> 14336
+    // 14.7 against 16.0, but 14336 -> 4096 20.0 against 16.0).
+    const int mb = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
     const int nb_tiles = (m > 16 && w->cols / 32 >= (size_t)ctx->num_cu) ? 2 : 1;
+    const int nst = mb == 1 ? 4 : (mb == 2 && nb_tiles == 2 ? 4 : 3);
+    const size_t ring = (size_t)nst * (nb_tiles + mb) * 2048;
+    const int per_cu = ring * 8 <= 160 * 1024 ? 8 : 4;
     const dim3 grid((unsigned)((w->cols + 16 * nb_tiles - 1) / (16 * nb_tiles)));
-    const size_t slots = (size_t)ctx->num_cu * (nb_tiles == 1 ? 8 : 4), units = w->k_pad / 128;
-    int nw = nb_tiles == 1 ? 8 : 4;
+    const size_t slots = (size_t)ctx->num_cu * per_cu, units = w->k_pad / 128;
+    int nw = per_cu;
     while (nw > 1 && ((size_t)grid.x * nw > slots || units / nw < 4)) nw >>= 1;
 #define PG_SKINNY_LAUNCH(MBB, NBB, NWW, NSTT)                                                                                \
     do {                                                                                                                     \
@@ -644,17 +651,26 @@ pg_status pg_launch_gemm_w8a8_skinny(pg_ctx *ctx, const int8_t *a_i8, size_t a_s
         return pg_launch(ctx, "gemm_w8a8_few_rows", kern, grid, dim3(64 * NWW), lds, a_i8, (const int8_t *)w->w_t,         \
                          (int)w->k_pad, (int)m, (int)w->cols, a_scales, (const float *)w->scales, out, acc);                 \
     } while (0)
-#define PG_SKINNY_NW(MBB, NBB, NSTT)                        \
+#define PG_SKINNY_NW8(MBB, NBB, NSTT)                       \
     switch (nw) {                                           \
         case 8: PG_SKINNY_LAUNCH(MBB, NBB, 8, NSTT);        \
         case 4: PG_SKINNY_LAUNCH(MBB, NBB, 4, NSTT);        \
         case 2: PG_SKINNY_LAUNCH(MBB, NBB, 2, NSTT);        \
         default: PG_SKINNY_LAUNCH(MBB, NBB, 1, NSTT);       \
     }
-    if (m <= 16) PG_SKINNY_NW(1, 1, 4)
-    if (nb_tiles == 1) PG_SKINNY_NW(2, 1, 3)
-    PG_SKINNY_NW(2, 2, 4)
-#undef PG_SKINNY_NW
+#define PG_SKINNY_NW4(MBB, NBB, NSTT)                       \
+    switch (nw) {                                           \
+        case 4: PG_SKINNY_LAUNCH(MBB, NBB, 4, NSTT);        \
+        case 2: PG_SKINNY_LAUNCH(MBB, NBB, 2, NSTT);        \
+        default: PG_SKINNY_LAUNCH(MBB, NBB, 1, NSTT);       \
+    }
+    if (mb == 1) PG_SKINNY_NW8(1, 1, 4)
+    if (mb == 2 && nb_tiles == 1) PG_SKINNY_NW8(2, 1, 3)
+    if (mb == 2) PG_SKINNY_NW4(2, 2, 4)
+    if (nb_tiles == 1) PG_SKINNY_NW4(4, 1, 3)
+    PG_SKINNY_NW4(4, 2, 3)
+#undef PG_SKINNY_NW8
+#undef PG_SKINNY_NW4
 #undef PG_SKINNY_LAUNCH
 }
 

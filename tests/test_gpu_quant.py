@@ -162,8 +162,10 @@ MATMUL_SHAPES = [
     # K of one unit of 128; more than 16 rows on a wide tensor: two weight tiles per workgroup)
     (5, 4096, 1000), (17, 4224, 520), (31, 512, 77), (2, 128, 16), (16, 130, 5), (9, 2000, 33), (20, 1024, 8200),
     (32, 4096, 14336), (17, 384, 8208), (24, 14336, 4096), (3, 14336, 4100),
-    # 33 .. 64 rows: K split over workgroups, i32 partial planes, finishing pass
-    (33, 1024, 4100), (40, 1024, 14336), (64, 14336, 300),
+    # 33 .. 64 rows on products at least as wide as long: the same with four activation tiles a unit
+    (33, 1024, 4100), (40, 1024, 14336), (64, 4096, 4096), (50, 384, 8300),
+    # 33 .. 64 rows on long, narrow products: K split over workgroups, i32 partial planes, finishing pass
+    (64, 14336, 300), (40, 8192, 4096),
     (100, 8192, 300), (130, 4096, 257), (256, 2048, 1000),   # up to 256 rows when K >= 2 N: 128-row tiles
 ]
 
