@@ -40,11 +40,17 @@ pg_status pg_launch_check(const char *what) {
 }
 
 pg_status pg_allow_dynamic_lds(pg_ctx *ctx, const void *kernel, size_t bytes) {
-    for (const void *k : ctx->lds_raised)
-        if (k == kernel) return PG_OK;
+    // (the limit only ever grows: a kernel launched with more than an earlier call asked for is raised again)
+    std::pair<const void *, size_t> *slot = nullptr;
+    for (auto &k : ctx->lds_raised)
+        if (k.first == kernel) {
+            if (k.second >= bytes) return PG_OK;
+            slot = &k;
+        }
     hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) return pg_fail(PG_EDEVICE, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    ctx->lds_raised.push_back(kernel);
+    if (slot) slot->second = bytes;
+    else ctx->lds_raised.emplace_back(kernel, bytes);
     return PG_OK;
 }
 
@@ -82,7 +88,7 @@ PG_API pg_status pg_ctx_create(int device, void *hip_stream, pg_ctx **out) {
     ctx->ws_bytes = 0;
     ctx->num_cu = prop.multiProcessorCount;
     ctx->profiling = false;
-    ctx->lds_raised.reserve(64);  // so that noting a kernel's raised LDS limit never allocates later
+    ctx->lds_raised.reserve(256);  // so that noting a kernel's raised LDS limit never allocates later
     if (hip_stream) {
         ctx->stream = static_cast<hipStream_t>(hip_stream);
         ctx->owns_stream = false;

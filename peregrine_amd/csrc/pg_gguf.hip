@@ -922,12 +922,13 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
 // 8192 weight rows (measured one launch against two: 4096 -> 4096 5.5 against 6.7 us, 14336 -> 4096 11.5
 // against 12.8 us; but 4096 -> 14336 10.9 against 10.3 us, and Q8_0 there 19.3 against 14.6 us).
 // k_in up to 32768 (the row's digits live in LDS).
-// Two rows at once, three or four over a small tensor (Q4_0; all their digits fit in LDS).  The kernel's time grows
-// by the arithmetic of every further row, the matrix-core route's hardly at all, but that one is three launches:
-// 4096 -> 14336 in us, rows 2 / 3 / 4: 12.2 / 16.2 / 19.9 against 17.5 / 17.5 / 17.7; 4096 -> 4096: 6.7 / 8.6 / 10.4
-// against 13.4; 14336 -> 4096: 17.8 / 24.1 against 21.4.
+// Two rows at once, three over a small tensor (Q4_0, K up to 8192; all their digits fit in LDS).  The kernel's time
+// grows by the arithmetic of every further row and by the digits of K m elements that every workgroup makes; the
+// matrix-core routes' hardly at all, but they start with a launch for the digits: us, rows 2 / 3 / 4, against
+// digits + one matrix-core launch at 4 rows: 4096 -> 14336 12.2 / 16.2 / 19.9 against 14.4; 4096 -> 4096 6.7 / 8.6 /
+// 10.4 against 8.2; 14336 -> 4096 17.8 / 24.1 / - against 14.3.
 bool pg_gguf_gemv_takes_few_rows(int ggml_type, size_t m, size_t n_out, size_t k_in, const float *x_f32) {
-    return ggml_type == PG_GGML_Q4_0 && (m == 2 || ((m == 3 || m == 4) && n_out * k_in <= ((size_t)1 << 25))) && k_in >= 32 &&
+    return ggml_type == PG_GGML_Q4_0 && (m == 2 || (m == 3 && n_out * k_in <= ((size_t)1 << 25))) && k_in >= 32 && k_in <= 8192 &&
            fewrows_lds(m, k_in) <= 150 * 1024 && (uintptr_t)x_f32 % 16 == 0;
 }
 
@@ -1036,6 +1037,12 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
         PG_TRY(pg_launch_x_to_digits(ctx, x_dev, m, w->k_in, w->ggml_type, xd));
         pg_gemv_batch batch = {(int)m, nullptr, nullptr, nullptr, 1};
         return pg_launch_gguf_gemv(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, batch, xd, y_dev, nullptr, w->m);
+    }
+    if (pg_gguf_skinny_takes(ctx, w->ggml_type, m, w->n_out, w->k_in)) {  // up to 16 rows: digits, then one launch
+        PG_TRY(pg_workspace(ctx, pg_mmdigits_bytes(m, w->k_in), &ws));
+        const pg_mmdigits md = pg_mmdigits_carve(ws, m, w->k_in);
+        PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, m, w->k_in, w->ggml_type, md));
+        return pg_launch_gguf_skinny(ctx, w->n_out, w->k_in, w->qs, w->d, m, md, y_dev);
     }
     const int ks = pg_gguf_mm_splitk(ctx, w->n_out, w->k_in, (m + 31) / 32, m, false, nullptr);
     const size_t sz_d = pg_mmdigits_bytes(m, w->k_in);

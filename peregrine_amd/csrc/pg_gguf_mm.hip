@@ -515,6 +515,208 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+// ---- up to 16 activation rows over a Q4_0 tensor in one launch after the digits ---------------------------------
+// The product above splits K between workgroups where one token tile meets a wide tensor, and a third launch adds
+// the planes.  Here a workgroup owns 16 NB weight rows and all of K: its NW wavefronts take one run of K each, every
+// wavefront with an LDS ring of its own (no barrier in the loop: it reads only what it loaded itself), and their
+// f32 tiles are added through LDS in a fixed order at the end.  A unit of the ring is 8 blocks (256 k): the weight
+// tiles as whole 128-byte lines per row (8 rows an instruction, 16-byte chunk p of row r at position
+// p ^ ((r >> 1) & 7)), their f16 scales, the two digit planes of the 16 token rows (256 bytes a row and plane,
+// chunk c of token t at position c ^ t) and the tokens' block scales; NST - 1 units are in flight while one is
+// consumed.  v_mfma_i32_16x16x32_i8 takes one block per instruction: lane -> (token or weight row lane % 16, 8 k at
+// lane / 16), result lane -> weight row lane % 16, tokens 4 (lane / 16) + i.  The weights are read in the row-major
+// planes every tensor has (no tile-major copy).  Each workgroup starts its walk through K at its own unit.
+// MT: token rows the ring holds (4, 8 or 16: the digits are most of a unit, and the fewer there are the more units
+// fit in flight); token slots from MT on read the rows of slots 0 .. MT - 1 again and are never stored.
+template <int NB, int MT, int NW, int NST>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void gguf_skinny_q4_0_kernel(const uint8_t *__restrict__ qs, const uint16_t *__restrict__ dsc,
+                                                                    int n_out, int nb, int nbp, int m,
+                                                                    const int8_t *__restrict__ digits, const float *__restrict__ xs,
+                                                                    float *__restrict__ y) {
+    constexpr int W_T = 2048, D_T = 256, DIG = MT * 512, XS_B = 512, GQ = MT / 2;  // GQ: digit fills per unit
+    constexpr int OFF_DS = NB * W_T, OFF_DG = OFF_DS + NB * D_T, OFF_X = OFF_DG + DIG, UNIT = OFF_X + XS_B;
+    constexpr int LPS = 2 * NB + 1 + GQ + 1;  // fills per unit
+    static_assert((NST - 1) * LPS < 64 && NST <= 6 && NB <= 2, "the wait counter holds 63");
+    extern __shared__ __attribute__((aligned(1024))) char lds[];  // NW rings of NST units; afterwards the wavefronts' tiles
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n0 = blockIdx.x * 16 * NB;
+    const int units = nb / 8, per = (units + NW - 1) / NW;
+    const int u_begin = wave * per, u_end = u_begin + per < units ? u_begin + per : units;
+    const int cnt = u_end - u_begin;
+    char *ring = lds + (size_t)wave * NST * UNIT;
+    const size_t row_bytes = pg_mm_row_bytes(nb);
+
+    // fill duties of this lane
+    const uint8_t *w_src[NB][2];  // weight rows 8 j + lane / 8 of tile c, chunk (lane % 8) ^ ((row >> 1) & 7); rows past the end: the last
+#pragma unroll
+    for (int c = 0; c < NB; ++c)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int r = 8 * j + (lane >> 3), ch = (lane & 7) ^ ((r >> 1) & 7);
+            const int row = n0 + 16 * c + r < n_out ? n0 + 16 * c + r : n_out - 1;
+            w_src[c][j] = qs + (size_t)row * nb * 16 + ch * 16;
+        }
+    // scales: lanes 0 .. 16 NB - 1: scale tile (n0 / 8 + lane / 8), blocks of the unit lane % 8 (16 bytes = 8 rows x f16)
+    const int ntile = (n_out + 7) / 8;
+    const int dt = (n0 >> 3) + (lane >> 3) < ntile ? (n0 >> 3) + (lane >> 3) : ntile - 1;
+    const char *d_src = reinterpret_cast<const char *>(dsc) + ((size_t)dt * nb + (lane & 7)) * 16;
+    // digits: instruction q covers runs 4 q .. 4 q + 3, run = 2 token + plane; lane -> run 4 q + lane / 16, position lane % 16
+    const int8_t *g_src[GQ];
+#pragma unroll
+    for (int q = 0; q < GQ; ++q) {
+        const int run = 4 * q + (lane >> 4), tok = run >> 1, pl = run & 1;
+        const int ch = (lane & 15) ^ tok;
+        g_src[q] = digits + (size_t)(tok < m ? tok : 0) * row_bytes + (size_t)pl * nb * 32 + ch * 16;
+    }
+    // token scales: lanes 0 .. 2 MT - 1: token lane / 2, blocks 4 (lane % 2) .. + 3 of the unit
+    const float *x_src = xs + (size_t)((lane >> 1) < m ? (lane >> 1) : 0) * nbp + 4 * (lane & 1);
+
+    const int rot = cnt > 0 ? (int)((blockIdx.x * 5u) % (unsigned)cnt) : 0;
+    auto issue = [&](auto slot, int t) {
+        const int r = t + rot;
+        const size_t unit = (size_t)(u_begin + (r >= cnt ? r - cnt : r));
+        char *base = ring + decltype(slot)::value * UNIT;
+#pragma unroll
+        for (int c = 0; c < NB; ++c)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                __builtin_amdgcn_global_load_lds((gptr_t)(w_src[c][j] + unit * 128), (lptr_t)(base + c * W_T + j * 1024), 16, 0, 2);
+        if (lane < 16 * NB) __builtin_amdgcn_global_load_lds((gptr_t)(d_src + unit * 128), (lptr_t)(base + OFF_DS), 16, 0, 0);
+#pragma unroll
+        for (int q = 0; q < GQ; ++q)
+            __builtin_amdgcn_global_load_lds((gptr_t)(g_src[q] + unit * 256), (lptr_t)(base + OFF_DG + q * 1024), 16, 0, 0);
+        if (lane < 2 * MT) __builtin_amdgcn_global_load_lds((gptr_t)(x_src + unit * 8), (lptr_t)(base + OFF_X), 16, 0, 0);
+    };
+
+    // fragment reads of this lane
+    const int fr = lane & 15, g4 = lane >> 4, ft = fr & (MT - 1);
+    const int w_rd = fr * 128 + 8 * (g4 & 1), w_sw = (fr >> 1) & 7;        // + ((j ^ w_sw) * 16): bytes 8 (g4 & 1) .. of block j
+    const int dg_rd = OFF_DG + ft * 512 + 8 * (g4 & 1);                     // + plane * 256 + (((2 j + (g4 >> 1)) ^ ft) * 16)
+    const int ds_rd = OFF_DS + (fr >> 3) * 128 + (fr & 7) * 2;              // + tile c * 256 + j * 16: this lane's weight row
+    const int x_rd = OFF_X + ((4 * g4) & (MT - 1)) * 32;                    // tokens 4 g4 .. + 3, 8 floats each
+    const int left = 4 - 4 * (g4 >> 1);                                     // low nibbles for the even elements' half
+
+    float acc[NB][4];
+#pragma unroll
+    for (int c = 0; c < NB; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[c][i] = 0.0f;
+
+    auto consume = [&](auto slot) {
+        const char *base = ring + decltype(slot)::value * UNIT;
+        // the scales of this lane's four tokens for the unit's eight blocks (read as integers: see gguf_mm_kernel)
+        int sx[4][8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const v4i t = *reinterpret_cast<const v4i *>(base + x_rd + i * 32 + h * 16);
+                const int t0 = t[0], t1 = t[1], t2 = t[2], t3 = t[3];
+                sx[i][4 * h] = t0; sx[i][4 * h + 1] = t1; sx[i][4 * h + 2] = t2; sx[i][4 * h + 3] = t3;
+            }
+        // Software pipeline over the unit's 8 blocks: while block j is scaled and accumulated on the vector ALU,
+        // the MFMAs of block j + 1 run and the LDS reads of block j + 2 return (one wavefront a SIMD: nothing else
+        // would fill those waits).
+        long dh[2], dl[2];
+        v2i wraw[2][NB];
+        unsigned db[2][NB];
+        v4i ihi[2][NB], ilo[2][NB];
+        auto read = [&](int buf, int j) {
+            const int dpos = (((2 * j + (g4 >> 1)) ^ ft) * 16);
+            dh[buf] = *reinterpret_cast<const long *>(base + dg_rd + dpos);
+            dl[buf] = *reinterpret_cast<const long *>(base + dg_rd + 256 + dpos);
+#pragma unroll
+            for (int c = 0; c < NB; ++c) wraw[buf][c] = *reinterpret_cast<const v2i *>(base + c * W_T + w_rd + ((j ^ w_sw) * 16));
+        };
+        auto read_d = [&](int buf, int j) {  // the blocks' weight scales of this lane's rows
+#pragma unroll
+            for (int c = 0; c < NB; ++c) db[buf][c] = *reinterpret_cast<const unsigned short *>(base + ds_rd + c * D_T + j * 16);
+        };
+        auto mfmas = [&](int buf, int c) {
+            const v4i zero = {0, 0, 0, 0};
+            {
+                v2i wq;
+                wq[0] = nibbles_to_i8x16(wraw[buf][c][0], left);
+                wq[1] = nibbles_to_i8x16(wraw[buf][c][1], left);
+                const long wl = __builtin_bit_cast(long, wq);
+                ihi[buf][c] = __builtin_amdgcn_mfma_i32_16x16x32_i8(dh[buf], wl, zero, 0, 0, 0);  // rows = tokens, columns = weight rows
+                ilo[buf][c] = __builtin_amdgcn_mfma_i32_16x16x32_i8(dl[buf], wl, zero, 0, 0, 0);
+            }
+        };
+        auto scale = [&](int buf, int j, int c) {
+            {
+                const float dv = half_bits_to_float(db[buf][c]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float fx = (float)(ihi[buf][c][i] * 256 + ilo[buf][c][i]) * __int_as_float(sx[i][j]);
+                    acc[c][i] = fmaf(dv, fx, acc[c][i]);
+                }
+            }
+        };
+        read(0, 0);
+        read_d(0, 0);
+        read(1, 1);
+#pragma unroll
+        for (int c = 0; c < NB; ++c) mfmas(0, c);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            // tile by tile: the two MFMAs of block j + 1 are issued, then block j of the same tile is scaled while
+            // they run (instructions issue in order: MFMAs back to back would hold the vector work behind them)
+            // (the LDS reads of block j + 2 go first and have the whole step to return; their buffers held block j,
+            // whose MFMAs were issued a step ago)
+            if (j + 1 < 8) read_d((j + 1) & 1, j + 1);
+            if (j + 2 < 8) read(j & 1, j + 2);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int c = 0; c < NB; ++c) {
+                if (j + 1 < 8) {
+                    mfmas((j + 1) & 1, c);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                scale(j & 1, j, c);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    if (cnt > 0) {
+#define PG_GS_PRO(U) if (U < NST - 1 && U < cnt) issue(std::integral_constant<int, (U < NST ? U : 0)>{}, U);
+        PG_GS_PRO(0) PG_GS_PRO(1) PG_GS_PRO(2) PG_GS_PRO(3) PG_GS_PRO(4)
+#undef PG_GS_PRO
+        for (int t0 = 0; t0 < cnt; t0 += NST) {
+#define PG_GS_STEP(U)                                                                                          \
+            if (U < NST && t0 + U < cnt) {                                                                     \
+                const int t = t0 + U;                                                                          \
+                /* unit t is the oldest of those in flight: all but the NST - 2 younger ones have landed */   \
+                if (t + NST - 2 < cnt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 2) * LPS) : "memory");  \
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                          \
+                if (t + NST - 1 < cnt) issue(std::integral_constant<int, (U + NST - 1) % NST>{}, t + NST - 1); \
+                __builtin_amdgcn_sched_barrier(0);                                                             \
+                consume(std::integral_constant<int, (U < NST ? U : 0)>{});                                     \
+                __builtin_amdgcn_sched_barrier(0);                                                             \
+            }
+            PG_GS_STEP(0) PG_GS_STEP(1) PG_GS_STEP(2) PG_GS_STEP(3) PG_GS_STEP(4) PG_GS_STEP(5)
+#undef PG_GS_STEP
+        }
+    }
+    __syncthreads();  // the rings are done with: their space takes the wavefronts' tiles
+    float *red = reinterpret_cast<float *>(lds);  // [NW][NB][4][64]
+#pragma unroll
+    for (int c = 0; c < NB; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[((wave * NB + c) * 4 + i) * 64 + lane] = acc[c][i];
+    __syncthreads();
+    for (int e = threadIdx.x; e < NB * 4 * 64; e += 64 * NW) {
+        const int l = e & 63, i = (e >> 6) & 3, c = e >> 8;
+        float sum = red[(c * 4 + i) * 64 + l];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) sum += red[((w * NB + c) * 4 + i) * 64 + l];  // ascending runs of K
+        const int tok = 4 * (l >> 4) + i, row = n0 + 16 * c + (l & 15);
+        if (tok < m && row < n_out) y[(size_t)tok * n_out + row] = sum * 0.0625f;  // the weight operand was 16 * (q - 8)
+    }
+}
+
 // y[i] = part[0][i] + part[1][i] + ... in a fixed order.
 __global__ void sum_parts_kernel(const float *__restrict__ part, size_t n, int ks, size_t stride, float *__restrict__ y) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -608,6 +810,55 @@ int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t group
     if (chunk_out) *chunk_out = (int)chunk;
     if (xcd_chunks) *xcd_chunks = by_xcd;
     return (int)ks_real;
+}
+
+// Up to 16 rows over a Q4_0 tensor whose K is a multiple of 256: the one-launch product (see the kernel).  The
+// kernel is bound by instruction issue (about 500 instructions per 8 blocks and weight tile pair, most of them the
+// per-block scaling), so what counts is wavefronts per SIMD, and LDS decides that: up to 8 token rows the rings are
+// small enough for eight wavefronts a CU (4096 -> 14336, us with the digits' launch: 4 rows 14.5, 8 rows 15.2,
+// against 19.5 and 18.0 for digits + product over four K chunks + their sum); with 16 token rows four fit, which
+// beats the three launches only where those are short of workgroups (14336 -> 4096: 19.0 against 24.3; 4096 -> 4096:
+// 9.1 against 13.3; but 4096 -> 14336: 21.1 against 20.3-22.0).
+bool pg_gguf_skinny_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_out, size_t k_in) {
+    return ggml_type == PG_GGML_Q4_0 && m >= 2 && (m <= 8 || (m <= 16 && n_out / 32 < (size_t)ctx->num_cu)) && k_in % 256 == 0 &&
+           k_in >= 1024 && n_out >= 1 && n_out < (1u << 30) && k_in < (1u << 24);
+}
+
+pg_status pg_launch_gguf_skinny(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, size_t m,
+                                const pg_mmdigits &md, float *y) {
+    if (!pg_gguf_skinny_takes(ctx, PG_GGML_Q4_0, m, n_out, k_in)) return pg_fail(PG_EINVAL, "gguf (few rows in one launch): [%zu x %zu] x %zu", m, k_in, n_out);
+    const int nb = (int)(k_in / 32), nbp = (int)pg_round_up(nb, 4);
+    // Wavefronts (runs of K) per workgroup: as many as keep every workgroup resident at once.
+    const int per_cu = m <= 8 ? 8 : 4;
+    const dim3 grid((unsigned)((n_out + 15) / 16));
+    const size_t slots = (size_t)ctx->num_cu * per_cu, units = (size_t)nb / 8;
+    int nw = per_cu;
+    while (nw > 1 && ((size_t)grid.x * nw > slots || units / nw < 4)) nw >>= 1;
+#define PG_GSK_LAUNCH(MTT, NWW, NSTT)                                                                                          \
+    do {                                                                                                                       \
+        auto kern = gguf_skinny_q4_0_kernel<1, MTT, NWW, NSTT>;                                                                \
+        const size_t lds = (size_t)NWW * NSTT * (2304 + MTT * 512 + 512);                                                      \
+        PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                            \
+        return pg_launch(ctx, "gguf_q4_0_few_rows_mm", kern, grid, dim3(64 * NWW), lds, qs, d, (int)n_out, nb, nbp, (int)m,   \
+                         (const int8_t *)md.digits, (const float *)md.xs, y);                                                  \
+    } while (0)
+#define PG_GSK_NW(MTT, NSTT)                      \
+    switch (nw) {                                 \
+        case 8: PG_GSK_LAUNCH(MTT, 8, NSTT);      \
+        case 4: PG_GSK_LAUNCH(MTT, 4, NSTT);      \
+        case 2: PG_GSK_LAUNCH(MTT, 2, NSTT);      \
+        default: PG_GSK_LAUNCH(MTT, 1, NSTT);     \
+    }
+    // ring stages: what the wavefronts' rings leave of 160 KiB (a unit: 4.75 / 6.75 / 10.75 KiB)
+    if (m <= 4) PG_GSK_NW(4, 4)
+    if (m <= 8) PG_GSK_NW(8, 2)
+    switch (nw) {
+        case 4: PG_GSK_LAUNCH(16, 4, 3);
+        case 2: PG_GSK_LAUNCH(16, 2, 3);
+        default: PG_GSK_LAUNCH(16, 1, 3);
+    }
+#undef PG_GSK_NW
+#undef PG_GSK_LAUNCH
 }
 
 pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,

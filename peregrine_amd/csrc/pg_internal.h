@@ -45,7 +45,7 @@ struct pg_ctx {
     };
     std::vector<moe_table> moe_tabs;
     // Kernels whose dynamic LDS limit was raised on this context's device (pg_allow_dynamic_lds).
-    std::vector<const void *> lds_raised;
+    std::vector<std::pair<const void *, size_t>> lds_raised;  // kernels whose dynamic-LDS limit was raised, and to what
     // W8A8 GEMM dispatch: the tile of the most recent launch (pg_gemm_w8a8_last_tile) and an
     // optional override of the dispatcher's choice (pg_gemm_w8a8_force_tile; 0 = automatic).
     int gemm_last_bm = 0, gemm_last_bn = 0, gemm_last_splits = 0;
@@ -296,6 +296,9 @@ struct pg_mmdigits {
 };
 size_t pg_mmdigits_bytes(size_t rows, size_t k);
 pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k);
+bool pg_gguf_skinny_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_out, size_t k_in);
+pg_status pg_launch_gguf_skinny(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, size_t m,
+                                const pg_mmdigits &md, float *y);
 pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows, size_t k, int ggml_type,
                                    const pg_mmdigits &md);
 // Q4_1 on the matrix-core route: the product is the Q4_0 product on the same nibbles and scales plus
