@@ -816,9 +816,9 @@ int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t group
 // kernel is bound by instruction issue (about 500 instructions per 8 blocks and weight tile pair, most of them the
 // per-block scaling), so what counts is wavefronts per SIMD, and LDS decides that: up to 8 token rows the rings are
 // small enough for eight wavefronts a CU (4096 -> 14336, us with the digits' launch: 4 rows 14.5, 8 rows 15.2,
-// against 19.5 and 18.0 for digits + product over four K chunks + their sum); with 16 token rows four fit, which
-// beats the three launches only where those are short of workgroups (14336 -> 4096: 19.0 against 24.3; 4096 -> 4096:
-// 9.1 against 13.3; but 4096 -> 14336: 21.1 against 20.3-22.0).
+// against 19.5 and 18.0 for digits + product over four K chunks + their sum); with 16 token rows seven fit at two
+// units a ring, which beats the three launches only where those are short of workgroups (14336 -> 4096: 18.2
+// against 24.3; 4096 -> 4096: 8.8 against 13.3; but 4096 -> 14336: 21.5 against 20.0-22.0).
 bool pg_gguf_skinny_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_out, size_t k_in) {
     return ggml_type == PG_GGML_Q4_0 && m >= 2 && (m <= 8 || (m <= 16 && n_out / 32 < (size_t)ctx->num_cu)) && k_in % 256 == 0 &&
            k_in >= 1024 && n_out >= 1 && n_out < (1u << 30) && k_in < (1u << 24);
@@ -829,10 +829,10 @@ pg_status pg_launch_gguf_skinny(pg_ctx *ctx, size_t n_out, size_t k_in, const ui
     if (!pg_gguf_skinny_takes(ctx, PG_GGML_Q4_0, m, n_out, k_in)) return pg_fail(PG_EINVAL, "gguf (few rows in one launch): [%zu x %zu] x %zu", m, k_in, n_out);
     const int nb = (int)(k_in / 32), nbp = (int)pg_round_up(nb, 4);
     // Wavefronts (runs of K) per workgroup: as many as keep every workgroup resident at once.
-    const int per_cu = m <= 8 ? 8 : 4;
+    const int per_cu = m <= 8 ? 8 : 7;  // (16 token rows: a ring of two units, 21.5 KiB; three units and four wavefronts a CU were slower)
     const dim3 grid((unsigned)((n_out + 15) / 16));
     const size_t slots = (size_t)ctx->num_cu * per_cu, units = (size_t)nb / 8;
-    int nw = per_cu;
+    int nw = m <= 8 ? 8 : 4;
     while (nw > 1 && ((size_t)grid.x * nw > slots || units / nw < 4)) nw >>= 1;
 #define PG_GSK_LAUNCH(MTT, NWW, NSTT)                                                                                          \
     do {                                                                                                                       \
@@ -849,13 +849,13 @@ pg_status pg_launch_gguf_skinny(pg_ctx *ctx, size_t n_out, size_t k_in, const ui
         case 2: PG_GSK_LAUNCH(MTT, 2, NSTT);      \
         default: PG_GSK_LAUNCH(MTT, 1, NSTT);     \
     }
-    // ring stages: what the wavefronts' rings leave of 160 KiB (a unit: 4.75 / 6.75 / 10.75 KiB)
+    // ring stages: what the wavefronts' rings can have of 160 KiB (a unit: 4.75 / 6.75 / 10.75 KiB)
     if (m <= 4) PG_GSK_NW(4, 4)
     if (m <= 8) PG_GSK_NW(8, 2)
     switch (nw) {
-        case 4: PG_GSK_LAUNCH(16, 4, 3);
-        case 2: PG_GSK_LAUNCH(16, 2, 3);
-        default: PG_GSK_LAUNCH(16, 1, 3);
+        case 4: PG_GSK_LAUNCH(16, 4, 2);
+        case 2: PG_GSK_LAUNCH(16, 2, 2);
+        default: PG_GSK_LAUNCH(16, 1, 2);
     }
 #undef PG_GSK_NW
 #undef PG_GSK_LAUNCH
