@@ -577,14 +577,14 @@ def section_gguf(B, line):
         mm_bytes = n_out * (k_in // 32) * 18 + 4 * m_q * k_in + 4 * m_q * n_out
         t_mm = B.timed(mm_step, B.dsteps, max(args.warmup, 8))
         prof, grids = B.profiled(mm_step, B.dsteps)
-        # up to 8 rows: one matrix-core launch after the digits (gguf_skinny_q4_0_kernel); more: product over K chunks + their sum
+        # up to 8 rows: one matrix-core launch after the digits (gguf_skinny_kernel); more: product over K chunks + their sum
         k_name = "gguf_q4_0_few_rows_mm" if "gguf_q4_0_few_rows_mm" in prof else "gguf_mm_q4_0"
         k_ms = prof[k_name][0]
         entry = {"workload": f"cfg4: M={m_q} Q4_0 dequant-matmul [{m_q}x4096]->[{m_q}x14336], weights read once",
                  "value": round(mm_bytes / (t_mm["ms_per_step"] * 1e-3) / 1e9, 1), "unit": "GB/s", **B.stats(t_mm),
                  "gflops": round(2 * m_q * n_out * k_in / (t_mm["ms_per_step"] * 1e-3) / 1e9, 1),
                  "kernels_ms": {k: round(v[0], 5) for k, v in prof.items()},
-                 "roofline": {"kernel": "gguf_skinny_q4_0_kernel" if k_name == "gguf_q4_0_few_rows_mm" else "gguf_mm_kernel<Q4_0>", "bound": "hbm",
+                 "roofline": {"kernel": "gguf_skinny_kernel<Q4_0>" if k_name == "gguf_q4_0_few_rows_mm" else "gguf_mm_kernel<Q4_0>", "bound": "hbm",
                               "achieved": round(mm_bytes / (k_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                               "frac": round(mm_bytes / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                               "traffic": B.traffic_for(k_name, grids),

@@ -515,7 +515,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
-// ---- up to 16 activation rows over a Q4_0 tensor in one launch after the digits ---------------------------------
+// ---- up to 16 activation rows over a Q4_0 or Q8_0 tensor in one launch after the digits ------------------------
 // The product above splits K between workgroups where one token tile meets a wide tensor, and a third launch adds
 // the planes.  Here a workgroup owns 16 NB weight rows and all of K: its NW wavefronts take one run of K each, every
 // wavefront with an LDS ring of its own (no barrier in the loop: it reads only what it loaded itself), and their
@@ -528,14 +528,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // planes every tensor has (no tile-major copy).  Each workgroup starts its walk through K at its own unit.
 // MT: token rows the ring holds (4, 8 or 16: the digits are most of a unit, and the fewer there are the more units
 // fit in flight); token slots from MT on read the rows of slots 0 .. MT - 1 again and are never stored.
-template <int NB, int MT, int NW, int NST>
-__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void gguf_skinny_q4_0_kernel(const uint8_t *__restrict__ qs, const uint16_t *__restrict__ dsc,
+// QT = 8 (Q8_0): a weight row is two streams (bytes 0 .. 15 and 16 .. 31 of its blocks, as the upload splits them), 32
+// streams a tile, kept in LDS half-major (stream slot 16 half + row) so that the fragment reads of 16 rows and one
+// half stay free of bank conflicts; no nibbles to unpack.
+template <int QT, int NB, int MT, int NW, int NST>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void gguf_skinny_kernel(const uint8_t *__restrict__ qs, const uint16_t *__restrict__ dsc,
                                                                     int n_out, int nb, int nbp, int m,
                                                                     const int8_t *__restrict__ digits, const float *__restrict__ xs,
                                                                     float *__restrict__ y) {
-    constexpr int W_T = 2048, D_T = 256, DIG = MT * 512, XS_B = 512, GQ = MT / 2;  // GQ: digit fills per unit
+    constexpr int WF = QT == 8 ? 4 : 2, W_T = WF * 1024, D_T = 256, DIG = MT * 512, XS_B = 512, GQ = MT / 2;  // WF, GQ: weight, digit fills per unit
     constexpr int OFF_DS = NB * W_T, OFF_DG = OFF_DS + NB * D_T, OFF_X = OFF_DG + DIG, UNIT = OFF_X + XS_B;
-    constexpr int LPS = 2 * NB + 1 + GQ + 1;  // fills per unit
+    constexpr int LPS = WF * NB + 1 + GQ + 1;  // fills per unit
     static_assert((NST - 1) * LPS < 64 && NST <= 6 && NB <= 2, "the wait counter holds 63");
     extern __shared__ __attribute__((aligned(1024))) char lds[];  // NW rings of NST units; afterwards the wavefronts' tiles
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -547,14 +550,14 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     const size_t row_bytes = pg_mm_row_bytes(nb);
 
     // fill duties of this lane
-    const uint8_t *w_src[NB][2];  // weight rows 8 j + lane / 8 of tile c, chunk (lane % 8) ^ ((row >> 1) & 7); rows past the end: the last
+    const uint8_t *w_src[NB][WF];  // stream slot 8 j + lane / 8 of tile c (Q4_0: slot = row; Q8_0: slot = 16 half + row), chunk (lane % 8) ^ ((row >> 1) & 7); rows past the end: the last
 #pragma unroll
     for (int c = 0; c < NB; ++c)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int r = 8 * j + (lane >> 3), ch = (lane & 7) ^ ((r >> 1) & 7);
+        for (int j = 0; j < WF; ++j) {
+            const int slot = 8 * j + (lane >> 3), r = slot & 15, half = slot >> 4, ch = (lane & 7) ^ ((r >> 1) & 7);
             const int row = n0 + 16 * c + r < n_out ? n0 + 16 * c + r : n_out - 1;
-            w_src[c][j] = qs + (size_t)row * nb * 16 + ch * 16;
+            w_src[c][j] = qs + (QT == 8 ? (size_t)row * 2 + half : (size_t)row) * nb * 16 + ch * 16;
         }
     // scales: lanes 0 .. 16 NB - 1: scale tile (n0 / 8 + lane / 8), blocks of the unit lane % 8 (16 bytes = 8 rows x f16)
     const int ntile = (n_out + 7) / 8;
@@ -579,7 +582,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
         for (int c = 0; c < NB; ++c)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < WF; ++j)
                 __builtin_amdgcn_global_load_lds((gptr_t)(w_src[c][j] + unit * 128), (lptr_t)(base + c * W_T + j * 1024), 16, 0, 2);
         if (lane < 16 * NB) __builtin_amdgcn_global_load_lds((gptr_t)(d_src + unit * 128), (lptr_t)(base + OFF_DS), 16, 0, 0);
 #pragma unroll
@@ -590,7 +593,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
     // fragment reads of this lane
     const int fr = lane & 15, g4 = lane >> 4, ft = fr & (MT - 1);
-    const int w_rd = fr * 128 + 8 * (g4 & 1), w_sw = (fr >> 1) & 7;        // + ((j ^ w_sw) * 16): bytes 8 (g4 & 1) .. of block j
+    const int w_rd = ((QT == 8 ? 16 * (g4 >> 1) : 0) + fr) * 128 + 8 * (g4 & 1), w_sw = (fr >> 1) & 7;  // + ((j ^ w_sw) * 16): bytes 8 (g4 & 1) .. of block j
     const int dg_rd = OFF_DG + ft * 512 + 8 * (g4 & 1);                     // + plane * 256 + (((2 j + (g4 >> 1)) ^ ft) * 16)
     const int ds_rd = OFF_DS + (fr >> 3) * 128 + (fr & 7) * 2;              // + tile c * 256 + j * 16: this lane's weight row
     const int x_rd = OFF_X + ((4 * g4) & (MT - 1)) * 32;                    // tokens 4 g4 .. + 3, 8 floats each
@@ -635,9 +638,11 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
         auto mfmas = [&](int buf, int c) {
             const v4i zero = {0, 0, 0, 0};
             {
-                v2i wq;
-                wq[0] = nibbles_to_i8x16(wraw[buf][c][0], left);
-                wq[1] = nibbles_to_i8x16(wraw[buf][c][1], left);
+                v2i wq = wraw[buf][c];
+                if constexpr (QT == 4) {
+                    wq[0] = nibbles_to_i8x16(wq[0], left);
+                    wq[1] = nibbles_to_i8x16(wq[1], left);
+                }
                 const long wl = __builtin_bit_cast(long, wq);
                 ihi[buf][c] = __builtin_amdgcn_mfma_i32_16x16x32_i8(dh[buf], wl, zero, 0, 0, 0);  // rows = tokens, columns = weight rows
                 ilo[buf][c] = __builtin_amdgcn_mfma_i32_16x16x32_i8(dl[buf], wl, zero, 0, 0, 0);
@@ -713,7 +718,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
         for (int w = 1; w < NW; ++w) sum += red[((w * NB + c) * 4 + i) * 64 + l];  // ascending runs of K
         const int tok = 4 * (l >> 4) + i, row = n0 + 16 * c + (l & 15);
-        if (tok < m && row < n_out) y[(size_t)tok * n_out + row] = sum * 0.0625f;  // the weight operand was 16 * (q - 8)
+        if (tok < m && row < n_out) y[(size_t)tok * n_out + row] = QT == 4 ? sum * 0.0625f : sum;  // (Q4_0: the weight operand was 16 * (q - 8))
     }
 }
 
@@ -820,44 +825,54 @@ int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t group
 // units a ring, which beats the three launches only where those are short of workgroups (14336 -> 4096: 18.2
 // against 24.3; 4096 -> 4096: 8.8 against 13.3; but 4096 -> 14336: 21.5 against 20.0-22.0).
 bool pg_gguf_skinny_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_out, size_t k_in) {
-    return ggml_type == PG_GGML_Q4_0 && m >= 2 && (m <= 8 || (m <= 16 && n_out / 32 < (size_t)ctx->num_cu)) && k_in % 256 == 0 &&
-           k_in >= 1024 && n_out >= 1 && n_out < (1u << 30) && k_in < (1u << 24);
+    return (ggml_type == PG_GGML_Q4_0 || ggml_type == PG_GGML_Q8_0) && m >= 2 && (m <= 8 || (m <= 16 && n_out / 32 < (size_t)ctx->num_cu)) &&
+           k_in % 256 == 0 && k_in >= 1024 && n_out >= 1 && n_out < (1u << 30) && k_in < (1u << 24);
 }
 
-pg_status pg_launch_gguf_skinny(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, size_t m,
+pg_status pg_launch_gguf_skinny(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, size_t m,
                                 const pg_mmdigits &md, float *y) {
-    if (!pg_gguf_skinny_takes(ctx, PG_GGML_Q4_0, m, n_out, k_in)) return pg_fail(PG_EINVAL, "gguf (few rows in one launch): [%zu x %zu] x %zu", m, k_in, n_out);
+    if (!pg_gguf_skinny_takes(ctx, ggml_type, m, n_out, k_in)) return pg_fail(PG_EINVAL, "gguf (few rows in one launch): [%zu x %zu] x %zu", m, k_in, n_out);
     const int nb = (int)(k_in / 32), nbp = (int)pg_round_up(nb, 4);
-    // Wavefronts (runs of K) per workgroup: as many as keep every workgroup resident at once.
-    const int per_cu = m <= 8 ? 8 : 7;  // (16 token rows: a ring of two units, 21.5 KiB; three units and four wavefronts a CU were slower)
+    const bool q8 = ggml_type == PG_GGML_Q8_0;
+    // Wavefronts (runs of K) per workgroup: as many as keep every workgroup resident at once.  The rings: units of
+    // 4.75 / 6.75 / 10.75 KiB for 4 / 8 / 16 token rows (Q8_0: 2 KiB more), as many stages as let eight wavefronts
+    // share a CU's LDS (16 token rows: two stages and six or seven wavefronts; three stages and four were slower).
+    const int per_cu = m <= 8 ? 8 : (q8 ? 6 : 7);
     const dim3 grid((unsigned)((n_out + 15) / 16));
     const size_t slots = (size_t)ctx->num_cu * per_cu, units = (size_t)nb / 8;
     int nw = m <= 8 ? 8 : 4;
     while (nw > 1 && ((size_t)grid.x * nw > slots || units / nw < 4)) nw >>= 1;
-#define PG_GSK_LAUNCH(MTT, NWW, NSTT)                                                                                          \
+#define PG_GSK_LAUNCH(QTT, MTT, NWW, NSTT)                                                                                     \
     do {                                                                                                                       \
-        auto kern = gguf_skinny_q4_0_kernel<1, MTT, NWW, NSTT>;                                                                \
-        const size_t lds = (size_t)NWW * NSTT * (2304 + MTT * 512 + 512);                                                      \
+        auto kern = gguf_skinny_kernel<QTT, 1, MTT, NWW, NSTT>;                                                                \
+        const size_t lds = (size_t)NWW * NSTT * ((QTT == 8 ? 4096 : 2048) + 256 + MTT * 512 + 512);                            \
         PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                            \
-        return pg_launch(ctx, "gguf_q4_0_few_rows_mm", kern, grid, dim3(64 * NWW), lds, qs, d, (int)n_out, nb, nbp, (int)m,   \
-                         (const int8_t *)md.digits, (const float *)md.xs, y);                                                  \
+        return pg_launch(ctx, QTT == 8 ? "gguf_q8_0_few_rows_mm" : "gguf_q4_0_few_rows_mm", kern, grid, dim3(64 * NWW), lds,  \
+                         qs, d, (int)n_out, nb, nbp, (int)m, (const int8_t *)md.digits, (const float *)md.xs, y);              \
     } while (0)
-#define PG_GSK_NW(MTT, NSTT)                      \
-    switch (nw) {                                 \
-        case 8: PG_GSK_LAUNCH(MTT, 8, NSTT);      \
-        case 4: PG_GSK_LAUNCH(MTT, 4, NSTT);      \
-        case 2: PG_GSK_LAUNCH(MTT, 2, NSTT);      \
-        default: PG_GSK_LAUNCH(MTT, 1, NSTT);     \
+#define PG_GSK_NW8(QTT, MTT, NSTT)                     \
+    switch (nw) {                                      \
+        case 8: PG_GSK_LAUNCH(QTT, MTT, 8, NSTT);      \
+        case 4: PG_GSK_LAUNCH(QTT, MTT, 4, NSTT);      \
+        case 2: PG_GSK_LAUNCH(QTT, MTT, 2, NSTT);      \
+        default: PG_GSK_LAUNCH(QTT, MTT, 1, NSTT);     \
     }
-    // ring stages: what the wavefronts' rings can have of 160 KiB (a unit: 4.75 / 6.75 / 10.75 KiB)
-    if (m <= 4) PG_GSK_NW(4, 4)
-    if (m <= 8) PG_GSK_NW(8, 2)
-    switch (nw) {
-        case 4: PG_GSK_LAUNCH(16, 4, 2);
-        case 2: PG_GSK_LAUNCH(16, 2, 2);
-        default: PG_GSK_LAUNCH(16, 1, 2);
+#define PG_GSK_NW4(QTT, MTT, NSTT)                     \
+    switch (nw) {                                      \
+        case 4: PG_GSK_LAUNCH(QTT, MTT, 4, NSTT);      \
+        case 2: PG_GSK_LAUNCH(QTT, MTT, 2, NSTT);      \
+        default: PG_GSK_LAUNCH(QTT, MTT, 1, NSTT);     \
     }
-#undef PG_GSK_NW
+    if (q8) {
+        if (m <= 4) PG_GSK_NW8(8, 4, 2)
+        if (m <= 8) PG_GSK_NW8(8, 8, 2)
+        PG_GSK_NW4(8, 16, 2)
+    }
+    if (m <= 4) PG_GSK_NW8(4, 4, 4)
+    if (m <= 8) PG_GSK_NW8(4, 8, 2)
+    PG_GSK_NW4(4, 16, 2)
+#undef PG_GSK_NW8
+#undef PG_GSK_NW4
 #undef PG_GSK_LAUNCH
 }
 

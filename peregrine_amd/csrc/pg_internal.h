@@ -297,7 +297,7 @@ struct pg_mmdigits {
 size_t pg_mmdigits_bytes(size_t rows, size_t k);
 pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k);
 bool pg_gguf_skinny_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_out, size_t k_in);
-pg_status pg_launch_gguf_skinny(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, size_t m,
+pg_status pg_launch_gguf_skinny(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, size_t m,
                                 const pg_mmdigits &md, float *y);
 pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows, size_t k, int ggml_type,
                                    const pg_mmdigits &md);

@@ -107,6 +107,8 @@ GGUF_SHAPES = [
     # a K of 4 and of 9 units; 12 rows over a wide tensor keep the product split over K
     (2, 1000, 4096, 7), (2, 333, 1024, 5), (2, 4100, 8192, 16), (2, 96, 2304, 9), (2, 14336, 4096, 12), (2, 4096, 14336, 8),
     (2, 4096, 4096, 5), (2, 40, 36864, 4),
+    # the same over Q8_0 (a weight row is two streams of 16-byte half blocks)
+    (8, 1000, 4096, 7), (8, 333, 1024, 2), (8, 4100, 8192, 16), (8, 96, 2304, 9), (8, 14336, 4096, 4), (8, 4096, 14336, 8), (8, 14336, 4096, 12),
     # Q4_1 (offset blocks): the streaming kernel with the block-sum term, one item per row
     (3, 256, 4096, 1), (3, 77, 96, 3), (3, 1000, 2048, 2), (3, 50, 11008, 1), (3, 64, 32768, 2), (3, 14336, 4096, 1), (3, 130, 224, 33),
     # Q4_1 from four rows on: the Q4_0 matrix-core product on the same nibbles plus the offsets times the rows' block sums
