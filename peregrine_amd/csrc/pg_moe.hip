@@ -129,7 +129,11 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
     //    of an output's error falls as 1 / sqrt(ffn) (measured 1.4e-3 of the row rms at ffn 64,
     //    below 2e-4 from ffn 2048 up).  Narrow experts are tiny products; the price is nil.
     const bool narrow = ffn < 512 && P <= 65535;
-    const bool up_stream = narrow || d / 32 < PG_MM_MIN_BLOCKS, down_stream = narrow || ffn / 32 < PG_MM_MIN_BLOCKS;
+    // 3. one token: its top_k pairs meet top_k different experts with one activation row each, which is the
+    //    streaming kernel's case (Grok-1-sized experts, Q8_0, top 2: 315 -> 227 us, the three products at 6.3 TB/s;
+    //    from two tokens on pairs share experts and the matrix-core kernel, which reads an expert once, wins)
+    const bool one_token = T == 1;
+    const bool up_stream = narrow || one_token || d / 32 < PG_MM_MIN_BLOCKS, down_stream = narrow || one_token || ffn / 32 < PG_MM_MIN_BLOCKS;
     PG_CHECK_ARG(!(up_stream || down_stream) || P <= 65535, "pg_moe_ffn: too many pairs for experts this small");
 
     // Arena layout.

@@ -48,6 +48,26 @@ def test_moe_small_vs_oracle(ctx, orc, typ, act):
         H.assert_close_rel(got[t], want[t], MOE_RTOL, f"token {t}")
 
 
+@pytest.mark.parametrize("typ", [8, 2])
+def test_moe_one_token_streams_its_experts(ctx, orc, typ):
+    """One token (a decode step): its top_k pairs go through the streaming kernel, one expert each, at widths where
+    more tokens take the matrix-core kernel; the same token inside a batch of three gives the same row to the
+    tolerance of that kernel."""
+    from peregrine_amd import gguf, moe
+    d, ffn, E, top_k = 512, 1536, 8, 2
+    say(f"moe one token typ={typ}")
+    raws = build(orc, 90, d, ffn, E, typ)
+    x = orc.rng_normal(5, 3 * d)
+    logits = orc.rng_normal(6, 3 * E).reshape(3, E)
+    mk = lambda rs, n_out, k_in: [gguf.GgufWeight(r, typ, n_out, k_in, ctx) for r in rs]
+    ex = moe.MoEExperts(mk(raws[0], ffn, d), mk(raws[1], ffn, d), mk(raws[2], d, ffn), top_k, moe.SILU, ctx)
+    got1 = ex.forward(x[:d], logits[:1]).reshape(-1)
+    want, _, _ = orc.moe_ffn(x[:d], 1, d, ffn, E, top_k, logits[:1], raws[0], raws[1], raws[2], typ, moe.SILU)
+    H.assert_close_rel(got1, want.reshape(-1), MOE_RTOL, "one token")
+    got3 = ex.forward(x, logits).reshape(3, d)
+    H.assert_close_rel(got3[0], got1, MOE_RTOL, "the same token in a batch")
+
+
 def test_moe_grok_shaped_reduced(ctx, orc):
     """benchmark configuration 5's structure (8 experts, top-2, 64 tokens, Q8_0, SiLU) at reduced
     width (d 512, ffn 1024) so the oracle finishes in seconds."""
