@@ -96,3 +96,47 @@ def test_block_step_replayed_from_a_graph(ctx, orc, typ, seq):
         hip.lib.hipGraphDestroy(graph)
     for w in ws:
         w.free()
+
+
+def test_few_row_products_replayed_from_a_graph(ctx, orc):
+    """The few-row products (W8A8 over 8 rows, Q4_0 over 5 and over 2 rows: one launch each after the rows'
+    quantisation / digits) captured together, after one eager call has made their buffers."""
+    from peregrine_amd import _ffi, gguf, quant
+    hip = Hip()
+    k, n = 1024, 520
+    qt = quant.quantize_weights(orc.rng_normal(31, k * n, 0.0, 0.02), k, n, ctx).to_gpu(ctx)
+    gw = gguf.GgufWeight(bytes(H.pack_q4_0(orc.rng_normal(32, n * k, 0.0, 0.03))), 2, n, k, ctx)
+    inputs = [orc.rng_normal(40 + i, 8 * k) for i in range(3)]
+    x = DevBuf(ctx, host=inputs[0])
+    outs = [DevBuf(ctx, 8 * n * 4) for _ in range(3)]
+
+    def step():
+        _ffi.check(_ffi.lib.pg_matmul_quantized_dev(ctx.handle, x.ptr, 8, k, qt._gpu, outs[0].ptr, None))
+        _ffi.check(_ffi.lib.pg_gguf_matmul_dev(ctx.handle, x.ptr, 5, gw._h, outs[1].ptr))
+        _ffi.check(_ffi.lib.pg_gguf_matmul_dev(ctx.handle, x.ptr, 2, gw._h, outs[2].ptr))
+
+    def eager(v):
+        _ffi.check(_ffi.lib.pg_memcpy_h2d(ctx.handle, x.ptr, C.c_void_p(v.ctypes.data), v.nbytes))
+        step()
+        ctx.sync()
+        return [o.to_host(np.float32) for o in outs]
+
+    want = [eager(v) for v in inputs]
+    say("capturing three few-row products")
+    graph, ex = hip.capture(ctx.stream, step)
+    try:
+        for i, v in enumerate(inputs):
+            _ffi.check(_ffi.lib.pg_gguf_matmul_dev(ctx.handle, x.ptr, 1, gw._h, outs[1].ptr))   # other work in between
+            _ffi.check(_ffi.lib.pg_memcpy_h2d(ctx.handle, x.ptr, C.c_void_p(v.ctypes.data), v.nbytes))
+            for o in outs:
+                _ffi.check(_ffi.lib.pg_memcpy_h2d(ctx.handle, o.ptr, C.c_void_p(np.full(8 * n, np.nan, np.float32).ctypes.data), 8 * n * 4))
+            ctx.sync()
+            hip.ok(hip.lib.hipGraphLaunch(ex, ctx.stream), "hipGraphLaunch")
+            ctx.sync()
+            for j, rows in enumerate((8, 5, 2)):
+                got = outs[j].to_host(np.float32)[: rows * n]
+                assert (got.view(np.uint32) == want[i][j][: rows * n].view(np.uint32)).all(), f"replay {i}, product {j} differs from the eager call"
+    finally:
+        hip.lib.hipGraphExecDestroy(ex)
+        hip.lib.hipGraphDestroy(graph)
+    gw.free()
