@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_kernel(
 #pragma unroll
         for (int j = 0; j < NCH; ++j) {
             const int c = lane + 64 * j;
-            w[j] = __builtin_nontemporal_load(wp + (c < nchunk ? c : lane));
+            w[j] = __builtin_nontemporal_load(wp + (c < nchunk ? c : 0));  // (past a short row: its first chunk, against zeros)
         }
         int acc = 0;
 #pragma unroll
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_w8a8_m1_f32x_kernel(
 #pragma unroll
         for (int j = 0; j < NCH; ++j) {
             const int c = lane + 64 * j;
-            w[j] = __builtin_nontemporal_load(wp + (c < nchunk ? c : lane));
+            w[j] = __builtin_nontemporal_load(wp + (c < nchunk ? c : 0));  // (past a short row: its first chunk, against zeros)
         }
     };
     // Loads return in issue order: the activation row (from L2) is requested first, so that its
