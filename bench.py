@@ -491,6 +491,24 @@ def section_decode_and_linear(B, line):
                            "launches_per_step": gemv_lps, "avg_launch_ms": round(gemv_avg_ms, 5)}}
     if B.cpu:
         decode["cpu_baseline"] = cpu_decode(B.orc, kept, x_d.cpu().numpy(), x_f.cpu().numpy(), dec_bytes)
+    # the same step over a small batch of rows (batched decode): the rows are quantised once, then one launch per weight
+    batched = []
+    for rows in (8, 32):
+        xb_d, xb_f = B.make_acts(rows, 4096, 1244), B.make_acts(rows, 14336, 1245)
+        yb_f, yb_u, yb_d = (torch.empty(rows, n, device=dev) for n in (14336, 14336, 4096))
+        gub_out = VP2(yb_f.data_ptr(), yb_u.data_ptr())
+
+        def batch_step():
+            r = B.i % LAYERS_ROT
+            B.i += 1
+            check(lib.pg_matmul_quantized_multi_dev(B.h, ptr(xb_d), rows, 4096, gu_tabs[r], 2, gub_out))
+            check(lib.pg_matmul_quantized_dev(B.h, ptr(xb_f), rows, 14336, dec_w[r][2], ptr(yb_d), None))
+
+        t_b = B.timed(batch_step, B.dsteps, max(args.warmup, 8))
+        prof_b, _ = B.profiled(batch_step, B.dsteps)
+        batched.append({"rows": rows, "ms_per_step": round(t_b["ms_per_step"], 5), "weight_gbs": round(3 * 4096 * 14336 / (t_b["ms_per_step"] * 1e-3) / 1e9, 1),
+                        "kernels_ms_x_launches": {k: [round(v[0], 5), v[1] / B.dsteps] for k, v in prof_b.items()}})
+    decode["batched"] = batched
     line["decode_gemv"] = decode
     del kept
     for trio in dec_w:
