@@ -429,16 +429,32 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const int32_t *__res
 // (src/quant.rs:163).  a_i8 has at least 16 MB rows of a_stride bytes (rows >= m feed accumulators never stored).
 // NB: tiles of 16 weight rows per workgroup (2 for more than 16 activation rows: every activation fragment then
 // meets two weight tiles, which halves what the CUs pull from L2).
+// Up to PG_GEMM_MAX_GROUP weights of equal K in one launch (the fused q|k|v and gate|up products of models::llama):
+// weight g owns the workgroups wg0[g] .. wg0[g + 1] - 1 (unused slots hold INT_MAX).
+struct skinny_wgroup {
+    const int8_t *w[PG_GEMM_MAX_GROUP];
+    const float *ws[PG_GEMM_MAX_GROUP];
+    float *out[PG_GEMM_MAX_GROUP];
+    int n[PG_GEMM_MAX_GROUP];
+    int wg0[PG_GEMM_MAX_GROUP];
+};
+
 template <int MB, int NB, int NW, int NST>
-__global__ __launch_bounds__(64 * NW) void gemm_w8a8_skinny_kernel(const int8_t *__restrict__ a_i8, const int8_t *__restrict__ w_t,
-                                                                    int k_pad, int m, int n, const float *__restrict__ a_scales,
-                                                                    const float *__restrict__ w_scales, float *__restrict__ out,
+__global__ __launch_bounds__(64 * NW) void gemm_w8a8_skinny_kernel(const int8_t *__restrict__ a_i8, const skinny_wgroup grp,
+                                                                    int k_pad, int m, const float *__restrict__ a_scales,
                                                                     int32_t *__restrict__ acc_out) {
+    int g = 0;
+#pragma unroll
+    for (int i = 1; i < PG_GEMM_MAX_GROUP; ++i) g = (int)blockIdx.x >= grp.wg0[i] ? i : g;
+    const int8_t *__restrict__ w_t = grp.w[g];
+    const float *__restrict__ w_scales = grp.ws[g];
+    float *__restrict__ out = grp.out[g];
+    const int n = grp.n[g];
     constexpr int TILE = 2048, UNIT = (NB + MB) * TILE, LPS = 2 * (NB + MB);  // bytes per tile and unit; fills per unit
     static_assert((NST - 1) * LPS < 64 && NST <= 6, "the wait counter holds 63");
     extern __shared__ __attribute__((aligned(1024))) char lds[];  // NW rings of NST units; afterwards the wavefronts' tiles
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int n0 = blockIdx.x * 16 * NB;
+    const int n0 = ((int)blockIdx.x - grp.wg0[g]) * 16 * NB;
     const int units = k_pad / 128, per = (units + NW - 1) / NW;
     const int u_begin = wave * per, u_end = u_begin + per < units ? u_begin + per : units;
     const int cnt = u_end - u_begin;
@@ -622,12 +638,21 @@ pg_status pg_launch_gemm_w8a8_few_rows(pg_ctx *ctx, const int8_t *a_i8, size_t a
 // 2 .. 64 rows in one launch (see gemm_w8a8_skinny_kernel).
 // (33 .. 64 rows, us with the quantisation launch: 4096 -> 14336 24.7 against 30.3 split over K with a finishing pass,
 // 4096 -> 4096 11.1 against 15.8, but 14336 -> 4096 27.8 against 26.2: long, narrow products keep the split.)
-bool pg_gemm_w8a8_takes_skinny(const pg_qtensor *w, size_t m) { return m >= 2 && (m <= 32 || (m <= 64 && w->cols >= w->k_pad)) && w->k_pad < (1ull << 30) && w->cols < (1ull << 30); }
+bool pg_gemm_w8a8_takes_skinny(const pg_qtensor *w, size_t m) { return m >= 2 && (m <= 32 || (m <= 64 && w->cols >= w->k_pad)) &&
+           w->k_pad < (1ull << 30) && w->cols < (1ull << 30); }
 
-pg_status pg_launch_gemm_w8a8_skinny(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
-                                     const pg_qtensor *w, size_t m, float *out, int32_t *acc) {
-    if (a_stride != w->k_pad) return pg_fail(PG_EINVAL, "gemm_w8a8: activation stride %zu != k_pad %zu", a_stride, w->k_pad);
-    if (!pg_gemm_w8a8_takes_skinny(w, m)) return pg_fail(PG_EINVAL, "gemm_w8a8 (few rows in one launch): m = %zu", m);
+// 2 .. 64 rows in one launch (see gemm_w8a8_skinny_kernel); `count` weights of equal K side by side.
+pg_status pg_launch_gemm_w8a8_skinny_group(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                                           const pg_qtensor *const *w, float *const *out, int count, size_t m, int32_t *acc) {
+    if (count < 1 || count > PG_GEMM_MAX_GROUP || (acc && count != 1))
+        return pg_fail(PG_EINVAL, "gemm_w8a8 (few rows in one launch): %d weights (1 .. %d; the accumulators of one only)", count, PG_GEMM_MAX_GROUP);
+    size_t cols = 0;
+    for (int i = 0; i < count; ++i) {
+        if (a_stride != w[i]->k_pad) return pg_fail(PG_EINVAL, "gemm_w8a8: activation stride %zu != k_pad %zu", a_stride, w[i]->k_pad);
+        if (!pg_gemm_w8a8_takes_skinny(w[i], m)) return pg_fail(PG_EINVAL, "gemm_w8a8 (few rows in one launch): m = %zu", m);
+        cols += w[i]->cols;
+    }
+    const size_t k_pad = w[0]->k_pad;
     // Wavefronts per workgroup (K runs): as many as keep every workgroup resident at once -- a second round of
     // workgroups would stream its weights after the first has drained.  The rings fill the CU's LDS: eight
     // wavefronts a CU with 16 to 18 KiB each up to 32 rows, four with 30 to 36 KiB where four activation tiles or
@@ -635,12 +660,23 @@ pg_status pg_launch_gemm_w8a8_skinny(pg_ctx *ctx, const int8_t *a_i8, size_t a_s
     // from L2 for the activations) pay while that still gives every CU a workgroup (32 rows, us: 4096 -> 14336
     // 14.7 against 16.0, but 14336 -> 4096 20.0 against 16.0).
     const int mb = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
-    const int nb_tiles = (m > 16 && w->cols / 32 >= (size_t)ctx->num_cu) ? 2 : 1;
+    const int nb_tiles = (m > 16 && cols / 32 >= (size_t)ctx->num_cu) ? 2 : 1;
     const int nst = mb == 1 ? 4 : (mb == 2 && nb_tiles == 2 ? 4 : 3);
     const size_t ring = (size_t)nst * (nb_tiles + mb) * 2048;
     const int per_cu = ring * 8 <= 160 * 1024 ? 8 : 4;
-    const dim3 grid((unsigned)((w->cols + 16 * nb_tiles - 1) / (16 * nb_tiles)));
-    const size_t slots = (size_t)ctx->num_cu * per_cu, units = w->k_pad / 128;
+    skinny_wgroup grp;
+    int wgs = 0;
+    for (int i = 0; i < PG_GEMM_MAX_GROUP; ++i) {
+        const bool used = i < count;
+        grp.w[i] = used ? w[i]->w_t : nullptr;
+        grp.ws[i] = used ? w[i]->scales : nullptr;
+        grp.out[i] = used ? out[i] : nullptr;
+        grp.n[i] = used ? (int)w[i]->cols : 0;
+        grp.wg0[i] = used ? wgs : INT_MAX;
+        if (used) wgs += (int)((w[i]->cols + 16 * nb_tiles - 1) / (16 * nb_tiles));
+    }
+    const dim3 grid((unsigned)wgs);
+    const size_t slots = (size_t)ctx->num_cu * per_cu, units = k_pad / 128;
     int nw = per_cu;
     while (nw > 1 && ((size_t)grid.x * nw > slots || units / nw < 4)) nw >>= 1;
 #define PG_SKINNY_LAUNCH(MBB, NBB, NWW, NSTT)                                                                                \
@@ -648,8 +684,7 @@ pg_status pg_launch_gemm_w8a8_skinny(pg_ctx *ctx, const int8_t *a_i8, size_t a_s
         auto kern = gemm_w8a8_skinny_kernel<MBB, NBB, NWW, NSTT>;                                                            \
         const size_t lds = (size_t)NWW * NSTT * (NBB + MBB) * 2048;                                                          \
         PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                          \
-        return pg_launch(ctx, "gemm_w8a8_few_rows", kern, grid, dim3(64 * NWW), lds, a_i8, (const int8_t *)w->w_t,         \
-                         (int)w->k_pad, (int)m, (int)w->cols, a_scales, (const float *)w->scales, out, acc);                 \
+        return pg_launch(ctx, "gemm_w8a8_few_rows", kern, grid, dim3(64 * NWW), lds, a_i8, grp, (int)k_pad, (int)m, a_scales, acc); \
     } while (0)
 #define PG_SKINNY_NW8(MBB, NBB, NSTT)                       \
     switch (nw) {                                           \
@@ -672,6 +707,11 @@ pg_status pg_launch_gemm_w8a8_skinny(pg_ctx *ctx, const int8_t *a_i8, size_t a_s
 #undef PG_SKINNY_NW8
 #undef PG_SKINNY_NW4
 #undef PG_SKINNY_LAUNCH
+}
+
+pg_status pg_launch_gemm_w8a8_skinny(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                                     const pg_qtensor *w, size_t m, float *out, int32_t *acc) {
+    return pg_launch_gemm_w8a8_skinny_group(ctx, a_i8, a_stride, a_scales, &w, &out, 1, m, acc);
 }
 
 // a_i8 must have at least round_up(m, 256) rows of a_stride bytes (rows >= m may

@@ -185,6 +185,8 @@ pg_status pg_launch_gemm_w8a8_group(pg_ctx *ctx, const int8_t *a_i8, size_t a_st
 pg_status pg_launch_gemm_w8a8_combine(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
                                       const pg_qtensor *w, size_t m, float *out, const int32_t *comb, size_t comb_plane);
 bool pg_gemm_w8a8_takes_skinny(const pg_qtensor *w, size_t m);
+pg_status pg_launch_gemm_w8a8_skinny_group(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
+                                           const pg_qtensor *const *w, float *const *out, int count, size_t m, int32_t *acc);
 pg_status pg_launch_gemm_w8a8_skinny(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,
                                      const pg_qtensor *w, size_t m, float *out, int32_t *acc);
 pg_status pg_launch_gemm_w8a8_few_rows(pg_ctx *ctx, const int8_t *a_i8, size_t a_stride, const float *a_scales,

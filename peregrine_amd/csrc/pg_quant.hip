@@ -620,15 +620,14 @@ PG_API pg_status pg_matmul_quantized_multi_dev(pg_ctx *ctx, const float *a_dev, 
         return pg_launch_gemv_w8a8_f32_row_group(ctx, a_dev, k, w, out_dev, (int)count, nullptr);
     bool skinny_group = count > 1;
     for (size_t i = 0; i < count && skinny_group; ++i) skinny_group = pg_gemm_w8a8_takes_skinny(w[i], m) && w[i]->k_pad == w[0]->k_pad;
-    if (skinny_group) {  // 2 .. 32 rows: quantised once, then one launch per weight
+    if (skinny_group) {  // 2 .. 64 rows: quantised once, then the weights side by side in one launch
         const size_t k_pad = w[0]->k_pad, a_bytes = pg_round_up(m, PG_MPAD) * k_pad;
         void *ws = nullptr;
         PG_TRY(pg_workspace(ctx, a_bytes + pg_round_up(PG_MPAD * sizeof(float), 256), &ws));
         int8_t *a_i8 = static_cast<int8_t *>(ws);
         float *a_scales = reinterpret_cast<float *>(a_i8 + a_bytes);
         PG_TRY(pg_launch_quantize_activations(ctx, a_dev, m, k, a_i8, k_pad, a_scales));
-        for (size_t i = 0; i < count; ++i) PG_TRY(pg_launch_gemm_w8a8_skinny(ctx, a_i8, k_pad, a_scales, w[i], m, out_dev[i], nullptr));
-        return PG_OK;
+        return pg_launch_gemm_w8a8_skinny_group(ctx, a_i8, k_pad, a_scales, w, out_dev, (int)count, m, nullptr);  // one launch for all
     }
     if (count == 1 || m <= 256) {  // few rows: the single products pick their own route (GEMV, split K)
         for (size_t i = 0; i < count; ++i) PG_TRY(pg_matmul_quantized_dev(ctx, a_dev, m, k, w[i], out_dev[i], nullptr));
