@@ -1042,7 +1042,7 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
         PG_TRY(pg_workspace(ctx, pg_mmdigits_bytes(m, w->k_in), &ws));
         const pg_mmdigits md = pg_mmdigits_carve(ws, m, w->k_in);
         PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, m, w->k_in, w->ggml_type, md));
-        return pg_launch_gguf_skinny(ctx, w->ggml_type, w->n_out, w->k_in, w->qs, w->d, m, md, y_dev);
+        return pg_launch_gguf_skinny_group(ctx, w->ggml_type, w->k_in, &w, &y_dev, 1, m, md);
     }
     const int ks = pg_gguf_mm_splitk(ctx, w->n_out, w->k_in, (m + 31) / 32, m, false, nullptr);
     const size_t sz_d = pg_mmdigits_bytes(m, w->k_in);

@@ -16,6 +16,7 @@
 // staged through LDS with direct global->LDS loads, two stages of 4 blocks ahead of the one
 // being consumed: each wavefront's own 32 weight rows and their f16 block scales, and the
 // token digits and scales of the stage, which the four wavefronts share.
+#include <limits.h>
 #include "pg_internal.h"
 #include "pg_digits.h"
 
@@ -531,18 +532,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // QT = 8 (Q8_0): a weight row is two streams (bytes 0 .. 15 and 16 .. 31 of its blocks, as the upload splits them), 32
 // streams a tile, kept in LDS half-major (stream slot 16 half + row) so that the fragment reads of 16 rows and one
 // half stay free of bank conflicts; no nibbles to unpack.
+// Up to three tensors of equal K in one launch (q|k|v, gate|up of models::llama): tensor g owns the workgroups
+// wg0[g] .. wg0[g + 1] - 1 (unused slots hold INT_MAX).
 template <int QT, int NB, int MT, int NW, int NST>
-__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void gguf_skinny_kernel(const uint8_t *__restrict__ qs, const uint16_t *__restrict__ dsc,
-                                                                    int n_out, int nb, int nbp, int m,
-                                                                    const int8_t *__restrict__ digits, const float *__restrict__ xs,
-                                                                    float *__restrict__ y) {
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void gguf_skinny_kernel(const pg_skinny_group grp, int nb, int nbp, int m,
+                                                                    const int8_t *__restrict__ digits, const float *__restrict__ xs) {
+    int tg = 0;
+#pragma unroll
+    for (int i = 1; i < 3; ++i) tg = (int)blockIdx.x >= grp.wg0[i] ? i : tg;
+    const uint8_t *__restrict__ qs = grp.qs[tg];
+    const uint16_t *__restrict__ dsc = grp.d[tg];
+    float *__restrict__ y = grp.y[tg];
+    const float *__restrict__ res = grp.res[tg];
+    const int n_out = grp.n[tg];
     constexpr int WF = QT == 8 ? 4 : 2, W_T = WF * 1024, D_T = 256, DIG = MT * 512, XS_B = 512, GQ = MT / 2;  // WF, GQ: weight, digit fills per unit
     constexpr int OFF_DS = NB * W_T, OFF_DG = OFF_DS + NB * D_T, OFF_X = OFF_DG + DIG, UNIT = OFF_X + XS_B;
     constexpr int LPS = WF * NB + 1 + GQ + 1;  // fills per unit
     static_assert((NST - 1) * LPS < 64 && NST <= 6 && NB <= 2, "the wait counter holds 63");
     extern __shared__ __attribute__((aligned(1024))) char lds[];  // NW rings of NST units; afterwards the wavefronts' tiles
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int n0 = blockIdx.x * 16 * NB;
+    const int n0 = ((int)blockIdx.x - grp.wg0[tg]) * 16 * NB;
     const int units = nb / 8, per = (units + NW - 1) / NW;
     const int u_begin = wave * per, u_end = u_begin + per < units ? u_begin + per : units;
     const int cnt = u_end - u_begin;
@@ -718,7 +727,10 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
         for (int w = 1; w < NW; ++w) sum += red[((w * NB + c) * 4 + i) * 64 + l];  // ascending runs of K
         const int tok = 4 * (l >> 4) + i, row = n0 + 16 * c + (l & 15);
-        if (tok < m && row < n_out) y[(size_t)tok * n_out + row] = QT == 4 ? sum * 0.0625f : sum;  // (Q4_0: the weight operand was 16 * (q - 8))
+        if (tok < m && row < n_out) {
+            const float v = QT == 4 ? sum * 0.0625f : sum;  // (Q4_0: the weight operand was 16 * (q - 8))
+            y[(size_t)tok * n_out + row] = res ? res[(size_t)tok * n_out + row] + v : v;
+        }
     }
 }
 
@@ -829,16 +841,34 @@ bool pg_gguf_skinny_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_o
            k_in % 256 == 0 && k_in >= 1024 && n_out >= 1 && n_out < (1u << 30) && k_in < (1u << 24);
 }
 
-pg_status pg_launch_gguf_skinny(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, size_t m,
-                                const pg_mmdigits &md, float *y) {
-    if (!pg_gguf_skinny_takes(ctx, ggml_type, m, n_out, k_in)) return pg_fail(PG_EINVAL, "gguf (few rows in one launch): [%zu x %zu] x %zu", m, k_in, n_out);
+pg_status pg_launch_gguf_skinny_group(pg_ctx *ctx, int ggml_type, size_t k_in, const pg_gguf_tensor *const *w, float *const *y, int count,
+                                      size_t m, const pg_mmdigits &md, const float *residual) {
+    if (count < 1 || count > 3) return pg_fail(PG_EINVAL, "gguf (few rows in one launch): %d tensors (1 .. 3)", count);
+    size_t n_total = 0;
+    for (int i = 0; i < count; ++i) {
+        if (w[i]->k_in != k_in || w[i]->ggml_type != ggml_type) return pg_fail(PG_EINVAL, "gguf (few rows in one launch): the tensors differ in K or type");
+        n_total += w[i]->n_out;
+    }
+    if (!pg_gguf_skinny_takes(ctx, ggml_type, m, n_total, k_in)) return pg_fail(PG_EINVAL, "gguf (few rows in one launch): [%zu x %zu] x %zu", m, k_in, n_total);
     const int nb = (int)(k_in / 32), nbp = (int)pg_round_up(nb, 4);
     const bool q8 = ggml_type == PG_GGML_Q8_0;
     // Wavefronts (runs of K) per workgroup: as many as keep every workgroup resident at once.  The rings: units of
     // 4.75 / 6.75 / 10.75 KiB for 4 / 8 / 16 token rows (Q8_0: 2 KiB more), as many stages as let eight wavefronts
     // share a CU's LDS (16 token rows: two stages and six or seven wavefronts; three stages and four were slower).
     const int per_cu = m <= 8 ? 8 : (q8 ? 6 : 7);
-    const dim3 grid((unsigned)((n_out + 15) / 16));
+    pg_skinny_group grp;
+    int wgs = 0;
+    for (int i = 0; i < 3; ++i) {
+        const bool used = i < count;
+        grp.qs[i] = used ? w[i]->qs : nullptr;
+        grp.d[i] = used ? w[i]->d : nullptr;
+        grp.y[i] = used ? y[i] : nullptr;
+        grp.res[i] = i == 0 ? residual : nullptr;
+        grp.n[i] = used ? (int)w[i]->n_out : 0;
+        grp.wg0[i] = used ? wgs : INT_MAX;
+        if (used) wgs += (int)((w[i]->n_out + 15) / 16);
+    }
+    const dim3 grid((unsigned)wgs);
     const size_t slots = (size_t)ctx->num_cu * per_cu, units = (size_t)nb / 8;
     int nw = m <= 8 ? 8 : 4;
     while (nw > 1 && ((size_t)grid.x * nw > slots || units / nw < 4)) nw >>= 1;
@@ -848,7 +878,7 @@ pg_status pg_launch_gguf_skinny(pg_ctx *ctx, int ggml_type, size_t n_out, size_t
         const size_t lds = (size_t)NWW * NSTT * ((QTT == 8 ? 4096 : 2048) + 256 + MTT * 512 + 512);                            \
         PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                            \
         return pg_launch(ctx, QTT == 8 ? "gguf_q8_0_few_rows_mm" : "gguf_q4_0_few_rows_mm", kern, grid, dim3(64 * NWW), lds,  \
-                         qs, d, (int)n_out, nb, nbp, (int)m, (const int8_t *)md.digits, (const float *)md.xs, y);              \
+                         grp, nb, nbp, (int)m, (const int8_t *)md.digits, (const float *)md.xs);                               \
     } while (0)
 #define PG_GSK_NW8(QTT, MTT, NSTT)                     \
     switch (nw) {                                      \

@@ -299,8 +299,16 @@ struct pg_mmdigits {
 size_t pg_mmdigits_bytes(size_t rows, size_t k);
 pg_mmdigits pg_mmdigits_carve(void *base, size_t rows, size_t k);
 bool pg_gguf_skinny_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_out, size_t k_in);
-pg_status pg_launch_gguf_skinny(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, size_t m,
-                                const pg_mmdigits &md, float *y);
+struct pg_skinny_group {  // the tensors of one few-rows launch (gguf_skinny_kernel)
+    const uint8_t *qs[3];
+    const uint16_t *d[3];
+    float *y[3];
+    const float *res[3];  // where set: y = res + product (same shape as y)
+    int n[3];
+    int wg0[3];
+};
+pg_status pg_launch_gguf_skinny_group(pg_ctx *ctx, int ggml_type, size_t k_in, const pg_gguf_tensor *const *w, float *const *y, int count,
+                                      size_t m, const pg_mmdigits &md, const float *residual = nullptr);  // residual: added to tensor 0's product
 pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows, size_t k, int ggml_type,
                                    const pg_mmdigits &md);
 // Q4_1 on the matrix-core route: the product is the Q4_0 product on the same nibbles and scales plus

@@ -2112,12 +2112,16 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     const size_t n_of[7] = {q_dim, kv_dim, kv_dim, d, ffn, ffn, d}, k_of[7] = {d, d, d, q_dim, d, d, ffn};
     // q|k|v and gate|up are one launch each (the tensors' 128-row groups one after the other): one K split for the launch
     const int first_of[7] = {0, 0, 0, 3, 4, 4, 6}, count_of[7] = {3, 3, 3, 1, 2, 2, 1};
+    // Up to eight tokens: the few-rows product (one launch per tensor group, no K split between workgroups, so every
+    // product leaves one plane; the weights are read in their row-major planes, no tile-major copy).
+    bool few = seq <= 8;
+    for (int i = 0; i < 7 && few; ++i) few = pg_gguf_skinny_takes(ctx, type, seq, n_of[i], k_of[i]);
     int ks[7];
     size_t part_off[7], floats = 0;
     for (int i = 0; i < 7; ++i) {
         size_t groups = 0;
         for (int j = first_of[i]; j < first_of[i] + count_of[i]; ++j) groups += (n_of[j] + 127) / 128;
-        ks[i] = pg_gguf_mm_splitk(ctx, groups * 128, k_of[i], tiles, seq, false, nullptr);
+        ks[i] = few ? 1 : pg_gguf_mm_splitk(ctx, groups * 128, k_of[i], tiles, seq, false, nullptr);
         if (ks[i] > PG_MAX_PLANES) return pg_fail(PG_EUNSUPPORTED, "llama block: a product in %d K chunks", ks[i]);
         part_off[i] = floats;
         floats += pg_round_up((size_t)ks[i] * seq * n_of[i], 64);
@@ -2141,6 +2145,10 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     pg_mm_group grp = {1, nullptr, nullptr, nullptr, nullptr, 0, (int)tiles, (int)seq, 1};
     grp.tiled = 1;
     auto product = [&](int i, const pg_mmdigits &md) -> pg_status {  // tensors i .. i + count_of[i] - 1
+        if (few) {
+            float *ys[3] = {part(i), count_of[i] > 1 ? part(i + 1) : nullptr, count_of[i] > 2 ? part(i + 2) : nullptr};
+            return pg_launch_gguf_skinny_group(ctx, type, k_of[i], b->w + i, ys, count_of[i], seq, md);
+        }
         pg_mm_group g = grp;
         size_t groups = 0;
         g.nseg = count_of[i] > 1 ? count_of[i] : 0;
@@ -2186,6 +2194,10 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
         PG_TRY(pg_launch(ctx, "swiglu_mm_digits", kern, dim3((unsigned)((nbf + 31) / 32), (unsigned)seq), dim3(256), 0,
                          (const float *)part(4), (const float *)part(5), ks[4], seq * ffn, nbf, (int)pg_round_up(nbf, 4),
                          md_f.digits, md_f.xs));
+    }
+    if (few) {  // the down product adds the residual itself
+        float *ys[1] = {out_dev};
+        return pg_launch_gguf_skinny_group(ctx, type, k_of[6], b->w + 6, ys, 1, seq, md_f, h1);
     }
     PG_TRY(product(6, md_f));
     return pg_launch(ctx, "residual_add", add_planes_kernel, dim3(blocks_for(seq * d)), dim3(256), 0, (const float *)h1,
