@@ -2114,14 +2114,18 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     const int first_of[7] = {0, 0, 0, 3, 4, 4, 6}, count_of[7] = {3, 3, 3, 1, 2, 2, 1};
     // Up to eight tokens: the few-rows product (one launch per tensor group, no K split between workgroups, so every
     // product leaves one plane; the weights are read in their row-major planes, no tile-major copy).
-    bool few = seq <= 8;
-    for (int i = 0; i < 7 && few; ++i) few = pg_gguf_skinny_takes(ctx, type, seq, n_of[i], k_of[i]);
+    // (Nine to sixteen tokens: only the products over fewer than 32 weight rows per CU, see pg_gguf_skinny_takes.)
+    bool few[7];
     int ks[7];
     size_t part_off[7], floats = 0;
     for (int i = 0; i < 7; ++i) {
-        size_t groups = 0;
-        for (int j = first_of[i]; j < first_of[i] + count_of[i]; ++j) groups += (n_of[j] + 127) / 128;
-        ks[i] = few ? 1 : pg_gguf_mm_splitk(ctx, groups * 128, k_of[i], tiles, seq, false, nullptr);
+        size_t groups = 0, rows = 0;
+        for (int j = first_of[i]; j < first_of[i] + count_of[i]; ++j) {
+            groups += (n_of[j] + 127) / 128;
+            rows += n_of[j];
+        }
+        few[i] = pg_gguf_skinny_takes(ctx, type, seq, rows, k_of[i]);
+        ks[i] = few[i] ? 1 : pg_gguf_mm_splitk(ctx, groups * 128, k_of[i], tiles, seq, false, nullptr);
         if (ks[i] > PG_MAX_PLANES) return pg_fail(PG_EUNSUPPORTED, "llama block: a product in %d K chunks", ks[i]);
         part_off[i] = floats;
         floats += pg_round_up((size_t)ks[i] * seq * n_of[i], 64);
@@ -2145,7 +2149,7 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     pg_mm_group grp = {1, nullptr, nullptr, nullptr, nullptr, 0, (int)tiles, (int)seq, 1};
     grp.tiled = 1;
     auto product = [&](int i, const pg_mmdigits &md) -> pg_status {  // tensors i .. i + count_of[i] - 1
-        if (few) {
+        if (few[i]) {
             float *ys[3] = {part(i), count_of[i] > 1 ? part(i + 1) : nullptr, count_of[i] > 2 ? part(i + 2) : nullptr};
             return pg_launch_gguf_skinny_group(ctx, type, k_of[i], b->w + i, ys, count_of[i], seq, md);
         }
@@ -2195,7 +2199,7 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
                          (const float *)part(4), (const float *)part(5), ks[4], seq * ffn, nbf, (int)pg_round_up(nbf, 4),
                          md_f.digits, md_f.xs));
     }
-    if (few) {  // the down product adds the residual itself
+    if (few[6]) {  // the down product adds the residual itself
         float *ys[1] = {out_dev};
         return pg_launch_gguf_skinny_group(ctx, type, k_of[6], b->w + 6, ys, 1, seq, md_f, h1);
     }
