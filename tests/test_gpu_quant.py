@@ -152,7 +152,7 @@ MATMUL_SHAPES = [
     (2, 4096, 1024), (3, 1000, 77), (4, 4096, 300),    # GEMV with m = 2..4, ragged k and n
     (32, 4096, 4096),                                  # benchmark configuration 1
     (5, 96, 40), (64, 200, 130), (65, 384, 129),       # 64x64 and 128x128 tiles, ragged
-    (196, 768, 3072),                                  # benches/wallclock.rs:758-786
+    (196, 768, 3072), (196, 1024, 4096),               # benches/wallclock.rs:758-786
     (300, 512, 1000),                                  # 128x128 tiles, ragged m and n
     (2048, 128, 4096),                                 # 128x256 tiles
     (2050, 192, 4100),                                 # 128x256 tiles, ragged m and n
@@ -380,9 +380,10 @@ def run_multi(ctx, da, m, k, qts, douts):
 
 @pytest.mark.parametrize("m,k,ns", [(300, 512, (1000, 130, 257)), (257, 128, (64, 64, 64, 64)), (40, 1024, (300, 77)),
                                      (1, 4096, (1024, 512)), (1, 14336, (300, 77, 4096)), (3, 200, (33,)), (2048, 4096, (4096, 1024, 1024)),
-                                     (2048, 4096, (14336, 14336)), (8, 4096, (4096, 1024, 1030)), (32, 1000, (8200, 520))],
+                                     (2048, 4096, (14336, 14336)), (8, 4096, (4096, 1024, 1030)), (32, 1000, (8200, 520)),
+                                     (1, 4096, (14336, 14336))],
                          ids=["ragged3", "four", "few-rows", "one-row", "one-row-long-k", "single", "qkv", "gate-up",
-                              "qkv-8-rows-quantised-once", "32-rows-quantised-once"])
+                              "qkv-8-rows-quantised-once", "32-rows-quantised-once", "one-row-gate-up-as-the-decode-benchmark-runs-it"])
 def test_matmul_quantized_multi_equals_the_single_products(ctx, orc, m, k, ns):
     """Several weights against one activation matrix (the reference's fused QKV / gate|up
     products): every output equals the single product bit for bit, and sampled rows equal the
