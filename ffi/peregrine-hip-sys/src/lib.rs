@@ -50,13 +50,6 @@ extern "C" {
     pub fn pg_ctx_stream(ctx: *mut pg_ctx) -> *mut c_void;
     pub fn pg_last_error() -> *const c_char;
     pub fn pg_status_string(st: pg_status) -> *const c_char;
-    pub fn pg_profile_begin(ctx: *mut pg_ctx) -> pg_status;
-    pub fn pg_profile_end(ctx: *mut pg_ctx, num_kernels: *mut usize) -> pg_status;
-    pub fn pg_profile_get(ctx: *mut pg_ctx, i: usize, name: *mut *const c_char, total_ms: *mut f64, launches: *mut usize) -> pg_status;
-    pub fn pg_profile_get_grids(ctx: *mut pg_ctx, i: usize, work_items: *mut usize, launches: *mut usize, cap: usize, count: *mut usize) -> pg_status;
-    pub fn pg_probe_mfma_i8(ctx: *mut pg_ctx, iters: c_int, tops: *mut f64, clock_ghz: *mut f64) -> pg_status;
-    pub fn pg_probe_hbm_read(ctx: *mut pg_ctx, bytes_per_pass: usize, buffers: c_int, passes: c_int, gbs: *mut f64) -> pg_status;
-    pub fn pg_probe_gemm_clock(ctx: *mut pg_ctx, m: usize, k: usize, n: usize, clock_ghz: *mut f64, loop_us: *mut f64) -> pg_status;
     pub fn pg_dev_alloc(ctx: *mut pg_ctx, bytes: usize, dptr: *mut *mut c_void) -> pg_status;
     pub fn pg_dev_free(ctx: *mut pg_ctx, dptr: *mut c_void) -> pg_status;
     pub fn pg_memcpy_h2d(ctx: *mut pg_ctx, dst_dev: *mut c_void, src_host: *const c_void, bytes: usize) -> pg_status;
@@ -76,8 +69,6 @@ extern "C" {
     pub fn pg_matmul_quantized_fixed_scratch_dev(ctx: *mut pg_ctx, a_dev: *const f32, m: usize, k: usize, w: *const pg_qtensor, out_dev: *mut f32) -> pg_status;
     pub fn pg_fixed_scratch_bytes() -> usize;
     pub fn pg_matmul_quantized_multi_dev(ctx: *mut pg_ctx, a_dev: *const f32, m: usize, k: usize, w: *const *const pg_qtensor, count: usize, out_dev: *const *mut f32) -> pg_status;
-    pub fn pg_gemm_w8a8_last_tile(ctx: *const pg_ctx, bm: *mut c_int, bn: *mut c_int, k_splits: *mut c_int) -> pg_status;
-    pub fn pg_gemm_w8a8_force_tile(ctx: *mut pg_ctx, tile: c_int) -> pg_status;
     pub fn pg_matmul_dequant_i8(ctx: *mut pg_ctx, a: *const f32, m: usize, k: usize, w: *const pg_qtensor, out: *mut f32) -> pg_status;
     pub fn pg_matmul_dequant_i8_dev(ctx: *mut pg_ctx, a_dev: *const f32, m: usize, k: usize, w: *const pg_qtensor, out_dev: *mut f32) -> pg_status;
     pub fn pg_f16_to_f32(ctx: *mut pg_ctx, bits: *const u16, n: usize, out: *mut f32) -> pg_status;
@@ -89,6 +80,9 @@ extern "C" {
     pub fn pg_gguf_free(ctx: *mut pg_ctx, t: *mut pg_gguf_tensor);
     pub fn pg_gguf_matmul(ctx: *mut pg_ctx, x: *const f32, m: usize, w: *const pg_gguf_tensor, y: *mut f32) -> pg_status;
     pub fn pg_gguf_matmul_dev(ctx: *mut pg_ctx, x_dev: *const f32, m: usize, w: *const pg_gguf_tensor, y_dev: *mut f32) -> pg_status;
+    pub fn pg_gguf_prepare(ctx: *mut pg_ctx, w: *const pg_gguf_tensor, max_rows: usize) -> pg_status;
+    pub fn pg_gguf_drop_prepared(ctx: *mut pg_ctx, w: *const pg_gguf_tensor) -> pg_status;
+    pub fn pg_gguf_device_bytes(w: *const pg_gguf_tensor, uploaded: *mut usize, derived: *mut usize) -> pg_status;
     pub fn pg_mxfp4_matmul(ctx: *mut pg_ctx, input: *const f32, blocks: *const u8, scales: *const u8, out_dim: usize, in_dim: usize, output: *mut f32) -> pg_status;
     pub fn pg_mxfp4_upload(ctx: *mut pg_ctx, blocks: *const u8, scales: *const u8, out_dim: usize, in_dim: usize, out: *mut *mut pg_gguf_tensor) -> pg_status;
     pub fn pg_mxfp4_expert_create(ctx: *mut pg_ctx, hidden: usize, intermediate: usize, alpha: f32, clamp: f32, mlp1_blocks: *const u8, mlp1_scales: *const u8, mlp2_blocks: *const u8, mlp2_scales: *const u8, mlp1_bias: *const f32, mlp2_bias: *const f32, out: *mut *mut pg_mxfp4_expert) -> pg_status;
@@ -128,6 +122,8 @@ extern "C" {
     pub fn pg_matmul_huffman(ctx: *mut pg_ctx, a: *const f32, m: usize, k: usize, t: *const pg_huffman_tensor, out: *mut f32) -> pg_status;
     pub fn pg_moe_ffn(ctx: *mut pg_ctx, x: *const f32, T: usize, router_logits: *const f32, E: usize, top_k: usize, gate: *const *const pg_gguf_tensor, up: *const *const pg_gguf_tensor, down: *const *const pg_gguf_tensor, act: c_int, out: *mut f32) -> pg_status;
     pub fn pg_moe_ffn_dev(ctx: *mut pg_ctx, x_dev: *const f32, T: usize, router_logits_dev: *const f32, E: usize, top_k: usize, gate: *const *const pg_gguf_tensor, up: *const *const pg_gguf_tensor, down: *const *const pg_gguf_tensor, act: c_int, out_dev: *mut f32) -> pg_status;
+    pub fn pg_moe_ffn_routed(ctx: *mut pg_ctx, x: *const f32, T: usize, expert_idx: *const i32, weight: *const f32, E: usize, top_k: usize, gate: *const *const pg_gguf_tensor, up: *const *const pg_gguf_tensor, down: *const *const pg_gguf_tensor, act: c_int, shared: *const f32, out: *mut f32) -> pg_status;
+    pub fn pg_moe_ffn_routed_dev(ctx: *mut pg_ctx, x_dev: *const f32, T: usize, expert_idx_dev: *const i32, weight_dev: *const f32, E: usize, top_k: usize, gate: *const *const pg_gguf_tensor, up: *const *const pg_gguf_tensor, down: *const *const pg_gguf_tensor, act: c_int, shared_dev: *const f32, out_dev: *mut f32) -> pg_status;
     pub fn pg_rmsnorm(ctx: *mut pg_ctx, x: *const f32, rows: usize, dim: usize, w: *const f32, eps: f32, out: *mut f32) -> pg_status;
     pub fn pg_rmsnorm_dev(ctx: *mut pg_ctx, x_dev: *const f32, rows: usize, dim: usize, w_dev: *const f32, eps: f32, out_dev: *mut f32) -> pg_status;
     pub fn pg_rope_create(ctx: *mut pg_ctx, head_dim: usize, max_seq_len: usize, base: f32, out: *mut *mut pg_rope) -> pg_status;
@@ -151,6 +147,15 @@ extern "C" {
     pub fn pg_llama_block_set_weights(ctx: *mut pg_ctx, block: *mut pg_llama_block, q_proj: *const pg_gguf_tensor, k_proj: *const pg_gguf_tensor, v_proj: *const pg_gguf_tensor, o_proj: *const pg_gguf_tensor, gate_proj: *const pg_gguf_tensor, up_proj: *const pg_gguf_tensor, down_proj: *const pg_gguf_tensor, attn_norm_w: *const f32, ffn_norm_w: *const f32) -> pg_status;
     pub fn pg_llama_block_forward(ctx: *mut pg_ctx, block: *mut pg_llama_block, h: *const f32, seq: usize, cache: *mut pg_kv_cache, out: *mut f32) -> pg_status;
     pub fn pg_llama_block_forward_dev(ctx: *mut pg_ctx, block: *mut pg_llama_block, h_dev: *const f32, seq: usize, cache: *mut pg_kv_cache, out_dev: *mut f32) -> pg_status;
+    pub fn pg_profile_begin(ctx: *mut pg_ctx) -> pg_status;
+    pub fn pg_profile_end(ctx: *mut pg_ctx, num_kernels: *mut usize) -> pg_status;
+    pub fn pg_profile_get(ctx: *mut pg_ctx, i: usize, name: *mut *const c_char, total_ms: *mut f64, launches: *mut usize) -> pg_status;
+    pub fn pg_profile_get_grids(ctx: *mut pg_ctx, i: usize, work_items: *mut usize, launches: *mut usize, cap: usize, count: *mut usize) -> pg_status;
+    pub fn pg_probe_mfma_i8(ctx: *mut pg_ctx, iters: c_int, tops: *mut f64, clock_ghz: *mut f64) -> pg_status;
+    pub fn pg_probe_hbm_read(ctx: *mut pg_ctx, bytes_per_pass: usize, buffers: c_int, passes: c_int, gbs: *mut f64) -> pg_status;
+    pub fn pg_probe_gemm_clock(ctx: *mut pg_ctx, m: usize, k: usize, n: usize, clock_ghz: *mut f64, loop_us: *mut f64) -> pg_status;
+    pub fn pg_gemm_w8a8_last_tile(ctx: *const pg_ctx, bm: *mut c_int, bn: *mut c_int, k_splits: *mut c_int) -> pg_status;
+    pub fn pg_gemm_w8a8_force_tile(ctx: *mut pg_ctx, tile: c_int) -> pg_status;
 }
 // ---- generated: end ----
 
@@ -183,6 +188,16 @@ pub fn sync() {
     ok(unsafe { pg_sync(ctx()) });
 }
 
+/// Stands where the reference's functions take `&GpuContext` (src/quant.rs:174,183,196-197): the
+/// device context itself is the calling thread's (`ctx()`), so the value carries nothing.
+pub struct GpuContext;
+impl GpuContext {
+    /// `gpu.sync()`  tests/quant_parity.rs:104.
+    pub fn sync(&self) {
+        sync();
+    }
+}
+
 /// `peregrine::quant` (src/quant.rs) over the library.
 pub mod quant {
     use super::*;
@@ -203,28 +218,35 @@ pub mod quant {
         pub scales: Vec<f32>,
         pub rows: usize,
         pub cols: usize,
-        pub hip: Option<HipQTensor>,
+        /// The device copy, made once.  A cell, because `matmul_quantized` takes `&QuantizedTensor`
+        /// (src/quant.rs:133) and still has to place the weights on the device on first use; the
+        /// reference's callers are single-threaded per tensor (src/tensor.rs:864), so is this.
+        pub hip: std::cell::OnceCell<HipQTensor>,
     }
 
     impl QuantizedTensor {
-        /// `QuantizedTensor::to_gpu`  src/quant.rs:174-181 (idempotent).
-        pub fn to_gpu(&mut self) {
-            if self.hip.is_none() {
+        fn upload(&self) -> *const pg_qtensor {
+            self.hip.get_or_init(|| {
                 let mut h = std::ptr::null_mut();
                 ok(unsafe { pg_qtensor_upload(ctx(), self.data_i8.as_ptr(), self.scales.as_ptr(), self.rows, self.cols, &mut h) });
-                self.hip = Some(HipQTensor(h));
-            }
+                HipQTensor(h)
+            }).0
+        }
+
+        /// `QuantizedTensor::to_gpu`  src/quant.rs:174-181 (idempotent).
+        pub fn to_gpu(&mut self, _gpu: &GpuContext) {
+            self.upload();
         }
 
         /// `QuantizedTensor::from_gpu`  src/quant.rs:183-190.
-        pub fn from_gpu(&mut self) {
-            if let Some(ref h) = self.hip {
+        pub fn from_gpu(&mut self, _gpu: &GpuContext) {
+            if let Some(h) = self.hip.get() {
                 ok(unsafe { pg_qtensor_download(ctx(), h.0, self.data_i8.as_mut_ptr(), self.data_i8_t.as_mut_ptr(), self.scales.as_mut_ptr()) });
             }
         }
 
         fn handle(&self) -> *const pg_qtensor {
-            self.hip.as_ref().expect("weights not on GPU").0 // src/quant.rs:208
+            self.hip.get().expect("weights not on GPU").0 // src/quant.rs:208
         }
     }
 
@@ -233,7 +255,7 @@ pub mod quant {
         assert_eq!(data.len(), rows * cols);
         let (mut q, mut q_t, mut s) = (vec![0i8; rows * cols], vec![0i8; rows * cols], vec![0f32; cols]);
         ok(unsafe { pg_quantize_weights(ctx(), data.as_ptr(), rows, cols, q.as_mut_ptr(), q_t.as_mut_ptr(), s.as_mut_ptr()) });
-        QuantizedTensor { data_i8: q, data_i8_t: q_t, scales: s, rows, cols, hip: None }
+        QuantizedTensor { data_i8: q, data_i8_t: q_t, scales: s, rows, cols, hip: std::cell::OnceCell::new() }
     }
 
     /// `quant::quantize_activations`  src/quant.rs:79-112.
@@ -253,29 +275,30 @@ pub mod quant {
 
     /// `quant::matmul_quantized`  src/quant.rs:129-169.  The weights go to the device on first
     /// use and stay there (the reference's CPU path has no such state; the result is the same).
-    pub fn matmul_quantized(a: &[f32], m: usize, k: usize, w: &mut QuantizedTensor) -> Vec<f32> {
+    pub fn matmul_quantized(a_data: &[f32], m: usize, k: usize, w: &QuantizedTensor) -> Vec<f32> {
         assert_eq!(w.rows, k);
-        assert_eq!(a.len(), m * k);
-        w.to_gpu();
+        assert_eq!(a_data.len(), m * k);
+        let h = w.upload();
         let mut out = vec![0f32; m * w.cols];
-        ok(unsafe { pg_matmul_quantized(ctx(), a.as_ptr(), m, k, w.handle(), out.as_mut_ptr()) });
+        ok(unsafe { pg_matmul_quantized(ctx(), a_data.as_ptr(), m, k, h, out.as_mut_ptr()) });
         out
     }
 
-    /// An unsynced device buffer of f32, the `GpuBuffer<f32>` that `matmul_quantized_gpu` returns.
-    pub struct DeviceBuffer {
-        pub ptr: *mut f32,
+    /// An unsynced device buffer, the `GpuBuffer<T>` that `matmul_quantized_gpu` returns
+    /// (src/quant.rs:202; only `GpuBuffer<f32>` is ever made here).
+    pub struct GpuBuffer<T> {
+        pub ptr: *mut T,
         pub len: usize,
     }
-    impl DeviceBuffer {
+    impl<T: Copy + Default> GpuBuffer<T> {
         /// `GpuBuffer::read` (after `sync()`).
-        pub fn read(&self) -> Vec<f32> {
-            let mut v = vec![0f32; self.len];
-            ok(unsafe { pg_memcpy_d2h(ctx(), v.as_mut_ptr() as *mut c_void, self.ptr as *const c_void, self.len * 4) });
+        pub fn read(&self) -> Vec<T> {
+            let mut v = vec![T::default(); self.len];
+            ok(unsafe { pg_memcpy_d2h(ctx(), v.as_mut_ptr() as *mut c_void, self.ptr as *const c_void, self.len * std::mem::size_of::<T>()) });
             v
         }
     }
-    impl Drop for DeviceBuffer {
+    impl<T> Drop for GpuBuffer<T> {
         fn drop(&mut self) {
             unsafe { pg_dev_free(ctx(), self.ptr as *mut c_void) };
         }
@@ -284,7 +307,7 @@ pub mod quant {
     /// `quant::matmul_quantized_gpu`  src/quant.rs:196-218: uploads `a`, enqueues the product,
     /// returns without waiting.  Numerics are the CPU path's W8A8; `matmul_dequant_i8_gpu` gives
     /// the Metal shader's W8A32.
-    pub fn matmul_quantized_gpu(a_data: &[f32], m: usize, k: usize, w: &QuantizedTensor) -> DeviceBuffer {
+    pub fn matmul_quantized_gpu(_gpu: &GpuContext, a_data: &[f32], m: usize, k: usize, w: &QuantizedTensor) -> GpuBuffer<f32> {
         assert_eq!(w.rows, k);
         assert_eq!(a_data.len(), m * k);
         let h = w.handle();
@@ -293,19 +316,19 @@ pub mod quant {
         ok(unsafe { pg_dev_alloc(ctx(), m * w.cols * 4, &mut out_dev) });
         ok(unsafe { pg_memcpy_h2d(ctx(), a_dev, a_data.as_ptr() as *const c_void, m * k * 4) });
         ok(unsafe { pg_matmul_quantized_dev(ctx(), a_dev as *const f32, m, k, h, out_dev as *mut f32, std::ptr::null_mut()) });
-        let out = DeviceBuffer { ptr: out_dev as *mut f32, len: m * w.cols };
-        drop(DeviceBuffer { ptr: a_dev as *mut f32, len: 0 }); // pg_dev_free waits for the stream first
+        let out = GpuBuffer { ptr: out_dev as *mut f32, len: m * w.cols };
+        drop(GpuBuffer { ptr: a_dev as *mut f32, len: 0 }); // pg_dev_free waits for the stream first
         out
     }
 
     /// The Metal shader's numerics for the same call (`matmul_dequant_i8`,
     /// src/metal/shaders.rs:2329-2375): f32 activations, dequantised weights, f32 accumulate.
-    pub fn matmul_dequant_i8(a: &[f32], m: usize, k: usize, w: &mut QuantizedTensor) -> Vec<f32> {
+    pub fn matmul_dequant_i8(a_data: &[f32], m: usize, k: usize, w: &QuantizedTensor) -> Vec<f32> {
         assert_eq!(w.rows, k);
-        assert_eq!(a.len(), m * k);
-        w.to_gpu();
+        assert_eq!(a_data.len(), m * k);
+        let h = w.upload();
         let mut out = vec![0f32; m * w.cols];
-        ok(unsafe { pg_matmul_dequant_i8(ctx(), a.as_ptr(), m, k, w.handle(), out.as_mut_ptr()) });
+        ok(unsafe { pg_matmul_dequant_i8(ctx(), a_data.as_ptr(), m, k, h, out.as_mut_ptr()) });
         out
     }
 }
@@ -345,8 +368,13 @@ pub mod gguf {
         out
     }
 
-    /// `gguf::f16_to_f32`  src/gguf.rs:354-382 on a slice.
-    pub fn f16_to_f32(bits: &[u16]) -> Vec<f32> {
+    /// `gguf::f16_to_f32`  src/gguf.rs:354-382 (one value; `f16_to_f32_slice` converts many at once).
+    pub fn f16_to_f32(bits: u16) -> f32 {
+        f16_to_f32_slice(&[bits])[0]
+    }
+
+    /// The same conversion over a slice in one call.
+    pub fn f16_to_f32_slice(bits: &[u16]) -> Vec<f32> {
         let mut out = vec![0f32; bits.len()];
         ok(unsafe { pg_f16_to_f32(ctx(), bits.as_ptr(), bits.len(), out.as_mut_ptr()) });
         out
@@ -367,6 +395,11 @@ pub mod gguf {
             let mut h = std::ptr::null_mut();
             ok(unsafe { pg_gguf_upload(ctx(), blocks.as_ptr() as *const c_void, ggml_type, n_out, k_in, &mut h) });
             GgufWeight(h, n_out, k_in)
+        }
+        /// The load-time step: the derived device copies that products over up to `max_rows` rows need are
+        /// made now, so that those products neither allocate nor wait.
+        pub fn prepare(&self, max_rows: usize) {
+            ok(unsafe { pg_gguf_prepare(ctx(), self.0, max_rows) });
         }
         /// y [m, n_out] = x [m, k_in] . dequant(w)^T  (src/tensor.rs:1342-1353 on the transposed weight).
         pub fn matmul(&self, x: &[f32], m: usize) -> Vec<f32> {

@@ -71,37 +71,6 @@ void *pg_ctx_stream(pg_ctx *ctx);
 const char *pg_last_error(void);
 const char *pg_status_string(pg_status st);
 
-/* Per-kernel timing.  No counterpart in the reference (it times whole calls with
- * Instant::now(), benches/wallclock.rs:28-41): between pg_profile_begin and
- * pg_profile_end every hot-path kernel the library launches on this context carries a
- * start and a stop HIP event stamped with the dispatch's own begin and end times
- * (hipExtLaunchKernel) on the context's stream; pg_profile_end waits for the stream and
- * aggregates elapsed time per kernel name, read back with pg_profile_get. */
-pg_status pg_profile_begin(pg_ctx *ctx);
-pg_status pg_profile_end(pg_ctx *ctx, size_t *num_kernels);
-pg_status pg_profile_get(pg_ctx *ctx, size_t i, const char **name, double *total_ms,
-                         size_t *launches);
-/* The distinct launch sizes (work-items = grid x workgroup, as a kernel trace lists them) behind
- * entry i and how many launches had each: up to `cap` pairs are written, *count gets their number.
- * Lets a benchmark check that a stored counter summary still describes the launches it makes. */
-pg_status pg_profile_get_grids(pg_ctx *ctx, size_t i, size_t *work_items, size_t *launches, size_t cap,
-                               size_t *count);
-
-/* Ceilings of the part, measured (no counterpart in the reference; a benchmark reports them
- * beside the published peaks):
- *   pg_probe_mfma_i8    int8 matrix-core rate with every operand in registers, in TOP/s (2 ops
- *                       per multiply-add), one workgroup of 8 wavefronts per CU for `iters` x 8
- *                       MFMAs per wavefront, and the shader clock the loop ran at;
- *   pg_probe_hbm_read   a pure 128-bit read stream: `passes` kernels, each reading
- *                       bytes_per_pass from one of `buffers` distinct buffers in turn (make
- *                       buffers x bytes_per_pass exceed the 256 MB last-level cache), in GB/s;
- *   pg_probe_gemm_clock the shader clock inside the K loop of the W8A8 GEMM's 256x256 tile on an
- *                       [m x k] . [k x n] product, and the mean duration of a workgroup's loop.
- * Each allocates its own buffers and waits for completion. */
-pg_status pg_probe_mfma_i8(pg_ctx *ctx, int iters, double *tops, double *clock_ghz);
-pg_status pg_probe_hbm_read(pg_ctx *ctx, size_t bytes_per_pass, int buffers, int passes, double *gbs);
-pg_status pg_probe_gemm_clock(pg_ctx *ctx, size_t m, size_t k, size_t n, double *clock_ghz, double *loop_us);
-
 /* Device memory for callers that have no HIP binding of their own
  * (GpuContext::alloc / upload / GpuBuffer::read, src/metal/buffer.rs). */
 pg_status pg_dev_alloc(pg_ctx *ctx, size_t bytes, void **dptr);
@@ -180,15 +149,6 @@ pg_status pg_matmul_quantized_multi_dev(pg_ctx *ctx, const float *a_dev, size_t 
                                         const pg_qtensor *const *w, size_t count,
                                         float *const *out_dev);
 
-/* Diagnostics of the matrix-core product.  No counterpart in the reference (its Metal
- * dispatcher picks between two shaders by size, src/metal/context.rs:2243, without a query):
- * the output tile (rows x columns) and the number of K splits of the most recent W8A8 GEMM
- * launch on this context, and an override of the dispatcher's tile choice (0 = automatic,
- * 1 = 64x64, 2 = 256x256, 3 = 128x256, 4 = 128x64, 5 = 128x128).  Every tile gives the same
- * bits; tests use the pair to prove each kernel instantiation ran. */
-pg_status pg_gemm_w8a8_last_tile(const pg_ctx *ctx, int *bm, int *bn, int *k_splits);
-pg_status pg_gemm_w8a8_force_tile(pg_ctx *ctx, int tile);
-
 /* The reference's GPU numerics for the same call (W8A32): f32 activations, weights
  * dequantised to f32, f32 accumulate, no activation quantisation --
  * GpuContext::dispatch_matmul_dequant_i8  src/metal/context.rs:2226-2306, shader
@@ -232,6 +192,21 @@ pg_status pg_gguf_matmul(pg_ctx *ctx, const float *x, size_t m, const pg_gguf_te
                          float *y);
 pg_status pg_gguf_matmul_dev(pg_ctx *ctx, const float *x_dev, size_t m,
                              const pg_gguf_tensor *w, float *y_dev);
+
+/* Load-time preparation.  The matrix-core block product reads a tile-major copy of a Q4_0 / Q8_0 / Q4_1 tensor's
+ * payload plane (as many bytes again as the payload), and an MXFP4 tensor's products over 16 rows or more (24 for
+ * tensors under 2^25 weights) go through a Q8_0 twin of the tensor (34 bytes per block, plus the twin's own
+ * tile-major copy of 32: about five times the 17 bytes per block as uploaded).  Left alone, the first product that
+ * needs such a copy makes it: a hipMalloc, a launch and a wait inside a call that is otherwise stream-ordered and
+ * allocation-free.  pg_gguf_prepare makes now whatever products over up to `max_rows` activation rows of this
+ * tensor (alone, in a group, inside a Llama block or as an expert of pg_moe_ffn) will need, as the reference
+ * rearranges weights at load (load_transposed_weight, src/models/llama/model.rs:243-257); afterwards those calls
+ * neither allocate nor wait, which a caller that captures them in a HIP graph requires.  max_rows < 2 makes
+ * nothing (one-row products read the planes as uploaded).  pg_gguf_drop_prepared frees the copies again (it waits
+ * for the stream); pg_gguf_device_bytes reports what the tensor holds. */
+pg_status pg_gguf_prepare(pg_ctx *ctx, const pg_gguf_tensor *w, size_t max_rows);
+pg_status pg_gguf_drop_prepared(pg_ctx *ctx, const pg_gguf_tensor *w);
+pg_status pg_gguf_device_bytes(const pg_gguf_tensor *w, size_t *uploaded, size_t *derived);
 
 /* ---- MXFP4 (the gpt_oss experts' format) ------------------------------------------ */
 
@@ -381,6 +356,24 @@ pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
                          const pg_gguf_tensor *const *gate, const pg_gguf_tensor *const *up,
                          const pg_gguf_tensor *const *down, int act, float *out_dev);
 
+/* The same expert FFN over a routing the caller's gate made: expert_idx / weight [T, top_k] (a token's experts
+ * distinct, each in 0 .. E - 1), out[t] = sum_k weight[t, k] * expert_{idx[t, k]}(x[t]) in k order, multiply then
+ * add, then + shared[t] when `shared` ([T, d], the shared experts' output) is not NULL --
+ * MoE::forward  examples/deepseek/moe.rs:271-300 after Gate::forward (:111-215: sigmoid or softmax scores, bias and
+ * group limits for the selection only, route_scale), and the gpt_oss layer (examples/gpt_oss/moe.rs:286-351: top-k
+ * on the logits, softmax over the k).  The host-pointer form rejects an index out of range or named twice
+ * (PG_EINVAL; the reference would panic on the first); the device form cannot look, and replaces such an entry by
+ * an unused expert with weight 0, so that it stays memory-safe. */
+pg_status pg_moe_ffn_routed(pg_ctx *ctx, const float *x, size_t T, const int32_t *expert_idx, const float *weight,
+                            size_t E, size_t top_k, const pg_gguf_tensor *const *gate,
+                            const pg_gguf_tensor *const *up, const pg_gguf_tensor *const *down, int act,
+                            const float *shared, float *out);
+pg_status pg_moe_ffn_routed_dev(pg_ctx *ctx, const float *x_dev, size_t T, const int32_t *expert_idx_dev,
+                                const float *weight_dev, size_t E, size_t top_k,
+                                const pg_gguf_tensor *const *gate, const pg_gguf_tensor *const *up,
+                                const pg_gguf_tensor *const *down, int act, const float *shared_dev,
+                                float *out_dev);
+
 /* ---- Llama decoder block: the glue around the quantised products -------------- */
 
 typedef struct pg_rope pg_rope;               /* nn::RoPE                  src/nn.rs:1250-1256 */
@@ -479,6 +472,50 @@ pg_status pg_llama_block_forward(pg_ctx *ctx, pg_llama_block *block, const float
                                  pg_kv_cache *cache, float *out);
 pg_status pg_llama_block_forward_dev(pg_ctx *ctx, pg_llama_block *block, const float *h_dev, size_t seq,
                                      pg_kv_cache *cache, float *out_dev);
+
+/* ---- diagnostics and measurement: nothing below has a counterpart in the reference ----
+ * Timing per kernel, probes of what the part delivers, and the hooks the tests use to name or
+ * force the matrix-core product's tile.  None of them is needed to run the path. */
+
+/* Per-kernel timing.  No counterpart in the reference (it times whole calls with
+ * Instant::now(), benches/wallclock.rs:28-41): between pg_profile_begin and
+ * pg_profile_end every hot-path kernel the library launches on this context carries a
+ * start and a stop HIP event stamped with the dispatch's own begin and end times
+ * (hipExtLaunchKernel) on the context's stream; pg_profile_end waits for the stream and
+ * aggregates elapsed time per kernel name, read back with pg_profile_get. */
+pg_status pg_profile_begin(pg_ctx *ctx);
+pg_status pg_profile_end(pg_ctx *ctx, size_t *num_kernels);
+pg_status pg_profile_get(pg_ctx *ctx, size_t i, const char **name, double *total_ms,
+                         size_t *launches);
+/* The distinct launch sizes (work-items = grid x workgroup, as a kernel trace lists them) behind
+ * entry i and how many launches had each: up to `cap` pairs are written, *count gets their number.
+ * Lets a benchmark check that a stored counter summary still describes the launches it makes. */
+pg_status pg_profile_get_grids(pg_ctx *ctx, size_t i, size_t *work_items, size_t *launches, size_t cap,
+                               size_t *count);
+
+/* Ceilings of the part, measured (no counterpart in the reference; a benchmark reports them
+ * beside the published peaks):
+ *   pg_probe_mfma_i8    int8 matrix-core rate with every operand in registers, in TOP/s (2 ops
+ *                       per multiply-add), one workgroup of 8 wavefronts per CU for `iters` x 8
+ *                       MFMAs per wavefront, and the shader clock the loop ran at;
+ *   pg_probe_hbm_read   a pure 128-bit read stream: `passes` kernels, each reading
+ *                       bytes_per_pass from one of `buffers` distinct buffers in turn (make
+ *                       buffers x bytes_per_pass exceed the 256 MB last-level cache), in GB/s;
+ *   pg_probe_gemm_clock the shader clock inside the K loop of the W8A8 GEMM's 256x256 tile on an
+ *                       [m x k] . [k x n] product, and the mean duration of a workgroup's loop.
+ * Each allocates its own buffers and waits for completion. */
+pg_status pg_probe_mfma_i8(pg_ctx *ctx, int iters, double *tops, double *clock_ghz);
+pg_status pg_probe_hbm_read(pg_ctx *ctx, size_t bytes_per_pass, int buffers, int passes, double *gbs);
+pg_status pg_probe_gemm_clock(pg_ctx *ctx, size_t m, size_t k, size_t n, double *clock_ghz, double *loop_us);
+
+/* Diagnostics of the matrix-core product.  No counterpart in the reference (its Metal
+ * dispatcher picks between two shaders by size, src/metal/context.rs:2243, without a query):
+ * the output tile (rows x columns) and the number of K splits of the most recent W8A8 GEMM
+ * launch on this context, and an override of the dispatcher's tile choice (0 = automatic,
+ * 1 = 64x64, 2 = 256x256, 3 = 128x256, 4 = 128x64, 5 = 128x128).  Every tile gives the same
+ * bits; tests use the pair to prove each kernel instantiation ran. */
+pg_status pg_gemm_w8a8_last_tile(const pg_ctx *ctx, int *bm, int *bn, int *k_splits);
+pg_status pg_gemm_w8a8_force_tile(pg_ctx *ctx, int tile);
 
 #ifdef __cplusplus
 }

@@ -222,6 +222,9 @@ public:
         check(pg_gguf_matmul(gpu_->raw(), x.data(), m, h_, y.data()), "BlockWeight::matmul");
         return y;
     }
+    // The load-time step: make now the derived device copies that products over up to `max_rows` rows need
+    // (afterwards those products neither allocate nor wait).
+    void prepare(size_t max_rows) { check(pg_gguf_prepare(gpu_->raw(), h_, max_rows), "BlockWeight::prepare"); }
     const pg_gguf_tensor *handle() const { return h_; }
     size_t n_out() const { return n_out_; }
     size_t k_in() const { return k_in_; }

@@ -401,6 +401,139 @@ done:
 }
 
 /* ------------------------------------------------------------------------
+ * The deepseek gate: which experts a token goes to and with what weights.
+ *                                    reference: examples/deepseek/moe.rs:111-215
+ *   scores[e] = x[t] . w[e]  (f32, d ascending); sigmoid per score, or the softmax of the row;
+ *   the weights come from these scores; the SELECTION uses scores + bias (if any), after the
+ *   experts of all but the topk_groups best groups are set to 0 (group score = the sum of the
+ *   group's two largest biased scores when there is a bias, else its largest; stable
+ *   descending order, ties keep the lower index); sigmoid weights are divided by their sum
+ *   when that is > 0; all weights are multiplied by route_scale.
+ *   x [T, dim], w [E, dim], bias [E] or NULL; idx / weight [T, topk].  Returns 0 on success.
+ * ---------------------------------------------------------------------- */
+static void stable_order_desc(const float *v, size_t n, size_t *order) {
+    for (size_t e = 0; e < n; ++e) {   /* insertion sort: an element only passes strictly smaller ones */
+        size_t j = e;
+        while (j > 0 && v[order[j - 1]] < v[e]) { order[j] = order[j - 1]; --j; }
+        order[j] = e;
+    }
+}
+
+ORC_API int orc_deepseek_gate(const float *x, size_t T, size_t dim, const float *w, const float *bias,
+                              size_t E, size_t topk, size_t n_groups, size_t topk_groups, float route_scale,
+                              int use_sigmoid, int32_t *idx, float *weight) {
+    if (topk > E || n_groups == 0 || E % n_groups != 0 || topk_groups > n_groups) return -3;
+    float *scores = (float *)malloc(E * sizeof(float)), *orig = (float *)malloc(E * sizeof(float));
+    float *gs = (float *)malloc(n_groups * sizeof(float)), *gv = (float *)malloc(E * sizeof(float));
+    size_t *order = (size_t *)malloc(E * sizeof(size_t)), *gorder = (size_t *)malloc(n_groups * sizeof(size_t));
+    if (!scores || !orig || !gs || !gv || !order || !gorder) { free(scores); free(orig); free(gs); free(gv); free(order); free(gorder); return -1; }
+    for (size_t t = 0; t < T; ++t) {
+        for (size_t e = 0; e < E; ++e) {
+            float dot = 0.0f;
+            for (size_t d = 0; d < dim; ++d) dot += x[t * dim + d] * w[e * dim + d];
+            scores[e] = use_sigmoid ? 1.0f / (1.0f + expf(-dot)) : dot;
+        }
+        if (!use_sigmoid) {
+            float mx = -INFINITY, sum = 0.0f;
+            for (size_t e = 0; e < E; ++e) mx = fmaxf(mx, scores[e]);
+            for (size_t e = 0; e < E; ++e) sum += expf(scores[e] - mx);
+            for (size_t e = 0; e < E; ++e) scores[e] = expf(scores[e] - mx) / sum;
+        }
+        memcpy(orig, scores, E * sizeof(float));
+        if (bias)
+            for (size_t e = 0; e < E; ++e) scores[e] += bias[e];
+        if (n_groups > 1) {
+            const size_t per = E / n_groups;
+            for (size_t g = 0; g < n_groups; ++g) {
+                const float *grp = scores + g * per;
+                stable_order_desc(grp, per, order);
+                gs[g] = bias ? (per >= 2 ? 0.0f + grp[order[0]] + grp[order[1]] : 0.0f + grp[order[0]]) : grp[order[0]];
+            }
+            stable_order_desc(gs, n_groups, gorder);
+            for (size_t g = 0; g < n_groups; ++g) {
+                int selected = 0;
+                for (size_t s = 0; s < topk_groups; ++s) selected |= gorder[s] == g;
+                if (!selected)
+                    for (size_t e = g * per; e < (g + 1) * per; ++e) scores[e] = 0.0f;
+            }
+        }
+        stable_order_desc(scores, E, order);
+        float sum = 0.0f;
+        for (size_t k = 0; k < topk; ++k) {
+            idx[t * topk + k] = (int32_t)order[k];
+            weight[t * topk + k] = orig[order[k]];
+            sum += orig[order[k]];
+        }
+        if (use_sigmoid && sum > 0.0f)
+            for (size_t k = 0; k < topk; ++k) weight[t * topk + k] /= sum;
+        for (size_t k = 0; k < topk; ++k) weight[t * topk + k] *= route_scale;
+    }
+    free(scores); free(orig); free(gs); free(gv); free(order); free(gorder);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------
+ * The gpt_oss router: top-k on the biased logits, then a softmax over those k.
+ *                                    reference: examples/gpt_oss/moe.rs:298-330
+ *   logits [T, E] (= x . gate), gate_bias [E]; idx / weight [T, topk].
+ * ---------------------------------------------------------------------- */
+ORC_API int orc_gpt_oss_route(const float *logits, const float *gate_bias, size_t T, size_t E, size_t topk,
+                              int32_t *idx, float *weight) {
+    if (topk > E) return -3;
+    float *tl = (float *)malloc(E * sizeof(float));
+    size_t *order = (size_t *)malloc(E * sizeof(size_t));
+    if (!tl || !order) { free(tl); free(order); return -1; }
+    for (size_t t = 0; t < T; ++t) {
+        for (size_t e = 0; e < E; ++e) tl[e] = logits[t * E + e] + gate_bias[e];
+        stable_order_desc(tl, E, order);
+        float mx = -INFINITY, sum = 0.0f;
+        for (size_t k = 0; k < topk; ++k) mx = fmaxf(mx, tl[order[k]]);
+        for (size_t k = 0; k < topk; ++k) sum += expf(tl[order[k]] - mx);
+        for (size_t k = 0; k < topk; ++k) {
+            idx[t * topk + k] = (int32_t)order[k];
+            weight[t * topk + k] = expf(tl[order[k]] - mx) / sum;
+        }
+    }
+    free(tl); free(order);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------
+ * Expert FFN over a routing that is given: out[t] = sum_k weight[t, k] * expert_{idx[t, k]}(x[t]) in k order,
+ * then + shared[t] if a shared-expert output is passed.
+ *                                    reference: examples/deepseek/moe.rs:271-300 (y_data += weight * out; y.add(&z)),
+ *                                               examples/gpt_oss/moe.rs:334-351
+ *   Expert and operand layout as orc_moe_ffn.  shared [T, d] or NULL.
+ * ---------------------------------------------------------------------- */
+ORC_API int orc_moe_ffn_routed(const float *x, size_t T, size_t d, size_t ffn, size_t E, size_t top_k,
+                               const int32_t *idx, const float *weight,
+                               const uint8_t *const *gate, const uint8_t *const *up, const uint8_t *const *down,
+                               int ggml_type, int act, const float *shared, float *out) {
+    float *g = (float *)malloc(ffn * sizeof(float)), *u = (float *)malloc(ffn * sizeof(float));
+    float *h = (float *)malloc(ffn * sizeof(float)), *y = (float *)malloc(d * sizeof(float));
+    int rc = 0;
+    if (!g || !u || !h || !y) { rc = -1; goto done; }
+    memset(out, 0, T * d * sizeof(float));
+    for (size_t t = 0; t < T; ++t) {
+        const float *xt = x + t * d;
+        for (size_t k = 0; k < top_k; ++k) {
+            const int32_t e = idx[t * top_k + k];
+            if (e < 0 || (size_t)e >= E) { rc = -3; goto done; }
+            if ((rc = orc_gguf_matmul(xt, 1, gate[e], ggml_type, ffn, d, g))) goto done;
+            if ((rc = orc_gguf_matmul(xt, 1, up[e], ggml_type, ffn, d, u))) goto done;
+            for (size_t i = 0; i < ffn; ++i) h[i] = (act == 1 ? gelu_tanh(g[i]) : silu_tensor(g[i])) * u[i];
+            if ((rc = orc_gguf_matmul(h, 1, down[e], ggml_type, d, ffn, y))) goto done;
+            for (size_t i = 0; i < d; ++i) out[t * d + i] += weight[t * top_k + k] * y[i];
+        }
+        if (shared)
+            for (size_t i = 0; i < d; ++i) out[t * d + i] = out[t * d + i] + shared[t * d + i];
+    }
+done:
+    free(g); free(u); free(h); free(y);
+    return rc;
+}
+
+/* ------------------------------------------------------------------------
  * Input synthesis: SplitMix64-seeded Xoshiro256++ and Box-Muller normals
  *                                    reference: src/random.rs:16-53, 311-380
  *   (the sequential generator; at 200 000 elements and more the reference

@@ -77,6 +77,9 @@ SIGNATURES = {
     "pg_gguf_free": [_vp, _vp],
     "pg_gguf_matmul": [_vp, _vp, _sz, _vp, _vp],
     "pg_gguf_matmul_dev": [_vp, _vp, _sz, _vp, _vp],
+    "pg_gguf_prepare": [_vp, _vp, _sz],
+    "pg_gguf_drop_prepared": [_vp, _vp],
+    "pg_gguf_device_bytes": [_vp, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "pg_gguf_file_parse": [_vp, _sz, _pp],
     "pg_gguf_file_open": [C.c_char_p, _pp],
     "pg_gguf_file_close": [_vp],
@@ -98,6 +101,8 @@ SIGNATURES = {
     "pg_qtensor_from_record": [_vp, _vp, _sz, _pp, C.POINTER(_sz)],
     "pg_moe_ffn": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
     "pg_moe_ffn_dev": [_vp, _vp, _sz, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp],
+    "pg_moe_ffn_routed": [_vp, _vp, _sz, _vp, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp, _vp],
+    "pg_moe_ffn_routed_dev": [_vp, _vp, _sz, _vp, _vp, _sz, _sz, _pp, _pp, _pp, _int, _vp, _vp],
     "pg_huffman_table_from_frequencies": [_vp, _vp, _vp],
     "pg_huffman_canonical_codes": [_vp, _vp],
     "pg_huffman_encode": [_vp, _vp, _sz, _vp, _sz, C.POINTER(_sz)],

@@ -44,6 +44,31 @@ __global__ void route_topk_kernel(const float *__restrict__ logits, int T, int E
     }
 }
 
+// A routing that the caller made (another gate: examples/deepseek/moe.rs:111-215, examples/gpt_oss/moe.rs:298-330)
+// is copied into the same arrays.  The grouped products assume what every top-k gate delivers: a token's experts are
+// distinct and inside 0 .. E - 1.  An entry that breaks this is replaced by the lowest expert the token does not use
+// yet, with weight 0, so that nothing downstream can index outside a table whatever the buffers hold (the entry's
+// own contribution is then 0 times a finite product).  One thread per token.
+__global__ void copy_routing_kernel(const int *__restrict__ idx_in, const float *__restrict__ w_in, int T, int E, int top_k,
+                                    int *__restrict__ topk_idx, float *__restrict__ topk_p) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= T) return;
+    unsigned taken[MAX_EXPERTS / 32];
+    for (int i = 0; i < MAX_EXPERTS / 32; ++i) taken[i] = 0u;
+    for (int k = 0; k < top_k; ++k) {
+        int e = idx_in[(size_t)t * top_k + k];
+        float w = w_in[(size_t)t * top_k + k];
+        if (e < 0 || e >= E || (taken[e >> 5] & (1u << (e & 31)))) {
+            e = 0;
+            while (taken[e >> 5] & (1u << (e & 31))) ++e;  // top_k <= E: a free expert exists
+            w = 0.0f;
+        }
+        taken[e >> 5] |= 1u << (e & 31);
+        topk_idx[(size_t)t * top_k + k] = e;
+        topk_p[(size_t)t * top_k + k] = w;
+    }
+}
+
 // Per expert, the (token, k) pairs routed to it, in ascending pair order.  One wavefront per
 // expert: ballot + prefix count over 64 pairs at a time.
 __global__ __launch_bounds__(64) void expert_lists_kernel(const int *__restrict__ topk_idx, int P, int stride,
@@ -78,8 +103,9 @@ __global__ void act_mul_kernel(const float *__restrict__ g, const float *__restr
     h[i] = a * u[i];
 }
 
+// `shared` (optional): the shared experts' output, added last (y.add(&z), examples/deepseek/moe.rs:298-300).
 __global__ void combine_kernel(const float *__restrict__ yb, const float *__restrict__ topk_p, int T,
-                               int d, int top_k, float *__restrict__ out) {
+                               int d, int top_k, const float *__restrict__ shared, float *__restrict__ out) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)T * d) return;
     const size_t t = i / d, c = i - t * d;
@@ -88,15 +114,17 @@ __global__ void combine_kernel(const float *__restrict__ yb, const float *__rest
         const float prod = topk_p[t * top_k + k] * yb[(t * top_k + k) * d + c];
         acc = acc + prod;
     }
-    out[i] = acc;
+    out[i] = shared ? acc + shared[i] : acc;
 }
 
 }  // namespace
 
-PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
-                                const float *router_logits_dev, size_t E, size_t top_k,
-                                const pg_gguf_tensor *const *gate, const pg_gguf_tensor *const *up,
-                                const pg_gguf_tensor *const *down, int act, float *out_dev) {
+// The expert FFN behind both entry points: the routing comes from `router_logits_dev` (grok1's softmax -> top-k) or,
+// when that is null, from `idx_dev` / `weight_dev` as the caller's gate made them.
+static pg_status moe_ffn_core(pg_ctx *ctx, const float *x_dev, size_t T, const float *router_logits_dev,
+                              const int *idx_dev, const float *weight_dev, size_t E, size_t top_k,
+                              const pg_gguf_tensor *const *gate, const pg_gguf_tensor *const *up,
+                              const pg_gguf_tensor *const *down, int act, const float *shared_dev, float *out_dev) {
     PG_TRY(pg_use(ctx));
     PG_CHECK_ARG(E >= 1 && E <= MAX_EXPERTS, "pg_moe_ffn: %zu experts (1..%d supported)", E, MAX_EXPERTS);
     PG_CHECK_ARG(top_k >= 1 && top_k <= E, "pg_moe_ffn: top_k %zu of %zu experts", top_k, E);
@@ -114,7 +142,7 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
                      "pg_moe_ffn: expert %zu mixes block types", e);
     }
     if (T == 0) return PG_OK;
-    PG_CHECK_ARG(x_dev && router_logits_dev && out_dev, "pg_moe_ffn: null pointer");
+    PG_CHECK_ARG(x_dev && (router_logits_dev || (idx_dev && weight_dev)) && out_dev, "pg_moe_ffn: null pointer");
     PG_CHECK_ARG((uintptr_t)x_dev % 16 == 0, "pg_moe_ffn: x must be 16-byte aligned");
     PG_CHECK_ARG(T * top_k < (1ull << 20), "pg_moe_ffn: too many (token, expert) pairs");
     const size_t P = T * top_k;
@@ -199,8 +227,12 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
         tab = static_cast<const void **>(dev);
     }
 
-    PG_TRY(pg_launch(ctx, "moe_route_topk", route_topk_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
-                     router_logits_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
+    if (router_logits_dev)
+        PG_TRY(pg_launch(ctx, "moe_route_topk", route_topk_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
+                         router_logits_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
+    else
+        PG_TRY(pg_launch(ctx, "moe_copy_routing", copy_routing_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
+                         idx_dev, weight_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
     PG_TRY(pg_launch(ctx, "moe_expert_lists", expert_lists_kernel, dim3((unsigned)E), dim3(64), 0, topk_idx, (int)P, (int)T,
                      lists, counts));
     auto table = [&](int which) { return reinterpret_cast<const uint8_t *const *>(tab + which * E); };
@@ -236,7 +268,59 @@ PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
         PG_TRY(pg_launch_gguf_mm(ctx, type, d, ffn, nullptr, nullptr, gd, P, hd, yb, part));
     }
     return pg_launch(ctx, "moe_combine", combine_kernel, dim3(grid_for(T * d, 256)), dim3(256), 0, yb, topk_p, (int)T,
-                     (int)d, (int)top_k, out_dev);
+                     (int)d, (int)top_k, shared_dev, out_dev);
+}
+
+PG_API pg_status pg_moe_ffn_dev(pg_ctx *ctx, const float *x_dev, size_t T,
+                                const float *router_logits_dev, size_t E, size_t top_k,
+                                const pg_gguf_tensor *const *gate, const pg_gguf_tensor *const *up,
+                                const pg_gguf_tensor *const *down, int act, float *out_dev) {
+    PG_CHECK_ARG(T == 0 || router_logits_dev, "pg_moe_ffn: null router logits");
+    return moe_ffn_core(ctx, x_dev, T, router_logits_dev, nullptr, nullptr, E, top_k, gate, up, down, act, nullptr, out_dev);
+}
+
+PG_API pg_status pg_moe_ffn_routed_dev(pg_ctx *ctx, const float *x_dev, size_t T, const int32_t *expert_idx_dev,
+                                       const float *weight_dev, size_t E, size_t top_k,
+                                       const pg_gguf_tensor *const *gate, const pg_gguf_tensor *const *up,
+                                       const pg_gguf_tensor *const *down, int act, const float *shared_dev, float *out_dev) {
+    PG_CHECK_ARG(T == 0 || (expert_idx_dev && weight_dev), "pg_moe_ffn_routed: null routing");
+    return moe_ffn_core(ctx, x_dev, T, nullptr, expert_idx_dev, weight_dev, E, top_k, gate, up, down, act, shared_dev, out_dev);
+}
+
+PG_API pg_status pg_moe_ffn_routed(pg_ctx *ctx, const float *x, size_t T, const int32_t *expert_idx, const float *weight,
+                                   size_t E, size_t top_k, const pg_gguf_tensor *const *gate,
+                                   const pg_gguf_tensor *const *up, const pg_gguf_tensor *const *down, int act,
+                                   const float *shared, float *out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(gate && gate[0], "pg_moe_ffn_routed: null expert table");
+    if (T == 0) return PG_OK;
+    PG_CHECK_ARG(x && expert_idx && weight && out, "pg_moe_ffn_routed: null pointer");
+    PG_CHECK_ARG(E >= 1 && E <= MAX_EXPERTS && top_k >= 1 && top_k <= E, "pg_moe_ffn_routed: top_k %zu of %zu experts", top_k, E);
+    // the reference indexes self.experts[expert_idx] and would panic on an index out of range; a token's experts are
+    // distinct in every gate on this path (the grouped products rely on it)
+    for (size_t t = 0; t < T; ++t)
+        for (size_t k = 0; k < top_k; ++k) {
+            const int32_t e = expert_idx[t * top_k + k];
+            PG_CHECK_ARG(e >= 0 && (size_t)e < E, "pg_moe_ffn_routed: token %zu names expert %d of %zu", t, (int)e, E);
+            for (size_t j = 0; j < k; ++j)
+                PG_CHECK_ARG(expert_idx[t * top_k + j] != e, "pg_moe_ffn_routed: token %zu names expert %d twice", t, (int)e);
+        }
+    const size_t d = gate[0]->k_in, P = T * top_k;
+    pg_tmp dx, di, dw, dsh, dout;
+    PG_TRY(dx.alloc(T * d * sizeof(float)));
+    PG_TRY(di.alloc(P * sizeof(int32_t)));
+    PG_TRY(dw.alloc(P * sizeof(float)));
+    PG_TRY(dout.alloc(T * d * sizeof(float)));
+    if (shared) PG_TRY(dsh.alloc(T * d * sizeof(float)));
+    PG_HIP(hipMemcpyAsync(dx.p, x, T * d * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(di.p, expert_idx, P * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(dw.p, weight, P * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    if (shared) PG_HIP(hipMemcpyAsync(dsh.p, shared, T * d * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_moe_ffn_routed_dev(ctx, dx.as<float>(), T, di.as<int32_t>(), dw.as<float>(), E, top_k, gate, up, down, act,
+                                 shared ? dsh.as<float>() : nullptr, dout.as<float>()));
+    PG_HIP(hipMemcpyAsync(out, dout.p, T * d * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
 }
 
 PG_API pg_status pg_moe_ffn(pg_ctx *ctx, const float *x, size_t T, const float *router_logits,

@@ -86,6 +86,21 @@ class GgufWeight:
         _ffi.check(_ffi.lib.pg_gguf_matmul(self.ctx.handle, _ptr(x), m, self._h, _ptr(y)))
         return y
 
+    def prepare(self, max_rows):
+        """Make now the derived device copies that products over up to `max_rows` rows would otherwise make on
+        their first call (the load-time step: afterwards those calls neither allocate nor wait)."""
+        _ffi.check(_ffi.lib.pg_gguf_prepare(self.ctx.handle, self._h, max_rows))
+        return self
+
+    def drop_prepared(self):
+        _ffi.check(_ffi.lib.pg_gguf_drop_prepared(self.ctx.handle, self._h))
+
+    def device_bytes(self):
+        """(bytes as uploaded, bytes of derived copies held now)."""
+        up, der = C.c_size_t(), C.c_size_t()
+        _ffi.check(_ffi.lib.pg_gguf_device_bytes(self._h, C.byref(up), C.byref(der)))
+        return up.value, der.value
+
     def free(self):
         if self._h:
             _ffi.lib.pg_gguf_free(self.ctx.handle, self._h)

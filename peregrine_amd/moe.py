@@ -42,3 +42,27 @@ class MoEExperts:
         _ffi.check(_ffi.lib.pg_moe_ffn(self.ctx.handle, _ptr(x), T, _ptr(logits), E, self.top_k,
                                        g, u, dn, self.act, _ptr(out)))
         return out.reshape(T, self.d)
+
+    def forward_routed(self, x, expert_idx, weight, shared=None):
+        """The expert FFN over a routing another gate made (Gate::forward, examples/deepseek/moe.rs:111-215, or the
+        gpt_oss top-k-then-softmax, examples/gpt_oss/moe.rs:298-330): expert_idx / weight [T, top_k]; `shared`
+        [T, d] is the shared experts' output, added last (examples/deepseek/moe.rs:298-300)."""
+        E = len(self.gate)
+        x = np.ascontiguousarray(x, np.float32).reshape(-1)
+        T = x.size // self.d
+        if x.size != T * self.d:
+            raise ValueError("MoEExperts.forward_routed: x is not [T, d]")
+        idx = np.ascontiguousarray(expert_idx, np.int32).reshape(-1)
+        w = np.ascontiguousarray(weight, np.float32).reshape(-1)
+        if idx.size != T * self.top_k or w.size != T * self.top_k:
+            raise ValueError("MoEExperts.forward_routed: expert_idx / weight are not [T, top_k]")
+        sh = None
+        if shared is not None:
+            sh = np.ascontiguousarray(shared, np.float32).reshape(-1)
+            if sh.size != T * self.d:
+                raise ValueError("MoEExperts.forward_routed: shared is not [T, d]")
+        out = np.empty(T * self.d, np.float32)
+        (g, _g), (u, _u), (dn, _d) = self._table(self.gate), self._table(self.up), self._table(self.down)
+        _ffi.check(_ffi.lib.pg_moe_ffn_routed(self.ctx.handle, _ptr(x), T, _ptr(idx), _ptr(w), E, self.top_k, g, u, dn,
+                                              self.act, _ptr(sh) if sh is not None else None, _ptr(out)))
+        return out.reshape(T, self.d)

@@ -96,3 +96,82 @@ def test_constants_and_opaque_types_match_the_header():
     for name, value in consts.items():
         m = re.search(r"pub const " + name + r": \w+ = (\d+);", lib)
         assert m and m.group(1) == value, f"{name}: header {value}, lib.rs {m.group(1) if m else None}"
+
+
+# The public functions of `peregrine::quant` and `peregrine::gguf` on this path, as the reference declares them
+# (name -> normalised "(parameter types) -> return type").  `self` receivers keep their form.
+REFERENCE_SIGNATURES = {
+    # /root/reference/src/quant.rs:27, 79, 115, 129-134, 174, 183, 196-202
+    "quant::quantize_weights": "(&[f32], usize, usize) -> QuantizedTensor",
+    "quant::quantize_activations": "(&[f32], usize, usize) -> (Vec<i8>, Vec<f32>)",
+    "quant::dequantize": "(&QuantizedTensor) -> Vec<f32>",
+    "quant::matmul_quantized": "(&[f32], usize, usize, &QuantizedTensor) -> Vec<f32>",
+    "quant::to_gpu": "(&mut self, &GpuContext)",
+    "quant::from_gpu": "(&mut self, &GpuContext)",
+    "quant::matmul_quantized_gpu": "(&GpuContext, &[f32], usize, usize, &QuantizedTensor) -> GpuBuffer<f32>",
+    # /root/reference/src/gguf.rs:286, 307, 331, 354, 386-390
+    "gguf::dequant_q8_0": "(&[u8], usize) -> Vec<f32>",
+    "gguf::dequant_q4_0": "(&[u8], usize) -> Vec<f32>",
+    "gguf::dequant_q4_1": "(&[u8], usize) -> Vec<f32>",
+    "gguf::f16_to_f32": "(u16) -> f32",
+    "gguf::load_tensor_q8_as_quantized": "(&[u8], usize, usize) -> crate::quant::QuantizedTensor",
+}
+
+
+def _pub_fn_signatures(src):
+    """{name: "(types) -> ret"} of every `pub fn` in a piece of Rust source (parameter names dropped)."""
+    out = {}
+    for m in re.finditer(r"pub fn (\w+)\s*\((.*?)\)\s*(?:->\s*(.*?))?\s*\{", src, flags=re.S):
+        params = []
+        depth, cur = 0, ""
+        for ch in m.group(2):  # split on top-level commas only
+            if ch in "<([":
+                depth += 1
+            elif ch in ">)]":
+                depth -= 1
+            if ch == "," and depth == 0:
+                params.append(cur)
+                cur = ""
+            else:
+                cur += ch
+        params.append(cur)
+        types = []
+        for p in (q.strip() for q in params):
+            if not p:
+                continue
+            types.append(p if "self" in p.split(":")[0] and ":" not in p else " ".join(p.split(":", 1)[1].split()))
+        sig = "(" + ", ".join(types) + ")"
+        if m.group(3):
+            sig += " -> " + " ".join(m.group(3).split())
+        out.setdefault(m.group(1), sig)
+    return out
+
+
+def _module(src, name):
+    a = src.index(f"pub mod {name} {{")
+    b = src.index("\n}\n", a)
+    return src[a:b]
+
+
+def test_quant_and_gguf_wrappers_keep_the_reference_signatures():
+    src = open(os.path.join(CRATE, "src", "lib.rs")).read()
+    ours = {}
+    for mod in ("quant", "gguf"):
+        for name, sig in _pub_fn_signatures(_module(src, mod)).items():
+            ours[f"{mod}::{name}"] = sig
+    for name, want in REFERENCE_SIGNATURES.items():
+        assert ours.get(name) == want, f"{name}: crate has {ours.get(name)!r}, the reference {want!r}"
+
+
+def test_reference_signature_table_matches_the_reference_text():
+    """Only where the reference's sources are at hand (they do not travel with the repository)."""
+    import pytest
+
+    ref = "/root/reference/src"
+    if not os.path.isdir(ref):
+        pytest.skip("reference sources not present on this machine")
+    for mod in ("quant", "gguf"):
+        theirs = _pub_fn_signatures(open(os.path.join(ref, f"{mod}.rs")).read())
+        for name, want in REFERENCE_SIGNATURES.items():
+            if name.startswith(mod + "::"):
+                assert theirs.get(name.split("::")[1]) == want, f"{name}: reference has {theirs.get(name.split('::')[1])!r}"

@@ -160,6 +160,37 @@ def test_gguf_matmul_full_size_m16_and_linearity(ctx, orc):
     gw.free()
 
 
+@pytest.mark.parametrize("typ", [2, 8])
+def test_prepare_makes_the_derived_copies_up_front(ctx, orc, typ):
+    """pg_gguf_prepare: the tile-major copy exists before the first many-row product, the product's bits do not
+    depend on who made it, one-row preparation makes nothing, and pg_gguf_drop_prepared gives the memory back."""
+    from peregrine_amd import gguf
+    n_out, k_in, m = 384, 1024, 40
+    say(f"gguf prepare typ={typ}")
+    raw = (H.pack_q4_0 if typ == 2 else H.pack_q8_0)(orc.rng_normal(77, n_out * k_in, 0.0, 0.02))
+    x = orc.rng_normal(78, m * k_in)
+    lazy = gguf.GgufWeight(raw, typ, n_out, k_in, ctx)
+    eager = gguf.GgufWeight(raw, typ, n_out, k_in, ctx)
+    up, der = eager.device_bytes()
+    assert up == n_out * k_in // 32 * (18 if typ == 2 else 34) and der == 0
+    eager.prepare(1)
+    assert eager.device_bytes()[1] == 0
+    eager.prepare(m)
+    der = eager.device_bytes()[1]
+    assert der >= n_out * k_in // 32 * (16 if typ == 2 else 32)
+    y_eager = eager.matmul(x, m)
+    assert eager.device_bytes()[1] == der           # the product made nothing more
+    y_lazy = lazy.matmul(x, m)                      # makes its own copy on the way
+    assert lazy.device_bytes()[1] == der
+    assert (y_eager.view(np.uint32) == y_lazy.view(np.uint32)).all()
+    H.assert_close_rel(y_eager, orc.gguf_matmul(x, m, raw, typ, n_out, k_in), RTOL_ACHIEVED_MM, "prepared product")
+    eager.drop_prepared()
+    assert eager.device_bytes()[1] == 0
+    assert (eager.matmul(x, m).view(np.uint32) == y_lazy.view(np.uint32)).all()
+    lazy.free()
+    eager.free()
+
+
 def test_gguf_matmul_special_inputs(ctx, orc):
     from peregrine_amd import gguf
     n_out, k_in = 40, 128
