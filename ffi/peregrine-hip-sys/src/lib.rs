@@ -435,4 +435,27 @@ pub mod moe {
         ok(unsafe { pg_moe_ffn(ctx(), x.as_ptr(), t, router_logits.as_ptr(), e, top_k, g.as_ptr(), u.as_ptr(), dn.as_ptr(), act, out.as_mut_ptr()) });
         out
     }
+
+    /// The same over a routing another gate made (`Gate::forward`, examples/deepseek/moe.rs:111-215, which returns
+    /// `Vec<Vec<(usize, f32)>>`; the gpt_oss router, examples/gpt_oss/moe.rs:298-330): `routing[t]` = the token's
+    /// `(expert_idx, weight)` list, every token with the same number of experts; `shared` = the shared experts'
+    /// output `[t, d]`, added last (examples/deepseek/moe.rs:298-300).
+    pub fn moe_ffn_routed(x: &[f32], routing: &[Vec<(usize, f32)>], gate: &[gguf::GgufWeight], up: &[gguf::GgufWeight],
+                          down: &[gguf::GgufWeight], act: c_int, shared: Option<&[f32]>) -> Vec<f32> {
+        let (e, t) = (gate.len(), routing.len());
+        assert!(e > 0 && up.len() == e && down.len() == e);
+        let d = gate[0].2;
+        assert_eq!(x.len(), t * d);
+        let top_k = routing.first().map_or(0, |r| r.len());
+        assert!(routing.iter().all(|r| r.len() == top_k));
+        let idx: Vec<i32> = routing.iter().flatten().map(|&(i, _)| i as i32).collect();
+        let w: Vec<f32> = routing.iter().flatten().map(|&(_, w)| w).collect();
+        if let Some(s) = shared { assert_eq!(s.len(), t * d); }
+        let tab = |w: &[gguf::GgufWeight]| w.iter().map(|g| g.0 as *const pg_gguf_tensor).collect::<Vec<_>>();
+        let (g, u, dn) = (tab(gate), tab(up), tab(down));
+        let mut out = vec![0f32; t * d];
+        ok(unsafe { pg_moe_ffn_routed(ctx(), x.as_ptr(), t, idx.as_ptr(), w.as_ptr(), e, top_k, g.as_ptr(), u.as_ptr(), dn.as_ptr(), act,
+                                      shared.map_or(std::ptr::null(), |s| s.as_ptr()), out.as_mut_ptr()) });
+        out
+    }
 }

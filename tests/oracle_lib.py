@@ -167,6 +167,42 @@ def moe_ffn(x, T, d, ffn, E, top_k, logits, gate, up, down, ggml_type, act):
     return out.reshape(T, d), idx.reshape(T, top_k), prob.reshape(T, top_k)
 
 
+def deepseek_gate(x, T, dim, w, bias, E, topk, n_groups, topk_groups, route_scale, use_sigmoid):
+    """Gate::forward (examples/deepseek/moe.rs:111-215): (expert indices [T, topk], weights [T, topk])."""
+    idx = np.empty(T * topk, np.int32)
+    wt = np.empty(T * topk, np.float32)
+    b = None if bias is None else _f32(bias).reshape(-1)
+    rc = lib.orc_deepseek_gate(_p(_f32(x).reshape(-1)), _sz(T), _sz(dim), _p(_f32(w).reshape(-1)), _p(b) if b is not None else None,
+                               _sz(E), _sz(topk), _sz(n_groups), _sz(topk_groups), C.c_float(route_scale), C.c_int(int(use_sigmoid)),
+                               _p(idx), _p(wt))
+    assert rc == 0, rc
+    return idx.reshape(T, topk), wt.reshape(T, topk)
+
+
+def gpt_oss_route(logits, gate_bias, T, E, topk):
+    """The gpt_oss router (examples/gpt_oss/moe.rs:298-330): top-k on logits + bias, softmax over the k."""
+    idx = np.empty(T * topk, np.int32)
+    wt = np.empty(T * topk, np.float32)
+    rc = lib.orc_gpt_oss_route(_p(_f32(logits).reshape(-1)), _p(_f32(gate_bias).reshape(-1)), _sz(T), _sz(E), _sz(topk), _p(idx), _p(wt))
+    assert rc == 0, rc
+    return idx.reshape(T, topk), wt.reshape(T, topk)
+
+
+def moe_ffn_routed(x, T, d, ffn, E, top_k, idx, weight, gate, up, down, ggml_type, act, shared=None):
+    """The expert FFN over a given routing, plus the shared experts' output if passed."""
+    keep = [np.frombuffer(bytes(b), np.uint8).copy() for b in list(gate) + list(up) + list(down)]
+    mk = lambda arrs: (C.c_void_p * E)(*[a.ctypes.data for a in arrs])
+    g, u, dn = mk(keep[:E]), mk(keep[E:2 * E]), mk(keep[2 * E:])
+    out = np.empty(T * d, np.float32)
+    ii = np.ascontiguousarray(idx, np.int32).reshape(-1)
+    ww = _f32(weight).reshape(-1)
+    sh = None if shared is None else _f32(shared).reshape(-1)
+    rc = lib.orc_moe_ffn_routed(_p(_f32(x).reshape(-1)), _sz(T), _sz(d), _sz(ffn), _sz(E), _sz(top_k), _p(ii), _p(ww),
+                                g, u, dn, C.c_int(ggml_type), C.c_int(act), _p(sh) if sh is not None else None, _p(out))
+    assert rc == 0, rc
+    return out.reshape(T, d)
+
+
 def philox_4x32_10(counter, key):
     """orc_philox_4x32_10 on one (counter[4], key[2]); returns the four u32 outputs."""
     c = (C.c_uint32 * 4)(*counter)

