@@ -153,9 +153,11 @@ extern "C" {
     pub fn pg_profile_get_grids(ctx: *mut pg_ctx, i: usize, work_items: *mut usize, launches: *mut usize, cap: usize, count: *mut usize) -> pg_status;
     pub fn pg_probe_mfma_i8(ctx: *mut pg_ctx, iters: c_int, tops: *mut f64, clock_ghz: *mut f64) -> pg_status;
     pub fn pg_probe_hbm_read(ctx: *mut pg_ctx, bytes_per_pass: usize, buffers: c_int, passes: c_int, gbs: *mut f64) -> pg_status;
+    pub fn pg_probe_hbm_read_shaped(ctx: *mut pg_ctx, bytes_per_pass: usize, buffers: c_int, passes: c_int, workgroups: c_int, threads: c_int, loads_in_flight: c_int, gbs: *mut f64) -> pg_status;
     pub fn pg_probe_gemm_clock(ctx: *mut pg_ctx, m: usize, k: usize, n: usize, clock_ghz: *mut f64, loop_us: *mut f64) -> pg_status;
     pub fn pg_gemm_w8a8_last_tile(ctx: *const pg_ctx, bm: *mut c_int, bn: *mut c_int, k_splits: *mut c_int) -> pg_status;
     pub fn pg_gemm_w8a8_force_tile(ctx: *mut pg_ctx, tile: c_int) -> pg_status;
+    pub fn pg_gemv_w8a8_force_shape(ctx: *mut pg_ctx, wavefronts: c_int, rows_per_wavefront: c_int) -> pg_status;
 }
 // ---- generated: end ----
 

@@ -506,6 +506,11 @@ pg_status pg_profile_get_grids(pg_ctx *ctx, size_t i, size_t *work_items, size_t
  * Each allocates its own buffers and waits for completion. */
 pg_status pg_probe_mfma_i8(pg_ctx *ctx, int iters, double *tops, double *clock_ghz);
 pg_status pg_probe_hbm_read(pg_ctx *ctx, size_t bytes_per_pass, int buffers, int passes, double *gbs);
+/* The same read stream with the launch shape named: `workgroups` of `threads` (256, 512 or 1024) threads, each lane
+ * with `loads_in_flight` (4, 8 or 16) 128-bit loads outstanding; pg_probe_hbm_read is 8 x CUs workgroups of 256
+ * with 8.  A benchmark sweeps the shape at the size of its own launches and quotes the best as the ceiling. */
+pg_status pg_probe_hbm_read_shaped(pg_ctx *ctx, size_t bytes_per_pass, int buffers, int passes, int workgroups,
+                                   int threads, int loads_in_flight, double *gbs);
 pg_status pg_probe_gemm_clock(pg_ctx *ctx, size_t m, size_t k, size_t n, double *clock_ghz, double *loop_us);
 
 /* Diagnostics of the matrix-core product.  No counterpart in the reference (its Metal
@@ -516,6 +521,10 @@ pg_status pg_probe_gemm_clock(pg_ctx *ctx, size_t m, size_t k, size_t n, double 
  * bits; tests use the pair to prove each kernel instantiation ran. */
 pg_status pg_gemm_w8a8_last_tile(const pg_ctx *ctx, int *bm, int *bn, int *k_splits);
 pg_status pg_gemm_w8a8_force_tile(pg_ctx *ctx, int tile);
+/* The one-row product that takes the activation row in f32: the workgroup shape (wavefronts per workgroup 4, 8 or
+ * 16; weight rows per wavefront 1 or 2, not 16 x 2) instead of the dispatcher's choice by row length; 0, 0 =
+ * automatic.  Every shape gives the same bits. */
+pg_status pg_gemv_w8a8_force_shape(pg_ctx *ctx, int wavefronts, int rows_per_wavefront);
 
 #ifdef __cplusplus
 }

@@ -43,6 +43,7 @@ SIGNATURES = {
     "pg_profile_get": [_vp, _sz, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(_sz)],
     "pg_probe_mfma_i8": [_vp, _int, C.POINTER(C.c_double), C.POINTER(C.c_double)],
     "pg_probe_hbm_read": [_vp, _sz, _int, _int, C.POINTER(C.c_double)],
+    "pg_probe_hbm_read_shaped": [_vp, _sz, _int, _int, _int, _int, _int, C.POINTER(C.c_double)],
     "pg_probe_gemm_clock": [_vp, _sz, _sz, _sz, C.POINTER(C.c_double), C.POINTER(C.c_double)],
     "pg_profile_get_grids": [_vp, _sz, C.POINTER(_sz), C.POINTER(_sz), _sz, C.POINTER(_sz)],
     "pg_dev_alloc": [_vp, _sz, _pp],
@@ -66,6 +67,7 @@ SIGNATURES = {
     "pg_fixed_scratch_bytes": [],
     "pg_gemm_w8a8_last_tile": [_vp, C.POINTER(_int), C.POINTER(_int), C.POINTER(_int)],
     "pg_gemm_w8a8_force_tile": [_vp, _int],
+    "pg_gemv_w8a8_force_shape": [_vp, _int, _int],
     "pg_matmul_dequant_i8": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_matmul_dequant_i8_dev": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_f16_to_f32": [_vp, _vp, _sz, _vp],

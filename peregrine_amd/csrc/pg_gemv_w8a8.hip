@@ -10,6 +10,7 @@
 #include <limits.h>
 #include "pg_internal.h"
 #include "pg_quant_dev.h"
+#include "pg_stream_addr.h"
 
 namespace {
 
@@ -95,7 +96,7 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_kernel(
     float *__restrict__ out, int32_t *__restrict__ acc_out) {
     const int nchunk = k_pad >> 4;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int row0 = (blockIdx.x * 4 + wave) * RPW;
+    const int row0 = pg_m1_row0(blockIdx.x, wave, 4, RPW);
     const v4i *xp = reinterpret_cast<const v4i *>(a_i8);
     v4i x[NCH];
 #pragma unroll
@@ -111,8 +112,7 @@ __global__ __launch_bounds__(256) void gemv_w8a8_m1_kernel(
         v4i w[NCH];
 #pragma unroll
         for (int j = 0; j < NCH; ++j) {
-            const int c = lane + 64 * j;
-            w[j] = __builtin_nontemporal_load(wp + (c < nchunk ? c : 0));  // (past a short row: its first chunk, against zeros)
+            w[j] = __builtin_nontemporal_load(wp + pg_m1_weight_chunk(lane, j, nchunk));  // (past a short row: its first chunk, against zeros)
         }
         int acc = 0;
 #pragma unroll
@@ -162,14 +162,12 @@ __global__ __launch_bounds__(64 * NW) void gemv_w8a8_m1_f32x_kernel(
     const int n = grp.n[g];
     const int nchunk = k_pad >> 4;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int row0 = (((int)blockIdx.x - grp.wg0[g]) * NW + wave) * RPW;
+    const int row0 = pg_m1_row0((int)blockIdx.x - grp.wg0[g], wave, NW, RPW);
     auto load_row = [&](int row, v4i (&w)[NCH]) {
         const v4i *wp = reinterpret_cast<const v4i *>(w_t + (size_t)row * k_pad);
 #pragma unroll
-        for (int j = 0; j < NCH; ++j) {
-            const int c = lane + 64 * j;
-            w[j] = __builtin_nontemporal_load(wp + (c < nchunk ? c : 0));  // (past a short row: its first chunk, against zeros)
-        }
+        for (int j = 0; j < NCH; ++j)
+            w[j] = __builtin_nontemporal_load(wp + pg_m1_weight_chunk(lane, j, nchunk));  // (past a short row: its first chunk, against zeros)
     };
     // Loads return in issue order: the activation row (from L2) is requested first, so that its
     // quantisation can start as soon as it is there; every weight row of this wavefront (from HBM)
@@ -180,8 +178,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_w8a8_m1_f32x_kernel(
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int idx = threadIdx.x + NT * i;
-        v[i] = x4[idx < nvec ? idx : nvec - 1];
+        v[i] = x4[pg_m1_x_vec(threadIdx.x, i, NT, nvec)];
     }
     v4i w[RPW][NCH];
 #pragma unroll
@@ -260,6 +257,15 @@ pg_status launch_m1_f32x_rows(pg_ctx *ctx, const float *x_f32, size_t k, const p
                               int32_t *acc) {
     size_t rows = 0;
     for (int i = 0; i < count; ++i) rows += w[i]->n_pad;
+    if (ctx->gemv_force_nw) {  // pg_gemv_w8a8_force_shape: a test or a sweep names the instantiation
+        const int nw = ctx->gemv_force_nw, rpw = ctx->gemv_force_rpw;
+        if (nw == 4 && rpw == 1) return launch_m1_f32x<NCH, 1, 4>(ctx, x_f32, k, w, out, count, acc);
+        if (nw == 4 && rpw == 2) return launch_m1_f32x<NCH, 2, 4>(ctx, x_f32, k, w, out, count, acc);
+        if (nw == 8 && rpw == 1) return launch_m1_f32x<NCH, 1, 8>(ctx, x_f32, k, w, out, count, acc);
+        if (nw == 8 && rpw == 2) return launch_m1_f32x<NCH, 2, 8>(ctx, x_f32, k, w, out, count, acc);
+        if (nw == 16 && rpw == 1) return launch_m1_f32x<NCH, 1, 16>(ctx, x_f32, k, w, out, count, acc);
+        return pg_fail(PG_EINVAL, "gemv_w8a8: no instantiation with %d wavefronts x %d rows", nw, rpw);
+    }
     constexpr int NW = NCH <= 4 ? 4 : (NCH <= 8 ? 8 : 16);
     if constexpr (NW < 16) {
         if (rows / 2 >= (size_t)ctx->num_cu * 8) return launch_m1_f32x<NCH, 2, NW>(ctx, x_f32, k, w, out, count, acc);

@@ -50,6 +50,7 @@ struct pg_ctx {
     // optional override of the dispatcher's choice (pg_gemm_w8a8_force_tile; 0 = automatic).
     int gemm_last_bm = 0, gemm_last_bn = 0, gemm_last_splits = 0;
     int gemm_force_tile = 0;
+    int gemv_force_nw = 0, gemv_force_rpw = 0;  // pg_gemv_w8a8_force_shape (0 = the dispatcher chooses)
 };
 
 // Device-resident quantised weight, K-contiguous and zero-padded:

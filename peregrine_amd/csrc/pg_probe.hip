@@ -5,6 +5,7 @@
 //   * a pure 128-bit read stream over buffers larger than the last-level cache,
 //   * the shader clock seen inside a W8A8 GEMM tile (pg_probe_gemm_clock, in pg_gemm_w8a8.hip).
 #include "pg_internal.h"
+#include "pg_stream_addr.h"
 
 namespace {
 
@@ -50,20 +51,25 @@ void probe_mfma_i8_kernel(int iters, const v4i *__restrict__ in, int *__restrict
     }
 }
 
-// Every workgroup streams a contiguous slice with 128-bit non-temporal loads, eight in flight
-// per lane; the sum is stored only if it has an impossible value (keeps the loads alive).
-__global__ __launch_bounds__(256) void probe_read_kernel(const v4i *__restrict__ src, size_t chunks_per_wg, int *__restrict__ out) {
-    const v4i *p = src + (size_t)blockIdx.x * chunks_per_wg;
+// Every workgroup streams a contiguous slice of `total` 16-byte chunks with 128-bit non-temporal loads, U in flight
+// per lane (a lane past the end of the slice loads nothing); the sum is stored only if it has an impossible value
+// (keeps the loads alive).
+template <int U>
+__global__ __launch_bounds__(1024) void probe_read_kernel(const v4i *__restrict__ src, size_t chunks_per_wg, size_t total, int *__restrict__ out) {
+    const size_t first = (size_t)blockIdx.x * chunks_per_wg;
+    const size_t n = first >= total ? 0 : (total - first < chunks_per_wg ? total - first : chunks_per_wg);
+    const v4i *p = src + first;
     v4i s = {0, 0, 0, 0};
-    for (size_t c = threadIdx.x; c < chunks_per_wg; c += 8 * 256) {
-        v4i v[8];
+    for (size_t c = threadIdx.x; c < n; c += (size_t)U * blockDim.x) {
+        v4i v[U];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const size_t i = c + (size_t)u * 256;
-            v[u] = __builtin_nontemporal_load(p + (i < chunks_per_wg ? i : c));
+        for (int u = 0; u < U; ++u) {
+            const size_t i = pg_probe_chunk(c, u, blockDim.x);
+            v[u] = v4i{0, 0, 0, 0};
+            if (i < n) v[u] = __builtin_nontemporal_load(p + i);
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) s += v[u];
+        for (int u = 0; u < U; ++u) s += v[u];
     }
     if (s.x == 0x12345678 && s.y == 0x0BADF00D) out[0] = s.z + s.w;
 }
@@ -128,13 +134,17 @@ PG_API pg_status pg_probe_mfma_i8(pg_ctx *ctx, int iters, double *tops, double *
     return PG_OK;
 }
 
-PG_API pg_status pg_probe_hbm_read(pg_ctx *ctx, size_t bytes_per_pass, int buffers, int passes, double *gbs) {
+PG_API pg_status pg_probe_hbm_read_shaped(pg_ctx *ctx, size_t bytes_per_pass, int buffers, int passes, int workgroups,
+                                          int threads, int loads_in_flight, double *gbs) {
     PG_TRY(pg_use(ctx));
     PG_CHECK_ARG(bytes_per_pass >= (1u << 20) && bytes_per_pass <= (1ull << 32), "pg_probe_hbm_read: %zu bytes per pass (1 MiB .. 4 GiB)", bytes_per_pass);
     PG_CHECK_ARG(buffers >= 1 && buffers <= 64 && passes >= 1 && passes <= 4096, "pg_probe_hbm_read: buffers %d, passes %d", buffers, passes);
-    const size_t wgs = (size_t)ctx->num_cu * 8;
-    const size_t chunks_per_wg = bytes_per_pass / 16 / wgs;
-    const size_t pass_bytes = chunks_per_wg * wgs * 16;
+    PG_CHECK_ARG(workgroups >= 1 && workgroups <= 65536 && (threads == 256 || threads == 512 || threads == 1024) &&
+                     (loads_in_flight == 4 || loads_in_flight == 8 || loads_in_flight == 16),
+                 "pg_probe_hbm_read: %d workgroups of %d threads, %d loads in flight (256 | 512 | 1024 threads; 4 | 8 | 16 loads)", workgroups, threads, loads_in_flight);
+    const size_t total = bytes_per_pass / 16, wgs = (size_t)workgroups;
+    const size_t chunks_per_wg = (total + wgs - 1) / wgs;
+    const size_t pass_bytes = total * 16;
     pg_tmp buf, out;
     PG_TRY(buf.alloc(pass_bytes * buffers));
     PG_TRY(out.alloc(256));
@@ -143,9 +153,12 @@ PG_API pg_status pg_probe_hbm_read(pg_ctx *ctx, size_t bytes_per_pass, int buffe
     PG_HIP(hipEventCreate(&e0));
     if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return pg_fail(PG_EDEVICE, "hipEventCreate failed"); }
     auto run = [&](int n) {
-        for (int i = 0; i < n; ++i)
-            probe_read_kernel<<<dim3((unsigned)wgs), dim3(256), 0, ctx->stream>>>(
-                reinterpret_cast<const v4i *>(buf.as<char>() + (size_t)(i % buffers) * pass_bytes), chunks_per_wg, out.as<int>());
+        for (int i = 0; i < n; ++i) {
+            const v4i *src = reinterpret_cast<const v4i *>(buf.as<char>() + (size_t)(i % buffers) * pass_bytes);
+            if (loads_in_flight == 4) probe_read_kernel<4><<<dim3((unsigned)wgs), dim3(threads), 0, ctx->stream>>>(src, chunks_per_wg, total, out.as<int>());
+            else if (loads_in_flight == 8) probe_read_kernel<8><<<dim3((unsigned)wgs), dim3(threads), 0, ctx->stream>>>(src, chunks_per_wg, total, out.as<int>());
+            else probe_read_kernel<16><<<dim3((unsigned)wgs), dim3(threads), 0, ctx->stream>>>(src, chunks_per_wg, total, out.as<int>());
+        }
     };
     run(buffers);  // warm-up: one pass over every buffer
     hipError_t e = hipEventRecord(e0, ctx->stream);
@@ -160,4 +173,10 @@ PG_API pg_status pg_probe_hbm_read(pg_ctx *ctx, size_t bytes_per_pass, int buffe
     if (e != hipSuccess) return pg_fail(PG_EDEVICE, "pg_probe_hbm_read: %s", hipGetErrorString(e));
     if (gbs) *gbs = (double)pass_bytes * passes / (ms * 1e-3) / 1e9;
     return PG_OK;
+}
+
+// The default shape: eight workgroups of 256 threads per CU, eight loads in flight per lane.
+PG_API pg_status pg_probe_hbm_read(pg_ctx *ctx, size_t bytes_per_pass, int buffers, int passes, double *gbs) {
+    PG_TRY(pg_use(ctx));
+    return pg_probe_hbm_read_shaped(ctx, bytes_per_pass, buffers, passes, ctx->num_cu * 8, 256, 8, gbs);
 }

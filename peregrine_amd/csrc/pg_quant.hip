@@ -677,6 +677,17 @@ PG_API pg_status pg_gemm_w8a8_force_tile(pg_ctx *ctx, int tile) {
     return PG_OK;
 }
 
+PG_API pg_status pg_gemv_w8a8_force_shape(pg_ctx *ctx, int wavefronts, int rows_per_wavefront) {
+    PG_CHECK_ARG(ctx != nullptr, "null context");
+    PG_CHECK_ARG((wavefronts == 0 && rows_per_wavefront == 0) ||
+                     ((wavefronts == 4 || wavefronts == 8 || wavefronts == 16) && (rows_per_wavefront == 1 || rows_per_wavefront == 2) &&
+                      !(wavefronts == 16 && rows_per_wavefront == 2)),
+                 "pg_gemv_w8a8_force_shape: %d wavefronts x %d rows (4 | 8 x 1 | 2, 16 x 1, or 0, 0 for automatic)", wavefronts, rows_per_wavefront);
+    ctx->gemv_force_nw = wavefronts;
+    ctx->gemv_force_rpw = rows_per_wavefront;
+    return PG_OK;
+}
+
 // The reference's GPU numerics for the same call: f32 activations times dequantised weights,
 // f32 accumulate (matmul_dequant_i8, src/metal/shaders.rs:2329-2375).  Here the activations
 // become 23/24-bit fixed point per row (power-of-two scale) and the product runs three times on the int8 matrix
