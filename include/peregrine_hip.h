@@ -526,6 +526,24 @@ pg_status pg_gemm_w8a8_force_tile(pg_ctx *ctx, int tile);
  * automatic.  Every shape gives the same bits. */
 pg_status pg_gemv_w8a8_force_shape(pg_ctx *ctx, int wavefronts, int rows_per_wavefront);
 
+/* Address audit of the streaming kernels, on the host (no device is touched): each function walks every
+ * (workgroup, wavefront, lane, step) of one launch of the named kernel shape with the very index functions the
+ * kernel uses and returns, per array it streams, the end of the furthest byte a load would touch and the bytes
+ * the library allocates for that array.  end <= bytes must hold for every shape the dispatchers can pick; a
+ * test without a GPU sweeps them. */
+pg_status pg_audit_gemv_w8a8_m1(size_t k, size_t n, int nch, int rows_per_wavefront, int wavefronts, int f32_row,
+                                size_t *w_end, size_t *w_bytes, size_t *x_end, size_t *x_bytes);
+pg_status pg_audit_gemm_w8a8_skinny(size_t m, size_t k, size_t n, int activation_tiles, int weight_tiles, int wavefronts,
+                                    size_t *w_end, size_t *w_bytes, size_t *a_end, size_t *a_bytes);
+pg_status pg_audit_gguf_gemv(size_t n_out, size_t k_in, int q8, int blocks_per_lane, int rows_per_wavefront,
+                             int wavefronts, size_t *qs_end, size_t *qs_bytes, size_t *d_end, size_t *d_bytes);
+pg_status pg_audit_gguf_skinny(size_t n_out, size_t k_in, int q8, int wavefronts, size_t *qs_end, size_t *qs_bytes,
+                               size_t *d_end, size_t *d_bytes);
+pg_status pg_audit_mxfp4_rows(size_t out_dim, size_t in_dim, int row_groups_per_workgroup, int wavefronts,
+                              size_t *qs_end, size_t *qs_bytes, size_t *sc_end, size_t *sc_bytes);
+pg_status pg_audit_probe_read(size_t bytes, int workgroups, int threads, int loads_in_flight, size_t *end,
+                              size_t *alloc);
+
 #ifdef __cplusplus
 }
 #endif

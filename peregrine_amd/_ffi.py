@@ -16,7 +16,7 @@ if not os.path.exists(LIB_PATH):
 # device ("no ROCm-capable device is detected" from pg_ctx_create).
 try:
     import torch  # noqa: F401
-except ImportError:
+except Exception:  # absent, or present but broken (a failing torch must not take this binding down with it)
     pass
 
 lib = C.CDLL(LIB_PATH)
@@ -66,6 +66,12 @@ SIGNATURES = {
     "pg_matmul_quantized_fixed_scratch_dev": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_fixed_scratch_bytes": [],
     "pg_gemm_w8a8_last_tile": [_vp, C.POINTER(_int), C.POINTER(_int), C.POINTER(_int)],
+    "pg_audit_gemv_w8a8_m1": [_sz, _sz, _int, _int, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
+    "pg_audit_gemm_w8a8_skinny": [_sz, _sz, _sz, _int, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
+    "pg_audit_gguf_gemv": [_sz, _sz, _int, _int, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
+    "pg_audit_gguf_skinny": [_sz, _sz, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
+    "pg_audit_mxfp4_rows": [_sz, _sz, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
+    "pg_audit_probe_read": [_sz, _int, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "pg_gemm_w8a8_force_tile": [_vp, _int],
     "pg_gemv_w8a8_force_shape": [_vp, _int, _int],
     "pg_matmul_dequant_i8": [_vp, _vp, _sz, _sz, _vp, _vp],

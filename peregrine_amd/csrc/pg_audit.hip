@@ -1,0 +1,202 @@
+// Host-side audit of the streaming kernels' load addresses.  No kernel runs and no HIP call is made: every function
+// walks the (workgroup, wavefront, lane, step) space of one launch with the index functions the kernels themselves
+// use (pg_stream_addr.h) and reports, per array, the end of the furthest byte any load would touch beside the size
+// of the allocation.  A test without a GPU sweeps ragged shapes over every instantiation and holds one against the
+// other: an over-read of a few hundred bytes only faults on the device when the tensor happens to end a mapping.
+#include <algorithm>
+#include "pg_internal.h"
+#include "pg_stream_addr.h"
+
+namespace {
+struct span_check {
+    size_t end = 0;
+    void touch(size_t offset, size_t bytes) { end = std::max(end, offset + bytes); }
+};
+}  // namespace
+
+// One-row W8A8 products over a [n_pad][k_pad] weight plane (gemv_w8a8_m1_kernel: nw = 4; gemv_w8a8_m1_f32x_kernel:
+// nw = 4, 8, 16).  nch = the kernel's NCH (64-lane steps over a row), rpw = rows per wavefront.  `f32_row`: the
+// row arrives in f32 (k elements, k % 4 == 0) and every thread fetches float4s of it.
+PG_API pg_status pg_audit_gemv_w8a8_m1(size_t k, size_t n, int nch, int rpw, int nw, int f32_row, size_t *w_end, size_t *w_bytes,
+                                       size_t *x_end, size_t *x_bytes) {
+    PG_CHECK_ARG(k > 0 && n > 0 && nch > 0 && rpw > 0 && nw > 0, "pg_audit_gemv_w8a8_m1: bad arguments");
+    const size_t k_pad = pg_round_up(k, PG_KPAD), n_pad = pg_round_up(n, PG_NPAD);
+    const int nchunk = (int)(k_pad >> 4);
+    PG_CHECK_ARG((size_t)nch * 64 >= (size_t)nchunk, "pg_audit_gemv_w8a8_m1: NCH %d does not cover a row of %zu bytes", nch, k_pad);
+    span_check w, x;
+    const int wgs = (int)(n_pad / ((size_t)nw * rpw));
+    for (int wg = 0; wg < wgs; ++wg)
+        for (int wave = 0; wave < nw; ++wave) {
+            const int row0 = pg_m1_row0(wg, wave, nw, rpw);
+            for (int r = 0; r < rpw; ++r)
+                for (int lane = 0; lane < 64; ++lane)
+                    for (int j = 0; j < nch; ++j) w.touch(((size_t)(row0 + r) * k_pad) + (size_t)pg_m1_weight_chunk(lane, j, nchunk) * 16, 16);
+        }
+    if (f32_row) {
+        const int nt = 64 * nw, nv = (nch * 256 + nt - 1) / nt, nvec = (int)(k >> 2);
+        for (int t = 0; t < nt; ++t)
+            for (int i = 0; i < nv; ++i) x.touch((size_t)pg_m1_x_vec(t, i, nt, nvec) * 16, 16);
+    }
+    if (w_end) *w_end = w.end;
+    if (w_bytes) *w_bytes = n_pad * k_pad;
+    if (x_end) *x_end = x.end;
+    if (x_bytes) *x_bytes = k * 4;
+    return PG_OK;
+}
+
+// 2 .. 64 rows in one launch over int8 weights (gemm_w8a8_skinny_kernel<MB, NB, NW, NST>): the weight plane
+// [n_pad][k_pad] and the quantised activation rows [m_pad][k_pad].
+PG_API pg_status pg_audit_gemm_w8a8_skinny(size_t m, size_t k, size_t n, int mb, int nb_tiles, int nw, size_t *w_end, size_t *w_bytes,
+                                           size_t *a_end, size_t *a_bytes) {
+    PG_CHECK_ARG(m > 0 && k > 0 && n > 0 && mb > 0 && nb_tiles > 0 && nw > 0, "pg_audit_gemm_w8a8_skinny: bad arguments");
+    PG_CHECK_ARG((size_t)16 * mb >= m, "pg_audit_gemm_w8a8_skinny: %d activation tiles for %zu rows", mb, m);
+    const size_t k_pad = pg_round_up(k, PG_KPAD), n_pad = pg_round_up(n, PG_NPAD), m_pad = pg_round_up(m, PG_MPAD);
+    span_check w, a;
+    const int wgs = (int)((n + 16 * nb_tiles - 1) / (16 * nb_tiles));
+    const int units = (int)(k_pad / 128), per = (units + nw - 1) / nw;
+    for (int wg = 0; wg < wgs; ++wg) {
+        const int n0 = wg * 16 * nb_tiles;
+        for (int wave = 0; wave < nw; ++wave) {
+            const int u_begin = wave * per, u_end = std::min(u_begin + per, units), cnt = u_end - u_begin;
+            if (cnt <= 0) continue;
+            const int rot = (int)(((unsigned)wg * 5u) % (unsigned)cnt);
+            for (int t = 0; t < cnt; ++t) {
+                const int unit = pg_skinny_walk_unit(u_begin, cnt, t, rot);
+                for (int lane = 0; lane < 64; ++lane)
+                    for (int j = 0; j < 2; ++j) {
+                        const int r = 8 * j + (lane >> 3), ch = (lane & 7) ^ ((r >> 1) & 7);
+                        for (int c = 0; c < nb_tiles; ++c) w.touch(pg_skinny_fill_offset(n0 + 16 * c + r, (int)k_pad, unit, ch), 16);
+                        for (int b = 0; b < mb; ++b) a.touch(pg_skinny_fill_offset(16 * b + r, (int)k_pad, unit, ch), 16);
+                    }
+            }
+        }
+    }
+    if (w_end) *w_end = w.end;
+    if (w_bytes) *w_bytes = n_pad * k_pad;
+    if (a_end) *a_end = a.end;
+    if (a_bytes) *a_bytes = m_pad * k_pad;
+    return PG_OK;
+}
+
+// One-row block products (gguf_gemv_kernel<QT, BPL, RW, R, ..., NW> and the few-rows form): the payload plane
+// [n_out][nh][nb][16 B] (nh = 2 for Q8_0, else 1) and the scale plane [ceil(n_out / 8)][nb][8 x f16].
+// bpl = blocks per lane and K segment, rw = rows per wavefront, nw = wavefronts per workgroup.
+PG_API pg_status pg_audit_gguf_gemv(size_t n_out, size_t k_in, int q8, int bpl, int rw, int nw, size_t *qs_end, size_t *qs_bytes,
+                                    size_t *d_end, size_t *d_bytes) {
+    PG_CHECK_ARG(n_out > 0 && k_in >= 32 && k_in % 32 == 0 && bpl >= 1 && bpl <= 4 && rw > 0 && nw > 0, "pg_audit_gguf_gemv: bad arguments");
+    const int nb = (int)(k_in / 32), nh = q8 ? 2 : 1, seg = 64 * bpl;
+    span_check qs, d;
+    const int wgs = (int)((n_out + (size_t)rw * nw - 1) / ((size_t)rw * nw));
+    for (int wg = 0; wg < wgs; ++wg)
+        for (int wave = 0; wave < nw; ++wave) {
+            const int row0 = (wg * nw + wave) * rw;
+            const bool live = (size_t)row0 < n_out;  // the wavefronts with no row of their own load no weights
+            if (!live) continue;
+            for (int seg0 = 0; seg0 < nb; seg0 += seg) {
+                const int seg_n = std::min(nb - seg0, seg);
+                for (int lane = 0; lane < 64; ++lane)
+                    for (int p = 0; p < bpl; ++p) {
+                        const int blk = pg_gemv_lane_block(seg0, lane, p, seg_n);
+                        d.touch(pg_gemv_scale_unit(row0, nb, blk) * 16, 16);
+                        for (int r = 0; r < rw; ++r) {
+                            const int row = pg_gemv_clamp_row(row0 + r, (int)n_out);
+                            for (int h = 0; h < nh; ++h) qs.touch(pg_gemv_weight_unit(row, h, nh, nb, blk) * 16, 16);
+                        }
+                    }
+            }
+        }
+    if (qs_end) *qs_end = qs.end;
+    if (qs_bytes) *qs_bytes = n_out * (size_t)nb * nh * 16;
+    if (d_end) *d_end = d.end;
+    if (d_bytes) *d_bytes = (n_out + 7) / 8 * 8 * (size_t)nb * sizeof(uint16_t);
+    return PG_OK;
+}
+
+// 2 .. 16 rows in one launch over a block tensor (gguf_skinny_kernel<QT, 1, MT, NW, NST>): K in units of 8 blocks
+// (k_in % 256 == 0), a workgroup of nw wavefronts per 16 weight rows.
+PG_API pg_status pg_audit_gguf_skinny(size_t n_out, size_t k_in, int q8, int nw, size_t *qs_end, size_t *qs_bytes, size_t *d_end,
+                                      size_t *d_bytes) {
+    PG_CHECK_ARG(n_out > 0 && k_in >= 256 && k_in % 256 == 0 && nw > 0, "pg_audit_gguf_skinny: bad arguments");
+    const int nb = (int)(k_in / 32), wf = q8 ? 4 : 2, units = nb / 8, per = (units + nw - 1) / nw, ntile = (int)((n_out + 7) / 8);
+    span_check qs, d;
+    const int wgs = (int)((n_out + 15) / 16);
+    for (int wg = 0; wg < wgs; ++wg) {
+        const int n0 = wg * 16;
+        for (int wave = 0; wave < nw; ++wave) {
+            const int u_begin = wave * per, u_end = std::min(u_begin + per, units), cnt = u_end - u_begin;
+            if (cnt <= 0) continue;
+            const int rot = (int)(((unsigned)wg * 5u) % (unsigned)cnt);
+            for (int t = 0; t < cnt; ++t) {
+                const int unit = pg_skinny_walk_unit(u_begin, cnt, t, rot);
+                for (int lane = 0; lane < 64; ++lane) {
+                    for (int j = 0; j < wf; ++j) {
+                        const int slot = 8 * j + (lane >> 3), r = slot & 15, half = slot >> 4, ch = (lane & 7) ^ ((r >> 1) & 7);
+                        const int row = pg_gemv_clamp_row(n0 + r, (int)n_out);
+                        qs.touch(pg_gskinny_weight_offset(q8 ? (size_t)row * 2 + half : (size_t)row, nb, unit, ch), 16);
+                    }
+                    if (lane < 16) d.touch(pg_gskinny_scale_offset(pg_gskinny_scale_tile(n0, lane, ntile), nb, unit, lane), 16);
+                }
+            }
+        }
+    }
+    if (qs_end) *qs_end = qs.end;
+    if (qs_bytes) *qs_bytes = n_out * (size_t)nb * (q8 ? 32 : 16);
+    if (d_end) *d_end = d.end;
+    if (d_bytes) *d_bytes = (n_out + 7) / 8 * 8 * (size_t)nb * sizeof(uint16_t);
+    return PG_OK;
+}
+
+// MXFP4 rows (mxfp4_rows_kernel<T, RG, NW>): the fragment-major code plane [row groups of 16][ncp chunks][64 lanes][16 B]
+// and the scale plane [row groups][ncp / 4][64 lanes][4 B]; a wavefront = (row group, K slice), 8 chunks per batch of loads.
+PG_API pg_status pg_audit_mxfp4_rows(size_t out_dim, size_t in_dim, int rg_per_wg, int nw, size_t *qs_end, size_t *qs_bytes,
+                                     size_t *sc_end, size_t *sc_bytes) {
+    PG_CHECK_ARG(out_dim > 0 && in_dim >= 32 && in_dim % 32 == 0 && rg_per_wg > 0 && nw >= rg_per_wg && nw % rg_per_wg == 0, "pg_audit_mxfp4_rows: bad arguments");
+    const int nb = (int)(in_dim / 32), ncp = (int)((((size_t)nb + 3) / 4 + 3) & ~(size_t)3), nrg = (int)((out_dim + 15) / 16), ks = nw / rg_per_wg;
+    const int mx_u = 8;
+    span_check qs, sc;
+    const int wgs = (nrg + rg_per_wg - 1) / rg_per_wg;
+    const int cps = ((ncp + ks - 1) / ks + 3) & ~3;
+    for (int wg = 0; wg < wgs; ++wg)
+        for (int wave = 0; wave < nw; ++wave) {
+            const int rgi = wave / ks, ksi = wave % ks;
+            int rg = wg * rg_per_wg + rgi;
+            rg = rg < nrg ? rg : nrg - 1;
+            const int c0 = ksi * cps, c1 = std::min(c0 + cps, ncp);
+            auto batch = [&](int cb) {
+                for (int lane = 0; lane < 64; ++lane) {
+                    for (int u = 0; u < mx_u; ++u) qs.touch((((size_t)rg * ncp + pg_mx_chunk(cb + u, ncp)) * 64 + lane) * 16, 16);
+                    for (int g = 0; g < mx_u / 4; ++g) sc.touch((((size_t)rg * (ncp / 4) + pg_mx_scale_word(cb + 4 * g, ncp)) * 64 + lane) * 4, 4);
+                }
+            };
+            batch(c0 < ncp ? c0 : 0);
+            for (int cb = c0; cb < c1; cb += 2 * mx_u) {
+                if (cb + mx_u < c1) batch(cb + mx_u);
+                if (cb + 2 * mx_u < c1) batch(cb + 2 * mx_u);
+            }
+        }
+    if (qs_end) *qs_end = qs.end;
+    if (qs_bytes) *qs_bytes = (size_t)nrg * ncp * 64 * 16;
+    if (sc_end) *sc_end = sc.end;
+    if (sc_bytes) *sc_bytes = (size_t)nrg * (ncp / 4) * 64 * 4;
+    return PG_OK;
+}
+
+// The read-stream probe (probe_read_kernel<U>): `total` 16-byte chunks cut into one slice per workgroup.
+PG_API pg_status pg_audit_probe_read(size_t bytes, int workgroups, int threads, int loads_in_flight, size_t *end, size_t *alloc) {
+    PG_CHECK_ARG(bytes >= 16 && workgroups > 0 && threads > 0 && loads_in_flight > 0, "pg_audit_probe_read: bad arguments");
+    const size_t total = bytes / 16, cpw = (total + workgroups - 1) / workgroups;
+    span_check s;
+    for (int wg = 0; wg < workgroups; ++wg) {
+        const size_t first = (size_t)wg * cpw;
+        const size_t n = first >= total ? 0 : std::min(total - first, cpw);
+        for (int t = 0; t < threads; ++t)
+            for (size_t c = t; c < n; c += (size_t)loads_in_flight * threads)
+                for (int u = 0; u < loads_in_flight; ++u) {
+                    const size_t i = pg_probe_chunk(c, u, (unsigned)threads);
+                    if (i < n) s.touch((first + i) * 16, 16);
+                }
+    }
+    if (end) *end = s.end;
+    if (alloc) *alloc = total * 16;
+    return PG_OK;
+}

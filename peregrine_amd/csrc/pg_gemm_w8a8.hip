@@ -28,6 +28,7 @@
 // MFMAs.
 #include <limits.h>
 #include "pg_internal.h"
+#include "pg_stream_addr.h"
 
 namespace {
 
@@ -465,9 +466,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_w8a8_skinny_kernel(const int8_t 
     for (int j = 0; j < 2; ++j) {
         const int r = 8 * j + (lane >> 3), ch = (lane & 7) ^ ((r >> 1) & 7);
 #pragma unroll
-        for (int c = 0; c < NB; ++c) src[c][j] = w_t + (size_t)(n0 + 16 * c + r) * k_pad + ch * 16;  // (weight rows are padded to 256)
+        for (int c = 0; c < NB; ++c) src[c][j] = w_t + pg_skinny_fill_offset(n0 + 16 * c + r, k_pad, 0, ch);  // (weight rows are padded to 256)
 #pragma unroll
-        for (int b = 0; b < MB; ++b) src[NB + b][j] = a_i8 + (size_t)(16 * b + r) * k_pad + ch * 16;
+        for (int b = 0; b < MB; ++b) src[NB + b][j] = a_i8 + pg_skinny_fill_offset(16 * b + r, k_pad, 0, ch);
     }
     // fragment reads: row lane % 16, chunk 4 s + lane / 16 of k-step s
     const int fr = lane & 15, fsw = (fr >> 1) & 7;
@@ -476,8 +477,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_w8a8_skinny_kernel(const int8_t 
     for (int st = 0; st < 2; ++st) rd[st] = fr * 128 + (((4 * st + (lane >> 4)) ^ fsw) * 16);
     const int rot = cnt > 0 ? (int)((blockIdx.x * 5u) % (unsigned)cnt) : 0;
     auto issue = [&](auto slot, int t) {  // t-th unit of the walk into ring slot `slot`
-        const int r = t + rot;
-        const size_t kb = (size_t)(u_begin + (r >= cnt ? r - cnt : r)) * 128;
+        const size_t kb = (size_t)pg_skinny_walk_unit(u_begin, cnt, t, rot) * 128;
         char *base = ring + decltype(slot)::value * UNIT;
 #pragma unroll
         for (int q = 0; q < NB; ++q)  // the weights: used once, non-temporal

@@ -19,6 +19,7 @@
 #include <mutex>
 #include <new>
 #include "pg_internal.h"
+#include "pg_stream_addr.h"
 #include "pg_digits.h"
 
 namespace {
@@ -292,17 +293,16 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
         const int seg_n = (nb - seg0 < SEG) ? nb - seg0 : SEG;
         int blk[BPL];  // this lane's blocks; lanes past the segment end re-read block seg0 with a zero scale
 #pragma unroll
-        for (int p = 0; p < BPL; ++p) blk[p] = seg0 + (lane + 64 * p < seg_n ? lane + 64 * p : 0);
+        for (int p = 0; p < BPL; ++p) blk[p] = pg_gemv_lane_block(seg0, lane, p, seg_n);
         auto load_rows = [&](RowLoads<QT, BPL, R> &L, int g) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                int row = row0 + (g % NG) * R + r;
-                row = row < n_out ? row : n_out - 1;  // clamped; masked at the store
+                const int row = pg_gemv_clamp_row(row0 + (g % NG) * R + r, n_out);  // clamped; masked at the store
 #pragma unroll
                 for (int p = 0; p < BPL; ++p)
 #pragma unroll
                     for (int h = 0; h < NH; ++h)
-                        L.w[r][p][h] = __builtin_nontemporal_load(qs_t[NT == 1 ? 0 : g / NG] + ((size_t)row * NH + h) * nb + blk[p]);
+                        L.w[r][p][h] = __builtin_nontemporal_load(qs_t[NT == 1 ? 0 : g / NG] + pg_gemv_weight_unit(row, h, NH, nb, blk[p]));
             }
         };
         // Loads return in issue order, so the (L2 / L1 resident) digits, block sums and scales
@@ -331,7 +331,7 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
             }
             if (live) {
 #pragma unroll
-                for (int p = 0; p < BPL; ++p) dtile[0][p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+                for (int p = 0; p < BPL; ++p) dtile[0][p] = dsc[pg_gemv_scale_unit(row0, nb, blk[p])];
                 load_rows(L[0], 0);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -364,14 +364,14 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_kernel(
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int b = b0 + u * 8 * NW;
-                    xv[u] = reinterpret_cast<const float4 *>(x_f32)[(size_t)(b < nb ? b : 0) * 8 + sub];
-                    if constexpr (NORM) gv[u] = reinterpret_cast<const float4 *>(epi.gamma)[(size_t)(b < nb ? b : 0) * 8 + sub];
+                    xv[u] = reinterpret_cast<const float4 *>(x_f32)[(size_t)pg_gemv_x_block(b, nb) * 8 + sub];
+                    if constexpr (NORM) gv[u] = reinterpret_cast<const float4 *>(epi.gamma)[(size_t)pg_gemv_x_block(b, nb) * 8 + sub];
                 }
             };
             if (seg0 == 0) fetch(bfirst);
             if (live) {
 #pragma unroll
-                for (int p = 0; p < BPL; ++p) dtile[0][p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+                for (int p = 0; p < BPL; ++p) dtile[0][p] = dsc[pg_gemv_scale_unit(row0, nb, blk[p])];
                 load_rows(L[0], 0);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -541,14 +541,13 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_fewrows_kernel(const uint8_
         const int seg_n = (nb - seg0 < SEG) ? nb - seg0 : SEG;
         int blk[BPL];  // this lane's blocks; lanes past the segment end re-read block seg0 with a zero scale
 #pragma unroll
-        for (int p = 0; p < BPL; ++p) blk[p] = seg0 + (lane + 64 * p < seg_n ? lane + 64 * p : 0);
+        for (int p = 0; p < BPL; ++p) blk[p] = pg_gemv_lane_block(seg0, lane, p, seg_n);
         auto load_rows = [&](RowLoads<4, BPL, R> &L, int g) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                int row = row0 + g * R + r;
-                row = row < n_out ? row : n_out - 1;  // clamped; masked at the store
+                const int row = pg_gemv_clamp_row(row0 + g * R + r, n_out);  // clamped; masked at the store
 #pragma unroll
-                for (int p = 0; p < BPL; ++p) L.w[r][p][0] = __builtin_nontemporal_load(qs + (size_t)row * nb + blk[p]);
+                for (int p = 0; p < BPL; ++p) L.w[r][p][0] = __builtin_nontemporal_load(qs + pg_gemv_weight_unit(row, 0, 1, nb, blk[p]));
             }
         };
         v4i dtile[BPL];
@@ -568,7 +567,7 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_fewrows_kernel(const uint8_
             fetch(bfirst);
             if (live) {
 #pragma unroll
-                for (int p = 0; p < BPL; ++p) dtile[p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+                for (int p = 0; p < BPL; ++p) dtile[p] = dsc[pg_gemv_scale_unit(row0, nb, blk[p])];
                 load_rows(L[0], 0);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -592,7 +591,7 @@ __global__ __launch_bounds__(64 * NW) void gguf_gemv_fewrows_kernel(const uint8_
             if (!live) return;  // after the workgroup's only barrier
         } else {
 #pragma unroll
-            for (int p = 0; p < BPL; ++p) dtile[p] = dsc[(size_t)(row0 >> 3) * nb + blk[p]];
+            for (int p = 0; p < BPL; ++p) dtile[p] = dsc[pg_gemv_scale_unit(row0, nb, blk[p])];
             load_rows(L[0], 0);
         }
         __builtin_amdgcn_sched_barrier(0);

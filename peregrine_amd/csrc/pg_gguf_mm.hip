@@ -18,6 +18,7 @@
 // token digits and scales of the stage, which the four wavefronts share.
 #include <limits.h>
 #include "pg_internal.h"
+#include "pg_stream_addr.h"
 #include "pg_digits.h"
 
 namespace {
@@ -565,13 +566,13 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
         for (int j = 0; j < WF; ++j) {
             const int slot = 8 * j + (lane >> 3), r = slot & 15, half = slot >> 4, ch = (lane & 7) ^ ((r >> 1) & 7);
-            const int row = n0 + 16 * c + r < n_out ? n0 + 16 * c + r : n_out - 1;
-            w_src[c][j] = qs + (QT == 8 ? (size_t)row * 2 + half : (size_t)row) * nb * 16 + ch * 16;
+            const int row = pg_gemv_clamp_row(n0 + 16 * c + r, n_out);
+            w_src[c][j] = qs + pg_gskinny_weight_offset(QT == 8 ? (size_t)row * 2 + half : (size_t)row, nb, 0, ch);
         }
     // scales: lanes 0 .. 16 NB - 1: scale tile (n0 / 8 + lane / 8), blocks of the unit lane % 8 (16 bytes = 8 rows x f16)
     const int ntile = (n_out + 7) / 8;
-    const int dt = (n0 >> 3) + (lane >> 3) < ntile ? (n0 >> 3) + (lane >> 3) : ntile - 1;
-    const char *d_src = reinterpret_cast<const char *>(dsc) + ((size_t)dt * nb + (lane & 7)) * 16;
+    const int dt = pg_gskinny_scale_tile(n0, lane, ntile);
+    const char *d_src = reinterpret_cast<const char *>(dsc) + pg_gskinny_scale_offset(dt, nb, 0, lane);
     // digits: instruction q covers runs 4 q .. 4 q + 3, run = 2 token + plane; lane -> run 4 q + lane / 16, position lane % 16
     const int8_t *g_src[GQ];
 #pragma unroll
@@ -585,8 +586,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
     const int rot = cnt > 0 ? (int)((blockIdx.x * 5u) % (unsigned)cnt) : 0;
     auto issue = [&](auto slot, int t) {
-        const int r = t + rot;
-        const size_t unit = (size_t)(u_begin + (r >= cnt ? r - cnt : r));
+        const size_t unit = (size_t)pg_skinny_walk_unit(u_begin, cnt, t, rot);
         char *base = ring + decltype(slot)::value * UNIT;
 #pragma unroll
         for (int c = 0; c < NB; ++c)

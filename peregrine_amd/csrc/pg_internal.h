@@ -91,6 +91,7 @@ constexpr size_t PG_MM_MIN_BLOCKS = 5;
 constexpr int PG_GEMM_MAX_GROUP = 4;  // weights one W8A8 launch can carry (fused q|k|v, gate|up)
 constexpr size_t PG_KPAD = 128;  // device K stride is a multiple of this
 constexpr size_t PG_NPAD = 256;  // device weight rows are padded to this
+constexpr size_t PG_MPAD = 256;  // quantised activation rows in the workspace are padded to this
 
 static inline size_t pg_round_up(size_t v, size_t m) { return (v + m - 1) / m * m; }
 

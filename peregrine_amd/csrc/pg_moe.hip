@@ -208,10 +208,19 @@ static pg_status moe_ffn_core(pg_ctx *ctx, const float *x_dev, size_t T, const f
         host_tab[4 * E + e] = down_stream ? down[e]->qs : down[e]->qs_tiled; host_tab[5 * E + e] = down[e]->d;
     }
     const void **tab = nullptr;
-    for (const auto &t : ctx->moe_tabs)
-        if (t.host.size() == 6 * E && memcmp(t.host.data(), host_tab, 6 * E * sizeof(void *)) == 0) tab = static_cast<const void **>(t.dev);
+    for (size_t i = 0; i < ctx->moe_tabs.size(); ++i) {
+        auto &t = ctx->moe_tabs[i];
+        if (t.host.size() == 6 * E && memcmp(t.host.data(), host_tab, 6 * E * sizeof(void *)) == 0) {
+            tab = static_cast<const void **>(t.dev);
+            if (i + 1 != ctx->moe_tabs.size()) std::rotate(ctx->moe_tabs.begin() + i, ctx->moe_tabs.begin() + i + 1, ctx->moe_tabs.end());  // most recent last
+            break;
+        }
+    }
     if (!tab) {
-        if (ctx->moe_tabs.size() >= 64) {  // a bounded cache: drop the oldest set once nothing can still read it
+        // Least recently used out first.  A layer has two sets (row-major planes for one token, tile-major ones for
+        // more), and a model alternates its layers: 512 sets hold both for 256 layers (the reference's Grok-1 has 64,
+        // examples/grok1/model.rs:35), so a decode loop after a prefill misses on no layer.
+        if (ctx->moe_tabs.size() >= 512) {  // a bounded cache: drop a set once nothing can still read it
             PG_HIP(hipStreamSynchronize(ctx->stream));
             (void)hipFree(ctx->moe_tabs.front().dev);
             ctx->moe_tabs.erase(ctx->moe_tabs.begin());

@@ -20,6 +20,7 @@
 #include <mutex>
 
 #include "pg_internal.h"
+#include "pg_stream_addr.h"
 #include "pg_digits.h"
 
 namespace {
@@ -152,12 +153,12 @@ __global__ __launch_bounds__(64 * NW) void mxfp4_rows_kernel(const uint8_t *__re
 #pragma unroll
         for (int u = 0; u < MX_U; ++u) {
             const int c = cb + u;
-            a[u] = __builtin_nontemporal_load(qa + (size_t)(c < ncp ? c : ncp - 1) * 64);
+            a[u] = __builtin_nontemporal_load(qa + (size_t)pg_mx_chunk(c, ncp) * 64);
         }
 #pragma unroll
         for (int g = 0; g < MX_U / 4; ++g) {
             const int c = cb + 4 * g;
-            s[g] = sa[(size_t)((c < ncp ? c : ncp - 4) >> 2) * 64];
+            s[g] = sa[(size_t)pg_mx_scale_word(c, ncp) * 64];
         }
     };
     // Loads return in issue order: the activation blocks of the first rounds (from L2) are requested

@@ -498,7 +498,6 @@ PG_API void pg_qtensor_free(pg_ctx *ctx, pg_qtensor *t) {
 
 // Rows of the quantised-activation scratch are padded to this many so the GEMM
 // tiles never read past the arena.
-constexpr size_t PG_MPAD = 256;
 // At or below this many activation rows the weight stream, not the matrix cores,
 // bounds the product: use the dot-product GEMV kernel.
 constexpr size_t PG_GEMV_MAX_M = 4;
@@ -701,7 +700,8 @@ PG_API pg_status pg_matmul_dequant_i8_dev(pg_ctx *ctx, const float *a_dev, size_
     if (m == 0) return PG_OK;
     PG_CHECK_ARG(a_dev && out_dev, "pg_matmul_dequant_i8: null pointer");
     PG_CHECK_ARG(m < (1ull << 24), "pg_matmul_dequant_i8: m = %zu too large", m);
-    PG_CHECK_ARG(k <= 133000, "pg_matmul_dequant_i8: k = %zu would overflow the i32 digit sums", k);  // 127 * 127 * k < 2^31
+    // a digit plane holds -128 .. 127 (the carry-free split yields -128), a weight -127 .. 127: 128 * 127 * k < 2^31
+    PG_CHECK_ARG(k <= 132104, "pg_matmul_dequant_i8: k = %zu would overflow the i32 digit sums", k);
     const size_t m_pad = pg_round_up(m, PG_MPAD), n = w->cols;
     // With enough rows the two low digit planes run as ONE product over the planes stacked row-wise (they lie
     // back to back in the scratch, each m_pad rows; the accumulator planes are then m_pad rows apart) and

@@ -31,3 +31,42 @@ PG_HD int pg_m1_x_vec(int thread, int i, int nt, int nvec) {
 }
 // first weight row of a wavefront: workgroup `wg` of its weight, NW wavefronts of RPW rows each
 PG_HD int pg_m1_row0(int wg, int wave, int nw, int rpw) { return (wg * nw + wave) * rpw; }
+
+// ---- block-quantised one-row products (gguf_gemv_kernel and its forms)
+// block of the K segment [seg0, seg0 + seg_n) that lane `lane` takes as its p-th: a lane past the segment's end
+// reads the segment's first block again (with a zero scale)
+PG_HD int pg_gemv_lane_block(int seg0, int lane, int p, int seg_n) {
+    const int b = lane + 64 * p;
+    return seg0 + (b < seg_n ? b : 0);
+}
+// weight row a wavefront reads for output row `row`: rows past the tensor repeat its last (masked at the store)
+PG_HD int pg_gemv_clamp_row(int row, int n_out) { return row < n_out ? row : n_out - 1; }
+// 16-byte unit of the payload plane: half `h` of NH (Q8_0: 2 half-blocks, else 1) of block `blk` of row `row`
+PG_HD size_t pg_gemv_weight_unit(int row, int h, int nh, int nb, int blk) { return ((size_t)row * nh + h) * nb + blk; }
+// 16-byte unit of the scale plane (8 rows x f16 per block): the tile of row0's eight rows, block `blk`
+PG_HD size_t pg_gemv_scale_unit(int row0, int nb, int blk) { return (size_t)(row0 >> 3) * nb + blk; }
+// block of the f32 activation row a digit-making thread fetches: past the row, its first
+PG_HD int pg_gemv_x_block(int b, int nb) { return b < nb ? b : 0; }
+
+// ---- few rows in one launch over int8 weights (gemm_w8a8_skinny_kernel): a wavefront walks its run of K units
+// (128 bytes of K each) from a start that differs per workgroup and wraps round
+PG_HD int pg_skinny_walk_unit(int u_begin, int cnt, int t, int rot) {
+    const int r = t + rot;
+    return u_begin + (r >= cnt ? r - cnt : r);
+}
+// byte offset of a 16-byte fill in a [rows][k_pad] plane: row, K unit, chunk within the unit's 128 bytes
+PG_HD size_t pg_skinny_fill_offset(int row, int k_pad, int unit, int ch) { return (size_t)row * k_pad + (size_t)unit * 128 + (size_t)ch * 16; }
+
+// ---- few rows in one launch over block tensors (gguf_skinny_kernel): units of 8 blocks
+// byte offset of a 16-byte fill of the payload plane: stream row (Q8_0: 2 row + half), unit, chunk = block within the unit
+PG_HD size_t pg_gskinny_weight_offset(size_t stream_row, int nb, int unit, int ch) { return stream_row * nb * 16 + (size_t)unit * 128 + (size_t)ch * 16; }
+// scale tile (8 rows) a lane group fetches: past the tensor's last tile, the last
+PG_HD int pg_gskinny_scale_tile(int n0, int lane, int ntile) {
+    const int t = (n0 >> 3) + (lane >> 3);
+    return t < ntile ? t : ntile - 1;
+}
+PG_HD size_t pg_gskinny_scale_offset(int tile, int nb, int unit, int lane) { return ((size_t)tile * nb + (lane & 7)) * 16 + (size_t)unit * 128; }
+
+// ---- MXFP4 rows (mxfp4_rows_kernel): fragment chunk and scale word a wavefront fetches for chunk index c
+PG_HD int pg_mx_chunk(int c, int ncp) { return c < ncp ? c : ncp - 1; }
+PG_HD int pg_mx_scale_word(int c, int ncp) { return (c < ncp ? c : ncp - 4) >> 2; }

@@ -25,7 +25,15 @@ class Hip:
     """The four runtime calls a capture needs, from the HIP runtime the library itself is linked with."""
 
     def __init__(self):
-        self.lib = C.CDLL("libamdhip64.so")
+        # the copy of the runtime that is already mapped into this process (torch's, which the library bound to): a bare
+        # name could resolve to another file and put a second runtime beside it
+        path = "libamdhip64.so"
+        with open("/proc/self/maps") as maps:
+            for line in maps:
+                if "libamdhip64" in line:
+                    path = line.split()[-1]
+                    break
+        self.lib = C.CDLL(path)
         for name, args in (("hipStreamBeginCapture", [C.c_void_p, C.c_int]), ("hipStreamEndCapture", [C.c_void_p, C.POINTER(C.c_void_p)]),
                            ("hipGraphInstantiate", [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
                            ("hipGraphLaunch", [C.c_void_p, C.c_void_p]), ("hipGraphExecDestroy", [C.c_void_p]),
