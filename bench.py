@@ -185,12 +185,20 @@ class Bench:
         self.check(self.lib.pg_probe_mfma_i8(self.h, 20000, C.byref(tops), C.byref(ghz)))
         self.check(self.lib.pg_probe_hbm_read(self.h, 256 << 20, 3, 30, C.byref(gbs)))
         self.check(self.lib.pg_probe_gemm_clock(self.h, 2048, 4096, 14336, C.byref(g_ghz), C.byref(loop_us)))
+        # a pure read of one launch's bytes, best of a few launch shapes (workgroups, threads, loads in flight):
+        # what a one-row product of that size could reach if it did nothing but read
         small = {}
-        for label, nbytes, bufs in (("33MB", 33103872, 10), ("59MB", 58851328, 6)):  # cfg4's and cfg2's largest launches
-            g = C.c_double()
-            self.check(self.lib.pg_probe_hbm_read(self.h, nbytes, bufs, 300, C.byref(g)))
-            small[label] = round(g.value, 1)
-        return {"hbm_read_stream_per_launch_size_gbs": small,"int8_mfma_registers_only_tops": round(tops.value, 1), "its_shader_clock_ghz": round(ghz.value, 3),
+        shapes = ((4096, 256, 4), (2048, 512, 4), (2048, 256, 8), (1024, 512, 8), (1024, 256, 16), (512, 1024, 4))
+        for label, nbytes, bufs in (("33MB", 33103872, 10), ("59MB", 58851328, 6), ("118MB", 117702656, 4)):
+            best = (0.0, None)   # cfg4's largest launch, cfg2's down, cfg2's gate|up
+            for wgs, thr, inflight in shapes:
+                g = C.c_double()
+                self.check(self.lib.pg_probe_hbm_read_shaped(self.h, nbytes, bufs, 200, wgs, thr, inflight, C.byref(g)))
+                if g.value > best[0]:
+                    best = (g.value, (wgs, thr, inflight))
+            small[label] = {"gbs": round(best[0], 1), "us": round(nbytes / best[0] / 1e3, 2),
+                            "workgroups_threads_loads_in_flight": list(best[1])}
+        return {"hbm_read_stream_per_launch_size": small, "int8_mfma_registers_only_tops": round(tops.value, 1), "its_shader_clock_ghz": round(ghz.value, 3),
                 "hbm_read_stream_gbs": round(gbs.value, 1), "gemm_tile_shader_clock_ghz": round(g_ghz.value, 3),
                 "gemm_tile_k_loop_us": round(loop_us.value, 2),
                 "int8_peak_at_gemm_clock_tops": round(256 * 8192 * g_ghz.value / 1e3, 1),

@@ -158,6 +158,7 @@ extern "C" {
     pub fn pg_gemm_w8a8_last_tile(ctx: *const pg_ctx, bm: *mut c_int, bn: *mut c_int, k_splits: *mut c_int) -> pg_status;
     pub fn pg_gemm_w8a8_force_tile(ctx: *mut pg_ctx, tile: c_int) -> pg_status;
     pub fn pg_gemv_w8a8_force_shape(ctx: *mut pg_ctx, wavefronts: c_int, rows_per_wavefront: c_int) -> pg_status;
+    pub fn pg_gguf_hmm_force(ctx: *mut pg_ctx, mode: c_int) -> pg_status;
     pub fn pg_audit_gemv_w8a8_m1(k: usize, n: usize, nch: c_int, rows_per_wavefront: c_int, wavefronts: c_int, f32_row: c_int, w_end: *mut usize, w_bytes: *mut usize, x_end: *mut usize, x_bytes: *mut usize) -> pg_status;
     pub fn pg_audit_gemm_w8a8_skinny(m: usize, k: usize, n: usize, activation_tiles: c_int, weight_tiles: c_int, wavefronts: c_int, w_end: *mut usize, w_bytes: *mut usize, a_end: *mut usize, a_bytes: *mut usize) -> pg_status;
     pub fn pg_audit_gguf_gemv(n_out: usize, k_in: usize, q8: c_int, blocks_per_lane: c_int, rows_per_wavefront: c_int, wavefronts: c_int, qs_end: *mut usize, qs_bytes: *mut usize, d_end: *mut usize, d_bytes: *mut usize) -> pg_status;

@@ -525,6 +525,12 @@ pg_status pg_gemm_w8a8_force_tile(pg_ctx *ctx, int tile);
  * 16; weight rows per wavefront 1 or 2, not 16 x 2) instead of the dispatcher's choice by row length; 0, 0 =
  * automatic.  Every shape gives the same bits. */
 pg_status pg_gemv_w8a8_force_shape(pg_ctx *ctx, int wavefronts, int rows_per_wavefront);
+/* The many-row Q4_0 product has two matrix-core routes: the int8 block product with 16-bit fixed-point activations
+ * per block, and, from about a hundred rows on where the launch fills the part, f16 tiles with the weights unpacked
+ * in registers and the activations as two f16 planes per row.  mode 0 = the dispatcher chooses, 1 = the f16 route
+ * wherever it can run (Q4_0, K a multiple of 64, at least two rows), 2 = never.  Both keep the weights exact; they
+ * round the activations differently (2^-22 of the row's largest value against 2^-16 of the block's). */
+pg_status pg_gguf_hmm_force(pg_ctx *ctx, int mode);
 
 /* Address audit of the streaming kernels, on the host (no device is touched): each function walks every
  * (workgroup, wavefront, lane, step) of one launch of the named kernel shape with the very index functions the

@@ -74,6 +74,7 @@ SIGNATURES = {
     "pg_audit_probe_read": [_sz, _int, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "pg_gemm_w8a8_force_tile": [_vp, _int],
     "pg_gemv_w8a8_force_shape": [_vp, _int, _int],
+    "pg_gguf_hmm_force": [_vp, _int],
     "pg_matmul_dequant_i8": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_matmul_dequant_i8_dev": [_vp, _vp, _sz, _sz, _vp, _vp],
     "pg_f16_to_f32": [_vp, _vp, _sz, _vp],

@@ -1005,6 +1005,22 @@ pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w) {
     return PG_OK;
 }
 
+// `count` Q4_0 products over the same many rows on the f16 matrix cores: the rows become two f16 planes once,
+// tensors of the same launch shape share a launch (up to PG_HMM_MAX_GROUP).
+static pg_status pg_gguf_hmm_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *const *w, float *const *y_dev,
+                                  int count, int ks) {
+    const size_t k_in = w[0]->k_in;
+    size_t n_total = 0;
+    for (int i = 0; i < count; ++i) n_total += w[i]->n_out;
+    const size_t sz_p = pg_hmm_planes_bytes(m, k_in), sz_part = pg_round_up(pg_gguf_hmm_part_floats(m, n_total, ks) * sizeof(float), 256);
+    void *ws = nullptr;
+    PG_TRY(pg_workspace(ctx, sz_p + sz_part, &ws));
+    const pg_hmm_planes planes = pg_hmm_planes_carve(ws, m, k_in);
+    float *part = ks > 1 ? reinterpret_cast<float *>(static_cast<char *>(ws) + sz_p) : nullptr;
+    PG_TRY(pg_launch_rows_to_f16_planes(ctx, x_dev, m, k_in, planes));
+    return pg_launch_gguf_hmm_group(ctx, k_in, w, y_dev, count, m, planes, ks, part);
+}
+
 // Quantise `m` activation rows (device) into the arena and run the fused product: the
 // streaming GEMV for one row, the matrix-core kernel (weights read once) for more.
 pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
@@ -1021,6 +1037,9 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
         }
         return pg_launch_mxfp4_rows(ctx, x_dev, m, w, y_dev);
     }
+    int hks = 1;
+    if (ctx->hmm_mode == 1 && pg_gguf_hmm_takes(ctx, w->ggml_type, m, w->n_out, w->k_in, &hks))  // forced (pg_gguf_hmm_force)
+        return pg_gguf_hmm_rows(ctx, x_dev, m, &w, &y_dev, 1, hks);
     // a K of a few blocks needs the streaming kernel's finer fixed point; so do up to seven rows of Q4_1 (its
     // matrix-core route is three launches more than the streaming one: 27 against 19 us at four rows of 4096 ->
     // 14336, 35 against 59 at sixteen) and Q4_1 rows too long for the offset kernel
@@ -1043,6 +1062,8 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
         PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, m, w->k_in, w->ggml_type, md));
         return pg_launch_gguf_skinny_group(ctx, w->ggml_type, w->k_in, &w, &y_dev, 1, m, md);
     }
+    if (pg_gguf_hmm_takes(ctx, w->ggml_type, m, w->n_out, w->k_in, &hks))  // many rows of Q4_0: the f16 matrix cores
+        return pg_gguf_hmm_rows(ctx, x_dev, m, &w, &y_dev, 1, hks);
     const int ks = pg_gguf_mm_splitk(ctx, w->n_out, w->k_in, (m + 31) / 32, m, false, nullptr);
     const size_t sz_d = pg_mmdigits_bytes(m, w->k_in);
     const size_t sz_part = ks > 1 ? pg_round_up((size_t)ks * m * w->n_out * sizeof(float), 256) : 0;
@@ -1091,6 +1112,16 @@ pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, c
         }
         return PG_OK;
     }
+    {   // many rows, all Q4_0: one launch on the f16 matrix cores
+        bool all_q4 = count <= PG_HMM_MAX_GROUP;
+        size_t n_total = 0;
+        for (int i = 0; i < count; ++i) {
+            all_q4 &= w[i]->ggml_type == PG_GGML_Q4_0;
+            n_total += w[i]->n_out;
+        }
+        int hks = 1;
+        if (all_q4 && pg_gguf_hmm_takes(ctx, PG_GGML_Q4_0, m, n_total, k_in, &hks)) return pg_gguf_hmm_rows(ctx, x_dev, m, w, y_dev, count, hks);
+    }
     const size_t sz_d = pg_mmdigits_bytes(m, k_in);
     size_t sz_part = 0;
     for (int i = 0; i < count; ++i) {
@@ -1113,6 +1144,13 @@ pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, c
         PG_TRY(pg_launch_gguf_mm(ctx, w[i]->ggml_type, w[i]->n_out, k_in, w[i]->qs_tiled, w[i]->d, grp, m, md, y_dev[i],
                                  ks > 1 ? part_base : nullptr));
     }
+    return PG_OK;
+}
+
+PG_API pg_status pg_gguf_hmm_force(pg_ctx *ctx, int mode) {
+    PG_CHECK_ARG(ctx != nullptr, "null context");
+    PG_CHECK_ARG(mode >= 0 && mode <= 2, "pg_gguf_hmm_force: mode %d (0 = automatic, 1 = wherever it can run, 2 = never)", mode);
+    ctx->hmm_mode = mode;
     return PG_OK;
 }
 

@@ -745,6 +745,11 @@ __global__ void sum_parts_kernel(const float *__restrict__ part, size_t n, int k
 
 }  // namespace
 
+pg_status pg_launch_sum_parts(pg_ctx *ctx, const float *part, size_t n, int ks, size_t stride, float *y) {
+    if (n == 0) return PG_OK;
+    return pg_launch(ctx, "gguf_mm_sum_parts", sum_parts_kernel, dim3(grid_for(n, 256)), dim3(256), 0, part, n, ks, stride, y);
+}
+
 size_t pg_mmdigits_bytes(size_t rows, size_t k) {
     const size_t nb = k / 32, nbp = pg_round_up(nb, 4);
     return rows * pg_mm_row_bytes(nb) + 2 * pg_round_up(rows * nbp * sizeof(float), 256);

@@ -51,6 +51,7 @@ struct pg_ctx {
     int gemm_last_bm = 0, gemm_last_bn = 0, gemm_last_splits = 0;
     int gemm_force_tile = 0;
     int gemv_force_nw = 0, gemv_force_rpw = 0;  // pg_gemv_w8a8_force_shape (0 = the dispatcher chooses)
+    int hmm_mode = 0;  // pg_gguf_hmm_force: 0 = the dispatcher chooses, 1 = the f16 matrix-core product wherever it can run, 2 = never
 };
 
 // Device-resident quantised weight, K-contiguous and zero-padded:
@@ -361,6 +362,25 @@ int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t group
 pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_in, const uint8_t *qs,
                             const uint16_t *d, const pg_mm_group &grp, size_t total_pairs, const pg_mmdigits &md,
                             float *y, float *part, bool keep_parts = false);  // keep_parts: the K chunks' planes are left in `part` unsummed
+// y[i] = part[0][i] + ... + part[ks - 1][i] (planes `stride` floats apart), in that order.
+pg_status pg_launch_sum_parts(pg_ctx *ctx, const float *part, size_t n, int ks, size_t stride, float *y);
+// The many-row Q4_0 product on the f16 matrix cores (pg_gguf_hmm.hip).  The activation rows as two f16 planes
+// [rows][k] (x * 2^e = hi + lo, e per row) and the rows' 2^-e as two f32 factors each.
+constexpr int PG_HMM_MAX_GROUP = 4;  // tensors one launch can carry (q|k|v, gate|up)
+struct pg_hmm_planes {
+    void *hi, *lo;
+    float *inv;  // [rows][2]
+    size_t rows, k;
+};
+size_t pg_hmm_planes_bytes(size_t rows, size_t k);
+pg_hmm_planes pg_hmm_planes_carve(void *base, size_t rows, size_t k);
+pg_status pg_launch_rows_to_f16_planes(pg_ctx *ctx, const float *x_dev, size_t rows, size_t k, const pg_hmm_planes &p);
+// Whether a product of m rows with n_total weight rows (all the tensors of the launch) runs there, and in how many
+// K chunks (*ks_out; their planes need pg_gguf_hmm_part_floats floats).
+bool pg_gguf_hmm_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_total, size_t k_in, int *ks_out);
+size_t pg_gguf_hmm_part_floats(size_t m, size_t n_total, int ks);
+pg_status pg_launch_gguf_hmm_group(pg_ctx *ctx, size_t k_in, const pg_gguf_tensor *const *w, float *const *y, int count, size_t m,
+                                   const pg_hmm_planes &planes, int ks, float *part);
 // y[m, n_out] = x[m, k_in] . dequant(w)^T on device pointers (uses the scratch arena).
 // MXFP4 tensors (pg_mxfp4.hip): qs holds the code bytes in matrix-core fragment order, d the E8M0 scale
 // bytes (four per dword); every product over them runs pg_launch_mxfp4_rows.

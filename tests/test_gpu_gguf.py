@@ -218,3 +218,106 @@ def test_gguf_matmul_special_inputs(ctx, orc):
     with pytest.raises(ValueError):
         gguf.GgufWeight(raw, 2, n_out, k_in + 1, ctx)                       # k_in % 32
     gw.free()
+
+
+# ---- many rows of Q4_0 on the f16 matrix cores (weights exact, activations as two f16 planes) -------------------
+RTOL_F16_ROUTE = 2e-5   # what that route is held to: the planes drop less than 2^-22 of a row's largest value
+
+# (n_out, k_in, m): forced onto the f16 route whatever the dispatcher would choose
+HMM_SHAPES = [
+    (512, 1024, 256),     # two full 256 x 256 tiles, K in two chunks
+    (515, 4160, 300),     # ragged rows, weight rows and K chunks (65 stages in 8 chunks)
+    (1400, 1088, 1000),   # 24 tiles, 17 stages, no split
+    (1100, 2048, 100),    # up to 128 rows: 128 x 512 tiles, ragged
+    (77, 256, 2),         # the smallest it takes: two rows, four stages, an odd number of weight rows
+    (256, 4096, 129),     # one row past the wide tile
+    (4096, 14336, 160),   # a long K in chunks under a half-empty row tile
+]
+
+
+@pytest.mark.parametrize("n_out,k_in,m", HMM_SHAPES)
+def test_gguf_matmul_f16_route_vs_oracle(ctx, orc, n_out, k_in, m):
+    from peregrine_amd import gguf, _ffi
+    say(f"gguf_matmul f16 route n_out={n_out} k_in={k_in} m={m}")
+    w = orc.rng_normal(1900 + n_out, n_out * k_in, 0.0, 0.02)
+    raw = H.pack_q4_0(w)
+    x = orc.rng_normal(117 + m, m * k_in)
+    x.reshape(m, k_in)[:, :: max(1, k_in // 40)] *= 20
+    gw = gguf.GgufWeight(raw, 2, n_out, k_in, ctx)
+    _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 1))
+    try:
+        ctx.profile_begin()
+        got = gw.matmul(x, m)
+        prof = ctx.profile_end()
+        again = gw.matmul(x, m)
+    finally:
+        _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 0))
+    assert "gguf_hmm_q4_0" in prof and "rows_to_f16_planes" in prof, prof
+    assert (bits(got) == bits(again)).all()
+    rows = range(m) if m * n_out * k_in <= 1 << 31 else sorted({0, 1, m // 2, m - 2, m - 1})
+    for r in rows:
+        want = orc.gguf_matmul(x.reshape(m, k_in)[r], 1, raw, 2, n_out, k_in)
+        H.assert_close_rel(got.reshape(m, n_out)[r], want, RTOL_F16_ROUTE, f"row {r}")
+    gw.free()
+
+
+def test_gguf_matmul_f16_route_prefill_size_is_the_dispatchers_choice(ctx, orc):
+    """1024 rows over [4096] -> [14336] (a prefill's gate projection): the dispatcher takes the f16 route by itself;
+    rows spot-checked against the oracle, and the int8 block route on the same input agrees within its own bar."""
+    from peregrine_amd import gguf, _ffi
+    n_out, k_in, m = 14336, 4096, 1024
+    say(f"gguf_matmul prefill size n_out={n_out} k_in={k_in} m={m}")
+    raw = H.pack_q4_0(orc.rng_normal(4343, n_out * k_in, 0.0, 0.02))
+    x = orc.rng_normal(4344, m * k_in)
+    gw = gguf.GgufWeight(raw, 2, n_out, k_in, ctx)
+    ctx.profile_begin()
+    got = gw.matmul(x, m).reshape(m, n_out)
+    prof = ctx.profile_end()
+    assert "gguf_hmm_q4_0" in prof, prof
+    for r in (0, 255, 256, 700, 1023):
+        want = orc.gguf_matmul(x.reshape(m, k_in)[r], 1, raw, 2, n_out, k_in)
+        H.assert_close_rel(got[r], want, RTOL_F16_ROUTE, f"row {r}")
+    _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 2))
+    try:
+        ctx.profile_begin()
+        blockwise = gw.matmul(x, m).reshape(m, n_out)
+        prof = ctx.profile_end()
+    finally:
+        _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 0))
+    assert "gguf_hmm_q4_0" not in prof and "gguf_mm_q4_0" in prof, prof
+    for r in (0, 511, 1023):
+        H.assert_close_rel(blockwise[r], got[r], RTOL_ACHIEVED_MM, f"int8 block route, row {r}")
+    gw.free()
+
+
+def test_gguf_matmul_f16_route_special_rows(ctx, orc):
+    """Zero, tiny, huge, denormal, NaN and infinite rows beside ordinary ones: each row has its own exponent."""
+    from peregrine_amd import gguf, _ffi
+    n_out, k_in, m = 300, 512, 130
+    raw = H.pack_q4_0(orc.rng_normal(55, n_out * k_in, 0.0, 0.02))
+    x = orc.rng_normal(56, m * k_in).reshape(m, k_in)
+    x[1] = 0
+    x[2] *= np.float32(1e-30)
+    x[3] *= np.float32(1e30)
+    x[4] *= np.float32(1e-41)      # denormal floats
+    x[5, 7] = np.nan
+    x[6, 9] = np.inf
+    x[7, :] = 0
+    x[7, 100] = 3.0                # one element: the result is 3 * that weight column, exactly representable inputs
+    gw = gguf.GgufWeight(raw, 2, n_out, k_in, ctx)
+    _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 1))
+    try:
+        got = gw.matmul(x.reshape(-1), m).reshape(m, n_out)
+    finally:
+        _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 0))
+    assert (got[1] == 0).all()
+    assert np.isnan(got[5]).all()
+    assert not np.isfinite(got[6]).any()
+    for r in (0, 2, 3, 7, 8, 129):
+        want = orc.gguf_matmul(x[r], 1, raw, 2, n_out, k_in)
+        H.assert_close_rel(got[r], want, RTOL_F16_ROUTE, f"row {r}")
+    want = orc.gguf_matmul(x[4], 1, raw, 2, n_out, k_in)
+    H.assert_close_rel(got[4], want, 1e-2, "denormal row")   # the inputs themselves carry only a few bits
+    w_col = orc.gguf_matmul(x[7], 1, raw, 2, n_out, k_in)
+    assert (bits(got[7]) == bits(w_col)).all()                # a single product per output: no rounding anywhere
+    gw.free()
