@@ -27,6 +27,7 @@
 // are summed in a fixed order by pg_launch_sum_parts.
 #include <limits.h>
 #include "pg_internal.h"
+#include "pg_f16_planes.h"
 
 namespace {
 
@@ -40,52 +41,30 @@ inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + bloc
 
 __device__ __forceinline__ int swz128(int r) { return ((r >> 1) & 7) ^ ((r & 1) << 2); }
 
-// ---- activation rows -> two f16 planes and the rows' inverse scales ---------------------
-// A row with a NaN or an infinity keeps e = 0: hi carries the special value (and every finite
-// element rounded to f16), lo is zero where the remainder is not finite.
+// ---- activation rows -> two f16 planes and the rows' inverse scales (pg_f16_planes.h) ----
 __global__ __launch_bounds__(256) void rows_to_f16_planes_kernel(const float *__restrict__ x, int K, _Float16 *__restrict__ hi,
                                                                  _Float16 *__restrict__ lo, float *__restrict__ inv) {
     const size_t row = blockIdx.x;
     const float *xr = x + row * K;
     __shared__ float red[4];
     float amax = 0.0f;
-    bool special = false;
     for (int i = threadIdx.x * 4; i < K; i += 1024) {
         const float4 v = *reinterpret_cast<const float4 *>(xr + i);
-        const float a = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        amax = fmaxf(amax, a);
-        special = special || !(fabsf(v.x) < INFINITY) || !(fabsf(v.y) < INFINITY) || !(fabsf(v.z) < INFINITY) || !(fabsf(v.w) < INFINITY);
+        amax = fmaxf(amax, fmaxf(fmaxf(pg_f16_mag(v.x), pg_f16_mag(v.y)), fmaxf(pg_f16_mag(v.z), pg_f16_mag(v.w))));
     }
-    if (special) amax = INFINITY;
     for (int o = 32; o; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
     __syncthreads();
     amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    int e = 0;
-    if (amax > 0.0f && amax < INFINITY) {
-        int ex;
-        (void)frexpf(amax, &ex);  // amax = f * 2^ex, f in [0.5, 1)
-        e = 15 - ex;              // amax * 2^e in [2^14, 2^15)
-    }
-    // 2^e and 2^-e as floats (|e| can pass 127 for denormal rows: two factors each)
-    const int e1 = e / 2, e2 = e - e1;
-    const float s1 = ldexpf(1.0f, e1), s2 = ldexpf(1.0f, e2);
+    const pg_f16_row_scale sc = pg_f16_row_scale_of(amax);
     if (threadIdx.x == 0) {
-        inv[2 * row] = ldexpf(1.0f, -e1);
-        inv[2 * row + 1] = ldexpf(1.0f, -e2);
+        inv[2 * row] = sc.i1;
+        inv[2 * row + 1] = sc.i2;
     }
     for (int i = threadIdx.x * 4; i < K; i += 1024) {
         const float4 v = *reinterpret_cast<const float4 *>(xr + i);
-        const float f[4] = {v.x * s1 * s2, v.y * s1 * s2, v.z * s1 * s2, v.w * s1 * s2};
-        _Float16 h[4], l[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            h[j] = (_Float16)f[j];
-            const float r = f[j] - (float)h[j];
-            l[j] = fabsf(r) < INFINITY ? (_Float16)r : (_Float16)0.0f;
-        }
-        *reinterpret_cast<uint2 *>(hi + row * K + i) = *reinterpret_cast<uint2 *>(h);
-        *reinterpret_cast<uint2 *>(lo + row * K + i) = *reinterpret_cast<uint2 *>(l);
+        const float f[4] = {v.x, v.y, v.z, v.w};
+        pg_f16_split4(f, sc, reinterpret_cast<uint2 *>(hi + row * K + i), reinterpret_cast<uint2 *>(lo + row * K + i));
     }
 }
 
@@ -353,6 +332,8 @@ bool pg_gguf_hmm_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_tota
     while (ks > 1 && stages / ks < 8) --ks;
     if (ks > 8) ks = 8;
     if (ks < 1) ks = 1;
+    const size_t per = (stages + ks - 1) / ks;
+    ks = (stages + per - 1) / per;   // chunks of `per` stages: none is empty
     if (ks_out) *ks_out = (int)ks;
     if (ctx->hmm_mode == 1) return true;
     // Measured against the int8 block product (us, f16 route : int8 route, [K] -> [N] at M rows): 4096 -> 14336 at
@@ -365,14 +346,16 @@ bool pg_gguf_hmm_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_tota
 
 size_t pg_gguf_hmm_part_floats(size_t m, size_t n_total, int ks) { return ks > 1 ? (size_t)ks * m * n_total : 0; }
 
+// ks > 1: the K chunks' planes go to `part` (tensor after tensor, ks planes of m x n_out each) and are summed into
+// y[i]; with keep_parts they go to y[i] instead (ks planes, m * n_out floats apart) and stay unsummed.
 pg_status pg_launch_gguf_hmm_group(pg_ctx *ctx, size_t k_in, const pg_gguf_tensor *const *w, float *const *y, int count, size_t m,
-                                   const pg_hmm_planes &planes, int ks, float *part) {
+                                   const pg_hmm_planes &planes, int ks, float *part, bool keep_parts) {
     if (count < 1 || count > PG_HMM_MAX_GROUP) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): %d tensors (1 .. %d)", count, PG_HMM_MAX_GROUP);
     if (m == 0) return PG_OK;
     for (int i = 0; i < count; ++i)
         if (w[i]->k_in != k_in || w[i]->ggml_type != PG_GGML_Q4_0) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): the tensors differ in K or are not Q4_0");
     if (k_in % 64 != 0 || planes.rows < m || planes.k != k_in) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): K = %zu, planes of %zu x %zu", k_in, planes.rows, planes.k);
-    if (ks < 1 || (ks > 1 && !part)) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): %d K chunks without a buffer for their planes", ks);
+    if (ks < 1 || (ks > 1 && !part && !keep_parts)) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): %d K chunks without a buffer for their planes", ks);
     const bool wide = m <= 128;   // 128 x 512 tiles
     const size_t bm = wide ? 128 : 256, bn = wide ? 512 : 256;
     hmm_group grp;
@@ -384,7 +367,7 @@ pg_status pg_launch_gguf_hmm_group(pg_ctx *ctx, size_t k_in, const pg_gguf_tenso
         grp.d[i] = used ? w[i]->d : nullptr;
         grp.n[i] = used ? (int)w[i]->n_out : 0;
         grp.panel0[i] = used ? panels : INT_MAX;
-        grp.out[i] = used ? (ks > 1 ? part + part_off : y[i]) : nullptr;
+        grp.out[i] = used ? (ks > 1 && !keep_parts ? part + part_off : y[i]) : nullptr;
         grp.stride[i] = used && ks > 1 ? (long long)(m * w[i]->n_out) : 0;
         if (used) {
             panels += (int)((w[i]->n_out + bn - 1) / bn);
@@ -394,6 +377,7 @@ pg_status pg_launch_gguf_hmm_group(pg_ctx *ctx, size_t k_in, const pg_gguf_tenso
     const int tiles_m = (int)((m + bm - 1) / bm), ntiles = tiles_m * panels;
     const int stages = (int)(k_in / 64), kt_per = (stages + ks - 1) / ks;
     const int ks_real = (stages + kt_per - 1) / kt_per;
+    if (ks_real != ks) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): %d K chunks of %d stages leave one empty", ks, kt_per);
     const dim3 grid((unsigned)((ntiles + 7) / 8 * 8), (unsigned)ks_real);
     const int nb = (int)(k_in / 32);
     if (wide) {
@@ -409,8 +393,7 @@ pg_status pg_launch_gguf_hmm_group(pg_ctx *ctx, size_t k_in, const pg_gguf_tenso
         PG_TRY(pg_launch(ctx, "gguf_hmm_q4_0", kern, grid, dim3(512), lds, (const _Float16 *)planes.hi, (const _Float16 *)planes.lo,
                          (const float *)planes.inv, grp, (int)m, nb, tiles_m, ntiles, kt_per));
     }
-    if (ks > 1) {
-        // (ks_real chunks were written; a plane that no chunk wrote does not exist: kt_per is rounded up)
+    if (ks > 1 && !keep_parts) {
         size_t off = 0;
         for (int i = 0; i < count; ++i) {
             const size_t plane = m * w[i]->n_out;

@@ -380,7 +380,7 @@ pg_status pg_launch_rows_to_f16_planes(pg_ctx *ctx, const float *x_dev, size_t r
 bool pg_gguf_hmm_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_total, size_t k_in, int *ks_out);
 size_t pg_gguf_hmm_part_floats(size_t m, size_t n_total, int ks);
 pg_status pg_launch_gguf_hmm_group(pg_ctx *ctx, size_t k_in, const pg_gguf_tensor *const *w, float *const *y, int count, size_t m,
-                                   const pg_hmm_planes &planes, int ks, float *part);
+                                   const pg_hmm_planes &planes, int ks, float *part, bool keep_parts = false);
 // y[m, n_out] = x[m, k_in] . dequant(w)^T on device pointers (uses the scratch arena).
 // MXFP4 tensors (pg_mxfp4.hip): qs holds the code bytes in matrix-core fragment order, d the E8M0 scale
 // bytes (four per dword); every product over them runs pg_launch_mxfp4_rows.

@@ -18,6 +18,7 @@
 #include <vector>
 #include "pg_internal.h"
 #include "pg_digits.h"
+#include "pg_f16_planes.h"
 
 struct pg_rope {
     float *cos_t, *sin_t;
@@ -103,7 +104,9 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(const float *a, const 
 // load of the row is issued before the first is needed.
 // DIG: 0 = write the normalised row as f32; 1 / 2 = write it as nibble / byte digits for the
 // streaming product instead (dim a multiple of 32, so that 8-lane groups hold whole blocks); 3 / 4 = as the
-// two byte-digit planes of the matrix-core block product (Q4_0 / Q8_0 element order).
+// two byte-digit planes of the matrix-core block product (Q4_0 / Q8_0 element order); 5 = as the two f16 planes of
+// the f16 matrix-core product (pg_f16_planes.h): hi plane at `digits`, lo plane at `out`, the rows' two inverse
+// scale factors at `xs`.
 // The second input may come as b_planes planes, b_stride4 float4 apart (the K chunks of a split product,
 // summed here in ascending order before the addition, as gguf_mm's own summing pass would).
 template <int MAXV, int DIG>
@@ -148,6 +151,32 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(const float4 *__re
     for (int j = 0; j < MAXV; ++j) ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
     ss = block_sum(ss, red);
     const float inv_rms = 1.0f / sqrtf(ss * (1.0f / (float)(dim4 * 4)) + eps);
+    if constexpr (DIG == 5) {
+        float amax = 0.f;
+#pragma unroll
+        for (int j = 0; j < MAXV; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            if (i < dim4) {
+                v[j] = float4{v[j].x * inv_rms * wv[j].x, v[j].y * inv_rms * wv[j].y, v[j].z * inv_rms * wv[j].z, v[j].w * inv_rms * wv[j].w};
+                amax = fmaxf(amax, fmaxf(fmaxf(pg_f16_mag(v[j].x), pg_f16_mag(v[j].y)), fmaxf(pg_f16_mag(v[j].z), pg_f16_mag(v[j].w))));
+            }
+        }
+        const pg_f16_row_scale sc = pg_f16_row_scale_of(block_max(amax, red));
+        if (threadIdx.x == 0) {
+            xs[2 * blockIdx.x] = sc.i1;
+            xs[2 * blockIdx.x + 1] = sc.i2;
+        }
+        _Float16 *hi = reinterpret_cast<_Float16 *>(digits), *lo = reinterpret_cast<_Float16 *>(out);
+#pragma unroll
+        for (int j = 0; j < MAXV; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            if (i < dim4) {
+                const float o[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+                pg_f16_split4(o, sc, reinterpret_cast<uint2 *>(hi + (row + i) * 4), reinterpret_cast<uint2 *>(lo + (row + i) * 4));
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < MAXV; ++j) {
         const int i = threadIdx.x + 256 * j;
@@ -1300,6 +1329,56 @@ __global__ __launch_bounds__(256) void swiglu_mm_digits_kernel(const float *__re
     pg_emit_mm_digits<NIB>(o, row, b, sub, nb, nbp, digits, xs);
 }
 
+// Rows of silu(g) * u written as the two f16 planes of the f16 matrix-core product (pg_f16_planes.h), a workgroup per
+// row with the row in registers (dim4 <= 256 * MAXV float4); g and u as the sums of `planes` planes, as above.
+template <int MAXV>
+__global__ __launch_bounds__(256) void swiglu_f16_planes_kernel(const float *__restrict__ g, const float *__restrict__ u, int planes,
+                                                                size_t stride, int dim4, _Float16 *__restrict__ hi,
+                                                                _Float16 *__restrict__ lo, float *__restrict__ inv) {
+    __shared__ float red[4];
+    const size_t row = (size_t)blockIdx.x * dim4;
+    float4 v[MAXV];
+    float amax = 0.f;
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        v[j] = float4{0.f, 0.f, 0.f, 0.f};
+        if (i < dim4) {
+            float4 gp[PG_MAX_PLANES], up[PG_MAX_PLANES];
+#pragma unroll
+            for (int pl = 0; pl < PG_MAX_PLANES; ++pl) {
+                const bool have = pl < planes;
+                gp[pl] = have ? reinterpret_cast<const float4 *>(g + pl * stride)[row + i] : float4{0.f, 0.f, 0.f, 0.f};
+                up[pl] = have ? reinterpret_cast<const float4 *>(u + pl * stride)[row + i] : float4{0.f, 0.f, 0.f, 0.f};
+            }
+            float4 gv = gp[0], uv = up[0];
+#pragma unroll
+            for (int pl = 1; pl < PG_MAX_PLANES; ++pl) {
+                if (pl < planes) {
+                    gv.x += gp[pl].x; gv.y += gp[pl].y; gv.z += gp[pl].z; gv.w += gp[pl].w;
+                    uv.x += up[pl].x; uv.y += up[pl].y; uv.z += up[pl].z; uv.w += up[pl].w;
+                }
+            }
+            v[j] = float4{gv.x / (1.0f + expf(-gv.x)) * uv.x, gv.y / (1.0f + expf(-gv.y)) * uv.y,
+                          gv.z / (1.0f + expf(-gv.z)) * uv.z, gv.w / (1.0f + expf(-gv.w)) * uv.w};
+            amax = fmaxf(amax, fmaxf(fmaxf(pg_f16_mag(v[j].x), pg_f16_mag(v[j].y)), fmaxf(pg_f16_mag(v[j].z), pg_f16_mag(v[j].w))));
+        }
+    }
+    const pg_f16_row_scale sc = pg_f16_row_scale_of(block_max(amax, red));
+    if (threadIdx.x == 0) {
+        inv[2 * blockIdx.x] = sc.i1;
+        inv[2 * blockIdx.x + 1] = sc.i2;
+    }
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        if (i < dim4) {
+            const float o[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+            pg_f16_split4(o, sc, reinterpret_cast<uint2 *>(hi + (row + i) * 4), reinterpret_cast<uint2 *>(lo + (row + i) * 4));
+        }
+    }
+}
+
 // out = a + (b as the sum of `planes` planes, in ascending order)
 __global__ __launch_bounds__(256) void add_planes_kernel(const float *__restrict__ a, const float *__restrict__ b, int planes,
                                                          size_t stride, float *__restrict__ out, size_t n) {
@@ -2115,7 +2194,7 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     // Up to eight tokens: the few-rows product (one launch per tensor group, no K split between workgroups, so every
     // product leaves one plane; the weights are read in their row-major planes, no tile-major copy).
     // (Nine to sixteen tokens: only the products over fewer than 32 weight rows per CU, see pg_gguf_skinny_takes.)
-    bool few[7];
+    bool few[7], hm[7];
     int ks[7];
     size_t part_off[7], floats = 0;
     for (int i = 0; i < 7; ++i) {
@@ -2126,12 +2205,20 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
         }
         few[i] = pg_gguf_skinny_takes(ctx, type, seq, rows, k_of[i]);
         ks[i] = few[i] ? 1 : pg_gguf_mm_splitk(ctx, groups * 128, k_of[i], tiles, seq, false, nullptr);
+        // Many tokens: the f16 matrix-core product where it is the faster one (its input then arrives as two f16
+        // planes, not as digit planes; the down projection's producer holds a row of the FFN width in registers).
+        int hks = 1;
+        hm[i] = !few[i] && (i != 6 || ffn <= 32768) && count_of[i] <= PG_HMM_MAX_GROUP &&
+                pg_gguf_hmm_takes(ctx, type, seq, rows, k_of[i], &hks);
+        if (hm[i]) ks[i] = hks;
         if (ks[i] > PG_MAX_PLANES) return pg_fail(PG_EUNSUPPORTED, "llama block: a product in %d K chunks", ks[i]);
         part_off[i] = floats;
         floats += pg_round_up((size_t)ks[i] * seq * n_of[i], 64);
     }
     const size_t sz_d = pg_mmdigits_bytes(seq, d), sz_q = pg_mmdigits_bytes(seq, q_dim), sz_f = pg_mmdigits_bytes(seq, ffn);
-    const size_t need = sz_d + sz_q + sz_f + floats * sizeof(float);
+    const size_t sz_hd = hm[0] || hm[4] ? pg_hmm_planes_bytes(seq, d) : 0, sz_hq = hm[3] ? pg_hmm_planes_bytes(seq, q_dim) : 0,
+                 sz_hf = hm[6] ? pg_hmm_planes_bytes(seq, ffn) : 0;
+    const size_t need = sz_d + sz_q + sz_f + floats * sizeof(float) + sz_hd + sz_hq + sz_hf;
     if (need > b->chain_bytes) {
         PG_HIP(hipStreamSynchronize(ctx->stream));
         if (b->chain) (void)hipFree(b->chain);
@@ -2146,9 +2233,17 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
                       md_f = pg_mmdigits_carve(base + sz_d + sz_q, seq, ffn);
     float *parts = reinterpret_cast<float *>(base + sz_d + sz_q + sz_f);
     auto part = [&](int i) { return parts + part_off[i]; };
+    char *hbase = base + sz_d + sz_q + sz_f + floats * sizeof(float);
+    const pg_hmm_planes pl_d = pg_hmm_planes_carve(hbase, seq, d), pl_q = pg_hmm_planes_carve(hbase + sz_hd, seq, q_dim),
+                        pl_f = pg_hmm_planes_carve(hbase + sz_hd + sz_hq, seq, ffn);  // (carved whether used or not: only those with bytes are touched)
     pg_mm_group grp = {1, nullptr, nullptr, nullptr, nullptr, 0, (int)tiles, (int)seq, 1};
     grp.tiled = 1;
     auto product = [&](int i, const pg_mmdigits &md) -> pg_status {  // tensors i .. i + count_of[i] - 1
+        if (hm[i]) {
+            float *ys[PG_HMM_MAX_GROUP] = {part(i), count_of[i] > 1 ? part(i + 1) : nullptr, count_of[i] > 2 ? part(i + 2) : nullptr, nullptr};
+            return pg_launch_gguf_hmm_group(ctx, k_of[i], b->w + i, ys, count_of[i], seq, i == 3 ? pl_q : (i == 6 ? pl_f : pl_d), ks[i],
+                                            nullptr, true);
+        }
         if (few[i]) {
             float *ys[3] = {part(i), count_of[i] > 1 ? part(i + 1) : nullptr, count_of[i] > 2 ? part(i + 2) : nullptr};
             return pg_launch_gguf_skinny_group(ctx, type, k_of[i], b->w + i, ys, count_of[i], seq, md);
@@ -2167,7 +2262,13 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
             return pg_launch_gguf_mm(ctx, type, n_of[i], k_of[i], b->w[i]->qs_tiled, b->w[i]->d, g, seq, md, part(i), part(i), true);
         return pg_launch_gguf_mm(ctx, type, groups * 128, k_of[i], nullptr, nullptr, g, seq, md, part(i), part(i), true);
     };
-    auto norm_digits = [&](const float *a, int bi, float *sum_out, const float *w) -> pg_status {
+    auto norm_digits = [&](const float *a, int bi, float *sum_out, const float *w, bool f16_planes) -> pg_status {
+        if (f16_planes) {
+            auto *kern = d <= 4096 ? add_rmsnorm_vec_kernel<4, 5> : add_rmsnorm_vec_kernel<8, 5>;
+            return pg_launch(ctx, "add_rmsnorm_f16_planes", kern, dim3((unsigned)seq), dim3(256), 0, (const float4 *)a,
+                             (const float4 *)(bi >= 0 ? part(bi) : nullptr), (float4 *)sum_out, (const float4 *)w, b->eps, (int)(d / 4),
+                             (float4 *)pl_d.lo, (int8_t *)pl_d.hi, pl_d.inv, bi >= 0 ? ks[bi] : 1, seq * d / 4);
+        }
         auto *kern = d <= 4096 ? (nib ? add_rmsnorm_vec_kernel<4, 3> : add_rmsnorm_vec_kernel<4, 4>)
                                : (nib ? add_rmsnorm_vec_kernel<8, 3> : add_rmsnorm_vec_kernel<8, 4>);
         return pg_launch(ctx, "add_rmsnorm_mm_digits", kern, dim3((unsigned)seq), dim3(256), 0, (const float4 *)a,
@@ -2176,7 +2277,7 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     };
     const int nbf = (int)(ffn / 32);
 
-    PG_TRY(norm_digits(h_dev, -1, nullptr, b->attn_norm_w));
+    PG_TRY(norm_digits(h_dev, -1, nullptr, b->attn_norm_w, hm[0]));
     PG_TRY(product(0, md_d));
     PG_TRY(cache_reserve(ctx, cache, offset + seq));
     rope_args ra = {};
@@ -2188,12 +2289,17 @@ static pg_status block_forward_chained(pg_ctx *ctx, pg_llama_block *b, const flo
     cache->len = offset + seq;
     bool md_written = false;  // (a merge of key runs writes the o-projection's digit planes itself)
     PG_TRY(launch_attention(ctx, q_rope, cache, cache, b->nqh, seq, 1.0f / sqrtf((float)hd), PG_MASK_CAUSAL, offset, 0, 0,
-                            0.0f, attn, 0, nullptr, type, nullptr, 0, nullptr, hd % 32 == 0 ? &md_q : nullptr, &md_written));
-    if (!md_written) PG_TRY(pg_launch_x_to_mm_digits(ctx, attn, seq, q_dim, type, md_q));
+                            0.0f, attn, 0, nullptr, type, nullptr, 0, nullptr, hd % 32 == 0 && !hm[3] ? &md_q : nullptr, &md_written));
+    if (hm[3]) PG_TRY(pg_launch_rows_to_f16_planes(ctx, attn, seq, q_dim, pl_q));
+    else if (!md_written) PG_TRY(pg_launch_x_to_mm_digits(ctx, attn, seq, q_dim, type, md_q));
     PG_TRY(product(3, md_q));
-    PG_TRY(norm_digits(h_dev, 3, h1, b->ffn_norm_w));  // h1 = h + attn . Wo, and its norm as digits
+    PG_TRY(norm_digits(h_dev, 3, h1, b->ffn_norm_w, hm[4]));  // h1 = h + attn . Wo, and its norm as digits
     PG_TRY(product(4, md_d));
-    {
+    if (hm[6]) {
+        auto *kern = ffn <= 16384 ? swiglu_f16_planes_kernel<16> : swiglu_f16_planes_kernel<32>;
+        PG_TRY(pg_launch(ctx, "swiglu_f16_planes", kern, dim3((unsigned)seq), dim3(256), 0, (const float *)part(4), (const float *)part(5),
+                         ks[4], seq * ffn, (int)(ffn / 4), (_Float16 *)pl_f.hi, (_Float16 *)pl_f.lo, pl_f.inv));
+    } else {
         auto *kern = nib ? swiglu_mm_digits_kernel<true> : swiglu_mm_digits_kernel<false>;
         PG_TRY(pg_launch(ctx, "swiglu_mm_digits", kern, dim3((unsigned)((nbf + 31) / 32), (unsigned)seq), dim3(256), 0,
                          (const float *)part(4), (const float *)part(5), ks[4], seq * ffn, nbf, (int)pg_round_up(nbf, 4),
