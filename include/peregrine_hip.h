@@ -525,10 +525,10 @@ pg_status pg_gemm_w8a8_force_tile(pg_ctx *ctx, int tile);
  * 16; weight rows per wavefront 1 or 2, not 16 x 2) instead of the dispatcher's choice by row length; 0, 0 =
  * automatic.  Every shape gives the same bits. */
 pg_status pg_gemv_w8a8_force_shape(pg_ctx *ctx, int wavefronts, int rows_per_wavefront);
-/* The many-row Q4_0 product has two matrix-core routes: the int8 block product with 16-bit fixed-point activations
+/* The many-row Q4_0 / Q8_0 product has two matrix-core routes: the int8 block product with 16-bit fixed-point activations
  * per block, and, from about a hundred rows on where the launch fills the part, f16 tiles with the weights unpacked
  * in registers and the activations as two f16 planes per row.  mode 0 = the dispatcher chooses, 1 = the f16 route
- * wherever it can run (Q4_0, K a multiple of 64, at least two rows), 2 = never.  Both keep the weights exact; they
+ * wherever it can run (Q4_0 or Q8_0, K a multiple of 64, at least two rows), 2 = never.  Both keep the weights exact; they
  * round the activations differently (2^-22 of the row's largest value against 2^-16 of the block's). */
 pg_status pg_gguf_hmm_force(pg_ctx *ctx, int mode);
 
@@ -545,6 +545,8 @@ pg_status pg_audit_gguf_gemv(size_t n_out, size_t k_in, int q8, int blocks_per_l
                              int wavefronts, size_t *qs_end, size_t *qs_bytes, size_t *d_end, size_t *d_bytes);
 pg_status pg_audit_gguf_skinny(size_t n_out, size_t k_in, int q8, int wavefronts, size_t *qs_end, size_t *qs_bytes,
                                size_t *d_end, size_t *d_bytes);
+pg_status pg_audit_gguf_hmm(size_t m, size_t n_out, size_t k_in, int q8, int wide_tiles, int k_chunks, size_t *plane_end,
+                            size_t *plane_bytes, size_t *qs_end, size_t *qs_bytes, size_t *d_end, size_t *d_bytes);
 pg_status pg_audit_mxfp4_rows(size_t out_dim, size_t in_dim, int row_groups_per_workgroup, int wavefronts,
                               size_t *qs_end, size_t *qs_bytes, size_t *sc_end, size_t *sc_bytes);
 pg_status pg_audit_probe_read(size_t bytes, int workgroups, int threads, int loads_in_flight, size_t *end,

@@ -146,6 +146,55 @@ PG_API pg_status pg_audit_gguf_skinny(size_t n_out, size_t k_in, int q8, int nw,
     return PG_OK;
 }
 
+// Many rows on the f16 matrix cores (gguf_hmm_kernel<QT, NWM, NWN>): 256 x 256 tiles (wide = 0) or 128 x 512 (wide = 1; Q8_0 always),
+// K in `ks` chunks of whole stages of 64; the planes are [m][k_in] f16, the payload [n_out][k_in / 32][16 B] (Q8_0: [n_out][2][k_in / 32][16 B]).
+// (Every offset is linear in the stage: the first and the last stage of a chunk bound the rest.)
+PG_API pg_status pg_audit_gguf_hmm(size_t m, size_t n_out, size_t k_in, int q8, int wide, int ks, size_t *plane_end, size_t *plane_bytes,
+                                   size_t *qs_end, size_t *qs_bytes, size_t *d_end, size_t *d_bytes) {
+    PG_CHECK_ARG(m > 0 && n_out >= 2 && k_in >= 64 && k_in % 64 == 0 && ks >= 1, "pg_audit_gguf_hmm: bad arguments");
+    const int nb = (int)(k_in / 32), K = (int)k_in, M = (int)m, N = (int)n_out;
+    PG_CHECK_ARG(!q8 || wide, "pg_audit_gguf_hmm: Q8_0 runs the 128 x 512 tiles only");
+    const int nwn = wide ? 8 : 4, bm = wide ? 128 : 256, bn = 64 * nwn, lx = bm / 64, lw = (bn * (q8 ? 64 : 32) / 1024 + 7) / 8;
+    const int stages = nb / 2, kt_per = (stages + ks - 1) / ks;
+    const int tiles_m = (M + bm - 1) / bm, panels = (N + bn - 1) / bn;
+    auto swz128 = [](int r) { return ((r >> 1) & 7) ^ ((r & 1) << 2); };
+    span_check pl, qs, d;
+    for (int split = 0; split * kt_per < stages; ++split) {
+        const int kt0 = split * kt_per, kt_n = std::min(kt_per, stages - kt0);
+        for (int tm = 0; tm < tiles_m; ++tm)
+            for (int np = 0; np < panels; ++np) {
+                const int m0 = tm * bm, n0 = np * bn;
+                for (int wave = 0; wave < 8; ++wave)
+                    for (int lane = 0; lane < 64; ++lane)
+                        for (int st : {kt0, kt0 + kt_n - 1}) {
+                            for (int i = 0; i < lx; ++i) {
+                                const int row = 8 * (wave + 8 * i) + (lane >> 3);
+                                pl.touch(pg_hmm_plane_offset(pg_hmm_clamp_row(m0 + row, M), K, st, (lane & 7) ^ swz128(row)), 16);
+                            }
+                            for (int i = 0; i < lw; ++i) {
+                                if (q8) {
+                                    const int row = 16 * (wave + 8 * i) + (lane >> 2), rc = row < bn ? row : bn - 1;
+                                    const int c = (lane & 3) ^ ((row >> 2) & 3);
+                                    qs.touch(pg_hmm_weight_offset_q8(pg_hmm_clamp_row(n0 + rc, N), c & 1, nb, st, c >> 1), 16);
+                                } else {
+                                    const int row = 32 * (wave + 8 * i) + (lane >> 1), rc = row < bn ? row : bn - 1;
+                                    qs.touch(pg_hmm_weight_offset(pg_hmm_clamp_row(n0 + rc, N), nb, st, (lane & 1) ^ ((row >> 3) & 1)), 16);
+                                }
+                            }
+                            const int row = (wave % nwn) * 64 + 2 * (lane & 31);
+                            d.touch(pg_hmm_scale_offset(pg_hmm_scale_row(n0 + row, N), nb, st, lane >> 5), 4);
+                        }
+            }
+    }
+    if (plane_end) *plane_end = pl.end;
+    if (plane_bytes) *plane_bytes = m * k_in * 2;
+    if (qs_end) *qs_end = qs.end;
+    if (qs_bytes) *qs_bytes = n_out * (size_t)nb * (q8 ? 32 : 16);
+    if (d_end) *d_end = d.end;
+    if (d_bytes) *d_bytes = (n_out + 7) / 8 * 8 * (size_t)nb * sizeof(uint16_t);
+    return PG_OK;
+}
+
 // MXFP4 rows (mxfp4_rows_kernel<T, RG, NW>): the fragment-major code plane [row groups of 16][ncp chunks][64 lanes][16 B]
 // and the scale plane [row groups][ncp / 4][64 lanes][4 B]; a wavefront = (row group, K slice), 8 chunks per batch of loads.
 PG_API pg_status pg_audit_mxfp4_rows(size_t out_dim, size_t in_dim, int rg_per_wg, int nw, size_t *qs_end, size_t *qs_bytes,

@@ -1005,7 +1005,7 @@ pg_status pg_gguf_ensure_tiled(pg_ctx *ctx, const pg_gguf_tensor *w) {
     return PG_OK;
 }
 
-// `count` Q4_0 products over the same many rows on the f16 matrix cores: the rows become two f16 planes once,
+// `count` products of one block type (Q4_0 or Q8_0) over the same many rows on the f16 matrix cores: the rows become two f16 planes once,
 // tensors of the same launch shape share a launch (up to PG_HMM_MAX_GROUP).
 static pg_status pg_gguf_hmm_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *const *w, float *const *y_dev,
                                   int count, int ks) {
@@ -1112,15 +1112,15 @@ pg_status pg_gguf_matmul_rows_multi(pg_ctx *ctx, const float *x_dev, size_t m, c
         }
         return PG_OK;
     }
-    {   // many rows, all Q4_0: one launch on the f16 matrix cores
-        bool all_q4 = count <= PG_HMM_MAX_GROUP;
+    {   // many rows, one block type: one launch on the f16 matrix cores
+        bool one_type = count <= PG_HMM_MAX_GROUP;
         size_t n_total = 0;
         for (int i = 0; i < count; ++i) {
-            all_q4 &= w[i]->ggml_type == PG_GGML_Q4_0;
+            one_type &= w[i]->ggml_type == w[0]->ggml_type;
             n_total += w[i]->n_out;
         }
         int hks = 1;
-        if (all_q4 && pg_gguf_hmm_takes(ctx, PG_GGML_Q4_0, m, n_total, k_in, &hks)) return pg_gguf_hmm_rows(ctx, x_dev, m, w, y_dev, count, hks);
+        if (one_type && pg_gguf_hmm_takes(ctx, w[0]->ggml_type, m, n_total, k_in, &hks)) return pg_gguf_hmm_rows(ctx, x_dev, m, w, y_dev, count, hks);
     }
     const size_t sz_d = pg_mmdigits_bytes(m, k_in);
     size_t sz_part = 0;

@@ -28,6 +28,7 @@
 #include <limits.h>
 #include "pg_internal.h"
 #include "pg_f16_planes.h"
+#include "pg_stream_addr.h"
 
 namespace {
 
@@ -84,6 +85,22 @@ __device__ __forceinline__ v8h nibbles_to_f16(uint32_t w) {
     return r.v;
 }
 
+// 8 Q8_0 quants (two dwords of int8, element order) -> 8 f16 values.  A byte q as q + 128 under 0x64 is the f16
+// 1152 + q; the bytes 0x64 come from the selector's second source.
+__device__ __forceinline__ v8h bytes_to_f16(uint32_t w0, uint32_t w1) {
+    w0 ^= 0x80808080u;
+    w1 ^= 0x80808080u;
+    const v2h bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+    union { uint32_t u[4]; v2h h[4]; v8h v; } r;
+    r.u[0] = __builtin_amdgcn_perm(w0, 0x64646464u, 0x00050004u);
+    r.u[1] = __builtin_amdgcn_perm(w0, 0x64646464u, 0x00070006u);
+    r.u[2] = __builtin_amdgcn_perm(w1, 0x64646464u, 0x00050004u);
+    r.u[3] = __builtin_amdgcn_perm(w1, 0x64646464u, 0x00070006u);
+#pragma unroll
+    for (int p = 0; p < 4; ++p) r.h[p] = r.h[p] - bias;
+    return r.v;
+}
+
 // The tensors of one launch: equal K, their panels of BN weight rows laid end to end in the launch's tile space.
 struct hmm_group {
     const uint8_t *qs[PG_HMM_MAX_GROUP];
@@ -96,13 +113,17 @@ struct hmm_group {
 
 constexpr int BKB = 2;  // blocks per stage
 
-template <int NWM, int NWN>
+// QT = 8 (Q8_0): a weight row is two streams of 16-byte half blocks (elements 0 .. 15 and 16 .. 31 of every block,
+// as the upload splits them); a stage holds 64 bytes a row, chunk 2 block + half at position chunk ^ ((row >> 2) & 3),
+// so that the 64-bit fragment reads of 16 rows spread over all banks.
+template <int QT, int NWM, int NWN>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void gguf_hmm_q4_kernel(const _Float16 *__restrict__ xh, const _Float16 *__restrict__ xl, const float *__restrict__ inv,
+void gguf_hmm_kernel(const _Float16 *__restrict__ xh, const _Float16 *__restrict__ xl, const float *__restrict__ inv,
                         const hmm_group grp, int M, int nb, int tiles_m, int ntiles, int kt_per_split) {
     static_assert(NWM * NWN == 8, "eight wavefronts");
     constexpr int BM = 128 * NWM, BN = 64 * NWN;
-    constexpr int LX = BM / 64, LW = (BN + 255) / 256;       // wave-loads per wavefront and stage: one plane, weights
+    constexpr int WROW = QT == 8 ? 64 : 32;                   // bytes of packed weights per row and stage
+    constexpr int LX = BM / 64, LW = (BN * WROW / 1024 + 7) / 8;  // wave-loads per wavefront and stage: one plane, weights
     constexpr int XP = BM * 128;                              // one activation plane of a stage
     constexpr int OFF_XL = XP, OFF_W = 2 * XP, OFF_D = OFF_W + 8 * LW * 1024, STAGE = OFF_D + 8 * 256;
     constexpr int LPS = 2 * LX + LW + 1;
@@ -141,25 +162,29 @@ void gguf_hmm_q4_kernel(const _Float16 *__restrict__ xh, const _Float16 *__restr
 #pragma unroll
         for (int i = 0; i < LX; ++i) {
             const int row = 8 * (wave + 8 * i) + lr;
-            const int mr = m0 + row < M ? m0 + row : M - 1;
-            xsrc[i] = reinterpret_cast<const char *>(xh) + ((size_t)mr * K + (size_t)kt0 * 64) * 2 + 16 * (pc ^ swz128(row));
+            xsrc[i] = reinterpret_cast<const char *>(xh) + pg_hmm_plane_offset(pg_hmm_clamp_row(m0 + row, M), K, kt0, pc ^ swz128(row));
         }
     }
     const ptrdiff_t lo_minus_hi = reinterpret_cast<const char *>(xl) - reinterpret_cast<const char *>(xh);
     const char *wsrc[LW];
 #pragma unroll
     for (int i = 0; i < LW; ++i) {
-        const int row = 32 * (wave + 8 * i) + (lane >> 1);
-        const int rc = row < BN ? row : BN - 1;
-        const int nr = n0 + rc < N ? n0 + rc : N - 1;
-        const int cb = (lane & 1) ^ ((row >> 3) & 1);
-        wsrc[i] = reinterpret_cast<const char *>(qs) + ((size_t)nr * nb + (size_t)kt0 * BKB + cb) * 16;
+        if constexpr (QT == 8) {
+            const int row = 16 * (wave + 8 * i) + (lane >> 2);
+            const int rc = row < BN ? row : BN - 1;
+            const int c = (lane & 3) ^ ((row >> 2) & 3);  // logical chunk: 2 block + half
+            wsrc[i] = reinterpret_cast<const char *>(qs) + pg_hmm_weight_offset_q8(pg_hmm_clamp_row(n0 + rc, N), c & 1, nb, kt0, c >> 1);
+        } else {
+            const int row = 32 * (wave + 8 * i) + (lane >> 1);
+            const int rc = row < BN ? row : BN - 1;
+            const int cb = (lane & 1) ^ ((row >> 3) & 1);
+            wsrc[i] = reinterpret_cast<const char *>(qs) + pg_hmm_weight_offset(pg_hmm_clamp_row(n0 + rc, N), nb, kt0, cb);
+        }
     }
     const char *dsrc;
     {
         const int row = wn * 64 + 2 * (lane & 31);   // this wavefront's own 64 weight rows, two per lane
-        const int nr = n0 + row < N ? n0 + row : (N - 1) & ~1;
-        dsrc = reinterpret_cast<const char *>(d) + (((size_t)(nr >> 3) * nb + (size_t)kt0 * BKB + (lane >> 5)) * 8 + (nr & 7)) * 2;
+        dsrc = reinterpret_cast<const char *>(d) + pg_hmm_scale_offset(pg_hmm_scale_row(n0 + row, N), nb, kt0, lane >> 5);
     }
     auto issue = [&](int stage, int kt) {   // kt: stage index within this workgroup's K chunk
         char *base = lds + stage * STAGE;
@@ -182,7 +207,8 @@ void gguf_hmm_q4_kernel(const _Float16 *__restrict__ xh, const _Float16 *__restr
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             a_off[b] = ra * 128 + (((4 * b + q4) ^ swz128(ra)) * 16);                    // + 16 rows per row tile
-            w_off[b] = OFF_W + rb * 32 + 16 * (b ^ ((rb >> 3) & 1)) + 4 * q4;            // + 16 rows per weight tile
+            if constexpr (QT == 8) w_off[b] = OFF_W + rb * 64 + 16 * ((2 * b + (q4 >> 1)) ^ ((rb >> 2) & 3)) + 8 * (q4 & 1);
+            else w_off[b] = OFF_W + rb * 32 + 16 * (b ^ ((rb >> 3) & 1)) + 4 * q4;       // + 16 rows per weight tile
             d_off[b] = OFF_D + wave * 256 + (b * 32 + (l15 >> 1)) * 4 + (l15 & 1) * 2;   // + 32 bytes per weight tile
         }
     }
@@ -205,13 +231,27 @@ void gguf_hmm_q4_kernel(const _Float16 *__restrict__ xh, const _Float16 *__restr
         const char *base = lds + s * STAGE;
         v8h fb[2][4];
         float df[2][4];
-        uint32_t wraw[4];
+        uint32_t wraw[4][QT == 8 ? 2 : 1];
         _Float16 draw[4];
+        auto read_w = [&](int b, int j, uint32_t (&raw)[QT == 8 ? 2 : 1]) {
+            if constexpr (QT == 8) {
+                const uint2 t = *reinterpret_cast<const uint2 *>(base + w_off[b] + j * 16 * WROW);
+                raw[0] = t.x;
+                raw[1] = t.y;
+            } else {
+                raw[0] = *reinterpret_cast<const uint32_t *>(base + w_off[b] + j * 16 * WROW);
+            }
+        };
+        auto unpack = [&](const uint32_t (&raw)[QT == 8 ? 2 : 1]) -> v8h {
+            if constexpr (QT == 8) return bytes_to_f16(raw[0], raw[1]);
+            else return nibbles_to_f16(raw[0]);
+        };
         v8h ah[2], al[2];
         v4f T[2][4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            fb[0][j] = nibbles_to_f16(*reinterpret_cast<const uint32_t *>(base + w_off[0] + j * 16 * 32));
+            read_w(0, j, wraw[j]);
+            fb[0][j] = unpack(wraw[j]);
             df[0][j] = (float)*reinterpret_cast<const _Float16 *>(base + d_off[0] + j * 32);
             asm volatile("" : "+v"(df[0][j]));   // a plain f32 register: the FMAs below are v_fma_f32, not mixed-precision ones
         }
@@ -228,12 +268,12 @@ void gguf_hmm_q4_kernel(const _Float16 *__restrict__ xh, const _Float16 *__restr
             if (q == 0) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    wraw[j] = *reinterpret_cast<const uint32_t *>(base + w_off[1] + j * 16 * 32);
+                    read_w(1, j, wraw[j]);
                     draw[j] = *reinterpret_cast<const _Float16 *>(base + d_off[1] + j * 32);
                 }
             }
             if (q >= 2 && q < 6) {
-                fb[1][q - 2] = nibbles_to_f16(wraw[q - 2]);
+                fb[1][q - 2] = unpack(wraw[q - 2]);
                 df[1][q - 2] = (float)draw[q - 2];
                 asm volatile("" : "+v"(df[1][q - 2]));
             }
@@ -287,8 +327,8 @@ void gguf_hmm_q4_kernel(const _Float16 *__restrict__ xh, const _Float16 *__restr
         }
 }
 
-template <int NWM, int NWN> constexpr size_t hmm_lds_bytes() {
-    return 2 * (size_t)(2 * 128 * NWM * 128 + 8 * ((64 * NWN + 255) / 256) * 1024 + 8 * 256);
+template <int QT, int NWM, int NWN> constexpr size_t hmm_lds_bytes() {
+    return 2 * (size_t)(2 * 128 * NWM * 128 + 8 * ((64 * NWN * (QT == 8 ? 64 : 32) / 1024 + 7) / 8) * 1024 + 8 * 256);
 }
 
 }  // namespace
@@ -322,10 +362,11 @@ pg_status pg_launch_rows_to_f16_planes(pg_ctx *ctx, const float *x_dev, size_t r
 // launch wants about one workgroup per CU: short of that, K is cut into up to 8 chunks of at least 512.
 bool pg_gguf_hmm_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_total, size_t k_in, int *ks_out) {
     if (ctx->hmm_mode == 2) return false;
-    if (ggml_type != PG_GGML_Q4_0 || k_in % 64 != 0 || k_in < 256 || k_in > ((size_t)1 << 24) || n_total < 2 || n_total > ((size_t)1 << 24) ||
+    if ((ggml_type != PG_GGML_Q4_0 && ggml_type != PG_GGML_Q8_0) || k_in % 64 != 0 || k_in < 256 || k_in > ((size_t)1 << 24) || n_total < 2 || n_total > ((size_t)1 << 24) ||
         m < 2 || m > ((size_t)1 << 20))
         return false;
-    const size_t bm = m <= 128 ? 128 : 256, bn = m <= 128 ? 512 : 256;
+    const bool wide = m <= 128 || ggml_type == PG_GGML_Q8_0;  // (Q8_0: a stage of 256 x 256 does not fit the LDS twice)
+    const size_t bm = wide ? 128 : 256, bn = wide ? 512 : 256;
     const size_t tiles = ((m + bm - 1) / bm) * ((n_total + bn - 1) / bn);
     size_t ks = (size_t)ctx->num_cu / tiles;
     const size_t stages = k_in / 64;
@@ -341,7 +382,9 @@ bool pg_gguf_hmm_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_tota
     // 144 : 175 / 268 : 345; 4096 -> 4096 at 512 / 1024 / 4096 74 : 59 / 105 : 106 / 281 : 389; 8192 -> 28672 at
     // 64 / 96 / 1024 143 : 115 / 149 : 172 / 899 : 1326.  The f16 route wins from about 18 G multiply-adds on:
     // below that its tiles leave CUs idle or its K chunks cost a pass over their planes.
-    return m >= 96 && (double)m * (double)n_total * (double)k_in >= 1.8e10;
+    // (Q8_0, always on 128 x 512 tiles: 4096 -> 14336 at 256 / 512 / 1024 rows 109 : 112 / 168 : 180 / 266 : 348, 14336 -> 4096 at
+    // 256 / 512 / 1024 143 : 105 / 166 : 188 / 287 : 351, 4096 -> 4096 at 1024 / 2048 111 : 110 / 186 : 202: from about 24 G.)
+    return m >= 96 && (double)m * (double)n_total * (double)k_in >= (ggml_type == PG_GGML_Q8_0 ? 2.4e10 : 1.8e10);
 }
 
 size_t pg_gguf_hmm_part_floats(size_t m, size_t n_total, int ks) { return ks > 1 ? (size_t)ks * m * n_total : 0; }
@@ -352,11 +395,13 @@ pg_status pg_launch_gguf_hmm_group(pg_ctx *ctx, size_t k_in, const pg_gguf_tenso
                                    const pg_hmm_planes &planes, int ks, float *part, bool keep_parts) {
     if (count < 1 || count > PG_HMM_MAX_GROUP) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): %d tensors (1 .. %d)", count, PG_HMM_MAX_GROUP);
     if (m == 0) return PG_OK;
+    const int type = w[0]->ggml_type;
+    if (type != PG_GGML_Q4_0 && type != PG_GGML_Q8_0) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): ggml type %d", type);
     for (int i = 0; i < count; ++i)
-        if (w[i]->k_in != k_in || w[i]->ggml_type != PG_GGML_Q4_0) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): the tensors differ in K or are not Q4_0");
+        if (w[i]->k_in != k_in || w[i]->ggml_type != type) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): the tensors differ in K or type");
     if (k_in % 64 != 0 || planes.rows < m || planes.k != k_in) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): K = %zu, planes of %zu x %zu", k_in, planes.rows, planes.k);
     if (ks < 1 || (ks > 1 && !part && !keep_parts)) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): %d K chunks without a buffer for their planes", ks);
-    const bool wide = m <= 128;   // 128 x 512 tiles
+    const bool q8 = type == PG_GGML_Q8_0, wide = m <= 128 || q8;   // 128 x 512 tiles
     const size_t bm = wide ? 128 : 256, bn = wide ? 512 : 256;
     hmm_group grp;
     int panels = 0;
@@ -380,19 +425,18 @@ pg_status pg_launch_gguf_hmm_group(pg_ctx *ctx, size_t k_in, const pg_gguf_tenso
     if (ks_real != ks) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): %d K chunks of %d stages leave one empty", ks, kt_per);
     const dim3 grid((unsigned)((ntiles + 7) / 8 * 8), (unsigned)ks_real);
     const int nb = (int)(k_in / 32);
-    if (wide) {
-        auto kern = gguf_hmm_q4_kernel<1, 8>;
-        const size_t lds = hmm_lds_bytes<1, 8>();
-        PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
-        PG_TRY(pg_launch(ctx, "gguf_hmm_q4_0", kern, grid, dim3(512), lds, (const _Float16 *)planes.hi, (const _Float16 *)planes.lo,
-                         (const float *)planes.inv, grp, (int)m, nb, tiles_m, ntiles, kt_per));
-    } else {
-        auto kern = gguf_hmm_q4_kernel<2, 4>;
-        const size_t lds = hmm_lds_bytes<2, 4>();
-        PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
-        PG_TRY(pg_launch(ctx, "gguf_hmm_q4_0", kern, grid, dim3(512), lds, (const _Float16 *)planes.hi, (const _Float16 *)planes.lo,
-                         (const float *)planes.inv, grp, (int)m, nb, tiles_m, ntiles, kt_per));
-    }
+#define PG_HMM_LAUNCH(QTT, NWMM, NWNN)                                                                                          \
+    do {                                                                                                                        \
+        auto kern = gguf_hmm_kernel<QTT, NWMM, NWNN>;                                                                           \
+        const size_t lds = hmm_lds_bytes<QTT, NWMM, NWNN>();                                                                    \
+        PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                             \
+        PG_TRY(pg_launch(ctx, QTT == 8 ? "gguf_hmm_q8_0" : "gguf_hmm_q4_0", kern, grid, dim3(512), lds, (const _Float16 *)planes.hi, \
+                         (const _Float16 *)planes.lo, (const float *)planes.inv, grp, (int)m, nb, tiles_m, ntiles, kt_per));    \
+    } while (0)
+    if (q8) PG_HMM_LAUNCH(8, 1, 8);
+    else if (wide) PG_HMM_LAUNCH(4, 1, 8);
+    else PG_HMM_LAUNCH(4, 2, 4);
+#undef PG_HMM_LAUNCH
     if (ks > 1 && !keep_parts) {
         size_t off = 0;
         for (int i = 0; i < count; ++i) {

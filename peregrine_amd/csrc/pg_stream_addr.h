@@ -70,3 +70,19 @@ PG_HD size_t pg_gskinny_scale_offset(int tile, int nb, int unit, int lane) { ret
 // ---- MXFP4 rows (mxfp4_rows_kernel): fragment chunk and scale word a wavefront fetches for chunk index c
 PG_HD int pg_mx_chunk(int c, int ncp) { return c < ncp ? c : ncp - 1; }
 PG_HD int pg_mx_scale_word(int c, int ncp) { return (c < ncp ? c : ncp - 4) >> 2; }
+
+// ---- many rows on the f16 matrix cores (gguf_hmm_kernel): per stage of two blocks a wavefront fills its share
+// of the two activation planes, of the packed weights and of their scales
+// activation or weight row a fill lane fetches: rows past the end repeat the last (their outputs are never stored)
+PG_HD int pg_hmm_clamp_row(int row, int rows) { return row < rows ? row : rows - 1; }
+// byte offset in an f16 plane [rows][k]: row, stage (64 k = 128 bytes), 16-byte chunk of the stage's run
+PG_HD size_t pg_hmm_plane_offset(int row, int k, int stage, int chunk) { return ((size_t)row * k + (size_t)stage * 64) * 2 + (size_t)chunk * 16; }
+// byte offset of a 16-byte block in the Q4_0 payload plane [rows][nb]: block `blk` (0 or 1) of the stage
+PG_HD size_t pg_hmm_weight_offset(int row, int nb, int stage, int blk) { return ((size_t)row * nb + (size_t)stage * 2 + blk) * 16; }
+// the same in the Q8_0 payload plane [rows][2 halves][nb]
+PG_HD size_t pg_hmm_weight_offset_q8(int row, int half, int nb, int stage, int blk) { return (((size_t)row * 2 + half) * nb + (size_t)stage * 2 + blk) * 16; }
+// the scale fill takes two neighbouring rows (4 bytes): the even row it starts at; past the end, the last even row
+// (the scale plane is padded to a multiple of 8 rows)
+PG_HD int pg_hmm_scale_row(int row, int rows) { return row < rows ? row : (rows - 1) & ~1; }
+// byte offset in the scale plane (8 rows x f16 per block and tile of 8 rows)
+PG_HD size_t pg_hmm_scale_offset(int row, int nb, int stage, int blk) { return (((size_t)(row >> 3) * nb + (size_t)stage * 2 + blk) * 8 + (row & 7)) * 2; }

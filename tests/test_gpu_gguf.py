@@ -220,7 +220,7 @@ def test_gguf_matmul_special_inputs(ctx, orc):
     gw.free()
 
 
-# ---- many rows of Q4_0 on the f16 matrix cores (weights exact, activations as two f16 planes) -------------------
+# ---- many rows of Q4_0 / Q8_0 on the f16 matrix cores (weights exact, activations as two f16 planes) -----------
 RTOL_F16_ROUTE = 2e-5   # what that route is held to: the planes drop less than 2^-22 of a row's largest value
 
 # (n_out, k_in, m): forced onto the f16 route whatever the dispatcher would choose
@@ -235,15 +235,16 @@ HMM_SHAPES = [
 ]
 
 
+@pytest.mark.parametrize("typ", [2, 8])
 @pytest.mark.parametrize("n_out,k_in,m", HMM_SHAPES)
-def test_gguf_matmul_f16_route_vs_oracle(ctx, orc, n_out, k_in, m):
+def test_gguf_matmul_f16_route_vs_oracle(ctx, orc, typ, n_out, k_in, m):
     from peregrine_amd import gguf, _ffi
-    say(f"gguf_matmul f16 route n_out={n_out} k_in={k_in} m={m}")
+    say(f"gguf_matmul f16 route type={typ} n_out={n_out} k_in={k_in} m={m}")
     w = orc.rng_normal(1900 + n_out, n_out * k_in, 0.0, 0.02)
-    raw = H.pack_q4_0(w)
+    raw = (H.pack_q4_0 if typ == 2 else H.pack_q8_0)(w)
     x = orc.rng_normal(117 + m, m * k_in)
     x.reshape(m, k_in)[:, :: max(1, k_in // 40)] *= 20
-    gw = gguf.GgufWeight(raw, 2, n_out, k_in, ctx)
+    gw = gguf.GgufWeight(raw, typ, n_out, k_in, ctx)
     _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 1))
     try:
         ctx.profile_begin()
@@ -252,11 +253,11 @@ def test_gguf_matmul_f16_route_vs_oracle(ctx, orc, n_out, k_in, m):
         again = gw.matmul(x, m)
     finally:
         _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 0))
-    assert "gguf_hmm_q4_0" in prof and "rows_to_f16_planes" in prof, prof
+    assert ("gguf_hmm_q4_0" if typ == 2 else "gguf_hmm_q8_0") in prof and "rows_to_f16_planes" in prof, prof
     assert (bits(got) == bits(again)).all()
     rows = range(m) if m * n_out * k_in <= 1 << 31 else sorted({0, 1, m // 2, m - 2, m - 1})
     for r in rows:
-        want = orc.gguf_matmul(x.reshape(m, k_in)[r], 1, raw, 2, n_out, k_in)
+        want = orc.gguf_matmul(x.reshape(m, k_in)[r], 1, raw, typ, n_out, k_in)
         H.assert_close_rel(got.reshape(m, n_out)[r], want, RTOL_F16_ROUTE, f"row {r}")
     gw.free()
 

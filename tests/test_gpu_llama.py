@@ -408,9 +408,10 @@ def test_llama_block_nine_to_sixteen_tokens_mixed_products(ctx, orc, typ):
     _block_case(ctx, orc, 1024, 8, 2, 128, 4096, typ, (20, 9, 16, 13, 5, 1), max_seq=80, seed=67)
 
 
+@pytest.mark.parametrize("typ", [2, 8])
 @pytest.mark.parametrize("shape", [(1024, 8, 2, 128, 2048, (40, 130, 9, 1)), (512, 8, 4, 64, 1280, (33, 17)),
                                    (5120, 5, 1, 128, 1024, (20,))])
-def test_llama_block_many_token_steps_on_the_f16_matrix_cores(ctx, orc, shape):
+def test_llama_block_many_token_steps_on_the_f16_matrix_cores(ctx, orc, shape, typ):
     """The many-token step with its four product launches forced onto the f16 route (at these sizes the dispatcher
     would keep the int8 block product): RMSNorm and SiLU.up write their rows as f16 planes, the attention output is
     converted, q|k|v and gate|up share a launch each, K chunks are left to the consumers to add up.  Steps of up to
@@ -421,11 +422,11 @@ def test_llama_block_many_token_steps_on_the_f16_matrix_cores(ctx, orc, shape):
     _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 1))
     try:
         ctx.profile_begin()
-        _block_case(ctx, orc, d, nqh, nkvh, hd, ffn, 2, steps, max_seq=192, seed=71)
+        _block_case(ctx, orc, d, nqh, nkvh, hd, ffn, typ, steps, max_seq=192, seed=71)
         prof = ctx.profile_end()
     finally:
         _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 0))
-    for name in ("gguf_hmm_q4_0", "add_rmsnorm_f16_planes", "swiglu_f16_planes", "rows_to_f16_planes"):
+    for name in ("gguf_hmm_q4_0" if typ == 2 else "gguf_hmm_q8_0", "add_rmsnorm_f16_planes", "swiglu_f16_planes", "rows_to_f16_planes"):
         assert name in prof, (name, sorted(prof))
 
 

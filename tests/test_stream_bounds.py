@@ -103,6 +103,23 @@ def test_block_few_rows_fills_stay_inside_payload_and_scale_planes():
             assert qs_end == qs_bytes and d_end == d_bytes
 
 
+def test_f16_matrix_core_fills_stay_inside_planes_payload_and_scales():
+    """gguf_hmm_kernel: Q4_0 and Q8_0, both tile shapes, ragged rows on both sides, every K chunk count the dispatcher can pick
+    (chunks of whole stages of 64), odd numbers of weight rows (the scale fill takes rows in pairs)."""
+    for m, n, k in itertools.product([2, 100, 128, 129, 256, 300, 1000], [2, 77, 256, 515, 1100, 4097], [256, 1088, 4096]):
+        for q8, wide in ((0, 1), (1, 1)) if m <= 128 else ((0, 0), (1, 1)):
+            for ks in (1, 2, 3, 5, 8):
+                if (k // 64) // ks < 1:
+                    continue
+                v = [C.c_size_t() for _ in range(6)]
+                check(lib.pg_audit_gguf_hmm(m, n, k, q8, wide, ks, *[C.byref(x) for x in v]))
+                pe, pb, qe, qb, de, db = (x.value for x in v)
+                what = f"gguf_hmm m={m} n={n} k={k} q8={q8} wide={wide} ks={ks}"
+                assert pe == pb, (what, pe, pb)       # the last row's last chunk is read by someone, and nothing past it
+                assert qe == qb, (what, qe, qb)
+                assert de <= db, (what, de, db)
+
+
 def test_mxfp4_rows_loads_stay_inside_the_fragment_planes():
     for k, n in itertools.product([32, 64, 512, 2880, 4096, 28160], [1, 15, 16, 17, 100, 2880]):
         for rg, nw in ((1, 16), (1, 8), (2, 8), (4, 8), (8, 8), (1, 4), (2, 4), (4, 4)):
