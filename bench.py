@@ -216,6 +216,9 @@ def main():
     ap.add_argument("--only-headline", action="store_true", help="cfg3 (and the ceilings) only")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain 512 MiB device copies (counter calibration under rocprofv3 --pmc)")
+    ap.add_argument("--probe-shapes", action="store_true",
+                    help="instead of the benchmark: the pure read probe over launch shapes (workgroups x threads x loads in "
+                         "flight) at the byte counts of the one-row products, one JSON line")
     ap.add_argument("--cache-residency", action="store_true",
                     help="instead of the benchmark: the one-row products timed with 1 .. 12 tensors rotated "
                          "(weights served by the L2s, the Infinity Cache, HBM), one JSON line")
@@ -228,6 +231,9 @@ def main():
 
     B = Bench(args)
     torch, lib, check, ptr, dev = B.torch, B.lib, B.check, B.ptr, B.dev
+    if args.probe_shapes:
+        print(json.dumps(probe_shapes(B)), flush=True)
+        return
     if args.cache_residency:
         print(json.dumps(cache_residency(B)), flush=True)
         return
@@ -400,6 +406,7 @@ def main():
         section_decode_and_linear(B, line)
         section_reference_shapes(B, line)
         section_gguf(B, line)
+        section_gguf_many_rows(B, line)
         section_mxfp4(B, line)
         section_moe(B, line)
         section_llama_block(B, line)
@@ -418,6 +425,21 @@ def main():
     line["cpu_baseline"] = cpu_baseline(B.orc, cpu_w, cpu_a) if B.cpu else None
     print(json.dumps(line), flush=True)
     B.ctx.close()
+
+
+def probe_shapes(B):
+    """What a launch that does nothing but read N bytes reaches, by launch shape: GB/s for every (workgroups, threads
+    per workgroup, 128-bit loads in flight per lane) at the byte counts of cfg4's product (33 MB), cfg2's down (59 MB)
+    and cfg2's gate|up (118 MB); the buffers are rotated so that neither the L2s nor the Infinity Cache serve them."""
+    out = {"what": " ".join(probe_shapes.__doc__.split()), "unit": "GB/s", "rows": []}
+    for label, nbytes, bufs in (("33MB", 33103872, 10), ("59MB", 58851328, 6), ("118MB", 117702656, 4)):
+        for wgs in (256, 512, 1024, 2048, 4096):
+            for thr in (256, 512, 1024):
+                for inflight in (4, 8, 16):
+                    g = C.c_double()
+                    B.check(B.lib.pg_probe_hbm_read_shaped(B.h, nbytes, bufs, 200, wgs, thr, inflight, C.byref(g)))
+                    out["rows"].append([label, wgs, thr, inflight, round(g.value, 1)])
+    return out
 
 
 def cache_residency(B):
@@ -692,6 +714,71 @@ def section_gguf(B, line):
         skinny.append(entry)
     line["gguf_q4_0_skinny"] = skinny
     for h in q4:
+        lib.pg_gguf_free(B.h, h)
+    torch.cuda.empty_cache()
+
+
+def section_gguf_many_rows(B, line):
+    """Row (a) at prefill size: 1024 rows through the Q4_0 dequant-matmul [4096] -> [14336] (a Llama-3-8B gate
+    projection).  The dispatcher's route (f16 matrix cores, weights exact) and, forced, the int8 block product."""
+    import numpy as np
+
+    torch, lib, check, ptr, dev, _ffi = B.torch, B.lib, B.check, B.ptr, B.dev, B.ffi
+    n_out, k_in, m = 14336, 4096, 1024
+    raw = np.frombuffer(B.synth.pack_q4_0(B.normal(7210, (n_out, k_in), 0.02).cpu().numpy()), np.uint8)
+    hs = []
+    for _ in range(8):  # 8 x 33 MB: past the Infinity Cache
+        h = C.c_void_p()
+        check(lib.pg_gguf_upload(B.h, C.c_void_p(raw.ctypes.data), _ffi.GGML_Q4_0, n_out, k_in, C.byref(h)))
+        hs.append(h)
+    x = B.make_acts(m, k_in, 1290)
+    y = torch.empty(m, n_out, device=dev)
+
+    def step():
+        check(lib.pg_gguf_matmul_dev(B.h, ptr(x), m, hs[B.i % len(hs)], ptr(y)))
+        B.i += 1
+
+    flop = 2 * m * n_out * k_in
+    t = B.timed(step, 24, 8)
+    prof, grids = B.profiled(step, 16)
+    k_ms = prof["gguf_hmm_q4_0"][0]
+    check(lib.pg_gguf_hmm_force(B.h, 2))
+    try:
+        t_i8 = B.timed(step, 24, 8)
+        prof_i8, _ = B.profiled(step, 16)
+    finally:
+        check(lib.pg_gguf_hmm_force(B.h, 0))
+    entry = {"workload": f"row (a), prefill size: Q4_0 dequant-matmul [{m}x{k_in}]->[{m}x{n_out}]; {len(hs)} tensors rotated",
+             "value": round(flop / (t["ms_per_step"] * 1e-3) / 1e12, 1), "unit": "TFLOP/s", **B.stats(t),
+             "kernels_ms": {k: round(v[0], 5) for k, v in prof.items()},
+             "roofline": {"kernel": "gguf_hmm_kernel<Q4_0, 2, 4> (v_mfma_f32_16x16x32_f16; weights unpacked exactly in registers, "
+                                    "activations as two f16 planes: twice the counted flops run on the matrix cores)",
+                          "bound": "mfma", "achieved": round(flop / (k_ms * 1e-3) / 1e12, 1), "peak": 2500.0, "unit": "TFLOP/s",
+                          "frac": round(flop / (k_ms * 1e-3) / 1e12 / 2500.0, 4), "executed_tflops": round(2 * flop / (k_ms * 1e-3) / 1e12, 1),
+                          "traffic": B.traffic_for("gguf_hmm_q4_0", grids), "flop_per_launch": flop, "avg_launch_ms": round(k_ms, 5)},
+             "int8_block_route": {"ms_per_step": t_i8["ms_per_step"], "tflops": round(flop / (t_i8["ms_per_step"] * 1e-3) / 1e12, 1),
+                                  "kernels_ms": {k: round(v[0], 5) for k, v in prof_i8.items()}}}
+    if B.cpu:
+        rows = 4
+        xs = x[:rows].cpu().numpy()
+        want = np.empty(rows * n_out, np.float32)
+        olib = B.orc["lib"]
+
+        def run():
+            assert olib.orc_gguf_matmul(_vp(xs), C.c_size_t(rows), _vp(raw), C.c_int(_ffi.GGML_Q4_0), C.c_size_t(n_out), C.c_size_t(k_in), _vp(want)) == 0
+
+        dt = _best_of(run, 1)
+        step()  # (the dispatcher's route again: y held the forced run's result)
+        torch.cuda.synchronize()
+        got = y[:rows].cpu().numpy().reshape(rows, n_out).astype(np.float64)
+        ref = want.reshape(rows, n_out).astype(np.float64)
+        floor = np.sqrt((ref * ref).mean(axis=1, keepdims=True))
+        entry["max_error_vs_cpu_oracle"] = float(f"{(np.abs(got - ref) / np.maximum(np.abs(ref), floor)).max():.3e}")
+        entry["cpu_baseline"] = {"value": round(2 * rows * n_out * k_in / dt / 1e12, 5), "unit": "TFLOP/s", "ms": round(dt * 1e3, 1), "cores": 1,
+                                 "kind": "port", "sample": f"{rows} of the {m} rows through the oracle's dequantise -> f32 product "
+                                                           f"(linear in the rows), single thread, gcc {B.orc['flags']}"}
+    line["gguf_q4_0_many_rows"] = entry
+    for h in hs:
         lib.pg_gguf_free(B.h, h)
     torch.cuda.empty_cache()
 
