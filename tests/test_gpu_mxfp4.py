@@ -123,10 +123,22 @@ def test_mxfp4_workgroup_shapes(ctx, orc, out_dim, in_dim, m):
     (2880, 2880, 24, 118, 124), (8192, 4096, 16, 118, 124), (5760, 2880, 100, 118, 124), (600, 4096, 300, 104, 144),   # every scale an f16: the Q8_0 twin
     (520, 512, 40, 100, 150),                                                               # some are not: the decode kernel
 ])
-def test_mxfp4_many_rows(ctx, orc, out_dim, in_dim, m, lo, hi):
+@pytest.mark.parametrize("f16_route", [False, True])
+def test_mxfp4_many_rows(ctx, orc, out_dim, in_dim, m, lo, hi, f16_route):
     """From 16 activation rows on (24 for a small tensor) a tensor whose block scales are all f16 values goes through the matrix-core
     block product (16-bit fixed-point activations per block: 4e-4); one with a scale outside f16 stays on the
-    decode kernel and keeps its tolerance.  One row on the same tensor afterwards still takes the decode kernel."""
+    decode kernel and keeps its tolerance.  One row on the same tensor afterwards still takes the decode kernel.
+    f16_route: the twin's product forced onto the f16 matrix cores (what the dispatcher picks at prefill sizes)."""
+    from peregrine_amd import mxfp4, _ffi
+    if f16_route:
+        _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 1))
+    try:
+        _mxfp4_many_rows(ctx, orc, out_dim, in_dim, m, lo, hi, f16_route)
+    finally:
+        _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 0))
+
+
+def _mxfp4_many_rows(ctx, orc, out_dim, in_dim, m, lo, hi, f16_route):
     from peregrine_amd import mxfp4
     say(f"mxfp4 many rows [{m} x {in_dim}] -> [{out_dim}] scales {lo}..{hi - 1}")
     rng = np.random.default_rng(out_dim + 3 * in_dim + m)
@@ -135,11 +147,14 @@ def test_mxfp4_many_rows(ctx, orc, out_dim, in_dim, m, lo, hi):
     w = mxfp4.upload(b, s, out_dim, in_dim, ctx)
     x = orc.rng_normal(m + 5, m * in_dim).reshape(m, in_dim)
     x[:, ::61] *= 25.0
+    ctx.profile_begin()
     got = w.matmul(x, m).reshape(m, out_dim)
+    prof = ctx.profile_end()
     rows = np.concatenate([[0], rng.choice(np.arange(1, out_dim), size=min(out_dim - 1, 95), replace=False)])
     bb = b.reshape(out_dim, -1)[rows].reshape(-1)
     ss = s.reshape(out_dim, -1)[rows].reshape(-1)
     twin = lo >= 104 and hi <= 144
+    assert ("gguf_hmm_q8_0" in prof) == (twin and f16_route), prof
     for i in list(range(0, m, max(1, m // 12))) + [m - 1]:
         want = orc.mxfp4_matmul(x[i], bb, ss, len(rows), in_dim)
         H.assert_close_rel(got[i][rows], want, RTOL_CONTRACT, f"row {i} (contract)")
