@@ -56,8 +56,20 @@ class Hip:
         return graph, ex
 
 
-@pytest.mark.parametrize("typ,seq", [(2, 1), (8, 1), (2, 4)])
-def test_block_step_replayed_from_a_graph(ctx, orc, typ, seq):
+@pytest.mark.parametrize("typ,seq,f16_route", [(2, 1, False), (8, 1, False), (2, 4, False), (2, 40, True), (8, 40, True)])
+def test_block_step_replayed_from_a_graph(ctx, orc, typ, seq, f16_route):
+    """f16_route: a many-token step with its products forced onto the f16 matrix cores (planes written by RMSNorm and
+    SiLU.up, K chunks summed by the consumers): what a captured prefill chunk of a large model runs."""
+    from peregrine_amd import _ffi
+    if f16_route:
+        _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 1))
+    try:
+        _block_step_replayed(ctx, orc, typ, seq)
+    finally:
+        _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 0))
+
+
+def _block_step_replayed(ctx, orc, typ, seq):
     from peregrine_amd import _ffi, gguf, llama
     hip = Hip()
     d, nqh, nkvh, hd, ffn, pre = 256, 8, 2, 64, 512, 300     # 300 positions: the keys are cut into splits / runs

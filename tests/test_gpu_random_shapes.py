@@ -74,6 +74,37 @@ def test_gguf_matmul_random_shapes(ctx, orc, seed):
         gw.free()
 
 
+@pytest.mark.parametrize("seed", [41, 42])
+def test_gguf_matmul_random_shapes_on_the_f16_matrix_cores(ctx, orc, seed):
+    """The many-row route forced for every shape it can take (K a multiple of 64, two rows and more): both tile shapes,
+    ragged rows and weight rows, 4 to 130 stages in 1 to 8 K chunks, Q4_0 and Q8_0, outlier channels, a zero row."""
+    from peregrine_amd import gguf, _ffi
+    rng = np.random.default_rng(seed)
+    _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 1))
+    try:
+        for case in range(30):
+            typ = _pick(rng, 2, 8)
+            m = _pick(rng, 2, 5, 16, 33, 100, 127, 128, 129, 200, 255, 256, 257, 300, 513)
+            k_in = 64 * _pick(rng, 4, 5, 8, 9, 16, 17, 33, 64, 65, 130)
+            n_out = _pick(rng, 2, 31, 64, 100, 255, 256, 257, 300, 511, 513, 777, 1025)
+            say(f"gguf f16-route random case {case}: type={typ} m={m} n_out={n_out} k_in={k_in}")
+            raw = (H.pack_q4_0 if typ == 2 else H.pack_q8_0)(orc.rng_normal(seed * 1000 + case, n_out * k_in, 0.0, 0.02))
+            x = orc.rng_normal(seed * 1000 + 500 + case, m * k_in).reshape(m, k_in)
+            x[:, :: max(1, k_in // 23)] *= 20
+            x[m // 2] = 0
+            gw = gguf.GgufWeight(raw, typ, n_out, k_in, ctx)
+            ctx.profile_begin()
+            got = gw.matmul(x.reshape(-1), m).reshape(m, n_out)
+            prof = ctx.profile_end()
+            assert any(k.startswith("gguf_hmm") for k in prof), prof
+            assert (got[m // 2] == 0).all()
+            for r in sorted({0, 1, m // 3, m - 2, m - 1} - {m // 2}):
+                H.assert_close_rel(got[r], orc.gguf_matmul(x[r], 1, raw, typ, n_out, k_in), 2e-5, f"row {r}")
+            gw.free()
+    finally:
+        _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 0))
+
+
 @pytest.mark.parametrize("seed", [31, 32])
 def test_attention_random_shapes_and_masks(ctx, orc, seed):
     from peregrine_amd import llama
