@@ -1062,8 +1062,17 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
         PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, m, w->k_in, w->ggml_type, md));
         return pg_launch_gguf_skinny_group(ctx, w->ggml_type, w->k_in, &w, &y_dev, 1, m, md);
     }
-    if (pg_gguf_hmm_takes(ctx, w->ggml_type, m, w->n_out, w->k_in, &hks))  // many rows of Q4_0: the f16 matrix cores
+    if (pg_gguf_hmm_takes(ctx, w->ggml_type, m, w->n_out, w->k_in, &hks))  // many rows of Q4_0 / Q8_0: the f16 matrix cores
         return pg_gguf_hmm_rows(ctx, x_dev, m, &w, &y_dev, 1, hks);
+    if (q41 && w->k_in <= 32768 && pg_gguf_hmm_takes(ctx, PG_GGML_Q4_0, m, w->n_out, w->k_in, &hks)) {
+        // Q4_1 at that size: the first term d sum (q - 8) x as the Q4_0 product on the f16 matrix cores, then the
+        // offsets times the rows' block sums (which the digit launch writes beside its planes)
+        PG_TRY(pg_gguf_hmm_rows(ctx, x_dev, m, &w, &y_dev, 1, hks));
+        PG_TRY(pg_workspace(ctx, pg_mmdigits_bytes(m, w->k_in), &ws));   // (the product is done with the arena)
+        const pg_mmdigits md = pg_mmdigits_carve(ws, m, w->k_in);
+        PG_TRY(pg_launch_x_to_mm_digits(ctx, x_dev, m, w->k_in, w->ggml_type, md));
+        return pg_launch_q41_offset(ctx, w, md, m, y_dev);
+    }
     const int ks = pg_gguf_mm_splitk(ctx, w->n_out, w->k_in, (m + 31) / 32, m, false, nullptr);
     const size_t sz_d = pg_mmdigits_bytes(m, w->k_in);
     const size_t sz_part = ks > 1 ? pg_round_up((size_t)ks * m * w->n_out * sizeof(float), 256) : 0;

@@ -395,10 +395,12 @@ pg_status pg_launch_gguf_hmm_group(pg_ctx *ctx, size_t k_in, const pg_gguf_tenso
                                    const pg_hmm_planes &planes, int ks, float *part, bool keep_parts) {
     if (count < 1 || count > PG_HMM_MAX_GROUP) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): %d tensors (1 .. %d)", count, PG_HMM_MAX_GROUP);
     if (m == 0) return PG_OK;
-    const int type = w[0]->ggml_type;
+    // (a Q4_1 tensor's nibbles and scales are laid out as a Q4_0 tensor's: its first term runs as the Q4_0 product)
+    auto kind = [](int t) { return t == PG_GGML_Q4_1 ? PG_GGML_Q4_0 : t; };
+    const int type = kind(w[0]->ggml_type);
     if (type != PG_GGML_Q4_0 && type != PG_GGML_Q8_0) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): ggml type %d", type);
     for (int i = 0; i < count; ++i)
-        if (w[i]->k_in != k_in || w[i]->ggml_type != type) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): the tensors differ in K or type");
+        if (w[i]->k_in != k_in || kind(w[i]->ggml_type) != type) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): the tensors differ in K or type");
     if (k_in % 64 != 0 || planes.rows < m || planes.k != k_in) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): K = %zu, planes of %zu x %zu", k_in, planes.rows, planes.k);
     if (ks < 1 || (ks > 1 && !part && !keep_parts)) return pg_fail(PG_EINVAL, "gguf (f16 matrix cores): %d K chunks without a buffer for their planes", ks);
     const bool q8 = type == PG_GGML_Q8_0, wide = m <= 128 || q8;   // 128 x 512 tiles

@@ -322,3 +322,28 @@ def test_gguf_matmul_f16_route_special_rows(ctx, orc):
     w_col = orc.gguf_matmul(x[7], 1, raw, 2, n_out, k_in)
     assert (bits(got[7]) == bits(w_col)).all()                # a single product per output: no rounding anywhere
     gw.free()
+
+
+@pytest.mark.parametrize("n_out,k_in,m", [(515, 4160, 300), (1100, 2048, 100), (256, 256, 129)])
+def test_gguf_matmul_f16_route_q4_1(ctx, orc, n_out, k_in, m):
+    """Q4_1 at prefill sizes: the first term as the Q4_0 product on the f16 matrix cores (same nibbles and scales),
+    then the launch that adds the blocks' offsets times the rows' block sums."""
+    from peregrine_amd import gguf, _ffi
+    say(f"gguf_matmul f16 route Q4_1 n_out={n_out} k_in={k_in} m={m}")
+    w = orc.rng_normal(2900 + n_out, n_out * k_in, 0.0, 0.02) + np.float32(0.03)
+    raw = H.pack_q4_1(w)
+    x = orc.rng_normal(217 + m, m * k_in)
+    x.reshape(m, k_in)[:, :: max(1, k_in // 40)] *= 20
+    gw = gguf.GgufWeight(raw, 3, n_out, k_in, ctx)
+    _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 1))
+    try:
+        ctx.profile_begin()
+        got = gw.matmul(x, m).reshape(m, n_out)
+        prof = ctx.profile_end()
+    finally:
+        _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 0))
+    assert "gguf_hmm_q4_0" in prof and "gguf_q4_1_offsets" in prof, prof
+    for r in sorted({0, 1, m // 2, m - 1}):
+        want = orc.gguf_matmul(x.reshape(m, k_in)[r], 1, raw, 3, n_out, k_in)
+        H.assert_close_rel(got[r], want, RTOL_ACHIEVED[3], f"row {r}")
+    gw.free()
