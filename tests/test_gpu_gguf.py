@@ -347,3 +347,30 @@ def test_gguf_matmul_f16_route_q4_1(ctx, orc, n_out, k_in, m):
         want = orc.gguf_matmul(x.reshape(m, k_in)[r], 1, raw, 3, n_out, k_in)
         H.assert_close_rel(got[r], want, RTOL_ACHIEVED[3], f"row {r}")
     gw.free()
+
+
+@pytest.mark.parametrize("typ,bb", [(2, 18), (8, 34)])
+def test_gguf_matmul_f16_route_every_quant_value(ctx, orc, typ, bb):
+    """Blocks of random bytes (every nibble and every int8 value, -128 included) with scales of both signs: the
+    unpacking of quants into f16 values is exact for all of them."""
+    from peregrine_amd import gguf, _ffi
+    n_out, k_in, m = 96, 512, 5
+    rng = np.random.default_rng(1234 + typ)
+    nblocks = n_out * k_in // 32
+    blocks = rng.integers(0, 256, size=(nblocks, bb), dtype=np.uint8)
+    scales = (rng.choice([0.5, -0.25, 0.0625, 1.5, -3.0, 0.0], size=nblocks) * 0.01).astype(np.float16)
+    blocks[:, :2] = scales.view(np.uint8).reshape(nblocks, 2)
+    if typ == 8:
+        blocks[0, 2:] = 0x80                       # a block of -128s
+    raw = blocks.tobytes()
+    x = orc.rng_normal(77, m * k_in)
+    gw = gguf.GgufWeight(raw, typ, n_out, k_in, ctx)
+    _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 1))
+    try:
+        got = gw.matmul(x, m).reshape(m, n_out)
+    finally:
+        _ffi.check(_ffi.lib.pg_gguf_hmm_force(ctx.handle, 0))
+    want = orc.gguf_matmul(x, m, raw, typ, n_out, k_in).reshape(m, n_out)
+    for r in range(m):
+        H.assert_close_rel(got[r], want[r], RTOL_F16_ROUTE, f"row {r}")
+    gw.free()
