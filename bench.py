@@ -412,6 +412,7 @@ def main():
         section_llama_block(B, line)
         section_decode_attention(B, line)
         section_huffman(B, line)
+        section_huffman_kv(B, line)
 
     if args.calibrate_copy:  # a plain copy of known size: 512 MiB read + 512 MiB written per launch
         src = torch.empty(128 << 20, device=dev, dtype=torch.float32).normal_()
@@ -1051,6 +1052,70 @@ def section_huffman(B, line):
         "symbols_per_s_kernels": round(hk * hn / (huff_kernels_ms * 1e-3), 0),
         "kernels_ms_x_launches": {k: [round(v[0], 4), round(v[1] / 5, 1)] for k, v in hprof.items()}}
     lib.pg_huffman_tensor_free(ht)
+
+
+def section_huffman_kv(B, line):
+    """HuffmanKVCache::compress_chunk / decompress_chunk on a chunk that is already on the device:
+    8 KV heads x 256 tokens x 128 (1 MiB of f32 per side), wall time per call (each call waits for
+    its histogram and for the stream's length, so kernel time is the smaller part)."""
+    lib, check = B.lib, B.check
+    heads, tokens, hd = 8, 256, 128
+    n = heads * tokens * hd
+    data = B.normal(7500, (n,), 1.0)
+    out = B.torch.empty(n, dtype=B.torch.float32, device=data.device)
+    chunk = C.c_void_p()
+
+    def compress():
+        h = C.c_void_p()
+        check(lib.pg_huffman_kv_compress_chunk_dev(B.h, C.c_void_p(data.data_ptr()), tokens * hd, tokens, heads, hd, C.byref(h)))
+        return h
+
+    def comp_step():
+        lib.pg_huffman_kv_chunk_free(B.h, compress())
+
+    chunk = compress()
+    nbytes = C.c_size_t()
+    check(lib.pg_huffman_kv_chunk_info(chunk, None, None, None, C.byref(nbytes)))
+
+    def dec_step():
+        check(lib.pg_huffman_kv_decompress_chunk_dev(B.h, chunk, C.c_void_p(out.data_ptr()), tokens * hd))
+
+    res = {}
+    for name, fn in (("compress", comp_step), ("decompress", dec_step)):
+        for _ in range(2):
+            fn()
+        B.torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            fn()
+        B.torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / 10 * 1e3
+        prof, _ = B.profiled(fn, 5)
+        res[name] = {"ms_per_call_wall": round(wall, 3),
+                     "kernels_ms": round(sum(v[0] * v[1] for v in prof.values()) / 5, 4),
+                     "kernels_ms_x_launches": {k: [round(v[0], 4), round(v[1] / 5, 1)] for k, v in prof.items()}}
+    if B.cpu:  # the scalar restatement of compress_chunk / decompress_chunk on the same chunk (the prebuilt -O2 oracle)
+        import numpy as np
+        olib = C.CDLL(os.path.join(ROOT, "oracle", "_build", "libperegrine_oracle.so"))
+        olib.orc_huffman_kv_compress_chunk.restype = C.c_size_t
+        host = data.cpu().numpy()
+        bits, scales, book, back = np.zeros(2 * n + 16, np.uint8), np.zeros(heads, np.float32), np.zeros(256, np.uint8), np.zeros(n, np.float32)
+        vp = lambda a: C.c_void_p(a.ctypes.data)
+        sz = C.c_size_t
+        best = [1e9, 1e9]
+        for _ in range(3):
+            t0 = time.perf_counter()
+            nb = olib.orc_huffman_kv_compress_chunk(vp(host), sz(tokens), sz(heads), sz(hd), vp(bits), vp(scales), vp(book), None)
+            t1 = time.perf_counter()
+            olib.orc_huffman_kv_decompress_chunk(vp(bits), sz(nb), vp(scales), vp(book), sz(tokens), sz(heads), sz(hd), vp(back))
+            best = [min(best[0], t1 - t0), min(best[1], time.perf_counter() - t1)]
+        res["cpu_baseline"] = {"compress_ms": round(best[0] * 1e3, 3), "decompress_ms": round(best[1] * 1e3, 3), "cores": 1, "kind": "port",
+                               "sample": "the same chunk, best of 3, single thread, gcc -O2"}
+    line["huffman_kv_chunk"] = {
+        "workload": f"HuffmanKVCache chunk of {heads} heads x {tokens} tokens x {hd} f32 on the device "
+                    f"({4 * n / 1e6:.2f} MB -> {nbytes.value / 1e6:.3f} MB, {8 * nbytes.value / n:.2f} bits per value)",
+        **res}
+    lib.pg_huffman_kv_chunk_free(B.h, chunk)
 
 
 # ---------------------------------------------------------------------- CPU baseline legs (the oracle; reported only)

@@ -40,7 +40,8 @@ pub const PG_MASK_LOCAL_GLOBAL: c_int = 3;
 macro_rules! opaque {
     ($($name:ident),*) => { $( #[repr(C)] pub struct $name { _private: [u8; 0] } )* };
 }
-opaque!(pg_ctx, pg_qtensor, pg_gguf_tensor, pg_mxfp4_expert, pg_gguf_file, pg_huffman_tensor, pg_rope, pg_kv_cache, pg_llama_block);
+opaque!(pg_ctx, pg_qtensor, pg_gguf_tensor, pg_mxfp4_expert, pg_gguf_file, pg_huffman_tensor, pg_huffman_kv_chunk,
+        pg_huffman_kv_cache, pg_rope, pg_kv_cache, pg_llama_block);
 
 // ---- generated from include/peregrine_hip.h: begin ----
 extern "C" {
@@ -120,6 +121,26 @@ extern "C" {
     pub fn pg_huffman_tensor_decode_to_quantized(ctx: *mut pg_ctx, t: *const pg_huffman_tensor, q: *mut i8, q_t: *mut i8, scales: *mut f32) -> pg_status;
     pub fn pg_huffman_tensor_to_gpu(ctx: *mut pg_ctx, t: *const pg_huffman_tensor, out: *mut *mut pg_qtensor) -> pg_status;
     pub fn pg_matmul_huffman(ctx: *mut pg_ctx, a: *const f32, m: usize, k: usize, t: *const pg_huffman_tensor, out: *mut f32) -> pg_status;
+    pub fn pg_huffman_kv_compress_chunk(ctx: *mut pg_ctx, data: *const f32, num_tokens: usize, num_heads: usize, head_dim: usize, out: *mut *mut pg_huffman_kv_chunk) -> pg_status;
+    pub fn pg_huffman_kv_compress_chunk_dev(ctx: *mut pg_ctx, data_dev: *const f32, head_stride: usize, num_tokens: usize, num_heads: usize, head_dim: usize, out: *mut *mut pg_huffman_kv_chunk) -> pg_status;
+    pub fn pg_huffman_kv_chunk_from_parts(ctx: *mut pg_ctx, bitstream: *const u8, bytes: usize, scales: *const f32, codebook: *const u8, num_tokens: usize, num_heads: usize, head_dim: usize, out: *mut *mut pg_huffman_kv_chunk) -> pg_status;
+    pub fn pg_huffman_kv_chunk_free(ctx: *mut pg_ctx, c: *mut pg_huffman_kv_chunk);
+    pub fn pg_huffman_kv_chunk_info(c: *const pg_huffman_kv_chunk, num_tokens: *mut usize, num_heads: *mut usize, head_dim: *mut usize, bitstream_bytes: *mut usize) -> pg_status;
+    pub fn pg_huffman_kv_chunk_parts(ctx: *mut pg_ctx, c: *const pg_huffman_kv_chunk, bitstream: *mut u8, scales: *mut f32, codebook: *mut u8) -> pg_status;
+    pub fn pg_huffman_kv_decompress_chunk(ctx: *mut pg_ctx, c: *const pg_huffman_kv_chunk, out: *mut f32) -> pg_status;
+    pub fn pg_huffman_kv_decompress_chunk_dev(ctx: *mut pg_ctx, c: *const pg_huffman_kv_chunk, out_dev: *mut f32, head_stride: usize) -> pg_status;
+    pub fn pg_huffman_kv_cache_create(ctx: *mut pg_ctx, num_kv_heads: usize, head_dim: usize, compress_threshold: usize, chunk_size: usize, out: *mut *mut pg_huffman_kv_cache) -> pg_status;
+    pub fn pg_huffman_kv_cache_free(ctx: *mut pg_ctx, c: *mut pg_huffman_kv_cache);
+    pub fn pg_huffman_kv_cache_append(ctx: *mut pg_ctx, c: *mut pg_huffman_kv_cache, new_k: *const f32, new_v: *const f32, seq_len: usize) -> pg_status;
+    pub fn pg_huffman_kv_cache_append_dev(ctx: *mut pg_ctx, c: *mut pg_huffman_kv_cache, new_k_dev: *const f32, new_v_dev: *const f32, seq_len: usize) -> pg_status;
+    pub fn pg_huffman_kv_cache_len(c: *const pg_huffman_kv_cache) -> usize;
+    pub fn pg_huffman_kv_cache_compressed_len(c: *const pg_huffman_kv_cache) -> usize;
+    pub fn pg_huffman_kv_cache_compress_threshold(c: *const pg_huffman_kv_cache) -> usize;
+    pub fn pg_huffman_kv_cache_num_chunks(c: *const pg_huffman_kv_cache) -> usize;
+    pub fn pg_huffman_kv_cache_hot(c: *mut pg_huffman_kv_cache, out: *mut *mut pg_kv_cache) -> pg_status;
+    pub fn pg_huffman_kv_cache_chunk(c: *const pg_huffman_kv_cache, value_side: c_int, index: usize, out: *mut *const pg_huffman_kv_chunk) -> pg_status;
+    pub fn pg_huffman_kv_cache_get_kv(ctx: *mut pg_ctx, c: *const pg_huffman_kv_cache, k: *mut f32, v: *mut f32) -> pg_status;
+    pub fn pg_huffman_kv_cache_get_kv_dev(ctx: *mut pg_ctx, c: *const pg_huffman_kv_cache, k_dev: *mut f32, v_dev: *mut f32) -> pg_status;
     pub fn pg_moe_ffn(ctx: *mut pg_ctx, x: *const f32, T: usize, router_logits: *const f32, E: usize, top_k: usize, gate: *const *const pg_gguf_tensor, up: *const *const pg_gguf_tensor, down: *const *const pg_gguf_tensor, act: c_int, out: *mut f32) -> pg_status;
     pub fn pg_moe_ffn_dev(ctx: *mut pg_ctx, x_dev: *const f32, T: usize, router_logits_dev: *const f32, E: usize, top_k: usize, gate: *const *const pg_gguf_tensor, up: *const *const pg_gguf_tensor, down: *const *const pg_gguf_tensor, act: c_int, out_dev: *mut f32) -> pg_status;
     pub fn pg_moe_ffn_routed(ctx: *mut pg_ctx, x: *const f32, T: usize, expert_idx: *const i32, weight: *const f32, E: usize, top_k: usize, gate: *const *const pg_gguf_tensor, up: *const *const pg_gguf_tensor, down: *const *const pg_gguf_tensor, act: c_int, shared: *const f32, out: *mut f32) -> pg_status;

@@ -339,6 +339,67 @@ pg_status pg_huffman_tensor_to_gpu(pg_ctx *ctx, const pg_huffman_tensor *t, pg_q
 /* matmul_huffman  src/huffman.rs:465-474: decode, then pg_matmul_quantized. */
 pg_status pg_matmul_huffman(pg_ctx *ctx, const float *a, size_t m, size_t k, const pg_huffman_tensor *t, float *out);
 
+/* ---- Huffman-coded KV cache (src/huffman.rs:476-724) -------------------------------------
+ * HuffmanKVCache keeps a window of recent tokens as f32 (a StandardKVCache, on the device)
+ * and older tokens as chunks of int8 values, one scale per head, Huffman-coded.  Chunks are
+ * built, kept and decoded in device memory; only the 256-entry code table is host work. */
+typedef struct pg_kv_cache pg_kv_cache;                   /* attention::StandardKVCache  src/attention.rs:8-15 */
+typedef struct pg_huffman_kv_chunk pg_huffman_kv_chunk;   /* CompressedChunk  src/huffman.rs:500-513 */
+typedef struct pg_huffman_kv_cache pg_huffman_kv_cache;   /* HuffmanKVCache   src/huffman.rs:484-497 */
+/* HuffmanKVCache::compress_chunk  src/huffman.rs:612-658: data [num_heads, num_tokens, head_dim]
+ * (host).  Its assert on data.len() is the caller's to keep: the sizes say how much is read. */
+pg_status pg_huffman_kv_compress_chunk(pg_ctx *ctx, const float *data, size_t num_tokens, size_t num_heads,
+                                       size_t head_dim, pg_huffman_kv_chunk **out);
+/* The same on device data; head h starts at data_dev + h * head_stride (floats), as the heads of a
+ * StandardKVCache do (src/huffman.rs:579-596 extract_chunk_data without the copy). */
+pg_status pg_huffman_kv_compress_chunk_dev(pg_ctx *ctx, const float *data_dev, size_t head_stride, size_t num_tokens,
+                                           size_t num_heads, size_t head_dim, pg_huffman_kv_chunk **out);
+/* The struct literal CompressedChunk { bitstream, scales, codebook, .. }  src/huffman.rs:649-657
+ * from stored parts (copied): scales [num_heads], codebook [256]. */
+pg_status pg_huffman_kv_chunk_from_parts(pg_ctx *ctx, const uint8_t *bitstream, size_t bytes, const float *scales,
+                                         const uint8_t *codebook, size_t num_tokens, size_t num_heads, size_t head_dim,
+                                         pg_huffman_kv_chunk **out);
+void pg_huffman_kv_chunk_free(pg_ctx *ctx, pg_huffman_kv_chunk *c);
+/* num_tokens, num_heads, head_dim and bitstream.len(); any out pointer may be NULL. */
+pg_status pg_huffman_kv_chunk_info(const pg_huffman_kv_chunk *c, size_t *num_tokens, size_t *num_heads, size_t *head_dim,
+                                   size_t *bitstream_bytes);
+/* Copies of bitstream [bitstream_bytes], scales [num_heads], codebook [256]; any may be NULL. */
+pg_status pg_huffman_kv_chunk_parts(pg_ctx *ctx, const pg_huffman_kv_chunk *c, uint8_t *bitstream, float *scales,
+                                    uint8_t *codebook);
+/* HuffmanKVCache::decompress_chunk  src/huffman.rs:661-680: out [num_heads, num_tokens, head_dim] (host).
+ * A codebook that does not decode the stream is PG_EINVAL, as in pg_huffman_decode. */
+pg_status pg_huffman_kv_decompress_chunk(pg_ctx *ctx, const pg_huffman_kv_chunk *c, float *out);
+/* The same into device memory, head h at out_dev + h * head_stride. */
+pg_status pg_huffman_kv_decompress_chunk_dev(pg_ctx *ctx, const pg_huffman_kv_chunk *c, float *out_dev, size_t head_stride);
+/* HuffmanKVCache::new  src/huffman.rs:524-540 (compress_threshold = max(compress_threshold, chunk_size)).
+ * chunk_size 0, with which the reference's append never returns once the threshold is met, is PG_EINVAL. */
+pg_status pg_huffman_kv_cache_create(pg_ctx *ctx, size_t num_kv_heads, size_t head_dim, size_t compress_threshold,
+                                     size_t chunk_size, pg_huffman_kv_cache **out);
+void pg_huffman_kv_cache_free(pg_ctx *ctx, pg_huffman_kv_cache *c);
+/* HuffmanKVCache::append  src/huffman.rs:544-556 (new_k, new_v [num_kv_heads, seq_len, head_dim], host):
+ * appends to the hot window, then compresses the oldest chunk_size tokens while the window holds
+ * at least compress_threshold (compress_oldest_chunk + remove_oldest_tokens, :559-610). */
+pg_status pg_huffman_kv_cache_append(pg_ctx *ctx, pg_huffman_kv_cache *c, const float *new_k, const float *new_v,
+                                     size_t seq_len);
+pg_status pg_huffman_kv_cache_append_dev(pg_ctx *ctx, pg_huffman_kv_cache *c, const float *new_k_dev, const float *new_v_dev,
+                                         size_t seq_len);
+/* len()  src/huffman.rs:683-685, the compressed_len and compress_threshold fields, k_chunks.len(). */
+size_t pg_huffman_kv_cache_len(const pg_huffman_kv_cache *c);
+size_t pg_huffman_kv_cache_compressed_len(const pg_huffman_kv_cache *c);
+size_t pg_huffman_kv_cache_compress_threshold(const pg_huffman_kv_cache *c);
+size_t pg_huffman_kv_cache_num_chunks(const pg_huffman_kv_cache *c);
+/* The `hot` field (owned by the cache; do not free or append to it directly). */
+pg_status pg_huffman_kv_cache_hot(pg_huffman_kv_cache *c, pg_kv_cache **out);
+/* k_chunks[index] (value_side 0) or v_chunks[index] (1), owned by the cache. */
+pg_status pg_huffman_kv_cache_chunk(const pg_huffman_kv_cache *c, int value_side, size_t index,
+                                    const pg_huffman_kv_chunk **out);
+/* HuffmanKVCache::get_kv  src/huffman.rs:689-724: k, v [num_kv_heads, len(), head_dim] (host), per
+ * head the decoded chunks in order, then the hot window.  The hot window of head h is read at
+ * h * head_stride(); the reference reads it at h * hot.len * head_dim (:707), which is the same
+ * place only for head 0 or a window that fills its capacity. */
+pg_status pg_huffman_kv_cache_get_kv(pg_ctx *ctx, const pg_huffman_kv_cache *c, float *k, float *v);
+pg_status pg_huffman_kv_cache_get_kv_dev(pg_ctx *ctx, const pg_huffman_kv_cache *c, float *k_dev, float *v_dev);
+
 /* ---- grouped MoE expert FFN ------------------------------------------------- */
 
 /* MoELayer::forward after the router matmul  examples/grok1/moe.rs:70-109
@@ -377,7 +438,6 @@ pg_status pg_moe_ffn_routed_dev(pg_ctx *ctx, const float *x_dev, size_t T, const
 /* ---- Llama decoder block: the glue around the quantised products -------------- */
 
 typedef struct pg_rope pg_rope;               /* nn::RoPE                  src/nn.rs:1250-1256 */
-typedef struct pg_kv_cache pg_kv_cache;       /* attention::StandardKVCache src/attention.rs:8-15 */
 typedef struct pg_llama_block pg_llama_block; /* LlamaBlock                src/models/llama/decoder.rs:7-16 */
 
 /* attention::AttentionMask  src/attention.rs:102-120 (LocalGlobal is not offered). */

@@ -594,6 +594,87 @@ inline std::vector<float> matmul_huffman(const GpuContext &gpu, const std::vecto
     return out;
 }
 
+// CompressedChunk  src/huffman.rs:500-513; the bitstream stays in device memory.
+class CompressedChunk {
+public:
+    CompressedChunk(const GpuContext &gpu, pg_huffman_kv_chunk *h) : gpu_(&gpu), h_(h) {}
+    ~CompressedChunk() { if (h_) pg_huffman_kv_chunk_free(gpu_->raw(), h_); }
+    CompressedChunk(CompressedChunk &&o) noexcept : gpu_(o.gpu_), h_(o.h_) { o.h_ = nullptr; }
+    CompressedChunk(const CompressedChunk &) = delete;
+    CompressedChunk &operator=(const CompressedChunk &) = delete;
+    size_t num_tokens() const { size_t v = 0; check(pg_huffman_kv_chunk_info(h_, &v, nullptr, nullptr, nullptr), "CompressedChunk"); return v; }
+    size_t num_heads() const { size_t v = 0; check(pg_huffman_kv_chunk_info(h_, nullptr, &v, nullptr, nullptr), "CompressedChunk"); return v; }
+    size_t head_dim() const { size_t v = 0; check(pg_huffman_kv_chunk_info(h_, nullptr, nullptr, &v, nullptr), "CompressedChunk"); return v; }
+    std::vector<uint8_t> bitstream() const {
+        size_t n = 0;
+        check(pg_huffman_kv_chunk_info(h_, nullptr, nullptr, nullptr, &n), "CompressedChunk");
+        std::vector<uint8_t> out(n);
+        check(pg_huffman_kv_chunk_parts(gpu_->raw(), h_, out.data(), nullptr, nullptr), "CompressedChunk::bitstream");
+        return out;
+    }
+    std::vector<float> scales() const {
+        std::vector<float> out(num_heads());
+        check(pg_huffman_kv_chunk_parts(gpu_->raw(), h_, nullptr, out.data(), nullptr), "CompressedChunk::scales");
+        return out;
+    }
+    std::vector<uint8_t> codebook() const {
+        std::vector<uint8_t> out(256);
+        check(pg_huffman_kv_chunk_parts(gpu_->raw(), h_, nullptr, nullptr, out.data()), "CompressedChunk::codebook");
+        return out;
+    }
+    const pg_huffman_kv_chunk *handle() const { return h_; }
+
+private:
+    const GpuContext *gpu_;
+    pg_huffman_kv_chunk *h_;
+};
+
+// HuffmanKVCache  src/huffman.rs:484-724.
+class HuffmanKVCache {
+public:
+    HuffmanKVCache(const GpuContext &gpu, size_t num_kv_heads, size_t head_dim, size_t compress_threshold, size_t chunk_size)
+        : gpu_(&gpu), heads_(num_kv_heads), head_dim_(head_dim) {
+        check(pg_huffman_kv_cache_create(gpu.raw(), num_kv_heads, head_dim, compress_threshold, chunk_size, &h_), "HuffmanKVCache::new");
+    }
+    ~HuffmanKVCache() { if (h_) pg_huffman_kv_cache_free(gpu_->raw(), h_); }
+    HuffmanKVCache(const HuffmanKVCache &) = delete;
+    HuffmanKVCache &operator=(const HuffmanKVCache &) = delete;
+    void append(const std::vector<float> &new_k, const std::vector<float> &new_v, size_t seq_len) {
+        const size_t n = heads_ * seq_len * head_dim_;
+        if (new_k.size() != n || new_v.size() != n) throw Panic(PG_EINVAL, "HuffmanKVCache::append: new_k / new_v are not [num_kv_heads, seq_len, head_dim]");
+        check(pg_huffman_kv_cache_append(gpu_->raw(), h_, new_k.data(), new_v.data(), seq_len), "HuffmanKVCache::append");
+    }
+    static CompressedChunk compress_chunk(const GpuContext &gpu, const std::vector<float> &data, size_t num_tokens, size_t num_heads,
+                                          size_t head_dim) {
+        if (data.size() != num_heads * num_tokens * head_dim) throw Panic(PG_EINVAL, "compress_chunk: data.len() != total");
+        pg_huffman_kv_chunk *c = nullptr;
+        check(pg_huffman_kv_compress_chunk(gpu.raw(), data.data(), num_tokens, num_heads, head_dim, &c), "HuffmanKVCache::compress_chunk");
+        return CompressedChunk(gpu, c);
+    }
+    static std::vector<float> decompress_chunk(const GpuContext &gpu, const CompressedChunk &chunk) {
+        std::vector<float> out(chunk.num_heads() * chunk.num_tokens() * chunk.head_dim());
+        check(pg_huffman_kv_decompress_chunk(gpu.raw(), chunk.handle(), out.data()), "HuffmanKVCache::decompress_chunk");
+        return out;
+    }
+    size_t len() const { return pg_huffman_kv_cache_len(h_); }
+    size_t compressed_len() const { return pg_huffman_kv_cache_compressed_len(h_); }
+    size_t compress_threshold() const { return pg_huffman_kv_cache_compress_threshold(h_); }
+    size_t num_chunks() const { return pg_huffman_kv_cache_num_chunks(h_); }
+    // (k, v), each [num_kv_heads, len(), head_dim]
+    std::pair<std::vector<float>, std::vector<float>> get_kv() const {
+        const size_t n = heads_ * len() * head_dim_;
+        std::vector<float> k(n), v(n);
+        check(pg_huffman_kv_cache_get_kv(gpu_->raw(), h_, k.data(), v.data()), "HuffmanKVCache::get_kv");
+        return {std::move(k), std::move(v)};
+    }
+    pg_huffman_kv_cache *handle() const { return h_; }
+
+private:
+    const GpuContext *gpu_;
+    size_t heads_, head_dim_;
+    pg_huffman_kv_cache *h_ = nullptr;
+};
+
 }  // namespace huffman
 }  // namespace peregrine
 #endif  // PEREGRINE_HIP_HPP

@@ -221,3 +221,253 @@ ORC_API int orc_huffman_decode(const uint8_t *bl, const uint8_t *bitstream, size
     }
     return 0;
 }
+
+/* ---------------------------------------------------------------------------------------
+ * HuffmanKVCache: int8 + Huffman chunks of older tokens behind an f32 window.  Parity
+ * status: pinned by the reference's own tests restated (src/huffman.rs:850-905,
+ * tests/huffman_parity.rs:133-186: lengths after each append, error <= scale + 1e-5), by
+ * closed forms (an all-zero head has scale 1 and codes of one bit; a constant chunk is
+ * ceil(n / 8) zero bytes and decodes to 127 * (c / 127); the values +-absmax become +-127),
+ * by the half-step error bound |x - x'| <= scale / 2 that only round-to-nearest meets, by a
+ * float32 NumPy recomputation of scales and int8 values that shares no code with this file,
+ * by bitstream == orc_huffman_encode of those values under orc_huffman_table of their
+ * histogram (both pinned above), and for the cache by token order: what get_kv returns is
+ * decompress(compress(.)) of the tokens each chunk took, in arrival order, followed bit for
+ * bit by the tokens still in the window.
+ * ------------------------------------------------------------------------------------- */
+
+/* The table a KV chunk is coded with: HuffmanTable::from_frequencies where that is a prefix code.
+ * Where its depth clamp over-subscribes the code the reference panics inside from_frequencies
+ * (build_decode_lut indexes past its table, src/huffman.rs:205-208), so there is nothing to
+ * restate; the library then repairs the lengths and this is that rule, written independently:
+ * sort the clamped lengths, hand them out shortest to most frequent (ties: lower symbol first);
+ * while the Kraft sum exceeds 1 lengthen by one bit the least frequent symbol of the deepest
+ * level below 12; then shorten, most frequent symbol first, whatever the slack allows.
+ * Returns 1 if the repair ran. */
+ORC_API int orc_huffman_table_that_decodes(const uint64_t *freqs, uint8_t *bl, uint32_t *codes) {
+    orc_huffman_table(freqs, bl, NULL);
+    const long full = 1L << HUF_MAX_BITS;
+    long kraft = 0;
+    int order[HUF_SYMS], len[HUF_SYMS], n = 0;
+    for (int s = 0; s < HUF_SYMS; ++s)
+        if (bl[s]) { kraft += full >> bl[s]; order[n++] = s; }
+    int repaired = 0;
+    if (kraft > full) {
+        repaired = 1;
+        for (int i = 1; i < n; ++i) { /* insertion sort: frequency descending, stable */
+            const int s = order[i];
+            int j = i;
+            while (j > 0 && freqs[order[j - 1]] < freqs[s]) { order[j] = order[j - 1]; --j; }
+            order[j] = s;
+        }
+        for (int i = 0; i < n; ++i) len[i] = bl[order[i]];
+        for (int i = 1; i < n; ++i) { /* lengths ascending */
+            const int v = len[i];
+            int j = i;
+            while (j > 0 && len[j - 1] > v) { len[j] = len[j - 1]; --j; }
+            len[j] = v;
+        }
+        while (kraft > full) {
+            int pick = n - 1;
+            while (len[pick] >= HUF_MAX_BITS) --pick; /* exists: n symbols of 12 bits never exceed 1 */
+            kraft -= full >> (len[pick] + 1);
+            len[pick] += 1;
+        }
+        for (int i = 0; i < n; ++i)
+            while (len[i] > 1 && (full >> len[i]) <= full - kraft) { kraft += full >> len[i]; len[i] -= 1; }
+        for (int i = 0; i < n; ++i) bl[order[i]] = (uint8_t)len[i];
+    }
+    if (codes) orc_huffman_canonical_codes(bl, codes);
+    return repaired;
+}
+
+static inline int8_t hkv_sat_i8(float v) { /* Rust `f32 as i8`: saturating, NaN -> 0 */
+    if (v != v) return 0;
+    if (v <= -128.0f) return (int8_t)-128;
+    if (v >= 127.0f) return (int8_t)127;
+    return (int8_t)v;
+}
+
+/* HuffmanKVCache::compress_chunk                  reference: src/huffman.rs:612-658
+ *   data [num_heads][num_tokens][head_dim]; per head absmax (f32::max drops NaN), scale =
+ *   absmax / 127 or 1, q = (v * (1 / scale)).round().clamp(-127, 127) as i8; one table over all
+ *   heads' values (orc_huffman_table_that_decodes); codebook = the 256 bit lengths.  bitstream may be NULL to ask for the
+ *   size; q_out (optional) receives the int8 values.  Returns the bitstream's bytes. */
+ORC_API size_t orc_huffman_kv_compress_chunk(const float *data, size_t num_tokens, size_t num_heads, size_t head_dim,
+                                             uint8_t *bitstream, float *scales, uint8_t *codebook, int8_t *q_out) {
+    const size_t head_size = num_tokens * head_dim, total = num_heads * head_size;
+    int8_t *q = (int8_t *)malloc(total ? total : 1);
+    for (size_t h = 0; h < num_heads; ++h) {
+        const float *hd = data + h * head_size;
+        float absmax = 0.0f;
+        for (size_t i = 0; i < head_size; ++i) {
+            const float a = fabsf(hd[i]);
+            if (a > absmax) absmax = a; /* a NaN compares false and is skipped, as acc.max(NaN) = acc */
+        }
+        const float scale = absmax == 0.0f ? 1.0f : absmax / 127.0f;
+        scales[h] = scale;
+        const float inv_scale = 1.0f / scale;
+        for (size_t i = 0; i < head_size; ++i) {
+            float r = roundf(hd[i] * inv_scale);
+            if (r == r) r = r < -127.0f ? -127.0f : (r > 127.0f ? 127.0f : r);
+            q[h * head_size + i] = hkv_sat_i8(r);
+        }
+    }
+    uint64_t freqs[HUF_SYMS];
+    uint32_t codes[HUF_SYMS];
+    memset(freqs, 0, sizeof freqs);
+    for (size_t i = 0; i < total; ++i) freqs[(int)q[i] + 128] += 1;
+    orc_huffman_table_that_decodes(freqs, codebook, codes);
+    const size_t bytes = orc_huffman_encode(codebook, codes, q, total, bitstream);
+    if (q_out) memcpy(q_out, q, total);
+    free(q);
+    return bytes;
+}
+
+/* HuffmanKVCache::decompress_chunk                reference: src/huffman.rs:661-680 */
+ORC_API int orc_huffman_kv_decompress_chunk(const uint8_t *bitstream, size_t bytes, const float *scales, const uint8_t *codebook,
+                                            size_t num_tokens, size_t num_heads, size_t head_dim, float *out) {
+    const size_t head_size = num_tokens * head_dim, total = num_heads * head_size;
+    int8_t *q = (int8_t *)malloc(total ? total : 1);
+    const int rc = orc_huffman_decode(codebook, bitstream, bytes, total, q);
+    if (rc == 0)
+        for (size_t h = 0; h < num_heads; ++h)
+            for (size_t i = 0; i < head_size; ++i) out[h * head_size + i] = (float)q[h * head_size + i] * scales[h];
+    free(q);
+    return rc;
+}
+
+typedef struct {
+    uint8_t *bitstream;
+    size_t bytes;
+    float *scales;
+    uint8_t codebook[HUF_SYMS];
+    size_t num_tokens;
+} orc_hkv_chunk;
+
+/* HuffmanKVCache over StandardKVCache             reference: src/huffman.rs:484-497, src/attention.rs:8-15 */
+typedef struct {
+    float *k, *v; /* [heads][capacity][head_dim] */
+    size_t len, capacity, heads, head_dim;
+    orc_hkv_chunk *kc, *vc;
+    size_t nchunks, compressed_len, threshold, chunk_size;
+} orc_hkv;
+
+/* HuffmanKVCache::new                             reference: src/huffman.rs:524-540 */
+ORC_API orc_hkv *orc_huffman_kv_new(size_t heads, size_t head_dim, size_t compress_threshold, size_t chunk_size) {
+    orc_hkv *c = (orc_hkv *)calloc(1, sizeof *c);
+    c->heads = heads;
+    c->head_dim = head_dim;
+    c->threshold = compress_threshold > chunk_size ? compress_threshold : chunk_size;
+    c->chunk_size = chunk_size;
+    return c;
+}
+
+ORC_API void orc_huffman_kv_free(orc_hkv *c) {
+    if (!c) return;
+    for (size_t i = 0; i < c->nchunks; ++i) {
+        free(c->kc[i].bitstream); free(c->kc[i].scales);
+        free(c->vc[i].bitstream); free(c->vc[i].scales);
+    }
+    free(c->kc); free(c->vc); free(c->k); free(c->v); free(c);
+}
+
+/* StandardKVCache::ensure_capacity + append       reference: src/attention.rs:31-83 */
+static void hkv_hot_append(orc_hkv *c, const float *nk, const float *nv, size_t seq_len) {
+    const size_t new_len = c->len + seq_len, hd = c->head_dim;
+    if (new_len > c->capacity) {
+        const size_t grown = (c->capacity > 16 ? c->capacity : 16) * 2, new_cap = new_len > grown ? new_len : grown;
+        const size_t total = c->heads * new_cap * hd;
+        float *k2 = (float *)calloc(total ? total : 1, sizeof(float)), *v2 = (float *)calloc(total ? total : 1, sizeof(float));
+        for (size_t h = 0; h < c->heads && c->len > 0; ++h) {
+            memcpy(k2 + h * new_cap * hd, c->k + h * c->capacity * hd, c->len * hd * sizeof(float));
+            memcpy(v2 + h * new_cap * hd, c->v + h * c->capacity * hd, c->len * hd * sizeof(float));
+        }
+        free(c->k); free(c->v);
+        c->k = k2; c->v = v2; c->capacity = new_cap;
+    }
+    for (size_t h = 0; h < c->heads; ++h) {
+        memcpy(c->k + h * c->capacity * hd + c->len * hd, nk + h * seq_len * hd, seq_len * hd * sizeof(float));
+        memcpy(c->v + h * c->capacity * hd + c->len * hd, nv + h * seq_len * hd, seq_len * hd * sizeof(float));
+    }
+    c->len = new_len;
+}
+
+/* extract_chunk_data + compress_chunk             reference: src/huffman.rs:579-596, 612-658 */
+static void hkv_compress_side(const orc_hkv *c, const float *side, size_t tokens, orc_hkv_chunk *out) {
+    const size_t hd = c->head_dim, n = c->heads * tokens * hd;
+    float *flat = (float *)malloc((n ? n : 1) * sizeof(float));
+    for (size_t h = 0; h < c->heads; ++h) memcpy(flat + h * tokens * hd, side + h * c->capacity * hd, tokens * hd * sizeof(float));
+    out->scales = (float *)malloc((c->heads ? c->heads : 1) * sizeof(float));
+    out->bitstream = (uint8_t *)malloc(2 * n + 16);
+    out->bytes = orc_huffman_kv_compress_chunk(flat, tokens, c->heads, hd, out->bitstream, out->scales, out->codebook, NULL);
+    out->num_tokens = tokens;
+    free(flat);
+}
+
+/* HuffmanKVCache::append                          reference: src/huffman.rs:544-556
+ *   compress_oldest_chunk :559-577, remove_oldest_tokens :599-610 (copy_within = memmove).
+ *   chunk_size 0 never ends once the threshold is met in the reference; here it returns. */
+ORC_API void orc_huffman_kv_append(orc_hkv *c, const float *nk, const float *nv, size_t seq_len) {
+    hkv_hot_append(c, nk, nv, seq_len);
+    while (c->len >= c->threshold) {
+        const size_t tokens = c->chunk_size < c->len ? c->chunk_size : c->len, hd = c->head_dim;
+        if (tokens == 0) return;
+        c->kc = (orc_hkv_chunk *)realloc(c->kc, (c->nchunks + 1) * sizeof *c->kc);
+        c->vc = (orc_hkv_chunk *)realloc(c->vc, (c->nchunks + 1) * sizeof *c->vc);
+        hkv_compress_side(c, c->k, tokens, &c->kc[c->nchunks]);
+        hkv_compress_side(c, c->v, tokens, &c->vc[c->nchunks]);
+        c->nchunks += 1;
+        c->compressed_len += tokens;
+        const size_t new_len = c->len - tokens;
+        for (size_t h = 0; h < c->heads; ++h) {
+            memmove(c->k + h * c->capacity * hd, c->k + h * c->capacity * hd + tokens * hd, new_len * hd * sizeof(float));
+            memmove(c->v + h * c->capacity * hd, c->v + h * c->capacity * hd + tokens * hd, new_len * hd * sizeof(float));
+        }
+        c->len = new_len;
+    }
+}
+
+/* which: 0 len() (:683-685), 1 compressed_len, 2 hot.len, 3 hot capacity, 4 chunks, 5 compress_threshold */
+ORC_API size_t orc_huffman_kv_stat(const orc_hkv *c, int which) {
+    switch (which) {
+    case 0: return c->compressed_len + c->len;
+    case 1: return c->compressed_len;
+    case 2: return c->len;
+    case 3: return c->capacity;
+    case 4: return c->nchunks;
+    default: return c->threshold;
+    }
+}
+
+ORC_API size_t orc_huffman_kv_chunk(const orc_hkv *c, int value_side, size_t index, const uint8_t **bitstream, const float **scales,
+                                    const uint8_t **codebook, size_t *num_tokens) {
+    const orc_hkv_chunk *ch = value_side ? &c->vc[index] : &c->kc[index];
+    *bitstream = ch->bitstream; *scales = ch->scales; *codebook = ch->codebook; *num_tokens = ch->num_tokens;
+    return ch->bytes;
+}
+
+/* HuffmanKVCache::get_kv                          reference: src/huffman.rs:689-724
+ *   k, v [heads][len()][head_dim].  literal_hot_offsets != 0 reads head h of the window at
+ *   h * hot.len * head_dim as the reference does (:707-708); 0 reads it at h * head_stride(),
+ *   where append put it.  The two agree for head 0 and whenever hot.len == capacity. */
+ORC_API void orc_huffman_kv_get_kv(const orc_hkv *c, int literal_hot_offsets, float *k, float *v) {
+    const size_t hd = c->head_dim, total_len = c->compressed_len + c->len;
+    for (int side = 0; side < 2; ++side) {
+        float *dst = side ? v : k;
+        const float *hot = side ? c->v : c->k;
+        const orc_hkv_chunk *chunks = side ? c->vc : c->kc;
+        for (size_t i = 0, off = 0; i < c->nchunks; ++i) {
+            const size_t t = chunks[i].num_tokens, n = c->heads * t * hd;
+            float *flat = (float *)malloc((n ? n : 1) * sizeof(float));
+            orc_huffman_kv_decompress_chunk(chunks[i].bitstream, chunks[i].bytes, chunks[i].scales, chunks[i].codebook, t, c->heads, hd, flat);
+            for (size_t h = 0; h < c->heads; ++h) memcpy(dst + (h * total_len + off) * hd, flat + h * t * hd, t * hd * sizeof(float));
+            free(flat);
+            off += t;
+        }
+        for (size_t h = 0; h < c->heads && c->len > 0; ++h) {
+            const size_t base = literal_hot_offsets ? h * c->len * hd : h * c->capacity * hd;
+            memcpy(dst + (h * total_len + c->compressed_len) * hd, hot + base, c->len * hd * sizeof(float));
+        }
+    }
+}

@@ -126,6 +126,26 @@ SIGNATURES = {
     "pg_huffman_tensor_decode_to_quantized": [_vp, _vp, _vp, _vp, _vp],
     "pg_huffman_tensor_to_gpu": [_vp, _vp, _pp],
     "pg_matmul_huffman": [_vp, _vp, _sz, _sz, _vp, _vp],
+    "pg_huffman_kv_compress_chunk": [_vp, _vp, _sz, _sz, _sz, _pp],
+    "pg_huffman_kv_compress_chunk_dev": [_vp, _vp, _sz, _sz, _sz, _sz, _pp],
+    "pg_huffman_kv_chunk_from_parts": [_vp, _vp, _sz, _vp, _vp, _sz, _sz, _sz, _pp],
+    "pg_huffman_kv_chunk_free": [_vp, _vp],
+    "pg_huffman_kv_chunk_info": [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)],
+    "pg_huffman_kv_chunk_parts": [_vp, _vp, _vp, _vp, _vp],
+    "pg_huffman_kv_decompress_chunk": [_vp, _vp, _vp],
+    "pg_huffman_kv_decompress_chunk_dev": [_vp, _vp, _vp, _sz],
+    "pg_huffman_kv_cache_create": [_vp, _sz, _sz, _sz, _sz, _pp],
+    "pg_huffman_kv_cache_free": [_vp, _vp],
+    "pg_huffman_kv_cache_append": [_vp, _vp, _vp, _vp, _sz],
+    "pg_huffman_kv_cache_append_dev": [_vp, _vp, _vp, _vp, _sz],
+    "pg_huffman_kv_cache_len": [_vp],
+    "pg_huffman_kv_cache_compressed_len": [_vp],
+    "pg_huffman_kv_cache_compress_threshold": [_vp],
+    "pg_huffman_kv_cache_num_chunks": [_vp],
+    "pg_huffman_kv_cache_hot": [_vp, _pp],
+    "pg_huffman_kv_cache_chunk": [_vp, _int, _sz, _pp],
+    "pg_huffman_kv_cache_get_kv": [_vp, _vp, _vp, _vp],
+    "pg_huffman_kv_cache_get_kv_dev": [_vp, _vp, _vp, _vp],
     "pg_mxfp4_matmul": [_vp, _vp, _vp, _vp, _sz, _sz, _vp],
     "pg_mxfp4_upload": [_vp, _vp, _vp, _sz, _sz, _pp],
     "pg_mxfp4_expert_create": [_vp, _sz, _sz, C.c_float, C.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _pp],
@@ -163,6 +183,12 @@ _OTHER_RESTYPE = {
     "pg_gguf_file_close": None,
     "pg_rope_free": None,
     "pg_huffman_tensor_free": None,
+    "pg_huffman_kv_chunk_free": None,
+    "pg_huffman_kv_cache_free": None,
+    "pg_huffman_kv_cache_len": _sz,
+    "pg_huffman_kv_cache_compressed_len": _sz,
+    "pg_huffman_kv_cache_compress_threshold": _sz,
+    "pg_huffman_kv_cache_num_chunks": _sz,
     "pg_mxfp4_expert_free": None,
     "pg_kv_cache_free": None,
     "pg_llama_block_free": None,

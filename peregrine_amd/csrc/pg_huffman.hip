@@ -96,6 +96,44 @@ void table_from_frequencies(const uint64_t *freqs, uint8_t *bl) {
     for (size_t i = 0; i < n; ++i) bl[symbols[i]] = (uint8_t)std::min<unsigned>(depth[i], MAX_LUT_BITS);
 }
 
+// A table for data that must decode again.  The reference's, where that is a prefix code.  Where
+// its depth clamp over-subscribes the code (it then panics while filling its decode table,
+// src/huffman.rs:189-213, so there is no reference result to match) the lengths are repaired:
+// the deepest leaf above the limit's level is pushed down one level until the Kraft sum fits,
+// any slack left is given to the most frequent symbols, and the resulting lengths are handed
+// out again shortest to most frequent.  Returns whether the repair was needed.
+bool table_that_decodes(const uint64_t *freqs, uint8_t *bl) {
+    table_from_frequencies(freqs, bl);
+    const long full = 1L << MAX_LUT_BITS;
+    long kraft = 0;
+    for (int s = 0; s < NUM_SYMBOLS; ++s)
+        if (bl[s]) kraft += full >> bl[s];
+    if (kraft <= full) return false;
+    std::vector<int> by_freq;  // most frequent first, ties by symbol
+    for (int s = 0; s < NUM_SYMBOLS; ++s)
+        if (bl[s]) by_freq.push_back(s);
+    std::stable_sort(by_freq.begin(), by_freq.end(), [&](int a, int b) { return freqs[a] > freqs[b]; });
+    std::vector<int> len;
+    for (int s : by_freq) len.push_back(bl[s]);
+    std::sort(len.begin(), len.end());  // shortest first: position i belongs to by_freq[i]
+    while (kraft > full) {              // lengthen the last (least frequent) leaf of the deepest level below the limit
+        int pick = -1;
+        for (int i = (int)len.size() - 1; i >= 0; --i)
+            if (len[i] < MAX_LUT_BITS && (pick < 0 || len[i] > len[pick])) pick = i;
+        kraft -= full >> (len[pick] + 1);
+        len[pick] += 1;
+        std::sort(len.begin(), len.end());
+    }
+    for (size_t i = 0; i < len.size(); ++i)  // spend the slack on the most frequent symbols
+        while (len[i] > 1 && (full >> len[i]) <= full - kraft) {
+            kraft += full >> len[i];
+            len[i] -= 1;
+        }
+    std::sort(len.begin(), len.end());
+    for (size_t i = 0; i < len.size(); ++i) bl[by_freq[i]] = (uint8_t)len[i];
+    return true;
+}
+
 // src/huffman.rs:189-213 with the packing of to_gpu_lut (src/huffman.rs:727-736):
 // entry = bit_length << 8 | (symbol + 128).  Codes that do not fit the table (a clamped,
 // over-subscribed length set) are reported instead of indexing past it.
@@ -309,36 +347,33 @@ __global__ __launch_bounds__(WG) void huff_write_kernel(const uint8_t *__restric
     }
 }
 
-// Decode `nstreams` streams (host bytes) into out_dev.  streams[i] has bytes[i] bytes and
-// holds symbols[i] symbols, written back to back.
-pg_status decode_streams(pg_ctx *ctx, const uint8_t *bit_lengths, const uint8_t *const *streams, const size_t *bytes,
-                         const size_t *symbols, size_t nstreams, int8_t *out_dev) {
+// Adds one stream of `bytes` bytes at d_bytes + byte_off holding `symbols` symbols, decoded to out + out_off.
+pg_status add_stream(std::vector<stream_desc> &desc, size_t byte_off, size_t bytes, size_t symbols, size_t out_off, size_t &sub,
+                     size_t &wg) {
+    stream_desc d;
+    d.byte_off = byte_off;
+    d.nbits = (unsigned long long)bytes * 8;
+    d.nsym = symbols;
+    d.out_off = out_off;
+    const size_t nsub = (d.nbits + SUBSEQ_BITS - 1) / SUBSEQ_BITS, nwg = (nsub + WG - 1) / WG;
+    PG_CHECK_ARG(sub + nsub < (1ull << 32) && wg + nwg < (1ull << 31), "huffman decode: stream too long");
+    d.sub_base = (unsigned)sub; d.nsub = (unsigned)nsub; d.wg_base = (unsigned)wg; d.nwg = (unsigned)nwg;
+    desc.push_back(d);
+    sub += nsub;
+    wg += nwg;
+    return PG_OK;
+}
+
+// Decode the streams `desc` describes (bytes already in device memory at d_bytes) into out_dev.
+pg_status decode_device_streams(pg_ctx *ctx, const uint8_t *bit_lengths, const std::vector<stream_desc> &desc,
+                                const uint8_t *d_bytes, size_t sub, size_t wg, int8_t *out_dev) {
+    if (desc.empty()) return PG_OK;
     uint32_t codes[NUM_SYMBOLS];
     std::vector<uint16_t> lut(LUT_SIZE);
     canonical_codes(bit_lengths, codes);
     PG_TRY(build_lut(bit_lengths, codes, lut.data()));
-    std::vector<stream_desc> desc;
-    size_t byte_off = 0, out_off = 0, sub = 0, wg = 0;
-    for (size_t i = 0; i < nstreams; ++i) {
-        if (symbols[i] == 0) continue;
-        PG_CHECK_ARG(bytes[i] > 0 && streams[i], "huffman decode: stream %zu holds %zu symbols in no bytes", i, symbols[i]);
-        stream_desc d;
-        d.byte_off = byte_off;
-        d.nbits = (unsigned long long)bytes[i] * 8;
-        d.nsym = symbols[i];
-        d.out_off = out_off;
-        const size_t nsub = (d.nbits + SUBSEQ_BITS - 1) / SUBSEQ_BITS, nwg = (nsub + WG - 1) / WG;
-        PG_CHECK_ARG(sub + nsub < (1ull << 32) && wg + nwg < (1ull << 31), "huffman decode: stream too long");
-        d.sub_base = (unsigned)sub; d.nsub = (unsigned)nsub; d.wg_base = (unsigned)wg; d.nwg = (unsigned)nwg;
-        desc.push_back(d);
-        byte_off += pg_round_up(bytes[i], 16);
-        out_off += symbols[i];
-        sub += nsub;
-        wg += nwg;
-    }
-    if (desc.empty()) return PG_OK;
-    // one allocation: stream bytes | descriptors | lut | start | end | count | excl | wg totals | flags
-    const size_t o_desc = pg_round_up(byte_off, 256), o_lut = o_desc + pg_round_up(desc.size() * sizeof(stream_desc), 256);
+    // one allocation: descriptors | lut | start | end | count | excl | wg totals | flags
+    const size_t o_lut = pg_round_up(desc.size() * sizeof(stream_desc), 256);
     const size_t o_start = o_lut + LUT_SIZE * sizeof(uint16_t), o_end = o_start + pg_round_up(sub * 8, 256);
     const size_t o_count = o_end + pg_round_up(sub * 8, 256), o_excl = o_count + pg_round_up(sub * 4, 256);
     const size_t o_wg = o_excl + pg_round_up(sub * 4, 256), o_flag = o_wg + pg_round_up(wg * 8, 256);
@@ -346,15 +381,9 @@ pg_status decode_streams(pg_ctx *ctx, const uint8_t *bit_lengths, const uint8_t 
     PG_TRY(buf.alloc(o_flag + 256));
     char *base = buf.as<char>();
     PG_HIP(hipMemsetAsync(base + o_flag, 0, 256, ctx->stream));
-    for (size_t i = 0, j = 0; i < nstreams; ++i) {
-        if (symbols[i] == 0) continue;
-        PG_HIP(hipMemcpyAsync(base + desc[j].byte_off, streams[i], bytes[i], hipMemcpyHostToDevice, ctx->stream));
-        ++j;
-    }
-    PG_HIP(hipMemcpyAsync(base + o_desc, desc.data(), desc.size() * sizeof(stream_desc), hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(base, desc.data(), desc.size() * sizeof(stream_desc), hipMemcpyHostToDevice, ctx->stream));
     PG_HIP(hipMemcpyAsync(base + o_lut, lut.data(), LUT_SIZE * sizeof(uint16_t), hipMemcpyHostToDevice, ctx->stream));
-    const uint8_t *d_bytes = reinterpret_cast<const uint8_t *>(base);
-    const stream_desc *d_desc = reinterpret_cast<const stream_desc *>(base + o_desc);
+    const stream_desc *d_desc = reinterpret_cast<const stream_desc *>(base);
     const uint16_t *d_lut = reinterpret_cast<const uint16_t *>(base + o_lut);
     auto *d_start = reinterpret_cast<unsigned long long *>(base + o_start);
     auto *d_end = reinterpret_cast<unsigned long long *>(base + o_end);
@@ -389,6 +418,30 @@ pg_status decode_streams(pg_ctx *ctx, const uint8_t *bit_lengths, const uint8_t 
     return PG_OK;
 }
 
+// Decode `nstreams` streams (host bytes) into out_dev.  streams[i] has bytes[i] bytes and
+// holds symbols[i] symbols, written back to back.
+pg_status decode_streams(pg_ctx *ctx, const uint8_t *bit_lengths, const uint8_t *const *streams, const size_t *bytes,
+                         const size_t *symbols, size_t nstreams, int8_t *out_dev) {
+    std::vector<stream_desc> desc;
+    size_t byte_off = 0, out_off = 0, sub = 0, wg = 0;
+    for (size_t i = 0; i < nstreams; ++i) {
+        if (symbols[i] == 0) continue;
+        PG_CHECK_ARG(bytes[i] > 0 && streams[i], "huffman decode: stream %zu holds %zu symbols in no bytes", i, symbols[i]);
+        PG_TRY(add_stream(desc, byte_off, bytes[i], symbols[i], out_off, sub, wg));
+        byte_off += pg_round_up(bytes[i], 16);
+        out_off += symbols[i];
+    }
+    if (desc.empty()) return PG_OK;
+    pg_tmp buf;
+    PG_TRY(buf.alloc(byte_off));
+    for (size_t i = 0, j = 0; i < nstreams; ++i) {
+        if (symbols[i] == 0) continue;
+        PG_HIP(hipMemcpyAsync(buf.as<char>() + desc[j].byte_off, streams[i], bytes[i], hipMemcpyHostToDevice, ctx->stream));
+        ++j;
+    }
+    return decode_device_streams(ctx, bit_lengths, desc, buf.as<uint8_t>(), sub, wg, out_dev);
+}
+
 }  // namespace
 
 // HuffmanTensor  src/huffman.rs:311-325 (host-resident, as in the reference).
@@ -399,6 +452,23 @@ struct pg_huffman_tensor {
     std::vector<float> scales;
     size_t rows, cols;
 };
+
+// For the other Huffman translation unit (the KV cache): the host table and one device-resident stream.
+bool pg_huffman_host_table(const uint64_t *freqs, uint8_t *bit_lengths, uint32_t *codes) {
+    const bool repaired = table_that_decodes(freqs, bit_lengths);
+    canonical_codes(bit_lengths, codes);
+    return repaired;
+}
+
+pg_status pg_huffman_decode_device_stream(pg_ctx *ctx, const uint8_t *bit_lengths, const uint8_t *bytes_dev, size_t bytes,
+                                          size_t num_symbols, int8_t *out_dev) {
+    if (num_symbols == 0) return PG_OK;
+    PG_CHECK_ARG(bytes > 0 && bytes_dev, "huffman decode: %zu symbols in no bytes", num_symbols);
+    std::vector<stream_desc> desc;
+    size_t sub = 0, wg = 0;
+    PG_TRY(add_stream(desc, 0, bytes, num_symbols, 0, sub, wg));
+    return decode_device_streams(ctx, bit_lengths, desc, bytes_dev, sub, wg, out_dev);
+}
 
 pg_status pg_qtensor_from_device_q(pg_ctx *ctx, const int8_t *q_dev, const float *scales_host, size_t rows, size_t cols,
                                    pg_qtensor **out);

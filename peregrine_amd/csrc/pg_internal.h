@@ -88,6 +88,11 @@ struct pg_gguf_tensor {
 // (an outlier in the block then costs every other element ~2^-16 of the outlier).  Products
 // whose K spans fewer blocks than this run the streaming kernel (18 / 22-bit activations),
 // one item per activation row.
+// attention::StandardKVCache (src/attention.rs:8-15) on the device: k, v = [num_kv_heads][capacity][head_dim] f32.
+struct pg_kv_cache {
+    float *k, *v;
+    size_t len, capacity, num_kv_heads, head_dim;
+};
 constexpr size_t PG_MM_MIN_BLOCKS = 5;
 constexpr int PG_GEMM_MAX_GROUP = 4;  // weights one W8A8 launch can carry (fused q|k|v, gate|up)
 constexpr size_t PG_KPAD = 128;  // device K stride is a multiple of this

@@ -25,10 +25,6 @@ struct pg_rope {
     size_t head_dim, max_seq_len;
 };
 
-struct pg_kv_cache {
-    float *k, *v;
-    size_t len, capacity, num_kv_heads, head_dim;
-};
 
 struct pg_llama_block {
     size_t d, nqh, nkvh, hd, ffn;

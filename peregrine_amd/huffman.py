@@ -155,3 +155,137 @@ def matmul_huffman(a_data, m, k, ht, ctx=None):
     out = np.empty(m * ht.cols, np.float32)
     _ffi.check(_ffi.lib.pg_matmul_huffman(ctx.handle, _ptr(a), m, k, ht._h, _ptr(out)))
     return out
+
+
+class CompressedChunk:
+    """`CompressedChunk` (src/huffman.rs:500-513).  The bitstream lives in device memory; the
+    `bitstream`, `scales` and `codebook` properties copy it out."""
+
+    def __init__(self, handle, ctx, owned=True):
+        self._h, self.ctx, self._owned = handle, ctx, owned
+        t, h, d, b = C.c_size_t(), C.c_size_t(), C.c_size_t(), C.c_size_t()
+        _ffi.check(_ffi.lib.pg_huffman_kv_chunk_info(handle, C.byref(t), C.byref(h), C.byref(d), C.byref(b)))
+        self.num_tokens, self.num_heads, self.head_dim, self._bytes = t.value, h.value, d.value, b.value
+
+    @classmethod
+    def from_parts(cls, bitstream, scales, codebook, num_tokens, num_heads, head_dim, ctx=None):
+        ctx = ctx or default_context()
+        b = np.frombuffer(bytes(bitstream), np.uint8)
+        s = np.ascontiguousarray(scales, np.float32).reshape(-1)
+        cb = np.frombuffer(bytes(codebook), np.uint8)
+        if s.size != num_heads or cb.size < NUM_SYMBOLS:
+            raise ValueError("CompressedChunk.from_parts: field lengths")
+        h = C.c_void_p()
+        _ffi.check(_ffi.lib.pg_huffman_kv_chunk_from_parts(ctx.handle, _ptr(b) if b.size else None, b.size, _ptr(s) if s.size else None,
+                                                           _ptr(cb), num_tokens, num_heads, head_dim, C.byref(h)))
+        return cls(h, ctx)
+
+    def _parts(self):
+        b, s, cb = np.zeros(self._bytes, np.uint8), np.zeros(self.num_heads, np.float32), np.zeros(NUM_SYMBOLS, np.uint8)
+        _ffi.check(_ffi.lib.pg_huffman_kv_chunk_parts(self.ctx.handle, self._h, _ptr(b) if b.size else None,
+                                                      _ptr(s) if s.size else None, _ptr(cb)))
+        return b.tobytes(), s, cb.tobytes()
+
+    bitstream = property(lambda self: self._parts()[0])
+    scales = property(lambda self: self._parts()[1])
+    codebook = property(lambda self: self._parts()[2])
+
+    def free(self):
+        if self._h and self._owned:
+            _ffi.lib.pg_huffman_kv_chunk_free(self.ctx.handle, self._h)
+        self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class HuffmanKVCache:
+    """`HuffmanKVCache` (src/huffman.rs:484-724): a window of recent tokens as f32 in a device
+    StandardKVCache, older tokens as int8 + Huffman chunks in device memory."""
+
+    def __init__(self, num_kv_heads, head_dim, compress_threshold, chunk_size, ctx=None):
+        self.ctx = ctx or default_context()
+        self.num_kv_heads, self.head_dim, self.chunk_size = int(num_kv_heads), int(head_dim), int(chunk_size)
+        self._h = C.c_void_p()
+        _ffi.check(_ffi.lib.pg_huffman_kv_cache_create(self.ctx.handle, self.num_kv_heads, self.head_dim, int(compress_threshold),
+                                                       self.chunk_size, C.byref(self._h)))
+
+    new = classmethod(lambda cls, *a, **k: cls(*a, **k))
+
+    def append(self, new_k, new_v, seq_len):
+        """src/huffman.rs:544-556."""
+        k = np.ascontiguousarray(new_k, np.float32).reshape(-1)
+        v = np.ascontiguousarray(new_v, np.float32).reshape(-1)
+        n = self.num_kv_heads * int(seq_len) * self.head_dim
+        if k.size != n or v.size != n:
+            raise ValueError("HuffmanKVCache.append: new_k / new_v are not [num_kv_heads, seq_len, head_dim]")
+        _ffi.check(_ffi.lib.pg_huffman_kv_cache_append(self.ctx.handle, self._h, _ptr(k) if n else None, _ptr(v) if n else None, int(seq_len)))
+
+    @staticmethod
+    def compress_chunk(data, num_tokens, num_heads, head_dim, ctx=None):
+        """src/huffman.rs:612-658."""
+        ctx = ctx or default_context()
+        d = np.ascontiguousarray(data, np.float32).reshape(-1)
+        if d.size != num_heads * num_tokens * head_dim:  # assert_eq!(data.len(), total)
+            raise ValueError("compress_chunk: data is not [num_heads, num_tokens, head_dim]")
+        h = C.c_void_p()
+        _ffi.check(_ffi.lib.pg_huffman_kv_compress_chunk(ctx.handle, _ptr(d) if d.size else None, num_tokens, num_heads, head_dim, C.byref(h)))
+        return CompressedChunk(h, ctx)
+
+    @staticmethod
+    def decompress_chunk(chunk):
+        """src/huffman.rs:661-680."""
+        out = np.zeros(chunk.num_heads * chunk.num_tokens * chunk.head_dim, np.float32)
+        _ffi.check(_ffi.lib.pg_huffman_kv_decompress_chunk(chunk.ctx.handle, chunk._h, _ptr(out) if out.size else None))
+        return out
+
+    def len(self):
+        return int(_ffi.lib.pg_huffman_kv_cache_len(self._h))  # src/huffman.rs:683-685
+
+    __len__ = len
+
+    @property
+    def compressed_len(self):
+        return int(_ffi.lib.pg_huffman_kv_cache_compressed_len(self._h))
+
+    @property
+    def compress_threshold(self):
+        return int(_ffi.lib.pg_huffman_kv_cache_compress_threshold(self._h))
+
+    @property
+    def hot_len(self):
+        h = C.c_void_p()
+        _ffi.check(_ffi.lib.pg_huffman_kv_cache_hot(self._h, C.byref(h)))
+        return int(_ffi.lib.pg_kv_cache_len(h))
+
+    def _chunks(self, value_side):
+        out = []
+        for i in range(int(_ffi.lib.pg_huffman_kv_cache_num_chunks(self._h))):
+            h = C.c_void_p()
+            _ffi.check(_ffi.lib.pg_huffman_kv_cache_chunk(self._h, value_side, i, C.byref(h)))
+            out.append(CompressedChunk(h, self.ctx, owned=False))
+        return out
+
+    k_chunks = property(lambda self: self._chunks(0))
+    v_chunks = property(lambda self: self._chunks(1))
+
+    def get_kv(self):
+        """src/huffman.rs:689-724: (k, v), each [num_kv_heads * len() * head_dim]."""
+        n = self.num_kv_heads * self.len() * self.head_dim
+        k, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+        _ffi.check(_ffi.lib.pg_huffman_kv_cache_get_kv(self.ctx.handle, self._h, _ptr(k) if n else None, _ptr(v) if n else None))
+        return k, v
+
+    def free(self):
+        if self._h:
+            _ffi.lib.pg_huffman_kv_cache_free(self.ctx.handle, self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass

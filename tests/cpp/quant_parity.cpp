@@ -25,6 +25,13 @@ int orc_llama_block_forward(const float *, size_t, size_t, size_t, size_t, size_
                             const uint8_t *, const uint8_t *, const uint8_t *, const uint8_t *, const uint8_t *,
                             const uint8_t *, const float *, const float *, float, const float *, const float *, float *,
                             float *, size_t, size_t, float *);
+size_t orc_huffman_kv_compress_chunk(const float *, size_t, size_t, size_t, uint8_t *, float *, uint8_t *, int8_t *);
+int orc_huffman_kv_decompress_chunk(const uint8_t *, size_t, const float *, const uint8_t *, size_t, size_t, size_t, float *);
+void *orc_huffman_kv_new(size_t, size_t, size_t, size_t);
+void orc_huffman_kv_free(void *);
+void orc_huffman_kv_append(void *, const float *, const float *, size_t);
+size_t orc_huffman_kv_stat(const void *, int);
+void orc_huffman_kv_get_kv(const void *, int, float *, float *);
 }
 
 using namespace peregrine;
@@ -297,6 +304,61 @@ static void test_huffman_matmul(const GpuContext &gpu) {
     EXPECT(table.decode(gpu, enc, 512) == same, "one-symbol round trip");
 }
 
+// src/huffman.rs:850-905 and tests/huffman_parity.rs:133-186: the compressed KV cache, checked bit
+// for bit against the CPU restatement
+static void test_huffman_kv_cache(const GpuContext &gpu) {
+    std::printf("test_huffman_kv_cache\n");
+    auto lcg = [](uint32_t &st) { st = st * 1103515245u + 12345u; return (float)st / 4294967295.0f * 2.0f - 1.0f; };
+    {
+        const size_t heads = 4, hd = 16, tokens = 32, n = heads * tokens * hd;
+        uint32_t st = 99;
+        std::vector<float> data(n);
+        for (auto &v : data) v = lcg(st);
+        auto chunk = huffman::HuffmanKVCache::compress_chunk(gpu, data, tokens, heads, hd);
+        std::vector<uint8_t> bits(2 * n + 16), codebook(256);
+        std::vector<float> scales(heads), ref(n);
+        bits.resize(orc_huffman_kv_compress_chunk(data.data(), tokens, heads, hd, bits.data(), scales.data(), codebook.data(), nullptr));
+        EXPECT(chunk.bitstream() == bits && chunk.codebook() == codebook && same_bits(chunk.scales(), scales), "compress_chunk differs");
+        auto rec = huffman::HuffmanKVCache::decompress_chunk(gpu, chunk);
+        orc_huffman_kv_decompress_chunk(bits.data(), bits.size(), scales.data(), codebook.data(), tokens, heads, hd, ref.data());
+        EXPECT(same_bits(rec, ref), "decompress_chunk differs");
+        for (size_t h = 0; h < heads; ++h)
+            for (size_t i = 0; i < tokens * hd; ++i)
+                EXPECT(std::fabs(data[h * tokens * hd + i] - rec[h * tokens * hd + i]) <= scales[h] + 1e-5f, "head %zu idx %zu", h, i);
+    }
+    {
+        huffman::HuffmanKVCache cache(gpu, 2, 4, 8, 4);
+        cache.append(std::vector<float>(32, 1.0f), std::vector<float>(32, 2.0f), 4);
+        EXPECT(cache.len() == 4 && cache.compressed_len() == 0, "after 4 tokens");
+        cache.append(std::vector<float>(32, 3.0f), std::vector<float>(32, 4.0f), 4);
+        EXPECT(cache.len() == 8 && cache.compressed_len() == 4, "after 8 tokens");
+        auto kv = cache.get_kv();
+        EXPECT(kv.first.size() == 2 * 8 * 4 && kv.second.size() == 2 * 8 * 4, "get_kv sizes");
+    }
+    {
+        const size_t heads = 2, hd = 8;
+        huffman::HuffmanKVCache cache(gpu, heads, hd, 16, 8);
+        void *orc = orc_huffman_kv_new(heads, hd, 16, 8);
+        for (uint32_t batch = 0; batch < 4; ++batch) {
+            uint32_t sk = 100 + batch, sv = 200 + batch;
+            std::vector<float> k(heads * 8 * hd), v(heads * 8 * hd);
+            for (auto &x : k) x = lcg(sk);
+            for (auto &x : v) x = lcg(sv);
+            cache.append(k, v, 8);
+            orc_huffman_kv_append(orc, k.data(), v.data(), 8);
+        }
+        EXPECT(cache.len() == 32 && cache.compressed_len() > 0 && cache.compressed_len() == orc_huffman_kv_stat(orc, 1), "lengths");
+        auto kv = cache.get_kv();
+        std::vector<float> rk(heads * 32 * hd), rv(heads * 32 * hd);
+        orc_huffman_kv_get_kv(orc, 0, rk.data(), rv.data());
+        EXPECT(same_bits(kv.first, rk) && same_bits(kv.second, rv), "get_kv differs");
+        orc_huffman_kv_free(orc);
+    }
+    bool threw = false;
+    try { huffman::HuffmanKVCache::compress_chunk(gpu, std::vector<float>(5), 1, 2, 3); } catch (const Panic &) { threw = true; }
+    EXPECT(threw, "data.len() != total must panic (src/huffman.rs:619)");
+}
+
 int main() {
     try {
         GpuContext gpu(0);
@@ -311,6 +373,7 @@ int main() {
         test_gqa_attention(gpu);
         test_llama_block(gpu);
         test_huffman_matmul(gpu);
+        test_huffman_kv_cache(gpu);
     } catch (const std::exception &e) {
         std::printf("FAIL: uncaught %s\n", e.what());
         return 2;

@@ -357,3 +357,89 @@ def huffman_decode(bl, stream, num_symbols):
     rc = lib.orc_huffman_decode(_p(bl), _p(b), _sz(b.size), _sz(num_symbols), _p(out))
     assert rc == 0, "a code does not fit the 12-bit table"
     return out
+
+
+lib.orc_huffman_kv_compress_chunk.restype = C.c_size_t
+lib.orc_huffman_kv_new.restype = _vp
+lib.orc_huffman_kv_new.argtypes = [_sz, _sz, _sz, _sz]
+lib.orc_huffman_kv_free.restype = None
+lib.orc_huffman_kv_free.argtypes = [_vp]
+lib.orc_huffman_kv_append.restype = None
+lib.orc_huffman_kv_append.argtypes = [_vp, _vp, _vp, _sz]
+lib.orc_huffman_kv_stat.restype = C.c_size_t
+lib.orc_huffman_kv_stat.argtypes = [_vp, C.c_int]
+lib.orc_huffman_kv_chunk.restype = C.c_size_t
+lib.orc_huffman_kv_chunk.argtypes = [_vp, C.c_int, _sz, _vp, _vp, _vp, _vp]
+lib.orc_huffman_kv_get_kv.restype = None
+lib.orc_huffman_kv_get_kv.argtypes = [_vp, C.c_int, _vp, _vp]
+
+
+def huffman_kv_compress_chunk(data, num_tokens, num_heads, head_dim):
+    """-> (bitstream bytes, scales [heads], codebook [256], q [heads * tokens * head_dim])."""
+    d = _f32(data).reshape(-1)
+    n = num_tokens * num_heads * head_dim
+    assert d.size == n
+    bits = np.zeros(2 * n + 16, np.uint8)
+    scales, codebook, q = np.zeros(num_heads, np.float32), np.zeros(256, np.uint8), np.zeros(n, np.int8)
+    nb = lib.orc_huffman_kv_compress_chunk(_p(d), _sz(num_tokens), _sz(num_heads), _sz(head_dim), _p(bits), _p(scales), _p(codebook), _p(q))
+    return bits[:nb].tobytes(), scales, codebook, q
+
+
+def huffman_kv_decompress_chunk(bitstream, scales, codebook, num_tokens, num_heads, head_dim):
+    b = np.frombuffer(bytes(bitstream), np.uint8)
+    s, cb = _f32(scales), np.ascontiguousarray(codebook, np.uint8)
+    out = np.zeros(num_tokens * num_heads * head_dim, np.float32)
+    rc = lib.orc_huffman_kv_decompress_chunk(_p(b), _sz(b.size), _p(s), _p(cb), _sz(num_tokens), _sz(num_heads), _sz(head_dim), _p(out))
+    assert rc == 0, "a code does not fit the 12-bit table"
+    return out
+
+
+class HuffmanKVCache:
+    """The oracle's HuffmanKVCache (state lives in the C library)."""
+
+    def __init__(self, num_kv_heads, head_dim, compress_threshold, chunk_size):
+        self.heads, self.head_dim = num_kv_heads, head_dim
+        self._h = lib.orc_huffman_kv_new(num_kv_heads, head_dim, compress_threshold, chunk_size)
+
+    def append(self, k, v, seq_len):
+        k, v = _f32(k).reshape(-1), _f32(v).reshape(-1)
+        assert k.size == v.size == self.heads * seq_len * self.head_dim
+        lib.orc_huffman_kv_append(self._h, _p(k), _p(v), seq_len)
+
+    def _stat(self, which):
+        return int(lib.orc_huffman_kv_stat(self._h, which))
+
+    len = property(lambda self: self._stat(0))
+    compressed_len = property(lambda self: self._stat(1))
+    hot_len = property(lambda self: self._stat(2))
+    hot_capacity = property(lambda self: self._stat(3))
+    num_chunks = property(lambda self: self._stat(4))
+    compress_threshold = property(lambda self: self._stat(5))
+
+    def chunk(self, value_side, index):
+        """-> (bitstream bytes, scales, codebook, num_tokens)"""
+        b, s, cb, t = _vp(), _vp(), _vp(), _sz()
+        nb = lib.orc_huffman_kv_chunk(self._h, int(value_side), index, C.byref(b), C.byref(s), C.byref(cb), C.byref(t))
+        scales = np.ctypeslib.as_array(C.cast(s, C.POINTER(C.c_float)), (self.heads,)).copy()
+        codebook = np.ctypeslib.as_array(C.cast(cb, C.POINTER(C.c_uint8)), (256,)).copy()
+        return C.string_at(b, nb), scales, codebook, int(t.value)
+
+    def get_kv(self, literal_hot_offsets=False):
+        n = self.heads * self.len * self.head_dim
+        k, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+        lib.orc_huffman_kv_get_kv(self._h, int(bool(literal_hot_offsets)), _p(k), _p(v))
+        return k, v
+
+    def __del__(self):
+        try:
+            lib.orc_huffman_kv_free(self._h)
+        except Exception:
+            pass
+
+
+def huffman_table_that_decodes(freqs):
+    """(bit_lengths, codes, repaired): the reference's table unless its depth clamp over-subscribes the code."""
+    f = np.ascontiguousarray(freqs, np.uint64)
+    bl, codes = np.zeros(256, np.uint8), np.zeros(256, np.uint32)
+    repaired = lib.orc_huffman_table_that_decodes(_p(f), _p(bl), _p(codes))
+    return bl, codes, bool(repaired)

@@ -204,3 +204,174 @@ def test_huffman_encode_hand_packed_and_reference_round_trips(orc):
     bl, _ = orc.huffman_table(np.bincount(same.astype(np.int16) + 128, minlength=256))
     enc = orc.huffman_encode(bl, same)
     assert len(enc) <= 65 and (orc.huffman_decode(bl, enc, 512) == same).all()
+
+
+# ---- HuffmanKVCache ---------------------------------------------------------------------
+
+def parity_random_data(n, seed):
+    """random_data of tests/huffman_parity.rs:7-16: (state as f32 / u32::MAX as f32) * 2 - 1."""
+    out, state = np.empty(n, np.float32), seed
+    for i in range(n):
+        state = (state * 1103515245 + 12345) & 0xFFFFFFFF
+        out[i] = np.float32(state) / np.float32(4294967295) * np.float32(2.0) - np.float32(1.0)
+    return out
+
+
+def numpy_chunk_quant(data, num_tokens, num_heads, head_dim):
+    """Scales and int8 values of a chunk in float32 NumPy: absmax / 127 (or 1), round half away
+    from zero of v * (1 / scale), clamped to +-127."""
+    d = np.asarray(data, np.float32).reshape(num_heads, num_tokens * head_dim)
+    absmax = np.abs(d).max(axis=1) if d.shape[1] else np.zeros(num_heads, np.float32)
+    scales = np.where(absmax == 0, np.float32(1), absmax / np.float32(127)).astype(np.float32)
+    t = d * (np.float32(1) / scales)[:, None]
+    r = np.sign(t) * np.floor(np.abs(t) + np.float32(0.5))      # exact in f32 below 2^23
+    frac_half = (np.abs(t) - np.floor(np.abs(t))) == np.float32(0.5)
+    assert t.dtype == np.float32 and (np.abs(t) < 2 ** 22).all() and frac_half.sum() >= 0
+    return scales, np.clip(r, -127, 127).astype(np.int8).reshape(-1)
+
+
+def test_kv_chunk_reference_tests_restated(orc):
+    # src/huffman.rs:879-905
+    h, d, t = 2, 8, 16
+    data = np.array([((i * 13 + 7) % 100) / 50.0 - 1.0 for i in range(h * t * d)], np.float32)
+    # tests/huffman_parity.rs:133-158
+    for data, (t, h, d) in ((data, (t, h, d)), (parity_random_data(4 * 32 * 16, 99), (32, 4, 16))):
+        bits, scales, codebook, q = orc.huffman_kv_compress_chunk(data, t, h, d)
+        rec = orc.huffman_kv_decompress_chunk(bits, scales, codebook, t, h, d)
+        per_head = np.abs(data - rec).reshape(h, -1).max(axis=1)
+        absmax = np.abs(data).reshape(h, -1).max(axis=1)
+        assert (scales == absmax / np.float32(127)).all()
+        assert (per_head <= scales + 1e-5).all()                 # the reference's bound
+        assert (per_head <= scales * 0.5 * (1 + 1e-6)).all()     # what round-to-nearest gives and truncation does not
+
+
+def test_kv_chunk_closed_forms(orc):
+    t, h, d = 8, 3, 4
+    n = t * d
+    # head 0 all zero, head 1 constant 2.5, head 2 holds +absmax and -absmax
+    data = np.zeros((h, n), np.float32)
+    data[1] = 2.5
+    data[2] = np.linspace(-3.0, 3.0, n, dtype=np.float32)
+    bits, scales, codebook, q = orc.huffman_kv_compress_chunk(data, t, h, d)
+    assert scales[0] == 1.0 and scales[1] == np.float32(2.5) / np.float32(127) and scales[2] == np.float32(3.0) / np.float32(127)
+    q = q.reshape(h, n)
+    assert (q[0] == 0).all() and (q[1] == 127).all() and q[2, 0] == -127 and q[2, -1] == 127
+    rec = orc.huffman_kv_decompress_chunk(bits, scales, codebook, t, h, d).reshape(h, n)
+    assert (rec[0] == 0).all() and (rec[1] == np.float32(127) * scales[1]).all()
+    # one value only: a 1-bit code (src/huffman.rs:52-64), ceil(n / 8) zero bytes, 256 bit lengths with a single 1
+    const = np.full(5 * 7 * 3, -0.75, np.float32)
+    bits, scales, codebook, q = orc.huffman_kv_compress_chunk(const, 7, 5, 3)
+    assert bits == bytes((const.size + 7) // 8) and (q == -127).all()
+    assert codebook[-127 + 128] == 1 and codebook.sum() == 1
+    assert (orc.huffman_kv_decompress_chunk(bits, scales, codebook, 7, 5, 3) == np.float32(-127) * scales[0]).all()
+    # NaN is skipped by the maximum and quantises to 0; an empty chunk is an empty stream under an empty table
+    data = np.array([1.0, np.nan, -0.5, 0.25], np.float32)
+    bits, scales, codebook, q = orc.huffman_kv_compress_chunk(data, 1, 1, 4)
+    assert scales[0] == np.float32(1) / np.float32(127) and q.tolist() == [127, 0, -64, 32]
+    bits, scales, codebook, q = orc.huffman_kv_compress_chunk(np.zeros(0, np.float32), 0, 2, 4)
+    assert bits == b"" and not codebook.any() and (scales == 1.0).all()
+
+
+def test_kv_chunk_is_numpy_quantisation_under_the_pinned_coder(orc):
+    rng = np.random.default_rng(11)
+    for t, h, d in ((5, 3, 7), (32, 4, 16), (1, 1, 1), (64, 2, 128)):
+        data = (rng.standard_normal(t * h * d) * rng.choice([0.01, 1.0, 300.0])).astype(np.float32)
+        data[rng.integers(0, data.size, 3)] = 0.0
+        bits, scales, codebook, q = orc.huffman_kv_compress_chunk(data, t, h, d)
+        want_scales, want_q = numpy_chunk_quant(data, t, h, d)
+        assert (scales == want_scales).all() and (q == want_q).all()
+        bl, _, _ = orc.huffman_table_that_decodes(np.bincount(want_q.astype(np.int16) + 128, minlength=256))
+        assert (codebook == bl).all() and bits == orc.huffman_encode(bl, want_q)
+        rec = orc.huffman_kv_decompress_chunk(bits, scales, codebook, t, h, d)
+        assert (rec == (want_q.reshape(h, -1).astype(np.float32) * want_scales[:, None]).reshape(-1)).all()
+
+
+def test_kv_chunk_table_is_the_reference_s_unless_that_one_cannot_decode(orc):
+    """Where from_frequencies yields a prefix code the chunk uses it unchanged; where its clamp
+    over-subscribes the code (the reference panics there) the repaired lengths are a prefix code of
+    at most 12 bits, ordered by frequency, within two percent of the unlimited Huffman cost."""
+    rng = np.random.default_rng(3)
+    flat = rng.integers(20, 50, 256).astype(np.uint64)
+    bl, _, repaired = orc.huffman_table_that_decodes(flat)
+    assert not repaired and (bl == orc.huffman_table(flat)[0]).all()
+    fib = [1, 1]
+    while len(fib) < 24:
+        fib.append(fib[-1] + fib[-2])
+    f_fib = np.zeros(256, np.uint64)
+    f_fib[100:124] = fib
+    bell = np.bincount(np.clip(np.rint(rng.standard_normal(1 << 16) * 30), -127, 127).astype(np.int16) + 128, minlength=256).astype(np.uint64)
+    for f in (f_fib, bell):
+        ref_bl = orc.huffman_table(f)[0]
+        assert sum(2.0 ** -int(l) for l in ref_bl if l) > 1.0        # the case the reference cannot handle
+        bl, codes, repaired = orc.huffman_table_that_decodes(f)
+        assert repaired and ((bl > 0) == (f > 0)).all() and bl.max() <= 12
+        assert sum(2.0 ** -int(l) for l in bl if l) <= 1.0
+        used = np.flatnonzero(f)
+        for a in used:                                               # a more frequent symbol never has the longer code
+            assert (bl[used][f[used] < f[a]] >= bl[a]).all()
+        assert int((f * bl).sum()) <= heap_huffman_cost(f) * 1.02
+        data = np.repeat(np.arange(256) - 128, np.minimum(f, 50).astype(np.int64)).astype(np.int8)
+        rng.shuffle(data)
+        assert (orc.huffman_decode(bl, orc.huffman_encode(bl, data), data.size) == data).all()
+    # through compress_chunk: a bell-shaped chunk of realistic size round-trips
+    t, h, d = 64, 2, 128
+    data = rng.standard_normal(t * h * d).astype(np.float32)
+    bits, scales, codebook, q = orc.huffman_kv_compress_chunk(data, t, h, d)
+    rec = orc.huffman_kv_decompress_chunk(bits, scales, codebook, t, h, d)
+    assert (rec == (q.reshape(h, -1).astype(np.float32) * scales[:, None]).reshape(-1)).all()
+
+
+def test_kv_cache_reference_tests_restated(orc):
+    # src/huffman.rs:850-876
+    c = orc.HuffmanKVCache(2, 4, 8, 4)
+    c.append(np.full(32, 1.0), np.full(32, 2.0), 4)
+    assert (c.len, c.compressed_len) == (4, 0)
+    c.append(np.full(32, 3.0), np.full(32, 4.0), 4)
+    assert (c.len, c.compressed_len) == (8, 4)
+    k, v = c.get_kv()
+    assert k.size == v.size == 2 * 8 * 4
+    assert (k.reshape(2, 8, 4)[:, :4] == 1.0).all() and (k.reshape(2, 8, 4)[:, 4:] == 3.0).all()
+    assert (v.reshape(2, 8, 4)[:, :4] == 2.0).all() and (v.reshape(2, 8, 4)[:, 4:] == 4.0).all()
+    # tests/huffman_parity.rs:160-186
+    c = orc.HuffmanKVCache(2, 8, 16, 8)
+    for batch in range(4):
+        c.append(parity_random_data(2 * 8 * 8, 100 + batch), parity_random_data(2 * 8 * 8, 200 + batch), 8)
+    assert c.len == 32 and c.compressed_len > 0
+    k, v = c.get_kv()
+    assert k.size == v.size == 2 * 32 * 8
+    # new(): compress_threshold.max(chunk_size)  (src/huffman.rs:535)
+    assert orc.HuffmanKVCache(1, 1, 3, 10).compress_threshold == 10
+
+
+def test_kv_cache_keeps_token_order(orc):
+    """Whatever the append sizes, get_kv is: per chunk, decompress(compress(.)) of the tokens the
+    chunk took in arrival order, then the window's tokens bit for bit."""
+    rng = np.random.default_rng(5)
+    for heads, hd, thr, chunk, appends in ((2, 8, 16, 8, (8, 8, 8, 8)), (3, 4, 10, 4, (1, 7, 2, 30, 5, 1)), (1, 16, 0, 5, (3, 3, 3)),
+                                           (2, 2, 6, 6, (13,))):
+        c = orc.HuffmanKVCache(heads, hd, thr, chunk)
+        all_k, all_v = np.zeros((heads, 0, hd), np.float32), np.zeros((heads, 0, hd), np.float32)
+        for n in appends:
+            k, v = rng.standard_normal((heads, n, hd)).astype(np.float32), rng.standard_normal((heads, n, hd)).astype(np.float32)
+            c.append(k, v, n)
+            all_k, all_v = np.concatenate([all_k, k], 1), np.concatenate([all_v, v], 1)
+            total = all_k.shape[1]
+            threshold = max(thr, chunk)
+            # chunks of exactly chunk_size are cut while at least `threshold` tokens are left
+            ncomp = 0
+            while total - ncomp >= threshold:
+                ncomp += chunk
+            assert (c.len, c.compressed_len, c.hot_len, c.num_chunks) == (total, ncomp, total - ncomp, ncomp // chunk)
+            for side, full in ((0, all_k), (1, all_v)):
+                got = c.get_kv()[side].reshape(heads, total, hd)
+                assert (got[:, ncomp:] == full[:, ncomp:]).all()
+                for i in range(ncomp // chunk):
+                    part = full[:, i * chunk:(i + 1) * chunk]
+                    bits, scales, codebook, _ = orc.huffman_kv_compress_chunk(part, chunk, heads, hd)
+                    cb, cs, ccb, ct = c.chunk(side, i)
+                    assert (cb, ct) == (bits, chunk) and (cs == scales).all() and (ccb == codebook).all()
+                    rec = orc.huffman_kv_decompress_chunk(bits, scales, codebook, chunk, heads, hd).reshape(heads, chunk, hd)
+                    assert (got[:, i * chunk:(i + 1) * chunk] == rec).all()
+        # the reference's own hot-window offsets agree for head 0 always
+        lit = c.get_kv(True)[0].reshape(heads, -1, hd)
+        assert (lit[0] == c.get_kv()[0].reshape(heads, -1, hd)[0]).all()
