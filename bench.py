@@ -1094,6 +1094,39 @@ def section_huffman_kv(B, line):
         res[name] = {"ms_per_call_wall": round(wall, 3),
                      "kernels_ms": round(sum(v[0] * v[1] for v in prof.values()) / 5, 4),
                      "kernels_ms_x_launches": {k: [round(v[0], 4), round(v[1] / 5, 1)] for k, v in prof.items()}}
+    # a cache of 8448 tokens: 32 chunks per side behind a window of 256 tokens; get_kv decodes all 64 streams in one pass
+    cache = C.c_void_p()
+    check(lib.pg_huffman_kv_cache_create(B.h, heads, hd, 2 * tokens, tokens, C.byref(cache)))
+    piece = 1056
+    kk, vv = B.normal(7501, (heads * piece * hd,), 1.0), B.normal(7502, (heads * piece * hd,), 2.0)
+    B.torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(8):
+        check(lib.pg_huffman_kv_cache_append_dev(B.h, cache, C.c_void_p(kk.data_ptr()), C.c_void_p(vv.data_ptr()), piece))
+    B.torch.cuda.synchronize()
+    append_ms = (time.perf_counter() - t0) / 8 * 1e3
+    total_len, comp_len = lib.pg_huffman_kv_cache_len(cache), lib.pg_huffman_kv_cache_compressed_len(cache)
+    full_k = B.torch.empty(heads * total_len * hd, dtype=B.torch.float32, device=data.device)
+    full_v = B.torch.empty_like(full_k)
+
+    def get_step():
+        check(lib.pg_huffman_kv_cache_get_kv_dev(B.h, cache, C.c_void_p(full_k.data_ptr()), C.c_void_p(full_v.data_ptr())))
+
+    for _ in range(2):
+        get_step()
+    B.torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        get_step()
+    B.torch.cuda.synchronize()
+    get_ms = (time.perf_counter() - t0) / 5 * 1e3
+    gprof, _ = B.profiled(get_step, 3)
+    res["cache"] = {"workload": f"{total_len} tokens ({comp_len} in {lib.pg_huffman_kv_cache_num_chunks(cache)} chunks per side), appended {piece} at a time from device tensors",
+                    "append_ms_per_call_wall": round(append_ms, 3), "get_kv_dev_ms_wall": round(get_ms, 3),
+                    "get_kv_dev_gbs_of_f32_out": round(2 * 4 * heads * total_len * hd / (get_ms * 1e-3) / 1e9, 1),
+                    "get_kv_kernels_ms_x_launches": {k: [round(v[0], 4), round(v[1] / 3, 1)] for k, v in gprof.items()}}
+    lib.pg_huffman_kv_cache_free(B.h, cache)
+    del full_k, full_v, kk, vv
     if B.cpu:  # the scalar restatement of compress_chunk / decompress_chunk on the same chunk (the prebuilt -O2 oracle)
         import numpy as np
         olib = C.CDLL(os.path.join(ROOT, "oracle", "_build", "libperegrine_oracle.so"))

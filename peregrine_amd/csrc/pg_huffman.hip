@@ -177,7 +177,8 @@ size_t encode_host(const uint8_t *bl, const uint32_t *codes, const int8_t *data,
 // ---- device: decode ----------------------------------------------------------------------
 
 struct stream_desc {
-    unsigned long long byte_off;  // into the concatenated stream bytes
+    const uint8_t *bytes;         // the stream, in device memory
+    const uint16_t *lut;          // its decode table (LUT_SIZE entries), in device memory
     unsigned long long nbits;     // 8 * stream bytes
     unsigned long long nsym;      // symbols to produce
     unsigned long long out_off;   // into the output
@@ -209,28 +210,32 @@ __device__ __forceinline__ void decode_span(const uint8_t *__restrict__ s, unsig
     count = c;
 }
 
+// The stream workgroup `wg` works on: the last one whose first workgroup is not past it.
 __device__ __forceinline__ int find_stream(const stream_desc *__restrict__ desc, int nstreams, unsigned wg) {
-    int s = 0;
-    while (s + 1 < nstreams && wg >= desc[s + 1].wg_base) ++s;
-    return s;
+    int lo = 0, hi = nstreams - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (desc[mid].wg_base <= wg) lo = mid;
+        else hi = mid - 1;
+    }
+    return lo;
 }
 
 // One round: every workgroup settles its 256 subsequences against the end its predecessor
 // workgroup reported last, and raises `changed` if anything moved.
-__global__ __launch_bounds__(WG) void huff_sync_kernel(const uint8_t *__restrict__ bytes, const stream_desc *__restrict__ desc,
-                                                       int nstreams, const uint16_t *__restrict__ lut_g, int first_round,
+__global__ __launch_bounds__(WG) void huff_sync_kernel(const stream_desc *__restrict__ desc, int nstreams, int first_round,
                                                        unsigned long long *__restrict__ start_g,
                                                        unsigned long long *end_g, unsigned *__restrict__ count_g,
                                                        int *__restrict__ changed) {
     __shared__ uint16_t lut[LUT_SIZE];
     __shared__ unsigned long long s_end[WG];
-    for (int i = threadIdx.x; i < LUT_SIZE; i += WG) lut[i] = lut_g[i];
     const int si = find_stream(desc, nstreams, blockIdx.x);
     const stream_desc d = desc[si];
+    for (int i = threadIdx.x; i < LUT_SIZE; i += WG) lut[i] = d.lut[i];
     const unsigned local = (blockIdx.x - d.wg_base) * WG + threadIdx.x;  // subsequence within the stream
     const bool live = local < d.nsub;
     const size_t g = (size_t)d.sub_base + local;
-    const uint8_t *s = bytes + d.byte_off;
+    const uint8_t *s = d.bytes;
     const unsigned long long limit = min((unsigned long long)(local + 1) * SUBSEQ_BITS, d.nbits);
     unsigned long long start = 0, end = 0;
     unsigned count = 0;
@@ -317,21 +322,20 @@ __global__ __launch_bounds__(64) void huff_scan_wg_kernel(const stream_desc *__r
     if (run < d.nsym) *err = 1;
 }
 
-__global__ __launch_bounds__(WG) void huff_write_kernel(const uint8_t *__restrict__ bytes, const stream_desc *__restrict__ desc,
-                                                        int nstreams, const uint16_t *__restrict__ lut_g,
+__global__ __launch_bounds__(WG) void huff_write_kernel(const stream_desc *__restrict__ desc, int nstreams,
                                                         const unsigned long long *__restrict__ start_g,
                                                         const unsigned *__restrict__ excl_g,
                                                         const unsigned long long *__restrict__ wg_excl,
                                                         int8_t *__restrict__ out, int *__restrict__ err) {
     __shared__ uint16_t lut[LUT_SIZE];
-    for (int i = threadIdx.x; i < LUT_SIZE; i += WG) lut[i] = lut_g[i];
-    __syncthreads();
     const int si = find_stream(desc, nstreams, blockIdx.x);
     const stream_desc d = desc[si];
+    for (int i = threadIdx.x; i < LUT_SIZE; i += WG) lut[i] = d.lut[i];
+    __syncthreads();
     const unsigned local = (blockIdx.x - d.wg_base) * WG + threadIdx.x;
     if (local >= d.nsub) return;
     const size_t g = (size_t)d.sub_base + local;
-    const uint8_t *s = bytes + d.byte_off;
+    const uint8_t *s = d.bytes;
     const unsigned long long limit = min((unsigned long long)(local + 1) * SUBSEQ_BITS, d.nbits);
     unsigned long long p = start_g[g], idx = wg_excl[blockIdx.x] + excl_g[g];
     while (p < limit && idx < d.nsym) {
@@ -347,11 +351,12 @@ __global__ __launch_bounds__(WG) void huff_write_kernel(const uint8_t *__restric
     }
 }
 
-// Adds one stream of `bytes` bytes at d_bytes + byte_off holding `symbols` symbols, decoded to out + out_off.
-pg_status add_stream(std::vector<stream_desc> &desc, size_t byte_off, size_t bytes, size_t symbols, size_t out_off, size_t &sub,
-                     size_t &wg) {
+// Adds one stream of `bytes` bytes at bytes_dev holding `symbols` symbols, decoded through lut_dev to out + out_off.
+pg_status add_stream(std::vector<stream_desc> &desc, const uint8_t *bytes_dev, const uint16_t *lut_dev, size_t bytes,
+                     size_t symbols, size_t out_off, size_t &sub, size_t &wg) {
     stream_desc d;
-    d.byte_off = byte_off;
+    d.bytes = bytes_dev;
+    d.lut = lut_dev;
     d.nbits = (unsigned long long)bytes * 8;
     d.nsym = symbols;
     d.out_off = out_off;
@@ -364,14 +369,11 @@ pg_status add_stream(std::vector<stream_desc> &desc, size_t byte_off, size_t byt
     return PG_OK;
 }
 
-// Decode the streams `desc` describes (bytes already in device memory at d_bytes) into out_dev.
-pg_status decode_device_streams(pg_ctx *ctx, const uint8_t *bit_lengths, const std::vector<stream_desc> &desc,
-                                const uint8_t *d_bytes, size_t sub, size_t wg, int8_t *out_dev) {
+// Decode the streams `desc` describes (bytes in device memory) into out_dev.  Streams without a
+// table of their own (lut == nullptr) share the one built here from bit_lengths.
+pg_status decode_device_streams(pg_ctx *ctx, const uint8_t *bit_lengths, std::vector<stream_desc> desc, size_t sub, size_t wg,
+                                int8_t *out_dev) {
     if (desc.empty()) return PG_OK;
-    uint32_t codes[NUM_SYMBOLS];
-    std::vector<uint16_t> lut(LUT_SIZE);
-    canonical_codes(bit_lengths, codes);
-    PG_TRY(build_lut(bit_lengths, codes, lut.data()));
     // one allocation: descriptors | lut | start | end | count | excl | wg totals | flags
     const size_t o_lut = pg_round_up(desc.size() * sizeof(stream_desc), 256);
     const size_t o_start = o_lut + LUT_SIZE * sizeof(uint16_t), o_end = o_start + pg_round_up(sub * 8, 256);
@@ -380,11 +382,21 @@ pg_status decode_device_streams(pg_ctx *ctx, const uint8_t *bit_lengths, const s
     pg_tmp buf;
     PG_TRY(buf.alloc(o_flag + 256));
     char *base = buf.as<char>();
+    std::vector<uint16_t> lut;
+    if (bit_lengths) {
+        uint32_t codes[NUM_SYMBOLS];
+        lut.resize(LUT_SIZE);
+        canonical_codes(bit_lengths, codes);
+        PG_TRY(build_lut(bit_lengths, codes, lut.data()));
+        PG_HIP(hipMemcpyAsync(base + o_lut, lut.data(), LUT_SIZE * sizeof(uint16_t), hipMemcpyHostToDevice, ctx->stream));
+    }
+    for (auto &d : desc) {
+        if (!d.lut) d.lut = reinterpret_cast<const uint16_t *>(base + o_lut);
+        PG_CHECK_ARG(d.lut != reinterpret_cast<const uint16_t *>(base + o_lut) || bit_lengths, "huffman decode: a stream without a table");
+    }
     PG_HIP(hipMemsetAsync(base + o_flag, 0, 256, ctx->stream));
     PG_HIP(hipMemcpyAsync(base, desc.data(), desc.size() * sizeof(stream_desc), hipMemcpyHostToDevice, ctx->stream));
-    PG_HIP(hipMemcpyAsync(base + o_lut, lut.data(), LUT_SIZE * sizeof(uint16_t), hipMemcpyHostToDevice, ctx->stream));
     const stream_desc *d_desc = reinterpret_cast<const stream_desc *>(base);
-    const uint16_t *d_lut = reinterpret_cast<const uint16_t *>(base + o_lut);
     auto *d_start = reinterpret_cast<unsigned long long *>(base + o_start);
     auto *d_end = reinterpret_cast<unsigned long long *>(base + o_end);
     auto *d_count = reinterpret_cast<unsigned *>(base + o_count);
@@ -392,12 +404,12 @@ pg_status decode_device_streams(pg_ctx *ctx, const uint8_t *bit_lengths, const s
     auto *d_wg = reinterpret_cast<unsigned long long *>(base + o_wg);
     int *d_changed = reinterpret_cast<int *>(base + o_flag), *d_err = d_changed + 1;
     const int ns = (int)desc.size();
-    PG_TRY(pg_launch(ctx, "huffman_sync", huff_sync_kernel, dim3((unsigned)wg), dim3(WG), 0, d_bytes, d_desc, ns, d_lut, 1,
-                     d_start, d_end, d_count, d_changed));
+    PG_TRY(pg_launch(ctx, "huffman_sync", huff_sync_kernel, dim3((unsigned)wg), dim3(WG), 0, d_desc, ns, 1, d_start, d_end, d_count,
+                     d_changed));
     for (size_t round = 0;; ++round) {
         if (round > wg + 1) return pg_fail(PG_EDEVICE, "huffman decode: the subsequence starts did not settle");
-        PG_TRY(pg_launch(ctx, "huffman_sync", huff_sync_kernel, dim3((unsigned)wg), dim3(WG), 0, d_bytes, d_desc, ns, d_lut, 0,
-                         d_start, d_end, d_count, d_changed));
+        PG_TRY(pg_launch(ctx, "huffman_sync", huff_sync_kernel, dim3((unsigned)wg), dim3(WG), 0, d_desc, ns, 0, d_start, d_end,
+                         d_count, d_changed));
         int changed = 0;
         PG_HIP(hipMemcpyAsync(&changed, d_changed, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
         PG_HIP(hipStreamSynchronize(ctx->stream));
@@ -407,7 +419,7 @@ pg_status decode_device_streams(pg_ctx *ctx, const uint8_t *bit_lengths, const s
     PG_TRY(pg_launch(ctx, "huffman_scan", huff_scan_local_kernel, dim3((unsigned)wg), dim3(WG), 0, d_desc, ns,
                      (const unsigned *)d_count, d_excl, d_wg));
     PG_TRY(pg_launch(ctx, "huffman_scan_wg", huff_scan_wg_kernel, dim3((unsigned)ns), dim3(64), 0, d_desc, d_wg, d_err));
-    PG_TRY(pg_launch(ctx, "huffman_write", huff_write_kernel, dim3((unsigned)wg), dim3(WG), 0, d_bytes, d_desc, ns, d_lut,
+    PG_TRY(pg_launch(ctx, "huffman_write", huff_write_kernel, dim3((unsigned)wg), dim3(WG), 0, d_desc, ns,
                      (const unsigned long long *)d_start, (const unsigned *)d_excl, (const unsigned long long *)d_wg, out_dev,
                      d_err));
     int err = 0;
@@ -422,24 +434,25 @@ pg_status decode_device_streams(pg_ctx *ctx, const uint8_t *bit_lengths, const s
 // holds symbols[i] symbols, written back to back.
 pg_status decode_streams(pg_ctx *ctx, const uint8_t *bit_lengths, const uint8_t *const *streams, const size_t *bytes,
                          const size_t *symbols, size_t nstreams, int8_t *out_dev) {
+    size_t total = 0;
+    for (size_t i = 0; i < nstreams; ++i) {
+        if (symbols[i] == 0) continue;
+        PG_CHECK_ARG(bytes[i] > 0 && streams[i], "huffman decode: stream %zu holds %zu symbols in no bytes", i, symbols[i]);
+        total += pg_round_up(bytes[i], 16);
+    }
+    if (total == 0) return PG_OK;
+    pg_tmp buf;
+    PG_TRY(buf.alloc(total));
     std::vector<stream_desc> desc;
     size_t byte_off = 0, out_off = 0, sub = 0, wg = 0;
     for (size_t i = 0; i < nstreams; ++i) {
         if (symbols[i] == 0) continue;
-        PG_CHECK_ARG(bytes[i] > 0 && streams[i], "huffman decode: stream %zu holds %zu symbols in no bytes", i, symbols[i]);
-        PG_TRY(add_stream(desc, byte_off, bytes[i], symbols[i], out_off, sub, wg));
+        PG_TRY(add_stream(desc, buf.as<uint8_t>() + byte_off, nullptr, bytes[i], symbols[i], out_off, sub, wg));
+        PG_HIP(hipMemcpyAsync(buf.as<char>() + byte_off, streams[i], bytes[i], hipMemcpyHostToDevice, ctx->stream));
         byte_off += pg_round_up(bytes[i], 16);
         out_off += symbols[i];
     }
-    if (desc.empty()) return PG_OK;
-    pg_tmp buf;
-    PG_TRY(buf.alloc(byte_off));
-    for (size_t i = 0, j = 0; i < nstreams; ++i) {
-        if (symbols[i] == 0) continue;
-        PG_HIP(hipMemcpyAsync(buf.as<char>() + desc[j].byte_off, streams[i], bytes[i], hipMemcpyHostToDevice, ctx->stream));
-        ++j;
-    }
-    return decode_device_streams(ctx, bit_lengths, desc, buf.as<uint8_t>(), sub, wg, out_dev);
+    return decode_device_streams(ctx, bit_lengths, desc, sub, wg, out_dev);
 }
 
 }  // namespace
@@ -460,14 +473,25 @@ bool pg_huffman_host_table(const uint64_t *freqs, uint8_t *bit_lengths, uint32_t
     return repaired;
 }
 
-pg_status pg_huffman_decode_device_stream(pg_ctx *ctx, const uint8_t *bit_lengths, const uint8_t *bytes_dev, size_t bytes,
-                                          size_t num_symbols, int8_t *out_dev) {
-    if (num_symbols == 0) return PG_OK;
-    PG_CHECK_ARG(bytes > 0 && bytes_dev, "huffman decode: %zu symbols in no bytes", num_symbols);
+// The decode table of a code (LUT entries of 16 bits, pg_huffman_lut_entries() of them) on the host.
+size_t pg_huffman_lut_entries() { return LUT_SIZE; }
+pg_status pg_huffman_host_lut(const uint8_t *bit_lengths, uint16_t *lut) {
+    uint32_t codes[NUM_SYMBOLS];
+    canonical_codes(bit_lengths, codes);
+    return build_lut(bit_lengths, codes, lut);
+}
+
+// Streams that sit in device memory, each with its own table there, decoded in one pass.
+pg_status pg_huffman_decode_device_streams(pg_ctx *ctx, const pg_huffman_dev_stream *streams, size_t count, int8_t *out_dev) {
     std::vector<stream_desc> desc;
     size_t sub = 0, wg = 0;
-    PG_TRY(add_stream(desc, 0, bytes, num_symbols, 0, sub, wg));
-    return decode_device_streams(ctx, bit_lengths, desc, bytes_dev, sub, wg, out_dev);
+    for (size_t i = 0; i < count; ++i) {
+        const pg_huffman_dev_stream &st = streams[i];
+        if (st.symbols == 0) continue;
+        PG_CHECK_ARG(st.bytes > 0 && st.bytes_dev && st.lut_dev, "huffman decode: %zu symbols in no bytes or without a table", st.symbols);
+        PG_TRY(add_stream(desc, st.bytes_dev, st.lut_dev, st.bytes, st.symbols, st.out_off, sub, wg));
+    }
+    return decode_device_streams(ctx, nullptr, desc, sub, wg, out_dev);
 }
 
 pg_status pg_qtensor_from_device_q(pg_ctx *ctx, const int8_t *q_dev, const float *scales_host, size_t rows, size_t cols,

@@ -10,16 +10,13 @@
 // from two kernels, the host builds the table from the histogram (2 KB down, 1 KB up), and the
 // encoder is a prefix sum over the code lengths followed by one pass in which every thread packs
 // 16 consecutive codes into the words of the MSB-first stream.  Coded chunks stay in device
-// memory; decoding is the self-synchronising decoder of the Huffman-coded weights followed by a
-// scaling kernel that writes straight into the caller's [heads, tokens, head_dim] layout.
+// memory, each with its 8 KB decode table beside it; decoding is the self-synchronising decoder of
+// the Huffman-coded weights over all chunks of a cache at once (every stream under its own table),
+// followed by one scaling kernel that writes straight into the caller's [heads, tokens, head_dim] layout.
 #include <new>
 #include <vector>
 #include "pg_internal.h"
 #include "pg_quant_dev.h"
-
-bool pg_huffman_host_table(const uint64_t *freqs, uint8_t *bit_lengths, uint32_t *codes);
-pg_status pg_huffman_decode_device_stream(pg_ctx *ctx, const uint8_t *bit_lengths, const uint8_t *bytes_dev, size_t bytes,
-                                          size_t num_symbols, int8_t *out_dev);
 
 namespace {
 
@@ -169,13 +166,20 @@ __global__ __launch_bounds__(KV_WG) void kv_encode_write_kernel(const int8_t *__
     if (nacc > 0) atomicOr(words + word, __builtin_bswap32((unsigned)(acc << (32 - nacc))));
 }
 
-// decoded_i8 as f32 * scale[head]   src/huffman.rs:669-677, into rows of out_stride floats per head.
-__global__ __launch_bounds__(KV_WG) void kv_dequant_kernel(const int8_t *__restrict__ q, const float *__restrict__ scales,
-                                                           size_t head_elems, float *__restrict__ out, size_t out_stride) {
-    const float scale = scales[blockIdx.y];
-    const int8_t *p = q + (size_t)blockIdx.y * head_elems;
-    float *o = out + (size_t)blockIdx.y * out_stride;
-    for (size_t i = (size_t)blockIdx.x * KV_WG + threadIdx.x; i < head_elems; i += (size_t)gridDim.x * KV_WG)
+// decoded_i8 as f32 * scale[head]   src/huffman.rs:669-677 for several chunks in one launch: grid
+// (splits, heads, chunks); chunk c's values start at q + q_off and go to rows of out_stride floats per head.
+struct dequant_item {
+    const float *scales;
+    float *out;
+    size_t q_off, head_elems, out_stride;
+};
+
+__global__ __launch_bounds__(KV_WG) void kv_dequant_kernel(const int8_t *__restrict__ q, const dequant_item *__restrict__ items) {
+    const dequant_item it = items[blockIdx.z];
+    const float scale = it.scales[blockIdx.y];
+    const int8_t *p = q + it.q_off + (size_t)blockIdx.y * it.head_elems;
+    float *o = it.out + (size_t)blockIdx.y * it.out_stride;
+    for (size_t i = (size_t)blockIdx.x * KV_WG + threadIdx.x; i < it.head_elems; i += (size_t)gridDim.x * KV_WG)
         o[i] = (float)p[i] * scale;
 }
 
@@ -190,12 +194,15 @@ unsigned splits_for(size_t head_elems) {
 struct pg_huffman_kv_chunk {
     uint8_t codebook[NUM_SYMBOLS];
     std::vector<float> scales;
-    char *dev = nullptr;  // [scales, 256-byte rounded][bitstream, zero padded to a whole word and 16 bytes on]
+    char *dev = nullptr;  // [scales, 256-byte rounded][decode table][bitstream, zero padded to a whole word and 16 bytes on]
     size_t bytes = 0;     // of the bitstream
     size_t num_tokens = 0, num_heads = 0, head_dim = 0;
+    bool decodable = false;  // the codebook fits the decode table (always, for chunks made here)
     size_t scales_bytes() const { return pg_round_up(num_heads * sizeof(float), 256); }
+    size_t head_bytes() const { return scales_bytes() + pg_huffman_lut_entries() * sizeof(uint16_t); }
     const float *scales_dev() const { return reinterpret_cast<const float *>(dev); }
-    const uint8_t *bits_dev() const { return reinterpret_cast<const uint8_t *>(dev + scales_bytes()); }
+    const uint16_t *lut_dev() const { return reinterpret_cast<const uint16_t *>(dev + scales_bytes()); }
+    const uint8_t *bits_dev() const { return reinterpret_cast<const uint8_t *>(dev + head_bytes()); }
     size_t symbols() const { return num_heads * num_tokens * head_dim; }
     ~pg_huffman_kv_chunk() { if (dev) (void)hipFree(dev); }
 };
@@ -216,13 +223,21 @@ static pg_status chunk_shape_ok(const char *who, size_t num_tokens, size_t num_h
     return PG_OK;
 }
 
-static pg_status chunk_alloc(pg_huffman_kv_chunk *c, size_t bytes) {
+// Allocates the chunk's device memory, zeroes it (stream ordered) and puts the decode table of c->codebook in place.
+static pg_status chunk_alloc(pg_ctx *ctx, pg_huffman_kv_chunk *c, size_t bytes) {
     c->bytes = bytes;
-    const size_t total = c->scales_bytes() + pg_round_up(bytes, 4) + 16;
+    const size_t total = c->head_bytes() + pg_round_up(bytes, 4) + 16;
     hipError_t e = hipMalloc((void **)&c->dev, total);
     if (e != hipSuccess) {
         c->dev = nullptr;
         return pg_fail(PG_ENOMEM, "hipMalloc(%zu) failed: %s", total, hipGetErrorString(e));
+    }
+    PG_HIP(hipMemsetAsync(c->dev, 0, total, ctx->stream));
+    std::vector<uint16_t> lut(pg_huffman_lut_entries());
+    c->decodable = pg_huffman_host_lut(c->codebook, lut.data()) == PG_OK;  // else: reported when the chunk is decoded
+    if (c->decodable) {
+        PG_HIP(hipMemcpyAsync(c->dev + c->scales_bytes(), lut.data(), lut.size() * sizeof(uint16_t), hipMemcpyHostToDevice, ctx->stream));
+        PG_HIP(hipStreamSynchronize(ctx->stream));  // lut is a local
     }
     return PG_OK;
 }
@@ -240,8 +255,7 @@ static pg_status compress_dev(pg_ctx *ctx, const float *data, size_t head_stride
     c->scales.assign(num_heads, 1.0f);  // absmax == 0.0 -> 1.0
     const size_t head_elems = num_tokens * head_dim, total = num_heads * head_elems;
     if (total == 0) {  // an empty table, an empty stream
-        PG_TRY(chunk_alloc(c, 0));
-        PG_HIP(hipMemsetAsync(c->dev, 0, c->scales_bytes() + 16, ctx->stream));
+        PG_TRY(chunk_alloc(ctx, c, 0));
         if (num_heads)
             PG_HIP(hipMemcpyAsync(c->dev, c->scales.data(), num_heads * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
         PG_HIP(hipStreamSynchronize(ctx->stream));
@@ -283,29 +297,52 @@ static pg_status compress_dev(pg_ctx *ctx, const float *data, size_t head_stride
     unsigned long long bits = 0;
     PG_HIP(hipMemcpyAsync(&bits, d_wg + nwg, sizeof bits, hipMemcpyDeviceToHost, ctx->stream));
     PG_HIP(hipStreamSynchronize(ctx->stream));
-    PG_TRY(chunk_alloc(c, (size_t)((bits + 7) / 8)));
-    PG_HIP(hipMemsetAsync(c->dev, 0, c->scales_bytes() + pg_round_up(c->bytes, 4) + 16, ctx->stream));
+    PG_TRY(chunk_alloc(ctx, c, (size_t)((bits + 7) / 8)));
     PG_HIP(hipMemcpyAsync(c->dev, d_scales, num_heads * sizeof(float), hipMemcpyDeviceToDevice, ctx->stream));
     PG_TRY(pg_launch(ctx, "huffman_kv_encode_write", kv_encode_write_kernel, dim3((unsigned)nwg), dim3(KV_WG), 0,
                      (const int8_t *)d_q, total, (const unsigned *)d_codes, (const unsigned long long *)d_wg,
-                     reinterpret_cast<unsigned *>(c->dev + c->scales_bytes())));
+                     reinterpret_cast<unsigned *>(c->dev + c->head_bytes())));
     PG_HIP(hipStreamSynchronize(ctx->stream));  // buf is freed on return
     g.c = nullptr;
     *out = c;
     return PG_OK;
 }
 
-// decompress_chunk into device memory: head h's values go to out + h * out_stride.
-static pg_status decompress_dev(pg_ctx *ctx, const pg_huffman_kv_chunk *c, float *out, size_t out_stride) {
-    const size_t total = c->symbols(), head_elems = c->num_tokens * c->head_dim;
-    if (total == 0) return PG_OK;
-    pg_tmp q;
-    PG_TRY(q.alloc(total));
-    PG_TRY(pg_huffman_decode_device_stream(ctx, c->codebook, c->bits_dev(), c->bytes, total, q.as<int8_t>()));
-    PG_TRY(pg_launch(ctx, "huffman_kv_dequant", kv_dequant_kernel, dim3(splits_for(head_elems), (unsigned)c->num_heads),
-                     dim3(KV_WG), 0, (const int8_t *)q.as<int8_t>(), c->scales_dev(), head_elems, out, out_stride));
-    PG_HIP(hipStreamSynchronize(ctx->stream));  // q is freed on return
+// decompress_chunk for several chunks in one pass: chunk i's head h goes to out[i] + h * out_stride[i].
+static pg_status decompress_many(pg_ctx *ctx, const pg_huffman_kv_chunk *const *chunks, float *const *out, const size_t *out_stride,
+                                 size_t count) {
+    std::vector<pg_huffman_dev_stream> streams;
+    std::vector<dequant_item> items;
+    size_t total = 0, max_head_elems = 0, heads = 0;
+    for (size_t i = 0; i < count; ++i) {
+        const pg_huffman_kv_chunk *c = chunks[i];
+        if (c->symbols() == 0) continue;
+        if (!c->decodable) {  // sets the message
+            std::vector<uint16_t> lut(pg_huffman_lut_entries());
+            PG_TRY(pg_huffman_host_lut(c->codebook, lut.data()));
+        }
+        PG_CHECK_ARG(heads == 0 || heads == c->num_heads, "huffman kv: chunks of %zu and %zu heads in one pass", heads, c->num_heads);
+        heads = c->num_heads;
+        streams.push_back({c->bits_dev(), c->bytes, c->symbols(), c->lut_dev(), total});
+        items.push_back({c->scales_dev(), out[i], total, c->num_tokens * c->head_dim, out_stride[i]});
+        max_head_elems = std::max(max_head_elems, c->num_tokens * c->head_dim);
+        total += pg_round_up(c->symbols(), 16);
+    }
+    if (items.empty()) return PG_OK;
+    PG_CHECK_ARG(items.size() < 65536, "huffman kv: %zu chunks in one pass", items.size());
+    const size_t o_items = pg_round_up(total, 256);
+    pg_tmp buf;
+    PG_TRY(buf.alloc(o_items + items.size() * sizeof(dequant_item)));
+    PG_HIP(hipMemcpyAsync(buf.as<char>() + o_items, items.data(), items.size() * sizeof(dequant_item), hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_huffman_decode_device_streams(ctx, streams.data(), streams.size(), buf.as<int8_t>()));
+    PG_TRY(pg_launch(ctx, "huffman_kv_dequant", kv_dequant_kernel, dim3(splits_for(max_head_elems), (unsigned)heads, (unsigned)items.size()),
+                     dim3(KV_WG), 0, (const int8_t *)buf.as<int8_t>(), reinterpret_cast<const dequant_item *>(buf.as<char>() + o_items)));
+    PG_HIP(hipStreamSynchronize(ctx->stream));  // buf is freed on return
     return PG_OK;
+}
+
+static pg_status decompress_dev(pg_ctx *ctx, const pg_huffman_kv_chunk *c, float *out, size_t out_stride) {
+    return decompress_many(ctx, &c, &out, &out_stride, 1);
 }
 
 PG_API pg_status pg_huffman_kv_compress_chunk_dev(pg_ctx *ctx, const float *data_dev, size_t head_stride, size_t num_tokens,
@@ -347,10 +384,9 @@ PG_API pg_status pg_huffman_kv_chunk_from_parts(pg_ctx *ctx, const uint8_t *bits
     c->num_tokens = num_tokens; c->num_heads = num_heads; c->head_dim = head_dim;
     std::copy(codebook, codebook + NUM_SYMBOLS, c->codebook);
     c->scales.assign(scales, scales + num_heads);
-    PG_TRY(chunk_alloc(c, bytes));
-    PG_HIP(hipMemsetAsync(c->dev, 0, c->scales_bytes() + pg_round_up(bytes, 4) + 16, ctx->stream));
+    PG_TRY(chunk_alloc(ctx, c, bytes));
     if (num_heads) PG_HIP(hipMemcpyAsync(c->dev, scales, num_heads * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
-    if (bytes) PG_HIP(hipMemcpyAsync(c->dev + c->scales_bytes(), bitstream, bytes, hipMemcpyHostToDevice, ctx->stream));
+    if (bytes) PG_HIP(hipMemcpyAsync(c->dev + c->head_bytes(), bitstream, bytes, hipMemcpyHostToDevice, ctx->stream));
     PG_HIP(hipStreamSynchronize(ctx->stream));
     g.c = nullptr;
     *out = c;
@@ -522,11 +558,17 @@ PG_API pg_status pg_huffman_kv_cache_get_kv_dev(pg_ctx *ctx, const pg_huffman_kv
     if (total_len * hd * heads == 0) return PG_OK;
     PG_CHECK_ARG(k_dev && v_dev, "pg_huffman_kv_cache_get_kv: null output");
     size_t off = 0;
-    for (size_t i = 0; i < c->k_chunks.size(); ++i) {
-        PG_TRY(decompress_dev(ctx, c->k_chunks[i], k_dev + off * hd, total_len * hd));
-        PG_TRY(decompress_dev(ctx, c->v_chunks[i], v_dev + off * hd, total_len * hd));
+    std::vector<const pg_huffman_kv_chunk *> chunks;
+    std::vector<float *> outs;
+    for (size_t i = 0; i < c->k_chunks.size(); ++i) {  // every chunk of both sides in one decoding pass
+        chunks.push_back(c->k_chunks[i]);
+        outs.push_back(k_dev + off * hd);
+        chunks.push_back(c->v_chunks[i]);
+        outs.push_back(v_dev + off * hd);
         off += c->k_chunks[i]->num_tokens;
     }
+    const std::vector<size_t> strides(chunks.size(), total_len * hd);
+    PG_TRY(decompress_many(ctx, chunks.data(), outs.data(), strides.data(), chunks.size()));
     if (hot->len > 0) {
         const size_t width = hot->len * hd * sizeof(float);
         PG_HIP(hipMemcpy2DAsync(k_dev + off * hd, total_len * hd * sizeof(float), hot->k, hot->capacity * hd * sizeof(float), width,

@@ -368,6 +368,17 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
                             const uint16_t *d, const pg_mm_group &grp, size_t total_pairs, const pg_mmdigits &md,
                             float *y, float *part, bool keep_parts = false);  // keep_parts: the K chunks' planes are left in `part` unsummed
 // y[i] = part[0][i] + ... + part[ks - 1][i] (planes `stride` floats apart), in that order.
+// Huffman pieces shared by the coded weights and the coded KV cache (pg_huffman.hip).
+struct pg_huffman_dev_stream {
+    const uint8_t *bytes_dev;   // the stream
+    size_t bytes, symbols;
+    const uint16_t *lut_dev;    // its decode table, pg_huffman_lut_entries() entries
+    size_t out_off;             // where its symbols go in the output
+};
+bool pg_huffman_host_table(const uint64_t *freqs, uint8_t *bit_lengths, uint32_t *codes);
+size_t pg_huffman_lut_entries();
+pg_status pg_huffman_host_lut(const uint8_t *bit_lengths, uint16_t *lut);
+pg_status pg_huffman_decode_device_streams(pg_ctx *ctx, const pg_huffman_dev_stream *streams, size_t count, int8_t *out_dev);
 pg_status pg_launch_sum_parts(pg_ctx *ctx, const float *part, size_t n, int ks, size_t stride, float *y);
 // The many-row Q4_0 product on the f16 matrix cores (pg_gguf_hmm.hip).  The activation rows as two f16 planes
 // [rows][k] (x * 2^e = hi + lo, e per row) and the rows' 2^-e as two f32 factors each.

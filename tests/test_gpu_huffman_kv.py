@@ -164,6 +164,7 @@ def test_reference_cache_tests(ctx, orc):
     (1, 16, 0, 5, (3, 3, 3, 20)),                  # threshold below the chunk size: raised to it
     (2, 2, 6, 6, (13,)),
     (8, 128, 512, 256, (300, 1, 1, 400, 1)),       # a Llama-sized cache: 262144 symbols per chunk
+    (2, 16, 8, 4, (5,) * 60),                      # 74 chunks per side: get_kv decodes 148 streams, each under its own table, in one pass
 ])
 def test_cache_follows_the_oracle(ctx, orc, heads, hd, thr, chunk, appends):
     from peregrine_amd import huffman
