@@ -825,6 +825,44 @@ def section_mxfp4(B, line):
     line["mxfp4_gemv"] = out
     torch.cuda.empty_cache()
 
+    # many rows: the tile kernel on the same instruction (prefill-sized, and the gpt-oss expert shapes at 128 tokens)
+    many = []
+    for m, n_out, k_in in ((1024, 14336, 4096), (1024, 4096, 14336), (128, 5760, 2880), (128, 2880, 2880)):
+        codes = rng.integers(0, 256, size=n_out * k_in // 2, dtype=np.uint8)
+        scales = rng.integers(118, 124, size=n_out * k_in // 32, dtype=np.uint8)
+        hs = []
+        for r in range(4):
+            codes[0] = r
+            h = C.c_void_p()
+            check(lib.pg_mxfp4_upload(B.h, C.c_void_p(codes.ctypes.data), C.c_void_p(scales.ctypes.data), n_out, k_in, C.byref(h)))
+            hs.append(h)
+        x = B.make_acts(m, k_in, 7420)
+        y = torch.empty(m, n_out, device=dev)
+
+        def step():
+            h = hs[B.i % 4]
+            B.i += 1
+            check(lib.pg_gguf_matmul_dev(B.h, ptr(x), m, h, ptr(y)))
+
+        t = B.timed(step, B.dsteps, max(args.warmup, 8))
+        prof, _ = B.profiled(step, B.dsteps)
+        flop = 2.0 * m * n_out * k_in
+        k_ms = prof["mxfp4_tiles"][0]
+        many.append({"workload": f"MXFP4 [{m} x {k_in}] -> [{n_out}]: activation rows as four planes of E4M3 base-32 digits, "
+                                 f"FP4 codes and both sides' block scales inside v_mfma_scale_f32_16x16x128_f8f6f4",
+                     "value": round(flop / (t["ms_per_step"] * 1e-3) / 1e12, 1), "unit": "TFLOP/s", **B.stats(t),
+                     "kernels_ms": {k: round(v[0], 5) for k, v in prof.items()},
+                     "roofline": {"kernel": "mxfp4_tiles_kernel", "bound": "mfma", "achieved": round(flop / (k_ms * 1e-3) / 1e12, 1),
+                                  "peak": 5000.0, "unit": "TFLOP/s", "frac": round(flop / (k_ms * 1e-3) / 1e12 / 5000.0, 4),
+                                  "executed_tflops": round(4 * flop / (k_ms * 1e-3) / 1e12, 1), "traffic": None,
+                                  "avg_launch_ms": round(k_ms, 5),
+                                  "note": "peak = the published dense FP8 rate (an FP4 x FP8 instruction runs at it); "
+                                          "executed = four digit planes per algorithmic multiply-add"}})
+        for h in hs:
+            lib.pg_gguf_free(B.h, h)
+    line["mxfp4_many_rows"] = many
+    torch.cuda.empty_cache()
+
 
 def section_moe(B, line):
     """cfg5: Grok-1-shaped MoE expert FFN, Q8_0 experts."""

@@ -194,16 +194,14 @@ pg_status pg_gguf_matmul_dev(pg_ctx *ctx, const float *x_dev, size_t m,
                              const pg_gguf_tensor *w, float *y_dev);
 
 /* Load-time preparation.  The matrix-core block product reads a tile-major copy of a Q4_0 / Q8_0 / Q4_1 tensor's
- * payload plane (as many bytes again as the payload), and an MXFP4 tensor's products over 16 rows or more (24 for
- * tensors under 2^25 weights) go through a Q8_0 twin of the tensor (34 bytes per block, plus the twin's own
- * tile-major copy of 32: about five times the 17 bytes per block as uploaded).  Left alone, the first product that
- * needs such a copy makes it: a hipMalloc, a launch and a wait inside a call that is otherwise stream-ordered and
- * allocation-free.  pg_gguf_prepare makes now whatever products over up to `max_rows` activation rows of this
- * tensor (alone, in a group, inside a Llama block or as an expert of pg_moe_ffn) will need, as the reference
- * rearranges weights at load (load_transposed_weight, src/models/llama/model.rs:243-257); afterwards those calls
- * neither allocate nor wait, which a caller that captures them in a HIP graph requires.  max_rows < 2 makes
- * nothing (one-row products read the planes as uploaded).  pg_gguf_drop_prepared frees the copies again (it waits
- * for the stream); pg_gguf_device_bytes reports what the tensor holds. */
+ * payload plane (as many bytes again as the payload).  Left alone, the first product that needs the copy makes it:
+ * a hipMalloc, a launch and a wait inside a call that is otherwise stream-ordered and allocation-free.
+ * pg_gguf_prepare makes now whatever products over up to `max_rows` activation rows of this tensor (alone, in a
+ * group, inside a Llama block or as an expert of pg_moe_ffn) will need, as the reference rearranges weights at load
+ * (load_transposed_weight, src/models/llama/model.rs:243-257); afterwards those calls neither allocate nor wait,
+ * which a caller that captures them in a HIP graph requires.  max_rows < 2 makes nothing (one-row products read
+ * the planes as uploaded), and neither does an MXFP4 tensor (all of its products do).  pg_gguf_drop_prepared frees
+ * the copy again (it waits for the stream); pg_gguf_device_bytes reports what the tensor holds. */
 pg_status pg_gguf_prepare(pg_ctx *ctx, const pg_gguf_tensor *w, size_t max_rows);
 pg_status pg_gguf_drop_prepared(pg_ctx *ctx, const pg_gguf_tensor *w);
 pg_status pg_gguf_device_bytes(const pg_gguf_tensor *w, size_t *uploaded, size_t *derived);
@@ -609,6 +607,12 @@ pg_status pg_audit_gguf_hmm(size_t m, size_t n_out, size_t k_in, int q8, int wid
                             size_t *plane_bytes, size_t *qs_end, size_t *qs_bytes, size_t *d_end, size_t *d_bytes);
 pg_status pg_audit_mxfp4_rows(size_t out_dim, size_t in_dim, int row_groups_per_workgroup, int wavefronts,
                               size_t *qs_end, size_t *qs_bytes, size_t *sc_end, size_t *sc_bytes);
+/* The MXFP4 tile kernel and its pre-pass under the plan the launcher makes for m rows on a part of num_cu CUs;
+ * rec_* = the token records between the two; ra, tb, ks report the plan (row groups per wavefront, token groups per
+ * workgroup, runs of K). */
+pg_status pg_audit_mxfp4_tiles(int num_cu, size_t out_dim, size_t in_dim, size_t m, size_t *qs_end, size_t *qs_bytes,
+                               size_t *sc_end, size_t *sc_bytes, size_t *rec_end, size_t *rec_bytes, int *ra, int *tb,
+                               int *ks);
 pg_status pg_audit_probe_read(size_t bytes, int workgroups, int threads, int loads_in_flight, size_t *end,
                               size_t *alloc);
 

@@ -230,6 +230,60 @@ PG_API pg_status pg_audit_mxfp4_rows(size_t out_dim, size_t in_dim, int rg_per_w
     return PG_OK;
 }
 
+// MXFP4 tiles (mxfp4_planes_kernel + mxfp4_tiles_kernel<RA, TB, BD>) with the plan the launcher makes for this shape on a
+// part of `num_cu` CUs: the weights' code and scale planes as above, and the token records the pre-pass writes and the
+// tile kernel reads ([token groups][ncp chunks][PG_MT_RECORD bytes]); rec_end covers both sides.
+PG_API pg_status pg_audit_mxfp4_tiles(int num_cu, size_t out_dim, size_t in_dim, size_t m, size_t *qs_end, size_t *qs_bytes,
+                                      size_t *sc_end, size_t *sc_bytes, size_t *rec_end, size_t *rec_bytes, int *ra, int *tb,
+                                      int *ks) {
+    PG_CHECK_ARG(num_cu > 0 && out_dim > 0 && in_dim >= 32 && in_dim % 32 == 0 && m > 0, "pg_audit_mxfp4_tiles: bad arguments");
+    const int nb = (int)(in_dim / 32), ncp = (int)pg_mx_chunks((size_t)nb), nrg = (int)((out_dim + 15) / 16);
+    const pg_mxfp4_tiles_plan p = pg_mxfp4_tiles_plan_for(num_cu, out_dim, m, ncp);
+    PG_CHECK_ARG(p.ra <= nrg && p.cps % 4 == 0 && p.cps >= 4 && (size_t)p.ks * p.cps >= (size_t)ncp && (size_t)(p.ks - 1) * p.cps < (size_t)ncp,
+                 "pg_audit_mxfp4_tiles: plan ra %d cps %d ks %d does not fit %d row groups / %d chunks", p.ra, p.cps, p.ks, nrg, ncp);
+    span_check qs, sc, rec;
+    // the pre-pass: a wavefront per (token group, pair of blocks)
+    for (size_t tg = 0; tg < p.groups; ++tg)
+        for (int b = 0; b < 4 * ncp; ++b)
+            for (int col = 0; col < 16; col += 15) {
+                for (int sub = 0; sub < 2; ++sub)
+                    for (int j = 0; j < PG_MT_PLANES; ++j) rec.touch(pg_mt_plane_store(tg, ncp, b, sub, col, j), 16);
+                rec.touch(pg_mt_scale_store(tg, ncp, b, col), 4);
+            }
+    // the tiles: every work item, wavefront and chunk of its run; lanes 0 and 63, threads 0 and 511
+    const int units = p.tb * (PG_MT_RECORD / 16), rounds = (units + 64 * PG_MT_NW - 1) / (64 * PG_MT_NW);
+    for (size_t wt = 0; wt < p.n_wt; ++wt)
+        for (int split = 0; split < p.ks; ++split) {
+            const int kc0 = split * p.cps, kc1 = pg_mt_run_end(split, p.cps, ncp);
+            PG_CHECK_ARG(kc1 > kc0 && (kc1 - kc0) % 4 == 0, "pg_audit_mxfp4_tiles: run %d is [%d, %d)", split, kc0, kc1);
+            for (int wave = 0; wave < PG_MT_NW; ++wave) {
+                const int rg0 = pg_mt_first_row_group((int)(wt * PG_MT_NW + wave) * p.ra, p.ra, nrg);
+                PG_CHECK_ARG(rg0 >= 0, "pg_audit_mxfp4_tiles: first row group %d", rg0);
+                for (int r = 0; r < p.ra; ++r)
+                    for (int c = kc0; c < kc1; ++c)
+                        for (int lane = 0; lane < 64; lane += 63) {
+                            qs.touch((((size_t)(rg0 + r) * ncp + c) * 64 + lane) * 16, 16);
+                            sc.touch((((size_t)(rg0 + r) * (ncp / 4) + (c >> 2)) * 64 + lane) * 4, 4);
+                        }
+            }
+            for (size_t tt = 0; tt < p.n_tt; ++tt)
+                for (int i = 0; i < rounds; ++i)
+                    for (int thread = 0; thread < 64 * PG_MT_NW; thread += 64 * PG_MT_NW - 1)
+                        rec.touch(tt * p.tb * ncp * PG_MT_RECORD + pg_mt_unit_offset(thread + i * 64 * PG_MT_NW, units, ncp) +
+                                      (size_t)(kc1 - 1) * PG_MT_RECORD, 16);
+        }
+    if (qs_end) *qs_end = qs.end;
+    if (qs_bytes) *qs_bytes = (size_t)nrg * ncp * 64 * 16;
+    if (sc_end) *sc_end = sc.end;
+    if (sc_bytes) *sc_bytes = (size_t)nrg * (ncp / 4) * 64 * 4;
+    if (rec_end) *rec_end = rec.end;
+    if (rec_bytes) *rec_bytes = p.groups * ncp * (size_t)PG_MT_RECORD;
+    if (ra) *ra = p.ra;
+    if (tb) *tb = p.tb;
+    if (ks) *ks = p.ks;
+    return PG_OK;
+}
+
 // The read-stream probe (probe_read_kernel<U>): `total` 16-byte chunks cut into one slice per workgroup.
 PG_API pg_status pg_audit_probe_read(size_t bytes, int workgroups, int threads, int loads_in_flight, size_t *end, size_t *alloc) {
     PG_CHECK_ARG(bytes >= 16 && workgroups > 0 && threads > 0 && loads_in_flight > 0, "pg_audit_probe_read: bad arguments");

@@ -1028,13 +1028,9 @@ pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const p
     void *ws = nullptr;
     if (w->ggml_type == PG_MXFP4) {
         // The MXFP4 kernel is a decode kernel (three rows per pass over the weights).  From 16 rows on (24 for a
-        // tensor under 2^25 weights, where the passes are short) the tensor's Q8_0 twin takes the matrix-core block
-        // product, which reads the weights once per 32 rows and tile.
-        if (m >= (w->n_out * w->k_in >= ((size_t)1 << 25) ? 16u : 24u) && w->k_in / 32 >= PG_MM_MIN_BLOCKS) {
-            const pg_gguf_tensor *twin = nullptr;
-            PG_TRY(pg_mxfp4_q8_twin(ctx, w, &twin));
-            if (twin) return pg_gguf_matmul_rows(ctx, x_dev, m, twin, y_dev);
-        }
+        // tensor under 2^25 weights, where the passes are short) the tile kernel on the same instruction takes over:
+        // the weights once per 64 rows, the rows as four planes of base-32 digits.
+        if (pg_mxfp4_tiles_takes(w, m)) return pg_launch_mxfp4_tiles(ctx, x_dev, m, w, y_dev);
         return pg_launch_mxfp4_rows(ctx, x_dev, m, w, y_dev);
     }
     int hks = 1;
@@ -1274,24 +1270,18 @@ PG_API void pg_gguf_free(pg_ctx *ctx, pg_gguf_tensor *t) {
     if (t->d) (void)hipFree(t->d);
     if (t->m) (void)hipFree(t->m);
     if (t->qs_tiled) (void)hipFree(t->qs_tiled);
-    if (t->twin) pg_gguf_free(nullptr, t->twin);  // (the stream was drained above)
     delete t;
 }
 
-// Load-time step: every derived copy that a product over up to `max_rows` activation rows would otherwise make
-// on its first call (pg_gguf_ensure_tiled, pg_mxfp4_q8_twin: an allocation, a launch and a wait each) is made now,
+// Load-time step: the derived copy that a product over up to `max_rows` activation rows would otherwise make
+// on its first call (pg_gguf_ensure_tiled: an allocation, a launch and a wait) is made now,
 // so that the `_dev` products, the Llama block and the expert FFN over this tensor neither allocate nor wait --
 // the place of the reference's own load-time rearrangement (load_transposed_weight, src/models/llama/model.rs:243-257).
 PG_API pg_status pg_gguf_prepare(pg_ctx *ctx, const pg_gguf_tensor *w, size_t max_rows) {
     PG_TRY(pg_use(ctx));
     PG_CHECK_ARG(w != nullptr, "pg_gguf_prepare: null tensor");
     if (max_rows < 2 || w->k_in / 32 < PG_MM_MIN_BLOCKS) return PG_OK;  // one row, or a K of a few blocks: the streaming kernels read the planes as uploaded
-    if (w->ggml_type == PG_MXFP4) {
-        if (max_rows < (w->n_out * w->k_in >= ((size_t)1 << 25) ? 16u : 24u)) return PG_OK;
-        const pg_gguf_tensor *twin = nullptr;
-        PG_TRY(pg_mxfp4_q8_twin(ctx, w, &twin));
-        return twin ? pg_gguf_ensure_tiled(ctx, twin) : PG_OK;
-    }
+    if (w->ggml_type == PG_MXFP4) return PG_OK;  // every MXFP4 product reads the planes as uploaded
     if (w->ggml_type == PG_GGML_Q4_0 || w->ggml_type == PG_GGML_Q8_0 || w->ggml_type == PG_GGML_Q4_1)
         return pg_gguf_ensure_tiled(ctx, w);
     return PG_OK;
@@ -1303,8 +1293,6 @@ PG_API pg_status pg_gguf_drop_prepared(pg_ctx *ctx, const pg_gguf_tensor *w) {
     PG_CHECK_ARG(w != nullptr, "pg_gguf_drop_prepared: null tensor");
     PG_HIP(hipStreamSynchronize(ctx->stream));
     if (w->qs_tiled) { (void)hipFree(w->qs_tiled); w->qs_tiled = nullptr; }
-    if (w->twin) { pg_gguf_free(nullptr, w->twin); w->twin = nullptr; }
-    if (w->twin_state > 0) w->twin_state = 0;
     return PG_OK;
 }
 
@@ -1316,7 +1304,7 @@ PG_API pg_status pg_gguf_device_bytes(const pg_gguf_tensor *w, size_t *uploaded,
         return t->qs_tiled ? ((t->n_out + 127) / 128) * pg_tiled_group_bytes((int)(t->k_in / 32), t->ggml_type == PG_GGML_Q8_0) : (size_t)0;
     };
     if (uploaded) *uploaded = blocks * (w->ggml_type == PG_GGML_Q8_0 ? 34 : (w->ggml_type == PG_GGML_Q4_1 ? 20 : (w->ggml_type == PG_MXFP4 ? 17 : 18)));
-    if (derived) *derived = tiled_bytes(w) + (w->twin ? blocks * 34 + tiled_bytes(w->twin) : 0);
+    if (derived) *derived = tiled_bytes(w);
     return PG_OK;
 }
 

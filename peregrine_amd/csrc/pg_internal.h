@@ -76,11 +76,6 @@ struct pg_gguf_tensor {
     mutable uint8_t *qs_tiled;
     int ggml_type;
     size_t n_out, k_in;
-    // MXFP4 only: the same tensor as Q8_0 blocks (i8 = twice the FP4 value, f16 scale 2^(e - 128): exact), made on
-    // the tensor's first product over many rows for the matrix-core block product; twin_state 0 = not tried,
-    // 1 = made, -1 = a block scale is not an f16 (the tensor keeps to its own kernel).
-    mutable pg_gguf_tensor *twin;
-    mutable int twin_state;
 };
 
 // The matrix-core block product carries 16-bit fixed-point activations per block: fine when a
@@ -322,7 +317,6 @@ pg_status pg_launch_x_to_mm_digits(pg_ctx *ctx, const float *x_dev, size_t rows,
 // Q4_1 on the matrix-core route: the product is the Q4_0 product on the same nibbles and scales plus
 // y[t][n] += sum_b (8 d + m)[n][b] * (sum of x over block b of row t); this adds the second term (md.xsum
 // as pg_launch_x_to_mm_digits leaves it for PG_GGML_Q4_1).  k_in up to 32768.
-pg_status pg_mxfp4_q8_twin(pg_ctx *ctx, const pg_gguf_tensor *w, const pg_gguf_tensor **twin);  // *twin null: not representable
 pg_status pg_launch_q41_offset(pg_ctx *ctx, const pg_gguf_tensor *w, const pg_mmdigits &md, size_t rows, float *y);
 // Which activation rows multiply which weights.  Without `counts`: one weight tensor and pairs
 // 0 .. max_count-1.  With `counts`: expert e owns counts[e] pairs, listed (in ascending order) in
@@ -401,6 +395,16 @@ pg_status pg_launch_gguf_hmm_group(pg_ctx *ctx, size_t k_in, const pg_gguf_tenso
 // MXFP4 tensors (pg_mxfp4.hip): qs holds the code bytes in matrix-core fragment order, d the E8M0 scale
 // bytes (four per dword); every product over them runs pg_launch_mxfp4_rows.
 pg_status pg_launch_mxfp4_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w, float *y_dev);
+// Many rows: the tile kernel on the same instruction (activations as three digit planes, weights read once per 64 rows).
+struct pg_mxfp4_tiles_plan {
+    int ra, tb;            // groups of 16 weight rows per wavefront, groups of 16 tokens per workgroup
+    int ks, cps;           // runs of K and chunks per run
+    size_t n_wt, n_tt;     // row tiles, token tiles
+    size_t groups;         // token groups the records are written for (n_tt * tb)
+};
+pg_mxfp4_tiles_plan pg_mxfp4_tiles_plan_for(int num_cu, size_t n_out, size_t m, int ncp);
+bool pg_mxfp4_tiles_takes(const pg_gguf_tensor *w, size_t m);
+pg_status pg_launch_mxfp4_tiles(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w, float *y_dev);
 pg_status pg_gguf_matmul_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w,
                               float *y_dev);
 // `count` such products over the same rows (equal k_in), the rows rewritten as digits once.

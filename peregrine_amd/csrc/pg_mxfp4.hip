@@ -17,8 +17,6 @@
 // j of a row is one column of B with block scale byte 127 + se + 5 j, so the instruction itself applies
 // both block scales and sums over K; the five columns of a row are added at the end.  Three activation
 // rows (15 columns) share one pass over the weights.
-#include <mutex>
-
 #include "pg_internal.h"
 #include "pg_stream_addr.h"
 #include "pg_digits.h"
@@ -35,8 +33,7 @@ constexpr int MX_U = 8;       // chunks (of 4 blocks) per batch of weight loads 
 constexpr int MX_MAX_T = 3;   // activation rows per pass over the weights
 
 inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
-// chunks of 4 blocks per row, rounded up to whole scale dwords (4 chunks)
-inline size_t mx_chunks(size_t nb) { return ((nb + 3) / 4 + 3) & ~(size_t)3; }
+inline size_t mx_chunks(size_t nb) { return pg_mx_chunks(nb); }  // chunks of 4 blocks per row, whole scale dwords
 
 // ---- device layout of a tensor ------------------------------------------------------
 // Fragment-major: for every group of 16 rows and every chunk of 4 blocks (128 k), the 64 lanes' 16 code
@@ -301,90 +298,358 @@ pg_status pg_launch_mxfp4_rows(pg_ctx *ctx, const float *x_dev, size_t m, const 
 #undef PG_MX_LAUNCH
 }
 
-// ---- ABI --------------------------------------------------------------------------------
-// A block is 16 bytes of FP4 (E2M1) codes, byte k = elements 2k (low nibble) and 2k+1, plus
-// one E8M0 scale byte: value = LUT[code] * 2^(scale - 127)   (examples/gpt_oss/moe.rs:5-53).
-// ---- the tensor as Q8_0 blocks (for products over many rows) ---------------------------------
-// Twice an FP4 (E2M1) value is an integer: 0, 1, 2, 3, 4, 6, 8, 12; with the block scale 2^(e - 128) as an f16 the
-// block is a Q8_0 block holding exactly the same numbers.  Planes as split_blocks_kernel lays Q8_0 out:
-// qs8[((n * 2 + h) * nb + b) * 16 + j] = element 16 h + j, d8 in tiles of 8 rows.  *bad is set when a scale has no
-// f16 (e above 143 or, for a block with nonzero codes, below 104).
-__global__ void mxfp4_to_q8_kernel(const uint4 *__restrict__ qs_frag, const uint8_t *__restrict__ sc_frag, int n_out, int nb, int ncp,
-                                   uint8_t *__restrict__ qs8, uint16_t *__restrict__ d8, int *__restrict__ bad) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t n_pad = ((size_t)n_out + 7) / 8 * 8;
-    if (i >= n_pad * nb) return;
-    const size_t n = i / nb, b = i - n * nb;
-    uint16_t *dd = d8 + ((n / 8) * nb + b) * 8 + (n % 8);
-    if (n >= (size_t)n_out) {
-        *dd = 0;
-        return;
-    }
-    const size_t rg = n / 16, c = b / 4;
-    const int lane = (int)(n % 16) + 16 * (int)(b % 4);
-    const uint4 v = qs_frag[(rg * ncp + c) * 64 + lane];
-    const int e = sc_frag[((rg * (ncp / 4) + c / 4) * 64 + lane) * 4 + (c & 3)];
-    const unsigned wv[4] = {v.x, v.y, v.z, v.w};
-    const bool zero = (v.x | v.y | v.z | v.w) == 0u;  // (an all-zero block, or one whose scale byte was 0)
-    const int ex = e - 128;
-    uint16_t bits = 0;
-    if (ex >= -14 && ex <= 15) bits = (uint16_t)((ex + 15) << 10);
-    else if (ex >= -24 && ex < -14) bits = (uint16_t)(1u << (ex + 24));  // subnormal f16: still a power of two
-    else if (!zero || ex > 15) atomicOr(bad, 1);  // (a huge scale times zero codes is not zero where the scale is inf / NaN)
-    *dd = bits;
+namespace {
+
+// ---- many activation rows: tiles on the scaled matrix-core instruction ------------------------
+// From a few dozen rows on the product is matrix-core work, and the instruction still does all of it: the block
+// scales of both sides are applied inside, so there is no rescaling of accumulators and nothing to dequantise.
+// An activation block becomes MT_PLANES balanced base-32 digits per value (20 bits under the block's largest
+// magnitude, |error| <= 2^-20 of it), each plane a B operand whose block scale carries the digit's weight; the
+// planes accumulate into the same tile, so a row costs MT_PLANES instructions per 16 x 16 x 128 tile and no
+// final sum.  A pre-pass writes the planes once, in the operand's own fragment order: per token group of 16
+// and chunk of 128 k one record of MT_RECORD bytes,
+//   [plane][half][64 lanes][16 B]   lane = token % 16 + 16 q holds k = 64 half + 16 q .. + 15 of the chunk
+//   [64 lanes] scale dwords         lane = token % 16 + 16 (block of the chunk), byte j = plane j
+constexpr int MT_PLANES = PG_MT_PLANES;
+constexpr int MT_NW = PG_MT_NW;            // wavefronts per workgroup
+constexpr int MT_FRAG = PG_MT_FRAG;        // bytes of one plane fragment
+constexpr int MT_RECORD = PG_MT_RECORD;    // one token group's planes and scales of a chunk
+constexpr int MT_UNITS = MT_RECORD / 16;   // in 16-byte units
+
+// One thread = 16 consecutive k of one token (half a block).  A wavefront = the 16 tokens of a group x two blocks x
+// their halves, tokens on consecutive lanes: what it writes are whole 256-byte runs of the records, and the
+// 256 bytes it reads of every token row are two full lines.
+__global__ __launch_bounds__(256) void mxfp4_planes_kernel(const float *__restrict__ x, int m, int nb, int ncp, int token_groups,
+                                                           char *__restrict__ bq) {
+    const size_t wv = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;  // (token group, pair of blocks)
+    const int lane = threadIdx.x & 63, col = lane & 15, sub = (lane >> 4) & 1, npair = 2 * ncp;
+    const size_t tg = wv / npair;
+    if (tg >= (size_t)token_groups) return;  // (whole wavefronts)
+    const int b = 2 * (int)(wv % npair) + (lane >> 5);
+    const size_t t = tg * 16 + col;
+    const bool valid = t < (size_t)m && b < nb;
+    float f[16];
 #pragma unroll
-    for (int el = 0; el < 32; ++el) {
-        const unsigned code = (wv[el >> 3] >> (4 * (el & 7))) & 15u;   // element el in nibble el
-        const int mag = (int)((0x0C08060403020100ull >> (8 * (code & 7u))) & 255u);  // 2 x {0, .5, 1, 1.5, 2, 3, 4, 6}
-        qs8[((n * 2 + (el >> 4)) * nb + b) * 16 + (el & 15)] = (uint8_t)(int8_t)((code & 8u) ? -mag : mag);
+    for (int e = 0; e < 4; ++e) {
+        float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (valid) v = reinterpret_cast<const float4 *>(x)[(t * nb + b) * 8 + sub * 4 + e];
+        f[4 * e] = v.x; f[4 * e + 1] = v.y; f[4 * e + 2] = v.z; f[4 * e + 3] = v.w;
+    }
+    float amax = 0.0f;
+    int bad = 0;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        amax = fmaxf(amax, fabsf(f[e]));
+        bad |= f[e] != f[e];
+    }
+    amax = fmaxf(amax, __shfl_xor(amax, 16, 64));  // the block's other half
+    bad |= __shfl_xor(bad, 16, 64);
+    int se = 0;
+    float inv = 1.0f;
+    if (bad || !(amax <= 3.4028234663852886e38f)) {
+        bad = 1;
+        inv = 0.0f;
+    } else if (amax > 0.0f) {
+        int ex;
+        (void)frexpf(amax, &ex);          // amax = f * 2^ex, f in [0.5, 1)
+        se = ex - (5 * MT_PLANES - 1);    // |x| / 2^se < 2^19 <= 16 (1 + 32 + 32^2 + 32^3)
+        if (se < -126) se = -126;
+        inv = ldexpf(1.0f, -se);
+    }
+    // Balanced base-32 digits, top down and all in f32 (every value is a small integer times a power of two, so
+    // each step is exact): n_j = round(r / 32^j), r -= n_j 32^j; |n_j| <= 16.  Small integers keep the
+    // instruction's own sum over k exact, which numbers spread over the format's exponent range do not (a split
+    // into E4M3 values of decreasing size, four significant bits a plane, stopped at 2e-4 of the output's rms
+    // however many planes it was given).
+    int packed[MT_PLANES][4];
+#pragma unroll
+    for (int e4 = 0; e4 < 4; ++e4) {
+        float r[4], d[MT_PLANES][4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float tt = f[4 * e4 + e] * inv;
+            r[e] = (tt != tt) ? 0.0f : rintf(tt);
+        }
+#pragma unroll
+        for (int j = MT_PLANES - 1; j >= 1; --j) {
+            const float down = __builtin_bit_cast(float, (127 - 5 * j) << 23), up = -__builtin_bit_cast(float, (127 + 5 * j) << 23);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                d[j][e] = rintf(r[e] * down);
+                r[e] = fmaf(d[j][e], up, r[e]);
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) d[0][e] = r[e];
+#pragma unroll
+        for (int j = 0; j < MT_PLANES; ++j) {  // integers in [-16, 16] are exact in E4M3
+            int pk = __builtin_amdgcn_cvt_pk_fp8_f32(d[j][0], d[j][1], 0, false);
+            packed[j][e4] = __builtin_amdgcn_cvt_pk_fp8_f32(d[j][2], d[j][3], pk, true);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < MT_PLANES; ++j)
+        *reinterpret_cast<v4i *>(bq + pg_mt_plane_store(tg, ncp, b, sub, col, j)) = v4i{packed[j][0], packed[j][1], packed[j][2], packed[j][3]};
+    if (sub == 0) {  // a NaN / inf block poisons every product it enters: scale byte 255 is NaN
+        unsigned word = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) word |= (unsigned)(j >= MT_PLANES ? 127 : (bad ? 255 : 127 + se + 5 * j)) << (8 * j);
+        *reinterpret_cast<unsigned *>(bq + pg_mt_scale_store(tg, ncp, b, col)) = word;
     }
 }
 
-static std::mutex g_twin_mutex;
+// A workgroup = MT_NW wavefronts x RA groups of 16 weight rows, against TB groups of 16 tokens, over one run of
+// chunks (all of K, or one of `ks` runs whose partial tiles a later launch adds).  The weights go from memory
+// straight into the A operand's registers (each wavefront streams its own rows: two chunks ahead for the widest
+// row tile, a batch of four chunks ahead otherwise); the token records of a chunk are shared through LDS (staged
+// through registers BD chunks ahead, two stages, one barrier per chunk).  Narrow tiles do little arithmetic per
+// chunk, so what they need is requests in flight: the deeper staging is theirs.
+template <int RA, int TB, int BD>
+__global__ __launch_bounds__(64 * MT_NW) void mxfp4_tiles_kernel(const uint8_t *__restrict__ qs_frag, const uint32_t *__restrict__ sc_frag,
+                                                                 const char *__restrict__ bq, float *__restrict__ y, int n_out,
+                                                                 int ncp, int m, int n_tt, int ks, int cps, size_t part_stride,
+                                                                 int items, int per_xcd) {
+    constexpr int STAGE = TB * MT_RECORD, UNITS = TB * MT_UNITS, ROUNDS = (UNITS + 64 * MT_NW - 1) / (64 * MT_NW);
+    constexpr bool RING = RA == 4;  // A two chunks ahead in a ring of two; else the next batch of four chunks
+    static_assert(BD == 1 || BD == 2 || BD == 4, "the staging depth divides the unrolled batch");
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // every XCD (workgroup id % 8) walks its own run of work items, token tiles of one row tile and K run first:
+    // that run's weights stay in the XCD's L2 while its token tiles pass
+    const int item = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per_xcd || item >= items) return;
+    const int tt = item % n_tt, split = (item / n_tt) % ks, wt = item / (n_tt * ks);
+    const int kc0 = split * cps, kc1 = pg_mt_run_end(split, cps, ncp);  // whole batches of four chunks
+    const int nrg = (n_out + 15) / 16;                       // >= RA (the launcher's choice of RA)
+    const int rg_mine = (wt * MT_NW + wave) * RA;            // the row groups whose tiles this wavefront stores
+    const int rg0 = pg_mt_first_row_group(rg_mine, RA, nrg);  // the ones it reads: a spare wavefront repeats the last ones
+    const size_t a_stride = (size_t)ncp * 64;                // v4i per row group
+    const gv4i_ptr qa = (gv4i_ptr)(uintptr_t)qs_frag + (size_t)rg0 * a_stride;
+    const uint32_t *const sa = sc_frag + (size_t)rg0 * (ncp / 4) * 64;
+    // this thread's share of a chunk's records: 16-byte unit u of the TB records, which lie ncp records apart
+    const char *const b_base = bq + (size_t)tt * TB * ncp * MT_RECORD;
+    unsigned b_off[ROUNDS];
+#pragma unroll
+    for (int i = 0; i < ROUNDS; ++i) b_off[i] = pg_mt_unit_offset((int)threadIdx.x + i * 64 * MT_NW, UNITS, ncp);
+    v4i sr[BD][ROUNDS];
+#define PG_MT_FETCH_B(SLOT, C)                                                                                          \
+    do {                                                                                                                \
+        _Pragma("unroll") for (int i = 0; i < ROUNDS; ++i)                                                              \
+            sr[SLOT][i] = *reinterpret_cast<const v4i *>(b_base + b_off[i] + (unsigned)(C) * MT_RECORD);                \
+    } while (0)
+#define PG_MT_PUT_B(STG, SLOT)                                                                                          \
+    do {                                                                                                                \
+        _Pragma("unroll") for (int i = 0; i < ROUNDS; ++i) {                                                            \
+            const int u = (int)threadIdx.x + i * 64 * MT_NW;                                                            \
+            if (u < UNITS) *reinterpret_cast<v4i *>(lds + (STG) * STAGE + u * 16) = sr[SLOT][i];                        \
+        }                                                                                                               \
+    } while (0)
+    v4i a[RING ? 2 : 4][RA], an[RING ? 1 : 4][RA];
+    uint32_t sca[RA], sca_next[RA];
+    auto fetch_a = [&](v4i (&dst)[RA], int c) {
+#pragma unroll
+        for (int r = 0; r < RA; ++r) dst[r] = __builtin_nontemporal_load(qa + (size_t)r * a_stride + (size_t)c * 64 + lane);
+    };
+    v4f acc[RA][TB];
+#pragma unroll
+    for (int r = 0; r < RA; ++r)
+#pragma unroll
+        for (int g = 0; g < TB; ++g) acc[r][g] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
-pg_status pg_mxfp4_q8_twin(pg_ctx *ctx, const pg_gguf_tensor *w, const pg_gguf_tensor **twin) {
-    // One maker at a time; the pointer is published once the planes are complete.
-    std::lock_guard<std::mutex> lock(g_twin_mutex);
-    *twin = nullptr;
-    if (w->twin_state != 0) {
-        *twin = w->twin_state > 0 ? w->twin : nullptr;
-        return PG_OK;
+    PG_MT_FETCH_B(0, kc0);
+    if (BD > 1) PG_MT_FETCH_B(BD > 1 ? 1 : 0, kc0 + 1);
+    if (BD > 2) {
+        PG_MT_FETCH_B(BD > 2 ? 2 : 0, kc0 + 2);
+        PG_MT_FETCH_B(BD > 2 ? 3 : 0, kc0 + 3);
     }
-    const size_t nb = w->k_in / 32, ncp = mx_chunks(nb), n_pad = (w->n_out + 7) / 8 * 8;
-    pg_gguf_tensor *t = new (std::nothrow) pg_gguf_tensor();
-    if (!t) return pg_fail(PG_ENOMEM, "host allocation failed");
-    t->ggml_type = PG_GGML_Q8_0;
-    t->n_out = w->n_out;
-    t->k_in = w->k_in;
-    int *bad_dev = nullptr, bad = 0;
-    hipError_t e = hipMalloc((void **)&t->qs, w->n_out * nb * 32);
-    if (e == hipSuccess) e = hipMalloc((void **)&t->d, n_pad * nb * sizeof(uint16_t));
-    if (e == hipSuccess) e = hipMalloc((void **)&bad_dev, sizeof(int));
-    if (e == hipSuccess) e = hipMemsetAsync(bad_dev, 0, sizeof(int), ctx->stream);  // (set-up, once per tensor: not a capturable path)
-    if (e == hipSuccess) {
-        mxfp4_to_q8_kernel<<<grid_for(n_pad * nb, 256), 256, 0, ctx->stream>>>(reinterpret_cast<const uint4 *>(w->qs),
-                                                                               reinterpret_cast<const uint8_t *>(w->d), (int)w->n_out,
-                                                                               (int)nb, (int)ncp, t->qs, t->d, bad_dev);
-        e = hipGetLastError();
+#pragma unroll
+    for (int u = 0; u < (RING ? 2 : 4); ++u) fetch_a(a[u], kc0 + u);
+#pragma unroll
+    for (int r = 0; r < RA; ++r) sca[r] = sa[((size_t)r * (ncp / 4) + (kc0 >> 2)) * 64 + lane];
+    PG_MT_PUT_B(0, 0);
+    if (kc0 + BD < kc1) PG_MT_FETCH_B(0, kc0 + BD);
+    __syncthreads();
+    for (int cb = kc0; cb < kc1; cb += 4) {
+        const bool more = cb + 4 < kc1;
+        if (more) {
+#pragma unroll
+            for (int r = 0; r < RA; ++r) sca_next[r] = sa[((size_t)r * (ncp / 4) + (cb >> 2) + 1) * 64 + lane];
+            if (!RING) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) fetch_a(an[RING ? 0 : u], cb + 4 + u);
+            }
+        }
+    // One plane of one token group: its two operand halves are read while the previous plane's instructions run.
+    // (The byte selectors of the two scale operands are immediates: chunk within the dword, plane within the dword.)
+#define PG_MT_READ(G, J, B0, B1)                                                                  \
+    do {                                                                                          \
+        B0 = *reinterpret_cast<const v4i *>(st + (G) * MT_RECORD + (J) * MT_FRAG + lane * 16);      \
+        B1 = *reinterpret_cast<const v4i *>(st + (G) * MT_RECORD + (J) * MT_FRAG + 1024 + lane * 16); \
+    } while (0)
+#define PG_MT_MUL(U, G, J, B0, B1)                                                                                          \
+    do {                                                                                                                    \
+        const v8i B = {B0[0], B0[1], B0[2], B0[3], B1[0], B1[1], B1[2], B1[3]};                                             \
+        _Pragma("unroll") for (int r = 0; r < RA; ++r) {                                                                    \
+            const v4i aw = a[RING ? (U) & 1 : (U)][r];                                                                      \
+            const v8i A = {aw[0], aw[1], aw[2], aw[3], 0, 0, 0, 0};                                                         \
+            acc[r][G] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, acc[r][G], 4, 0, (U), (int)sca[r], (J), sbv[G]); \
+            asm volatile("" : "+v"(acc[r][G]));  /* (or the compiler sinks every product to the end of the loop body) */  \
+        }                                                                                                                   \
+    } while (0)
+#define PG_MT_GROUP(U, G)                                                 \
+    do {                                                                  \
+        if ((G) < TB) {                                                   \
+            PG_MT_READ(G, 1, y0, y1);                                     \
+            PG_MT_MUL(U, G, 0, x0, x1);                                   \
+            __builtin_amdgcn_sched_barrier(0);                            \
+            PG_MT_READ(G, 2, x0, x1);                                     \
+            PG_MT_MUL(U, G, 1, y0, y1);                                   \
+            __builtin_amdgcn_sched_barrier(0);                            \
+            PG_MT_READ(G, 3, y0, y1);                                     \
+            PG_MT_MUL(U, G, 2, x0, x1);                                   \
+            __builtin_amdgcn_sched_barrier(0);                            \
+            if ((G) + 1 < TB) PG_MT_READ((G) + 1 < TB ? (G) + 1 : 0, 0, x0, x1); \
+            PG_MT_MUL(U, G, 3, y0, y1);                                   \
+            __builtin_amdgcn_sched_barrier(0);                            \
+        }                                                                 \
+    } while (0)
+#define PG_MT_CHUNK(U)                                                                                   \
+    do {                                                                                                 \
+        const int c = cb + (U);                                                                          \
+        const char *st = lds + ((U) & 1) * STAGE;                                                        \
+        int sbv[TB];                                                                                     \
+        _Pragma("unroll") for (int g = 0; g < TB; ++g)                                                   \
+            sbv[g] = *reinterpret_cast<const int *>(st + g * MT_RECORD + MT_PLANES * MT_FRAG + lane * 4); \
+        v4i x0, x1, y0, y1;                                                                              \
+        PG_MT_READ(0, 0, x0, x1);                                                                        \
+        __builtin_amdgcn_sched_barrier(0);                                                               \
+        PG_MT_GROUP(U, 0);                                                                               \
+        PG_MT_GROUP(U, 1);                                                                               \
+        PG_MT_GROUP(U, 2);                                                                               \
+        PG_MT_GROUP(U, 3);                                                                               \
+        if (c + 1 < kc1) {                                                                               \
+            PG_MT_PUT_B(((U) + 1) & 1, ((U) + 1) % BD);                                                  \
+            if (c + 1 + BD < kc1) PG_MT_FETCH_B(((U) + 1) % BD, c + 1 + BD);                             \
+        }                                                                                                \
+        if (RING && c + 2 < kc1) fetch_a(a[RING ? (U) & 1 : 0], c + 2);                                  \
+        __syncthreads();                                                                                 \
+    } while (0)
+        static_assert(MT_PLANES == 4 && TB <= 4, "the plane steps are written out");
+        PG_MT_CHUNK(0);
+        PG_MT_CHUNK(1);
+        PG_MT_CHUNK(2);
+        PG_MT_CHUNK(3);
+#undef PG_MT_CHUNK
+#undef PG_MT_GROUP
+#undef PG_MT_MUL
+#undef PG_MT_READ
+        if (more) {
+#pragma unroll
+            for (int r = 0; r < RA; ++r) sca[r] = sca_next[r];
+            if (!RING) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+#pragma unroll
+                    for (int r = 0; r < RA; ++r) a[RING ? 0 : u][r] = an[RING ? 0 : u][r];
+            }
+        }
     }
-    if (e == hipSuccess) e = hipMemcpyAsync(&bad, bad_dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
-    if (bad_dev) (void)hipFree(bad_dev);
-    if (e != hipSuccess) {
-        pg_gguf_free(nullptr, t);
-        return pg_fail(e == hipErrorOutOfMemory ? PG_ENOMEM : PG_EDEVICE, "mxfp4 Q8_0 twin: %s", hipGetErrorString(e));
+#undef PG_MT_FETCH_B
+#undef PG_MT_PUT_B
+    // D: lane holds token lane % 16 of its group, weight rows 4 (lane / 16) .. + 3 of the row group
+    float *const out = y + (size_t)split * part_stride;
+#pragma unroll
+    for (int r = 0; r < RA; ++r) {
+        if (rg_mine != rg0 && rg0 + r < rg_mine) continue;   // rows a spare wavefront only repeated
+        if (rg_mine >= nrg) continue;
+        const size_t row = (size_t)(rg0 + r) * 16 + 4 * (lane >> 4);
+#pragma unroll
+        for (int g = 0; g < TB; ++g) {
+            const size_t token = ((size_t)tt * TB + g) * 16 + (lane & 15);
+            if (token >= (size_t)m) continue;
+            float *o = out + token * n_out + row;
+            if (row + 3 < (size_t)n_out && (n_out & 3) == 0) {
+                *reinterpret_cast<v4f *>(o) = acc[r][g];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (row + i < (size_t)n_out) o[i] = acc[r][g][i];
+            }
+        }
     }
-    if (bad) {
-        pg_gguf_free(nullptr, t);
-        w->twin_state = -1;
-        return PG_OK;
-    }
-    w->twin = t;
-    w->twin_state = 1;
-    *twin = t;
+}
+
+using mt_plan = pg_mxfp4_tiles_plan;
+
+template <int RA, int TB, int BD>
+pg_status launch_tiles(pg_ctx *ctx, const pg_gguf_tensor *w, const char *bq, float *y, size_t m, int ncp, const mt_plan &p) {
+    const size_t lds = 2 * (size_t)TB * MT_RECORD;
+    auto kern = mxfp4_tiles_kernel<RA, TB, BD>;
+    PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
+    const size_t items = p.n_wt * p.n_tt * p.ks, per_xcd = (items + 7) / 8;
+    return pg_launch(ctx, "mxfp4_tiles", kern, dim3((unsigned)(8 * per_xcd)), dim3(64 * MT_NW), lds, (const uint8_t *)w->qs,
+                     reinterpret_cast<const uint32_t *>(w->d), bq, y, (int)w->n_out, ncp, (int)m, (int)p.n_tt, p.ks, p.cps,
+                     m * w->n_out, (int)items, (int)per_xcd);
+}
+
+}  // namespace
+
+// The tile shape and K split for m rows of an [n_out, 32 nb] tensor: the widest row tile that still gives every CU a
+// workgroup (and no wider than the tensor); with the narrowest still short of that, K in runs of at least 8 chunks.
+pg_mxfp4_tiles_plan pg_mxfp4_tiles_plan_for(int num_cu, size_t n_out, size_t m, int ncp) {
+    pg_mxfp4_tiles_plan p;
+    p.tb = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
+    p.n_tt = (m + 16 * p.tb - 1) / (16 * p.tb);
+    p.groups = p.n_tt * p.tb;
+    const size_t nrg = (n_out + 15) / 16;
+    p.ra = 4;
+    while (p.ra > 1 && ((size_t)p.ra > nrg || (nrg + MT_NW * p.ra - 1) / (MT_NW * p.ra) * p.n_tt < (size_t)num_cu)) p.ra >>= 1;
+    p.n_wt = (nrg + MT_NW * p.ra - 1) / (MT_NW * p.ra);
+    const size_t tiles = p.n_wt * p.n_tt;
+    p.ks = 1;
+    if (tiles < (size_t)num_cu) p.ks = (int)std::min<size_t>(std::min<size_t>((size_t)num_cu / tiles, (size_t)ncp / 8), 16);
+    if (p.ks < 1) p.ks = 1;
+    p.cps = ((ncp / 4 + p.ks - 1) / p.ks) * 4;       // chunks per run: whole batches of four
+    p.ks = (ncp + p.cps - 1) / p.cps;                // (no empty run)
+    return p;
+}
+
+// Whether the tile kernel takes `m` activation rows of this tensor (otherwise the decode kernel's passes of three
+// rows): from 16 rows, or 24 for a tensor under 2^25 weights, whose passes are short.
+bool pg_mxfp4_tiles_takes(const pg_gguf_tensor *w, size_t m) {
+    return w->ggml_type == PG_MXFP4 && m >= (w->n_out * w->k_in >= ((size_t)1 << 25) ? 16u : 24u) && m < ((size_t)1 << 27) &&
+           w->n_out < ((size_t)1 << 27);
+}
+
+// y[m, n_out] = x[m, k_in] . W^T for an MXFP4 tensor over many rows; x 16-byte aligned.
+pg_status pg_launch_mxfp4_tiles(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w, float *y_dev) {
+    const int nb = (int)(w->k_in / 32), ncp = (int)mx_chunks((size_t)nb);
+    const mt_plan p = pg_mxfp4_tiles_plan_for(ctx->num_cu, w->n_out, m, ncp);
+    PG_CHECK_ARG(p.n_wt * p.n_tt * p.ks < ((size_t)1 << 28), "mxfp4: %zu x %zu tiles", p.n_wt, p.n_tt);
+    void *ws = nullptr;
+    const size_t sz_b = pg_round_up(p.groups * ncp * (size_t)MT_RECORD, 256);
+    const size_t sz_part = p.ks > 1 ? (size_t)p.ks * m * w->n_out * sizeof(float) : 0;
+    PG_TRY(pg_workspace(ctx, sz_b + sz_part, &ws));
+    char *bq = static_cast<char *>(ws);
+    float *part = p.ks > 1 ? reinterpret_cast<float *>(bq + sz_b) : y_dev;
+    const size_t threads = p.groups * 2 * (size_t)ncp * 64;  // a wavefront per token group and pair of blocks
+    PG_CHECK_ARG((threads + 255) / 256 < ((size_t)1 << 31), "mxfp4: %zu rows x %zu is too much for one pre-pass", m, w->k_in);
+    PG_TRY(pg_launch(ctx, "mxfp4_planes", mxfp4_planes_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, x_dev, (int)m, nb,
+                     ncp, (int)p.groups, bq));
+    // the staging depth: the less arithmetic a chunk holds, the more chunks ahead
+#define PG_MT_LAUNCH(RA_, BD1, BD2, BD4) \
+    (p.tb == 1 ? launch_tiles<RA_, 1, BD1>(ctx, w, bq, part, m, ncp, p) \
+     : p.tb == 2 ? launch_tiles<RA_, 2, BD2>(ctx, w, bq, part, m, ncp, p) \
+                 : launch_tiles<RA_, 4, BD4>(ctx, w, bq, part, m, ncp, p))
+    PG_TRY(p.ra == 4 ? PG_MT_LAUNCH(4, 4, 2, 1) : (p.ra == 2 ? PG_MT_LAUNCH(2, 4, 4, 2) : PG_MT_LAUNCH(1, 4, 4, 4)));
+#undef PG_MT_LAUNCH
+    if (p.ks > 1) PG_TRY(pg_launch_sum_parts(ctx, part, m * w->n_out, p.ks, m * w->n_out, y_dev));
     return PG_OK;
 }
 
+// ---- ABI --------------------------------------------------------------------------------
+// A block is 16 bytes of FP4 (E2M1) codes, byte k = elements 2k (low nibble) and 2k+1, plus
+// one E8M0 scale byte: value = LUT[code] * 2^(scale - 127)   (examples/gpt_oss/moe.rs:5-53).
 PG_API pg_status pg_mxfp4_upload(pg_ctx *ctx, const uint8_t *blocks, const uint8_t *scales, size_t out_dim,
                                  size_t in_dim, pg_gguf_tensor **out) {
     PG_TRY(pg_use(ctx));

@@ -71,6 +71,31 @@ PG_HD size_t pg_gskinny_scale_offset(int tile, int nb, int unit, int lane) { ret
 PG_HD int pg_mx_chunk(int c, int ncp) { return c < ncp ? c : ncp - 1; }
 PG_HD int pg_mx_scale_word(int c, int ncp) { return (c < ncp ? c : ncp - 4) >> 2; }
 
+// ---- MXFP4 over many rows (mxfp4_planes_kernel writes the token records, mxfp4_tiles_kernel reads them and the weights)
+// A record = one token group of 16 and one chunk of 128 k: PG_MT_PLANES operand fragments of 2 KiB, then 64 scale dwords.
+constexpr int PG_MT_PLANES = 4, PG_MT_FRAG = 2048, PG_MT_RECORD = PG_MT_PLANES * PG_MT_FRAG + 256, PG_MT_NW = 8;
+// chunks a row of nb blocks is padded to: whole scale dwords (4 chunks of 4 blocks)
+PG_HD size_t pg_mx_chunks(size_t nb) { return ((nb + 3) / 4 + 3) & ~(size_t)3; }
+// first of the `ra` row groups a wavefront reads, from the first one it owns: past the tensor's end it repeats the last ones
+PG_HD int pg_mt_first_row_group(int rg_mine, int ra, int nrg) { return rg_mine + ra <= nrg ? rg_mine : nrg - ra; }
+// the run of chunks a work item covers: `split` of runs of `cps` chunks
+PG_HD int pg_mt_run_end(int split, int cps, int ncp) { return split * cps + cps < ncp ? split * cps + cps : ncp; }
+// byte offset, from the token tile's first record of chunk 0, of 16-byte unit u of the tile's records of one chunk
+// (the tile's records of a chunk lie ncp records apart; spare threads repeat the last unit)
+PG_HD unsigned pg_mt_unit_offset(int u, int units, int ncp) {
+    u = u < units ? u : units - 1;
+    return (unsigned)(u / (PG_MT_RECORD / 16)) * (unsigned)ncp * PG_MT_RECORD + (unsigned)(u % (PG_MT_RECORD / 16)) * 16;
+}
+// byte offset of the 16 bytes of plane j that hold k = 32 (b % 4) + 16 sub .. + 15 of chunk b / 4 for token `col` of group tg
+PG_HD size_t pg_mt_plane_store(size_t tg, int ncp, int b, int sub, int col, int j) {
+    const int k0 = 32 * (b & 3) + 16 * sub, half = k0 >> 6, q = (k0 & 63) >> 4;
+    return (tg * ncp + (size_t)(b >> 2)) * PG_MT_RECORD + (size_t)j * PG_MT_FRAG + half * 1024 + (col + 16 * q) * 16;
+}
+// byte offset of the scale dword of block b for token `col` of group tg
+PG_HD size_t pg_mt_scale_store(size_t tg, int ncp, int b, int col) {
+    return (tg * ncp + (size_t)(b >> 2)) * PG_MT_RECORD + (size_t)PG_MT_PLANES * PG_MT_FRAG + (size_t)(col + 16 * (b & 3)) * 4;
+}
+
 // ---- many rows on the f16 matrix cores (gguf_hmm_kernel): per stage of two blocks a wavefront fills its share
 // of the two activation planes, of the packed weights and of their scales
 // activation or weight row a fill lane fetches: rows past the end repeat the last (their outputs are never stored)

@@ -128,6 +128,23 @@ def test_mxfp4_rows_loads_stay_inside_the_fragment_planes():
             _inside(v, f"mxfp4_rows n={n} k={k} RG={rg} NW={nw}")
 
 
+def test_mxfp4_tiles_stay_inside_the_planes_and_the_token_records():
+    """mxfp4_planes_kernel + mxfp4_tiles_kernel under the launcher's own plan, for every row-tile width (1, 2, 4 groups
+    of 16 rows per wavefront), token-tile width (1, 2, 4 groups of 16 tokens) and K split it can pick."""
+    seen = set()
+    for num_cu in (256, 64):
+        for k, n, m in itertools.product([32, 96, 512, 2880, 4096, 14336], [1, 15, 16, 17, 100, 2880, 8192, 70000], [16, 17, 32, 33, 100, 640]):
+            v = [C.c_size_t() for _ in range(6)]
+            plan = [C.c_int() for _ in range(3)]
+            check(lib.pg_audit_mxfp4_tiles(num_cu, n, k, m, *[C.byref(x) for x in v], *[C.byref(x) for x in plan]))
+            what = f"mxfp4_tiles n={n} k={k} m={m} cus={num_cu} plan={[x.value for x in plan]}"
+            _inside(v[:4], what)
+            assert v[4].value == v[5].value, f"{what}: the records are used up to byte {v[4].value} of {v[5].value}"
+            seen.add((plan[0].value, plan[1].value, min(plan[2].value, 2)))
+    assert {(ra, tb) for ra, tb, _ in seen} == {(ra, tb) for ra in (1, 2, 4) for tb in (1, 2, 4)}, seen
+    assert {ks for _, _, ks in seen} == {1, 2}
+
+
 def test_probe_read_covers_its_buffer_exactly_once_in_bounds():
     for nbytes in (1 << 20, 33103872, 58851328, (1 << 20) + 16):
         for wgs, threads, nl in itertools.product((256, 2048, 4096), (256, 1024), (4, 16)):
