@@ -90,6 +90,8 @@ extern "C" {
     pub fn pg_mxfp4_expert_free(ctx: *mut pg_ctx, expert: *mut pg_mxfp4_expert);
     pub fn pg_mxfp4_expert_forward(ctx: *mut pg_ctx, expert: *const pg_mxfp4_expert, x: *const f32, m: usize, out: *mut f32) -> pg_status;
     pub fn pg_mxfp4_expert_forward_dev(ctx: *mut pg_ctx, expert: *const pg_mxfp4_expert, x_dev: *const f32, m: usize, scratch_dev: *mut f32, out_dev: *mut f32) -> pg_status;
+    pub fn pg_mxfp4_moe_ffn_routed(ctx: *mut pg_ctx, x: *const f32, T: usize, expert_idx: *const i32, weight: *const f32, top_k: usize, experts: *const *const pg_mxfp4_expert, E: usize, out: *mut f32) -> pg_status;
+    pub fn pg_mxfp4_moe_ffn_routed_dev(ctx: *mut pg_ctx, x_dev: *const f32, T: usize, expert_idx_dev: *const i32, weight_dev: *const f32, top_k: usize, experts: *const *const pg_mxfp4_expert, E: usize, out_dev: *mut f32) -> pg_status;
     pub fn pg_gguf_file_parse(data: *const c_void, len: usize, out: *mut *mut pg_gguf_file) -> pg_status;
     pub fn pg_gguf_file_open(path: *const c_char, out: *mut *mut pg_gguf_file) -> pg_status;
     pub fn pg_gguf_file_close(f: *mut pg_gguf_file);

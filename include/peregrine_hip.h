@@ -237,6 +237,17 @@ pg_status pg_mxfp4_expert_forward(pg_ctx *ctx, const pg_mxfp4_expert *expert, co
 /* scratch_dev: m * 3 * intermediate floats, 16-byte aligned. */
 pg_status pg_mxfp4_expert_forward_dev(pg_ctx *ctx, const pg_mxfp4_expert *expert, const float *x_dev, size_t m,
                                       float *scratch_dev, float *out_dev);
+/* MoELayer::forward after its router, over MXFP4 experts  examples/gpt_oss/moe.rs:286-352 (the router itself:
+ * logits = x . gate + bias, top-k, softmax over the k, :289-330, is the caller's): x, out [T, hidden];
+ * expert_idx, weight [T, top_k]; out[t] = sum_k weight[t, k] * experts[expert_idx[t, k]].forward(x[t]), the terms
+ * added in k order.  All experts of one launch share hidden, intermediate, alpha and clamp.  The reference calls an
+ * expert once per (token, k); here the tokens of each expert are gathered and every product is one launch over all
+ * experts.  An index outside 0..E-1 or repeated within a token contributes nothing (its weight counts as 0). */
+pg_status pg_mxfp4_moe_ffn_routed(pg_ctx *ctx, const float *x, size_t T, const int32_t *expert_idx, const float *weight,
+                                  size_t top_k, const pg_mxfp4_expert *const *experts, size_t E, float *out);
+pg_status pg_mxfp4_moe_ffn_routed_dev(pg_ctx *ctx, const float *x_dev, size_t T, const int32_t *expert_idx_dev,
+                                      const float *weight_dev, size_t top_k, const pg_mxfp4_expert *const *experts,
+                                      size_t E, float *out_dev);
 
 /* ---- GGUF container (gguf::GgufFile, src/gguf.rs:403-561) ---------------------
  * Parsing needs no device.  A malformed or truncated file is PG_EINVAL (the reference

@@ -81,6 +81,33 @@ ORC_API int orc_mxfp4_expert_forward(const float *x, size_t hidden, size_t inter
     return 0;
 }
 
+/* MoELayer::forward after its router, MXFP4 experts          reference: examples/gpt_oss/moe.rs:286-352
+ *   out[t] = sum over the token's k experts, in the order given, of weight * expert.forward(x[t]) (one multiply, one
+ *   add per term, from 0.0).  Expert e's operands are entry e of the six arrays.  Parity status: a composition of
+ *   orc_mxfp4_expert_forward (pinned above); the accumulation is pinned by recomputing it in float32 NumPy from
+ *   that function's own outputs, bit for bit, on routings where the order of the terms matters. */
+ORC_API int orc_mxfp4_moe_routed(const float *x, size_t T, size_t hidden, size_t intermediate, float alpha, float clamp, size_t E,
+                                 size_t top_k, const int32_t *idx, const float *weight, const uint8_t *const *mlp1_blocks,
+                                 const uint8_t *const *mlp1_scales, const uint8_t *const *mlp2_blocks, const uint8_t *const *mlp2_scales,
+                                 const float *const *mlp1_bias, const float *const *mlp2_bias, float *out) {
+    float *y = (float *)malloc(hidden * sizeof(float));
+    if (!y) return -1;
+    int rc = 0;
+    for (size_t t = 0; t < T && rc == 0; ++t) {
+        for (size_t i = 0; i < hidden; ++i) out[t * hidden + i] = 0.0f;
+        for (size_t k = 0; k < top_k; ++k) {
+            const int32_t e = idx[t * top_k + k];
+            if (e < 0 || (size_t)e >= E) { rc = -3; break; }
+            rc = orc_mxfp4_expert_forward(x + t * hidden, hidden, intermediate, alpha, clamp, mlp1_blocks[e], mlp1_scales[e],
+                                          mlp2_blocks[e], mlp2_scales[e], mlp1_bias[e], mlp2_bias[e], y);
+            if (rc) break;
+            for (size_t i = 0; i < hidden; ++i) out[t * hidden + i] += weight[t * top_k + k] * y[i];
+        }
+    }
+    free(y);
+    return rc;
+}
+
 /* ---------------------------------------------------------------------------------------
  * Canonical Huffman over i8 symbols.  Parity status: orc_huffman_table is pinned by hand-
  * worked small cases that fix the tie-breaking (stable sort, leaf before internal node), by

@@ -153,6 +153,8 @@ SIGNATURES = {
     "pg_mxfp4_expert_free": [_vp, _vp],
     "pg_mxfp4_expert_forward": [_vp, _vp, _vp, _sz, _vp],
     "pg_mxfp4_expert_forward_dev": [_vp, _vp, _vp, _sz, _vp, _vp],
+    "pg_mxfp4_moe_ffn_routed": [_vp, _vp, _sz, _vp, _vp, _sz, _pp, _sz, _vp],
+    "pg_mxfp4_moe_ffn_routed_dev": [_vp, _vp, _sz, _vp, _vp, _sz, _pp, _sz, _vp],
     "pg_rmsnorm": [_vp, _vp, _sz, _sz, _vp, C.c_float, _vp],
     "pg_rmsnorm_dev": [_vp, _vp, _sz, _sz, _vp, C.c_float, _vp],
     "pg_rope_create": [_vp, _sz, _sz, C.c_float, _pp],

@@ -396,6 +396,11 @@ pg_status pg_launch_gguf_hmm_group(pg_ctx *ctx, size_t k_in, const pg_gguf_tenso
 // bytes (four per dword); every product over them runs pg_launch_mxfp4_rows.
 pg_status pg_launch_mxfp4_rows(pg_ctx *ctx, const float *x_dev, size_t m, const pg_gguf_tensor *w, float *y_dev);
 // Many rows: the tile kernel on the same instruction (activations as three digit planes, weights read once per 64 rows).
+// MoE pieces shared by the block-tensor experts (pg_moe.hip) and the MXFP4 experts (pg_mxfp4.hip).
+constexpr int PG_MOE_MAX_EXPERTS = 256;
+pg_status pg_moe_cached_table(pg_ctx *ctx, const void *const *host_tab, size_t n, const void ***dev_tab);
+pg_status pg_launch_moe_routing(pg_ctx *ctx, const float *router_logits_dev, const int *idx_dev, const float *weight_dev, size_t T,
+                                size_t E, size_t top_k, int *topk_idx, float *topk_p, int *lists, int *counts);
 struct pg_mxfp4_tiles_plan {
     int ra, tb;            // groups of 16 weight rows per wavefront, groups of 16 tokens per workgroup
     int ks, cps;           // runs of K and chunks per run

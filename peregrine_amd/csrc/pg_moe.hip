@@ -14,7 +14,7 @@ namespace {
 
 inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
 
-constexpr int MAX_EXPERTS = 256;
+constexpr int MAX_EXPERTS = PG_MOE_MAX_EXPERTS;
 
 // One thread per token.
 __global__ void route_topk_kernel(const float *__restrict__ logits, int T, int E, int top_k,
@@ -119,6 +119,52 @@ __global__ void combine_kernel(const float *__restrict__ yb, const float *__rest
 
 }  // namespace
 
+// A table of device pointers (an expert set's planes) in a device buffer kept with the context, one per distinct
+// table; uploaded (blocking: the source is the caller's stack frame) only on a table's first use.
+pg_status pg_moe_cached_table(pg_ctx *ctx, const void *const *host_tab, size_t n, const void ***dev_tab) {
+    for (size_t i = 0; i < ctx->moe_tabs.size(); ++i) {
+        auto &t = ctx->moe_tabs[i];
+        if (t.host.size() == n && memcmp(t.host.data(), host_tab, n * sizeof(void *)) == 0) {
+            *dev_tab = static_cast<const void **>(t.dev);
+            if (i + 1 != ctx->moe_tabs.size()) std::rotate(ctx->moe_tabs.begin() + i, ctx->moe_tabs.begin() + i + 1, ctx->moe_tabs.end());  // most recent last
+            return PG_OK;
+        }
+    }
+    // Least recently used out first.  A layer has two sets (row-major planes for one token, tile-major ones for
+    // more), and a model alternates its layers: 512 sets hold both for 256 layers (the reference's Grok-1 has 64,
+    // examples/grok1/model.rs:35), so a decode loop after a prefill misses on no layer.
+    if (ctx->moe_tabs.size() >= 512) {  // a bounded cache: drop a set once nothing can still read it
+        PG_HIP(hipStreamSynchronize(ctx->stream));
+        (void)hipFree(ctx->moe_tabs.front().dev);
+        ctx->moe_tabs.erase(ctx->moe_tabs.begin());
+    }
+    void *dev = nullptr;
+    PG_HIP(hipMalloc(&dev, n * sizeof(void *)));
+    const hipError_t ce = hipMemcpy(dev, host_tab, n * sizeof(void *), hipMemcpyHostToDevice);
+    if (ce != hipSuccess) {
+        (void)hipFree(dev);
+        return pg_fail(PG_EDEVICE, "uploading an expert table: %s", hipGetErrorString(ce));
+    }
+    ctx->moe_tabs.push_back({std::vector<const void *>(host_tab, host_tab + n), dev});
+    *dev_tab = static_cast<const void **>(dev);
+    return PG_OK;
+}
+
+// The routing of T tokens as the expert products want it: topk_idx / topk_p [T * top_k] (from the router's logits,
+// grok1's softmax -> top-k, or a copy of the caller's own choice with out-of-range and repeated experts made
+// harmless), and per expert the (token, k) pairs routed to it in ascending order (lists [E][T], counts [E]).
+pg_status pg_launch_moe_routing(pg_ctx *ctx, const float *router_logits_dev, const int *idx_dev, const float *weight_dev, size_t T,
+                                size_t E, size_t top_k, int *topk_idx, float *topk_p, int *lists, int *counts) {
+    if (router_logits_dev)
+        PG_TRY(pg_launch(ctx, "moe_route_topk", route_topk_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
+                         router_logits_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
+    else
+        PG_TRY(pg_launch(ctx, "moe_copy_routing", copy_routing_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
+                         idx_dev, weight_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
+    return pg_launch(ctx, "moe_expert_lists", expert_lists_kernel, dim3((unsigned)E), dim3(64), 0, (const int *)topk_idx,
+                     (int)(T * top_k), (int)T, lists, counts);
+}
+
 // The expert FFN behind both entry points: the routing comes from `router_logits_dev` (grok1's softmax -> top-k) or,
 // when that is null, from `idx_dev` / `weight_dev` as the caller's gate made them.
 static pg_status moe_ffn_core(pg_ctx *ctx, const float *x_dev, size_t T, const float *router_logits_dev,
@@ -208,42 +254,9 @@ static pg_status moe_ffn_core(pg_ctx *ctx, const float *x_dev, size_t T, const f
         host_tab[4 * E + e] = down_stream ? down[e]->qs : down[e]->qs_tiled; host_tab[5 * E + e] = down[e]->d;
     }
     const void **tab = nullptr;
-    for (size_t i = 0; i < ctx->moe_tabs.size(); ++i) {
-        auto &t = ctx->moe_tabs[i];
-        if (t.host.size() == 6 * E && memcmp(t.host.data(), host_tab, 6 * E * sizeof(void *)) == 0) {
-            tab = static_cast<const void **>(t.dev);
-            if (i + 1 != ctx->moe_tabs.size()) std::rotate(ctx->moe_tabs.begin() + i, ctx->moe_tabs.begin() + i + 1, ctx->moe_tabs.end());  // most recent last
-            break;
-        }
-    }
-    if (!tab) {
-        // Least recently used out first.  A layer has two sets (row-major planes for one token, tile-major ones for
-        // more), and a model alternates its layers: 512 sets hold both for 256 layers (the reference's Grok-1 has 64,
-        // examples/grok1/model.rs:35), so a decode loop after a prefill misses on no layer.
-        if (ctx->moe_tabs.size() >= 512) {  // a bounded cache: drop a set once nothing can still read it
-            PG_HIP(hipStreamSynchronize(ctx->stream));
-            (void)hipFree(ctx->moe_tabs.front().dev);
-            ctx->moe_tabs.erase(ctx->moe_tabs.begin());
-        }
-        void *dev = nullptr;
-        PG_HIP(hipMalloc(&dev, 6 * E * sizeof(void *)));
-        const hipError_t ce = hipMemcpy(dev, host_tab, 6 * E * sizeof(void *), hipMemcpyHostToDevice);
-        if (ce != hipSuccess) {
-            (void)hipFree(dev);
-            return pg_fail(PG_EDEVICE, "pg_moe_ffn: uploading the expert table: %s", hipGetErrorString(ce));
-        }
-        ctx->moe_tabs.push_back({std::vector<const void *>(host_tab, host_tab + 6 * E), dev});
-        tab = static_cast<const void **>(dev);
-    }
+    PG_TRY(pg_moe_cached_table(ctx, host_tab, 6 * E, &tab));
 
-    if (router_logits_dev)
-        PG_TRY(pg_launch(ctx, "moe_route_topk", route_topk_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
-                         router_logits_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
-    else
-        PG_TRY(pg_launch(ctx, "moe_copy_routing", copy_routing_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
-                         idx_dev, weight_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
-    PG_TRY(pg_launch(ctx, "moe_expert_lists", expert_lists_kernel, dim3((unsigned)E), dim3(64), 0, topk_idx, (int)P, (int)T,
-                     lists, counts));
+    PG_TRY(pg_launch_moe_routing(ctx, router_logits_dev, idx_dev, weight_dev, T, E, top_k, topk_idx, topk_p, lists, counts));
     auto table = [&](int which) { return reinterpret_cast<const uint8_t *const *>(tab + which * E); };
     auto dtable = [&](int which) { return reinterpret_cast<const uint16_t *const *>(tab + which * E); };
     // Each token reaches an expert at most once, so an expert owns at most T pairs.

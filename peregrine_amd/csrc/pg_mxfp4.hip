@@ -316,18 +316,56 @@ constexpr int MT_FRAG = PG_MT_FRAG;        // bytes of one plane fragment
 constexpr int MT_RECORD = PG_MT_RECORD;    // one token group's planes and scales of a chunk
 constexpr int MT_UNITS = MT_RECORD / 16;   // in 16-byte units
 
+// Experts' token lists, for the grouped products of an MoE layer: the token tiles (TB groups of 16 slots) of all
+// experts follow one another, expert e's from tile goff[e]; slot i of an expert holds pair lists[e * stride + i].
+struct mt_gather {
+    const int *lists, *counts, *goff;  // [E][stride], [E], [E + 1]
+    int stride, experts, tb, div;      // row of the source matrix = pair / div
+};
+// the expert whose tiles include token tile gt (gt < goff[experts])
+__device__ __forceinline__ int mt_expert_of(const mt_gather &g, int gt) {
+    int lo = 0, hi = g.experts;
+    while (lo + 1 < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (g.goff[mid] <= gt) lo = mid;
+        else hi = mid;
+    }
+    return lo;
+}
+
+// First token tile of every expert: goff[e] = sum over e' < e of ceil(counts[e'] / (16 tb)); goff[experts] = all.
+__global__ __launch_bounds__(64) void mxfp4_tile_offsets_kernel(const int *__restrict__ counts, int experts, int tb, int *__restrict__ goff) {
+    if (threadIdx.x != 0) return;
+    int run = 0;
+    for (int e = 0; e < experts; ++e) {
+        goff[e] = run;
+        run += (counts[e] + 16 * tb - 1) / (16 * tb);
+    }
+    goff[experts] = run;
+}
+
 // One thread = 16 consecutive k of one token (half a block).  A wavefront = the 16 tokens of a group x two blocks x
 // their halves, tokens on consecutive lanes: what it writes are whole 256-byte runs of the records, and the
 // 256 bytes it reads of every token row are two full lines.
+// GATHER: the token groups are the experts' slots (mt_gather) instead of the rows in order.
+template <bool GATHER>
 __global__ __launch_bounds__(256) void mxfp4_planes_kernel(const float *__restrict__ x, int m, int nb, int ncp, int token_groups,
-                                                           char *__restrict__ bq) {
+                                                           char *__restrict__ bq, const mt_gather gat) {
     const size_t wv = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;  // (token group, pair of blocks)
     const int lane = threadIdx.x & 63, col = lane & 15, sub = (lane >> 4) & 1, npair = 2 * ncp;
     const size_t tg = wv / npair;
     if (tg >= (size_t)token_groups) return;  // (whole wavefronts)
     const int b = 2 * (int)(wv % npair) + (lane >> 5);
-    const size_t t = tg * 16 + col;
-    const bool valid = t < (size_t)m && b < nb;
+    size_t t = tg * 16 + col;
+    bool valid = t < (size_t)m && b < nb;
+    if (GATHER) {
+        const int gt = (int)(tg / gat.tb);
+        if (gt >= gat.goff[gat.experts]) return;  // past the last expert's tiles (whole wavefronts)
+        const int e = mt_expert_of(gat, gt);
+        const int slot = ((gt - gat.goff[e]) * gat.tb + (int)(tg % gat.tb)) * 16 + col;
+        valid = slot < gat.counts[e] && b < nb;
+        t = valid ? (size_t)(gat.lists[(size_t)e * gat.stride + slot] / gat.div) : 0;
+    }
     float f[16];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -404,11 +442,19 @@ __global__ __launch_bounds__(256) void mxfp4_planes_kernel(const float *__restri
 // row tile, a batch of four chunks ahead otherwise); the token records of a chunk are shared through LDS (staged
 // through registers BD chunks ahead, two stages, one barrier per chunk).  Narrow tiles do little arithmetic per
 // chunk, so what they need is requests in flight: the deeper staging is theirs.
-template <int RA, int TB, int BD>
+// GROUPED: the token tiles are the experts' (mt_gather), the weights come from the expert's entry of two pointer
+// tables, an output row is the pair the slot holds; one run of K; items walk the row tiles of one token tile first
+// (that tile's records stay in the XCD's L2).
+struct mt_experts {
+    const uint8_t *const *qs_tab;
+    const uint32_t *const *sc_tab;
+};
+
+template <int RA, int TB, int BD, bool GROUPED>
 __global__ __launch_bounds__(64 * MT_NW) void mxfp4_tiles_kernel(const uint8_t *__restrict__ qs_frag, const uint32_t *__restrict__ sc_frag,
                                                                  const char *__restrict__ bq, float *__restrict__ y, int n_out,
                                                                  int ncp, int m, int n_tt, int ks, int cps, size_t part_stride,
-                                                                 int items, int per_xcd) {
+                                                                 int items, int per_xcd, const mt_gather gat, const mt_experts ex) {
     constexpr int STAGE = TB * MT_RECORD, UNITS = TB * MT_UNITS, ROUNDS = (UNITS + 64 * MT_NW - 1) / (64 * MT_NW);
     constexpr bool RING = RA == 4;  // A two chunks ahead in a ring of two; else the next batch of four chunks
     static_assert(BD == 1 || BD == 2 || BD == 4, "the staging depth divides the unrolled batch");
@@ -418,7 +464,16 @@ __global__ __launch_bounds__(64 * MT_NW) void mxfp4_tiles_kernel(const uint8_t *
     // that run's weights stay in the XCD's L2 while its token tiles pass
     const int item = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
     if ((int)(blockIdx.x >> 3) >= per_xcd || item >= items) return;
-    const int tt = item % n_tt, split = (item / n_tt) % ks, wt = item / (n_tt * ks);
+    int tt = item % n_tt, split = (item / n_tt) % ks, wt = item / (n_tt * ks), expert = 0;
+    if (GROUPED) {  // n_tt = the row tiles here
+        wt = item % n_tt;
+        tt = item / n_tt;
+        split = 0;
+        if (tt >= gat.goff[gat.experts]) return;
+        expert = mt_expert_of(gat, tt);
+        qs_frag = ex.qs_tab[expert];
+        sc_frag = ex.sc_tab[expert];
+    }
     const int kc0 = split * cps, kc1 = pg_mt_run_end(split, cps, ncp);  // whole batches of four chunks
     const int nrg = (n_out + 15) / 16;                       // >= RA (the launcher's choice of RA)
     const int rg_mine = (wt * MT_NW + wave) * RA;            // the row groups whose tiles this wavefront stores
@@ -565,8 +620,14 @@ __global__ __launch_bounds__(64 * MT_NW) void mxfp4_tiles_kernel(const uint8_t *
         const size_t row = (size_t)(rg0 + r) * 16 + 4 * (lane >> 4);
 #pragma unroll
         for (int g = 0; g < TB; ++g) {
-            const size_t token = ((size_t)tt * TB + g) * 16 + (lane & 15);
-            if (token >= (size_t)m) continue;
+            size_t token = ((size_t)tt * TB + g) * 16 + (lane & 15);
+            if (GROUPED) {
+                const int slot = ((tt - gat.goff[expert]) * TB + g) * 16 + (lane & 15);
+                if (slot >= gat.counts[expert]) continue;
+                token = (size_t)gat.lists[(size_t)expert * gat.stride + slot];
+            } else if (token >= (size_t)m) {
+                continue;
+            }
             float *o = out + token * n_out + row;
             if (row + 3 < (size_t)n_out && (n_out & 3) == 0) {
                 *reinterpret_cast<v4f *>(o) = acc[r][g];
@@ -584,12 +645,24 @@ using mt_plan = pg_mxfp4_tiles_plan;
 template <int RA, int TB, int BD>
 pg_status launch_tiles(pg_ctx *ctx, const pg_gguf_tensor *w, const char *bq, float *y, size_t m, int ncp, const mt_plan &p) {
     const size_t lds = 2 * (size_t)TB * MT_RECORD;
-    auto kern = mxfp4_tiles_kernel<RA, TB, BD>;
+    auto kern = mxfp4_tiles_kernel<RA, TB, BD, false>;
     PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
     const size_t items = p.n_wt * p.n_tt * p.ks, per_xcd = (items + 7) / 8;
     return pg_launch(ctx, "mxfp4_tiles", kern, dim3((unsigned)(8 * per_xcd)), dim3(64 * MT_NW), lds, (const uint8_t *)w->qs,
                      reinterpret_cast<const uint32_t *>(w->d), bq, y, (int)w->n_out, ncp, (int)m, (int)p.n_tt, p.ks, p.cps,
-                     m * w->n_out, (int)items, (int)per_xcd);
+                     m * w->n_out, (int)items, (int)per_xcd, mt_gather{}, mt_experts{});
+}
+
+// The grouped form: `max_tiles` token tiles at most (the launch covers them all; those past the experts' last exit).
+template <int RA, int TB, int BD>
+pg_status launch_tiles_grouped(pg_ctx *ctx, size_t n_out, int ncp, const char *bq, float *y, size_t n_wt, size_t max_tiles,
+                               const mt_gather &gat, const mt_experts &ex) {
+    const size_t lds = 2 * (size_t)TB * MT_RECORD;
+    auto kern = mxfp4_tiles_kernel<RA, TB, BD, true>;
+    PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
+    const size_t items = n_wt * max_tiles, per_xcd = (items + 7) / 8;
+    return pg_launch(ctx, "mxfp4_tiles_grouped", kern, dim3((unsigned)(8 * per_xcd)), dim3(64 * MT_NW), lds, (const uint8_t *)nullptr,
+                     (const uint32_t *)nullptr, bq, y, (int)n_out, ncp, 0, (int)n_wt, 1, ncp, (size_t)0, (int)items, (int)per_xcd, gat, ex);
 }
 
 }  // namespace
@@ -634,8 +707,8 @@ pg_status pg_launch_mxfp4_tiles(pg_ctx *ctx, const float *x_dev, size_t m, const
     float *part = p.ks > 1 ? reinterpret_cast<float *>(bq + sz_b) : y_dev;
     const size_t threads = p.groups * 2 * (size_t)ncp * 64;  // a wavefront per token group and pair of blocks
     PG_CHECK_ARG((threads + 255) / 256 < ((size_t)1 << 31), "mxfp4: %zu rows x %zu is too much for one pre-pass", m, w->k_in);
-    PG_TRY(pg_launch(ctx, "mxfp4_planes", mxfp4_planes_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, x_dev, (int)m, nb,
-                     ncp, (int)p.groups, bq));
+    PG_TRY(pg_launch(ctx, "mxfp4_planes", mxfp4_planes_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, x_dev, (int)m, nb,
+                     ncp, (int)p.groups, bq, mt_gather{}));
     // the staging depth: the less arithmetic a chunk holds, the more chunks ahead
 #define PG_MT_LAUNCH(RA_, BD1, BD2, BD4) \
     (p.tb == 1 ? launch_tiles<RA_, 1, BD1>(ctx, w, bq, part, m, ncp, p) \
@@ -810,3 +883,150 @@ PG_API pg_status pg_mxfp4_expert_forward(pg_ctx *ctx, const pg_mxfp4_expert *e, 
     return PG_OK;
 }
 
+
+// ---- the MoE layer over MXFP4 experts, grouped ------------------------------------------------
+// MoELayer::forward after its router  examples/gpt_oss/moe.rs:286-352: the reference walks the tokens and calls
+// Mxfp4Expert::forward once per (token, chosen expert).  Here every expert's tokens form token tiles of the tile
+// kernel, all experts in one launch per product: routing lists, the pairs' activation rows gathered into digit
+// records, mlp1 of all experts, bias + swiglu per pair, records again, mlp2, and out[t] = sum_k w[t,k] (y + bias2)
+// in k order.
+namespace {
+
+// biased = h + bias1[expert]; the gpt-oss swiglu (examples/gpt_oss/moe.rs:155-166) per pair
+__global__ __launch_bounds__(256) void mxfp4_moe_swiglu_kernel(const float *__restrict__ h, const float *const *__restrict__ bias_tab,
+                                                               const int *__restrict__ topk_idx, size_t pairs, size_t inter,
+                                                               float alpha, float clamp, float *__restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= pairs * inter) return;
+    const size_t p = i / inter, c = i - p * inter;
+    const float *bias = bias_tab[topk_idx[p]];
+    const float g0 = h[p * 2 * inter + 2 * c] + bias[2 * c], l0 = h[p * 2 * inter + 2 * c + 1] + bias[2 * c + 1];
+    const float gate = fminf(g0, clamp);                                     // f32::min: a NaN operand loses
+    const float linear = l0 != l0 ? l0 : fminf(fmaxf(l0, -clamp), clamp);    // f32::clamp keeps NaN
+    const float activated = gate * (1.0f / (1.0f + expf(-alpha * gate)));
+    out[i] = activated * (linear + 1.0f);
+}
+
+// output[t] += weight * (out + mlp2_bias) over the token's experts in the order given  (examples/gpt_oss/moe.rs:104-108, 330-334)
+__global__ __launch_bounds__(256) void mxfp4_moe_combine_kernel(const float *__restrict__ yb, const float *const *__restrict__ bias_tab,
+                                                                const int *__restrict__ topk_idx, const float *__restrict__ topk_p,
+                                                                size_t tokens, size_t hidden, int top_k, float *__restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= tokens * hidden) return;
+    const size_t t = i / hidden, c = i - t * hidden;
+    float acc = 0.0f;
+    for (int k = 0; k < top_k; ++k) {
+        const size_t p = t * top_k + k;
+        const float result = yb[p * hidden + c] + bias_tab[topk_idx[p]][c];
+        const float prod = topk_p[p] * result;
+        acc = acc + prod;
+    }
+    out[i] = acc;
+}
+
+// One grouped product: rows `src` (pair / div) of the experts' slots -> records -> tiles against tensor table `which`.
+pg_status moe_product(pg_ctx *ctx, const float *src, size_t k_in, size_t n_out, int tb, size_t max_tiles, mt_gather gat, int div,
+                      const void **tab, size_t experts, int which, char *bq, float *y) {
+    const int nb = (int)(k_in / 32), ncp = (int)mx_chunks((size_t)nb);
+    gat.div = div;
+    const size_t groups = max_tiles * tb, threads = groups * 2 * (size_t)ncp * 64;
+    PG_CHECK_ARG((threads + 255) / 256 < ((size_t)1 << 31), "mxfp4 moe: too many pairs x %zu for one pre-pass", k_in);
+    PG_TRY(pg_launch(ctx, "mxfp4_planes_gather", mxfp4_planes_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, src, 0, nb,
+                     ncp, (int)groups, bq, gat));
+    const size_t nrg = (n_out + 15) / 16;
+    int ra = 4;
+    while (ra > 1 && ((size_t)ra > nrg || (nrg + MT_NW * ra - 1) / (MT_NW * ra) * max_tiles < 2 * (size_t)ctx->num_cu)) ra >>= 1;
+    const size_t n_wt = (nrg + MT_NW * ra - 1) / (MT_NW * ra);
+    PG_CHECK_ARG(n_wt * max_tiles < ((size_t)1 << 28), "mxfp4 moe: %zu x %zu tiles", n_wt, max_tiles);
+    const mt_experts ex = {reinterpret_cast<const uint8_t *const *>(tab + (size_t)(2 * which) * experts),
+                           reinterpret_cast<const uint32_t *const *>(tab + (size_t)(2 * which + 1) * experts)};
+#define PG_MTG(RA_, BD1, BD2, BD4) \
+    (tb == 1 ? launch_tiles_grouped<RA_, 1, BD1>(ctx, n_out, ncp, bq, y, n_wt, max_tiles, gat, ex) \
+     : tb == 2 ? launch_tiles_grouped<RA_, 2, BD2>(ctx, n_out, ncp, bq, y, n_wt, max_tiles, gat, ex) \
+               : launch_tiles_grouped<RA_, 4, BD4>(ctx, n_out, ncp, bq, y, n_wt, max_tiles, gat, ex))
+    return ra == 4 ? PG_MTG(4, 4, 2, 1) : (ra == 2 ? PG_MTG(2, 4, 4, 2) : PG_MTG(1, 4, 4, 4));
+#undef PG_MTG
+}
+
+}  // namespace
+
+PG_API pg_status pg_mxfp4_moe_ffn_routed_dev(pg_ctx *ctx, const float *x_dev, size_t T, const int32_t *expert_idx_dev,
+                                             const float *weight_dev, size_t top_k, const pg_mxfp4_expert *const *experts, size_t E,
+                                             float *out_dev) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(E >= 1 && E <= (size_t)PG_MOE_MAX_EXPERTS, "pg_mxfp4_moe_ffn: %zu experts (1..%d supported)", E, PG_MOE_MAX_EXPERTS);
+    PG_CHECK_ARG(top_k >= 1 && top_k <= E, "pg_mxfp4_moe_ffn: top_k %zu of %zu experts", top_k, E);
+    PG_CHECK_ARG(experts && experts[0], "pg_mxfp4_moe_ffn: null expert table");
+    const size_t hidden = experts[0]->hidden, inter = experts[0]->intermediate;
+    const float alpha = experts[0]->alpha, clamp = experts[0]->clamp;
+    for (size_t e = 0; e < E; ++e) {
+        PG_CHECK_ARG(experts[e] != nullptr, "pg_mxfp4_moe_ffn: expert %zu is null", e);
+        PG_CHECK_ARG(experts[e]->hidden == hidden && experts[e]->intermediate == inter && experts[e]->alpha == alpha &&
+                         experts[e]->clamp == clamp, "pg_mxfp4_moe_ffn: expert %zu differs in shape, alpha or clamp", e);
+    }
+    if (T == 0) return PG_OK;
+    PG_CHECK_ARG(x_dev && expert_idx_dev && weight_dev && out_dev, "pg_mxfp4_moe_ffn: null pointer");
+    PG_CHECK_ARG((uintptr_t)x_dev % 16 == 0, "pg_mxfp4_moe_ffn: x must be 16-byte aligned");
+    PG_CHECK_ARG(T * top_k < (1ull << 20), "pg_mxfp4_moe_ffn: too many (token, expert) pairs");
+    const size_t P = T * top_k;
+    // token tiles: groups of 16 slots, as many to a tile as an expert's average share suggests
+    const int tb = P / E <= 16 ? 1 : (P / E <= 32 ? 2 : 4);
+    const size_t max_tiles = P / (16 * (size_t)tb) + E;  // sum over experts of ceil(count / (16 tb)) stays below
+    const int ncp1 = (int)mx_chunks(hidden / 32), ncp2 = (int)mx_chunks(inter / 32);
+    const size_t sz_idx = pg_round_up(P * sizeof(int), 256), sz_p = pg_round_up(P * sizeof(float), 256);
+    const size_t sz_lists = pg_round_up(E * T * sizeof(int), 256), sz_counts = pg_round_up((2 * E + 1) * sizeof(int), 256);
+    const size_t sz_rec = pg_round_up(max_tiles * tb * (size_t)std::max(ncp1, ncp2) * MT_RECORD, 256);
+    const size_t sz_h = pg_round_up(P * 2 * inter * sizeof(float), 256), sz_act = pg_round_up(P * inter * sizeof(float), 256);
+    const size_t sz_y = pg_round_up(P * hidden * sizeof(float), 256);
+    void *ws = nullptr;
+    PG_TRY(pg_workspace(ctx, sz_idx + sz_p + sz_lists + sz_counts + sz_rec + sz_h + sz_act + sz_y, &ws));
+    char *p = static_cast<char *>(ws);
+    int *topk_idx = reinterpret_cast<int *>(p); p += sz_idx;
+    float *topk_p = reinterpret_cast<float *>(p); p += sz_p;
+    int *lists = reinterpret_cast<int *>(p); p += sz_lists;
+    int *counts = reinterpret_cast<int *>(p), *goff = counts + E; p += sz_counts;
+    char *rec = p; p += sz_rec;
+    float *h = reinterpret_cast<float *>(p); p += sz_h;
+    float *act = reinterpret_cast<float *>(p); p += sz_act;
+    float *yb = reinterpret_cast<float *>(p);
+    // [mlp1 codes | mlp1 scales | mlp2 codes | mlp2 scales | bias1 | bias2], E each
+    const void *host_tab[6 * PG_MOE_MAX_EXPERTS];
+    for (size_t e = 0; e < E; ++e) {
+        host_tab[0 * E + e] = experts[e]->mlp1->qs; host_tab[1 * E + e] = experts[e]->mlp1->d;
+        host_tab[2 * E + e] = experts[e]->mlp2->qs; host_tab[3 * E + e] = experts[e]->mlp2->d;
+        host_tab[4 * E + e] = experts[e]->bias1;    host_tab[5 * E + e] = experts[e]->bias2;
+    }
+    const void **tab = nullptr;
+    PG_TRY(pg_moe_cached_table(ctx, host_tab, 6 * E, &tab));
+    PG_TRY(pg_launch_moe_routing(ctx, nullptr, expert_idx_dev, weight_dev, T, E, top_k, topk_idx, topk_p, lists, counts));
+    PG_TRY(pg_launch(ctx, "mxfp4_tile_offsets", mxfp4_tile_offsets_kernel, dim3(1), dim3(64), 0, (const int *)counts, (int)E, tb, goff));
+    const mt_gather gat = {lists, counts, goff, (int)T, (int)E, tb, 1};
+    PG_TRY(moe_product(ctx, x_dev, hidden, 2 * inter, tb, max_tiles, gat, (int)top_k, tab, E, 0, rec, h));
+    PG_TRY(pg_launch(ctx, "mxfp4_moe_swiglu", mxfp4_moe_swiglu_kernel, dim3(grid_for(P * inter, 256)), dim3(256), 0, (const float *)h,
+                     reinterpret_cast<const float *const *>(tab + 4 * E), (const int *)topk_idx, P, inter, alpha, clamp, act));
+    PG_TRY(moe_product(ctx, act, inter, hidden, tb, max_tiles, gat, 1, tab, E, 1, rec, yb));
+    return pg_launch(ctx, "mxfp4_moe_combine", mxfp4_moe_combine_kernel, dim3(grid_for(T * hidden, 256)), dim3(256), 0, (const float *)yb,
+                     reinterpret_cast<const float *const *>(tab + 5 * E), (const int *)topk_idx, (const float *)topk_p, T, hidden,
+                     (int)top_k, out_dev);
+}
+
+PG_API pg_status pg_mxfp4_moe_ffn_routed(pg_ctx *ctx, const float *x, size_t T, const int32_t *expert_idx, const float *weight,
+                                         size_t top_k, const pg_mxfp4_expert *const *experts, size_t E, float *out) {
+    PG_TRY(pg_use(ctx));
+    PG_CHECK_ARG(experts && experts[0], "pg_mxfp4_moe_ffn: null expert table");
+    if (T == 0) return PG_OK;
+    PG_CHECK_ARG(x && expert_idx && weight && out, "pg_mxfp4_moe_ffn: null pointer");
+    const size_t hidden = experts[0]->hidden;
+    pg_tmp dx, di, dw, dout;
+    PG_TRY(dx.alloc(T * hidden * sizeof(float)));
+    PG_TRY(di.alloc(T * top_k * sizeof(int32_t)));
+    PG_TRY(dw.alloc(T * top_k * sizeof(float)));
+    PG_TRY(dout.alloc(T * hidden * sizeof(float)));
+    PG_HIP(hipMemcpyAsync(dx.p, x, T * hidden * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(di.p, expert_idx, T * top_k * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
+    PG_HIP(hipMemcpyAsync(dw.p, weight, T * top_k * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    PG_TRY(pg_mxfp4_moe_ffn_routed_dev(ctx, dx.as<float>(), T, di.as<int32_t>(), dw.as<float>(), top_k, experts, E, dout.as<float>()));
+    PG_HIP(hipMemcpyAsync(out, dout.p, T * hidden * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    PG_HIP(hipStreamSynchronize(ctx->stream));
+    return PG_OK;
+}

@@ -85,3 +85,22 @@ class Mxfp4Expert:
             self.free()
         except Exception:
             pass
+
+
+def moe_forward_routed(x, expert_idx, weight, experts, ctx=None):
+    """`MoELayer::forward` after its router, over `Mxfp4Expert`s (examples/gpt_oss/moe.rs:286-352): x [T, hidden],
+    expert_idx / weight [T, top_k] as the router chose them -> [T, hidden]; every product is one launch over all
+    experts."""
+    ctx = ctx or default_context()
+    hidden = experts[0].hidden
+    x = np.ascontiguousarray(x, np.float32).reshape(-1, hidden)
+    T = x.shape[0]
+    idx = np.ascontiguousarray(expert_idx, np.int32).reshape(T, -1)
+    w = np.ascontiguousarray(weight, np.float32).reshape(T, -1)
+    if idx.shape != w.shape:
+        raise ValueError("moe_forward_routed: expert_idx and weight differ in shape")
+    tab = (C.c_void_p * len(experts))(*[e._h.value for e in experts])
+    out = np.empty((T, hidden), np.float32)
+    _ffi.check(_ffi.lib.pg_mxfp4_moe_ffn_routed(ctx.handle, _ptr(x.reshape(-1)), T, _ptr(idx.reshape(-1)), _ptr(w.reshape(-1)), idx.shape[1],
+                                                C.cast(tab, C.POINTER(C.c_void_p)), len(experts), _ptr(out.reshape(-1))))
+    return out

@@ -320,6 +320,19 @@ def mxfp4_expert_forward(x, hidden, intermediate, alpha, clamp, b1, s1, b2, s2, 
     return out
 
 
+def mxfp4_moe_routed(x, T, hidden, intermediate, alpha, clamp, top_k, idx, weight, experts):
+    """experts: list of (mlp1_blocks, mlp1_scales, mlp2_blocks, mlp2_scales, mlp1_bias, mlp2_bias)."""
+    E = len(experts)
+    cols = [[_u8(ex[j]) if j < 4 else _f32(ex[j]) for ex in experts] for j in range(6)]
+    tabs = [(C.c_void_p * E)(*[a.ctypes.data for a in col]) for col in cols]
+    out = np.empty(T * hidden, np.float32)
+    rc = lib.orc_mxfp4_moe_routed(_p(_f32(x).reshape(-1)), _sz(T), _sz(hidden), _sz(intermediate), C.c_float(alpha), C.c_float(clamp),
+                                  _sz(E), _sz(top_k), _p(np.ascontiguousarray(idx, np.int32).reshape(-1)), _p(_f32(weight).reshape(-1)),
+                                  *tabs, _p(out))
+    assert rc == 0, rc
+    return out.reshape(T, hidden)
+
+
 lib.orc_huffman_table.restype = None
 lib.orc_huffman_canonical_codes.restype = None
 lib.orc_huffman_encode.restype = C.c_size_t

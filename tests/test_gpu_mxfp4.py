@@ -205,3 +205,40 @@ def test_mxfp4_limits_and_non_finite(ctx, orc):
     s3[5, :] = 0                                # f32::from_bits(0) = 0.0: the row is exactly zero
     got = mxfp4.mxfp4_matmul(x, b, s3.reshape(-1), out_dim, in_dim, ctx)
     assert got[5] == 0.0 and orc.mxfp4_matmul(x, b, s3.reshape(-1), out_dim, in_dim)[5] == 0.0
+
+
+@pytest.mark.parametrize("hidden,inter,E,top_k,T", [
+    (64, 96, 4, 2, 1), (64, 96, 5, 3, 7), (256, 160, 8, 2, 64), (512, 512, 8, 4, 300), (128, 64, 32, 4, 40),
+    (2880, 2880, 4, 2, 150),        # the gpt-oss expert shape; 75 tokens an expert on average
+])
+def test_mxfp4_moe_routed_follows_the_oracle(ctx, orc, hidden, inter, E, top_k, T):
+    """MoELayer::forward over MXFP4 experts (examples/gpt_oss/moe.rs:286-352), every product one launch over all
+    experts, against the reference's per-token walk; experts with no token, with one, and with more than a tile's."""
+    from peregrine_amd import mxfp4
+    from test_oracle_formats_pins import _mx_expert
+    say(f"mxfp4 moe hidden={hidden} inter={inter} E={E} top_k={top_k} T={T}")
+    rng = np.random.default_rng(hidden + inter + E + T)
+    raw = [_mx_expert(rng, hidden, inter) for _ in range(E)]
+    experts = [mxfp4.Mxfp4Expert(hidden, inter, 1.702, 7.0, *r, ctx=ctx) for r in raw]
+    x = orc.rng_normal(T + 11, T * hidden).reshape(T, hidden)
+    x[:, ::37] *= 10.0
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 0] -= 8.0                                    # expert 0 is (almost) never chosen
+    idx, w = orc.gpt_oss_route(logits, np.zeros(E, np.float32), T, E, top_k)
+    got = mxfp4.moe_forward_routed(x, idx, w, experts, ctx)
+    rows = list(range(0, T, max(1, T // 10))) + [T - 1]
+    want = orc.mxfp4_moe_routed(x[rows], len(rows), hidden, inter, 1.702, 7.0, top_k, np.asarray(idx).reshape(T, top_k)[rows],
+                                np.asarray(w).reshape(T, top_k)[rows], raw)
+    for j, t in enumerate(rows):
+        H.assert_close_rel(got[t], want[j], RTOL_CONTRACT, f"token {t} (contract)")
+        H.assert_close_rel(got[t], want[j], 2e-4, f"token {t} (achieved)")
+    # one expert called alone on the tokens routed to it gives the same rows as the grouped launch did for those pairs
+    e = int(np.bincount(np.asarray(idx).reshape(-1), minlength=E).argmax())
+    toks = [t for t in range(T) if e in np.asarray(idx).reshape(T, top_k)[t]][:5]
+    if top_k == 1 and toks:
+        alone = experts[e].forward(x[toks])
+        H.assert_close_rel(got[toks] / np.asarray(w).reshape(T, top_k)[toks], alone, 2e-4, "one expert alone")
+    with pytest.raises(ValueError):
+        mxfp4.moe_forward_routed(x, np.asarray(idx).reshape(T, top_k), np.asarray(w).reshape(T, top_k)[:, :1], experts, ctx)
+    for ex in experts:
+        ex.free()

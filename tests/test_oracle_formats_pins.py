@@ -106,6 +106,37 @@ def test_mxfp4_expert_closed_forms_and_float64(orc):
     assert np.abs(got - want).max() <= 5e-6 * np.abs(want).max()
 
 
+def _mx_expert(rng, hidden, inter):
+    return (rng.integers(0, 256, 2 * inter * hidden // 2, dtype=np.uint8), rng.integers(118, 126, 2 * inter * hidden // 32, dtype=np.uint8),
+            rng.integers(0, 256, hidden * inter // 2, dtype=np.uint8), rng.integers(118, 126, hidden * inter // 32, dtype=np.uint8),
+            rng.standard_normal(2 * inter).astype(np.float32), rng.standard_normal(hidden).astype(np.float32))
+
+
+def test_mxfp4_moe_is_the_experts_outputs_added_in_the_routing_s_order(orc):
+    """examples/gpt_oss/moe.rs:330-351: output += weight * expert_out, experts in the order the router listed them.
+    Recomputed in float32 NumPy from orc_mxfp4_expert_forward's own outputs; equal bit for bit, and a swapped order
+    is not (so the order is what is pinned)."""
+    rng = np.random.default_rng(77)
+    hidden, inter, E, top_k, T = 64, 96, 5, 3, 6
+    experts = [_mx_expert(rng, hidden, inter) for _ in range(E)]
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    idx = np.array([rng.permutation(E)[:top_k] for _ in range(T)], np.int32)
+    w = rng.random((T, top_k)).astype(np.float32)
+    got = orc.mxfp4_moe_routed(x, T, hidden, inter, 1.702, 7.0, top_k, idx, w, experts)
+    differs = False
+    for t in range(T):
+        ys = [orc.mxfp4_expert_forward(x[t], hidden, inter, 1.702, 7.0, *experts[e]) for e in idx[t]]
+        acc = np.zeros(hidden, np.float32)
+        for k in range(top_k):
+            acc = (acc + (w[t, k] * ys[k]).astype(np.float32)).astype(np.float32)
+        assert (got[t].view(np.uint32) == acc.view(np.uint32)).all()
+        rev = np.zeros(hidden, np.float32)
+        for k in reversed(range(top_k)):
+            rev = (rev + (w[t, k] * ys[k]).astype(np.float32)).astype(np.float32)
+        differs |= bool((rev.view(np.uint32) != acc.view(np.uint32)).any())
+    assert differs
+
+
 # ---- canonical Huffman ------------------------------------------------------------------
 
 def biased_i8(n, seed):
