@@ -863,6 +863,66 @@ def section_mxfp4(B, line):
     line["mxfp4_many_rows"] = many
     torch.cuda.empty_cache()
 
+    # the gpt-oss-20b MoE layer after its router: 32 MXFP4 experts (hidden = intermediate = 2880), top 4
+    hidden = inter = 2880
+    E, top_k = 32, 4
+    experts = []
+    for e in range(E):
+        b1 = rng.integers(0, 256, size=2 * inter * hidden // 2, dtype=np.uint8)
+        s1 = rng.integers(118, 124, size=2 * inter * hidden // 32, dtype=np.uint8)
+        b2 = rng.integers(0, 256, size=hidden * inter // 2, dtype=np.uint8)
+        s2 = rng.integers(118, 124, size=hidden * inter // 32, dtype=np.uint8)
+        bias1 = rng.standard_normal(2 * inter).astype(np.float32)
+        bias2 = rng.standard_normal(hidden).astype(np.float32)
+        h = C.c_void_p()
+        check(lib.pg_mxfp4_expert_create(B.h, hidden, inter, C.c_float(1.702), C.c_float(7.0), C.c_void_p(b1.ctypes.data), C.c_void_p(s1.ctypes.data),
+                                         C.c_void_p(b2.ctypes.data), C.c_void_p(s2.ctypes.data), C.c_void_p(bias1.ctypes.data),
+                                         C.c_void_p(bias2.ctypes.data), C.byref(h)))
+        experts.append(h)
+    tab = (C.c_void_p * E)(*[h.value for h in experts])
+    weight_bytes = E * 3 * inter * (hidden // 32) * 17
+    moe = []
+    for T in (1024, 1):
+        x = B.make_acts(T, hidden, 7430)
+        logits = B.normal(7431, (T, E), 1.0)
+        top = torch.topk(logits, top_k, dim=1)
+        idx = top.indices.to(torch.int32).contiguous()
+        wt = torch.softmax(top.values, dim=1).contiguous()
+        out = torch.empty(T, hidden, device=dev)
+        torch.cuda.synchronize()
+
+        def step():
+            check(lib.pg_mxfp4_moe_ffn_routed_dev(B.h, ptr(x), T, ptr(idx), ptr(wt), top_k, C.cast(tab, C.POINTER(C.c_void_p)), E, ptr(out)))
+
+        t = B.timed(step, B.dsteps, max(args.warmup, 8))
+        prof, _ = B.profiled(step, B.dsteps)
+        # the same layer as the reference walks it, batched per expert: one Mxfp4Expert::forward per expert over its tokens
+        lists = [torch.nonzero((idx == e).any(dim=1)).flatten() for e in range(E)]
+        xs = [x[l].contiguous() for l in lists]
+        scratch = torch.empty(max(1, max(l.numel() for l in lists)) * 3 * inter, device=dev)
+        outs = [torch.empty(max(1, l.numel()), hidden, device=dev) for l in lists]
+
+        def loop_step():
+            for e in range(E):
+                if lists[e].numel():
+                    check(lib.pg_mxfp4_expert_forward_dev(B.h, experts[e], ptr(xs[e]), lists[e].numel(), ptr(scratch), ptr(outs[e])))
+
+        tl = B.timed(loop_step, max(3, B.dsteps // 4), 3)
+        flop = 2.0 * T * top_k * 3 * inter * hidden
+        touched = min(E, T * top_k) / E * weight_bytes if T == 1 else weight_bytes
+        entry = {"workload": f"gpt-oss-20b MoE layer after its router: {T} token(s), {E} MXFP4 experts of {hidden} -> 2 x {inter} -> {hidden}, top {top_k}; "
+                             f"routing from N(0,1) logits (top-k, softmax over the k)",
+                 "ms_per_step": round(t["ms_per_step"], 5), **B.stats(t),
+                 "value": round(flop / (t["ms_per_step"] * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+                 "weights_gbs": round(touched / (t["ms_per_step"] * 1e-3) / 1e9, 1),
+                 "per_expert_calls_ms": round(tl["ms_per_step"], 5),
+                 "kernels_ms_x_launches": {k: [round(v[0], 5), round(v[1] / B.dsteps, 1)] for k, v in prof.items()}}
+        moe.append(entry)
+    for h in experts:
+        lib.pg_mxfp4_expert_free(B.h, h)
+    line["mxfp4_moe_layer"] = moe
+    torch.cuda.empty_cache()
+
 
 def section_moe(B, line):
     """cfg5: Grok-1-shaped MoE expert FFN, Q8_0 experts."""

@@ -161,6 +161,7 @@ pg_status pg_launch_moe_routing(pg_ctx *ctx, const float *router_logits_dev, con
     else
         PG_TRY(pg_launch(ctx, "moe_copy_routing", copy_routing_kernel, dim3(grid_for(T, 64)), dim3(64), 0,
                          idx_dev, weight_dev, (int)T, (int)E, (int)top_k, topk_idx, topk_p));
+    if (!lists) return PG_OK;  // (a caller that works pair by pair)
     return pg_launch(ctx, "moe_expert_lists", expert_lists_kernel, dim3((unsigned)E), dim3(64), 0, (const int *)topk_idx,
                      (int)(T * top_k), (int)T, lists, counts);
 }

@@ -124,11 +124,28 @@ __device__ __forceinline__ void mx_emit_digits(const float (&f)[4], int b, int s
 // LDS while its first weight loads are in flight.  Each wavefront then walks its K slice in batches of
 // MX_U chunks, the next batch requested before the current one is consumed, and the partial tiles of
 // the KS slices and the 5 planes are added through LDS in a fixed order.
-template <int T, int RG, int NW>
+// PAIRS (T = 1): blockIdx.y is a (token, expert) pair of an MoE layer: the weights are the pair's expert's entry of
+// two pointer tables, the activation row is pair / div, the output row the pair.
+struct mx_pairs {
+    const uint8_t *const *qs_tab;
+    const uint32_t *const *sc_tab;
+    const int *expert_of;  // [pairs]
+    int div;
+};
+
+template <int T, int RG, int NW, bool PAIRS = false>
 __global__ __launch_bounds__(64 * NW) void mxfp4_rows_kernel(const uint8_t *__restrict__ qs_frag, const uint32_t *__restrict__ sc_frag,
                                                                   const float *__restrict__ x, float *__restrict__ y,
-                                                                  int n_out, int nb, int ncp, int m) {
+                                                                  int n_out, int nb, int ncp, int m, const mx_pairs pr) {
+    static_assert(!PAIRS || T == 1, "a pair is one activation row");
     constexpr int KS = NW / RG, COLS = MX_PLANES * T;
+    size_t x_row0 = (size_t)blockIdx.y * T;  // first activation row of this workgroup
+    if (PAIRS) {
+        const int expert = pr.expert_of[blockIdx.y];
+        qs_frag = pr.qs_tab[expert];
+        sc_frag = pr.sc_tab[expert];
+        x_row0 = blockIdx.y / (unsigned)pr.div;
+    }
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const int kp = ncp * 128, stride = kp + 64;  // plane stride: not a multiple of the LDS bank span
     char *const dig = lds;
@@ -167,11 +184,11 @@ __global__ __launch_bounds__(64 * NW) void mxfp4_rows_kernel(const uint8_t *__re
     auto row_of = [&](int id) { return T == 1 ? 0 : (id >= nblk) + (T > 2 && id >= 2 * nblk); };  // id / nblk
     auto x_valid = [&](int id) {
         const int t = row_of(id), b = id - t * nblk;
-        return b < nb && (size_t)blockIdx.y * T + t < (size_t)m;  // blocks nb .. 4 ncp - 1 and rows past m are zeros
+        return b < nb && x_row0 + t < (size_t)m;  // blocks nb .. 4 ncp - 1 and rows past m are zeros
     };
     auto load_x = [&](int id) {
         const int t = row_of(id), b = id - t * nblk;
-        const size_t at = x_valid(id) ? (((size_t)blockIdx.y * T + t) * nb + b) * 8 + sub : 0;
+        const size_t at = x_valid(id) ? ((x_row0 + t) * nb + b) * 8 + sub : 0;
         return reinterpret_cast<const float4 *>(x)[at];
     };
     auto emit = [&](int id, const float4 v) {
@@ -249,8 +266,8 @@ __global__ __launch_bounds__(64 * NW) void mxfp4_rows_kernel(const uint8_t *__re
 #pragma unroll
             for (int k = 0; k < KS; ++k)
                 sum += part[((size_t)(g * KS + k) * 64 + 16 * (i >> 2) + t * MX_PLANES + j) * 4 + (i & 3)];
-        const size_t row = ((size_t)blockIdx.x * RG + g) * 16 + i, item = (size_t)blockIdx.y * T + t;
-        if (row < (size_t)n_out && item < (size_t)m) y[item * n_out + row] = sum;
+        const size_t row = ((size_t)blockIdx.x * RG + g) * 16 + i, item = (size_t)blockIdx.y * T + t;  // (PAIRS: the pair)
+        if (row < (size_t)n_out && (PAIRS || item < (size_t)m)) y[item * n_out + row] = sum;
     }
 }
 
@@ -266,7 +283,19 @@ pg_status launch_rows(pg_ctx *ctx, const pg_gguf_tensor *w, const float *x, floa
     PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
     const dim3 grid(grid_for((w->n_out + 15) / 16, RG), grid_for(m, T));
     return pg_launch(ctx, "mxfp4_rows", kern, grid, dim3(64 * NW), lds, (const uint8_t *)w->qs,
-                     reinterpret_cast<const uint32_t *>(w->d), x, y, (int)w->n_out, (int)(w->k_in / 32), ncp, (int)m);
+                     reinterpret_cast<const uint32_t *>(w->d), x, y, (int)w->n_out, (int)(w->k_in / 32), ncp, (int)m, mx_pairs{});
+}
+
+// One launch for `pairs` (token, expert) pairs: pair p = row p / div of x against expert expert_of[p]; x has x_rows rows.
+template <int RG, int NW>
+pg_status launch_rows_pairs(pg_ctx *ctx, size_t n_out, size_t k_in, const float *x, size_t x_rows, float *y, size_t pairs, int ncp,
+                            const mx_pairs &pr) {
+    const size_t lds = mx_lds_bytes(1, ncp, NW);
+    auto kern = mxfp4_rows_kernel<1, RG, NW, true>;
+    PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
+    const dim3 grid(grid_for((n_out + 15) / 16, RG), (unsigned)pairs);
+    return pg_launch(ctx, "mxfp4_rows_pairs", kern, grid, dim3(64 * NW), lds, (const uint8_t *)nullptr, (const uint32_t *)nullptr, x, y,
+                     (int)n_out, (int)(k_in / 32), ncp, (int)x_rows, pr);
 }
 
 }  // namespace
@@ -948,6 +977,22 @@ pg_status moe_product(pg_ctx *ctx, const float *src, size_t k_in, size_t n_out, 
 #undef PG_MTG
 }
 
+// The same product pair by pair on the decode kernel (few pairs).
+bool pairs_fit(int ncp) { return mx_lds_bytes(1, ncp) <= (160u << 10); }
+pg_status moe_product_pairs(pg_ctx *ctx, const float *src, size_t src_rows, size_t k_in, size_t n_out, size_t pairs, int div,
+                            const void **tab, size_t experts, int which, const int *topk_idx, float *y) {
+    const int ncp = (int)mx_chunks(k_in / 32);
+    const mx_pairs pr = {reinterpret_cast<const uint8_t *const *>(tab + (size_t)(2 * which) * experts),
+                         reinterpret_cast<const uint32_t *const *>(tab + (size_t)(2 * which + 1) * experts), topk_idx, div};
+    // as pg_launch_mxfp4_rows chooses: 16 wavefronts on a row group while there is at most one group per CU, else 8
+    // on the fewest row groups that keep every workgroup resident at once
+    const size_t groups = (n_out + 15) / 16 * pairs, slots = (size_t)ctx->num_cu * 2;
+    if (groups <= (size_t)ctx->num_cu) return launch_rows_pairs<1, 16>(ctx, n_out, k_in, src, src_rows, y, pairs, ncp, pr);
+    if (groups <= slots) return launch_rows_pairs<1, 8>(ctx, n_out, k_in, src, src_rows, y, pairs, ncp, pr);
+    if ((groups + 1) / 2 <= slots) return launch_rows_pairs<2, 8>(ctx, n_out, k_in, src, src_rows, y, pairs, ncp, pr);
+    return launch_rows_pairs<4, 8>(ctx, n_out, k_in, src, src_rows, y, pairs, ncp, pr);
+}
+
 }  // namespace
 
 PG_API pg_status pg_mxfp4_moe_ffn_routed_dev(pg_ctx *ctx, const float *x_dev, size_t T, const int32_t *expert_idx_dev,
@@ -998,13 +1043,23 @@ PG_API pg_status pg_mxfp4_moe_ffn_routed_dev(pg_ctx *ctx, const float *x_dev, si
     }
     const void **tab = nullptr;
     PG_TRY(pg_moe_cached_table(ctx, host_tab, 6 * E, &tab));
-    PG_TRY(pg_launch_moe_routing(ctx, nullptr, expert_idx_dev, weight_dev, T, E, top_k, topk_idx, topk_p, lists, counts));
-    PG_TRY(pg_launch(ctx, "mxfp4_tile_offsets", mxfp4_tile_offsets_kernel, dim3(1), dim3(64), 0, (const int *)counts, (int)E, tb, goff));
+    // With few pairs hardly two of them meet in an expert, and a pair is a one-row product: the decode kernel, one
+    // workgroup column per pair (exact activations; no expert lists).  Otherwise the experts' token tiles on the tile kernel.
+    const bool by_pairs = P <= 2 * E && P <= 64 && pairs_fit(ncp1) && pairs_fit(ncp2);
+    PG_TRY(pg_launch_moe_routing(ctx, nullptr, expert_idx_dev, weight_dev, T, E, top_k, topk_idx, topk_p, by_pairs ? nullptr : lists, counts));
+    if (!by_pairs)
+        PG_TRY(pg_launch(ctx, "mxfp4_tile_offsets", mxfp4_tile_offsets_kernel, dim3(1), dim3(64), 0, (const int *)counts, (int)E, tb, goff));
     const mt_gather gat = {lists, counts, goff, (int)T, (int)E, tb, 1};
-    PG_TRY(moe_product(ctx, x_dev, hidden, 2 * inter, tb, max_tiles, gat, (int)top_k, tab, E, 0, rec, h));
+    if (by_pairs)
+        PG_TRY(moe_product_pairs(ctx, x_dev, T, hidden, 2 * inter, P, (int)top_k, tab, E, 0, topk_idx, h));
+    else
+        PG_TRY(moe_product(ctx, x_dev, hidden, 2 * inter, tb, max_tiles, gat, (int)top_k, tab, E, 0, rec, h));
     PG_TRY(pg_launch(ctx, "mxfp4_moe_swiglu", mxfp4_moe_swiglu_kernel, dim3(grid_for(P * inter, 256)), dim3(256), 0, (const float *)h,
                      reinterpret_cast<const float *const *>(tab + 4 * E), (const int *)topk_idx, P, inter, alpha, clamp, act));
-    PG_TRY(moe_product(ctx, act, inter, hidden, tb, max_tiles, gat, 1, tab, E, 1, rec, yb));
+    if (by_pairs)
+        PG_TRY(moe_product_pairs(ctx, act, P, inter, hidden, P, 1, tab, E, 1, topk_idx, yb));
+    else
+        PG_TRY(moe_product(ctx, act, inter, hidden, tb, max_tiles, gat, 1, tab, E, 1, rec, yb));
     return pg_launch(ctx, "mxfp4_moe_combine", mxfp4_moe_combine_kernel, dim3(grid_for(T * hidden, 256)), dim3(256), 0, (const float *)yb,
                      reinterpret_cast<const float *const *>(tab + 5 * E), (const int *)topk_idx, (const float *)topk_p, T, hidden,
                      (int)top_k, out_dev);

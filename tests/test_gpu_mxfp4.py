@@ -208,7 +208,8 @@ def test_mxfp4_limits_and_non_finite(ctx, orc):
 
 
 @pytest.mark.parametrize("hidden,inter,E,top_k,T", [
-    (64, 96, 4, 2, 1), (64, 96, 5, 3, 7), (256, 160, 8, 2, 64), (512, 512, 8, 4, 300), (128, 64, 32, 4, 40),
+    (64, 96, 4, 2, 1), (128, 64, 32, 4, 8), (2880, 2880, 8, 4, 2),      # few pairs: the decode kernel, a workgroup column per pair
+    (64, 96, 5, 3, 7), (256, 160, 8, 2, 64), (512, 512, 8, 4, 300), (128, 64, 32, 4, 40),
     (2880, 2880, 4, 2, 150),        # the gpt-oss expert shape; 75 tokens an expert on average
 ])
 def test_mxfp4_moe_routed_follows_the_oracle(ctx, orc, hidden, inter, E, top_k, T):
