@@ -845,7 +845,7 @@ def section_mxfp4(B, line):
             check(lib.pg_gguf_matmul_dev(B.h, ptr(x), m, h, ptr(y)))
 
         t = B.timed(step, B.dsteps, max(args.warmup, 8))
-        prof, _ = B.profiled(step, B.dsteps)
+        prof, grids = B.profiled(step, B.dsteps)
         flop = 2.0 * m * n_out * k_in
         k_ms = prof["mxfp4_tiles"][0]
         many.append({"workload": f"MXFP4 [{m} x {k_in}] -> [{n_out}]: activation rows as four planes of E4M3 base-32 digits, "
@@ -854,7 +854,7 @@ def section_mxfp4(B, line):
                      "kernels_ms": {k: round(v[0], 5) for k, v in prof.items()},
                      "roofline": {"kernel": "mxfp4_tiles_kernel", "bound": "mfma", "achieved": round(flop / (k_ms * 1e-3) / 1e12, 1),
                                   "peak": 5000.0, "unit": "TFLOP/s", "frac": round(flop / (k_ms * 1e-3) / 1e12 / 5000.0, 4),
-                                  "executed_tflops": round(4 * flop / (k_ms * 1e-3) / 1e12, 1), "traffic": None,
+                                  "executed_tflops": round(4 * flop / (k_ms * 1e-3) / 1e12, 1), "traffic": B.traffic_for("mxfp4_tiles", grids) if not many else None,
                                   "avg_launch_ms": round(k_ms, 5),
                                   "note": "peak = the published dense FP8 rate (an FP4 x FP8 instruction runs at it); "
                                           "executed = four digit planes per algorithmic multiply-add"}})

@@ -493,15 +493,19 @@ __global__ __launch_bounds__(64 * MT_NW) void mxfp4_tiles_kernel(const uint8_t *
     // that run's weights stay in the XCD's L2 while its token tiles pass
     const int item = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
     if ((int)(blockIdx.x >> 3) >= per_xcd || item >= items) return;
-    int tt = item % n_tt, split = (item / n_tt) % ks, wt = item / (n_tt * ks), expert = 0;
-    if (GROUPED) {  // n_tt = the row tiles here
-        wt = item % n_tt;
-        tt = item / n_tt;
+    int tt = item % n_tt, split = (item / n_tt) % ks, wt = item / (n_tt * ks), expert = 0, live = TB;
+    if (GROUPED) {  // n_tt = the row tiles here; token tile 8 i + x belongs to XCD x (the unused tail tiles spread evenly)
+        const int slot = (int)(blockIdx.x >> 3);
+        wt = slot % n_tt;
+        tt = (slot / n_tt) * 8 + (int)(blockIdx.x & 7);
         split = 0;
         if (tt >= gat.goff[gat.experts]) return;
         expert = mt_expert_of(gat, tt);
         qs_frag = ex.qs_tab[expert];
         sc_frag = ex.sc_tab[expert];
+        // an expert's last tile is rarely full: token groups without a slot in use are skipped (their records hold zeros)
+        const int left = gat.counts[expert] - (tt - gat.goff[expert]) * TB * 16;
+        live = __builtin_amdgcn_readfirstlane(left >= TB * 16 ? TB : (left + 15) / 16);
     }
     const int kc0 = split * cps, kc1 = pg_mt_run_end(split, cps, ncp);  // whole batches of four chunks
     const int nrg = (n_out + 15) / 16;                       // >= RA (the launcher's choice of RA)
@@ -582,7 +586,7 @@ __global__ __launch_bounds__(64 * MT_NW) void mxfp4_tiles_kernel(const uint8_t *
     } while (0)
 #define PG_MT_GROUP(U, G)                                                 \
     do {                                                                  \
-        if ((G) < TB) {                                                   \
+        if ((G) < TB && (!GROUPED || (G) < live)) {                       \
             PG_MT_READ(G, 1, y0, y1);                                     \
             PG_MT_MUL(U, G, 0, x0, x1);                                   \
             __builtin_amdgcn_sched_barrier(0);                            \
@@ -689,7 +693,7 @@ pg_status launch_tiles_grouped(pg_ctx *ctx, size_t n_out, int ncp, const char *b
     const size_t lds = 2 * (size_t)TB * MT_RECORD;
     auto kern = mxfp4_tiles_kernel<RA, TB, BD, true>;
     PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
-    const size_t items = n_wt * max_tiles, per_xcd = (items + 7) / 8;
+    const size_t per_xcd = (max_tiles + 7) / 8 * n_wt, items = 8 * per_xcd;
     return pg_launch(ctx, "mxfp4_tiles_grouped", kern, dim3((unsigned)(8 * per_xcd)), dim3(64 * MT_NW), lds, (const uint8_t *)nullptr,
                      (const uint32_t *)nullptr, bq, y, (int)n_out, ncp, 0, (int)n_wt, 1, ncp, (size_t)0, (int)items, (int)per_xcd, gat, ex);
 }
