@@ -160,3 +160,61 @@ def test_few_row_products_replayed_from_a_graph(ctx, orc):
         hip.lib.hipGraphExecDestroy(ex)
         hip.lib.hipGraphDestroy(graph)
     gw.free()
+
+
+def test_mxfp4_products_and_moe_replayed_from_a_graph(ctx, orc):
+    """MXFP4 over many rows (digit records, tiles over two runs of K, their sum) and the gpt-oss MoE layer over
+    MXFP4 experts in both its forms (token tiles of all experts in one launch; pair by pair for a few pairs),
+    captured together after one eager call has made the buffers and the experts' pointer table."""
+    from peregrine_amd import _ffi, mxfp4
+    from test_oracle_formats_pins import _mx_expert
+    hip = Hip()
+    rng = np.random.default_rng(5)
+    n, k, m = 600, 2048, 40
+    w = mxfp4.upload(rng.integers(0, 256, n * k // 2, dtype=np.uint8), rng.integers(110, 130, n * k // 32, dtype=np.uint8), n, k, ctx)
+    hidden, inter, E, top_k, T = 256, 128, 8, 2, 48
+    experts = [mxfp4.Mxfp4Expert(hidden, inter, 1.702, 7.0, *_mx_expert(rng, hidden, inter), ctx=ctx) for _ in range(E)]
+    tab = (C.c_void_p * E)(*[e._h.value for e in experts])
+    idx = np.stack([rng.permutation(E)[:top_k] for _ in range(T)]).astype(np.int32)
+    wt = rng.random((T, top_k)).astype(np.float32)
+    inputs = [orc.rng_normal(60 + i, max(m * k, T * hidden)) for i in range(3)]
+    x = DevBuf(ctx, host=inputs[0])
+    d_idx, d_wt = DevBuf(ctx, host=idx), DevBuf(ctx, host=wt)
+    outs = [DevBuf(ctx, m * n * 4), DevBuf(ctx, T * hidden * 4), DevBuf(ctx, 3 * hidden * 4)]
+    sizes = [m * n, T * hidden, 3 * hidden]
+
+    def step():
+        _ffi.check(_ffi.lib.pg_gguf_matmul_dev(ctx.handle, x.ptr, m, w._h, outs[0].ptr))
+        _ffi.check(_ffi.lib.pg_mxfp4_moe_ffn_routed_dev(ctx.handle, x.ptr, T, d_idx.ptr, d_wt.ptr, top_k, C.cast(tab, C.POINTER(C.c_void_p)), E, outs[1].ptr))
+        _ffi.check(_ffi.lib.pg_mxfp4_moe_ffn_routed_dev(ctx.handle, x.ptr, 3, d_idx.ptr, d_wt.ptr, top_k, C.cast(tab, C.POINTER(C.c_void_p)), E, outs[2].ptr))
+
+    def eager(v):
+        _ffi.check(_ffi.lib.pg_memcpy_h2d(ctx.handle, x.ptr, C.c_void_p(v.ctypes.data), v.nbytes))
+        ctx.profile_begin()
+        step()
+        prof = ctx.profile_end()
+        ctx.sync()
+        return [o.to_host(np.float32) for o in outs], prof
+
+    want, prof = zip(*[eager(v) for v in inputs])
+    assert {"mxfp4_tiles", "gguf_mm_sum_parts", "mxfp4_tiles_grouped", "mxfp4_rows_pairs"} <= set(prof[0]), prof[0]
+    say("capturing an MXFP4 product and two MoE layers")
+    graph, ex = hip.capture(ctx.stream, step)
+    try:
+        for i, v in enumerate(inputs):
+            _ffi.check(_ffi.lib.pg_gguf_matmul_dev(ctx.handle, x.ptr, 1, w._h, outs[0].ptr))   # other work in between
+            _ffi.check(_ffi.lib.pg_memcpy_h2d(ctx.handle, x.ptr, C.c_void_p(v.ctypes.data), v.nbytes))
+            for o, sz in zip(outs, sizes):
+                _ffi.check(_ffi.lib.pg_memcpy_h2d(ctx.handle, o.ptr, C.c_void_p(np.full(sz, np.nan, np.float32).ctypes.data), sz * 4))
+            ctx.sync()
+            hip.ok(hip.lib.hipGraphLaunch(ex, ctx.stream), "hipGraphLaunch")
+            ctx.sync()
+            for j in range(3):
+                got = outs[j].to_host(np.float32)
+                assert (got.view(np.uint32) == want[i][j].view(np.uint32)).all(), f"replay {i}, call {j} differs from the eager call"
+    finally:
+        hip.lib.hipGraphExecDestroy(ex)
+        hip.lib.hipGraphDestroy(graph)
+    w.free()
+    for e in experts:
+        e.free()
