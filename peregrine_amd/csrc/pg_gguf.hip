@@ -968,7 +968,7 @@ __global__ void tile_weights_kernel(const uint8_t *__restrict__ qs, int n_out, i
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;    // chunk within the row group
     if (i >= (size_t)nsg * 4 * CH) return;
     const int lane = (int)(i & 63), q = (int)((i >> 6) % FILLS), wave = (int)((i / CH) & 3), sg = (int)(i / (4 * CH));
-    const int st = 16 * q + (lane >> 2), j = (lane & 3) ^ ((lane >> 3) & 3);
+    const int st = 16 * q + (lane >> 2), j = (lane & 3) ^ ((lane >> 4) & 3);
     const int row = rg * 128 + wave * 32 + (st & 31), half = st >> 5, block = sg * 4 + j;
     uint4 v = {0, 0, 0, 0};
     if (row < n_out && block < nb)

@@ -36,8 +36,11 @@ constexpr int NBU = 4;                              // blocks per stage
 constexpr int RING = 3;                             // LDS stages (two in flight beyond the one consumed)
 // LDS stage layout.  Every fill is arranged so that neighbouring lanes fetch neighbouring
 // 16-byte chunks of global memory (whole 64- or 128-byte runs per request); the chunk order
-// inside a run is XOR-swizzled so that the 128-bit LDS reads of 8 neighbouring lanes fall
-// into 8 different 16-byte bank groups.
+// inside a run is XOR-swizzled so that the 128-bit LDS reads of 16 neighbouring lanes fall
+// into 16 different 16-byte bank groups (gfx950 serves a 128-bit read over 256 bytes of banks a
+// pass: with 8 distinct groups per 8 lanes only, lanes l and l + 8 collided and every such read
+// took 8 cycles instead of 4).  For the digits that means: tokens 8 .. 15 (mod 16) keep their two
+// planes in swapped places.
 constexpr int DIG_STAGE = 64 * 128;                 // [token][plane] units of 128 B: 4 blocks x 2 halves  8 KiB
 constexpr int D_STAGE = 4 * 256;                    // [wave][row group of 8][j][8 f16]                     1 KiB
 constexpr int XS_STAGE = 32 * 16;                   // [token][4 block scales]                              512 B
@@ -221,7 +224,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     int dig_jb[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-        const int unit = (2 * wave + u) * 8 + (lane >> 3), tok = unit >> 1, pl = unit & 1;
+        const int unit = (2 * wave + u) * 8 + (lane >> 3), tok = unit >> 1, pl = (unit & 1) ^ ((tok >> 3) & 1);
         const int ch = (lane & 7) ^ (tok & 7);
         dig_jb[u] = ch >> 1;
         dig_src[u] = digits + xrow_of(tok) * pg_mm_row_bytes(nb) + (size_t)pl * nb * 32 + (ch & 1) * 16;
@@ -231,7 +234,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // weights: fill q covers streams 16q .. 16q+15 (Q8_0: stream = 32*half + row, Q4_0: stream = row);
     // the lane fetches block (lane & 3) ^ swizzle of the stream's 4 blocks.
     const int row0 = bx * 128 + wave * 32;
-    const int w_jb = (lane & 3) ^ ((lane >> 3) & 3);  // stream >> 1 = 8q + (lane >> 3)
+    const int w_jb = (lane & 3) ^ ((lane >> 4) & 3);  // (stream >> 2) & 3, stream = 16q + (lane >> 2)
     const int8_t *w_src[W_FILLS];
 #pragma unroll
     for (int q = 0; q < W_FILLS; ++q) {
@@ -283,13 +286,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     // One block of the stage at `base`: operands from LDS, two MFMAs, scale-and-accumulate.
     // Split into three phases so that the full-stage path can overlap them across blocks.
-    const int w_rd = OFF_W + wave * W_WAVE + (QT == 8 ? lane : l31) * 64, w_sw = ((QT == 8 ? lane : l31) >> 1) & 3;
-    const int dig_rd = l31 * 256, dig_sw = l31 & 7;
+    const int w_rd = OFF_W + wave * W_WAVE + (QT == 8 ? lane : l31) * 64, w_sw = ((QT == 8 ? lane : l31) >> 2) & 3;
+    const int dig_rd = l31 * 256, dig_sw = l31 & 7, dig_hi = ((l31 >> 3) & 1) * 128;  // tokens 8 .. 15 (mod 16) keep their planes swapped
     const int d_rd = OFF_D + wave * 256 + (l31 >> 3) * 64 + (l31 & 7) * 2;  // this lane's weight row: [group of 8][j][8 f16]
     auto read_ab = [&](const char *base, int j, v4i (&ab)[3]) {
         ab[0] = *reinterpret_cast<const v4i *>(base + w_rd + ((j ^ w_sw) * 16));
-        ab[1] = *reinterpret_cast<const v4i *>(base + dig_rd + (((2 * j + hh) ^ dig_sw) * 16));
-        ab[2] = *reinterpret_cast<const v4i *>(base + dig_rd + 128 + (((2 * j + hh) ^ dig_sw) * 16));
+        ab[1] = *reinterpret_cast<const v4i *>(base + dig_rd + dig_hi + (((2 * j + hh) ^ dig_sw) * 16));
+        ab[2] = *reinterpret_cast<const v4i *>(base + dig_rd + (128 - dig_hi) + (((2 * j + hh) ^ dig_sw) * 16));
     };
     // the block's weight scale of this lane's row
     // (read as integers: a float-typed LDS read makes the compiler wait for every fill in flight)
