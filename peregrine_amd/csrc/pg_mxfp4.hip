@@ -147,7 +147,7 @@ __global__ __launch_bounds__(64 * NW) void mxfp4_rows_kernel(const uint8_t *__re
         x_row0 = blockIdx.y / (unsigned)pr.div;
     }
     extern __shared__ __attribute__((aligned(16))) char lds[];
-    const int kp = ncp * 128, stride = kp + 64;  // plane stride: not a multiple of the LDS bank span
+    const int kp = ncp * 128, stride = kp + 16;  // plane stride = 16 (mod 256): the 16 columns of a 128-bit read fall into 16 different bank groups
     char *const dig = lds;
     uint8_t *const sb = reinterpret_cast<uint8_t *>(lds + (size_t)COLS * stride);
     float *const part = reinterpret_cast<float *>(lds + (size_t)COLS * stride + (((size_t)COLS * 4 * ncp + 15) & ~(size_t)15));
@@ -273,7 +273,7 @@ __global__ __launch_bounds__(64 * NW) void mxfp4_rows_kernel(const uint8_t *__re
 
 size_t mx_lds_bytes(int t, int ncp, int nw = 16) {
     const size_t cols = (size_t)MX_PLANES * t;
-    return cols * ((size_t)ncp * 128 + 64) + ((cols * 4 * ncp + 15) & ~(size_t)15) + (size_t)nw * 64 * 4 * sizeof(float);
+    return cols * ((size_t)ncp * 128 + 16) + ((cols * 4 * ncp + 15) & ~(size_t)15) + (size_t)nw * 64 * 4 * sizeof(float);
 }
 
 template <int T, int RG, int NW>
