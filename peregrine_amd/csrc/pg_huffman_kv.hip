@@ -568,7 +568,9 @@ PG_API pg_status pg_huffman_kv_cache_get_kv_dev(pg_ctx *ctx, const pg_huffman_kv
         off += c->k_chunks[i]->num_tokens;
     }
     const std::vector<size_t> strides(chunks.size(), total_len * hd);
-    PG_TRY(decompress_many(ctx, chunks.data(), outs.data(), strides.data(), chunks.size()));
+    for (size_t first = 0; first < chunks.size(); first += 16384)  // (a launch takes up to 65535 chunks)
+        PG_TRY(decompress_many(ctx, chunks.data() + first, outs.data() + first, strides.data() + first,
+                               std::min<size_t>(16384, chunks.size() - first)));
     if (hot->len > 0) {
         const size_t width = hot->len * hd * sizeof(float);
         PG_HIP(hipMemcpy2DAsync(k_dev + off * hd, total_len * hd * sizeof(float), hot->k, hot->capacity * hd * sizeof(float), width,
