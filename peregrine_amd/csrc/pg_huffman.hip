@@ -20,7 +20,6 @@
 // A prefix sum over the per-subsequence symbol counts then gives every thread its output
 // offset and a last pass writes the symbols.
 #include <algorithm>
-#include <deque>
 #include <new>
 #include "pg_internal.h"
 
@@ -52,48 +51,53 @@ void canonical_codes(const uint8_t *bl, uint32_t *codes) {
         if (bl[s] > 0) codes[s] = next_code[bl[s]]++;
 }
 
-// src/huffman.rs:35-150: two-queue Huffman over the symbols in use (stable sort by frequency,
-// a leaf wins a tie against an internal node), depths clamped to MAX_LUT_BITS.
+// Code lengths equal to those of src/huffman.rs:35-150 (two queues over the symbols in use,
+// stably sorted by frequency; a leaf wins a tie against an internal node; depths clamped to
+// MAX_LUT_BITS), computed in place in the sorted weight array without building the tree
+// (Moffat & Katajainen's three passes).  Both give the same lengths because the two-queue
+// construction consumes leaves in sorted order and a node consumed earlier never ends up
+// shallower than one consumed later: the depth of the i-th leaf in sorted order is fixed by
+// how many internal nodes each level holds, which is what the passes below count.
 void table_from_frequencies(const uint64_t *freqs, uint8_t *bl) {
     std::fill(bl, bl + NUM_SYMBOLS, (uint8_t)0);
-    std::vector<int> symbols;
-    std::vector<uint64_t> fv;
+    int sym[NUM_SYMBOLS], n = 0;
     for (int s = 0; s < NUM_SYMBOLS; ++s)
-        if (freqs[s] > 0) { symbols.push_back(s); fv.push_back(freqs[s]); }
-    const size_t n = symbols.size();
+        if (freqs[s] > 0) sym[n++] = s;
     if (n == 0) return;
-    if (n == 1) { bl[symbols[0]] = 1; return; }
-    std::vector<size_t> parent(2 * n - 1, 0);
-    std::vector<unsigned> depth(2 * n - 1, 0);
-    std::vector<size_t> order(n);
-    for (size_t i = 0; i < n; ++i) order[i] = i;
-    std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) { return fv[a] < fv[b]; });
-    std::deque<std::pair<uint64_t, size_t>> leaf_q, int_q;
-    for (size_t i : order) leaf_q.emplace_back(fv[i], i);
-    auto pick = [&]() {
-        std::pair<uint64_t, size_t> r;
-        if (!leaf_q.empty() && (int_q.empty() || leaf_q.front().first <= int_q.front().first)) {
-            r = leaf_q.front();
-            leaf_q.pop_front();
-        } else {
-            r = int_q.front();
-            int_q.pop_front();
+    if (n == 1) { bl[sym[0]] = 1; return; }
+    std::stable_sort(sym, sym + n, [&](int a, int b) { return freqs[a] < freqs[b]; });
+    uint64_t w[NUM_SYMBOLS];  // weights, then parent indices, then depths
+    for (int i = 0; i < n; ++i) w[i] = freqs[sym[i]];
+    // Pass 1: w[t] becomes the weight of internal node t; a consumed internal node's slot holds
+    // its parent.  `leaf` walks the unconsumed leaves, `node` the unconsumed internal nodes.
+    int leaf = 0, node = 0;
+    for (int t = 0; t < n - 1; ++t) {
+        uint64_t sum = 0;
+        for (int half = 0; half < 2; ++half) {
+            const bool take_node = leaf >= n || (node < t && w[node] < w[leaf]);
+            if (take_node) { sum += w[node]; w[node++] = (uint64_t)t; }
+            else sum += w[leaf++];
         }
-        return r;
-    };
-    size_t next_node = n;
-    for (size_t it = 0; it + 1 < n; ++it) {
-        const auto a = pick();
-        const auto b = pick();
-        parent[a.second] = next_node;
-        parent[b.second] = next_node;
-        int_q.emplace_back(a.first + b.first, next_node);
-        ++next_node;
+        // Leaves are consumed from the front and node t's slot is behind `leaf` by now (each
+        // step consumes at least as many slots as it fills), so the write never lands on a
+        // weight still to be read.
+        w[t] = sum;
     }
-    const size_t root = 2 * n - 2;
-    depth[root] = 0;
-    for (size_t i = root; i-- > 0;) depth[i] = depth[parent[i]] + 1;
-    for (size_t i = 0; i < n; ++i) bl[symbols[i]] = (uint8_t)std::min<unsigned>(depth[i], MAX_LUT_BITS);
+    // Pass 2: parent indices to depths of the internal nodes, root (node n-2) first.
+    w[n - 2] = 0;
+    for (int t = n - 3; t >= 0; --t) w[t] = w[w[t]] + 1;
+    // Pass 3: a level with `slots` places of which `inner` are internal nodes holds
+    // slots - inner leaves, handed out from the most frequent symbol down.
+    uint64_t depth = 0;
+    int slots = 1, t = n - 2, next = n - 1;
+    while (slots > 0) {
+        int inner = 0;
+        while (t >= 0 && w[t] == depth) { ++inner; --t; }
+        for (; slots > inner; --slots) w[next--] = depth;
+        slots = 2 * inner;
+        ++depth;
+    }
+    for (int i = 0; i < n; ++i) bl[sym[i]] = (uint8_t)std::min<uint64_t>(w[i], MAX_LUT_BITS);
 }
 
 // A table for data that must decode again.  The reference's, where that is a prefix code.  Where

@@ -23,6 +23,16 @@ def test_table_and_codes_equal_the_oracle(orc):
     for k in (2, 7, 64, 256):
         f = np.zeros(256, np.uint64); f[rng.choice(256, k, replace=False)] = rng.integers(1, 1000, k); cases.append(f)
     cases.append(_freqs(np.clip(np.rint(rng.standard_normal(1 << 16) * 20), -127, 127)))   # weight-like
+    for i in range(3000):                                                             # many ties, few to all symbols, wide ranges
+        k = int(rng.integers(2, 257))
+        f = np.zeros(256, np.uint64)
+        hi = (2, 3, 5, 50, 1 << 20, 1 << 40)[i % 6]
+        f[rng.choice(256, k, replace=False)] = rng.integers(1, hi, k)
+        if i % 7 == 0:
+            f[f > 0] = np.sort(f[f > 0])[::-1]                                        # falling with the symbol
+        if i % 11 == 0:
+            f[f > 0] = 2 ** rng.integers(0, 30, int((f > 0).sum()))                   # powers of two: sums that tie with leaves
+        cases.append(f)
     for f in cases:
         t = huffman.HuffmanTable.from_frequencies(f)
         bl, codes = orc.huffman_table(f)
