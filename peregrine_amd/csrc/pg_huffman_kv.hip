@@ -519,16 +519,13 @@ static pg_status compress_hot(pg_ctx *ctx, pg_huffman_kv_cache *c) {
     }
     if (done == 0) return st;
     const size_t rest = hot->len - done;
-    if (rest > 0) {  // through a staging buffer: source and destination may overlap
-        const size_t width = rest * hd * sizeof(float), pitch = stride * sizeof(float);
-        pg_tmp tmp;
-        PG_TRY(tmp.alloc(2 * heads * width));
-        char *tk = tmp.as<char>(), *tv = tk + heads * width;
-        PG_HIP(hipMemcpy2DAsync(tk, width, hot->k + done * hd, pitch, width, heads, hipMemcpyDeviceToDevice, ctx->stream));
-        PG_HIP(hipMemcpy2DAsync(tv, width, hot->v + done * hd, pitch, width, heads, hipMemcpyDeviceToDevice, ctx->stream));
-        PG_HIP(hipMemcpy2DAsync(hot->k, pitch, tk, width, width, heads, hipMemcpyDeviceToDevice, ctx->stream));
-        PG_HIP(hipMemcpy2DAsync(hot->v, pitch, tv, width, width, heads, hipMemcpyDeviceToDevice, ctx->stream));
-        PG_HIP(hipStreamSynchronize(ctx->stream));
+    // The rest moves to the front in slices no longer than the distance it moves, oldest first on
+    // the one stream, so that no copy reads what it writes; nothing is allocated and nothing waited for.
+    const size_t pitch = stride * sizeof(float);
+    for (size_t at = 0; at < rest && hd * heads > 0; at += done) {
+        const size_t width = std::min(done, rest - at) * hd * sizeof(float);
+        PG_HIP(hipMemcpy2DAsync(hot->k + at * hd, pitch, hot->k + (done + at) * hd, pitch, width, heads, hipMemcpyDeviceToDevice, ctx->stream));
+        PG_HIP(hipMemcpy2DAsync(hot->v + at * hd, pitch, hot->v + (done + at) * hd, pitch, width, heads, hipMemcpyDeviceToDevice, ctx->stream));
     }
     hot->len = rest;
     return st;

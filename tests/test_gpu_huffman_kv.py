@@ -163,6 +163,7 @@ def test_reference_cache_tests(ctx, orc):
     (3, 4, 10, 4, (1, 7, 2, 30, 5, 1, 0, 3)),      # one append that cuts several chunks, an empty append
     (1, 16, 0, 5, (3, 3, 3, 20)),                  # threshold below the chunk size: raised to it
     (2, 2, 6, 6, (13,)),
+    (2, 8, 64, 4, (70, 3, 3, 1)),                  # a window much longer than a chunk: it moves to the front in many slices
     (8, 128, 512, 256, (300, 1, 1, 400, 1)),       # a Llama-sized cache: 262144 symbols per chunk
     (2, 16, 8, 4, (5,) * 60),                      # 74 chunks per side: get_kv decodes 148 streams, each under its own table, in one pass
 ])
