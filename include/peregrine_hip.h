@@ -242,7 +242,9 @@ pg_status pg_mxfp4_expert_forward_dev(pg_ctx *ctx, const pg_mxfp4_expert *expert
  * expert_idx, weight [T, top_k]; out[t] = sum_k weight[t, k] * experts[expert_idx[t, k]].forward(x[t]), the terms
  * added in k order.  All experts of one launch share hidden, intermediate, alpha and clamp.  The reference calls an
  * expert once per (token, k); here the tokens of each expert are gathered and every product is one launch over all
- * experts.  An index outside 0..E-1 or repeated within a token contributes nothing (its weight counts as 0). */
+ * experts.  An index outside 0..E-1, or an expert named twice by one token (the reference would panic on the first
+ * and never produces the second), is PG_EINVAL from the host-pointer form, which reads the indices; the _dev form
+ * cannot look without waiting for the stream, and there such an entry contributes nothing (its weight counts as 0). */
 pg_status pg_mxfp4_moe_ffn_routed(pg_ctx *ctx, const float *x, size_t T, const int32_t *expert_idx, const float *weight,
                                   size_t top_k, const pg_mxfp4_expert *const *experts, size_t E, float *out);
 pg_status pg_mxfp4_moe_ffn_routed_dev(pg_ctx *ctx, const float *x_dev, size_t T, const int32_t *expert_idx_dev,

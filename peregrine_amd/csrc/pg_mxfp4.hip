@@ -1075,6 +1075,16 @@ PG_API pg_status pg_mxfp4_moe_ffn_routed(pg_ctx *ctx, const float *x, size_t T, 
     PG_CHECK_ARG(experts && experts[0], "pg_mxfp4_moe_ffn: null expert table");
     if (T == 0) return PG_OK;
     PG_CHECK_ARG(x && expert_idx && weight && out, "pg_mxfp4_moe_ffn: null pointer");
+    PG_CHECK_ARG(E >= 1 && E <= (size_t)PG_MOE_MAX_EXPERTS && top_k >= 1 && top_k <= E, "pg_mxfp4_moe_ffn: top_k %zu of %zu experts", top_k, E);
+    // the reference indexes self.experts[expert_idx] (examples/gpt_oss/moe.rs:104-108) and would panic on an index out
+    // of range; its top-k never names an expert twice for a token, which the grouped products rely on
+    for (size_t t = 0; t < T; ++t)
+        for (size_t k = 0; k < top_k; ++k) {
+            const int32_t e = expert_idx[t * top_k + k];
+            PG_CHECK_ARG(e >= 0 && (size_t)e < E, "pg_mxfp4_moe_ffn: token %zu names expert %d of %zu", t, (int)e, E);
+            for (size_t j = 0; j < k; ++j)
+                PG_CHECK_ARG(expert_idx[t * top_k + j] != e, "pg_mxfp4_moe_ffn: token %zu names expert %d twice", t, (int)e);
+        }
     const size_t hidden = experts[0]->hidden;
     pg_tmp dx, di, dw, dout;
     PG_TRY(dx.alloc(T * hidden * sizeof(float)));

@@ -241,5 +241,14 @@ def test_mxfp4_moe_routed_follows_the_oracle(ctx, orc, hidden, inter, E, top_k, 
         H.assert_close_rel(got[toks] / np.asarray(w).reshape(T, top_k)[toks], alone, 2e-4, "one expert alone")
     with pytest.raises(ValueError):
         mxfp4.moe_forward_routed(x, np.asarray(idx).reshape(T, top_k), np.asarray(w).reshape(T, top_k)[:, :1], experts, ctx)
+    from peregrine_amd import _ffi
+    bad = np.asarray(idx, np.int32).reshape(T, top_k).copy()
+    bad[T - 1, 0] = E                                      # the reference's self.experts[expert_idx] would panic
+    with pytest.raises(_ffi.PeregrineError):
+        mxfp4.moe_forward_routed(x, bad, w, experts, ctx)
+    if top_k > 1:
+        bad[T - 1, 0] = bad[T - 1, 1]                      # an expert named twice by one token
+        with pytest.raises(_ffi.PeregrineError):
+            mxfp4.moe_forward_routed(x, bad, w, experts, ctx)
     for ex in experts:
         ex.free()
