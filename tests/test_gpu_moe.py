@@ -126,6 +126,37 @@ def test_moe_full_size_equal_experts_property(ctx, orc):
         H.assert_close_rel(got[t], want[t], 1e-3, f"token {t}")
 
 
+def test_moe_full_size_distinct_experts_against_the_oracle(ctx, orc):
+    """Benchmark configuration 5 at full width with eight DIFFERENT experts (5.1 GB of Q8_0 blocks): the whole layer
+    on 64 tokens, of which three are walked by the oracle (a token's output depends on no other token, so the oracle
+    is given just those rows and their logits: 18 one-row products of 201 M weights each)."""
+    from peregrine_amd import gguf, moe
+    T, d, ffn, E, top_k = 64, 6144, 32768, 8, 2
+    say("moe full size, distinct experts, sampled tokens against the oracle")
+    rng = np.random.default_rng(51)
+    def blocks(n_out, k_in):
+        b = np.empty((n_out * k_in // 32, 34), np.uint8)
+        b[:, 2:] = rng.integers(0, 256, size=(b.shape[0], 32), dtype=np.uint8)
+        b[:, :2] = np.frombuffer(np.float16(0.02 / 127).tobytes(), np.uint8)
+        b[::7, :2] = np.frombuffer(np.float16(-0.035 / 127).tobytes(), np.uint8)   # scales differ between blocks, in sign too
+        return b.tobytes()
+    raws = [[blocks(ffn, d) for _ in range(E)], [blocks(ffn, d) for _ in range(E)], [blocks(d, ffn) for _ in range(E)]]
+    mk = lambda rs, n_out, k_in: [gguf.GgufWeight(r, 8, n_out, k_in, ctx) for r in rs]
+    ex = moe.MoEExperts(mk(raws[0], ffn, d), mk(raws[1], ffn, d), mk(raws[2], d, ffn), top_k, moe.SILU, ctx)
+    x = orc.rng_normal(8, T * d)
+    logits = orc.rng_normal(9, T * E).reshape(T, E)
+    got = ex.forward(x, logits).reshape(T, d)
+    rows = [0, 29, 63]
+    xs = np.ascontiguousarray(x.reshape(T, d)[rows]).reshape(-1)
+    want, idx, _ = orc.moe_ffn(xs, len(rows), d, ffn, E, top_k, np.ascontiguousarray(logits[rows]), raws[0], raws[1], raws[2], 8, 0)
+    assert len(set(np.asarray(idx).reshape(-1).tolist())) >= 3      # the sampled tokens reach several experts
+    want = np.asarray(want).reshape(len(rows), d)
+    for j, t in enumerate(rows):
+        H.assert_close_rel(got[t], want[j], MOE_RTOL, f"token {t}")
+    for w in ex.gate + ex.up + ex.down:
+        w.free()
+
+
 def test_moe_many_tokens_per_expert(ctx, orc):
     """More than 32 tokens reach one expert (two token tiles), another expert gets none, and the
     widths are not multiples of the kernel's 128-row / 4-block tiles."""
