@@ -325,6 +325,35 @@ inline std::vector<float> expert_ffn(const GpuContext &gpu, const std::vector<fl
     return out;
 }
 
+// The same expert FFN over a routing another gate made: routing[t] = the token's (expert, weight) pairs, as
+// Gate::forward returns them (examples/deepseek/moe.rs:111-215, 271-297; the gpt_oss router,
+// examples/gpt_oss/moe.rs:298-330, gives the same per token).  Every token names the same number of experts.
+// `shared`, if not empty: the shared experts' output [tokens, d], added last (examples/deepseek/moe.rs:298-300).
+inline std::vector<float> expert_ffn_routed(const GpuContext &gpu, const std::vector<float> &x,
+                                            const std::vector<std::vector<std::pair<size_t, float>>> &routing,
+                                            const std::vector<const gguf::BlockWeight *> &gate,
+                                            const std::vector<const gguf::BlockWeight *> &up,
+                                            const std::vector<const gguf::BlockWeight *> &down, int act,
+                                            const std::vector<float> &shared = {}) {
+    const size_t E = gate.size(), tokens = routing.size();
+    if (E == 0 || up.size() != E || down.size() != E) throw Panic(PG_EINVAL, "expert_ffn_routed: expert tables differ in length");
+    std::vector<const pg_gguf_tensor *> g(E), u(E), d(E);
+    for (size_t e = 0; e < E; ++e) { g[e] = gate[e]->handle(); u[e] = up[e]->handle(); d[e] = down[e]->handle(); }
+    const size_t dm = gate[0]->k_in(), top_k = tokens ? routing[0].size() : 1;
+    if (x.size() != tokens * dm || (!shared.empty() && shared.size() != tokens * dm)) throw Panic(PG_EINVAL, "expert_ffn_routed: input sizes");
+    std::vector<int32_t> idx;
+    std::vector<float> w;
+    for (const auto &r : routing) {
+        if (r.size() != top_k) throw Panic(PG_EINVAL, "expert_ffn_routed: tokens name different numbers of experts");
+        for (const auto &pr : r) { idx.push_back((int32_t)pr.first); w.push_back(pr.second); }
+    }
+    std::vector<float> out(tokens * dm);
+    check(pg_moe_ffn_routed(gpu.raw(), x.data(), tokens, idx.data(), w.data(), E, top_k, g.data(), u.data(), d.data(), act,
+                            shared.empty() ? nullptr : shared.data(), out.data()),
+          "expert_ffn_routed");
+    return out;
+}
+
 }  // namespace moe
 
 namespace llama {
@@ -510,11 +539,37 @@ public:
         return out;
     }
 
+    const pg_mxfp4_expert *handle() const { return h_; }
+    size_t hidden() const { return hidden_; }
+
 private:
     const GpuContext *gpu_;
     pg_mxfp4_expert *h_ = nullptr;
     size_t hidden_;
 };
+
+// MoELayer::forward after its router, over Mxfp4Experts  examples/gpt_oss/moe.rs:286-352: x [tokens, hidden],
+// routing[t] = the token's (expert, weight) pairs in the order the router chose them; every product is one launch
+// over all experts.
+inline std::vector<float> moe_forward_routed(const GpuContext &gpu, const std::vector<float> &x,
+                                             const std::vector<std::vector<std::pair<size_t, float>>> &routing,
+                                             const std::vector<const Mxfp4Expert *> &experts) {
+    if (experts.empty()) throw Panic(PG_EINVAL, "moe_forward_routed: no experts");
+    const size_t tokens = routing.size(), hidden = experts[0]->hidden(), top_k = tokens ? routing[0].size() : 1;
+    if (x.size() != tokens * hidden) throw Panic(PG_EINVAL, "moe_forward_routed: x.len() != tokens * hidden");
+    std::vector<const pg_mxfp4_expert *> tab;
+    for (const auto *e : experts) tab.push_back(e->handle());
+    std::vector<int32_t> idx;
+    std::vector<float> w;
+    for (const auto &r : routing) {
+        if (r.size() != top_k) throw Panic(PG_EINVAL, "moe_forward_routed: tokens name different numbers of experts");
+        for (const auto &pr : r) { idx.push_back((int32_t)pr.first); w.push_back(pr.second); }
+    }
+    std::vector<float> out(tokens * hidden);
+    check(pg_mxfp4_moe_ffn_routed(gpu.raw(), x.data(), tokens, idx.data(), w.data(), top_k, tab.data(), tab.size(), out.data()),
+          "moe_forward_routed");
+    return out;
+}
 
 }  // namespace mxfp4
 

@@ -32,6 +32,12 @@ void orc_huffman_kv_free(void *);
 void orc_huffman_kv_append(void *, const float *, const float *, size_t);
 size_t orc_huffman_kv_stat(const void *, int);
 void orc_huffman_kv_get_kv(const void *, int, float *, float *);
+int orc_gpt_oss_route(const float *, const float *, size_t, size_t, size_t, int32_t *, float *);
+int orc_moe_ffn_routed(const float *, size_t, size_t, size_t, size_t, size_t, const int32_t *, const float *, const uint8_t *const *,
+                       const uint8_t *const *, const uint8_t *const *, int, int, const float *, float *);
+int orc_mxfp4_moe_routed(const float *, size_t, size_t, size_t, float, float, size_t, size_t, const int32_t *, const float *,
+                         const uint8_t *const *, const uint8_t *const *, const uint8_t *const *, const uint8_t *const *,
+                         const float *const *, const float *const *, float *);
 }
 
 using namespace peregrine;
@@ -359,6 +365,106 @@ static void test_huffman_kv_cache(const GpuContext &gpu) {
     EXPECT(threw, "data.len() != total must panic (src/huffman.rs:619)");
 }
 
+// The expert FFNs behind a routing the caller made (examples/deepseek/moe.rs:271-300, examples/gpt_oss/moe.rs:286-352),
+// against the CPU restatement's per-token walk.
+static void test_moe_routed(const GpuContext &gpu) {
+    std::printf("test_moe_routed\n");
+    auto lcg = [](uint32_t &st) { st = st * 1103515245u + 12345u; return (float)st / 4294967295.0f * 2.0f - 1.0f; };
+    auto rel_err = [](const std::vector<float> &got, const std::vector<float> &want) {
+        double num = 0, den = 0;
+        for (size_t i = 0; i < got.size(); ++i) { num = std::fmax(num, std::fabs((double)got[i] - want[i])); den += (double)want[i] * want[i]; }
+        return num / std::fmax(std::sqrt(den / (double)got.size()), 1e-30);
+    };
+    const size_t T = 9, E = 6, top_k = 2;
+    uint32_t st = 7;
+    std::vector<float> logits(T * E), zero_bias(E, 0.0f), w(T * top_k);
+    for (auto &v : logits) v = 3.0f * lcg(st);
+    std::vector<int32_t> idx(T * top_k);
+    orc_gpt_oss_route(logits.data(), zero_bias.data(), T, E, top_k, idx.data(), w.data());
+    std::vector<std::vector<std::pair<size_t, float>>> routing(T);
+    for (size_t t = 0; t < T; ++t)
+        for (size_t k = 0; k < top_k; ++k) routing[t].push_back({(size_t)idx[t * top_k + k], w[t * top_k + k]});
+    {   // Q8_0 experts, SiLU, with a shared-expert term
+        const size_t d = 64, ffn = 96;
+        auto blocks = [&](size_t n_out, size_t k_in) {
+            std::vector<uint8_t> b(n_out * k_in / 32 * 34);
+            for (size_t i = 0; i < b.size(); i += 34) {
+                b[i] = 0x00; b[i + 1] = 0x1E + (uint8_t)((i / 34) % 3);   // f16 scales around 2^-8
+                for (size_t j = 2; j < 34; ++j) { st = st * 1103515245u + 12345u; b[i + j] = (uint8_t)(st >> 24); }
+            }
+            return b;
+        };
+        std::vector<std::vector<uint8_t>> raw[3];
+        std::vector<std::unique_ptr<gguf::BlockWeight>> own;
+        std::vector<const gguf::BlockWeight *> tabs[3];
+        std::vector<const uint8_t *> rp[3];
+        for (int which = 0; which < 3; ++which)
+            for (size_t e = 0; e < E; ++e) {
+                raw[which].push_back(which == 2 ? blocks(d, ffn) : blocks(ffn, d));
+                own.push_back(std::make_unique<gguf::BlockWeight>(gpu, raw[which].back(), 8, which == 2 ? d : ffn, which == 2 ? ffn : d));
+                tabs[which].push_back(own.back().get());
+            }
+        for (int which = 0; which < 3; ++which)
+            for (size_t e = 0; e < E; ++e) rp[which].push_back(raw[which][e].data());
+        std::vector<float> x(T * d), shared(T * d), want(T * d);
+        for (auto &v : x) v = lcg(st);
+        for (auto &v : shared) v = 0.1f * lcg(st);
+        auto got = moe::expert_ffn_routed(gpu, x, routing, tabs[0], tabs[1], tabs[2], PG_ACT_SILU, shared);
+        EXPECT(orc_moe_ffn_routed(x.data(), T, d, ffn, E, top_k, idx.data(), w.data(), rp[0].data(), rp[1].data(), rp[2].data(), 8, 0,
+                                  shared.data(), want.data()) == 0, "oracle");
+        EXPECT(rel_err(got, want) < 4e-4, "expert_ffn_routed: %.3g of the rms", rel_err(got, want));
+        bool threw = false;
+        auto bad = routing;
+        bad[3][1].first = E;
+        try { moe::expert_ffn_routed(gpu, x, bad, tabs[0], tabs[1], tabs[2], PG_ACT_SILU); } catch (const Panic &) { threw = true; }
+        EXPECT(threw, "an expert index out of range must panic");
+    }
+    {   // MXFP4 experts
+        const size_t hidden = 64, inter = 96;
+        const float alpha = 1.702f, clamp = 7.0f;
+        auto bytes = [&](size_t n, uint8_t lo, uint8_t span) {
+            std::vector<uint8_t> b(n);
+            for (auto &v : b) { st = st * 1103515245u + 12345u; v = (uint8_t)(lo + (st >> 24) % span); }
+            return b;
+        };
+        std::vector<std::vector<uint8_t>> b1, s1, b2, s2;
+        std::vector<std::vector<float>> bias1, bias2;
+        std::vector<std::unique_ptr<mxfp4::Mxfp4Expert>> own;
+        std::vector<const mxfp4::Mxfp4Expert *> tab;
+        for (size_t e = 0; e < E; ++e) {
+            b1.push_back(bytes(2 * inter * hidden / 2, 0, 255));
+            s1.push_back(bytes(2 * inter * hidden / 32, 118, 6));     // E8M0 scales 2^-9 .. 2^-4
+            b2.push_back(bytes(hidden * inter / 2, 0, 255));
+            s2.push_back(bytes(hidden * inter / 32, 118, 6));
+            bias1.emplace_back(2 * inter);
+            bias2.emplace_back(hidden);
+            for (auto &v : bias1.back()) v = 0.2f * lcg(st);
+            for (auto &v : bias2.back()) v = 0.2f * lcg(st);
+            own.push_back(std::make_unique<mxfp4::Mxfp4Expert>(gpu, hidden, inter, alpha, clamp, b1[e], s1[e], b2[e], s2[e], bias1[e], bias2[e]));
+            tab.push_back(own.back().get());
+        }
+        std::vector<const uint8_t *> pb1, ps1, pb2, ps2;
+        std::vector<const float *> pbi1, pbi2;
+        for (size_t e = 0; e < E; ++e) {
+            pb1.push_back(b1[e].data()); ps1.push_back(s1[e].data()); pb2.push_back(b2[e].data()); ps2.push_back(s2[e].data());
+            pbi1.push_back(bias1[e].data()); pbi2.push_back(bias2[e].data());
+        }
+        std::vector<float> x(T * hidden), want(T * hidden);
+        for (auto &v : x) v = lcg(st);
+        auto got = mxfp4::moe_forward_routed(gpu, x, routing, tab);
+        EXPECT(orc_mxfp4_moe_routed(x.data(), T, hidden, inter, alpha, clamp, E, top_k, idx.data(), w.data(), pb1.data(), ps1.data(),
+                                    pb2.data(), ps2.data(), pbi1.data(), pbi2.data(), want.data()) == 0, "oracle");
+        EXPECT(rel_err(got, want) < 2e-4, "mxfp4 moe_forward_routed: %.3g of the rms", rel_err(got, want));
+        // one token, one expert: the layer is weight * expert.forward(x)
+        std::vector<float> x0(x.begin(), x.begin() + hidden);
+        auto alone = tab[2]->forward(x0);
+        auto one = mxfp4::moe_forward_routed(gpu, x0, {{{2, 0.5f}}}, tab);
+        double worst = 0;
+        for (size_t i = 0; i < hidden; ++i) worst = std::fmax(worst, std::fabs(one[i] - 0.5f * alone[i]));
+        EXPECT(worst < 1e-5, "one pair against the expert alone: %.3g", worst);
+    }
+}
+
 int main() {
     try {
         GpuContext gpu(0);
@@ -374,6 +480,7 @@ int main() {
         test_llama_block(gpu);
         test_huffman_matmul(gpu);
         test_huffman_kv_cache(gpu);
+        test_moe_routed(gpu);
     } catch (const std::exception &e) {
         std::printf("FAIL: uncaught %s\n", e.what());
         return 2;
