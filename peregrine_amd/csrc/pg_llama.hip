@@ -231,6 +231,48 @@ __global__ __launch_bounds__(128) void rope_kernel(rope_args ra) {
     }
 }
 
+// The same for head sizes that are multiples of 8 with every pointer and stride a multiple of four floats: a
+// thread takes dims 4j .. 4j+3 and their partners half + 4j .. as 128-bit loads and stores, 256 / (hd / 8)
+// heads of one token to a workgroup (the operations per element are those of rope_kernel, in its order).
+__global__ __launch_bounds__(256) void rope_v4_kernel(rope_args ra, int total_heads) {
+    const int t = blockIdx.x, per = ra.hd >> 3;
+    const int idx = blockIdx.y * 256 + threadIdx.x;
+    int h = idx / per, s = 0;
+    const int j = idx - h * per;
+    if (h >= total_heads) return;
+    while (s < ra.nseg - 1 && h >= ra.seg[s].heads) h -= ra.seg[s++].heads;
+    const rope_seg sg = ra.seg[s];
+    const float *src = sg.src + (size_t)t * sg.src_tstride + (size_t)h * ra.hd;
+    float *dst = sg.dst + (size_t)h * sg.dst_hstride + (size_t)t * ra.hd;
+    const int half = ra.hd / 2;
+    auto at = [&](int i) {
+        float4 xp[PG_MAX_PLANES];
+#pragma unroll
+        for (int pl = 0; pl < PG_MAX_PLANES; ++pl)
+            xp[pl] = pl < sg.planes ? *reinterpret_cast<const float4 *>(src + pl * sg.plane_stride + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+        float4 x = xp[0];
+#pragma unroll
+        for (int pl = 1; pl < PG_MAX_PLANES; ++pl)
+            if (pl < sg.planes) { x.x += xp[pl].x; x.y += xp[pl].y; x.z += xp[pl].z; x.w += xp[pl].w; }
+        return x;
+    };
+    const float4 x0 = at(4 * j), x1 = at(half + 4 * j);
+    if (!sg.rotate) {
+        *reinterpret_cast<float4 *>(dst + 4 * j) = x0;
+        *reinterpret_cast<float4 *>(dst + half + 4 * j) = x1;
+        return;
+    }
+    const size_t row = (size_t)(ra.pos0 + t) * ra.hd + 4 * j;
+    const float4 c = *reinterpret_cast<const float4 *>(ra.cos_t + row), sn = *reinterpret_cast<const float4 *>(ra.sin_t + row);
+    float4 lo, hi;
+    lo.x = x0.x * c.x - x1.x * sn.x; hi.x = x0.x * sn.x + x1.x * c.x;
+    lo.y = x0.y * c.y - x1.y * sn.y; hi.y = x0.y * sn.y + x1.y * c.y;
+    lo.z = x0.z * c.z - x1.z * sn.z; hi.z = x0.z * sn.z + x1.z * c.z;
+    lo.w = x0.w * c.w - x1.w * sn.w; hi.w = x0.w * sn.w + x1.w * c.w;
+    *reinterpret_cast<float4 *>(dst + 4 * j) = lo;
+    *reinterpret_cast<float4 *>(dst + half + 4 * j) = hi;
+}
+
 // Mask kinds 0..2 as in the header; 3 = LocalGlobal (src/attention.rs:287-299): `window` is the
 // local window and bit kt of `gbits` says that key position kt is a global one.
 __device__ __forceinline__ bool attn_masked(int mask_kind, int offset, int window, int sink, const uint32_t *gbits, int qt,
@@ -1691,6 +1733,16 @@ pg_status cache_reserve(pg_ctx *ctx, pg_kv_cache *c, size_t needed) {
 
 pg_status launch_rope(pg_ctx *ctx, const rope_args &ra, size_t seq, size_t heads) {
     if (seq == 0 || heads == 0) return PG_OK;
+    bool vec = ra.hd % 8 == 0 && ra.hd <= 2048 && ((uintptr_t)ra.cos_t | (uintptr_t)ra.sin_t) % 16 == 0;
+    for (int i = 0; i < ra.nseg && vec; ++i) {
+        const rope_seg &sg = ra.seg[i];
+        vec = ((uintptr_t)sg.src | (uintptr_t)sg.dst) % 16 == 0 && sg.src_tstride % 4 == 0 && sg.dst_hstride % 4 == 0 &&
+              (sg.planes <= 1 || sg.plane_stride % 4 == 0);
+    }
+    if (vec) {
+        const size_t threads = heads * (size_t)(ra.hd / 8);
+        return pg_launch(ctx, "rope", rope_v4_kernel, dim3((unsigned)seq, (unsigned)((threads + 255) / 256)), dim3(256), 0, ra, (int)heads);
+    }
     return pg_launch(ctx, "rope", rope_kernel, dim3((unsigned)seq, (unsigned)heads), dim3(128), 0, ra);
 }
 
