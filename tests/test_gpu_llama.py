@@ -47,7 +47,7 @@ def test_rmsnorm_closed_form(ctx):
     assert (llama.RMSNorm(64, 1e-5, ctx).forward(np.zeros((1, 64), np.float32)) == 0).all()
 
 
-@pytest.mark.parametrize("hd,seq,offset", [(8, 5, 3), (128, 7, 0), (64, 1, 100), (2, 4, 1)])
+@pytest.mark.parametrize("hd,seq,offset", [(8, 5, 3), (128, 7, 0), (64, 1, 100), (2, 4, 1), (24, 9, 2), (12, 3, 0), (256, 100, 17)])
 def test_rope(ctx, orc, hd, seq, offset):
     from peregrine_amd import llama, _ffi
     say(f"rope hd={hd} seq={seq} offset={offset}")
