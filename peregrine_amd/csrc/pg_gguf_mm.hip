@@ -33,7 +33,6 @@ typedef const v4i __attribute__((address_space(1))) *gv4i_ptr;
 inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
 
 constexpr int NBU = 4;                              // blocks per stage
-constexpr int RING = 3;                             // LDS stages (two in flight beyond the one consumed)
 // LDS stage layout.  Every fill is arranged so that neighbouring lanes fetch neighbouring
 // 16-byte chunks of global memory (whole 64- or 128-byte runs per request); the chunk order
 // inside a run is XOR-swizzled so that the 128-bit LDS reads of 16 neighbouring lanes fall
@@ -49,6 +48,13 @@ template <int QT> struct MMCfg {
     static constexpr int W_WAVE = QT == 8 ? 64 * 64 : 32 * 64;  // per wavefront: [stream][4 blocks][16 B]
     static constexpr int W_FILLS = W_WAVE / 1024;               // weight fills per wavefront and stage
     static constexpr int STAGE = OFF_W + 4 * W_WAVE;            // 25.5 KiB (Q8_0) / 17.5 KiB (Q4_0)
+    // Two LDS stages (one in flight beyond the one consumed), so that THREE workgroups share a CU (three wavefronts
+    // a SIMD, 168 registers each).  Against two workgroups of three stages the expert products ran 2 % faster, the
+    // 16-row product 6 % and the 1024-row o projection 7 %: a third wavefront fills the issue slots the other two
+    // leave while they wait, which counts for more than the deeper ring.  (Three stages of the smaller Q4_0 stage,
+    // 3 x 52.5 KiB a CU, measured like two workgroups: they do not fit three at a time.)
+    static constexpr int RING = 2;
+    static constexpr int AHEAD = RING - 1;
     static constexpr int LPS = 2 + 1 + 1 + W_FILLS;             // LDS fills per wavefront and stage
 };
 
@@ -139,14 +145,14 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
 // grid: x = tiles of 128 weight rows, y = expert * tiles_per_expert + token tile, z = K chunk.
 // `chunk` (blocks per K chunk) is a multiple of NBU and no chunk is empty.
 // out: [K chunks][total pairs][n_out] (plain y with one chunk).
-// (Two wavefronts per SIMD: with at most 256 registers per lane the MFMA results are written
-// to ordinary VGPRs, not to accumulation registers that would have to be copied out first.)
+// (Three wavefronts per SIMD, 168 registers each: the MFMA results are written to ordinary VGPRs,
+// not to accumulation registers that would have to be copied out first.)
 // NT: the weight fills carry the non-temporal hint.  Right for the expert products, where a
 // weight byte is used by one or two workgroups and 1.7 GB of them per launch would otherwise
 // push the activations, digits and partial sums of the neighbouring kernels out of the caches
 // (MoE step 1.22 -> 1.17 ms); wrong for a prefill, where 32 token tiles re-read every weight.
 template <int QT, bool NT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gguf_mm_kernel(const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void gguf_mm_kernel(const uint8_t *__restrict__ qs0, const uint16_t *__restrict__ d0,
                                                       pg_mm_group grp, int n_out_arg, int nb, int nbp, int chunk,
                                                       const int8_t *__restrict__ digits, const float *__restrict__ xs,
                                                       float *__restrict__ out_arg, size_t part_stride_arg) {
@@ -454,20 +460,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n s_barrier" ::: "memory");
     };
 
+    constexpr int RING = MMCfg<QT>::RING, AHEAD = MMCfg<QT>::AHEAD;
     issue(std::integral_constant<int, 0>{}, 0);
-    if (nst > 1) issue(std::integral_constant<int, 1>{}, 1);
+    if (AHEAD > 1 && nst > 1) issue(std::integral_constant<int, 1 % RING>{}, 1);
     auto k_loop = [&](auto nr) {
         for (int s0 = 0; s0 < nst; s0 += RING) {
 #define PG_MM_STEP(U)                                                                     \
             if (s0 + U < nst) {                                                           \
                 const int s = s0 + U;                                                     \
-                wait_barrier(s + 1 < nst);                                                \
-                if (s + 2 < nst) issue(std::integral_constant<int, (U + 2) % RING>{}, s + 2); \
+                wait_barrier(AHEAD > 1 && s + 1 < nst);                                   \
+                if (s + AHEAD < nst) issue(std::integral_constant<int, (U + AHEAD) % RING>{}, s + AHEAD); \
                 compute(nr, std::integral_constant<int, U>{}, s);                         \
             }
             PG_MM_STEP(0)
             PG_MM_STEP(1)
-            PG_MM_STEP(2)
+            if constexpr (RING > 2) { PG_MM_STEP(2) }
 #undef PG_MM_STEP
         }
     };
@@ -476,13 +483,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #define PG_MM_STEP(U)                                                                     \
             if (s0 + U < nst) {                                                           \
                 const int s = s0 + U;                                                     \
-                wait_barrier(s + 1 < nst);                                                \
-                if (s + 2 < nst) issue(std::integral_constant<int, (U + 2) % RING>{}, s + 2); \
+                wait_barrier(AHEAD > 1 && s + 1 < nst);                                   \
+                if (s + AHEAD < nst) issue(std::integral_constant<int, (U + AHEAD) % RING>{}, s + AHEAD); \
                 compute_rows(std::integral_constant<int, U>{}, s);                        \
             }
             PG_MM_STEP(0)
             PG_MM_STEP(1)
-            PG_MM_STEP(2)
+            if constexpr (RING > 2) { PG_MM_STEP(2) }
 #undef PG_MM_STEP
         }
         const bool tok_ok = tt * 32 + l31 < count;  // the token whose outputs this lane accumulated
@@ -948,7 +955,7 @@ pg_status pg_launch_gguf_mm(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k_i
     }
     float *dst = ks > 1 ? part : y;
     const size_t stride = total_pairs * n_out;
-    const size_t lds = (size_t)RING * (ggml_type == PG_GGML_Q4_0 ? MMCfg<4>::STAGE : MMCfg<8>::STAGE);
+    const size_t lds = ggml_type == PG_GGML_Q4_0 ? (size_t)MMCfg<4>::RING * MMCfg<4>::STAGE : (size_t)MMCfg<8>::RING * MMCfg<8>::STAGE;
     auto launch = [&](auto kern, const char *name) -> pg_status {
         PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));
         return pg_launch(ctx, name, kern, grid, dim3(256), lds, qs, d, g2, (int)n_out, nb, nbp, chunk, md.digits, md.xs, dst,
