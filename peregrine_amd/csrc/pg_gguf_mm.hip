@@ -817,8 +817,9 @@ int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t group
                       int *chunk_out, bool *xcd_chunks) {
     const size_t nb = k_in / 32;
     const size_t wgs = ((n_out + 127) / 128) * (groups ? groups : 1);
-    // Two workgroups fit on a CU.  A short K is split only as far as every workgroup is still
-    // resident at once: a second round of workgroups would pay the start-up latency again.
+    // A short K is split only as far as every workgroup is still resident at once: a second round of
+    // workgroups would pay the start-up latency again.  (Three workgroups fit on a CU; splitting for
+    // three a CU instead of two measured the same on the 16-row product, with more partial planes to sum.)
     const size_t slots = 2 * (size_t)ctx->num_cu;
     size_t ks = slots / wgs;
     if (ks > 8) ks = 8;
