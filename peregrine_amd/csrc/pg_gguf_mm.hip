@@ -618,13 +618,83 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     const int x_rd = OFF_X + ((4 * g4) & (MT - 1)) * 32;                    // tokens 4 g4 .. + 3, 8 floats each
     const int left = 4 - 4 * (g4 >> 1);                                     // low nibbles for the even elements' half
 
-    float acc[NB][4];
+    // Up to 8 token rows (QUAD): v_mfma_i32_4x4x4_i8 instead, sixteen independent 4 x 4 x 4 products an instruction.
+    // Product b of a lane quad takes weight rows 4 (b % 4) .. + 3 against four tokens for FOUR DIFFERENT blocks of K
+    // (block lane / 16 of a group of four): lane -> weight row lane % 16 of block lane / 16, its eight operand
+    // dwords the block's 32 k; the token operand comes from lane % 4's token (one more set of instructions for
+    // tokens 4 .. 7).  The result registers are the four tokens of the lane's own row and block, so nothing of the
+    // 16 x 16 tile is padding: per block and 16 rows a quarter of the instructions of the form above, which spends
+    // them on 16 token slots whatever the count.  A lane sums blocks lane / 16, + 4, ...; the four partial sums of a
+    // row meet in the final pass through LDS.
+    constexpr bool QUAD = MT <= 8 && NB == 1;
+    constexpr int NS = QUAD ? MT / 4 : NB;  // accumulator sets: token quads, or weight tiles
+    float acc[NS][4];
 #pragma unroll
-    for (int c = 0; c < NB; ++c)
+    for (int c = 0; c < NS; ++c)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[c][i] = 0.0f;
 
+    auto consume_quad = [&](auto slot) {
+        const char *base = ring + decltype(slot)::value * UNIT;
+        const int tq = lane & 3;  // the token (of each set) whose digits this lane hands to its quad
+#pragma unroll
+        for (int J = 0; J < 2; ++J) {
+            const int blk = 4 * J + g4;
+            // the lane's row and block: 32 weight bytes as eight dwords in the order of the digit halves
+            int wk[8];
+            if constexpr (QT == 4) {
+                const v4i wr = *reinterpret_cast<const v4i *>(base + fr * 128 + ((blk ^ w_sw) * 16));
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    wk[p] = nibbles_to_i8x16(wr[p], 4);      // low nibbles: the even elements (digit half 0)
+                    wk[4 + p] = nibbles_to_i8x16(wr[p], 0);  // high nibbles: the odd ones (half 1)
+                }
+            } else {
+                const v4i w0 = *reinterpret_cast<const v4i *>(base + fr * 128 + ((blk ^ w_sw) * 16));
+                const v4i w1 = *reinterpret_cast<const v4i *>(base + (16 + fr) * 128 + ((blk ^ w_sw) * 16));
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    wk[p] = w0[p];
+                    wk[4 + p] = w1[p];
+                }
+            }
+            const float dv = half_bits_to_float(*reinterpret_cast<const unsigned short *>(base + ds_rd + blk * 16));
+#pragma unroll
+            for (int s2 = 0; s2 < NS; ++s2) {
+                const int tok = 4 * s2 + tq;
+                const char *dg = base + OFF_DG + tok * 512;
+                const v4i h0 = *reinterpret_cast<const v4i *>(dg + (((2 * blk) ^ tok) * 16));
+                const v4i h1 = *reinterpret_cast<const v4i *>(dg + (((2 * blk + 1) ^ tok) * 16));
+                const v4i l0 = *reinterpret_cast<const v4i *>(dg + 256 + (((2 * blk) ^ tok) * 16));
+                const v4i l1 = *reinterpret_cast<const v4i *>(dg + 256 + (((2 * blk + 1) ^ tok) * 16));
+                int sx[4];  // the scales of tokens 4 s2 .. + 3 for this lane's block (read as integers: see gguf_mm_kernel)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sx[i] = *reinterpret_cast<const int *>(base + OFF_X + (4 * s2 + i) * 32 + blk * 4);
+                v4i ihi = {0, 0, 0, 0}, ilo = {0, 0, 0, 0};
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    ihi = __builtin_amdgcn_mfma_i32_4x4x4i8(h0[p], wk[p], ihi, 0, 0, 0);  // rows = tokens, columns = weight rows
+                    ilo = __builtin_amdgcn_mfma_i32_4x4x4i8(l0[p], wk[p], ilo, 0, 0, 0);
+                }
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    ihi = __builtin_amdgcn_mfma_i32_4x4x4i8(h1[p], wk[4 + p], ihi, 0, 0, 0);
+                    ilo = __builtin_amdgcn_mfma_i32_4x4x4i8(l1[p], wk[4 + p], ilo, 0, 0, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float fx = (float)(ihi[i] * 256 + ilo[i]) * __int_as_float(sx[i]);
+                    acc[s2][i] = fmaf(dv, fx, acc[s2][i]);
+                }
+            }
+        }
+    };
+
     auto consume = [&](auto slot) {
+        if constexpr (QUAD) {
+            consume_quad(slot);
+            return;
+        }
         const char *base = ring + decltype(slot)::value * UNIT;
         // the scales of this lane's four tokens for the unit's eight blocks (read as integers: see gguf_mm_kernel)
         int sx[4][8];
@@ -725,12 +795,28 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
         }
     }
     __syncthreads();  // the rings are done with: their space takes the wavefronts' tiles
-    float *red = reinterpret_cast<float *>(lds);  // [NW][NB][4][64]
+    float *red = reinterpret_cast<float *>(lds);  // [NW][NS][4][64]
 #pragma unroll
-    for (int c = 0; c < NB; ++c)
+    for (int c = 0; c < NS; ++c)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) red[((wave * NB + c) * 4 + i) * 64 + lane] = acc[c][i];
+        for (int i = 0; i < 4; ++i) red[((wave * NS + c) * 4 + i) * 64 + lane] = acc[c][i];
     __syncthreads();
+    if constexpr (QUAD) {
+        for (int e = threadIdx.x; e < NS * 4 * 16; e += 64 * NW) {
+            const int r = e & 15, i = (e >> 4) & 3, c = e >> 6;
+            float sum = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w)  // ascending runs of K, within a run the four block classes in order
+#pragma unroll
+                for (int q = 0; q < 4; ++q) sum += red[((w * NS + c) * 4 + i) * 64 + 16 * q + r];
+            const int tok = 4 * c + i, row = n0 + r;
+            if (tok < m && row < n_out) {
+                const float v = QT == 4 ? sum * 0.0625f : sum;  // (Q4_0: the weight operand was 16 * (q - 8))
+                y[(size_t)tok * n_out + row] = res ? res[(size_t)tok * n_out + row] + v : v;
+            }
+        }
+        return;
+    }
     for (int e = threadIdx.x; e < NB * 4 * 64; e += 64 * NW) {
         const int l = e & 63, i = (e >> 6) & 3, c = e >> 8;
         float sum = red[(c * 4 + i) * 64 + l];
