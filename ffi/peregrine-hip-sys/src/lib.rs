@@ -185,7 +185,7 @@ extern "C" {
     pub fn pg_audit_gemv_w8a8_m1(k: usize, n: usize, nch: c_int, rows_per_wavefront: c_int, wavefronts: c_int, f32_row: c_int, w_end: *mut usize, w_bytes: *mut usize, x_end: *mut usize, x_bytes: *mut usize) -> pg_status;
     pub fn pg_audit_gemm_w8a8_skinny(m: usize, k: usize, n: usize, activation_tiles: c_int, weight_tiles: c_int, wavefronts: c_int, w_end: *mut usize, w_bytes: *mut usize, a_end: *mut usize, a_bytes: *mut usize) -> pg_status;
     pub fn pg_audit_gguf_gemv(n_out: usize, k_in: usize, q8: c_int, blocks_per_lane: c_int, rows_per_wavefront: c_int, wavefronts: c_int, qs_end: *mut usize, qs_bytes: *mut usize, d_end: *mut usize, d_bytes: *mut usize) -> pg_status;
-    pub fn pg_audit_gguf_skinny(n_out: usize, k_in: usize, q8: c_int, wavefronts: c_int, qs_end: *mut usize, qs_bytes: *mut usize, d_end: *mut usize, d_bytes: *mut usize) -> pg_status;
+    pub fn pg_audit_gguf_skinny(n_out: usize, k_in: usize, q8: c_int, wavefronts: c_int, weight_tiles: c_int, qs_end: *mut usize, qs_bytes: *mut usize, d_end: *mut usize, d_bytes: *mut usize) -> pg_status;
     pub fn pg_audit_gguf_hmm(m: usize, n_out: usize, k_in: usize, q8: c_int, wide_tiles: c_int, k_chunks: c_int, plane_end: *mut usize, plane_bytes: *mut usize, qs_end: *mut usize, qs_bytes: *mut usize, d_end: *mut usize, d_bytes: *mut usize) -> pg_status;
     pub fn pg_audit_mxfp4_rows(out_dim: usize, in_dim: usize, row_groups_per_workgroup: c_int, wavefronts: c_int, qs_end: *mut usize, qs_bytes: *mut usize, sc_end: *mut usize, sc_bytes: *mut usize) -> pg_status;
     pub fn pg_audit_mxfp4_tiles(num_cu: c_int, out_dim: usize, in_dim: usize, m: usize, qs_end: *mut usize, qs_bytes: *mut usize, sc_end: *mut usize, sc_bytes: *mut usize, rec_end: *mut usize, rec_bytes: *mut usize, ra: *mut c_int, tb: *mut c_int, ks: *mut c_int) -> pg_status;

@@ -614,8 +614,8 @@ pg_status pg_audit_gemm_w8a8_skinny(size_t m, size_t k, size_t n, int activation
                                     size_t *w_end, size_t *w_bytes, size_t *a_end, size_t *a_bytes);
 pg_status pg_audit_gguf_gemv(size_t n_out, size_t k_in, int q8, int blocks_per_lane, int rows_per_wavefront,
                              int wavefronts, size_t *qs_end, size_t *qs_bytes, size_t *d_end, size_t *d_bytes);
-pg_status pg_audit_gguf_skinny(size_t n_out, size_t k_in, int q8, int wavefronts, size_t *qs_end, size_t *qs_bytes,
-                               size_t *d_end, size_t *d_bytes);
+pg_status pg_audit_gguf_skinny(size_t n_out, size_t k_in, int q8, int wavefronts, int weight_tiles, size_t *qs_end,
+                               size_t *qs_bytes, size_t *d_end, size_t *d_bytes);
 pg_status pg_audit_gguf_hmm(size_t m, size_t n_out, size_t k_in, int q8, int wide_tiles, int k_chunks, size_t *plane_end,
                             size_t *plane_bytes, size_t *qs_end, size_t *qs_bytes, size_t *d_end, size_t *d_bytes);
 pg_status pg_audit_mxfp4_rows(size_t out_dim, size_t in_dim, int row_groups_per_workgroup, int wavefronts,

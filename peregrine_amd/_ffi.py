@@ -70,7 +70,7 @@ SIGNATURES = {
     "pg_audit_gemm_w8a8_skinny": [_sz, _sz, _sz, _int, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "pg_audit_gguf_gemv": [_sz, _sz, _int, _int, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "pg_audit_gguf_hmm": [_sz, _sz, _sz, _int, _int, _int] + [C.POINTER(C.c_size_t)] * 6,
-    "pg_audit_gguf_skinny": [_sz, _sz, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
+    "pg_audit_gguf_skinny": [_sz, _sz, _int, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "pg_audit_mxfp4_tiles": [_int, _sz, _sz, _sz] + [C.POINTER(C.c_size_t)] * 6 + [C.POINTER(_int)] * 3,
     "pg_audit_mxfp4_rows": [_sz, _sz, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "pg_audit_probe_read": [_sz, _int, _int, _int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],

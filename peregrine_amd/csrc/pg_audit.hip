@@ -112,16 +112,16 @@ PG_API pg_status pg_audit_gguf_gemv(size_t n_out, size_t k_in, int q8, int bpl, 
     return PG_OK;
 }
 
-// 2 .. 16 rows in one launch over a block tensor (gguf_skinny_kernel<QT, 1, MT, NW, NST>): K in units of 8 blocks
-// (k_in % 256 == 0), a workgroup of nw wavefronts per 16 weight rows.
-PG_API pg_status pg_audit_gguf_skinny(size_t n_out, size_t k_in, int q8, int nw, size_t *qs_end, size_t *qs_bytes, size_t *d_end,
-                                      size_t *d_bytes) {
-    PG_CHECK_ARG(n_out > 0 && k_in >= 256 && k_in % 256 == 0 && nw > 0, "pg_audit_gguf_skinny: bad arguments");
+// 2 .. 16 rows in one launch over a block tensor (gguf_skinny_kernel<QT, NB, MT, NW, NST>): K in units of 8 blocks
+// (k_in % 256 == 0), a workgroup of nw wavefronts per `tiles` tiles of 16 weight rows.
+PG_API pg_status pg_audit_gguf_skinny(size_t n_out, size_t k_in, int q8, int nw, int tiles, size_t *qs_end, size_t *qs_bytes,
+                                      size_t *d_end, size_t *d_bytes) {
+    PG_CHECK_ARG(n_out > 0 && k_in >= 256 && k_in % 256 == 0 && nw > 0 && (tiles == 1 || tiles == 2), "pg_audit_gguf_skinny: bad arguments");
     const int nb = (int)(k_in / 32), wf = q8 ? 4 : 2, units = nb / 8, per = (units + nw - 1) / nw, ntile = (int)((n_out + 7) / 8);
     span_check qs, d;
-    const int wgs = (int)((n_out + 15) / 16);
+    const int wgs = (int)((n_out + 16 * tiles - 1) / (16 * tiles));
     for (int wg = 0; wg < wgs; ++wg) {
-        const int n0 = wg * 16;
+        const int n0 = wg * 16 * tiles;
         for (int wave = 0; wave < nw; ++wave) {
             const int u_begin = wave * per, u_end = std::min(u_begin + per, units), cnt = u_end - u_begin;
             if (cnt <= 0) continue;
@@ -131,10 +131,12 @@ PG_API pg_status pg_audit_gguf_skinny(size_t n_out, size_t k_in, int q8, int nw,
                 for (int lane = 0; lane < 64; ++lane) {
                     for (int j = 0; j < wf; ++j) {
                         const int slot = 8 * j + (lane >> 3), r = slot & 15, half = slot >> 4, ch = (lane & 7) ^ ((r >> 1) & 7);
-                        const int row = pg_gemv_clamp_row(n0 + r, (int)n_out);
-                        qs.touch(pg_gskinny_weight_offset(q8 ? (size_t)row * 2 + half : (size_t)row, nb, unit, ch), 16);
+                        for (int c = 0; c < tiles; ++c) {
+                            const int row = pg_gemv_clamp_row(n0 + 16 * c + r, (int)n_out);
+                            qs.touch(pg_gskinny_weight_offset(q8 ? (size_t)row * 2 + half : (size_t)row, nb, unit, ch), 16);
+                        }
                     }
-                    if (lane < 16) d.touch(pg_gskinny_scale_offset(pg_gskinny_scale_tile(n0, lane, ntile), nb, unit, lane), 16);
+                    if (lane < 16 * tiles) d.touch(pg_gskinny_scale_offset(pg_gskinny_scale_tile(n0, lane, ntile), nb, unit, lane), 16);
                 }
             }
         }

@@ -546,7 +546,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 // Up to three tensors of equal K in one launch (q|k|v, gate|up of models::llama): tensor g owns the workgroups
 // wg0[g] .. wg0[g + 1] - 1 (unused slots hold INT_MAX).
 template <int QT, int NB, int MT, int NW, int NST>
-__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void gguf_skinny_kernel(const pg_skinny_group grp, int nb, int nbp, int m,
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, (MT <= 8 && NST <= 2) ? 4 : 2))) void gguf_skinny_kernel(const pg_skinny_group grp, int nb, int nbp, int m,
                                                                     const int8_t *__restrict__ digits, const float *__restrict__ xs) {
     int tg = 0;
 #pragma unroll
@@ -626,8 +626,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     // 16 x 16 tile is padding: per block and 16 rows a quarter of the instructions of the form above, which spends
     // them on 16 token slots whatever the count.  A lane sums blocks lane / 16, + 4, ...; the four partial sums of a
     // row meet in the final pass through LDS.
-    constexpr bool QUAD = MT <= 8 && NB == 1;
-    constexpr int NS = QUAD ? MT / 4 : NB;  // accumulator sets: token quads, or weight tiles
+    constexpr bool QUAD = MT <= 8;
+    constexpr int NQ = QUAD ? MT / 4 : 1, NS = NB * NQ;  // accumulator sets: weight tiles x token quads
     float acc[NS][4];
 #pragma unroll
     for (int c = 0; c < NS; ++c)
@@ -640,27 +640,32 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
         for (int J = 0; J < 2; ++J) {
             const int blk = 4 * J + g4;
-            // the lane's row and block: 32 weight bytes as eight dwords in the order of the digit halves
-            int wk[8];
-            if constexpr (QT == 4) {
-                const v4i wr = *reinterpret_cast<const v4i *>(base + fr * 128 + ((blk ^ w_sw) * 16));
+            // the lane's rows (one a tile) and block: 32 weight bytes each as eight dwords in the order of the digit halves
+            int wk[NB][8];
+            float dv[NB];
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    wk[p] = nibbles_to_i8x16(wr[p], 4);      // low nibbles: the even elements (digit half 0)
-                    wk[4 + p] = nibbles_to_i8x16(wr[p], 0);  // high nibbles: the odd ones (half 1)
-                }
-            } else {
-                const v4i w0 = *reinterpret_cast<const v4i *>(base + fr * 128 + ((blk ^ w_sw) * 16));
-                const v4i w1 = *reinterpret_cast<const v4i *>(base + (16 + fr) * 128 + ((blk ^ w_sw) * 16));
+            for (int c = 0; c < NB; ++c) {
+                const char *wt = base + c * W_T;
+                if constexpr (QT == 4) {
+                    const v4i wr = *reinterpret_cast<const v4i *>(wt + fr * 128 + ((blk ^ w_sw) * 16));
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    wk[p] = w0[p];
-                    wk[4 + p] = w1[p];
+                    for (int p = 0; p < 4; ++p) {
+                        wk[c][p] = nibbles_to_i8x16(wr[p], 4);      // low nibbles: the even elements (digit half 0)
+                        wk[c][4 + p] = nibbles_to_i8x16(wr[p], 0);  // high nibbles: the odd ones (half 1)
+                    }
+                } else {
+                    const v4i w0 = *reinterpret_cast<const v4i *>(wt + fr * 128 + ((blk ^ w_sw) * 16));
+                    const v4i w1 = *reinterpret_cast<const v4i *>(wt + (16 + fr) * 128 + ((blk ^ w_sw) * 16));
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        wk[c][p] = w0[p];
+                        wk[c][4 + p] = w1[p];
+                    }
                 }
+                dv[c] = half_bits_to_float(*reinterpret_cast<const unsigned short *>(base + ds_rd + c * D_T + blk * 16));
             }
-            const float dv = half_bits_to_float(*reinterpret_cast<const unsigned short *>(base + ds_rd + blk * 16));
 #pragma unroll
-            for (int s2 = 0; s2 < NS; ++s2) {
+            for (int s2 = 0; s2 < NQ; ++s2) {
                 const int tok = 4 * s2 + tq;
                 const char *dg = base + OFF_DG + tok * 512;
                 const v4i h0 = *reinterpret_cast<const v4i *>(dg + (((2 * blk) ^ tok) * 16));
@@ -670,21 +675,24 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 int sx[4];  // the scales of tokens 4 s2 .. + 3 for this lane's block (read as integers: see gguf_mm_kernel)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) sx[i] = *reinterpret_cast<const int *>(base + OFF_X + (4 * s2 + i) * 32 + blk * 4);
-                v4i ihi = {0, 0, 0, 0}, ilo = {0, 0, 0, 0};
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    ihi = __builtin_amdgcn_mfma_i32_4x4x4i8(h0[p], wk[p], ihi, 0, 0, 0);  // rows = tokens, columns = weight rows
-                    ilo = __builtin_amdgcn_mfma_i32_4x4x4i8(l0[p], wk[p], ilo, 0, 0, 0);
-                }
+                for (int c = 0; c < NB; ++c) {
+                    v4i ihi = {0, 0, 0, 0}, ilo = {0, 0, 0, 0};
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    ihi = __builtin_amdgcn_mfma_i32_4x4x4i8(h1[p], wk[4 + p], ihi, 0, 0, 0);
-                    ilo = __builtin_amdgcn_mfma_i32_4x4x4i8(l1[p], wk[4 + p], ilo, 0, 0, 0);
-                }
+                    for (int p = 0; p < 4; ++p) {
+                        ihi = __builtin_amdgcn_mfma_i32_4x4x4i8(h0[p], wk[c][p], ihi, 0, 0, 0);  // rows = tokens, columns = weight rows
+                        ilo = __builtin_amdgcn_mfma_i32_4x4x4i8(l0[p], wk[c][p], ilo, 0, 0, 0);
+                    }
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float fx = (float)(ihi[i] * 256 + ilo[i]) * __int_as_float(sx[i]);
-                    acc[s2][i] = fmaf(dv, fx, acc[s2][i]);
+                    for (int p = 0; p < 4; ++p) {
+                        ihi = __builtin_amdgcn_mfma_i32_4x4x4i8(h1[p], wk[c][4 + p], ihi, 0, 0, 0);
+                        ilo = __builtin_amdgcn_mfma_i32_4x4x4i8(l1[p], wk[c][4 + p], ilo, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float fx = (float)(ihi[i] * 256 + ilo[i]) * __int_as_float(sx[i]);
+                        acc[c * NQ + s2][i] = fmaf(dv[c], fx, acc[c * NQ + s2][i]);
+                    }
                 }
             }
         }
@@ -803,13 +811,13 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     __syncthreads();
     if constexpr (QUAD) {
         for (int e = threadIdx.x; e < NS * 4 * 16; e += 64 * NW) {
-            const int r = e & 15, i = (e >> 4) & 3, c = e >> 6;
+            const int r = e & 15, i = (e >> 4) & 3, c = e >> 6;  // c = tile * NQ + token quad
             float sum = 0.0f;
 #pragma unroll
             for (int w = 0; w < NW; ++w)  // ascending runs of K, within a run the four block classes in order
 #pragma unroll
                 for (int q = 0; q < 4; ++q) sum += red[((w * NS + c) * 4 + i) * 64 + 16 * q + r];
-            const int tok = 4 * c + i, row = n0 + r;
+            const int tok = 4 * (c % NQ) + i, row = n0 + 16 * (c / NQ) + r;
             if (tok < m && row < n_out) {
                 const float v = QT == 4 ? sum * 0.0625f : sum;  // (Q4_0: the weight operand was 16 * (q - 8))
                 y[(size_t)tok * n_out + row] = res ? res[(size_t)tok * n_out + row] + v : v;
@@ -957,7 +965,12 @@ pg_status pg_launch_gguf_skinny_group(pg_ctx *ctx, int ggml_type, size_t k_in, c
     // Wavefronts (runs of K) per workgroup: as many as keep every workgroup resident at once.  The rings: units of
     // 4.75 / 6.75 / 10.75 KiB for 4 / 8 / 16 token rows (Q8_0: 2 KiB more), as many stages as let eight wavefronts
     // share a CU's LDS (16 token rows: two stages and six or seven wavefronts; three stages and four were slower).
-    const int per_cu = m <= 8 ? 8 : (q8 ? 6 : 7);
+    // Two weight tiles a workgroup (32 rows) where that still leaves a workgroup for every CU: the digits, which
+    // every workgroup fetches for all of K, then cost half as much per weight byte.
+    const int tiles = (m <= 8 && n_total / 32 >= (size_t)ctx->num_cu) ? 2 : 1;
+    const size_t unit_bytes = (size_t)tiles * ((q8 ? 4096 : 2048) + 256) + (m <= 4 ? 4 : (m <= 8 ? 8 : 16)) * 512 + 512;
+    const int stages = 2;
+    const int per_cu = m <= 8 ? (int)std::min<size_t>(16, (160u << 10) / (stages * unit_bytes)) : (q8 ? 6 : 7);
     pg_skinny_group grp;
     int wgs = 0;
     for (int i = 0; i < 3; ++i) {
@@ -968,40 +981,40 @@ pg_status pg_launch_gguf_skinny_group(pg_ctx *ctx, int ggml_type, size_t k_in, c
         grp.res[i] = i == 0 ? residual : nullptr;
         grp.n[i] = used ? (int)w[i]->n_out : 0;
         grp.wg0[i] = used ? wgs : INT_MAX;
-        if (used) wgs += (int)((w[i]->n_out + 15) / 16);
+        if (used) wgs += (int)((w[i]->n_out + 16 * tiles - 1) / (16 * tiles));
     }
     const dim3 grid((unsigned)wgs);
     const size_t slots = (size_t)ctx->num_cu * per_cu, units = (size_t)nb / 8;
     int nw = m <= 8 ? 8 : 4;
     while (nw > 1 && ((size_t)grid.x * nw > slots || units / nw < 4)) nw >>= 1;
-#define PG_GSK_LAUNCH(QTT, MTT, NWW, NSTT)                                                                                     \
+#define PG_GSK_LAUNCH(QTT, NBB, MTT, NWW, NSTT)                                                                                \
     do {                                                                                                                       \
-        auto kern = gguf_skinny_kernel<QTT, 1, MTT, NWW, NSTT>;                                                                \
-        const size_t lds = (size_t)NWW * NSTT * ((QTT == 8 ? 4096 : 2048) + 256 + MTT * 512 + 512);                            \
+        auto kern = gguf_skinny_kernel<QTT, NBB, MTT, NWW, NSTT>;                                                              \
+        const size_t lds = (size_t)NWW * NSTT * (NBB * ((QTT == 8 ? 4096 : 2048) + 256) + MTT * 512 + 512);                    \
         PG_TRY(pg_allow_dynamic_lds(ctx, (const void *)kern, lds));                                                            \
         return pg_launch(ctx, QTT == 8 ? "gguf_q8_0_few_rows_mm" : "gguf_q4_0_few_rows_mm", kern, grid, dim3(64 * NWW), lds,  \
                          grp, nb, nbp, (int)m, (const int8_t *)md.digits, (const float *)md.xs);                               \
     } while (0)
-#define PG_GSK_NW8(QTT, MTT, NSTT)                     \
-    switch (nw) {                                      \
-        case 8: PG_GSK_LAUNCH(QTT, MTT, 8, NSTT);      \
-        case 4: PG_GSK_LAUNCH(QTT, MTT, 4, NSTT);      \
-        case 2: PG_GSK_LAUNCH(QTT, MTT, 2, NSTT);      \
-        default: PG_GSK_LAUNCH(QTT, MTT, 1, NSTT);     \
+#define PG_GSK_NW8(QTT, NBB, MTT, NSTT)                     \
+    switch (nw) {                                           \
+        case 8: PG_GSK_LAUNCH(QTT, NBB, MTT, 8, NSTT);      \
+        case 4: PG_GSK_LAUNCH(QTT, NBB, MTT, 4, NSTT);      \
+        case 2: PG_GSK_LAUNCH(QTT, NBB, MTT, 2, NSTT);      \
+        default: PG_GSK_LAUNCH(QTT, NBB, MTT, 1, NSTT);     \
     }
-#define PG_GSK_NW4(QTT, MTT, NSTT)                     \
-    switch (nw) {                                      \
-        case 4: PG_GSK_LAUNCH(QTT, MTT, 4, NSTT);      \
-        case 2: PG_GSK_LAUNCH(QTT, MTT, 2, NSTT);      \
-        default: PG_GSK_LAUNCH(QTT, MTT, 1, NSTT);     \
+#define PG_GSK_NW4(QTT, MTT, NSTT)                        \
+    switch (nw) {                                         \
+        case 4: PG_GSK_LAUNCH(QTT, 1, MTT, 4, NSTT);      \
+        case 2: PG_GSK_LAUNCH(QTT, 1, MTT, 2, NSTT);      \
+        default: PG_GSK_LAUNCH(QTT, 1, MTT, 1, NSTT);     \
     }
     if (q8) {
-        if (m <= 4) PG_GSK_NW8(8, 4, 2)
-        if (m <= 8) PG_GSK_NW8(8, 8, 2)
+        if (m <= 4) { if (tiles == 2) PG_GSK_NW8(8, 2, 4, 2) else PG_GSK_NW8(8, 1, 4, 2) }
+        if (m <= 8) { if (tiles == 2) PG_GSK_NW8(8, 2, 8, 2) else PG_GSK_NW8(8, 1, 8, 2) }
         PG_GSK_NW4(8, 16, 2)
     }
-    if (m <= 4) PG_GSK_NW8(4, 4, 4)
-    if (m <= 8) PG_GSK_NW8(4, 8, 2)
+    if (m <= 4) { if (tiles == 2) PG_GSK_NW8(4, 2, 4, 2) else PG_GSK_NW8(4, 1, 4, 2) }
+    if (m <= 8) { if (tiles == 2) PG_GSK_NW8(4, 2, 8, 2) else PG_GSK_NW8(4, 1, 8, 2) }
     PG_GSK_NW4(4, 16, 2)
 #undef PG_GSK_NW8
 #undef PG_GSK_NW4

@@ -94,12 +94,12 @@ def test_block_gemv_loads_stay_inside_payload_and_scale_planes():
 
 
 def test_block_few_rows_fills_stay_inside_payload_and_scale_planes():
-    """gguf_skinny_kernel: K a multiple of 256, every wavefront count."""
+    """gguf_skinny_kernel: K a multiple of 256, every wavefront count, one or two weight tiles a workgroup."""
     for k, n in itertools.product([1024, 1280, 4096, 14336, 32768], RAGGED_N + [14336]):
-        for q8, nw in itertools.product((0, 1), (1, 2, 4, 8)):
+        for q8, nw, tiles in itertools.product((0, 1), (1, 2, 4, 8), (1, 2)):
             v = _four()
-            check(lib.pg_audit_gguf_skinny(n, k, q8, nw, *[C.byref(x) for x in v]))
-            qs_end, qs_bytes, d_end, d_bytes = _inside(v, f"gguf_skinny n={n} k={k} q8={q8} NW={nw}")
+            check(lib.pg_audit_gguf_skinny(n, k, q8, nw, tiles, *[C.byref(x) for x in v]))
+            qs_end, qs_bytes, d_end, d_bytes = _inside(v, f"gguf_skinny n={n} k={k} q8={q8} NW={nw} NB={tiles}")
             assert qs_end == qs_bytes and d_end == d_bytes
 
 
@@ -158,4 +158,4 @@ def test_audit_argument_errors():
     with pytest.raises(_ffi.PeregrineError):
         check(lib.pg_audit_gemv_w8a8_m1(4096, 16, 1, 1, 4, 0, *[C.byref(x) for x in v]))   # NCH too small for the row
     with pytest.raises(_ffi.PeregrineError):
-        check(lib.pg_audit_gguf_skinny(16, 1000, 0, 4, *[C.byref(x) for x in v]))          # K not a multiple of 256
+        check(lib.pg_audit_gguf_skinny(16, 1000, 0, 4, 1, *[C.byref(x) for x in v]))          # K not a multiple of 256
