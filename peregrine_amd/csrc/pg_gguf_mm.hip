@@ -546,7 +546,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 // Up to three tensors of equal K in one launch (q|k|v, gate|up of models::llama): tensor g owns the workgroups
 // wg0[g] .. wg0[g + 1] - 1 (unused slots hold INT_MAX).
 template <int QT, int NB, int MT, int NW, int NST>
-__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, (MT <= 8 && NST <= 2) ? 4 : 2))) void gguf_skinny_kernel(const pg_skinny_group grp, int nb, int nbp, int m,
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, MT <= 8 ? 4 : 2))) void gguf_skinny_kernel(const pg_skinny_group grp, int nb, int nbp, int m,
                                                                     const int8_t *__restrict__ digits, const float *__restrict__ xs) {
     int tg = 0;
 #pragma unroll
@@ -939,13 +939,14 @@ int pg_gguf_mm_splitk(const pg_ctx *ctx, size_t n_out, size_t k_in, size_t group
     return (int)ks_real;
 }
 
-// Up to 16 rows over a Q4_0 tensor whose K is a multiple of 256: the one-launch product (see the kernel).  The
-// kernel is bound by instruction issue (about 500 instructions per 8 blocks and weight tile pair, most of them the
-// per-block scaling), so what counts is wavefronts per SIMD, and LDS decides that: up to 8 token rows the rings are
-// small enough for eight wavefronts a CU (4096 -> 14336, us with the digits' launch: 4 rows 14.5, 8 rows 15.2,
-// against 19.5 and 18.0 for digits + product over four K chunks + their sum); with 16 token rows seven fit at two
-// units a ring, which beats the three launches only where those are short of workgroups (14336 -> 4096: 18.2
-// against 24.3; 4096 -> 4096: 8.8 against 13.3; but 4096 -> 14336: 21.5 against 20.0-22.0).
+// Up to 16 rows over a Q4_0 or Q8_0 tensor whose K is a multiple of 256: the one-launch product (see the kernel).
+// With 9 .. 16 token rows (the 16 x 16 x 32 form) the kernel is bound by instruction issue (about 500 instructions per
+// 8 blocks and weight tile, most of them the per-block scaling of 16 token slots), seven wavefronts fit a CU at two
+// units a ring, and it beats digits + product over K chunks + their sum only where those are short of workgroups
+// (14336 -> 4096: 18.2 against 24.3 us; 4096 -> 4096: 8.8 against 13.3; but 4096 -> 14336: 21.5 against 20.0 - 22.0).
+// Up to 8 token rows (the 4 x 4 x 4 form) a quarter of those instructions remain and the kernel is bound by how many
+// bytes its rings keep in flight: 4 x 4096 -> 14336 takes 9.0 us (with its arithmetic switched off 8.6 - 9.1; in the
+// 16 x 16 x 32 form it took 11.9).
 bool pg_gguf_skinny_takes(const pg_ctx *ctx, int ggml_type, size_t m, size_t n_out, size_t k_in) {
     return (ggml_type == PG_GGML_Q4_0 || ggml_type == PG_GGML_Q8_0) && m >= 2 && (m <= 8 || (m <= 16 && n_out / 32 < (size_t)ctx->num_cu)) &&
            k_in % 256 == 0 && k_in >= 1024 && n_out >= 1 && n_out < (1u << 30) && k_in < (1u << 24);
@@ -969,8 +970,8 @@ pg_status pg_launch_gguf_skinny_group(pg_ctx *ctx, int ggml_type, size_t k_in, c
     // every workgroup fetches for all of K, then cost half as much per weight byte.
     const int tiles = (m <= 8 && n_total / 32 >= (size_t)ctx->num_cu) ? 2 : 1;
     const size_t unit_bytes = (size_t)tiles * ((q8 ? 4096 : 2048) + 256) + (m <= 4 ? 4 : (m <= 8 ? 8 : 16)) * 512 + 512;
-    const int stages = 2;
-    const int per_cu = m <= 8 ? (int)std::min<size_t>(16, (160u << 10) / (stages * unit_bytes)) : (q8 ? 6 : 7);
+    const int stages = 2;  // (three stages on fewer wavefronts: 10.7 - 10.9 against 9.0 us on 4 x 4096 -> 14336)
+    const size_t lds_cu = 160u << 10;
     pg_skinny_group grp;
     int wgs = 0;
     for (int i = 0; i < 3; ++i) {
@@ -984,9 +985,15 @@ pg_status pg_launch_gguf_skinny_group(pg_ctx *ctx, int ggml_type, size_t k_in, c
         if (used) wgs += (int)((w[i]->n_out + 16 * tiles - 1) / (16 * tiles));
     }
     const dim3 grid((unsigned)wgs);
-    const size_t slots = (size_t)ctx->num_cu * per_cu, units = (size_t)nb / 8;
+    // LDS is handed out per workgroup: nw wavefronts' rings each; up to 16 wavefronts a CU (4 a SIMD)
+    const size_t units = (size_t)nb / 8;
+    auto fits = [&](int nw_) {
+        if (m > 8) return (size_t)grid.x * nw_ <= (size_t)ctx->num_cu * (q8 ? 6 : 7);
+        const size_t per_cu = std::min<size_t>(lds_cu / ((size_t)nw_ * stages * unit_bytes), 16 / nw_);
+        return (size_t)grid.x <= (size_t)ctx->num_cu * per_cu;
+    };
     int nw = m <= 8 ? 8 : 4;
-    while (nw > 1 && ((size_t)grid.x * nw > slots || units / nw < 4)) nw >>= 1;
+    while (nw > 1 && (!fits(nw) || units / nw < 4)) nw >>= 1;
 #define PG_GSK_LAUNCH(QTT, NBB, MTT, NWW, NSTT)                                                                                \
     do {                                                                                                                       \
         auto kern = gguf_skinny_kernel<QTT, NBB, MTT, NWW, NSTT>;                                                              \
