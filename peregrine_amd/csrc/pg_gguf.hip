@@ -925,19 +925,18 @@ pg_status pg_launch_gguf_gemv(pg_ctx *ctx, int ggml_type, size_t n_out, size_t k
 // grows by the arithmetic of every further row and by the digits of K m elements that every workgroup makes; the
 // matrix-core routes' hardly at all, but they start with a launch for the digits: us, rows 2 / 3 / 4, against
 // digits + one matrix-core launch at 4 rows: 4096 -> 14336 12.2 / 16.2 / 19.9 against 14.4; 4096 -> 4096 6.7 / 8.6 /
-// 10.4 against 8.2; 14336 -> 4096 17.8 / 24.1 / - against 14.3.
+// 10.4 against 8.2; 14336 -> 4096 17.8 / 24.1 / - against 14.3.  Since the matrix-core route for up to 8 rows moved to
+// 4 x 4 x 4 products (4096 -> 14336 11.0 us, 14336 -> 4096 11.8, 4096 -> 4096 7.7, 4096 -> 6144 8.4 at 2 .. 4 rows)
+// this kernel keeps two rows over small tensors only (4096 -> 4096: 6.8).
 bool pg_gguf_gemv_takes_few_rows(int ggml_type, size_t m, size_t n_out, size_t k_in, const float *x_f32) {
-    return ggml_type == PG_GGML_Q4_0 && (m == 2 || (m == 3 && n_out * k_in <= ((size_t)1 << 25))) && k_in >= 32 && k_in <= 8192 &&
+    return ggml_type == PG_GGML_Q4_0 && m == 2 && n_out * k_in <= ((size_t)1 << 24) && k_in >= 32 && k_in <= 8192 &&
            fewrows_lds(m, k_in) <= 150 * 1024 && (uintptr_t)x_f32 % 16 == 0;
 }
 
 pg_status pg_launch_gguf_gemv_few_rows(pg_ctx *ctx, size_t n_out, size_t k_in, const uint8_t *qs, const uint16_t *d, const float *x_f32,
                                        size_t m, float *y) {
-#define PG_FEWROWS_BPL(B)                                                                   \
-    (m == 2 ? launch_gemv_fewrows_bpl<B, 2>(ctx, n_out, k_in, qs, d, x_f32, y)                  \
-            : m == 3 ? launch_gemv_fewrows_bpl<B, 3>(ctx, n_out, k_in, qs, d, x_f32, y)         \
-                     : launch_gemv_fewrows_bpl<B, 4>(ctx, n_out, k_in, qs, d, x_f32, y))
-    if (m < 2 || m > 4) return pg_fail(PG_EINVAL, "gguf_gemv (few rows): %zu rows", m);
+#define PG_FEWROWS_BPL(B) launch_gemv_fewrows_bpl<B, 2>(ctx, n_out, k_in, qs, d, x_f32, y)
+    if (m != 2) return pg_fail(PG_EINVAL, "gguf_gemv (few rows): %zu rows", m);
     switch ((k_in / 32 + 63) / 64) {
         case 1: return PG_FEWROWS_BPL(1);
         case 2: return PG_FEWROWS_BPL(2);
