@@ -98,15 +98,18 @@ GGUF_SHAPES = [
     (8, 4096, 14336, 1), (8, 300, 8192, 1), (8, 24, 16384, 1),  # two rows a wavefront under a long row: the digits shared through LDS (ragged last workgroups)
     # more than one row: matrix-core path (token tiles of 32, row tiles of 128, split K)
     (2, 130, 224, 33), (8, 131, 160, 40), (2, 515, 4096, 64), (8, 257, 6144, 35), (2, 14336, 4096, 4), (8, 4096, 14336, 16),
-    # Q4_0, two rows (three over up to 2^25 weights), K up to 8192: one launch, every wavefront's weight rows against all
-    # the activation rows (the one-row kernel's arithmetic: its tolerance); ragged rows and K segments
-    (2, 14336, 4096, 2), (2, 4096, 4096, 3), (2, 1003, 2080, 3), (2, 33, 96, 2), (2, 520, 8192, 2), (2, 8190, 1024, 3),
-    (2, 4096, 14336, 2), (2, 4096, 14336, 3), (2, 33, 96, 4),   # (longer K, more weights or four rows: matrix cores)
+    # Q4_0, two rows over at most 2^24 weights, K up to 8192: one launch, every wavefront's weight rows against both
+    # activation rows (the one-row kernel's arithmetic: its tolerance); ragged rows and K segments
+    (2, 4096, 4096, 2), (2, 1003, 2080, 2), (2, 33, 96, 2), (2, 520, 8192, 2), (2, 8190, 1024, 2),
+    (2, 14336, 4096, 2), (2, 4096, 4096, 3), (2, 1003, 2080, 3), (2, 8190, 1024, 3),
+    (2, 4096, 14336, 2), (2, 4096, 14336, 3), (2, 33, 96, 4),   # (more weights, longer K or more rows: matrix cores)
     # Q4_0, 3 .. 16 rows, K a multiple of 256: digits, then ONE matrix-core launch (a workgroup per 16 weight rows, its
     # wavefronts on runs of K with private LDS rings): rings of 4, 8 and 16 token rows, 1 to 8 wavefronts, ragged rows,
     # a K of 4 and of 9 units; 12 rows over a wide tensor keep the product split over K
     (2, 1000, 4096, 7), (2, 333, 1024, 5), (2, 4100, 8192, 16), (2, 96, 2304, 9), (2, 14336, 4096, 12), (2, 4096, 14336, 8),
     (2, 4096, 4096, 5), (2, 40, 36864, 4),
+    # up to 8 rows: 4 x 4 x 4 products; from 32 weight rows a CU on two weight tiles a workgroup (ragged last workgroup)
+    (2, 14336, 4096, 7), (2, 8200, 1024, 6), (2, 8200, 1024, 3), (8, 8200, 1280, 5), (8, 8200, 1280, 2),
     # the same over Q8_0 (a weight row is two streams of 16-byte half blocks)
     (8, 1000, 4096, 7), (8, 333, 1024, 2), (8, 4100, 8192, 16), (8, 96, 2304, 9), (8, 14336, 4096, 4), (8, 4096, 14336, 8), (8, 14336, 4096, 12),
     # Q4_1 (offset blocks): the streaming kernel with the block-sum term, one item per row
