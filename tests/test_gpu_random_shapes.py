@@ -74,6 +74,35 @@ def test_gguf_matmul_random_shapes(ctx, orc, seed):
         gw.free()
 
 
+@pytest.mark.parametrize("seed", [31, 32])
+def test_gguf_few_rows_random_shapes(ctx, orc, seed):
+    """2 .. 16 rows over K a multiple of 256: the one-launch matrix-core product (4 x 4 x 4 products up to 8 rows,
+    one or two weight tiles a workgroup, 16 x 16 x 32 above), ragged weight rows, outlier channels, a NaN."""
+    from peregrine_amd import gguf
+    rng = np.random.default_rng(seed)
+    for case in range(24):
+        typ = _pick(rng, 2, 8)
+        m = _pick(rng, 2, 3, 4, 5, 6, 7, 8, 9, 12, 16)
+        k_in = 256 * _pick(rng, 4, 5, 8, 9, 16, 17)
+        n_out = _pick(rng, 16, 17, 100, 333, 520, 1000, 4100, 8192, 8200, 9001)
+        say(f"gguf few rows random case {case}: type={typ} m={m} n_out={n_out} k_in={k_in}")
+        w = orc.rng_normal(seed * 1000 + case, n_out * k_in, 0.0, 0.02)
+        raw = {2: H.pack_q4_0, 8: H.pack_q8_0}[typ](w)
+        x = orc.rng_normal(seed * 1000 + 500 + case, m * k_in)
+        x.reshape(m, k_in)[:, :: max(1, k_in // 37)] *= 20
+        poisoned = rng.random() < 0.25
+        if poisoned:
+            x.reshape(m, k_in)[m - 1, int(rng.integers(k_in))] = np.nan      # that row is lost, the others are not
+        gw = gguf.GgufWeight(raw, typ, n_out, k_in, ctx)
+        got = gw.matmul(x, m).reshape(m, n_out)
+        want = orc.gguf_matmul(x, m, raw, typ, n_out, k_in).reshape(m, n_out)
+        for r in range(m - 1 if poisoned else m):
+            H.assert_close_rel(got[r], want[r], 1e-3, f"row {r}")
+        if poisoned:
+            assert np.isnan(got[m - 1]).all() and np.isnan(want[m - 1]).all()
+        gw.free()
+
+
 @pytest.mark.parametrize("seed", [41, 42])
 def test_gguf_matmul_random_shapes_on_the_f16_matrix_cores(ctx, orc, seed):
     """The many-row route forced for every shape it can take (K a multiple of 64, two rows and more): both tile shapes,
