@@ -714,6 +714,21 @@ def section_gguf(B, line):
             entry["cpu_baseline"] = cpu_q4[m_q]
         skinny.append(entry)
     line["gguf_q4_0_skinny"] = skinny
+    # the same tensors at the other small row counts (a few draft tokens being verified): whole call, digits' launch included
+    other = []
+    for m_q in (2, 3, 8, 12):
+        x_m = B.normal(1270 + m_q, (m_q, k_in))
+        y_m = torch.empty(m_q, n_out, device=dev)
+
+        def mm_step():
+            h = q4[B.i % Q4_ROT]
+            B.i += 1
+            check(lib.pg_gguf_matmul_dev(B.h, ptr(x_m), m_q, h, ptr(y_m)))
+
+        t_mm = B.timed(mm_step, B.dsteps, max(args.warmup, 8))
+        other.append({"rows": m_q, "ms_per_step": round(t_mm["ms_per_step"], 5),
+                      "weight_gbs": round(n_out * (k_in // 32) * 18 / (t_mm["ms_per_step"] * 1e-3) / 1e9, 1)})
+    line["gguf_q4_0_other_row_counts"] = other
     for h in q4:
         lib.pg_gguf_free(B.h, h)
     torch.cuda.empty_cache()
